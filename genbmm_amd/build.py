@@ -1,0 +1,75 @@
+"""Build step: compile the HIP sources into libgenbmm_gfx950.so (in-tree).
+
+    python -m genbmm_amd.build
+
+This takes the place of the reference's setup.py (setup.py:1-27, a
+torch CUDAExtension named `_genbmm`): there is no pybind11 / torch extension
+here, only a plain shared library with a C ABI (include/genbmm_gfx950.h) that
+genbmm_amd/_lib.py loads with ctypes.  hipcc cross-compiles for gfx950 without
+a GPU being present.
+"""
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIBDIR = os.path.join(HERE, "lib")
+LIBNAME = "libgenbmm_gfx950.so"
+SOURCES = ["dense_fwd.hip", "dense_bwd.hip", "banded.hip"]
+
+# -packed-fp32-ops is switched OFF: v_pk_{add,mul,fma}_f32 are not used by any
+# kernel here, and the compiler must not form them on its own either.
+HIPCC_FLAGS = [
+    "-O3",
+    "-std=c++17",
+    "--offload-arch=gfx950",
+    "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-fno-gpu-rdc",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def lib_path():
+    return os.path.join(LIBDIR, LIBNAME)
+
+
+def hipcc():
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; it is needed to build " + LIBNAME)
+    return exe
+
+
+def build(verbose=True):
+    """Compile every source for gfx950 and link the shared library. Always recompiles."""
+    os.makedirs(LIBDIR, exist_ok=True)
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    cc = hipcc()
+    procs = []
+    for src in SOURCES:
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        cmd = [cc] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src, obj, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
+    objs = []
+    for src, obj, proc in procs:
+        out = proc.communicate()[0].decode()
+        if proc.returncode != 0:
+            raise RuntimeError("hipcc failed on %s:\n%s" % (src, out))
+        objs.append(obj)
+    tmp = lib_path() + ".tmp"
+    cmd = [cc, "-shared", "-fPIC", "--offload-arch=gfx950", "-fno-gpu-rdc"] + objs + ["-o", tmp]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    os.replace(tmp, lib_path())
+    return lib_path()
+
+
+if __name__ == "__main__":
+    print(build(verbose="-q" not in sys.argv))

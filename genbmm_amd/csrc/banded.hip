@@ -1,0 +1,352 @@
+// Banded-matrix semiring multiply: forward, backward (both operands) and the
+// log-semiring second-order terms (gfx950).
+//
+// Band storage (reference genbmm/sparse.py:12-30): data[b, c, k] is the dense
+// element (row c + k - lu, column c); row c of `data` is dense column c.
+// For operands a (lu=a_lu, ld=a_ld, width Wa) and b (b_lu, b_ld, Wb) the
+// product has lu = a_lu + b_ld, ld = a_ld + b_lu, width Wo = Wa + Wb - 1 and
+//
+//   out[i, j] = (+)_k a[i, k] (x) b[o, k2],   o  = i + j - lu_out,
+//                                            k2 = k - j + (Wb - 1),
+//
+// over the k with 0 <= k < Wa, 0 <= k2 < Wb and 0 <= i + k - a_lu < n
+// (reference banded_cuda_kernel.cu:32-51; k2 there is (pos - o) + b_lu with
+// pos = i + k - a_lu, which simplifies to the expression above).  k2 does not
+// depend on i, so for a fixed output diagonal j the operands are walked as
+// two straight runs: a[i, klo..khi] and b[o, klo-j+Wb-1 ..].
+//
+// One lane per output element with lanes along the band axis (the contiguous
+// axis of every tensor), so stores are coalesced and neighbouring lanes read
+// overlapping runs that the vector L1 / L2 serve.
+#include "common.h"
+
+namespace genbmm {
+namespace {
+
+struct BandArgs {
+  const float* a;
+  const float* b;
+  const float* out;
+  const float* g;
+  const float* ua;
+  const float* ub;
+  const int32_t* idx;
+  float* o0;      // out        | grad_a
+  float* o1;      // -          | grad_b
+  float* o2;      // -          | grad_g
+  int32_t* oidx;  // forward argmax
+  int n, a_lu, Wa, b_lu, Wb, r_lu, Wo;
+};
+
+__device__ __forceinline__ int imax3(int a, int b, int c) { return max(a, max(b, c)); }
+__device__ __forceinline__ int imin3(int a, int b, int c) { return min(a, min(b, c)); }
+
+// Valid k range [klo, khi] of output cell (i, j); needs 0 <= o < n.
+__device__ __forceinline__ void k_range(const BandArgs& p, int i, int j, int& klo, int& khi) {
+  klo = imax3(0, j - (p.Wb - 1), p.a_lu - i);
+  khi = imin3(p.Wa - 1, j, p.n - 1 + p.a_lu - i);
+}
+
+// ------------------------------------------------------------------ forward
+// Reference banded_cuda_forward_kernel_mul (banded_cuda_kernel.cu:13-100).
+template <int MODE>
+__global__ __launch_bounds__(256) void k_band_fwd(const BandArgs p, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int j = (int)(e % p.Wo);
+  const long bi = e / p.Wo;  // batch*n + i
+  const int i = (int)(bi % p.n);
+  const int o = i + j - p.r_lu;
+  if (o < 0 || o >= p.n) {  // outside the matrix: the reference leaves its zero fill
+    p.o0[e] = 0.f;
+    if (MODE == GENBMM_BAND_MAX) p.oidx[e] = 0;
+    return;
+  }
+  int klo, khi;
+  k_range(p, i, j, klo, khi);
+  const float* ar = p.a + bi * p.Wa;
+  const float* br = p.b + (bi + (o - i)) * p.Wb + (p.Wb - 1 - j);  // br[k] = b[o][k2(k)]
+  if (MODE == GENBMM_BAND_MUL) {
+    float v = 0.f;
+    for (int k = klo; k <= khi; ++k) v = __builtin_fmaf(ar[k], br[k], v);
+    p.o0[e] = v;
+  } else if (MODE == GENBMM_BAND_MAX) {
+    float m = kFloor;
+    int ind = -1;
+    for (int k = klo; k <= khi; ++k) {
+      const float v = ar[k] + br[k];
+      if (v > m) {
+        m = v;
+        ind = k;
+      }
+    }
+    p.o0[e] = m;
+    p.oidx[e] = ind;
+  } else {
+    float m = kFloor;
+    for (int k = klo; k <= khi; ++k) m = fmaxf(m, ar[k] + br[k]);
+    const float nm = -m * kLog2e;
+    float s = 0.f;
+    for (int k = klo; k <= khi; ++k) s += fast_exp2(__builtin_fmaf(ar[k] + br[k], kLog2e, nm));
+    p.o0[e] = logf(s) + m;
+  }
+}
+
+// ----------------------------------------------------------------- backward
+// d out[i,j] / d a[i,k]: MUL b[o,k2]; LOG exp(a[i,k]+b[o,k2]-out[i,j]);
+// MAX [k == idx[i,j]].  grad_a[i,k] sums over j ascending (reference
+// banded_cuda_backward_kernel_mul, banded_cuda_kernel.cu:104-152).
+template <int MODE>
+__global__ __launch_bounds__(256) void k_band_bwd_a(const BandArgs p, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int k = (int)(e % p.Wa);
+  const long bi = e / p.Wa;
+  const int i = (int)(bi % p.n);
+  const int pos = i + k - p.a_lu;
+  float acc = 0.f;
+  if (pos >= 0 && pos < p.n) {
+    const int jlo = imax3(k, p.r_lu - i, 0);
+    const int jhi = imin3(k + p.Wb - 1, p.n - 1 + p.r_lu - i, p.Wo - 1);
+    const float* gr = p.g + bi * p.Wo;
+    // b[o][k2] = bw[j * (Wb - 1)] with o = i + j - r_lu, k2 = k - j + Wb - 1
+    const float* bw = p.b + (bi - p.r_lu) * p.Wb + k + p.Wb - 1;
+    if (MODE == GENBMM_BAND_MUL) {
+      for (int j = jlo; j <= jhi; ++j) acc = __builtin_fmaf(bw[(long)j * (p.Wb - 1)], gr[j], acc);
+    } else if (MODE == GENBMM_BAND_MAX) {
+      const int32_t* ir = p.idx + bi * p.Wo;
+      for (int j = jlo; j <= jhi; ++j) acc += (ir[j] == k) ? gr[j] : 0.f;
+    } else {
+      const float av = p.a[e];
+      const float* orow = p.out + bi * p.Wo;
+      for (int j = jlo; j <= jhi; ++j) {
+        const float w = fast_exp(av + bw[(long)j * (p.Wb - 1)] - orow[j]);
+        acc = __builtin_fmaf(w, gr[j], acc);
+      }
+    }
+  }
+  p.o0[e] = acc;
+}
+
+// grad_b[o,k2] sums, in ascending i, over the cells (i, j = o - i + r_lu) that
+// read b[o,k2], with k = k2 + j - (Wb - 1).  The reference gets the same
+// numbers by transposing g / out in band form on the host and calling the
+// kernel above with the operands swapped (sparse.py:436-446, 523-545, 625-635).
+template <int MODE>
+__global__ __launch_bounds__(256) void k_band_bwd_b(const BandArgs p, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int k2 = (int)(e % p.Wb);
+  const long bo = e / p.Wb;
+  const int o = (int)(bo % p.n);
+  const int prow = o + k2 - p.b_lu;
+  float acc = 0.f;
+  if (prow >= 0 && prow < p.n) {
+    const int jhi_k = p.Wb - 1 - k2 + p.Wa - 1;  // j with k = Wa-1
+    const int jlo_k = p.Wb - 1 - k2;             // j with k = 0
+    const int ilo = imax3(0, o + p.r_lu - min(jhi_k, p.Wo - 1), o + p.r_lu - (p.Wo - 1));
+    const int ihi = imin3(p.n - 1, o + p.r_lu - max(jlo_k, 0), o + p.r_lu);
+    const long base = bo - o;  // batch*n
+    const float bv = p.b[e];
+    for (int i = ilo; i <= ihi; ++i) {
+      const int j = o - i + p.r_lu;
+      const int k = k2 + j - (p.Wb - 1);
+      const long gi = (base + i) * p.Wo + j;
+      if (MODE == GENBMM_BAND_MUL) {
+        acc = __builtin_fmaf(p.a[(base + i) * p.Wa + k], p.g[gi], acc);
+      } else if (MODE == GENBMM_BAND_MAX) {
+        acc += (p.idx[gi] == k) ? p.g[gi] : 0.f;
+      } else {
+        const float w = fast_exp(p.a[(base + i) * p.Wa + k] + bv - p.out[gi]);
+        acc = __builtin_fmaf(w, p.g[gi], acc);
+      }
+    }
+  }
+  p.o1[e] = acc;
+}
+
+// ------------------------------------------------------ log second order
+// p = exp(a[i,k] + b[o,k2] - out[i,j]),  w = u_a[i,k] + u_b[o,k2]:
+//   t[i,j]       = sum_k p*w                        (gradient w.r.t. g)
+//   grad_a[i,k]  = sum_j g[i,j]*p*(w - t[i,j])
+//   grad_b[o,k2] = sum_i g[i,j]*p*(w - t[i,j])
+// With u_b = 0 these equal the reference's banded_cuda_backbackward_kernel_A/
+// _B/_C (banded_cuda_kernel.cu:154-350), whose inner loop sum_m (delta*s -
+// s*s2)*u[m] is s*(u[k] - t).
+__global__ __launch_bounds__(256) void k_band_bb_t(const BandArgs p, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int j = (int)(e % p.Wo);
+  const long bi = e / p.Wo;
+  const int i = (int)(bi % p.n);
+  const int o = i + j - p.r_lu;
+  float t = 0.f;
+  if (o >= 0 && o < p.n) {
+    int klo, khi;
+    k_range(p, i, j, klo, khi);
+    const long boff = (bi + (o - i)) * p.Wb + (p.Wb - 1 - j);
+    const float ov = p.out[e];
+    for (int k = klo; k <= khi; ++k) {
+      const float pr = fast_exp(p.a[bi * p.Wa + k] + p.b[boff + k] - ov);
+      const float w = (p.ua ? p.ua[bi * p.Wa + k] : 0.f) + (p.ub ? p.ub[boff + k] : 0.f);
+      t = __builtin_fmaf(pr, w, t);
+    }
+  }
+  p.o2[e] = t;
+}
+
+__global__ __launch_bounds__(256) void k_band_bb_a(const BandArgs p, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int k = (int)(e % p.Wa);
+  const long bi = e / p.Wa;
+  const int i = (int)(bi % p.n);
+  const int pos = i + k - p.a_lu;
+  float acc = 0.f;
+  if (pos >= 0 && pos < p.n) {
+    const int jlo = imax3(k, p.r_lu - i, 0);
+    const int jhi = imin3(k + p.Wb - 1, p.n - 1 + p.r_lu - i, p.Wo - 1);
+    const long bw = (bi - p.r_lu) * p.Wb + k + p.Wb - 1;
+    const float av = p.a[e];
+    const float uav = p.ua ? p.ua[e] : 0.f;
+    for (int j = jlo; j <= jhi; ++j) {
+      const long bj = bw + (long)j * (p.Wb - 1);
+      const long gi = bi * p.Wo + j;
+      const float pr = fast_exp(av + p.b[bj] - p.out[gi]);
+      const float w = uav + (p.ub ? p.ub[bj] : 0.f) - p.o2[gi];
+      acc = __builtin_fmaf(p.g[gi] * pr, w, acc);
+    }
+  }
+  p.o0[e] = acc;
+}
+
+__global__ __launch_bounds__(256) void k_band_bb_b(const BandArgs p, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int k2 = (int)(e % p.Wb);
+  const long bo = e / p.Wb;
+  const int o = (int)(bo % p.n);
+  const int prow = o + k2 - p.b_lu;
+  float acc = 0.f;
+  if (prow >= 0 && prow < p.n) {
+    const int jhi_k = p.Wb - 1 - k2 + p.Wa - 1;
+    const int jlo_k = p.Wb - 1 - k2;
+    const int ilo = imax3(0, o + p.r_lu - min(jhi_k, p.Wo - 1), o + p.r_lu - (p.Wo - 1));
+    const int ihi = imin3(p.n - 1, o + p.r_lu - max(jlo_k, 0), o + p.r_lu);
+    const long base = bo - o;
+    const float bv = p.b[e];
+    const float ubv = p.ub ? p.ub[e] : 0.f;
+    for (int i = ilo; i <= ihi; ++i) {
+      const int j = o - i + p.r_lu;
+      const int k = k2 + j - (p.Wb - 1);
+      const long gi = (base + i) * p.Wo + j;
+      const long ai = (base + i) * p.Wa + k;
+      const float pr = fast_exp(p.a[ai] + bv - p.out[gi]);
+      const float w = (p.ua ? p.ua[ai] : 0.f) + ubv - p.o2[gi];
+      acc = __builtin_fmaf(p.g[gi] * pr, w, acc);
+    }
+  }
+  p.o1[e] = acc;
+}
+
+int fill_band(BandArgs& p, int a_lu, int a_ld, int b_lu, int b_ld, int B, int n) {
+  if (a_lu < 0 || a_ld < 0 || b_lu < 0 || b_ld < 0) return GENBMM_E_BAND;
+  if (B < 0 || n < 0) return GENBMM_E_SHAPE;
+  const int64_t Wa = (int64_t)a_lu + a_ld + 1, Wb = (int64_t)b_lu + b_ld + 1;
+  const int64_t Wo = Wa + Wb - 1;
+  if (Wo > 0x3fffffff || (int64_t)B * n * Wo > ((int64_t)1 << 40)) return GENBMM_E_SHAPE;
+  p.n = n; p.a_lu = a_lu; p.Wa = (int)Wa; p.b_lu = b_lu; p.Wb = (int)Wb;
+  p.r_lu = a_lu + b_ld; p.Wo = (int)Wo;
+  return GENBMM_OK;
+}
+
+inline dim3 blocks_for(long total) { return dim3((unsigned)((total + 255) / 256)); }
+
+}  // namespace
+}  // namespace genbmm
+
+extern "C" {
+
+int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
+                      float* out, int32_t* idx, int B, int n, int mode, void* stream) {
+  using namespace genbmm;
+  if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
+    return GENBMM_E_MODE;
+  if (!a || !b || !out || (mode == GENBMM_BAND_MAX && !idx)) return GENBMM_E_NULLPTR;
+  BandArgs p{};
+  if (int e = fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return e;
+  p.a = a; p.b = b; p.o0 = out; p.oidx = idx;
+  const long total = (long)B * n * p.Wo;
+  if (total == 0) return GENBMM_OK;
+  hipStream_t s = (hipStream_t)stream;
+  if (mode == GENBMM_BAND_LOG)
+    hipLaunchKernelGGL(k_band_fwd<GENBMM_BAND_LOG>, blocks_for(total), dim3(256), 0, s, p, total);
+  else if (mode == GENBMM_BAND_MAX)
+    hipLaunchKernelGGL(k_band_fwd<GENBMM_BAND_MAX>, blocks_for(total), dim3(256), 0, s, p, total);
+  else
+    hipLaunchKernelGGL(k_band_fwd<GENBMM_BAND_MUL>, blocks_for(total), dim3(256), 0, s, p, total);
+  return launch_status();
+}
+
+int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
+                      const float* out, const int32_t* idx, const float* g, float* grad_a,
+                      float* grad_b, int B, int n, int mode, void* stream) {
+  using namespace genbmm;
+  if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
+    return GENBMM_E_MODE;
+  if (!a || !b || !g || !grad_a || !grad_b || (mode == GENBMM_BAND_LOG && !out) ||
+      (mode == GENBMM_BAND_MAX && !idx))
+    return GENBMM_E_NULLPTR;
+  BandArgs p{};
+  if (int e = fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return e;
+  p.a = a; p.b = b; p.out = out; p.idx = idx; p.g = g; p.o0 = grad_a; p.o1 = grad_b;
+  const long ta = (long)B * n * p.Wa, tb = (long)B * n * p.Wb;
+  if (ta == 0) return GENBMM_OK;
+  hipStream_t s = (hipStream_t)stream;
+  if (mode == GENBMM_BAND_LOG) {
+    hipLaunchKernelGGL(k_band_bwd_a<GENBMM_BAND_LOG>, blocks_for(ta), dim3(256), 0, s, p, ta);
+    hipLaunchKernelGGL(k_band_bwd_b<GENBMM_BAND_LOG>, blocks_for(tb), dim3(256), 0, s, p, tb);
+  } else if (mode == GENBMM_BAND_MAX) {
+    hipLaunchKernelGGL(k_band_bwd_a<GENBMM_BAND_MAX>, blocks_for(ta), dim3(256), 0, s, p, ta);
+    hipLaunchKernelGGL(k_band_bwd_b<GENBMM_BAND_MAX>, blocks_for(tb), dim3(256), 0, s, p, tb);
+  } else {
+    hipLaunchKernelGGL(k_band_bwd_a<GENBMM_BAND_MUL>, blocks_for(ta), dim3(256), 0, s, p, ta);
+    hipLaunchKernelGGL(k_band_bwd_b<GENBMM_BAND_MUL>, blocks_for(tb), dim3(256), 0, s, p, tb);
+  }
+  return launch_status();
+}
+
+int genbmm_banded_bwdbwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
+                         const float* out, const float* g, const float* u_a, const float* u_b,
+                         float* grad_a, float* grad_b, float* grad_g, int B, int n,
+                         void* stream) {
+  using namespace genbmm;
+  if (!a || !b || !out || !g || !grad_a || !grad_b || !grad_g || (!u_a && !u_b))
+    return GENBMM_E_NULLPTR;
+  BandArgs p{};
+  if (int e = fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return e;
+  p.a = a; p.b = b; p.out = out; p.g = g; p.ua = u_a; p.ub = u_b;
+  p.o0 = grad_a; p.o1 = grad_b; p.o2 = grad_g;
+  const long ta = (long)B * n * p.Wa, tb = (long)B * n * p.Wb, to = (long)B * n * p.Wo;
+  if (to == 0) return GENBMM_OK;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(k_band_bb_t, blocks_for(to), dim3(256), 0, s, p, to);
+  hipLaunchKernelGGL(k_band_bb_a, blocks_for(ta), dim3(256), 0, s, p, ta);
+  hipLaunchKernelGGL(k_band_bb_b, blocks_for(tb), dim3(256), 0, s, p, tb);
+  return launch_status();
+}
+
+const char* genbmm_version(void) { return "genbmm-gfx950 0.1"; }
+
+const char* genbmm_error_string(int code) {
+  switch (code) {
+    case GENBMM_OK: return "ok";
+    case GENBMM_E_NULLPTR: return "a required pointer argument is NULL";
+    case GENBMM_E_SHAPE: return "a dimension is negative or too large";
+    case GENBMM_E_MODE: return "unknown semiring mode";
+    case GENBMM_E_BAND: return "negative band width";
+    default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
+  }
+}
+
+}  // extern "C"

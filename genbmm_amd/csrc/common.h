@@ -1,0 +1,202 @@
+// Shared device/host helpers for the gfx950 semiring-matmul kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/genbmm_gfx950.h"
+
+namespace genbmm {
+
+// Floor of every running maximum, as in the reference kernels
+// (matmul_cuda_kernel.cu:31,62,93,139; banded_cuda_kernel.cu:44,79).
+constexpr float kFloor = -1e9f;
+constexpr float kLog2e = 1.44269504088896340736f;
+constexpr float kLn2 = 0.69314718055994530942f;
+
+// v_exp_f32 / v_log_f32: base-2 hardware transcendentals.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// exp(x) for x that is already a difference (x <= ~0): one multiply + v_exp_f32.
+__device__ __forceinline__ float fast_exp(float x) { return fast_exp2(x * kLog2e); }
+
+constexpr int kPad = 4;  // LDS row padding (floats); keeps float4 alignment
+
+// ---------------------------------------------------------------- tile loaders
+//
+// Both loaders move a [RED x OUT] tile into LDS laid out as lds[red][out]
+// (row stride OUT + kPad) through registers, so that the global loads of the
+// next tile can be in flight while the current tile is being consumed.
+// Out-of-range elements are filled with 0; kernels never let those reach a
+// stored result (reduction loops stop at the true extent, stores are masked).
+
+// Operand stored in global memory as [out][red] (contiguous along the
+// reduction axis), leading dimension ld.
+template <int OUT, int RED, int NT>
+struct TileOutMajor {
+  static constexpr int C4 = RED / 4;
+  static constexpr int NV = OUT * C4;
+  static constexpr int PER = (NV + NT - 1) / NT;
+  static constexpr int LD = OUT + kPad;
+  float4 r[PER];
+
+  __device__ __forceinline__ void gload(const float* __restrict__ base, long ld,
+                                        int out0, int red0, int out_lim,
+                                        int red_lim, bool vec, int tid) {
+#pragma unroll
+    for (int l = 0; l < PER; ++l) {
+      const int idx = tid + l * NT;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (NV % NT == 0 || idx < NV) {
+        const int row = idx / C4, c4 = idx % C4;
+        const int go = out0 + row, gr = red0 + c4 * 4;
+        if (go < out_lim && gr < red_lim) {
+          const float* p = base + (long)go * ld + gr;
+          if (vec && gr + 3 < red_lim) {
+            v = *reinterpret_cast<const float4*>(p);
+          } else {
+            v.x = p[0];
+            if (gr + 1 < red_lim) v.y = p[1];
+            if (gr + 2 < red_lim) v.z = p[2];
+            if (gr + 3 < red_lim) v.w = p[3];
+          }
+        }
+      }
+      r[l] = v;
+    }
+  }
+
+  __device__ __forceinline__ void sstore(float* __restrict__ lds, int tid) const {
+#pragma unroll
+    for (int l = 0; l < PER; ++l) {
+      const int idx = tid + l * NT;
+      if (NV % NT == 0 || idx < NV) {
+        const int row = idx / C4, c4 = idx % C4;
+        float* p = lds + (c4 * 4) * LD + row;
+        p[0] = r[l].x;
+        p[LD] = r[l].y;
+        p[2 * LD] = r[l].z;
+        p[3 * LD] = r[l].w;
+      }
+    }
+  }
+};
+
+// Operand stored in global memory as [red][out] (contiguous along the output
+// axis), leading dimension ld.
+template <int OUT, int RED, int NT>
+struct TileRedMajor {
+  static constexpr int C4 = OUT / 4;
+  static constexpr int NV = RED * C4;
+  static constexpr int PER = (NV + NT - 1) / NT;
+  static constexpr int LD = OUT + kPad;
+  float4 r[PER];
+
+  __device__ __forceinline__ void gload(const float* __restrict__ base, long ld,
+                                        int out0, int red0, int out_lim,
+                                        int red_lim, bool vec, int tid) {
+#pragma unroll
+    for (int l = 0; l < PER; ++l) {
+      const int idx = tid + l * NT;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (NV % NT == 0 || idx < NV) {
+        const int row = idx / C4, c4 = idx % C4;
+        const int gr = red0 + row, go = out0 + c4 * 4;
+        if (gr < red_lim && go < out_lim) {
+          const float* p = base + (long)gr * ld + go;
+          if (vec && go + 3 < out_lim) {
+            v = *reinterpret_cast<const float4*>(p);
+          } else {
+            v.x = p[0];
+            if (go + 1 < out_lim) v.y = p[1];
+            if (go + 2 < out_lim) v.z = p[2];
+            if (go + 3 < out_lim) v.w = p[3];
+          }
+        }
+      }
+      r[l] = v;
+    }
+  }
+
+  __device__ __forceinline__ void sstore(float* __restrict__ lds, int tid) const {
+#pragma unroll
+    for (int l = 0; l < PER; ++l) {
+      const int idx = tid + l * NT;
+      if (NV % NT == 0 || idx < NV) {
+        const int row = idx / C4, c4 = idx % C4;
+        *reinterpret_cast<float4*>(lds + row * LD + c4 * 4) = r[l];
+      }
+    }
+  }
+};
+
+// Read NV4 float4 fragments lds[off + q*stride4 .. +4) into dst[4*NV4].
+template <int NV4>
+__device__ __forceinline__ void lds_frag(const float* __restrict__ row, int off,
+                                         int stride, float* dst) {
+#pragma unroll
+  for (int q = 0; q < NV4; ++q) {
+    const float4 v = *reinterpret_cast<const float4*>(row + off + q * stride);
+    dst[4 * q + 0] = v.x;
+    dst[4 * q + 1] = v.y;
+    dst[4 * q + 2] = v.z;
+    dst[4 * q + 3] = v.w;
+  }
+}
+
+// 16-byte alignment test used to enable float4 global accesses.
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ------------------------------------------------------------------- Philox
+// Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3",
+// SC'11): multipliers 0xD2511F53 / 0xCD9E8D57, Weyl key increments
+// 0x9E3779B9 / 0xBB67AE85, ten rounds.
+struct Philox4 {
+  uint32_t x[4];
+};
+
+__host__ __device__ inline Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2,
+                                                 uint32_t c3, uint32_t k0, uint32_t k1) {
+#pragma unroll
+  for (int round = 0; round < 10; ++round) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+    const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    const uint32_t n1 = (uint32_t)p1;
+    const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    const uint32_t n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  Philox4 r;
+  r.x[0] = c0; r.x[1] = c1; r.x[2] = c2; r.x[3] = c3;
+  return r;
+}
+
+// Uniform in [0,1) of output cell `i` for stream (seed, offset).
+__host__ __device__ inline float philox_uniform(uint64_t i, uint64_t seed, uint64_t offset) {
+  const Philox4 r = philox4x32_10((uint32_t)i, (uint32_t)(i >> 32), (uint32_t)offset,
+                                  (uint32_t)(offset >> 32), (uint32_t)seed,
+                                  (uint32_t)(seed >> 32));
+  return (float)(r.x[0] >> 8) * (1.0f / 16777216.0f);
+}
+
+// ------------------------------------------------------------- host helpers
+inline int check_dense_dims(int B, int M, int K, int N) {
+  if (B < 0 || M < 0 || K < 0 || N < 0) return GENBMM_E_SHAPE;
+  const int64_t lim = (int64_t)1 << 40;  // element counts are 64-bit inside
+  if ((int64_t)B * M * K > lim || (int64_t)B * K * N > lim || (int64_t)B * M * N > lim)
+    return GENBMM_E_SHAPE;
+  return GENBMM_OK;
+}
+
+inline int launch_status() {
+  const hipError_t e = hipGetLastError();
+  return e == hipSuccess ? GENBMM_OK : (int)e;
+}
+
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+}  // namespace genbmm

@@ -1,0 +1,210 @@
+"""Dense semiring batched matmul with autograd: logbmm, maxbmm, samplebmm, prodmaxbmm.
+
+Same public contract as the reference's genbmm/genmul.py:100-103: each op takes
+contiguous device tensors a (B, M, K) and b (B, K, N) and returns (B, M, N);
+all four are differentiable and logbmm is twice differentiable.  The work is
+done by the HIP kernels behind the C ABI in include/genbmm_gfx950.h.
+
+Differences in mechanism (not in results):
+  * logbmm's backward produces grad_a and grad_b from one library call that
+    reads every operand in place; the reference calls its kernel twice and
+    transposes b, a, g, out, maxes and the result in between (genmul.py:35-41).
+  * no `maxes` tensor is saved: exp(a+b-mx)/exp(out-mx) == exp(a+b-out).
+  * the arg-max / sample index stays int32 into the backward; the reference
+    converts it (and a, b, g) to float first (genmul.py:62-65).
+  * samplebmm draws its uniforms from a counter-based Philox4x32-10 stream
+    keyed by torch's CUDA generator seed instead of torch::rand
+    (matmul_cuda_kernel.cu:517).
+"""
+import torch
+
+from . import _lib
+
+_COMPUTE = torch.float32
+_UPCAST = (torch.float16, torch.bfloat16)
+
+
+def _prep(a, b):
+    """Validate, and widen half types to the fp32 the kernels compute in."""
+    if not isinstance(a, torch.Tensor) or not isinstance(b, torch.Tensor):
+        raise RuntimeError("a and b must be tensors")
+    if a.dtype != b.dtype:
+        raise RuntimeError("a and b must have the same dtype, got %s and %s" % (a.dtype, b.dtype))
+    if a.dtype in _UPCAST:
+        _lib.require(a, "a", dtype=a.dtype)
+        _lib.require(b, "b", dtype=b.dtype)
+        a, b = a.float(), b.float()
+    elif a.dtype != _COMPUTE:
+        raise RuntimeError(
+            "genbmm_amd computes in float32; %s inputs are not supported" % a.dtype
+        )
+    dims = _lib.dense_dims(a, b)
+    return a, b, dims
+
+
+def _call(name, t, *args):
+    lib = _lib.load()
+    with _lib.device_of(t):
+        _lib.check(getattr(lib, name)(*args, _lib.stream_of(t)), name)
+
+
+# --------------------------------------------------------------------- logbmm
+class _LogBmmGrad(torch.autograd.Function):
+    """(a, b, g, out) -> (grad_a, grad_b); itself differentiable in (a, b, g).
+
+    Plays the role of the reference's LogMatMulBack (genmul.py:11-24), which
+    yields grad_a only and is applied twice per backward.
+    """
+
+    @staticmethod
+    def forward(ctx, a, b, g, out):
+        B, M, K, N = _lib.dense_dims(a, b)
+        grad_a = torch.empty_like(a)
+        grad_b = torch.empty_like(b)
+        _call("genbmm_logbmm_bwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g),
+              _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
+        ctx.save_for_backward(a, b, g, out)
+        ctx.set_materialize_grads(False)
+        return grad_a, grad_b
+
+    @staticmethod
+    def backward(ctx, u_a, u_b):
+        if u_a is None and u_b is None:
+            return None, None, None, None
+        a, b, g, out = ctx.saved_tensors
+        B, M, K, N = _lib.dense_dims(a, b)
+        u_a = None if u_a is None else u_a.contiguous()
+        u_b = None if u_b is None else u_b.contiguous()
+        ga = torch.empty_like(a)
+        gb = torch.empty_like(b)
+        gg = torch.empty_like(g)
+        _call("genbmm_logbmm_bwdbwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g),
+              _lib.ptr(u_a), _lib.ptr(u_b), _lib.ptr(ga), _lib.ptr(gb), _lib.ptr(gg), B, M, K, N)
+        return ga, gb, gg, None
+
+
+class LogMatMul(torch.autograd.Function):
+    """out[b,m,n] = logsumexp_k(a[b,m,k] + b[b,k,n])   (reference genmul.py:27-41)."""
+
+    @staticmethod
+    def forward(ctx, a, b):
+        in_dtype = a.dtype if isinstance(a, torch.Tensor) else None
+        a, b, (B, M, K, N) = _prep(a, b)
+        out = torch.empty(B, M, N, dtype=_COMPUTE, device=a.device)
+        _call("genbmm_logbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), B, M, K, N)
+        ctx.save_for_backward(a, b, out)
+        ctx.in_dtype = in_dtype
+        return out.to(in_dtype)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        a, b, out = ctx.saved_tensors
+        grad_a, grad_b = _LogBmmGrad.apply(a, b, grad_output.to(_COMPUTE).contiguous(), out)
+        return grad_a.to(ctx.in_dtype), grad_b.to(ctx.in_dtype)
+
+
+# ------------------------------------------------- max / sample / prod-max
+def _argmax_backward(ctx, grad_output, prod):
+    a, b, idx = ctx.saved_tensors
+    B, M, K, N = ctx.dims
+    g = grad_output.to(_COMPUTE).contiguous()
+    grad_a = torch.empty(B, M, K, dtype=_COMPUTE, device=g.device)
+    grad_b = torch.empty(B, K, N, dtype=_COMPUTE, device=g.device)
+    if prod:
+        _call("genbmm_prodmax_bwd", g, _lib.ptr(a), _lib.ptr(b), _lib.ptr(idx), _lib.ptr(g),
+              _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
+    else:
+        _call("genbmm_argmax_bwd", g, _lib.ptr(idx), _lib.ptr(g), _lib.ptr(grad_a),
+              _lib.ptr(grad_b), B, M, K, N)
+    return grad_a.to(ctx.in_dtype), grad_b.to(ctx.in_dtype)
+
+
+class MaxMatMul(torch.autograd.Function):
+    """out = max_k(a + b), ties to the lowest k   (reference genmul.py:52-65)."""
+
+    @staticmethod
+    def forward(ctx, a, b):
+        in_dtype = a.dtype if isinstance(a, torch.Tensor) else None
+        a, b, dims = _prep(a, b)
+        B, M, K, N = dims
+        out = torch.empty(B, M, N, dtype=_COMPUTE, device=a.device)
+        idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
+        _call("genbmm_maxbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
+              B, M, K, N)
+        empty = a.new_empty(0)
+        ctx.save_for_backward(empty, empty, idx)
+        ctx.dims, ctx.in_dtype = dims, in_dtype
+        return out.to(in_dtype)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return _argmax_backward(ctx, grad_output, prod=False)
+
+
+class ProdMaxMatMul(torch.autograd.Function):
+    """out = max_k(a * b)   (reference genmul.py:84-97)."""
+
+    @staticmethod
+    def forward(ctx, a, b):
+        in_dtype = a.dtype if isinstance(a, torch.Tensor) else None
+        a, b, dims = _prep(a, b)
+        B, M, K, N = dims
+        out = torch.empty(B, M, N, dtype=_COMPUTE, device=a.device)
+        idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
+        _call("genbmm_prodmaxbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
+              B, M, K, N)
+        ctx.save_for_backward(a, b, idx)
+        ctx.dims, ctx.in_dtype = dims, in_dtype
+        return out.to(in_dtype)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return _argmax_backward(ctx, grad_output, prod=True)
+
+
+_SEED_SALT = 0x67656E626D6D  # keeps the stream apart from torch's own Philox use
+
+
+def _next_stream(device):
+    """(seed, offset) for the next samplebmm call: follows torch.manual_seed and
+    advances the CUDA generator's offset so that successive calls differ."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    gen = torch.cuda.default_generators[index]
+    seed = (gen.initial_seed() ^ _SEED_SALT) & 0xFFFFFFFFFFFFFFFF
+    offset = gen.get_offset()
+    gen.set_offset(offset + 4)
+    return seed, offset
+
+
+class SampleMatMul(torch.autograd.Function):
+    """out = logsumexp_k(a + b); the gradient is a one-hot sample k ~ softmax_k(a + b)
+    (reference genmul.py:68-81).  `stream` = (seed, offset) pins the Philox stream."""
+
+    @staticmethod
+    def forward(ctx, a, b, stream=None):
+        in_dtype = a.dtype if isinstance(a, torch.Tensor) else None
+        a, b, dims = _prep(a, b)
+        B, M, K, N = dims
+        seed, offset = _next_stream(a.device) if stream is None else stream
+        out = torch.empty(B, M, N, dtype=_COMPUTE, device=a.device)
+        idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
+        _call("genbmm_samplebmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
+              int(seed) & 0xFFFFFFFFFFFFFFFF, int(offset) & 0xFFFFFFFFFFFFFFFF, B, M, K, N)
+        empty = a.new_empty(0)
+        ctx.save_for_backward(empty, empty, idx)
+        ctx.dims, ctx.in_dtype = dims, in_dtype
+        return out.to(in_dtype)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return _argmax_backward(ctx, grad_output, prod=False) + (None,)
+
+
+def samplebmm(a, b, stream=None):
+    """genbmm.samplebmm(a, b); `stream=(seed, offset)` makes the draw reproducible."""
+    return SampleMatMul.apply(a, b, stream)
+
+
+logbmm = LogMatMul.apply
+maxbmm = MaxMatMul.apply
+prodmaxbmm = ProdMaxMatMul.apply

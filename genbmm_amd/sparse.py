@@ -1,0 +1,297 @@
+"""Banded matrices in band storage and their semiring products.
+
+Public surface of the reference's genbmm/sparse.py: `banddiag` (:12-30) and
+`BandedMatrix` (:80-266) with `multiply`, `multiply_log`, `multiply_max`,
+`transpose`, `to_dense`, `op`, `band_shift`, `band_pad`, `band_unshift`,
+`col_shift`, `col_unshift`, `_expand`.
+
+Layout: `data` is (batch, n, lu + ld + 1) and data[b, c, k] is the dense
+element at row c + k - lu, column c: row c of `data` holds dense column c,
+`lu` entries above the diagonal, the diagonal, `ld` entries below.
+
+The three products run on the GPU through include/genbmm_gfx950.h
+(genbmm_banded_fwd / _bwd / _bwdbwd).  The structural operations are index
+arithmetic in plain torch and work on any device.  The reference's Python
+triple-loop products (`multiply_simple` and friends, :268-401), which it uses
+when its extension is absent, have no counterpart here: a product on CPU
+tensors raises.
+"""
+import torch
+import torch.nn.functional as F
+
+from . import _lib
+
+MODE_LOG, MODE_MAX, MODE_MUL = 0, 1, 3
+
+
+def _band_rows(n_cols, lu, ld, n_rows, device):
+    """row[c, k] = c + k - lu (dense row of band cell (c, k)) and its validity mask."""
+    c = torch.arange(n_cols, device=device).unsqueeze(1)
+    k = torch.arange(lu + ld + 1, device=device).unsqueeze(0)
+    row = c + k - lu
+    return row, (row >= 0) & (row < n_rows)
+
+
+def banddiag(orig_x, lu, ld, fill=0):
+    """Band storage of the dense (..., n, n) matrix `orig_x`, keeping `lu` super- and
+    `ld` sub-diagonals.  Returns (band, orig_x) like the reference (sparse.py:12-30),
+    whose second value is the input seen through its padded copy.  Cells that fall
+    outside the matrix hold 0 (the reference ignores `fill` here as well)."""
+    n_rows, n_cols = orig_x.shape[-2], orig_x.shape[-1]
+    row, ok = _band_rows(n_cols, lu, ld, n_rows, orig_x.device)
+    col = torch.arange(n_cols, device=orig_x.device).unsqueeze(1).expand_as(row)
+    band = orig_x[..., row.clamp(0, max(n_rows - 1, 0)), col]
+    band = torch.where(ok, band, torch.zeros((), dtype=band.dtype, device=band.device))
+    return band, orig_x
+
+
+def _band_transpose(data, lu, ld):
+    """Band data of the transposed matrix (which has lu' = ld, ld' = lu):
+    T[i, k] = data[i + k - ld, W - 1 - k] when that row exists, else 0
+    (reference Transpose / repdiag, sparse.py:33-77)."""
+    n, width = data.shape[-2], data.shape[-1]
+    i = torch.arange(n, device=data.device).unsqueeze(1)
+    k = torch.arange(width, device=data.device).unsqueeze(0)
+    src = i + k - ld
+    ok = (src >= 0) & (src < n)
+    gathered = data[..., src.clamp(0, max(n - 1, 0)), (width - 1 - k).expand_as(src)]
+    return torch.where(ok, gathered, torch.zeros((), dtype=data.dtype, device=data.device))
+
+
+class BandedMatrix:
+    def __init__(self, data, lu, ld, fill=0):
+        batch, n, off = data.shape
+        assert off == lu + ld + 1, "Offsets need to add up."
+        self.data = data
+        self.fill = fill
+        self.lu, self.ld = lu, ld
+        self.width = lu + ld + 1
+
+    # ------------------------------------------------------------ structure
+    def _new(self, lu, ld):
+        batch, n, _ = self.data.shape
+        return self.data.new_full((batch, n, lu + ld + 1), self.fill)
+
+    def band_shift(self, t):
+        """Drop `t` leading band cells and pad `t` at the end (t < 0: the other way);
+        the same numbers are re-labelled lu + t / ld - t (reference sparse.py:96-110)."""
+        if t == 0:
+            return self
+        if t > 0:
+            v = F.pad(self.data[:, :, t:], (0, t), value=self.fill)
+        else:
+            v = F.pad(self.data[:, :, :t], (-t, 0), value=self.fill)
+        return BandedMatrix(v, self.lu + t, self.ld - t, self.fill)
+
+    def band_pad(self, t):
+        """Widen the band by `t` fill cells on both sides (reference sparse.py:112-123)."""
+        if t == 0:
+            return self
+        v = F.pad(self.data, (abs(t), abs(t)), value=self.fill)
+        return BandedMatrix(v, self.lu + t, self.ld + t, self.fill)
+
+    def band_unshift(self):
+        """One fill cell in front, last cell dropped; lu - 1 / ld + 1 (sparse.py:137-152)."""
+        v = F.pad(self.data[:, :, :-1], (1, 0), value=self.fill)
+        return BandedMatrix(v, self.lu - 1, self.ld + 1, self.fill)
+
+    def col_shift(self, t):
+        """Drop the first `t` columns and append `t` fill columns (t < 0: the other
+        way); lu - t / ld + t (reference sparse.py:154-165)."""
+        if t == 0:
+            return self
+        if t > 0:
+            v = F.pad(self.data[:, t:, :], (0, 0, 0, t), value=self.fill)
+        else:
+            v = F.pad(self.data[:, :t, :], (0, 0, -t, 0), value=self.fill)
+        return BandedMatrix(v, self.lu - t, self.ld + t, self.fill)
+
+    def col_unshift(self):
+        """One fill column in front, last column dropped; lu + 1 / ld - 1 (sparse.py:167-182)."""
+        v = F.pad(self.data[:, :-1, :], (0, 0, 1, 0), value=self.fill)
+        return BandedMatrix(v, self.lu + 1, self.ld - 1, self.fill)
+
+    def to_dense(self):
+        """Dense (batch, n, n) matrix; cells outside the band hold `fill` (sparse.py:184-190)."""
+        batch, n, _ = self.data.shape
+        row, ok = _band_rows(n, self.lu, self.ld, n, self.data.device)
+        col = torch.arange(n, device=self.data.device).unsqueeze(1).expand_as(row)
+        full = self.data.new_full((batch, n, n), self.fill)
+        full[:, row[ok], col[ok]] = self.data[:, ok]
+        return full
+
+    def _expand(self, lu, ld):
+        """Same matrix in a wider band (lu >= self.lu, ld >= self.ld) (sparse.py:192-197)."""
+        data = self._new(lu, ld)
+        s = lu - self.lu
+        data[:, :, s : s + self.width] = self.data
+        return BandedMatrix(data, lu, ld, self.fill)
+
+    def op(self, other, op, zero=0):
+        """Element-wise `op(self, other)` on the union band; cells only one operand
+        covers see `zero` for the other (reference sparse.py:199-212)."""
+        lu = max(self.lu, other.lu)
+        ld = max(self.ld, other.ld)
+        data = self._new(lu, ld).fill_(zero)
+        s1 = lu - self.lu
+        data[:, :, s1 : s1 + self.width] = self.data
+        s2 = lu - other.lu
+        data[:, :, s2 : s2 + other.width] = op(data[:, :, s2 : s2 + other.width], other.data)
+        return BandedMatrix(data, lu, ld, self.fill)
+
+    def transpose(self):
+        """Band form of the transposed matrix (reference sparse.py:214-218)."""
+        return BandedMatrix(_band_transpose(self.data, self.lu, self.ld), self.ld, self.lu, self.fill)
+
+    # ------------------------------------------------------------- products
+    def _product(self, other, fn):
+        batch, n, _ = self.data.shape
+        assert other.data.shape[1] == n
+        lu = self.lu + other.ld
+        ld = self.ld + other.lu
+        out = fn(self.data, self.lu, self.ld, other.data, other.lu, other.ld, lu, ld)
+        return BandedMatrix(out, lu, ld, self.fill)
+
+    def multiply(self, other):
+        """Dense(other)^T @ Dense(self) in band form (reference sparse.py:229-240)."""
+        return self._product(other, bandedbmm)
+
+    def multiply_log(self, other):
+        """The same product in the (logsumexp, +) semiring (reference sparse.py:242-253)."""
+        return self._product(other, bandedlogbmm)
+
+    def multiply_max(self, other):
+        """The same product in the (max, +) semiring (reference sparse.py:255-266)."""
+        return self._product(other, bandedmaxbmm)
+
+
+# ------------------------------------------------------------------ autograd
+def _check_pair(a, b):
+    _lib.require(a, "a")
+    _lib.require(b, "b", device=a.device)
+    if a.shape[:2] != b.shape[:2]:
+        raise RuntimeError("banded operands disagree: %s vs %s" % (tuple(a.shape), tuple(b.shape)))
+    return a.shape[0], a.shape[1]
+
+
+def _call(name, t, *args):
+    lib = _lib.load()
+    with _lib.device_of(t):
+        _lib.check(getattr(lib, name)(*args, _lib.stream_of(t)), name)
+
+
+def _forward(a, a_lu, a_ld, b, b_lu, b_ld, mode):
+    a = a.contiguous()
+    b = b.contiguous()
+    B, n = _check_pair(a, b)
+    if a.shape[2] != a_lu + a_ld + 1 or b.shape[2] != b_lu + b_ld + 1:
+        raise RuntimeError("band widths do not match lu + ld + 1")
+    wo = a.shape[2] + b.shape[2] - 1
+    out = torch.empty(B, n, wo, dtype=torch.float32, device=a.device)
+    idx = torch.empty(B, n, wo, dtype=torch.int32, device=a.device) if mode == MODE_MAX else None
+    _call("genbmm_banded_fwd", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
+          _lib.ptr(out), _lib.ptr(idx), B, n, mode)
+    return a, b, out, idx
+
+
+def _backward(a, b, bands, out, idx, g, mode):
+    a_lu, a_ld, b_lu, b_ld = bands
+    B, n = a.shape[0], a.shape[1]
+    g = g.to(torch.float32).contiguous()
+    grad_a = torch.empty_like(a)
+    grad_b = torch.empty_like(b)
+    _call("genbmm_banded_bwd", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
+          _lib.ptr(out), _lib.ptr(idx), _lib.ptr(g), _lib.ptr(grad_a), _lib.ptr(grad_b),
+          B, n, mode)
+    return grad_a, grad_b
+
+
+_NO_BAND_GRADS = (None,) * 6
+
+
+class BandedMul(torch.autograd.Function):
+    """(+, *) banded product (reference sparse.py:404-447)."""
+
+    @staticmethod
+    def forward(ctx, a, a_lu, a_ld, b, b_lu, b_ld, o_lu, o_ld):
+        a, b, out, _ = _forward(a, a_lu, a_ld, b, b_lu, b_ld, MODE_MUL)
+        ctx.save_for_backward(a, b)
+        ctx.bands = (a_lu, a_ld, b_lu, b_ld)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        a, b = ctx.saved_tensors
+        grad_a, grad_b = _backward(a, b, ctx.bands, None, None, grad_output, MODE_MUL)
+        return (grad_a, None, None, grad_b) + (None,) * 4
+
+
+class _BandedLogGrad(torch.autograd.Function):
+    """(a, b, g, out) -> (grad_a, grad_b) of the log product, differentiable in
+    (a, b, g).  Plays the role of the reference's BandedLogMulBack
+    (sparse.py:466-508), which yields one gradient per call and needs g, out and
+    maxes transposed in band form for the second operand."""
+
+    @staticmethod
+    def forward(ctx, a, b, g, out, bands):
+        grad_a, grad_b = _backward(a, b, bands, out, None, g, MODE_LOG)
+        ctx.save_for_backward(a, b, g, out)
+        ctx.bands = bands
+        ctx.set_materialize_grads(False)
+        return grad_a, grad_b
+
+    @staticmethod
+    def backward(ctx, u_a, u_b):
+        if u_a is None and u_b is None:
+            return (None,) * 5
+        a, b, g, out = ctx.saved_tensors
+        a_lu, a_ld, b_lu, b_ld = ctx.bands
+        u_a = None if u_a is None else u_a.contiguous()
+        u_b = None if u_b is None else u_b.contiguous()
+        ga, gb, gg = torch.empty_like(a), torch.empty_like(b), torch.empty_like(g)
+        _call("genbmm_banded_bwdbwd", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
+              _lib.ptr(out), _lib.ptr(g), _lib.ptr(u_a), _lib.ptr(u_b),
+              _lib.ptr(ga), _lib.ptr(gb), _lib.ptr(gg), a.shape[0], a.shape[1])
+        return ga, gb, gg, None, None
+
+
+class BandedLogMul(torch.autograd.Function):
+    """(logsumexp, +) banded product, twice differentiable (reference sparse.py:510-545)."""
+
+    @staticmethod
+    def forward(ctx, a, a_lu, a_ld, b, b_lu, b_ld, o_lu, o_ld):
+        a, b, out, _ = _forward(a, a_lu, a_ld, b, b_lu, b_ld, MODE_LOG)
+        ctx.save_for_backward(a, b, out)
+        ctx.bands = (a_lu, a_ld, b_lu, b_ld)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        a, b, out = ctx.saved_tensors
+        g = grad_output.to(torch.float32).contiguous()
+        grad_a, grad_b = _BandedLogGrad.apply(a, b, g, out, ctx.bands)
+        return (grad_a, None, None, grad_b) + (None,) * 4
+
+
+class BandedMaxMul(torch.autograd.Function):
+    """(max, +) banded product (reference sparse.py:579-637).  One forward launch:
+    the arg-max is kept in a's band frame and both gradients read it there, where the
+    reference runs the forward a second time with the operands swapped."""
+
+    @staticmethod
+    def forward(ctx, a, a_lu, a_ld, b, b_lu, b_ld, o_lu, o_ld):
+        a, b, out, idx = _forward(a, a_lu, a_ld, b, b_lu, b_ld, MODE_MAX)
+        ctx.save_for_backward(a, b, idx)
+        ctx.bands = (a_lu, a_ld, b_lu, b_ld)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        a, b, idx = ctx.saved_tensors
+        grad_a, grad_b = _backward(a, b, ctx.bands, None, idx, grad_output, MODE_MAX)
+        return (grad_a, None, None, grad_b) + (None,) * 4
+
+
+bandedbmm = BandedMul.apply
+bandedlogbmm = BandedLogMul.apply
+bandedmaxbmm = BandedMaxMul.apply

@@ -1,0 +1,201 @@
+/*
+ * genbmm_gfx950.h — C ABI of libgenbmm_gfx950.so
+ *
+ * Generalized-semiring batched matrix multiply (log / max / sample / prod-max)
+ * and banded-matrix multiply for AMD MI355X (gfx950, CDNA4), as hand-written
+ * HIP kernels behind plain C entry points.
+ *
+ * This library replaces the private pybind11 module `_genbmm` of
+ * harvardnlp/genbmm (reference matmul_cuda.cpp:165-172) whose six functions
+ * `forward, backward, backbackward, forward_band, backward_band,
+ * backbackward_band` return freshly allocated torch tensors.  Here the entry
+ * points take raw device pointers instead:
+ *
+ *   - every pointer is a DEVICE pointer to a dense row-major fp32 (or int32)
+ *     buffer that the CALLER allocated; outputs are fully overwritten, they
+ *     need no initialisation;
+ *   - the library never allocates, frees or synchronises; every call only
+ *     enqueues kernels on `stream` (a hipStream_t passed as void*; NULL is the
+ *     legacy default stream);
+ *   - return value: 0 = enqueued; < 0 = argument error (GENBMM_E_*);
+ *     > 0 = the hipError_t reported by the launch;
+ *   - no global state; calls are re-entrant and thread safe.
+ *
+ * Dense operands: a is (B, M, K), b is (B, K, N), results are (B, M, N).
+ * Banded operands: band data is (B, n, W) with W = lu + ld + 1 and
+ * data[b, c, k] = Dense[b, c + k - lu, c]  (reference genbmm/sparse.py:12-30).
+ */
+#ifndef GENBMM_GFX950_H
+#define GENBMM_GFX950_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Argument errors (negative return values). */
+#define GENBMM_OK 0
+#define GENBMM_E_NULLPTR (-1) /* a required pointer is NULL            */
+#define GENBMM_E_SHAPE (-2)   /* a dimension is < 0 or overflows int32 */
+#define GENBMM_E_MODE (-3)    /* unknown semiring mode                 */
+#define GENBMM_E_BAND (-4)    /* negative band width                   */
+
+/* Banded semiring modes (reference banded_cuda_kernel.cu:42,64,76). */
+#define GENBMM_BAND_LOG 0
+#define GENBMM_BAND_MAX 1
+#define GENBMM_BAND_MUL 3
+
+/* Library version string, e.g. "genbmm-gfx950 0.1". */
+const char* genbmm_version(void);
+
+/* Human-readable text for a return value of any function below. */
+const char* genbmm_error_string(int code);
+
+/* ------------------------------------------------------------------ dense */
+
+/*
+ * out[b,m,n] = log sum_k exp(a[b,m,k] + b[b,k,n]).
+ * Replaces _genbmm.forward(a, b, 0): matmul_cuda.cpp:69-77 ->
+ * matmul_cuda_forward mode 0 (matmul_cuda_kernel.cu:465-497, kernel :13-45).
+ * The reference's second output `maxes` is not produced: the backward below
+ * does not need it.  The running maximum starts at -1e9 as in the reference
+ * (kernel :31), so an output whose terms are all <= -1e9 is -inf.
+ */
+int genbmm_logbmm_fwd(const float* a, const float* b, float* out,
+                      int B, int M, int K, int N, void* stream);
+
+/*
+ * grad_a[b,m,k] = sum_n exp(a[m,k] + b[k,n] - out[m,n]) * g[m,n]
+ * grad_b[b,k,n] = sum_m exp(a[m,k] + b[k,n] - out[m,n]) * g[m,n]
+ * Replaces the two _genbmm.backward(..., 0) calls plus six transposes of
+ * LogMatMul.backward (genmul.py:35-41; matmul_cuda.cpp:79-92;
+ * matmul_cuda_kernel.cu:625-664, kernel :159-184).
+ */
+int genbmm_logbmm_bwd(const float* a, const float* b, const float* out,
+                      const float* g, float* grad_a, float* grad_b,
+                      int B, int M, int K, int N, void* stream);
+
+/*
+ * Second-order terms of logbmm: the gradients with respect to (a, b, g) of
+ * <u_a, grad_a> + <u_b, grad_b> where (grad_a, grad_b) are the outputs of
+ * genbmm_logbmm_bwd.  u_a or u_b may be NULL (treated as zeros), not both.
+ * With u_b == NULL this is _genbmm.backbackward(a, b, g, out, maxes, u_a, 0):
+ * matmul_cuda.cpp:94-109, matmul_cuda_kernel.cu:547-622, kernels :220-331.
+ */
+int genbmm_logbmm_bwdbwd(const float* a, const float* b, const float* out,
+                         const float* g, const float* u_a, const float* u_b,
+                         float* grad_a, float* grad_b, float* grad_g,
+                         int B, int M, int K, int N, void* stream);
+
+/*
+ * out[b,m,n] = max_k (a[m,k] + b[k,n]); idx = the k attaining it.
+ * Ascending k, strict '>' against a running maximum that starts at -1e9
+ * with index -1: ties resolve to the lowest k.
+ * Replaces _genbmm.forward(a, b, 1): matmul_cuda_kernel.cu:498-511,
+ * kernel :47-75.
+ */
+int genbmm_maxbmm_fwd(const float* a, const float* b, float* out, int32_t* idx,
+                      int B, int M, int K, int N, void* stream);
+
+/*
+ * out[b,m,n] = max_k (a[m,k] * b[k,n]); idx as above.
+ * Replaces _genbmm.forward(a, b, 3): matmul_cuda_kernel.cu:527-541,
+ * kernel :124-152.
+ */
+int genbmm_prodmaxbmm_fwd(const float* a, const float* b, float* out,
+                          int32_t* idx, int B, int M, int K, int N,
+                          void* stream);
+
+/*
+ * out = log-sum-exp as genbmm_logbmm_fwd; idx[b,m,n] ~ Categorical(softmax_k
+ * (a[m,k] + b[k,n])) by inverse CDF in ascending k against one uniform per
+ * output cell.  The uniform of cell i = (b*M + m)*N + n is
+ * (x >> 8) * 2^-24 with x = word 0 of Philox4x32-10(counter = {lo32(i),
+ * hi32(i), lo32(offset), hi32(offset)}, key = {lo32(seed), hi32(seed)}).
+ * A cell whose scan never crosses its uniform keeps index 0, as in the
+ * reference.  Replaces _genbmm.forward(a, b, 2): matmul_cuda_kernel.cu:512-526
+ * (torch::rand at :517), kernel :77-121.
+ */
+int genbmm_samplebmm_fwd(const float* a, const float* b, float* out,
+                         int32_t* idx, uint64_t seed, uint64_t offset,
+                         int B, int M, int K, int N, void* stream);
+
+/*
+ * grad_a[b,m,k] = sum_n [k == idx[m,n]] * g[m,n]   (terms added in ascending n)
+ * grad_b[b,k,n] = sum_m [k == idx[m,n]] * g[m,n]   (terms added in ascending m)
+ * Backward of maxbmm and samplebmm.  Replaces _genbmm.backward(..., 1|2):
+ * matmul_cuda_kernel.cu:676-696, kernels :336-395 (which take the index as a
+ * float tensor, genmul.py:62-65).
+ */
+int genbmm_argmax_bwd(const int32_t* idx, const float* g,
+                      float* grad_a, float* grad_b,
+                      int B, int M, int K, int N, void* stream);
+
+/*
+ * grad_a[b,m,k] = sum_n [k == idx[m,n]] * b[k,n] * g[m,n]
+ * grad_b[b,k,n] = sum_m [k == idx[m,n]] * a[m,k] * g[m,n]
+ * Each term is rounded as a product and then added (no fused multiply-add),
+ * in ascending n (resp. m).  Replaces _genbmm.backward(..., 3):
+ * matmul_cuda_kernel.cu:697-718, kernels :399-456.
+ */
+int genbmm_prodmax_bwd(const float* a, const float* b, const int32_t* idx,
+                       const float* g, float* grad_a, float* grad_b,
+                       int B, int M, int K, int N, void* stream);
+
+/* ----------------------------------------------------------------- banded */
+
+/*
+ * Banded product of a (B, n, a_lu+a_ld+1) with b (B, n, b_lu+b_ld+1) in band
+ * storage; the result has lu = a_lu + b_ld, ld = a_ld + b_lu and shape
+ * (B, n, Wo), Wo = (a_lu+a_ld+1) + (b_lu+b_ld+1) - 1.  In dense terms the
+ * result is  Dense(b)^T (x) Dense(a)  in the chosen semiring.
+ *   out[i,j] = (+)_k a[i,k] (x) b[o,k2],  o = i + j - lu_out,
+ *              k2 = k - j + (b_lu + b_ld),  0 <= i+k-a_lu < n.
+ * mode GENBMM_BAND_LOG: log-sum-exp; GENBMM_BAND_MAX: max-plus, idx (B,n,Wo)
+ * receives the arg-max k (index into a's band; -1e9 floor, strict '>');
+ * GENBMM_BAND_MUL: ordinary (+,*).  Cells with o outside [0,n) are written
+ * as 0 (idx 0).  idx may be NULL unless mode is GENBMM_BAND_MAX.
+ * Replaces _genbmm.forward_band: matmul_cuda.cpp:112-124,
+ * banded_cuda_kernel.cu:354-402, kernel :13-100.
+ */
+int genbmm_banded_fwd(const float* a, int a_lu, int a_ld,
+                      const float* b, int b_lu, int b_ld,
+                      float* out, int32_t* idx,
+                      int B, int n, int mode, void* stream);
+
+/*
+ * Gradients of genbmm_banded_fwd with respect to BOTH operands, reading g,
+ * out and idx in the frame the forward wrote them (no banded transposes).
+ * `out` is read in mode LOG only, `idx` in mode MAX only (others may be NULL).
+ * grad_a terms are added in ascending j (result band index), grad_b terms in
+ * ascending i (row of a), which is the order of the reference's two calls.
+ * Replaces the two _genbmm.backward_band calls and the Python-side banded
+ * transposes of BandedMul / BandedLogMul / BandedMaxMul.backward
+ * (sparse.py:404-447, 466-545, 579-637; matmul_cuda.cpp:126-143;
+ * banded_cuda_kernel.cu:404-450, kernel :104-152).
+ */
+int genbmm_banded_bwd(const float* a, int a_lu, int a_ld,
+                      const float* b, int b_lu, int b_ld,
+                      const float* out, const int32_t* idx, const float* g,
+                      float* grad_a, float* grad_b,
+                      int B, int n, int mode, void* stream);
+
+/*
+ * Log-semiring second-order terms: gradients with respect to (a, b, g) of
+ * <u_a, grad_a> + <u_b, grad_b> for the outputs of genbmm_banded_bwd in mode
+ * LOG.  u_a or u_b may be NULL (zeros), not both.
+ * Replaces _genbmm.backbackward_band: matmul_cuda.cpp:145-161,
+ * banded_cuda_kernel.cu:453-546, kernels :154-350.
+ */
+int genbmm_banded_bwdbwd(const float* a, int a_lu, int a_ld,
+                         const float* b, int b_lu, int b_ld,
+                         const float* out, const float* g,
+                         const float* u_a, const float* u_b,
+                         float* grad_a, float* grad_b, float* grad_g,
+                         int B, int n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GENBMM_GFX950_H */
