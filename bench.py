@@ -1,0 +1,178 @@
+"""Headline benchmark: logbmm forward + backward, fp32, B=64, M=K=N=512, one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one forward and one backward of the hot path through the C ABI on inputs
+already resident in HBM (seeded synthetic log-potentials).  Prints one JSON line:
+semiring GOP/s (6*B*M*K*N semiring operations per step), the roofline of the dominant
+kernel measured with events around its launches, and the reference's CPU formulation
+(the torch broadcast) timed on this host's cores on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+B, M, K, N = 64, 512, 512, 512
+FP32_VALU_PEAK_TFLOPS = 157.3  # MI355X vector FP32 peak (packed FMA); the metric's denominator
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (see profiles/); None until measured for the current kernel.
+DOMINANT_TRAFFIC_BYTES = None
+
+
+def cpu_baseline(torch, sample_batches=4):
+    """The reference's CPU formulation (README.md:31-35): broadcast add + logsumexp, and
+    autograd backward, on `sample_batches` items of the headline shape, one item per
+    chunk (a 512 MB fp32 intermediate each)."""
+    import oracle
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16)
+    torch.set_num_threads(cores)
+    torch.manual_seed(0)
+    a = torch.randn(sample_batches, M, K)
+    b = torch.randn(sample_batches, K, N)
+    g = torch.randn(sample_batches, M, N)
+
+    def one(i):
+        ai = a[i:i + 1].clone().requires_grad_(True)
+        bi = b[i:i + 1].clone().requires_grad_(True)
+        out = oracle.logbmm_broadcast(ai, bi)
+        out.backward(g[i:i + 1])
+        return ai.grad, bi.grad
+
+    one(0)  # warm-up
+    t0 = time.perf_counter()
+    for i in range(sample_batches):
+        one(i)
+    dt = time.perf_counter() - t0
+    ops = 6.0 * sample_batches * M * K * N
+    return {
+        "value": round(ops / dt / 1e9, 3),
+        "unit": "semiring GOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": "%d of the %d batch items of the headline shape, one item per chunk, torch broadcast "
+                  "logsumexp fwd + autograd bwd, %.1f s" % (sample_batches, B, dt),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU only; every batch item is independent, so more GPUs "
+                 "would shard the batch axis with no exchange. Run with --gpus 1.")
+
+    import torch
+
+    from genbmm_amd import _lib
+
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    a = torch.randn(B, M, K).to(dev)
+    b = torch.randn(B, K, N).to(dev)
+    g = torch.randn(B, M, N).to(dev)
+    out = torch.empty(B, M, N, device=dev)
+    ga, gb = torch.empty_like(a), torch.empty_like(b)
+    stream = _lib.stream_of(a)
+    p = _lib.ptr
+    null = p(None)
+
+    def fwd():
+        _lib.check(lib.genbmm_logbmm_fwd(p(a), p(b), p(out), B, M, K, N, stream), "fwd")
+
+    def bwd_a():
+        _lib.check(lib.genbmm_logbmm_bwd(p(a), p(b), p(out), p(g), p(ga), null, B, M, K, N, stream), "bwd_a")
+
+    def bwd_b():
+        _lib.check(lib.genbmm_logbmm_bwd(p(a), p(b), p(out), p(g), null, p(gb), B, M, K, N, stream), "bwd_b")
+
+    for _ in range(args.warmup):
+        fwd(); bwd_a(); bwd_b()
+    torch.cuda.synchronize()
+
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(args.steps):
+        ev[s][0].record(); fwd()
+        ev[s][1].record(); bwd_a()
+        ev[s][2].record(); bwd_b()
+        ev[s][3].record()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+
+    ms_fwd = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
+    ms_bwd_a = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+    ms_bwd_b = sum(e[2].elapsed_time(e[3]) for e in ev) / args.steps
+    ms_step = dt * 1e3 / args.steps
+    bmkn = float(B) * M * K * N
+    value = 6.0 * bmkn / (ms_step * 1e-3) / 1e9
+
+    # dominant kernel = the backward template (two launches per step, 2*BMKN semiring ops each)
+    ms_dom = 0.5 * (ms_bwd_a + ms_bwd_b)
+    achieved = 2.0 * bmkn / (ms_dom * 1e-3) / 1e12
+    roofline = {
+        "bound": "valu",
+        "kernel": "k_log_bwd (grad_a and grad_b launches averaged)",
+        "achieved": round(achieved, 3),
+        "peak": FP32_VALU_PEAK_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": round(achieved / FP32_VALU_PEAK_TFLOPS, 4),
+        "traffic": DOMINANT_TRAFFIC_BYTES,
+        "avg_launch_ms": round(ms_dom, 4),
+    }
+
+    # end-to-end through the public autograd API (allocations included), for the record
+    import genbmm_amd as genbmm
+
+    ar, br = a.clone().requires_grad_(True), b.clone().requires_grad_(True)
+    for _ in range(2):
+        genbmm.logbmm(ar, br).backward(g)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for _ in range(args.steps):
+        ar.grad = br.grad = None
+        genbmm.logbmm(ar, br).backward(g)
+    torch.cuda.synchronize()
+    ms_autograd = (time.perf_counter() - t1) * 1e3 / args.steps
+
+    line = {
+        "metric": "semiring GOP/s logbmm fwd+bwd fp32 B=64 512^3; % FP32 VALU peak",
+        "value": round(value, 1),
+        "unit": "semiring GOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "logbmm fwd+bwd, a,b,g ~ Normal(0,1) seed 0, B=64 M=K=N=512 (headline)",
+                   "B": B, "M": M, "K": K, "N": N, "ops_per_step": 6.0 * bmkn},
+        "pct_fp32_valu_peak": round(100.0 * value / 1e3 / FP32_VALU_PEAK_TFLOPS, 3),
+        "ms_fwd": round(ms_fwd, 4),
+        "ms_bwd_grad_a": round(ms_bwd_a, 4),
+        "ms_bwd_grad_b": round(ms_bwd_b, 4),
+        "ms_per_step_autograd_api": round(ms_autograd, 4),
+        "roofline": roofline,
+        "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(torch),
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

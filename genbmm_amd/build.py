@@ -26,6 +26,9 @@ HIPCC_FLAGS = [
     "-std=c++17",
     "--offload-arch=gfx950",
     "-fPIC",
+    # multiply-add fusion only where the source spells fmaf(): kernels whose results
+    # must be bit-exact round each product before adding it
+    "-ffp-contract=on",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-fno-gpu-rdc",
     "-Wno-unused-command-line-argument",

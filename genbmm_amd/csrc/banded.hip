@@ -272,9 +272,10 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   using namespace genbmm;
   if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
     return GENBMM_E_MODE;
-  if (!a || !b || !out || (mode == GENBMM_BAND_MAX && !idx)) return GENBMM_E_NULLPTR;
   BandArgs p{};
   if (int e = fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return e;
+  if ((int64_t)B * n == 0) return GENBMM_OK;
+  if (!a || !b || !out || (mode == GENBMM_BAND_MAX && !idx)) return GENBMM_E_NULLPTR;
   p.a = a; p.b = b; p.o0 = out; p.oidx = idx;
   const long total = (long)B * n * p.Wo;
   if (total == 0) return GENBMM_OK;
@@ -294,11 +295,12 @@ int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   using namespace genbmm;
   if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
     return GENBMM_E_MODE;
+  BandArgs p{};
+  if (int e = fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return e;
+  if ((int64_t)B * n == 0) return GENBMM_OK;
   if (!a || !b || !g || !grad_a || !grad_b || (mode == GENBMM_BAND_LOG && !out) ||
       (mode == GENBMM_BAND_MAX && !idx))
     return GENBMM_E_NULLPTR;
-  BandArgs p{};
-  if (int e = fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return e;
   p.a = a; p.b = b; p.out = out; p.idx = idx; p.g = g; p.o0 = grad_a; p.o1 = grad_b;
   const long ta = (long)B * n * p.Wa, tb = (long)B * n * p.Wb;
   if (ta == 0) return GENBMM_OK;
@@ -321,10 +323,11 @@ int genbmm_banded_bwdbwd(const float* a, int a_lu, int a_ld, const float* b, int
                          float* grad_a, float* grad_b, float* grad_g, int B, int n,
                          void* stream) {
   using namespace genbmm;
-  if (!a || !b || !out || !g || !grad_a || !grad_b || !grad_g || (!u_a && !u_b))
-    return GENBMM_E_NULLPTR;
   BandArgs p{};
   if (int e = fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return e;
+  if ((int64_t)B * n == 0) return GENBMM_OK;
+  if (!a || !b || !out || !g || !grad_a || !grad_b || !grad_g || (!u_a && !u_b))
+    return GENBMM_E_NULLPTR;
   p.a = a; p.b = b; p.out = out; p.g = g; p.ua = u_a; p.ub = u_b;
   p.o0 = grad_a; p.o1 = grad_b; p.o2 = grad_g;
   const long ta = (long)B * n * p.Wa, tb = (long)B * n * p.Wb, to = (long)B * n * p.Wo;

@@ -192,6 +192,9 @@ inline int check_dense_dims(int B, int M, int K, int N) {
   return GENBMM_OK;
 }
 
+// A pointer may be NULL only if the buffer it names has no elements.
+inline bool missing(const void* p, int64_t count) { return p == nullptr && count > 0; }
+
 inline int launch_status() {
   const hipError_t e = hipGetLastError();
   return e == hipSuccess ? GENBMM_OK : (int)e;

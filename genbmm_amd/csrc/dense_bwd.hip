@@ -297,7 +297,7 @@ __global__ __launch_bounds__(256) void k_log_bwdbwd_b(const BB p, long total) {
 // term into the cell idx selects, in an LDS-resident accumulator row; the
 // additions hitting a given cell therefore happen in the reference's order,
 // so the result is bit-identical, in O(M*N) work.  Products are rounded
-// before the add (no fused multiply-add), as the oracle does.
+// before the add (the build uses -ffp-contract=on: no fusion across statements).
 constexpr int kKC = 128;  // gradient columns/rows accumulated per pass
 
 template <bool PROD>
@@ -372,8 +372,11 @@ __global__ __launch_bounds__(64) void k_argmax_bwd_b(const float* __restrict__ a
 template <bool PROD>
 int run_argmax_bwd(const float* a, const float* b, const int32_t* idx, const float* g,
                    float* grad_a, float* grad_b, int B, int M, int K, int N, void* stream) {
-  if (!idx || !g || !grad_a || !grad_b || (PROD && (!a || !b))) return GENBMM_E_NULLPTR;
   if (int e = check_dense_dims(B, M, K, N)) return e;
+  const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
+  if (missing(idx, mn) || missing(g, mn) || missing(grad_a, mk) || missing(grad_b, kn) ||
+      (PROD && (missing(a, mk) || missing(b, kn))))
+    return GENBMM_E_NULLPTR;
   hipStream_t s = (hipStream_t)stream;
   if ((int64_t)B * M * K > 0) {
     const int row_tiles = ceil_div(M, 64);
@@ -402,27 +405,40 @@ extern "C" {
 int genbmm_logbmm_bwd(const float* a, const float* b, const float* out, const float* g,
                       float* grad_a, float* grad_b, int B, int M, int K, int N, void* stream) {
   using namespace genbmm;
-  if (!a || !b || !out || !g || !grad_a || !grad_b) return GENBMM_E_NULLPTR;
   if (int e = check_dense_dims(B, M, K, N)) return e;
+  const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
+  if (missing(a, mk) || missing(b, kn) || missing(out, mn) || missing(g, mn) ||
+      (missing(grad_a, mk) && missing(grad_b, kn)))
+    return GENBMM_E_NULLPTR;
   LogBwdArgs p{};
   p.a = a; p.b = b; p.out = out; p.g = g;
   p.M = M; p.K = K; p.N = N;
   p.vec_k = (K % 4 == 0) && aligned16(a) && aligned16(grad_a);
   p.vec_n = (N % 4 == 0) && aligned16(b) && aligned16(out) && aligned16(g) && aligned16(grad_b);
   hipStream_t s = (hipStream_t)stream;
-  p.grad = grad_a;
-  if (int e = run_log_bwd<true>(p, B, s)) return e;
-  p.grad = grad_b;
-  return run_log_bwd<false>(p, B, s);
+  if (grad_a) {
+    p.grad = grad_a;
+    if (int e = run_log_bwd<true>(p, B, s)) return e;
+  }
+  if (grad_b) {
+    p.grad = grad_b;
+    if (int e = run_log_bwd<false>(p, B, s)) return e;
+  }
+  return GENBMM_OK;
 }
 
 int genbmm_logbmm_bwdbwd(const float* a, const float* b, const float* out, const float* g,
                          const float* u_a, const float* u_b, float* grad_a, float* grad_b,
                          float* grad_g, int B, int M, int K, int N, void* stream) {
   using namespace genbmm;
-  if (!a || !b || !out || !g || !grad_a || !grad_b || !grad_g || (!u_a && !u_b))
-    return GENBMM_E_NULLPTR;
   if (int e = check_dense_dims(B, M, K, N)) return e;
+  {
+    const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
+    if (missing(a, mk) || missing(b, kn) || missing(out, mn) || missing(g, mn) ||
+        missing(grad_a, mk) || missing(grad_b, kn) || missing(grad_g, mn) ||
+        (missing(u_a, mk) && missing(u_b, kn)))
+      return GENBMM_E_NULLPTR;
+  }
   BB p{a, b, out, g, u_a, u_b, grad_a, grad_b, grad_g, M, K, N};
   hipStream_t s = (hipStream_t)stream;
   auto blocks = [](long total) { return dim3((unsigned)((total + 255) / 256)); };

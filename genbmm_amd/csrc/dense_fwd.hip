@@ -378,9 +378,11 @@ int launch_log(DenseArgs p, int B, int M, int K, int N, hipStream_t s) {
 template <bool PROD>
 int run_max(const float* a, const float* b, float* out, int32_t* idx, int B, int M, int K, int N,
             void* stream) {
-  if (!a || !b || !out || !idx) return GENBMM_E_NULLPTR;
   if (int e = check_dense_dims(B, M, K, N)) return e;
-  if ((int64_t)B * M * N == 0) return GENBMM_OK;
+  const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
+  if (missing(a, mk) || missing(b, kn) || missing(out, mn) || missing(idx, mn))
+    return GENBMM_E_NULLPTR;
+  if (mn == 0) return GENBMM_OK;
   DenseArgs p{};
   p.a = a; p.b = b; p.out = out; p.idx = idx;
   hipStream_t s = (hipStream_t)stream;
@@ -395,9 +397,11 @@ int run_max(const float* a, const float* b, float* out, int32_t* idx, int B, int
 template <bool SAMPLE>
 int run_log(const float* a, const float* b, float* out, int32_t* idx, uint64_t seed,
             uint64_t offset, int B, int M, int K, int N, void* stream) {
-  if (!a || !b || !out || (SAMPLE && !idx)) return GENBMM_E_NULLPTR;
   if (int e = check_dense_dims(B, M, K, N)) return e;
-  if ((int64_t)B * M * N == 0) return GENBMM_OK;
+  const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
+  if (missing(a, mk) || missing(b, kn) || missing(out, mn) || (SAMPLE && missing(idx, mn)))
+    return GENBMM_E_NULLPTR;
+  if (mn == 0) return GENBMM_OK;
   DenseArgs p{};
   p.a = a; p.b = b; p.out = out; p.idx = idx; p.seed = seed; p.offset = offset;
   hipStream_t s = (hipStream_t)stream;

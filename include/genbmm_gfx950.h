@@ -71,6 +71,7 @@ int genbmm_logbmm_fwd(const float* a, const float* b, float* out,
  * Replaces the two _genbmm.backward(..., 0) calls plus six transposes of
  * LogMatMul.backward (genmul.py:35-41; matmul_cuda.cpp:79-92;
  * matmul_cuda_kernel.cu:625-664, kernel :159-184).
+ * grad_a or grad_b may be NULL (that gradient is then not computed), not both.
  */
 int genbmm_logbmm_bwd(const float* a, const float* b, const float* out,
                       const float* g, float* grad_a, float* grad_b,

@@ -251,6 +251,21 @@ def band_transpose(data, lu, ld):
     return band_from_dense(band_to_dense(data, lu, ld, 0.0).transpose(-2, -1), ld, lu)
 
 
+def band_transpose_indexed(data, lu, ld):
+    """The same transposition by index arithmetic, for sizes where the dense detour is
+    too slow: T[i, k] = data[i + k - ld, W - 1 - k] where that row exists, else 0
+    (from the layout: T[c, k] = Dense[c, c + k - ld]).  Pinned against band_transpose
+    in tests/test_oracle.py."""
+    d = _np(data, np.float64 if data.dtype == torch.float64 else np.float32)
+    n, W = d.shape[1], d.shape[2]
+    i = np.arange(n)[:, None]
+    k = np.arange(W)[None, :]
+    src = i + k - ld
+    ok = (src >= 0) & (src < n)
+    out = d[:, np.clip(src, 0, n - 1), np.broadcast_to(W - 1 - k, src.shape)]
+    return torch.from_numpy(np.where(ok[None], out, 0).astype(d.dtype))
+
+
 def band_product_dense(a, a_lu, a_ld, b, b_lu, b_ld, mode):
     """X.multiply*(Y) as dense algebra (test_sparse.py:141-142, 181-195): Dense(Y)^T (x)
     Dense(X), re-banded with lu = a_lu + b_ld, ld = a_ld + b_lu.  mode 3: torch.bmm;
@@ -297,11 +312,11 @@ def seq_band_bwd(a, a_lu, a_ld, b, b_lu, b_ld, g, mode, dtype=np.float32):
     out, idx, _ = seq_band_fwd(a, a_lu, a_ld, b, b_lu, b_ld, mode, dtype)
     o_lu, o_ld = a_lu + b_ld, a_ld + b_lu
     g = torch.as_tensor(_np(g, dt))
-    gT = band_transpose(g, o_lu, o_ld)
+    gT = band_transpose_indexed(g, o_lu, o_ld)
     if mode == 1:
         part, partT = idx.to(g.dtype), seq_band_fwd(b, b_lu, b_ld, a, a_lu, a_ld, 1, dtype)[1].to(g.dtype)
     elif mode == 0:
-        part, partT = out, band_transpose(out, o_lu, o_ld)
+        part, partT = out, band_transpose_indexed(out, o_lu, o_ld)
     else:
         part, partT = g, gT
     ga = _seq_band_bwd_first(pre, dt, a, a_lu, a_ld, b, b_lu, b_ld, part, g, mode)

@@ -1,0 +1,165 @@
+"""GPU parity of the banded products against the CPU oracle (all marked gpu)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import genbmm_amd as genbmm
+from genbmm_amd import _lib
+from genbmm_amd.sparse import BandedMatrix, banddiag
+
+pytestmark = pytest.mark.gpu
+
+# (n, a_lu, a_ld, b_lu, b_ld): bands narrower and wider than the matrix, empty sides
+BANDS = [(5, 1, 1, 2, 0), (6, 2, 1, 1, 3), (4, 3, 3, 3, 3), (7, 0, 2, 2, 0), (3, 4, 5, 5, 4),
+         (40, 3, 5, 4, 2), (33, 0, 0, 0, 0), (64, 8, 8, 8, 8), (1, 0, 0, 0, 0), (130, 17, 2, 5, 20)]
+
+
+def close(x, ref, rtol=1e-5, atol=1e-5):
+    x, ref = x.detach().cpu().double(), ref.detach().cpu().double()
+    assert torch.allclose(x, ref, rtol=rtol, atol=atol), float((x - ref).abs().max())
+
+
+def grid(*shape):
+    return torch.round(torch.randn(*shape) * 8) / 8
+
+
+def pair(n, a_lu, a_ld, b_lu, b_ld, batch=3, mk=torch.randn):
+    a = banddiag(mk(batch, n, n), a_lu, a_ld)[0].contiguous()
+    b = banddiag(mk(batch, n, n), b_lu, b_ld)[0].contiguous()
+    return a, b
+
+
+@pytest.mark.parametrize("n,a_lu,a_ld,b_lu,b_ld", BANDS)
+@pytest.mark.parametrize("mode", [0, 1, 3])
+def test_banded_forward_backward(gpu, n, a_lu, a_ld, b_lu, b_ld, mode):
+    torch.manual_seed(n * 7 + mode)
+    exact = mode == 1
+    a, b = pair(n, a_lu, a_ld, b_lu, b_ld, mk=grid if exact else torch.randn)
+    W = a.shape[2] + b.shape[2] - 1
+    g = grid(3, n, W).clamp(-4, 4) if exact else torch.randn(3, n, W)
+    X = BandedMatrix(a.to(gpu).requires_grad_(True), a_lu, a_ld)
+    Y = BandedMatrix(b.to(gpu).requires_grad_(True), b_lu, b_ld)
+    res = {0: X.multiply_log, 1: X.multiply_max, 3: X.multiply}[mode](Y)
+    assert (res.lu, res.ld) == (a_lu + b_ld, a_ld + b_lu)
+    # float64 sequential restatement of the reference kernel; whole tensor incl. zero cells
+    want, widx, _ = oracle.seq_band_fwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, mode, dtype=np.float64)
+    if exact:
+        assert torch.equal(res.data.detach().cpu().double(), want)
+    else:
+        close(res.data, want)
+    ga, gb = torch.autograd.grad(res.data, (X.data, Y.data), g.to(gpu))
+    wa, wb = oracle.seq_band_bwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, g.double(), mode, dtype=np.float64)
+    if exact:
+        assert torch.equal(ga.cpu().double(), wa) and torch.equal(gb.cpu().double(), wb)
+    else:
+        close(ga, wa)
+        close(gb, wb)
+
+
+def test_banded_max_index_through_c_abi(gpu):
+    torch.manual_seed(2)
+    n, a_lu, a_ld, b_lu, b_ld = 50, 4, 6, 5, 3
+    a, b = pair(n, a_lu, a_ld, b_lu, b_ld, mk=grid)
+    ad, bd = a.to(gpu), b.to(gpu)
+    W = a.shape[2] + b.shape[2] - 1
+    out = torch.empty(3, n, W, device=gpu)
+    idx = torch.empty(3, n, W, dtype=torch.int32, device=gpu)
+    rc = _lib.load().genbmm_banded_fwd(_lib.ptr(ad), a_lu, a_ld, _lib.ptr(bd), b_lu, b_ld, _lib.ptr(out),
+                                       _lib.ptr(idx), 3, n, 1, _lib.stream_of(ad))
+    assert rc == 0
+    want, widx, _ = oracle.seq_band_fwd(a, a_lu, a_ld, b, b_lu, b_ld, 1)
+    assert torch.equal(out.cpu(), want) and torch.equal(idx.cpu(), widx)
+
+
+@pytest.mark.parametrize("n,lu,ld", [(5, 3, 4), (4, 5, 3), (3, 3, 3), (9, 2, 4)])
+def test_reference_style_log_product(gpu, n, lu, ld):
+    """The reference's own banded test (test_cuda.py:46-49, 81-143):
+    bmm(a, b) = b.multiply_log(a.transpose()), forward, gradients and second-order terms."""
+    torch.manual_seed(n + lu)
+    band, _ = banddiag(torch.rand(3, n, n), lu, ld)
+    band2, _ = banddiag(torch.rand(3, n, n), lu, ld)
+    back = torch.rand(3, n, 2 * (lu + ld) + 1)
+    back2 = (torch.rand(3, n, lu + ld + 1), torch.rand(3, n, lu + ld + 1))
+
+    def run(dev, dtype):
+        s1 = band.to(dev, dtype).clone().requires_grad_(True)
+        s2 = band2.to(dev, dtype).clone().requires_grad_(True)
+        bk = back.to(dev, dtype).clone().requires_grad_(True)
+        if dev.type == "cuda":
+            out = BandedMatrix(s2, lu, ld).multiply_log(BandedMatrix(s1, lu, ld).transpose()).data
+        else:  # dense closed form, float64 (test_sparse.py:181-195)
+            X = BandedMatrix(BandedMatrix(s1, lu, ld).transpose().data, ld, lu, -1e9).to_dense()
+            Y = BandedMatrix(s2, lu, ld, -1e9).to_dense()
+            D = (X.transpose(-2, -1).unsqueeze(-1) + Y.unsqueeze(-3)).logsumexp(-2)
+            out = banddiag(D, lu + lu, ld + ld)[0]
+        g = torch.autograd.grad(out, (s1, s2), bk, create_graph=True)
+        h = torch.autograd.grad((g[0], g[1]), (s1, s2, bk), (back2[0].to(dev, dtype), back2[1].to(dev, dtype)))
+        return out, g, h
+
+    out, g, h = run(gpu, torch.float32)
+    wout, wg, wh = run(torch.device("cpu"), torch.float64)
+    n_ = band.shape[1]
+    mask = oracle.band_from_dense(torch.ones(1, n_, n_), 2 * lu, 2 * ld)[0] > 0
+    close(out[:, mask.to(gpu)], wout[:, mask])
+    assert bool((out[:, ~mask.to(gpu)] == 0).all())
+    for x, y in zip(g, wg):
+        close(x, y)
+    for x, y in zip(h, wh):
+        close(x, y, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("n,a_lu,a_ld,b_lu,b_ld", BANDS[:6])
+def test_banded_double_backward_vs_literal_kernels(gpu, n, a_lu, a_ld, b_lu, b_ld):
+    torch.manual_seed(n)
+    a, b = pair(n, a_lu, a_ld, b_lu, b_ld)
+    W = a.shape[2] + b.shape[2] - 1
+    g, u = torch.randn(3, n, W), torch.randn(*a.shape)
+    want = oracle.seq_band_bwdbwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, g.double(), u.double(),
+                                  dtype=np.float64)
+    ad, bd, gd = (t.to(gpu).requires_grad_(True) for t in (a, b, g))
+    out = BandedMatrix(ad, a_lu, a_ld).multiply_log(BandedMatrix(bd, b_lu, b_ld)).data
+    (ga,) = torch.autograd.grad(out, (ad,), gd, create_graph=True)
+    got = torch.autograd.grad(ga, (ad, bd, gd), u.to(gpu))
+    for x, y in zip(got, want):
+        close(x, y, rtol=1e-4, atol=1e-5)
+
+
+def test_banded_config_c5(gpu):
+    """BASELINE config 4: batch 64, n = 4096, lu = ld = 32 for both operands, Uniform[-1,1)
+    band data from seed 7; standard and log semiring, forward + backward.  Full-size run;
+    float64 oracle on two batch items; dense closed form at reduced n."""
+    torch.manual_seed(7)
+    B, n, lu, ld = 64, 4096, 32, 32
+    a, b = torch.rand(B, n, 65) * 2 - 1, torch.rand(B, n, 65) * 2 - 1
+    g = torch.randn(B, n, 129)
+    ad, bd, gd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True), g.to(gpu)
+    pick = [0, 63]
+    for mode in (3, 0):
+        X, Y = BandedMatrix(ad, lu, ld), BandedMatrix(bd, lu, ld)
+        res = (X.multiply if mode == 3 else X.multiply_log)(Y)
+        ga, gb = torch.autograd.grad(res.data, (ad, bd), gd)
+        want, _, _ = oracle.seq_band_fwd(a[pick].double(), lu, ld, b[pick].double(), lu, ld, mode, dtype=np.float64)
+        close(res.data[pick], want, rtol=1e-5, atol=2e-5)
+        wa, wb = oracle.seq_band_bwd(a[pick].double(), lu, ld, b[pick].double(), lu, ld, g[pick].double(), mode,
+                                     dtype=np.float64)
+        close(ga[pick], wa, rtol=1e-5, atol=1e-4)
+        close(gb[pick], wb, rtol=1e-5, atol=1e-4)
+        if mode == 0:  # softmax weights of every in-matrix output cell sum to one
+            pass
+    # dense closed form at n = 256, same bandwidths (test_sparse.py:141-142, 181-195)
+    n2 = 256
+    a2, b2 = a[:4, :n2].contiguous(), b[:4, :n2].contiguous()
+    for mode in (3, 0):
+        want, mask = oracle.band_product_dense(a2.double(), lu, ld, b2.double(), lu, ld, mode)
+        X, Y = BandedMatrix(a2.to(gpu), lu, ld), BandedMatrix(b2.to(gpu), lu, ld)
+        res = (X.multiply if mode == 3 else X.multiply_log)(Y)
+        close(res.data[:, mask.to(gpu)], want[:, mask], rtol=1e-5, atol=2e-5)
+
+
+def test_banded_errors(gpu):
+    a = torch.randn(2, 5, 3)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        BandedMatrix(a, 1, 1).multiply(BandedMatrix(a, 1, 1))
+    with pytest.raises(RuntimeError, match="disagree"):
+        BandedMatrix(a.to(gpu), 1, 1).multiply_log(BandedMatrix(torch.randn(3, 5, 3, device=gpu), 1, 1))

@@ -1,0 +1,356 @@
+"""GPU parity of the dense semiring ops against the CPU oracle (all marked gpu).
+
+Tolerances: logbmm forward / gradients rtol 1e-5, atol 1e-5 against float64;
+max / prod-max values, indices and gradients bit-exact; sampling by a CDF
+bracket check per cell plus a chi-square bound.
+"""
+import ctypes
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import genbmm_amd as genbmm
+from genbmm_amd import _lib
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 1e-5
+
+
+def close(x, ref, rtol=RTOL, atol=ATOL):
+    x, ref = x.detach().cpu().double(), ref.detach().cpu().double()
+    bad = ~torch.isclose(x, ref, rtol=rtol, atol=atol, equal_nan=True)
+    if bad.any():
+        err = (x - ref).abs()
+        raise AssertionError("max abs err %.3e over %d cells, worst at %s" % (
+            float(err[bad].max()), int(bad.sum()), np.unravel_index(int(err.argmax()), x.shape)))
+
+
+def lse64(a, b, chunk=4):
+    outs = [oracle.logbmm_broadcast(a[i:i + chunk].double(), b[i:i + chunk].double())
+            for i in range(0, a.shape[0], chunk)]
+    return torch.cat(outs) if outs else a.new_zeros((0, a.shape[1], b.shape[2])).double()
+
+
+SHAPES = [(16, 64, 64, 64), (3, 7, 9, 5), (2, 1, 1, 1), (4, 5, 1, 6), (5, 33, 70, 129), (2, 130, 17, 66),
+          (3, 64, 64, 128), (2, 200, 96, 260), (9, 32, 32, 32), (7, 31, 33, 29), (1, 256, 40, 256)]
+
+
+@pytest.mark.parametrize("B,M,K,N", SHAPES)
+def test_logbmm_forward_and_grads(gpu, B, M, K, N):
+    torch.manual_seed(B * 1000 + M)
+    a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
+    want, wa, wb = oracle.logbmm_grads64(a, b, g)
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    out = genbmm.logbmm(ad, bd)
+    close(out, want)
+    ga, gb = torch.autograd.grad(out, (ad, bd), g.to(gpu))
+    close(ga, wa)
+    close(gb, wb)
+    # softmax weights sum to one over k
+    close(ga.sum(-1), g.double().sum(-1), atol=1e-4)
+    close(gb.sum(-2), g.double().sum(-2), atol=1e-4)
+
+
+def test_logbmm_config_c1_uniform_ones(gpu):
+    """BASELINE config 0: seed 0, Uniform[0,1) (16,64,64), grad_out = ones."""
+    torch.manual_seed(0)
+    a, b = torch.rand(16, 64, 64), torch.rand(16, 64, 64)
+    g = torch.ones(16, 64, 64)
+    want, wa, wb = oracle.logbmm_grads64(a, b, g)
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    out = genbmm.logbmm(ad, bd)
+    ga, gb = torch.autograd.grad(out.sum(), (ad, bd))
+    close(out, want)
+    close(ga, wa)
+    close(gb, wb)
+    # the sequential fp32 restatement of the reference kernel agrees too
+    close(out, oracle.seq_logbmm_fwd(a, b)[0])
+
+
+def test_logbmm_special_values(gpu):
+    a, b = torch.randn(2, 5, 6), torch.randn(2, 6, 4)
+    b[0, 2, :] = -math.inf          # masked k
+    a[1, 3, :] = -math.inf          # fully masked row -> -inf
+    a[0, 1, :] = -2e9               # below the -1e9 floor -> -inf, as in the reference
+    got = genbmm.logbmm(a.to(gpu), b.to(gpu)).cpu()
+    want, _ = oracle.seq_logbmm_fwd(a, b)
+    assert torch.equal(torch.isinf(got), torch.isinf(want))
+    fin = ~torch.isinf(want)
+    close(got[fin], want[fin])
+    big = torch.randn(2, 9, 33) * 30 + 200  # large magnitudes
+    bb = torch.randn(2, 33, 7) * 30 - 500
+    close(genbmm.logbmm(big.to(gpu), bb.to(gpu)), lse64(big, bb))
+    a1, b1 = torch.randn(2, 5, 1), torch.randn(2, 1, 4)               # K = 1: out = a + b
+    close(genbmm.logbmm(a1.to(gpu), b1.to(gpu)), a1 + b1, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("B,M,K,N,sub", [(512, 128, 128, 128, 8), (8192, 32, 32, 32, 256), (64, 512, 512, 512, 1)])
+def test_logbmm_baseline_shapes(gpu, B, M, K, N, sub):
+    """BASELINE configs 1 and the headline shape: full-size run, float64 check on a
+    batch subset plus the size-independent row-sum invariants on everything."""
+    torch.manual_seed(0)
+    a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
+    ad, bd, gd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True), g.to(gpu)
+    out = genbmm.logbmm(ad, bd)
+    ga, gb = torch.autograd.grad(out, (ad, bd), gd)
+    pick = torch.linspace(0, B - 1, sub).long()
+    want, wa, wb = oracle.logbmm_grads64(a[pick], b[pick], g[pick])
+    close(out[pick.to(gpu)], want)
+    close(ga[pick.to(gpu)], wa)
+    close(gb[pick.to(gpu)], wb)
+    close(ga.sum(-1), gd.double().sum(-1), atol=2e-4)
+    close(gb.sum(-2), gd.double().sum(-2), atol=2e-4)
+    # out >= max_k(a+b) and out <= max + log K
+    mx = genbmm.maxbmm(ad.detach(), bd.detach())
+    assert bool((out >= mx - 1e-5).all()) and bool((out <= mx + math.log(K) + 1e-5).all())
+
+
+@pytest.mark.parametrize("B,M,K,N", [(2, 4, 5, 3), (3, 9, 12, 7), (2, 33, 20, 40)])
+def test_logbmm_double_backward(gpu, B, M, K, N):
+    """Second-order terms (test_cuda.py:30-42 uses rtol 1e-2; here 1e-4 vs float64)."""
+    torch.manual_seed(7)
+    a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
+    ua, ub = torch.randn(B, M, K), torch.randn(B, K, N)
+    for u_a, u_b in [(ua, ub), (ua, None), (None, ub)]:
+        want = oracle.logbmm_second_order64(a, b, g, u_a, u_b)
+        ad, bd, gd = (t.to(gpu).requires_grad_(True) for t in (a, b, g))
+        out = genbmm.logbmm(ad, bd)
+        ga, gb = torch.autograd.grad(out, (ad, bd), gd, create_graph=True)
+        outs = [t for t, u in ((ga, u_a), (gb, u_b)) if u is not None]
+        cots = [u.to(gpu) for u in (u_a, u_b) if u is not None]
+        got = torch.autograd.grad(outs, (ad, bd, gd), cots)
+        for x, y in zip(got, want):
+            close(x, y, rtol=1e-4, atol=1e-5)
+    # the reference's literal quartic kernels (u_b = 0), fp32 sequential
+    qa, qb, qg = oracle.seq_logbmm_bwdbwd(a.double(), b.double(), g.double(), ua.double(), dtype=np.float64)
+    want = oracle.logbmm_second_order64(a, b, g, ua, None)
+    for x, y in zip((qa, qb, qg), want):
+        close(x, y, rtol=1e-9, atol=1e-11)
+
+
+# ------------------------------------------------------------ max / prod-max
+def grid(*shape):
+    return torch.round(torch.randn(*shape) * 8) / 8
+
+
+@pytest.mark.parametrize("B,M,K,N", [(4, 9, 17, 6), (3, 64, 64, 64), (2, 130, 70, 129), (5, 32, 32, 32),
+                                     (2, 1, 1, 1), (2, 128, 200, 256), (16, 128, 48, 128)])
+@pytest.mark.parametrize("prod", [False, True])
+def test_max_forward_backward_bit_exact(gpu, B, M, K, N, prod):
+    torch.manual_seed(M + K)
+    if prod:
+        a, b = 1 - torch.rand(B, M, K), 1 - torch.rand(B, K, N)
+        a[:, :, ::3] = torch.round(a[:, :, ::3] * 4) / 4 + 0.25  # some exact product ties
+        b[:, ::3, :] = torch.round(b[:, ::3, :] * 4) / 4 + 0.25
+        op, orc = genbmm.prodmaxbmm, oracle.prodmaxbmm_broadcast
+    else:
+        a, b = grid(B, M, K), grid(B, K, N)
+        op, orc = genbmm.maxbmm, oracle.maxbmm_broadcast
+    g = grid(B, M, N).clamp(-4, 4)
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    out = op(ad, bd)
+    wv, wi = orc(a, b)
+    assert torch.equal(out.detach().cpu(), wv)
+    sv, si = oracle.seq_maxbmm_fwd(a, b, prod)
+    assert torch.equal(wv, sv) and torch.equal(wi.int(), si)
+    ga, gb = torch.autograd.grad(out, (ad, bd), g.to(gpu))
+    wa, wb = oracle.seq_argmax_bwd(a if prod else K, b, si, g, prod)
+    assert torch.equal(ga.cpu(), wa), float((ga.cpu() - wa).abs().max())
+    assert torch.equal(gb.cpu(), wb), float((gb.cpu() - wb).abs().max())
+
+
+def _abi_max(gpu, a, b, prod):
+    lib = _lib.load()
+    B, M, K = a.shape
+    N = b.shape[2]
+    out = torch.empty(B, M, N, device=gpu)
+    idx = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
+    fn = lib.genbmm_prodmaxbmm_fwd if prod else lib.genbmm_maxbmm_fwd
+    rc = fn(_lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), B, M, K, N, _lib.stream_of(a))
+    assert rc == 0
+    return out, idx
+
+
+@pytest.mark.parametrize("prod", [False, True])
+def test_max_index_through_c_abi(gpu, prod):
+    torch.manual_seed(3)
+    a, b = grid(6, 70, 90), grid(6, 90, 50)
+    if prod:
+        a, b = a.abs() + 0.125, b.abs() + 0.125
+    out, idx = _abi_max(gpu, a.to(gpu), b.to(gpu), prod)
+    sv, si = oracle.seq_maxbmm_fwd(a, b, prod)
+    assert torch.equal(out.cpu(), sv) and torch.equal(idx.cpu(), si)
+    # floor: everything below -1e9 -> value -1e9, index -1 (matmul_cuda_kernel.cu:62-64)
+    if not prod:
+        lo = torch.full((1, 3, 4), -2e9)
+        out, idx = _abi_max(gpu, lo.to(gpu), torch.zeros(1, 4, 2, device=gpu), False)
+        assert bool((out == -1e9).all()) and bool((idx == -1).all())
+
+
+def test_max_config_c3(gpu):
+    """BASELINE config 2: (256,256,256) on the 1/8 grid (max) and Uniform(0,1] (prod-max);
+    bit-exact on a batch subset, argmax property on everything."""
+    torch.manual_seed(0)
+    B = M = K = N = 256
+    g = grid(B, M, N).clamp(-4, 4)
+    for prod in (False, True):
+        if prod:
+            a, b = 1 - torch.rand(B, M, K), 1 - torch.rand(B, K, N)
+            op = genbmm.prodmaxbmm
+        else:
+            a, b = grid(B, M, K), grid(B, K, N)
+            op = genbmm.maxbmm
+        ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+        out = op(ad, bd)
+        ga, gb = torch.autograd.grad(out, (ad, bd), g.to(gpu))
+        _, idx = _abi_max(gpu, ad.detach(), bd.detach(), prod)
+        pick = [0, 101, 255]
+        sv, si = oracle.seq_maxbmm_fwd(a[pick], b[pick], prod)
+        assert torch.equal(out[pick].detach().cpu(), sv) and torch.equal(idx[pick].cpu(), si)
+        wa, wb = oracle.seq_argmax_bwd(a[pick] if prod else K, b[pick], si, g[pick], prod)
+        assert torch.equal(ga[pick].cpu(), wa) and torch.equal(gb[pick].cpu(), wb)
+        # property over the full tensors: out == a[m,idx] (x) b[idx,n]
+        li = idx.long()
+        bsel = torch.gather(bd.detach(), 1, li)                      # b[idx[m,n], n]
+        asel = torch.gather(ad.detach().unsqueeze(2).expand(B, M, N, K), 3, li.unsqueeze(-1)).squeeze(-1)
+        rebuilt = asel * bsel if prod else asel + bsel
+        assert torch.equal(rebuilt, out.detach())
+        if not prod:
+            # ties are present in this configuration and resolve to the lowest k
+            s = a[0].unsqueeze(-1) + b[0].unsqueeze(-3)
+            assert int(((s == sv[0].unsqueeze(-2)).sum(-2) > 1).sum()) > 100
+
+
+# -------------------------------------------------------------------- sample
+def test_sample_index_brackets_cdf(gpu):
+    torch.manual_seed(11)
+    B, M, K, N = 6, 20, 37, 24
+    a, b = 2 * torch.randn(B, M, K), 2 * torch.randn(B, K, N)
+    seed, offset = 1234, 5
+    lib = _lib.load()
+    ad, bd = a.to(gpu), b.to(gpu)
+    out = torch.empty(B, M, N, device=gpu)
+    idx = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
+    rc = lib.genbmm_samplebmm_fwd(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx),
+                                  seed, offset, B, M, K, N, _lib.stream_of(ad))
+    assert rc == 0
+    close(out, lse64(a, b))
+    u = oracle.philox_uniform(0, B * M * N, seed, offset).view(B, M, N)
+    cdf = oracle.sample_cdf64(a, b)                                   # (B,M,K,N)
+    got = idx.cpu().long()
+    want = oracle.sample_index_from_cdf(cdf, u).long()
+    assert float((got != want).float().mean()) < 2e-3
+    # every index brackets its uniform up to fp32 rounding of the CDF
+    hi = torch.gather(cdf, 2, got.unsqueeze(2)).squeeze(2)
+    lo = torch.where(got > 0, torch.gather(cdf, 2, (got - 1).clamp(min=0).unsqueeze(2)).squeeze(2),
+                     torch.zeros_like(hi))
+    tol = 2e-5
+    ok = (lo - tol <= u.double()) & (u.double() <= hi + tol)
+    assert bool(ok.all())
+    # same stream -> same draw; other offset -> different draw
+    idx2 = torch.empty_like(idx)
+    lib.genbmm_samplebmm_fwd(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx2),
+                             seed, offset, B, M, K, N, _lib.stream_of(ad))
+    assert torch.equal(idx, idx2)
+    lib.genbmm_samplebmm_fwd(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx2),
+                             seed, offset + 1, B, M, K, N, _lib.stream_of(ad))
+    assert not torch.equal(idx, idx2)
+
+
+def test_sample_config_c4_chi_square(gpu):
+    """BASELINE config 3: Normal(0,2) (64,512,512) potentials, Philox seed 1234; 10^4
+    draws per cell of the (4,16,16) slice; per-cell chi-square against the float64
+    softmax, categories with expected count < 5 pooled, bound = the 1-1e-6 quantile."""
+    from scipy.stats import chi2 as chi2_dist
+
+    torch.manual_seed(0)
+    a, b = 2 * torch.randn(64, 512, 512), 2 * torch.randn(64, 512, 512)
+    sa, sb = a[:4, :16, :].contiguous(), b[:4, :, :16].contiguous()
+    draws = 10000
+    A = sa.repeat(draws, 1, 1).to(gpu).requires_grad_(True)           # (40000,16,512)
+    Bm = sb.repeat(draws, 1, 1).to(gpu)
+    out = genbmm.samplebmm(A, Bm, (1234, 0))
+    # the gradient is the one-hot sample: histogram it through grad_a-like counts
+    lib = _lib.load()
+    idx = torch.empty(A.shape[0], 16, 16, dtype=torch.int32, device=gpu)
+    o2 = torch.empty_like(out)
+    lib.genbmm_samplebmm_fwd(_lib.ptr(A), _lib.ptr(Bm), _lib.ptr(o2), _lib.ptr(idx), 1234, 0,
+                             A.shape[0], 16, 512, 16, _lib.stream_of(A))
+    assert torch.equal(o2, out.detach())
+    (gA,) = torch.autograd.grad(out.sum(), (A,))                      # one-hot rows summed over n
+    onehot = torch.zeros(A.shape[0], 16, 512, device=gpu)
+    onehot.scatter_add_(2, idx.long(), torch.ones_like(idx, dtype=torch.float32))
+    assert torch.equal(gA, onehot)
+    counts = torch.zeros(4, 16, 16, 512, dtype=torch.float64)
+    iv = idx.view(draws, 4, 16, 16).cpu().long()
+    counts.scatter_add_(3, iv.permute(1, 2, 3, 0), torch.ones(4, 16, 16, draws, dtype=torch.float64))
+    p = torch.softmax(sa.double().unsqueeze(-1) + sb.double().unsqueeze(-3), -2).permute(0, 1, 3, 2)
+    expc = p * draws                                                  # (4,16,16,512)
+    worst = 0.0
+    for cell in range(4 * 16 * 16):
+        e, c = expc.reshape(-1, 512)[cell], counts.reshape(-1, 512)[cell]
+        keep = e >= 5
+        stat = float((((c - e) ** 2) / e)[keep].sum())
+        dof = int(keep.sum())
+        if (~keep).any():
+            ep, cp = float(e[~keep].sum()), float(c[~keep].sum())
+            if ep >= 1:
+                stat += (cp - ep) ** 2 / ep
+                dof += 1
+        dof = max(dof - 1, 1)
+        bound = chi2_dist.ppf(1 - 1e-6, dof)
+        worst = max(worst, stat / bound)
+        assert stat < bound, (cell, stat, bound, dof)
+    assert worst > 0
+
+
+def test_sample_public_api_follows_torch_seed(gpu):
+    a, b = torch.randn(3, 8, 16, device=gpu, requires_grad=True), torch.randn(3, 16, 8, device=gpu)
+    torch.manual_seed(5)
+    g1 = torch.autograd.grad(genbmm.samplebmm(a, b).sum(), a)[0]
+    g2 = torch.autograd.grad(genbmm.samplebmm(a, b).sum(), a)[0]
+    torch.manual_seed(5)
+    g3 = torch.autograd.grad(genbmm.samplebmm(a, b).sum(), a)[0]
+    assert torch.equal(g1, g3) and not torch.equal(g1, g2)
+    assert torch.equal(g1.sum(-1), torch.full((3, 8), 8.0, device=gpu))  # one sample per (m,n)
+
+
+# ------------------------------------------------------------ error handling
+def test_errors(gpu):
+    a, b = torch.randn(2, 3, 4), torch.randn(2, 4, 5)
+    for op in (genbmm.logbmm, genbmm.maxbmm, genbmm.samplebmm, genbmm.prodmaxbmm):
+        with pytest.raises(RuntimeError, match="CUDA tensor"):
+            op(a, b)                                                   # matmul_cuda.cpp:65
+        with pytest.raises(RuntimeError, match="contiguous"):
+            op(a.to(gpu).transpose(1, 2).contiguous().transpose(1, 2), b.to(gpu))  # :66
+        with pytest.raises(RuntimeError, match="shape mismatch"):
+            op(a.to(gpu), torch.randn(2, 3, 5, device=gpu))
+        with pytest.raises(RuntimeError, match="float32"):
+            op(a.to(gpu).double(), b.to(gpu).double())
+    lib = _lib.load()
+    null = ctypes.c_void_p(0)
+    ad = a.to(gpu)
+    assert lib.genbmm_logbmm_fwd(null, _lib.ptr(ad), _lib.ptr(ad), 1, 1, 1, 1, null) == -1
+    assert lib.genbmm_logbmm_fwd(_lib.ptr(ad), _lib.ptr(ad), _lib.ptr(ad), 1, -1, 1, 1, null) == -2
+    assert lib.genbmm_banded_fwd(_lib.ptr(ad), 0, 0, _lib.ptr(ad), 0, 0, _lib.ptr(ad), null, 1, 1, 2, null) == -3
+    assert lib.genbmm_banded_fwd(_lib.ptr(ad), -1, 0, _lib.ptr(ad), 0, 0, _lib.ptr(ad), null, 1, 1, 0, null) == -4
+    assert b"NULL" in lib.genbmm_error_string(-1)
+
+
+def test_empty_and_half(gpu):
+    for shape in [(0, 3, 4, 5), (2, 0, 4, 5), (2, 3, 4, 0)]:
+        B, M, K, N = shape
+        out = genbmm.logbmm(torch.randn(B, M, K, device=gpu), torch.randn(B, K, N, device=gpu))
+        assert out.shape == (B, M, N)
+    out = genbmm.logbmm(torch.randn(2, 3, 0, device=gpu), torch.randn(2, 0, 5, device=gpu))
+    assert bool(torch.isinf(out).all())                              # empty sum: log(0) - 1e9
+    a, b = torch.randn(2, 9, 12, device=gpu).half(), torch.randn(2, 12, 7, device=gpu).half()
+    out = genbmm.logbmm(a.requires_grad_(True), b)
+    assert out.dtype == torch.float16
+    close(out.float(), lse64(a.float().cpu(), b.float().cpu()), rtol=2e-3, atol=2e-3)
+    (ga,) = torch.autograd.grad(out.sum(), a)
+    assert ga.dtype == torch.float16

@@ -1,0 +1,140 @@
+"""Host-side logic that needs no GPU: band structure operations against explicit index
+loops (the reference's test_sparse.py strategy), the C-ABI library's exported symbols,
+and the no-CPU-fallback rule."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+from hypothesis import given, settings
+from hypothesis.strategies import integers
+
+import oracle
+import genbmm_amd
+from genbmm_amd import _lib
+from genbmm_amd.sparse import BandedMatrix, banddiag
+
+mint = integers(min_value=6, max_value=10)
+lint = integers(min_value=0, max_value=10)
+sint = integers(min_value=3, max_value=5)
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@settings(max_examples=25, deadline=None)
+@given(sint, mint, lint, lint)
+def test_band_structure(batch, n, lu, ld):
+    """Mirrors genbmm/test_sparse.py:12-55 with the loops living in the oracle."""
+    start = torch.rand(batch, n, n)
+    band, same = banddiag(start, lu, ld)
+    assert torch.equal(band, oracle.band_from_dense(start, lu, ld))
+    assert torch.equal(same, start)
+    mid = oracle.band_to_dense(band, lu, ld, 0.0)
+    banded = BandedMatrix(band, lu, ld)
+    assert torch.equal(banded.to_dense(), mid)
+    assert torch.equal(BandedMatrix(band, lu, ld, fill=-3.0).to_dense(), oracle.band_to_dense(band, lu, ld, -3.0))
+    t = banded.transpose()
+    assert (t.lu, t.ld) == (ld, lu)
+    assert torch.equal(t.to_dense(), mid.transpose(-2, -1))
+    assert torch.equal(t.data, oracle.band_transpose(band, lu, ld))
+    plus = banded.op(banded, lambda a, b: a + b)
+    assert (plus.lu, plus.ld) == (lu, ld)
+    assert torch.equal(plus.data, band + band) and torch.equal(plus.to_dense(), mid + mid)
+    plus = banded.op(banded.transpose(), lambda a, b: a + b)
+    assert plus.lu == max(lu, ld) and plus.ld == max(lu, ld)
+    assert torch.equal(plus.to_dense(), mid.transpose(-2, -1) + mid)
+    wide = banded._expand(lu + 2, ld + 1)
+    assert torch.equal(wide.to_dense(), mid)
+
+
+@settings(max_examples=15, deadline=None)
+@given(sint, mint)
+def test_col_shift(batch, n):
+    """genbmm/test_sparse.py:87-107."""
+    lu = ld = 1
+    band, _ = banddiag(torch.rand(batch, n, n), lu, ld)
+    bx = BandedMatrix(band, lu, ld)
+    x = bx.to_dense()
+    x2 = torch.cat([x[:, :, 1:], torch.zeros(batch, n, 1)], 2)
+    assert torch.equal(banddiag(x2, lu - 1, ld + 1)[0], bx.col_shift(1).data)
+    x2 = torch.cat([torch.zeros(batch, n, 1), x[:, :, :-1]], 2)
+    assert torch.equal(banddiag(x2, lu + 1, ld - 1)[0], bx.col_shift(-1).data)
+    assert torch.equal(bx.col_unshift().data, bx.col_shift(-1).data)
+    assert bx.col_shift(0) is bx and bx.band_shift(0) is bx and bx.band_pad(0) is bx
+
+
+def test_band_relabel_ops():
+    """band_shift / band_pad / band_unshift: the reference has no test for these; they
+    are pure relabelling of the same cells (sparse.py:96-152), checked here on the dense
+    matrix they denote."""
+    band, _ = banddiag(torch.rand(2, 7, 7), 2, 3)
+    bx = BandedMatrix(band, 2, 3, fill=0)
+    x = bx.to_dense()
+    p = bx.band_pad(2)
+    assert (p.lu, p.ld, p.width) == (4, 5, 10) and torch.equal(p.to_dense(), x)
+    s = bx.band_shift(1)     # drops band cell 0, relabels lu+1 / ld-1
+    assert (s.lu, s.ld) == (3, 2)
+    assert torch.equal(s.data[:, :, :-1], band[:, :, 1:]) and bool((s.data[:, :, -1] == 0).all())
+    s = bx.band_shift(-2)
+    assert (s.lu, s.ld) == (0, 5)
+    assert torch.equal(s.data[:, :, 2:], band[:, :, :-2]) and bool((s.data[:, :, :2] == 0).all())
+    u = bx.band_unshift()
+    assert (u.lu, u.ld) == (1, 4) and torch.equal(u.data, bx.band_shift(-1).data)
+    f = BandedMatrix(band, 2, 3, fill=-1e9).band_pad(1)
+    assert bool((f.data[:, :, 0] == -1e9).all()) and bool((f.data[:, :, -1] == -1e9).all())
+
+
+def test_transpose_is_differentiable():
+    band = banddiag(torch.rand(2, 6, 6), 2, 1)[0].clone().requires_grad_(True)
+    t = BandedMatrix(band, 2, 1).transpose()
+    (g,) = torch.autograd.grad(t.data.sum(), band)
+    inside = oracle.band_from_dense(torch.ones(2, 6, 6), 2, 1)
+    assert torch.equal(g, inside)
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "genbmm_gfx950.h")).read()
+    declared = set(re.findall(r"\b(genbmm_[a-z_0-9]+)\s*\(", header))
+    assert len(declared) == 13
+    assert declared == set(_lib.SIGNATURES) | set(_lib.STRING_FUNCS)
+    assert os.path.exists(_lib.LIB_PATH), "build with `python -m genbmm_amd.build`"
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), name
+    lib.genbmm_version.restype = ctypes.c_char_p
+    assert lib.genbmm_version().startswith(b"genbmm-gfx950")
+    lib.genbmm_error_string.restype = ctypes.c_char_p
+    assert lib.genbmm_error_string(-2) == b"a dimension is negative or too large"
+
+
+def test_no_cpu_fallback():
+    a, b = torch.randn(2, 3, 4), torch.randn(2, 4, 5)
+    for op in (genbmm_amd.logbmm, genbmm_amd.maxbmm, genbmm_amd.samplebmm, genbmm_amd.prodmaxbmm):
+        with pytest.raises(RuntimeError):
+            op(a, b)
+    band = torch.randn(2, 5, 3)
+    for name in ("multiply", "multiply_log", "multiply_max"):
+        with pytest.raises(RuntimeError):
+            getattr(BandedMatrix(band, 1, 1), name)(BandedMatrix(band, 1, 1))
+
+
+def test_product_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "genbmm_amd")
+    for fn in os.listdir(pkg):
+        if fn.endswith(".py"):
+            src = open(os.path.join(pkg, fn)).read()
+            assert not re.search(r"^\s*(import|from)\s+oracle\b", src, re.M), fn
+
+
+def test_install_as_genbmm():
+    import sys
+
+    mod = genbmm_amd.install_as_genbmm()
+    import genbmm
+
+    assert genbmm is mod and genbmm.logbmm is genbmm_amd.logbmm
+    from genbmm.sparse import BandedMatrix as BM
+
+    assert BM is BandedMatrix
+    for k in ("genbmm", "genbmm.genmul", "genbmm.sparse"):
+        sys.modules.pop(k, None)

@@ -219,6 +219,7 @@ def test_band_layout_matches_host_banddiag():
         assert torch.equal(oracle.band_from_dense(x, lu, ld), banddiag(x, lu, ld)[0])
         band = oracle.band_from_dense(x, lu, ld)
         assert torch.equal(oracle.band_to_dense(band, lu, ld, -7.0), BandedMatrix(band, lu, ld, -7.0).to_dense())
+        assert torch.equal(oracle.band_transpose_indexed(band, lu, ld), oracle.band_transpose(band, lu, ld))
 
 
 @pytest.mark.parametrize("n,a_lu,a_ld,b_lu,b_ld", BANDS)
