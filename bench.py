@@ -25,14 +25,14 @@ FP32_VALU_PEAK_TFLOPS = 157.3  # MI355X vector FP32 peak (packed FMA); the metri
 DOMINANT_TRAFFIC_BYTES = None
 
 
-def cpu_baseline(torch, sample_batches=4):
+def cpu_baseline(torch, sample_batches=64):
     """The reference's CPU formulation (README.md:31-35): broadcast add + logsumexp, and
     autograd backward, on `sample_batches` items of the headline shape, one item per
     chunk (a 512 MB fp32 intermediate each)."""
     import oracle
 
     cores = os.cpu_count() or 1
-    cores = min(cores, 16)
+    cores = min(cores, 16)  # the GPU box grants 16 host cores to a one-GPU job
     torch.set_num_threads(cores)
     torch.manual_seed(0)
     a = torch.randn(sample_batches, M, K)
@@ -85,18 +85,19 @@ def main():
     g = torch.randn(B, M, N).to(dev)
     out = torch.empty(B, M, N, device=dev)
     ga, gb = torch.empty_like(a), torch.empty_like(b)
+    stats = torch.empty(B, M + N, device=dev)
     stream = _lib.stream_of(a)
     p = _lib.ptr
     null = p(None)
 
     def fwd():
-        _lib.check(lib.genbmm_logbmm_fwd(p(a), p(b), p(out), B, M, K, N, stream), "fwd")
+        _lib.check(lib.genbmm_logbmm_fwd(p(a), p(b), p(out), p(stats), B, M, K, N, stream), "fwd")
 
     def bwd_a():
-        _lib.check(lib.genbmm_logbmm_bwd(p(a), p(b), p(out), p(g), p(ga), null, B, M, K, N, stream), "bwd_a")
+        _lib.check(lib.genbmm_logbmm_bwd(p(a), p(b), p(out), p(g), p(stats), p(ga), null, B, M, K, N, stream), "bwd_a")
 
     def bwd_b():
-        _lib.check(lib.genbmm_logbmm_bwd(p(a), p(b), p(out), p(g), null, p(gb), B, M, K, N, stream), "bwd_b")
+        _lib.check(lib.genbmm_logbmm_bwd(p(a), p(b), p(out), p(g), p(stats), null, p(gb), B, M, K, N, stream), "bwd_b")
 
     for _ in range(args.warmup):
         fwd(); bwd_a(); bwd_b()

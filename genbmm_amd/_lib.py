@@ -29,8 +29,8 @@ _BAND = [_c_float_p, _i, _i, _c_float_p, _i, _i]  # a, a_lu, a_ld, b, b_lu, b_ld
 # name -> argtypes (every function returns int unless noted); mirrors
 # include/genbmm_gfx950.h
 SIGNATURES = {
-    "genbmm_logbmm_fwd": [_c_float_p] * 3 + _DENSE_DIMS,
-    "genbmm_logbmm_bwd": [_c_float_p] * 6 + _DENSE_DIMS,
+    "genbmm_logbmm_fwd": [_c_float_p] * 4 + _DENSE_DIMS,
+    "genbmm_logbmm_bwd": [_c_float_p] * 7 + _DENSE_DIMS,
     "genbmm_logbmm_bwdbwd": [_c_float_p] * 9 + _DENSE_DIMS,
     "genbmm_maxbmm_fwd": [_c_float_p] * 3 + [_c_int_p] + _DENSE_DIMS,
     "genbmm_prodmaxbmm_fwd": [_c_float_p] * 3 + [_c_int_p] + _DENSE_DIMS,
@@ -42,6 +42,7 @@ SIGNATURES = {
     "genbmm_banded_bwdbwd": _BAND + [_c_float_p] * 7 + [_i, _i, _vp],
 }
 STRING_FUNCS = {"genbmm_version": [], "genbmm_error_string": [_i]}
+VOID_FUNCS = {"genbmm_logbmm_force_exact": [_i]}
 
 _lib = None
 
@@ -67,6 +68,10 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = argtypes
         fn.restype = ctypes.c_char_p
+    for name, argtypes in VOID_FUNCS.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = None
     _lib = lib
     return lib
 

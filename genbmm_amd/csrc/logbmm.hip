@@ -1,0 +1,570 @@
+// logbmm forward and backward (gfx950): the exact online-log-sum-exp kernels and
+// the factored kernels that replace the per-element exponential by one fused
+// multiply-add whenever that is provably as accurate.
+//
+// Factored form.  With row/column shifts alpha[m] = max_k a[m,k] and
+// beta[n] = max_k b[k,n] (the "stats" vector, alpha then beta per batch item):
+//
+//   EA[m,k] = exp(a[m,k] - alpha[m])  in (0,1]     EB[k,n] = exp(b[k,n] - beta[n])
+//   S[m,n]  = sum_k EA[m,k] * EB[k,n]              out = log S + alpha + beta
+//   H[m,n]  = g[m,n] * exp(alpha[m] + beta[n] - out[m,n])            ( = g / S )
+//   grad_a[m,k] = EA[m,k] * sum_n H[m,n] * EB[k,n]
+//   grad_b[k,n] = EB[k,n] * sum_m EA[m,k] * H[m,n]
+//
+// The exponentials are taken while a tile is staged into LDS (once per tile
+// element, not once per (m,k,n)), the contraction itself is v_fma_f32 on
+// register blocks.  A factor can only underflow for a term that is below
+// 2^-126 of the bound exp(alpha+beta); as long as S >= 2^-40 such terms are
+// below 2^-86 of the result, i.e. invisible in fp32.  Each workgroup checks that
+// condition for its own tile (forward: on S; backward: on alpha+beta-out while
+// staging H) and, if any cell fails it - or is NaN/inf, or sits at the
+// reference's -1e9 floor - recomputes the whole tile with the exact kernel's
+// routine (online running-max log-sum-exp forward, exp(a+b-out) backward), so
+// the result never depends on the factoring being applicable.
+#include <atomic>
+
+#include "dense_tiles.h"
+#include "log_bwd_tile.h"
+
+namespace genbmm {
+namespace {
+
+constexpr float kLog2eLo = 1.92596299e-8f;  // log2(e) - (float)log2(e)
+constexpr float kGuardBits = 40.f;          // factored path needs S >= 2^-40
+
+// exp(d) through v_exp_f32 with the rounding error of d*log2e compensated.
+__device__ __forceinline__ float exp_comp(float d) {
+  const float hi = d * kLog2e;
+  const float lo = __builtin_fmaf(d, kLog2e, -hi) + d * kLog2eLo;
+  const float e = fast_exp2(hi);
+  return __builtin_fmaf(e, lo * kLn2, e);
+}
+
+// ------------------------------------------------------------------ stats
+// stats[b][0..M) = max_k a[b,m,k],  stats[b][M..M+N) = max_k b[b,k,n].
+__global__ __launch_bounds__(256) void k_log_stats(const float* __restrict__ a,
+                                                   const float* __restrict__ b,
+                                                   float* __restrict__ stats, int M, int K, int N,
+                                                   int row_wgs, int col_wgs, int vec_a,
+                                                   int vec_b) {
+  __shared__ float part[8][128];
+  const int per = row_wgs + col_wgs;
+  const int batch = blockIdx.x / per;
+  const int wg = blockIdx.x - batch * per;
+  const int tid = threadIdx.x;
+  float* st = stats + (long)batch * (M + N);
+  if (wg < row_wgs) {  // one wave per row of a
+    const int lane = tid & 63, m = wg * 4 + (tid >> 6);
+    if (m >= M) return;
+    const float* row = a + ((long)batch * M + m) * K;
+    float v = -INFINITY;
+    if (vec_a) {
+      for (int k = lane * 4; k < K; k += 256) {
+        const float4 x = *reinterpret_cast<const float4*>(row + k);
+        v = fmaxf(v, fmaxf(fmaxf(x.x, x.y), fmaxf(x.z, x.w)));
+      }
+    } else {
+      for (int k = lane; k < K; k += 64) v = fmaxf(v, row[k]);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    if (lane == 0) st[m] = v;
+  } else {  // 128 columns of b: 32 column quads x 8 row groups
+    const int c4 = tid & 31, rg = tid >> 5;
+    const int n = (wg - row_wgs) * 128 + c4 * 4;
+    const float* col = b + (long)batch * K * N + n;
+    float4 v = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+    if (n < N) {
+      for (int k = rg; k < K; k += 8) {
+        const float* p = col + (long)k * N;
+        if (vec_b) {
+          const float4 x = *reinterpret_cast<const float4*>(p);
+          v.x = fmaxf(v.x, x.x); v.y = fmaxf(v.y, x.y); v.z = fmaxf(v.z, x.z); v.w = fmaxf(v.w, x.w);
+        } else {
+          v.x = fmaxf(v.x, p[0]);
+          if (n + 1 < N) v.y = fmaxf(v.y, p[1]);
+          if (n + 2 < N) v.z = fmaxf(v.z, p[2]);
+          if (n + 3 < N) v.w = fmaxf(v.w, p[3]);
+        }
+      }
+    }
+    part[rg][c4 * 4 + 0] = v.x; part[rg][c4 * 4 + 1] = v.y;
+    part[rg][c4 * 4 + 2] = v.z; part[rg][c4 * 4 + 3] = v.w;
+    __syncthreads();
+    if (tid < 128) {
+      const int nn = (wg - row_wgs) * 128 + tid;
+      if (nn < N) {
+        float r = part[0][tid];
+#pragma unroll
+        for (int q = 1; q < 8; ++q) r = fmaxf(r, part[q][tid]);
+        st[M + nn] = r;
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------ exact kernels
+template <class C>
+__global__ __launch_bounds__(C::NT) void k_log_fwd_exact(const DenseArgs p) {
+  __shared__ __attribute__((aligned(16))) float smem[C::KT * (C::LDA + C::LDB)];
+  int batch, m0, n0;
+  decode_tile<C>(p, batch, m0, n0);
+  log_fwd_tile<C, false>(p, batch, m0, n0, smem, smem + C::KT * C::LDA);
+}
+
+template <class C, bool GRAD_A>
+__global__ __launch_bounds__(C::NT) void k_log_bwd_exact(const LogBwdArgs p) {
+  __shared__ __attribute__((aligned(16))) float smem[LogBwdLds<C, GRAD_A>::FLOATS];
+  const int per = p.tiles_r * p.tiles_c;
+  const int batch = blockIdx.x / per;
+  const int rem = blockIdx.x - batch * per;
+  log_bwd_tile<C, GRAD_A>(p, batch, (rem / p.tiles_c) * C::BR, (rem % p.tiles_c) * C::BC, smem);
+}
+
+// --------------------------------------------------------- factored forward
+// C: tile of the factored pass; CX: tile of the exact routine used for the
+// recompute, covering the same BN and NX * CX::BM = C::BM rows.
+template <class C, class CX, int NX>
+__global__ __launch_bounds__(C::NT) void k_log_fwd_fast(const DenseArgs p,
+                                                        const float* __restrict__ stats) {
+  static_assert(CX::BN == C::BN && CX::BM * NX == C::BM && CX::NT == C::NT && CX::KT <= C::KT, "");
+  __shared__ __attribute__((aligned(16))) float smem[C::KT * (C::LDA + C::LDB) + C::BM + C::BN];
+  float* As = smem;
+  float* Bs = As + C::KT * C::LDA;
+  float* al = Bs + C::KT * C::LDB;
+  float* be = al + C::BM;
+  const int tid = threadIdx.x, tx = tid % C::TX, ty = tid / C::TX;
+  int batch, m0, n0;
+  decode_tile<C>(p, batch, m0, n0);
+  const int M = p.M, K = p.K, N = p.N;
+  const float* ab = p.a + (long)batch * M * K;
+  const float* bb = p.b + (long)batch * K * N;
+  const float* st = stats + (long)batch * (M + N);
+  for (int t = tid; t < C::BM; t += C::NT) al[t] = (m0 + t < M) ? st[m0 + t] : 0.f;
+  for (int t = tid; t < C::BN; t += C::NT) be[t] = (n0 + t < N) ? st[M + n0 + t] : 0.f;
+  __syncthreads();
+
+  float acc[C::TM][C::TN];
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) acc[i][j] = 0.f;
+
+  using TA = TileOutMajor<C::BM, C::KT, C::NT>;
+  using TB = TileRedMajor<C::BN, C::KT, C::NT>;
+  TA ta;
+  TB tb;
+  if (K > 0) {
+    ta.gload(ab, K, m0, 0, M, K, p.vec_a, tid);
+    tb.gload(bb, N, n0, 0, N, K, p.vec_b, tid);
+  }
+  for (int k0 = 0; k0 < K; k0 += C::KT) {
+    __syncthreads();
+#pragma unroll
+    for (int l = 0; l < TA::PER; ++l) {  // EA = exp(a - alpha[row])
+      const float s = al[((tid + l * C::NT) / TA::C4) % C::BM];
+      ta.r[l].x = exp_comp(ta.r[l].x - s); ta.r[l].y = exp_comp(ta.r[l].y - s);
+      ta.r[l].z = exp_comp(ta.r[l].z - s); ta.r[l].w = exp_comp(ta.r[l].w - s);
+    }
+#pragma unroll
+    for (int l = 0; l < TB::PER; ++l) {  // EB = exp(b - beta[col])
+      const float4 s = *reinterpret_cast<const float4*>(be + ((tid + l * C::NT) % TB::C4) * 4);
+      tb.r[l].x = exp_comp(tb.r[l].x - s.x); tb.r[l].y = exp_comp(tb.r[l].y - s.y);
+      tb.r[l].z = exp_comp(tb.r[l].z - s.z); tb.r[l].w = exp_comp(tb.r[l].w - s.w);
+    }
+    ta.sstore(As, tid);
+    tb.sstore(Bs, tid);
+    __syncthreads();
+    if (k0 + C::KT < K) {
+      ta.gload(ab, K, m0, k0 + C::KT, M, K, p.vec_a, tid);
+      tb.gload(bb, N, n0, k0 + C::KT, N, K, p.vec_b, tid);
+    }
+    const int kn = min(C::KT, K - k0);
+    auto step = [&](int kk) __attribute__((always_inline)) {
+      float av[C::TM], bv[C::TN];
+      lds_frag<C::TM / 4>(As + kk * C::LDA, ty * C::TM, 4, av);
+      lds_frag<C::TN / 4>(Bs + kk * C::LDB, tx * 4, C::TX * 4, bv);
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
+    };
+    if (kn == C::KT) {
+#pragma unroll
+      for (int kk = 0; kk < C::KT; ++kk) step(kk);
+    } else {
+      for (int kk = 0; kk < kn; ++kk) step(kk);
+    }
+  }
+
+  // guard + epilogue
+  const float thr = __builtin_amdgcn_exp2f(-kGuardBits);
+  int bad = 0;
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i) {
+    const int r = ty * C::TM + i;
+    const float ai = al[r];
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) {
+      const int c = col_of<C>(tx, j);
+      const float shift = ai + be[c];
+      const float s = acc[i][j];
+      const bool ok = (s >= thr) && (s < INFINITY) && (shift > 0.9f * kFloor) && (shift < INFINITY);
+      if (!ok && m0 + r < M && n0 + c < N) bad = 1;
+      acc[i][j] = logf(s) + shift;
+    }
+  }
+  if (__syncthreads_or(bad)) {
+#pragma unroll
+    for (int h = 0; h < NX; ++h)
+      if (m0 + h * CX::BM < M) {
+        log_fwd_tile<CX, false>(p, batch, m0 + h * CX::BM, n0, smem, smem + CX::KT * CX::LDA);
+        __syncthreads();
+      }
+    return;
+  }
+  store_tile_f<C>(p.out + (long)batch * M * N, acc, m0, n0, M, N, p.vec_o, tx, ty);
+}
+
+// -------------------------------------------------------- factored backward
+// Output tile (rows r, cols c) = (m,k) for grad_a, (k,n) for grad_b; the
+// reduction index q is n or m.  Y = the other operand, staged as exp(y - shift);
+// H = g*exp(alpha+beta-out), staged from out and g; X = the operand shaped like
+// the output, read once in the epilogue.
+template <class C, class CX, int NX, bool GRAD_A>
+__global__ __launch_bounds__(C::NT) void k_log_bwd_fast(const LogBwdArgs p,
+                                                        const float* __restrict__ stats) {
+  constexpr int BY = GRAD_A ? C::BC : C::BR;
+  constexpr int BO = GRAD_A ? C::BR : C::BC;
+  using TYt = std::conditional_t<GRAD_A, TileOutMajor<BY, C::RT, C::NT>, TileRedMajor<BY, C::RT, C::NT>>;
+  using TOt = std::conditional_t<GRAD_A, TileOutMajor<BO, C::RT, C::NT>, TileRedMajor<BO, C::RT, C::NT>>;
+  constexpr int LDY = BY + kPad, LDO = BO + kPad;
+  constexpr int FAST_FLOATS = C::RT * (LDY + LDO);
+  constexpr int EXACT_FLOATS = LogBwdLds<CX, GRAD_A>::FLOATS;
+  __shared__ __attribute__((aligned(16))) float smem[FAST_FLOATS > EXACT_FLOATS ? FAST_FLOATS : EXACT_FLOATS];
+  float* Ys = smem;
+  float* Hs = smem + C::RT * LDY;
+
+  const int tid = threadIdx.x, tx = tid % C::TX, ty = tid / C::TX;
+  const int M = p.M, K = p.K, N = p.N;
+  const int R = GRAD_A ? M : K, Cc = GRAD_A ? K : N, Q = GRAD_A ? N : M;
+  const int per = p.tiles_r * p.tiles_c;
+  const int batch = blockIdx.x / per;
+  const int rem = blockIdx.x - batch * per;
+  const int r0 = (rem / p.tiles_c) * C::BR, c0 = (rem % p.tiles_c) * C::BC;
+
+  const float* ab = p.a + (long)batch * M * K;
+  const float* bb = p.b + (long)batch * K * N;
+  const float* ob = p.out + (long)batch * M * N;
+  const float* gb = p.g + (long)batch * M * N;
+  const float* xb = GRAD_A ? ab : bb;
+  const float* yb = GRAD_A ? bb : ab;
+  const float* al = stats + (long)batch * (M + N);  // alpha[m]
+  const float* be = al + M;                         // beta[n]
+  const long ldy = GRAD_A ? N : K;
+  const bool vec_x = GRAD_A ? p.vec_k : p.vec_n;
+  const bool vec_y = GRAD_A ? p.vec_n : p.vec_k;
+  const bool vec_o = p.vec_n;
+  const int y0 = GRAD_A ? c0 : r0;
+  const int o0 = GRAD_A ? r0 : c0, olim = GRAD_A ? M : N;
+  const float lim = kGuardBits * kLn2 + 1e-3f;  // alpha+beta-out above this: S < 2^-40
+
+  auto col_of = [&](int j) { return (j >> 2) * (C::TX * 4) + tx * 4 + (j & 3); };
+  auto safe = [](const float* v, int i, int n) { return i < n ? v[i] : 0.f; };
+
+  float acc[C::TR][C::TC];
+#pragma unroll
+  for (int i = 0; i < C::TR; ++i)
+#pragma unroll
+    for (int j = 0; j < C::TC; ++j) acc[i][j] = 0.f;
+
+  // Shifts that do not change from slab to slab.
+  // GRAD_A: H rows are m (out axis): alpha per float4 of the H tile.
+  // GRAD_B: H cols are n (out axis): beta float4 per float4 of the H tile.
+  float fix_s[TOt::PER];
+  float4 fix_v[TOt::PER];
+#pragma unroll
+  for (int l = 0; l < TOt::PER; ++l) {
+    const int idx = tid + l * C::NT;
+    if (GRAD_A) {
+      fix_s[l] = safe(al, o0 + idx / TOt::C4, M);
+    } else {
+      const int n = o0 + (idx % TOt::C4) * 4;
+      fix_v[l] = make_float4(safe(be, n, N), safe(be, n + 1, N), safe(be, n + 2, N), safe(be, n + 3, N));
+    }
+  }
+
+  TYt tyl;
+  TOt tol, tgl;
+  auto load = [&](int q0) __attribute__((always_inline)) {
+    tyl.gload(yb, ldy, y0, q0, K, Q, vec_y, tid);
+    tol.gload(ob, N, o0, q0, olim, Q, vec_o, tid);
+    tgl.gload(gb, N, o0, q0, olim, Q, vec_o, tid);
+  };
+  int bad = 0;
+  if (Q > 0) load(0);
+  for (int q0 = 0; q0 < Q; q0 += C::RT) {
+    __syncthreads();
+    if (GRAD_A) {
+      // red axis = n (4 consecutive n per float4): beta float4 shared by Y and H
+      {
+        const int n = q0 + (tid % TYt::C4) * 4;  // C4 == RT/4 for both tiles; NT % C4 == 0
+        const float4 bq = make_float4(safe(be, n, N), safe(be, n + 1, N), safe(be, n + 2, N), safe(be, n + 3, N));
+#pragma unroll
+        for (int l = 0; l < TYt::PER; ++l) {
+          tyl.r[l].x = exp_comp(tyl.r[l].x - bq.x); tyl.r[l].y = exp_comp(tyl.r[l].y - bq.y);
+          tyl.r[l].z = exp_comp(tyl.r[l].z - bq.z); tyl.r[l].w = exp_comp(tyl.r[l].w - bq.w);
+        }
+#pragma unroll
+        for (int l = 0; l < TOt::PER; ++l) {
+          const int m = o0 + (tid + l * C::NT) / TOt::C4;
+          const float ex = fix_s[l] + bq.x - tol.r[l].x, ey = fix_s[l] + bq.y - tol.r[l].y;
+          const float ez = fix_s[l] + bq.z - tol.r[l].z, ew = fix_s[l] + bq.w - tol.r[l].w;
+          if (m < M) {
+            if (n < N && !(ex <= lim)) bad = 1;
+            if (n + 1 < N && !(ey <= lim)) bad = 1;
+            if (n + 2 < N && !(ez <= lim)) bad = 1;
+            if (n + 3 < N && !(ew <= lim)) bad = 1;
+          }
+          tol.r[l].x = tgl.r[l].x * exp_comp(ex); tol.r[l].y = tgl.r[l].y * exp_comp(ey);
+          tol.r[l].z = tgl.r[l].z * exp_comp(ez); tol.r[l].w = tgl.r[l].w * exp_comp(ew);
+        }
+      }
+    } else {
+      // red axis = m (one m per float4 row)
+#pragma unroll
+      for (int l = 0; l < TYt::PER; ++l) {
+        const float s = safe(al, q0 + (tid + l * C::NT) / TYt::C4, M);
+        tyl.r[l].x = exp_comp(tyl.r[l].x - s); tyl.r[l].y = exp_comp(tyl.r[l].y - s);
+        tyl.r[l].z = exp_comp(tyl.r[l].z - s); tyl.r[l].w = exp_comp(tyl.r[l].w - s);
+      }
+#pragma unroll
+      for (int l = 0; l < TOt::PER; ++l) {
+        const int idx = tid + l * C::NT;
+        const int m = q0 + idx / TOt::C4, n = o0 + (idx % TOt::C4) * 4;
+        const float s = safe(al, m, M);
+        const float ex = s + fix_v[l].x - tol.r[l].x, ey = s + fix_v[l].y - tol.r[l].y;
+        const float ez = s + fix_v[l].z - tol.r[l].z, ew = s + fix_v[l].w - tol.r[l].w;
+        if (m < M) {
+          if (n < N && !(ex <= lim)) bad = 1;
+          if (n + 1 < N && !(ey <= lim)) bad = 1;
+          if (n + 2 < N && !(ez <= lim)) bad = 1;
+          if (n + 3 < N && !(ew <= lim)) bad = 1;
+        }
+        tol.r[l].x = tgl.r[l].x * exp_comp(ex); tol.r[l].y = tgl.r[l].y * exp_comp(ey);
+        tol.r[l].z = tgl.r[l].z * exp_comp(ez); tol.r[l].w = tgl.r[l].w * exp_comp(ew);
+      }
+    }
+    tyl.sstore(Ys, tid);
+    tol.sstore(Hs, tid);
+    __syncthreads();
+    if (q0 + C::RT < Q) load(q0 + C::RT);
+    const int qn = min(C::RT, Q - q0);
+    auto step = [&](int qq) __attribute__((always_inline)) {
+      if (GRAD_A) {
+        float yv[C::TC], hv[C::TR];
+        lds_frag<C::TC / 4>(Ys + qq * LDY, tx * 4, C::TX * 4, yv);
+        lds_frag<C::TR / 4>(Hs + qq * LDO, ty * C::TR, 4, hv);
+#pragma unroll
+        for (int i = 0; i < C::TR; ++i)
+#pragma unroll
+          for (int j = 0; j < C::TC; ++j) acc[i][j] = __builtin_fmaf(hv[i], yv[j], acc[i][j]);
+      } else {
+        float yv[C::TR], hv[C::TC];
+        lds_frag<C::TR / 4>(Ys + qq * LDY, ty * C::TR, 4, yv);
+        lds_frag<C::TC / 4>(Hs + qq * LDO, tx * 4, C::TX * 4, hv);
+#pragma unroll
+        for (int i = 0; i < C::TR; ++i)
+#pragma unroll
+          for (int j = 0; j < C::TC; ++j) acc[i][j] = __builtin_fmaf(yv[i], hv[j], acc[i][j]);
+      }
+    };
+    if (qn == C::RT) {
+#pragma unroll
+      for (int qq = 0; qq < C::RT; ++qq) step(qq);
+    } else {
+      for (int qq = 0; qq < qn; ++qq) step(qq);
+    }
+  }
+
+  if (__syncthreads_or(bad)) {
+#pragma unroll
+    for (int h = 0; h < NX; ++h)
+      if (r0 + h * CX::BR < R) {
+        log_bwd_tile<CX, GRAD_A>(p, batch, r0 + h * CX::BR, c0, smem);
+        __syncthreads();
+      }
+    return;
+  }
+
+  // epilogue: grad = exp(x - shift) * acc, x re-read from global memory
+  float* gradb = p.grad + (long)batch * R * Cc;
+  const float* xshift = GRAD_A ? al : be;  // alpha by row (m) / beta by column (n)
+#pragma unroll
+  for (int i = 0; i < C::TR; ++i) {
+    const int r = r0 + ty * C::TR + i;
+    if (r >= R) continue;
+    const float rs = GRAD_A ? xshift[r] : 0.f;
+#pragma unroll
+    for (int q4 = 0; q4 < C::TC / 4; ++q4) {
+      const int c = c0 + col_of(4 * q4);
+      if (c >= Cc) continue;
+      const float* src = xb + (long)r * Cc + c;
+      float* dst = gradb + (long)r * Cc + c;
+      float xv[4], sv[4];
+      const bool full = vec_x && c + 3 < Cc;
+      if (full) {
+        const float4 v = *reinterpret_cast<const float4*>(src);
+        xv[0] = v.x; xv[1] = v.y; xv[2] = v.z; xv[3] = v.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) xv[e] = (c + e < Cc) ? src[e] : 0.f;
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        sv[e] = GRAD_A ? rs : safe(xshift, c + e, Cc);
+        xv[e] = exp_comp(xv[e] - sv[e]) * acc[i][4 * q4 + e];
+      }
+      if (full) {
+        *reinterpret_cast<float4*>(dst) = make_float4(xv[0], xv[1], xv[2], xv[3]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (c + e < Cc) dst[e] = xv[e];
+      }
+    }
+  }
+}
+
+// ----------------------------------------------------------------- dispatch
+std::atomic<int> g_force_exact{0};
+
+template <class C>
+int launch_fwd_exact(DenseArgs p, int B, int M, int K, int N, hipStream_t s) {
+  dim3 grid;
+  if (int e = fill_args<C>(p, B, M, K, N, grid)) return e;
+  hipLaunchKernelGGL((k_log_fwd_exact<C>), grid, dim3(C::NT), 0, s, p);
+  return launch_status();
+}
+
+template <class C, class CX, int NX>
+int launch_fwd_fast(DenseArgs p, const float* stats, int B, int M, int K, int N, hipStream_t s) {
+  dim3 grid;
+  if (int e = fill_args<C>(p, B, M, K, N, grid)) return e;
+  hipLaunchKernelGGL((k_log_fwd_fast<C, CX, NX>), grid, dim3(C::NT), 0, s, p, stats);
+  return launch_status();
+}
+
+int launch_stats(const float* a, const float* b, float* stats, int B, int M, int K, int N,
+                 hipStream_t s) {
+  const int row_wgs = ceil_div(M, 4), col_wgs = ceil_div(N, 128);
+  const int64_t total = (int64_t)B * (row_wgs + col_wgs);
+  if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
+  if (total == 0) return GENBMM_OK;
+  hipLaunchKernelGGL(k_log_stats, dim3((unsigned)total), dim3(256), 0, s, a, b, stats, M, K, N,
+                     row_wgs, col_wgs, (int)((K % 4 == 0) && aligned16(a)),
+                     (int)((N % 4 == 0) && aligned16(b)));
+  return launch_status();
+}
+
+template <class C, bool GRAD_A>
+int launch_bwd_exact(LogBwdArgs p, int B, hipStream_t s) {
+  const int R = GRAD_A ? p.M : p.K, Cc = GRAD_A ? p.K : p.N;
+  p.tiles_r = ceil_div(R, C::BR);
+  p.tiles_c = ceil_div(Cc, C::BC);
+  const int64_t total = (int64_t)B * p.tiles_r * p.tiles_c;
+  if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
+  hipLaunchKernelGGL((k_log_bwd_exact<C, GRAD_A>), dim3((unsigned)total), dim3(C::NT), 0, s, p);
+  return launch_status();
+}
+
+template <class C, class CX, int NX, bool GRAD_A>
+int launch_bwd_fast(LogBwdArgs p, const float* stats, int B, hipStream_t s) {
+  const int R = GRAD_A ? p.M : p.K, Cc = GRAD_A ? p.K : p.N;
+  p.tiles_r = ceil_div(R, C::BR);
+  p.tiles_c = ceil_div(Cc, C::BC);
+  const int64_t total = (int64_t)B * p.tiles_r * p.tiles_c;
+  if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
+  hipLaunchKernelGGL((k_log_bwd_fast<C, CX, NX, GRAD_A>), dim3((unsigned)total), dim3(C::NT), 0, s,
+                     p, stats);
+  return launch_status();
+}
+
+template <bool GRAD_A>
+int run_bwd(const LogBwdArgs& p, const float* stats, int B, hipStream_t s) {
+  const int R = GRAD_A ? p.M : p.K, Cc = GRAD_A ? p.K : p.N;
+  if ((int64_t)B * R * Cc == 0) return GENBMM_OK;
+  auto wgs = [&](int br, int bc) { return (int64_t)B * ceil_div(R, br) * ceil_div(Cc, bc); };
+  const bool small = R <= 32 && Cc <= 32;
+  const bool big = R >= 128 && Cc >= 128 && wgs(128, 128) >= 512;
+  if (stats) {
+    if (small) return launch_bwd_fast<BCfgSmall, BCfgSmall, 1, GRAD_A>(p, stats, B, s);
+    if (big) return launch_bwd_fast<BCfgBig, BCfgWide, 2, GRAD_A>(p, stats, B, s);
+    return launch_bwd_fast<BCfgMid, BCfgMid, 1, GRAD_A>(p, stats, B, s);
+  }
+  if (small) return launch_bwd_exact<BCfgSmall, GRAD_A>(p, B, s);
+  if (R >= 64 && Cc >= 128 && wgs(64, 128) >= 512) return launch_bwd_exact<BCfgWide, GRAD_A>(p, B, s);
+  return launch_bwd_exact<BCfgMid, GRAD_A>(p, B, s);
+}
+
+}  // namespace
+}  // namespace genbmm
+
+extern "C" {
+
+void genbmm_logbmm_force_exact(int on) { genbmm::g_force_exact.store(on ? 1 : 0); }
+
+int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats, int B, int M,
+                      int K, int N, void* stream) {
+  using namespace genbmm;
+  if (int e = check_dense_dims(B, M, K, N)) return e;
+  const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
+  if (missing(a, mk) || missing(b, kn) || missing(out, mn)) return GENBMM_E_NULLPTR;
+  hipStream_t s = (hipStream_t)stream;
+  if (stats) {
+    if (int e = launch_stats(a, b, stats, B, M, K, N, s)) return e;
+  }
+  if (mn == 0) return GENBMM_OK;
+  DenseArgs p{};
+  p.a = a; p.b = b; p.out = out; p.idx = nullptr;
+  if (stats && K > 0 && !g_force_exact.load()) {
+    if (M <= 32 && N <= 32) return launch_fwd_fast<CfgSmall, CfgSmall, 1>(p, stats, B, M, K, N, s);
+    if (M >= 128 && N >= 128 && (int64_t)B * ceil_div(M, 128) * ceil_div(N, 128) >= 512)
+      return launch_fwd_fast<CfgBig, CfgWide, 2>(p, stats, B, M, K, N, s);
+    return launch_fwd_fast<CfgMid, CfgMid, 1>(p, stats, B, M, K, N, s);
+  }
+  switch (pick_shape(B, M, N, false)) {
+    case kWide: return launch_fwd_exact<CfgWide>(p, B, M, K, N, s);
+    case kMid: return launch_fwd_exact<CfgMid>(p, B, M, K, N, s);
+    default: return launch_fwd_exact<CfgSmall>(p, B, M, K, N, s);
+  }
+}
+
+int genbmm_logbmm_bwd(const float* a, const float* b, const float* out, const float* g,
+                      const float* stats, float* grad_a, float* grad_b, int B, int M, int K,
+                      int N, void* stream) {
+  using namespace genbmm;
+  if (int e = check_dense_dims(B, M, K, N)) return e;
+  const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
+  if (missing(a, mk) || missing(b, kn) || missing(out, mn) || missing(g, mn) ||
+      (missing(grad_a, mk) && missing(grad_b, kn)))
+    return GENBMM_E_NULLPTR;
+  LogBwdArgs p{};
+  p.a = a; p.b = b; p.out = out; p.g = g;
+  p.M = M; p.K = K; p.N = N;
+  p.vec_k = (K % 4 == 0) && aligned16(a) && aligned16(grad_a);
+  p.vec_n = (N % 4 == 0) && aligned16(b) && aligned16(out) && aligned16(g) && aligned16(grad_b);
+  hipStream_t s = (hipStream_t)stream;
+  const float* st = (g_force_exact.load() || mn == 0) ? nullptr : stats;
+  if (grad_a) {
+    p.grad = grad_a;
+    if (int e = run_bwd<true>(p, st, B, s)) return e;
+  }
+  if (grad_b) {
+    p.grad = grad_b;
+    if (int e = run_bwd<false>(p, st, B, s)) return e;
+  }
+  return GENBMM_OK;
+}
+
+}  // extern "C"

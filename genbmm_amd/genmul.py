@@ -9,7 +9,9 @@ Differences in mechanism (not in results):
   * logbmm's backward produces grad_a and grad_b from one library call that
     reads every operand in place; the reference calls its kernel twice and
     transposes b, a, g, out, maxes and the result in between (genmul.py:35-41).
-  * no `maxes` tensor is saved: exp(a+b-mx)/exp(out-mx) == exp(a+b-out).
+  * instead of the (B, M, N) `maxes` tensor the forward saves a (B, M + N) vector of
+    row maxima of a and column maxima of b, which lets forward and backward factor
+    exp(a + b) wherever that is exact (see csrc/logbmm.hip).
   * the arg-max / sample index stays int32 into the backward; the reference
     converts it (and a, b, g) to float first (genmul.py:62-65).
   * samplebmm draws its uniforms from a counter-based Philox4x32-10 stream
@@ -57,12 +59,12 @@ class _LogBmmGrad(torch.autograd.Function):
     """
 
     @staticmethod
-    def forward(ctx, a, b, g, out):
+    def forward(ctx, a, b, g, out, stats):
         B, M, K, N = _lib.dense_dims(a, b)
         grad_a = torch.empty_like(a)
         grad_b = torch.empty_like(b)
         _call("genbmm_logbmm_bwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g),
-              _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
+              _lib.ptr(stats), _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
         ctx.save_for_backward(a, b, g, out)
         ctx.set_materialize_grads(False)
         return grad_a, grad_b
@@ -70,7 +72,7 @@ class _LogBmmGrad(torch.autograd.Function):
     @staticmethod
     def backward(ctx, u_a, u_b):
         if u_a is None and u_b is None:
-            return None, None, None, None
+            return None, None, None, None, None
         a, b, g, out = ctx.saved_tensors
         B, M, K, N = _lib.dense_dims(a, b)
         u_a = None if u_a is None else u_a.contiguous()
@@ -80,7 +82,7 @@ class _LogBmmGrad(torch.autograd.Function):
         gg = torch.empty_like(g)
         _call("genbmm_logbmm_bwdbwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g),
               _lib.ptr(u_a), _lib.ptr(u_b), _lib.ptr(ga), _lib.ptr(gb), _lib.ptr(gg), B, M, K, N)
-        return ga, gb, gg, None
+        return ga, gb, gg, None, None
 
 
 class LogMatMul(torch.autograd.Function):
@@ -91,15 +93,18 @@ class LogMatMul(torch.autograd.Function):
         in_dtype = a.dtype if isinstance(a, torch.Tensor) else None
         a, b, (B, M, K, N) = _prep(a, b)
         out = torch.empty(B, M, N, dtype=_COMPUTE, device=a.device)
-        _call("genbmm_logbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), B, M, K, N)
-        ctx.save_for_backward(a, b, out)
+        # row maxima of a, column maxima of b: what the reference's `maxes` becomes
+        stats = torch.empty(B, M + N, dtype=_COMPUTE, device=a.device)
+        _call("genbmm_logbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(stats),
+              B, M, K, N)
+        ctx.save_for_backward(a, b, out, stats)
         ctx.in_dtype = in_dtype
         return out.to(in_dtype)
 
     @staticmethod
     def backward(ctx, grad_output):
-        a, b, out = ctx.saved_tensors
-        grad_a, grad_b = _LogBmmGrad.apply(a, b, grad_output.to(_COMPUTE).contiguous(), out)
+        a, b, out, stats = ctx.saved_tensors
+        grad_a, grad_b = _LogBmmGrad.apply(a, b, grad_output.to(_COMPUTE).contiguous(), out, stats)
         return grad_a.to(ctx.in_dtype), grad_b.to(ctx.in_dtype)
 
 

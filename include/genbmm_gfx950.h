@@ -19,7 +19,8 @@
  *     legacy default stream);
  *   - return value: 0 = enqueued; < 0 = argument error (GENBMM_E_*);
  *     > 0 = the hipError_t reported by the launch;
- *   - no global state; calls are re-entrant and thread safe.
+ *   - calls are re-entrant and thread safe; the only global state is the
+ *     switch genbmm_logbmm_force_exact().
  *
  * Dense operands: a is (B, M, K), b is (B, K, N), results are (B, M, N).
  * Banded operands: band data is (B, n, W) with W = lu + ld + 1 and
@@ -58,11 +59,18 @@ const char* genbmm_error_string(int code);
  * out[b,m,n] = log sum_k exp(a[b,m,k] + b[b,k,n]).
  * Replaces _genbmm.forward(a, b, 0): matmul_cuda.cpp:69-77 ->
  * matmul_cuda_forward mode 0 (matmul_cuda_kernel.cu:465-497, kernel :13-45).
- * The reference's second output `maxes` is not produced: the backward below
- * does not need it.  The running maximum starts at -1e9 as in the reference
- * (kernel :31), so an output whose terms are all <= -1e9 is -inf.
+ * The running maximum starts at -1e9 as in the reference (kernel :31), so an
+ * output whose terms are all <= -1e9 is -inf.
+ *
+ * `stats` is an optional (B, M + N) fp32 buffer.  NULL: the online
+ * (running-max) log-sum-exp kernel runs.  Non-NULL: it receives, per batch
+ * item, max_k a[m,k] for every m followed by max_k b[k,n] for every n, and the
+ * forward uses them to factor exp(a+b) = exp(a-max)*exp(b-max) wherever that
+ * is exact to fp32 (tiles where it is not are recomputed by the online
+ * kernel's routine).  It takes the place of the reference's (B, M, N) `maxes`
+ * output; pass the same buffer to genbmm_logbmm_bwd.
  */
-int genbmm_logbmm_fwd(const float* a, const float* b, float* out,
+int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats,
                       int B, int M, int K, int N, void* stream);
 
 /*
@@ -72,10 +80,20 @@ int genbmm_logbmm_fwd(const float* a, const float* b, float* out,
  * LogMatMul.backward (genmul.py:35-41; matmul_cuda.cpp:79-92;
  * matmul_cuda_kernel.cu:625-664, kernel :159-184).
  * grad_a or grad_b may be NULL (that gradient is then not computed), not both.
+ * `stats`: NULL, or the buffer genbmm_logbmm_fwd filled for the same (a, b).
  */
 int genbmm_logbmm_bwd(const float* a, const float* b, const float* out,
-                      const float* g, float* grad_a, float* grad_b,
+                      const float* g, const float* stats,
+                      float* grad_a, float* grad_b,
                       int B, int M, int K, int N, void* stream);
+
+/*
+ * Process-wide switch for tests and measurements: non-zero makes
+ * genbmm_logbmm_fwd / _bwd ignore `stats` and always run the online / exact
+ * kernels.  The only piece of global state in the library; default 0.
+ * No counterpart in the reference.
+ */
+void genbmm_logbmm_force_exact(int on);
 
 /*
  * Second-order terms of logbmm: the gradients with respect to (a, b, g) of

@@ -35,12 +35,22 @@ def lse64(a, b, chunk=4):
     return torch.cat(outs) if outs else a.new_zeros((0, a.shape[1], b.shape[2])).double()
 
 
+@pytest.fixture(params=["factored", "exact"])
+def path(request, gpu):
+    """Run a logbmm test on both code paths: the factored kernels (default) and the
+    online/exact kernels alone."""
+    lib = _lib.load()
+    lib.genbmm_logbmm_force_exact(1 if request.param == "exact" else 0)
+    yield request.param
+    lib.genbmm_logbmm_force_exact(0)
+
+
 SHAPES = [(16, 64, 64, 64), (3, 7, 9, 5), (2, 1, 1, 1), (4, 5, 1, 6), (5, 33, 70, 129), (2, 130, 17, 66),
           (3, 64, 64, 128), (2, 200, 96, 260), (9, 32, 32, 32), (7, 31, 33, 29), (1, 256, 40, 256)]
 
 
 @pytest.mark.parametrize("B,M,K,N", SHAPES)
-def test_logbmm_forward_and_grads(gpu, B, M, K, N):
+def test_logbmm_forward_and_grads(gpu, path, B, M, K, N):
     torch.manual_seed(B * 1000 + M)
     a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
     want, wa, wb = oracle.logbmm_grads64(a, b, g)
@@ -55,7 +65,7 @@ def test_logbmm_forward_and_grads(gpu, B, M, K, N):
     close(gb.sum(-2), g.double().sum(-2), atol=1e-4)
 
 
-def test_logbmm_config_c1_uniform_ones(gpu):
+def test_logbmm_config_c1_uniform_ones(gpu, path):
     """BASELINE config 0: seed 0, Uniform[0,1) (16,64,64), grad_out = ones."""
     torch.manual_seed(0)
     a, b = torch.rand(16, 64, 64), torch.rand(16, 64, 64)
@@ -71,7 +81,7 @@ def test_logbmm_config_c1_uniform_ones(gpu):
     close(out, oracle.seq_logbmm_fwd(a, b)[0])
 
 
-def test_logbmm_special_values(gpu):
+def test_logbmm_special_values(gpu, path):
     a, b = torch.randn(2, 5, 6), torch.randn(2, 6, 4)
     b[0, 2, :] = -math.inf          # masked k
     a[1, 3, :] = -math.inf          # fully masked row -> -inf
@@ -89,7 +99,7 @@ def test_logbmm_special_values(gpu):
 
 
 @pytest.mark.parametrize("B,M,K,N,sub", [(512, 128, 128, 128, 8), (8192, 32, 32, 32, 256), (64, 512, 512, 512, 1)])
-def test_logbmm_baseline_shapes(gpu, B, M, K, N, sub):
+def test_logbmm_baseline_shapes(gpu, path, B, M, K, N, sub):
     """BASELINE configs 1 and the headline shape: full-size run, float64 check on a
     batch subset plus the size-independent row-sum invariants on everything."""
     torch.manual_seed(0)
@@ -107,6 +117,41 @@ def test_logbmm_baseline_shapes(gpu, B, M, K, N, sub):
     # out >= max_k(a+b) and out <= max + log K
     mx = genbmm.maxbmm(ad.detach(), bd.detach())
     assert bool((out >= mx - 1e-5).all()) and bool((out <= mx + math.log(K) + 1e-5).all())
+
+
+@pytest.mark.parametrize("B,M,K,N", [(2, 40, 48, 36), (3, 130, 64, 140), (2, 256, 32, 256), (5, 32, 32, 32)])
+def test_logbmm_factoring_guard(gpu, B, M, K, N):
+    """Inputs for which exp(a - rowmax) * exp(b - colmax) underflows although the true
+    terms do not: the factored kernels must detect it per tile and fall back."""
+    torch.manual_seed(B + M)
+    a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
+    # every second row of a peaks at k = 0 while b's row 0 is 200 below the rest
+    a[:, ::2, 0] += 200.0
+    b[:, 0, :] -= 200.0
+    # one batch item carries -2e9 masks on disjoint halves of k: every term is below the
+    # -1e9 floor -> -inf (matmul_cuda_kernel.cu:31-41)
+    a[-1, :, ::2] = -2e9
+    b[-1, 1::2, :] = -2e9
+    want, wa, wb = oracle.logbmm_grads64(a[:-1], b[:-1], g[:-1])
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    out = genbmm.logbmm(ad, bd)
+    close(out[:-1], want)
+    ref32, _ = oracle.seq_logbmm_fwd(a[-1:], b[-1:])
+    assert bool(torch.isinf(ref32).all()) and bool(torch.isinf(out[-1]).all())
+    ga, gb = torch.autograd.grad(out[:-1].sum() * 0 + (out[:-1] * g[:-1].to(gpu)).sum(), (ad, bd))
+    close(ga[:-1], wa)
+    close(gb[:-1], wb)
+    # the two paths agree with each other on these inputs as well
+    lib = _lib.load()
+    lib.genbmm_logbmm_force_exact(1)
+    try:
+        out2 = genbmm.logbmm(ad, bd)
+        ga2, gb2 = torch.autograd.grad((out2[:-1] * g[:-1].to(gpu)).sum(), (ad, bd))
+    finally:
+        lib.genbmm_logbmm_force_exact(0)
+    close(out2[:-1], want)
+    close(ga2[:-1], wa)
+    close(gb2[:-1], wb)
 
 
 @pytest.mark.parametrize("B,M,K,N", [(2, 4, 5, 3), (3, 9, 12, 7), (2, 33, 20, 40)])
@@ -334,8 +379,8 @@ def test_errors(gpu):
     lib = _lib.load()
     null = ctypes.c_void_p(0)
     ad = a.to(gpu)
-    assert lib.genbmm_logbmm_fwd(null, _lib.ptr(ad), _lib.ptr(ad), 1, 1, 1, 1, null) == -1
-    assert lib.genbmm_logbmm_fwd(_lib.ptr(ad), _lib.ptr(ad), _lib.ptr(ad), 1, -1, 1, 1, null) == -2
+    assert lib.genbmm_logbmm_fwd(null, _lib.ptr(ad), _lib.ptr(ad), null, 1, 1, 1, 1, null) == -1
+    assert lib.genbmm_logbmm_fwd(_lib.ptr(ad), _lib.ptr(ad), _lib.ptr(ad), null, 1, -1, 1, 1, null) == -2
     assert lib.genbmm_banded_fwd(_lib.ptr(ad), 0, 0, _lib.ptr(ad), 0, 0, _lib.ptr(ad), null, 1, 1, 2, null) == -3
     assert lib.genbmm_banded_fwd(_lib.ptr(ad), -1, 0, _lib.ptr(ad), 0, 0, _lib.ptr(ad), null, 1, 1, 0, null) == -4
     assert b"NULL" in lib.genbmm_error_string(-1)
