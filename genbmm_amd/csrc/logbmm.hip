@@ -29,10 +29,18 @@
 namespace genbmm {
 namespace {
 
+#ifndef GENBMM_WPE
+#define GENBMM_WPE 2
+#endif
 constexpr float kLog2eLo = 1.92596299e-8f;  // log2(e) - (float)log2(e)
 constexpr float kGuardBits = 40.f;          // factored path needs S >= 2^-40
 
-// exp(d) through v_exp_f32 with the rounding error of d*log2e compensated.
+// exp(d) for staged tile elements: one multiply and v_exp_f32.  The rounding of
+// d*log2e costs |d| * 6e-8 relative; terms that matter have |d| < ~28 (guard).
+__device__ __forceinline__ float exp_stage(float d) { return fast_exp2(d * kLog2e); }
+
+// exp(d) through v_exp_f32 with the rounding error of d*log2e compensated
+// (used once per output element).
 __device__ __forceinline__ float exp_comp(float d) {
   const float hi = d * kLog2e;
   const float lo = __builtin_fmaf(d, kLog2e, -hi) + d * kLog2eLo;
@@ -125,7 +133,7 @@ __global__ __launch_bounds__(C::NT) void k_log_bwd_exact(const LogBwdArgs p) {
 // C: tile of the factored pass; CX: tile of the exact routine used for the
 // recompute, covering the same BN and NX * CX::BM = C::BM rows.
 template <class C, class CX, int NX>
-__global__ __launch_bounds__(C::NT) void k_log_fwd_fast(const DenseArgs p,
+__global__ __launch_bounds__(C::NT) __attribute__((amdgpu_waves_per_eu(GENBMM_WPE, GENBMM_WPE))) void k_log_fwd_fast(const DenseArgs p,
                                                         const float* __restrict__ stats) {
   static_assert(CX::BN == C::BN && CX::BM * NX == C::BM && CX::NT == C::NT && CX::KT <= C::KT, "");
   __shared__ __attribute__((aligned(16))) float smem[C::KT * (C::LDA + C::LDB) + C::BM + C::BN];
@@ -163,14 +171,14 @@ __global__ __launch_bounds__(C::NT) void k_log_fwd_fast(const DenseArgs p,
 #pragma unroll
     for (int l = 0; l < TA::PER; ++l) {  // EA = exp(a - alpha[row])
       const float s = al[((tid + l * C::NT) / TA::C4) % C::BM];
-      ta.r[l].x = exp_comp(ta.r[l].x - s); ta.r[l].y = exp_comp(ta.r[l].y - s);
-      ta.r[l].z = exp_comp(ta.r[l].z - s); ta.r[l].w = exp_comp(ta.r[l].w - s);
+      ta.r[l].x = exp_stage(ta.r[l].x - s); ta.r[l].y = exp_stage(ta.r[l].y - s);
+      ta.r[l].z = exp_stage(ta.r[l].z - s); ta.r[l].w = exp_stage(ta.r[l].w - s);
     }
 #pragma unroll
     for (int l = 0; l < TB::PER; ++l) {  // EB = exp(b - beta[col])
       const float4 s = *reinterpret_cast<const float4*>(be + ((tid + l * C::NT) % TB::C4) * 4);
-      tb.r[l].x = exp_comp(tb.r[l].x - s.x); tb.r[l].y = exp_comp(tb.r[l].y - s.y);
-      tb.r[l].z = exp_comp(tb.r[l].z - s.z); tb.r[l].w = exp_comp(tb.r[l].w - s.w);
+      tb.r[l].x = exp_stage(tb.r[l].x - s.x); tb.r[l].y = exp_stage(tb.r[l].y - s.y);
+      tb.r[l].z = exp_stage(tb.r[l].z - s.z); tb.r[l].w = exp_stage(tb.r[l].w - s.w);
     }
     ta.sstore(As, tid);
     tb.sstore(Bs, tid);
@@ -190,7 +198,7 @@ __global__ __launch_bounds__(C::NT) void k_log_fwd_fast(const DenseArgs p,
         for (int j = 0; j < C::TN; ++j) acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
     };
     if (kn == C::KT) {
-#pragma unroll
+#pragma unroll 2
       for (int kk = 0; kk < C::KT; ++kk) step(kk);
     } else {
       for (int kk = 0; kk < kn; ++kk) step(kk);
@@ -232,7 +240,7 @@ __global__ __launch_bounds__(C::NT) void k_log_fwd_fast(const DenseArgs p,
 // H = g*exp(alpha+beta-out), staged from out and g; X = the operand shaped like
 // the output, read once in the epilogue.
 template <class C, class CX, int NX, bool GRAD_A>
-__global__ __launch_bounds__(C::NT) void k_log_bwd_fast(const LogBwdArgs p,
+__global__ __launch_bounds__(C::NT) __attribute__((amdgpu_waves_per_eu(GENBMM_WPE, GENBMM_WPE))) void k_log_bwd_fast(const LogBwdArgs p,
                                                         const float* __restrict__ stats) {
   constexpr int BY = GRAD_A ? C::BC : C::BR;
   constexpr int BO = GRAD_A ? C::BR : C::BC;
@@ -312,8 +320,8 @@ __global__ __launch_bounds__(C::NT) void k_log_bwd_fast(const LogBwdArgs p,
         const float4 bq = make_float4(safe(be, n, N), safe(be, n + 1, N), safe(be, n + 2, N), safe(be, n + 3, N));
 #pragma unroll
         for (int l = 0; l < TYt::PER; ++l) {
-          tyl.r[l].x = exp_comp(tyl.r[l].x - bq.x); tyl.r[l].y = exp_comp(tyl.r[l].y - bq.y);
-          tyl.r[l].z = exp_comp(tyl.r[l].z - bq.z); tyl.r[l].w = exp_comp(tyl.r[l].w - bq.w);
+          tyl.r[l].x = exp_stage(tyl.r[l].x - bq.x); tyl.r[l].y = exp_stage(tyl.r[l].y - bq.y);
+          tyl.r[l].z = exp_stage(tyl.r[l].z - bq.z); tyl.r[l].w = exp_stage(tyl.r[l].w - bq.w);
         }
 #pragma unroll
         for (int l = 0; l < TOt::PER; ++l) {
@@ -326,8 +334,8 @@ __global__ __launch_bounds__(C::NT) void k_log_bwd_fast(const LogBwdArgs p,
             if (n + 2 < N && !(ez <= lim)) bad = 1;
             if (n + 3 < N && !(ew <= lim)) bad = 1;
           }
-          tol.r[l].x = tgl.r[l].x * exp_comp(ex); tol.r[l].y = tgl.r[l].y * exp_comp(ey);
-          tol.r[l].z = tgl.r[l].z * exp_comp(ez); tol.r[l].w = tgl.r[l].w * exp_comp(ew);
+          tol.r[l].x = tgl.r[l].x * exp_stage(ex); tol.r[l].y = tgl.r[l].y * exp_stage(ey);
+          tol.r[l].z = tgl.r[l].z * exp_stage(ez); tol.r[l].w = tgl.r[l].w * exp_stage(ew);
         }
       }
     } else {
@@ -335,8 +343,8 @@ __global__ __launch_bounds__(C::NT) void k_log_bwd_fast(const LogBwdArgs p,
 #pragma unroll
       for (int l = 0; l < TYt::PER; ++l) {
         const float s = safe(al, q0 + (tid + l * C::NT) / TYt::C4, M);
-        tyl.r[l].x = exp_comp(tyl.r[l].x - s); tyl.r[l].y = exp_comp(tyl.r[l].y - s);
-        tyl.r[l].z = exp_comp(tyl.r[l].z - s); tyl.r[l].w = exp_comp(tyl.r[l].w - s);
+        tyl.r[l].x = exp_stage(tyl.r[l].x - s); tyl.r[l].y = exp_stage(tyl.r[l].y - s);
+        tyl.r[l].z = exp_stage(tyl.r[l].z - s); tyl.r[l].w = exp_stage(tyl.r[l].w - s);
       }
 #pragma unroll
       for (int l = 0; l < TOt::PER; ++l) {
@@ -351,8 +359,8 @@ __global__ __launch_bounds__(C::NT) void k_log_bwd_fast(const LogBwdArgs p,
           if (n + 2 < N && !(ez <= lim)) bad = 1;
           if (n + 3 < N && !(ew <= lim)) bad = 1;
         }
-        tol.r[l].x = tgl.r[l].x * exp_comp(ex); tol.r[l].y = tgl.r[l].y * exp_comp(ey);
-        tol.r[l].z = tgl.r[l].z * exp_comp(ez); tol.r[l].w = tgl.r[l].w * exp_comp(ew);
+        tol.r[l].x = tgl.r[l].x * exp_stage(ex); tol.r[l].y = tgl.r[l].y * exp_stage(ey);
+        tol.r[l].z = tgl.r[l].z * exp_stage(ez); tol.r[l].w = tgl.r[l].w * exp_stage(ew);
       }
     }
     tyl.sstore(Ys, tid);
@@ -380,7 +388,7 @@ __global__ __launch_bounds__(C::NT) void k_log_bwd_fast(const LogBwdArgs p,
       }
     };
     if (qn == C::RT) {
-#pragma unroll
+#pragma unroll 2
       for (int qq = 0; qq < C::RT; ++qq) step(qq);
     } else {
       for (int qq = 0; qq < qn; ++qq) step(qq);
