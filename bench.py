@@ -85,7 +85,7 @@ def main():
     g = torch.randn(B, M, N).to(dev)
     out = torch.empty(B, M, N, device=dev)
     ga, gb = torch.empty_like(a), torch.empty_like(b)
-    stats = torch.empty(B, M + N, device=dev)
+    stats = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=dev)
     stream = _lib.stream_of(a)
     p = _lib.ptr
     null = p(None)

@@ -43,6 +43,7 @@ SIGNATURES = {
 }
 STRING_FUNCS = {"genbmm_version": [], "genbmm_error_string": [_i]}
 VOID_FUNCS = {"genbmm_logbmm_force_exact": [_i]}
+SIZE_FUNCS = {"genbmm_logbmm_stats_size": [_i, _i, _i, _i]}
 
 _lib = None
 
@@ -72,6 +73,10 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = argtypes
         fn.restype = None
+    for name, argtypes in SIZE_FUNCS.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = ctypes.c_size_t
     _lib = lib
     return lib
 

@@ -18,20 +18,24 @@
 // below 2^-86 of the result, i.e. invisible in fp32.  Each workgroup checks that
 // condition for its own tile (forward: on S; backward: on alpha+beta-out while
 // staging H) and, if any cell fails it - or is NaN/inf, or sits at the
-// reference's -1e9 floor - recomputes the whole tile with the exact kernel's
-// routine (online running-max log-sum-exp forward, exp(a+b-out) backward), so
-// the result never depends on the factoring being applicable.
+// reference's -1e9 floor - raises that tile's flag instead of storing; a fix-up
+// kernel launched right behind recomputes exactly the flagged tiles with the
+// exact kernel's routine (online running-max log-sum-exp forward, exp(a+b-out)
+// backward), so the result never depends on the factoring being applicable.
+// The flags live behind the shifts in the caller's `stats` buffer.
+//
+// Two implementations of the factored contraction: v_fma_f32 on register blocks
+// (any shape, this file) and the fp32 matrix-core instruction for problems made
+// of full 128x128 tiles (logbmm_mfma.h).
 #include <atomic>
 
 #include "dense_tiles.h"
 #include "log_bwd_tile.h"
+#include "logbmm_mfma.h"
 
 namespace genbmm {
 namespace {
 
-#ifndef GENBMM_WPE
-#define GENBMM_WPE 2
-#endif
 constexpr float kLog2eLo = 1.92596299e-8f;  // log2(e) - (float)log2(e)
 constexpr float kGuardBits = 40.f;          // factored path needs S >= 2^-40
 
@@ -130,12 +134,10 @@ __global__ __launch_bounds__(C::NT) void k_log_bwd_exact(const LogBwdArgs p) {
 }
 
 // --------------------------------------------------------- factored forward
-// C: tile of the factored pass; CX: tile of the exact routine used for the
-// recompute, covering the same BN and NX * CX::BM = C::BM rows.
-template <class C, class CX, int NX>
-__global__ __launch_bounds__(C::NT) __attribute__((amdgpu_waves_per_eu(GENBMM_WPE, GENBMM_WPE))) void k_log_fwd_fast(const DenseArgs p,
-                                                        const float* __restrict__ stats) {
-  static_assert(CX::BN == C::BN && CX::BM * NX == C::BM && CX::NT == C::NT && CX::KT <= C::KT, "");
+template <class C>
+__global__ __launch_bounds__(C::NT, 2) void k_log_fwd_fast(const DenseArgs p,
+                                                           const float* __restrict__ stats,
+                                                           int* __restrict__ flags) {
   __shared__ __attribute__((aligned(16))) float smem[C::KT * (C::LDA + C::LDB) + C::BM + C::BN];
   float* As = smem;
   float* Bs = As + C::KT * C::LDA;
@@ -219,19 +221,57 @@ __global__ __launch_bounds__(C::NT) __attribute__((amdgpu_waves_per_eu(GENBMM_WP
       const float s = acc[i][j];
       const bool ok = (s >= thr) && (s < INFINITY) && (shift > 0.9f * kFloor) && (shift < INFINITY);
       if (!ok && m0 + r < M && n0 + c < N) bad = 1;
-      acc[i][j] = logf(s) + shift;
+      acc[i][j] = __builtin_fmaf(fast_log2(s), kLn2, shift);  // v_log_f32
     }
   }
-  if (__syncthreads_or(bad)) {
+  bad = __syncthreads_or(bad);
+  if (tid == 0) flags[blockIdx.x] = bad;
+  if (bad) return;  // the fix-up launch recomputes this tile
+  store_tile_f<C>(p.out + (long)batch * M * N, acc, m0, n0, M, N, p.vec_o, tx, ty);
+}
+
+// Recompute the flagged tiles of a factored forward launch with the online
+// routine.  FBM x FBN is the factored launch's tile, CX the exact routine's
+// tile (CX::BN == FBN, NX * CX::BM == FBM).  Workgroups stride over the tile list.
+template <class CX, int NX, int FBM, int FBN>
+__global__ __launch_bounds__(CX::NT) void k_log_fwd_fixup(const DenseArgs p,
+                                                          const int* __restrict__ flags,
+                                                          int total_tiles) {
+  static_assert(CX::BN == FBN && CX::BM * NX == FBM, "");
+  __shared__ __attribute__((aligned(16))) float smem[CX::KT * (CX::LDA + CX::LDB)];
+  const int per = p.tiles_m * p.tiles_n;  // of the factored launch
+  for (int t = blockIdx.x; t < total_tiles; t += gridDim.x) {
+    if (!flags[t]) continue;
+    const int batch = t / per, r = t - batch * per;
+    const int m0 = (r / p.tiles_n) * FBM, n0 = (r % p.tiles_n) * FBN;
 #pragma unroll
     for (int h = 0; h < NX; ++h)
-      if (m0 + h * CX::BM < M) {
+      if (m0 + h * CX::BM < p.M) {
         log_fwd_tile<CX, false>(p, batch, m0 + h * CX::BM, n0, smem, smem + CX::KT * CX::LDA);
         __syncthreads();
       }
-    return;
   }
-  store_tile_f<C>(p.out + (long)batch * M * N, acc, m0, n0, M, N, p.vec_o, tx, ty);
+}
+
+template <class CX, int NX, int FBR, int FBC, bool GRAD_A>
+__global__ __launch_bounds__(CX::NT) void k_log_bwd_fixup(const LogBwdArgs p,
+                                                          const int* __restrict__ flags,
+                                                          int total_tiles) {
+  static_assert(CX::BC == FBC && CX::BR * NX == FBR, "");
+  __shared__ __attribute__((aligned(16))) float smem[LogBwdLds<CX, GRAD_A>::FLOATS];
+  const int per = p.tiles_r * p.tiles_c;  // of the factored launch
+  const int R = GRAD_A ? p.M : p.K;
+  for (int t = blockIdx.x; t < total_tiles; t += gridDim.x) {
+    if (!flags[t]) continue;
+    const int batch = t / per, r = t - batch * per;
+    const int r0 = (r / p.tiles_c) * FBR, c0 = (r % p.tiles_c) * FBC;
+#pragma unroll
+    for (int h = 0; h < NX; ++h)
+      if (r0 + h * CX::BR < R) {
+        log_bwd_tile<CX, GRAD_A>(p, batch, r0 + h * CX::BR, c0, smem);
+        __syncthreads();
+      }
+  }
 }
 
 // -------------------------------------------------------- factored backward
@@ -239,17 +279,16 @@ __global__ __launch_bounds__(C::NT) __attribute__((amdgpu_waves_per_eu(GENBMM_WP
 // reduction index q is n or m.  Y = the other operand, staged as exp(y - shift);
 // H = g*exp(alpha+beta-out), staged from out and g; X = the operand shaped like
 // the output, read once in the epilogue.
-template <class C, class CX, int NX, bool GRAD_A>
-__global__ __launch_bounds__(C::NT) __attribute__((amdgpu_waves_per_eu(GENBMM_WPE, GENBMM_WPE))) void k_log_bwd_fast(const LogBwdArgs p,
-                                                        const float* __restrict__ stats) {
+template <class C, bool GRAD_A>
+__global__ __launch_bounds__(C::NT, 2) void k_log_bwd_fast(const LogBwdArgs p,
+                                                           const float* __restrict__ stats,
+                                                           int* __restrict__ flags) {
   constexpr int BY = GRAD_A ? C::BC : C::BR;
   constexpr int BO = GRAD_A ? C::BR : C::BC;
   using TYt = std::conditional_t<GRAD_A, TileOutMajor<BY, C::RT, C::NT>, TileRedMajor<BY, C::RT, C::NT>>;
   using TOt = std::conditional_t<GRAD_A, TileOutMajor<BO, C::RT, C::NT>, TileRedMajor<BO, C::RT, C::NT>>;
   constexpr int LDY = BY + kPad, LDO = BO + kPad;
-  constexpr int FAST_FLOATS = C::RT * (LDY + LDO);
-  constexpr int EXACT_FLOATS = LogBwdLds<CX, GRAD_A>::FLOATS;
-  __shared__ __attribute__((aligned(16))) float smem[FAST_FLOATS > EXACT_FLOATS ? FAST_FLOATS : EXACT_FLOATS];
+  __shared__ __attribute__((aligned(16))) float smem[C::RT * (LDY + LDO)];
   float* Ys = smem;
   float* Hs = smem + C::RT * LDY;
 
@@ -395,15 +434,9 @@ __global__ __launch_bounds__(C::NT) __attribute__((amdgpu_waves_per_eu(GENBMM_WP
     }
   }
 
-  if (__syncthreads_or(bad)) {
-#pragma unroll
-    for (int h = 0; h < NX; ++h)
-      if (r0 + h * CX::BR < R) {
-        log_bwd_tile<CX, GRAD_A>(p, batch, r0 + h * CX::BR, c0, smem);
-        __syncthreads();
-      }
-    return;
-  }
+  bad = __syncthreads_or(bad);
+  if (tid == 0) flags[blockIdx.x] = bad;
+  if (bad) return;  // the fix-up launch recomputes this tile
 
   // epilogue: grad = exp(x - shift) * acc, x re-read from global memory
   float* gradb = p.grad + (long)batch * R * Cc;
@@ -445,7 +478,19 @@ __global__ __launch_bounds__(C::NT) __attribute__((amdgpu_waves_per_eu(GENBMM_WP
 }
 
 // ----------------------------------------------------------------- dispatch
-std::atomic<int> g_force_exact{0};
+std::atomic<int> g_path{0};  // 0 default, 1 exact only, 2 factored without matrix cores
+constexpr int kFixupGrid = 1024;
+
+// Layout of the caller's stats buffer: B*(M+N) shifts, then one int flag per
+// 32x32 tile of (M,N), of (M,K) and of (K,N) (an upper bound on any launch's
+// tile count).
+inline int64_t tiles32(int B, int X, int Y) { return (int64_t)B * ceil_div(X, 32) * ceil_div(Y, 32); }
+inline int* flags_of(const float* stats, int B, int M, int K, int N, int which) {
+  int* f = reinterpret_cast<int*>(const_cast<float*>(stats) + (int64_t)B * (M + N));
+  if (which >= 1) f += tiles32(B, M, N);
+  if (which >= 2) f += tiles32(B, M, K);
+  return f;
+}
 
 template <class C>
 int launch_fwd_exact(DenseArgs p, int B, int M, int K, int N, hipStream_t s) {
@@ -455,12 +500,31 @@ int launch_fwd_exact(DenseArgs p, int B, int M, int K, int N, hipStream_t s) {
   return launch_status();
 }
 
+template <class CX, int NX, int FBM, int FBN>
+int launch_fwd_fixup(const DenseArgs& p, const int* flags, int tiles, hipStream_t s) {
+  hipLaunchKernelGGL((k_log_fwd_fixup<CX, NX, FBM, FBN>), dim3(min(tiles, kFixupGrid)),
+                     dim3(CX::NT), 0, s, p, flags, tiles);
+  return launch_status();
+}
+
 template <class C, class CX, int NX>
-int launch_fwd_fast(DenseArgs p, const float* stats, int B, int M, int K, int N, hipStream_t s) {
+int launch_fwd_fast(DenseArgs p, const float* stats, int* flags, int B, int M, int K, int N,
+                    hipStream_t s) {
   dim3 grid;
   if (int e = fill_args<C>(p, B, M, K, N, grid)) return e;
-  hipLaunchKernelGGL((k_log_fwd_fast<C, CX, NX>), grid, dim3(C::NT), 0, s, p, stats);
-  return launch_status();
+  hipLaunchKernelGGL((k_log_fwd_fast<C>), grid, dim3(C::NT), 0, s, p, stats, flags);
+  if (int e = launch_status()) return e;
+  return launch_fwd_fixup<CX, NX, C::BM, C::BN>(p, flags, (int)grid.x, s);
+}
+
+int launch_fwd_mfma(DenseArgs p, const float* stats, int* flags, int B, int M, int K, int N,
+                    hipStream_t s) {
+  dim3 grid;
+  if (int e = fill_args<CfgBig>(p, B, M, K, N, grid)) return e;
+  hipLaunchKernelGGL(k_log_fwd_mfma, grid, dim3(256), 0, s, p.a, p.b, p.out, stats, flags, M, K, N,
+                     p.tiles_m, p.tiles_n);
+  if (int e = launch_status()) return e;
+  return launch_fwd_fixup<CfgWide, 2, 128, 128>(p, flags, (int)grid.x, s);
 }
 
 int launch_stats(const float* a, const float* b, float* stats, int B, int M, int K, int N,
@@ -486,29 +550,46 @@ int launch_bwd_exact(LogBwdArgs p, int B, hipStream_t s) {
   return launch_status();
 }
 
-template <class C, class CX, int NX, bool GRAD_A>
-int launch_bwd_fast(LogBwdArgs p, const float* stats, int B, hipStream_t s) {
+template <class C, class CX, int NX, bool GRAD_A, bool MFMA>
+int launch_bwd_fast(LogBwdArgs p, const float* stats, int* flags, int B, hipStream_t s) {
   const int R = GRAD_A ? p.M : p.K, Cc = GRAD_A ? p.K : p.N;
   p.tiles_r = ceil_div(R, C::BR);
   p.tiles_c = ceil_div(Cc, C::BC);
   const int64_t total = (int64_t)B * p.tiles_r * p.tiles_c;
   if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
-  hipLaunchKernelGGL((k_log_bwd_fast<C, CX, NX, GRAD_A>), dim3((unsigned)total), dim3(C::NT), 0, s,
-                     p, stats);
+  if (MFMA)
+    hipLaunchKernelGGL((k_log_bwd_mfma<GRAD_A>), dim3((unsigned)total), dim3(256), 0, s, p.a, p.b,
+                       p.out, p.g, stats, p.grad, flags, p.M, p.K, p.N, p.tiles_r, p.tiles_c);
+  else
+    hipLaunchKernelGGL((k_log_bwd_fast<C, GRAD_A>), dim3((unsigned)total), dim3(C::NT), 0, s, p,
+                       stats, flags);
+  if (int e = launch_status()) return e;
+  hipLaunchKernelGGL((k_log_bwd_fixup<CX, NX, C::BR, C::BC, GRAD_A>),
+                     dim3(min((int)total, kFixupGrid)), dim3(CX::NT), 0, s, p, flags, (int)total);
   return launch_status();
+}
+
+// All tiles full and every access 16-byte aligned: the matrix-core kernels apply.
+inline bool mfma_ok(int out_r, int out_c, int red, bool aligned, int64_t tiles) {
+  return g_path.load() == 0 && aligned && red > 0 && out_r % 128 == 0 && out_c % 128 == 0 &&
+         red % 16 == 0 && tiles >= 128;
 }
 
 template <bool GRAD_A>
 int run_bwd(const LogBwdArgs& p, const float* stats, int B, hipStream_t s) {
-  const int R = GRAD_A ? p.M : p.K, Cc = GRAD_A ? p.K : p.N;
+  const int R = GRAD_A ? p.M : p.K, Cc = GRAD_A ? p.K : p.N, Q = GRAD_A ? p.N : p.M;
   if ((int64_t)B * R * Cc == 0) return GENBMM_OK;
   auto wgs = [&](int br, int bc) { return (int64_t)B * ceil_div(R, br) * ceil_div(Cc, bc); };
   const bool small = R <= 32 && Cc <= 32;
-  const bool big = R >= 128 && Cc >= 128 && wgs(128, 128) >= 512;
   if (stats) {
-    if (small) return launch_bwd_fast<BCfgSmall, BCfgSmall, 1, GRAD_A>(p, stats, B, s);
-    if (big) return launch_bwd_fast<BCfgBig, BCfgWide, 2, GRAD_A>(p, stats, B, s);
-    return launch_bwd_fast<BCfgMid, BCfgMid, 1, GRAD_A>(p, stats, B, s);
+    int* fl = flags_of(stats, B, p.M, p.K, p.N, GRAD_A ? 1 : 2);
+    const bool al = p.vec_k && p.vec_n && aligned16(stats) && p.M % 4 == 0 && p.N % 4 == 0;
+    if (mfma_ok(R, Cc, Q, al, wgs(128, 128)))
+      return launch_bwd_fast<BCfgBig, BCfgWide, 2, GRAD_A, true>(p, stats, fl, B, s);
+    if (small) return launch_bwd_fast<BCfgSmall, BCfgSmall, 1, GRAD_A, false>(p, stats, fl, B, s);
+    if (R >= 128 && Cc >= 128 && wgs(128, 128) >= 512)
+      return launch_bwd_fast<BCfgBig, BCfgWide, 2, GRAD_A, false>(p, stats, fl, B, s);
+    return launch_bwd_fast<BCfgMid, BCfgMid, 1, GRAD_A, false>(p, stats, fl, B, s);
   }
   if (small) return launch_bwd_exact<BCfgSmall, GRAD_A>(p, B, s);
   if (R >= 64 && Cc >= 128 && wgs(64, 128) >= 512) return launch_bwd_exact<BCfgWide, GRAD_A>(p, B, s);
@@ -520,7 +601,13 @@ int run_bwd(const LogBwdArgs& p, const float* stats, int B, hipStream_t s) {
 
 extern "C" {
 
-void genbmm_logbmm_force_exact(int on) { genbmm::g_force_exact.store(on ? 1 : 0); }
+size_t genbmm_logbmm_stats_size(int B, int M, int K, int N) {
+  using namespace genbmm;
+  if (check_dense_dims(B, M, K, N)) return 0;
+  return (size_t)((int64_t)B * (M + N) + tiles32(B, M, N) + tiles32(B, M, K) + tiles32(B, K, N));
+}
+
+void genbmm_logbmm_force_exact(int on) { genbmm::g_path.store(on == 1 || on == 2 ? on : 0); }
 
 int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats, int B, int M,
                       int K, int N, void* stream) {
@@ -535,11 +622,16 @@ int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats, 
   if (mn == 0) return GENBMM_OK;
   DenseArgs p{};
   p.a = a; p.b = b; p.out = out; p.idx = nullptr;
-  if (stats && K > 0 && !g_force_exact.load()) {
-    if (M <= 32 && N <= 32) return launch_fwd_fast<CfgSmall, CfgSmall, 1>(p, stats, B, M, K, N, s);
-    if (M >= 128 && N >= 128 && (int64_t)B * ceil_div(M, 128) * ceil_div(N, 128) >= 512)
-      return launch_fwd_fast<CfgBig, CfgWide, 2>(p, stats, B, M, K, N, s);
-    return launch_fwd_fast<CfgMid, CfgMid, 1>(p, stats, B, M, K, N, s);
+  if (stats && K > 0 && g_path.load() != 1) {
+    int* fl = flags_of(stats, B, M, K, N, 0);
+    const int64_t big_tiles = (int64_t)B * ceil_div(M, 128) * ceil_div(N, 128);
+    const bool al = K % 4 == 0 && N % 4 == 0 && aligned16(a) && aligned16(b) && aligned16(stats);
+    if (mfma_ok(M, N, K, al, big_tiles)) return launch_fwd_mfma(p, stats, fl, B, M, K, N, s);
+    if (M <= 32 && N <= 32)
+      return launch_fwd_fast<CfgSmall, CfgSmall, 1>(p, stats, fl, B, M, K, N, s);
+    if (M >= 128 && N >= 128 && big_tiles >= 512)
+      return launch_fwd_fast<CfgBig, CfgWide, 2>(p, stats, fl, B, M, K, N, s);
+    return launch_fwd_fast<CfgMid, CfgMid, 1>(p, stats, fl, B, M, K, N, s);
   }
   switch (pick_shape(B, M, N, false)) {
     case kWide: return launch_fwd_exact<CfgWide>(p, B, M, K, N, s);
@@ -563,7 +655,7 @@ int genbmm_logbmm_bwd(const float* a, const float* b, const float* out, const fl
   p.vec_k = (K % 4 == 0) && aligned16(a) && aligned16(grad_a);
   p.vec_n = (N % 4 == 0) && aligned16(b) && aligned16(out) && aligned16(g) && aligned16(grad_b);
   hipStream_t s = (hipStream_t)stream;
-  const float* st = (g_force_exact.load() || mn == 0) ? nullptr : stats;
+  const float* st = (g_path.load() == 1 || mn == 0) ? nullptr : stats;
   if (grad_a) {
     p.grad = grad_a;
     if (int e = run_bwd<true>(p, st, B, s)) return e;

@@ -9,8 +9,8 @@ Differences in mechanism (not in results):
   * logbmm's backward produces grad_a and grad_b from one library call that
     reads every operand in place; the reference calls its kernel twice and
     transposes b, a, g, out, maxes and the result in between (genmul.py:35-41).
-  * instead of the (B, M, N) `maxes` tensor the forward saves a (B, M + N) vector of
-    row maxima of a and column maxima of b, which lets forward and backward factor
+  * instead of the (B, M, N) `maxes` tensor the forward saves a B*(M+N) vector of
+    row maxima of a and column maxima of b (plus a few per-tile flags), which lets forward and backward factor
     exp(a + b) wherever that is exact (see csrc/logbmm.hip).
   * the arg-max / sample index stays int32 into the backward; the reference
     converts it (and a, b, g) to float first (genmul.py:62-65).
@@ -94,7 +94,8 @@ class LogMatMul(torch.autograd.Function):
         a, b, (B, M, K, N) = _prep(a, b)
         out = torch.empty(B, M, N, dtype=_COMPUTE, device=a.device)
         # row maxima of a, column maxima of b: what the reference's `maxes` becomes
-        stats = torch.empty(B, M + N, dtype=_COMPUTE, device=a.device)
+        stats = torch.empty(_lib.load().genbmm_logbmm_stats_size(B, M, K, N), dtype=_COMPUTE,
+                            device=a.device)
         _call("genbmm_logbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(stats),
               B, M, K, N)
         ctx.save_for_backward(a, b, out, stats)

@@ -29,6 +29,7 @@
 #ifndef GENBMM_GFX950_H
 #define GENBMM_GFX950_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -62,13 +63,15 @@ const char* genbmm_error_string(int code);
  * The running maximum starts at -1e9 as in the reference (kernel :31), so an
  * output whose terms are all <= -1e9 is -inf.
  *
- * `stats` is an optional (B, M + N) fp32 buffer.  NULL: the online
- * (running-max) log-sum-exp kernel runs.  Non-NULL: it receives, per batch
- * item, max_k a[m,k] for every m followed by max_k b[k,n] for every n, and the
- * forward uses them to factor exp(a+b) = exp(a-max)*exp(b-max) wherever that
- * is exact to fp32 (tiles where it is not are recomputed by the online
- * kernel's routine).  It takes the place of the reference's (B, M, N) `maxes`
- * output; pass the same buffer to genbmm_logbmm_bwd.
+ * `stats` is an optional fp32 buffer of genbmm_logbmm_stats_size(B,M,K,N)
+ * elements.  NULL: the online (running-max) log-sum-exp kernel runs.
+ * Non-NULL: its first B*(M+N) elements receive, per batch item, max_k a[m,k]
+ * for every m followed by max_k b[k,n] for every n, and the forward uses them
+ * to factor exp(a+b) = exp(a-max)*exp(b-max) wherever that is exact to fp32;
+ * the rest of the buffer holds per-tile flags naming the tiles where it is
+ * not, which a fix-up launch recomputes with the online kernel's routine.
+ * The buffer takes the place of the reference's (B, M, N) `maxes` output;
+ * pass the same buffer to genbmm_logbmm_bwd.
  */
 int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats,
                       int B, int M, int K, int N, void* stream);
@@ -87,10 +90,15 @@ int genbmm_logbmm_bwd(const float* a, const float* b, const float* out,
                       float* grad_a, float* grad_b,
                       int B, int M, int K, int N, void* stream);
 
+/* Number of fp32 elements genbmm_logbmm_fwd / _bwd need in `stats`. */
+size_t genbmm_logbmm_stats_size(int B, int M, int K, int N);
+
 /*
- * Process-wide switch for tests and measurements: non-zero makes
- * genbmm_logbmm_fwd / _bwd ignore `stats` and always run the online / exact
- * kernels.  The only piece of global state in the library; default 0.
+ * Process-wide switch for tests and measurements.  1: genbmm_logbmm_fwd / _bwd
+ * ignore `stats` and always run the online / exact kernels.  2: the factored
+ * kernels contract with v_fma_f32 on the vector ALU instead of the fp32
+ * matrix-core instruction.  0 (default): factored kernels, matrix cores for
+ * 128x128 tiles.  The only piece of global state in the library.
  * No counterpart in the reference.
  */
 void genbmm_logbmm_force_exact(int on);

@@ -35,12 +35,12 @@ def lse64(a, b, chunk=4):
     return torch.cat(outs) if outs else a.new_zeros((0, a.shape[1], b.shape[2])).double()
 
 
-@pytest.fixture(params=["factored", "exact"])
+@pytest.fixture(params=["factored", "exact", "factored-valu"])
 def path(request, gpu):
-    """Run a logbmm test on both code paths: the factored kernels (default) and the
-    online/exact kernels alone."""
+    """Run a logbmm test on every code path: the factored kernels (default: matrix cores
+    for 128x128 tiles), the online/exact kernels alone, the factored kernels on v_fma."""
     lib = _lib.load()
-    lib.genbmm_logbmm_force_exact(1 if request.param == "exact" else 0)
+    lib.genbmm_logbmm_force_exact({"factored": 0, "exact": 1, "factored-valu": 2}[request.param])
     yield request.param
     lib.genbmm_logbmm_force_exact(0)
 
