@@ -31,6 +31,14 @@ constexpr int kMS = 16;         // slab depth
 constexpr int kMLD = kMT + 4;   // LDS row stride of a [slab][tile] buffer
 constexpr float kMfmaGuardBits = 40.f;
 
+// Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
+// Renumber them so that every XCD works on one contiguous run of tiles (the 16
+// tiles of a batch item share their operands).
+__device__ __forceinline__ int xcd_tile_id() {
+  const int w = blockIdx.x, n = gridDim.x;
+  return (n & 7) == 0 ? (w & 7) * (n >> 3) + (w >> 3) : w;
+}
+
 __device__ __forceinline__ float exp_st(float d) { return fast_exp2(d * kLog2e); }
 
 // 32 matrix-core steps over one staged slab: rows from R[q][0..128), columns
@@ -63,7 +71,7 @@ __device__ __forceinline__ void lds_put(float* __restrict__ buf, int red, int ou
 }
 
 // ----------------------------------------------------------------- forward
-__global__ __launch_bounds__(256, 2) void k_log_fwd_mfma(const float* __restrict__ a,
+__global__ __launch_bounds__(256, 4) void k_log_fwd_mfma(const float* __restrict__ a,
                                                          const float* __restrict__ b,
                                                          float* __restrict__ out,
                                                          const float* __restrict__ stats,
@@ -73,8 +81,8 @@ __global__ __launch_bounds__(256, 2) void k_log_fwd_mfma(const float* __restrict
   __shared__ __attribute__((aligned(16))) float Bs[2][kMS * kMLD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm0 = (wave >> 1) * 64, wn0 = (wave & 1) * 64;
-  const int per = tiles_m * tiles_n;
-  const int batch = blockIdx.x / per, rem = blockIdx.x - batch * per;
+  const int per = tiles_m * tiles_n, tile = xcd_tile_id();
+  const int batch = tile / per, rem = tile - batch * per;
   const int m0 = (rem / tiles_n) * kMT, n0 = (rem % tiles_n) * kMT;
   const float* st = stats + (long)batch * (M + N);
 
@@ -140,7 +148,7 @@ __global__ __launch_bounds__(256, 2) void k_log_fwd_mfma(const float* __restrict
       acc[x >> 1][x & 1][i] = __builtin_fmaf(fast_log2(s), kLn2, shift);
     }
   bad = __syncthreads_or(bad);
-  if (tid == 0) flags[blockIdx.x] = bad;
+  if (tid == 0) flags[tile] = bad;
   if (bad) return;  // the fix-up launch recomputes this tile
   float* ob = out + ((long)batch * M + m0 + wm0) * N + n0 + wn0 + lrow;
 #pragma unroll
@@ -156,7 +164,7 @@ __global__ __launch_bounds__(256, 2) void k_log_fwd_mfma(const float* __restrict
 // H = g * exp(alpha[m] + beta[n] - out[m,n]);  the epilogue multiplies by
 // exp(x - shift) of the operand shaped like the output.
 template <bool GRAD_A>
-__global__ __launch_bounds__(256, 2) void k_log_bwd_mfma(const float* __restrict__ a,
+__global__ __launch_bounds__(256, GRAD_A ? 2 : 4) void k_log_bwd_mfma(const float* __restrict__ a,
                                                          const float* __restrict__ b,
                                                          const float* __restrict__ outp,
                                                          const float* __restrict__ g,
@@ -168,8 +176,8 @@ __global__ __launch_bounds__(256, 2) void k_log_bwd_mfma(const float* __restrict
   __shared__ __attribute__((aligned(16))) float Hs[2][kMS * kMLD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wr0 = (wave >> 1) * 64, wc0 = (wave & 1) * 64;
-  const int per = tiles_r * tiles_c;
-  const int batch = blockIdx.x / per, rem = blockIdx.x - batch * per;
+  const int per = tiles_r * tiles_c, tile = xcd_tile_id();
+  const int batch = tile / per, rem = tile - batch * per;
   const int r0 = (rem / tiles_c) * kMT, c0 = (rem % tiles_c) * kMT;
   const int Q = GRAD_A ? N : M;
   const float* al = stats + (long)batch * (M + N);
@@ -276,7 +284,7 @@ __global__ __launch_bounds__(256, 2) void k_log_bwd_mfma(const float* __restrict
   }
 
   bad = __syncthreads_or(bad);
-  if (tid == 0) flags[blockIdx.x] = bad;
+  if (tid == 0) flags[tile] = bad;
   if (bad) return;  // the fix-up launch recomputes this tile
 
   // grad = exp(x - shift) * acc
