@@ -1,0 +1,207 @@
+"""Timing of every BASELINE.json configuration on one MI355X (bench.py covers only the
+headline line the driver reads).
+
+    python bench_configs.py [--reps 20] [--cpu]
+
+For each configuration: median device time of the C-ABI calls on pre-allocated outputs
+(HIP events on torch's current stream, 5 warm-ups), semiring GOP/s and % of the FP32
+vector peak (157.3 TFLOP/s) from the algorithmic operation count, and HBM GB/s from the
+algorithmic byte count.  --cpu adds the reference's CPU formulation (torch broadcast) for
+configuration 0.  One JSON object per line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+import torch  # noqa: E402
+
+from genbmm_amd import _lib  # noqa: E402
+
+PEAK_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def timed(fn, reps):
+    for _ in range(5):
+        fn()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        e1.synchronize()
+        ts.append(e0.elapsed_time(e1))
+    ts.sort()
+    return ts[len(ts) // 2]
+
+
+def report(name, ms, ops, nbytes, extra=None):
+    line = {
+        "config": name,
+        "ms": round(ms, 4),
+        "semiring_GOPs": round(ops / ms / 1e6, 1),
+        "pct_fp32_vector_peak": round(100 * ops / (ms * 1e-3) / (PEAK_TFLOPS * 1e12), 2),
+        "algorithmic_GBs": round(nbytes / ms / 1e6, 1),
+        "pct_hbm_peak": round(100 * nbytes / (ms * 1e-3) / (PEAK_HBM_GBS * 1e9), 2),
+    }
+    if extra:
+        line.update(extra)
+    print(json.dumps(line), flush=True)
+
+
+def dense_log(lib, dev, B, M, K, N, reps, name, dist="randn", path=0):
+    torch.manual_seed(0)
+    mk = torch.randn if dist == "randn" else torch.rand
+    a, b = mk(B, M, K).to(dev), mk(B, K, N).to(dev)
+    g = (torch.ones(B, M, N) if dist == "rand" else torch.randn(B, M, N)).to(dev)
+    out, ga, gb = torch.empty(B, M, N, device=dev), torch.empty_like(a), torch.empty_like(b)
+    stats = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=dev)
+    s, p = _lib.stream_of(a), _lib.ptr
+    lib.genbmm_logbmm_force_exact(path)
+
+    def step():
+        _lib.check(lib.genbmm_logbmm_fwd(p(a), p(b), p(out), p(stats), B, M, K, N, s), "fwd")
+        _lib.check(lib.genbmm_logbmm_bwd(p(a), p(b), p(out), p(g), p(stats), p(ga), p(gb), B, M, K, N, s), "bwd")
+
+    ms = timed(step, reps)
+    lib.genbmm_logbmm_force_exact(0)
+    bmkn = float(B) * M * K * N
+    nbytes = 4.0 * B * (3 * M * K + 3 * K * N + 3 * M * N)
+    report(name, ms, 6 * bmkn, nbytes, {"path": {0: "factored", 1: "online-exact", 2: "factored-valu"}[path]})
+
+
+def dense_max(lib, dev, B, M, K, N, reps, prod):
+    torch.manual_seed(0)
+    if prod:
+        a, b = (1 - torch.rand(B, M, K)).to(dev), (1 - torch.rand(B, K, N)).to(dev)
+    else:
+        a, b = (torch.round(torch.randn(B, M, K) * 8) / 8).to(dev), (torch.round(torch.randn(B, K, N) * 8) / 8).to(dev)
+    g = (torch.round(torch.randn(B, M, N) * 8) / 8).clamp(-4, 4).to(dev)
+    out = torch.empty(B, M, N, device=dev)
+    idx = torch.empty(B, M, N, dtype=torch.int32, device=dev)
+    ga, gb = torch.empty_like(a), torch.empty_like(b)
+    s, p = _lib.stream_of(a), _lib.ptr
+    fwd = lib.genbmm_prodmaxbmm_fwd if prod else lib.genbmm_maxbmm_fwd
+
+    def f():
+        _lib.check(fwd(p(a), p(b), p(out), p(idx), B, M, K, N, s), "fwd")
+
+    def bw():
+        if prod:
+            _lib.check(lib.genbmm_prodmax_bwd(p(a), p(b), p(idx), p(g), p(ga), p(gb), B, M, K, N, s), "bwd")
+        else:
+            _lib.check(lib.genbmm_argmax_bwd(p(idx), p(g), p(ga), p(gb), B, M, K, N, s), "bwd")
+
+    mf, mb = timed(f, reps), timed(bw, reps)
+    bmkn = float(B) * M * K * N
+    nbytes = 4.0 * B * (2 * M * K + 2 * K * N + 4 * M * N)
+    report(("prodmaxbmm" if prod else "maxbmm") + " fwd+bwd (%d,%d,%d,%d)" % (B, M, K, N), mf + mb, 6 * bmkn, nbytes,
+           {"ms_fwd": round(mf, 4), "ms_bwd": round(mb, 4)})
+
+
+def dense_sample(lib, dev, B, M, K, N, reps):
+    torch.manual_seed(0)
+    a, b = (2 * torch.randn(B, M, K)).to(dev), (2 * torch.randn(B, K, N)).to(dev)
+    g = torch.randn(B, M, N).to(dev)
+    out = torch.empty(B, M, N, device=dev)
+    idx = torch.empty(B, M, N, dtype=torch.int32, device=dev)
+    ga, gb = torch.empty_like(a), torch.empty_like(b)
+    s, p = _lib.stream_of(a), _lib.ptr
+
+    def f():
+        _lib.check(lib.genbmm_samplebmm_fwd(p(a), p(b), p(out), p(idx), 1234, 0, B, M, K, N, s), "fwd")
+
+    def bw():
+        _lib.check(lib.genbmm_argmax_bwd(p(idx), p(g), p(ga), p(gb), B, M, K, N, s), "bwd")
+
+    mf, mb = timed(f, reps), timed(bw, reps)
+    bmkn = float(B) * M * K * N
+    nbytes = 4.0 * B * (2 * M * K + 2 * K * N + 4 * M * N)
+    report("samplebmm fwd+bwd (%d,%d,%d,%d)" % (B, M, K, N), mf + mb, 6 * bmkn, nbytes,
+           {"ms_fwd": round(mf, 4), "ms_bwd": round(mb, 4)})
+
+
+def banded(lib, dev, B, n, lu, ld, mode, reps):
+    torch.manual_seed(7)
+    W = lu + ld + 1
+    Wo = 2 * W - 1
+    a, b = (torch.rand(B, n, W) * 2 - 1).to(dev), (torch.rand(B, n, W) * 2 - 1).to(dev)
+    g = torch.randn(B, n, Wo).to(dev)
+    out = torch.empty(B, n, Wo, device=dev)
+    idx = torch.empty(B, n, Wo, dtype=torch.int32, device=dev) if mode == 1 else None
+    ga, gb = torch.empty_like(a), torch.empty_like(b)
+    s, p = _lib.stream_of(a), _lib.ptr
+
+    def f():
+        _lib.check(lib.genbmm_banded_fwd(p(a), lu, ld, p(b), lu, ld, p(out), p(idx), B, n, mode, s), "fwd")
+
+    def bw():
+        _lib.check(lib.genbmm_banded_bwd(p(a), lu, ld, p(b), lu, ld, p(out), p(idx), p(g), p(ga), p(gb), B, n, mode, s),
+                   "bwd")
+
+    mf, mb = timed(f, reps), timed(bw, reps)
+    pairs = float(B) * n * W * W
+    fb = 4.0 * B * n * (2 * W + Wo) + (4.0 * B * n * Wo if mode == 1 else 0)
+    bb = 4.0 * B * n * (4 * W + Wo + (Wo if mode in (0, 1) else 0))
+    name = {0: "multiply_log", 1: "multiply_max", 3: "multiply"}[mode]
+    report("banded %s fwd+bwd (B=%d,n=%d,lu=ld=%d)" % (name, B, n, lu), mf + mb, 6 * pairs, fb + bb,
+           {"ms_fwd": round(mf, 4), "ms_bwd": round(mb, 4),
+            "fwd_GBs": round(fb / mf / 1e6, 1), "bwd_GBs": round(bb / mb / 1e6, 1)})
+
+
+def cpu_c1():
+    import oracle
+
+    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    torch.manual_seed(0)
+    a = torch.rand(16, 64, 64, requires_grad=True)
+    b = torch.rand(16, 64, 64, requires_grad=True)
+
+    def one():
+        a.grad = b.grad = None
+        oracle.logbmm_broadcast(a, b).backward(torch.ones(16, 64, 64))
+
+    one()
+    ts = []
+    for _ in range(11):
+        t0 = time.perf_counter()
+        one()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    ops = 6.0 * 16 * 64 * 64 * 64
+    print(json.dumps({"config": "logbmm fwd+bwd (16,64,64,64) CPU torch broadcast", "ms": round(ts[5] * 1e3, 3),
+                      "semiring_GOPs": round(ops / ts[5] / 1e9, 2), "cores": torch.get_num_threads()}), flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--reps", type=int, default=20)
+    ap.add_argument("--cpu", action="store_true")
+    args = ap.parse_args()
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    r = args.reps
+    dense_log(lib, dev, 16, 64, 64, 64, r, "logbmm fwd+bwd (16,64,64,64) config 0", dist="rand")
+    dense_log(lib, dev, 512, 128, 128, 128, r, "logbmm fwd+bwd (512,128,128,128) config 1")
+    dense_log(lib, dev, 8192, 32, 32, 32, r, "logbmm fwd+bwd (8192,32,32,32) config 1 skinny")
+    for path in (0, 2, 1):
+        dense_log(lib, dev, 64, 512, 512, 512, r, "logbmm fwd+bwd (64,512,512,512) headline", path=path)
+    dense_max(lib, dev, 256, 256, 256, 256, r, prod=False)
+    dense_max(lib, dev, 256, 256, 256, 256, r, prod=True)
+    dense_sample(lib, dev, 64, 512, 512, 512, r)
+    for mode in (3, 0, 1):
+        banded(lib, dev, 64, 4096, 32, 32, mode, r)
+    if args.cpu:
+        cpu_c1()
+
+
+if __name__ == "__main__":
+    main()
