@@ -185,20 +185,26 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--cpu", action="store_true")
+    ap.add_argument("--only", default="", help="comma-separated subset: log,max,sample,banded")
     args = ap.parse_args()
+    want = set(args.only.split(",")) if args.only else {"log", "max", "sample", "banded"}
     lib = _lib.load()
     dev = torch.device("cuda:0")
     r = args.reps
-    dense_log(lib, dev, 16, 64, 64, 64, r, "logbmm fwd+bwd (16,64,64,64) config 0", dist="rand")
-    dense_log(lib, dev, 512, 128, 128, 128, r, "logbmm fwd+bwd (512,128,128,128) config 1")
-    dense_log(lib, dev, 8192, 32, 32, 32, r, "logbmm fwd+bwd (8192,32,32,32) config 1 skinny")
-    for path in (0, 2, 1):
-        dense_log(lib, dev, 64, 512, 512, 512, r, "logbmm fwd+bwd (64,512,512,512) headline", path=path)
-    dense_max(lib, dev, 256, 256, 256, 256, r, prod=False)
-    dense_max(lib, dev, 256, 256, 256, 256, r, prod=True)
-    dense_sample(lib, dev, 64, 512, 512, 512, r)
-    for mode in (3, 0, 1):
-        banded(lib, dev, 64, 4096, 32, 32, mode, r)
+    if "log" in want:
+        dense_log(lib, dev, 16, 64, 64, 64, r, "logbmm fwd+bwd (16,64,64,64) config 0", dist="rand")
+        dense_log(lib, dev, 512, 128, 128, 128, r, "logbmm fwd+bwd (512,128,128,128) config 1")
+        dense_log(lib, dev, 8192, 32, 32, 32, r, "logbmm fwd+bwd (8192,32,32,32) config 1 skinny")
+        for path in (0, 2, 1):
+            dense_log(lib, dev, 64, 512, 512, 512, r, "logbmm fwd+bwd (64,512,512,512) headline", path=path)
+    if "max" in want:
+        dense_max(lib, dev, 256, 256, 256, 256, r, prod=False)
+        dense_max(lib, dev, 256, 256, 256, 256, r, prod=True)
+    if "sample" in want:
+        dense_sample(lib, dev, 64, 512, 512, 512, r)
+    if "banded" in want:
+        for mode in (3, 0, 1):
+            banded(lib, dev, 64, 4096, 32, 32, mode, r)
     if args.cpu:
         cpu_c1()
 

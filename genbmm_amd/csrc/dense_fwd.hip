@@ -121,7 +121,7 @@ int run_max(const float* a, const float* b, float* out, int32_t* idx, int B, int
   DenseArgs p{};
   p.a = a; p.b = b; p.out = out; p.idx = idx;
   hipStream_t s = (hipStream_t)stream;
-  switch (pick_shape(B, M, N, true)) {
+  switch (pick_shape(B, M, N, false)) {
     case kBig: return launch_max<CfgBig, PROD>(p, B, M, K, N, s);
     case kWide: return launch_max<CfgWide, PROD>(p, B, M, K, N, s);
     case kMid: return launch_max<CfgMid, PROD>(p, B, M, K, N, s);
