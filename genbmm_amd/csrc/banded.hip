@@ -18,151 +18,33 @@
 // One lane per output element with lanes along the band axis (the contiguous
 // axis of every tensor), so stores are coalesced and neighbouring lanes read
 // overlapping runs that the vector L1 / L2 serve.
-#include "common.h"
+#include "banded_strip.h"
 
 namespace genbmm {
 namespace {
 
-struct BandArgs {
-  const float* a;
-  const float* b;
-  const float* out;
-  const float* g;
-  const float* ua;
-  const float* ub;
-  const int32_t* idx;
-  float* o0;      // out        | grad_a
-  float* o1;      // -          | grad_b
-  float* o2;      // -          | grad_g
-  int32_t* oidx;  // forward argmax
-  int n, a_lu, Wa, b_lu, Wb, r_lu, Wo;
-};
-
-__device__ __forceinline__ int imax3(int a, int b, int c) { return max(a, max(b, c)); }
-__device__ __forceinline__ int imin3(int a, int b, int c) { return min(a, min(b, c)); }
-
-// Valid k range [klo, khi] of output cell (i, j); needs 0 <= o < n.
-__device__ __forceinline__ void k_range(const BandArgs& p, int i, int j, int& klo, int& khi) {
-  klo = imax3(0, j - (p.Wb - 1), p.a_lu - i);
-  khi = imin3(p.Wa - 1, j, p.n - 1 + p.a_lu - i);
-}
-
-// ------------------------------------------------------------------ forward
-// Reference banded_cuda_forward_kernel_mul (banded_cuda_kernel.cu:13-100).
 template <int MODE>
 __global__ __launch_bounds__(256) void k_band_fwd(const BandArgs p, long total) {
   const long e = (long)blockIdx.x * 256 + threadIdx.x;
   if (e >= total) return;
-  const int j = (int)(e % p.Wo);
   const long bi = e / p.Wo;  // batch*n + i
-  const int i = (int)(bi % p.n);
-  const int o = i + j - p.r_lu;
-  if (o < 0 || o >= p.n) {  // outside the matrix: the reference leaves its zero fill
-    p.o0[e] = 0.f;
-    if (MODE == GENBMM_BAND_MAX) p.oidx[e] = 0;
-    return;
-  }
-  int klo, khi;
-  k_range(p, i, j, klo, khi);
-  const float* ar = p.a + bi * p.Wa;
-  const float* br = p.b + (bi + (o - i)) * p.Wb + (p.Wb - 1 - j);  // br[k] = b[o][k2(k)]
-  if (MODE == GENBMM_BAND_MUL) {
-    float v = 0.f;
-    for (int k = klo; k <= khi; ++k) v = __builtin_fmaf(ar[k], br[k], v);
-    p.o0[e] = v;
-  } else if (MODE == GENBMM_BAND_MAX) {
-    float m = kFloor;
-    int ind = -1;
-    for (int k = klo; k <= khi; ++k) {
-      const float v = ar[k] + br[k];
-      if (v > m) {
-        m = v;
-        ind = k;
-      }
-    }
-    p.o0[e] = m;
-    p.oidx[e] = ind;
-  } else {
-    float m = kFloor;
-    for (int k = klo; k <= khi; ++k) m = fmaxf(m, ar[k] + br[k]);
-    const float nm = -m * kLog2e;
-    float s = 0.f;
-    for (int k = klo; k <= khi; ++k) s += fast_exp2(__builtin_fmaf(ar[k] + br[k], kLog2e, nm));
-    p.o0[e] = logf(s) + m;
-  }
+  band_fwd_cell<MODE>(p, bi, (int)(bi % p.n), (int)(e - bi * p.Wo));
 }
 
-// ----------------------------------------------------------------- backward
-// d out[i,j] / d a[i,k]: MUL b[o,k2]; LOG exp(a[i,k]+b[o,k2]-out[i,j]);
-// MAX [k == idx[i,j]].  grad_a[i,k] sums over j ascending (reference
-// banded_cuda_backward_kernel_mul, banded_cuda_kernel.cu:104-152).
 template <int MODE>
 __global__ __launch_bounds__(256) void k_band_bwd_a(const BandArgs p, long total) {
   const long e = (long)blockIdx.x * 256 + threadIdx.x;
   if (e >= total) return;
-  const int k = (int)(e % p.Wa);
   const long bi = e / p.Wa;
-  const int i = (int)(bi % p.n);
-  const int pos = i + k - p.a_lu;
-  float acc = 0.f;
-  if (pos >= 0 && pos < p.n) {
-    const int jlo = imax3(k, p.r_lu - i, 0);
-    const int jhi = imin3(k + p.Wb - 1, p.n - 1 + p.r_lu - i, p.Wo - 1);
-    const float* gr = p.g + bi * p.Wo;
-    // b[o][k2] = bw[j * (Wb - 1)] with o = i + j - r_lu, k2 = k - j + Wb - 1
-    const float* bw = p.b + (bi - p.r_lu) * p.Wb + k + p.Wb - 1;
-    if (MODE == GENBMM_BAND_MUL) {
-      for (int j = jlo; j <= jhi; ++j) acc = __builtin_fmaf(bw[(long)j * (p.Wb - 1)], gr[j], acc);
-    } else if (MODE == GENBMM_BAND_MAX) {
-      const int32_t* ir = p.idx + bi * p.Wo;
-      for (int j = jlo; j <= jhi; ++j) acc += (ir[j] == k) ? gr[j] : 0.f;
-    } else {
-      const float av = p.a[e];
-      const float* orow = p.out + bi * p.Wo;
-      for (int j = jlo; j <= jhi; ++j) {
-        const float w = fast_exp(av + bw[(long)j * (p.Wb - 1)] - orow[j]);
-        acc = __builtin_fmaf(w, gr[j], acc);
-      }
-    }
-  }
-  p.o0[e] = acc;
+  band_bwd_a_cell<MODE>(p, bi, (int)(bi % p.n), (int)(e - bi * p.Wa));
 }
 
-// grad_b[o,k2] sums, in ascending i, over the cells (i, j = o - i + r_lu) that
-// read b[o,k2], with k = k2 + j - (Wb - 1).  The reference gets the same
-// numbers by transposing g / out in band form on the host and calling the
-// kernel above with the operands swapped (sparse.py:436-446, 523-545, 625-635).
 template <int MODE>
 __global__ __launch_bounds__(256) void k_band_bwd_b(const BandArgs p, long total) {
   const long e = (long)blockIdx.x * 256 + threadIdx.x;
   if (e >= total) return;
-  const int k2 = (int)(e % p.Wb);
   const long bo = e / p.Wb;
-  const int o = (int)(bo % p.n);
-  const int prow = o + k2 - p.b_lu;
-  float acc = 0.f;
-  if (prow >= 0 && prow < p.n) {
-    const int jhi_k = p.Wb - 1 - k2 + p.Wa - 1;  // j with k = Wa-1
-    const int jlo_k = p.Wb - 1 - k2;             // j with k = 0
-    const int ilo = imax3(0, o + p.r_lu - min(jhi_k, p.Wo - 1), o + p.r_lu - (p.Wo - 1));
-    const int ihi = imin3(p.n - 1, o + p.r_lu - max(jlo_k, 0), o + p.r_lu);
-    const long base = bo - o;  // batch*n
-    const float bv = p.b[e];
-    for (int i = ilo; i <= ihi; ++i) {
-      const int j = o - i + p.r_lu;
-      const int k = k2 + j - (p.Wb - 1);
-      const long gi = (base + i) * p.Wo + j;
-      if (MODE == GENBMM_BAND_MUL) {
-        acc = __builtin_fmaf(p.a[(base + i) * p.Wa + k], p.g[gi], acc);
-      } else if (MODE == GENBMM_BAND_MAX) {
-        acc += (p.idx[gi] == k) ? p.g[gi] : 0.f;
-      } else {
-        const float w = fast_exp(p.a[(base + i) * p.Wa + k] + bv - p.out[gi]);
-        acc = __builtin_fmaf(w, p.g[gi], acc);
-      }
-    }
-  }
-  p.o1[e] = acc;
+  band_bwd_b_cell<MODE>(p, bo, (int)(bo % p.n), (int)(e - bo * p.Wb));
 }
 
 // ------------------------------------------------------ log second order
@@ -260,6 +142,8 @@ int fill_band(BandArgs& p, int a_lu, int a_ld, int b_lu, int b_ld, int B, int n)
   return GENBMM_OK;
 }
 
+constexpr size_t kStripLdsLimit = 64 * 1024;  // dynamic LDS available without opting in
+
 inline dim3 blocks_for(long total) { return dim3((unsigned)((total + 255) / 256)); }
 
 }  // namespace
@@ -280,6 +164,20 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   const long total = (long)B * n * p.Wo;
   if (total == 0) return GENBMM_OK;
   hipStream_t s = (hipStream_t)stream;
+  const StripDims sd = strip_dims(p.Wa, p.Wb);
+  if (mode != GENBMM_BAND_MAX && sd.ld_own <= 256 && sd.ld_sl <= 256 && sd.bytes <= kStripLdsLimit) {
+    const int strips = ceil_div(n, kBT);
+    const dim3 grid((unsigned)((long)B * strips));
+    const int nq = ceil_div(max(sd.ld_own, sd.ld_sl), 64);
+    auto go = [&](auto kern) {
+      hipLaunchKernelGGL(kern, grid, dim3(256), sd.bytes, s, p, strips, sd.ld_own, sd.ld_sl);
+    };
+    const bool lg = mode == GENBMM_BAND_LOG;
+    if (nq <= 1) lg ? go(k_band_fwd_strip<true, 1>) : go(k_band_fwd_strip<false, 1>);
+    else if (nq == 2) lg ? go(k_band_fwd_strip<true, 2>) : go(k_band_fwd_strip<false, 2>);
+    else lg ? go(k_band_fwd_strip<true, 4>) : go(k_band_fwd_strip<false, 4>);
+    return launch_status();
+  }
   if (mode == GENBMM_BAND_LOG)
     hipLaunchKernelGGL(k_band_fwd<GENBMM_BAND_LOG>, blocks_for(total), dim3(256), 0, s, p, total);
   else if (mode == GENBMM_BAND_MAX)
@@ -305,6 +203,34 @@ int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   const long ta = (long)B * n * p.Wa, tb = (long)B * n * p.Wb;
   if (ta == 0) return GENBMM_OK;
   hipStream_t s = (hipStream_t)stream;
+  if (mode != GENBMM_BAND_MAX && p.Wa <= 8 * 4 * kMaxKB && p.Wb <= 8 * 4 * kMaxKB) {
+    const bool lg = mode == GENBMM_BAND_LOG;
+    const StripDims da = strip_dims(p.Wa, p.Wb), db = strip_dims(p.Wb, p.Wa);
+    const size_t na = bwd_strip_bytes(da, lg), nb = bwd_strip_bytes(db, lg);
+    if (max(na, nb) <= kStripLdsLimit && max(max(da.ld_own, da.ld_sl), max(db.ld_own, db.ld_sl)) <= 128) {
+      const int strips = ceil_div(n, kBT);
+      const dim3 grid((unsigned)((long)B * strips));
+      const int nq = ceil_div(max(max(da.ld_own, da.ld_sl), max(db.ld_own, db.ld_sl)), 64);
+      if (nq <= 1) {
+        if (lg) {
+          hipLaunchKernelGGL((k_band_bwd_strip<true, true, 1>), grid, dim3(256), na, s, p, strips, da.ld_own, da.ld_sl, bwd_sl_floats(da));
+          hipLaunchKernelGGL((k_band_bwd_strip<true, false, 1>), grid, dim3(256), nb, s, p, strips, db.ld_own, db.ld_sl, bwd_sl_floats(db));
+        } else {
+          hipLaunchKernelGGL((k_band_bwd_strip<false, true, 1>), grid, dim3(256), na, s, p, strips, da.ld_own, da.ld_sl, bwd_sl_floats(da));
+          hipLaunchKernelGGL((k_band_bwd_strip<false, false, 1>), grid, dim3(256), nb, s, p, strips, db.ld_own, db.ld_sl, bwd_sl_floats(db));
+        }
+      } else {
+        if (lg) {
+          hipLaunchKernelGGL((k_band_bwd_strip<true, true, 2>), grid, dim3(256), na, s, p, strips, da.ld_own, da.ld_sl, bwd_sl_floats(da));
+          hipLaunchKernelGGL((k_band_bwd_strip<true, false, 2>), grid, dim3(256), nb, s, p, strips, db.ld_own, db.ld_sl, bwd_sl_floats(db));
+        } else {
+          hipLaunchKernelGGL((k_band_bwd_strip<false, true, 2>), grid, dim3(256), na, s, p, strips, da.ld_own, da.ld_sl, bwd_sl_floats(da));
+          hipLaunchKernelGGL((k_band_bwd_strip<false, false, 2>), grid, dim3(256), nb, s, p, strips, db.ld_own, db.ld_sl, bwd_sl_floats(db));
+        }
+      }
+      return launch_status();
+    }
+  }
   if (mode == GENBMM_BAND_LOG) {
     hipLaunchKernelGGL(k_band_bwd_a<GENBMM_BAND_LOG>, blocks_for(ta), dim3(256), 0, s, p, ta);
     hipLaunchKernelGGL(k_band_bwd_b<GENBMM_BAND_LOG>, blocks_for(tb), dim3(256), 0, s, p, tb);

@@ -1,0 +1,383 @@
+// Strip kernels for the banded (+,*) and log products: the operands of a strip
+// of 64 matrix columns are staged through LDS, so every band element is read
+// from memory once per strip (plus the halo of the sliding operand) and every
+// load and store is a run along the band axis.
+//
+// Walking the diagonals.  With k2 = k - j + (Wb - 1) independent of i,
+//   forward   out[i,j]  = sum_k  a[i,k]       * b[i+j-lu_o, k-j+Wb-1]
+//   grad_a    ga[i,k]   = sum_j  g'[i,j]      * b[i+j-lu_o, k-j+Wb-1]
+//   grad_b    gb[o,k2]  = sum_j  g'[o-j+lu_o,j] * a[o-j+lu_o, k2+j-(Wb-1)]
+// a lane owns one row (i, resp. o) and a block of 8 adjacent outputs along the
+// band axis (j, k, k2); one step of the sum reads one value of the lane's own
+// row and 8 values of the other operand, which sit on an anti-diagonal of its
+// LDS tile: row + 1, column - 1 per output.  Row strides are odd, so the 64
+// lanes of a wave (64 consecutive rows) hit 64 different banks at every step.
+// The other operand's rows carry 7 cells of padding on both sides holding the
+// semiring zero, and matrix-edge cells are zeroed while staging, so the inner
+// loop has no predicates.  The band axis of the sum/outputs is cut into chunks
+// of 32 (8 per wave); the sliding operand's 64 + 31 rows are re-staged per chunk.
+//
+// Log semiring: factored like the dense logbmm.  alpha[i] = max_k a[i,k],
+// beta[o] = max_k2 b[o,k2] (over the cells inside the matrix) are taken by the
+// wave that stages the row, the tiles hold exp(a - alpha), exp(b - beta) and
+// the sum is a multiply-add; out = log S + alpha + beta.  The backward stages
+// H = g * exp(alpha + beta - out) in place of g.  A cell whose S falls below
+// 2^-40 (forward) or whose alpha + beta - out exceeds 40 ln 2 (backward) is
+// recomputed - the cell, resp. the gradient rows it feeds - by the per-cell
+// routine from global memory.
+#pragma once
+
+#include "banded_cells.h"
+
+namespace genbmm {
+
+constexpr int kBT = 64;              // rows per strip = lanes of a wave
+constexpr int kBJ = 32;              // band-axis chunk: 4 waves x 8
+constexpr int kBR = kBT + kBJ - 1;   // rows of the sliding operand per chunk
+constexpr int kBP = 7;               // padding cells on both sides of its rows
+constexpr int kBC = kBJ + 1;         // row stride of the output staging tile
+constexpr float kBandGuardBits = 40.f;
+
+struct StripDims {
+  int ld_own;    // row stride of the lane's own operand tile
+  int ld_sl;     // row stride of the sliding operand tile (padded)
+  size_t bytes;  // dynamic LDS
+};
+
+inline int odd(int x) { return x | 1; }
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+// Staging of `ROWS` rows of a band operand (width W, lu given) starting at
+// matrix column row0 into tile[r * ld + pad + k]; columns [0, pad) and
+// [pad + W, ld) and every cell outside the matrix get the semiring zero.  LOG:
+// the tile gets exp(x - rowmax) and shift[r] the row maximum (over cells inside
+// the matrix).  One wave per row (rows wave, wave+4, ...), lanes along the band
+// axis, NQ = ceil(ld / 64) cells per lane.  load() only issues the global
+// loads into registers, store() consumes them - a whole chunk is in flight while
+// the previous one is being multiplied.
+template <bool LOG, int NQ, int ROWS>
+struct RowStage {
+  static constexpr int U = (ROWS + 3) / 4;
+  float v[U][NQ];
+
+  __device__ __forceinline__ void load(const float* __restrict__ src, int W, int lu, int n, int row0,
+                                       int ld, int pad, int wave, int lane) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int r = wave + 4 * u, c = row0 + r;  // c: matrix column = row of the band tensor
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        const int col = lane + 64 * q, k = col - pad;
+        const int prow = c + k - lu;  // dense row of this cell
+        const bool ok = r < ROWS && col < ld && c >= 0 && c < n && k >= 0 && k < W && prow >= 0 && prow < n;
+        v[u][q] = ok ? src[(long)c * W + k] : (LOG ? -INFINITY : 0.f);
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(float* __restrict__ tile, int ld, float* __restrict__ shift,
+                                        int wave, int lane) const {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int r = wave + 4 * u;
+      if (r < ROWS) {
+        float m = 0.f;
+        if (LOG) {
+          m = v[u][0];
+#pragma unroll
+          for (int q = 1; q < NQ; ++q) m = fmaxf(m, v[u][q]);
+          m = wave_max(m);
+          if (lane == 0) shift[r] = m;
+          if (m == -INFINITY) m = 0.f;  // row without a cell inside the matrix: all zeros
+        }
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+          const int col = lane + 64 * q;
+          if (col < ld) tile[r * ld + col] = LOG ? fast_exp2((v[u][q] - m) * kLog2e) : v[u][q];
+        }
+      }
+    }
+  }
+};
+
+// ------------------------------------------------------------------ forward
+// Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each): renumber so
+// that an XCD works on consecutive strips, whose halos overlap.
+__device__ __forceinline__ int xcd_strip_id() {
+  const int w = blockIdx.x, n = gridDim.x;
+  return (n & 7) == 0 ? (w & 7) * (n >> 3) + (w >> 3) : w;
+}
+
+template <bool LOG, int NQ>
+__global__ __launch_bounds__(256, LOG ? 2 : 3) void k_band_fwd_strip(const BandArgs p, int strips, int ld_own,
+                                                           int ld_sl) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  float* As = smem;                 // [64][ld_own]
+  float* Bs = As + kBT * ld_own;    // [95][ld_sl]; reused as the [64][33] output staging tile
+  float* al = Bs + kBR * ld_sl;     // [64]
+  float* be = al + kBT;             // [95]
+  float* Cs = Bs;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wg = xcd_strip_id();
+  const int batch = wg / strips, i0 = (wg - batch * strips) * kBT;
+  const int n = p.n, Wa = p.Wa, Wb = p.Wb, Wo = p.Wo;
+  const float* ab = p.a + (long)batch * n * Wa;
+  const float* bb = p.b + (long)batch * n * Wb;
+  float* ob = p.o0 + (long)batch * n * Wo;
+  const long bn = (long)batch * n;
+  const float thr = fast_exp2(-kBandGuardBits);
+
+  {
+    RowStage<LOG, NQ, kBT> sa;
+    sa.load(ab, Wa, p.a_lu, n, i0, ld_own, 0, wave, lane);
+    sa.store(As, ld_own, al, wave, lane);
+  }
+  RowStage<LOG, NQ, kBR> sb;
+  sb.load(bb, Wb, p.b_lu, n, i0 - p.r_lu, ld_sl, kBP, wave, lane);
+
+  for (int jc = 0; jc < Wo; jc += kBJ) {
+    __syncthreads();  // the previous chunk's output tile has been written out
+    sb.store(Bs, ld_sl, be, wave, lane);
+    __syncthreads();
+    if (jc + kBJ < Wo) sb.load(bb, Wb, p.b_lu, n, i0 + jc + kBJ - p.r_lu, ld_sl, kBP, wave, lane);
+
+    const int j0 = jc + 8 * wave;
+    float acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) acc[t] = 0.f;
+    if (j0 < Wo) {
+      const int klo = max(0, j0 - (Wb - 1)), khi = min(Wa - 1, j0 + 7);
+      const float* ap = As + lane * ld_own;
+      // element (t, k): Bs[(lane + 8*wave + t)][k - j0 - t + Wb - 1 + pad]
+      const float* bp = Bs + (lane + 8 * wave) * ld_sl + (Wb - 1 + kBP - j0);
+      const int dt = ld_sl - 1;
+      int k = klo;
+      for (; k + 3 <= khi; k += 4) {
+        float av[4], bv[4][8];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          av[x] = ap[k + x];
+#pragma unroll
+          for (int t = 0; t < 8; ++t) bv[x][t] = bp[t * dt + k + x];
+        }
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+#pragma unroll
+          for (int t = 0; t < 8; ++t) acc[t] = __builtin_fmaf(av[x], bv[x][t], acc[t]);
+      }
+      for (; k <= khi; ++k) {
+        const float av = ap[k];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc[t] = __builtin_fmaf(av, bp[t * dt + k], acc[t]);
+      }
+    }
+    float sh[8];
+    if (LOG) {
+#pragma unroll
+      for (int t = 0; t < 8; ++t) sh[t] = al[lane] + be[min(lane + 8 * wave + t, kBR - 1)];
+    }
+    __syncthreads();  // every wave is done with Bs: it becomes the output tile
+    const int i = i0 + lane;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      float v = acc[t];
+      if (LOG) {
+        const int j = j0 + t, o = i + j - p.r_lu;
+        if (i < n && j < Wo && o >= 0 && o < n) {
+          if ((v >= thr) && (v < INFINITY) && (sh[t] > 0.9f * kFloor) && (sh[t] < INFINITY)) {
+            v = __builtin_fmaf(fast_log2(v), kLn2, sh[t]);
+          } else {  // factoring not exact for this cell: recompute it from memory
+            band_fwd_cell<GENBMM_BAND_LOG>(p, bn + i, i, j);
+            v = ob[(long)i * Wo + j];
+          }
+        } else {
+          v = 0.f;  // outside the matrix: the reference's zero fill
+        }
+      }
+      Cs[lane * kBC + 8 * wave + t] = v;
+    }
+    __syncthreads();
+    // rows of 32 consecutive outputs
+    for (int e = tid; e < kBT * kBJ; e += 256) {
+      const int r = e >> 5, c = e & 31;
+      if (i0 + r < n && jc + c < Wo) ob[(long)(i0 + r) * Wo + jc + c] = Cs[r * kBC + c];
+    }
+  }
+}
+
+// ----------------------------------------------------------------- backward
+// Shared by both gradients: the lane owns row x of the OUTPUT operand (a for
+// grad_a, b for grad_b) and up to kMaxKB blocks of 8 cells along its band axis;
+// per chunk of 32 result diagonals j it multiplies one value of g' (g, or
+// H = g*exp(alpha+beta-out) in the log semiring) with 8 values of the other
+// operand on an anti-diagonal of its tile.
+//   grad_a: g'[x][j]            * b'[x + j - lu_o][kk - j + Wb - 1]
+//   grad_b: g'[x - j + lu_o][j] * a'[x - j + lu_o][kk + j - (Wb - 1)]
+constexpr int kMaxKB = 3;  // band-axis blocks of 8 per wave: widths up to 96
+
+template <bool LOG, bool GRAD_A, int NQ>
+__global__ __launch_bounds__(256, 2) void k_band_bwd_strip(const BandArgs p, int strips, int ld_own,
+                                                           int ld_sl, int sl_floats) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  // own: the output operand's strip (LOG: exp(x - shift), for the epilogue)
+  // sl : 95 rows of the other operand, padded (LOG: exp(y - shift))
+  // gt : g' tile; grad_a [64][33] (row x), grad_b [95][33] (row x - j + lu_o)
+  float* own = smem;
+  float* sl = own + (LOG ? kBT * ld_own : 0);
+  float* gt = sl + sl_floats;      // sl_floats = max(95 * ld_sl, 64 * ld_own)
+  float* sh_own = gt + kBR * kBC;  // [64] shift of the lane's own row
+  float* sh_sl = sh_own + kBT;     // [95] shifts of the staged other-operand rows
+  int* badrow = reinterpret_cast<int*>(sh_sl + kBR);  // [64]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wg = xcd_strip_id();
+  const int batch = wg / strips, x0 = (wg - batch * strips) * kBT;
+  const int n = p.n, Wa = p.Wa, Wb = p.Wb, Wo = p.Wo;
+  const long bn = (long)batch * n;
+  const float* ab = p.a + bn * Wa;
+  const float* bb = p.b + bn * Wb;
+  const float* gb = p.g + bn * Wo;
+  const float* ob = LOG ? p.out + bn * Wo : nullptr;
+  // output operand / other operand
+  const float* xo = GRAD_A ? ab : bb;
+  const float* yo = GRAD_A ? bb : ab;
+  const int Wx = GRAD_A ? Wa : Wb, Wy = GRAD_A ? Wb : Wa;
+  const int lux = GRAD_A ? p.a_lu : p.b_lu, luy = GRAD_A ? p.b_lu : p.a_lu;
+  float* gradb = (GRAD_A ? p.o0 : p.o1) + bn * Wx;
+  const float lim = kBandGuardBits * kLn2 + 1e-3f;
+
+  if (tid < kBT) badrow[tid] = 0;
+  if (LOG) {
+    RowStage<true, NQ, kBT> so;
+    so.load(xo, Wx, lux, n, x0, ld_own, 0, wave, lane);
+    so.store(own, ld_own, sh_own, wave, lane);
+  }
+  float acc[kMaxKB][8];
+#pragma unroll
+  for (int q = 0; q < kMaxKB; ++q)
+#pragma unroll
+    for (int t = 0; t < 8; ++t) acc[q][t] = 0.f;
+
+  // first row of the other operand needed by chunk jc
+  auto row0_of = [&](int jc) { return GRAD_A ? x0 + jc - p.r_lu : x0 - jc - (kBJ - 1) + p.r_lu; };
+  RowStage<LOG, NQ, kBR> ss;
+  ss.load(yo, Wy, luy, n, row0_of(0), ld_sl, kBP, wave, lane);
+
+  for (int jc = 0; jc < Wo; jc += kBJ) {
+    const int yb = row0_of(jc);
+    __syncthreads();  // previous chunk fully consumed
+    ss.store(sl, ld_sl, sh_sl, wave, lane);
+    __syncthreads();  // sh_sl visible
+    if (jc + kBJ < Wo) ss.load(yo, Wy, luy, n, row0_of(jc + kBJ), ld_sl, kBP, wave, lane);
+    // ---- g' tile
+    {
+      const int rows = GRAD_A ? kBT : kBR;
+      for (int e = tid; e < rows * kBJ; e += 256) {
+        const int r = e >> 5, c = e & 31, j = jc + c;
+        const int i = GRAD_A ? x0 + r : yb + r;  // row of g / out (a's row index)
+        const int o = i + j - p.r_lu;            // b's row index of this cell
+        float v = 0.f;
+        const bool inside = i >= 0 && i < n && j < Wo && o >= 0 && o < n;
+        // grad_b only uses cells whose o lies in this strip
+        const bool used = inside && (GRAD_A || (o >= x0 && o < x0 + kBT));
+        if (used) {
+          v = gb[(long)i * Wo + j];
+          if (LOG) {
+            // alpha[i] + beta[o] - out[i,j]
+            const float sa = GRAD_A ? sh_own[r] : sh_sl[r];
+            const float sb = GRAD_A ? sh_sl[r + c] : sh_own[o - x0];
+            const float ex = sa + sb - ob[(long)i * Wo + j];
+            if (!(ex <= lim)) badrow[GRAD_A ? r : o - x0] = 1;  // factoring not exact: row redone
+            v *= fast_exp2(ex * kLog2e);
+          }
+        }
+        gt[r * kBC + c] = v;
+      }
+    }
+    __syncthreads();
+    // ---- multiply
+#pragma unroll
+    for (int q = 0; q < kMaxKB; ++q) {
+      const int k0 = 8 * (wave + 4 * q);  // first band cell of this block
+      if (k0 >= Wx) break;
+      // j range (within the chunk) that can meet cells k0 .. k0+7
+      int jlo, jhi;
+      if (GRAD_A) {  // k2 = k - j + Wb - 1 in [0, Wb)
+        jlo = max(jc, k0);
+        jhi = min(min(jc + kBJ - 1, Wo - 1), k0 + 7 + Wb - 1);
+      } else {       // k = k2 + j - (Wb - 1) in [0, Wa)
+        jlo = max(jc, Wb - 1 - k0 - 7);
+        jhi = min(min(jc + kBJ - 1, Wo - 1), Wb - 1 - k0 + Wa - 1);
+      }
+      const float* gp;
+      const float* yp;
+      int gstep, ystep;
+      if (GRAD_A) {
+        // g'[lane][jj], b'[lane + jj][k0 + t - (jc + jj) + Wb - 1 + pad]
+        gp = gt + lane * kBC;
+        gstep = 1;
+        yp = sl + lane * ld_sl + (k0 - jc + Wb - 1 + kBP);
+        ystep = ld_sl - 1;
+      } else {
+        // row r = lane - jj + 31: g'[r][jj], a'[r][k0 + t + (jc + jj) - (Wb - 1) + pad]
+        gp = gt + (lane + kBJ - 1) * kBC;
+        gstep = 1 - kBC;
+        yp = sl + (lane + kBJ - 1) * ld_sl + (k0 + jc - (Wb - 1) + kBP);
+        ystep = 1 - ld_sl;
+      }
+      for (int j = jlo; j <= jhi; ++j) {
+        const int jj = j - jc;
+        const float gv = gp[jj * gstep];
+        const float* yr = yp + jj * ystep;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc[q][t] = __builtin_fmaf(gv, yr[t], acc[q][t]);
+      }
+    }
+  }
+
+  // ---- epilogue: grad = (LOG ? exp(x - shift) : 1) * acc, staged for row-wise stores
+  __syncthreads();
+  float* ct = sl;  // [64][ld_own]
+#pragma unroll
+  for (int q = 0; q < kMaxKB; ++q) {
+    const int k0 = 8 * (wave + 4 * q);
+    if (k0 >= Wx) break;
+#pragma unroll
+    for (int t = 0; t < 8; ++t)
+      if (k0 + t < Wx)
+        ct[lane * ld_own + k0 + t] = LOG ? own[lane * ld_own + k0 + t] * acc[q][t] : acc[q][t];
+  }
+  __syncthreads();
+  for (int r = wave; r < kBT; r += 4) {
+    const int x = x0 + r;
+    if (x >= n) break;
+    if (LOG && badrow[r]) {  // recompute this row cell by cell from memory
+      for (int k = lane; k < Wx; k += 64) {
+        if (GRAD_A) band_bwd_a_cell<GENBMM_BAND_LOG>(p, bn + x, x, k);
+        else band_bwd_b_cell<GENBMM_BAND_LOG>(p, bn + x, x, k);
+      }
+    } else {
+      for (int k = lane; k < Wx; k += 64) gradb[(long)x * Wx + k] = ct[r * ld_own + k];
+    }
+  }
+}
+
+inline int bwd_sl_floats(const StripDims& d) { return max(kBR * d.ld_sl, kBT * d.ld_own); }
+inline size_t bwd_strip_bytes(const StripDims& d, bool log_mode) {
+  return sizeof(float) * ((log_mode ? (size_t)kBT * d.ld_own : 0) + (size_t)bwd_sl_floats(d) +
+                          (size_t)kBR * kBC + kBT + kBR + kBT);
+}
+
+inline StripDims strip_dims(int w_own, int w_sl) {
+  StripDims d;
+  d.ld_own = odd(w_own);
+  d.ld_sl = odd(w_sl + 2 * kBP);
+  d.bytes = sizeof(float) * ((size_t)kBT * d.ld_own + (size_t)kBR * d.ld_sl + kBT + kBR);
+  return d;
+}
+
+}  // namespace genbmm

@@ -12,7 +12,8 @@ pytestmark = pytest.mark.gpu
 
 # (n, a_lu, a_ld, b_lu, b_ld): bands narrower and wider than the matrix, empty sides
 BANDS = [(5, 1, 1, 2, 0), (6, 2, 1, 1, 3), (4, 3, 3, 3, 3), (7, 0, 2, 2, 0), (3, 4, 5, 5, 4),
-         (40, 3, 5, 4, 2), (33, 0, 0, 0, 0), (64, 8, 8, 8, 8), (1, 0, 0, 0, 0), (130, 17, 2, 5, 20)]
+         (40, 3, 5, 4, 2), (33, 0, 0, 0, 0), (64, 8, 8, 8, 8), (1, 0, 0, 0, 0), (130, 17, 2, 5, 20),
+         (257, 32, 32, 32, 32), (100, 60, 50, 40, 70)]
 
 
 def close(x, ref, rtol=1e-5, atol=1e-5):
@@ -55,6 +56,31 @@ def test_banded_forward_backward(gpu, n, a_lu, a_ld, b_lu, b_ld, mode):
     else:
         close(ga, wa)
         close(gb, wb)
+
+
+@pytest.mark.parametrize("n,a_lu,a_ld,b_lu,b_ld", [(70, 3, 5, 4, 2), (200, 20, 12, 9, 30), (64, 8, 8, 8, 8)])
+def test_banded_log_factoring_guard(gpu, n, a_lu, a_ld, b_lu, b_ld):
+    """Band rows whose maxima sit on cells that never meet: exp(a - rowmax) * exp(b - rowmax)
+    underflows although the true terms do not; those cells / gradient rows must be recomputed
+    exactly.  Also -inf entries (masked cells) and a fully masked row."""
+    torch.manual_seed(n)
+    a, b = pair(n, a_lu, a_ld, b_lu, b_ld)
+    a[:, ::3, 0] += 150.0            # first band cell of every third column of a
+    b[:, :, 0] -= 150.0
+    b[:, 1::4, -1] += 120.0
+    a[1, 5:9, 1:3] = -float("inf")   # masked cells
+    W = a.shape[2] + b.shape[2] - 1
+    g = torch.randn(3, n, W)
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    res = BandedMatrix(ad, a_lu, a_ld).multiply_log(BandedMatrix(bd, b_lu, b_ld))
+    want, _, _ = oracle.seq_band_fwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, 0, dtype=np.float64)
+    close(res.data, want)
+    ga, gb = torch.autograd.grad(res.data, (ad, bd), g.to(gpu))
+    wa, wb = oracle.seq_band_bwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, g.double(), 0, dtype=np.float64)
+    # |a|, |b| reach 150 here: one fp32 ulp of a + b - out is 1.5e-5, which is the
+    # relative accuracy any fp32 evaluation of exp(a + b - out) can have
+    close(ga, wa, rtol=1e-4, atol=1e-4)
+    close(gb, wb, rtol=1e-4, atol=1e-4)
 
 
 def test_banded_max_index_through_c_abi(gpu):
