@@ -98,75 +98,110 @@ __global__ __launch_bounds__(256) void k_log_bwdbwd_b(const BB p, long total) {
 // additions hitting a given cell therefore happen in the reference's order,
 // so the result is bit-identical, in O(M*N) work.  Products are rounded
 // before the add (the build uses -ffp-contract=on: no fusion across statements).
-constexpr int kKC = 128;  // gradient columns/rows accumulated per pass
+constexpr int kKC = 128;  // gradient columns/rows accumulated per workgroup
 
+// One wave: lane = row m of a 64-row tile, k in [c0, c0 + kKC).  The row is read
+// 16 cells at a time (int4 / float4 when the rows are 16-byte aligned), then the
+// 16 additions are made in order.
 template <bool PROD>
 __global__ __launch_bounds__(64) void k_argmax_bwd_a(const float* __restrict__ bmat,
                                                     const int32_t* __restrict__ idx,
                                                     const float* __restrict__ g,
                                                     float* __restrict__ grad_a, int M, int K,
-                                                    int N, int row_tiles) {
+                                                    int N, int row_tiles, int k_chunks, int vec) {
   __shared__ float accs[64 * (kKC + 1)];
   const int lane = threadIdx.x;
-  const int batch = blockIdx.x / row_tiles;
-  const int m0 = (blockIdx.x - batch * row_tiles) * 64;
+  const int kc_id = blockIdx.x % k_chunks, rt = blockIdx.x / k_chunks;
+  const int batch = rt / row_tiles;
+  const int m0 = (rt - batch * row_tiles) * 64;
+  const int c0 = kc_id * kKC, kc = min(kKC, K - c0);
   const int m = m0 + lane;
   const bool live = m < M;
   const int32_t* irow = idx + ((long)batch * M + (live ? m : 0)) * N;
   const float* grow = g + ((long)batch * M + (live ? m : 0)) * N;
   const float* bb = PROD ? bmat + (long)batch * K * N : nullptr;
   float* mine = accs + lane * (kKC + 1);
-  for (int c0 = 0; c0 < K; c0 += kKC) {
-    const int kc = min(kKC, K - c0);
-    for (int kk = 0; kk < kKC; ++kk) mine[kk] = 0.f;
-    if (live) {
-      for (int n = 0; n < N; ++n) {
-        const int k = irow[n] - c0;
-        if (k >= 0 && k < kc) {
-          float v = grow[n];
-          if (PROD) v = __fmul_rn(bb[(long)(k + c0) * N + n], v);
-          mine[k] = __fadd_rn(mine[k], v);
+  for (int kk = 0; kk < kKC; ++kk) mine[kk] = 0.f;
+  auto add = [&](int n, int ki, float gv) __attribute__((always_inline)) {
+    const int k = ki - c0;
+    if (k >= 0 && k < kc) {
+      float v = gv;
+      if (PROD) v = __fmul_rn(bb[(long)ki * N + n], v);
+      mine[k] = __fadd_rn(mine[k], v);
+    }
+  };
+  if (live) {
+    int n = 0;
+    if (vec) {
+      for (; n + 16 <= N; n += 16) {
+        int4 iv[4];
+        float4 gv[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          iv[q] = *reinterpret_cast<const int4*>(irow + n + 4 * q);
+          gv[q] = *reinterpret_cast<const float4*>(grow + n + 4 * q);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          add(n + 4 * q, iv[q].x, gv[q].x);
+          add(n + 4 * q + 1, iv[q].y, gv[q].y);
+          add(n + 4 * q + 2, iv[q].z, gv[q].z);
+          add(n + 4 * q + 3, iv[q].w, gv[q].w);
         }
       }
     }
-    __syncthreads();
-    const int rows = min(64, M - m0);
-    for (int r = 0; r < rows; ++r) {
-      float* dst = grad_a + ((long)batch * M + m0 + r) * K + c0;
-      for (int kk = lane; kk < kc; kk += 64) dst[kk] = accs[r * (kKC + 1) + kk];
-    }
-    __syncthreads();
+    for (; n < N; ++n) add(n, irow[n], grow[n]);
+  }
+  __syncthreads();
+  const int rows = min(64, M - m0);
+  for (int r = 0; r < rows; ++r) {
+    float* dst = grad_a + ((long)batch * M + m0 + r) * K + c0;
+    for (int kk = lane; kk < kc; kk += 64) dst[kk] = accs[r * (kKC + 1) + kk];
   }
 }
 
+// One wave: lane = column n of a 64-column tile, k in [c0, c0 + kKC); the column is
+// read 8 rows at a time (coalesced across the lanes), then added in order.
 template <bool PROD>
 __global__ __launch_bounds__(64) void k_argmax_bwd_b(const float* __restrict__ amat,
                                                     const int32_t* __restrict__ idx,
                                                     const float* __restrict__ g,
                                                     float* __restrict__ grad_b, int M, int K,
-                                                    int N, int col_tiles) {
+                                                    int N, int col_tiles, int k_chunks) {
   __shared__ float accs[kKC * 64];
   const int lane = threadIdx.x;
-  const int batch = blockIdx.x / col_tiles;
-  const int n = (blockIdx.x - batch * col_tiles) * 64 + lane;
+  const int kc_id = blockIdx.x % k_chunks, ct = blockIdx.x / k_chunks;
+  const int batch = ct / col_tiles;
+  const int n = (ct - batch * col_tiles) * 64 + lane;
+  const int c0 = kc_id * kKC, kc = min(kKC, K - c0);
   if (n >= N) return;  // lanes are independent: no barriers below
   const int32_t* icol = idx + (long)batch * M * N + n;
   const float* gcol = g + (long)batch * M * N + n;
   const float* ab = PROD ? amat + (long)batch * M * K : nullptr;
-  for (int c0 = 0; c0 < K; c0 += kKC) {
-    const int kc = min(kKC, K - c0);
-    for (int kk = 0; kk < kKC; ++kk) accs[kk * 64 + lane] = 0.f;
-    for (int m = 0; m < M; ++m) {
-      const int k = icol[(long)m * N] - c0;
-      if (k >= 0 && k < kc) {
-        float v = gcol[(long)m * N];
-        if (PROD) v = __fmul_rn(ab[(long)m * K + k + c0], v);
-        accs[k * 64 + lane] = __fadd_rn(accs[k * 64 + lane], v);
-      }
+  for (int kk = 0; kk < kKC; ++kk) accs[kk * 64 + lane] = 0.f;
+  auto add = [&](int m, int ki, float gv) __attribute__((always_inline)) {
+    const int k = ki - c0;
+    if (k >= 0 && k < kc) {
+      float v = gv;
+      if (PROD) v = __fmul_rn(ab[(long)m * K + ki], v);
+      accs[k * 64 + lane] = __fadd_rn(accs[k * 64 + lane], v);
     }
-    for (int kk = 0; kk < kc; ++kk)
-      grad_b[((long)batch * K + c0 + kk) * N + n] = accs[kk * 64 + lane];
+  };
+  int m = 0;
+  for (; m + 8 <= M; m += 8) {
+    int iv[8];
+    float gv[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      iv[q] = icol[(long)(m + q) * N];
+      gv[q] = gcol[(long)(m + q) * N];
+    }
+#pragma unroll
+    for (int q = 0; q < 8; ++q) add(m + q, iv[q], gv[q]);
   }
+  for (; m < M; ++m) add(m, icol[(long)m * N], gcol[(long)m * N]);
+  for (int kk = 0; kk < kc; ++kk)
+    grad_b[((long)batch * K + c0 + kk) * N + n] = accs[kk * 64 + lane];
 }
 
 template <bool PROD>
@@ -179,19 +214,20 @@ int run_argmax_bwd(const float* a, const float* b, const int32_t* idx, const flo
     return GENBMM_E_NULLPTR;
   hipStream_t s = (hipStream_t)stream;
   if ((int64_t)B * M * K > 0) {
-    const int row_tiles = ceil_div(M, 64);
-    const int64_t total = (int64_t)B * row_tiles;
+    const int row_tiles = ceil_div(M, 64), k_chunks = ceil_div(K, kKC);
+    const int64_t total = (int64_t)B * row_tiles * k_chunks;
     if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
+    const int vec = (N % 4 == 0) && aligned16(idx) && aligned16(g);
     hipLaunchKernelGGL((k_argmax_bwd_a<PROD>), dim3((unsigned)total), dim3(64), 0, s, b, idx, g,
-                       grad_a, M, K, N, row_tiles);
+                       grad_a, M, K, N, row_tiles, k_chunks, vec);
     if (int e = launch_status()) return e;
   }
   if ((int64_t)B * K * N > 0) {
-    const int col_tiles = ceil_div(N, 64);
-    const int64_t total = (int64_t)B * col_tiles;
+    const int col_tiles = ceil_div(N, 64), k_chunks = ceil_div(K, kKC);
+    const int64_t total = (int64_t)B * col_tiles * k_chunks;
     if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
     hipLaunchKernelGGL((k_argmax_bwd_b<PROD>), dim3((unsigned)total), dim3(64), 0, s, a, idx, g,
-                       grad_b, M, K, N, col_tiles);
+                       grad_b, M, K, N, col_tiles, k_chunks);
     if (int e = launch_status()) return e;
   }
   return GENBMM_OK;
