@@ -116,8 +116,10 @@ def dense_sample(lib, dev, B, M, K, N, reps):
     ga, gb = torch.empty_like(a), torch.empty_like(b)
     s, p = _lib.stream_of(a), _lib.ptr
 
+    stats = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=dev)
+
     def f():
-        _lib.check(lib.genbmm_samplebmm_fwd(p(a), p(b), p(out), p(idx), 1234, 0, B, M, K, N, s), "fwd")
+        _lib.check(lib.genbmm_samplebmm_fwd(p(a), p(b), p(out), p(idx), p(stats), 1234, 0, B, M, K, N, s), "fwd")
 
     def bw():
         _lib.check(lib.genbmm_argmax_bwd(p(idx), p(g), p(ga), p(gb), B, M, K, N, s), "bwd")

@@ -93,6 +93,118 @@ __global__ __launch_bounds__(C::NT) void k_sample_fwd(const DenseArgs p) {
   log_fwd_tile<C, true>(p, batch, m0, n0, As, Bs);
 }
 
+// Sampling sweep on top of a finished log-sum-exp (out) and the row / column
+// maxima alpha, beta (stats): with EA = exp(a - alpha), EB = exp(b - beta) staged
+// per tile, the unnormalised mass of term k is EA*EB and the target is
+// u * S, S = exp(out - alpha - beta): one multiply per (m,k,n) instead of an
+// exponential.  A tile in which any cell has S < 2^-40 (or is not finite) runs
+// the online routine + exact sweep instead.
+template <class C>
+__global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
+                                                           const float* __restrict__ stats) {
+  __shared__ __attribute__((aligned(16))) float smem[C::KT * (C::LDA + C::LDB) + C::BM + C::BN];
+  float* As = smem;
+  float* Bs = As + C::KT * C::LDA;
+  float* al = Bs + C::KT * C::LDB;
+  float* be = al + C::BM;
+  const int tid = threadIdx.x, tx = tid % C::TX, ty = tid / C::TX;
+  int batch, m0, n0;
+  decode_tile<C>(p, batch, m0, n0);
+  const int M = p.M, K = p.K, N = p.N;
+  const float* ab = p.a + (long)batch * M * K;
+  const float* bb = p.b + (long)batch * K * N;
+  const float* ob = p.out + (long)batch * M * N;
+  const float* st = stats + (long)batch * (M + N);
+  for (int t = tid; t < C::BM; t += C::NT) al[t] = (m0 + t < M) ? st[m0 + t] : 0.f;
+  for (int t = tid; t < C::BN; t += C::NT) be[t] = (n0 + t < N) ? st[M + n0 + t] : 0.f;
+  __syncthreads();
+
+  // tgt = u*S; the sampled index is the number of prefix sums that do not exceed it
+  // (prefix sums never decrease), which costs a multiply-add, a compare and an
+  // add-with-carry per term.
+  float tgt[C::TM][C::TN], cum[C::TM][C::TN];
+  int ind[C::TM][C::TN];
+  const float lim = 40.f * kLn2 + 1e-3f;
+  int bad = 0;
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) {
+      const int r = ty * C::TM + i, c = col_of<C>(tx, j);
+      const int m = m0 + r, n = n0 + c;
+      ind[i][j] = 0;
+      cum[i][j] = 0.f;
+      tgt[i][j] = 0.f;
+      if (m < M && n < N) {
+        const float e = al[r] + be[c] - ob[(long)m * N + n];   // -log S
+        if (!(e <= lim) || !(e > -INFINITY)) bad = 1;
+        const uint64_t cell = ((uint64_t)batch * M + m) * (uint64_t)N + n;
+        tgt[i][j] = philox_uniform(cell, p.seed, p.offset) * fast_exp2(-e * kLog2e);
+      }
+    }
+  if (__syncthreads_or(bad)) {  // workgroup-uniform
+    log_fwd_tile<C, true>(p, batch, m0, n0, As, Bs);
+    return;
+  }
+
+  using TA = TileOutMajor<C::BM, C::KT, C::NT>;
+  using TB = TileRedMajor<C::BN, C::KT, C::NT>;
+  TA ta;
+  TB tb;
+  if (K > 0) {
+    ta.gload(ab, K, m0, 0, M, K, p.vec_a, tid);
+    tb.gload(bb, N, n0, 0, N, K, p.vec_b, tid);
+  }
+  for (int k0 = 0; k0 < K; k0 += C::KT) {
+    __syncthreads();
+#pragma unroll
+    for (int l = 0; l < TA::PER; ++l) {
+      const float s = al[((tid + l * C::NT) / TA::C4) % C::BM];
+      ta.r[l].x = fast_exp2((ta.r[l].x - s) * kLog2e); ta.r[l].y = fast_exp2((ta.r[l].y - s) * kLog2e);
+      ta.r[l].z = fast_exp2((ta.r[l].z - s) * kLog2e); ta.r[l].w = fast_exp2((ta.r[l].w - s) * kLog2e);
+    }
+#pragma unroll
+    for (int l = 0; l < TB::PER; ++l) {
+      const float4 s = *reinterpret_cast<const float4*>(be + ((tid + l * C::NT) % TB::C4) * 4);
+      tb.r[l].x = fast_exp2((tb.r[l].x - s.x) * kLog2e); tb.r[l].y = fast_exp2((tb.r[l].y - s.y) * kLog2e);
+      tb.r[l].z = fast_exp2((tb.r[l].z - s.z) * kLog2e); tb.r[l].w = fast_exp2((tb.r[l].w - s.w) * kLog2e);
+    }
+    ta.sstore(As, tid);
+    tb.sstore(Bs, tid);
+    __syncthreads();
+    if (k0 + C::KT < K) {
+      ta.gload(ab, K, m0, k0 + C::KT, M, K, p.vec_a, tid);
+      tb.gload(bb, N, n0, k0 + C::KT, N, K, p.vec_b, tid);
+    }
+    const int kn = min(C::KT, K - k0);
+    auto scan = [&](int kk) __attribute__((always_inline)) {
+      float av[C::TM], bv[C::TN];
+      lds_frag<C::TM / 4>(As + kk * C::LDA, ty * C::TM, 4, av);
+      lds_frag<C::TN / 4>(Bs + kk * C::LDB, tx * 4, C::TX * 4, bv);
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) {
+          cum[i][j] = __builtin_fmaf(av[i], bv[j], cum[i][j]);
+          ind[i][j] += (cum[i][j] <= tgt[i][j]) ? 1 : 0;
+        }
+    };
+    if (kn == C::KT) {
+#pragma unroll 4
+      for (int kk = 0; kk < C::KT; ++kk) scan(kk);
+    } else {
+      for (int kk = 0; kk < kn; ++kk) scan(kk);
+    }
+  }
+  // rounding can leave the last prefix sum a hair under u*S: no crossing -> index 0,
+  // as when the reference's walk never exceeds its draw
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) ind[i][j] = ind[i][j] >= K ? 0 : ind[i][j];
+  store_tile_i<C>(p.idx + (long)batch * M * N, ind, m0, n0, M, N, p.vec_o, tx, ty);
+}
+
 // ---------------------------------------------------------------- dispatch
 template <class C, bool PROD>
 int launch_max(DenseArgs p, int B, int M, int K, int N, hipStream_t s) {
@@ -129,8 +241,16 @@ int run_max(const float* a, const float* b, float* out, int32_t* idx, int B, int
   }
 }
 
-int run_sample(const float* a, const float* b, float* out, int32_t* idx, uint64_t seed,
-               uint64_t offset, int B, int M, int K, int N, void* stream) {
+template <class C>
+int launch_sweep(DenseArgs p, const float* stats, int B, int M, int K, int N, hipStream_t s) {
+  dim3 grid;
+  if (int e = fill_args<C>(p, B, M, K, N, grid)) return e;
+  hipLaunchKernelGGL((k_sample_sweep<C>), grid, dim3(C::NT), 0, s, p, stats);
+  return launch_status();
+}
+
+int run_sample(const float* a, const float* b, float* out, int32_t* idx, float* stats,
+               uint64_t seed, uint64_t offset, int B, int M, int K, int N, void* stream) {
   if (int e = check_dense_dims(B, M, K, N)) return e;
   const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
   if (missing(a, mk) || missing(b, kn) || missing(out, mn) || missing(idx, mn))
@@ -139,6 +259,14 @@ int run_sample(const float* a, const float* b, float* out, int32_t* idx, uint64_
   DenseArgs p{};
   p.a = a; p.b = b; p.out = out; p.idx = idx; p.seed = seed; p.offset = offset;
   hipStream_t s = (hipStream_t)stream;
+  if (stats && K > 0) {  // log-sum-exp by the logbmm forward, then the multiply-only sweep
+    if (int e = genbmm_logbmm_fwd(a, b, out, stats, B, M, K, N, stream)) return e;
+    switch (pick_shape(B, M, N, false)) {
+      case kWide: return launch_sweep<CfgWide>(p, stats, B, M, K, N, s);
+      case kMid: return launch_sweep<CfgMid>(p, stats, B, M, K, N, s);
+      default: return launch_sweep<CfgSmall>(p, stats, B, M, K, N, s);
+    }
+  }
   switch (pick_shape(B, M, N, false)) {
     case kWide: return launch_sample<CfgWide>(p, B, M, K, N, s);
     case kMid: return launch_sample<CfgMid>(p, B, M, K, N, s);
@@ -151,9 +279,10 @@ int run_sample(const float* a, const float* b, float* out, int32_t* idx, uint64_
 
 extern "C" {
 
-int genbmm_samplebmm_fwd(const float* a, const float* b, float* out, int32_t* idx, uint64_t seed,
-                         uint64_t offset, int B, int M, int K, int N, void* stream) {
-  return genbmm::run_sample(a, b, out, idx, seed, offset, B, M, K, N, stream);
+int genbmm_samplebmm_fwd(const float* a, const float* b, float* out, int32_t* idx, float* stats,
+                         uint64_t seed, uint64_t offset, int B, int M, int K, int N,
+                         void* stream) {
+  return genbmm::run_sample(a, b, out, idx, stats, seed, offset, B, M, K, N, stream);
 }
 
 int genbmm_maxbmm_fwd(const float* a, const float* b, float* out, int32_t* idx, int B, int M,

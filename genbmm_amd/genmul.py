@@ -194,8 +194,11 @@ class SampleMatMul(torch.autograd.Function):
         seed, offset = _next_stream(a.device) if stream is None else stream
         out = torch.empty(B, M, N, dtype=_COMPUTE, device=a.device)
         idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
+        stats = torch.empty(_lib.load().genbmm_logbmm_stats_size(B, M, K, N), dtype=_COMPUTE,
+                            device=a.device)
         _call("genbmm_samplebmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
-              int(seed) & 0xFFFFFFFFFFFFFFFF, int(offset) & 0xFFFFFFFFFFFFFFFF, B, M, K, N)
+              _lib.ptr(stats), int(seed) & 0xFFFFFFFFFFFFFFFF, int(offset) & 0xFFFFFFFFFFFFFFFF,
+              B, M, K, N)
         empty = a.new_empty(0)
         ctx.save_for_backward(empty, empty, idx)
         ctx.dims, ctx.in_dtype = dims, in_dtype

@@ -143,9 +143,14 @@ int genbmm_prodmaxbmm_fwd(const float* a, const float* b, float* out,
  * A cell whose scan never crosses its uniform keeps index 0, as in the
  * reference.  Replaces _genbmm.forward(a, b, 2): matmul_cuda_kernel.cu:512-526
  * (torch::rand at :517), kernel :77-121.
+ * `stats`: NULL, or a buffer of genbmm_logbmm_stats_size(B,M,K,N) floats as for
+ * genbmm_logbmm_fwd; with it the log-sum-exp comes from the logbmm forward and
+ * the CDF walk multiplies staged exp(a-max)*exp(b-max) instead of taking one
+ * exponential per term (tiles where that is not exact walk the exact way).
  */
 int genbmm_samplebmm_fwd(const float* a, const float* b, float* out,
-                         int32_t* idx, uint64_t seed, uint64_t offset,
+                         int32_t* idx, float* stats,
+                         uint64_t seed, uint64_t offset,
                          int B, int M, int K, int N, void* stream);
 
 /*

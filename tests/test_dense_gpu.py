@@ -271,16 +271,20 @@ def test_max_config_c3(gpu):
 
 
 # -------------------------------------------------------------------- sample
-def test_sample_index_brackets_cdf(gpu):
+@pytest.mark.parametrize("use_stats", [True, False])
+@pytest.mark.parametrize("B,M,K,N", [(6, 20, 37, 24), (3, 130, 64, 132), (2, 64, 100, 128)])
+def test_sample_index_brackets_cdf(gpu, use_stats, B, M, K, N):
     torch.manual_seed(11)
-    B, M, K, N = 6, 20, 37, 24
     a, b = 2 * torch.randn(B, M, K), 2 * torch.randn(B, K, N)
+    a[0, ::2, 0] += 150.0      # batch item 0: the factored walk is not exact -> exact walk
+    b[0, 0, :] -= 150.0
     seed, offset = 1234, 5
     lib = _lib.load()
     ad, bd = a.to(gpu), b.to(gpu)
     out = torch.empty(B, M, N, device=gpu)
     idx = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
-    rc = lib.genbmm_samplebmm_fwd(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx),
+    stats = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=gpu) if use_stats else None
+    rc = lib.genbmm_samplebmm_fwd(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx), _lib.ptr(stats),
                                   seed, offset, B, M, K, N, _lib.stream_of(ad))
     assert rc == 0
     close(out, lse64(a, b))
@@ -298,10 +302,10 @@ def test_sample_index_brackets_cdf(gpu):
     assert bool(ok.all())
     # same stream -> same draw; other offset -> different draw
     idx2 = torch.empty_like(idx)
-    lib.genbmm_samplebmm_fwd(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx2),
+    lib.genbmm_samplebmm_fwd(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx2), _lib.ptr(stats),
                              seed, offset, B, M, K, N, _lib.stream_of(ad))
     assert torch.equal(idx, idx2)
-    lib.genbmm_samplebmm_fwd(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx2),
+    lib.genbmm_samplebmm_fwd(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx2), _lib.ptr(stats),
                              seed, offset + 1, B, M, K, N, _lib.stream_of(ad))
     assert not torch.equal(idx, idx2)
 
@@ -323,7 +327,8 @@ def test_sample_config_c4_chi_square(gpu):
     lib = _lib.load()
     idx = torch.empty(A.shape[0], 16, 16, dtype=torch.int32, device=gpu)
     o2 = torch.empty_like(out)
-    lib.genbmm_samplebmm_fwd(_lib.ptr(A), _lib.ptr(Bm), _lib.ptr(o2), _lib.ptr(idx), 1234, 0,
+    st = torch.empty(lib.genbmm_logbmm_stats_size(A.shape[0], 16, 512, 16), device=gpu)
+    lib.genbmm_samplebmm_fwd(_lib.ptr(A), _lib.ptr(Bm), _lib.ptr(o2), _lib.ptr(idx), _lib.ptr(st), 1234, 0,
                              A.shape[0], 16, 512, 16, _lib.stream_of(A))
     assert torch.equal(o2, out.detach())
     (gA,) = torch.autograd.grad(out.sum(), (A,))                      # one-hot rows summed over n
