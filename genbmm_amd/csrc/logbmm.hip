@@ -54,45 +54,73 @@ __device__ __forceinline__ float exp_comp(float d) {
 
 // ------------------------------------------------------------------ stats
 // stats[b][0..M) = max_k a[b,m,k],  stats[b][M..M+N) = max_k b[b,k,n].
+// Workgroups [0, row_wgs) of a batch item take kStatRows rows of a each (a wave
+// owns four rows and keeps their loads in flight together); the remaining
+// col_wgs take kStatCols columns of b each (8 float4 lanes across, 32 row
+// groups down, reduced through LDS).
+constexpr int kStatRows = 16, kStatCols = 32;
+
 __global__ __launch_bounds__(256) void k_log_stats(const float* __restrict__ a,
                                                    const float* __restrict__ b,
-                                                   float* __restrict__ stats, int M, int K, int N,
-                                                   int row_wgs, int col_wgs, int vec_a,
-                                                   int vec_b) {
-  __shared__ float part[8][128];
+                                                   float* __restrict__ stats, int* __restrict__ hdr,
+                                                   int M, int K, int N, int row_wgs, int col_wgs,
+                                                   int vec_a, int vec_b) {
+  __shared__ float part[32][kStatCols + 1];
+  if (blockIdx.x == 0 && threadIdx.x == 0) hdr[0] = 0;  // by-products of an earlier forward are stale
   const int per = row_wgs + col_wgs;
   const int batch = blockIdx.x / per;
   const int wg = blockIdx.x - batch * per;
   const int tid = threadIdx.x;
   float* st = stats + (long)batch * (M + N);
-  if (wg < row_wgs) {  // one wave per row of a
-    const int lane = tid & 63, m = wg * 4 + (tid >> 6);
-    if (m >= M) return;
-    const float* row = a + ((long)batch * M + m) * K;
-    float v = -INFINITY;
-    if (vec_a) {
+  if (wg < row_wgs) {
+    const int lane = tid & 63, m0 = wg * kStatRows + (tid >> 6) * 4;
+    const float* base = a + ((long)batch * M + m0) * K;
+    float v[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    if (vec_a && m0 + 3 < M) {
       for (int k = lane * 4; k < K; k += 256) {
-        const float4 x = *reinterpret_cast<const float4*>(row + k);
-        v = fmaxf(v, fmaxf(fmaxf(x.x, x.y), fmaxf(x.z, x.w)));
+        float4 x[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) x[r] = *reinterpret_cast<const float4*>(base + (long)r * K + k);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = fmaxf(v[r], fmaxf(fmaxf(x[r].x, x[r].y), fmaxf(x[r].z, x[r].w)));
       }
     } else {
-      for (int k = lane; k < K; k += 64) v = fmaxf(v, row[k]);
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (m0 + r < M)
+          for (int k = lane; k < K; k += 64) v[r] = fmaxf(v[r], base[(long)r * K + k]);
     }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-    if (lane == 0) st[m] = v;
-  } else {  // 128 columns of b: 32 column quads x 8 row groups
-    const int c4 = tid & 31, rg = tid >> 5;
-    const int n = (wg - row_wgs) * 128 + c4 * 4;
+    for (int r = 0; r < 4; ++r) {
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) v[r] = fmaxf(v[r], __shfl_xor(v[r], off, 64));
+      if (lane == 0 && m0 + r < M) st[m0 + r] = v[r];
+    }
+  } else {
+    const int c4 = tid & 7, rg = tid >> 3;
+    const int n = (wg - row_wgs) * kStatCols + c4 * 4;
     const float* col = b + (long)batch * K * N + n;
     float4 v = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
     if (n < N) {
-      for (int k = rg; k < K; k += 8) {
-        const float* p = col + (long)k * N;
-        if (vec_b) {
-          const float4 x = *reinterpret_cast<const float4*>(p);
+      if (vec_b) {
+        int k = rg;
+        for (; k + 96 < K; k += 128) {  // four rows in flight
+          float4 x[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) x[r] = *reinterpret_cast<const float4*>(col + (long)(k + 32 * r) * N);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            v.x = fmaxf(v.x, x[r].x); v.y = fmaxf(v.y, x[r].y);
+            v.z = fmaxf(v.z, x[r].z); v.w = fmaxf(v.w, x[r].w);
+          }
+        }
+        for (; k < K; k += 32) {
+          const float4 x = *reinterpret_cast<const float4*>(col + (long)k * N);
           v.x = fmaxf(v.x, x.x); v.y = fmaxf(v.y, x.y); v.z = fmaxf(v.z, x.z); v.w = fmaxf(v.w, x.w);
-        } else {
+        }
+      } else {
+        for (int k = rg; k < K; k += 32) {
+          const float* p = col + (long)k * N;
           v.x = fmaxf(v.x, p[0]);
           if (n + 1 < N) v.y = fmaxf(v.y, p[1]);
           if (n + 2 < N) v.z = fmaxf(v.z, p[2]);
@@ -103,12 +131,12 @@ __global__ __launch_bounds__(256) void k_log_stats(const float* __restrict__ a,
     part[rg][c4 * 4 + 0] = v.x; part[rg][c4 * 4 + 1] = v.y;
     part[rg][c4 * 4 + 2] = v.z; part[rg][c4 * 4 + 3] = v.w;
     __syncthreads();
-    if (tid < 128) {
-      const int nn = (wg - row_wgs) * 128 + tid;
+    if (tid < kStatCols) {
+      const int nn = (wg - row_wgs) * kStatCols + tid;
       if (nn < N) {
         float r = part[0][tid];
 #pragma unroll
-        for (int q = 1; q < 8; ++q) r = fmaxf(r, part[q][tid]);
+        for (int q = 1; q < 32; ++q) r = fmaxf(r, part[q][tid]);
         st[M + nn] = r;
       }
     }
@@ -232,45 +260,46 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_fwd_fast(const DenseArgs p,
 
 // Recompute the flagged tiles of a factored forward launch with the online
 // routine.  FBM x FBN is the factored launch's tile, CX the exact routine's
-// tile (CX::BN == FBN, NX * CX::BM == FBM).  Workgroups stride over the tile list.
-template <class CX, int NX, int FBM, int FBN>
+// tile (which divides it).  Workgroups stride over the tile list.
+template <class CX, int FBM, int FBN>
 __global__ __launch_bounds__(CX::NT) void k_log_fwd_fixup(const DenseArgs p,
                                                           const int* __restrict__ flags,
                                                           int total_tiles) {
-  static_assert(CX::BN == FBN && CX::BM * NX == FBM, "");
+  static_assert(FBM % CX::BM == 0 && FBN % CX::BN == 0, "");
   __shared__ __attribute__((aligned(16))) float smem[CX::KT * (CX::LDA + CX::LDB)];
   const int per = p.tiles_m * p.tiles_n;  // of the factored launch
   for (int t = blockIdx.x; t < total_tiles; t += gridDim.x) {
     if (!flags[t]) continue;
     const int batch = t / per, r = t - batch * per;
     const int m0 = (r / p.tiles_n) * FBM, n0 = (r % p.tiles_n) * FBN;
-#pragma unroll
-    for (int h = 0; h < NX; ++h)
-      if (m0 + h * CX::BM < p.M) {
-        log_fwd_tile<CX, false>(p, batch, m0 + h * CX::BM, n0, smem, smem + CX::KT * CX::LDA);
-        __syncthreads();
-      }
+    for (int h = 0; h < FBM / CX::BM; ++h)
+      for (int w = 0; w < FBN / CX::BN; ++w)
+        if (m0 + h * CX::BM < p.M && n0 + w * CX::BN < p.N) {
+          log_fwd_tile<CX, false>(p, batch, m0 + h * CX::BM, n0 + w * CX::BN, smem,
+                                  smem + CX::KT * CX::LDA);
+          __syncthreads();
+        }
   }
 }
 
-template <class CX, int NX, int FBR, int FBC, bool GRAD_A>
+template <class CX, int FBR, int FBC, bool GRAD_A>
 __global__ __launch_bounds__(CX::NT) void k_log_bwd_fixup(const LogBwdArgs p,
                                                           const int* __restrict__ flags,
                                                           int total_tiles) {
-  static_assert(CX::BC == FBC && CX::BR * NX == FBR, "");
+  static_assert(FBR % CX::BR == 0 && FBC % CX::BC == 0, "");
   __shared__ __attribute__((aligned(16))) float smem[LogBwdLds<CX, GRAD_A>::FLOATS];
   const int per = p.tiles_r * p.tiles_c;  // of the factored launch
-  const int R = GRAD_A ? p.M : p.K;
+  const int R = GRAD_A ? p.M : p.K, Cc = GRAD_A ? p.K : p.N;
   for (int t = blockIdx.x; t < total_tiles; t += gridDim.x) {
     if (!flags[t]) continue;
     const int batch = t / per, r = t - batch * per;
     const int r0 = (r / p.tiles_c) * FBR, c0 = (r % p.tiles_c) * FBC;
-#pragma unroll
-    for (int h = 0; h < NX; ++h)
-      if (r0 + h * CX::BR < R) {
-        log_bwd_tile<CX, GRAD_A>(p, batch, r0 + h * CX::BR, c0, smem);
-        __syncthreads();
-      }
+    for (int h = 0; h < FBR / CX::BR; ++h)
+      for (int w = 0; w < FBC / CX::BC; ++w)
+        if (r0 + h * CX::BR < R && c0 + w * CX::BC < Cc) {
+          log_bwd_tile<CX, GRAD_A>(p, batch, r0 + h * CX::BR, c0 + w * CX::BC, smem);
+          __syncthreads();
+        }
   }
 }
 
@@ -481,15 +510,37 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_bwd_fast(const LogBwdArgs p,
 std::atomic<int> g_path{0};  // 0 default, 1 exact only, 2 factored without matrix cores
 constexpr int kFixupGrid = 1024;
 
-// Layout of the caller's stats buffer: B*(M+N) shifts, then one int flag per
-// 32x32 tile of (M,N), of (M,K) and of (K,N) (an upper bound on any launch's
-// tile count).
+// Layout of the caller's stats buffer: B*(M+N) shifts; one int flag per 32x32
+// tile of (M,N), of (M,K) and of (K,N) (an upper bound on any launch's tile
+// count); a header of four ints; and, for shapes the matrix-core forward can
+// take, its by-products EA (B*M*K), EB (B*K*N) and R (B*M*N) on a 16-byte
+// boundary.
 inline int64_t tiles32(int B, int X, int Y) { return (int64_t)B * ceil_div(X, 32) * ceil_div(Y, 32); }
 inline int* flags_of(const float* stats, int B, int M, int K, int N, int which) {
   int* f = reinterpret_cast<int*>(const_cast<float*>(stats) + (int64_t)B * (M + N));
   if (which >= 1) f += tiles32(B, M, N);
   if (which >= 2) f += tiles32(B, M, K);
+  if (which >= 3) f += tiles32(B, K, N);
   return f;
+}
+inline int64_t header_offset(int B, int M, int K, int N) {
+  const int64_t o = (int64_t)B * (M + N) + tiles32(B, M, N) + tiles32(B, M, K) + tiles32(B, K, N);
+  return (o + 3) & ~(int64_t)3;
+}
+// Shapes whose forward runs on the matrix cores (given alignment and path).
+inline bool fwd_mfma_shape(int B, int M, int K, int N) {
+  if (K <= 0 || K % kMS != 0 || M % 128 != 0 || N % 128 != 0 || M == 0 || N == 0) return false;
+  const int64_t t128 = (int64_t)B * (M / 128) * (N / 128);
+  return t128 >= 128 && t128 <= 0x7fffffff;
+}
+inline LogPrepared prepared_of(const float* stats, int B, int M, int K, int N) {
+  float* base = const_cast<float*>(stats) + header_offset(B, M, K, N);
+  LogPrepared w;
+  w.hdr = reinterpret_cast<int*>(base);
+  w.ea = base + 4;
+  w.eb = w.ea + (int64_t)B * M * K;
+  w.r = w.eb + (int64_t)B * K * N;
+  return w;
 }
 
 template <class C>
@@ -500,41 +551,47 @@ int launch_fwd_exact(DenseArgs p, int B, int M, int K, int N, hipStream_t s) {
   return launch_status();
 }
 
-template <class CX, int NX, int FBM, int FBN>
+template <class CX, int FBM, int FBN>
 int launch_fwd_fixup(const DenseArgs& p, const int* flags, int tiles, hipStream_t s) {
-  hipLaunchKernelGGL((k_log_fwd_fixup<CX, NX, FBM, FBN>), dim3(min(tiles, kFixupGrid)),
+  hipLaunchKernelGGL((k_log_fwd_fixup<CX, FBM, FBN>), dim3(min(tiles, kFixupGrid)),
                      dim3(CX::NT), 0, s, p, flags, tiles);
   return launch_status();
 }
 
-template <class C, class CX, int NX>
+template <class C, class CX>
 int launch_fwd_fast(DenseArgs p, const float* stats, int* flags, int B, int M, int K, int N,
                     hipStream_t s) {
   dim3 grid;
   if (int e = fill_args<C>(p, B, M, K, N, grid)) return e;
   hipLaunchKernelGGL((k_log_fwd_fast<C>), grid, dim3(C::NT), 0, s, p, stats, flags);
   if (int e = launch_status()) return e;
-  return launch_fwd_fixup<CX, NX, C::BM, C::BN>(p, flags, (int)grid.x, s);
+  return launch_fwd_fixup<CX, C::BM, C::BN>(p, flags, (int)grid.x, s);
 }
 
+// Matrix-core launches: T is the MTile; the problem is made of full tiles.
+template <class T>
 int launch_fwd_mfma(DenseArgs p, const float* stats, int* flags, int B, int M, int K, int N,
                     hipStream_t s) {
-  dim3 grid;
-  if (int e = fill_args<CfgBig>(p, B, M, K, N, grid)) return e;
-  hipLaunchKernelGGL(k_log_fwd_mfma, grid, dim3(256), 0, s, p.a, p.b, p.out, stats, flags, M, K, N,
-                     p.tiles_m, p.tiles_n);
+  p.M = M; p.K = K; p.N = N;
+  p.tiles_m = M / T::TR;
+  p.tiles_n = N / T::TC;
+  p.vec_a = p.vec_b = p.vec_o = 1;
+  const int total = B * p.tiles_m * p.tiles_n;
+  const LogPrepared ws = prepared_of(stats, B, M, K, N);
+  hipLaunchKernelGGL((k_log_fwd_mfma<T>), dim3(total), dim3(T::NT), 0, s, p.a, p.b, p.out, stats,
+                     flags, ws.ea, ws.eb, ws.r, ws.hdr, M, K, N, p.tiles_m, p.tiles_n);
   if (int e = launch_status()) return e;
-  return launch_fwd_fixup<CfgWide, 2, 128, 128>(p, flags, (int)grid.x, s);
+  return launch_fwd_fixup<CfgWide, T::TR, T::TC>(p, flags, total, s);
 }
 
 int launch_stats(const float* a, const float* b, float* stats, int B, int M, int K, int N,
                  hipStream_t s) {
-  const int row_wgs = ceil_div(M, 4), col_wgs = ceil_div(N, 128);
+  const int row_wgs = ceil_div(M, kStatRows), col_wgs = ceil_div(N, kStatCols);
   const int64_t total = (int64_t)B * (row_wgs + col_wgs);
   if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
   if (total == 0) return GENBMM_OK;
-  hipLaunchKernelGGL(k_log_stats, dim3((unsigned)total), dim3(256), 0, s, a, b, stats, M, K, N,
-                     row_wgs, col_wgs, (int)((K % 4 == 0) && aligned16(a)),
+  hipLaunchKernelGGL(k_log_stats, dim3((unsigned)total), dim3(256), 0, s, a, b, stats,
+                     prepared_of(stats, B, M, K, N).hdr, M, K, N, row_wgs, col_wgs, (int)((K % 4 == 0) && aligned16(a)),
                      (int)((N % 4 == 0) && aligned16(b)));
   return launch_status();
 }
@@ -550,30 +607,52 @@ int launch_bwd_exact(LogBwdArgs p, int B, hipStream_t s) {
   return launch_status();
 }
 
-template <class C, class CX, int NX, bool GRAD_A, bool MFMA>
+template <class C, class CX, bool GRAD_A>
 int launch_bwd_fast(LogBwdArgs p, const float* stats, int* flags, int B, hipStream_t s) {
   const int R = GRAD_A ? p.M : p.K, Cc = GRAD_A ? p.K : p.N;
   p.tiles_r = ceil_div(R, C::BR);
   p.tiles_c = ceil_div(Cc, C::BC);
   const int64_t total = (int64_t)B * p.tiles_r * p.tiles_c;
   if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
-  if (MFMA)
-    hipLaunchKernelGGL((k_log_bwd_mfma<GRAD_A>), dim3((unsigned)total), dim3(256), 0, s, p.a, p.b,
-                       p.out, p.g, stats, p.grad, flags, p.M, p.K, p.N, p.tiles_r, p.tiles_c);
-  else
-    hipLaunchKernelGGL((k_log_bwd_fast<C, GRAD_A>), dim3((unsigned)total), dim3(C::NT), 0, s, p,
-                       stats, flags);
+  hipLaunchKernelGGL((k_log_bwd_fast<C, GRAD_A>), dim3((unsigned)total), dim3(C::NT), 0, s, p,
+                     stats, flags);
   if (int e = launch_status()) return e;
-  hipLaunchKernelGGL((k_log_bwd_fixup<CX, NX, C::BR, C::BC, GRAD_A>),
+  hipLaunchKernelGGL((k_log_bwd_fixup<CX, C::BR, C::BC, GRAD_A>),
                      dim3(min((int)total, kFixupGrid)), dim3(CX::NT), 0, s, p, flags, (int)total);
   return launch_status();
 }
 
-// All tiles full and every access 16-byte aligned: the matrix-core kernels apply.
-inline bool mfma_ok(int out_r, int out_c, int red, bool aligned, int64_t tiles) {
-  return g_path.load() == 0 && aligned && red > 0 && out_r % 128 == 0 && out_c % 128 == 0 &&
-         red % 16 == 0 && tiles >= 128;
+template <class T, bool GRAD_A>
+int launch_bwd_mfma(LogBwdArgs p, const float* stats, int* flags, int B, hipStream_t s) {
+  const int R = GRAD_A ? p.M : p.K, Cc = GRAD_A ? p.K : p.N;
+  p.tiles_r = R / T::TR;
+  p.tiles_c = Cc / T::TC;
+  const int total = B * p.tiles_r * p.tiles_c;
+  const LogPrepared ws = prepared_of(stats, B, p.M, p.K, p.N);
+  hipLaunchKernelGGL((k_log_bwd_mfma<T, GRAD_A>), dim3(total), dim3(T::NT), 0, s, p.g, ws.ea, ws.eb,
+                     ws.r, ws.hdr, flags_of(stats, B, p.M, p.K, p.N, 0), p.grad, flags, p.M, p.K,
+                     p.N, p.tiles_r, p.tiles_c);
+  if (int e = launch_status()) return e;
+  hipLaunchKernelGGL((k_log_bwd_fixup<BCfgWide, T::TR, T::TC, GRAD_A>),
+                     dim3(min(total, kFixupGrid)), dim3(BCfgWide::NT), 0, s, p, flags, total);
+  return launch_status();
 }
+
+// All tiles full and every access 16-byte aligned: the matrix-core kernels apply.
+// Returns 2 for the 256-wide tile (enough tiles to give every compute unit two
+// workgroups of eight waves), 1 for 128x128, 0 for neither.  `long_cols`: the
+// 256 side is the column side of the output.
+inline int mfma_kind(int B, int out_r, int out_c, int red, bool aligned, bool long_cols) {
+  if (g_path.load() != 0 || !aligned || red <= 0 || red % kMS != 0) return 0;
+  if (out_r % 128 != 0 || out_c % 128 != 0) return 0;
+  const int64_t t128 = (int64_t)B * (out_r / 128) * (out_c / 128);
+  if ((long_cols ? out_c : out_r) % 256 == 0 && t128 >= 1024 && t128 / 2 <= 0x7fffffff) return 2;
+  return t128 >= 128 && t128 <= 0x7fffffff ? 1 : 0;
+}
+
+using MT128 = MTile<128, 128>;
+using MTWide = MTile<128, 256>;  // forward (m x n) and grad_a (m x k)
+using MTTall = MTile<256, 128>;  // grad_b (k x n)
 
 template <bool GRAD_A>
 int run_bwd(const LogBwdArgs& p, const float* stats, int B, hipStream_t s) {
@@ -584,12 +663,18 @@ int run_bwd(const LogBwdArgs& p, const float* stats, int B, hipStream_t s) {
   if (stats) {
     int* fl = flags_of(stats, B, p.M, p.K, p.N, GRAD_A ? 1 : 2);
     const bool al = p.vec_k && p.vec_n && aligned16(stats) && p.M % 4 == 0 && p.N % 4 == 0;
-    if (mfma_ok(R, Cc, Q, al, wgs(128, 128)))
-      return launch_bwd_fast<BCfgBig, BCfgWide, 2, GRAD_A, true>(p, stats, fl, B, s);
-    if (small) return launch_bwd_fast<BCfgSmall, BCfgSmall, 1, GRAD_A, false>(p, stats, fl, B, s);
+    // the matrix-core kernels run on what the matrix-core forward left behind
+    switch (fwd_mfma_shape(B, p.M, p.K, p.N) ? mfma_kind(B, R, Cc, Q, al, GRAD_A) : 0) {
+      case 2:
+        if constexpr (GRAD_A) return launch_bwd_mfma<MTWide, true>(p, stats, fl, B, s);
+        else return launch_bwd_mfma<MTTall, false>(p, stats, fl, B, s);
+      case 1: return launch_bwd_mfma<MT128, GRAD_A>(p, stats, fl, B, s);
+      default: break;
+    }
+    if (small) return launch_bwd_fast<BCfgSmall, BCfgSmall, GRAD_A>(p, stats, fl, B, s);
     if (R >= 128 && Cc >= 128 && wgs(128, 128) >= 512)
-      return launch_bwd_fast<BCfgBig, BCfgWide, 2, GRAD_A, false>(p, stats, fl, B, s);
-    return launch_bwd_fast<BCfgMid, BCfgMid, 1, GRAD_A, false>(p, stats, fl, B, s);
+      return launch_bwd_fast<BCfgBig, BCfgWide, GRAD_A>(p, stats, fl, B, s);
+    return launch_bwd_fast<BCfgMid, BCfgMid, GRAD_A>(p, stats, fl, B, s);
   }
   if (small) return launch_bwd_exact<BCfgSmall, GRAD_A>(p, B, s);
   if (R >= 64 && Cc >= 128 && wgs(64, 128) >= 512) return launch_bwd_exact<BCfgWide, GRAD_A>(p, B, s);
@@ -604,7 +689,9 @@ extern "C" {
 size_t genbmm_logbmm_stats_size(int B, int M, int K, int N) {
   using namespace genbmm;
   if (check_dense_dims(B, M, K, N)) return 0;
-  return (size_t)((int64_t)B * (M + N) + tiles32(B, M, N) + tiles32(B, M, K) + tiles32(B, K, N));
+  int64_t n = header_offset(B, M, K, N) + 4;
+  if (fwd_mfma_shape(B, M, K, N)) n += (int64_t)B * ((int64_t)M * K + (int64_t)K * N + (int64_t)M * N);
+  return (size_t)n;
 }
 
 void genbmm_logbmm_force_exact(int on) { genbmm::g_path.store(on == 1 || on == 2 ? on : 0); }
@@ -626,12 +713,15 @@ int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats, 
     int* fl = flags_of(stats, B, M, K, N, 0);
     const int64_t big_tiles = (int64_t)B * ceil_div(M, 128) * ceil_div(N, 128);
     const bool al = K % 4 == 0 && N % 4 == 0 && aligned16(a) && aligned16(b) && aligned16(stats);
-    if (mfma_ok(M, N, K, al, big_tiles)) return launch_fwd_mfma(p, stats, fl, B, M, K, N, s);
-    if (M <= 32 && N <= 32)
-      return launch_fwd_fast<CfgSmall, CfgSmall, 1>(p, stats, fl, B, M, K, N, s);
+    switch (fwd_mfma_shape(B, M, K, N) ? mfma_kind(B, M, N, K, al, true) : 0) {
+      case 2: return launch_fwd_mfma<MTWide>(p, stats, fl, B, M, K, N, s);
+      case 1: return launch_fwd_mfma<MT128>(p, stats, fl, B, M, K, N, s);
+      default: break;
+    }
+    if (M <= 32 && N <= 32) return launch_fwd_fast<CfgSmall, CfgSmall>(p, stats, fl, B, M, K, N, s);
     if (M >= 128 && N >= 128 && big_tiles >= 512)
-      return launch_fwd_fast<CfgBig, CfgWide, 2>(p, stats, fl, B, M, K, N, s);
-    return launch_fwd_fast<CfgMid, CfgMid, 1>(p, stats, fl, B, M, K, N, s);
+      return launch_fwd_fast<CfgBig, CfgWide>(p, stats, fl, B, M, K, N, s);
+    return launch_fwd_fast<CfgMid, CfgMid>(p, stats, fl, B, M, K, N, s);
   }
   switch (pick_shape(B, M, N, false)) {
     case kWide: return launch_fwd_exact<CfgWide>(p, B, M, K, N, s);

@@ -25,14 +25,16 @@ __device__ __forceinline__ floatx16 mfma_32x32x2(float a, float b, floatx16 c) {
 __device__ __forceinline__ int mfma_row(int i, int lane) {
   return 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
 }
+// The same split into a part that is uniform over the wave and the lane's part.
+__device__ __forceinline__ constexpr int mfma_row_u(int i) { return 8 * (i >> 2) + (i & 3); }
+__device__ __forceinline__ int mfma_row_l(int lane) { return 4 * (lane >> 5); }
 
-constexpr int kMT = 128;        // tile edge
 constexpr int kMS = 16;         // slab depth
-constexpr int kMLD = kMT + 4;   // LDS row stride of a [slab][tile] buffer
+constexpr int kMPad = 4;        // LDS row padding (floats) of a [slab][tile] buffer
 constexpr float kMfmaGuardBits = 40.f;
 
 // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
-// Renumber them so that every XCD works on one contiguous run of tiles (the 16
+// Renumber them so that every XCD works on one contiguous run of tiles (the
 // tiles of a batch item share their operands).
 __device__ __forceinline__ int xcd_tile_id() {
   const int w = blockIdx.x, n = gridDim.x;
@@ -41,57 +43,186 @@ __device__ __forceinline__ int xcd_tile_id() {
 
 __device__ __forceinline__ float exp_st(float d) { return fast_exp2(d * kLog2e); }
 
-// 32 matrix-core steps over one staged slab: rows from R[q][0..128), columns
-// from Cs[q][0..128).
+// The matrix-core instruction runs on the same lanes as ordinary vector
+// instructions (the hardware counters show no cycle of overlap), so every
+// vector instruction spent on staging is taken from the contraction.  A tile is
+// therefore TR x TC with one side 256 when the problem allows: each staged
+// element then serves twice as many products, and the side whose staging is
+// dearer (H in the backward kernels, the transposed stores elsewhere) is the
+// short one.  (TR/64) x (TC/64) waves, each keeping a 64x64 block as 2x2
+// accumulators of v_mfma_f32_32x32x2_f32.
+template <int TR_, int TC_, int WPE_ = 4>
+struct MTile {
+  static constexpr int TR = TR_, TC = TC_;
+  static constexpr int WPE = WPE_;              // waves per SIMD the kernel is compiled for
+  static constexpr int WC = TC / 64;            // waves across
+  static constexpr int NT = (TR / 64) * WC * 64;
+  static constexpr int LDR = TR + kMPad, LDC = TC + kMPad;
+};
+
+// 32 matrix-core steps over one staged slab: rows from R[q][0..TR), columns
+// from Cs[q][0..TC).
+template <int LDR, int LDC>
 __device__ __forceinline__ void mfma_slab(const float* __restrict__ R, const float* __restrict__ Cs,
                                           int wr0, int wc0, int lane, floatx16 (&acc)[2][2]) {
   const int lrow = lane & 31, lk = lane >> 5;
-  const float* rp = R + lk * kMLD + wr0 + lrow;
-  const float* cp = Cs + lk * kMLD + wc0 + lrow;
+  const float* rp = R + lk * LDR + wr0 + lrow;
+  const float* cp = Cs + lk * LDC + wc0 + lrow;
+  // operands of step q+2 are read while the four products of step q run
+  float fa[2][2], fb[2][2];
+  fa[0][0] = rp[0]; fa[0][1] = rp[32];
+  fb[0][0] = cp[0]; fb[0][1] = cp[32];
+  __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
 #pragma unroll
   for (int q = 0; q < kMS; q += 2) {
-    const float a0 = rp[q * kMLD], a1 = rp[q * kMLD + 32];
-    const float b0 = cp[q * kMLD], b1 = cp[q * kMLD + 32];
-    acc[0][0] = mfma_32x32x2(a0, b0, acc[0][0]);
-    acc[0][1] = mfma_32x32x2(a0, b1, acc[0][1]);
-    acc[1][0] = mfma_32x32x2(a1, b0, acc[1][0]);
-    acc[1][1] = mfma_32x32x2(a1, b1, acc[1][1]);
+    const int c = (q >> 1) & 1, n = c ^ 1;
+    if (q + 2 < kMS) {
+      fa[n][0] = rp[(q + 2) * LDR]; fa[n][1] = rp[(q + 2) * LDR + 32];
+      fb[n][0] = cp[(q + 2) * LDC]; fb[n][1] = cp[(q + 2) * LDC + 32];
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+    acc[0][0] = mfma_32x32x2(fa[c][0], fb[c][0], acc[0][0]);
+    acc[0][1] = mfma_32x32x2(fa[c][0], fb[c][1], acc[0][1]);
+    acc[1][0] = mfma_32x32x2(fa[c][1], fb[c][0], acc[1][0]);
+    acc[1][1] = mfma_32x32x2(fa[c][1], fb[c][1], acc[1][1]);
+    __builtin_amdgcn_sched_group_barrier(0x8, 4, 0);
   }
 }
 
-// Store a float4 read along the reduction axis of an [out][red] tile into a
-// [red][out] LDS buffer (transposing), and one read along the out axis of a
-// [red][out] tile (straight).
-__device__ __forceinline__ void lds_put_t(float* __restrict__ buf, int out, int red4, float4 v) {
-  float* p = buf + (red4 * 4) * kMLD + out;
-  p[0] = v.x; p[kMLD] = v.y; p[2 * kMLD] = v.z; p[3 * kMLD] = v.w;
+// A staged operand tile of OUT lines x kMS reduction steps, one float4 per
+// thread and piece.  Transposed: the source is [out][red] (float4 along red,
+// four scalar LDS stores);  straight: the source is [red][out] (float4 along
+// out, one 16-byte store).
+template <int OUT, int NT, int LD>
+struct StageT {
+  static constexpr int PER = OUT * 4 / NT;
+  static constexpr int STEP = NT / 4;  // source lines between a thread's pieces
+  static_assert(PER >= 1 && OUT * 4 % NT == 0, "");
+  static __device__ __forceinline__ int line(int tid, int l) { return (tid >> 2) + l * (NT / 4); }
+  static __device__ __forceinline__ int quad(int tid) { return tid & 3; }
+  static __device__ __forceinline__ void put(float* __restrict__ buf, int tid, int l, float4 v) {
+    float* p = buf + (quad(tid) * 4) * LD + line(tid, l);
+    p[0] = v.x; p[LD] = v.y; p[2 * LD] = v.z; p[3 * LD] = v.w;
+  }
+};
+template <int OUT, int NT, int LD>
+struct StageS {
+  static constexpr int Q = OUT / 4;
+  static constexpr int PER = kMS * Q / NT;
+  static constexpr int STEP = NT / Q;  // source lines between a thread's pieces
+  static_assert(PER >= 1 && kMS * Q % NT == 0 && NT % Q == 0, "");
+  static __device__ __forceinline__ int red(int tid, int l) { return tid / Q + l * (NT / Q); }
+  static __device__ __forceinline__ int quad(int tid) { return tid % Q; }
+  static __device__ __forceinline__ void put(float* __restrict__ buf, int tid, int l, float4 v) {
+    *reinterpret_cast<float4*>(buf + red(tid, l) * LD + quad(tid) * 4) = v;
+  }
+};
+
+__device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 exp4(float4 x, float4 s) {
+  return make_float4(exp_st(x.x - s.x), exp_st(x.y - s.y), exp_st(x.z - s.z), exp_st(x.w - s.w));
 }
-__device__ __forceinline__ void lds_put(float* __restrict__ buf, int red, int out4, float4 v) {
-  *reinterpret_cast<float4*>(buf + red * kMLD + out4 * 4) = v;
+__device__ __forceinline__ float4 exp4(float4 x, float s) {
+  return make_float4(exp_st(x.x - s), exp_st(x.y - s), exp_st(x.z - s), exp_st(x.w - s));
+}
+
+// What the forward leaves in the caller's workspace for the backward kernels:
+// EA = exp(a - alpha), EB = exp(b - beta) (each written by the tiles of the
+// first column / row block while they stage them anyway) and R = 1/S per output
+// cell, so that the backward contraction needs no exponential at all:
+// H = g * R.  hdr[0] = 1 once they are valid, hdr[1], hdr[2] = the forward's
+// tile shape (its flags tell which cells of R are not usable).  The kernels take
+// the members as separate __restrict__ parameters: through a struct the
+// compiler must assume that they alias the output and serialises the epilogue.
+struct LogPrepared {
+  float* ea;
+  float* eb;
+  float* r;
+  int* hdr;
+};
+
+// Compiler-level ordering point for a wave's own LDS traffic (the hardware
+// executes one wave's LDS instructions in order).
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
+constexpr int kStripFloats = 16 * 64;  // per wave: 16 rows of its 64-column block
+
+// Hands a wave's 64x64 accumulator block back in row-major order, so that global
+// memory is touched 16 bytes per lane and 256 contiguous bytes per row instead
+// of 4 and 128: f(q, t, v) receives, for quarter q = 0..3 and t = 0..3, the four
+// consecutive columns (lane & 15) * 4 .. +3 of block row 16*q + 4*t + (lane >> 4).
+// `pre(q)` runs before quarter q is exchanged (a place to start loads).  The
+// exchange goes through a wave-private LDS strip; the caller guarantees that no
+// wave still reads the staging buffers the strip overlays.
+template <class P, class F>
+__device__ __forceinline__ void acc_rows(const floatx16 (&acc)[2][2], float* __restrict__ strip,
+                                         int lane, P&& pre, F&& f) {
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    pre(q);
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        strip[(mfma_row_u(i) + mfma_row_l(lane)) * 64 + c * 32 + (lane & 31)] =
+            acc[q >> 1][c][(q & 1) * 8 + i];
+    wave_lds_sync();
+    float4 v[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      v[t] = *reinterpret_cast<const float4*>(strip + ((lane >> 4) + 4 * t) * 64 + (lane & 15) * 4);
+    wave_lds_sync();
+#pragma unroll
+    for (int t = 0; t < 4; ++t) f(q, t, v[t]);
+  }
 }
 
 // ----------------------------------------------------------------- forward
-__global__ __launch_bounds__(256, 4) void k_log_fwd_mfma(const float* __restrict__ a,
-                                                         const float* __restrict__ b,
-                                                         float* __restrict__ out,
-                                                         const float* __restrict__ stats,
-                                                         int* __restrict__ flags, int M, int K,
-                                                         int N, int tiles_m, int tiles_n) {
-  __shared__ __attribute__((aligned(16))) float As[2][kMS * kMLD];
-  __shared__ __attribute__((aligned(16))) float Bs[2][kMS * kMLD];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm0 = (wave >> 1) * 64, wn0 = (wave & 1) * 64;
+// rows <- EA from a[m][k] (transposed stage), columns <- EB from b[k][n].
+template <class T>
+__global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WPE, T::WPE)))
+void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
+                    float* __restrict__ out, const float* __restrict__ stats,
+                    int* __restrict__ flags, float* __restrict__ ws_ea,
+                    float* __restrict__ ws_eb, float* __restrict__ ws_r, int* __restrict__ ws_hdr,
+                    int M, int K, int N, int tiles_m, int tiles_n) {
+  constexpr int NT = T::NT, LDR = T::LDR, LDC = T::LDC;
+  using SA = StageT<T::TR, NT, LDR>;
+  using SB = StageS<T::TC, NT, LDC>;
+  __shared__ __attribute__((aligned(16))) float smem[2 * kMS * (LDR + LDC)];
+  static_assert(2 * kMS * (LDR + LDC) >= (NT / 64) * kStripFloats, "");
+  float(*As)[kMS * LDR] = reinterpret_cast<float(*)[kMS * LDR]>(smem);
+  float(*Bs)[kMS * LDC] = reinterpret_cast<float(*)[kMS * LDC]>(smem + 2 * kMS * LDR);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps tile offsets scalar
+  const int wm0 = (wave / T::WC) * 64, wn0 = (wave % T::WC) * 64;
   const int per = tiles_m * tiles_n, tile = xcd_tile_id();
   const int batch = tile / per, rem = tile - batch * per;
-  const int m0 = (rem / tiles_n) * kMT, n0 = (rem % tiles_n) * kMT;
+  const int m0 = (rem / tiles_n) * T::TR, n0 = (rem % tiles_n) * T::TC;
   const float* st = stats + (long)batch * (M + N);
+  // EA / EB are written out by the tiles that stage them anyway: the tiles of
+  // one row block share the slabs of EA between them (slab s goes to column
+  // block s mod tiles_n), likewise EB, so that every workgroup stores the same.
+  const int nblk = rem % tiles_n, mblk = rem / tiles_n;
 
-  // a tile [m][k]: lane reads rows ar, ar+64 at k quad aq;  b tile [k][n]: rows br, br+8
-  const int ar = tid >> 2, aq = tid & 3, br = tid >> 5, bq = tid & 31;
-  const float* pa = a + ((long)batch * M + m0 + ar) * K + aq * 4;
-  const float* pb = b + ((long)batch * K + br) * N + n0 + bq * 4;
-  const float al0 = st[m0 + ar], al1 = st[m0 + ar + 64];
-  const float4 be = *reinterpret_cast<const float4*>(st + M + n0 + bq * 4);
+  const long offa = ((long)batch * M + m0 + SA::line(tid, 0)) * K + SA::quad(tid) * 4;
+  const long offb = ((long)batch * K + SB::red(tid, 0)) * N + n0 + SB::quad(tid) * 4;
+  const float* pa = a + offa;
+  const float* pb = b + offb;
+  float* qa = ws_ea + offa;
+  float* qb = ws_eb + offb;
+  float al[SA::PER];
+#pragma unroll
+  for (int l = 0; l < SA::PER; ++l) al[l] = st[m0 + SA::line(tid, l)];
+  const float4 be = ld4(st + M + n0 + SB::quad(tid) * 4);
+  if (tile == 0 && tid == 0) {
+    ws_hdr[1] = T::TR;
+    ws_hdr[2] = T::TC;
+    ws_hdr[0] = 1;
+  }
 
   floatx16 acc[2][2];
 #pragma unroll
@@ -99,90 +230,134 @@ __global__ __launch_bounds__(256, 4) void k_log_fwd_mfma(const float* __restrict
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[x >> 1][x & 1][i] = 0.f;
 
-  float4 ra0, ra1, rb0, rb1;
+  float4 ra[SA::PER], rb[SB::PER];
   auto load = [&]() __attribute__((always_inline)) {
-    ra0 = *reinterpret_cast<const float4*>(pa);
-    ra1 = *reinterpret_cast<const float4*>(pa + 64l * K);
-    rb0 = *reinterpret_cast<const float4*>(pb);
-    rb1 = *reinterpret_cast<const float4*>(pb + 8l * N);
+#pragma unroll
+    for (int l = 0; l < SA::PER; ++l) ra[l] = ld4(pa + (long)l * SA::STEP * K);
+#pragma unroll
+    for (int l = 0; l < SB::PER; ++l) rb[l] = ld4(pb + (long)l * SB::STEP * N);
     pa += kMS;
     pb += (long)kMS * N;
   };
-  auto stage = [&](int buf) __attribute__((always_inline)) {
-    lds_put_t(As[buf], ar, aq, make_float4(exp_st(ra0.x - al0), exp_st(ra0.y - al0),
-                                           exp_st(ra0.z - al0), exp_st(ra0.w - al0)));
-    lds_put_t(As[buf], ar + 64, aq, make_float4(exp_st(ra1.x - al1), exp_st(ra1.y - al1),
-                                                exp_st(ra1.z - al1), exp_st(ra1.w - al1)));
-    lds_put(Bs[buf], br, bq, make_float4(exp_st(rb0.x - be.x), exp_st(rb0.y - be.y),
-                                         exp_st(rb0.z - be.z), exp_st(rb0.w - be.w)));
-    lds_put(Bs[buf], br + 8, bq, make_float4(exp_st(rb1.x - be.x), exp_st(rb1.y - be.y),
-                                             exp_st(rb1.z - be.z), exp_st(rb1.w - be.w)));
+  auto stage = [&](int buf, bool keep_a, bool keep_b) __attribute__((always_inline)) {
+#pragma unroll
+    for (int l = 0; l < SA::PER; ++l) {
+      const float4 e = exp4(ra[l], al[l]);
+      SA::put(As[buf], tid, l, e);
+      if (keep_a) *reinterpret_cast<float4*>(qa + (long)l * SA::STEP * K) = e;
+    }
+#pragma unroll
+    for (int l = 0; l < SB::PER; ++l) {
+      const float4 e = exp4(rb[l], be);
+      SB::put(Bs[buf], tid, l, e);
+      if (keep_b) *reinterpret_cast<float4*>(qb + (long)l * SB::STEP * N) = e;
+    }
+    qa += kMS;
+    qb += (long)kMS * N;
   };
 
   const int slabs = K / kMS;
   load();
-  stage(0);
+  stage(0, nblk == 0, mblk == 0);
   __syncthreads();
+  int sa = 1 % tiles_n, sb = 1 % tiles_m;  // (s + 1) mod tiles_n, mod tiles_m
   for (int s = 0; s < slabs; ++s) {
     const bool more = s + 1 < slabs;
     if (more) load();
-    mfma_slab(As[s & 1], Bs[s & 1], wm0, wn0, lane, acc);
-    if (more) stage((s + 1) & 1);
+    mfma_slab<LDR, LDC>(As[s & 1], Bs[s & 1], wm0, wn0, lane, acc);
+    if (more) stage((s + 1) & 1, sa == nblk, sb == mblk);
+    sa = sa + 1 == tiles_n ? 0 : sa + 1;
+    sb = sb + 1 == tiles_m ? 0 : sb + 1;
     __syncthreads();
   }
 
-  // guard: S >= 2^-40, finite, and the shift above the reference's -1e9 floor
+  // guard: S >= 2^-40 and finite; every shift of the tile finite and far above
+  // the reference's -1e9 floor (checked per row and column, which is stricter
+  // than per cell and only sends more tiles to the exact routine).
   const float thr = fast_exp2(-kMfmaGuardBits);
-  const int lrow = lane & 31;
   int bad = 0;
-  float be_c[2];
-  be_c[0] = st[M + n0 + wn0 + lrow];
-  be_c[1] = st[M + n0 + wn0 + 32 + lrow];
 #pragma unroll
   for (int x = 0; x < 4; ++x)
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const float shift = st[m0 + wm0 + (x >> 1) * 32 + mfma_row(i, lane)] + be_c[x & 1];
       const float s = acc[x >> 1][x & 1][i];
-      if (!((s >= thr) && (s < INFINITY) && (shift > 0.9f * kFloor) && (shift < INFINITY))) bad = 1;
-      acc[x >> 1][x & 1][i] = __builtin_fmaf(fast_log2(s), kLn2, shift);
+      if (!((s >= thr) && (s < INFINITY))) bad = 1;
     }
-  bad = __syncthreads_or(bad);
+  for (int t = tid; t < T::TR + T::TC; t += NT) {
+    const float sh = t < T::TR ? st[m0 + t] : st[M + n0 + t - T::TR];
+    if (!((sh > 0.45f * kFloor) && (sh < INFINITY))) bad = 1;
+  }
+  bad = __syncthreads_or(bad);  // also: every wave is done with the staging buffers
   if (tid == 0) flags[tile] = bad;
   if (bad) return;  // the fix-up launch recomputes this tile
-  float* ob = out + ((long)batch * M + m0 + wm0) * N + n0 + wn0 + lrow;
-#pragma unroll
-  for (int x = 0; x < 4; ++x)
-#pragma unroll
-    for (int i = 0; i < 16; ++i)
-      ob[(long)((x >> 1) * 32 + mfma_row(i, lane)) * N + (x & 1) * 32] = acc[x >> 1][x & 1][i];
+
+  // out = log S + alpha + beta and R = 1/S, written row-wise
+  const int lr = lane >> 4, lc = (lane & 15) * 4;
+  const float4 be4 = ld4(st + M + n0 + wn0 + lc);
+  const float* alw = st + m0 + wm0 + lr;
+  const long ubase = ((long)batch * M + m0 + wm0) * N + n0 + wn0;
+  const int voff = lr * N + lc;
+  acc_rows(acc, smem + wave * kStripFloats, lane, [](int) {},
+           [&](int q, int t, float4 sv) __attribute__((always_inline)) {
+             const int ru = 16 * q + 4 * t;
+             const float alr = alw[ru];
+             const long u = ubase + (long)ru * N;
+             *reinterpret_cast<float4*>(ws_r + u + voff) =
+                 make_float4(__builtin_amdgcn_rcpf(sv.x), __builtin_amdgcn_rcpf(sv.y),
+                             __builtin_amdgcn_rcpf(sv.z), __builtin_amdgcn_rcpf(sv.w));
+             *reinterpret_cast<float4*>(out + u + voff) =
+                 make_float4(__builtin_fmaf(fast_log2(sv.x), kLn2, alr + be4.x),
+                             __builtin_fmaf(fast_log2(sv.y), kLn2, alr + be4.y),
+                             __builtin_fmaf(fast_log2(sv.z), kLn2, alr + be4.z),
+                             __builtin_fmaf(fast_log2(sv.w), kLn2, alr + be4.w));
+           });
 }
 
 // ---------------------------------------------------------------- backward
-// GRAD_A: tile (m,k) of grad_a, reduction over n.  rows <- H[n][m], cols <- EB[n][k].
-// GRAD_B: tile (k,n) of grad_b, reduction over m.  rows <- EA[m][k], cols <- H[m][n].
-// H = g * exp(alpha[m] + beta[n] - out[m,n]);  the epilogue multiplies by
-// exp(x - shift) of the operand shaped like the output.
-template <bool GRAD_A>
-__global__ __launch_bounds__(256, GRAD_A ? 2 : 4) void k_log_bwd_mfma(const float* __restrict__ a,
-                                                         const float* __restrict__ b,
-                                                         const float* __restrict__ outp,
-                                                         const float* __restrict__ g,
-                                                         const float* __restrict__ stats,
-                                                         float* __restrict__ grad,
-                                                         int* __restrict__ flags, int M, int K,
-                                                         int N, int tiles_r, int tiles_c) {
-  __shared__ __attribute__((aligned(16))) float Ys[2][kMS * kMLD];
-  __shared__ __attribute__((aligned(16))) float Hs[2][kMS * kMLD];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wr0 = (wave >> 1) * 64, wc0 = (wave & 1) * 64;
+// On the forward's by-products:  H = g * R.
+// GRAD_A: tile (m,k) of grad_a = EA * sum_n H[m][n] EB[k][n]; rows <- H, columns
+//         <- EB, both sources [out][red] (transposed stage).
+// GRAD_B: tile (k,n) of grad_b = EB * sum_m EA[m][k] H[m][n]; rows <- EA,
+//         columns <- H, both sources [red][out].
+// A tile that touches a cell the forward flagged (R unusable there), or runs
+// on a workspace the matrix-core forward did not fill, raises its own flag and
+// leaves the work to the fix-up launch.
+template <class T, bool GRAD_A>
+__global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WPE, T::WPE)))
+void k_log_bwd_mfma(const float* __restrict__ g, const float* __restrict__ ws_ea,
+                    const float* __restrict__ ws_eb, const float* __restrict__ ws_r,
+                    const int* __restrict__ ws_hdr, const int* __restrict__ fwd_flags,
+                    float* __restrict__ grad,
+                    int* __restrict__ flags, int M, int K, int N, int tiles_r, int tiles_c) {
+  constexpr int NT = T::NT, LDR = T::LDR, LDC = T::LDC;
+  using SH = std::conditional_t<GRAD_A, StageT<T::TR, NT, LDR>, StageS<T::TC, NT, LDC>>;
+  using SY = std::conditional_t<GRAD_A, StageT<T::TC, NT, LDC>, StageS<T::TR, NT, LDR>>;
+  __shared__ __attribute__((aligned(16))) float smem[2 * kMS * (LDR + LDC)];
+  static_assert(2 * kMS * (LDR + LDC) >= (NT / 64) * kStripFloats, "");
+  float(*Rs)[kMS * LDR] = reinterpret_cast<float(*)[kMS * LDR]>(smem);
+  float(*Cs)[kMS * LDC] = reinterpret_cast<float(*)[kMS * LDC]>(smem + 2 * kMS * LDR);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps tile offsets scalar
+  const int wr0 = (wave / T::WC) * 64, wc0 = (wave % T::WC) * 64;
   const int per = tiles_r * tiles_c, tile = xcd_tile_id();
   const int batch = tile / per, rem = tile - batch * per;
-  const int r0 = (rem / tiles_c) * kMT, c0 = (rem % tiles_c) * kMT;
+  const int r0 = (rem / tiles_c) * T::TR, c0 = (rem % tiles_c) * T::TC;
   const int Q = GRAD_A ? N : M;
-  const float* al = stats + (long)batch * (M + N);
-  const float* be = al + M;
-  const float lim = kMfmaGuardBits * kLn2 + 1e-3f;
+
+  {  // forward flags over the cells this tile reduces over
+    int bad = ws_hdr[0] != 1;
+    const int ftr = max(ws_hdr[1], 1), ftc = max(ws_hdr[2], 1);
+    const int fm = M / ftr, fn = N / ftc;
+    const int mlo = GRAD_A ? r0 / ftr : 0, mhi = GRAD_A ? (r0 + T::TR - 1) / ftr : fm - 1;
+    const int nlo = GRAD_A ? 0 : c0 / ftc, nhi = GRAD_A ? fn - 1 : (c0 + T::TC - 1) / ftc;
+    const int nn = nhi - nlo + 1, cnt = (mhi - mlo + 1) * nn;
+    if (!bad)
+      for (int t = tid; t < cnt; t += NT)
+        bad |= fwd_flags[((long)batch * fm + mlo + t / nn) * fn + nlo + t % nn];
+    bad = __syncthreads_or(bad);
+    if (tid == 0) flags[tile] = bad;
+    if (bad) return;
+  }
 
   floatx16 acc[2][2];
 #pragma unroll
@@ -190,82 +365,44 @@ __global__ __launch_bounds__(256, GRAD_A ? 2 : 4) void k_log_bwd_mfma(const floa
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[x >> 1][x & 1][i] = 0.f;
 
-  float4 ry0, ry1, ro0, ro1, rg0, rg1, sh;   // sh: shifts that change with the slab
-  float sh0 = 0.f, sh1 = 0.f;
-  int bad = 0;
-  const float* py;
-  const float* po;
-  const float* pg;
-  const float* ps;
-  // fixed shifts
-  float fa0 = 0.f, fa1 = 0.f;
-  float4 fb = make_float4(0.f, 0.f, 0.f, 0.f);
-  const int tr = tid >> 2, tq = tid & 3;    // [out][red] tiles: out row tr (+64), red quad tq
-  const int ur = tid >> 5, uq = tid & 31;   // [red][out] tiles: red row ur (+8), out quad uq
+  float4 ry[SY::PER], rr[SH::PER], rg[SH::PER];
+  const float *py, *pr, *pg;
   if constexpr (GRAD_A) {
-    py = b + ((long)batch * K + c0 + tr) * N + tq * 4;      // b[k = c0+tr][n]
-    po = outp + ((long)batch * M + r0 + tr) * N + tq * 4;   // out[m = r0+tr][n]
-    pg = g + ((long)batch * M + r0 + tr) * N + tq * 4;
-    ps = be + tq * 4;                                       // beta[n] of the slab
-    fa0 = al[r0 + tr];
-    fa1 = al[r0 + tr + 64];
+    py = ws_eb + ((long)batch * K + c0 + SY::line(tid, 0)) * N + SY::quad(tid) * 4;  // EB[k][n]
+    const long o = ((long)batch * M + r0 + SH::line(tid, 0)) * N + SH::quad(tid) * 4;
+    pr = ws_r + o;
+    pg = g + o;
   } else {
-    py = a + ((long)batch * M + ur) * K + r0 + uq * 4;      // a[m][k = r0 + ...]
-    po = outp + ((long)batch * M + ur) * N + c0 + uq * 4;   // out[m][n = c0 + ...]
-    pg = g + ((long)batch * M + ur) * N + c0 + uq * 4;
-    ps = al + ur;                                           // alpha[m] of the slab
-    fb = *reinterpret_cast<const float4*>(be + c0 + uq * 4);
+    py = ws_ea + ((long)batch * M + SY::red(tid, 0)) * K + r0 + SY::quad(tid) * 4;   // EA[m][k]
+    const long o = ((long)batch * M + SH::red(tid, 0)) * N + c0 + SH::quad(tid) * 4;
+    pr = ws_r + o;
+    pg = g + o;
   }
+  constexpr long kYStep = SY::STEP, kHStep = SH::STEP;
+  const long ldy = GRAD_A ? N : K;
   auto load = [&]() __attribute__((always_inline)) {
-    if constexpr (GRAD_A) {
-      ry0 = *reinterpret_cast<const float4*>(py);
-      ry1 = *reinterpret_cast<const float4*>(py + 64l * N);
-      ro0 = *reinterpret_cast<const float4*>(po);
-      ro1 = *reinterpret_cast<const float4*>(po + 64l * N);
-      rg0 = *reinterpret_cast<const float4*>(pg);
-      rg1 = *reinterpret_cast<const float4*>(pg + 64l * N);
-      sh = *reinterpret_cast<const float4*>(ps);
-      py += kMS; po += kMS; pg += kMS; ps += kMS;
-    } else {
-      ry0 = *reinterpret_cast<const float4*>(py);
-      ry1 = *reinterpret_cast<const float4*>(py + 8l * K);
-      ro0 = *reinterpret_cast<const float4*>(po);
-      ro1 = *reinterpret_cast<const float4*>(po + 8l * N);
-      rg0 = *reinterpret_cast<const float4*>(pg);
-      rg1 = *reinterpret_cast<const float4*>(pg + 8l * N);
-      sh0 = ps[0];
-      sh1 = ps[8];
-      py += (long)kMS * K; po += (long)kMS * N; pg += (long)kMS * N; ps += kMS;
+#pragma unroll
+    for (int l = 0; l < SY::PER; ++l) ry[l] = ld4(py + l * kYStep * ldy);
+#pragma unroll
+    for (int l = 0; l < SH::PER; ++l) {
+      rr[l] = ld4(pr + l * kHStep * N);
+      rg[l] = ld4(pg + l * kHStep * N);
     }
-  };
-  auto hval = [&](float gv, float e) __attribute__((always_inline)) {
-    if (!(e <= lim)) bad = 1;  // S < 2^-40 (or NaN): factoring not exact here
-    return gv * exp_st(e);
+    if constexpr (GRAD_A) {
+      py += kMS; pr += kMS; pg += kMS;
+    } else {
+      py += (long)kMS * K; pr += (long)kMS * N; pg += (long)kMS * N;
+    }
   };
   auto stage = [&](int buf) __attribute__((always_inline)) {
-    if constexpr (GRAD_A) {
-      lds_put_t(Ys[buf], tr, tq, make_float4(exp_st(ry0.x - sh.x), exp_st(ry0.y - sh.y),
-                                             exp_st(ry0.z - sh.z), exp_st(ry0.w - sh.w)));
-      lds_put_t(Ys[buf], tr + 64, tq, make_float4(exp_st(ry1.x - sh.x), exp_st(ry1.y - sh.y),
-                                                  exp_st(ry1.z - sh.z), exp_st(ry1.w - sh.w)));
-      lds_put_t(Hs[buf], tr, tq,
-                make_float4(hval(rg0.x, fa0 + sh.x - ro0.x), hval(rg0.y, fa0 + sh.y - ro0.y),
-                            hval(rg0.z, fa0 + sh.z - ro0.z), hval(rg0.w, fa0 + sh.w - ro0.w)));
-      lds_put_t(Hs[buf], tr + 64, tq,
-                make_float4(hval(rg1.x, fa1 + sh.x - ro1.x), hval(rg1.y, fa1 + sh.y - ro1.y),
-                            hval(rg1.z, fa1 + sh.z - ro1.z), hval(rg1.w, fa1 + sh.w - ro1.w)));
-    } else {
-      lds_put(Ys[buf], ur, uq, make_float4(exp_st(ry0.x - sh0), exp_st(ry0.y - sh0),
-                                           exp_st(ry0.z - sh0), exp_st(ry0.w - sh0)));
-      lds_put(Ys[buf], ur + 8, uq, make_float4(exp_st(ry1.x - sh1), exp_st(ry1.y - sh1),
-                                               exp_st(ry1.z - sh1), exp_st(ry1.w - sh1)));
-      lds_put(Hs[buf], ur, uq,
-              make_float4(hval(rg0.x, sh0 + fb.x - ro0.x), hval(rg0.y, sh0 + fb.y - ro0.y),
-                          hval(rg0.z, sh0 + fb.z - ro0.z), hval(rg0.w, sh0 + fb.w - ro0.w)));
-      lds_put(Hs[buf], ur + 8, uq,
-              make_float4(hval(rg1.x, sh1 + fb.x - ro1.x), hval(rg1.y, sh1 + fb.y - ro1.y),
-                          hval(rg1.z, sh1 + fb.z - ro1.z), hval(rg1.w, sh1 + fb.w - ro1.w)));
-    }
+    float* ybuf = GRAD_A ? Cs[buf] : Rs[buf];
+    float* hbuf = GRAD_A ? Rs[buf] : Cs[buf];
+#pragma unroll
+    for (int l = 0; l < SY::PER; ++l) SY::put(ybuf, tid, l, ry[l]);
+#pragma unroll
+    for (int l = 0; l < SH::PER; ++l)
+      SH::put(hbuf, tid, l, make_float4(rg[l].x * rr[l].x, rg[l].y * rr[l].y, rg[l].z * rr[l].z,
+                                        rg[l].w * rr[l].w));
   };
 
   const int slabs = Q / kMS;
@@ -275,37 +412,32 @@ __global__ __launch_bounds__(256, GRAD_A ? 2 : 4) void k_log_bwd_mfma(const floa
   for (int s = 0; s < slabs; ++s) {
     const bool more = s + 1 < slabs;
     if (more) load();
-    if constexpr (GRAD_A)
-      mfma_slab(Hs[s & 1], Ys[s & 1], wr0, wc0, lane, acc);
-    else
-      mfma_slab(Ys[s & 1], Hs[s & 1], wr0, wc0, lane, acc);
+    mfma_slab<LDR, LDC>(Rs[s & 1], Cs[s & 1], wr0, wc0, lane, acc);
     if (more) stage((s + 1) & 1);
     __syncthreads();
   }
 
-  bad = __syncthreads_or(bad);
-  if (tid == 0) flags[tile] = bad;
-  if (bad) return;  // the fix-up launch recomputes this tile
-
-  // grad = exp(x - shift) * acc
+  // grad = EX * acc, EX = EA or EB, row-wise; the loads of a quarter are started
+  // before the previous quarter is exchanged.
   const int Cc = GRAD_A ? K : N;
-  const int lrow = lane & 31;
-  const float* xb = (GRAD_A ? a : b) + ((long)batch * (GRAD_A ? M : K) + r0 + wr0) * Cc + c0 + wc0 + lrow;
-  float* gp = grad + ((long)batch * (GRAD_A ? M : K) + r0 + wr0) * Cc + c0 + wc0 + lrow;
-  float cs[2] = {0.f, 0.f};
-  if constexpr (!GRAD_A) {
-    cs[0] = be[c0 + wc0 + lrow];
-    cs[1] = be[c0 + wc0 + 32 + lrow];
-  }
+  const int lr = lane >> 4, lc = (lane & 15) * 4;
+  const int voff = lr * Cc + lc;
+  const long ubase = ((long)batch * (GRAD_A ? M : K) + r0 + wr0) * Cc + c0 + wc0;
+  const float* xb = (GRAD_A ? ws_ea : ws_eb) + ubase + voff;
+  float* gp = grad + ubase + voff;
+  float4 xq[2][4];
+  auto fetch = [&](int q) __attribute__((always_inline)) {
 #pragma unroll
-  for (int x = 0; x < 4; ++x)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int rr = (x >> 1) * 32 + mfma_row(i, lane);
-      const long off = (long)rr * Cc + (x & 1) * 32;
-      const float shv = GRAD_A ? al[r0 + wr0 + rr] : cs[x & 1];
-      gp[off] = exp_st(xb[off] - shv) * acc[x >> 1][x & 1][i];
-    }
+    for (int t = 0; t < 4; ++t) xq[q & 1][t] = ld4(xb + (long)(16 * q + 4 * t) * Cc);
+  };
+  fetch(0);
+  acc_rows(acc, smem + wave * kStripFloats, lane,
+           [&](int q) __attribute__((always_inline)) { if (q + 1 < 4) fetch(q + 1); },
+           [&](int q, int t, float4 v) __attribute__((always_inline)) {
+             const float4 x = xq[q & 1][t];
+             *reinterpret_cast<float4*>(gp + (long)(16 * q + 4 * t) * Cc) =
+                 make_float4(x.x * v.x, x.y * v.y, x.z * v.z, x.w * v.w);
+           });
 }
 
 }  // namespace genbmm

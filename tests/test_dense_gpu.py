@@ -154,6 +154,55 @@ def test_logbmm_factoring_guard(gpu, B, M, K, N):
     close(gb2[:-1], wb)
 
 
+@pytest.mark.parametrize("B,M,K,N", [(32, 256, 128, 256), (64, 512, 128, 512)])
+def test_logbmm_factoring_guard_matrix_core_tiles(gpu, B, M, K, N):
+    """Shapes that run on the matrix-core kernels (128x128 and 128x256 / 256x128 tiles).
+    Some batch items need the exact fall-back in every tile, one in a single row, the
+    rest in none: flagged and unflagged tiles side by side, and the backward kernels
+    must honour the forward's flags (they read 1/S from the forward's workspace)."""
+    torch.manual_seed(B + M)
+    a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
+    a[: B // 4, ::2, 0] += 200.0
+    b[: B // 4, 0, :] -= 200.0
+    a[B // 4, 37, 5] += 200.0
+    b[B // 4, 5, :] -= 200.0
+    pick = torch.tensor([0, 1, B // 4, B // 4 + 1, B - 1])
+    want, wa, wb = oracle.logbmm_grads64(a[pick], b[pick], g[pick])
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    out = genbmm.logbmm(ad, bd)
+    ga, gb = torch.autograd.grad(out, (ad, bd), g.to(gpu))
+    close(out[pick.to(gpu)], want)
+    close(ga[pick.to(gpu)], wa)
+    close(gb[pick.to(gpu)], wb)
+    close(ga.sum(-1), g.double().sum(-1), atol=2e-4)
+    close(gb.sum(-2), g.double().sum(-2), atol=2e-4)
+
+
+def test_logbmm_backward_on_foreign_workspace(gpu):
+    """The matrix-core backward runs on by-products of the matrix-core forward; handed
+    a workspace that another forward path filled, it must notice and still be right."""
+    lib = _lib.load()
+    torch.manual_seed(3)
+    B, M, K, N = 32, 256, 128, 256
+    a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
+    ad, bd, gd = a.to(gpu), b.to(gpu), g.to(gpu)
+    out, ga, gb = torch.empty(B, M, N, device=gpu), torch.empty_like(ad), torch.empty_like(bd)
+    stats = torch.full((lib.genbmm_logbmm_stats_size(B, M, K, N),), float("nan"), device=gpu)
+    p, s = _lib.ptr, _lib.stream_of(ad)
+    lib.genbmm_logbmm_force_exact(2)
+    try:
+        assert lib.genbmm_logbmm_fwd(p(ad), p(bd), p(out), p(stats), B, M, K, N, s) == 0
+    finally:
+        lib.genbmm_logbmm_force_exact(0)
+    assert lib.genbmm_logbmm_bwd(p(ad), p(bd), p(out), p(gd), p(stats), p(ga), p(gb), B, M, K, N, s) == 0
+    pick = torch.tensor([0, B - 1])
+    want, wa, wb = oracle.logbmm_grads64(a[pick], b[pick], g[pick])
+    close(out[pick.to(gpu)], want)
+    close(ga[pick.to(gpu)], wa)
+    close(gb[pick.to(gpu)], wb)
+    close(ga.sum(-1), g.double().sum(-1), atol=2e-4)
+
+
 @pytest.mark.parametrize("B,M,K,N", [(2, 4, 5, 3), (3, 9, 12, 7), (2, 33, 20, 40)])
 def test_logbmm_double_backward(gpu, B, M, K, N):
     """Second-order terms (test_cuda.py:30-42 uses rtol 1e-2; here 1e-4 vs float64)."""
