@@ -67,15 +67,22 @@ def dense_log(lib, dev, B, M, K, N, reps, name, dist="randn", path=0):
     s, p = _lib.stream_of(a), _lib.ptr
     lib.genbmm_logbmm_force_exact(path)
 
-    def step():
+    def f():
         _lib.check(lib.genbmm_logbmm_fwd(p(a), p(b), p(out), p(stats), B, M, K, N, s), "fwd")
+
+    def bw():
         _lib.check(lib.genbmm_logbmm_bwd(p(a), p(b), p(out), p(g), p(stats), p(ga), p(gb), B, M, K, N, s), "bwd")
 
-    ms = timed(step, reps)
+    def step():
+        f()
+        bw()
+
+    ms, mf, mb = timed(step, reps), timed(f, reps), timed(bw, reps)
     lib.genbmm_logbmm_force_exact(0)
     bmkn = float(B) * M * K * N
     nbytes = 4.0 * B * (3 * M * K + 3 * K * N + 3 * M * N)
-    report(name, ms, 6 * bmkn, nbytes, {"path": {0: "factored", 1: "online-exact", 2: "factored-valu"}[path]})
+    report(name, ms, 6 * bmkn, nbytes, {"path": {0: "factored", 1: "online-exact", 2: "factored-valu"}[path],
+                                        "ms_fwd": round(mf, 4), "ms_bwd": round(mb, 4)})
 
 
 def dense_max(lib, dev, B, M, K, N, reps, prod):

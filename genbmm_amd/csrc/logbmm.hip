@@ -27,6 +27,7 @@
 // Two implementations of the factored contraction: v_fma_f32 on register blocks
 // (any shape, this file) and the fp32 matrix-core instruction for problems made
 // of full 128x128 tiles (logbmm_mfma.h).
+#include <algorithm>
 #include <atomic>
 
 #include "dense_tiles.h"
@@ -298,6 +299,36 @@ __global__ __launch_bounds__(CX::NT) void k_log_bwd_fixup(const LogBwdArgs p,
       for (int w = 0; w < FBC / CX::BC; ++w)
         if (r0 + h * CX::BR < R && c0 + w * CX::BC < Cc) {
           log_bwd_tile<CX, GRAD_A>(p, batch, r0 + h * CX::BR, c0 + w * CX::BC, smem);
+          __syncthreads();
+        }
+  }
+}
+
+// Fix-up of both gradients' flagged tiles in one launch (workgroups stride over
+// the grad_a list, then over the grad_b list).
+template <class CX, int AR, int AC, int BR, int BC>
+__global__ __launch_bounds__(CX::NT) void k_log_bwd_fixup_both(const LogBwdArgs pa,
+                                                               const LogBwdArgs pb,
+                                                               const int* __restrict__ flags_a,
+                                                               const int* __restrict__ flags_b,
+                                                               int tiles_a, int tiles_b) {
+  constexpr int kFa = LogBwdLds<CX, true>::FLOATS, kFb = LogBwdLds<CX, false>::FLOATS;
+  __shared__ __attribute__((aligned(16))) float smem[kFa > kFb ? kFa : kFb];
+  for (int t = blockIdx.x; t < tiles_a + tiles_b; t += gridDim.x) {
+    const bool is_a = t < tiles_a;
+    const int u = is_a ? t : t - tiles_a;
+    if (!(is_a ? flags_a[u] : flags_b[u])) continue;
+    const LogBwdArgs& p = is_a ? pa : pb;
+    const int per = p.tiles_r * p.tiles_c;
+    const int batch = u / per, r = u - batch * per;
+    const int FR = is_a ? AR : BR, FC = is_a ? AC : BC;
+    const int R = is_a ? p.M : p.K, Cc = is_a ? p.K : p.N;
+    const int r0 = (r / p.tiles_c) * FR, c0 = (r % p.tiles_c) * FC;
+    for (int h = 0; h < FR / CX::BR; ++h)
+      for (int w = 0; w < FC / CX::BC; ++w)
+        if (r0 + h * CX::BR < R && c0 + w * CX::BC < Cc) {
+          if (is_a) log_bwd_tile<CX, true>(p, batch, r0 + h * CX::BR, c0 + w * CX::BC, smem);
+          else log_bwd_tile<CX, false>(p, batch, r0 + h * CX::BR, c0 + w * CX::BC, smem);
           __syncthreads();
         }
   }
@@ -638,6 +669,28 @@ int launch_bwd_mfma(LogBwdArgs p, const float* stats, int* flags, int B, hipStre
   return launch_status();
 }
 
+// grad_a and grad_b of a matrix-core problem in one launch (+ one fix-up launch).
+template <class TA, class TB>
+int launch_bwd_mfma_both(LogBwdArgs pa, LogBwdArgs pb, const float* stats, int B, hipStream_t s) {
+  const int M = pa.M, K = pa.K, N = pa.N;
+  pa.tiles_r = M / TA::TR; pa.tiles_c = K / TA::TC;
+  pb.tiles_r = K / TB::TR; pb.tiles_c = N / TB::TC;
+  const int64_t ta = (int64_t)B * pa.tiles_r * pa.tiles_c, tb = (int64_t)B * pb.tiles_r * pb.tiles_c;
+  if (ta + tb > 0x7fffffffLL) return GENBMM_E_SHAPE;
+  const LogPrepared ws = prepared_of(stats, B, M, K, N);
+  int* fa = flags_of(stats, B, M, K, N, 1);
+  int* fb = flags_of(stats, B, M, K, N, 2);
+  hipLaunchKernelGGL((k_log_bwd_mfma_both<TA, TB>), dim3((unsigned)(ta + tb)), dim3(TA::NT), 0, s,
+                     pa.g, ws.ea, ws.eb, ws.r, ws.hdr, flags_of(stats, B, M, K, N, 0), pa.grad,
+                     pb.grad, fa, fb, M, K, N, (int)ta, pa.tiles_r, pa.tiles_c, pb.tiles_r,
+                     pb.tiles_c);
+  if (int e = launch_status()) return e;
+  hipLaunchKernelGGL((k_log_bwd_fixup_both<BCfgWide, TA::TR, TA::TC, TB::TR, TB::TC>),
+                     dim3((unsigned)std::min<int64_t>(ta + tb, kFixupGrid)), dim3(BCfgWide::NT), 0,
+                     s, pa, pb, fa, fb, (int)ta, (int)tb);
+  return launch_status();
+}
+
 // All tiles full and every access 16-byte aligned: the matrix-core kernels apply.
 // Returns 2 for the 256-wide tile (enough tiles to give every compute unit two
 // workgroups of eight waves), 1 for 128x128, 0 for neither.  `long_cols`: the
@@ -746,6 +799,17 @@ int genbmm_logbmm_bwd(const float* a, const float* b, const float* out, const fl
   p.vec_n = (N % 4 == 0) && aligned16(b) && aligned16(out) && aligned16(g) && aligned16(grad_b);
   hipStream_t s = (hipStream_t)stream;
   const float* st = (g_path.load() == 1 || mn == 0) ? nullptr : stats;
+  if (st && grad_a && grad_b && mk > 0 && kn > 0 && fwd_mfma_shape(B, M, K, N)) {
+    const bool al = p.vec_k && p.vec_n && aligned16(st) && M % 4 == 0 && N % 4 == 0;
+    const int ka = mfma_kind(B, M, K, N, al, true), kb = mfma_kind(B, K, N, M, al, false);
+    if (ka == kb && ka != 0) {
+      LogBwdArgs pa = p, pb = p;
+      pa.grad = grad_a;
+      pb.grad = grad_b;
+      return ka == 2 ? launch_bwd_mfma_both<MTWide, MTTall>(pa, pb, st, B, s)
+                     : launch_bwd_mfma_both<MT128, MT128>(pa, pb, st, B, s);
+    }
+  }
   if (grad_a) {
     p.grad = grad_a;
     if (int e = run_bwd<true>(p, st, B, s)) return e;

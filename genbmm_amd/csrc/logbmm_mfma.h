@@ -36,10 +36,10 @@ constexpr float kMfmaGuardBits = 40.f;
 // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
 // Renumber them so that every XCD works on one contiguous run of tiles (the
 // tiles of a batch item share their operands).
-__device__ __forceinline__ int xcd_tile_id() {
-  const int w = blockIdx.x, n = gridDim.x;
+__device__ __forceinline__ int xcd_renumber(int w, int n) {
   return (n & 7) == 0 ? (w & 7) * (n >> 3) + (w >> 3) : w;
 }
+__device__ __forceinline__ int xcd_tile_id() { return xcd_renumber(blockIdx.x, gridDim.x); }
 
 __device__ __forceinline__ float exp_st(float d) { return fast_exp2(d * kLog2e); }
 
@@ -323,23 +323,22 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
 // on a workspace the matrix-core forward did not fill, raises its own flag and
 // leaves the work to the fix-up launch.
 template <class T, bool GRAD_A>
-__global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WPE, T::WPE)))
-void k_log_bwd_mfma(const float* __restrict__ g, const float* __restrict__ ws_ea,
-                    const float* __restrict__ ws_eb, const float* __restrict__ ws_r,
-                    const int* __restrict__ ws_hdr, const int* __restrict__ fwd_flags,
-                    float* __restrict__ grad,
-                    int* __restrict__ flags, int M, int K, int N, int tiles_r, int tiles_c) {
+__device__ __forceinline__ void log_bwd_mfma_tile(
+    float* __restrict__ smem, int tile, const float* __restrict__ g,
+    const float* __restrict__ ws_ea, const float* __restrict__ ws_eb,
+    const float* __restrict__ ws_r, const int* __restrict__ ws_hdr,
+    const int* __restrict__ fwd_flags, float* __restrict__ grad, int* __restrict__ flags, int M,
+    int K, int N, int tiles_r, int tiles_c) {
   constexpr int NT = T::NT, LDR = T::LDR, LDC = T::LDC;
   using SH = std::conditional_t<GRAD_A, StageT<T::TR, NT, LDR>, StageS<T::TC, NT, LDC>>;
   using SY = std::conditional_t<GRAD_A, StageT<T::TC, NT, LDC>, StageS<T::TR, NT, LDR>>;
-  __shared__ __attribute__((aligned(16))) float smem[2 * kMS * (LDR + LDC)];
   static_assert(2 * kMS * (LDR + LDC) >= (NT / 64) * kStripFloats, "");
   float(*Rs)[kMS * LDR] = reinterpret_cast<float(*)[kMS * LDR]>(smem);
   float(*Cs)[kMS * LDC] = reinterpret_cast<float(*)[kMS * LDC]>(smem + 2 * kMS * LDR);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps tile offsets scalar
   const int wr0 = (wave / T::WC) * 64, wc0 = (wave % T::WC) * 64;
-  const int per = tiles_r * tiles_c, tile = xcd_tile_id();
+  const int per = tiles_r * tiles_c;
   const int batch = tile / per, rem = tile - batch * per;
   const int r0 = (rem / tiles_c) * T::TR, c0 = (rem % tiles_c) * T::TC;
   const int Q = GRAD_A ? N : M;
@@ -438,6 +437,45 @@ void k_log_bwd_mfma(const float* __restrict__ g, const float* __restrict__ ws_ea
              *reinterpret_cast<float4*>(gp + (long)(16 * q + 4 * t) * Cc) =
                  make_float4(x.x * v.x, x.y * v.y, x.z * v.z, x.w * v.w);
            });
+}
+
+template <class T, bool GRAD_A>
+__global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WPE, T::WPE)))
+void k_log_bwd_mfma(const float* __restrict__ g, const float* __restrict__ ws_ea,
+                    const float* __restrict__ ws_eb, const float* __restrict__ ws_r,
+                    const int* __restrict__ ws_hdr, const int* __restrict__ fwd_flags,
+                    float* __restrict__ grad, int* __restrict__ flags, int M, int K, int N,
+                    int tiles_r, int tiles_c) {
+  __shared__ __attribute__((aligned(16))) float smem[2 * kMS * (T::LDR + T::LDC)];
+  log_bwd_mfma_tile<T, GRAD_A>(smem, xcd_tile_id(), g, ws_ea, ws_eb, ws_r, ws_hdr, fwd_flags, grad,
+                               flags, M, K, N, tiles_r, tiles_c);
+}
+
+// Both gradients in one launch: workgroups [0, tiles_a) take the tiles of grad_a
+// (shape TA), the rest those of grad_b (shape TB).  Workgroups are dispatched in
+// index order, so the first grad_b tiles start while the last grad_a tiles are
+// still writing their results back.
+template <class TA, class TB>
+__global__ __launch_bounds__(TA::NT) __attribute__((amdgpu_waves_per_eu(TA::WPE, TA::WPE)))
+void k_log_bwd_mfma_both(const float* __restrict__ g, const float* __restrict__ ws_ea,
+                         const float* __restrict__ ws_eb, const float* __restrict__ ws_r,
+                         const int* __restrict__ ws_hdr, const int* __restrict__ fwd_flags,
+                         float* __restrict__ grad_a, float* __restrict__ grad_b,
+                         int* __restrict__ flags_a, int* __restrict__ flags_b, int M, int K, int N,
+                         int tiles_a, int ar, int ac, int br, int bc) {
+  static_assert(TA::NT == TB::NT && TA::WPE == TB::WPE, "");
+  constexpr int kA = 2 * kMS * (TA::LDR + TA::LDC), kB = 2 * kMS * (TB::LDR + TB::LDC);
+  __shared__ __attribute__((aligned(16))) float smem[kA > kB ? kA : kB];
+  const int w = blockIdx.x, n = gridDim.x;
+  // XCD-aware numbering inside each half (needs both halves to be multiples of 8)
+  const bool renum = (tiles_a & 7) == 0 && (n & 7) == 0;
+  if (w < tiles_a)
+    log_bwd_mfma_tile<TA, true>(smem, renum ? xcd_renumber(w, tiles_a) : w, g, ws_ea, ws_eb, ws_r,
+                                ws_hdr, fwd_flags, grad_a, flags_a, M, K, N, ar, ac);
+  else
+    log_bwd_mfma_tile<TB, false>(smem, renum ? xcd_renumber(w - tiles_a, n - tiles_a) : w - tiles_a,
+                                 g, ws_ea, ws_eb, ws_r, ws_hdr, fwd_flags, grad_b, flags_b, M, K, N,
+                                 br, bc);
 }
 
 }  // namespace genbmm
