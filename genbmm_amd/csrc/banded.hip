@@ -18,6 +18,9 @@
 // One lane per output element with lanes along the band axis (the contiguous
 // axis of every tensor), so stores are coalesced and neighbouring lanes read
 // overlapping runs that the vector L1 / L2 serve.
+#include <type_traits>
+
+#include "banded_argmax.h"
 #include "banded_strip.h"
 
 namespace genbmm {
@@ -165,17 +168,24 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   if (total == 0) return GENBMM_OK;
   hipStream_t s = (hipStream_t)stream;
   const StripDims sd = strip_dims(p.Wa, p.Wb);
-  if (mode != GENBMM_BAND_MAX && sd.ld_own <= 256 && sd.ld_sl <= 256 && sd.bytes <= kStripLdsLimit) {
+  // the sliding tile doubles as the output staging tile(s): [64][33] values (+ indices)
+  const bool tiles_fit = (size_t)kBR * sd.ld_sl >= (size_t)2 * kBT * kBC;
+  if (tiles_fit && sd.ld_own <= 256 && sd.ld_sl <= 256 && sd.bytes <= kStripLdsLimit) {
     const int strips = ceil_div(n, kBT);
     const dim3 grid((unsigned)((long)B * strips));
     const int nq = ceil_div(max(sd.ld_own, sd.ld_sl), 64);
     auto go = [&](auto kern) {
       hipLaunchKernelGGL(kern, grid, dim3(256), sd.bytes, s, p, strips, sd.ld_own, sd.ld_sl);
     };
-    const bool lg = mode == GENBMM_BAND_LOG;
-    if (nq <= 1) lg ? go(k_band_fwd_strip<true, 1>) : go(k_band_fwd_strip<false, 1>);
-    else if (nq == 2) lg ? go(k_band_fwd_strip<true, 2>) : go(k_band_fwd_strip<false, 2>);
-    else lg ? go(k_band_fwd_strip<true, 4>) : go(k_band_fwd_strip<false, 4>);
+    auto pick = [&](auto nqc) {
+      constexpr int Q = decltype(nqc)::value;
+      if (mode == GENBMM_BAND_LOG) go(k_band_fwd_strip<kSemLog, Q>);
+      else if (mode == GENBMM_BAND_MAX) go(k_band_fwd_strip<kSemMax, Q>);
+      else go(k_band_fwd_strip<kSemMul, Q>);
+    };
+    if (nq <= 1) pick(std::integral_constant<int, 1>{});
+    else if (nq == 2) pick(std::integral_constant<int, 2>{});
+    else pick(std::integral_constant<int, 4>{});
     return launch_status();
   }
   if (mode == GENBMM_BAND_LOG)
@@ -230,6 +240,14 @@ int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_
       }
       return launch_status();
     }
+  }
+  if (mode == GENBMM_BAND_MAX &&
+      max(argmax_bwd_a_bytes(p.Wa), argmax_bwd_b_bytes(p.Wb)) <= kStripLdsLimit) {
+    const int strips = ceil_div(n, kAT);
+    const dim3 grid((unsigned)((long)B * strips));
+    hipLaunchKernelGGL(k_band_argmax_bwd_a, grid, dim3(256), argmax_bwd_a_bytes(p.Wa), s, p, strips);
+    hipLaunchKernelGGL(k_band_argmax_bwd_b, grid, dim3(256), argmax_bwd_b_bytes(p.Wb), s, p, strips);
+    return launch_status();
   }
   if (mode == GENBMM_BAND_LOG) {
     hipLaunchKernelGGL(k_band_bwd_a<GENBMM_BAND_LOG>, blocks_for(ta), dim3(256), 0, s, p, ta);

@@ -60,8 +60,11 @@ __device__ __forceinline__ float wave_max(float v) {
 // axis, NQ = ceil(ld / 64) cells per lane.  load() only issues the global
 // loads into registers, store() consumes them - a whole chunk is in flight while
 // the previous one is being multiplied.
-template <bool LOG, int NQ, int ROWS>
+constexpr int kSemMul = 0, kSemLog = 1, kSemMax = 2;  // what a staged tile is used for
+
+template <int SEM, int NQ, int ROWS>
 struct RowStage {
+  static constexpr bool LOG = SEM == kSemLog;
   static constexpr int U = (ROWS + 3) / 4;
   float v[U][NQ];
 
@@ -75,7 +78,7 @@ struct RowStage {
         const int col = lane + 64 * q, k = col - pad;
         const int prow = c + k - lu;  // dense row of this cell
         const bool ok = r < ROWS && col < ld && c >= 0 && c < n && k >= 0 && k < W && prow >= 0 && prow < n;
-        v[u][q] = ok ? src[(long)c * W + k] : (LOG ? -INFINITY : 0.f);
+        v[u][q] = ok ? src[(long)c * W + k] : (SEM == kSemMul ? 0.f : -INFINITY);
       }
     }
   }
@@ -113,15 +116,17 @@ __device__ __forceinline__ int xcd_strip_id() {
   return (n & 7) == 0 ? (w & 7) * (n >> 3) + (w >> 3) : w;
 }
 
-template <bool LOG, int NQ>
-__global__ __launch_bounds__(256, LOG ? 2 : 3) void k_band_fwd_strip(const BandArgs p, int strips, int ld_own,
-                                                           int ld_sl) {
+template <int SEM, int NQ>
+__global__ __launch_bounds__(256, SEM == kSemMul ? 3 : 2) void k_band_fwd_strip(const BandArgs p, int strips,
+                                                                          int ld_own, int ld_sl) {
+  constexpr bool LOG = SEM == kSemLog, MAXP = SEM == kSemMax;
   extern __shared__ __attribute__((aligned(16))) float smem[];
   float* As = smem;                 // [64][ld_own]
   float* Bs = As + kBT * ld_own;    // [95][ld_sl]; reused as the [64][33] output staging tile
   float* al = Bs + kBR * ld_sl;     // [64]
   float* be = al + kBT;             // [95]
   float* Cs = Bs;
+  int* Is = reinterpret_cast<int*>(Bs + kBT * kBC);  // max product: the argmax tile behind it
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wg = xcd_strip_id();
   const int batch = wg / strips, i0 = (wg - batch * strips) * kBT;
@@ -129,15 +134,16 @@ __global__ __launch_bounds__(256, LOG ? 2 : 3) void k_band_fwd_strip(const BandA
   const float* ab = p.a + (long)batch * n * Wa;
   const float* bb = p.b + (long)batch * n * Wb;
   float* ob = p.o0 + (long)batch * n * Wo;
+  int32_t* ib = MAXP ? p.oidx + (long)batch * n * Wo : nullptr;
   const long bn = (long)batch * n;
   const float thr = fast_exp2(-kBandGuardBits);
 
   {
-    RowStage<LOG, NQ, kBT> sa;
+    RowStage<SEM, NQ, kBT> sa;
     sa.load(ab, Wa, p.a_lu, n, i0, ld_own, 0, wave, lane);
     sa.store(As, ld_own, al, wave, lane);
   }
-  RowStage<LOG, NQ, kBR> sb;
+  RowStage<SEM, NQ, kBR> sb;
   sb.load(bb, Wb, p.b_lu, n, i0 - p.r_lu, ld_sl, kBP, wave, lane);
 
   for (int jc = 0; jc < Wo; jc += kBJ) {
@@ -147,9 +153,26 @@ __global__ __launch_bounds__(256, LOG ? 2 : 3) void k_band_fwd_strip(const BandA
     if (jc + kBJ < Wo) sb.load(bb, Wb, p.b_lu, n, i0 + jc + kBJ - p.r_lu, ld_sl, kBP, wave, lane);
 
     const int j0 = jc + 8 * wave;
+    // acc: the sum; max product: the running maximum (strictly above the reference's
+    // -1e9 floor to count) and its k, lowest k on ties since k ascends
     float acc[8];
+    int ind[8];
 #pragma unroll
-    for (int t = 0; t < 8; ++t) acc[t] = 0.f;
+    for (int t = 0; t < 8; ++t) {
+      acc[t] = MAXP ? kFloor : 0.f;
+      ind[t] = -1;
+    }
+    auto fold = [&](int t, float av, float bv, int k) __attribute__((always_inline)) {
+      if (MAXP) {
+        const float v = av + bv;
+        if (v > acc[t]) {
+          acc[t] = v;
+          ind[t] = k;
+        }
+      } else {
+        acc[t] = __builtin_fmaf(av, bv, acc[t]);
+      }
+    };
     if (j0 < Wo) {
       const int klo = max(0, j0 - (Wb - 1)), khi = min(Wa - 1, j0 + 7);
       const float* ap = As + lane * ld_own;
@@ -168,12 +191,12 @@ __global__ __launch_bounds__(256, LOG ? 2 : 3) void k_band_fwd_strip(const BandA
 #pragma unroll
         for (int x = 0; x < 4; ++x)
 #pragma unroll
-          for (int t = 0; t < 8; ++t) acc[t] = __builtin_fmaf(av[x], bv[x][t], acc[t]);
+          for (int t = 0; t < 8; ++t) fold(t, av[x], bv[x][t], k + x);
       }
       for (; k <= khi; ++k) {
         const float av = ap[k];
 #pragma unroll
-        for (int t = 0; t < 8; ++t) acc[t] = __builtin_fmaf(av, bp[t * dt + k], acc[t]);
+        for (int t = 0; t < 8; ++t) fold(t, av, bp[t * dt + k], k);
       }
     }
     float sh[8];
@@ -199,13 +222,22 @@ __global__ __launch_bounds__(256, LOG ? 2 : 3) void k_band_fwd_strip(const BandA
           v = 0.f;  // outside the matrix: the reference's zero fill
         }
       }
+      if (MAXP) {
+        const int o = i + j0 + t - p.r_lu;
+        const bool inside = o >= 0 && o < n;
+        if (!inside) v = 0.f;  // outside the matrix: the reference's zero fill (index 0 too)
+        Is[lane * kBC + 8 * wave + t] = inside ? ind[t] : 0;
+      }
       Cs[lane * kBC + 8 * wave + t] = v;
     }
     __syncthreads();
     // rows of 32 consecutive outputs
     for (int e = tid; e < kBT * kBJ; e += 256) {
       const int r = e >> 5, c = e & 31;
-      if (i0 + r < n && jc + c < Wo) ob[(long)(i0 + r) * Wo + jc + c] = Cs[r * kBC + c];
+      if (i0 + r < n && jc + c < Wo) {
+        ob[(long)(i0 + r) * Wo + jc + c] = Cs[r * kBC + c];
+        if (MAXP) ib[(long)(i0 + r) * Wo + jc + c] = Is[r * kBC + c];
+      }
     }
   }
 }
@@ -252,7 +284,7 @@ __global__ __launch_bounds__(256, 2) void k_band_bwd_strip(const BandArgs p, int
 
   if (tid < kBT) badrow[tid] = 0;
   if (LOG) {
-    RowStage<true, NQ, kBT> so;
+    RowStage<kSemLog, NQ, kBT> so;
     so.load(xo, Wx, lux, n, x0, ld_own, 0, wave, lane);
     so.store(own, ld_own, sh_own, wave, lane);
   }
@@ -264,7 +296,7 @@ __global__ __launch_bounds__(256, 2) void k_band_bwd_strip(const BandArgs p, int
 
   // first row of the other operand needed by chunk jc
   auto row0_of = [&](int jc) { return GRAD_A ? x0 + jc - p.r_lu : x0 - jc - (kBJ - 1) + p.r_lu; };
-  RowStage<LOG, NQ, kBR> ss;
+  RowStage<LOG ? kSemLog : kSemMul, NQ, kBR> ss;
   ss.load(yo, Wy, luy, n, row0_of(0), ld_sl, kBP, wave, lane);
 
   for (int jc = 0; jc < Wo; jc += kBJ) {
