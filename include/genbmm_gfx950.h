@@ -68,10 +68,13 @@ const char* genbmm_error_string(int code);
  * Non-NULL: its first B*(M+N) elements receive, per batch item, max_k a[m,k]
  * for every m followed by max_k b[k,n] for every n, and the forward uses them
  * to factor exp(a+b) = exp(a-max)*exp(b-max) wherever that is exact to fp32;
- * the rest of the buffer holds per-tile flags naming the tiles where it is
- * not, which a fix-up launch recomputes with the online kernel's routine.
- * The buffer takes the place of the reference's (B, M, N) `maxes` output;
- * pass the same buffer to genbmm_logbmm_bwd.
+ * behind them sit per-tile flags naming the tiles where it is not, which a
+ * fix-up launch recomputes with the online kernel's routine, and - for shapes
+ * that run on the matrix cores (M, N multiples of 128, K of 16, at least 128
+ * tiles) - exp(a-max), exp(b-max) and 1/sum, which the backward then reads
+ * instead of taking any exponential itself.  The contents belong to the
+ * library; the buffer takes the place of the reference's (B, M, N) `maxes`
+ * output; pass the same buffer, unchanged, to genbmm_logbmm_bwd.
  */
 int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats,
                       int B, int M, int K, int N, void* stream);
@@ -83,7 +86,10 @@ int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats,
  * LogMatMul.backward (genmul.py:35-41; matmul_cuda.cpp:79-92;
  * matmul_cuda_kernel.cu:625-664, kernel :159-184).
  * grad_a or grad_b may be NULL (that gradient is then not computed), not both.
- * `stats`: NULL, or the buffer genbmm_logbmm_fwd filled for the same (a, b).
+ * `stats`: NULL, or the buffer genbmm_logbmm_fwd filled for the same (a, b)
+ * (the per-tile flags in it are rewritten, hence usable for any number of
+ * backward calls).  With both gradients requested a matrix-core problem is one
+ * launch.
  */
 int genbmm_logbmm_bwd(const float* a, const float* b, const float* out,
                       const float* g, const float* stats,
