@@ -189,3 +189,27 @@ def test_banded_errors(gpu):
         BandedMatrix(a, 1, 1).multiply(BandedMatrix(a, 1, 1))
     with pytest.raises(RuntimeError, match="disagree"):
         BandedMatrix(a.to(gpu), 1, 1).multiply_log(BandedMatrix(torch.randn(3, 5, 3, device=gpu), 1, 1))
+
+
+@pytest.mark.parametrize("case", range(4))
+def test_banded_products_match_reference_cpu_vectors(gpu, case):
+    """Outputs of the reference's own CPU loops (sparse.py:268-401), stored by
+    tests/golden/make_band_struct_fixtures.py: max is bit-exact, (+,x) and log to fp32
+    rounding (the GPU sums with fused multiply-adds / in factored form)."""
+    import os
+
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "band_struct.npz"),
+                allow_pickle=False)
+    p = "c%d_" % case
+    B, n, lu, ld, olu, old = (int(v) for v in z[p + "meta"])
+    a = BandedMatrix(torch.from_numpy(z[p + "zband"]).to(gpu), lu, ld)
+    b = BandedMatrix(torch.from_numpy(z[p + "zoband"]).to(gpu), olu, old)
+    for fn, name, exact in ((a.multiply, "multiply_simple", False), (a.multiply_log, "multiply_log_simple", False),
+                            (a.multiply_max, "multiply_max_simple", True)):
+        got = fn(b)
+        want = torch.from_numpy(z[p + name])
+        assert [got.lu, got.ld] == [int(v) for v in z[p + name + "_luld"]]
+        if exact:
+            assert torch.equal(got.data.cpu(), want), name
+        else:
+            assert torch.allclose(got.data.cpu(), want, rtol=1e-5, atol=1e-5), name

@@ -138,3 +138,43 @@ def test_install_as_genbmm():
     assert BM is BandedMatrix
     for k in ("genbmm", "genbmm.genmul", "genbmm.sparse"):
         sys.modules.pop(k, None)
+
+
+# ---------------------------------------------------------------- golden fixtures
+# tests/golden/band_struct.npz holds input / output vectors written by running the
+# reference's own pure-Python BandedMatrix methods (sparse.py:81-218) on the CPU
+# (tests/golden/make_band_struct_fixtures.py): the reference has no test for them.
+GOLDEN = os.path.join(ROOT, "tests", "golden", "band_struct.npz")
+
+
+def _golden():
+    import numpy as np
+
+    return np.load(GOLDEN, allow_pickle=False)
+
+
+@pytest.mark.parametrize("case", range(4))
+def test_band_structural_ops_match_reference_vectors(case):
+    z = _golden()
+    p = "c%d_" % case
+    B, n, lu, ld, olu, old = (int(v) for v in z[p + "meta"])
+    fill = float(z[p + "fill"])
+    bm = BandedMatrix(torch.from_numpy(z[p + "band"]), lu, ld, fill)
+    om = BandedMatrix(torch.from_numpy(z[p + "oband"]), olu, old, fill)
+
+    def same(name, m):
+        assert [m.lu, m.ld] == [int(v) for v in z[p + name + "_luld"]], name
+        assert torch.equal(m.data, torch.from_numpy(z[p + name])), name
+
+    same("band_shift_p1", bm.band_shift(1))
+    same("band_shift_m2", bm.band_shift(-2))
+    same("band_pad_2", bm.band_pad(2))
+    same("band_unshift", bm.band_unshift())
+    same("col_shift_p1", bm.col_shift(1))
+    same("col_shift_m2", bm.col_shift(-2))
+    same("col_unshift", bm.col_unshift())
+    same("expand", bm._expand(lu + 2, ld + 1))
+    same("op_add", bm.op(om, lambda x, y: x + y, zero=0))
+    same("op_max", bm.op(om, torch.max, zero=-1e9))
+    same("transpose", bm.transpose())
+    assert torch.equal(bm.to_dense(), torch.from_numpy(z[p + "to_dense"]))

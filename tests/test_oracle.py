@@ -278,3 +278,27 @@ def test_seq_band_bwdbwd_matches_autograd(n, a_lu, a_ld, b_lu, b_ld):
     want = torch.autograd.grad(ga, (ar, br, gr), u)
     for x, y in zip(got, want):
         assert torch.allclose(x, y, rtol=1e-9, atol=1e-11)
+
+
+# ------------------------------------------------------------- golden fixtures
+# Vectors written by the reference's own CPU code (the *_simple Python loops of
+# genbmm/sparse.py:268-401, run by tests/golden/make_band_struct_fixtures.py).
+@pytest.mark.parametrize("case", range(4))
+def test_band_products_match_reference_cpu_loops(case):
+    import os
+
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "band_struct.npz"),
+                allow_pickle=False)
+    p = "c%d_" % case
+    B, n, lu, ld, olu, old = (int(v) for v in z[p + "meta"])
+    a, b = torch.from_numpy(z[p + "zband"]), torch.from_numpy(z[p + "zoband"])
+    for mode, name in ((3, "multiply_simple"), (0, "multiply_log_simple"), (1, "multiply_max_simple")):
+        got = oracle.seq_band_fwd(a, lu, ld, b, olu, old, mode)[0]
+        assert [lu + old, ld + olu] == [int(v) for v in z[p + name + "_luld"]]
+        assert torch.equal(got, torch.from_numpy(z[p + name])), name   # same loop order, fp32: bit for bit
+    # multiply_back_simple returns the first operand's gradient in transposed band form
+    g = torch.from_numpy(z[p + "grad_out"])
+    ga, _ = oracle.seq_band_bwd(a, lu, ld, b, olu, old, g, 3)
+    want = torch.from_numpy(z[p + "multiply_back_simple"])
+    assert [ld, lu] == [int(v) for v in z[p + "multiply_back_simple_luld"]]
+    assert torch.allclose(oracle.band_transpose(ga, lu, ld), want, rtol=1e-6, atol=1e-6)
