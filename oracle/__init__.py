@@ -13,8 +13,11 @@ Two layers:
   of Philox4x32-10.
 
 What pins the oracle itself is listed in tests/test_oracle.py.  The reference
-has no stored vectors for this path; it cannot be built here (CUDA only), so
-there is no oracle/_ref.
+has no stored vectors for this path and cannot be built here (CUDA only), so
+there is no oracle/_ref; the band products are additionally pinned by vectors
+that the reference's own CPU loops produced (tests/golden/band_struct.npz).
+Parity unpinned: only the random stream of samplebmm (the reference draws from
+torch's CUDA generator); its decision rule and distribution are pinned.
 """
 import ctypes
 import os

@@ -64,9 +64,9 @@ def test_col_shift(batch, n):
 
 
 def test_band_relabel_ops():
-    """band_shift / band_pad / band_unshift: the reference has no test for these; they
-    are pure relabelling of the same cells (sparse.py:96-152), checked here on the dense
-    matrix they denote."""
+    """band_shift / band_pad / band_unshift are pure relabelling of the same cells
+    (sparse.py:96-152): checked here on the dense matrix they denote, and further down
+    against the reference's own outputs."""
     band, _ = banddiag(torch.rand(2, 7, 7), 2, 3)
     bx = BandedMatrix(band, 2, 3, fill=0)
     x = bx.to_dense()
