@@ -57,7 +57,7 @@ def report(name, ms, ops, nbytes, extra=None):
     print(json.dumps(line), flush=True)
 
 
-def dense_log(lib, dev, B, M, K, N, reps, name, dist="randn", path=0):
+def dense_log(lib, dev, B, M, K, N, reps, name, dist="randn", path=0, graph=False):
     torch.manual_seed(0)
     mk = torch.randn if dist == "randn" else torch.rand
     a, b = mk(B, M, K).to(dev), mk(B, K, N).to(dev)
@@ -78,11 +78,20 @@ def dense_log(lib, dev, B, M, K, N, reps, name, dist="randn", path=0):
         bw()
 
     ms, mf, mb = timed(step, reps), timed(f, reps), timed(bw, reps)
+    extra_graph = {}
+    if graph:  # the same step captured once into a HIP graph and replayed (launch-bound shapes)
+        gr, cap = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+        cap.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.graph(gr, stream=cap):
+            s = _lib.stream_of(a)
+            step()
+        s = _lib.stream_of(a)
+        extra_graph = {"ms_graph_replay": round(timed(gr.replay, reps), 4)}
     lib.genbmm_logbmm_force_exact(0)
     bmkn = float(B) * M * K * N
     nbytes = 4.0 * B * (3 * M * K + 3 * K * N + 3 * M * N)
     report(name, ms, 6 * bmkn, nbytes, {"path": {0: "factored", 1: "online-exact", 2: "factored-valu"}[path],
-                                        "ms_fwd": round(mf, 4), "ms_bwd": round(mb, 4)})
+                                        "ms_fwd": round(mf, 4), "ms_bwd": round(mb, 4), **extra_graph})
 
 
 def dense_max(lib, dev, B, M, K, N, reps, prod):
@@ -201,7 +210,7 @@ def main():
     dev = torch.device("cuda:0")
     r = args.reps
     if "log" in want:
-        dense_log(lib, dev, 16, 64, 64, 64, r, "logbmm fwd+bwd (16,64,64,64) config 0", dist="rand")
+        dense_log(lib, dev, 16, 64, 64, 64, r, "logbmm fwd+bwd (16,64,64,64) config 0", dist="rand", graph=True)
         dense_log(lib, dev, 512, 128, 128, 128, r, "logbmm fwd+bwd (512,128,128,128) config 1")
         dense_log(lib, dev, 8192, 32, 32, 32, r, "logbmm fwd+bwd (8192,32,32,32) config 1 skinny")
         for path in (0, 2, 1):

@@ -453,3 +453,85 @@ def test_empty_and_half(gpu):
     close(out.float(), lse64(a.float().cpu(), b.float().cpu()), rtol=2e-3, atol=2e-3)
     (ga,) = torch.autograd.grad(out.sum(), a)
     assert ga.dtype == torch.float16
+
+
+# ------------------------------------------------------- streams and HIP graphs
+@pytest.mark.parametrize("B,M,K,N", [(5, 33, 70, 129), (32, 256, 128, 256)])
+def test_logbmm_on_a_side_stream_and_in_a_graph(gpu, B, M, K, N):
+    """The library only enqueues kernels on the stream it is handed (no allocation, no
+    synchronisation, no memset): the same calls must give the same bits on a side stream
+    and when captured into a HIP graph and replayed, with eager work between replays."""
+    lib = _lib.load()
+    torch.manual_seed(B + N)
+    a, b, g = (torch.randn(s, device=gpu) for s in ((B, M, K), (B, K, N), (B, M, N)))
+    p = _lib.ptr
+
+    def buffers():
+        return (torch.empty(B, M, N, device=gpu), torch.empty_like(a), torch.empty_like(b),
+                torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=gpu))
+
+    def enqueue(out, ga, gb, stats, stream):
+        s = ctypes.c_void_p(stream.cuda_stream)
+        assert lib.genbmm_logbmm_fwd(p(a), p(b), p(out), p(stats), B, M, K, N, s) == 0
+        assert lib.genbmm_logbmm_bwd(p(a), p(b), p(out), p(g), p(stats), p(ga), p(gb), B, M, K, N, s) == 0
+
+    out0, ga0, gb0, st0 = buffers()
+    enqueue(out0, ga0, gb0, st0, torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    want, wa, wb = oracle.logbmm_grads64(a[:2].cpu(), b[:2].cpu(), g[:2].cpu())
+    close(out0[:2], want)
+    close(ga0[:2], wa)
+    close(gb0[:2], wb)
+
+    side = torch.cuda.Stream()               # default priority
+    out1, ga1, gb1, st1 = buffers()
+    side.wait_stream(torch.cuda.current_stream())
+    enqueue(out1, ga1, gb1, st1, side)
+    side.synchronize()
+    assert torch.equal(out1, out0) and torch.equal(ga1, ga0) and torch.equal(gb1, gb0)
+
+    out2, ga2, gb2, st2 = buffers()
+    graph = torch.cuda.CUDAGraph()
+    cap = torch.cuda.Stream()
+    cap.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.graph(graph, stream=cap):
+        enqueue(out2, ga2, gb2, st2, torch.cuda.current_stream())
+    for rep in range(3):
+        out2.fill_(float("nan")); ga2.fill_(float("nan")); gb2.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out2, out0) and torch.equal(ga2, ga0) and torch.equal(gb2, gb0), rep
+        (a * 2).sum().item()                 # eager work and a sync between replays
+
+
+def test_maxbmm_and_banded_in_a_graph(gpu):
+    lib = _lib.load()
+    torch.manual_seed(5)
+    B, M, K, N = 4, 40, 50, 36
+    a, b = torch.randn(B, M, K, device=gpu), torch.randn(B, K, N, device=gpu)
+    out, idx = torch.empty(B, M, N, device=gpu), torch.empty(B, M, N, dtype=torch.int32, device=gpu)
+    n, lu, ld = 70, 3, 2
+    W = lu + ld + 1
+    xa, xb = torch.randn(B, n, W, device=gpu), torch.randn(B, n, W, device=gpu)
+    bo = torch.empty(B, n, 2 * W - 1, device=gpu)
+    p = _lib.ptr
+
+    def enqueue(stream):
+        s = ctypes.c_void_p(stream.cuda_stream)
+        assert lib.genbmm_maxbmm_fwd(p(a), p(b), p(out), p(idx), B, M, K, N, s) == 0
+        assert lib.genbmm_banded_fwd(p(xa), lu, ld, p(xb), lu, ld, p(bo), p(None), B, n, 0, s) == 0
+
+    enqueue(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    ref = (out.clone(), idx.clone(), bo.clone())
+    graph = torch.cuda.CUDAGraph()
+    cap = torch.cuda.Stream()
+    cap.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.graph(graph, stream=cap):
+        enqueue(torch.cuda.current_stream())
+    for rep in range(3):
+        out.zero_(); idx.zero_(); bo.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref[0]) and torch.equal(idx, ref[1]) and torch.equal(bo, ref[2]), rep
+        (a + 1).sum().item()
