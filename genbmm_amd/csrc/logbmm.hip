@@ -32,6 +32,7 @@
 
 #include "dense_tiles.h"
 #include "log_bwd_tile.h"
+#include "logbmm_item.h"
 #include "logbmm_mfma.h"
 
 namespace genbmm {
@@ -558,6 +559,11 @@ inline int64_t header_offset(int B, int M, int K, int N) {
   const int64_t o = (int64_t)B * (M + N) + tiles32(B, M, N) + tiles32(B, M, K) + tiles32(B, K, N);
   return (o + 3) & ~(int64_t)3;
 }
+// Small matrices: a whole batch item per workgroup (logbmm_item.h).
+inline bool item_shape(int M, int K, int N) {
+  return M >= 1 && K >= 1 && N >= 1 && M <= 64 && K <= 64 && N <= 64;
+}
+
 // Shapes whose forward runs on the matrix cores (given alignment and path).
 inline bool fwd_mfma_shape(int B, int M, int K, int N) {
   if (K <= 0 || K % kMS != 0 || M % 128 != 0 || N % 128 != 0 || M == 0 || N == 0) return false;
@@ -756,6 +762,13 @@ int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats, 
   const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
   if (missing(a, mk) || missing(b, kn) || missing(out, mn)) return GENBMM_E_NULLPTR;
   hipStream_t s = (hipStream_t)stream;
+  if (stats && B > 0 && item_shape(M, K, N) && g_path.load() == 0) {  // whole items per workgroup
+    if (max(max(M, K), N) <= 32)
+      hipLaunchKernelGGL((k_log_item_fwd<16, 2>), dim3(B), dim3(256), 0, s, a, b, out, stats, M, K, N);
+    else
+      hipLaunchKernelGGL((k_log_item_fwd<16, 4>), dim3(B), dim3(256), 0, s, a, b, out, stats, M, K, N);
+    return launch_status();
+  }
   if (stats) {
     if (int e = launch_stats(a, b, stats, B, M, K, N, s)) return e;
   }
@@ -799,6 +812,13 @@ int genbmm_logbmm_bwd(const float* a, const float* b, const float* out, const fl
   p.vec_n = (N % 4 == 0) && aligned16(b) && aligned16(out) && aligned16(g) && aligned16(grad_b);
   hipStream_t s = (hipStream_t)stream;
   const float* st = (g_path.load() == 1 || mn == 0) ? nullptr : stats;
+  if (st && B > 0 && item_shape(M, K, N) && g_path.load() == 0) {
+    if (max(max(M, K), N) <= 32)
+      hipLaunchKernelGGL((k_log_item_bwd<16, 2>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
+    else
+      hipLaunchKernelGGL((k_log_item_bwd<16, 4>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
+    return launch_status();
+  }
   if (st && grad_a && grad_b && mk > 0 && kn > 0 && fwd_mfma_shape(B, M, K, N)) {
     const bool al = p.vec_k && p.vec_n && aligned16(st) && M % 4 == 0 && N % 4 == 0;
     const int ka = mfma_kind(B, M, K, N, al, true), kb = mfma_kind(B, K, N, M, al, false);

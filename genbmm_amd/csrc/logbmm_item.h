@@ -1,0 +1,284 @@
+// logbmm for small matrices (M, K, N <= 64): one workgroup per batch item, the
+// whole item in LDS, one launch for the forward and one for both gradients.
+// At these sizes the problem is launch- and HBM-bound (a 32^3 item is 12 KB of
+// operands and 0.2 M products), so the kernels read every operand exactly once
+// and write every result exactly once, in contiguous runs.
+//
+// Same factored form as the large kernels: alpha[m] = max_k a, beta[n] = max_k b
+// are taken inside the workgroup, EA = exp(a - alpha), EB = exp(b - beta),
+// S = EA * EB, out = log S + alpha + beta, H = g * exp(alpha + beta - out),
+// grad_a = EA .* (H * EB^T), grad_b = EB .* (EA^T * H).  A cell (forward) or an
+// item (backward) for which the factoring is not exact to fp32 - S < 2^-40, a
+// shift at the reference's -1e9 floor, anything non-finite - is recomputed inside
+// the same kernel from global memory with the reference's own two-pass form.
+#pragma once
+
+#include "common.h"
+
+namespace genbmm {
+
+constexpr float kItemGuardBits = 40.f;
+
+// log-sum-exp of a[m,:] + b[:,n] the way the reference's kernel does it
+// (matmul_cuda_kernel.cu:27-41): running maximum from -1e9, then the sum.
+__device__ __forceinline__ float item_exact_out(const float* __restrict__ arow,
+                                                const float* __restrict__ bcol, int K, int N) {
+  float mx = kFloor;
+  for (int k = 0; k < K; ++k) mx = fmaxf(mx, arow[k] + bcol[(long)k * N]);
+  const float nm = -mx * kLog2e;
+  float s = 0.f;
+  for (int k = 0; k < K; ++k) s += fast_exp2(__builtin_fmaf(arow[k] + bcol[(long)k * N], kLog2e, nm));
+  return logf(s) + mx;
+}
+
+// (row, column) of elements tid, tid + nt, tid + 2 nt, ... of a row-major array
+// with C columns, without a division per element.
+struct RowMajorWalk {
+  int r, c, dr, dc, C;
+  __device__ __forceinline__ RowMajorWalk(int tid, int nt, int cols) : C(cols) {
+    r = tid / C;
+    c = tid - r * C;
+    dr = nt / C;
+    dc = nt - dr * C;
+  }
+  __device__ __forceinline__ void next() {
+    r += dr;
+    c += dc;
+    if (c >= C) {
+      c -= C;
+      ++r;
+    }
+  }
+};
+
+// exp(x - shift), with the all -inf row / column (shift = -inf) giving zeros
+__device__ __forceinline__ float item_exp(float x, float shift) {
+  return fast_exp2((x - (shift == -INFINITY ? 0.f : shift)) * kLog2e);
+}
+
+// TB x TB outputs per thread on a G x G thread grid.  Used with G = 16: TB = 2
+// covers items up to 32 x 32, TB = 4 up to 64 x 64.  (One wave per item, G = 8 and
+// TB = 4, measured slower at 8192 items of 32^3: the chain of dependent phases of
+// an item gets longer than the extra items in flight make up for.)
+template <int G, int TB>
+__global__ __launch_bounds__(G * G) void k_log_item_fwd(const float* __restrict__ a,
+                                                      const float* __restrict__ b,
+                                                      float* __restrict__ out,
+                                                      float* __restrict__ stats, int M, int K,
+                                                      int N) {
+  constexpr int NT = G * G, S = G * TB, LD = S + 1;
+  static_assert(2 * S <= NT, "row and column scans use 2*S threads");
+  __shared__ float At[S * LD];  // [k][m]: a, then EA; finally the output tile [m][n]
+  __shared__ float Bs[S * LD];  // [k][n]: b, then EB
+  __shared__ float al[S], be[S];
+  const int tid = threadIdx.x, batch = blockIdx.x;
+  const float* ab = a + (long)batch * M * K;
+  const float* bb = b + (long)batch * K * N;
+  for (RowMajorWalk w(tid, NT, K); w.r < M; w.next()) {
+    const int m = w.r, k = w.c, e = w.r * K + w.c;
+    At[k * LD + m] = ab[e];
+  }
+  for (RowMajorWalk w(tid, NT, N); w.r < K; w.next()) {
+    const int k = w.r, n = w.c, e = w.r * N + w.c;
+    Bs[k * LD + n] = bb[e];
+  }
+  __syncthreads();
+  // row / column maxima: one thread per row, one per column (LDS atomics on the
+  // shared maximum while loading measured slower: 32 lanes on one address)
+  if (tid < M) {
+    float mx = -INFINITY;
+    for (int k = 0; k < K; ++k) mx = fmaxf(mx, At[k * LD + tid]);
+    al[tid] = mx;
+  } else if (tid >= S && tid - S < N) {
+    float mx = -INFINITY;
+    for (int k = 0; k < K; ++k) mx = fmaxf(mx, Bs[k * LD + tid - S]);
+    be[tid - S] = mx;
+  }
+  __syncthreads();
+  for (RowMajorWalk w(tid, NT, K); w.r < M; w.next()) {
+    const int m = w.r, k = w.c;
+    At[k * LD + m] = item_exp(At[k * LD + m], al[m]);
+  }
+  for (RowMajorWalk w(tid, NT, N); w.r < K; w.next()) {
+    const int k = w.r, n = w.c, e = w.r * N + w.c;
+    Bs[k * LD + n] = item_exp(Bs[k * LD + n], be[n]);
+  }
+  if (stats) {
+    float* st = stats + (long)batch * (M + N);
+    if (tid < M) st[tid] = al[tid];
+    else if (tid >= S && tid - S < N) st[M + tid - S] = be[tid - S];
+  }
+  __syncthreads();
+
+  const int ty = tid / G, tx = tid % G;
+  float acc[TB][TB];
+#pragma unroll
+  for (int i = 0; i < TB; ++i)
+#pragma unroll
+    for (int j = 0; j < TB; ++j) acc[i][j] = 0.f;
+#pragma unroll 4
+  for (int k = 0; k < K; ++k) {
+    float av[TB], bv[TB];
+#pragma unroll
+    for (int i = 0; i < TB; ++i) av[i] = At[k * LD + ty * TB + i];
+#pragma unroll
+    for (int j = 0; j < TB; ++j) bv[j] = Bs[k * LD + tx * TB + j];
+#pragma unroll
+    for (int i = 0; i < TB; ++i)
+#pragma unroll
+      for (int j = 0; j < TB; ++j) acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
+  }
+  __syncthreads();  // At becomes the output tile
+  const float thr = fast_exp2(-kItemGuardBits);
+#pragma unroll
+  for (int i = 0; i < TB; ++i)
+#pragma unroll
+    for (int j = 0; j < TB; ++j) {
+      const int m = ty * TB + i, n = tx * TB + j;
+      if (m < M && n < N) {
+        const float shift = al[m] + be[n], s = acc[i][j];
+        const bool ok = (s >= thr) && (s < INFINITY) && (shift > 0.9f * kFloor) && (shift < INFINITY);
+        At[m * LD + n] = ok ? __builtin_fmaf(fast_log2(s), kLn2, shift)
+                            : item_exact_out(ab + (long)m * K, bb + n, K, N);
+      }
+    }
+  __syncthreads();
+  float* ob = out + (long)batch * M * N;
+  for (RowMajorWalk w(tid, NT, N); w.r < M; w.next()) {
+    const int m = w.r, n = w.c, e = w.r * N + w.c;
+    ob[e] = At[m * LD + n];
+  }
+}
+
+template <int G, int TB>
+__global__ __launch_bounds__(G * G) void k_log_item_bwd(const float* __restrict__ a,
+                                                      const float* __restrict__ b,
+                                                      const float* __restrict__ outp,
+                                                      const float* __restrict__ g,
+                                                      float* __restrict__ grad_a,
+                                                      float* __restrict__ grad_b, int M, int K,
+                                                      int N) {
+  constexpr int NT = G * G, S = G * TB, LD = S + 1;
+  static_assert(2 * S <= NT, "row and column scans use 2*S threads");
+  __shared__ float Ea[S * LD];  // [m][k]: a, EA, finally grad_a
+  __shared__ float Eb[S * LD];  // [k][n]: b, EB, finally grad_b
+  __shared__ float Hs[S * LD];  // [m][n]: H
+  __shared__ float al[S], be[S];
+  const int tid = threadIdx.x, batch = blockIdx.x;
+  const float* ab = a + (long)batch * M * K;
+  const float* bb = b + (long)batch * K * N;
+  const float* ob = outp + (long)batch * M * N;
+  const float* gb = g + (long)batch * M * N;
+  float* gab = grad_a ? grad_a + (long)batch * M * K : nullptr;
+  float* gbb = grad_b ? grad_b + (long)batch * K * N : nullptr;
+  for (RowMajorWalk w(tid, NT, K); w.r < M; w.next()) {
+    const int m = w.r, k = w.c, e = w.r * K + w.c;
+    Ea[m * LD + k] = ab[e];
+  }
+  for (RowMajorWalk w(tid, NT, N); w.r < K; w.next()) {
+    const int k = w.r, n = w.c, e = w.r * N + w.c;
+    Eb[k * LD + n] = bb[e];
+  }
+  __syncthreads();
+  if (tid < M) {
+    float mx = -INFINITY;
+    for (int k = 0; k < K; ++k) mx = fmaxf(mx, Ea[tid * LD + k]);
+    al[tid] = mx;
+  } else if (tid >= S && tid - S < N) {
+    float mx = -INFINITY;
+    for (int k = 0; k < K; ++k) mx = fmaxf(mx, Eb[k * LD + tid - S]);
+    be[tid - S] = mx;
+  }
+  __syncthreads();
+  const float lim = kItemGuardBits * kLn2 + 1e-3f;
+  int bad = 0;
+  for (RowMajorWalk w(tid, NT, K); w.r < M; w.next()) {
+    const int m = w.r, k = w.c, e = w.r * K + w.c;
+    Ea[m * LD + k] = item_exp(Ea[m * LD + k], al[m]);
+  }
+  for (RowMajorWalk w(tid, NT, N); w.r < K; w.next()) {
+    const int k = w.r, n = w.c, e = w.r * N + w.c;
+    Eb[k * LD + n] = item_exp(Eb[k * LD + n], be[n]);
+  }
+  for (RowMajorWalk w(tid, NT, N); w.r < M; w.next()) {
+    const int m = w.r, n = w.c, e = w.r * N + w.c;
+    const float ex = al[m] + be[n] - ob[e];
+    if (!(ex <= lim) || !(ex > -INFINITY)) bad = 1;  // S < 2^-40, NaN or infinities: not exact
+    Hs[m * LD + n] = gb[e] * fast_exp2(ex * kLog2e);
+  }
+  bad = __syncthreads_or(bad);
+  if (bad) {
+    // the reference's form for the whole item (matmul_cuda_kernel.cu:159-184):
+    // exp(a + b - out) * g summed over n (grad_a) / m (grad_b), from global memory
+    if (gab)
+      for (int e = tid; e < M * K; e += NT) {
+        const int m = e / K, k = e - m * K;
+        const float av = ab[e];
+        float s = 0.f;
+        for (int n = 0; n < N; ++n)
+          s = __builtin_fmaf(fast_exp(av + bb[(long)k * N + n] - ob[(long)m * N + n]), gb[(long)m * N + n], s);
+        gab[e] = s;
+      }
+    if (gbb)
+      for (int e = tid; e < K * N; e += NT) {
+        const int k = e / N, n = e - k * N;
+        const float bv = bb[e];
+        float s = 0.f;
+        for (int m = 0; m < M; ++m)
+          s = __builtin_fmaf(fast_exp(ab[(long)m * K + k] + bv - ob[(long)m * N + n]), gb[(long)m * N + n], s);
+        gbb[e] = s;
+      }
+    return;
+  }
+
+  const int ty = tid / G, tx = tid % G;
+  float ga[TB][TB], gw[TB][TB];
+#pragma unroll
+  for (int i = 0; i < TB; ++i)
+#pragma unroll
+    for (int j = 0; j < TB; ++j) ga[i][j] = gw[i][j] = 0.f;
+  if (gab) {  // rows m = ty*TB+i, columns k = tx*TB+j, sum over n
+#pragma unroll 4
+    for (int n = 0; n < N; ++n) {
+      float hv[TB], ev[TB];
+#pragma unroll
+      for (int i = 0; i < TB; ++i) hv[i] = Hs[(ty * TB + i) * LD + n];
+#pragma unroll
+      for (int j = 0; j < TB; ++j) ev[j] = Eb[(tx * TB + j) * LD + n];
+#pragma unroll
+      for (int i = 0; i < TB; ++i)
+#pragma unroll
+        for (int j = 0; j < TB; ++j) ga[i][j] = __builtin_fmaf(hv[i], ev[j], ga[i][j]);
+    }
+  }
+  if (gbb) {  // rows k = ty*TB+i, columns n = tx*TB+j, sum over m
+#pragma unroll 4
+    for (int m = 0; m < M; ++m) {
+      float ev[TB], hv[TB];
+#pragma unroll
+      for (int i = 0; i < TB; ++i) ev[i] = Ea[m * LD + ty * TB + i];
+#pragma unroll
+      for (int j = 0; j < TB; ++j) hv[j] = Hs[m * LD + tx * TB + j];
+#pragma unroll
+      for (int i = 0; i < TB; ++i)
+#pragma unroll
+        for (int j = 0; j < TB; ++j) gw[i][j] = __builtin_fmaf(ev[i], hv[j], gw[i][j]);
+    }
+  }
+  __syncthreads();  // all sums taken: scale in place, each thread its own cells
+#pragma unroll
+  for (int i = 0; i < TB; ++i)
+#pragma unroll
+    for (int j = 0; j < TB; ++j) {
+      const int r = ty * TB + i, c = tx * TB + j;
+      Ea[r * LD + c] *= ga[i][j];
+      Eb[r * LD + c] *= gw[i][j];
+    }
+  __syncthreads();
+  if (gab)
+    for (RowMajorWalk w(tid, NT, K); w.r < M; w.next()) gab[w.r * K + w.c] = Ea[w.r * LD + w.c];
+  if (gbb)
+    for (RowMajorWalk w(tid, NT, N); w.r < K; w.next()) gbb[w.r * N + w.c] = Eb[w.r * LD + w.c];
+}
+
+}  // namespace genbmm
