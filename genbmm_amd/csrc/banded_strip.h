@@ -70,6 +70,28 @@ struct RowStage {
 
   __device__ __forceinline__ void load(const float* __restrict__ src, int W, int lu, int n, int row0,
                                        int ld, int pad, int wave, int lane) {
+    const float fill = SEM == kSemMul ? 0.f : -INFINITY;
+    // Strips away from the matrix edges (all but a few per batch item): every staged
+    // row exists and every band cell of it lies inside the matrix, so the only
+    // predicate left is the lane's own column - one masked region per q instead of
+    // five comparisons per element.
+    const bool interior = row0 - lu >= 0 && row0 + ROWS + W - 2 - lu <= n - 1;  // uniform
+    if (interior) {
+      const float* base = src + (long)(row0 + wave) * W - pad + lane;
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        const int col = lane + 64 * q, k = col - pad;
+        const bool kin = col < ld && k >= 0 && k < W;
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u][q] = fill;
+        if (kin) {
+#pragma unroll
+          for (int u = 0; u < U; ++u)
+            if (4 * u + 3 < ROWS || wave + 4 * u < ROWS) v[u][q] = base[(long)(4 * u) * W + 64 * q];
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int r = wave + 4 * u, c = row0 + r;  // c: matrix column = row of the band tensor
@@ -78,7 +100,7 @@ struct RowStage {
         const int col = lane + 64 * q, k = col - pad;
         const int prow = c + k - lu;  // dense row of this cell
         const bool ok = r < ROWS && col < ld && c >= 0 && c < n && k >= 0 && k < W && prow >= 0 && prow < n;
-        v[u][q] = ok ? src[(long)c * W + k] : (SEM == kSemMul ? 0.f : -INFINITY);
+        v[u][q] = ok ? src[(long)c * W + k] : fill;
       }
     }
   }
@@ -101,7 +123,7 @@ struct RowStage {
 #pragma unroll
         for (int q = 0; q < NQ; ++q) {
           const int col = lane + 64 * q;
-          if (col < ld) tile[r * ld + col] = LOG ? fast_exp2((v[u][q] - m) * kLog2e) : v[u][q];
+          if (tile && col < ld) tile[r * ld + col] = LOG ? fast_exp2((v[u][q] - m) * kLog2e) : v[u][q];
         }
       }
     }
@@ -250,17 +272,69 @@ __global__ __launch_bounds__(256, SEM == kSemMul ? 3 : 2) void k_band_fwd_strip(
 // operand on an anti-diagonal of its tile.
 //   grad_a: g'[x][j]            * b'[x + j - lu_o][kk - j + Wb - 1]
 //   grad_b: g'[x - j + lu_o][j] * a'[x - j + lu_o][kk + j - (Wb - 1)]
+// The g' tile of one chunk of 32 diagonals: rows x of g (grad_a, 64 rows) or rows
+// x - j + lu_o (grad_b, 95 rows).  load() issues all global reads of g (and out)
+// of the tile, store() turns them into g' = g (or H = g * exp(alpha + beta - out))
+// in LDS.  A cell
+// counts if it lies inside the matrix and, for grad_b, if its b row is in the strip.
+template <bool LOG, bool GRAD_A>
+struct GStage {
+  static constexpr int ROWS = GRAD_A ? kBT : kBR;
+  static constexpr int PER = (ROWS * kBJ + 255) / 256;
+  float gv[PER], ov[PER];
+  unsigned used;
+
+  __device__ __forceinline__ void load(const float* __restrict__ gb, const float* __restrict__ ob,
+                                       int x0, int yb, int jc, int n, int Wo, int r_lu, int tid) {
+    used = 0;
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int e = tid + 256 * u, r = e >> 5, c = e & 31, j = jc + c;
+      const int i = GRAD_A ? x0 + r : yb + r;  // row of g / out (a's row index)
+      const int o = i + j - r_lu;              // b's row index of this cell
+      const bool inside = r < ROWS && i >= 0 && i < n && j < Wo && o >= 0 && o < n;
+      const bool use = inside && (GRAD_A || (o >= x0 && o < x0 + kBT));
+      gv[u] = use ? gb[(long)i * Wo + j] : 0.f;
+      ov[u] = (LOG && use) ? ob[(long)i * Wo + j] : 0.f;
+      used |= (use ? 1u : 0u) << u;
+    }
+  }
+
+  __device__ __forceinline__ void store(float* __restrict__ gt, const float* __restrict__ sh_own,
+                                        const float* __restrict__ sh_sl, int* __restrict__ badrow,
+                                        int x0, int yb, int jc, int r_lu, float lim, int tid) const {
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int e = tid + 256 * u, r = e >> 5, c = e & 31;
+      if (r >= ROWS) continue;
+      float v = gv[u];
+      if (LOG && ((used >> u) & 1u)) {
+        const int o = (GRAD_A ? x0 + r : yb + r) + jc + c - r_lu;
+        // alpha[i] + beta[o] - out[i,j]
+        const float sa = GRAD_A ? sh_own[r] : sh_sl[r];
+        const float sb = GRAD_A ? sh_sl[r + c] : sh_own[o - x0];
+        const float ex = sa + sb - ov[u];
+        if (!(ex <= lim)) badrow[GRAD_A ? r : o - x0] = 1;  // factoring not exact: row redone
+        v *= fast_exp2(ex * kLog2e);
+      }
+      gt[r * kBC + c] = v;
+    }
+  }
+};
+
 constexpr int kMaxKB = 3;  // band-axis blocks of 8 per wave: widths up to 96
 
 template <bool LOG, bool GRAD_A, int NQ>
-__global__ __launch_bounds__(256, 2) void k_band_bwd_strip(const BandArgs p, int strips, int ld_own,
+__global__ __launch_bounds__(256, 3) void k_band_bwd_strip(const BandArgs p, int strips, int ld_own,
                                                            int ld_sl, int sl_floats) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  // own: the output operand's strip (LOG: exp(x - shift), for the epilogue)
-  // sl : 95 rows of the other operand, padded (LOG: exp(y - shift))
+  // sl : 95 rows of the other operand, padded (LOG: exp(y - shift)); reused as the
+  //      [64][ld_own] result tile at the end
   // gt : g' tile; grad_a [64][33] (row x), grad_b [95][33] (row x - j + lu_o)
-  float* own = smem;
-  float* sl = own + (LOG ? kBT * ld_own : 0);
+  // The output operand itself is only needed for its row maxima (LOG) and, in the
+  // epilogue, as the factor exp(x - shift), which is taken while the rows are
+  // written out.
+  float* sl = smem;
   float* gt = sl + sl_floats;      // sl_floats = max(95 * ld_sl, 64 * ld_own)
   float* sh_own = gt + kBR * kBC;  // [64] shift of the lane's own row
   float* sh_sl = sh_own + kBT;     // [95] shifts of the staged other-operand rows
@@ -286,7 +360,7 @@ __global__ __launch_bounds__(256, 2) void k_band_bwd_strip(const BandArgs p, int
   if (LOG) {
     RowStage<kSemLog, NQ, kBT> so;
     so.load(xo, Wx, lux, n, x0, ld_own, 0, wave, lane);
-    so.store(own, ld_own, sh_own, wave, lane);
+    so.store(nullptr, ld_own, sh_own, wave, lane);  // row maxima only
   }
   float acc[kMaxKB][8];
 #pragma unroll
@@ -305,30 +379,29 @@ __global__ __launch_bounds__(256, 2) void k_band_bwd_strip(const BandArgs p, int
     ss.store(sl, ld_sl, sh_sl, wave, lane);
     __syncthreads();  // sh_sl visible
     if (jc + kBJ < Wo) ss.load(yo, Wy, luy, n, row0_of(jc + kBJ), ld_sl, kBP, wave, lane);
-    // ---- g' tile
-    {
-      const int rows = GRAD_A ? kBT : kBR;
-      for (int e = tid; e < rows * kBJ; e += 256) {
+    // ---- g' tile.  (Starting these reads one chunk ahead, like the operand rows,
+    // measured slower: the extra live registers cost more than the latency.)
+    // The log kernels are short of registers: they go element by element.
+    if (LOG) {
+      for (int e = tid; e < GStage<LOG, GRAD_A>::ROWS * kBJ; e += 256) {
         const int r = e >> 5, c = e & 31, j = jc + c;
-        const int i = GRAD_A ? x0 + r : yb + r;  // row of g / out (a's row index)
-        const int o = i + j - p.r_lu;            // b's row index of this cell
-        float v = 0.f;
+        const int i = GRAD_A ? x0 + r : yb + r;
+        const int o = i + j - p.r_lu;
         const bool inside = i >= 0 && i < n && j < Wo && o >= 0 && o < n;
-        // grad_b only uses cells whose o lies in this strip
-        const bool used = inside && (GRAD_A || (o >= x0 && o < x0 + kBT));
-        if (used) {
-          v = gb[(long)i * Wo + j];
-          if (LOG) {
-            // alpha[i] + beta[o] - out[i,j]
-            const float sa = GRAD_A ? sh_own[r] : sh_sl[r];
-            const float sb = GRAD_A ? sh_sl[r + c] : sh_own[o - x0];
-            const float ex = sa + sb - ob[(long)i * Wo + j];
-            if (!(ex <= lim)) badrow[GRAD_A ? r : o - x0] = 1;  // factoring not exact: row redone
-            v *= fast_exp2(ex * kLog2e);
-          }
+        float v = 0.f;
+        if (inside && (GRAD_A || (o >= x0 && o < x0 + kBT))) {
+          const float sa = GRAD_A ? sh_own[r] : sh_sl[r];
+          const float sb = GRAD_A ? sh_sl[r + c] : sh_own[o - x0];
+          const float ex = sa + sb - ob[(long)i * Wo + j];  // alpha[i] + beta[o] - out[i,j]
+          if (!(ex <= lim)) badrow[GRAD_A ? r : o - x0] = 1;  // factoring not exact: row redone
+          v = gb[(long)i * Wo + j] * fast_exp2(ex * kLog2e);
         }
         gt[r * kBC + c] = v;
       }
+    } else {
+      GStage<LOG, GRAD_A> gs;
+      gs.load(gb, ob, x0, yb, jc, n, Wo, p.r_lu, tid);
+      gs.store(gt, sh_own, sh_sl, badrow, x0, yb, jc, p.r_lu, lim, tid);
     }
     __syncthreads();
     // ---- multiply
@@ -381,7 +454,7 @@ __global__ __launch_bounds__(256, 2) void k_band_bwd_strip(const BandArgs p, int
 #pragma unroll
     for (int t = 0; t < 8; ++t)
       if (k0 + t < Wx)
-        ct[lane * ld_own + k0 + t] = LOG ? own[lane * ld_own + k0 + t] * acc[q][t] : acc[q][t];
+        ct[lane * ld_own + k0 + t] = acc[q][t];
   }
   __syncthreads();
   for (int r = wave; r < kBT; r += 4) {
@@ -393,15 +466,25 @@ __global__ __launch_bounds__(256, 2) void k_band_bwd_strip(const BandArgs p, int
         else band_bwd_b_cell<GENBMM_BAND_LOG>(p, bn + x, x, k);
       }
     } else {
-      for (int k = lane; k < Wx; k += 64) gradb[(long)x * Wx + k] = ct[r * ld_own + k];
+      if (LOG) {
+        const float sh = sh_own[r] == -INFINITY ? 0.f : sh_own[r];
+        for (int k = lane; k < Wx; k += 64) {
+          // exp(x - shift); cells outside the matrix are excluded from the row maximum
+          // and their sum is 0
+          const float acv = ct[r * ld_own + k];
+          gradb[(long)x * Wx + k] = acv == 0.f ? 0.f : fast_exp2((xo[(long)x * Wx + k] - sh) * kLog2e) * acv;
+        }
+      } else {
+        for (int k = lane; k < Wx; k += 64) gradb[(long)x * Wx + k] = ct[r * ld_own + k];
+      }
     }
   }
 }
 
 inline int bwd_sl_floats(const StripDims& d) { return max(kBR * d.ld_sl, kBT * d.ld_own); }
 inline size_t bwd_strip_bytes(const StripDims& d, bool log_mode) {
-  return sizeof(float) * ((log_mode ? (size_t)kBT * d.ld_own : 0) + (size_t)bwd_sl_floats(d) +
-                          (size_t)kBR * kBC + kBT + kBR + kBT);
+  (void)log_mode;
+  return sizeof(float) * ((size_t)bwd_sl_floats(d) + (size_t)kBR * kBC + kBT + kBR + kBT);
 }
 
 inline StripDims strip_dims(int w_own, int w_sl) {
