@@ -9,9 +9,12 @@ Differences in mechanism (not in results):
   * logbmm's backward produces grad_a and grad_b from one library call that
     reads every operand in place; the reference calls its kernel twice and
     transposes b, a, g, out, maxes and the result in between (genmul.py:35-41).
-  * instead of the (B, M, N) `maxes` tensor the forward saves a B*(M+N) vector of
-    row maxima of a and column maxima of b (plus a few per-tile flags), which lets forward and backward factor
-    exp(a + b) wherever that is exact (see csrc/logbmm.hip).
+  * instead of the (B, M, N) `maxes` tensor the forward saves a workspace sized by
+    the library: row maxima of a, column maxima of b and a few per-tile flags,
+    which let forward and backward factor exp(a + b) wherever that is exact
+    (csrc/logbmm.hip), and - for shapes that run on the matrix cores - the
+    factors exp(a - max), exp(b - max) and 1/sum, so that the backward takes no
+    exponential at all (csrc/logbmm_mfma.h).
   * the arg-max / sample index stays int32 into the backward; the reference
     converts it (and a, b, g) to float first (genmul.py:62-65).
   * samplebmm draws its uniforms from a counter-based Philox4x32-10 stream
@@ -93,7 +96,7 @@ class LogMatMul(torch.autograd.Function):
         in_dtype = a.dtype if isinstance(a, torch.Tensor) else None
         a, b, (B, M, K, N) = _prep(a, b)
         out = torch.empty(B, M, N, dtype=_COMPUTE, device=a.device)
-        # row maxima of a, column maxima of b: what the reference's `maxes` becomes
+        # the library's workspace: what the reference's `maxes` becomes
         stats = torch.empty(_lib.load().genbmm_logbmm_stats_size(B, M, K, N), dtype=_COMPUTE,
                             device=a.device)
         _call("genbmm_logbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(stats),
