@@ -119,11 +119,14 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
   for (int t = tid; t < C::BN; t += C::NT) be[t] = (n0 + t < N) ? st[M + n0 + t] : 0.f;
   __syncthreads();
 
-  // tgt = u*S; the sampled index is the number of prefix sums that do not exceed it
-  // (prefix sums never decrease), which costs a multiply-add, a compare and an
-  // add-with-carry per term.
-  float tgt[C::TM][C::TN], cum[C::TM][C::TN];
-  int ind[C::TM][C::TN];
+  // With the target t = u*S, the sampled index is the number of prefix sums that do
+  // not exceed t (prefix sums never decrease).  Per cell: rem = t - prefix sum,
+  // updated by one multiply-add per term; its sign bit (set once the prefix sum
+  // has passed t; t - t = +0 keeps it clear) is shifted into a bit string by one
+  // v_alignbit_b32 and the bits of a slab are counted once per slab.
+  float rem[C::TM][C::TN];
+  uint32_t bits[C::TM][C::TN];
+  int ind[C::TM][C::TN];  // number of terms whose prefix sum exceeded t
   const float lim = 40.f * kLn2 + 1e-3f;
   int bad = 0;
 #pragma unroll
@@ -133,13 +136,12 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
       const int r = ty * C::TM + i, c = col_of<C>(tx, j);
       const int m = m0 + r, n = n0 + c;
       ind[i][j] = 0;
-      cum[i][j] = 0.f;
-      tgt[i][j] = 0.f;
+      rem[i][j] = 0.f;
       if (m < M && n < N) {
         const float e = al[r] + be[c] - ob[(long)m * N + n];   // -log S
         if (!(e <= lim) || !(e > -INFINITY)) bad = 1;
         const uint64_t cell = ((uint64_t)batch * M + m) * (uint64_t)N + n;
-        tgt[i][j] = philox_uniform(cell, p.seed, p.offset) * fast_exp2(-e * kLog2e);
+        rem[i][j] = philox_uniform(cell, p.seed, p.offset) * fast_exp2(-e * kLog2e);
       }
     }
   if (__syncthreads_or(bad)) {  // workgroup-uniform
@@ -177,6 +179,11 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
       tb.gload(bb, N, n0, k0 + C::KT, N, K, p.vec_b, tid);
     }
     const int kn = min(C::KT, K - k0);
+    static_assert(C::KT <= 32, "one bit per term of a slab");
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < C::TN; ++j) bits[i][j] = 0u;
     auto scan = [&](int kk) __attribute__((always_inline)) {
       float av[C::TM], bv[C::TN];
       lds_frag<C::TM / 4>(As + kk * C::LDA, ty * C::TM, 4, av);
@@ -185,8 +192,8 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
       for (int i = 0; i < C::TM; ++i)
 #pragma unroll
         for (int j = 0; j < C::TN; ++j) {
-          cum[i][j] = __builtin_fmaf(av[i], bv[j], cum[i][j]);
-          ind[i][j] += (cum[i][j] <= tgt[i][j]) ? 1 : 0;
+          rem[i][j] = __builtin_fmaf(-av[i], bv[j], rem[i][j]);
+          bits[i][j] = __builtin_amdgcn_alignbit(bits[i][j], __float_as_uint(rem[i][j]), 31);
         }
     };
     if (kn == C::KT) {
@@ -195,13 +202,17 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
     } else {
       for (int kk = 0; kk < kn; ++kk) scan(kk);
     }
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < C::TN; ++j) ind[i][j] += __builtin_popcount(bits[i][j]);
   }
-  // rounding can leave the last prefix sum a hair under u*S: no crossing -> index 0,
-  // as when the reference's walk never exceeds its draw
+  // index = K - (terms past t).  Rounding can leave the last prefix sum a hair under
+  // u*S: no crossing -> index 0, as when the reference's walk never exceeds its draw
 #pragma unroll
   for (int i = 0; i < C::TM; ++i)
 #pragma unroll
-    for (int j = 0; j < C::TN; ++j) ind[i][j] = ind[i][j] >= K ? 0 : ind[i][j];
+    for (int j = 0; j < C::TN; ++j) ind[i][j] = ind[i][j] == 0 ? 0 : K - ind[i][j];
   store_tile_i<C>(p.idx + (long)batch * M * N, ind, m0, n0, M, N, p.vec_o, tx, ty);
 }
 
