@@ -565,9 +565,18 @@ inline bool item_shape(int M, int K, int N) {
 }
 
 // Shapes whose forward runs on the matrix cores (given alignment and path).
+// Extents are multiples of 4 (a float4 is inside or outside the matrix as a whole),
+// large enough for 128-wide tiles to pay, and there are tiles enough for the chip;
+// ragged edges are handled by the kernels.
+inline bool mfma_extents(int out_r, int out_c, int red) {
+  return out_r % 4 == 0 && out_c % 4 == 0 && red % 4 == 0 && out_r >= 96 && out_c >= 96 && red >= kMS;
+}
+inline int64_t tiles128(int B, int out_r, int out_c) {
+  return (int64_t)B * ceil_div(out_r, 128) * ceil_div(out_c, 128);
+}
 inline bool fwd_mfma_shape(int B, int M, int K, int N) {
-  if (K <= 0 || K % kMS != 0 || M % 128 != 0 || N % 128 != 0 || M == 0 || N == 0) return false;
-  const int64_t t128 = (int64_t)B * (M / 128) * (N / 128);
+  if (!mfma_extents(M, N, K)) return false;
+  const int64_t t128 = tiles128(B, M, N);
   return t128 >= 128 && t128 <= 0x7fffffff;
 }
 inline LogPrepared prepared_of(const float* stats, int B, int M, int K, int N) {
@@ -605,18 +614,23 @@ int launch_fwd_fast(DenseArgs p, const float* stats, int* flags, int B, int M, i
   return launch_fwd_fixup<CX, C::BM, C::BN>(p, flags, (int)grid.x, s);
 }
 
-// Matrix-core launches: T is the MTile; the problem is made of full tiles.
+// Matrix-core launches: T is the MTile; the ragged variant of a kernel is used only
+// when some extent is not a multiple of its tile / slab.
 template <class T>
 int launch_fwd_mfma(DenseArgs p, const float* stats, int* flags, int B, int M, int K, int N,
                     hipStream_t s) {
   p.M = M; p.K = K; p.N = N;
-  p.tiles_m = M / T::TR;
-  p.tiles_n = N / T::TC;
+  p.tiles_m = ceil_div(M, T::TR);
+  p.tiles_n = ceil_div(N, T::TC);
   p.vec_a = p.vec_b = p.vec_o = 1;
   const int total = B * p.tiles_m * p.tiles_n;
   const LogPrepared ws = prepared_of(stats, B, M, K, N);
-  hipLaunchKernelGGL((k_log_fwd_mfma<T>), dim3(total), dim3(T::NT), 0, s, p.a, p.b, p.out, stats,
-                     flags, ws.ea, ws.eb, ws.r, ws.hdr, M, K, N, p.tiles_m, p.tiles_n);
+  auto go = [&](auto kern) {
+    hipLaunchKernelGGL(kern, dim3(total), dim3(T::NT), 0, s, p.a, p.b, p.out, stats, flags, ws.ea,
+                       ws.eb, ws.r, ws.hdr, M, K, N, p.tiles_m, p.tiles_n);
+  };
+  if (M % T::TR != 0 || N % T::TC != 0 || K % kMS != 0) go(k_log_fwd_mfma<T, true>);
+  else go(k_log_fwd_mfma<T, false>);
   if (int e = launch_status()) return e;
   return launch_fwd_fixup<CfgWide, T::TR, T::TC>(p, flags, total, s);
 }
@@ -662,13 +676,18 @@ int launch_bwd_fast(LogBwdArgs p, const float* stats, int* flags, int B, hipStre
 template <class T, bool GRAD_A>
 int launch_bwd_mfma(LogBwdArgs p, const float* stats, int* flags, int B, hipStream_t s) {
   const int R = GRAD_A ? p.M : p.K, Cc = GRAD_A ? p.K : p.N;
-  p.tiles_r = R / T::TR;
-  p.tiles_c = Cc / T::TC;
+  const int Q = GRAD_A ? p.N : p.M;
+  p.tiles_r = ceil_div(R, T::TR);
+  p.tiles_c = ceil_div(Cc, T::TC);
   const int total = B * p.tiles_r * p.tiles_c;
   const LogPrepared ws = prepared_of(stats, B, p.M, p.K, p.N);
-  hipLaunchKernelGGL((k_log_bwd_mfma<T, GRAD_A>), dim3(total), dim3(T::NT), 0, s, p.g, ws.ea, ws.eb,
-                     ws.r, ws.hdr, flags_of(stats, B, p.M, p.K, p.N, 0), p.grad, flags, p.M, p.K,
-                     p.N, p.tiles_r, p.tiles_c);
+  auto go = [&](auto kern) {
+    hipLaunchKernelGGL(kern, dim3(total), dim3(T::NT), 0, s, p.g, ws.ea, ws.eb, ws.r, ws.hdr,
+                       flags_of(stats, B, p.M, p.K, p.N, 0), p.grad, flags, p.M, p.K, p.N,
+                       p.tiles_r, p.tiles_c);
+  };
+  if (R % T::TR != 0 || Cc % T::TC != 0 || Q % kMS != 0) go(k_log_bwd_mfma<T, GRAD_A, true>);
+  else go(k_log_bwd_mfma<T, GRAD_A, false>);
   if (int e = launch_status()) return e;
   hipLaunchKernelGGL((k_log_bwd_fixup<BCfgWide, T::TR, T::TC, GRAD_A>),
                      dim3(min(total, kFixupGrid)), dim3(BCfgWide::NT), 0, s, p, flags, total);
@@ -679,17 +698,22 @@ int launch_bwd_mfma(LogBwdArgs p, const float* stats, int* flags, int B, hipStre
 template <class TA, class TB>
 int launch_bwd_mfma_both(LogBwdArgs pa, LogBwdArgs pb, const float* stats, int B, hipStream_t s) {
   const int M = pa.M, K = pa.K, N = pa.N;
-  pa.tiles_r = M / TA::TR; pa.tiles_c = K / TA::TC;
-  pb.tiles_r = K / TB::TR; pb.tiles_c = N / TB::TC;
+  pa.tiles_r = ceil_div(M, TA::TR); pa.tiles_c = ceil_div(K, TA::TC);
+  pb.tiles_r = ceil_div(K, TB::TR); pb.tiles_c = ceil_div(N, TB::TC);
   const int64_t ta = (int64_t)B * pa.tiles_r * pa.tiles_c, tb = (int64_t)B * pb.tiles_r * pb.tiles_c;
   if (ta + tb > 0x7fffffffLL) return GENBMM_E_SHAPE;
   const LogPrepared ws = prepared_of(stats, B, M, K, N);
   int* fa = flags_of(stats, B, M, K, N, 1);
   int* fb = flags_of(stats, B, M, K, N, 2);
-  hipLaunchKernelGGL((k_log_bwd_mfma_both<TA, TB>), dim3((unsigned)(ta + tb)), dim3(TA::NT), 0, s,
-                     pa.g, ws.ea, ws.eb, ws.r, ws.hdr, flags_of(stats, B, M, K, N, 0), pa.grad,
-                     pb.grad, fa, fb, M, K, N, (int)ta, pa.tiles_r, pa.tiles_c, pb.tiles_r,
-                     pb.tiles_c);
+  auto go = [&](auto kern) {
+    hipLaunchKernelGGL(kern, dim3((unsigned)(ta + tb)), dim3(TA::NT), 0, s, pa.g, ws.ea, ws.eb, ws.r,
+                       ws.hdr, flags_of(stats, B, M, K, N, 0), pa.grad, pb.grad, fa, fb, M, K, N,
+                       (int)ta, pa.tiles_r, pa.tiles_c, pb.tiles_r, pb.tiles_c);
+  };
+  const bool ragged = M % TA::TR != 0 || K % TA::TC != 0 || N % kMS != 0 || K % TB::TR != 0 ||
+                      N % TB::TC != 0 || M % kMS != 0;
+  if (ragged) go(k_log_bwd_mfma_both<TA, TB, true>);
+  else go(k_log_bwd_mfma_both<TA, TB, false>);
   if (int e = launch_status()) return e;
   hipLaunchKernelGGL((k_log_bwd_fixup_both<BCfgWide, TA::TR, TA::TC, TB::TR, TB::TC>),
                      dim3((unsigned)std::min<int64_t>(ta + tb, kFixupGrid)), dim3(BCfgWide::NT), 0,
@@ -697,16 +721,18 @@ int launch_bwd_mfma_both(LogBwdArgs pa, LogBwdArgs pb, const float* stats, int B
   return launch_status();
 }
 
-// All tiles full and every access 16-byte aligned: the matrix-core kernels apply.
-// Returns 2 for the 256-wide tile (enough tiles to give every compute unit two
-// workgroups of eight waves), 1 for 128x128, 0 for neither.  `long_cols`: the
-// 256 side is the column side of the output.
+// Which matrix-core tiling an output of out_r x out_c (reduction over red) gets:
+// 2 for the 256-wide tile (when the long side splits into 256s without extra
+// padding and there are tiles enough to give every compute unit two workgroups of
+// eight waves), 1 for 128x128, 0 for none.  `long_cols`: the 256 side is the
+// column side of the output.
 inline int mfma_kind(int B, int out_r, int out_c, int red, bool aligned, bool long_cols) {
-  if (g_path.load() != 0 || !aligned || red <= 0 || red % kMS != 0) return 0;
-  if (out_r % 128 != 0 || out_c % 128 != 0) return 0;
-  const int64_t t128 = (int64_t)B * (out_r / 128) * (out_c / 128);
-  if ((long_cols ? out_c : out_r) % 256 == 0 && t128 >= 1024 && t128 / 2 <= 0x7fffffff) return 2;
-  return t128 >= 128 && t128 <= 0x7fffffff ? 1 : 0;
+  if (g_path.load() != 0 || !aligned || !mfma_extents(out_r, out_c, red)) return 0;
+  const int64_t t128 = tiles128(B, out_r, out_c);
+  if (t128 > 0x7fffffff) return 0;
+  const int L = long_cols ? out_c : out_r;
+  if (ceil_div(L, 256) * 2 == ceil_div(L, 128) && t128 >= 1024) return 2;
+  return t128 >= 128 ? 1 : 0;
 }
 
 using MT128 = MTile<128, 128>;

@@ -100,6 +100,8 @@ struct StageT {
   static_assert(PER >= 1 && OUT * 4 % NT == 0, "");
   static __device__ __forceinline__ int line(int tid, int l) { return (tid >> 2) + l * (NT / 4); }
   static __device__ __forceinline__ int quad(int tid) { return tid & 3; }
+  // first reduction step (within the slab) of piece l; a piece spans four of them
+  static __device__ __forceinline__ int redpos(int tid, int) { return (tid & 3) * 4; }
   static __device__ __forceinline__ void put(float* __restrict__ buf, int tid, int l, float4 v) {
     float* p = buf + (quad(tid) * 4) * LD + line(tid, l);
     p[0] = v.x; p[LD] = v.y; p[2 * LD] = v.z; p[3 * LD] = v.w;
@@ -113,6 +115,8 @@ struct StageS {
   static_assert(PER >= 1 && kMS * Q % NT == 0 && NT % Q == 0, "");
   static __device__ __forceinline__ int red(int tid, int l) { return tid / Q + l * (NT / Q); }
   static __device__ __forceinline__ int quad(int tid) { return tid % Q; }
+  // the reduction step (within the slab) of piece l
+  static __device__ __forceinline__ int redpos(int tid, int l) { return red(tid, l); }
   static __device__ __forceinline__ void put(float* __restrict__ buf, int tid, int l, float4 v) {
     *reinterpret_cast<float4*>(buf + red(tid, l) * LD + quad(tid) * 4) = v;
   }
@@ -182,7 +186,14 @@ __device__ __forceinline__ void acc_rows(const floatx16 (&acc)[2][2], float* __r
 
 // ----------------------------------------------------------------- forward
 // rows <- EA from a[m][k] (transposed stage), columns <- EB from b[k][n].
-template <class T>
+//
+// RAGGED: M, N need not be multiples of the tile nor K of the slab (all three are
+// multiples of 4, so a float4 is inside or outside as a whole).  Lines of a tile
+// beyond the matrix re-read the last line and get the shift +inf, i.e. exp -> 0,
+// at no cost in the loop; the reduction tail is filled with -inf (exp -> 0) by a
+// loader used for the last slab only; results and by-products are stored under
+// masks.  Full-tile problems compile without any of it.
+template <class T, bool RAGGED>
 __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WPE, T::WPE)))
 void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
                     float* __restrict__ out, const float* __restrict__ stats,
@@ -208,16 +219,26 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
   // block s mod tiles_n), likewise EB, so that every workgroup stores the same.
   const int nblk = rem % tiles_n, mblk = rem / tiles_n;
 
-  const long offa = ((long)batch * M + m0 + SA::line(tid, 0)) * K + SA::quad(tid) * 4;
-  const long offb = ((long)batch * K + SB::red(tid, 0)) * N + n0 + SB::quad(tid) * 4;
-  const float* pa = a + offa;
-  const float* pb = b + offb;
-  float* qa = ws_ea + offa;
-  float* qb = ws_eb + offb;
+  // a pieces: lines m0 + line(l), four k from quad*4;  b pieces: rows red(l), four n
+  const int bcol = n0 + SB::quad(tid) * 4;
+  const bool vb = !RAGGED || bcol < N;
+  bool va[SA::PER];
+  const float* pa[SA::PER];
+  const float* pb[SB::PER];
   float al[SA::PER];
 #pragma unroll
-  for (int l = 0; l < SA::PER; ++l) al[l] = st[m0 + SA::line(tid, l)];
-  const float4 be = ld4(st + M + n0 + SB::quad(tid) * 4);
+  for (int l = 0; l < SA::PER; ++l) {
+    const int line = m0 + SA::line(tid, l);
+    va[l] = !RAGGED || line < M;
+    pa[l] = a + ((long)batch * M + (va[l] ? line : M - 1)) * K + SA::quad(tid) * 4;
+    al[l] = va[l] ? st[line] : INFINITY;
+  }
+#pragma unroll
+  for (int l = 0; l < SB::PER; ++l)
+    pb[l] = b + ((long)batch * K + SB::red(tid, l)) * N + (vb ? bcol : N - 4);
+  const float4 be = vb ? ld4(st + M + bcol) : make_float4(INFINITY, INFINITY, INFINITY, INFINITY);
+  // by-products live at the same offsets in their own arrays
+  const long da = (ws_ea - a) - kMS, db = (ws_eb - b) - (long)kMS * N;  // loads run one slab ahead
   if (tile == 0 && tid == 0) {
     ws_hdr[1] = T::TR;
     ws_hdr[2] = T::TC;
@@ -230,40 +251,56 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[x >> 1][x & 1][i] = 0.f;
 
+  const int ktail = RAGGED ? K % kMS : 0;          // reduction steps of a partial last slab
+  const int slabs = RAGGED ? (K + kMS - 1) / kMS : K / kMS;
+  const float4 ninf = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
   float4 ra[SA::PER], rb[SB::PER];
-  auto load = [&]() __attribute__((always_inline)) {
+  bool ta = true, tb[SB::PER];                     // pieces inside the reduction range
 #pragma unroll
-    for (int l = 0; l < SA::PER; ++l) ra[l] = ld4(pa + (long)l * SA::STEP * K);
+  for (int l = 0; l < SB::PER; ++l) tb[l] = true;
+  auto load = [&](bool tail) __attribute__((always_inline)) {
+    if (RAGGED && tail) {
+      ta = SA::quad(tid) * 4 < ktail;
 #pragma unroll
-    for (int l = 0; l < SB::PER; ++l) rb[l] = ld4(pb + (long)l * SB::STEP * N);
-    pa += kMS;
-    pb += (long)kMS * N;
+      for (int l = 0; l < SA::PER; ++l) ra[l] = ta ? ld4(pa[l]) : ninf;
+#pragma unroll
+      for (int l = 0; l < SB::PER; ++l) {
+        tb[l] = SB::red(tid, l) < ktail;
+        rb[l] = tb[l] ? ld4(pb[l]) : ninf;
+      }
+    } else {
+#pragma unroll
+      for (int l = 0; l < SA::PER; ++l) ra[l] = ld4(pa[l]);
+#pragma unroll
+      for (int l = 0; l < SB::PER; ++l) rb[l] = ld4(pb[l]);
+    }
+#pragma unroll
+    for (int l = 0; l < SA::PER; ++l) pa[l] += kMS;
+#pragma unroll
+    for (int l = 0; l < SB::PER; ++l) pb[l] += (long)kMS * N;
   };
   auto stage = [&](int buf, bool keep_a, bool keep_b) __attribute__((always_inline)) {
 #pragma unroll
     for (int l = 0; l < SA::PER; ++l) {
       const float4 e = exp4(ra[l], al[l]);
       SA::put(As[buf], tid, l, e);
-      if (keep_a) *reinterpret_cast<float4*>(qa + (long)l * SA::STEP * K) = e;
+      if (keep_a && (!RAGGED || (va[l] && ta))) *reinterpret_cast<float4*>(const_cast<float*>(pa[l]) + da) = e;
     }
 #pragma unroll
     for (int l = 0; l < SB::PER; ++l) {
       const float4 e = exp4(rb[l], be);
       SB::put(Bs[buf], tid, l, e);
-      if (keep_b) *reinterpret_cast<float4*>(qb + (long)l * SB::STEP * N) = e;
+      if (keep_b && (!RAGGED || (vb && tb[l]))) *reinterpret_cast<float4*>(const_cast<float*>(pb[l]) + db) = e;
     }
-    qa += kMS;
-    qb += (long)kMS * N;
   };
 
-  const int slabs = K / kMS;
-  load();
+  load(slabs == 1 && ktail != 0);
   stage(0, nblk == 0, mblk == 0);
   __syncthreads();
   int sa = 1 % tiles_n, sb = 1 % tiles_m;  // (s + 1) mod tiles_n, mod tiles_m
   for (int s = 0; s < slabs; ++s) {
     const bool more = s + 1 < slabs;
-    if (more) load();
+    if (more) load(s + 2 == slabs && ktail != 0);
     mfma_slab<LDR, LDC>(As[s & 1], Bs[s & 1], wm0, wn0, lane, acc);
     if (more) stage((s + 1) & 1, sa == nblk, sb == mblk);
     sa = sa + 1 == tiles_n ? 0 : sa + 1;
@@ -276,16 +313,25 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
   // than per cell and only sends more tiles to the exact routine).
   const float thr = fast_exp2(-kMfmaGuardBits);
   int bad = 0;
+  {
+    const int rlim = M - (m0 + wm0) - mfma_row_l(lane);   // rows of this lane below rlim exist
+    const int clim = N - (n0 + wn0) - (lane & 31);        // column blocks at offset < clim exist
 #pragma unroll
-  for (int x = 0; x < 4; ++x)
+    for (int x = 0; x < 4; ++x)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const float s = acc[x >> 1][x & 1][i];
-      if (!((s >= thr) && (s < INFINITY))) bad = 1;
-    }
+      for (int i = 0; i < 16; ++i) {
+        const float s = acc[x >> 1][x & 1][i];
+        const bool here = !RAGGED || ((x >> 1) * 32 + mfma_row_u(i) < rlim && (x & 1) * 32 < clim);
+        if (here && !((s >= thr) && (s < INFINITY))) bad = 1;
+      }
+  }
   for (int t = tid; t < T::TR + T::TC; t += NT) {
-    const float sh = t < T::TR ? st[m0 + t] : st[M + n0 + t - T::TR];
-    if (!((sh > 0.45f * kFloor) && (sh < INFINITY))) bad = 1;
+    const bool row = t < T::TR;
+    const bool here = !RAGGED || (row ? m0 + t < M : n0 + t - T::TR < N);
+    if (here) {
+      const float sh = row ? st[m0 + t] : st[M + n0 + t - T::TR];
+      if (!((sh > 0.45f * kFloor) && (sh < INFINITY))) bad = 1;
+    }
   }
   bad = __syncthreads_or(bad);  // also: every wave is done with the staging buffers
   if (tid == 0) flags[tile] = bad;
@@ -293,13 +339,16 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
 
   // out = log S + alpha + beta and R = 1/S, written row-wise
   const int lr = lane >> 4, lc = (lane & 15) * 4;
-  const float4 be4 = ld4(st + M + n0 + wn0 + lc);
+  const bool cok = !RAGGED || n0 + wn0 + lc < N;
+  const float4 be4 = cok ? ld4(st + M + n0 + wn0 + lc) : make_float4(0.f, 0.f, 0.f, 0.f);
   const float* alw = st + m0 + wm0 + lr;
   const long ubase = ((long)batch * M + m0 + wm0) * N + n0 + wn0;
   const int voff = lr * N + lc;
+  const int rows_left = M - (m0 + wm0) - lr;
   acc_rows(acc, smem + wave * kStripFloats, lane, [](int) {},
            [&](int q, int t, float4 sv) __attribute__((always_inline)) {
              const int ru = 16 * q + 4 * t;
+             if (RAGGED && !(cok && ru < rows_left)) return;
              const float alr = alw[ru];
              const long u = ubase + (long)ru * N;
              *reinterpret_cast<float4*>(ws_r + u + voff) =
@@ -322,7 +371,10 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
 // A tile that touches a cell the forward flagged (R unusable there), or runs
 // on a workspace the matrix-core forward did not fill, raises its own flag and
 // leaves the work to the fix-up launch.
-template <class T, bool GRAD_A>
+// RAGGED: lines of a tile beyond the matrix re-read the last line (they only feed
+// results that are not stored); the reduction tail is zero-filled in both
+// operands by the loader of the last slab; the epilogue is masked.
+template <class T, bool GRAD_A, bool RAGGED>
 __device__ __forceinline__ void log_bwd_mfma_tile(
     float* __restrict__ smem, int tile, const float* __restrict__ g,
     const float* __restrict__ ws_ea, const float* __restrict__ ws_eb,
@@ -341,14 +393,15 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
   const int per = tiles_r * tiles_c;
   const int batch = tile / per, rem = tile - batch * per;
   const int r0 = (rem / tiles_c) * T::TR, c0 = (rem % tiles_c) * T::TC;
-  const int Q = GRAD_A ? N : M;
+  const int Q = GRAD_A ? N : M;                      // reduction extent
+  const int R = GRAD_A ? M : K, Cc = GRAD_A ? K : N;  // output extents
 
   {  // forward flags over the cells this tile reduces over
     int bad = ws_hdr[0] != 1;
     const int ftr = max(ws_hdr[1], 1), ftc = max(ws_hdr[2], 1);
-    const int fm = M / ftr, fn = N / ftc;
-    const int mlo = GRAD_A ? r0 / ftr : 0, mhi = GRAD_A ? (r0 + T::TR - 1) / ftr : fm - 1;
-    const int nlo = GRAD_A ? 0 : c0 / ftc, nhi = GRAD_A ? fn - 1 : (c0 + T::TC - 1) / ftc;
+    const int fm = (M + ftr - 1) / ftr, fn = (N + ftc - 1) / ftc;
+    const int mlo = GRAD_A ? r0 / ftr : 0, mhi = GRAD_A ? min((r0 + T::TR - 1) / ftr, fm - 1) : fm - 1;
+    const int nlo = GRAD_A ? 0 : c0 / ftc, nhi = GRAD_A ? fn - 1 : min((c0 + T::TC - 1) / ftc, fn - 1);
     const int nn = nhi - nlo + 1, cnt = (mhi - mlo + 1) * nn;
     if (!bad)
       for (int t = tid; t < cnt; t += NT)
@@ -365,33 +418,49 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
     for (int i = 0; i < 16; ++i) acc[x >> 1][x & 1][i] = 0.f;
 
   float4 ry[SY::PER], rr[SH::PER], rg[SH::PER];
-  const float *py, *pr, *pg;
+  const float* py[SY::PER];
+  const float* pr[SH::PER];
+  long dg;  // g sits at the same offsets as R
   if constexpr (GRAD_A) {
-    py = ws_eb + ((long)batch * K + c0 + SY::line(tid, 0)) * N + SY::quad(tid) * 4;  // EB[k][n]
-    const long o = ((long)batch * M + r0 + SH::line(tid, 0)) * N + SH::quad(tid) * 4;
-    pr = ws_r + o;
-    pg = g + o;
-  } else {
-    py = ws_ea + ((long)batch * M + SY::red(tid, 0)) * K + r0 + SY::quad(tid) * 4;   // EA[m][k]
-    const long o = ((long)batch * M + SH::red(tid, 0)) * N + c0 + SH::quad(tid) * 4;
-    pr = ws_r + o;
-    pg = g + o;
-  }
-  constexpr long kYStep = SY::STEP, kHStep = SH::STEP;
-  const long ldy = GRAD_A ? N : K;
-  auto load = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int l = 0; l < SY::PER; ++l) ry[l] = ld4(py + l * kYStep * ldy);
+    for (int l = 0; l < SY::PER; ++l) {  // EB[k][n]: line k, four n from quad*4
+      const int k = c0 + SY::line(tid, l);
+      py[l] = ws_eb + ((long)batch * K + (RAGGED ? min(k, K - 1) : k)) * N + SY::quad(tid) * 4;
+    }
 #pragma unroll
     for (int l = 0; l < SH::PER; ++l) {
-      rr[l] = ld4(pr + l * kHStep * N);
-      rg[l] = ld4(pg + l * kHStep * N);
+      const int m = r0 + SH::line(tid, l);
+      pr[l] = ws_r + ((long)batch * M + (RAGGED ? min(m, M - 1) : m)) * N + SH::quad(tid) * 4;
     }
-    if constexpr (GRAD_A) {
-      py += kMS; pr += kMS; pg += kMS;
-    } else {
-      py += (long)kMS * K; pr += (long)kMS * N; pg += (long)kMS * N;
+  } else {
+    const int kc = r0 + SY::quad(tid) * 4, nc = c0 + SH::quad(tid) * 4;
+#pragma unroll
+    for (int l = 0; l < SY::PER; ++l)    // EA[m][k]: row m = red, four k
+      py[l] = ws_ea + ((long)batch * M + SY::red(tid, l)) * K + (RAGGED ? min(kc, K - 4) : kc);
+#pragma unroll
+    for (int l = 0; l < SH::PER; ++l)
+      pr[l] = ws_r + ((long)batch * M + SH::red(tid, l)) * N + (RAGGED ? min(nc, N - 4) : nc);
+  }
+  dg = g - ws_r;
+  const int qtail = RAGGED ? Q % kMS : 0;
+  const int slabs = RAGGED ? (Q + kMS - 1) / kMS : Q / kMS;
+  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  auto load = [&](bool tail) __attribute__((always_inline)) {
+#pragma unroll
+    for (int l = 0; l < SY::PER; ++l) {
+      const bool in = !(RAGGED && tail) || SY::redpos(tid, l) < qtail;
+      ry[l] = in ? ld4(py[l]) : zero4;
     }
+#pragma unroll
+    for (int l = 0; l < SH::PER; ++l) {
+      const bool in = !(RAGGED && tail) || SH::redpos(tid, l) < qtail;
+      rr[l] = in ? ld4(pr[l]) : zero4;
+      rg[l] = in ? ld4(pr[l] + dg) : zero4;
+    }
+#pragma unroll
+    for (int l = 0; l < SY::PER; ++l) py[l] += GRAD_A ? (long)kMS : (long)kMS * K;
+#pragma unroll
+    for (int l = 0; l < SH::PER; ++l) pr[l] += GRAD_A ? (long)kMS : (long)kMS * N;
   };
   auto stage = [&](int buf) __attribute__((always_inline)) {
     float* ybuf = GRAD_A ? Cs[buf] : Rs[buf];
@@ -404,13 +473,12 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
                                         rg[l].w * rr[l].w));
   };
 
-  const int slabs = Q / kMS;
-  load();
+  load(slabs == 1 && qtail != 0);
   stage(0);
   __syncthreads();
   for (int s = 0; s < slabs; ++s) {
     const bool more = s + 1 < slabs;
-    if (more) load();
+    if (more) load(s + 2 == slabs && qtail != 0);
     mfma_slab<LDR, LDC>(Rs[s & 1], Cs[s & 1], wr0, wc0, lane, acc);
     if (more) stage((s + 1) & 1);
     __syncthreads();
@@ -418,28 +486,31 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
 
   // grad = EX * acc, EX = EA or EB, row-wise; the loads of a quarter are started
   // before the previous quarter is exchanged.
-  const int Cc = GRAD_A ? K : N;
   const int lr = lane >> 4, lc = (lane & 15) * 4;
   const int voff = lr * Cc + lc;
-  const long ubase = ((long)batch * (GRAD_A ? M : K) + r0 + wr0) * Cc + c0 + wc0;
+  const long ubase = ((long)batch * R + r0 + wr0) * Cc + c0 + wc0;
   const float* xb = (GRAD_A ? ws_ea : ws_eb) + ubase + voff;
   float* gp = grad + ubase + voff;
+  const bool cok = !RAGGED || c0 + wc0 + lc < Cc;
+  const int rows_left = R - (r0 + wr0) - lr;
   float4 xq[2][4];
   auto fetch = [&](int q) __attribute__((always_inline)) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t) xq[q & 1][t] = ld4(xb + (long)(16 * q + 4 * t) * Cc);
+    for (int t = 0; t < 4; ++t)
+      if (!RAGGED || (cok && 16 * q + 4 * t < rows_left)) xq[q & 1][t] = ld4(xb + (long)(16 * q + 4 * t) * Cc);
   };
   fetch(0);
   acc_rows(acc, smem + wave * kStripFloats, lane,
            [&](int q) __attribute__((always_inline)) { if (q + 1 < 4) fetch(q + 1); },
            [&](int q, int t, float4 v) __attribute__((always_inline)) {
+             if (RAGGED && !(cok && 16 * q + 4 * t < rows_left)) return;
              const float4 x = xq[q & 1][t];
              *reinterpret_cast<float4*>(gp + (long)(16 * q + 4 * t) * Cc) =
                  make_float4(x.x * v.x, x.y * v.y, x.z * v.z, x.w * v.w);
            });
 }
 
-template <class T, bool GRAD_A>
+template <class T, bool GRAD_A, bool RAGGED>
 __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WPE, T::WPE)))
 void k_log_bwd_mfma(const float* __restrict__ g, const float* __restrict__ ws_ea,
                     const float* __restrict__ ws_eb, const float* __restrict__ ws_r,
@@ -447,15 +518,15 @@ void k_log_bwd_mfma(const float* __restrict__ g, const float* __restrict__ ws_ea
                     float* __restrict__ grad, int* __restrict__ flags, int M, int K, int N,
                     int tiles_r, int tiles_c) {
   __shared__ __attribute__((aligned(16))) float smem[2 * kMS * (T::LDR + T::LDC)];
-  log_bwd_mfma_tile<T, GRAD_A>(smem, xcd_tile_id(), g, ws_ea, ws_eb, ws_r, ws_hdr, fwd_flags, grad,
-                               flags, M, K, N, tiles_r, tiles_c);
+  log_bwd_mfma_tile<T, GRAD_A, RAGGED>(smem, xcd_tile_id(), g, ws_ea, ws_eb, ws_r, ws_hdr, fwd_flags,
+                                       grad, flags, M, K, N, tiles_r, tiles_c);
 }
 
 // Both gradients in one launch: workgroups [0, tiles_a) take the tiles of grad_a
 // (shape TA), the rest those of grad_b (shape TB).  Workgroups are dispatched in
 // index order, so the first grad_b tiles start while the last grad_a tiles are
 // still writing their results back.
-template <class TA, class TB>
+template <class TA, class TB, bool RAGGED>
 __global__ __launch_bounds__(TA::NT) __attribute__((amdgpu_waves_per_eu(TA::WPE, TA::WPE)))
 void k_log_bwd_mfma_both(const float* __restrict__ g, const float* __restrict__ ws_ea,
                          const float* __restrict__ ws_eb, const float* __restrict__ ws_r,
@@ -470,12 +541,12 @@ void k_log_bwd_mfma_both(const float* __restrict__ g, const float* __restrict__ 
   // XCD-aware numbering inside each half (needs both halves to be multiples of 8)
   const bool renum = (tiles_a & 7) == 0 && (n & 7) == 0;
   if (w < tiles_a)
-    log_bwd_mfma_tile<TA, true>(smem, renum ? xcd_renumber(w, tiles_a) : w, g, ws_ea, ws_eb, ws_r,
-                                ws_hdr, fwd_flags, grad_a, flags_a, M, K, N, ar, ac);
+    log_bwd_mfma_tile<TA, true, RAGGED>(smem, renum ? xcd_renumber(w, tiles_a) : w, g, ws_ea, ws_eb,
+                                        ws_r, ws_hdr, fwd_flags, grad_a, flags_a, M, K, N, ar, ac);
   else
-    log_bwd_mfma_tile<TB, false>(smem, renum ? xcd_renumber(w - tiles_a, n - tiles_a) : w - tiles_a,
-                                 g, ws_ea, ws_eb, ws_r, ws_hdr, fwd_flags, grad_b, flags_b, M, K, N,
-                                 br, bc);
+    log_bwd_mfma_tile<TB, false, RAGGED>(smem, renum ? xcd_renumber(w - tiles_a, n - tiles_a) : w - tiles_a,
+                                         g, ws_ea, ws_eb, ws_r, ws_hdr, fwd_flags, grad_b, flags_b, M,
+                                         K, N, br, bc);
 }
 
 }  // namespace genbmm
