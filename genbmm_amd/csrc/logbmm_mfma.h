@@ -1,14 +1,15 @@
-// Factored logbmm on the fp32 matrix cores, for problems whose tiles are all
-// full: M, N (forward) resp. the output and reduction extents (backward) are
-// multiples of 128 / 16 and every row is 16-byte aligned.  No bounds checks, no
-// index arithmetic in the loop: each lane walks fixed pointers slab by slab.
+// Factored logbmm on the fp32 matrix cores.  Every extent is a multiple of 4 and
+// every row 16-byte aligned; the loop has no bounds checks and no index
+// arithmetic - each lane walks fixed pointers slab by slab - and ragged edges are
+// dealt with outside it (see the RAGGED notes at the kernels).
 //
-// A workgroup of four waves (2x2) owns a 128x128 output tile; each wave keeps a
-// 64x64 quarter as 2x2 accumulator blocks of v_mfma_f32_32x32x2_f32 (fp32 in,
-// fp32 accumulate).  The reduction axis is consumed in slabs of 16 through two
-// LDS buffers: while the matrix cores work on slab s, the global loads of slab
-// s+1 are in flight; they are turned into exp(x - shift) and written to the
-// other buffer before the single barrier of the iteration.
+// A workgroup of (TR/64) x (TC/64) waves owns a TR x TC output tile (128x128,
+// 128x256 or 256x128); each wave keeps a 64x64 block as 2x2 accumulator blocks of
+// v_mfma_f32_32x32x2_f32 (fp32 in, fp32 accumulate).  The reduction axis is
+// consumed in slabs of 16 through two LDS buffers: while the matrix cores work on
+// slab s, the global loads of slab s+1 are in flight; they are staged (forward:
+// turned into exp(x - shift)) into the other buffer before the single barrier of
+// the iteration.
 #pragma once
 
 #include "common.h"
