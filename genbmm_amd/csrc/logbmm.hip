@@ -565,9 +565,10 @@ inline bool item_shape(int M, int K, int N) {
 }
 
 // Shapes whose forward runs on the matrix cores (given alignment and path).
-// Extents are multiples of 4 (a float4 is inside or outside the matrix as a whole),
-// large enough for 128-wide tiles to pay, and there are tiles enough for the chip;
-// ragged edges are handled by the kernels.
+// Extents are multiples of 4 (a float4 is inside or outside the matrix as a whole)
+// and large enough for 128-wide tiles to pay; ragged edges are handled by the
+// kernels.  (Measured down to a single batch item of 512^3, 16 tiles: the
+// matrix-core kernels beat the vector-ALU ones at every tile count.)
 inline bool mfma_extents(int out_r, int out_c, int red) {
   return out_r % 4 == 0 && out_c % 4 == 0 && red % 4 == 0 && out_r >= 96 && out_c >= 96 && red >= kMS;
 }
@@ -577,7 +578,7 @@ inline int64_t tiles128(int B, int out_r, int out_c) {
 inline bool fwd_mfma_shape(int B, int M, int K, int N) {
   if (!mfma_extents(M, N, K)) return false;
   const int64_t t128 = tiles128(B, M, N);
-  return t128 >= 128 && t128 <= 0x7fffffff;
+  return t128 <= 0x7fffffff;
 }
 inline LogPrepared prepared_of(const float* stats, int B, int M, int K, int N) {
   float* base = const_cast<float*>(stats) + header_offset(B, M, K, N);
@@ -724,7 +725,7 @@ int launch_bwd_mfma_both(LogBwdArgs pa, LogBwdArgs pb, const float* stats, int B
 // Which matrix-core tiling an output of out_r x out_c (reduction over red) gets:
 // 2 for the 256-wide tile (when the long side splits into 256s without extra
 // padding and there are tiles enough to give every compute unit two workgroups of
-// eight waves), 1 for 128x128, 0 for none.  `long_cols`: the 256 side is the
+// eight waves), 1 for 128x128, 0 for none (extents too small or not multiples of 4).  `long_cols`: the 256 side is the
 // column side of the output.
 inline int mfma_kind(int B, int out_r, int out_c, int red, bool aligned, bool long_cols) {
   if (g_path.load() != 0 || !aligned || !mfma_extents(out_r, out_c, red)) return 0;
@@ -732,7 +733,7 @@ inline int mfma_kind(int B, int out_r, int out_c, int red, bool aligned, bool lo
   if (t128 > 0x7fffffff) return 0;
   const int L = long_cols ? out_c : out_r;
   if (ceil_div(L, 256) * 2 == ceil_div(L, 128) && t128 >= 1024) return 2;
-  return t128 >= 128 ? 1 : 0;
+  return 1;
 }
 
 using MT128 = MTile<128, 128>;

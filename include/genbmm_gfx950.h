@@ -71,7 +71,7 @@ const char* genbmm_error_string(int code);
  * behind them sit per-tile flags naming the tiles where it is not, which a
  * fix-up launch recomputes with the online kernel's routine, and - for shapes
  * that run on the matrix cores (M, K, N multiples of 4, M and N at least 96,
- * at least 128 tiles of 128x128) - exp(a-max), exp(b-max) and 1/sum, which the backward then reads
+ * K at least 16) - exp(a-max), exp(b-max) and 1/sum, which the backward then reads
  * instead of taking any exponential itself.  The contents belong to the
  * library; the buffer takes the place of the reference's (B, M, N) `maxes`
  * output; pass the same buffer, unchanged, to genbmm_logbmm_bwd.
@@ -103,8 +103,8 @@ size_t genbmm_logbmm_stats_size(int B, int M, int K, int N);
  * Process-wide switch for tests and measurements.  1: genbmm_logbmm_fwd / _bwd
  * ignore `stats` and always run the online / exact kernels.  2: the factored
  * kernels contract with v_fma_f32 on the vector ALU instead of the fp32
- * matrix-core instruction.  0 (default): factored kernels, matrix cores for
- * 128x128 tiles.  The only piece of global state in the library.
+ * matrix-core instruction.  0 (default): factored kernels, on the matrix cores
+ * wherever the shape allows.  The only piece of global state in the library.
  * No counterpart in the reference.
  */
 void genbmm_logbmm_force_exact(int on);
