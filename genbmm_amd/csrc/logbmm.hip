@@ -565,12 +565,11 @@ inline bool item_shape(int M, int K, int N) {
 }
 
 // Shapes whose forward runs on the matrix cores (given alignment and path).
-// Extents are multiples of 4 (a float4 is inside or outside the matrix as a whole)
-// and large enough for 128-wide tiles to pay; ragged edges are handled by the
-// kernels.  (Measured down to a single batch item of 512^3, 16 tiles: the
+// Extents large enough for 128-wide tiles to pay; ragged edges, odd sizes and
+// unaligned rows are handled by the kernels.  (Measured down to a single batch item of 512^3, 16 tiles: the
 // matrix-core kernels beat the vector-ALU ones at every tile count.)
 inline bool mfma_extents(int out_r, int out_c, int red) {
-  return out_r % 4 == 0 && out_c % 4 == 0 && red % 4 == 0 && out_r >= 96 && out_c >= 96 && red >= kMS;
+  return out_r >= 96 && out_c >= 96 && red >= kMS;
 }
 inline int64_t tiles128(int B, int out_r, int out_c) {
   return (int64_t)B * ceil_div(out_r, 128) * ceil_div(out_c, 128);
@@ -748,7 +747,7 @@ int run_bwd(const LogBwdArgs& p, const float* stats, int B, hipStream_t s) {
   const bool small = R <= 32 && Cc <= 32;
   if (stats) {
     int* fl = flags_of(stats, B, p.M, p.K, p.N, GRAD_A ? 1 : 2);
-    const bool al = p.vec_k && p.vec_n && aligned16(stats) && p.M % 4 == 0 && p.N % 4 == 0;
+    const bool al = true;  // the matrix-core kernels assume 4-byte alignment only
     // the matrix-core kernels run on what the matrix-core forward left behind
     switch (fwd_mfma_shape(B, p.M, p.K, p.N) ? mfma_kind(B, R, Cc, Q, al, GRAD_A) : 0) {
       case 2:
@@ -805,7 +804,7 @@ int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats, 
   if (stats && K > 0 && g_path.load() != 1) {
     int* fl = flags_of(stats, B, M, K, N, 0);
     const int64_t big_tiles = (int64_t)B * ceil_div(M, 128) * ceil_div(N, 128);
-    const bool al = K % 4 == 0 && N % 4 == 0 && aligned16(a) && aligned16(b) && aligned16(stats);
+    const bool al = true;  // the matrix-core kernels assume 4-byte alignment only
     switch (fwd_mfma_shape(B, M, K, N) ? mfma_kind(B, M, N, K, al, true) : 0) {
       case 2: return launch_fwd_mfma<MTWide>(p, stats, fl, B, M, K, N, s);
       case 1: return launch_fwd_mfma<MT128>(p, stats, fl, B, M, K, N, s);
@@ -847,7 +846,7 @@ int genbmm_logbmm_bwd(const float* a, const float* b, const float* out, const fl
     return launch_status();
   }
   if (st && grad_a && grad_b && mk > 0 && kn > 0 && fwd_mfma_shape(B, M, K, N)) {
-    const bool al = p.vec_k && p.vec_n && aligned16(st) && M % 4 == 0 && N % 4 == 0;
+    const bool al = true;
     const int ka = mfma_kind(B, M, K, N, al, true), kb = mfma_kind(B, K, N, M, al, false);
     if (ka == kb && ka != 0) {
       LogBwdArgs pa = p, pb = p;

@@ -123,7 +123,37 @@ struct StageS {
   }
 };
 
-__device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+// Global memory is touched four floats at a time with only 4-byte alignment
+// assumed (the hardware takes misaligned dwordx4; rows of odd-sized matrices start
+// anywhere).  The masked forms touch the first cnt (<= 0: none, >= 4: all) elements.
+typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
+__device__ __forceinline__ float4 ld4(const float* p) {
+  const float4u v = *reinterpret_cast<const float4u*>(p);
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void st4(float* p, float4 v) {
+  float4u u;
+  u.x = v.x; u.y = v.y; u.z = v.z; u.w = v.w;
+  *reinterpret_cast<float4u*>(p) = u;
+}
+__device__ __forceinline__ float4 ld4m(const float* p, int cnt, float fill) {
+  if (cnt >= 4) return ld4(p);
+  float4 r = make_float4(fill, fill, fill, fill);
+  if (cnt > 0) r.x = p[0];
+  if (cnt > 1) r.y = p[1];
+  if (cnt > 2) r.z = p[2];
+  return r;
+}
+__device__ __forceinline__ void st4m(float* p, int cnt, float4 v) {
+  if (cnt >= 4) {
+    st4(p, v);
+    return;
+  }
+  if (cnt > 0) p[0] = v.x;
+  if (cnt > 1) p[1] = v.y;
+  if (cnt > 2) p[2] = v.z;
+}
+__device__ __forceinline__ int clamp4(int x) { return min(max(x, 0), 4); }
 __device__ __forceinline__ float4 exp4(float4 x, float4 s) {
   return make_float4(exp_st(x.x - s.x), exp_st(x.y - s.y), exp_st(x.z - s.z), exp_st(x.w - s.w));
 }
@@ -188,12 +218,13 @@ __device__ __forceinline__ void acc_rows(const floatx16 (&acc)[2][2], float* __r
 // ----------------------------------------------------------------- forward
 // rows <- EA from a[m][k] (transposed stage), columns <- EB from b[k][n].
 //
-// RAGGED: M, N need not be multiples of the tile nor K of the slab (all three are
-// multiples of 4, so a float4 is inside or outside as a whole).  Lines of a tile
-// beyond the matrix re-read the last line and get the shift +inf, i.e. exp -> 0,
-// at no cost in the loop; the reduction tail is filled with -inf (exp -> 0) by a
-// loader used for the last slab only; results and by-products are stored under
-// masks.  Full-tile problems compile without any of it.
+// RAGGED: M, N need not be multiples of the tile nor K of the slab - any sizes.
+// Lines of a tile beyond the matrix re-read the last line and get the shift +inf,
+// i.e. exp -> 0, at no cost in the loop; a piece of four that straddles the right
+// edge is read element by element by the few lanes that own one; the reduction
+// tail is filled with -inf (exp -> 0) by a loader used for the last slab only;
+// results and by-products are stored under masks.  Full-tile problems compile
+// without any of it.
 template <class T, bool RAGGED>
 __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WPE, T::WPE)))
 void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
@@ -222,7 +253,8 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
 
   // a pieces: lines m0 + line(l), four k from quad*4;  b pieces: rows red(l), four n
   const int bcol = n0 + SB::quad(tid) * 4;
-  const bool vb = !RAGGED || bcol < N;
+  const int cb = RAGGED ? clamp4(N - bcol) : 4;  // columns of this lane's b pieces inside the matrix
+  const bool vb = cb > 0;
   bool va[SA::PER];
   const float* pa[SA::PER];
   const float* pb[SB::PER];
@@ -236,8 +268,8 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
   }
 #pragma unroll
   for (int l = 0; l < SB::PER; ++l)
-    pb[l] = b + ((long)batch * K + SB::red(tid, l)) * N + (vb ? bcol : N - 4);
-  const float4 be = vb ? ld4(st + M + bcol) : make_float4(INFINITY, INFINITY, INFINITY, INFINITY);
+    pb[l] = b + ((long)batch * K + SB::red(tid, l)) * N + (vb ? bcol : 0);
+  const float4 be = RAGGED ? ld4m(st + M + (vb ? bcol : 0), cb, INFINITY) : ld4(st + M + bcol);
   // by-products live at the same offsets in their own arrays
   const long da = (ws_ea - a) - kMS, db = (ws_eb - b) - (long)kMS * N;  // loads run one slab ahead
   if (tile == 0 && tid == 0) {
@@ -256,24 +288,25 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
   const int slabs = RAGGED ? (K + kMS - 1) / kMS : K / kMS;
   const float4 ninf = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
   float4 ra[SA::PER], rb[SB::PER];
-  bool ta = true, tb[SB::PER];                     // pieces inside the reduction range
+  int ca = 4;                                      // reduction steps of the a pieces inside K
+  bool tb[SB::PER];                                // b pieces inside K
 #pragma unroll
   for (int l = 0; l < SB::PER; ++l) tb[l] = true;
   auto load = [&](bool tail) __attribute__((always_inline)) {
     if (RAGGED && tail) {
-      ta = SA::quad(tid) * 4 < ktail;
+      ca = clamp4(ktail - SA::quad(tid) * 4);
 #pragma unroll
-      for (int l = 0; l < SA::PER; ++l) ra[l] = ta ? ld4(pa[l]) : ninf;
+      for (int l = 0; l < SA::PER; ++l) ra[l] = ld4m(pa[l], ca, -INFINITY);
 #pragma unroll
       for (int l = 0; l < SB::PER; ++l) {
         tb[l] = SB::red(tid, l) < ktail;
-        rb[l] = tb[l] ? ld4(pb[l]) : ninf;
+        rb[l] = tb[l] ? ld4m(pb[l], cb, -INFINITY) : ninf;
       }
     } else {
 #pragma unroll
       for (int l = 0; l < SA::PER; ++l) ra[l] = ld4(pa[l]);
 #pragma unroll
-      for (int l = 0; l < SB::PER; ++l) rb[l] = ld4(pb[l]);
+      for (int l = 0; l < SB::PER; ++l) rb[l] = RAGGED ? ld4m(pb[l], cb, -INFINITY) : ld4(pb[l]);
     }
 #pragma unroll
     for (int l = 0; l < SA::PER; ++l) pa[l] += kMS;
@@ -285,13 +318,19 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
     for (int l = 0; l < SA::PER; ++l) {
       const float4 e = exp4(ra[l], al[l]);
       SA::put(As[buf], tid, l, e);
-      if (keep_a && (!RAGGED || (va[l] && ta))) *reinterpret_cast<float4*>(const_cast<float*>(pa[l]) + da) = e;
+      if (keep_a) {
+        if (!RAGGED) st4(const_cast<float*>(pa[l]) + da, e);
+        else if (va[l]) st4m(const_cast<float*>(pa[l]) + da, ca, e);
+      }
     }
 #pragma unroll
     for (int l = 0; l < SB::PER; ++l) {
       const float4 e = exp4(rb[l], be);
       SB::put(Bs[buf], tid, l, e);
-      if (keep_b && (!RAGGED || (vb && tb[l]))) *reinterpret_cast<float4*>(const_cast<float*>(pb[l]) + db) = e;
+      if (keep_b) {
+        if (!RAGGED) st4(const_cast<float*>(pb[l]) + db, e);
+        else if (tb[l]) st4m(const_cast<float*>(pb[l]) + db, cb, e);
+      }
     }
   };
 
@@ -340,8 +379,9 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
 
   // out = log S + alpha + beta and R = 1/S, written row-wise
   const int lr = lane >> 4, lc = (lane & 15) * 4;
-  const bool cok = !RAGGED || n0 + wn0 + lc < N;
-  const float4 be4 = cok ? ld4(st + M + n0 + wn0 + lc) : make_float4(0.f, 0.f, 0.f, 0.f);
+  const int cc = RAGGED ? clamp4(N - (n0 + wn0 + lc)) : 4;  // columns of this lane's pieces that exist
+  const bool cok = cc > 0;
+  const float4 be4 = RAGGED ? ld4m(st + M + (cok ? n0 + wn0 + lc : 0), cc, 0.f) : ld4(st + M + n0 + wn0 + lc);
   const float* alw = st + m0 + wm0 + lr;
   const long ubase = ((long)batch * M + m0 + wm0) * N + n0 + wn0;
   const int voff = lr * N + lc;
@@ -352,14 +392,19 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
              if (RAGGED && !(cok && ru < rows_left)) return;
              const float alr = alw[ru];
              const long u = ubase + (long)ru * N;
-             *reinterpret_cast<float4*>(ws_r + u + voff) =
-                 make_float4(__builtin_amdgcn_rcpf(sv.x), __builtin_amdgcn_rcpf(sv.y),
-                             __builtin_amdgcn_rcpf(sv.z), __builtin_amdgcn_rcpf(sv.w));
-             *reinterpret_cast<float4*>(out + u + voff) =
-                 make_float4(__builtin_fmaf(fast_log2(sv.x), kLn2, alr + be4.x),
-                             __builtin_fmaf(fast_log2(sv.y), kLn2, alr + be4.y),
-                             __builtin_fmaf(fast_log2(sv.z), kLn2, alr + be4.z),
-                             __builtin_fmaf(fast_log2(sv.w), kLn2, alr + be4.w));
+             const float4 rv = make_float4(__builtin_amdgcn_rcpf(sv.x), __builtin_amdgcn_rcpf(sv.y),
+                                           __builtin_amdgcn_rcpf(sv.z), __builtin_amdgcn_rcpf(sv.w));
+             const float4 ov = make_float4(__builtin_fmaf(fast_log2(sv.x), kLn2, alr + be4.x),
+                                           __builtin_fmaf(fast_log2(sv.y), kLn2, alr + be4.y),
+                                           __builtin_fmaf(fast_log2(sv.z), kLn2, alr + be4.z),
+                                           __builtin_fmaf(fast_log2(sv.w), kLn2, alr + be4.w));
+             if (RAGGED) {
+               st4m(ws_r + u + voff, cc, rv);
+               st4m(out + u + voff, cc, ov);
+             } else {
+               st4(ws_r + u + voff, rv);
+               st4(out + u + voff, ov);
+             }
            });
 }
 
@@ -372,9 +417,10 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
 // A tile that touches a cell the forward flagged (R unusable there), or runs
 // on a workspace the matrix-core forward did not fill, raises its own flag and
 // leaves the work to the fix-up launch.
-// RAGGED: lines of a tile beyond the matrix re-read the last line (they only feed
-// results that are not stored); the reduction tail is zero-filled in both
-// operands by the loader of the last slab; the epilogue is masked.
+// RAGGED (any sizes): lines of a tile beyond the matrix re-read the last line (they
+// only feed results that are not stored); pieces straddling the right edge are
+// read element by element; the reduction tail is zero-filled in both operands by
+// the loader of the last slab; the epilogue is masked.
 template <class T, bool GRAD_A, bool RAGGED>
 __device__ __forceinline__ void log_bwd_mfma_tile(
     float* __restrict__ smem, int tile, const float* __restrict__ g,
@@ -422,6 +468,9 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
   const float* py[SY::PER];
   const float* pr[SH::PER];
   long dg;  // g sits at the same offsets as R
+  // elements of this lane's pieces inside the matrix: grad_b pieces run along the
+  // output axis (fixed per lane), grad_a pieces along the reduction (last slab only)
+  int cy = 4, ch = 4;
   if constexpr (GRAD_A) {
 #pragma unroll
     for (int l = 0; l < SY::PER; ++l) {  // EB[k][n]: line k, four n from quad*4
@@ -435,28 +484,42 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
     }
   } else {
     const int kc = r0 + SY::quad(tid) * 4, nc = c0 + SH::quad(tid) * 4;
+    cy = RAGGED ? clamp4(K - kc) : 4;
+    ch = RAGGED ? clamp4(N - nc) : 4;
 #pragma unroll
     for (int l = 0; l < SY::PER; ++l)    // EA[m][k]: row m = red, four k
-      py[l] = ws_ea + ((long)batch * M + SY::red(tid, l)) * K + (RAGGED ? min(kc, K - 4) : kc);
+      py[l] = ws_ea + ((long)batch * M + SY::red(tid, l)) * K + (cy > 0 ? kc : 0);
 #pragma unroll
     for (int l = 0; l < SH::PER; ++l)
-      pr[l] = ws_r + ((long)batch * M + SH::red(tid, l)) * N + (RAGGED ? min(nc, N - 4) : nc);
+      pr[l] = ws_r + ((long)batch * M + SH::red(tid, l)) * N + (ch > 0 ? nc : 0);
   }
   dg = g - ws_r;
   const int qtail = RAGGED ? Q % kMS : 0;
   const int slabs = RAGGED ? (Q + kMS - 1) / kMS : Q / kMS;
   const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
   auto load = [&](bool tail) __attribute__((always_inline)) {
+    if (!RAGGED) {
 #pragma unroll
-    for (int l = 0; l < SY::PER; ++l) {
-      const bool in = !(RAGGED && tail) || SY::redpos(tid, l) < qtail;
-      ry[l] = in ? ld4(py[l]) : zero4;
-    }
+      for (int l = 0; l < SY::PER; ++l) ry[l] = ld4(py[l]);
 #pragma unroll
-    for (int l = 0; l < SH::PER; ++l) {
-      const bool in = !(RAGGED && tail) || SH::redpos(tid, l) < qtail;
-      rr[l] = in ? ld4(pr[l]) : zero4;
-      rg[l] = in ? ld4(pr[l] + dg) : zero4;
+      for (int l = 0; l < SH::PER; ++l) {
+        rr[l] = ld4(pr[l]);
+        rg[l] = ld4(pr[l] + dg);
+      }
+    } else {
+      // grad_a: a piece covers reduction steps redpos .. redpos+3; grad_b: one step
+#pragma unroll
+      for (int l = 0; l < SY::PER; ++l) {
+        const int left = tail ? qtail - SY::redpos(tid, l) : 4;
+        ry[l] = ld4m(py[l], GRAD_A ? left : (left > 0 ? cy : 0), 0.f);
+      }
+#pragma unroll
+      for (int l = 0; l < SH::PER; ++l) {
+        const int left = tail ? qtail - SH::redpos(tid, l) : 4;
+        const int cnt = GRAD_A ? left : (left > 0 ? ch : 0);
+        rr[l] = ld4m(pr[l], cnt, 0.f);
+        rg[l] = ld4m(pr[l] + dg, cnt, 0.f);
+      }
     }
 #pragma unroll
     for (int l = 0; l < SY::PER; ++l) py[l] += GRAD_A ? (long)kMS : (long)kMS * K;
@@ -492,13 +555,16 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
   const long ubase = ((long)batch * R + r0 + wr0) * Cc + c0 + wc0;
   const float* xb = (GRAD_A ? ws_ea : ws_eb) + ubase + voff;
   float* gp = grad + ubase + voff;
-  const bool cok = !RAGGED || c0 + wc0 + lc < Cc;
+  const int cc = RAGGED ? clamp4(Cc - (c0 + wc0 + lc)) : 4;  // columns of this lane's pieces that exist
+  const bool cok = cc > 0;
   const int rows_left = R - (r0 + wr0) - lr;
   float4 xq[2][4];
   auto fetch = [&](int q) __attribute__((always_inline)) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
-      if (!RAGGED || (cok && 16 * q + 4 * t < rows_left)) xq[q & 1][t] = ld4(xb + (long)(16 * q + 4 * t) * Cc);
+    for (int t = 0; t < 4; ++t) {
+      if (!RAGGED) xq[q & 1][t] = ld4(xb + (long)(16 * q + 4 * t) * Cc);
+      else if (cok && 16 * q + 4 * t < rows_left) xq[q & 1][t] = ld4m(xb + (long)(16 * q + 4 * t) * Cc, cc, 0.f);
+    }
   };
   fetch(0);
   acc_rows(acc, smem + wave * kStripFloats, lane,
@@ -506,8 +572,9 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
            [&](int q, int t, float4 v) __attribute__((always_inline)) {
              if (RAGGED && !(cok && 16 * q + 4 * t < rows_left)) return;
              const float4 x = xq[q & 1][t];
-             *reinterpret_cast<float4*>(gp + (long)(16 * q + 4 * t) * Cc) =
-                 make_float4(x.x * v.x, x.y * v.y, x.z * v.z, x.w * v.w);
+             const float4 r = make_float4(x.x * v.x, x.y * v.y, x.z * v.z, x.w * v.w);
+             if (RAGGED) st4m(gp + (long)(16 * q + 4 * t) * Cc, cc, r);
+             else st4(gp + (long)(16 * q + 4 * t) * Cc, r);
            });
 }
 

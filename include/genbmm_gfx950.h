@@ -70,8 +70,7 @@ const char* genbmm_error_string(int code);
  * to factor exp(a+b) = exp(a-max)*exp(b-max) wherever that is exact to fp32;
  * behind them sit per-tile flags naming the tiles where it is not, which a
  * fix-up launch recomputes with the online kernel's routine, and - for shapes
- * that run on the matrix cores (M, K, N multiples of 4, M and N at least 96,
- * K at least 16) - exp(a-max), exp(b-max) and 1/sum, which the backward then reads
+ * that run on the matrix cores (M and N at least 96, K at least 16) - exp(a-max), exp(b-max) and 1/sum, which the backward then reads
  * instead of taking any exponential itself.  The contents belong to the
  * library; the buffer takes the place of the reference's (B, M, N) `maxes`
  * output; pass the same buffer, unchanged, to genbmm_logbmm_bwd.

@@ -155,10 +155,12 @@ def test_logbmm_factoring_guard(gpu, B, M, K, N):
 
 
 @pytest.mark.parametrize("B,M,K,N", [(32, 256, 128, 256), (64, 512, 128, 512), (64, 200, 100, 260),
-                                     (64, 500, 132, 500), (128, 260, 388, 132)])
+                                     (64, 500, 132, 500), (128, 260, 388, 132), (24, 201, 103, 259),
+                                     (3, 130, 97, 391), (64, 257, 255, 129)])
 def test_logbmm_factoring_guard_matrix_core_tiles(gpu, B, M, K, N):
     """Shapes that run on the matrix-core kernels (128x128 and 128x256 / 256x128 tiles),
-    the last three with ragged edges in every dimension (partial tiles, partial slabs).
+    all but the first two with ragged edges in every dimension (partial tiles, partial slabs),
+    the last three with odd sizes (rows not 16-byte aligned, pieces straddling the edge).
     Some batch items need the exact fall-back in every tile, one in a single row, the
     rest in none: flagged and unflagged tiles side by side, and the backward kernels
     must honour the forward's flags (they read 1/S from the forward's workspace)."""
