@@ -1,7 +1,6 @@
-// Factored logbmm on the fp32 matrix cores.  Every extent is a multiple of 4 and
-// every row 16-byte aligned; the loop has no bounds checks and no index
-// arithmetic - each lane walks fixed pointers slab by slab - and ragged edges are
-// dealt with outside it (see the RAGGED notes at the kernels).
+// Factored logbmm on the fp32 matrix cores, for any sizes.  The loop has no bounds
+// checks and no index arithmetic - each lane walks fixed pointers slab by slab -
+// and ragged edges are dealt with outside it (see the RAGGED notes at the kernels).
 //
 // A workgroup of (TR/64) x (TC/64) waves owns a TR x TC output tile (128x128,
 // 128x256 or 256x128); each wave keeps a 64x64 block as 2x2 accumulator blocks of
