@@ -731,7 +731,7 @@ inline int mfma_kind(int B, int out_r, int out_c, int red, bool aligned, bool lo
   const int64_t t128 = tiles128(B, out_r, out_c);
   if (t128 > 0x7fffffff) return 0;
   const int L = long_cols ? out_c : out_r;
-  if (ceil_div(L, 256) * 2 == ceil_div(L, 128) && t128 >= 1024) return 2;
+  if (ceil_div(L, 256) * 2 == ceil_div(L, 128) && t128 >= 512) return 2;
   return 1;
 }
 
