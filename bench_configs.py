@@ -156,13 +156,14 @@ def banded(lib, dev, B, n, lu, ld, mode, reps):
     out = torch.empty(B, n, Wo, device=dev)
     idx = torch.empty(B, n, Wo, dtype=torch.int32, device=dev) if mode == 1 else None
     ga, gb = torch.empty_like(a), torch.empty_like(b)
+    ws = torch.empty(lib.genbmm_banded_workspace_size(lu, ld, lu, ld, B, n), device=dev) if mode == 0 else None
     s, p = _lib.stream_of(a), _lib.ptr
 
     def f():
-        _lib.check(lib.genbmm_banded_fwd(p(a), lu, ld, p(b), lu, ld, p(out), p(idx), B, n, mode, s), "fwd")
+        _lib.check(lib.genbmm_banded_fwd(p(a), lu, ld, p(b), lu, ld, p(out), p(idx), p(ws), B, n, mode, s), "fwd")
 
     def bw():
-        _lib.check(lib.genbmm_banded_bwd(p(a), lu, ld, p(b), lu, ld, p(out), p(idx), p(g), p(ga), p(gb), B, n, mode, s),
+        _lib.check(lib.genbmm_banded_bwd(p(a), lu, ld, p(b), lu, ld, p(out), p(idx), p(ws), p(g), p(ga), p(gb), B, n, mode, s),
                    "bwd")
 
     mf, mb = timed(f, reps), timed(bw, reps)

@@ -37,13 +37,14 @@ SIGNATURES = {
     "genbmm_samplebmm_fwd": [_c_float_p] * 3 + [_c_int_p, _c_float_p, _u64, _u64] + _DENSE_DIMS,
     "genbmm_argmax_bwd": [_c_int_p] + [_c_float_p] * 3 + _DENSE_DIMS,
     "genbmm_prodmax_bwd": [_c_float_p] * 2 + [_c_int_p] + [_c_float_p] * 3 + _DENSE_DIMS,
-    "genbmm_banded_fwd": _BAND + [_c_float_p, _c_int_p, _i, _i, _i, _vp],
-    "genbmm_banded_bwd": _BAND + [_c_float_p, _c_int_p] + [_c_float_p] * 3 + [_i, _i, _i, _vp],
+    "genbmm_banded_fwd": _BAND + [_c_float_p, _c_int_p, _c_float_p, _i, _i, _i, _vp],
+    "genbmm_banded_bwd": _BAND + [_c_float_p, _c_int_p] + [_c_float_p] * 4 + [_i, _i, _i, _vp],
     "genbmm_banded_bwdbwd": _BAND + [_c_float_p] * 7 + [_i, _i, _vp],
 }
 STRING_FUNCS = {"genbmm_version": [], "genbmm_error_string": [_i]}
 VOID_FUNCS = {"genbmm_logbmm_force_exact": [_i]}
-SIZE_FUNCS = {"genbmm_logbmm_stats_size": [_i, _i, _i, _i]}
+SIZE_FUNCS = {"genbmm_logbmm_stats_size": [_i, _i, _i, _i],
+              "genbmm_banded_workspace_size": [_i, _i, _i, _i, _i, _i]}
 
 _lib = None
 

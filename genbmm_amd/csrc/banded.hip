@@ -147,6 +147,44 @@ int fill_band(BandArgs& p, int a_lu, int a_ld, int b_lu, int b_ld, int B, int n)
 
 constexpr size_t kStripLdsLimit = 64 * 1024;  // dynamic LDS available without opting in
 
+// Workspace of the log product: EA (B*n*Wa), EB (B*n*Wb), alpha (B*n), beta (B*n),
+// R (B*n*Wo) floats.
+inline size_t band_ws_floats(const BandArgs& p, int B) {
+  return (size_t)B * p.n * ((size_t)p.Wa + p.Wb + p.Wo + 2);
+}
+// Which bands the strip kernels take (forward / backward): tiles within 64 KB of
+// LDS, the sliding tile large enough to double as the output staging tiles.
+inline bool fwd_strip_ok(const BandArgs& p) {
+  const StripDims sd = strip_dims(p.Wa, p.Wb);
+  const bool tiles_fit = (size_t)kBR * sd.ld_sl >= (size_t)2 * kBT * kBC;
+  return tiles_fit && sd.ld_own <= 256 && sd.ld_sl <= 256 && sd.bytes <= kStripLdsLimit;
+}
+inline bool bwd_strip_ok(const BandArgs& p) {
+  if (p.Wa > 8 * 4 * kMaxKB || p.Wb > 8 * 4 * kMaxKB) return false;
+  const StripDims da = strip_dims(p.Wa, p.Wb), db = strip_dims(p.Wb, p.Wa);
+  return max(bwd_strip_bytes(da, true), bwd_strip_bytes(db, true)) <= kStripLdsLimit &&
+         max(max(da.ld_own, da.ld_sl), max(db.ld_own, db.ld_sl)) <= 128;
+}
+// The workspace is filled and used only when both directions run strip kernels, so
+// that forward and backward always agree on whether it holds anything.
+inline bool workspace_used(const BandArgs& p) {
+  return fwd_strip_ok(p) && bwd_strip_ok(p) &&
+         strip_dims(p.Wa, p.Wb).bytes + sizeof(float) * (kBT + p.Wo + kBJ) <= kStripLdsLimit;
+}
+
+inline bool prep_fwd(const BandArgs& p, int mode, const float* workspace) {
+  return mode == GENBMM_BAND_LOG && workspace != nullptr && workspace_used(p);
+}
+
+inline void set_workspace(BandArgs& p, float* ws, int B) {
+  const size_t rows = (size_t)B * p.n;
+  p.ws_ea = ws;
+  p.ws_eb = p.ws_ea + rows * p.Wa;
+  p.ws_al = p.ws_eb + rows * p.Wb;
+  p.ws_be = p.ws_al + rows;
+  p.ws_r = p.ws_be + rows;
+}
+
 inline dim3 blocks_for(long total) { return dim3((unsigned)((total + 255) / 256)); }
 
 }  // namespace
@@ -154,8 +192,16 @@ inline dim3 blocks_for(long total) { return dim3((unsigned)((total + 255) / 256)
 
 extern "C" {
 
+size_t genbmm_banded_workspace_size(int a_lu, int a_ld, int b_lu, int b_ld, int B, int n) {
+  using namespace genbmm;
+  BandArgs p{};
+  if (fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return 0;
+  return band_ws_floats(p, B);
+}
+
 int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
-                      float* out, int32_t* idx, int B, int n, int mode, void* stream) {
+                      float* out, int32_t* idx, float* workspace, int B, int n, int mode,
+                      void* stream) {
   using namespace genbmm;
   if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
     return GENBMM_E_MODE;
@@ -168,18 +214,30 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   if (total == 0) return GENBMM_OK;
   hipStream_t s = (hipStream_t)stream;
   const StripDims sd = strip_dims(p.Wa, p.Wb);
-  // the sliding tile doubles as the output staging tile(s): [64][33] values (+ indices)
-  const bool tiles_fit = (size_t)kBR * sd.ld_sl >= (size_t)2 * kBT * kBC;
-  if (tiles_fit && sd.ld_own <= 256 && sd.ld_sl <= 256 && sd.bytes <= kStripLdsLimit) {
+  if (fwd_strip_ok(p)) {
     const int strips = ceil_div(n, kBT);
     const dim3 grid((unsigned)((long)B * strips));
     const int nq = ceil_div(max(sd.ld_own, sd.ld_sl), 64);
+    // the prepared log product also stages beta for every row its outputs can meet
+    const size_t lds = sd.bytes + (prep_fwd(p, mode, workspace) ? sizeof(float) * (kBT + p.Wo + kBJ) : 0);
     auto go = [&](auto kern) {
-      hipLaunchKernelGGL(kern, grid, dim3(256), sd.bytes, s, p, strips, sd.ld_own, sd.ld_sl);
+      hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, p, strips, sd.ld_own, sd.ld_sl);
     };
+    const bool prep = prep_fwd(p, mode, workspace);
+    if (prep) {  // EA, alpha and EB, beta once, instead of per strip and chunk
+      set_workspace(p, workspace, B);
+      const long rows = (long)B * n;
+      const dim3 pg((unsigned)((rows + kPrepRows - 1) / kPrepRows));
+      const int lda = odd(p.Wa), ldb = odd(p.Wb);
+      hipLaunchKernelGGL(k_band_prep, pg, dim3(256), sizeof(float) * kPrepRows * lda, s, a, p.ws_ea,
+                         p.ws_al, p.Wa, a_lu, n, rows, lda);
+      hipLaunchKernelGGL(k_band_prep, pg, dim3(256), sizeof(float) * kPrepRows * ldb, s, b, p.ws_eb,
+                         p.ws_be, p.Wb, b_lu, n, rows, ldb);
+    }
     auto pick = [&](auto nqc) {
       constexpr int Q = decltype(nqc)::value;
-      if (mode == GENBMM_BAND_LOG) go(k_band_fwd_strip<kSemLog, Q>);
+      if (prep) go(k_band_fwd_strip<kSemLogPrep, Q>);
+      else if (mode == GENBMM_BAND_LOG) go(k_band_fwd_strip<kSemLog, Q>);
       else if (mode == GENBMM_BAND_MAX) go(k_band_fwd_strip<kSemMax, Q>);
       else go(k_band_fwd_strip<kSemMul, Q>);
     };
@@ -198,8 +256,8 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
 }
 
 int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
-                      const float* out, const int32_t* idx, const float* g, float* grad_a,
-                      float* grad_b, int B, int n, int mode, void* stream) {
+                      const float* out, const int32_t* idx, const float* workspace, const float* g,
+                      float* grad_a, float* grad_b, int B, int n, int mode, void* stream) {
   using namespace genbmm;
   if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
     return GENBMM_E_MODE;
@@ -213,14 +271,25 @@ int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   const long ta = (long)B * n * p.Wa, tb = (long)B * n * p.Wb;
   if (ta == 0) return GENBMM_OK;
   hipStream_t s = (hipStream_t)stream;
-  if (mode != GENBMM_BAND_MAX && p.Wa <= 8 * 4 * kMaxKB && p.Wb <= 8 * 4 * kMaxKB) {
+  if (mode != GENBMM_BAND_MAX && bwd_strip_ok(p)) {
     const bool lg = mode == GENBMM_BAND_LOG;
     const StripDims da = strip_dims(p.Wa, p.Wb), db = strip_dims(p.Wb, p.Wa);
     const size_t na = bwd_strip_bytes(da, lg), nb = bwd_strip_bytes(db, lg);
-    if (max(na, nb) <= kStripLdsLimit && max(max(da.ld_own, da.ld_sl), max(db.ld_own, db.ld_sl)) <= 128) {
+    {
       const int strips = ceil_div(n, kBT);
       const dim3 grid((unsigned)((long)B * strips));
       const int nq = ceil_div(max(max(da.ld_own, da.ld_sl), max(db.ld_own, db.ld_sl)), 64);
+      if (lg && workspace && workspace_used(p)) {  // on the forward's workspace: a (+,x) backward plus epilogue
+        set_workspace(p, const_cast<float*>(workspace), B);
+        if (nq <= 1) {
+          hipLaunchKernelGGL((k_band_bwd_strip<false, true, 1, true>), grid, dim3(256), na, s, p, strips, da.ld_own, da.ld_sl, bwd_sl_floats(da));
+          hipLaunchKernelGGL((k_band_bwd_strip<false, false, 1, true>), grid, dim3(256), nb, s, p, strips, db.ld_own, db.ld_sl, bwd_sl_floats(db));
+        } else {
+          hipLaunchKernelGGL((k_band_bwd_strip<false, true, 2, true>), grid, dim3(256), na, s, p, strips, da.ld_own, da.ld_sl, bwd_sl_floats(da));
+          hipLaunchKernelGGL((k_band_bwd_strip<false, false, 2, true>), grid, dim3(256), nb, s, p, strips, db.ld_own, db.ld_sl, bwd_sl_floats(db));
+        }
+        return launch_status();
+      }
       if (nq <= 1) {
         if (lg) {
           hipLaunchKernelGGL((k_band_bwd_strip<true, true, 1>), grid, dim3(256), na, s, p, strips, da.ld_own, da.ld_sl, bwd_sl_floats(da));

@@ -20,6 +20,14 @@ struct BandArgs {
   float* o1;      // -          | grad_b
   float* o2;      // -          | grad_g
   int32_t* oidx;  // forward argmax
+  // log product with a workspace: EA = exp(a - alpha), EB = exp(b - beta) with the
+  // row maxima alpha, beta (over cells inside the matrix), and R = 1/S per output
+  // cell (-1: the cell was computed exactly, S is not usable)
+  float* ws_ea;
+  float* ws_eb;
+  float* ws_al;
+  float* ws_be;
+  float* ws_r;
   int n, a_lu, Wa, b_lu, Wb, r_lu, Wo;
 };
 

@@ -61,6 +61,7 @@ __device__ __forceinline__ float wave_max(float v) {
 // loads into registers, store() consumes them - a whole chunk is in flight while
 // the previous one is being multiplied.
 constexpr int kSemMul = 0, kSemLog = 1, kSemMax = 2;  // what a staged tile is used for
+constexpr int kSemLogPrep = 3;  // log product on operands prepared by k_band_prep (forward kernel only)
 
 template <int SEM, int NQ, int ROWS>
 struct RowStage {
@@ -130,6 +131,55 @@ struct RowStage {
   }
 };
 
+// ------------------------------------------------------------ prepared operands
+// One wave per band row: shift = maximum over the cells inside the matrix (-inf if
+// there is none), e = exp(x - shift), 0 for cells outside.  With these the log
+// product is a (+,x) product of e's plus an epilogue, and no kernel downstream
+// takes an exponential per staged element again.
+constexpr int kPrepRows = 64;  // band rows per workgroup: one contiguous block of memory
+
+__global__ __launch_bounds__(256) void k_band_prep(const float* __restrict__ x, float* __restrict__ e,
+                                                   float* __restrict__ shift, int W, int lu, int n,
+                                                   long rows, int ld) {
+  extern __shared__ __attribute__((aligned(16))) float tile[];  // [64][ld], ld odd
+  const int tid = threadIdx.x;
+  const long row0 = (long)blockIdx.x * kPrepRows;
+  const int nr = (int)min((long)kPrepRows, rows - row0);
+  const float* xb = x + row0 * W;
+  float* eb = e + row0 * W;
+  // the block is contiguous in memory: coalesced in, row per lane inside, coalesced out
+  for (int i = tid, r = tid / W, k = tid - (tid / W) * W; i < nr * W; i += 256) {
+    tile[r * ld + k] = xb[i];
+    r += 256 / W;
+    k += 256 % W;
+    if (k >= W) {
+      k -= W;
+      ++r;
+    }
+  }
+  __syncthreads();
+  if (tid < nr) {
+    const int c = (int)((row0 + tid) % n);
+    const int klo = max(0, lu - c), khi = min(W - 1, n - 1 + lu - c);  // cells inside the matrix
+    float* tr = tile + tid * ld;
+    float m = -INFINITY;
+    for (int k = klo; k <= khi; ++k) m = fmaxf(m, tr[k]);
+    shift[row0 + tid] = m;
+    const float sh = m == -INFINITY ? 0.f : m;
+    for (int k = 0; k < W; ++k) tr[k] = (k >= klo && k <= khi) ? fast_exp2((tr[k] - sh) * kLog2e) : 0.f;
+  }
+  __syncthreads();
+  for (int i = tid, r = tid / W, k = tid - (tid / W) * W; i < nr * W; i += 256) {
+    eb[i] = tile[r * ld + k];
+    r += 256 / W;
+    k += 256 % W;
+    if (k >= W) {
+      k -= W;
+      ++r;
+    }
+  }
+}
+
 // ------------------------------------------------------------------ forward
 // Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each): renumber so
 // that an XCD works on consecutive strips, whose halos overlap.
@@ -138,10 +188,18 @@ __device__ __forceinline__ int xcd_strip_id() {
   return (n & 7) == 0 ? (w & 7) * (n >> 3) + (w >> 3) : w;
 }
 
+// The exact recompute of one cell, kept out of line: it is rare, and inlined it costs
+// the strip kernels registers they do not have.
+__device__ __attribute__((noinline)) float band_fwd_cell_log_exact(const BandArgs& p, long bi, int i, int j) {
+  band_fwd_cell<GENBMM_BAND_LOG>(p, bi, i, j);
+  return p.o0[bi * p.Wo + j];
+}
+
 template <int SEM, int NQ>
-__global__ __launch_bounds__(256, SEM == kSemMul ? 3 : 2) void k_band_fwd_strip(const BandArgs p, int strips,
+__global__ __launch_bounds__(256, (SEM == kSemMul || SEM == kSemLogPrep) ? 3 : 2) void k_band_fwd_strip(const BandArgs p, int strips,
                                                                           int ld_own, int ld_sl) {
-  constexpr bool LOG = SEM == kSemLog, MAXP = SEM == kSemMax;
+  constexpr bool LOG = SEM == kSemLog, MAXP = SEM == kSemMax, PREP = SEM == kSemLogPrep;
+  constexpr int SS = PREP ? kSemMul : SEM;  // how the tiles are staged
   extern __shared__ __attribute__((aligned(16))) float smem[];
   float* As = smem;                 // [64][ld_own]
   float* Bs = As + kBT * ld_own;    // [95][ld_sl]; reused as the [64][33] output staging tile
@@ -149,23 +207,33 @@ __global__ __launch_bounds__(256, SEM == kSemMul ? 3 : 2) void k_band_fwd_strip(
   float* be = al + kBT;             // [95]
   float* Cs = Bs;
   int* Is = reinterpret_cast<int*>(Bs + kBT * kBC);  // max product: the argmax tile behind it
+  float* Rt = Bs + kBT * kBC;                        // prepared log product: the 1/S tile
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wg = xcd_strip_id();
   const int batch = wg / strips, i0 = (wg - batch * strips) * kBT;
   const int n = p.n, Wa = p.Wa, Wb = p.Wb, Wo = p.Wo;
-  const float* ab = p.a + (long)batch * n * Wa;
-  const float* bb = p.b + (long)batch * n * Wb;
+  const float* ab = (PREP ? p.ws_ea : p.a) + (long)batch * n * Wa;
+  const float* bb = (PREP ? p.ws_eb : p.b) + (long)batch * n * Wb;
   float* ob = p.o0 + (long)batch * n * Wo;
   int32_t* ib = MAXP ? p.oidx + (long)batch * n * Wo : nullptr;
+  float* rb = PREP ? p.ws_r + (long)batch * n * Wo : nullptr;
   const long bn = (long)batch * n;
   const float thr = fast_exp2(-kBandGuardBits);
 
   {
-    RowStage<SEM, NQ, kBT> sa;
+    RowStage<SS, NQ, kBT> sa;
     sa.load(ab, Wa, p.a_lu, n, i0, ld_own, 0, wave, lane);
     sa.store(As, ld_own, al, wave, lane);
   }
-  RowStage<SEM, NQ, kBR> sb;
+  float* bw = be + kBR;  // prepared log product: beta[i0 - lu_out + t], t < 64 + Wo (+ chunk round-up)
+  if (PREP) {
+    if (tid < kBT) al[tid] = i0 + tid < n ? p.ws_al[bn + i0 + tid] : 0.f;
+    for (int t = tid; t < kBT + Wo + kBJ; t += 256) {
+      const int o = i0 - p.r_lu + t;
+      bw[t] = (o >= 0 && o < n) ? p.ws_be[bn + o] : 0.f;
+    }
+  }
+  RowStage<SS, NQ, kBR> sb;
   sb.load(bb, Wb, p.b_lu, n, i0 - p.r_lu, ld_sl, kBP, wave, lane);
 
   for (int jc = 0; jc < Wo; jc += kBJ) {
@@ -226,23 +294,30 @@ __global__ __launch_bounds__(256, SEM == kSemMul ? 3 : 2) void k_band_fwd_strip(
 #pragma unroll
       for (int t = 0; t < 8; ++t) sh[t] = al[lane] + be[min(lane + 8 * wave + t, kBR - 1)];
     }
+    if (PREP) {  // alpha[i] + beta[o], o = i + j - lu_out, staged once per strip
+#pragma unroll
+      for (int t = 0; t < 8; ++t) sh[t] = al[lane] + bw[lane + j0 + t];
+    }
     __syncthreads();  // every wave is done with Bs: it becomes the output tile
     const int i = i0 + lane;
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
       float v = acc[t];
-      if (LOG) {
+      if (LOG || PREP) {
         const int j = j0 + t, o = i + j - p.r_lu;
+        float rv = 0.f;
         if (i < n && j < Wo && o >= 0 && o < n) {
           if ((v >= thr) && (v < INFINITY) && (sh[t] > 0.9f * kFloor) && (sh[t] < INFINITY)) {
+            rv = __builtin_amdgcn_rcpf(v);
             v = __builtin_fmaf(fast_log2(v), kLn2, sh[t]);
           } else {  // factoring not exact for this cell: recompute it from memory
-            band_fwd_cell<GENBMM_BAND_LOG>(p, bn + i, i, j);
-            v = ob[(long)i * Wo + j];
+            v = band_fwd_cell_log_exact(p, bn + i, i, j);
+            rv = -1.f;  // tells the backward that 1/S is not usable here
           }
         } else {
           v = 0.f;  // outside the matrix: the reference's zero fill
         }
+        if (PREP) Rt[lane * kBC + 8 * wave + t] = rv;
       }
       if (MAXP) {
         const int o = i + j0 + t - p.r_lu;
@@ -259,6 +334,7 @@ __global__ __launch_bounds__(256, SEM == kSemMul ? 3 : 2) void k_band_fwd_strip(
       if (i0 + r < n && jc + c < Wo) {
         ob[(long)(i0 + r) * Wo + jc + c] = Cs[r * kBC + c];
         if (MAXP) ib[(long)(i0 + r) * Wo + jc + c] = Is[r * kBC + c];
+        if (PREP) rb[(long)(i0 + r) * Wo + jc + c] = Rt[r * kBC + c];
       }
     }
   }
@@ -277,37 +353,68 @@ __global__ __launch_bounds__(256, SEM == kSemMul ? 3 : 2) void k_band_fwd_strip(
 // of the tile, store() turns them into g' = g (or H = g * exp(alpha + beta - out))
 // in LDS.  A cell
 // counts if it lies inside the matrix and, for grad_b, if its b row is in the strip.
-template <bool LOG, bool GRAD_A>
+template <bool LOG, bool GRAD_A, bool PREP = false>
 struct GStage {
   static constexpr int ROWS = GRAD_A ? kBT : kBR;
   static constexpr int PER = (ROWS * kBJ + 255) / 256;
   float gv[PER], ov[PER];
   unsigned used;
 
+  // [U0, U1): the pieces handled by this call (all of them, or a few at a time where
+  // registers are short)
+  template <int U0 = 0, int U1 = PER>
   __device__ __forceinline__ void load(const float* __restrict__ gb, const float* __restrict__ ob,
                                        int x0, int yb, int jc, int n, int Wo, int r_lu, int tid) {
-    used = 0;
+    if (U0 == 0) used = 0;
 #pragma unroll
-    for (int u = 0; u < PER; ++u) {
+    for (int u = U0; u < (U1 < PER ? U1 : PER); ++u) {
       const int e = tid + 256 * u, r = e >> 5, c = e & 31, j = jc + c;
       const int i = GRAD_A ? x0 + r : yb + r;  // row of g / out (a's row index)
       const int o = i + j - r_lu;              // b's row index of this cell
       const bool inside = r < ROWS && i >= 0 && i < n && j < Wo && o >= 0 && o < n;
       const bool use = inside && (GRAD_A || (o >= x0 && o < x0 + kBT));
       gv[u] = use ? gb[(long)i * Wo + j] : 0.f;
-      ov[u] = (LOG && use) ? ob[(long)i * Wo + j] : 0.f;
+      ov[u] = ((LOG || PREP) && use) ? ob[(long)i * Wo + j] : 0.f;  // out, or 1/S of the workspace
       used |= (use ? 1u : 0u) << u;
     }
   }
 
+  // gv holds 1/S (or -1: not usable, the row this cell feeds is redone) of the cells
+  // whose g' the same thread has just stored: g' *= 1/S
+  __device__ __forceinline__ void scale(float* __restrict__ gt, int* __restrict__ badrow, int x0,
+                                        int yb, int jc, int r_lu, int tid) const {
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int e = tid + 256 * u, r = e >> 5, c = e & 31;
+      if (r >= ROWS || !((used >> u) & 1u)) continue;
+      if (gv[u] < 0.f) {
+        const int o = (GRAD_A ? x0 + r : yb + r) + jc + c - r_lu;
+        badrow[GRAD_A ? r : o - x0] = 1;
+        gt[r * kBC + c] = 0.f;
+      } else {
+        gt[r * kBC + c] *= gv[u];
+      }
+    }
+  }
+
+  template <int U0 = 0, int U1 = PER>
   __device__ __forceinline__ void store(float* __restrict__ gt, const float* __restrict__ sh_own,
                                         const float* __restrict__ sh_sl, int* __restrict__ badrow,
                                         int x0, int yb, int jc, int r_lu, float lim, int tid) const {
 #pragma unroll
-    for (int u = 0; u < PER; ++u) {
+    for (int u = U0; u < (U1 < PER ? U1 : PER); ++u) {
       const int e = tid + 256 * u, r = e >> 5, c = e & 31;
       if (r >= ROWS) continue;
       float v = gv[u];
+      if (PREP && ((used >> u) & 1u)) {
+        const int o = (GRAD_A ? x0 + r : yb + r) + jc + c - r_lu;
+        if (ov[u] < 0.f) {  // the cell was computed exactly: 1/S not usable, the row is redone
+          badrow[GRAD_A ? r : o - x0] = 1;
+          v = 0.f;
+        } else {
+          v *= ov[u];
+        }
+      }
       if (LOG && ((used >> u) & 1u)) {
         const int o = (GRAD_A ? x0 + r : yb + r) + jc + c - r_lu;
         // alpha[i] + beta[o] - out[i,j]
@@ -324,9 +431,13 @@ struct GStage {
 
 constexpr int kMaxKB = 3;  // band-axis blocks of 8 per wave: widths up to 96
 
-template <bool LOG, bool GRAD_A, int NQ>
-__global__ __launch_bounds__(256, 3) void k_band_bwd_strip(const BandArgs p, int strips, int ld_own,
+// PREP (with LOG = false): the log product on the forward's workspace - operands
+// EA / EB staged like a (+,x) product, g' = g * R, result times the own operand's
+// EA / EB; rows fed by a cell whose R is marked unusable are recomputed exactly.
+template <bool LOG, bool GRAD_A, int NQ, bool PREP = false>
+__global__ __launch_bounds__(256, (PREP && !GRAD_A) ? 2 : 3) void k_band_bwd_strip(const BandArgs p, int strips, int ld_own,
                                                            int ld_sl, int sl_floats) {
+  static_assert(!(LOG && PREP), "");
   extern __shared__ __attribute__((aligned(16))) float smem[];
   // sl : 95 rows of the other operand, padded (LOG: exp(y - shift)); reused as the
   //      [64][ld_own] result tile at the end
@@ -344,10 +455,10 @@ __global__ __launch_bounds__(256, 3) void k_band_bwd_strip(const BandArgs p, int
   const int batch = wg / strips, x0 = (wg - batch * strips) * kBT;
   const int n = p.n, Wa = p.Wa, Wb = p.Wb, Wo = p.Wo;
   const long bn = (long)batch * n;
-  const float* ab = p.a + bn * Wa;
-  const float* bb = p.b + bn * Wb;
+  const float* ab = (PREP ? p.ws_ea : p.a) + bn * Wa;
+  const float* bb = (PREP ? p.ws_eb : p.b) + bn * Wb;
   const float* gb = p.g + bn * Wo;
-  const float* ob = LOG ? p.out + bn * Wo : nullptr;
+  const float* ob = LOG ? p.out + bn * Wo : (PREP ? p.ws_r + bn * Wo : nullptr);
   // output operand / other operand
   const float* xo = GRAD_A ? ab : bb;
   const float* yo = GRAD_A ? bb : ab;
@@ -382,7 +493,14 @@ __global__ __launch_bounds__(256, 3) void k_band_bwd_strip(const BandArgs p, int
     // ---- g' tile.  (Starting these reads one chunk ahead, like the operand rows,
     // measured slower: the extra live registers cost more than the latency.)
     // The log kernels are short of registers: they go element by element.
-    if (LOG) {
+    if (PREP) {
+      // two passes over the same cells (g, then 1/S) keep half as many values live
+      GStage<false, GRAD_A> gs;
+      gs.load(gb, nullptr, x0, yb, jc, n, Wo, p.r_lu, tid);
+      gs.store(gt, sh_own, sh_sl, badrow, x0, yb, jc, p.r_lu, lim, tid);
+      gs.load(ob, nullptr, x0, yb, jc, n, Wo, p.r_lu, tid);
+      gs.scale(gt, badrow, x0, yb, jc, p.r_lu, tid);
+    } else if (LOG) {
       for (int e = tid; e < GStage<LOG, GRAD_A>::ROWS * kBJ; e += 256) {
         const int r = e >> 5, c = e & 31, j = jc + c;
         const int i = GRAD_A ? x0 + r : yb + r;
@@ -460,7 +578,7 @@ __global__ __launch_bounds__(256, 3) void k_band_bwd_strip(const BandArgs p, int
   for (int r = wave; r < kBT; r += 4) {
     const int x = x0 + r;
     if (x >= n) break;
-    if (LOG && badrow[r]) {  // recompute this row cell by cell from memory
+    if ((LOG || PREP) && badrow[r]) {  // recompute this row cell by cell from memory
       for (int k = lane; k < Wx; k += 64) {
         if (GRAD_A) band_bwd_a_cell<GENBMM_BAND_LOG>(p, bn + x, x, k);
         else band_bwd_b_cell<GENBMM_BAND_LOG>(p, bn + x, x, k);
@@ -474,6 +592,8 @@ __global__ __launch_bounds__(256, 3) void k_band_bwd_strip(const BandArgs p, int
           const float acv = ct[r * ld_own + k];
           gradb[(long)x * Wx + k] = acv == 0.f ? 0.f : fast_exp2((xo[(long)x * Wx + k] - sh) * kLog2e) * acv;
         }
+      } else if (PREP) {
+        for (int k = lane; k < Wx; k += 64) gradb[(long)x * Wx + k] = xo[(long)x * Wx + k] * ct[r * ld_own + k];
       } else {
         for (int k = lane; k < Wx; k += 64) gradb[(long)x * Wx + k] = ct[r * ld_own + k];
       }

@@ -189,20 +189,26 @@ def _forward(a, a_lu, a_ld, b, b_lu, b_ld, mode):
     wo = a.shape[2] + b.shape[2] - 1
     out = torch.empty(B, n, wo, dtype=torch.float32, device=a.device)
     idx = torch.empty(B, n, wo, dtype=torch.int32, device=a.device) if mode == MODE_MAX else None
+    # log product: the library's workspace (exp(a - max), exp(b - max), maxima, 1/sum),
+    # which stands where the reference's `maxes` stands
+    ws = None
+    if mode == MODE_LOG:
+        size = _lib.load().genbmm_banded_workspace_size(a_lu, a_ld, b_lu, b_ld, B, n)
+        ws = torch.empty(size, dtype=torch.float32, device=a.device)
     _call("genbmm_banded_fwd", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
-          _lib.ptr(out), _lib.ptr(idx), B, n, mode)
-    return a, b, out, idx
+          _lib.ptr(out), _lib.ptr(idx), _lib.ptr(ws), B, n, mode)
+    return a, b, out, (ws if mode == MODE_LOG else idx)
 
 
-def _backward(a, b, bands, out, idx, g, mode):
+def _backward(a, b, bands, out, idx, g, mode, ws=None):
     a_lu, a_ld, b_lu, b_ld = bands
     B, n = a.shape[0], a.shape[1]
     g = g.to(torch.float32).contiguous()
     grad_a = torch.empty_like(a)
     grad_b = torch.empty_like(b)
     _call("genbmm_banded_bwd", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
-          _lib.ptr(out), _lib.ptr(idx), _lib.ptr(g), _lib.ptr(grad_a), _lib.ptr(grad_b),
-          B, n, mode)
+          _lib.ptr(out), _lib.ptr(idx), _lib.ptr(ws), _lib.ptr(g), _lib.ptr(grad_a),
+          _lib.ptr(grad_b), B, n, mode)
     return grad_a, grad_b
 
 
@@ -233,8 +239,8 @@ class _BandedLogGrad(torch.autograd.Function):
     maxes transposed in band form for the second operand."""
 
     @staticmethod
-    def forward(ctx, a, b, g, out, bands):
-        grad_a, grad_b = _backward(a, b, bands, out, None, g, MODE_LOG)
+    def forward(ctx, a, b, g, out, ws, bands):
+        grad_a, grad_b = _backward(a, b, bands, out, None, g, MODE_LOG, ws)
         ctx.save_for_backward(a, b, g, out)
         ctx.bands = bands
         ctx.set_materialize_grads(False)
@@ -243,7 +249,7 @@ class _BandedLogGrad(torch.autograd.Function):
     @staticmethod
     def backward(ctx, u_a, u_b):
         if u_a is None and u_b is None:
-            return (None,) * 5
+            return (None,) * 6
         a, b, g, out = ctx.saved_tensors
         a_lu, a_ld, b_lu, b_ld = ctx.bands
         u_a = None if u_a is None else u_a.contiguous()
@@ -252,7 +258,7 @@ class _BandedLogGrad(torch.autograd.Function):
         _call("genbmm_banded_bwdbwd", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
               _lib.ptr(out), _lib.ptr(g), _lib.ptr(u_a), _lib.ptr(u_b),
               _lib.ptr(ga), _lib.ptr(gb), _lib.ptr(gg), a.shape[0], a.shape[1])
-        return ga, gb, gg, None, None
+        return ga, gb, gg, None, None, None
 
 
 class BandedLogMul(torch.autograd.Function):
@@ -260,16 +266,16 @@ class BandedLogMul(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, a, a_lu, a_ld, b, b_lu, b_ld, o_lu, o_ld):
-        a, b, out, _ = _forward(a, a_lu, a_ld, b, b_lu, b_ld, MODE_LOG)
-        ctx.save_for_backward(a, b, out)
+        a, b, out, ws = _forward(a, a_lu, a_ld, b, b_lu, b_ld, MODE_LOG)
+        ctx.save_for_backward(a, b, out, ws)
         ctx.bands = (a_lu, a_ld, b_lu, b_ld)
         return out
 
     @staticmethod
     def backward(ctx, grad_output):
-        a, b, out = ctx.saved_tensors
+        a, b, out, ws = ctx.saved_tensors
         g = grad_output.to(torch.float32).contiguous()
-        grad_a, grad_b = _BandedLogGrad.apply(a, b, g, out, ctx.bands)
+        grad_a, grad_b = _BandedLogGrad.apply(a, b, g, out, ws, ctx.bands)
         return (grad_a, None, None, grad_b) + (None,) * 4
 
 

@@ -193,18 +193,29 @@ int genbmm_prodmax_bwd(const float* a, const float* b, const int32_t* idx,
  * receives the arg-max k (index into a's band; -1e9 floor, strict '>');
  * GENBMM_BAND_MUL: ordinary (+,*).  Cells with o outside [0,n) are written
  * as 0 (idx 0).  idx may be NULL unless mode is GENBMM_BAND_MAX.
+ * `workspace`: NULL, or (used in mode LOG only) a buffer of
+ * genbmm_banded_workspace_size floats.  With it the forward takes every
+ * exponential once - exp(a - rowmax), exp(b - rowmax) in a pass of its own,
+ * kept together with the maxima and 1/sum per output cell - and
+ * genbmm_banded_bwd, handed the same buffer, takes none.  It stands where the
+ * reference's `maxes` output stands.
  * Replaces _genbmm.forward_band: matmul_cuda.cpp:112-124,
  * banded_cuda_kernel.cu:354-402, kernel :13-100.
  */
 int genbmm_banded_fwd(const float* a, int a_lu, int a_ld,
                       const float* b, int b_lu, int b_ld,
-                      float* out, int32_t* idx,
+                      float* out, int32_t* idx, float* workspace,
                       int B, int n, int mode, void* stream);
+
+/* Number of fp32 elements of the log product's workspace (0 on bad arguments). */
+size_t genbmm_banded_workspace_size(int a_lu, int a_ld, int b_lu, int b_ld,
+                                    int B, int n);
 
 /*
  * Gradients of genbmm_banded_fwd with respect to BOTH operands, reading g,
  * out and idx in the frame the forward wrote them (no banded transposes).
- * `out` is read in mode LOG only, `idx` in mode MAX only (others may be NULL).
+ * `out` is read in mode LOG only, `idx` in mode MAX only (others may be NULL);
+ * `workspace`: NULL or, in mode LOG, the buffer the forward filled.
  * grad_a terms are added in ascending j (result band index), grad_b terms in
  * ascending i (row of a), which is the order of the reference's two calls.
  * Replaces the two _genbmm.backward_band calls and the Python-side banded
@@ -214,7 +225,8 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld,
  */
 int genbmm_banded_bwd(const float* a, int a_lu, int a_ld,
                       const float* b, int b_lu, int b_ld,
-                      const float* out, const int32_t* idx, const float* g,
+                      const float* out, const int32_t* idx,
+                      const float* workspace, const float* g,
                       float* grad_a, float* grad_b,
                       int B, int n, int mode, void* stream);
 

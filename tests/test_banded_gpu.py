@@ -92,7 +92,7 @@ def test_banded_max_index_through_c_abi(gpu):
     out = torch.empty(3, n, W, device=gpu)
     idx = torch.empty(3, n, W, dtype=torch.int32, device=gpu)
     rc = _lib.load().genbmm_banded_fwd(_lib.ptr(ad), a_lu, a_ld, _lib.ptr(bd), b_lu, b_ld, _lib.ptr(out),
-                                       _lib.ptr(idx), 3, n, 1, _lib.stream_of(ad))
+                                       _lib.ptr(idx), _lib.ptr(None), 3, n, 1, _lib.stream_of(ad))
     assert rc == 0
     want, widx, _ = oracle.seq_band_fwd(a, a_lu, a_ld, b, b_lu, b_ld, 1)
     assert torch.equal(out.cpu(), want) and torch.equal(idx.cpu(), widx)

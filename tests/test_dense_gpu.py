@@ -439,8 +439,8 @@ def test_errors(gpu):
     ad = a.to(gpu)
     assert lib.genbmm_logbmm_fwd(null, _lib.ptr(ad), _lib.ptr(ad), null, 1, 1, 1, 1, null) == -1
     assert lib.genbmm_logbmm_fwd(_lib.ptr(ad), _lib.ptr(ad), _lib.ptr(ad), null, 1, -1, 1, 1, null) == -2
-    assert lib.genbmm_banded_fwd(_lib.ptr(ad), 0, 0, _lib.ptr(ad), 0, 0, _lib.ptr(ad), null, 1, 1, 2, null) == -3
-    assert lib.genbmm_banded_fwd(_lib.ptr(ad), -1, 0, _lib.ptr(ad), 0, 0, _lib.ptr(ad), null, 1, 1, 0, null) == -4
+    assert lib.genbmm_banded_fwd(_lib.ptr(ad), 0, 0, _lib.ptr(ad), 0, 0, _lib.ptr(ad), null, null, 1, 1, 2, null) == -3
+    assert lib.genbmm_banded_fwd(_lib.ptr(ad), -1, 0, _lib.ptr(ad), 0, 0, _lib.ptr(ad), null, null, 1, 1, 0, null) == -4
     assert b"NULL" in lib.genbmm_error_string(-1)
 
 
@@ -518,12 +518,13 @@ def test_maxbmm_and_banded_in_a_graph(gpu):
     W = lu + ld + 1
     xa, xb = torch.randn(B, n, W, device=gpu), torch.randn(B, n, W, device=gpu)
     bo = torch.empty(B, n, 2 * W - 1, device=gpu)
+    bws = torch.empty(lib.genbmm_banded_workspace_size(lu, ld, lu, ld, B, n), device=gpu)
     p = _lib.ptr
 
     def enqueue(stream):
         s = ctypes.c_void_p(stream.cuda_stream)
         assert lib.genbmm_maxbmm_fwd(p(a), p(b), p(out), p(idx), B, M, K, N, s) == 0
-        assert lib.genbmm_banded_fwd(p(xa), lu, ld, p(xb), lu, ld, p(bo), p(None), B, n, 0, s) == 0
+        assert lib.genbmm_banded_fwd(p(xa), lu, ld, p(xb), lu, ld, p(bo), p(None), p(bws), B, n, 0, s) == 0
 
     enqueue(torch.cuda.current_stream())
     torch.cuda.synchronize()
