@@ -213,3 +213,26 @@ def test_banded_products_match_reference_cpu_vectors(gpu, case):
             assert torch.equal(got.data.cpu(), want), name
         else:
             assert torch.allclose(got.data.cpu(), want, rtol=1e-5, atol=1e-5), name
+
+
+@pytest.mark.parametrize("n,a_lu,a_ld,b_lu,b_ld", BANDS)
+def test_banded_log_without_workspace(gpu, n, a_lu, a_ld, b_lu, b_ld):
+    """The log product through the C ABI with workspace = NULL (every exponential taken
+    in the strip kernels) against the float64 oracle; the Python layer always passes a
+    workspace, so this is the only caller of that path."""
+    lib = _lib.load()
+    torch.manual_seed(n + a_lu)
+    a, b = pair(n, a_lu, a_ld, b_lu, b_ld)
+    W = a.shape[2] + b.shape[2] - 1
+    g = torch.randn(3, n, W)
+    ad, bd, gd = a.to(gpu), b.to(gpu), g.to(gpu)
+    out, ga, gb = torch.empty(3, n, W, device=gpu), torch.empty_like(ad), torch.empty_like(bd)
+    p, s, null = _lib.ptr, _lib.stream_of(ad), _lib.ptr(None)
+    assert lib.genbmm_banded_fwd(p(ad), a_lu, a_ld, p(bd), b_lu, b_ld, p(out), null, null, 3, n, 0, s) == 0
+    assert lib.genbmm_banded_bwd(p(ad), a_lu, a_ld, p(bd), b_lu, b_ld, p(out), null, null, p(gd), p(ga), p(gb),
+                                 3, n, 0, s) == 0
+    want, _, _ = oracle.seq_band_fwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, 0, dtype=np.float64)
+    wa, wb = oracle.seq_band_bwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, g.double(), 0, dtype=np.float64)
+    close(out, want)
+    close(ga, wa)
+    close(gb, wb)
