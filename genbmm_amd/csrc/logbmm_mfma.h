@@ -153,6 +153,16 @@ __device__ __forceinline__ void st4m(float* p, int cnt, float4 v) {
   if (cnt > 2) p[2] = v.z;
 }
 __device__ __forceinline__ int clamp4(int x) { return min(max(x, 0), 4); }
+
+// Two arrays of the same shape are walked with one pointer plus the byte distance
+// between them (integer arithmetic on addresses, not pointer arithmetic across
+// objects).
+__device__ __forceinline__ long byte_distance(const void* to, const void* from) {
+  return (long)(reinterpret_cast<uintptr_t>(to) - reinterpret_cast<uintptr_t>(from));
+}
+__device__ __forceinline__ float* shifted(const float* p, long bytes) {
+  return reinterpret_cast<float*>(reinterpret_cast<uintptr_t>(p) + (uintptr_t)bytes);
+}
 __device__ __forceinline__ float4 exp4(float4 x, float4 s) {
   return make_float4(exp_st(x.x - s.x), exp_st(x.y - s.y), exp_st(x.z - s.z), exp_st(x.w - s.w));
 }
@@ -270,7 +280,8 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
     pb[l] = b + ((long)batch * K + SB::red(tid, l)) * N + (vb ? bcol : 0);
   const float4 be = RAGGED ? ld4m(st + M + (vb ? bcol : 0), cb, INFINITY) : ld4(st + M + bcol);
   // by-products live at the same offsets in their own arrays
-  const long da = (ws_ea - a) - kMS, db = (ws_eb - b) - (long)kMS * N;  // loads run one slab ahead
+  // (the source pointers run one slab ahead of what is being staged)
+  const long da = byte_distance(ws_ea, a) - 4l * kMS, db = byte_distance(ws_eb, b) - 4l * kMS * N;
   if (tile == 0 && tid == 0) {
     ws_hdr[1] = T::TR;
     ws_hdr[2] = T::TC;
@@ -318,8 +329,8 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
       const float4 e = exp4(ra[l], al[l]);
       SA::put(As[buf], tid, l, e);
       if (keep_a) {
-        if (!RAGGED) st4(const_cast<float*>(pa[l]) + da, e);
-        else if (va[l]) st4m(const_cast<float*>(pa[l]) + da, ca, e);
+        if (!RAGGED) st4(shifted(pa[l], da), e);
+        else if (va[l]) st4m(shifted(pa[l], da), ca, e);
       }
     }
 #pragma unroll
@@ -327,8 +338,8 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
       const float4 e = exp4(rb[l], be);
       SB::put(Bs[buf], tid, l, e);
       if (keep_b) {
-        if (!RAGGED) st4(const_cast<float*>(pb[l]) + db, e);
-        else if (tb[l]) st4m(const_cast<float*>(pb[l]) + db, cb, e);
+        if (!RAGGED) st4(shifted(pb[l], db), e);
+        else if (tb[l]) st4m(shifted(pb[l], db), cb, e);
       }
     }
   };
@@ -466,7 +477,7 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
   float4 ry[SY::PER], rr[SH::PER], rg[SH::PER];
   const float* py[SY::PER];
   const float* pr[SH::PER];
-  long dg;  // g sits at the same offsets as R
+  long dg;  // g sits at the same offsets as R: byte distance between the arrays
   // elements of this lane's pieces inside the matrix: grad_b pieces run along the
   // output axis (fixed per lane), grad_a pieces along the reduction (last slab only)
   int cy = 4, ch = 4;
@@ -492,7 +503,7 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
     for (int l = 0; l < SH::PER; ++l)
       pr[l] = ws_r + ((long)batch * M + SH::red(tid, l)) * N + (ch > 0 ? nc : 0);
   }
-  dg = g - ws_r;
+  dg = byte_distance(g, ws_r);
   const int qtail = RAGGED ? Q % kMS : 0;
   const int slabs = RAGGED ? (Q + kMS - 1) / kMS : Q / kMS;
   const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -503,7 +514,7 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
 #pragma unroll
       for (int l = 0; l < SH::PER; ++l) {
         rr[l] = ld4(pr[l]);
-        rg[l] = ld4(pr[l] + dg);
+        rg[l] = ld4(shifted(pr[l], dg));
       }
     } else {
       // grad_a: a piece covers reduction steps redpos .. redpos+3; grad_b: one step
@@ -517,7 +528,7 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
         const int left = tail ? qtail - SH::redpos(tid, l) : 4;
         const int cnt = GRAD_A ? left : (left > 0 ? ch : 0);
         rr[l] = ld4m(pr[l], cnt, 0.f);
-        rg[l] = ld4m(pr[l] + dg, cnt, 0.f);
+        rg[l] = ld4m(shifted(pr[l], dg), cnt, 0.f);
       }
     }
 #pragma unroll
