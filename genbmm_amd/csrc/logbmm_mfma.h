@@ -70,6 +70,7 @@ __device__ __forceinline__ void mfma_slab(const float* __restrict__ R, const flo
   const float* cp = Cs + lk * LDC + wc0 + lrow;
   // operands of step q+2 are read while the four products of step q run
   float fa[2][2], fb[2][2];
+  __builtin_amdgcn_s_setprio(1);
   fa[0][0] = rp[0]; fa[0][1] = rp[32];
   fb[0][0] = cp[0]; fb[0][1] = cp[32];
   __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
@@ -87,6 +88,7 @@ __device__ __forceinline__ void mfma_slab(const float* __restrict__ R, const flo
     acc[1][1] = mfma_32x32x2(fa[c][1], fb[c][1], acc[1][1]);
     __builtin_amdgcn_sched_group_barrier(0x8, 4, 0);
   }
+  __builtin_amdgcn_s_setprio(0);
 }
 
 // A staged operand tile of OUT lines x kMS reduction steps, one float4 per
