@@ -736,8 +736,8 @@ inline int mfma_kind(int B, int out_r, int out_c, int red, bool aligned, bool lo
 }
 
 using MT128 = MTile<128, 128>;
-using MTWide = MTile<128, 256>;  // forward (m x n) and grad_a (m x k)
-using MTTall = MTile<256, 128>;  // grad_b (k x n)
+using MTWide = MTile<128, 256>;  // grad_a (m x k)
+using MTTall = MTile<256, 128>;  // forward (m x n; measured 1-2 % ahead of 128x256) and grad_b (k x n)
 
 template <bool GRAD_A>
 int run_bwd(const LogBwdArgs& p, const float* stats, int B, hipStream_t s) {
@@ -805,8 +805,8 @@ int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats, 
     int* fl = flags_of(stats, B, M, K, N, 0);
     const int64_t big_tiles = (int64_t)B * ceil_div(M, 128) * ceil_div(N, 128);
     const bool al = true;  // the matrix-core kernels assume 4-byte alignment only
-    switch (fwd_mfma_shape(B, M, K, N) ? mfma_kind(B, M, N, K, al, true) : 0) {
-      case 2: return launch_fwd_mfma<MTWide>(p, stats, fl, B, M, K, N, s);
+    switch (fwd_mfma_shape(B, M, K, N) ? mfma_kind(B, M, N, K, al, false) : 0) {
+      case 2: return launch_fwd_mfma<MTTall>(p, stats, fl, B, M, K, N, s);
       case 1: return launch_fwd_mfma<MT128>(p, stats, fl, B, M, K, N, s);
       default: break;
     }
