@@ -289,6 +289,32 @@ def test_max_index_through_c_abi(gpu, prod):
         assert bool((out == -1e9).all()) and bool((idx == -1).all())
 
 
+@pytest.mark.parametrize("B,M,K,N", [(2, 70, 261, 65), (1, 40, 600, 130), (3, 33, 7, 20), (2, 64, 512, 128)])
+@pytest.mark.parametrize("prod", [False, True])
+def test_max_index_groups_and_special_values(gpu, prod, B, M, K, N):
+    """The forward finds the index in two levels (group of consecutive k, then k inside
+    the group, with the rows of b staged 256 at a time): K across several stages and
+    not a multiple of the group, many ties, and NaN / infinite / signed-zero terms.
+    Values are compared as bit patterns."""
+    torch.manual_seed(K + N)
+    a, b = grid(B, M, K) / 2, grid(B, K, N) / 2
+    if prod:
+        a, b = a.abs(), b.abs()       # zeros stay: products tie at 0 and signs of zero matter
+        b[:, 1::5, :] *= -1
+    a[:, ::7, 3::11] = float("nan")
+    a[:, 1::9, 2::13] = float("inf")
+    b[:, 4::17, ::6] = float("-inf")
+    b[:, 5::19, 1::4] = -0.0
+    a[:, 2::5, 5::19] = -0.0
+    a[0, 0, :] = -0.0                 # a whole row of zero terms of both signs
+    b[0, :, 0] = torch.where(torch.arange(K) % 3 == 0, 0.0, -0.0)
+    out, idx = _abi_max(gpu, a.to(gpu), b.to(gpu), prod)
+    sv, si = oracle.seq_maxbmm_fwd(a, b, prod)
+    assert torch.equal(idx.cpu(), si)
+    assert torch.equal(out.cpu().view(torch.int32), sv.view(torch.int32))
+    assert int((si >= 0).sum()) > 0
+
+
 def test_max_config_c3(gpu):
     """BASELINE config 2: (256,256,256) on the 1/8 grid (max) and Uniform(0,1] (prod-max);
     bit-exact on a batch subset, argmax property on everything."""
