@@ -105,14 +105,17 @@ def dense_max(lib, dev, B, M, K, N, reps, prod):
     idx = torch.empty(B, M, N, dtype=torch.int32, device=dev)
     ga, gb = torch.empty_like(a), torch.empty_like(b)
     s, p = _lib.stream_of(a), _lib.ptr
-    fwd = lib.genbmm_prodmaxbmm_fwd if prod else lib.genbmm_maxbmm_fwd
+    fac = torch.empty(2, B, M, N, device=dev) if prod else None
 
     def f():
-        _lib.check(fwd(p(a), p(b), p(out), p(idx), B, M, K, N, s), "fwd")
+        if prod:
+            _lib.check(lib.genbmm_prodmaxbmm_fwd(p(a), p(b), p(out), p(idx), p(fac), B, M, K, N, s), "fwd")
+        else:
+            _lib.check(lib.genbmm_maxbmm_fwd(p(a), p(b), p(out), p(idx), B, M, K, N, s), "fwd")
 
     def bw():
         if prod:
-            _lib.check(lib.genbmm_prodmax_bwd(p(a), p(b), p(idx), p(g), p(ga), p(gb), B, M, K, N, s), "bwd")
+            _lib.check(lib.genbmm_prodmax_bwd(p(a), p(b), p(idx), p(fac), p(g), p(ga), p(gb), B, M, K, N, s), "bwd")
         else:
             _lib.check(lib.genbmm_argmax_bwd(p(idx), p(g), p(ga), p(gb), B, M, K, N, s), "bwd")
 

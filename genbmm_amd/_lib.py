@@ -33,10 +33,10 @@ SIGNATURES = {
     "genbmm_logbmm_bwd": [_c_float_p] * 7 + _DENSE_DIMS,
     "genbmm_logbmm_bwdbwd": [_c_float_p] * 9 + _DENSE_DIMS,
     "genbmm_maxbmm_fwd": [_c_float_p] * 3 + [_c_int_p] + _DENSE_DIMS,
-    "genbmm_prodmaxbmm_fwd": [_c_float_p] * 3 + [_c_int_p] + _DENSE_DIMS,
+    "genbmm_prodmaxbmm_fwd": [_c_float_p] * 3 + [_c_int_p, _c_float_p] + _DENSE_DIMS,
     "genbmm_samplebmm_fwd": [_c_float_p] * 3 + [_c_int_p, _c_float_p, _u64, _u64] + _DENSE_DIMS,
     "genbmm_argmax_bwd": [_c_int_p] + [_c_float_p] * 3 + _DENSE_DIMS,
-    "genbmm_prodmax_bwd": [_c_float_p] * 2 + [_c_int_p] + [_c_float_p] * 3 + _DENSE_DIMS,
+    "genbmm_prodmax_bwd": [_c_float_p] * 2 + [_c_int_p] + [_c_float_p] * 4 + _DENSE_DIMS,
     "genbmm_banded_fwd": _BAND + [_c_float_p, _c_int_p, _c_float_p, _i, _i, _i, _vp],
     "genbmm_banded_bwd": _BAND + [_c_float_p, _c_int_p] + [_c_float_p] * 4 + [_i, _i, _i, _vp],
     "genbmm_banded_bwdbwd": _BAND + [_c_float_p] * 7 + [_i, _i, _vp],

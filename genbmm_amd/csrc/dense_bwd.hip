@@ -103,8 +103,11 @@ constexpr int kKC = 128;  // gradient columns/rows accumulated per workgroup
 // One wave: lane = row m of a 64-row tile, k in [c0, c0 + kKC).  The row is read
 // 16 cells at a time (int4 / float4 when the rows are 16-byte aligned), then the
 // 16 additions are made in order.
-template <bool PROD>
+// PROD: 0 plain sum of g, 1 times b[idx, n] gathered from b, 2 times the factor the
+// forward stored per cell (fac[m,n] = b[idx[m,n], n], read like g).
+template <int PROD>
 __global__ __launch_bounds__(64) void k_argmax_bwd_a(const float* __restrict__ bmat,
+                                                    const float* __restrict__ fac,
                                                     const int32_t* __restrict__ idx,
                                                     const float* __restrict__ g,
                                                     float* __restrict__ grad_a, int M, int K,
@@ -119,16 +122,20 @@ __global__ __launch_bounds__(64) void k_argmax_bwd_a(const float* __restrict__ b
   const bool live = m < M;
   const int32_t* irow = idx + ((long)batch * M + (live ? m : 0)) * N;
   const float* grow = g + ((long)batch * M + (live ? m : 0)) * N;
-  const float* bb = PROD ? bmat + (long)batch * K * N : nullptr;
+  const float* bb = PROD == 1 ? bmat + (long)batch * K * N : nullptr;
+  const float* frow = PROD == 2 ? fac + ((long)batch * M + (live ? m : 0)) * N : nullptr;
   float* mine = accs + lane * (kKC + 1);
   for (int kk = 0; kk < kKC; ++kk) mine[kk] = 0.f;
-  auto add = [&](int n, int ki, float gv) __attribute__((always_inline)) {
+  // the term of cell n: g, times b[idx, n] for the product semiring (read only when
+  // the index falls into this workgroup's k range)
+  auto term = [&](int n, int ki, float gv) __attribute__((always_inline)) {
     const int k = ki - c0;
-    if (k >= 0 && k < kc) {
-      float v = gv;
-      if (PROD) v = __fmul_rn(bb[(long)ki * N + n], v);
-      mine[k] = __fadd_rn(mine[k], v);
-    }
+    if (PROD == 1 && k >= 0 && k < kc) return __fmul_rn(bb[(long)ki * N + n], gv);
+    return gv;
+  };
+  auto add = [&](int ki, float v) __attribute__((always_inline)) {
+    const int k = ki - c0;
+    if (k >= 0 && k < kc) mine[k] = __fadd_rn(mine[k], v);
   };
   if (live) {
     int n = 0;
@@ -141,16 +148,35 @@ __global__ __launch_bounds__(64) void k_argmax_bwd_a(const float* __restrict__ b
           iv[q] = *reinterpret_cast<const int4*>(irow + n + 4 * q);
           gv[q] = *reinterpret_cast<const float4*>(grow + n + 4 * q);
         }
+        if (PROD == 2) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float4 f = *reinterpret_cast<const float4*>(frow + n + 4 * q);
+            gv[q].x = __fmul_rn(f.x, gv[q].x);
+            gv[q].y = __fmul_rn(f.y, gv[q].y);
+            gv[q].z = __fmul_rn(f.z, gv[q].z);
+            gv[q].w = __fmul_rn(f.w, gv[q].w);
+          }
+        }
+        // all sixteen factors are requested before the first (ordered) addition
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          add(n + 4 * q, iv[q].x, gv[q].x);
-          add(n + 4 * q + 1, iv[q].y, gv[q].y);
-          add(n + 4 * q + 2, iv[q].z, gv[q].z);
-          add(n + 4 * q + 3, iv[q].w, gv[q].w);
+          gv[q].x = term(n + 4 * q, iv[q].x, gv[q].x);
+          gv[q].y = term(n + 4 * q + 1, iv[q].y, gv[q].y);
+          gv[q].z = term(n + 4 * q + 2, iv[q].z, gv[q].z);
+          gv[q].w = term(n + 4 * q + 3, iv[q].w, gv[q].w);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          add(iv[q].x, gv[q].x);
+          add(iv[q].y, gv[q].y);
+          add(iv[q].z, gv[q].z);
+          add(iv[q].w, gv[q].w);
         }
       }
     }
-    for (; n < N; ++n) add(n, irow[n], grow[n]);
+    for (; n < N; ++n)
+      add(irow[n], PROD == 2 ? __fmul_rn(frow[n], grow[n]) : term(n, irow[n], grow[n]));
   }
   __syncthreads();
   const int rows = min(64, M - m0);
@@ -162,8 +188,9 @@ __global__ __launch_bounds__(64) void k_argmax_bwd_a(const float* __restrict__ b
 
 // One wave: lane = column n of a 64-column tile, k in [c0, c0 + kKC); the column is
 // read 8 rows at a time (coalesced across the lanes), then added in order.
-template <bool PROD>
+template <int PROD>
 __global__ __launch_bounds__(64) void k_argmax_bwd_b(const float* __restrict__ amat,
+                                                    const float* __restrict__ fac,
                                                     const int32_t* __restrict__ idx,
                                                     const float* __restrict__ g,
                                                     float* __restrict__ grad_b, int M, int K,
@@ -177,15 +204,18 @@ __global__ __launch_bounds__(64) void k_argmax_bwd_b(const float* __restrict__ a
   if (n >= N) return;  // lanes are independent: no barriers below
   const int32_t* icol = idx + (long)batch * M * N + n;
   const float* gcol = g + (long)batch * M * N + n;
-  const float* ab = PROD ? amat + (long)batch * M * K : nullptr;
+  const float* ab = PROD == 1 ? amat + (long)batch * M * K : nullptr;
+  const float* fcol = PROD == 2 ? fac + (long)batch * M * N + n : nullptr;
   for (int kk = 0; kk < kKC; ++kk) accs[kk * 64 + lane] = 0.f;
-  auto add = [&](int m, int ki, float gv) __attribute__((always_inline)) {
+  auto term = [&](int m, int ki, float gv) __attribute__((always_inline)) {
     const int k = ki - c0;
-    if (k >= 0 && k < kc) {
-      float v = gv;
-      if (PROD) v = __fmul_rn(ab[(long)m * K + ki], v);
-      accs[k * 64 + lane] = __fadd_rn(accs[k * 64 + lane], v);
-    }
+    if (PROD == 1 && k >= 0 && k < kc) return __fmul_rn(ab[(long)m * K + ki], gv);
+    if (PROD == 2) return __fmul_rn(fcol[(long)m * N], gv);
+    return gv;
+  };
+  auto add = [&](int ki, float v) __attribute__((always_inline)) {
+    const int k = ki - c0;
+    if (k >= 0 && k < kc) accs[k * 64 + lane] = __fadd_rn(accs[k * 64 + lane], v);
   };
   int m = 0;
   for (; m + 8 <= M; m += 8) {
@@ -197,37 +227,51 @@ __global__ __launch_bounds__(64) void k_argmax_bwd_b(const float* __restrict__ a
       gv[q] = gcol[(long)(m + q) * N];
     }
 #pragma unroll
-    for (int q = 0; q < 8; ++q) add(m + q, iv[q], gv[q]);
+    for (int q = 0; q < 8; ++q) gv[q] = term(m + q, iv[q], gv[q]);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) add(iv[q], gv[q]);
   }
-  for (; m < M; ++m) add(m, icol[(long)m * N], gcol[(long)m * N]);
+  for (; m < M; ++m) add(icol[(long)m * N], term(m, icol[(long)m * N], gcol[(long)m * N]));
   for (int kk = 0; kk < kc; ++kk)
     grad_b[((long)batch * K + c0 + kk) * N + n] = accs[kk * 64 + lane];
 }
 
 template <bool PROD>
-int run_argmax_bwd(const float* a, const float* b, const int32_t* idx, const float* g,
-                   float* grad_a, float* grad_b, int B, int M, int K, int N, void* stream) {
+int run_argmax_bwd(const float* a, const float* b, const int32_t* idx, const float* factors,
+                   const float* g, float* grad_a, float* grad_b, int B, int M, int K, int N,
+                   void* stream) {
   if (int e = check_dense_dims(B, M, K, N)) return e;
   const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
   if (missing(idx, mn) || missing(g, mn) || missing(grad_a, mk) || missing(grad_b, kn) ||
-      (PROD && (missing(a, mk) || missing(b, kn))))
+      (PROD && !factors && (missing(a, mk) || missing(b, kn))))
     return GENBMM_E_NULLPTR;
+  // factors = [a[m, idx] | b[idx, n]], each B*M*N: grad_a needs the second, grad_b the first
+  constexpr int kGather = PROD ? 1 : 0;
   hipStream_t s = (hipStream_t)stream;
   if ((int64_t)B * M * K > 0) {
     const int row_tiles = ceil_div(M, 64), k_chunks = ceil_div(K, kKC);
     const int64_t total = (int64_t)B * row_tiles * k_chunks;
     if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
     const int vec = (N % 4 == 0) && aligned16(idx) && aligned16(g);
-    hipLaunchKernelGGL((k_argmax_bwd_a<PROD>), dim3((unsigned)total), dim3(64), 0, s, b, idx, g,
-                       grad_a, M, K, N, row_tiles, k_chunks, vec);
+    if (PROD && factors && mn > 0)
+      hipLaunchKernelGGL((k_argmax_bwd_a<2>), dim3((unsigned)total), dim3(64), 0, s, b,
+                         factors + mn, idx, g, grad_a, M, K, N, row_tiles,
+                         k_chunks, vec && aligned16(factors + mn));
+    else
+      hipLaunchKernelGGL((k_argmax_bwd_a<kGather>), dim3((unsigned)total), dim3(64), 0, s, b,
+                         (const float*)nullptr, idx, g, grad_a, M, K, N, row_tiles, k_chunks, vec);
     if (int e = launch_status()) return e;
   }
   if ((int64_t)B * K * N > 0) {
     const int col_tiles = ceil_div(N, 64), k_chunks = ceil_div(K, kKC);
     const int64_t total = (int64_t)B * col_tiles * k_chunks;
     if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
-    hipLaunchKernelGGL((k_argmax_bwd_b<PROD>), dim3((unsigned)total), dim3(64), 0, s, a, idx, g,
-                       grad_b, M, K, N, col_tiles, k_chunks);
+    if (PROD && factors && mn > 0)
+      hipLaunchKernelGGL((k_argmax_bwd_b<2>), dim3((unsigned)total), dim3(64), 0, s, a, factors,
+                         idx, g, grad_b, M, K, N, col_tiles, k_chunks);
+    else
+      hipLaunchKernelGGL((k_argmax_bwd_b<kGather>), dim3((unsigned)total), dim3(64), 0, s, a,
+                         (const float*)nullptr, idx, g, grad_b, M, K, N, col_tiles, k_chunks);
     if (int e = launch_status()) return e;
   }
   return GENBMM_OK;
@@ -271,13 +315,14 @@ int genbmm_logbmm_bwdbwd(const float* a, const float* b, const float* out, const
 
 int genbmm_argmax_bwd(const int32_t* idx, const float* g, float* grad_a, float* grad_b, int B,
                       int M, int K, int N, void* stream) {
-  return genbmm::run_argmax_bwd<false>(nullptr, nullptr, idx, g, grad_a, grad_b, B, M, K, N,
-                                       stream);
+  return genbmm::run_argmax_bwd<false>(nullptr, nullptr, idx, nullptr, g, grad_a, grad_b, B, M,
+                                       K, N, stream);
 }
 
-int genbmm_prodmax_bwd(const float* a, const float* b, const int32_t* idx, const float* g,
-                       float* grad_a, float* grad_b, int B, int M, int K, int N, void* stream) {
-  return genbmm::run_argmax_bwd<true>(a, b, idx, g, grad_a, grad_b, B, M, K, N, stream);
+int genbmm_prodmax_bwd(const float* a, const float* b, const int32_t* idx, const float* factors,
+                       const float* g, float* grad_a, float* grad_b, int B, int M, int K, int N,
+                       void* stream) {
+  return genbmm::run_argmax_bwd<true>(a, b, idx, factors, g, grad_a, grad_b, B, M, K, N, stream);
 }
 
 }  // extern "C"

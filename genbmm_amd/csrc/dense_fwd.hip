@@ -141,7 +141,8 @@ typedef float float4_u __attribute__((ext_vector_type(4), aligned(4)));
 template <bool PROD, bool TAIL>
 __global__ __launch_bounds__(kResWaves * 64) void k_max_resolve(
     const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ out,
-    int32_t* __restrict__ idx, int M, int K, int N, int panels, int row_chunks, int rows_per) {
+    int32_t* __restrict__ idx, float* __restrict__ fac_a, float* __restrict__ fac_b, int M, int K,
+    int N, int panels, int row_chunks, int rows_per) {
   __shared__ float Bs[kResK * kResCols];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -158,6 +159,9 @@ __global__ __launch_bounds__(kResWaves * 64) void k_max_resolve(
   const float* bb = b + (long)batch * K * N;
   float* ob = out + (long)batch * M * N;
   int32_t* ib = idx + (long)batch * M * N;
+  // optional: the two factors of the winning term per cell (product semiring)
+  float* fa = fac_a ? fac_a + (long)batch * M * N : nullptr;
+  float* fb = fac_b ? fac_b + (long)batch * M * N : nullptr;
 
   constexpr int R = kResRows, G = kMaxGroup, STEP = kResWaves * kResRows;
   // codes of R rows; 0 (nothing to do) outside the matrix
@@ -196,15 +200,21 @@ __global__ __launch_bounds__(kResWaves * 64) void k_max_resolve(
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const long e = (long)(mb + r) * N + n;
-      if (code[r] == -1 && kc == 0) ob[e] = kFloor;
+      if (code[r] == -1 && kc == 0) {
+        ob[e] = kFloor;
+        if (fa) {
+          fa[e] = 0.f;
+          fb[e] = 0.f;
+        }
+      }
       if (kb[r] < 0) continue;
       const int rel = kb[r] - kc;
       const float* br = Bs + rel * kResCols + lane;
-      float t[G];
+      float t[G], bv[G];
 #pragma unroll
       for (int j = 0; j < G; ++j) {
-        const float bv = br[(TAIL ? min(j, rows - 1 - rel) : j) * kResCols];
-        t[j] = PROD ? av[r][j] * bv : av[r][j] + bv;
+        bv[j] = br[(TAIL ? min(j, rows - 1 - rel) : j) * kResCols];
+        t[j] = PROD ? av[r][j] * bv[j] : av[r][j] + bv[j];
         if (TAIL && kb[r] + j >= K) t[j] = -INFINITY;
       }
       float v = __builtin_fmaxf(__builtin_fmaxf(t[0], t[1]), t[2]);
@@ -222,6 +232,16 @@ __global__ __launch_bounds__(kResWaves * 64) void k_max_resolve(
       }
       ib[e] = kb[r] + first;
       ob[e] = v;
+      if (fa) {
+        float sa = av[r][0], sb = bv[0];
+#pragma unroll
+        for (int j = 1; j < G; ++j) {
+          sa = j == first ? av[r][j] : sa;
+          sb = j == first ? bv[j] : sb;
+        }
+        fa[e] = sa;
+        fb[e] = sb;
+      }
     }
   };
 
@@ -399,7 +419,7 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
 
 // ---------------------------------------------------------------- dispatch
 template <class C, bool PROD>
-int launch_max(DenseArgs p, int B, int M, int K, int N, hipStream_t s) {
+int launch_max(DenseArgs p, float* factors, int B, int M, int K, int N, hipStream_t s) {
   dim3 grid;
   if (int e = fill_args<C>(p, B, M, K, N, grid)) return e;
   hipLaunchKernelGGL((k_max_fwd<C, PROD>), grid, dim3(C::NT), 0, s, p);
@@ -414,12 +434,14 @@ int launch_max(DenseArgs p, int B, int M, int K, int N, hipStream_t s) {
   row_chunks = ceil_div(M, rows_per);
   const int64_t total = (int64_t)B * panels * row_chunks;
   if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
+  float* fa = factors;
+  float* fb = factors ? factors + (int64_t)B * M * N : nullptr;
   if (K % kMaxGroup == 0)
     hipLaunchKernelGGL((k_max_resolve<PROD, false>), dim3((unsigned)total), dim3(kResWaves * 64), 0,
-                       s, p.a, p.b, p.out, p.idx, M, K, N, panels, row_chunks, rows_per);
+                       s, p.a, p.b, p.out, p.idx, fa, fb, M, K, N, panels, row_chunks, rows_per);
   else
     hipLaunchKernelGGL((k_max_resolve<PROD, true>), dim3((unsigned)total), dim3(kResWaves * 64), 0,
-                       s, p.a, p.b, p.out, p.idx, M, K, N, panels, row_chunks, rows_per);
+                       s, p.a, p.b, p.out, p.idx, fa, fb, M, K, N, panels, row_chunks, rows_per);
   return launch_status();
 }
 
@@ -432,8 +454,8 @@ int launch_sample(DenseArgs p, int B, int M, int K, int N, hipStream_t s) {
 }
 
 template <bool PROD>
-int run_max(const float* a, const float* b, float* out, int32_t* idx, int B, int M, int K, int N,
-            void* stream) {
+int run_max(const float* a, const float* b, float* out, int32_t* idx, float* factors, int B,
+            int M, int K, int N, void* stream) {
   if (int e = check_dense_dims(B, M, K, N)) return e;
   const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
   if (missing(a, mk) || missing(b, kn) || missing(out, mn) || missing(idx, mn))
@@ -443,10 +465,10 @@ int run_max(const float* a, const float* b, float* out, int32_t* idx, int B, int
   p.a = a; p.b = b; p.out = out; p.idx = idx;
   hipStream_t s = (hipStream_t)stream;
   switch (pick_shape(B, M, N, false)) {
-    case kBig: return launch_max<CfgBig, PROD>(p, B, M, K, N, s);
-    case kWide: return launch_max<CfgWide, PROD>(p, B, M, K, N, s);
-    case kMid: return launch_max<CfgMid, PROD>(p, B, M, K, N, s);
-    default: return launch_max<CfgSmall, PROD>(p, B, M, K, N, s);
+    case kBig: return launch_max<CfgBig, PROD>(p, factors, B, M, K, N, s);
+    case kWide: return launch_max<CfgWide, PROD>(p, factors, B, M, K, N, s);
+    case kMid: return launch_max<CfgMid, PROD>(p, factors, B, M, K, N, s);
+    default: return launch_max<CfgSmall, PROD>(p, factors, B, M, K, N, s);
   }
 }
 
@@ -496,12 +518,12 @@ int genbmm_samplebmm_fwd(const float* a, const float* b, float* out, int32_t* id
 
 int genbmm_maxbmm_fwd(const float* a, const float* b, float* out, int32_t* idx, int B, int M,
                       int K, int N, void* stream) {
-  return genbmm::run_max<false>(a, b, out, idx, B, M, K, N, stream);
+  return genbmm::run_max<false>(a, b, out, idx, nullptr, B, M, K, N, stream);
 }
 
-int genbmm_prodmaxbmm_fwd(const float* a, const float* b, float* out, int32_t* idx, int B, int M,
-                          int K, int N, void* stream) {
-  return genbmm::run_max<true>(a, b, out, idx, B, M, K, N, stream);
+int genbmm_prodmaxbmm_fwd(const float* a, const float* b, float* out, int32_t* idx,
+                          float* factors, int B, int M, int K, int N, void* stream) {
+  return genbmm::run_max<true>(a, b, out, idx, factors, B, M, K, N, stream);
 }
 
 }  // extern "C"

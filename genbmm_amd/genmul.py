@@ -114,13 +114,17 @@ class LogMatMul(torch.autograd.Function):
 
 # ------------------------------------------------- max / sample / prod-max
 def _argmax_backward(ctx, grad_output, prod):
-    a, b, idx = ctx.saved_tensors
+    if prod:
+        idx, factors = ctx.saved_tensors
+    else:
+        a, b, idx = ctx.saved_tensors
     B, M, K, N = ctx.dims
     g = grad_output.to(_COMPUTE).contiguous()
     grad_a = torch.empty(B, M, K, dtype=_COMPUTE, device=g.device)
     grad_b = torch.empty(B, K, N, dtype=_COMPUTE, device=g.device)
     if prod:
-        _call("genbmm_prodmax_bwd", g, _lib.ptr(a), _lib.ptr(b), _lib.ptr(idx), _lib.ptr(g),
+        # the factors a[m, idx], b[idx, n] were stored by the forward: a and b are not read
+        _call("genbmm_prodmax_bwd", g, _lib.ptr(None), _lib.ptr(None), _lib.ptr(idx), _lib.ptr(factors), _lib.ptr(g),
               _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
     else:
         _call("genbmm_argmax_bwd", g, _lib.ptr(idx), _lib.ptr(g), _lib.ptr(grad_a),
@@ -160,9 +164,10 @@ class ProdMaxMatMul(torch.autograd.Function):
         B, M, K, N = dims
         out = torch.empty(B, M, N, dtype=_COMPUTE, device=a.device)
         idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
+        factors = torch.empty(2, B, M, N, dtype=_COMPUTE, device=a.device)
         _call("genbmm_prodmaxbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
-              B, M, K, N)
-        ctx.save_for_backward(a, b, idx)
+              _lib.ptr(factors), B, M, K, N)
+        ctx.save_for_backward(idx, factors)
         ctx.dims, ctx.in_dtype = dims, in_dtype
         return out.to(in_dtype)
 

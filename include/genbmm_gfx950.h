@@ -132,12 +132,16 @@ int genbmm_maxbmm_fwd(const float* a, const float* b, float* out, int32_t* idx,
 
 /*
  * out[b,m,n] = max_k (a[m,k] * b[k,n]); idx as above.
+ * factors (optional, may be NULL): 2*B*M*N floats of workspace for
+ * genbmm_prodmax_bwd; receives a[m, idx[m,n]] for every cell, then
+ * b[idx[m,n], n] for every cell (0 where idx is -1; nothing when K = 0), so
+ * that the backward reads its factors in order instead of gathering them.
  * Replaces _genbmm.forward(a, b, 3): matmul_cuda_kernel.cu:527-541,
  * kernel :124-152.
  */
 int genbmm_prodmaxbmm_fwd(const float* a, const float* b, float* out,
-                          int32_t* idx, int B, int M, int K, int N,
-                          void* stream);
+                          int32_t* idx, float* factors, int B, int M, int K,
+                          int N, void* stream);
 
 /*
  * out = log-sum-exp as genbmm_logbmm_fwd; idx[b,m,n] ~ Categorical(softmax_k
@@ -173,12 +177,14 @@ int genbmm_argmax_bwd(const int32_t* idx, const float* g,
  * grad_a[b,m,k] = sum_n [k == idx[m,n]] * b[k,n] * g[m,n]
  * grad_b[b,k,n] = sum_m [k == idx[m,n]] * a[m,k] * g[m,n]
  * Each term is rounded as a product and then added (no fused multiply-add),
- * in ascending n (resp. m).  Replaces _genbmm.backward(..., 3):
- * matmul_cuda_kernel.cu:697-718, kernels :399-456.
+ * in ascending n (resp. m).  factors: NULL, or the workspace filled by
+ * genbmm_prodmaxbmm_fwd for these a, b, idx; a and b are then not read (and may
+ * be NULL) and the results are the same bit for bit.  Replaces
+ * _genbmm.backward(..., 3): matmul_cuda_kernel.cu:697-718, kernels :399-456.
  */
 int genbmm_prodmax_bwd(const float* a, const float* b, const int32_t* idx,
-                       const float* g, float* grad_a, float* grad_b,
-                       int B, int M, int K, int N, void* stream);
+                       const float* factors, const float* g, float* grad_a,
+                       float* grad_b, int B, int M, int K, int N, void* stream);
 
 /* ----------------------------------------------------------------- banded */
 

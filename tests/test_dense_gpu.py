@@ -261,16 +261,59 @@ def test_max_forward_backward_bit_exact(gpu, B, M, K, N, prod):
     assert torch.equal(gb.cpu(), wb), float((gb.cpu() - wb).abs().max())
 
 
-def _abi_max(gpu, a, b, prod):
+def _abi_max(gpu, a, b, prod, factors=None):
     lib = _lib.load()
     B, M, K = a.shape
     N = b.shape[2]
     out = torch.empty(B, M, N, device=gpu)
     idx = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
-    fn = lib.genbmm_prodmaxbmm_fwd if prod else lib.genbmm_maxbmm_fwd
-    rc = fn(_lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), B, M, K, N, _lib.stream_of(a))
+    if prod:
+        rc = lib.genbmm_prodmaxbmm_fwd(_lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
+                                       _lib.ptr(factors), B, M, K, N, _lib.stream_of(a))
+    else:
+        rc = lib.genbmm_maxbmm_fwd(_lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), B, M, K, N,
+                                   _lib.stream_of(a))
     assert rc == 0
     return out, idx
+
+
+@pytest.mark.parametrize("B,M,K,N", [(3, 70, 90, 50), (2, 64, 261, 130), (2, 130, 16, 64)])
+def test_prodmax_factors_workspace(gpu, B, M, K, N):
+    """The optional workspace of the prod-max forward holds a[m, idx] and b[idx, n]; the
+    backward gives the same bits from it (a, b not passed) as from gathering a and b."""
+    torch.manual_seed(N)
+    a, b = grid(B, M, K), grid(B, K, N)
+    a[:, ::5, ::3] *= 0
+    g = grid(B, M, N).clamp(-4, 4)
+    ad, bd, gd = a.to(gpu), b.to(gpu), g.to(gpu)
+    fac = torch.full((2, B, M, N), float("nan"), device=gpu)
+    out, idx = _abi_max(gpu, ad, bd, True, fac)
+    out0, idx0 = _abi_max(gpu, ad, bd, True, None)
+    sv, si = oracle.seq_maxbmm_fwd(a, b, True)
+    assert torch.equal(out.cpu(), sv) and torch.equal(idx.cpu(), si)
+    assert torch.equal(out0.cpu(), sv) and torch.equal(idx0.cpu(), si)
+    li = si.long().clamp(min=0)
+    want_a = torch.gather(a.unsqueeze(2).expand(B, M, N, K), 3, li.unsqueeze(-1)).squeeze(-1)
+    want_b = torch.gather(b, 1, li)
+    hit = si >= 0
+    assert torch.equal(fac[0].cpu()[hit], want_a[hit]) and torch.equal(fac[1].cpu()[hit], want_b[hit])
+    assert bool((fac[0].cpu()[~hit] == 0).all()) and bool((fac[1].cpu()[~hit] == 0).all())
+    lib = _lib.load()
+    res = []
+    for use in (True, False):
+        ga, gb = torch.full_like(ad, float("nan")), torch.full_like(bd, float("nan"))
+        rc = lib.genbmm_prodmax_bwd(_lib.ptr(None if use else ad), _lib.ptr(None if use else bd), _lib.ptr(idx),
+                                    _lib.ptr(fac if use else None), _lib.ptr(gd), _lib.ptr(ga), _lib.ptr(gb),
+                                    B, M, K, N, _lib.stream_of(ad))
+        assert rc == 0
+        res.append((ga.cpu(), gb.cpu()))
+    wa, wb = oracle.seq_argmax_bwd(a, b, si, g, True)
+    for ga, gb in res:
+        assert torch.equal(ga, wa) and torch.equal(gb, wb)
+    # neither a/b nor the workspace: refused
+    rc = lib.genbmm_prodmax_bwd(_lib.ptr(None), _lib.ptr(None), _lib.ptr(idx), _lib.ptr(None), _lib.ptr(gd),
+                                _lib.ptr(ga.to(gpu)), _lib.ptr(gb.to(gpu)), B, M, K, N, _lib.stream_of(ad))
+    assert rc != 0
 
 
 @pytest.mark.parametrize("prod", [False, True])
