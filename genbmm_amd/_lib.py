@@ -40,6 +40,11 @@ SIGNATURES = {
     "genbmm_banded_fwd": _BAND + [_c_float_p, _c_int_p, _c_float_p, _i, _i, _i, _vp],
     "genbmm_banded_bwd": _BAND + [_c_float_p, _c_int_p] + [_c_float_p] * 4 + [_i, _i, _i, _vp],
     "genbmm_banded_bwdbwd": _BAND + [_c_float_p] * 7 + [_i, _i, _vp],
+    "genbmm_band_shift": [_c_float_p, _c_float_p] + [_i] * 6 + [ctypes.c_float, _vp],
+    "genbmm_band_op": _BAND + [_c_float_p, _i, _i, _i, ctypes.c_float, _vp],
+    "genbmm_band_transpose": [_c_float_p, _c_float_p, _i, _i, _i, _i, _vp],
+    "genbmm_band_to_dense": [_c_float_p, _c_float_p, _i, _i, _i, _i, ctypes.c_float, _vp],
+    "genbmm_band_from_dense": [_c_float_p, _c_float_p, _i, _i, _i, _i, _i, _vp],
 }
 STRING_FUNCS = {"genbmm_version": [], "genbmm_error_string": [_i]}
 VOID_FUNCS = {"genbmm_logbmm_force_exact": [_i]}

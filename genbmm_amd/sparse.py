@@ -10,12 +10,17 @@ element at row c + k - lu, column c: row c of `data` holds dense column c,
 `lu` entries above the diagonal, the diagonal, `ld` entries below.
 
 The three products run on the GPU through include/genbmm_gfx950.h
-(genbmm_banded_fwd / _bwd / _bwdbwd).  The structural operations are index
-arithmetic in plain torch and work on any device.  The reference's Python
+(genbmm_banded_fwd / _bwd / _bwdbwd).  The structural operations on float32
+device tensors are single-pass kernels of the same library (genbmm_band_shift,
+_op, _transpose, _to_dense, _from_dense), each an autograd Function whose
+backward is the adjoint kernel; on host tensors (and other dtypes) they are
+index arithmetic in plain torch, as in the reference.  The reference's Python
 triple-loop products (`multiply_simple` and friends, :268-401), which it uses
 when its extension is absent, have no counterpart here: a product on CPU
 tensors raises.
 """
+import operator
+
 import torch
 import torch.nn.functional as F
 
@@ -32,12 +37,106 @@ def _band_rows(n_cols, lu, ld, n_rows, device):
     return row, (row >= 0) & (row < n_rows)
 
 
+def _native(t):
+    """Device tensors in the library's element type take the kernels."""
+    return t.is_cuda and t.dtype == torch.float32
+
+
+def _struct_call(name, t, *args):
+    lib = _lib.load()
+    with _lib.device_of(t):
+        _lib.check(getattr(lib, name)(*args, _lib.stream_of(t)), name)
+
+
+class _BandShift(torch.autograd.Function):
+    """out[b, c, k] = data[b, c + dcol, k + dband] or fill (genbmm_band_shift)."""
+
+    @staticmethod
+    def forward(ctx, data, w_out, dcol, dband, fill):
+        data = data.contiguous()
+        B, n, w_in = data.shape
+        out = torch.empty(B, n, w_out, dtype=data.dtype, device=data.device)
+        _struct_call("genbmm_band_shift", data, _lib.ptr(data), _lib.ptr(out), B, n, w_in, w_out,
+                     dcol, dband, float(fill))
+        ctx.args = (w_in, dcol, dband)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        w_in, dcol, dband = ctx.args
+        return _BandShift.apply(g, w_in, -dcol, -dband, 0.0), None, None, None, None
+
+
+class _BandTranspose(torch.autograd.Function):
+    """Band data of the transposed matrix (genbmm_band_transpose); the adjoint is the
+    transpose back."""
+
+    @staticmethod
+    def forward(ctx, data, lu, ld):
+        data = data.contiguous()
+        B, n, _ = data.shape
+        out = torch.empty_like(data)
+        _struct_call("genbmm_band_transpose", data, _lib.ptr(data), _lib.ptr(out), B, n, lu, ld)
+        ctx.bands = (lu, ld)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        lu, ld = ctx.bands
+        return _BandTranspose.apply(g, ld, lu), None, None
+
+
+class _BandToDense(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, data, lu, ld, fill):
+        data = data.contiguous()
+        B, n, _ = data.shape
+        out = torch.empty(B, n, n, dtype=data.dtype, device=data.device)
+        _struct_call("genbmm_band_to_dense", data, _lib.ptr(data), _lib.ptr(out), B, n, lu, ld,
+                     float(fill))
+        ctx.bands = (lu, ld)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        lu, ld = ctx.bands
+        return _BandFromDense.apply(g, lu, ld), None, None, None
+
+
+class _BandFromDense(torch.autograd.Function):
+    """Square (B, n, n) dense -> band (genbmm_band_from_dense)."""
+
+    @staticmethod
+    def forward(ctx, dense, lu, ld):
+        dense = dense.contiguous()
+        B, n_rows, n = dense.shape
+        out = torch.empty(B, n, lu + ld + 1, dtype=dense.dtype, device=dense.device)
+        _struct_call("genbmm_band_from_dense", dense, _lib.ptr(dense), _lib.ptr(out), B, n_rows, n,
+                     lu, ld)
+        ctx.bands = (lu, ld)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        lu, ld = ctx.bands
+        return _BandToDense.apply(g, lu, ld, 0.0), None, None
+
+
+# element-wise callables the library applies in one pass (others are applied by torch)
+_FUSED_OPS = {torch.add: 0, operator.add: 0, torch.mul: 1, operator.mul: 1,
+              torch.max: 2, torch.maximum: 2, torch.min: 3, torch.minimum: 3}
+
+
 def banddiag(orig_x, lu, ld, fill=0):
     """Band storage of the dense (..., n, n) matrix `orig_x`, keeping `lu` super- and
     `ld` sub-diagonals.  Returns (band, orig_x) like the reference (sparse.py:12-30),
     whose second value is the input seen through its padded copy.  Cells that fall
     outside the matrix hold 0 (the reference ignores `fill` here as well)."""
     n_rows, n_cols = orig_x.shape[-2], orig_x.shape[-1]
+    if _native(orig_x) and n_rows == n_cols and orig_x.dim() >= 3:
+        flat = orig_x.reshape(-1, n_rows, n_cols)
+        band = _BandFromDense.apply(flat, lu, ld)
+        return band.reshape(orig_x.shape[:-2] + (n_cols, lu + ld + 1)), orig_x
     row, ok = _band_rows(n_cols, lu, ld, n_rows, orig_x.device)
     col = torch.arange(n_cols, device=orig_x.device).unsqueeze(1).expand_as(row)
     band = orig_x[..., row.clamp(0, max(n_rows - 1, 0)), col]
@@ -50,6 +149,8 @@ def _band_transpose(data, lu, ld):
     T[i, k] = data[i + k - ld, W - 1 - k] when that row exists, else 0
     (reference Transpose / repdiag, sparse.py:33-77)."""
     n, width = data.shape[-2], data.shape[-1]
+    if _native(data) and data.dim() == 3:
+        return _BandTranspose.apply(data, lu, ld)
     i = torch.arange(n, device=data.device).unsqueeze(1)
     k = torch.arange(width, device=data.device).unsqueeze(0)
     src = i + k - ld
@@ -77,7 +178,9 @@ class BandedMatrix:
         the same numbers are re-labelled lu + t / ld - t (reference sparse.py:96-110)."""
         if t == 0:
             return self
-        if t > 0:
+        if _native(self.data):
+            v = _BandShift.apply(self.data, self.width, 0, t, self.fill)
+        elif t > 0:
             v = F.pad(self.data[:, :, t:], (0, t), value=self.fill)
         else:
             v = F.pad(self.data[:, :, :t], (-t, 0), value=self.fill)
@@ -87,12 +190,18 @@ class BandedMatrix:
         """Widen the band by `t` fill cells on both sides (reference sparse.py:112-123)."""
         if t == 0:
             return self
-        v = F.pad(self.data, (abs(t), abs(t)), value=self.fill)
+        if _native(self.data):
+            v = _BandShift.apply(self.data, self.width + 2 * abs(t), 0, -abs(t), self.fill)
+        else:
+            v = F.pad(self.data, (abs(t), abs(t)), value=self.fill)
         return BandedMatrix(v, self.lu + t, self.ld + t, self.fill)
 
     def band_unshift(self):
         """One fill cell in front, last cell dropped; lu - 1 / ld + 1 (sparse.py:137-152)."""
-        v = F.pad(self.data[:, :, :-1], (1, 0), value=self.fill)
+        if _native(self.data):
+            v = _BandShift.apply(self.data, self.width, 0, -1, self.fill)
+        else:
+            v = F.pad(self.data[:, :, :-1], (1, 0), value=self.fill)
         return BandedMatrix(v, self.lu - 1, self.ld + 1, self.fill)
 
     def col_shift(self, t):
@@ -100,7 +209,9 @@ class BandedMatrix:
         way); lu - t / ld + t (reference sparse.py:154-165)."""
         if t == 0:
             return self
-        if t > 0:
+        if _native(self.data):
+            v = _BandShift.apply(self.data, self.width, t, 0, self.fill)
+        elif t > 0:
             v = F.pad(self.data[:, t:, :], (0, 0, 0, t), value=self.fill)
         else:
             v = F.pad(self.data[:, :t, :], (0, 0, -t, 0), value=self.fill)
@@ -108,12 +219,17 @@ class BandedMatrix:
 
     def col_unshift(self):
         """One fill column in front, last column dropped; lu + 1 / ld - 1 (sparse.py:167-182)."""
-        v = F.pad(self.data[:, :-1, :], (0, 0, 1, 0), value=self.fill)
+        if _native(self.data):
+            v = _BandShift.apply(self.data, self.width, -1, 0, self.fill)
+        else:
+            v = F.pad(self.data[:, :-1, :], (0, 0, 1, 0), value=self.fill)
         return BandedMatrix(v, self.lu + 1, self.ld - 1, self.fill)
 
     def to_dense(self):
         """Dense (batch, n, n) matrix; cells outside the band hold `fill` (sparse.py:184-190)."""
         batch, n, _ = self.data.shape
+        if _native(self.data):
+            return _BandToDense.apply(self.data, self.lu, self.ld, self.fill)
         row, ok = _band_rows(n, self.lu, self.ld, n, self.data.device)
         col = torch.arange(n, device=self.data.device).unsqueeze(1).expand_as(row)
         full = self.data.new_full((batch, n, n), self.fill)
@@ -122,9 +238,12 @@ class BandedMatrix:
 
     def _expand(self, lu, ld):
         """Same matrix in a wider band (lu >= self.lu, ld >= self.ld) (sparse.py:192-197)."""
-        data = self._new(lu, ld)
         s = lu - self.lu
-        data[:, :, s : s + self.width] = self.data
+        if _native(self.data):
+            data = _BandShift.apply(self.data, lu + ld + 1, 0, -s, self.fill)
+        else:
+            data = self._new(lu, ld)
+            data[:, :, s : s + self.width] = self.data
         return BandedMatrix(data, lu, ld, self.fill)
 
     def op(self, other, op, zero=0):
@@ -132,6 +251,16 @@ class BandedMatrix:
         covers see `zero` for the other (reference sparse.py:199-212)."""
         lu = max(self.lu, other.lu)
         ld = max(self.ld, other.ld)
+        code = _FUSED_OPS.get(op) if callable(op) and getattr(op, "__hash__", None) else None
+        needs_grad = torch.is_grad_enabled() and (self.data.requires_grad or other.data.requires_grad)
+        if (code is not None and not needs_grad and _native(self.data) and _native(other.data)
+                and self.data.shape[:2] == other.data.shape[:2]):
+            a, b = self.data.contiguous(), other.data.contiguous()
+            batch, n, _ = a.shape
+            data = torch.empty(batch, n, lu + ld + 1, dtype=a.dtype, device=a.device)
+            _struct_call("genbmm_band_op", a, _lib.ptr(a), self.lu, self.ld, _lib.ptr(b), other.lu,
+                         other.ld, _lib.ptr(data), batch, n, code, float(zero))
+            return BandedMatrix(data, lu, ld, self.fill)
         data = self._new(lu, ld).fill_(zero)
         s1 = lu - self.lu
         data[:, :, s1 : s1 + self.width] = self.data

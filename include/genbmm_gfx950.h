@@ -250,6 +250,62 @@ int genbmm_banded_bwdbwd(const float* a, int a_lu, int a_ld,
                          float* grad_a, float* grad_b, float* grad_g,
                          int B, int n, void* stream);
 
+/* ------------------------------------------------- band storage, structure */
+
+/*
+ * The reference has no native entry points for these: genbmm/sparse.py builds
+ * them from torch cat / flip / unfold / diagonal / contiguous calls on the band
+ * tensor.  Each one below is a single pass (one read, one write).  data is
+ * (B, n, W = lu + ld + 1), data[b, c, k] = Dense[b, c + k - lu, c].
+ */
+
+/*
+ * out[b, c, k] = data[b, c + dcol, k + dband] where that lies inside
+ * (n, w_in), else fill; out is (B, n, w_out).  With the band offsets
+ * re-labelled by the caller this is band_shift(t) (dband = t, sparse.py:96-110),
+ * band_pad(t) (dband = -|t|, w_out = w_in + 2|t|, :112-123), band_unshift
+ * (dband = -1, :137-152), col_shift(t) (dcol = t, :154-165), col_unshift
+ * (dcol = -1, :167-182) and _expand (dband = -(lu' - lu), :192-197).
+ */
+int genbmm_band_shift(const float* data, float* out, int B, int n, int w_in,
+                      int w_out, int dcol, int dband, float fill, void* stream);
+
+/*
+ * Element-wise op on the union band (lu = max(a_lu, b_lu), ld = max(a_ld,
+ * b_ld)): out = zero; out[a's cells] = a; out[b's cells] = op(out, b), as
+ * BandedMatrix.op does (sparse.py:199-212).
+ */
+#define GENBMM_OP_ADD 0
+#define GENBMM_OP_MUL 1
+#define GENBMM_OP_MAX 2
+#define GENBMM_OP_MIN 3
+int genbmm_band_op(const float* a, int a_lu, int a_ld,
+                   const float* b, int b_lu, int b_ld, float* out,
+                   int B, int n, int op, float zero, void* stream);
+
+/*
+ * Band storage of the transposed matrix (its lu is ld, its ld is lu):
+ * out[b, c, k] = data[b, c + k - ld, W - 1 - k], 0 where that row does not
+ * exist (Transpose / repdiag and BandedMatrix.transpose, sparse.py:33-77,
+ * 214-218).
+ */
+int genbmm_band_transpose(const float* data, float* out, int B, int n,
+                          int lu, int ld, void* stream);
+
+/*
+ * out (B, n, n): out[b, r, c] = data[b, c, r - c + lu] inside the band, else
+ * fill (BandedMatrix.to_dense, sparse.py:184-190).
+ */
+int genbmm_band_to_dense(const float* data, float* out, int B, int n,
+                         int lu, int ld, float fill, void* stream);
+
+/*
+ * Band storage of dense (B, n_rows, n): out[b, c, k] = dense[b, c + k - lu, c],
+ * 0 where that row does not exist (banddiag, sparse.py:12-30).
+ */
+int genbmm_band_from_dense(const float* dense, float* out, int B, int n_rows,
+                           int n, int lu, int ld, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -269,6 +269,45 @@ def band_transpose_indexed(data, lu, ld):
     return torch.from_numpy(np.where(ok[None], out, 0).astype(d.dtype))
 
 
+def band_relabel(data, dcol, dband, w_out, fill):
+    """out[b, c, k] = data[b, c + dcol, k + dband] where that cell exists, else `fill`:
+    the one index rule behind the reference's slicing-and-padding methods
+    (genbmm/sparse.py): band_shift(t) :96-110 is dband = t; band_pad(t) :112-123 is
+    dband = -|t| with 2|t| more cells; band_unshift :137-152 is dband = -1;
+    col_shift(t) :154-165 is dcol = t; col_unshift :167-182 is dcol = -1; _expand
+    :192-197 is dband = -(lu' - lu).  Explicit loops; pinned against the reference's own
+    outputs (tests/golden/band_struct.npz) in tests/test_oracle.py."""
+    d = data.detach().cpu().numpy()
+    batch, n, w = d.shape
+    out = np.full((batch, n, w_out), fill, dtype=d.dtype)
+    for c in range(n):
+        cs = c + dcol
+        if cs < 0 or cs >= n:
+            continue
+        for k in range(w_out):
+            ks = k + dband
+            if 0 <= ks < w:
+                out[:, c, k] = d[:, cs, ks]
+    return torch.from_numpy(out)
+
+
+def band_op(a, a_lu, a_ld, b, b_lu, b_ld, fn, zero):
+    """BandedMatrix.op (genbmm/sparse.py:199-212) cell by cell on the union band:
+    `zero` where neither operand has a cell, a's value where only a has one,
+    fn(zero, b) where only b has one, fn(a, b) where both do.  `fn` works on numpy
+    arrays.  Returns (data, lu, ld)."""
+    x, y = a.detach().cpu().numpy(), b.detach().cpu().numpy()
+    batch, n, wa = x.shape
+    wb = y.shape[2]
+    lu, ld = max(a_lu, b_lu), max(a_ld, b_ld)
+    out = np.full((batch, n, lu + ld + 1), zero, dtype=x.dtype)
+    for k in range(lu + ld + 1):
+        ka, kb = k - (lu - a_lu), k - (lu - b_lu)
+        cur = x[:, :, ka] if 0 <= ka < wa else out[:, :, k]
+        out[:, :, k] = fn(cur, y[:, :, kb]) if 0 <= kb < wb else cur
+    return torch.from_numpy(out), lu, ld
+
+
 def band_product_dense(a, a_lu, a_ld, b, b_lu, b_ld, mode):
     """X.multiply*(Y) as dense algebra (test_sparse.py:141-142, 181-195): Dense(Y)^T (x)
     Dense(X), re-banded with lu = a_lu + b_ld, ld = a_ld + b_lu.  mode 3: torch.bmm;

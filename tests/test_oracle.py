@@ -13,6 +13,7 @@ pinned against something independent of its own formula:
     autograd through them.
 """
 import math
+import os
 
 import numpy as np
 import pytest
@@ -302,3 +303,33 @@ def test_band_products_match_reference_cpu_loops(case):
     want = torch.from_numpy(z[p + "multiply_back_simple"])
     assert [ld, lu] == [int(v) for v in z[p + "multiply_back_simple_luld"]]
     assert torch.allclose(oracle.band_transpose(ga, lu, ld), want, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("case", range(4))
+def test_band_relabel_and_op_match_reference_vectors(case):
+    """oracle.band_relabel / band_op / band_transpose_indexed / band_to_dense against the
+    outputs of the reference's own BandedMatrix methods (tests/golden/band_struct.npz)."""
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "band_struct.npz"), allow_pickle=False)
+    p = "c%d_" % case
+    B, n, lu, ld, olu, old = (int(v) for v in z[p + "meta"])
+    fill = float(z[p + "fill"])
+    band, oband = torch.from_numpy(z[p + "band"]), torch.from_numpy(z[p + "oband"])
+    W = lu + ld + 1
+
+    def same(name, got):
+        assert torch.equal(got, torch.from_numpy(z[p + name])), name
+
+    same("band_shift_p1", oracle.band_relabel(band, 0, 1, W, fill))
+    same("band_shift_m2", oracle.band_relabel(band, 0, -2, W, fill))
+    same("band_pad_2", oracle.band_relabel(band, 0, -2, W + 4, fill))
+    same("band_unshift", oracle.band_relabel(band, 0, -1, W, fill))
+    same("col_shift_p1", oracle.band_relabel(band, 1, 0, W, fill))
+    same("col_shift_m2", oracle.band_relabel(band, -2, 0, W, fill))
+    same("col_unshift", oracle.band_relabel(band, -1, 0, W, fill))
+    same("expand", oracle.band_relabel(band, 0, -2, W + 3, fill))
+    got, glu, gld = oracle.band_op(band, lu, ld, oband, olu, old, np.add, 0.0)
+    assert [glu, gld] == [int(v) for v in z[p + "op_add_luld"]]
+    same("op_add", got)
+    same("op_max", oracle.band_op(band, lu, ld, oband, olu, old, np.maximum, -1e9)[0])
+    same("transpose", oracle.band_transpose_indexed(band, lu, ld))
+    same("to_dense", oracle.band_to_dense(band, lu, ld, fill))
