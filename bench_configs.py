@@ -179,6 +179,57 @@ def banded(lib, dev, B, n, lu, ld, mode, reps):
             "fwd_GBs": round(fb / mf / 1e6, 1), "bwd_GBs": round(bb / mb / 1e6, 1)})
 
 
+def band_structure(lib, dev, B, n, lu, ld, reps):
+    """The structural kernels at the banded configuration's size: HBM-bound copies, the
+    figure is algorithmic GB/s (one read of the source + one write of the result).  The
+    same operation written as torch index arithmetic (the host layer's formulation for
+    CPU tensors, run here on the device) is timed beside it."""
+    W = lu + ld + 1
+    torch.manual_seed(7)
+    data = (torch.rand(B, n, W) * 2 - 1).to(dev)
+    s, p = _lib.stream_of(data), _lib.ptr
+    out = torch.empty_like(data)
+    wide = torch.empty(B, n, W + 8, device=dev)
+    band_bytes = 4.0 * B * n * W
+
+    def line(name, ms, nbytes, torch_ms=None):
+        d = {"config": "band %s (B=%d,n=%d,lu=ld=%d)" % (name, B, n, lu), "ms": round(ms, 4),
+             "algorithmic_GBs": round(nbytes / ms / 1e6, 1),
+             "pct_hbm_peak": round(100 * nbytes / (ms * 1e-3) / (PEAK_HBM_GBS * 1e9), 2)}
+        if torch_ms is not None:
+            d["torch_index_ops_ms"] = round(torch_ms, 4)
+        print(json.dumps(d), flush=True)
+
+    import torch.nn.functional as F
+
+    def idx_transpose():
+        i = torch.arange(n, device=dev).unsqueeze(1)
+        k = torch.arange(W, device=dev).unsqueeze(0)
+        src = i + k - ld
+        ok = (src >= 0) & (src < n)
+        g = data[..., src.clamp(0, n - 1), (W - 1 - k).expand_as(src)]
+        return torch.where(ok, g, torch.zeros((), device=dev))
+
+    ms = timed(lambda: _lib.check(lib.genbmm_band_transpose(p(data), p(out), B, n, lu, ld, s), "t"), reps)
+    line("transpose", ms, 2 * band_bytes, timed(idx_transpose, max(3, reps // 4)))
+    ms = timed(lambda: _lib.check(lib.genbmm_band_shift(p(data), p(out), B, n, W, W, 0, 3, 0.0, s), "s"), reps)
+    line("band_shift(3)", ms, 2 * band_bytes, timed(lambda: F.pad(data[:, :, 3:], (0, 3)), reps))
+    ms = timed(lambda: _lib.check(lib.genbmm_band_shift(p(data), p(out), B, n, W, W, 5, 0, 0.0, s), "c"), reps)
+    line("col_shift(5)", ms, 2 * band_bytes, timed(lambda: F.pad(data[:, 5:, :], (0, 0, 0, 5)), reps))
+    ms = timed(lambda: _lib.check(lib.genbmm_band_shift(p(data), p(wide), B, n, W, W + 8, 0, -4, 0.0, s), "p"), reps)
+    line("band_pad(4)", ms, band_bytes + 4.0 * B * n * (W + 8), timed(lambda: F.pad(data, (4, 4)), reps))
+    ms = timed(lambda: _lib.check(lib.genbmm_band_op(p(data), lu, ld, p(data), lu, ld, p(out), B, n, 0, 0.0, s), "o"), reps)
+    line("op(add)", ms, 3 * band_bytes, timed(lambda: torch.add(data, data), reps))
+    # dense forms: B * n * n * 4 bytes (4.3 GB at B=64, n=4096)
+    Bd = B
+    dense = torch.empty(Bd, n, n, device=dev)
+    sub = data[:Bd].contiguous()
+    ms = timed(lambda: _lib.check(lib.genbmm_band_to_dense(p(sub), p(dense), Bd, n, lu, ld, 0.0, s), "d"), reps)
+    line("to_dense", ms, 4.0 * Bd * n * (n + W))
+    ms = timed(lambda: _lib.check(lib.genbmm_band_from_dense(p(dense), p(out), Bd, n, n, lu, ld, s), "f"), reps)
+    line("banddiag", ms, 4.0 * Bd * n * 2 * W)
+
+
 def cpu_c1():
     import oracle
 
@@ -207,9 +258,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--cpu", action="store_true")
-    ap.add_argument("--only", default="", help="comma-separated subset: log,max,sample,banded")
+    ap.add_argument("--only", default="", help="comma-separated subset: log,max,sample,banded,struct")
     args = ap.parse_args()
-    want = set(args.only.split(",")) if args.only else {"log", "max", "sample", "banded"}
+    want = set(args.only.split(",")) if args.only else {"log", "max", "sample", "banded", "struct"}
     lib = _lib.load()
     dev = torch.device("cuda:0")
     r = args.reps
@@ -227,6 +278,8 @@ def main():
     if "banded" in want:
         for mode in (3, 0, 1):
             banded(lib, dev, 64, 4096, 32, 32, mode, r)
+    if "struct" in want:
+        band_structure(lib, dev, 64, 4096, 32, 32, r)
     if args.cpu:
         cpu_c1()
 

@@ -15,6 +15,8 @@ constexpr int kBlockCells = 8192;        // cells of the result per workgroup (r
 constexpr int kMaxLine = 1 << 20;        // longest row (band width or n) the kernels take
 constexpr int kTileBytes = 64 * 1024;    // LDS tile budget of the skewed kernels
 
+typedef float float4_u __attribute__((ext_vector_type(4), aligned(4)));  // any 4-byte address
+
 // i / d for 0 <= i < 2^21 through the float unit (inv = 1/d rounded): (i + 0.5)/d
 // is at least 0.5/d away from every integer and the rounding error is below that.
 __device__ __forceinline__ int small_div(int i, float inv) {
@@ -36,6 +38,7 @@ __global__ __launch_bounds__(kST) void k_band_shift(const float* __restrict__ in
   const float* ib = in + (long)batch * n * w_in;
   float* ob = out + ((long)batch * n + c0) * w_out;
   const int total = rows * w_out;
+#pragma unroll 4
   for (int i = threadIdx.x; i < total; i += kST) {
     const int r = small_div(i, inv_w), k = i - r * w_out;
     const int cs = c0 + r + dcol, ks = k + dband;
@@ -72,6 +75,7 @@ __global__ __launch_bounds__(kST) void k_band_op(const float* __restrict__ a,
   const float* bb = b + ((long)batch * n + c0) * wb;
   float* ob = out + ((long)batch * n + c0) * wo;
   const int total = rows * wo;
+#pragma unroll 4
   for (int i = threadIdx.x; i < total; i += kST) {
     const int r = small_div(i, inv_w), k = i - r * wo;
     const int ka = k - sa, kb = k - sb;
@@ -99,14 +103,40 @@ __global__ __launch_bounds__(kST) void k_band_transpose(const float* __restrict_
   const float* ib = in + (long)batch * n * W;
   float* ob = out + ((long)batch * n + c0) * W;
   const int first = c0 - ld, src_rows = cols + W - 1;
-  for (int i = threadIdx.x; i < src_rows * W; i += kST) {
-    const int r = small_div(i, inv_w), k = i - r * W;
-    const int src = first + r;
-    const bool ok = src >= 0 && src < n;
-    const float v = ib[ok ? (long)src * W + k : 0];
-    tile[r * pitch + k] = ok ? v : 0.f;
+  // the source rows that exist are one contiguous run of cells: four per lane and load
+  const int lo = max(first, 0), hi = min(first + src_rows, n);      // rows [lo, hi)
+  const int cells = (hi - lo) * W, skip = (lo - first) * W;
+  const float* run = ib + (long)lo * W;
+  for (int i = threadIdx.x; i < skip; i += kST) {                   // rows before row 0
+    const int r = small_div(i, inv_w);
+    tile[r * pitch + (i - r * W)] = 0.f;
+  }
+  for (int i = skip + cells + threadIdx.x; i < src_rows * W; i += kST) {   // rows past n - 1
+    const int r = small_div(i, inv_w);
+    tile[r * pitch + (i - r * W)] = 0.f;
+  }
+#pragma unroll 2
+  for (int i = threadIdx.x * 4; i < cells; i += kST * 4) {
+    float v[4];
+    if (i + 4 <= cells) {
+      const float4_u x = *reinterpret_cast<const float4_u*>(run + i);
+      v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = run[min(i + j, cells - 1)];
+    }
+    int r = small_div(skip + i, inv_w), k = skip + i - r * W;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (i + j < cells) tile[r * pitch + k] = v[j];
+      if (++k == W) {
+        k = 0;
+        ++r;
+      }
+    }
   }
   __syncthreads();
+#pragma unroll 4
   for (int i = threadIdx.x; i < cols * W; i += kST) {
     const int c = small_div(i, inv_w), k = i - c * W;
     ob[i] = tile[(c + k) * pitch + (W - 1 - k)];
@@ -148,7 +178,8 @@ __global__ __launch_bounds__(kST) void k_band_to_dense(const float* __restrict__
   if (VEC) {
     const int quads = n >> 2, total = rows * quads;
     const float inv_q = inv_n * 4.f;
-    for (int i = threadIdx.x; i < total; i += kST) {
+  #pragma unroll 4
+  for (int i = threadIdx.x; i < total; i += kST) {
       const int rl = small_div(i, inv_q), c = (i - rl * quads) * 4;
       const int r = r0 + rl;
       float4 v = make_float4(fill, fill, fill, fill);
@@ -158,7 +189,8 @@ __global__ __launch_bounds__(kST) void k_band_to_dense(const float* __restrict__
     }
   } else {
     const int total = rows * n;
-    for (int i = threadIdx.x; i < total; i += kST) {
+  #pragma unroll 4
+  for (int i = threadIdx.x; i < total; i += kST) {
       const int rl = small_div(i, inv_n), c = i - rl * n;
       ob[i] = cell(r0 + rl, c);
     }
@@ -180,6 +212,7 @@ __global__ __launch_bounds__(kST) void k_band_from_dense(const float* __restrict
   const float* db = dense + (long)batch * n_rows * n;
   float* ob = out + ((long)batch * n + c0) * W;
   const int first = c0 - lu, src_rows = cols + W - 1, pitch = cb + 1;
+#pragma unroll 4
   for (int i = threadIdx.x; i < (src_rows << cb_shift); i += kST) {
     const int r = i >> cb_shift, cc = i & (cb - 1);
     const int src = first + r;
@@ -188,6 +221,7 @@ __global__ __launch_bounds__(kST) void k_band_from_dense(const float* __restrict
     tile[r * pitch + cc] = ok ? v : 0.f;
   }
   __syncthreads();
+#pragma unroll 4
   for (int i = threadIdx.x; i < cols * W; i += kST) {
     const int c = small_div(i, inv_w), k = i - c * W;
     ob[i] = tile[(c + k) * pitch + c];
@@ -229,9 +263,10 @@ int row_blocks(int B, int n, int line, int& rows_per, int& chunks, unsigned& gri
   return GENBMM_OK;
 }
 
-// Largest power-of-two count of result rows (<= 64) whose LDS tile fits.
+// Largest power-of-two count of result rows whose LDS tile fits: the more rows, the
+// smaller the share of the W - 1 halo rows each workgroup reads on top of its own.
 int tile_rows(int W, bool from_dense, int& pitch) {
-  for (int cb = 64; cb >= 8; cb >>= 1) {
+  for (int cb = from_dense ? 64 : 128; cb >= 8; cb >>= 1) {
     pitch = from_dense ? cb + 1 : W + (W & 1);
     if ((int64_t)(cb + W - 1) * pitch * 4 <= kTileBytes) return cb;
   }
