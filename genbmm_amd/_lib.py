@@ -40,6 +40,17 @@ SIGNATURES = {
     "genbmm_banded_fwd": _BAND + [_c_float_p, _c_int_p, _c_float_p, _i, _i, _i, _vp],
     "genbmm_banded_bwd": _BAND + [_c_float_p, _c_int_p] + [_c_float_p] * 4 + [_i, _i, _i, _vp],
     "genbmm_banded_bwdbwd": _BAND + [_c_float_p] * 7 + [_i, _i, _vp],
+    "genbmm_logbmm_fwd_f64": [_c_float_p] * 3 + _DENSE_DIMS,
+    "genbmm_logbmm_bwd_f64": [_c_float_p] * 6 + _DENSE_DIMS,
+    "genbmm_logbmm_bwdbwd_f64": [_c_float_p] * 9 + _DENSE_DIMS,
+    "genbmm_maxbmm_fwd_f64": [_c_float_p] * 3 + [_c_int_p] + _DENSE_DIMS,
+    "genbmm_prodmaxbmm_fwd_f64": [_c_float_p] * 3 + [_c_int_p] + _DENSE_DIMS,
+    "genbmm_samplebmm_fwd_f64": [_c_float_p] * 3 + [_c_int_p, _u64, _u64] + _DENSE_DIMS,
+    "genbmm_argmax_bwd_f64": [_c_int_p] + [_c_float_p] * 3 + _DENSE_DIMS,
+    "genbmm_prodmax_bwd_f64": [_c_float_p] * 2 + [_c_int_p] + [_c_float_p] * 3 + _DENSE_DIMS,
+    "genbmm_banded_fwd_f64": _BAND + [_c_float_p, _c_int_p, _i, _i, _i, _vp],
+    "genbmm_banded_bwd_f64": _BAND + [_c_float_p, _c_int_p] + [_c_float_p] * 3 + [_i, _i, _i, _vp],
+    "genbmm_banded_bwdbwd_f64": _BAND + [_c_float_p] * 7 + [_i, _i, _vp],
     "genbmm_band_shift": [_c_float_p, _c_float_p] + [_i] * 6 + [ctypes.c_float, _vp],
     "genbmm_band_op": _BAND + [_c_float_p, _i, _i, _i, ctypes.c_float, _vp],
     "genbmm_band_transpose": [_c_float_p, _c_float_p, _i, _i, _i, _i, _vp],
@@ -123,9 +134,11 @@ def require(t, name, dtype=torch.float32, ndim=3, device=None):
 
 
 def dense_dims(a, b):
-    """(B, M, K, N) of a (B,M,K) x (B,K,N) product, with agreement checks."""
-    require(a, "a")
-    require(b, "b", device=a.device)
+    """(B, M, K, N) of a (B,M,K) x (B,K,N) product, with agreement checks; a's element
+    type (float32 or float64) is the one both must have."""
+    dtype = torch.float64 if isinstance(a, torch.Tensor) and a.dtype == torch.float64 else torch.float32
+    require(a, "a", dtype=dtype)
+    require(b, "b", dtype=dtype, device=a.device)
     B, M, K = a.shape
     if b.shape[0] != B or b.shape[1] != K:
         raise RuntimeError(

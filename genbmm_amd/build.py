@@ -17,7 +17,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIBNAME = "libgenbmm_gfx950.so"
-SOURCES = ["logbmm.hip", "dense_fwd.hip", "dense_bwd.hip", "banded.hip", "band_struct.hip"]
+SOURCES = ["logbmm.hip", "dense_fwd.hip", "dense_bwd.hip", "banded.hip", "band_struct.hip", "f64.hip"]
 
 # -packed-fp32-ops is switched OFF: v_pk_{add,mul,fma}_f32 are not used by any
 # kernel here, and the compiler must not form them on its own either.

@@ -26,125 +26,6 @@
 namespace genbmm {
 namespace {
 
-template <int MODE>
-__global__ __launch_bounds__(256) void k_band_fwd(const BandArgs p, long total) {
-  const long e = (long)blockIdx.x * 256 + threadIdx.x;
-  if (e >= total) return;
-  const long bi = e / p.Wo;  // batch*n + i
-  band_fwd_cell<MODE>(p, bi, (int)(bi % p.n), (int)(e - bi * p.Wo));
-}
-
-template <int MODE>
-__global__ __launch_bounds__(256) void k_band_bwd_a(const BandArgs p, long total) {
-  const long e = (long)blockIdx.x * 256 + threadIdx.x;
-  if (e >= total) return;
-  const long bi = e / p.Wa;
-  band_bwd_a_cell<MODE>(p, bi, (int)(bi % p.n), (int)(e - bi * p.Wa));
-}
-
-template <int MODE>
-__global__ __launch_bounds__(256) void k_band_bwd_b(const BandArgs p, long total) {
-  const long e = (long)blockIdx.x * 256 + threadIdx.x;
-  if (e >= total) return;
-  const long bo = e / p.Wb;
-  band_bwd_b_cell<MODE>(p, bo, (int)(bo % p.n), (int)(e - bo * p.Wb));
-}
-
-// ------------------------------------------------------ log second order
-// p = exp(a[i,k] + b[o,k2] - out[i,j]),  w = u_a[i,k] + u_b[o,k2]:
-//   t[i,j]       = sum_k p*w                        (gradient w.r.t. g)
-//   grad_a[i,k]  = sum_j g[i,j]*p*(w - t[i,j])
-//   grad_b[o,k2] = sum_i g[i,j]*p*(w - t[i,j])
-// With u_b = 0 these equal the reference's banded_cuda_backbackward_kernel_A/
-// _B/_C (banded_cuda_kernel.cu:154-350), whose inner loop sum_m (delta*s -
-// s*s2)*u[m] is s*(u[k] - t).
-__global__ __launch_bounds__(256) void k_band_bb_t(const BandArgs p, long total) {
-  const long e = (long)blockIdx.x * 256 + threadIdx.x;
-  if (e >= total) return;
-  const int j = (int)(e % p.Wo);
-  const long bi = e / p.Wo;
-  const int i = (int)(bi % p.n);
-  const int o = i + j - p.r_lu;
-  float t = 0.f;
-  if (o >= 0 && o < p.n) {
-    int klo, khi;
-    k_range(p, i, j, klo, khi);
-    const long boff = (bi + (o - i)) * p.Wb + (p.Wb - 1 - j);
-    const float ov = p.out[e];
-    for (int k = klo; k <= khi; ++k) {
-      const float pr = fast_exp(p.a[bi * p.Wa + k] + p.b[boff + k] - ov);
-      const float w = (p.ua ? p.ua[bi * p.Wa + k] : 0.f) + (p.ub ? p.ub[boff + k] : 0.f);
-      t = __builtin_fmaf(pr, w, t);
-    }
-  }
-  p.o2[e] = t;
-}
-
-__global__ __launch_bounds__(256) void k_band_bb_a(const BandArgs p, long total) {
-  const long e = (long)blockIdx.x * 256 + threadIdx.x;
-  if (e >= total) return;
-  const int k = (int)(e % p.Wa);
-  const long bi = e / p.Wa;
-  const int i = (int)(bi % p.n);
-  const int pos = i + k - p.a_lu;
-  float acc = 0.f;
-  if (pos >= 0 && pos < p.n) {
-    const int jlo = imax3(k, p.r_lu - i, 0);
-    const int jhi = imin3(k + p.Wb - 1, p.n - 1 + p.r_lu - i, p.Wo - 1);
-    const long bw = (bi - p.r_lu) * p.Wb + k + p.Wb - 1;
-    const float av = p.a[e];
-    const float uav = p.ua ? p.ua[e] : 0.f;
-    for (int j = jlo; j <= jhi; ++j) {
-      const long bj = bw + (long)j * (p.Wb - 1);
-      const long gi = bi * p.Wo + j;
-      const float pr = fast_exp(av + p.b[bj] - p.out[gi]);
-      const float w = uav + (p.ub ? p.ub[bj] : 0.f) - p.o2[gi];
-      acc = __builtin_fmaf(p.g[gi] * pr, w, acc);
-    }
-  }
-  p.o0[e] = acc;
-}
-
-__global__ __launch_bounds__(256) void k_band_bb_b(const BandArgs p, long total) {
-  const long e = (long)blockIdx.x * 256 + threadIdx.x;
-  if (e >= total) return;
-  const int k2 = (int)(e % p.Wb);
-  const long bo = e / p.Wb;
-  const int o = (int)(bo % p.n);
-  const int prow = o + k2 - p.b_lu;
-  float acc = 0.f;
-  if (prow >= 0 && prow < p.n) {
-    const int jhi_k = p.Wb - 1 - k2 + p.Wa - 1;
-    const int jlo_k = p.Wb - 1 - k2;
-    const int ilo = imax3(0, o + p.r_lu - min(jhi_k, p.Wo - 1), o + p.r_lu - (p.Wo - 1));
-    const int ihi = imin3(p.n - 1, o + p.r_lu - max(jlo_k, 0), o + p.r_lu);
-    const long base = bo - o;
-    const float bv = p.b[e];
-    const float ubv = p.ub ? p.ub[e] : 0.f;
-    for (int i = ilo; i <= ihi; ++i) {
-      const int j = o - i + p.r_lu;
-      const int k = k2 + j - (p.Wb - 1);
-      const long gi = (base + i) * p.Wo + j;
-      const long ai = (base + i) * p.Wa + k;
-      const float pr = fast_exp(p.a[ai] + bv - p.out[gi]);
-      const float w = (p.ua ? p.ua[ai] : 0.f) + ubv - p.o2[gi];
-      acc = __builtin_fmaf(p.g[gi] * pr, w, acc);
-    }
-  }
-  p.o1[e] = acc;
-}
-
-int fill_band(BandArgs& p, int a_lu, int a_ld, int b_lu, int b_ld, int B, int n) {
-  if (a_lu < 0 || a_ld < 0 || b_lu < 0 || b_ld < 0) return GENBMM_E_BAND;
-  if (B < 0 || n < 0) return GENBMM_E_SHAPE;
-  const int64_t Wa = (int64_t)a_lu + a_ld + 1, Wb = (int64_t)b_lu + b_ld + 1;
-  const int64_t Wo = Wa + Wb - 1;
-  if (Wo > 0x3fffffff || (int64_t)B * n * Wo > ((int64_t)1 << 40)) return GENBMM_E_SHAPE;
-  p.n = n; p.a_lu = a_lu; p.Wa = (int)Wa; p.b_lu = b_lu; p.Wb = (int)Wb;
-  p.r_lu = a_lu + b_ld; p.Wo = (int)Wo;
-  return GENBMM_OK;
-}
-
 constexpr size_t kStripLdsLimit = 64 * 1024;  // dynamic LDS available without opting in
 
 // Workspace of the log product: EA (B*n*Wa), EB (B*n*Wb), alpha (B*n), beta (B*n),
@@ -184,8 +65,6 @@ inline void set_workspace(BandArgs& p, float* ws, int B) {
   p.ws_be = p.ws_al + rows;
   p.ws_r = p.ws_be + rows;
 }
-
-inline dim3 blocks_for(long total) { return dim3((unsigned)((total + 255) / 256)); }
 
 }  // namespace
 }  // namespace genbmm
@@ -247,11 +126,11 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
     return launch_status();
   }
   if (mode == GENBMM_BAND_LOG)
-    hipLaunchKernelGGL(k_band_fwd<GENBMM_BAND_LOG>, blocks_for(total), dim3(256), 0, s, p, total);
+    hipLaunchKernelGGL((k_band_fwd<GENBMM_BAND_LOG, float>), blocks_for(total), dim3(256), 0, s, p, total);
   else if (mode == GENBMM_BAND_MAX)
-    hipLaunchKernelGGL(k_band_fwd<GENBMM_BAND_MAX>, blocks_for(total), dim3(256), 0, s, p, total);
+    hipLaunchKernelGGL((k_band_fwd<GENBMM_BAND_MAX, float>), blocks_for(total), dim3(256), 0, s, p, total);
   else
-    hipLaunchKernelGGL(k_band_fwd<GENBMM_BAND_MUL>, blocks_for(total), dim3(256), 0, s, p, total);
+    hipLaunchKernelGGL((k_band_fwd<GENBMM_BAND_MUL, float>), blocks_for(total), dim3(256), 0, s, p, total);
   return launch_status();
 }
 
@@ -319,14 +198,14 @@ int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_
     return launch_status();
   }
   if (mode == GENBMM_BAND_LOG) {
-    hipLaunchKernelGGL(k_band_bwd_a<GENBMM_BAND_LOG>, blocks_for(ta), dim3(256), 0, s, p, ta);
-    hipLaunchKernelGGL(k_band_bwd_b<GENBMM_BAND_LOG>, blocks_for(tb), dim3(256), 0, s, p, tb);
+    hipLaunchKernelGGL((k_band_bwd_a<GENBMM_BAND_LOG, float>), blocks_for(ta), dim3(256), 0, s, p, ta);
+    hipLaunchKernelGGL((k_band_bwd_b<GENBMM_BAND_LOG, float>), blocks_for(tb), dim3(256), 0, s, p, tb);
   } else if (mode == GENBMM_BAND_MAX) {
-    hipLaunchKernelGGL(k_band_bwd_a<GENBMM_BAND_MAX>, blocks_for(ta), dim3(256), 0, s, p, ta);
-    hipLaunchKernelGGL(k_band_bwd_b<GENBMM_BAND_MAX>, blocks_for(tb), dim3(256), 0, s, p, tb);
+    hipLaunchKernelGGL((k_band_bwd_a<GENBMM_BAND_MAX, float>), blocks_for(ta), dim3(256), 0, s, p, ta);
+    hipLaunchKernelGGL((k_band_bwd_b<GENBMM_BAND_MAX, float>), blocks_for(tb), dim3(256), 0, s, p, tb);
   } else {
-    hipLaunchKernelGGL(k_band_bwd_a<GENBMM_BAND_MUL>, blocks_for(ta), dim3(256), 0, s, p, ta);
-    hipLaunchKernelGGL(k_band_bwd_b<GENBMM_BAND_MUL>, blocks_for(tb), dim3(256), 0, s, p, tb);
+    hipLaunchKernelGGL((k_band_bwd_a<GENBMM_BAND_MUL, float>), blocks_for(ta), dim3(256), 0, s, p, ta);
+    hipLaunchKernelGGL((k_band_bwd_b<GENBMM_BAND_MUL, float>), blocks_for(tb), dim3(256), 0, s, p, tb);
   }
   return launch_status();
 }
@@ -346,9 +225,9 @@ int genbmm_banded_bwdbwd(const float* a, int a_lu, int a_ld, const float* b, int
   const long ta = (long)B * n * p.Wa, tb = (long)B * n * p.Wb, to = (long)B * n * p.Wo;
   if (to == 0) return GENBMM_OK;
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(k_band_bb_t, blocks_for(to), dim3(256), 0, s, p, to);
-  hipLaunchKernelGGL(k_band_bb_a, blocks_for(ta), dim3(256), 0, s, p, ta);
-  hipLaunchKernelGGL(k_band_bb_b, blocks_for(tb), dim3(256), 0, s, p, tb);
+  hipLaunchKernelGGL(k_band_bb_t<float>, blocks_for(to), dim3(256), 0, s, p, to);
+  hipLaunchKernelGGL(k_band_bb_a<float>, blocks_for(ta), dim3(256), 0, s, p, ta);
+  hipLaunchKernelGGL(k_band_bb_b<float>, blocks_for(tb), dim3(256), 0, s, p, tb);
   return launch_status();
 }
 

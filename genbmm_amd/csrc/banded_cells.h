@@ -8,17 +8,20 @@
 
 namespace genbmm {
 
-struct BandArgs {
-  const float* a;
-  const float* b;
-  const float* out;
-  const float* g;
-  const float* ua;
-  const float* ub;
+// T: element type of the operands and results (float; double for the fp64 entry
+// points, which run these per-cell kernels only).
+template <class T>
+struct BandArgsT {
+  const T* a;
+  const T* b;
+  const T* out;
+  const T* g;
+  const T* ua;
+  const T* ub;
   const int32_t* idx;
-  float* o0;      // out        | grad_a
-  float* o1;      // -          | grad_b
-  float* o2;      // -          | grad_g
+  T* o0;          // out        | grad_a
+  T* o1;          // -          | grad_b
+  T* o2;          // -          | grad_g
   int32_t* oidx;  // forward argmax
   // log product with a workspace: EA = exp(a - alpha), EB = exp(b - beta) with the
   // row maxima alpha, beta (over cells inside the matrix), and R = 1/S per output
@@ -30,12 +33,21 @@ struct BandArgs {
   float* ws_r;
   int n, a_lu, Wa, b_lu, Wb, r_lu, Wo;
 };
+using BandArgs = BandArgsT<float>;
+
+// exp of a difference and fused multiply-add per element type: float takes the
+// hardware base-2 exponential, double the library routine.
+__device__ __forceinline__ float sr_exp(float x) { return fast_exp(x); }
+__device__ __forceinline__ double sr_exp(double x) { return exp(x); }
+__device__ __forceinline__ float sr_fma(float x, float y, float z) { return __builtin_fmaf(x, y, z); }
+__device__ __forceinline__ double sr_fma(double x, double y, double z) { return __builtin_fma(x, y, z); }
 
 __device__ __forceinline__ int imax3(int a, int b, int c) { return max(a, max(b, c)); }
 __device__ __forceinline__ int imin3(int a, int b, int c) { return min(a, min(b, c)); }
 
 // Valid k range [klo, khi] of output cell (i, j); needs 0 <= o < n.
-__device__ __forceinline__ void k_range(const BandArgs& p, int i, int j, int& klo, int& khi) {
+template <class T>
+__device__ __forceinline__ void k_range(const BandArgsT<T>& p, int i, int j, int& klo, int& khi) {
   klo = imax3(0, j - (p.Wb - 1), p.a_lu - i);
   khi = imin3(p.Wa - 1, j, p.n - 1 + p.a_lu - i);
 }
@@ -43,28 +55,28 @@ __device__ __forceinline__ void k_range(const BandArgs& p, int i, int j, int& kl
 // ------------------------------------------------------------------ forward
 // Reference banded_cuda_forward_kernel_mul (banded_cuda_kernel.cu:13-100).
 // One output cell e = (bi*Wo + j), bi = batch*n + i.
-template <int MODE>
-__device__ __forceinline__ void band_fwd_cell(const BandArgs& p, long bi, int i, int j) {
+template <int MODE, class T>
+__device__ __forceinline__ void band_fwd_cell(const BandArgsT<T>& p, long bi, int i, int j) {
   const long e = bi * p.Wo + j;
   const int o = i + j - p.r_lu;
   if (o < 0 || o >= p.n) {  // outside the matrix: the reference leaves its zero fill
-    p.o0[e] = 0.f;
+    p.o0[e] = 0;
     if (MODE == GENBMM_BAND_MAX) p.oidx[e] = 0;
     return;
   }
   int klo, khi;
   k_range(p, i, j, klo, khi);
-  const float* ar = p.a + bi * p.Wa;
-  const float* br = p.b + (bi + (o - i)) * p.Wb + (p.Wb - 1 - j);  // br[k] = b[o][k2(k)]
+  const T* ar = p.a + bi * p.Wa;
+  const T* br = p.b + (bi + (o - i)) * p.Wb + (p.Wb - 1 - j);  // br[k] = b[o][k2(k)]
   if (MODE == GENBMM_BAND_MUL) {
-    float v = 0.f;
-    for (int k = klo; k <= khi; ++k) v = __builtin_fmaf(ar[k], br[k], v);
+    T v = 0;
+    for (int k = klo; k <= khi; ++k) v = sr_fma(ar[k], br[k], v);
     p.o0[e] = v;
   } else if (MODE == GENBMM_BAND_MAX) {
-    float m = kFloor;
+    T m = kFloor;
     int ind = -1;
     for (int k = klo; k <= khi; ++k) {
-      const float v = ar[k] + br[k];
+      const T v = ar[k] + br[k];
       if (v > m) {
         m = v;
         ind = k;
@@ -72,13 +84,19 @@ __device__ __forceinline__ void band_fwd_cell(const BandArgs& p, long bi, int i,
     }
     p.o0[e] = m;
     p.oidx[e] = ind;
-  } else {
+  } else if constexpr (sizeof(T) == sizeof(float)) {
     float m = kFloor;
     for (int k = klo; k <= khi; ++k) m = fmaxf(m, ar[k] + br[k]);
     const float nm = -m * kLog2e;
     float s = 0.f;
     for (int k = klo; k <= khi; ++k) s += fast_exp2(__builtin_fmaf(ar[k] + br[k], kLog2e, nm));
     p.o0[e] = logf(s) + m;
+  } else {
+    T m = kFloor;
+    for (int k = klo; k <= khi; ++k) m = fmax(m, ar[k] + br[k]);
+    T s = 0;
+    for (int k = klo; k <= khi; ++k) s += exp(ar[k] + br[k] - m);
+    p.o0[e] = log(s) + m;
   }
 }
 
@@ -86,28 +104,28 @@ __device__ __forceinline__ void band_fwd_cell(const BandArgs& p, long bi, int i,
 // d out[i,j] / d a[i,k]: MUL b[o,k2]; LOG exp(a[i,k]+b[o,k2]-out[i,j]);
 // MAX [k == idx[i,j]].  grad_a[i,k] sums over j ascending (reference
 // banded_cuda_backward_kernel_mul, banded_cuda_kernel.cu:104-152).
-template <int MODE>
-__device__ __forceinline__ void band_bwd_a_cell(const BandArgs& p, long bi, int i, int k) {
+template <int MODE, class T>
+__device__ __forceinline__ void band_bwd_a_cell(const BandArgsT<T>& p, long bi, int i, int k) {
   const long e = bi * p.Wa + k;
   const int pos = i + k - p.a_lu;
-  float acc = 0.f;
+  T acc = 0;
   if (pos >= 0 && pos < p.n) {
     const int jlo = imax3(k, p.r_lu - i, 0);
     const int jhi = imin3(k + p.Wb - 1, p.n - 1 + p.r_lu - i, p.Wo - 1);
-    const float* gr = p.g + bi * p.Wo;
+    const T* gr = p.g + bi * p.Wo;
     // b[o][k2] = bw[j * (Wb - 1)] with o = i + j - r_lu, k2 = k - j + Wb - 1
-    const float* bw = p.b + (bi - p.r_lu) * p.Wb + k + p.Wb - 1;
+    const T* bw = p.b + (bi - p.r_lu) * p.Wb + k + p.Wb - 1;
     if (MODE == GENBMM_BAND_MUL) {
-      for (int j = jlo; j <= jhi; ++j) acc = __builtin_fmaf(bw[(long)j * (p.Wb - 1)], gr[j], acc);
+      for (int j = jlo; j <= jhi; ++j) acc = sr_fma(bw[(long)j * (p.Wb - 1)], gr[j], acc);
     } else if (MODE == GENBMM_BAND_MAX) {
       const int32_t* ir = p.idx + bi * p.Wo;
-      for (int j = jlo; j <= jhi; ++j) acc += (ir[j] == k) ? gr[j] : 0.f;
+      for (int j = jlo; j <= jhi; ++j) acc += (ir[j] == k) ? gr[j] : T(0);
     } else {
-      const float av = p.a[e];
-      const float* orow = p.out + bi * p.Wo;
+      const T av = p.a[e];
+      const T* orow = p.out + bi * p.Wo;
       for (int j = jlo; j <= jhi; ++j) {
-        const float w = fast_exp(av + bw[(long)j * (p.Wb - 1)] - orow[j]);
-        acc = __builtin_fmaf(w, gr[j], acc);
+        const T w = sr_exp(av + bw[(long)j * (p.Wb - 1)] - orow[j]);
+        acc = sr_fma(w, gr[j], acc);
       }
     }
   }
@@ -118,33 +136,160 @@ __device__ __forceinline__ void band_bwd_a_cell(const BandArgs& p, long bi, int 
 // read b[o,k2], with k = k2 + j - (Wb - 1).  The reference gets the same
 // numbers by transposing g / out in band form on the host and calling the
 // kernel above with the operands swapped (sparse.py:436-446, 523-545, 625-635).
-template <int MODE>
-__device__ __forceinline__ void band_bwd_b_cell(const BandArgs& p, long bo, int o, int k2) {
+template <int MODE, class T>
+__device__ __forceinline__ void band_bwd_b_cell(const BandArgsT<T>& p, long bo, int o, int k2) {
   const long e = bo * p.Wb + k2;
   const int prow = o + k2 - p.b_lu;
-  float acc = 0.f;
+  T acc = 0;
   if (prow >= 0 && prow < p.n) {
     const int jhi_k = p.Wb - 1 - k2 + p.Wa - 1;  // j with k = Wa-1
     const int jlo_k = p.Wb - 1 - k2;             // j with k = 0
     const int ilo = imax3(0, o + p.r_lu - min(jhi_k, p.Wo - 1), o + p.r_lu - (p.Wo - 1));
     const int ihi = imin3(p.n - 1, o + p.r_lu - max(jlo_k, 0), o + p.r_lu);
     const long base = bo - o;  // batch*n
-    const float bv = p.b[e];
+    const T bv = p.b[e];
     for (int i = ilo; i <= ihi; ++i) {
       const int j = o - i + p.r_lu;
       const int k = k2 + j - (p.Wb - 1);
       const long gi = (base + i) * p.Wo + j;
       if (MODE == GENBMM_BAND_MUL) {
-        acc = __builtin_fmaf(p.a[(base + i) * p.Wa + k], p.g[gi], acc);
+        acc = sr_fma(p.a[(base + i) * p.Wa + k], p.g[gi], acc);
       } else if (MODE == GENBMM_BAND_MAX) {
-        acc += (p.idx[gi] == k) ? p.g[gi] : 0.f;
+        acc += (p.idx[gi] == k) ? p.g[gi] : T(0);
       } else {
-        const float w = fast_exp(p.a[(base + i) * p.Wa + k] + bv - p.out[gi]);
-        acc = __builtin_fmaf(w, p.g[gi], acc);
+        const T w = sr_exp(p.a[(base + i) * p.Wa + k] + bv - p.out[gi]);
+        acc = sr_fma(w, p.g[gi], acc);
       }
     }
   }
   p.o1[e] = acc;
 }
+
+// ------------------------------------------------ one lane per cell kernels
+template <int MODE, class T>
+__global__ __launch_bounds__(256) void k_band_fwd(const BandArgsT<T> p, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const long bi = e / p.Wo;  // batch*n + i
+  band_fwd_cell<MODE>(p, bi, (int)(bi % p.n), (int)(e - bi * p.Wo));
+}
+
+template <int MODE, class T>
+__global__ __launch_bounds__(256) void k_band_bwd_a(const BandArgsT<T> p, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const long bi = e / p.Wa;
+  band_bwd_a_cell<MODE>(p, bi, (int)(bi % p.n), (int)(e - bi * p.Wa));
+}
+
+template <int MODE, class T>
+__global__ __launch_bounds__(256) void k_band_bwd_b(const BandArgsT<T> p, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const long bo = e / p.Wb;
+  band_bwd_b_cell<MODE>(p, bo, (int)(bo % p.n), (int)(e - bo * p.Wb));
+}
+
+// ------------------------------------------------------ log second order
+// p = exp(a[i,k] + b[o,k2] - out[i,j]),  w = u_a[i,k] + u_b[o,k2]:
+//   t[i,j]       = sum_k p*w                        (gradient w.r.t. g)
+//   grad_a[i,k]  = sum_j g[i,j]*p*(w - t[i,j])
+//   grad_b[o,k2] = sum_i g[i,j]*p*(w - t[i,j])
+// With u_b = 0 these equal the reference's banded_cuda_backbackward_kernel_A/
+// _B/_C (banded_cuda_kernel.cu:154-350), whose inner loop sum_m (delta*s -
+// s*s2)*u[m] is s*(u[k] - t).
+template <class T>
+__global__ __launch_bounds__(256) void k_band_bb_t(const BandArgsT<T> p, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int j = (int)(e % p.Wo);
+  const long bi = e / p.Wo;
+  const int i = (int)(bi % p.n);
+  const int o = i + j - p.r_lu;
+  T t = 0;
+  if (o >= 0 && o < p.n) {
+    int klo, khi;
+    k_range(p, i, j, klo, khi);
+    const long boff = (bi + (o - i)) * p.Wb + (p.Wb - 1 - j);
+    const T ov = p.out[e];
+    for (int k = klo; k <= khi; ++k) {
+      const T pr = sr_exp(p.a[bi * p.Wa + k] + p.b[boff + k] - ov);
+      const T w = (p.ua ? p.ua[bi * p.Wa + k] : T(0)) + (p.ub ? p.ub[boff + k] : T(0));
+      t = sr_fma(pr, w, t);
+    }
+  }
+  p.o2[e] = t;
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void k_band_bb_a(const BandArgsT<T> p, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int k = (int)(e % p.Wa);
+  const long bi = e / p.Wa;
+  const int i = (int)(bi % p.n);
+  const int pos = i + k - p.a_lu;
+  T acc = 0;
+  if (pos >= 0 && pos < p.n) {
+    const int jlo = imax3(k, p.r_lu - i, 0);
+    const int jhi = imin3(k + p.Wb - 1, p.n - 1 + p.r_lu - i, p.Wo - 1);
+    const long bw = (bi - p.r_lu) * p.Wb + k + p.Wb - 1;
+    const T av = p.a[e];
+    const T uav = p.ua ? p.ua[e] : T(0);
+    for (int j = jlo; j <= jhi; ++j) {
+      const long bj = bw + (long)j * (p.Wb - 1);
+      const long gi = bi * p.Wo + j;
+      const T pr = sr_exp(av + p.b[bj] - p.out[gi]);
+      const T w = uav + (p.ub ? p.ub[bj] : T(0)) - p.o2[gi];
+      acc = sr_fma(p.g[gi] * pr, w, acc);
+    }
+  }
+  p.o0[e] = acc;
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void k_band_bb_b(const BandArgsT<T> p, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int k2 = (int)(e % p.Wb);
+  const long bo = e / p.Wb;
+  const int o = (int)(bo % p.n);
+  const int prow = o + k2 - p.b_lu;
+  T acc = 0;
+  if (prow >= 0 && prow < p.n) {
+    const int jhi_k = p.Wb - 1 - k2 + p.Wa - 1;
+    const int jlo_k = p.Wb - 1 - k2;
+    const int ilo = imax3(0, o + p.r_lu - min(jhi_k, p.Wo - 1), o + p.r_lu - (p.Wo - 1));
+    const int ihi = imin3(p.n - 1, o + p.r_lu - max(jlo_k, 0), o + p.r_lu);
+    const long base = bo - o;
+    const T bv = p.b[e];
+    const T ubv = p.ub ? p.ub[e] : T(0);
+    for (int i = ilo; i <= ihi; ++i) {
+      const int j = o - i + p.r_lu;
+      const int k = k2 + j - (p.Wb - 1);
+      const long gi = (base + i) * p.Wo + j;
+      const long ai = (base + i) * p.Wa + k;
+      const T pr = sr_exp(p.a[ai] + bv - p.out[gi]);
+      const T w = (p.ua ? p.ua[ai] : T(0)) + ubv - p.o2[gi];
+      acc = sr_fma(p.g[gi] * pr, w, acc);
+    }
+  }
+  p.o1[e] = acc;
+}
+
+// ------------------------------------------------------------------- host
+template <class T>
+inline int fill_band(BandArgsT<T>& p, int a_lu, int a_ld, int b_lu, int b_ld, int B, int n) {
+  if (a_lu < 0 || a_ld < 0 || b_lu < 0 || b_ld < 0) return GENBMM_E_BAND;
+  if (B < 0 || n < 0) return GENBMM_E_SHAPE;
+  const int64_t Wa = (int64_t)a_lu + a_ld + 1, Wb = (int64_t)b_lu + b_ld + 1;
+  const int64_t Wo = Wa + Wb - 1;
+  if (Wo > 0x3fffffff || (int64_t)B * n * Wo > ((int64_t)1 << 40)) return GENBMM_E_SHAPE;
+  p.n = n; p.a_lu = a_lu; p.Wa = (int)Wa; p.b_lu = b_lu; p.Wb = (int)Wb;
+  p.r_lu = a_lu + b_ld; p.Wo = (int)Wo;
+  return GENBMM_OK;
+}
+
+inline dim3 blocks_for(long total) { return dim3((unsigned)((total + 255) / 256)); }
 
 }  // namespace genbmm

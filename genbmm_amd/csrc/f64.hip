@@ -1,0 +1,429 @@
+// Double-precision entry points (gfx950).  The reference instantiates every kernel
+// for double as well (AT_DISPATCH_FLOATING_TYPES_AND_HALF, matmul_cuda_kernel.cu:489
+// and on, banded_cuda_kernel.cu:389 and on).  These are its algorithms in the plain
+// form - one lane per result cell, the reduction axis walked in ascending order,
+// lanes along the contiguous axis so that loads and stores coalesce - without the
+// tiling, factoring and matrix-core work of the float path: double arithmetic runs
+// at half the vector rate and exp / log are software routines, so these kernels are
+// bound by that arithmetic, not by how operands are staged.
+#include "banded_cells.h"
+
+namespace genbmm {
+namespace {
+
+constexpr double kFloorD = -1e9;
+
+enum { kLog = 0, kMax = 1, kSample = 2, kProdMax = 3 };  // the reference's dense modes
+
+// --------------------------------------------------------------- dense forward
+// Reference kernels matmul_cuda_kernel.cu:13-45 (log), :47-75 (max), :77-121
+// (sample), :124-152 (prod-max): two passes (maximum, then sum of exponentials)
+// for the log-sum-exp, strict '>' from -1e9 / index -1 for the arg-max modes.
+template <int MODE>
+__global__ __launch_bounds__(256) void k64_fwd(const double* __restrict__ a,
+                                              const double* __restrict__ b,
+                                              double* __restrict__ out, int32_t* __restrict__ idx,
+                                              uint64_t seed, uint64_t offset, int M, int K, int N,
+                                              long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int n = (int)(e % N);
+  const long bm = e / N;  // batch*M + m
+  const long batch = bm / M;
+  const double* arow = a + bm * K;
+  const double* bcol = b + batch * K * N + n;
+  double m = kFloorD;
+  if (MODE == kMax || MODE == kProdMax) {
+    int ind = -1;
+    for (int k = 0; k < K; ++k) {
+      const double v = MODE == kProdMax ? arow[k] * bcol[(long)k * N] : arow[k] + bcol[(long)k * N];
+      if (v > m) {
+        m = v;
+        ind = k;
+      }
+    }
+    out[e] = m;
+    idx[e] = ind;
+    return;
+  }
+  for (int k = 0; k < K; ++k) {
+    const double v = arow[k] + bcol[(long)k * N];
+    if (v > m) m = v;
+  }
+  double val = 0.0;
+  for (int k = 0; k < K; ++k) val += exp(arow[k] + bcol[(long)k * N] - m);
+  const double o = log(val) + m;
+  out[e] = o;
+  if (MODE == kSample) {
+    // inverse CDF in ascending k (:109-118); index 0 when the walk never brackets r.
+    // One uniform per cell from the same Philox4x32-10 stream as the float path.
+    const double r = (double)philox_uniform((uint64_t)e, seed, offset);
+    double acc = 0.0;
+    int ind = 0;
+    for (int k = 0; k < K; ++k) {
+      const double p = exp(arow[k] + bcol[(long)k * N] - o);
+      if (acc < r && acc + p > r) {
+        ind = k;
+        break;
+      }
+      acc += p;
+    }
+    idx[e] = ind;
+  }
+}
+
+// -------------------------------------------------------------- logbmm backward
+// grad_b[k,n] = sum_m exp(a[m,k] + b[k,n] - out[m,n]) g[m,n]: one lane per cell,
+// lanes along n (reference :190-217, the transposed second call of genmul.py:38-41).
+__global__ __launch_bounds__(256) void k64_log_bwd_b(const double* __restrict__ a,
+                                                    const double* __restrict__ b,
+                                                    const double* __restrict__ out,
+                                                    const double* __restrict__ g,
+                                                    double* __restrict__ grad_b, int M, int K,
+                                                    int N, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int n = (int)(e % N);
+  const long bk = e / N;
+  const long batch = bk / K;
+  const int k = (int)(bk - batch * K);
+  const double bv = b[e];
+  const double* acol = a + batch * M * K + k;
+  const double* ocol = out + batch * M * N + n;
+  const double* gcol = g + batch * M * N + n;
+  double acc = 0.0;
+  for (int m = 0; m < M; ++m)
+    acc = __builtin_fma(exp(acol[(long)m * K] + bv - ocol[(long)m * N]), gcol[(long)m * N], acc);
+  grad_b[e] = acc;
+}
+
+// grad_a[m,k] = sum_n exp(a[m,k] + b[k,n] - out[m,n]) g[m,n] (reference :159-184).
+// One wave per row m: the lanes split n (b, out and g are read along their
+// contiguous axis) and the 64 partial sums are added across the wave per k.
+__global__ __launch_bounds__(256) void k64_log_bwd_a(const double* __restrict__ a,
+                                                    const double* __restrict__ b,
+                                                    const double* __restrict__ out,
+                                                    const double* __restrict__ g,
+                                                    double* __restrict__ grad_a, int M, int K,
+                                                    int N, long rows) {
+  const int lane = threadIdx.x & 63;
+  const long bm = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (bm >= rows) return;  // whole waves leave together
+  const long batch = bm / M;
+  const double* arow = a + bm * K;
+  const double* orow = out + bm * N;
+  const double* grow = g + bm * N;
+  const double* bb = b + batch * K * N;
+  for (int k = 0; k < K; ++k) {
+    const double av = arow[k];
+    double acc = 0.0;
+    for (int n = lane; n < N; n += 64)
+      acc = __builtin_fma(exp(av + bb[(long)k * N + n] - orow[n]), grow[n], acc);
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) acc += __shfl_xor(acc, s, 64);
+    if (lane == 0) grad_a[bm * K + k] = acc;
+  }
+}
+
+// ------------------------------------------------------ logbmm second order
+// Same closed form as the float kernels: with p = exp(a+b-out), w = u_a + u_b,
+//   t = sum_k p w;  grad_a = sum_n g p (w - t);  grad_b = sum_m g p (w - t)
+// (reference :220-331 computes them as quartic loops).
+struct BB64 {
+  const double* a; const double* b; const double* out; const double* g;
+  const double* ua; const double* ub;
+  double* ga; double* gb; double* gg;
+  int M, K, N;
+};
+
+__global__ __launch_bounds__(256) void k64_bb_t(const BB64 p, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int n = (int)(e % p.N);
+  const long bm = e / p.N;
+  const long batch = bm / p.M;
+  const double* arow = p.a + bm * p.K;
+  const double* uarow = p.ua ? p.ua + bm * p.K : nullptr;
+  const double* bcol = p.b + batch * p.K * p.N + n;
+  const double* ubcol = p.ub ? p.ub + batch * p.K * p.N + n : nullptr;
+  const double o = p.out[e];
+  double t = 0.0;
+  for (int k = 0; k < p.K; ++k) {
+    const double pr = exp(arow[k] + bcol[(long)k * p.N] - o);
+    const double w = (uarow ? uarow[k] : 0.0) + (ubcol ? ubcol[(long)k * p.N] : 0.0);
+    t = __builtin_fma(pr, w, t);
+  }
+  p.gg[e] = t;
+}
+
+__global__ __launch_bounds__(256) void k64_bb_a(const BB64 p, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int k = (int)(e % p.K);
+  const long bm = e / p.K;
+  const long batch = bm / p.M;
+  const double av = p.a[e];
+  const double uav = p.ua ? p.ua[e] : 0.0;
+  const double* brow = p.b + (batch * p.K + k) * p.N;
+  const double* ubrow = p.ub ? p.ub + (batch * p.K + k) * p.N : nullptr;
+  const double* orow = p.out + bm * p.N;
+  const double* grow = p.g + bm * p.N;
+  const double* trow = p.gg + bm * p.N;
+  double acc = 0.0;
+  for (int n = 0; n < p.N; ++n) {
+    const double pr = exp(av + brow[n] - orow[n]);
+    const double w = uav + (ubrow ? ubrow[n] : 0.0) - trow[n];
+    acc = __builtin_fma(grow[n] * pr, w, acc);
+  }
+  p.ga[e] = acc;
+}
+
+__global__ __launch_bounds__(256) void k64_bb_b(const BB64 p, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int n = (int)(e % p.N);
+  const long bk = e / p.N;
+  const long batch = bk / p.K;
+  const int k = (int)(bk - batch * p.K);
+  const double bv = p.b[e];
+  const double ubv = p.ub ? p.ub[e] : 0.0;
+  const double* acol = p.a + batch * p.M * p.K + k;
+  const double* uacol = p.ua ? p.ua + batch * p.M * p.K + k : nullptr;
+  const double* ocol = p.out + batch * p.M * p.N + n;
+  const double* gcol = p.g + batch * p.M * p.N + n;
+  const double* tcol = p.gg + batch * p.M * p.N + n;
+  double acc = 0.0;
+  for (int m = 0; m < p.M; ++m) {
+    const long mn = (long)m * p.N;
+    const double pr = exp(acol[(long)m * p.K] + bv - ocol[mn]);
+    const double w = (uacol ? uacol[(long)m * p.K] : 0.0) + ubv - tcol[mn];
+    acc = __builtin_fma(gcol[mn] * pr, w, acc);
+  }
+  p.gb[e] = acc;
+}
+
+// ---------------------------------------------------------- arg-max backward
+// grad_a[m,k] = sum_n [k == idx[m,n]] g[m,n] (* b[k,n]); grad_b[k,n] = sum_m [...]
+// g[m,n] (* a[m,k]): one lane per gradient cell scanning the reduced axis in
+// ascending order, products rounded before the add - the reference's kernels
+// :336-456 as they stand, so the sums are bit-identical to a sequential loop.
+template <bool PROD>
+__global__ __launch_bounds__(256) void k64_argmax_bwd_a(const double* __restrict__ b,
+                                                       const int32_t* __restrict__ idx,
+                                                       const double* __restrict__ g,
+                                                       double* __restrict__ grad_a, int M, int K,
+                                                       int N, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int k = (int)(e % K);
+  const long bm = e / K;
+  const long batch = bm / M;
+  const int32_t* irow = idx + bm * N;
+  const double* grow = g + bm * N;
+  const double* brow = PROD ? b + (batch * K + k) * N : nullptr;
+  double acc = 0.0;
+  for (int n = 0; n < N; ++n)
+    if (irow[n] == k) acc = __dadd_rn(acc, PROD ? __dmul_rn(brow[n], grow[n]) : grow[n]);
+  grad_a[e] = acc;
+}
+
+template <bool PROD>
+__global__ __launch_bounds__(256) void k64_argmax_bwd_b(const double* __restrict__ a,
+                                                       const int32_t* __restrict__ idx,
+                                                       const double* __restrict__ g,
+                                                       double* __restrict__ grad_b, int M, int K,
+                                                       int N, long total) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int n = (int)(e % N);
+  const long bk = e / N;
+  const long batch = bk / K;
+  const int k = (int)(bk - batch * K);
+  const int32_t* icol = idx + batch * M * N + n;
+  const double* gcol = g + batch * M * N + n;
+  const double* acol = PROD ? a + batch * M * K + k : nullptr;
+  double acc = 0.0;
+  for (int m = 0; m < M; ++m)
+    if (icol[(long)m * N] == k)
+      acc = __dadd_rn(acc, PROD ? __dmul_rn(acol[(long)m * K], gcol[(long)m * N]) : gcol[(long)m * N]);
+  grad_b[e] = acc;
+}
+
+// ---------------------------------------------------------------- dispatch
+template <int MODE>
+int run_fwd64(const double* a, const double* b, double* out, int32_t* idx, uint64_t seed,
+              uint64_t offset, int B, int M, int K, int N, void* stream) {
+  if (int e = check_dense_dims(B, M, K, N)) return e;
+  const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
+  if (missing(a, mk) || missing(b, kn) || missing(out, mn) || (MODE != kLog && missing(idx, mn)))
+    return GENBMM_E_NULLPTR;
+  if (mn == 0) return GENBMM_OK;
+  hipLaunchKernelGGL((k64_fwd<MODE>), blocks_for(mn), dim3(256), 0, (hipStream_t)stream, a, b, out,
+                     idx, seed, offset, M, K, N, (long)mn);
+  return launch_status();
+}
+
+template <bool PROD>
+int run_argmax_bwd64(const double* a, const double* b, const int32_t* idx, const double* g,
+                     double* grad_a, double* grad_b, int B, int M, int K, int N, void* stream) {
+  if (int e = check_dense_dims(B, M, K, N)) return e;
+  const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
+  if (missing(idx, mn) || missing(g, mn) || missing(grad_a, mk) || missing(grad_b, kn) ||
+      (PROD && (missing(a, mk) || missing(b, kn))))
+    return GENBMM_E_NULLPTR;
+  hipStream_t s = (hipStream_t)stream;
+  if (mk > 0) hipLaunchKernelGGL((k64_argmax_bwd_a<PROD>), blocks_for(mk), dim3(256), 0, s, b, idx, g,
+                                 grad_a, M, K, N, (long)mk);
+  if (kn > 0) hipLaunchKernelGGL((k64_argmax_bwd_b<PROD>), blocks_for(kn), dim3(256), 0, s, a, idx, g,
+                                 grad_b, M, K, N, (long)kn);
+  return launch_status();
+}
+
+}  // namespace
+}  // namespace genbmm
+
+extern "C" {
+
+int genbmm_logbmm_fwd_f64(const double* a, const double* b, double* out, int B, int M, int K, int N,
+                          void* stream) {
+  return genbmm::run_fwd64<genbmm::kLog>(a, b, out, nullptr, 0, 0, B, M, K, N, stream);
+}
+
+int genbmm_maxbmm_fwd_f64(const double* a, const double* b, double* out, int32_t* idx, int B, int M,
+                          int K, int N, void* stream) {
+  return genbmm::run_fwd64<genbmm::kMax>(a, b, out, idx, 0, 0, B, M, K, N, stream);
+}
+
+int genbmm_prodmaxbmm_fwd_f64(const double* a, const double* b, double* out, int32_t* idx, int B,
+                              int M, int K, int N, void* stream) {
+  return genbmm::run_fwd64<genbmm::kProdMax>(a, b, out, idx, 0, 0, B, M, K, N, stream);
+}
+
+int genbmm_samplebmm_fwd_f64(const double* a, const double* b, double* out, int32_t* idx,
+                             uint64_t seed, uint64_t offset, int B, int M, int K, int N,
+                             void* stream) {
+  return genbmm::run_fwd64<genbmm::kSample>(a, b, out, idx, seed, offset, B, M, K, N, stream);
+}
+
+int genbmm_logbmm_bwd_f64(const double* a, const double* b, const double* out, const double* g,
+                          double* grad_a, double* grad_b, int B, int M, int K, int N,
+                          void* stream) {
+  using namespace genbmm;
+  if (int e = check_dense_dims(B, M, K, N)) return e;
+  const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
+  if (missing(a, mk) || missing(b, kn) || missing(out, mn) || missing(g, mn) ||
+      missing(grad_a, mk) || missing(grad_b, kn))
+    return GENBMM_E_NULLPTR;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t rows = (int64_t)B * M;
+  if (mk > 0) {
+    if ((rows + 3) / 4 > 0x7fffffffLL) return GENBMM_E_SHAPE;
+    hipLaunchKernelGGL(k64_log_bwd_a, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, a, b, out, g,
+                       grad_a, M, K, N, (long)rows);
+  }
+  if (kn > 0)
+    hipLaunchKernelGGL(k64_log_bwd_b, blocks_for(kn), dim3(256), 0, s, a, b, out, g, grad_b, M, K, N,
+                       (long)kn);
+  return launch_status();
+}
+
+int genbmm_logbmm_bwdbwd_f64(const double* a, const double* b, const double* out, const double* g,
+                             const double* u_a, const double* u_b, double* grad_a, double* grad_b,
+                             double* grad_g, int B, int M, int K, int N, void* stream) {
+  using namespace genbmm;
+  if (int e = check_dense_dims(B, M, K, N)) return e;
+  const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
+  if (missing(a, mk) || missing(b, kn) || missing(out, mn) || missing(g, mn) ||
+      missing(grad_a, mk) || missing(grad_b, kn) || missing(grad_g, mn) ||
+      (missing(u_a, mk) && missing(u_b, kn)))
+    return GENBMM_E_NULLPTR;
+  BB64 p{a, b, out, g, u_a, u_b, grad_a, grad_b, grad_g, M, K, N};
+  hipStream_t s = (hipStream_t)stream;
+  if (mn > 0) hipLaunchKernelGGL(k64_bb_t, blocks_for(mn), dim3(256), 0, s, p, (long)mn);
+  if (mk > 0) hipLaunchKernelGGL(k64_bb_a, blocks_for(mk), dim3(256), 0, s, p, (long)mk);
+  if (kn > 0) hipLaunchKernelGGL(k64_bb_b, blocks_for(kn), dim3(256), 0, s, p, (long)kn);
+  return launch_status();
+}
+
+int genbmm_argmax_bwd_f64(const int32_t* idx, const double* g, double* grad_a, double* grad_b, int B,
+                          int M, int K, int N, void* stream) {
+  return genbmm::run_argmax_bwd64<false>(nullptr, nullptr, idx, g, grad_a, grad_b, B, M, K, N,
+                                         stream);
+}
+
+int genbmm_prodmax_bwd_f64(const double* a, const double* b, const int32_t* idx, const double* g,
+                           double* grad_a, double* grad_b, int B, int M, int K, int N,
+                           void* stream) {
+  return genbmm::run_argmax_bwd64<true>(a, b, idx, g, grad_a, grad_b, B, M, K, N, stream);
+}
+
+int genbmm_banded_fwd_f64(const double* a, int a_lu, int a_ld, const double* b, int b_lu, int b_ld,
+                          double* out, int32_t* idx, int B, int n, int mode, void* stream) {
+  using namespace genbmm;
+  if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
+    return GENBMM_E_MODE;
+  BandArgsT<double> p{};
+  if (int e = fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return e;
+  const long total = (long)B * n * p.Wo;
+  if (total == 0) return GENBMM_OK;
+  if (!a || !b || !out || (mode == GENBMM_BAND_MAX && !idx)) return GENBMM_E_NULLPTR;
+  p.a = a; p.b = b; p.o0 = out; p.oidx = idx;
+  hipStream_t s = (hipStream_t)stream;
+  if (mode == GENBMM_BAND_LOG)
+    hipLaunchKernelGGL((k_band_fwd<GENBMM_BAND_LOG, double>), blocks_for(total), dim3(256), 0, s, p, total);
+  else if (mode == GENBMM_BAND_MAX)
+    hipLaunchKernelGGL((k_band_fwd<GENBMM_BAND_MAX, double>), blocks_for(total), dim3(256), 0, s, p, total);
+  else
+    hipLaunchKernelGGL((k_band_fwd<GENBMM_BAND_MUL, double>), blocks_for(total), dim3(256), 0, s, p, total);
+  return launch_status();
+}
+
+int genbmm_banded_bwd_f64(const double* a, int a_lu, int a_ld, const double* b, int b_lu, int b_ld,
+                          const double* out, const int32_t* idx, const double* g, double* grad_a,
+                          double* grad_b, int B, int n, int mode, void* stream) {
+  using namespace genbmm;
+  if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
+    return GENBMM_E_MODE;
+  BandArgsT<double> p{};
+  if (int e = fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return e;
+  if ((int64_t)B * n == 0) return GENBMM_OK;
+  if (!a || !b || !g || !grad_a || !grad_b || (mode == GENBMM_BAND_LOG && !out) ||
+      (mode == GENBMM_BAND_MAX && !idx))
+    return GENBMM_E_NULLPTR;
+  p.a = a; p.b = b; p.out = out; p.idx = idx; p.g = g; p.o0 = grad_a; p.o1 = grad_b;
+  const long ta = (long)B * n * p.Wa, tb = (long)B * n * p.Wb;
+  hipStream_t s = (hipStream_t)stream;
+  if (mode == GENBMM_BAND_LOG) {
+    hipLaunchKernelGGL((k_band_bwd_a<GENBMM_BAND_LOG, double>), blocks_for(ta), dim3(256), 0, s, p, ta);
+    hipLaunchKernelGGL((k_band_bwd_b<GENBMM_BAND_LOG, double>), blocks_for(tb), dim3(256), 0, s, p, tb);
+  } else if (mode == GENBMM_BAND_MAX) {
+    hipLaunchKernelGGL((k_band_bwd_a<GENBMM_BAND_MAX, double>), blocks_for(ta), dim3(256), 0, s, p, ta);
+    hipLaunchKernelGGL((k_band_bwd_b<GENBMM_BAND_MAX, double>), blocks_for(tb), dim3(256), 0, s, p, tb);
+  } else {
+    hipLaunchKernelGGL((k_band_bwd_a<GENBMM_BAND_MUL, double>), blocks_for(ta), dim3(256), 0, s, p, ta);
+    hipLaunchKernelGGL((k_band_bwd_b<GENBMM_BAND_MUL, double>), blocks_for(tb), dim3(256), 0, s, p, tb);
+  }
+  return launch_status();
+}
+
+int genbmm_banded_bwdbwd_f64(const double* a, int a_lu, int a_ld, const double* b, int b_lu,
+                             int b_ld, const double* out, const double* g, const double* u_a,
+                             const double* u_b, double* grad_a, double* grad_b, double* grad_g,
+                             int B, int n, void* stream) {
+  using namespace genbmm;
+  BandArgsT<double> p{};
+  if (int e = fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return e;
+  if ((int64_t)B * n == 0) return GENBMM_OK;
+  if (!a || !b || !out || !g || !grad_a || !grad_b || !grad_g || (!u_a && !u_b))
+    return GENBMM_E_NULLPTR;
+  p.a = a; p.b = b; p.out = out; p.g = g; p.ua = u_a; p.ub = u_b;
+  p.o0 = grad_a; p.o1 = grad_b; p.o2 = grad_g;
+  const long ta = (long)B * n * p.Wa, tb = (long)B * n * p.Wb, to = (long)B * n * p.Wo;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(k_band_bb_t<double>, blocks_for(to), dim3(256), 0, s, p, to);
+  hipLaunchKernelGGL(k_band_bb_a<double>, blocks_for(ta), dim3(256), 0, s, p, ta);
+  hipLaunchKernelGGL(k_band_bb_b<double>, blocks_for(tb), dim3(256), 0, s, p, tb);
+  return launch_status();
+}
+
+}  // extern "C"

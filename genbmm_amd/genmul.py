@@ -20,6 +20,11 @@ Differences in mechanism (not in results):
   * samplebmm draws its uniforms from a counter-based Philox4x32-10 stream
     keyed by torch's CUDA generator seed instead of torch::rand
     (matmul_cuda_kernel.cu:517).
+
+Element types: float32 takes the kernels above; float64 takes the library's
+double-precision entry points (`*_f64`, the reference's algorithms as they stand,
+no workspaces); float16 / bfloat16 are widened to float32 and the result is
+narrowed again.
 """
 import torch
 
@@ -29,8 +34,12 @@ _COMPUTE = torch.float32
 _UPCAST = (torch.float16, torch.bfloat16)
 
 
+def _f64(t):
+    return t.dtype == torch.float64
+
+
 def _prep(a, b):
-    """Validate, and widen half types to the fp32 the kernels compute in."""
+    """Validate, and widen half types to float32; float32 and float64 stay."""
     if not isinstance(a, torch.Tensor) or not isinstance(b, torch.Tensor):
         raise RuntimeError("a and b must be tensors")
     if a.dtype != b.dtype:
@@ -39,9 +48,9 @@ def _prep(a, b):
         _lib.require(a, "a", dtype=a.dtype)
         _lib.require(b, "b", dtype=b.dtype)
         a, b = a.float(), b.float()
-    elif a.dtype != _COMPUTE:
+    elif a.dtype not in (_COMPUTE, torch.float64):
         raise RuntimeError(
-            "genbmm_amd computes in float32; %s inputs are not supported" % a.dtype
+            "genbmm_amd computes in float32 or float64; %s inputs are not supported" % a.dtype
         )
     dims = _lib.dense_dims(a, b)
     return a, b, dims
@@ -66,8 +75,12 @@ class _LogBmmGrad(torch.autograd.Function):
         B, M, K, N = _lib.dense_dims(a, b)
         grad_a = torch.empty_like(a)
         grad_b = torch.empty_like(b)
-        _call("genbmm_logbmm_bwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g),
-              _lib.ptr(stats), _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
+        if _f64(a):
+            _call("genbmm_logbmm_bwd_f64", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g),
+                  _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
+        else:
+            _call("genbmm_logbmm_bwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g),
+                  _lib.ptr(stats), _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
         ctx.save_for_backward(a, b, g, out)
         ctx.set_materialize_grads(False)
         return grad_a, grad_b
@@ -83,8 +96,9 @@ class _LogBmmGrad(torch.autograd.Function):
         ga = torch.empty_like(a)
         gb = torch.empty_like(b)
         gg = torch.empty_like(g)
-        _call("genbmm_logbmm_bwdbwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g),
-              _lib.ptr(u_a), _lib.ptr(u_b), _lib.ptr(ga), _lib.ptr(gb), _lib.ptr(gg), B, M, K, N)
+        _call("genbmm_logbmm_bwdbwd_f64" if _f64(a) else "genbmm_logbmm_bwdbwd", a, _lib.ptr(a),
+              _lib.ptr(b), _lib.ptr(out), _lib.ptr(g), _lib.ptr(u_a), _lib.ptr(u_b), _lib.ptr(ga),
+              _lib.ptr(gb), _lib.ptr(gg), B, M, K, N)
         return ga, gb, gg, None, None
 
 
@@ -95,12 +109,16 @@ class LogMatMul(torch.autograd.Function):
     def forward(ctx, a, b):
         in_dtype = a.dtype if isinstance(a, torch.Tensor) else None
         a, b, (B, M, K, N) = _prep(a, b)
-        out = torch.empty(B, M, N, dtype=_COMPUTE, device=a.device)
-        # the library's workspace: what the reference's `maxes` becomes
-        stats = torch.empty(_lib.load().genbmm_logbmm_stats_size(B, M, K, N), dtype=_COMPUTE,
-                            device=a.device)
-        _call("genbmm_logbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(stats),
-              B, M, K, N)
+        out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)
+        if _f64(a):
+            stats = a.new_empty(0)
+            _call("genbmm_logbmm_fwd_f64", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), B, M, K, N)
+        else:
+            # the library's workspace: what the reference's `maxes` becomes
+            stats = torch.empty(_lib.load().genbmm_logbmm_stats_size(B, M, K, N), dtype=_COMPUTE,
+                                device=a.device)
+            _call("genbmm_logbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(stats),
+                  B, M, K, N)
         ctx.save_for_backward(a, b, out, stats)
         ctx.in_dtype = in_dtype
         return out.to(in_dtype)
@@ -108,21 +126,29 @@ class LogMatMul(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         a, b, out, stats = ctx.saved_tensors
-        grad_a, grad_b = _LogBmmGrad.apply(a, b, grad_output.to(_COMPUTE).contiguous(), out, stats)
+        grad_a, grad_b = _LogBmmGrad.apply(a, b, grad_output.to(a.dtype).contiguous(), out, stats)
         return grad_a.to(ctx.in_dtype), grad_b.to(ctx.in_dtype)
 
 
 # ------------------------------------------------- max / sample / prod-max
 def _argmax_backward(ctx, grad_output, prod):
+    ct = ctx.compute
     if prod:
-        idx, factors = ctx.saved_tensors
+        idx, factors, a, b = ctx.saved_tensors
     else:
-        a, b, idx = ctx.saved_tensors
+        (idx,) = ctx.saved_tensors
     B, M, K, N = ctx.dims
-    g = grad_output.to(_COMPUTE).contiguous()
-    grad_a = torch.empty(B, M, K, dtype=_COMPUTE, device=g.device)
-    grad_b = torch.empty(B, K, N, dtype=_COMPUTE, device=g.device)
-    if prod:
+    g = grad_output.to(ct).contiguous()
+    grad_a = torch.empty(B, M, K, dtype=ct, device=g.device)
+    grad_b = torch.empty(B, K, N, dtype=ct, device=g.device)
+    if ct == torch.float64:
+        if prod:
+            _call("genbmm_prodmax_bwd_f64", g, _lib.ptr(a), _lib.ptr(b), _lib.ptr(idx), _lib.ptr(g),
+                  _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
+        else:
+            _call("genbmm_argmax_bwd_f64", g, _lib.ptr(idx), _lib.ptr(g), _lib.ptr(grad_a),
+                  _lib.ptr(grad_b), B, M, K, N)
+    elif prod:
         # the factors a[m, idx], b[idx, n] were stored by the forward: a and b are not read
         _call("genbmm_prodmax_bwd", g, _lib.ptr(None), _lib.ptr(None), _lib.ptr(idx), _lib.ptr(factors), _lib.ptr(g),
               _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
@@ -140,13 +166,12 @@ class MaxMatMul(torch.autograd.Function):
         in_dtype = a.dtype if isinstance(a, torch.Tensor) else None
         a, b, dims = _prep(a, b)
         B, M, K, N = dims
-        out = torch.empty(B, M, N, dtype=_COMPUTE, device=a.device)
+        out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)
         idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
-        _call("genbmm_maxbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
-              B, M, K, N)
-        empty = a.new_empty(0)
-        ctx.save_for_backward(empty, empty, idx)
-        ctx.dims, ctx.in_dtype = dims, in_dtype
+        _call("genbmm_maxbmm_fwd_f64" if _f64(a) else "genbmm_maxbmm_fwd", a, _lib.ptr(a),
+              _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), B, M, K, N)
+        ctx.save_for_backward(idx)
+        ctx.dims, ctx.in_dtype, ctx.compute = dims, in_dtype, a.dtype
         return out.to(in_dtype)
 
     @staticmethod
@@ -162,13 +187,19 @@ class ProdMaxMatMul(torch.autograd.Function):
         in_dtype = a.dtype if isinstance(a, torch.Tensor) else None
         a, b, dims = _prep(a, b)
         B, M, K, N = dims
-        out = torch.empty(B, M, N, dtype=_COMPUTE, device=a.device)
+        out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)
         idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
-        factors = torch.empty(2, B, M, N, dtype=_COMPUTE, device=a.device)
-        _call("genbmm_prodmaxbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
-              _lib.ptr(factors), B, M, K, N)
-        ctx.save_for_backward(idx, factors)
-        ctx.dims, ctx.in_dtype = dims, in_dtype
+        empty = a.new_empty(0)
+        if _f64(a):
+            _call("genbmm_prodmaxbmm_fwd_f64", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out),
+                  _lib.ptr(idx), B, M, K, N)
+            ctx.save_for_backward(idx, empty, a, b)
+        else:
+            factors = torch.empty(2, B, M, N, dtype=_COMPUTE, device=a.device)
+            _call("genbmm_prodmaxbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
+                  _lib.ptr(factors), B, M, K, N)
+            ctx.save_for_backward(idx, factors, empty, empty)
+        ctx.dims, ctx.in_dtype, ctx.compute = dims, in_dtype, a.dtype
         return out.to(in_dtype)
 
     @staticmethod
@@ -200,16 +231,19 @@ class SampleMatMul(torch.autograd.Function):
         a, b, dims = _prep(a, b)
         B, M, K, N = dims
         seed, offset = _next_stream(a.device) if stream is None else stream
-        out = torch.empty(B, M, N, dtype=_COMPUTE, device=a.device)
+        out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)
         idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
-        stats = torch.empty(_lib.load().genbmm_logbmm_stats_size(B, M, K, N), dtype=_COMPUTE,
-                            device=a.device)
-        _call("genbmm_samplebmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
-              _lib.ptr(stats), int(seed) & 0xFFFFFFFFFFFFFFFF, int(offset) & 0xFFFFFFFFFFFFFFFF,
-              B, M, K, N)
-        empty = a.new_empty(0)
-        ctx.save_for_backward(empty, empty, idx)
-        ctx.dims, ctx.in_dtype = dims, in_dtype
+        seed, offset = int(seed) & 0xFFFFFFFFFFFFFFFF, int(offset) & 0xFFFFFFFFFFFFFFFF
+        if _f64(a):
+            _call("genbmm_samplebmm_fwd_f64", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out),
+                  _lib.ptr(idx), seed, offset, B, M, K, N)
+        else:
+            stats = torch.empty(_lib.load().genbmm_logbmm_stats_size(B, M, K, N), dtype=_COMPUTE,
+                                device=a.device)
+            _call("genbmm_samplebmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
+                  _lib.ptr(stats), seed, offset, B, M, K, N)
+        ctx.save_for_backward(idx)
+        ctx.dims, ctx.in_dtype, ctx.compute = dims, in_dtype, a.dtype
         return out.to(in_dtype)
 
     @staticmethod

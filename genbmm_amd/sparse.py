@@ -295,9 +295,14 @@ class BandedMatrix:
 
 
 # ------------------------------------------------------------------ autograd
+def _f64(t):
+    return t.dtype == torch.float64
+
+
 def _check_pair(a, b):
-    _lib.require(a, "a")
-    _lib.require(b, "b", device=a.device)
+    dtype = torch.float64 if isinstance(a, torch.Tensor) and _f64(a) else torch.float32
+    _lib.require(a, "a", dtype=dtype)
+    _lib.require(b, "b", dtype=dtype, device=a.device)
     if a.shape[:2] != b.shape[:2]:
         raise RuntimeError("banded operands disagree: %s vs %s" % (tuple(a.shape), tuple(b.shape)))
     return a.shape[0], a.shape[1]
@@ -316,8 +321,12 @@ def _forward(a, a_lu, a_ld, b, b_lu, b_ld, mode):
     if a.shape[2] != a_lu + a_ld + 1 or b.shape[2] != b_lu + b_ld + 1:
         raise RuntimeError("band widths do not match lu + ld + 1")
     wo = a.shape[2] + b.shape[2] - 1
-    out = torch.empty(B, n, wo, dtype=torch.float32, device=a.device)
+    out = torch.empty(B, n, wo, dtype=a.dtype, device=a.device)
     idx = torch.empty(B, n, wo, dtype=torch.int32, device=a.device) if mode == MODE_MAX else None
+    if _f64(a):  # the double-precision entry points take no workspace
+        _call("genbmm_banded_fwd_f64", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
+              _lib.ptr(out), _lib.ptr(idx), B, n, mode)
+        return a, b, out, (None if mode == MODE_LOG else idx)
     # log product: the library's workspace (exp(a - max), exp(b - max), maxima, 1/sum),
     # which stands where the reference's `maxes` stands
     ws = None
@@ -332,9 +341,13 @@ def _forward(a, a_lu, a_ld, b, b_lu, b_ld, mode):
 def _backward(a, b, bands, out, idx, g, mode, ws=None):
     a_lu, a_ld, b_lu, b_ld = bands
     B, n = a.shape[0], a.shape[1]
-    g = g.to(torch.float32).contiguous()
+    g = g.to(a.dtype).contiguous()
     grad_a = torch.empty_like(a)
     grad_b = torch.empty_like(b)
+    if _f64(a):
+        _call("genbmm_banded_bwd_f64", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
+              _lib.ptr(out), _lib.ptr(idx), _lib.ptr(g), _lib.ptr(grad_a), _lib.ptr(grad_b), B, n, mode)
+        return grad_a, grad_b
     _call("genbmm_banded_bwd", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
           _lib.ptr(out), _lib.ptr(idx), _lib.ptr(ws), _lib.ptr(g), _lib.ptr(grad_a),
           _lib.ptr(grad_b), B, n, mode)
@@ -384,8 +397,8 @@ class _BandedLogGrad(torch.autograd.Function):
         u_a = None if u_a is None else u_a.contiguous()
         u_b = None if u_b is None else u_b.contiguous()
         ga, gb, gg = torch.empty_like(a), torch.empty_like(b), torch.empty_like(g)
-        _call("genbmm_banded_bwdbwd", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
-              _lib.ptr(out), _lib.ptr(g), _lib.ptr(u_a), _lib.ptr(u_b),
+        _call("genbmm_banded_bwdbwd_f64" if _f64(a) else "genbmm_banded_bwdbwd", a, _lib.ptr(a),
+              a_lu, a_ld, _lib.ptr(b), b_lu, b_ld, _lib.ptr(out), _lib.ptr(g), _lib.ptr(u_a), _lib.ptr(u_b),
               _lib.ptr(ga), _lib.ptr(gb), _lib.ptr(gg), a.shape[0], a.shape[1])
         return ga, gb, gg, None, None, None
 
@@ -403,7 +416,7 @@ class BandedLogMul(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         a, b, out, ws = ctx.saved_tensors
-        g = grad_output.to(torch.float32).contiguous()
+        g = grad_output.to(a.dtype).contiguous()
         grad_a, grad_b = _BandedLogGrad.apply(a, b, g, out, ws, ctx.bands)
         return (grad_a, None, None, grad_b) + (None,) * 4
 

@@ -306,6 +306,57 @@ int genbmm_band_to_dense(const float* data, float* out, int B, int n,
 int genbmm_band_from_dense(const float* dense, float* out, int B, int n_rows,
                            int n, int lu, int ld, void* stream);
 
+/* ------------------------------------------------------- double precision */
+
+/*
+ * The reference instantiates all of its kernels for double as well
+ * (AT_DISPATCH_FLOATING_TYPES_AND_HALF, matmul_cuda_kernel.cu:489 and on,
+ * banded_cuda_kernel.cu:389 and on).  The functions below are the same
+ * operations as their float namesakes above on double buffers, with the same
+ * argument meaning and return codes, minus the float path's workspaces
+ * (stats / factors / workspace): one lane per result cell, the reduction walked
+ * in ascending order as the reference does.  samplebmm draws the same uniform
+ * (24 random bits) per cell as the float function for a given seed and offset.
+ */
+int genbmm_logbmm_fwd_f64(const double* a, const double* b, double* out,
+                          int B, int M, int K, int N, void* stream);
+int genbmm_logbmm_bwd_f64(const double* a, const double* b, const double* out,
+                          const double* g, double* grad_a, double* grad_b,
+                          int B, int M, int K, int N, void* stream);
+int genbmm_logbmm_bwdbwd_f64(const double* a, const double* b, const double* out,
+                             const double* g, const double* u_a, const double* u_b,
+                             double* grad_a, double* grad_b, double* grad_g,
+                             int B, int M, int K, int N, void* stream);
+int genbmm_maxbmm_fwd_f64(const double* a, const double* b, double* out,
+                          int32_t* idx, int B, int M, int K, int N, void* stream);
+int genbmm_prodmaxbmm_fwd_f64(const double* a, const double* b, double* out,
+                              int32_t* idx, int B, int M, int K, int N,
+                              void* stream);
+int genbmm_samplebmm_fwd_f64(const double* a, const double* b, double* out,
+                             int32_t* idx, uint64_t seed, uint64_t offset,
+                             int B, int M, int K, int N, void* stream);
+int genbmm_argmax_bwd_f64(const int32_t* idx, const double* g, double* grad_a,
+                          double* grad_b, int B, int M, int K, int N,
+                          void* stream);
+int genbmm_prodmax_bwd_f64(const double* a, const double* b, const int32_t* idx,
+                           const double* g, double* grad_a, double* grad_b,
+                           int B, int M, int K, int N, void* stream);
+int genbmm_banded_fwd_f64(const double* a, int a_lu, int a_ld,
+                          const double* b, int b_lu, int b_ld,
+                          double* out, int32_t* idx,
+                          int B, int n, int mode, void* stream);
+int genbmm_banded_bwd_f64(const double* a, int a_lu, int a_ld,
+                          const double* b, int b_lu, int b_ld,
+                          const double* out, const int32_t* idx, const double* g,
+                          double* grad_a, double* grad_b,
+                          int B, int n, int mode, void* stream);
+int genbmm_banded_bwdbwd_f64(const double* a, int a_lu, int a_ld,
+                             const double* b, int b_lu, int b_ld,
+                             const double* out, const double* g,
+                             const double* u_a, const double* u_b,
+                             double* grad_a, double* grad_b, double* grad_g,
+                             int B, int n, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

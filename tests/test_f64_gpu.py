@@ -1,0 +1,178 @@
+"""GPU parity of the double-precision entry points (`*_f64`) against the CPU oracle's
+double instantiation of the reference kernels, through the public API and the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import genbmm_amd as genbmm
+from genbmm_amd import _lib
+from genbmm_amd.sparse import BandedMatrix, banddiag
+
+pytestmark = pytest.mark.gpu
+F64 = np.float64
+SHAPES = [(3, 9, 12, 7), (2, 33, 70, 129), (4, 64, 64, 64), (2, 1, 1, 1), (1, 130, 5, 66)]
+
+
+def close(x, ref, rtol=1e-12, atol=1e-12):
+    x, ref = x.detach().cpu(), ref.detach().cpu()
+    assert x.dtype == torch.float64 and ref.dtype == torch.float64
+    assert torch.allclose(x, ref, rtol=rtol, atol=atol), float((x - ref).abs().max())
+
+
+def grid(*shape):
+    return (torch.round(torch.randn(*shape) * 8) / 8).double()
+
+
+@pytest.mark.parametrize("B,M,K,N", SHAPES)
+def test_logbmm_f64(gpu, B, M, K, N):
+    torch.manual_seed(K)
+    a, b, g = torch.randn(B, M, K).double() * 3, torch.randn(B, K, N).double() * 3, torch.randn(B, M, N).double()
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    out = genbmm.logbmm(ad, bd)
+    assert out.dtype == torch.float64
+    close(out, oracle.seq_logbmm_fwd(a, b, dtype=F64)[0])
+    close(out, oracle.logbmm_broadcast(a, b))
+    ga, gb = torch.autograd.grad(out, (ad, bd), g.to(gpu), create_graph=True)
+    wa, wb = oracle.seq_logbmm_bwd(a, b, g, dtype=F64)
+    close(ga, wa)
+    close(gb, wb)
+    _, wa64, wb64 = oracle.logbmm_grads64(a, b, g)
+    close(ga, wa64, 1e-10, 1e-12)
+    close(gb, wb64, 1e-10, 1e-12)
+    # second order: gradients of <u_a, grad_a> + <u_b, grad_b>
+    ua, ub = torch.randn(B, M, K).double(), torch.randn(B, K, N).double()
+    got = torch.autograd.grad((ga * ua.to(gpu)).sum() + (gb * ub.to(gpu)).sum(), (ad, bd))
+    want = oracle.logbmm_second_order64(a, b, g, ua, ub)
+    close(got[0], want[0], 1e-9, 1e-11)
+    close(got[1], want[1], 1e-9, 1e-11)
+
+
+def test_logbmm_f64_special_values(gpu):
+    a = torch.tensor([[[0.0, -1e9, float("-inf")], [5.0, 5.0, 5.0]]], dtype=torch.float64)
+    b = torch.zeros(1, 3, 2, dtype=torch.float64)
+    out = genbmm.logbmm(a.to(gpu), b.to(gpu)).cpu()
+    assert torch.allclose(out[0, 0], torch.zeros(2, dtype=torch.float64), atol=1e-15)
+    assert torch.allclose(out[0, 1], torch.full((2,), 5 + np.log(3.0), dtype=torch.float64), rtol=1e-15)
+    # a term float32 loses: log(1 + e^-30) = 9.36e-14, within the rounding of 1 + e^-30
+    tiny = torch.tensor([[[0.0, -30.0]]], dtype=torch.float64)
+    got = genbmm.logbmm(tiny.to(gpu), torch.zeros(1, 2, 1, dtype=torch.float64, device=gpu)).item()
+    assert abs(got - np.log1p(np.exp(-30.0))) < 3e-16 and got != 0.0
+
+
+@pytest.mark.parametrize("B,M,K,N", SHAPES)
+@pytest.mark.parametrize("prod", [False, True])
+def test_max_f64_bit_exact(gpu, B, M, K, N, prod):
+    torch.manual_seed(M + N)
+    if prod:
+        a, b = (1 - torch.rand(B, M, K)).double(), (1 - torch.rand(B, K, N)).double()
+        a[:, :, ::3] = torch.round(a[:, :, ::3] * 4) / 4 + 0.25
+        b[:, ::3, :] = torch.round(b[:, ::3, :] * 4) / 4 + 0.25
+        op = genbmm.prodmaxbmm
+    else:
+        a, b = grid(B, M, K), grid(B, K, N)
+        op = genbmm.maxbmm
+    g = grid(B, M, N).clamp(-4, 4)
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    out = op(ad, bd)
+    sv, si = oracle.seq_maxbmm_fwd(a, b, prod, dtype=F64)
+    assert out.dtype == torch.float64 and torch.equal(out.detach().cpu(), sv)
+    ga, gb = torch.autograd.grad(out, (ad, bd), g.to(gpu))
+    wa, wb = oracle.seq_argmax_bwd(a if prod else K, b, si, g, prod, dtype=F64)
+    assert torch.equal(ga.cpu(), wa) and torch.equal(gb.cpu(), wb)
+    # index through the C ABI
+    lib = _lib.load()
+    o2 = torch.empty(B, M, N, dtype=torch.float64, device=gpu)
+    i2 = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
+    fn = lib.genbmm_prodmaxbmm_fwd_f64 if prod else lib.genbmm_maxbmm_fwd_f64
+    assert fn(_lib.ptr(ad.detach()), _lib.ptr(bd.detach()), _lib.ptr(o2), _lib.ptr(i2), B, M, K, N,
+              _lib.stream_of(o2)) == 0
+    assert torch.equal(i2.cpu(), si) and torch.equal(o2.cpu(), sv)
+
+
+def test_sample_f64_follows_the_cdf_rule(gpu):
+    """Index = the reference's walk (matmul_cuda_kernel.cu:109-118) on the uniform of the
+    cell, which is the float path's Philox draw for the same seed and offset."""
+    torch.manual_seed(4)
+    B, M, K, N = 3, 20, 37, 24
+    a, b = torch.randn(B, M, K).double() * 2, torch.randn(B, K, N).double() * 2
+    seed, offset = 1234, 8
+    lib = _lib.load()
+    ad, bd = a.to(gpu), b.to(gpu)
+    out = torch.empty(B, M, N, dtype=torch.float64, device=gpu)
+    idx = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
+    assert lib.genbmm_samplebmm_fwd_f64(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx), seed, offset,
+                                        B, M, K, N, _lib.stream_of(ad)) == 0
+    close(out, oracle.logbmm_broadcast(a, b))
+    u = oracle.philox_uniform(0, B * M * N, seed, offset).view(B, M, N).double()
+    sv, si = oracle.seq_samplebmm_fwd(a, b, u, dtype=F64)
+    got = idx.cpu()
+    # exp() of the device library and the host's differ in the last bits: a draw within
+    # that distance of a CDF step may land on the neighbouring index
+    assert float((got != si).float().mean()) < 1e-3
+    cdf = oracle.sample_cdf64(a, b)
+    gl = got.long()
+    hi = torch.gather(cdf, 2, gl.unsqueeze(2)).squeeze(2)
+    lo = torch.where(gl > 0, torch.gather(cdf, 2, (gl - 1).clamp(min=0).unsqueeze(2)).squeeze(2), torch.zeros_like(hi))
+    assert bool(((lo - 1e-12 <= u) & (u <= hi + 1e-12)).all())
+    # the float entry point draws the same uniforms: same index wherever float rounding allows
+    o32 = torch.empty(B, M, N, device=gpu)
+    i32 = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
+    assert lib.genbmm_samplebmm_fwd(_lib.ptr(ad.float()), _lib.ptr(bd.float()), _lib.ptr(o32), _lib.ptr(i32),
+                                    _lib.ptr(None), seed, offset, B, M, K, N, _lib.stream_of(ad)) == 0
+    assert float((i32.cpu() != got).float().mean()) < 5e-3
+    # through autograd: the gradient is the one-hot of the index times g
+    ar, br = ad.clone().requires_grad_(True), bd.clone().requires_grad_(True)
+    o = genbmm.samplebmm(ar, br, (seed, offset))
+    g = torch.randn(B, M, N).double()
+    ga, gb = torch.autograd.grad(o, (ar, br), g.to(gpu))
+    onehot = torch.nn.functional.one_hot(got.long(), K).double()          # (B, M, N, K)
+    assert torch.allclose(ga.cpu(), (onehot * g.unsqueeze(-1)).sum(2), rtol=1e-12, atol=1e-12)
+    assert torch.allclose(gb.cpu().sum(1), g.sum(1), rtol=1e-12, atol=1e-12)
+
+
+BANDS = [(5, 1, 1, 2, 0), (7, 0, 2, 2, 0), (3, 4, 5, 5, 4), (40, 3, 5, 4, 2), (130, 17, 2, 5, 20)]
+
+
+@pytest.mark.parametrize("n,a_lu,a_ld,b_lu,b_ld", BANDS)
+@pytest.mark.parametrize("mode", [0, 1, 3])
+def test_banded_f64(gpu, n, a_lu, a_ld, b_lu, b_ld, mode):
+    torch.manual_seed(n + mode)
+    exact = mode == 1
+    mk = grid if exact else (lambda *s: torch.randn(*s).double())
+    a = banddiag(mk(3, n, n), a_lu, a_ld)[0].contiguous()
+    b = banddiag(mk(3, n, n), b_lu, b_ld)[0].contiguous()
+    W = a.shape[2] + b.shape[2] - 1
+    g = grid(3, n, W).clamp(-4, 4) if exact else torch.randn(3, n, W).double()
+    X = BandedMatrix(a.to(gpu).requires_grad_(True), a_lu, a_ld)
+    Y = BandedMatrix(b.to(gpu).requires_grad_(True), b_lu, b_ld)
+    res = {0: X.multiply_log, 1: X.multiply_max, 3: X.multiply}[mode](Y)
+    assert res.data.dtype == torch.float64
+    want, widx, _ = oracle.seq_band_fwd(a, a_lu, a_ld, b, b_lu, b_ld, mode, dtype=F64)
+    if exact:
+        assert torch.equal(res.data.detach().cpu(), want)
+    else:
+        close(res.data, want, 1e-12, 1e-12)
+    ga, gb = torch.autograd.grad(res.data, (X.data, Y.data), g.to(gpu), create_graph=(mode == 0))
+    wa, wb = oracle.seq_band_bwd(a, a_lu, a_ld, b, b_lu, b_ld, g, mode, dtype=F64)
+    if exact:
+        assert torch.equal(ga.cpu(), wa) and torch.equal(gb.cpu(), wb)
+    else:
+        close(ga, wa, 1e-11, 1e-12)
+        close(gb, wb, 1e-11, 1e-12)
+    if mode == 0 and n <= 40:
+        u = torch.randn_like(a)
+        got = torch.autograd.grad((ga * u.to(gpu)).sum(), (X.data, Y.data))
+        want = oracle.seq_band_bwdbwd(a, a_lu, a_ld, b, b_lu, b_ld, g, u, dtype=F64)
+        close(got[0], want[0], 1e-10, 1e-11)
+        close(got[1], want[1], 1e-10, 1e-11)
+
+
+def test_f64_and_f32_disagree_only_by_float_rounding(gpu):
+    torch.manual_seed(0)
+    a, b = torch.randn(4, 64, 96), torch.randn(4, 96, 80)
+    o32 = genbmm.logbmm(a.to(gpu), b.to(gpu)).double().cpu()
+    o64 = genbmm.logbmm(a.double().to(gpu), b.double().to(gpu)).cpu()
+    assert torch.allclose(o32, o64, rtol=1e-5, atol=1e-5) and not torch.equal(o32, o64)
+    with pytest.raises(RuntimeError):
+        genbmm.logbmm(a.double().to(gpu), b.to(gpu))
