@@ -230,6 +230,32 @@ def band_structure(lib, dev, B, n, lu, ld, reps):
     line("banddiag", ms, 4.0 * Bd * n * 2 * W)
 
 
+def dense_f64(lib, dev, B, M, K, N, reps):
+    """logbmm / maxbmm forward + backward on the double-precision entry points (plain
+    kernels: the figure of merit is % of the FP64 vector peak, 78.6 TFLOP/s)."""
+    torch.manual_seed(0)
+    a, b, g = (torch.randn(B, M, K).double().to(dev), torch.randn(B, K, N).double().to(dev),
+               torch.randn(B, M, N).double().to(dev))
+    out = torch.empty(B, M, N, dtype=torch.float64, device=dev)
+    idx = torch.empty(B, M, N, dtype=torch.int32, device=dev)
+    ga, gb = torch.empty_like(a), torch.empty_like(b)
+    s, p = _lib.stream_of(a), _lib.ptr
+    bmkn = float(B) * M * K * N
+    for name, f, bw in (
+        ("logbmm", lambda: lib.genbmm_logbmm_fwd_f64(p(a), p(b), p(out), B, M, K, N, s),
+         lambda: lib.genbmm_logbmm_bwd_f64(p(a), p(b), p(out), p(g), p(ga), p(gb), B, M, K, N, s)),
+        ("maxbmm", lambda: lib.genbmm_maxbmm_fwd_f64(p(a), p(b), p(out), p(idx), B, M, K, N, s),
+         lambda: lib.genbmm_argmax_bwd_f64(p(idx), p(g), p(ga), p(gb), B, M, K, N, s)),
+    ):
+        mf = timed(lambda: _lib.check(f(), "fwd"), reps)
+        mb = timed(lambda: _lib.check(bw(), "bwd"), reps)
+        ms = mf + mb
+        print(json.dumps({"config": "%s f64 fwd+bwd (%d,%d,%d,%d)" % (name, B, M, K, N), "ms": round(ms, 4),
+                          "semiring_GOPs": round(6 * bmkn / ms / 1e6, 1),
+                          "pct_fp64_vector_peak": round(100 * 6 * bmkn / (ms * 1e-3) / 78.6e12, 2),
+                          "ms_fwd": round(mf, 4), "ms_bwd": round(mb, 4)}), flush=True)
+
+
 def cpu_c1():
     import oracle
 
@@ -258,9 +284,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--cpu", action="store_true")
-    ap.add_argument("--only", default="", help="comma-separated subset: log,max,sample,banded,struct")
+    ap.add_argument("--only", default="", help="comma-separated subset: log,max,sample,banded,struct,f64")
     args = ap.parse_args()
-    want = set(args.only.split(",")) if args.only else {"log", "max", "sample", "banded", "struct"}
+    want = set(args.only.split(",")) if args.only else {"log", "max", "sample", "banded", "struct", "f64"}
     lib = _lib.load()
     dev = torch.device("cuda:0")
     r = args.reps
@@ -280,6 +306,8 @@ def main():
             banded(lib, dev, 64, 4096, 32, 32, mode, r)
     if "struct" in want:
         band_structure(lib, dev, 64, 4096, 32, 32, r)
+    if "f64" in want:
+        dense_f64(lib, dev, 512, 128, 128, 128, max(3, r // 4))
     if args.cpu:
         cpu_c1()
 
