@@ -501,8 +501,10 @@ def test_errors(gpu):
             op(a.to(gpu).transpose(1, 2).contiguous().transpose(1, 2), b.to(gpu))  # :66
         with pytest.raises(RuntimeError, match="shape mismatch"):
             op(a.to(gpu), torch.randn(2, 3, 5, device=gpu))
-        with pytest.raises(RuntimeError, match="float32"):
-            op(a.to(gpu).double(), b.to(gpu).double())
+        with pytest.raises(RuntimeError, match="same dtype"):
+            op(a.to(gpu).double(), b.to(gpu))
+        with pytest.raises(RuntimeError, match="not supported"):
+            op(a.to(gpu).long(), b.to(gpu).long())
     lib = _lib.load()
     null = ctypes.c_void_p(0)
     ad = a.to(gpu)
