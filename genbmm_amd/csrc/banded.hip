@@ -29,9 +29,9 @@ namespace {
 constexpr size_t kStripLdsLimit = 64 * 1024;  // dynamic LDS available without opting in
 
 // Workspace of the log product: EA (B*n*Wa), EB (B*n*Wb), alpha (B*n), beta (B*n),
-// R (B*n*Wo) floats.
+// R (B*n*Wo) floats from the forward, and H (B*n*Wo) that the backward fills.
 inline size_t band_ws_floats(const BandArgs& p, int B) {
-  return (size_t)B * p.n * ((size_t)p.Wa + p.Wb + p.Wo + 2);
+  return (size_t)B * p.n * ((size_t)p.Wa + p.Wb + 2 * (size_t)p.Wo + 2);
 }
 // Which bands the strip kernels take (forward / backward): tiles within 64 KB of
 // LDS, the sliding tile large enough to double as the output staging tiles.
@@ -64,6 +64,7 @@ inline void set_workspace(BandArgs& p, float* ws, int B) {
   p.ws_al = p.ws_eb + rows * p.Wb;
   p.ws_be = p.ws_al + rows;
   p.ws_r = p.ws_be + rows;
+  p.ws_h = p.ws_r + rows * p.Wo;
 }
 
 }  // namespace
@@ -135,7 +136,7 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
 }
 
 int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
-                      const float* out, const int32_t* idx, const float* workspace, const float* g,
+                      const float* out, const int32_t* idx, float* workspace, const float* g,
                       float* grad_a, float* grad_b, int B, int n, int mode, void* stream) {
   using namespace genbmm;
   if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
@@ -159,7 +160,11 @@ int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_
       const dim3 grid((unsigned)((long)B * strips));
       const int nq = ceil_div(max(max(da.ld_own, da.ld_sl), max(db.ld_own, db.ld_sl)), 64);
       if (lg && workspace && workspace_used(p)) {  // on the forward's workspace: a (+,x) backward plus epilogue
-        set_workspace(p, const_cast<float*>(workspace), B);
+        set_workspace(p, workspace, B);
+        // H = g * R once for both gradients (NaN marks a cell whose R is not usable)
+        const long cells = (long)B * n * p.Wo;
+        hipLaunchKernelGGL(k_band_h, dim3((unsigned)min((cells + 1023) / 1024, (long)0x7fffffff)),
+                           dim3(256), 0, s, g, p.ws_r, p.ws_h, cells);
         if (nq <= 1) {
           hipLaunchKernelGGL((k_band_bwd_strip<false, true, 1, true>), grid, dim3(256), na, s, p, strips, da.ld_own, da.ld_sl, bwd_sl_floats(da));
           hipLaunchKernelGGL((k_band_bwd_strip<false, false, 1, true>), grid, dim3(256), nb, s, p, strips, db.ld_own, db.ld_sl, bwd_sl_floats(db));

@@ -31,6 +31,7 @@ struct BandArgsT {
   float* ws_al;
   float* ws_be;
   float* ws_r;
+  float* ws_h;    // backward scratch: g * R per output cell (NaN where R is not usable)
   int n, a_lu, Wa, b_lu, Wb, r_lu, Wo;
 };
 using BandArgs = BandArgsT<float>;

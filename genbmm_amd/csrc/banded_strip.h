@@ -374,26 +374,8 @@ struct GStage {
       const bool inside = r < ROWS && i >= 0 && i < n && j < Wo && o >= 0 && o < n;
       const bool use = inside && (GRAD_A || (o >= x0 && o < x0 + kBT));
       gv[u] = use ? gb[(long)i * Wo + j] : 0.f;
-      ov[u] = ((LOG || PREP) && use) ? ob[(long)i * Wo + j] : 0.f;  // out, or 1/S of the workspace
+      ov[u] = (LOG && use) ? ob[(long)i * Wo + j] : 0.f;
       used |= (use ? 1u : 0u) << u;
-    }
-  }
-
-  // gv holds 1/S (or -1: not usable, the row this cell feeds is redone) of the cells
-  // whose g' the same thread has just stored: g' *= 1/S
-  __device__ __forceinline__ void scale(float* __restrict__ gt, int* __restrict__ badrow, int x0,
-                                        int yb, int jc, int r_lu, int tid) const {
-#pragma unroll
-    for (int u = 0; u < PER; ++u) {
-      const int e = tid + 256 * u, r = e >> 5, c = e & 31;
-      if (r >= ROWS || !((used >> u) & 1u)) continue;
-      if (gv[u] < 0.f) {
-        const int o = (GRAD_A ? x0 + r : yb + r) + jc + c - r_lu;
-        badrow[GRAD_A ? r : o - x0] = 1;
-        gt[r * kBC + c] = 0.f;
-      } else {
-        gt[r * kBC + c] *= gv[u];
-      }
     }
   }
 
@@ -406,14 +388,10 @@ struct GStage {
       const int e = tid + 256 * u, r = e >> 5, c = e & 31;
       if (r >= ROWS) continue;
       float v = gv[u];
-      if (PREP && ((used >> u) & 1u)) {
+      if (PREP && v != v) {  // H is NaN: the cell's 1/S is not usable (or g is NaN), the row is redone
         const int o = (GRAD_A ? x0 + r : yb + r) + jc + c - r_lu;
-        if (ov[u] < 0.f) {  // the cell was computed exactly: 1/S not usable, the row is redone
-          badrow[GRAD_A ? r : o - x0] = 1;
-          v = 0.f;
-        } else {
-          v *= ov[u];
-        }
+        badrow[GRAD_A ? r : o - x0] = 1;
+        v = 0.f;
       }
       if (LOG && ((used >> u) & 1u)) {
         const int o = (GRAD_A ? x0 + r : yb + r) + jc + c - r_lu;
@@ -431,11 +409,30 @@ struct GStage {
 
 constexpr int kMaxKB = 3;  // band-axis blocks of 8 per wave: widths up to 96
 
+// H = g * R for the prepared log backward, once for both gradients; R < 0 marks a
+// cell that the forward computed exactly (its 1/S is not usable): NaN there, which
+// the gradient kernels turn into "redo this row exactly".
+__global__ __launch_bounds__(256) void k_band_h(const float* __restrict__ g,
+                                               const float* __restrict__ r,
+                                               float* __restrict__ h, long cells) {
+  const long stride = (long)gridDim.x * 1024;
+  for (long e = (long)blockIdx.x * 1024 + threadIdx.x; e < cells; e += stride) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const long i = e + 256 * u;
+      if (i < cells) {
+        const float rv = r[i];
+        h[i] = rv < 0.f ? __builtin_nanf("") : g[i] * rv;
+      }
+    }
+  }
+}
+
 // PREP (with LOG = false): the log product on the forward's workspace - operands
-// EA / EB staged like a (+,x) product, g' = g * R, result times the own operand's
-// EA / EB; rows fed by a cell whose R is marked unusable are recomputed exactly.
+// EA / EB staged like a (+,x) product, g' = H = g * R from k_band_h, result times
+// the own operand's EA / EB; rows fed by a cell whose H is NaN are recomputed exactly.
 template <bool LOG, bool GRAD_A, int NQ, bool PREP = false>
-__global__ __launch_bounds__(256, (PREP && !GRAD_A) ? 2 : 3) void k_band_bwd_strip(const BandArgs p, int strips, int ld_own,
+__global__ __launch_bounds__(256, 3) void k_band_bwd_strip(const BandArgs p, int strips, int ld_own,
                                                            int ld_sl, int sl_floats) {
   static_assert(!(LOG && PREP), "");
   extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -457,8 +454,8 @@ __global__ __launch_bounds__(256, (PREP && !GRAD_A) ? 2 : 3) void k_band_bwd_str
   const long bn = (long)batch * n;
   const float* ab = (PREP ? p.ws_ea : p.a) + bn * Wa;
   const float* bb = (PREP ? p.ws_eb : p.b) + bn * Wb;
-  const float* gb = p.g + bn * Wo;
-  const float* ob = LOG ? p.out + bn * Wo : (PREP ? p.ws_r + bn * Wo : nullptr);
+  const float* gb = (PREP ? p.ws_h : p.g) + bn * Wo;  // PREP: H = g / S, staged once for both gradients
+  const float* ob = LOG ? p.out + bn * Wo : nullptr;
   // output operand / other operand
   const float* xo = GRAD_A ? ab : bb;
   const float* yo = GRAD_A ? bb : ab;
@@ -493,14 +490,7 @@ __global__ __launch_bounds__(256, (PREP && !GRAD_A) ? 2 : 3) void k_band_bwd_str
     // ---- g' tile.  (Starting these reads one chunk ahead, like the operand rows,
     // measured slower: the extra live registers cost more than the latency.)
     // The log kernels are short of registers: they go element by element.
-    if (PREP) {
-      // two passes over the same cells (g, then 1/S) keep half as many values live
-      GStage<false, GRAD_A> gs;
-      gs.load(gb, nullptr, x0, yb, jc, n, Wo, p.r_lu, tid);
-      gs.store(gt, sh_own, sh_sl, badrow, x0, yb, jc, p.r_lu, lim, tid);
-      gs.load(ob, nullptr, x0, yb, jc, n, Wo, p.r_lu, tid);
-      gs.scale(gt, badrow, x0, yb, jc, p.r_lu, tid);
-    } else if (LOG) {
+    if (LOG) {
       for (int e = tid; e < GStage<LOG, GRAD_A>::ROWS * kBJ; e += 256) {
         const int r = e >> 5, c = e & 31, j = jc + c;
         const int i = GRAD_A ? x0 + r : yb + r;
@@ -517,7 +507,7 @@ __global__ __launch_bounds__(256, (PREP && !GRAD_A) ? 2 : 3) void k_band_bwd_str
         gt[r * kBC + c] = v;
       }
     } else {
-      GStage<LOG, GRAD_A> gs;
+      GStage<LOG, GRAD_A, PREP> gs;
       gs.load(gb, ob, x0, yb, jc, n, Wo, p.r_lu, tid);
       gs.store(gt, sh_own, sh_sl, badrow, x0, yb, jc, p.r_lu, lim, tid);
     }
@@ -562,7 +552,20 @@ __global__ __launch_bounds__(256, (PREP && !GRAD_A) ? 2 : 3) void k_band_bwd_str
     }
   }
 
-  // ---- epilogue: grad = (LOG ? exp(x - shift) : 1) * acc, staged for row-wise stores
+  // ---- epilogue: grad = (LOG ? exp(x - shift) : PREP ? EX : 1) * acc, staged for row-wise
+  // stores.  The own operand's rows are requested before the tile is staged, all at
+  // once: read row by row inside the store loop, each wave would wait sixteen times.
+  constexpr int kRowsPerWave = kBT / 4;
+  float xv[(LOG || PREP) ? kRowsPerWave : 1][(LOG || PREP) ? NQ : 1];
+  if (LOG || PREP) {
+#pragma unroll
+    for (int rr = 0; rr < kRowsPerWave; ++rr)
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        const int x = x0 + wave + 4 * rr, k = lane + 64 * q;
+        xv[rr][q] = (x < n && k < Wx) ? xo[(long)x * Wx + k] : 0.f;
+      }
+  }
   __syncthreads();
   float* ct = sl;  // [64][ld_own]
 #pragma unroll
@@ -575,28 +578,34 @@ __global__ __launch_bounds__(256, (PREP && !GRAD_A) ? 2 : 3) void k_band_bwd_str
         ct[lane * ld_own + k0 + t] = acc[q][t];
   }
   __syncthreads();
-  for (int r = wave; r < kBT; r += 4) {
-    const int x = x0 + r;
+#pragma unroll
+  for (int rr = 0; rr < kRowsPerWave; ++rr) {
+    const int r = wave + 4 * rr, x = x0 + r;
     if (x >= n) break;
     if ((LOG || PREP) && badrow[r]) {  // recompute this row cell by cell from memory
       for (int k = lane; k < Wx; k += 64) {
         if (GRAD_A) band_bwd_a_cell<GENBMM_BAND_LOG>(p, bn + x, x, k);
         else band_bwd_b_cell<GENBMM_BAND_LOG>(p, bn + x, x, k);
       }
-    } else {
-      if (LOG) {
-        const float sh = sh_own[r] == -INFINITY ? 0.f : sh_own[r];
-        for (int k = lane; k < Wx; k += 64) {
-          // exp(x - shift); cells outside the matrix are excluded from the row maximum
-          // and their sum is 0
-          const float acv = ct[r * ld_own + k];
-          gradb[(long)x * Wx + k] = acv == 0.f ? 0.f : fast_exp2((xo[(long)x * Wx + k] - sh) * kLog2e) * acv;
-        }
-      } else if (PREP) {
-        for (int k = lane; k < Wx; k += 64) gradb[(long)x * Wx + k] = xo[(long)x * Wx + k] * ct[r * ld_own + k];
-      } else {
-        for (int k = lane; k < Wx; k += 64) gradb[(long)x * Wx + k] = ct[r * ld_own + k];
+    } else if (LOG) {
+      const float sh = sh_own[r] == -INFINITY ? 0.f : sh_own[r];
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        const int k = lane + 64 * q;
+        if (k >= Wx) break;
+        // exp(x - shift); cells outside the matrix are excluded from the row maximum
+        // and their sum is 0
+        const float acv = ct[r * ld_own + k];
+        gradb[(long)x * Wx + k] = acv == 0.f ? 0.f : fast_exp2((xv[rr][q] - sh) * kLog2e) * acv;
       }
+    } else if (PREP) {
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        const int k = lane + 64 * q;
+        if (k < Wx) gradb[(long)x * Wx + k] = xv[rr][q] * ct[r * ld_own + k];
+      }
+    } else {
+      for (int k = lane; k < Wx; k += 64) gradb[(long)x * Wx + k] = ct[r * ld_own + k];
     }
   }
 }

@@ -221,7 +221,9 @@ size_t genbmm_banded_workspace_size(int a_lu, int a_ld, int b_lu, int b_ld,
  * Gradients of genbmm_banded_fwd with respect to BOTH operands, reading g,
  * out and idx in the frame the forward wrote them (no banded transposes).
  * `out` is read in mode LOG only, `idx` in mode MAX only (others may be NULL);
- * `workspace`: NULL or, in mode LOG, the buffer the forward filled.
+ * `workspace`: NULL or, in mode LOG, the buffer the forward filled; the backward
+ * writes its own part of it (g/S per output cell, shared by both gradients), so
+ * two backward calls on one workspace must not overlap in time.
  * grad_a terms are added in ascending j (result band index), grad_b terms in
  * ascending i (row of a), which is the order of the reference's two calls.
  * Replaces the two _genbmm.backward_band calls and the Python-side banded
@@ -232,7 +234,7 @@ size_t genbmm_banded_workspace_size(int a_lu, int a_ld, int b_lu, int b_ld,
 int genbmm_banded_bwd(const float* a, int a_lu, int a_ld,
                       const float* b, int b_lu, int b_ld,
                       const float* out, const int32_t* idx,
-                      const float* workspace, const float* g,
+                      float* workspace, const float* g,
                       float* grad_a, float* grad_b,
                       int B, int n, int mode, void* stream);
 
