@@ -11,6 +11,7 @@
 // registers.  Lanes run along n, so the reads of b and the writes of out/idx
 // are coalesced (the reference puts threadIdx.x on rows and strides by K/N).
 #include "dense_tiles.h"
+#include "logbmm_ws.h"
 
 namespace genbmm {
 namespace {
@@ -124,65 +125,74 @@ __global__ __launch_bounds__(C::NT) void k_max_fwd(const DenseArgs p) {
   store_tile_i<C>(p.idx + (long)batch * M * N, ind, m0, n0, M, N, p.vec_o, tx, ty);
 }
 
-// Second level: group code -> value and index.  A workgroup owns kResCols columns
-// of one batch item and a range of rows; the rows of b that the groups can point
-// at are staged kResK at a time in LDS as [k][column], so that lane = column reads
-// its own bank whatever k it needs, and the kMaxGroup values of a come from the
-// row of a the whole wave shares.  The maximum of the group's terms is the
-// maximum of the cell (the group raised it last); descending k keeps the first
-// term equal to it.  Rows are taken kResRows at a time.
-constexpr int kResCols = 64, kResK = 256, kResWaves = 8, kResRows = 4, kResStage = 8;
-static_assert(kResK % kMaxGroup == 0, "a group lies in one staged chunk");
-static_assert(kMaxGroup == 8, "the maximum chain below is written for eight terms");
+// Second level (max / prod-max and the sampling sweep): group code -> result.
+// A workgroup owns COLS columns of one batch item and a range of rows; the rows of
+// the second operand that the groups can point at are staged in LDS as [k][column]
+// - 64 KB: 256 rows of 64 columns or 512 rows of 32 - so that a lane reads the bank
+// of its own column whatever k it needs (COLS = 32: a wave takes two rows at a time
+// and the two halves may meet in a bank).  The kResGroup values of the first operand
+// come from the row the lanes of a half-wave share.  Rows are taken kResRows at a time,
+// software-pipelined: the codes two steps ahead and the first operand's values one step
+// ahead are requested before the current rows are finished and stored.
+//
+// Op supplies what differs: Extra load(e) (read together with the code of cell e),
+// none(e) (a cell whose code is -1) and cell(e, kb, av, br, stride, valid, extra) with
+// av[j] = first operand at k = kb + j, br[j * stride] = second operand, valid = number
+// of terms of the group that lie inside K.
+constexpr int kResGroup = 8, kResWaves = 8, kResRows = 4, kResStage = 8;
+constexpr int kResFloats = 16384;  // 64 KB of LDS
+static_assert(kMaxGroup == kResGroup, "");
 
 typedef float float4_u __attribute__((ext_vector_type(4), aligned(4)));
 
-// TAIL: K is not a multiple of the group, the last group is cut at K.
-template <bool PROD, bool TAIL>
-__global__ __launch_bounds__(kResWaves * 64) void k_max_resolve(
-    const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ out,
-    int32_t* __restrict__ idx, float* __restrict__ fac_a, float* __restrict__ fac_b, int M, int K,
-    int N, int panels, int row_chunks, int rows_per) {
-  __shared__ float Bs[kResK * kResCols];
-  const int lane = threadIdx.x & 63;
+template <int COLS, bool TAIL, class Op>
+__device__ __forceinline__ void resolve_walk(const float* __restrict__ first, const float* __restrict__ second,
+                                             int32_t* __restrict__ idx, Op& op, int M, int K, int N,
+                                             int panels, int row_chunks, int rows_per, float* Bs) {
+  constexpr int RPW = 64 / COLS;           // rows a wave takes per step
+  constexpr int KSTAGE = kResFloats / COLS;  // rows of the second operand staged at a time
+  constexpr int R = kResRows, G = kResGroup, STEP = kResWaves * R * RPW;
+  static_assert(KSTAGE % G == 0, "a group lies in one staged chunk");
+  const int lane = threadIdx.x & 63, col = lane % COLS, sub = lane / COLS;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   int wg = blockIdx.x;
   const int panel = wg % panels;
   wg /= panels;
   const int chunk = wg % row_chunks;
   const int batch = wg / row_chunks;
-  const int n = panel * kResCols + lane;
+  const int n = panel * COLS + col;
   const bool live = n < N;
   const int nc = min(n, N - 1);
   const int m_beg = chunk * rows_per, m_end = min(M, m_beg + rows_per);
-  const float* ab = a + (long)batch * M * K;
-  const float* bb = b + (long)batch * K * N;
-  float* ob = out + (long)batch * M * N;
-  int32_t* ib = idx + (long)batch * M * N;
-  // optional: the two factors of the winning term per cell (product semiring)
-  float* fa = fac_a ? fac_a + (long)batch * M * N : nullptr;
-  float* fb = fac_b ? fac_b + (long)batch * M * N : nullptr;
+  const float* ab = first + (long)batch * M * K;
+  const float* bb = second + (long)batch * K * N;
+  const long cell0 = (long)batch * M * N;
+  const int32_t* ib = idx + cell0;
+  using Extra = typename Op::Extra;
+  auto row_of = [&](int mb, int r) { return mb + r * RPW + sub; };
 
-  constexpr int R = kResRows, G = kMaxGroup, STEP = kResWaves * kResRows;
-  // codes of R rows; 0 (nothing to do) outside the matrix
-  auto load_codes = [&](int mb, int (&code)[R]) __attribute__((always_inline)) {
+  // codes of R rows (0: nothing to do, also outside the matrix) and what Op reads with them
+  auto load_codes = [&](int mb, int (&code)[R], Extra (&ex)[R]) __attribute__((always_inline)) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const int c = ib[(long)min(mb + r, M - 1) * N + nc];
-      code[r] = (live && mb + r < m_end) ? c : 0;
+      const int m = row_of(mb, r);
+      const long e = (long)min(m, M - 1) * N + nc;
+      const int c = ib[e];
+      ex[r] = op.load(cell0 + e);
+      code[r] = (live && m < m_end) ? c : 0;
     }
   };
-  // first k of the group of each row (-1: not a group of the staged rows kc..) and
-  // the group's values of a
-  auto gather_a = [&](int mb, int kc, const int (&code)[R], int (&kb)[R], float (&av)[R][G])
-                      __attribute__((always_inline)) {
+  // first k of each row's group (-1: not a group of the staged rows kc..) and the
+  // group's values of the first operand
+  auto gather = [&](int mb, int kc, const int (&code)[R], int (&kb)[R], float (&av)[R][G])
+                    __attribute__((always_inline)) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int k = (-2 - code[r]) * G;
-      const bool act = code[r] <= -2 && k >= kc && k < kc + kResK;
+      const bool act = code[r] <= -2 && k >= kc && k < kc + KSTAGE;
       kb[r] = act ? k : -1;
       const int ks = act ? k : kc;
-      const float* ar = ab + (long)min(mb + r, M - 1) * K + ks;
+      const float* ar = ab + (long)min(row_of(mb, r), M - 1) * K + ks;
       if (!TAIL) {
 #pragma unroll
         for (int q = 0; q < G / 4; ++q) {
@@ -195,93 +205,140 @@ __global__ __launch_bounds__(kResWaves * 64) void k_max_resolve(
       }
     }
   };
-  auto finish = [&](int mb, int kc, int rows, const int (&code)[R], const int (&kb)[R],
-                    const float (&av)[R][G]) __attribute__((always_inline)) {
+  auto finish = [&](int mb, int kc, int rows, const int (&code)[R], const Extra (&ex)[R],
+                    const int (&kb)[R], const float (&av)[R][G]) __attribute__((always_inline)) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const long e = (long)(mb + r) * N + n;
-      if (code[r] == -1 && kc == 0) {
-        ob[e] = kFloor;
-        if (fa) {
-          fa[e] = 0.f;
-          fb[e] = 0.f;
-        }
-      }
+      const long e = cell0 + (long)row_of(mb, r) * N + n;
+      if (code[r] == -1 && kc == 0) op.none(e);
       if (kb[r] < 0) continue;
       const int rel = kb[r] - kc;
-      const float* br = Bs + rel * kResCols + lane;
-      float t[G], bv[G];
-#pragma unroll
-      for (int j = 0; j < G; ++j) {
-        bv[j] = br[(TAIL ? min(j, rows - 1 - rel) : j) * kResCols];
-        t[j] = PROD ? av[r][j] * bv[j] : av[r][j] + bv[j];
-        if (TAIL && kb[r] + j >= K) t[j] = -INFINITY;
-      }
-      float v = __builtin_fmaxf(__builtin_fmaxf(t[0], t[1]), t[2]);
-      v = __builtin_fmaxf(__builtin_fmaxf(v, t[3]), t[4]);
-      v = __builtin_fmaxf(__builtin_fmaxf(v, t[5]), t[6]);
-      v = __builtin_fmaxf(v, t[7]);
-      int first = G - 1;
-#pragma unroll
-      for (int j = G - 2; j >= 0; --j)
-        if (t[j] == v) first = j;
-      if (v == 0.f) {  // +0 and -0 compare equal: the value is the first one's
-#pragma unroll
-        for (int j = G - 1; j >= 0; --j)
-          if (j == first) v = t[j];
-      }
-      ib[e] = kb[r] + first;
-      ob[e] = v;
-      if (fa) {
-        float sa = av[r][0], sb = bv[0];
-#pragma unroll
-        for (int j = 1; j < G; ++j) {
-          sa = j == first ? av[r][j] : sa;
-          sb = j == first ? bv[j] : sb;
-        }
-        fa[e] = sa;
-        fb[e] = sb;
-      }
+      // the last group of a ragged K: its rows past K are not staged; point at row rows - 1
+      const float* br = Bs + rel * COLS + col;
+      const int valid = TAIL ? min(G, K - kb[r]) : G;
+      op.cell(e, kb[r], av[r], br, COLS, valid, min(G, rows - rel), ex[r]);
     }
   };
 
-  for (int kc = 0; kc < K; kc += kResK) {
-    const int rows = min(kResK, K - kc);
-    int mb = m_beg + wave * R;
+  for (int kc = 0; kc < K; kc += KSTAGE) {
+    const int rows = min(KSTAGE, K - kc);
+    int mb = m_beg + wave * R * RPW;
     int c0[R], c1[R], kb0[R];
+    Extra e0[R], e1[R];
     float a0[R][G];
-    load_codes(mb, c0);
+    load_codes(mb, c0, e0);
     __syncthreads();
-    for (int r0 = wave; r0 < rows; r0 += kResWaves * kResStage) {
+    for (int r0 = wave * RPW + sub; r0 < rows; r0 += kResWaves * RPW * kResStage) {
       float x[kResStage];
 #pragma unroll
       for (int u = 0; u < kResStage; ++u)
-        x[u] = bb[(long)(kc + min(r0 + u * kResWaves, rows - 1)) * N + nc];
+        x[u] = bb[(long)(kc + min(r0 + u * kResWaves * RPW, rows - 1)) * N + nc];
 #pragma unroll
       for (int u = 0; u < kResStage; ++u)
-        if (r0 + u * kResWaves < rows) Bs[(r0 + u * kResWaves) * kResCols + lane] = x[u];
+        if (r0 + u * kResWaves * RPW < rows) Bs[(r0 + u * kResWaves * RPW) * COLS + col] = x[u];
     }
-    gather_a(mb, kc, c0, kb0, a0);
-    load_codes(mb + STEP, c1);
+    gather(mb, kc, c0, kb0, a0);
+    load_codes(mb + STEP, c1, e1);
     __syncthreads();
-    // two sets of rows in flight: the codes two ahead and the values of a one ahead
-    // are requested before the current rows are finished and stored
-    for (; mb < m_end; mb += STEP) {
+    for (; mb < m_end; mb += STEP) {   // mb is wave-uniform; rows past m_end carry code 0
       int c2[R], kb1[R];
+      Extra e2[R];
       float a1[R][G];
-      gather_a(mb + STEP, kc, c1, kb1, a1);
-      load_codes(mb + 2 * STEP, c2);
-      finish(mb, kc, rows, c0, kb0, a0);
+      gather(mb + STEP, kc, c1, kb1, a1);
+      load_codes(mb + 2 * STEP, c2, e2);
+      finish(mb, kc, rows, c0, e0, kb0, a0);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        c0[r] = c1[r];
-        c1[r] = c2[r];
+        c0[r] = c1[r]; c1[r] = c2[r];
+        e0[r] = e1[r]; e1[r] = e2[r];
         kb0[r] = kb1[r];
 #pragma unroll
         for (int j = 0; j < G; ++j) a0[r][j] = a1[r][j];
       }
     }
   }
+}
+
+// Rows per workgroup (all of them unless that leaves the compute units short) and
+// the grid of a resolve launch.
+inline int resolve_grid(int B, int M, int N, int cols, int& panels, int& row_chunks, int& rows_per,
+                        unsigned& grid) {
+  panels = ceil_div(N, cols);
+  row_chunks = 1;
+  const int step = kResWaves * kResRows * (64 / cols);
+  while ((int64_t)B * panels * row_chunks < 1024 && ceil_div(M, row_chunks) > 2 * step) row_chunks *= 2;
+  rows_per = ceil_div(M, row_chunks);
+  row_chunks = ceil_div(M, rows_per);
+  const int64_t total = (int64_t)B * panels * row_chunks;
+  if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
+  grid = (unsigned)total;
+  return GENBMM_OK;
+}
+
+// max / prod-max: the maximum of the group's terms is the maximum of the cell (the
+// group raised it last); descending k keeps the first term equal to it.
+template <bool PROD>
+struct MaxResolve {
+  struct Extra {};
+  float* out;
+  int32_t* idx;
+  float* fa;  // optional: the two factors of the winning term per cell (product semiring)
+  float* fb;
+  __device__ __forceinline__ Extra load(long) const { return Extra{}; }
+  __device__ __forceinline__ void none(long e) const {
+    out[e] = kFloor;
+    if (fa) {
+      fa[e] = 0.f;
+      fb[e] = 0.f;
+    }
+  }
+  __device__ __forceinline__ void cell(long e, int kb, const float (&av)[kResGroup], const float* br,
+                                       int stride, int valid, int staged, Extra) const {
+    constexpr int G = kResGroup;
+    float t[G], bv[G];
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+      bv[j] = br[min(j, staged - 1) * stride];
+      t[j] = PROD ? av[j] * bv[j] : av[j] + bv[j];
+      if (j >= valid) t[j] = -INFINITY;
+    }
+    float v = __builtin_fmaxf(__builtin_fmaxf(t[0], t[1]), t[2]);
+    v = __builtin_fmaxf(__builtin_fmaxf(v, t[3]), t[4]);
+    v = __builtin_fmaxf(__builtin_fmaxf(v, t[5]), t[6]);
+    v = __builtin_fmaxf(v, t[7]);
+    int first = G - 1;
+#pragma unroll
+    for (int j = G - 2; j >= 0; --j)
+      if (t[j] == v) first = j;
+    if (v == 0.f) {  // +0 and -0 compare equal: the value is the first one's
+#pragma unroll
+      for (int j = G - 1; j >= 0; --j)
+        if (j == first) v = t[j];
+    }
+    idx[e] = kb + first;
+    out[e] = v;
+    if (fa) {
+      float sa = av[0], sb = bv[0];
+#pragma unroll
+      for (int j = 1; j < G; ++j) {
+        sa = j == first ? av[j] : sa;
+        sb = j == first ? bv[j] : sb;
+      }
+      fa[e] = sa;
+      fb[e] = sb;
+    }
+  }
+};
+
+// TAIL: K is not a multiple of the group, the last group is cut at K.
+template <bool PROD, int COLS, bool TAIL>
+__global__ __launch_bounds__(kResWaves * 64, 4) void k_max_resolve(
+    const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ out,
+    int32_t* __restrict__ idx, float* __restrict__ fac_a, float* __restrict__ fac_b, int M, int K,
+    int N, int panels, int row_chunks, int rows_per) {
+  __shared__ float Bs[kResFloats];
+  MaxResolve<PROD> op{out, idx, fac_a, fac_b};
+  resolve_walk<COLS, TAIL>(a, b, idx, op, M, K, N, panels, row_chunks, rows_per, Bs);
 }
 
 // ------------------------------------------------------------ sample forward
@@ -300,9 +357,23 @@ __global__ __launch_bounds__(C::NT) void k_sample_fwd(const DenseArgs p) {
 // u * S, S = exp(out - alpha - beta): one multiply per (m,k,n) instead of an
 // exponential.  A tile in which any cell has S < 2^-40 (or is not finite) runs
 // the online routine + exact sweep instead.
-template <class C>
+//
+// TWO (shapes whose logbmm forward left EA, EB and a B*M*N scratch array in the
+// workspace): two levels like the max forward.  The sweep reads EA / EB as they are,
+// spends one multiply-add per term on the running rem = t - prefix sum, and looks at it
+// only at the end of every group of kSampleGroup terms: its sign goes into the bit
+// string (-> the group in which the prefix sum passes t), its smallest non-negative
+// value (-> rem at the start of that group; non-negative floats order as unsigned
+// integers and every negative one is larger) into the scratch array.
+// k_sample_resolve then redoes the same multiply-adds for that one group.
+constexpr int kSampleGroup = 8;
+
+template <class C, bool TWO>
 __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
-                                                           const float* __restrict__ stats) {
+                                                           const float* __restrict__ stats,
+                                                           const float* __restrict__ ws_ea,
+                                                           const float* __restrict__ ws_eb,
+                                                           float* __restrict__ ws_rem) {
   __shared__ __attribute__((aligned(16))) float smem[C::KT * (C::LDA + C::LDB) + C::BM + C::BN];
   float* As = smem;
   float* Bs = As + C::KT * C::LDA;
@@ -312,8 +383,8 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
   int batch, m0, n0;
   decode_tile<C>(p, batch, m0, n0);
   const int M = p.M, K = p.K, N = p.N;
-  const float* ab = p.a + (long)batch * M * K;
-  const float* bb = p.b + (long)batch * K * N;
+  const float* ab = (TWO ? ws_ea : p.a) + (long)batch * M * K;
+  const float* bb = (TWO ? ws_eb : p.b) + (long)batch * K * N;
   const float* ob = p.out + (long)batch * M * N;
   const float* st = stats + (long)batch * (M + N);
   for (int t = tid; t < C::BM; t += C::NT) al[t] = (m0 + t < M) ? st[m0 + t] : 0.f;
@@ -327,7 +398,8 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
   // v_alignbit_b32 and the bits of a slab are counted once per slab.
   float rem[C::TM][C::TN];
   uint32_t bits[C::TM][C::TN];
-  int ind[C::TM][C::TN];  // number of terms whose prefix sum exceeded t
+  int ind[C::TM][C::TN];  // number of terms (TWO: groups) whose prefix sum exceeded t
+  uint32_t low[TWO ? C::TM : 1][TWO ? C::TN : 1];  // TWO: smallest rem >= 0 seen at a group end
   const float lim = 40.f * kLn2 + 1e-3f;
   int bad = 0;
 #pragma unroll
@@ -343,6 +415,10 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
         if (!(e <= lim) || !(e > -INFINITY)) bad = 1;
         const uint64_t cell = ((uint64_t)batch * M + m) * (uint64_t)N + n;
         rem[i][j] = philox_uniform(cell, p.seed, p.offset) * fast_exp2(-e * kLog2e);
+      }
+      if (TWO) {
+        low[i][j] = __float_as_uint(rem[i][j]);
+        bits[i][j] = 0u;
       }
     }
   if (__syncthreads_or(bad)) {  // workgroup-uniform
@@ -361,13 +437,13 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
   for (int k0 = 0; k0 < K; k0 += C::KT) {
     __syncthreads();
 #pragma unroll
-    for (int l = 0; l < TA::PER; ++l) {
+    for (int l = 0; l < (TWO ? 0 : TA::PER); ++l) {
       const float s = al[((tid + l * C::NT) / TA::C4) % C::BM];
       ta.r[l].x = fast_exp2((ta.r[l].x - s) * kLog2e); ta.r[l].y = fast_exp2((ta.r[l].y - s) * kLog2e);
       ta.r[l].z = fast_exp2((ta.r[l].z - s) * kLog2e); ta.r[l].w = fast_exp2((ta.r[l].w - s) * kLog2e);
     }
 #pragma unroll
-    for (int l = 0; l < TB::PER; ++l) {
+    for (int l = 0; l < (TWO ? 0 : TB::PER); ++l) {
       const float4 s = *reinterpret_cast<const float4*>(be + ((tid + l * C::NT) % TB::C4) * 4);
       tb.r[l].x = fast_exp2((tb.r[l].x - s.x) * kLog2e); tb.r[l].y = fast_exp2((tb.r[l].y - s.y) * kLog2e);
       tb.r[l].z = fast_exp2((tb.r[l].z - s.z) * kLog2e); tb.r[l].w = fast_exp2((tb.r[l].w - s.w) * kLog2e);
@@ -381,6 +457,43 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
     }
     const int kn = min(C::KT, K - k0);
     static_assert(C::KT <= 32, "one bit per term of a slab");
+    if (TWO) {
+      // terms past K are zero (the loaders fill with 0): every slab is walked in full
+      static_assert(C::KT % kSampleGroup == 0, "whole groups per slab");
+#pragma unroll
+      for (int g = 0; g < C::KT / kSampleGroup; ++g) {
+#pragma unroll
+        for (int kk = g * kSampleGroup; kk < (g + 1) * kSampleGroup; ++kk) {
+          float av[C::TM], bv[C::TN];
+          lds_frag<C::TM / 4>(As + kk * C::LDA, ty * C::TM, 4, av);
+          lds_frag<C::TN / 4>(Bs + kk * C::LDB, tx * 4, C::TX * 4, bv);
+#pragma unroll
+          for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+            for (int j = 0; j < C::TN; ++j) rem[i][j] = __builtin_fmaf(-av[i], bv[j], rem[i][j]);
+        }
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+          for (int j = 0; j < C::TN; ++j) {
+            const uint32_t rb = __float_as_uint(rem[i][j]);
+            bits[i][j] = __builtin_amdgcn_alignbit(bits[i][j], rb, 31);
+            low[i][j] = min(low[i][j], rb);
+          }
+      }
+      // the bit string holds 32 groups
+      constexpr int kFold = 32 / (C::KT / kSampleGroup);
+      if ((k0 / C::KT) % kFold == kFold - 1 || k0 + C::KT >= K) {
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+          for (int j = 0; j < C::TN; ++j) {
+            ind[i][j] += __builtin_popcount(bits[i][j]);
+            bits[i][j] = 0u;
+          }
+      }
+      continue;
+    }
 #pragma unroll
     for (int i = 0; i < C::TM; ++i)
 #pragma unroll
@@ -408,6 +521,23 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
 #pragma unroll
       for (int j = 0; j < C::TN; ++j) ind[i][j] += __builtin_popcount(bits[i][j]);
   }
+  if (TWO) {
+    // group = groups walked - groups past t (none past t: rounding left the last prefix
+    // sum a hair under t -> index 0, as below); the code -2 - group goes to idx, rem at
+    // the start of that group to the scratch array
+    const int walked = ((K + C::KT - 1) / C::KT) * (C::KT / kSampleGroup);
+    float remv[C::TM][C::TN];
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < C::TN; ++j) {
+        ind[i][j] = ind[i][j] == 0 ? 0 : -2 - (walked - ind[i][j]);
+        remv[i][j] = __uint_as_float(low[i][j]);
+      }
+    store_tile_i<C>(p.idx + (long)batch * M * N, ind, m0, n0, M, N, p.vec_o, tx, ty);
+    store_tile_f<C>(ws_rem + (long)batch * M * N, remv, m0, n0, M, N, p.vec_o && (reinterpret_cast<uintptr_t>(ws_rem) & 15u) == 0, tx, ty);
+    return;
+  }
   // index = K - (terms past t).  Rounding can leave the last prefix sum a hair under
   // u*S: no crossing -> index 0, as when the reference's walk never exceeds its draw
 #pragma unroll
@@ -415,6 +545,41 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
 #pragma unroll
     for (int j = 0; j < C::TN; ++j) ind[i][j] = ind[i][j] == 0 ? 0 : K - ind[i][j];
   store_tile_i<C>(p.idx + (long)batch * M * N, ind, m0, n0, M, N, p.vec_o, tx, ty);
+}
+
+// Second level of the sampling sweep: rem at the start of the group goes through the
+// same multiply-adds as in the sweep; the index is the group's first term plus the
+// number of terms after which rem is still >= 0 (rem only falls).
+struct SampleResolve {
+  typedef float Extra;
+  const float* rem;
+  int32_t* idx;
+  int K;
+  __device__ __forceinline__ float load(long e) const { return rem[e]; }
+  __device__ __forceinline__ void none(long) const {}
+  __device__ __forceinline__ void cell(long e, int kb, const float (&av)[kResGroup], const float* br,
+                                       int stride, int valid, int staged, float r) const {
+    uint32_t past = 0u;
+#pragma unroll
+    for (int j = 0; j < kResGroup; ++j) {
+      const float ea = j < valid ? av[j] : 0.f;
+      r = __builtin_fmaf(-ea, br[min(j, staged - 1) * stride], r);
+      past = __builtin_amdgcn_alignbit(past, __float_as_uint(r), 31);
+    }
+    idx[e] = min(kb + kResGroup - __builtin_popcount(past), K - 1);
+  }
+};
+
+template <int COLS, bool TAIL>
+__global__ __launch_bounds__(kResWaves * 64, 4) void k_sample_resolve(
+    const float* __restrict__ ea, const float* __restrict__ eb, const float* __restrict__ remw,
+    int32_t* __restrict__ idx, int* __restrict__ valid, int M, int K, int N, int panels,
+    int row_chunks, int rows_per) {
+  __shared__ float Bs[kResFloats];
+  static_assert(kSampleGroup == kResGroup, "");
+  if (blockIdx.x == 0 && threadIdx.x == 0) *valid = 0;  // the 1/S array of the workspace is gone
+  SampleResolve op{remw, idx, K};
+  resolve_walk<COLS, TAIL>(ea, eb, idx, op, M, K, N, panels, row_chunks, rows_per, Bs);
 }
 
 // ---------------------------------------------------------------- dispatch
@@ -425,23 +590,24 @@ int launch_max(DenseArgs p, float* factors, int B, int M, int K, int N, hipStrea
   hipLaunchKernelGGL((k_max_fwd<C, PROD>), grid, dim3(C::NT), 0, s, p);
   if (int e = launch_status()) return e;
   if (K == 0) return GENBMM_OK;  // every code is -1 already
-  // rows per workgroup: all of them unless that leaves the compute units short
-  const int panels = ceil_div(N, kResCols);
-  int row_chunks = 1;
-  while ((int64_t)B * panels * row_chunks < 1024 && ceil_div(M, row_chunks) > 2 * kResWaves * kResRows)
-    row_chunks *= 2;
-  const int rows_per = ceil_div(M, row_chunks);
-  row_chunks = ceil_div(M, rows_per);
-  const int64_t total = (int64_t)B * panels * row_chunks;
-  if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
   float* fa = factors;
   float* fb = factors ? factors + (int64_t)B * M * N : nullptr;
-  if (K % kMaxGroup == 0)
-    hipLaunchKernelGGL((k_max_resolve<PROD, false>), dim3((unsigned)total), dim3(kResWaves * 64), 0,
-                       s, p.a, p.b, p.out, p.idx, fa, fb, M, K, N, panels, row_chunks, rows_per);
-  else
-    hipLaunchKernelGGL((k_max_resolve<PROD, true>), dim3((unsigned)total), dim3(kResWaves * 64), 0,
-                       s, p.a, p.b, p.out, p.idx, fa, fb, M, K, N, panels, row_chunks, rows_per);
+  const int cols = K > 256 ? 32 : 64;  // 512 or 256 staged rows: one pass up to K = 512
+  int panels, row_chunks, rows_per;
+  unsigned rgrid;
+  if (int e = resolve_grid(B, M, N, cols, panels, row_chunks, rows_per, rgrid)) return e;
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(rgrid), dim3(kResWaves * 64), 0, s, p.a, p.b, p.out, p.idx, fa, fb,
+                       M, K, N, panels, row_chunks, rows_per);
+  };
+  const bool tail = K % kMaxGroup != 0;
+  if (cols == 64) {
+    if (tail) go(k_max_resolve<PROD, 64, true>);
+    else go(k_max_resolve<PROD, 64, false>);
+  } else {
+    if (tail) go(k_max_resolve<PROD, 32, true>);
+    else go(k_max_resolve<PROD, 32, false>);
+  }
   return launch_status();
 }
 
@@ -476,7 +642,36 @@ template <class C>
 int launch_sweep(DenseArgs p, const float* stats, int B, int M, int K, int N, hipStream_t s) {
   dim3 grid;
   if (int e = fill_args<C>(p, B, M, K, N, grid)) return e;
-  hipLaunchKernelGGL((k_sample_sweep<C>), grid, dim3(C::NT), 0, s, p, stats);
+  hipLaunchKernelGGL((k_sample_sweep<C, false>), grid, dim3(C::NT), 0, s, p, stats,
+                     (const float*)nullptr, (const float*)nullptr, (float*)nullptr);
+  return launch_status();
+}
+
+// Two levels on the factors the logbmm forward left in the workspace.
+template <class C>
+int launch_sweep_two(DenseArgs p, const float* stats, const LogFactors& f, int B, int M, int K,
+                     int N, hipStream_t s) {
+  dim3 grid;
+  if (int e = fill_args<C>(p, B, M, K, N, grid)) return e;
+  hipLaunchKernelGGL((k_sample_sweep<C, true>), grid, dim3(C::NT), 0, s, p, stats, f.ea, f.eb,
+                     f.scratch);
+  if (int e = launch_status()) return e;
+  const int cols = K > 256 ? 32 : 64;
+  int panels, row_chunks, rows_per;
+  unsigned rgrid;
+  if (int e = resolve_grid(B, M, N, cols, panels, row_chunks, rows_per, rgrid)) return e;
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(rgrid), dim3(kResWaves * 64), 0, s, f.ea, f.eb, f.scratch, p.idx,
+                       f.valid, M, K, N, panels, row_chunks, rows_per);
+  };
+  const bool tail = K % kSampleGroup != 0;
+  if (cols == 64) {
+    if (tail) go(k_sample_resolve<64, true>);
+    else go(k_sample_resolve<64, false>);
+  } else {
+    if (tail) go(k_sample_resolve<32, true>);
+    else go(k_sample_resolve<32, false>);
+  }
   return launch_status();
 }
 
@@ -492,6 +687,13 @@ int run_sample(const float* a, const float* b, float* out, int32_t* idx, float* 
   hipStream_t s = (hipStream_t)stream;
   if (stats && K > 0) {  // log-sum-exp by the logbmm forward, then the multiply-only sweep
     if (int e = genbmm_logbmm_fwd(a, b, out, stats, B, M, K, N, stream)) return e;
+    LogFactors f;
+    if (log_fwd_writes_factors(stats, B, M, K, N, &f)) {
+      switch (pick_shape(B, M, N, false)) {
+        case kWide: return launch_sweep_two<CfgWide>(p, stats, f, B, M, K, N, s);
+        default: return launch_sweep_two<CfgMid>(p, stats, f, B, M, K, N, s);
+      }
+    }
     switch (pick_shape(B, M, N, false)) {
       case kWide: return launch_sweep<CfgWide>(p, stats, B, M, K, N, s);
       case kMid: return launch_sweep<CfgMid>(p, stats, B, M, K, N, s);

@@ -34,6 +34,7 @@
 #include "log_bwd_tile.h"
 #include "logbmm_item.h"
 #include "logbmm_mfma.h"
+#include "logbmm_ws.h"
 
 namespace genbmm {
 namespace {
@@ -767,6 +768,22 @@ int run_bwd(const LogBwdArgs& p, const float* stats, int B, hipStream_t s) {
 }
 
 }  // namespace
+
+// The forward's own decision (genbmm_logbmm_fwd below): factors are written by the
+// matrix-core kernels only.
+bool log_fwd_writes_factors(const float* stats, int B, int M, int K, int N, LogFactors* f) {
+  if (!stats || K <= 0 || (int64_t)B * M * N == 0) return false;
+  if (B > 0 && item_shape(M, K, N) && g_path.load() == 0) return false;   // whole-item kernels
+  if (g_path.load() == 1 || !fwd_mfma_shape(B, M, K, N)) return false;
+  if (mfma_kind(B, M, N, K, true, false) == 0) return false;
+  const LogPrepared ws = prepared_of(stats, B, M, K, N);
+  f->ea = ws.ea;
+  f->eb = ws.eb;
+  f->scratch = ws.r;
+  f->valid = ws.hdr;
+  return true;
+}
+
 }  // namespace genbmm
 
 extern "C" {

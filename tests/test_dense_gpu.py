@@ -394,7 +394,10 @@ def test_max_config_c3(gpu):
 
 # -------------------------------------------------------------------- sample
 @pytest.mark.parametrize("use_stats", [True, False])
-@pytest.mark.parametrize("B,M,K,N", [(6, 20, 37, 24), (3, 130, 64, 132), (2, 64, 100, 128)])
+@pytest.mark.parametrize("B,M,K,N", [(6, 20, 37, 24), (3, 130, 64, 132), (2, 64, 100, 128),
+                                     # shapes whose forward leaves the factors: two-level sweep (groups of 8
+                                     # terms; K not a multiple of 8, K across several staged chunks / folds)
+                                     (2, 128, 96, 160), (2, 200, 100, 260), (2, 256, 520, 128), (1, 97, 1030, 96)])
 def test_sample_index_brackets_cdf(gpu, use_stats, B, M, K, N):
     torch.manual_seed(11)
     a, b = 2 * torch.randn(B, M, K), 2 * torch.randn(B, K, N)
