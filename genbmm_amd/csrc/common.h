@@ -175,12 +175,44 @@ __host__ __device__ inline Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint3
   return r;
 }
 
+// One Philox block serves four consecutive output cells: cell i takes word i & 3 of
+// Philox(counter = {lo(i >> 2), hi(i >> 2), lo(offset), hi(offset)}, key = seed); its
+// top 24 bits scaled by 2^-24 are the uniform in [0,1).  (The 64-bit products of the
+// ten rounds are the cost of a draw: a lane that owns four adjacent cells pays once.)
+__host__ __device__ inline Philox4 philox_block(uint64_t block, uint64_t seed, uint64_t offset) {
+  return philox4x32_10((uint32_t)block, (uint32_t)(block >> 32), (uint32_t)offset,
+                       (uint32_t)(offset >> 32), (uint32_t)seed, (uint32_t)(seed >> 32));
+}
+__host__ __device__ inline float philox_scale(uint32_t word) {
+  return (float)(word >> 8) * (1.0f / 16777216.0f);
+}
 // Uniform in [0,1) of output cell `i` for stream (seed, offset).
 __host__ __device__ inline float philox_uniform(uint64_t i, uint64_t seed, uint64_t offset) {
-  const Philox4 r = philox4x32_10((uint32_t)i, (uint32_t)(i >> 32), (uint32_t)offset,
-                                  (uint32_t)(offset >> 32), (uint32_t)seed,
-                                  (uint32_t)(seed >> 32));
-  return (float)(r.x[0] >> 8) * (1.0f / 16777216.0f);
+  const Philox4 r = philox_block(i >> 2, seed, offset);
+  const uint32_t w = (i & 2) ? ((i & 1) ? r.x[3] : r.x[2]) : ((i & 1) ? r.x[1] : r.x[0]);
+  return philox_scale(w);
+}
+
+// Uniforms of the four consecutive cells i .. i+3.  aligned: i is a multiple of four
+// (one block); otherwise the cells straddle two blocks.
+__host__ __device__ inline void philox_uniform4(uint64_t i, bool aligned, uint64_t seed,
+                                                uint64_t offset, float (&u)[4]) {
+  const Philox4 r0 = philox_block(i >> 2, seed, offset);
+  if (aligned) {
+    u[0] = philox_scale(r0.x[0]); u[1] = philox_scale(r0.x[1]);
+    u[2] = philox_scale(r0.x[2]); u[3] = philox_scale(r0.x[3]);
+    return;
+  }
+  const Philox4 r1 = philox_block((i >> 2) + 1, seed, offset);
+  const uint32_t w[8] = {r0.x[0], r0.x[1], r0.x[2], r0.x[3], r1.x[0], r1.x[1], r1.x[2], r1.x[3]};
+  const int s = (int)(i & 3);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    uint32_t v = w[q];
+#pragma unroll
+    for (int t = 1; t < 4; ++t) v = s == t ? w[q + t] : v;
+    u[q] = philox_scale(v);
+  }
 }
 
 // ------------------------------------------------------------- host helpers

@@ -402,23 +402,30 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
   uint32_t low[TWO ? C::TM : 1][TWO ? C::TN : 1];  // TWO: smallest rem >= 0 seen at a group end
   const float lim = 40.f * kLn2 + 1e-3f;
   int bad = 0;
+  const bool blocks = (N & 3) == 0;  // a lane's four adjacent cells then share one Philox block
 #pragma unroll
   for (int i = 0; i < C::TM; ++i)
 #pragma unroll
-    for (int j = 0; j < C::TN; ++j) {
-      const int r = ty * C::TM + i, c = col_of<C>(tx, j);
-      const int m = m0 + r, n = n0 + c;
-      ind[i][j] = 0;
-      rem[i][j] = 0.f;
-      if (m < M && n < N) {
-        const float e = al[r] + be[c] - ob[(long)m * N + n];   // -log S
-        if (!(e <= lim) || !(e > -INFINITY)) bad = 1;
-        const uint64_t cell = ((uint64_t)batch * M + m) * (uint64_t)N + n;
-        rem[i][j] = philox_uniform(cell, p.seed, p.offset) * fast_exp2(-e * kLog2e);
-      }
-      if (TWO) {
-        low[i][j] = __float_as_uint(rem[i][j]);
-        bits[i][j] = 0u;
+    for (int jq = 0; jq < C::TN; jq += 4) {
+      const int r = ty * C::TM + i, c0 = col_of<C>(tx, jq);
+      const int m = m0 + r;
+      float u[4] = {0.f, 0.f, 0.f, 0.f};
+      if (m < M && n0 + c0 < N)
+        philox_uniform4(((uint64_t)batch * M + m) * (uint64_t)N + (n0 + c0), blocks, p.seed, p.offset, u);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int j = jq + q, c = c0 + q, n = n0 + c;
+        ind[i][j] = 0;
+        rem[i][j] = 0.f;
+        if (m < M && n < N) {
+          const float e = al[r] + be[c] - ob[(long)m * N + n];   // -log S
+          if (!(e <= lim) || !(e > -INFINITY)) bad = 1;
+          rem[i][j] = u[q] * fast_exp2(-e * kLog2e);
+        }
+        if (TWO) {
+          low[i][j] = __float_as_uint(rem[i][j]);
+          bits[i][j] = 0u;
+        }
       }
     }
   if (__syncthreads_or(bad)) {  // workgroup-uniform

@@ -198,16 +198,21 @@ __device__ __forceinline__ void log_fwd_tile(const DenseArgs& p, int batch, int 
   // the reference's `total < r && total + p > r` with total = r - rem.
   float rem[C::TM][C::TN];
   int ind[C::TM][C::TN];
+  const bool blocks = (N & 3) == 0;  // a lane's four adjacent cells then share one Philox block
 #pragma unroll
   for (int i = 0; i < C::TM; ++i)
 #pragma unroll
-    for (int j = 0; j < C::TN; ++j) {
+    for (int jq = 0; jq < C::TN; jq += 4) {
       const int m = m0 + ty * C::TM + i;
-      const int n = n0 + col_of<C>(tx, j);
-      const uint64_t cell = ((uint64_t)batch * M + m) * (uint64_t)N + n;
-      rem[i][j] = philox_uniform(cell, p.seed, p.offset);
-      ind[i][j] = 0;
-      mx[i][j] = -mx[i][j] * kLog2e;  // -out*log2e
+      const int n = n0 + col_of<C>(tx, jq);
+      float u[4];
+      philox_uniform4(((uint64_t)batch * M + m) * (uint64_t)N + n, blocks, p.seed, p.offset, u);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        rem[i][jq + q] = u[q];
+        ind[i][jq + q] = 0;
+        mx[i][jq + q] = -mx[i][jq + q] * kLog2e;  // -out*log2e
+      }
     }
   if (K > 0) {
     ta.gload(ab, K, m0, 0, M, K, p.vec_a, tid);

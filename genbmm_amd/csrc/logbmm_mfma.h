@@ -629,4 +629,169 @@ void k_log_bwd_mfma_both(const float* __restrict__ g, const float* __restrict__ 
                                          K, N, br, bc);
 }
 
+// ------------------------------------------------------- sampling sweep
+// samplebmm on the forward's factors: index = first k whose prefix sum
+// sum_{k' <= k} EA[m,k'] EB[k',n] passes the target t = u * S (one Philox uniform
+// u per cell, S = exp(out - alpha - beta)).  The accumulators start at -t, so after
+// every slab they hold prefix - t.  Per slab and cell two vector instructions look
+// at that value: its sign bit (prefix still below t) is shifted into a bit string
+// (slabs <= 32) or added to a counter, and a signed-integer minimum keeps the
+// negative value closest to zero (negative floats order backwards as integers and
+// lie below every non-negative one) - minus that is rem = t - prefix at the start
+// of the slab in which the prefix passes t.  Results: the code -2 - slab in idx (0
+// if the prefix never reaches t) and rem in `remw`; the terms of that one slab are
+// walked by the resolve kernel.  A tile with a cell whose S is below 2^-40 or not
+// finite, or that the forward flagged, sets its flag and leaves: it is redone exactly.
+template <class T, bool RAGGED>
+__global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::NT / 256, T::NT / 256)))
+void k_sample_sweep_mfma(const float* __restrict__ ws_ea, const float* __restrict__ ws_eb,
+                         const float* __restrict__ out, const float* __restrict__ stats,
+                         int* __restrict__ flags, float* __restrict__ remw,
+                         int32_t* __restrict__ idx, uint64_t seed, uint64_t offset, int M, int K,
+                         int N, int tiles_m, int tiles_n) {
+  constexpr int NT = T::NT, LDR = T::LDR, LDC = T::LDC;
+  using SA = StageT<T::TR, NT, LDR>;
+  using SB = StageS<T::TC, NT, LDC>;
+  __shared__ __attribute__((aligned(16))) float smem[2 * kMS * (LDR + LDC)];
+  float(*As)[kMS * LDR] = reinterpret_cast<float(*)[kMS * LDR]>(smem);
+  float(*Bs)[kMS * LDC] = reinterpret_cast<float(*)[kMS * LDC]>(smem + 2 * kMS * LDR);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = (wave / T::WC) * 64, wn0 = (wave % T::WC) * 64;
+  const int per = tiles_m * tiles_n, tile = xcd_tile_id();
+  const int batch = tile / per, rem = tile - batch * per;
+  const int m0 = (rem / tiles_n) * T::TR, n0 = (rem % tiles_n) * T::TC;
+  const float* st = stats + (long)batch * (M + N);
+
+  // ---- targets: acc = -t, low = its bit pattern, in the accumulator layout
+  floatx16 acc[2][2];
+  int low[2][2][16];
+  uint32_t cnt[2][2][16];
+  const int col = lane & 31;
+  const float lim = kMfmaGuardBits * kLn2 + 1e-3f;
+  int bad = flags[tile];
+#pragma unroll
+  for (int br = 0; br < 2; ++br)
+#pragma unroll
+    for (int bc = 0; bc < 2; ++bc) {
+      const int n = n0 + wn0 + bc * 32 + col;
+      const bool nok = !RAGGED || n < N;
+      const float be = nok ? st[M + n] : 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int m = m0 + wm0 + br * 32 + mfma_row(i, lane);
+        const bool ok = nok && (!RAGGED || m < M);
+        float t = 0.f;
+        if (ok) {
+          const long cell = ((long)batch * M + m) * N + n;
+          const float e = st[m] + be - out[cell];  // -log S
+          if (!(e <= lim) || !(e > -INFINITY)) bad = 1;
+          t = philox_uniform((uint64_t)cell, seed, offset) * fast_exp2(-e * kLog2e);
+        }
+        acc[br][bc][i] = -t;
+        low[br][bc][i] = __float_as_int(-t);
+        cnt[br][bc][i] = 0u;
+      }
+    }
+  bad = __syncthreads_or(bad);
+  if (bad) {
+    if (tid == 0) flags[tile] = 1;
+    return;
+  }
+
+  // ---- staging of EA (transposed) and EB, one slab ahead
+  const int bcol = n0 + SB::quad(tid) * 4;
+  const int cb = RAGGED ? clamp4(N - bcol) : 4;
+  const bool vb = cb > 0;
+  bool va[SA::PER];
+  const float* pa[SA::PER];
+  const float* pb[SB::PER];
+#pragma unroll
+  for (int l = 0; l < SA::PER; ++l) {
+    const int line = m0 + SA::line(tid, l);
+    va[l] = !RAGGED || line < M;
+    pa[l] = ws_ea + ((long)batch * M + (va[l] ? line : M - 1)) * K + SA::quad(tid) * 4;
+  }
+#pragma unroll
+  for (int l = 0; l < SB::PER; ++l)
+    pb[l] = ws_eb + ((long)batch * K + SB::red(tid, l)) * N + (vb ? bcol : 0);
+  const int ktail = RAGGED ? K % kMS : 0;
+  const int slabs = RAGGED ? (K + kMS - 1) / kMS : K / kMS;
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 ra[SA::PER], rb[SB::PER];
+  auto load = [&](bool tail) __attribute__((always_inline)) {
+    if (RAGGED && tail) {
+      const int ca = clamp4(ktail - SA::quad(tid) * 4);
+#pragma unroll
+      for (int l = 0; l < SA::PER; ++l) ra[l] = va[l] ? ld4m(pa[l], ca, 0.f) : zero;
+#pragma unroll
+      for (int l = 0; l < SB::PER; ++l) rb[l] = SB::red(tid, l) < ktail ? ld4m(pb[l], cb, 0.f) : zero;
+    } else {
+#pragma unroll
+      for (int l = 0; l < SA::PER; ++l) ra[l] = (!RAGGED || va[l]) ? ld4(pa[l]) : zero;
+#pragma unroll
+      for (int l = 0; l < SB::PER; ++l) rb[l] = RAGGED ? ld4m(pb[l], cb, 0.f) : ld4(pb[l]);
+    }
+#pragma unroll
+    for (int l = 0; l < SA::PER; ++l) pa[l] += kMS;
+#pragma unroll
+    for (int l = 0; l < SB::PER; ++l) pb[l] += (long)kMS * N;
+  };
+  auto stage = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int l = 0; l < SA::PER; ++l) SA::put(As[buf], tid, l, ra[l]);
+#pragma unroll
+    for (int l = 0; l < SB::PER; ++l) SB::put(Bs[buf], tid, l, rb[l]);
+  };
+
+  const bool strings = slabs <= 32;  // one bit per slab fits the register
+  load(slabs == 1 && ktail != 0);
+  stage(0);
+  __syncthreads();
+  for (int s = 0; s < slabs; ++s) {
+    const bool more = s + 1 < slabs;
+    if (more) load(s + 2 == slabs && ktail != 0);
+    mfma_slab<LDR, LDC>(As[s & 1], Bs[s & 1], wm0, wn0, lane, acc);
+    if (more) stage((s + 1) & 1);
+    if (strings) {
+#pragma unroll
+      for (int x = 0; x < 4; ++x)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int v = __float_as_int(acc[x >> 1][x & 1][i]);
+          low[x >> 1][x & 1][i] = min(low[x >> 1][x & 1][i], v);
+          cnt[x >> 1][x & 1][i] = __builtin_amdgcn_alignbit(cnt[x >> 1][x & 1][i], (uint32_t)v, 31);
+        }
+    } else {
+#pragma unroll
+      for (int x = 0; x < 4; ++x)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int v = __float_as_int(acc[x >> 1][x & 1][i]);
+          low[x >> 1][x & 1][i] = min(low[x >> 1][x & 1][i], v);
+          cnt[x >> 1][x & 1][i] += (uint32_t)v >> 31;
+        }
+    }
+    __syncthreads();
+  }
+
+  // ---- slab in which the prefix passes t, and rem at its start
+#pragma unroll
+  for (int br = 0; br < 2; ++br)
+#pragma unroll
+    for (int bc = 0; bc < 2; ++bc) {
+      const int n = n0 + wn0 + bc * 32 + col;
+      if (RAGGED && n >= N) continue;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int m = m0 + wm0 + br * 32 + mfma_row(i, lane);
+        if (RAGGED && m >= M) continue;
+        const long cell = ((long)batch * M + m) * N + n;
+        const int below = strings ? __builtin_popcount(cnt[br][bc][i]) : (int)cnt[br][bc][i];
+        idx[cell] = below >= slabs ? 0 : -2 - below;
+        remw[cell] = -__int_as_float(low[br][bc][i]);
+      }
+    }
+}
+
 }  // namespace genbmm

@@ -147,8 +147,9 @@ int genbmm_prodmaxbmm_fwd(const float* a, const float* b, float* out,
  * out = log-sum-exp as genbmm_logbmm_fwd; idx[b,m,n] ~ Categorical(softmax_k
  * (a[m,k] + b[k,n])) by inverse CDF in ascending k against one uniform per
  * output cell.  The uniform of cell i = (b*M + m)*N + n is
- * (x >> 8) * 2^-24 with x = word 0 of Philox4x32-10(counter = {lo32(i),
- * hi32(i), lo32(offset), hi32(offset)}, key = {lo32(seed), hi32(seed)}).
+ * (x >> 8) * 2^-24 with x = word (i & 3) of Philox4x32-10(counter = {lo32(i >> 2),
+ * hi32(i >> 2), lo32(offset), hi32(offset)}, key = {lo32(seed), hi32(seed)}):
+ * four consecutive cells share one Philox block.
  * A cell whose scan never crosses its uniform keeps index 0, as in the
  * reference.  Replaces _genbmm.forward(a, b, 2): matmul_cuda_kernel.cu:512-526
  * (torch::rand at :517), kernel :77-121.

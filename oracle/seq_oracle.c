@@ -51,16 +51,17 @@ void orc_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t ou
   out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
 }
 
-/* Uniforms of cells first..first+count-1 of stream (seed, offset): word 0 of
- * Philox(counter = {lo(i), hi(i), lo(offset), hi(offset)}, key = {lo(seed),
- * hi(seed)}), top 24 bits scaled by 2^-24. */
+/* Uniforms of cells first..first+count-1 of stream (seed, offset): cell i takes word
+ * i & 3 of Philox(counter = {lo(i >> 2), hi(i >> 2), lo(offset), hi(offset)}, key =
+ * {lo(seed), hi(seed)}), top 24 bits scaled by 2^-24. */
 void orc_philox_uniform(uint64_t first, uint64_t count, uint64_t seed, uint64_t offset, float* out) {
   for (uint64_t e = 0; e < count; ++e) {
     uint64_t i = first + e;
-    uint32_t ctr[4] = {(uint32_t)i, (uint32_t)(i >> 32), (uint32_t)offset, (uint32_t)(offset >> 32)};
+    uint64_t blk = i >> 2;
+    uint32_t ctr[4] = {(uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)offset, (uint32_t)(offset >> 32)};
     uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
     uint32_t x[4];
     orc_philox4x32_10(ctr, key, x);
-    out[e] = (float)(x[0] >> 8) * (1.0f / 16777216.0f);
+    out[e] = (float)(x[i & 3] >> 8) * (1.0f / 16777216.0f);
   }
 }

@@ -42,13 +42,14 @@ def test_philox_known_answers(ctr, key, want):
 
 def test_philox_uniform_mapping():
     seed, offset = 0x1234_5678_9ABC_DEF0, 0x0FED_CBA9_8765_4321
-    first = (1 << 32) - 3  # crosses the 32-bit boundary of the cell index
-    u = oracle.philox_uniform(first, 8, seed, offset)
-    for e in range(8):
+    first = (1 << 34) - 6  # crosses the 32-bit boundary of the block index (cell >> 2)
+    u = oracle.philox_uniform(first, 12, seed, offset)
+    for e in range(12):
         i = first + e
-        x = oracle.philox4x32_10_py((i & 0xFFFFFFFF, i >> 32, offset & 0xFFFFFFFF, offset >> 32),
+        blk = i >> 2                       # four consecutive cells share one Philox block
+        x = oracle.philox4x32_10_py((blk & 0xFFFFFFFF, blk >> 32, offset & 0xFFFFFFFF, offset >> 32),
                                     (seed & 0xFFFFFFFF, seed >> 32))
-        assert float(u[e]) == (x[0] >> 8) / 16777216.0
+        assert float(u[e]) == (x[i & 3] >> 8) / 16777216.0
     big = oracle.philox_uniform(0, 200000, 1234, 0)
     assert 0.0 <= float(big.min()) and float(big.max()) < 1.0
     assert abs(float(big.mean()) - 0.5) < 0.005
