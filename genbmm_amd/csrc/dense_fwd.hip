@@ -145,14 +145,14 @@ static_assert(kMaxGroup == kResGroup, "");
 
 typedef float float4_u __attribute__((ext_vector_type(4), aligned(4)));
 
-template <int COLS, bool TAIL, class Op>
+template <int COLS, bool TAIL, int G, int R, class Op>
 __device__ __forceinline__ void resolve_walk(const float* __restrict__ first, const float* __restrict__ second,
                                              int32_t* __restrict__ idx, Op& op, int M, int K, int N,
                                              int panels, int row_chunks, int rows_per, float* Bs) {
   constexpr int RPW = 64 / COLS;           // rows a wave takes per step
   constexpr int KSTAGE = kResFloats / COLS;  // rows of the second operand staged at a time
-  constexpr int R = kResRows, G = kResGroup, STEP = kResWaves * R * RPW;
-  static_assert(KSTAGE % G == 0, "a group lies in one staged chunk");
+  constexpr int STEP = kResWaves * R * RPW;
+  static_assert(KSTAGE % G == 0 && G % 4 == 0, "a group lies in one staged chunk");
   const int lane = threadIdx.x & 63, col = lane % COLS, sub = lane / COLS;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   int wg = blockIdx.x;
@@ -261,11 +261,11 @@ __device__ __forceinline__ void resolve_walk(const float* __restrict__ first, co
 
 // Rows per workgroup (all of them unless that leaves the compute units short) and
 // the grid of a resolve launch.
-inline int resolve_grid(int B, int M, int N, int cols, int& panels, int& row_chunks, int& rows_per,
-                        unsigned& grid) {
+inline int resolve_grid(int B, int M, int N, int cols, int rows_step, int& panels, int& row_chunks,
+                        int& rows_per, unsigned& grid) {
   panels = ceil_div(N, cols);
   row_chunks = 1;
-  const int step = kResWaves * kResRows * (64 / cols);
+  const int step = kResWaves * rows_step * (64 / cols);
   while ((int64_t)B * panels * row_chunks < 1024 && ceil_div(M, row_chunks) > 2 * step) row_chunks *= 2;
   rows_per = ceil_div(M, row_chunks);
   row_chunks = ceil_div(M, rows_per);
@@ -338,7 +338,7 @@ __global__ __launch_bounds__(kResWaves * 64, 4) void k_max_resolve(
     int N, int panels, int row_chunks, int rows_per) {
   __shared__ float Bs[kResFloats];
   MaxResolve<PROD> op{out, idx, fac_a, fac_b};
-  resolve_walk<COLS, TAIL>(a, b, idx, op, M, K, N, panels, row_chunks, rows_per, Bs);
+  resolve_walk<COLS, TAIL, kResGroup, kResRows>(a, b, idx, op, M, K, N, panels, row_chunks, rows_per, Bs);
 }
 
 // ------------------------------------------------------------ sample forward
@@ -554,9 +554,10 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
   store_tile_i<C>(p.idx + (long)batch * M * N, ind, m0, n0, M, N, p.vec_o, tx, ty);
 }
 
-// Second level of the sampling sweep: rem at the start of the group goes through the
-// same multiply-adds as in the sweep; the index is the group's first term plus the
+// Second level of the sampling sweep: rem at the start of the group (G terms) goes
+// through multiply-adds term by term; the index is the group's first term plus the
 // number of terms after which rem is still >= 0 (rem only falls).
+template <int G>
 struct SampleResolve {
   typedef float Extra;
   const float* rem;
@@ -564,29 +565,30 @@ struct SampleResolve {
   int K;
   __device__ __forceinline__ float load(long e) const { return rem[e]; }
   __device__ __forceinline__ void none(long) const {}
-  __device__ __forceinline__ void cell(long e, int kb, const float (&av)[kResGroup], const float* br,
-                                       int stride, int valid, int staged, float r) const {
+  __device__ __forceinline__ void cell(long e, int kb, const float (&av)[G], const float* br, int stride,
+                                       int valid, int staged, float r) const {
     uint32_t past = 0u;
 #pragma unroll
-    for (int j = 0; j < kResGroup; ++j) {
+    for (int j = 0; j < G; ++j) {
       const float ea = j < valid ? av[j] : 0.f;
       r = __builtin_fmaf(-ea, br[min(j, staged - 1) * stride], r);
       past = __builtin_amdgcn_alignbit(past, __float_as_uint(r), 31);
     }
-    idx[e] = min(kb + kResGroup - __builtin_popcount(past), K - 1);
+    idx[e] = min(kb + G - __builtin_popcount(past), K - 1);
   }
 };
 
-template <int COLS, bool TAIL>
+template <int COLS, bool TAIL, int G>
 __global__ __launch_bounds__(kResWaves * 64, 4) void k_sample_resolve(
     const float* __restrict__ ea, const float* __restrict__ eb, const float* __restrict__ remw,
     int32_t* __restrict__ idx, int* __restrict__ valid, int M, int K, int N, int panels,
     int row_chunks, int rows_per) {
   __shared__ float Bs[kResFloats];
-  static_assert(kSampleGroup == kResGroup, "");
   if (blockIdx.x == 0 && threadIdx.x == 0) *valid = 0;  // the 1/S array of the workspace is gone
-  SampleResolve op{remw, idx, K};
-  resolve_walk<COLS, TAIL>(ea, eb, idx, op, M, K, N, panels, row_chunks, rows_per, Bs);
+  SampleResolve<G> op{remw, idx, K};
+  // 16-term groups: two rows per step keep the pipelined values within the registers
+  resolve_walk<COLS, TAIL, G, (G > 8 ? 2 : kResRows)>(ea, eb, idx, op, M, K, N, panels, row_chunks,
+                                                     rows_per, Bs);
 }
 
 // ---------------------------------------------------------------- dispatch
@@ -602,7 +604,7 @@ int launch_max(DenseArgs p, float* factors, int B, int M, int K, int N, hipStrea
   const int cols = K > 256 ? 32 : 64;  // 512 or 256 staged rows: one pass up to K = 512
   int panels, row_chunks, rows_per;
   unsigned rgrid;
-  if (int e = resolve_grid(B, M, N, cols, panels, row_chunks, rows_per, rgrid)) return e;
+  if (int e = resolve_grid(B, M, N, cols, kResRows, panels, row_chunks, rows_per, rgrid)) return e;
   auto go = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3(rgrid), dim3(kResWaves * 64), 0, s, p.a, p.b, p.out, p.idx, fa, fb,
                        M, K, N, panels, row_chunks, rows_per);
@@ -654,7 +656,32 @@ int launch_sweep(DenseArgs p, const float* stats, int B, int M, int K, int N, hi
   return launch_status();
 }
 
-// Two levels on the factors the logbmm forward left in the workspace.
+// Second level of a sweep that left group codes (groups of `group` terms) in idx and
+// rem in the workspace's scratch array.
+template <int G>
+int launch_sample_resolve(DenseArgs p, const LogFactors& f, int B, int M, int K, int N, hipStream_t s) {
+  const int cols = K > 256 ? 32 : 64;
+  int panels, row_chunks, rows_per;
+  unsigned rgrid;
+  if (int e = resolve_grid(B, M, N, cols, G > 8 ? 2 : kResRows, panels, row_chunks, rows_per, rgrid))
+    return e;
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(rgrid), dim3(kResWaves * 64), 0, s, f.ea, f.eb, f.scratch, p.idx,
+                       f.valid, M, K, N, panels, row_chunks, rows_per);
+  };
+  const bool tail = K % G != 0;
+  if (cols == 64) {
+    if (tail) go(k_sample_resolve<64, true, G>);
+    else go(k_sample_resolve<64, false, G>);
+  } else {
+    if (tail) go(k_sample_resolve<32, true, G>);
+    else go(k_sample_resolve<32, false, G>);
+  }
+  return launch_status();
+}
+
+// Two levels on the factors the logbmm forward left in the workspace, sweep on the
+// vector ALU.
 template <class C>
 int launch_sweep_two(DenseArgs p, const float* stats, const LogFactors& f, int B, int M, int K,
                      int N, hipStream_t s) {
@@ -663,23 +690,7 @@ int launch_sweep_two(DenseArgs p, const float* stats, const LogFactors& f, int B
   hipLaunchKernelGGL((k_sample_sweep<C, true>), grid, dim3(C::NT), 0, s, p, stats, f.ea, f.eb,
                      f.scratch);
   if (int e = launch_status()) return e;
-  const int cols = K > 256 ? 32 : 64;
-  int panels, row_chunks, rows_per;
-  unsigned rgrid;
-  if (int e = resolve_grid(B, M, N, cols, panels, row_chunks, rows_per, rgrid)) return e;
-  auto go = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, dim3(rgrid), dim3(kResWaves * 64), 0, s, f.ea, f.eb, f.scratch, p.idx,
-                       f.valid, M, K, N, panels, row_chunks, rows_per);
-  };
-  const bool tail = K % kSampleGroup != 0;
-  if (cols == 64) {
-    if (tail) go(k_sample_resolve<64, true>);
-    else go(k_sample_resolve<64, false>);
-  } else {
-    if (tail) go(k_sample_resolve<32, true>);
-    else go(k_sample_resolve<32, false>);
-  }
-  return launch_status();
+  return launch_sample_resolve<kSampleGroup>(p, f, B, M, K, N, s);
 }
 
 int run_sample(const float* a, const float* b, float* out, int32_t* idx, float* stats,
@@ -696,6 +707,10 @@ int run_sample(const float* a, const float* b, float* out, int32_t* idx, float* 
     if (int e = genbmm_logbmm_fwd(a, b, out, stats, B, M, K, N, stream)) return e;
     LogFactors f;
     if (log_fwd_writes_factors(stats, B, M, K, N, &f)) {
+      if (log_sample_mfma_ok(K)) {  // sweep on the matrix cores, groups of 16 terms
+        if (int e = log_sample_sweep_mfma(a, b, out, idx, stats, seed, offset, B, M, K, N, s)) return e;
+        return launch_sample_resolve<16>(p, f, B, M, K, N, s);
+      }
       switch (pick_shape(B, M, N, false)) {
         case kWide: return launch_sweep_two<CfgWide>(p, stats, f, B, M, K, N, s);
         default: return launch_sweep_two<CfgMid>(p, stats, f, B, M, K, N, s);

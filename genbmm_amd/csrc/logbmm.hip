@@ -285,6 +285,28 @@ __global__ __launch_bounds__(CX::NT) void k_log_fwd_fixup(const DenseArgs p,
   }
 }
 
+// The same for samplebmm: log-sum-exp and index of the flagged tiles by the exact walk.
+template <class CX, int FBM, int FBN>
+__global__ __launch_bounds__(CX::NT) void k_sample_fixup(const DenseArgs p,
+                                                         const int* __restrict__ flags,
+                                                         int total_tiles) {
+  static_assert(FBM % CX::BM == 0 && FBN % CX::BN == 0, "");
+  __shared__ __attribute__((aligned(16))) float smem[CX::KT * (CX::LDA + CX::LDB)];
+  const int per = p.tiles_m * p.tiles_n;
+  for (int t = blockIdx.x; t < total_tiles; t += gridDim.x) {
+    if (!flags[t]) continue;
+    const int batch = t / per, r = t - batch * per;
+    const int m0 = (r / p.tiles_n) * FBM, n0 = (r % p.tiles_n) * FBN;
+    for (int h = 0; h < FBM / CX::BM; ++h)
+      for (int w = 0; w < FBN / CX::BN; ++w)
+        if (m0 + h * CX::BM < p.M && n0 + w * CX::BN < p.N) {
+          log_fwd_tile<CX, true>(p, batch, m0 + h * CX::BM, n0 + w * CX::BN, smem,
+                                 smem + CX::KT * CX::LDA);
+          __syncthreads();
+        }
+  }
+}
+
 template <class CX, int FBR, int FBC, bool GRAD_A>
 __global__ __launch_bounds__(CX::NT) void k_log_bwd_fixup(const LogBwdArgs p,
                                                           const int* __restrict__ flags,
@@ -636,6 +658,28 @@ int launch_fwd_mfma(DenseArgs p, const float* stats, int* flags, int B, int M, i
   return launch_fwd_fixup<CfgWide, T::TR, T::TC>(p, flags, total, s);
 }
 
+template <class T>
+int launch_sample_sweep_mfma(DenseArgs p, const float* stats, int* flags, int B, int M, int K, int N,
+                             hipStream_t s) {
+  p.M = M; p.K = K; p.N = N;
+  p.tiles_m = ceil_div(M, T::TR);
+  p.tiles_n = ceil_div(N, T::TC);
+  p.vec_a = (K % 4 == 0) && aligned16(p.a);
+  p.vec_b = (N % 4 == 0) && aligned16(p.b);
+  p.vec_o = (N % 4 == 0) && aligned16(p.out) && aligned16(p.idx);
+  const int total = B * p.tiles_m * p.tiles_n;
+  const LogPrepared ws = prepared_of(stats, B, M, K, N);
+  auto go = [&](auto kern) {
+    hipLaunchKernelGGL(kern, dim3(total), dim3(T::NT), 0, s, ws.ea, ws.eb, p.out, stats, flags, ws.r,
+                       p.idx, p.seed, p.offset, M, K, N, p.tiles_m, p.tiles_n);
+  };
+  go(k_sample_sweep_mfma<T>);
+  if (int e = launch_status()) return e;
+  hipLaunchKernelGGL((k_sample_fixup<CfgWide, T::TR, T::TC>), dim3(min(total, kFixupGrid)),
+                     dim3(CfgWide::NT), 0, s, p, flags, total);
+  return launch_status();
+}
+
 int launch_stats(const float* a, const float* b, float* stats, int B, int M, int K, int N,
                  hipStream_t s) {
   const int row_wgs = ceil_div(M, kStatRows), col_wgs = ceil_div(N, kStatCols);
@@ -782,6 +826,23 @@ bool log_fwd_writes_factors(const float* stats, int B, int M, int K, int N, LogF
   f->scratch = ws.r;
   f->valid = ws.hdr;
   return true;
+}
+
+bool log_sample_mfma_ok(int K) { return ceil_div(K, kMS) <= kSampleSlabs; }
+
+int log_sample_sweep_mfma(const float* a, const float* b, float* out, int32_t* idx,
+                          const float* stats, uint64_t seed, uint64_t offset, int B, int M, int K,
+                          int N, hipStream_t s) {
+  DenseArgs p{};
+  p.a = a; p.b = b; p.out = out; p.idx = idx; p.seed = seed; p.offset = offset;
+  if (ceil_div(K, kMS) > kSampleSlabs) return GENBMM_E_SHAPE;  // the caller checks log_sample_mfma_ok
+  int* fl = flags_of(stats, B, M, K, N, 0);
+  // the forward's tile shape: its flags are indexed by it
+  switch (mfma_kind(B, M, N, K, true, false)) {
+    case 2: return launch_sample_sweep_mfma<MTTall>(p, stats, fl, B, M, K, N, s);
+    case 1: return launch_sample_sweep_mfma<MT128>(p, stats, fl, B, M, K, N, s);
+    default: return GENBMM_E_SHAPE;
+  }
 }
 
 }  // namespace genbmm

@@ -633,22 +633,31 @@ void k_log_bwd_mfma_both(const float* __restrict__ g, const float* __restrict__ 
 // samplebmm on the forward's factors: index = first k whose prefix sum
 // sum_{k' <= k} EA[m,k'] EB[k',n] passes the target t = u * S (one Philox uniform
 // u per cell, S = exp(out - alpha - beta)).  The accumulators start at -t, so after
-// every slab they hold prefix - t.  Per slab and cell two vector instructions look
-// at that value: its sign bit (prefix still below t) is shifted into a bit string
-// (slabs <= 32) or added to a counter, and a signed-integer minimum keeps the
-// negative value closest to zero (negative floats order backwards as integers and
-// lie below every non-negative one) - minus that is rem = t - prefix at the start
-// of the slab in which the prefix passes t.  Results: the code -2 - slab in idx (0
-// if the prefix never reaches t) and rem in `remw`; the terms of that one slab are
-// walked by the resolve kernel.  A tile with a cell whose S is below 2^-40 or not
-// finite, or that the forward flagged, sets its flag and leaves: it is redone exactly.
-template <class T, bool RAGGED>
-__global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::NT / 256, T::NT / 256)))
+// every slab they hold prefix - t: negative while the prefix is below the target, and
+// closer to zero slab by slab.  One register per cell keeps what is needed of that
+// history: the low six bits of the value's bit pattern are replaced by 62 - slab and
+// a signed-integer minimum is taken (negative floats order backwards as integers and
+// lie below every non-negative one; of two slabs the later has the smaller magnitude
+// and the smaller tag, so it always wins).  At the end the tag gives the number of
+// slabs that ended below the target = the slab in which the prefix passes it, and the
+// value (six mantissa bits short) is -(t - prefix at the start of that slab) = -rem.
+// Two vector instructions per cell and slab beside the matrix-core work.  Results:
+// the code -2 - slab in idx (0 if the prefix never reaches t) and rem in `remw`; the
+// terms of that one slab are walked by the resolve kernel.  At most kSampleSlabs
+// slabs (the tag's range).  A tile with a cell whose S is below 2^-40 or not finite,
+// or that the forward flagged, sets its flag and leaves: it is redone exactly.
+constexpr int kSampleSlabs = 62;
+
+// (Always the any-size form of the loaders: with this kernel's register budget the
+// full-tile form compiled to spills and measured no faster.)
+template <class T>
+__global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void k_sample_sweep_mfma(const float* __restrict__ ws_ea, const float* __restrict__ ws_eb,
                          const float* __restrict__ out, const float* __restrict__ stats,
                          int* __restrict__ flags, float* __restrict__ remw,
                          int32_t* __restrict__ idx, uint64_t seed, uint64_t offset, int M, int K,
                          int N, int tiles_m, int tiles_n) {
+  constexpr bool RAGGED = true;
   constexpr int NT = T::NT, LDR = T::LDR, LDC = T::LDC;
   using SA = StageT<T::TR, NT, LDR>;
   using SB = StageS<T::TC, NT, LDC>;
@@ -663,41 +672,57 @@ void k_sample_sweep_mfma(const float* __restrict__ ws_ea, const float* __restric
   const int m0 = (rem / tiles_n) * T::TR, n0 = (rem % tiles_n) * T::TC;
   const float* st = stats + (long)batch * (M + N);
 
-  // ---- targets: acc = -t, low = its bit pattern, in the accumulator layout
-  floatx16 acc[2][2];
-  int low[2][2][16];
-  uint32_t cnt[2][2][16];
-  const int col = lane & 31;
+  // ---- targets.  First -t = -u * S per cell into `remw`, row by row, four adjacent
+  // cells per lane and step (they share one Philox block when rows are a multiple of
+  // four cells); a rolled loop, its body is long.  Then the accumulators pick their
+  // cells up in the matrix-core layout.
   const float lim = kMfmaGuardBits * kLn2 + 1e-3f;
   int bad = flags[tile];
+  {
+    constexpr int QR = T::TC / 4;  // quads per tile row
+    const bool blocks = (N & 3) == 0;
+    for (int q = tid; q < T::TR * QR; q += NT) {
+      const int r = q / QR, m = m0 + r, n = n0 + (q - r * QR) * 4;
+      if (RAGGED && (m >= M || n >= N)) continue;
+      const long cell = ((long)batch * M + m) * N + n;
+      const int cn = RAGGED ? clamp4(N - n) : 4;
+      float u[4];
+      philox_uniform4((uint64_t)cell, blocks, seed, offset, u);
+      const float alr = st[m];
+      const float4 be4 = ld4m(st + M + n, cn, 0.f), o4 = ld4m(out + cell, cn, 0.f);
+      const float bev[4] = {be4.x, be4.y, be4.z, be4.w}, ov[4] = {o4.x, o4.y, o4.z, o4.w};
+      float tv[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float e = alr + bev[j] - ov[j];  // -log S
+        if (j < cn && (!(e <= lim) || !(e > -INFINITY))) bad = 1;
+        tv[j] = -u[j] * fast_exp2(-e * kLog2e);
+      }
+      st4m(remw + cell, cn, make_float4(tv[0], tv[1], tv[2], tv[3]));
+    }
+  }
+  bad = __syncthreads_or(bad);  // also: the tile's -t are visible to the whole workgroup
+  if (bad) {
+    if (tid == 0) flags[tile] = 1;
+    return;
+  }
+  floatx16 acc[2][2];
+  int low[2][2][16];
+  const int col = lane & 31;
 #pragma unroll
   for (int br = 0; br < 2; ++br)
 #pragma unroll
     for (int bc = 0; bc < 2; ++bc) {
       const int n = n0 + wn0 + bc * 32 + col;
-      const bool nok = !RAGGED || n < N;
-      const float be = nok ? st[M + n] : 0.f;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int m = m0 + wm0 + br * 32 + mfma_row(i, lane);
-        const bool ok = nok && (!RAGGED || m < M);
-        float t = 0.f;
-        if (ok) {
-          const long cell = ((long)batch * M + m) * N + n;
-          const float e = st[m] + be - out[cell];  // -log S
-          if (!(e <= lim) || !(e > -INFINITY)) bad = 1;
-          t = philox_uniform((uint64_t)cell, seed, offset) * fast_exp2(-e * kLog2e);
-        }
-        acc[br][bc][i] = -t;
-        low[br][bc][i] = __float_as_int(-t);
-        cnt[br][bc][i] = 0u;
+        const bool ok = !RAGGED || (m < M && n < N);
+        const float nt = ok ? remw[((long)batch * M + m) * N + n] : 0.f;
+        acc[br][bc][i] = nt;
+        low[br][bc][i] = __float_as_int(nt) | 63;  // tag 63: no slab has ended below t
       }
     }
-  bad = __syncthreads_or(bad);
-  if (bad) {
-    if (tid == 0) flags[tile] = 1;
-    return;
-  }
 
   // ---- staging of EA (transposed) and EB, one slab ahead
   const int bcol = n0 + SB::quad(tid) * 4;
@@ -744,7 +769,6 @@ void k_sample_sweep_mfma(const float* __restrict__ ws_ea, const float* __restric
     for (int l = 0; l < SB::PER; ++l) SB::put(Bs[buf], tid, l, rb[l]);
   };
 
-  const bool strings = slabs <= 32;  // one bit per slab fits the register
   load(slabs == 1 && ktail != 0);
   stage(0);
   __syncthreads();
@@ -753,25 +777,14 @@ void k_sample_sweep_mfma(const float* __restrict__ ws_ea, const float* __restric
     if (more) load(s + 2 == slabs && ktail != 0);
     mfma_slab<LDR, LDC>(As[s & 1], Bs[s & 1], wm0, wn0, lane, acc);
     if (more) stage((s + 1) & 1);
-    if (strings) {
+    const int tag = 62 - s;
 #pragma unroll
-      for (int x = 0; x < 4; ++x)
+    for (int x = 0; x < 4; ++x)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int v = __float_as_int(acc[x >> 1][x & 1][i]);
-          low[x >> 1][x & 1][i] = min(low[x >> 1][x & 1][i], v);
-          cnt[x >> 1][x & 1][i] = __builtin_amdgcn_alignbit(cnt[x >> 1][x & 1][i], (uint32_t)v, 31);
-        }
-    } else {
-#pragma unroll
-      for (int x = 0; x < 4; ++x)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int v = __float_as_int(acc[x >> 1][x & 1][i]);
-          low[x >> 1][x & 1][i] = min(low[x >> 1][x & 1][i], v);
-          cnt[x >> 1][x & 1][i] += (uint32_t)v >> 31;
-        }
-    }
+      for (int i = 0; i < 16; ++i) {
+        const int v = (__float_as_int(acc[x >> 1][x & 1][i]) & ~63) | tag;
+        low[x >> 1][x & 1][i] = min(low[x >> 1][x & 1][i], v);
+      }
     __syncthreads();
   }
 
@@ -787,9 +800,9 @@ void k_sample_sweep_mfma(const float* __restrict__ ws_ea, const float* __restric
         const int m = m0 + wm0 + br * 32 + mfma_row(i, lane);
         if (RAGGED && m >= M) continue;
         const long cell = ((long)batch * M + m) * N + n;
-        const int below = strings ? __builtin_popcount(cnt[br][bc][i]) : (int)cnt[br][bc][i];
+        const int below = 63 - (low[br][bc][i] & 63);
         idx[cell] = below >= slabs ? 0 : -2 - below;
-        remw[cell] = -__int_as_float(low[br][bc][i]);
+        remw[cell] = -__int_as_float(low[br][bc][i] & ~63);
       }
     }
 }

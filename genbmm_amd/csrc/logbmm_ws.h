@@ -2,6 +2,9 @@
 // library (the sampling sweep reads the factors instead of taking exponentials again).
 #pragma once
 
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
 namespace genbmm {
 
 struct LogFactors {
@@ -14,5 +17,15 @@ struct LogFactors {
 // True (and *f filled) if a genbmm_logbmm_fwd call with this workspace and these sizes
 // writes the factors: the same decision the forward takes, made on the host.
 bool log_fwd_writes_factors(const float* stats, int B, int M, int K, int N, LogFactors* f);
+
+// For a workspace that log_fwd_writes_factors() accepts: the sampling sweep on the
+// matrix cores.  Leaves in idx the code -2 - group (groups of 16 terms; 0: the prefix
+// sums never reach the target) and in the scratch array rem at the start of that
+// group; tiles that the forward or the sweep flagged are redone exactly (out and the
+// final index).  The caller resolves the codes.
+bool log_sample_mfma_ok(int K);  // the sweep below takes reductions up to 62 slabs of 16 terms
+int log_sample_sweep_mfma(const float* a, const float* b, float* out, int32_t* idx,
+                          const float* stats, uint64_t seed, uint64_t offset, int B, int M, int K,
+                          int N, hipStream_t s);
 
 }  // namespace genbmm
