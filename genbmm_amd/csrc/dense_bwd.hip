@@ -92,42 +92,74 @@ __global__ __launch_bounds__(256) void k_log_bwdbwd_b(const BB p, long total) {
 //                      grad_b[k,n] = sum_m [k == idx[m,n]] g[m,n]
 // prodmaxbmm: the terms are b[k,n]*g[m,n] and a[m,k]*g[m,n].
 // (reference matmul_cuda_kernel.cu:336-456: one thread per gradient cell
-// scanning the whole reduction axis, O(M*K*N).)  Here one lane owns one row m
-// (resp. column n) and walks it once in ascending n (resp. m), adding each
-// term into the cell idx selects, in an LDS-resident accumulator row; the
-// additions hitting a given cell therefore happen in the reference's order,
-// so the result is bit-identical, in O(M*N) work.  Products are rounded
-// before the add (the build uses -ffp-contract=on: no fusion across statements).
-constexpr int kKC = 128;  // gradient columns/rows accumulated per workgroup
+// scanning the whole reduction axis, O(M*K*N).)  Here a lane owns a row m (resp.
+// column n) and a range of k, walks the row once in ascending n (resp. the column
+// in ascending m) and adds each term whose idx falls into its range to that
+// cell of an LDS-resident accumulator; the additions hitting a given cell
+// therefore happen in the reference's order, so the result is bit-identical, in
+// O(M*N) work.  Products are rounded before the add (the build uses
+// -ffp-contract=on: no fusion across statements).
+constexpr int kKC = 128;  // cells of the reduction axis per lane
 
-// One wave: lane = row m of a 64-row tile, k in [c0, c0 + kKC).  The row is read
-// 16 cells at a time (int4 / float4 when the rows are 16-byte aligned), then the
-// 16 additions are made in order.
-// PROD: 0 plain sum of g, 1 times b[idx, n] gathered from b, 2 times the factor the
-// forward stored per cell (fac[m,n] = b[idx[m,n], n], read like g).
+// The 64 lanes of a workgroup are (line, part): 64 >> ps lines (rows m of grad_a,
+// columns n of grad_b) times 2^ps parts of kKC consecutive k, so that one workgroup
+// covers every k of its lines (up to 64 * kKC; longer K: further workgroups) and idx
+// and g are read from memory once - the lanes of a line read the same addresses.
+// Each lane walks its whole line and adds the terms whose k falls into its part.
+
+// Four ordered additions with one LDS round trip: the four cells are read together,
+// the sums are chained in registers (a cell that was already hit earlier in the group
+// takes that sum instead of what it read), and written back in order.  A term whose k
+// is not this lane's goes to the lane's spare cell.
+__device__ __forceinline__ void add4_ordered(float* __restrict__ accs, const int (&s)[4],
+                                             const float (&v)[4]) {
+  const float r0 = accs[s[0]], r1 = accs[s[1]], r2 = accs[s[2]], r3 = accs[s[3]];
+  const float v0 = __fadd_rn(r0, v[0]);
+  const float v1 = __fadd_rn(s[1] == s[0] ? v0 : r1, v[1]);
+  const float v2 = __fadd_rn(s[2] == s[1] ? v1 : (s[2] == s[0] ? v0 : r2), v[2]);
+  const float v3 = __fadd_rn(s[3] == s[2] ? v2 : (s[3] == s[1] ? v1 : (s[3] == s[0] ? v0 : r3)), v[3]);
+  accs[s[0]] = v0;
+  accs[s[1]] = v1;
+  accs[s[2]] = v2;
+  accs[s[3]] = v3;
+}
+
+// grad_a: line = row m.  The row is read 16 cells at a time (int4 / float4 when the
+// rows are 16-byte aligned), then the 16 additions are made in order.
 template <int PROD>
 __global__ __launch_bounds__(64) void k_argmax_bwd_a(const float* __restrict__ bmat,
                                                     const float* __restrict__ fac,
                                                     const int32_t* __restrict__ idx,
                                                     const float* __restrict__ g,
                                                     float* __restrict__ grad_a, int M, int K,
-                                                    int N, int row_tiles, int k_chunks, int vec) {
-  __shared__ float accs[64 * (kKC + 1)];
-  const int lane = threadIdx.x;
+                                                    int N, int row_tiles, int k_chunks, int ps,
+                                                    int vec) {
+  __shared__ float accs[64 * kKC + 64 + 64];
+  const int lane = threadIdx.x, parts = 1 << ps, lines = 64 >> ps;
+  const int part = lane & (parts - 1), line = lane >> ps;
+  const int spare = 64 * kKC + 64 + lane;
   const int kc_id = blockIdx.x % k_chunks, rt = blockIdx.x / k_chunks;
   const int batch = rt / row_tiles;
-  const int m0 = (rt - batch * row_tiles) * 64;
-  const int c0 = kc_id * kKC, kc = min(kKC, K - c0);
-  const int m = m0 + lane;
+  const int m0 = (rt - batch * row_tiles) * lines;
+  const int kw = parts * kKC;                       // k covered by the workgroup
+  const int w0 = kc_id * kw, c0 = w0 + part * kKC;  // first k of the workgroup / of this lane
+  const int kc = min(kKC, K - c0);                  // <= 0: the part lies beyond K
+  const int m = m0 + line;
   const bool live = m < M;
   const int32_t* irow = idx + ((long)batch * M + (live ? m : 0)) * N;
   const float* grow = g + ((long)batch * M + (live ? m : 0)) * N;
   const float* bb = PROD == 1 ? bmat + (long)batch * K * N : nullptr;
   const float* frow = PROD == 2 ? fac + ((long)batch * M + (live ? m : 0)) * N : nullptr;
-  float* mine = accs + lane * (kKC + 1);
+  const int base = line * (kw + 1) + part * kKC;
+  float* mine = accs + base;
   for (int kk = 0; kk < kKC; ++kk) mine[kk] = 0.f;
+  accs[spare] = 0.f;
+  auto slot = [&](int ki) __attribute__((always_inline)) {
+    const int k = ki - c0;
+    return (k >= 0 && k < kc) ? base + k : spare;
+  };
   // the term of cell n: g, times b[idx, n] for the product semiring (read only when
-  // the index falls into this workgroup's k range)
+  // the index falls into this lane's k range)
   auto term = [&](int n, int ki, float gv) __attribute__((always_inline)) {
     const int k = ki - c0;
     if (PROD == 1 && k >= 0 && k < kc) return __fmul_rn(bb[(long)ki * N + n], gv);
@@ -168,10 +200,9 @@ __global__ __launch_bounds__(64) void k_argmax_bwd_a(const float* __restrict__ b
         }
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          add(iv[q].x, gv[q].x);
-          add(iv[q].y, gv[q].y);
-          add(iv[q].z, gv[q].z);
-          add(iv[q].w, gv[q].w);
+          const int sl[4] = {slot(iv[q].x), slot(iv[q].y), slot(iv[q].z), slot(iv[q].w)};
+          const float tv[4] = {gv[q].x, gv[q].y, gv[q].z, gv[q].w};
+          add4_ordered(accs, sl, tv);
         }
       }
     }
@@ -179,34 +210,46 @@ __global__ __launch_bounds__(64) void k_argmax_bwd_a(const float* __restrict__ b
       add(irow[n], PROD == 2 ? __fmul_rn(frow[n], grow[n]) : term(n, irow[n], grow[n]));
   }
   __syncthreads();
-  const int rows = min(64, M - m0);
+  const int rows = min(lines, M - m0), kn = min(kw, K - w0);
   for (int r = 0; r < rows; ++r) {
-    float* dst = grad_a + ((long)batch * M + m0 + r) * K + c0;
-    for (int kk = lane; kk < kc; kk += 64) dst[kk] = accs[r * (kKC + 1) + kk];
+    float* dst = grad_a + ((long)batch * M + m0 + r) * K + w0;
+    for (int kk = lane; kk < kn; kk += 64) dst[kk] = accs[r * (kw + 1) + kk];
   }
 }
 
-// One wave: lane = column n of a 64-column tile, k in [c0, c0 + kKC); the column is
-// read 8 rows at a time (coalesced across the lanes), then added in order.
+// grad_b: line = column n; the column is read 16 rows at a time, then added in order.
+// Accumulators are [k][line].
 template <int PROD>
 __global__ __launch_bounds__(64) void k_argmax_bwd_b(const float* __restrict__ amat,
                                                     const float* __restrict__ fac,
                                                     const int32_t* __restrict__ idx,
                                                     const float* __restrict__ g,
                                                     float* __restrict__ grad_b, int M, int K,
-                                                    int N, int col_tiles, int k_chunks) {
-  __shared__ float accs[kKC * 64];
-  const int lane = threadIdx.x;
+                                                    int N, int col_tiles, int k_chunks, int ps) {
+  __shared__ float accs[kKC * 64 + 64];
+  const int lane = threadIdx.x, parts = 1 << ps, lines = 64 >> ps;
+  const int part = lane & (parts - 1), line = lane >> ps;
+  const int spare = kKC * 64 + lane;
   const int kc_id = blockIdx.x % k_chunks, ct = blockIdx.x / k_chunks;
   const int batch = ct / col_tiles;
-  const int n = (ct - batch * col_tiles) * 64 + lane;
-  const int c0 = kc_id * kKC, kc = min(kKC, K - c0);
-  if (n >= N) return;  // lanes are independent: no barriers below
-  const int32_t* icol = idx + (long)batch * M * N + n;
-  const float* gcol = g + (long)batch * M * N + n;
+  const int n0 = (ct - batch * col_tiles) * lines, n = n0 + line;
+  const int kw = parts * kKC;
+  const int w0 = kc_id * kw, c0 = w0 + part * kKC;
+  const int kc = min(kKC, K - c0);
+  const bool live = n < N;
+  const int nn = live ? n : N - 1;
+  const int32_t* icol = idx + (long)batch * M * N + nn;
+  const float* gcol = g + (long)batch * M * N + nn;
   const float* ab = PROD == 1 ? amat + (long)batch * M * K : nullptr;
-  const float* fcol = PROD == 2 ? fac + (long)batch * M * N + n : nullptr;
-  for (int kk = 0; kk < kKC; ++kk) accs[kk * 64 + lane] = 0.f;
+  const float* fcol = PROD == 2 ? fac + (long)batch * M * N + nn : nullptr;
+  const int base = (part * kKC) * lines + line;  // cell k of this lane: accs[base + k * lines]
+  float* mine = accs + base;
+  for (int kk = 0; kk < kKC; ++kk) mine[kk * lines] = 0.f;
+  accs[spare] = 0.f;
+  auto slot = [&](int ki) __attribute__((always_inline)) {
+    const int k = ki - c0;
+    return (k >= 0 && k < kc) ? base + k * lines : spare;
+  };
   auto term = [&](int m, int ki, float gv) __attribute__((always_inline)) {
     const int k = ki - c0;
     if (PROD == 1 && k >= 0 && k < kc) return __fmul_rn(ab[(long)m * K + ki], gv);
@@ -215,25 +258,44 @@ __global__ __launch_bounds__(64) void k_argmax_bwd_b(const float* __restrict__ a
   };
   auto add = [&](int ki, float v) __attribute__((always_inline)) {
     const int k = ki - c0;
-    if (k >= 0 && k < kc) accs[k * 64 + lane] = __fadd_rn(accs[k * 64 + lane], v);
+    if (k >= 0 && k < kc) mine[k * lines] = __fadd_rn(mine[k * lines], v);
   };
-  int m = 0;
-  for (; m + 8 <= M; m += 8) {
-    int iv[8];
-    float gv[8];
+  if (live) {
+    int m = 0;
+    for (; m + 16 <= M; m += 16) {
+      int iv[16];
+      float gv[16];
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      iv[q] = icol[(long)(m + q) * N];
-      gv[q] = gcol[(long)(m + q) * N];
+      for (int q = 0; q < 16; ++q) {
+        iv[q] = icol[(long)(m + q) * N];
+        gv[q] = gcol[(long)(m + q) * N];
+      }
+#pragma unroll
+      for (int q = 0; q < 16; ++q) gv[q] = term(m + q, iv[q], gv[q]);
+#pragma unroll
+      for (int q = 0; q < 16; q += 4) {
+        const int sl[4] = {slot(iv[q]), slot(iv[q + 1]), slot(iv[q + 2]), slot(iv[q + 3])};
+        const float tv[4] = {gv[q], gv[q + 1], gv[q + 2], gv[q + 3]};
+        add4_ordered(accs, sl, tv);
+      }
     }
-#pragma unroll
-    for (int q = 0; q < 8; ++q) gv[q] = term(m + q, iv[q], gv[q]);
-#pragma unroll
-    for (int q = 0; q < 8; ++q) add(iv[q], gv[q]);
+    for (; m < M; ++m) add(icol[(long)m * N], term(m, icol[(long)m * N], gcol[(long)m * N]));
   }
-  for (; m < M; ++m) add(icol[(long)m * N], term(m, icol[(long)m * N], gcol[(long)m * N]));
-  for (int kk = 0; kk < kc; ++kk)
-    grad_b[((long)batch * K + c0 + kk) * N + n] = accs[kk * 64 + lane];
+  __syncthreads();
+  // rows k of the result: `lines` consecutive columns each
+  const int cols = min(lines, N - n0), kn = min(kw, K - w0);
+  const int lc = lane & (lines - 1), lk = lane / lines;
+  if (lc < cols)
+    for (int kk = lk; kk < kn; kk += parts)
+      grad_b[((long)batch * K + w0 + kk) * N + n0 + lc] = accs[kk * lines + lc];
+}
+
+// Parts per workgroup for a reduction axis of K cells: the smallest power of two that
+// covers it (at most 64).
+inline int argmax_parts_shift(int K) {
+  int ps = 0;
+  while (ps < 6 && (kKC << ps) < K) ++ps;
+  return ps;
 }
 
 template <bool PROD>
@@ -249,29 +311,33 @@ int run_argmax_bwd(const float* a, const float* b, const int32_t* idx, const flo
   constexpr int kGather = PROD ? 1 : 0;
   hipStream_t s = (hipStream_t)stream;
   if ((int64_t)B * M * K > 0) {
-    const int row_tiles = ceil_div(M, 64), k_chunks = ceil_div(K, kKC);
+    const int ps = argmax_parts_shift(K);
+    const int row_tiles = ceil_div(M, 64 >> ps), k_chunks = ceil_div(K, kKC << ps);
     const int64_t total = (int64_t)B * row_tiles * k_chunks;
     if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
     const int vec = (N % 4 == 0) && aligned16(idx) && aligned16(g);
     if (PROD && factors && mn > 0)
       hipLaunchKernelGGL((k_argmax_bwd_a<2>), dim3((unsigned)total), dim3(64), 0, s, b,
                          factors + mn, idx, g, grad_a, M, K, N, row_tiles,
-                         k_chunks, vec && aligned16(factors + mn));
+                         k_chunks, ps, vec && aligned16(factors + mn));
     else
       hipLaunchKernelGGL((k_argmax_bwd_a<kGather>), dim3((unsigned)total), dim3(64), 0, s, b,
-                         (const float*)nullptr, idx, g, grad_a, M, K, N, row_tiles, k_chunks, vec);
+                         (const float*)nullptr, idx, g, grad_a, M, K, N, row_tiles, k_chunks, ps, vec);
     if (int e = launch_status()) return e;
   }
   if ((int64_t)B * K * N > 0) {
-    const int col_tiles = ceil_div(N, 64), k_chunks = ceil_div(K, kKC);
+    // columns: two parts at most - narrower groups of columns cost more in the strided
+    // reads of idx and g than reading them again saves
+    const int ps = min(argmax_parts_shift(K), 1);
+    const int col_tiles = ceil_div(N, 64 >> ps), k_chunks = ceil_div(K, kKC << ps);
     const int64_t total = (int64_t)B * col_tiles * k_chunks;
     if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
     if (PROD && factors && mn > 0)
       hipLaunchKernelGGL((k_argmax_bwd_b<2>), dim3((unsigned)total), dim3(64), 0, s, a, factors,
-                         idx, g, grad_b, M, K, N, col_tiles, k_chunks);
+                         idx, g, grad_b, M, K, N, col_tiles, k_chunks, ps);
     else
       hipLaunchKernelGGL((k_argmax_bwd_b<kGather>), dim3((unsigned)total), dim3(64), 0, s, a,
-                         (const float*)nullptr, idx, g, grad_b, M, K, N, col_tiles, k_chunks);
+                         (const float*)nullptr, idx, g, grad_b, M, K, N, col_tiles, k_chunks, ps);
     if (int e = launch_status()) return e;
   }
   return GENBMM_OK;
