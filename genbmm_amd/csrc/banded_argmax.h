@@ -25,9 +25,10 @@ constexpr int kAJ = 32;        // diagonals per tile
 constexpr int kAC = kAJ + 1;   // tile row stride
 constexpr int kAS = kAT + 1;   // accumulator stride
 
-inline size_t argmax_bwd_a_bytes(int Wa) { return sizeof(float) * ((size_t)Wa * kAS + 2 * kAT * kAC); }
+// accumulators [W][65], one spare cell per lane (terms that are not the lane's), tiles
+inline size_t argmax_bwd_a_bytes(int Wa) { return sizeof(float) * ((size_t)Wa * kAS + 256 + 2 * kAT * kAC); }
 inline size_t argmax_bwd_b_bytes(int Wb) {
-  return sizeof(float) * ((size_t)Wb * kAS + 2 * (kAT + kAJ - 1) * kAC);
+  return sizeof(float) * ((size_t)Wb * kAS + 256 + 2 * (kAT + kAJ - 1) * kAC);
 }
 
 // Tile of ROWS x 32 cells of g and idx: load() starts the global reads (masked
@@ -66,19 +67,21 @@ struct ArgTile {
 
 // Four waves per strip: all walk the same cells in the same order, wave w adds
 // only the cells whose target index is w mod 4, so the per-target order is kept
-// and the dependent read-modify-write chains are a quarter as long.
+// and the dependent read-modify-write chains are a quarter as long; the additions
+// go four at a time through add4_ordered (one LDS round trip for four cells).
 __global__ __launch_bounds__(256) void k_band_argmax_bwd_a(const BandArgs p, int strips) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   const int n = p.n, Wa = p.Wa, Wo = p.Wo;
-  float* acc = smem;                                      // [Wa][65]
-  float* gt = acc + Wa * kAS;                             // [64][33]
+  float* acc = smem;                                      // [Wa][65] + 256 spare cells
+  float* gt = acc + Wa * kAS + 256;                       // [64][33]
   int* it = reinterpret_cast<int*>(gt + kAT * kAC);       // [64][33]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int batch = blockIdx.x / strips, i0 = (blockIdx.x - batch * strips) * kAT;
   const long bn = (long)batch * n;
   const float* gb = p.g + bn * Wo;
   const int32_t* ib = p.idx + bn * Wo;
-  for (int e = tid; e < Wa * kAS; e += 256) acc[e] = 0.f;
+  for (int e = tid; e < Wa * kAS + 256; e += 256) acc[e] = 0.f;
+  const int spare = Wa * kAS + tid;
   ArgTile<kAT> tile;
   tile.load(gb, ib, i0, 0, n, Wo, p.r_lu, true, tid);
   for (int jc = 0; jc < Wo; jc += kAJ) {
@@ -86,10 +89,17 @@ __global__ __launch_bounds__(256) void k_band_argmax_bwd_a(const BandArgs p, int
     tile.store(gt, it, tid);
     __syncthreads();
     if (jc + kAJ < Wo) tile.load(gb, ib, i0, jc + kAJ, n, Wo, p.r_lu, true, tid);
-#pragma unroll 8
-    for (int c = 0; c < kAJ; ++c) {
-      const int k = it[lane * kAC + c];
-      if (k >= 0 && k < Wa && (k & 3) == wave) acc[k * kAS + lane] += gt[lane * kAC + c];
+#pragma unroll 2
+    for (int c = 0; c < kAJ; c += 4) {
+      int sl[4];
+      float tv[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int k = it[lane * kAC + c + q];
+        sl[q] = (k >= 0 && k < Wa && (k & 3) == wave) ? k * kAS + lane : spare;
+        tv[q] = gt[lane * kAC + c + q];
+      }
+      add4_ordered(acc, sl, tv);
     }
   }
   __syncthreads();
@@ -105,15 +115,16 @@ __global__ __launch_bounds__(256) void k_band_argmax_bwd_b(const BandArgs p, int
   extern __shared__ __attribute__((aligned(16))) float smem[];
   constexpr int kRows = kAT + kAJ - 1;  // 95 rows of g / idx feed 64 rows of b per tile
   const int n = p.n, Wb = p.Wb, Wo = p.Wo;
-  float* acc = smem;                                      // [Wb][65]
-  float* gt = acc + Wb * kAS;                             // [95][33]
+  float* acc = smem;                                      // [Wb][65] + 256 spare cells
+  float* gt = acc + Wb * kAS + 256;                       // [95][33]
   int* it = reinterpret_cast<int*>(gt + kRows * kAC);     // [95][33]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int batch = blockIdx.x / strips, o0 = (blockIdx.x - batch * strips) * kAT;
   const long bn = (long)batch * n;
   const float* gb = p.g + bn * Wo;
   const int32_t* ib = p.idx + bn * Wo;
-  for (int e = tid; e < Wb * kAS; e += 256) acc[e] = 0.f;
+  for (int e = tid; e < Wb * kAS + 256; e += 256) acc[e] = 0.f;
+  const int spare = Wb * kAS + tid;
   // i = o + r_lu - j ascends as j descends: last tile first, columns right to left;
   // tile row 0 holds g row o0 + r_lu - jc - 31
   const int jlast = ((Wo - 1) / kAJ) * kAJ;
@@ -126,13 +137,20 @@ __global__ __launch_bounds__(256) void k_band_argmax_bwd_b(const BandArgs p, int
     __syncthreads();
     if (jc > 0) tile.load(gb, ib, row0_of(jc - kAJ), jc - kAJ, n, Wo, p.r_lu, false, tid);
     if (o0 + lane < n) {
-#pragma unroll 8
-      for (int c = kAJ - 1; c >= 0; --c) {
-        // cell (i, j) with i + j - r_lu = o0 + lane sits in tile row lane + 31 - c
-        const int r = lane + (kAJ - 1) - c;
-        const int k = it[r * kAC + c];
-        const int k2 = k - (jc + c) + Wb - 1;
-        if (k >= 0 && k2 >= 0 && k2 < Wb && (k2 & 3) == wave) acc[k2 * kAS + lane] += gt[r * kAC + c];
+#pragma unroll 2
+      for (int c4 = kAJ - 1; c4 >= 0; c4 -= 4) {
+        int sl[4];
+        float tv[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          // cell (i, j) with i + j - r_lu = o0 + lane sits in tile row lane + 31 - c
+          const int c = c4 - q, r = lane + (kAJ - 1) - c;
+          const int k = it[r * kAC + c];
+          const int k2 = k - (jc + c) + Wb - 1;
+          sl[q] = (k >= 0 && k2 >= 0 && k2 < Wb && (k2 & 3) == wave) ? k2 * kAS + lane : spare;
+          tv[q] = gt[r * kAC + c];
+        }
+        add4_ordered(acc, sl, tv);
       }
     }
   }

@@ -215,6 +215,23 @@ __host__ __device__ inline void philox_uniform4(uint64_t i, bool aligned, uint64
   }
 }
 
+// Four ordered additions with one LDS round trip: the four cells are read together,
+// the sums are chained in registers (a cell that was already hit earlier in the group
+// takes that sum instead of what it read), and written back in order.  A term whose k
+// is not this lane's goes to the lane's spare cell.
+__device__ __forceinline__ void add4_ordered(float* __restrict__ accs, const int (&s)[4],
+                                             const float (&v)[4]) {
+  const float r0 = accs[s[0]], r1 = accs[s[1]], r2 = accs[s[2]], r3 = accs[s[3]];
+  const float v0 = __fadd_rn(r0, v[0]);
+  const float v1 = __fadd_rn(s[1] == s[0] ? v0 : r1, v[1]);
+  const float v2 = __fadd_rn(s[2] == s[1] ? v1 : (s[2] == s[0] ? v0 : r2), v[2]);
+  const float v3 = __fadd_rn(s[3] == s[2] ? v2 : (s[3] == s[1] ? v1 : (s[3] == s[0] ? v0 : r3)), v[3]);
+  accs[s[0]] = v0;
+  accs[s[1]] = v1;
+  accs[s[2]] = v2;
+  accs[s[3]] = v3;
+}
+
 // ------------------------------------------------------------- host helpers
 inline int check_dense_dims(int B, int M, int K, int N) {
   if (B < 0 || M < 0 || K < 0 || N < 0) return GENBMM_E_SHAPE;

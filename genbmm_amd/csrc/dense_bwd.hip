@@ -107,23 +107,6 @@ constexpr int kKC = 128;  // cells of the reduction axis per lane
 // and g are read from memory once - the lanes of a line read the same addresses.
 // Each lane walks its whole line and adds the terms whose k falls into its part.
 
-// Four ordered additions with one LDS round trip: the four cells are read together,
-// the sums are chained in registers (a cell that was already hit earlier in the group
-// takes that sum instead of what it read), and written back in order.  A term whose k
-// is not this lane's goes to the lane's spare cell.
-__device__ __forceinline__ void add4_ordered(float* __restrict__ accs, const int (&s)[4],
-                                             const float (&v)[4]) {
-  const float r0 = accs[s[0]], r1 = accs[s[1]], r2 = accs[s[2]], r3 = accs[s[3]];
-  const float v0 = __fadd_rn(r0, v[0]);
-  const float v1 = __fadd_rn(s[1] == s[0] ? v0 : r1, v[1]);
-  const float v2 = __fadd_rn(s[2] == s[1] ? v1 : (s[2] == s[0] ? v0 : r2), v[2]);
-  const float v3 = __fadd_rn(s[3] == s[2] ? v2 : (s[3] == s[1] ? v1 : (s[3] == s[0] ? v0 : r3)), v[3]);
-  accs[s[0]] = v0;
-  accs[s[1]] = v1;
-  accs[s[2]] = v2;
-  accs[s[3]] = v3;
-}
-
 // grad_a: line = row m.  The row is read 16 cells at a time (int4 / float4 when the
 // rows are 16-byte aligned), then the 16 additions are made in order.
 template <int PROD>
