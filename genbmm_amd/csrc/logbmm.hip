@@ -658,25 +658,29 @@ int launch_fwd_mfma(DenseArgs p, const float* stats, int* flags, int B, int M, i
   return launch_fwd_fixup<CfgWide, T::TR, T::TC>(p, flags, total, s);
 }
 
-template <class T>
+// TF: the forward's tile shape (its flags and the exact fix-up go by it); the sweep
+// itself always runs 128 x 128 tiles.
+template <class TF>
 int launch_sample_sweep_mfma(DenseArgs p, const float* stats, int* flags, int B, int M, int K, int N,
                              hipStream_t s) {
+  using T = MTile<128, 128>;
   p.M = M; p.K = K; p.N = N;
-  p.tiles_m = ceil_div(M, T::TR);
-  p.tiles_n = ceil_div(N, T::TC);
+  const int tiles_m = ceil_div(M, T::TR), tiles_n = ceil_div(N, T::TC);
+  p.tiles_m = ceil_div(M, TF::TR);
+  p.tiles_n = ceil_div(N, TF::TC);
   p.vec_a = (K % 4 == 0) && aligned16(p.a);
   p.vec_b = (N % 4 == 0) && aligned16(p.b);
   p.vec_o = (N % 4 == 0) && aligned16(p.out) && aligned16(p.idx);
-  const int total = B * p.tiles_m * p.tiles_n;
+  const int64_t total = (int64_t)B * tiles_m * tiles_n;
+  if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
   const LogPrepared ws = prepared_of(stats, B, M, K, N);
-  auto go = [&](auto kern) {
-    hipLaunchKernelGGL(kern, dim3(total), dim3(T::NT), 0, s, ws.ea, ws.eb, p.out, stats, flags, ws.r,
-                       p.idx, p.seed, p.offset, M, K, N, p.tiles_m, p.tiles_n);
-  };
-  go(k_sample_sweep_mfma<T>);
+  hipLaunchKernelGGL(k_sample_sweep_mfma<T>, dim3((unsigned)total), dim3(T::NT), 0, s, ws.ea, ws.eb,
+                     p.out, stats, flags, ws.r, p.idx, p.seed, p.offset, M, K, N, tiles_m, tiles_n,
+                     TF::TR, TF::TC, p.tiles_m, p.tiles_n);
   if (int e = launch_status()) return e;
-  hipLaunchKernelGGL((k_sample_fixup<CfgWide, T::TR, T::TC>), dim3(min(total, kFixupGrid)),
-                     dim3(CfgWide::NT), 0, s, p, flags, total);
+  const int ftotal = B * p.tiles_m * p.tiles_n;
+  hipLaunchKernelGGL((k_sample_fixup<CfgWide, TF::TR, TF::TC>), dim3(min(ftotal, kFixupGrid)),
+                     dim3(CfgWide::NT), 0, s, p, flags, ftotal);
   return launch_status();
 }
 

@@ -645,7 +645,10 @@ void k_log_bwd_mfma_both(const float* __restrict__ g, const float* __restrict__ 
 // the code -2 - slab in idx (0 if the prefix never reaches t) and rem in `remw`; the
 // terms of that one slab are walked by the resolve kernel.  At most kSampleSlabs
 // slabs (the tag's range).  A tile with a cell whose S is below 2^-40 or not finite,
-// or that the forward flagged, sets its flag and leaves: it is redone exactly.
+// or that lies in a tile the forward flagged, sets that flag and leaves: the forward's
+// tile is redone exactly.  The sweep's own tile shape is free: 128 x 128 with four
+// waves lets two workgroups share a compute unit within the 256 registers per lane,
+// so that one's vector work overlaps the other's matrix-core work.
 constexpr int kSampleSlabs = 62;
 
 // (Always the any-size form of the loaders: with this kernel's register budget the
@@ -656,7 +659,8 @@ void k_sample_sweep_mfma(const float* __restrict__ ws_ea, const float* __restric
                          const float* __restrict__ out, const float* __restrict__ stats,
                          int* __restrict__ flags, float* __restrict__ remw,
                          int32_t* __restrict__ idx, uint64_t seed, uint64_t offset, int M, int K,
-                         int N, int tiles_m, int tiles_n) {
+                         int N, int tiles_m, int tiles_n, int ftr, int ftc, int ftiles_m,
+                         int ftiles_n) {
   constexpr bool RAGGED = true;
   constexpr int NT = T::NT, LDR = T::LDR, LDC = T::LDC;
   using SA = StageT<T::TR, NT, LDR>;
@@ -676,11 +680,14 @@ void k_sample_sweep_mfma(const float* __restrict__ ws_ea, const float* __restric
   // cells per lane and step (they share one Philox block when rows are a multiple of
   // four cells); a rolled loop, its body is long.  Then the accumulators pick their
   // cells up in the matrix-core layout.
+  // the flags are the forward's, one per tile of ITS shape (ftr x ftc)
+  int* flag = flags + (batch * ftiles_m + m0 / ftr) * ftiles_n + n0 / ftc;
   const float lim = kMfmaGuardBits * kLn2 + 1e-3f;
-  int bad = flags[tile];
+  int bad = *flag;
   {
     constexpr int QR = T::TC / 4;  // quads per tile row
     const bool blocks = (N & 3) == 0;
+#pragma unroll 4
     for (int q = tid; q < T::TR * QR; q += NT) {
       const int r = q / QR, m = m0 + r, n = n0 + (q - r * QR) * 4;
       if (RAGGED && (m >= M || n >= N)) continue;
@@ -703,7 +710,7 @@ void k_sample_sweep_mfma(const float* __restrict__ ws_ea, const float* __restric
   }
   bad = __syncthreads_or(bad);  // also: the tile's -t are visible to the whole workgroup
   if (bad) {
-    if (tid == 0) flags[tile] = 1;
+    if (tid == 0) *flag = 1;
     return;
   }
   floatx16 acc[2][2];
