@@ -1,4 +1,4 @@
-"""Timing of every BASELINE.json configuration on one MI355X (bench.py covers only the
+"""Timing of every benchmark configuration (BASELINE.json) on one MI355X (bench.py covers only the
 headline line the driver reads).
 
     python bench_configs.py [--reps 20] [--cpu]

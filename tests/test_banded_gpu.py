@@ -152,7 +152,7 @@ def test_banded_double_backward_vs_literal_kernels(gpu, n, a_lu, a_ld, b_lu, b_l
 
 
 def test_banded_config_c5(gpu):
-    """BASELINE config 4: batch 64, n = 4096, lu = ld = 32 for both operands, Uniform[-1,1)
+    """Benchmark configuration 4: batch 64, n = 4096, lu = ld = 32 for both operands, Uniform[-1,1)
     band data from seed 7; standard and log semiring, forward + backward.  Full-size run;
     float64 oracle on two batch items; dense closed form at reduced n."""
     torch.manual_seed(7)

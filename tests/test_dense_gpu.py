@@ -66,7 +66,7 @@ def test_logbmm_forward_and_grads(gpu, path, B, M, K, N):
 
 
 def test_logbmm_config_c1_uniform_ones(gpu, path):
-    """BASELINE config 0: seed 0, Uniform[0,1) (16,64,64), grad_out = ones."""
+    """Benchmark configuration 0: seed 0, Uniform[0,1) (16,64,64), grad_out = ones."""
     torch.manual_seed(0)
     a, b = torch.rand(16, 64, 64), torch.rand(16, 64, 64)
     g = torch.ones(16, 64, 64)
@@ -100,7 +100,7 @@ def test_logbmm_special_values(gpu, path):
 
 @pytest.mark.parametrize("B,M,K,N,sub", [(512, 128, 128, 128, 8), (8192, 32, 32, 32, 256), (64, 512, 512, 512, 1)])
 def test_logbmm_baseline_shapes(gpu, path, B, M, K, N, sub):
-    """BASELINE configs 1 and the headline shape: full-size run, float64 check on a
+    """Benchmark configuration 1 and the headline shape: full-size run, float64 check on a
     batch subset plus the size-independent row-sum invariants on everything."""
     torch.manual_seed(0)
     a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
@@ -359,7 +359,7 @@ def test_max_index_groups_and_special_values(gpu, prod, B, M, K, N):
 
 
 def test_max_config_c3(gpu):
-    """BASELINE config 2: (256,256,256) on the 1/8 grid (max) and Uniform(0,1] (prod-max);
+    """Benchmark configuration 2: (256,256,256) on the 1/8 grid (max) and Uniform(0,1] (prod-max);
     bit-exact on a batch subset, argmax property on everything."""
     torch.manual_seed(0)
     B = M = K = N = 256
@@ -436,7 +436,7 @@ def test_sample_index_brackets_cdf(gpu, use_stats, B, M, K, N):
 
 
 def test_sample_config_c4_chi_square(gpu):
-    """BASELINE config 3: Normal(0,2) (64,512,512) potentials, Philox seed 1234; 10^4
+    """Benchmark configuration 3: Normal(0,2) (64,512,512) potentials, Philox seed 1234; 10^4
     draws per cell of the (4,16,16) slice; per-cell chi-square against the float64
     softmax, categories with expected count < 5 pooled, bound = the 1-1e-6 quantile."""
     from scipy.stats import chi2 as chi2_dist
