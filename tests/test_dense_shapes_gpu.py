@@ -89,3 +89,37 @@ def test_sample_on_many_shapes(gpu):
         assert bool(ok.all()), ((B, M, K, N), float((~ok).float().mean()))
         want = oracle.sample_index_from_cdf(cdf, u).long()
         assert float((got != want).float().mean()) < 5e-3, (B, M, K, N)
+
+
+@pytest.mark.parametrize("scale", [0.05, 2.0, 12.0, 40.0])
+def test_sample_on_flat_and_peaked_distributions(gpu, scale):
+    """From nearly uniform to one-term-takes-all, with masked terms (-inf, -1e9), on a shape
+    that takes the matrix-core sweep (and its exact fix-up where S underflows)."""
+    lib = _lib.load()
+    torch.manual_seed(int(scale * 10))
+    B, M, K, N = 2, 128, 200, 160
+    a, b = scale * torch.randn(B, M, K), scale * torch.randn(B, K, N)
+    a[:, ::3, ::5] = float("-inf")
+    b[:, 1::7, ::2] = -1e9
+    a[1, 5, :] = float("-inf")          # a row without any mass: out = -inf, index 0
+    ad, bd = a.to(gpu), b.to(gpu)
+    out = torch.empty(B, M, N, device=gpu)
+    idx = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
+    stats = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=gpu)
+    assert lib.genbmm_samplebmm_fwd(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx), _lib.ptr(stats),
+                                    5, 11, B, M, K, N, _lib.stream_of(ad)) == 0
+    u = oracle.philox_uniform(0, B * M * N, 5, 11).view(B, M, N).double()
+    want_out, want_idx = oracle.seq_samplebmm_fwd(a, b, u.float())
+    got = idx.cpu().long()
+    live = torch.ones(B, M, N, dtype=torch.bool)
+    live[1, 5, :] = False
+    assert bool((got[~live] == 0).all()) and bool((out.cpu()[~live] == want_out[~live]).all())
+    assert torch.allclose(out.cpu()[live], want_out[live], rtol=1e-5, atol=1e-5)
+    cdf = oracle.sample_cdf64(a, b)
+    hi = torch.gather(cdf, 2, got.unsqueeze(2)).squeeze(2)
+    lo = torch.where(got > 0, torch.gather(cdf, 2, (got - 1).clamp(min=0).unsqueeze(2)).squeeze(2), torch.zeros_like(hi))
+    ok = ((lo - 2e-5 <= u) & (u <= hi + 2e-5)) | ~live
+    assert bool(ok.all()), float((~ok).float().mean())
+    # a sampled term always has mass (never a masked one)
+    picked = torch.gather(a.unsqueeze(-1) + b.unsqueeze(-3), 2, got.unsqueeze(2)).squeeze(2)
+    assert bool((picked[live] > -1e8).all())
