@@ -21,6 +21,7 @@
 #include <type_traits>
 
 #include "banded_argmax.h"
+#include "banded_mfma.h"
 #include "banded_strip.h"
 
 namespace genbmm {
@@ -55,6 +56,27 @@ inline bool workspace_used(const BandArgs& p) {
 
 inline bool prep_fwd(const BandArgs& p, int mode, const float* workspace) {
   return mode == GENBMM_BAND_LOG && workspace != nullptr && workspace_used(p);
+}
+
+// Which bands the matrix-core kernels take: the tiles of all three products fit in LDS.
+constexpr size_t kMmLdsLimit = 160 * 1024;
+inline bool mm_ok(const BandArgs& p) {
+  if (!mm_tiles_ok(p.Wa, p.Wb, p.Wo) || min(p.Wa, p.Wb) < 4) return false;
+  for (int kind = 0; kind < 3; ++kind)
+    if (mm_dims(kind, p.Wa, p.Wb, p.Wo).bytes > kMmLdsLimit) return false;
+  return true;
+}
+template <int KIND, bool PREP>
+inline void launch_mm(const BandArgs& p, int B, hipStream_t s) {
+  const MmDims d = mm_dims(KIND, p.Wa, p.Wb, p.Wo);
+  const int strips = ceil_div(p.n, mm_rows(KIND));
+  auto kern = k_band_mm<KIND, PREP>;
+  if (d.bytes > kStripLdsLimit)
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)d.bytes);
+  const long rows = (long)B * p.n;
+  hipLaunchKernelGGL(kern, dim3((unsigned)((long)B * strips)), dim3(256), d.bytes, s, p, strips, d,
+                     rows * p.Wa, rows * p.Wb, rows * p.Wo);
 }
 
 inline void set_workspace(BandArgs& p, float* ws, int B) {
@@ -94,6 +116,22 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   if (total == 0) return GENBMM_OK;
   hipStream_t s = (hipStream_t)stream;
   const StripDims sd = strip_dims(p.Wa, p.Wb);
+  if (mode != GENBMM_BAND_MAX && mm_ok(p) && (mode == GENBMM_BAND_MUL || prep_fwd(p, mode, workspace))) {
+    if (mode == GENBMM_BAND_LOG) {
+      set_workspace(p, workspace, B);
+      const long rows = (long)B * n;
+      const dim3 pg((unsigned)((rows + kPrepRows - 1) / kPrepRows));
+      const int lda = odd(p.Wa), ldb = odd(p.Wb);
+      hipLaunchKernelGGL(k_band_prep, pg, dim3(256), sizeof(float) * kPrepRows * lda, s, a, p.ws_ea,
+                         p.ws_al, p.Wa, a_lu, n, rows, lda);
+      hipLaunchKernelGGL(k_band_prep, pg, dim3(256), sizeof(float) * kPrepRows * ldb, s, b, p.ws_eb,
+                         p.ws_be, p.Wb, b_lu, n, rows, ldb);
+      launch_mm<kMmFwd, true>(p, B, s);
+    } else {
+      launch_mm<kMmFwd, false>(p, B, s);
+    }
+    return launch_status();
+  }
   if (fwd_strip_ok(p)) {
     const int strips = ceil_div(n, kBT);
     const dim3 grid((unsigned)((long)B * strips));
@@ -151,6 +189,20 @@ int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   const long ta = (long)B * n * p.Wa, tb = (long)B * n * p.Wb;
   if (ta == 0) return GENBMM_OK;
   hipStream_t s = (hipStream_t)stream;
+  if (mode == GENBMM_BAND_MUL && mm_ok(p)) {
+    launch_mm<kMmGradA, false>(p, B, s);
+    launch_mm<kMmGradB, false>(p, B, s);
+    return launch_status();
+  }
+  if (mode == GENBMM_BAND_LOG && workspace && workspace_used(p) && mm_ok(p)) {
+    set_workspace(p, workspace, B);
+    const long cells = (long)B * n * p.Wo;
+    hipLaunchKernelGGL(k_band_h, dim3((unsigned)min((cells + 1023) / 1024, (long)0x7fffffff)), dim3(256), 0,
+                       s, g, p.ws_r, p.ws_h, cells);
+    launch_mm<kMmGradA, true>(p, B, s);
+    launch_mm<kMmGradB, true>(p, B, s);
+    return launch_status();
+  }
   if (mode != GENBMM_BAND_MAX && bwd_strip_ok(p)) {
     const bool lg = mode == GENBMM_BAND_LOG;
     const StripDims da = strip_dims(p.Wa, p.Wb), db = strip_dims(p.Wb, p.Wa);

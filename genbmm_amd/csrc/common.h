@@ -215,6 +215,12 @@ __host__ __device__ inline void philox_uniform4(uint64_t i, bool aligned, uint64
   }
 }
 
+// Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
+// Renumber them so that every XCD works on one contiguous run of tiles (the
+// tiles of a batch item share their operands).
+__device__ __forceinline__ int xcd_renumber(int w, int n) {
+  return (n & 7) == 0 ? (w & 7) * (n >> 3) + (w >> 3) : w;
+}
 // Four ordered additions with one LDS round trip: the four cells are read together,
 // the sums are chained in registers (a cell that was already hit earlier in the group
 // takes that sum instead of what it read), and written back in order.  A term whose k

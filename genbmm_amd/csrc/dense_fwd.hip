@@ -155,7 +155,8 @@ __device__ __forceinline__ void resolve_walk(const float* __restrict__ first, co
   static_assert(KSTAGE % G == 0 && G % 4 == 0, "a group lies in one staged chunk");
   const int lane = threadIdx.x & 63, col = lane % COLS, sub = lane / COLS;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  int wg = blockIdx.x;
+  // the panels of a batch item share its rows of the first operand: keep them on one XCD (one L2)
+  int wg = xcd_renumber(blockIdx.x, gridDim.x);
   const int panel = wg % panels;
   wg /= panels;
   const int chunk = wg % row_chunks;

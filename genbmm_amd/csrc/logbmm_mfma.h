@@ -33,12 +33,6 @@ constexpr int kMS = 16;         // slab depth
 constexpr int kMPad = 4;        // LDS row padding (floats) of a [slab][tile] buffer
 constexpr float kMfmaGuardBits = 40.f;
 
-// Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
-// Renumber them so that every XCD works on one contiguous run of tiles (the
-// tiles of a batch item share their operands).
-__device__ __forceinline__ int xcd_renumber(int w, int n) {
-  return (n & 7) == 0 ? (w & 7) * (n >> 3) + (w >> 3) : w;
-}
 __device__ __forceinline__ int xcd_tile_id() { return xcd_renumber(blockIdx.x, gridDim.x); }
 
 __device__ __forceinline__ float exp_st(float d) { return fast_exp2(d * kLog2e); }
