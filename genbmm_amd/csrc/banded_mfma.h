@@ -98,8 +98,11 @@ struct MmFlat {
   int nvec, lead, W, gap;
   unsigned magic;  // ceil(2^32 / W)
   const float* abeg;
+  bool inside;     // every piece lies inside the tensor
 
-  __device__ __forceinline__ void init(const float* tensor, long first, int count, int W_, int pitch) {
+  // [tensor, tensor_end): the whole tensor; a piece that crosses its ends is read float by float
+  __device__ __forceinline__ void init(const float* tensor, const float* tensor_end, long first, int count,
+                                       int W_, int pitch) {
     const float* beg = tensor + first;
     lead = (int)((reinterpret_cast<uintptr_t>(beg) & 15) >> 2);
     abeg = beg - lead;
@@ -107,25 +110,30 @@ struct MmFlat {
     W = W_;
     gap = pitch - W_;
     magic = (unsigned)((0x100000000ull + (unsigned)W - 1) / (unsigned)W);
+    inside = abeg >= tensor && abeg + 4 * (long)nvec <= tensor_end;
   }
   __device__ __forceinline__ int origin() const { return lead + gap; }
   __device__ __forceinline__ bool more(int batch) const { return batch * 256 * U < nvec; }
-  // [lo, hi): the tensor; a piece that crosses its ends is read float by float
   __device__ __forceinline__ void load(const float* lo, const float* hi, int batch, int tid) {
+    if (inside) {  // uniform
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int vi = tid + 256 * (u + batch * U);
+        v[u] = mm_f4{0.f, 0.f, 0.f, 0.f};
+        if (vi < nvec) v[u] = *reinterpret_cast<const mm_f4*>(abeg + 4 * vi);
+      }
+      return;
+    }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int vi = tid + 256 * (u + batch * U);
-      v[u] = mm_f4{0.f, 0.f, 0.f, 0.f};
+      mm_f4 x = mm_f4{0.f, 0.f, 0.f, 0.f};
       if (vi < nvec) {
         const float* q = abeg + 4 * vi;
-        if (q >= lo && q + 4 <= hi) {
-          v[u] = *reinterpret_cast<const mm_f4*>(q);
-        } else {
-#pragma unroll
-          for (int t = 0; t < 4; ++t)
-            if (q + t >= lo && q + t < hi) v[u][t] = q[t];
-        }
+        for (int t = 0; t < 4; ++t)
+          if (q + t >= lo && q + t < hi) x[t] = q[t];
       }
+      v[u] = x;
     }
   }
   // returns whether this thread saw a value that is not finite.  Piece v holds the flat
@@ -143,9 +151,11 @@ struct MmFlat {
                !(fabsf(x[3]) <= FLT_MAX);
         const int f = 4 * vi, uu = f + W - lead;
         const int r1 = (int)__umulhi((unsigned)uu, magic), k = uu - r1 * W;
-        const int at = f + r1 * gap;
+        float* at = L + (f + r1 * gap);
+        const int nb = W - k;  // cells of the piece before its row ends, at least one
+        at[0] = x[0];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) L[at + t + (k + t >= W ? gap : 0)] = x[t];
+        for (int t = 1; t < 4; ++t) at[t + (t >= nb ? gap : 0)] = x[t];
       }
     }
     return bad;
@@ -242,14 +252,14 @@ __global__ __launch_bounds__(256, 2) void k_band_mm(const BandArgs p, int strips
   MmFlat<14> sq;
   MmFlat<6> sp;
   MmSkew<PREP, 20> sk;
-  sq.init(qt, (bn + qr0) * Wq, (qr1 - qr0) * Wq, Wq, d.qp);
+  sq.init(qt, qt + cells_q, (bn + qr0) * Wq, (qr1 - qr0) * Wq, Wq, d.qp);
   sq.load(qt, qt + cells_q, 0, tid);
   if (GB) {
     sk.init(Wo);
     sk.load(gt + bn * Wo, Wo, r_lu, n, x0, 0, tid);
   } else {
     const float* pt = FWD ? at : gt;
-    sp.init(pt, (bn + x0) * Wp, (pr1 - x0) * Wp, Wp, d.pp);
+    sp.init(pt, pt + (FWD ? cells_a : cells_o), (bn + x0) * Wp, (pr1 - x0) * Wp, Wp, d.pp);
     sp.load(pt, pt + (FWD ? cells_a : cells_o), 0, tid);
   }
   if (tid <= ROWS) badrow[tid] = 0;
@@ -291,8 +301,6 @@ __global__ __launch_bounds__(256, 2) void k_band_mm(const BandArgs p, int strips
   const int pp = d.pp, qp = d.qp;
   const float* Pt = GB ? PL : PL + sp.origin();
   const float* Qt = QL + sq.origin() - (qr0 - q0) * qp;
-  const int p_last = ROWS * pp - 1;                                      // indices of Pt / Qt that
-  const int q_first = (qr0 - q0) * qp, q_last = (qr1 - q0) * qp - 1;    // lie in the staged rows
 
   // ---- tiles
   const int xt = wave / SPLIT, part = wave % SPLIT;
@@ -362,16 +370,22 @@ __global__ __launch_bounds__(256, 2) void k_band_mm(const BandArgs p, int strips
         const int qbase = FWD ? (y - q0) * qp - y + luq : y + luq - q0 * qp;
         const int qz = FWD ? 1 : qp - 1;
         mm_f4 c = acc[ty];
+        // a lane outside feeds zero; what it reads instead (possibly beyond the staged
+        // rows, LDS has no faults) does not matter
         auto masked = [&](int sa, int sb) {
-          int z = zlo + 4 * sa + zq;
+          const int z = zlo + 4 * sa + zq;
+          const float* pa = Pt + pbase + psign * z;
+          const float* pb = Qt + qbase + qz * z;
+          unsigned zp = (unsigned)(z - plo), zy = (unsigned)(z - qlo);
           for (int s = sa; s < sb; ++s) {
-            const int ia = mm_clamp(pbase + psign * z, 0, p_last);
-            const int ib = mm_clamp(qbase + qz * z, q_first, q_last);
-            float a = Pt[ia], b = Qt[ib];
-            a = (unsigned)(z - plo) <= (unsigned)pspan ? a : 0.f;
-            b = (unsigned)(z - qlo) <= (unsigned)qspan ? b : 0.f;
+            float a = *pa, b = *pb;
+            a = zp <= (unsigned)pspan ? a : 0.f;
+            b = zy <= (unsigned)qspan ? b : 0.f;
             c = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
-            z += 4;
+            pa += 4 * psign;
+            pb += dq;
+            zp += 4;
+            zy += 4;
           }
         };
         masked(s0, sc0);
@@ -405,18 +419,21 @@ __global__ __launch_bounds__(256, 2) void k_band_mm(const BandArgs p, int strips
   __syncthreads();  // the operands are consumed: their place becomes the result tile
 
   // lane holds rows 4 zq + r, column l15 of each of its tiles; result column 16 ty + l15 - row
+  int srow[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) srow[r] = (16 * xt + 4 * zq + r) * Wout + l15 - (4 * zq + r);
 #pragma unroll
   for (int phase = 0; phase < SPLIT; ++phase) {
     if (part == phase) {
 #pragma unroll
       for (int ty = 0; ty < kMmTiles; ++ty) {
         if (ty < ny && (phase == 0 || ((mine >> ty) & 1u))) {
+          const bool inner = 16 * ty - 15 >= 0 && 16 * ty + 15 < Wout;  // no lane of the tile is outside
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const int xr = 4 * zq + r;
-            const int col = 16 * ty + l15 - xr;
-            if (col >= 0 && col < Wout) {
-              float* sc = S + (16 * xt + xr) * Wout + col;
+            const int col = 16 * ty + l15 - (4 * zq + r);
+            if (inner || (col >= 0 && col < Wout)) {
+              float* sc = S + srow[r] + 16 * ty;
               *sc = phase == 0 ? acc[ty][r] : *sc + acc[ty][r];
             }
           }
