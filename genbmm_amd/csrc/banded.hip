@@ -58,13 +58,17 @@ inline bool prep_fwd(const BandArgs& p, int mode, const float* workspace) {
   return mode == GENBMM_BAND_LOG && workspace != nullptr && workspace_used(p);
 }
 
-// Which bands the matrix-core kernels take: the tiles of all three products fit in LDS.
-constexpr size_t kMmLdsLimit = 160 * 1024;
-inline bool mm_ok(const BandArgs& p) {
-  if (!mm_tiles_ok(p.Wa, p.Wb, p.Wo) || min(p.Wa, p.Wb) < 4) return false;
-  for (int kind = 0; kind < 3; ++kind)
-    if (mm_dims(kind, p.Wa, p.Wb, p.Wo).bytes > kMmLdsLimit) return false;
-  return true;
+// Which bands the matrix-core kernels take: wide enough for 16 x 16 tiles to pay (measured
+// against the strip kernels at 64 x 4096: forward from 9 diagonals on, gradients from 25),
+// and two workgroups' tiles fit in a compute unit's LDS.
+constexpr size_t kMmLdsLimit = 80 * 1024;
+inline bool mm_fwd_ok(const BandArgs& p) {
+  return mm_tiles_ok(p.Wa, p.Wb, p.Wo) && min(p.Wa, p.Wb) >= 8 &&
+         mm_dims(kMmFwd, p.Wa, p.Wb, p.Wo).bytes <= kMmLdsLimit;
+}
+inline bool mm_bwd_ok(const BandArgs& p) {
+  return mm_tiles_ok(p.Wa, p.Wb, p.Wo) && min(p.Wa, p.Wb) >= 25 &&
+         max(mm_dims(kMmGradA, p.Wa, p.Wb, p.Wo).bytes, mm_dims(kMmGradB, p.Wa, p.Wb, p.Wo).bytes) <= kMmLdsLimit;
 }
 template <int KIND, bool PREP>
 inline void launch_mm(const BandArgs& p, int B, hipStream_t s) {
@@ -116,7 +120,7 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   if (total == 0) return GENBMM_OK;
   hipStream_t s = (hipStream_t)stream;
   const StripDims sd = strip_dims(p.Wa, p.Wb);
-  if (mode != GENBMM_BAND_MAX && mm_ok(p) && (mode == GENBMM_BAND_MUL || prep_fwd(p, mode, workspace))) {
+  if (mode != GENBMM_BAND_MAX && mm_fwd_ok(p) && (mode == GENBMM_BAND_MUL || prep_fwd(p, mode, workspace))) {
     if (mode == GENBMM_BAND_LOG) {
       set_workspace(p, workspace, B);
       const long rows = (long)B * n;
@@ -189,12 +193,12 @@ int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   const long ta = (long)B * n * p.Wa, tb = (long)B * n * p.Wb;
   if (ta == 0) return GENBMM_OK;
   hipStream_t s = (hipStream_t)stream;
-  if (mode == GENBMM_BAND_MUL && mm_ok(p)) {
+  if (mode == GENBMM_BAND_MUL && mm_bwd_ok(p)) {
     launch_mm<kMmGradA, false>(p, B, s);
     launch_mm<kMmGradB, false>(p, B, s);
     return launch_status();
   }
-  if (mode == GENBMM_BAND_LOG && workspace && workspace_used(p) && mm_ok(p)) {
+  if (mode == GENBMM_BAND_LOG && workspace && workspace_used(p) && mm_bwd_ok(p)) {
     set_workspace(p, workspace, B);
     const long cells = (long)B * n * p.Wo;
     hipLaunchKernelGGL(k_band_h, dim3((unsigned)min((cells + 1023) / 1024, (long)0x7fffffff)), dim3(256), 0,

@@ -1,0 +1,122 @@
+"""GPU parity of the banded (+,x) and log products on bands wide enough for the
+matrix-core kernels (9 diagonals forward, 25 backward): edges of the matrix inside a
+strip, strips cut by n, one-sided bands, operands that do not start on 16 bytes, values
+that are not finite.  All against the float64 sequential restatement of the reference
+kernel (oracle.seq_band_fwd / seq_band_bwd)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from genbmm_amd.sparse import BandedMatrix, banddiag
+
+pytestmark = pytest.mark.gpu
+
+# (n, a_lu, a_ld, b_lu, b_ld)
+WIDE = [(300, 12, 12, 12, 12), (95, 20, 9, 14, 16), (513, 32, 32, 32, 32), (64, 30, 0, 0, 30),
+        (33, 16, 16, 16, 16), (1000, 3, 30, 28, 2), (129, 4, 4, 20, 20), (40, 28, 28, 30, 30),
+        (257, 0, 31, 31, 0), (70, 10, 5, 3, 8)]
+
+
+def close(x, ref, rtol=1e-5, atol=1e-5):
+    x, ref = x.detach().cpu().double(), ref.detach().cpu().double()
+    assert torch.allclose(x, ref, rtol=rtol, atol=atol, equal_nan=True), float((x - ref).abs().nan_to_num().max())
+
+
+def pair(n, a_lu, a_ld, b_lu, b_ld, batch=2):
+    a = banddiag(torch.randn(batch, n, n), a_lu, a_ld)[0].contiguous()
+    b = banddiag(torch.randn(batch, n, n), b_lu, b_ld)[0].contiguous()
+    return a, b
+
+
+def offset_copy(t, gpu, shift):
+    """The same values in device memory that starts `shift` floats past a 16-byte boundary."""
+    flat = torch.empty(t.numel() + 8, device=gpu)
+    view = flat[shift:shift + t.numel()].view(t.shape)
+    view.copy_(t)
+    assert view.data_ptr() % 16 == 4 * (shift % 4) and view.is_contiguous()
+    return view
+
+
+@pytest.mark.parametrize("n,a_lu,a_ld,b_lu,b_ld", WIDE)
+@pytest.mark.parametrize("mode", [0, 3])
+def test_wide_bands_forward_backward(gpu, n, a_lu, a_ld, b_lu, b_ld, mode):
+    torch.manual_seed(n + 31 * mode)
+    a, b = pair(n, a_lu, a_ld, b_lu, b_ld)
+    W = a.shape[2] + b.shape[2] - 1
+    g = torch.randn(2, n, W)
+    X = BandedMatrix(a.to(gpu).requires_grad_(True), a_lu, a_ld)
+    Y = BandedMatrix(b.to(gpu).requires_grad_(True), b_lu, b_ld)
+    res = (X.multiply_log if mode == 0 else X.multiply)(Y)
+    want, _, _ = oracle.seq_band_fwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, mode, dtype=np.float64)
+    close(res.data, want)
+    ga, gb = torch.autograd.grad(res.data, (X.data, Y.data), g.to(gpu))
+    wa, wb = oracle.seq_band_bwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, g.double(), mode, dtype=np.float64)
+    close(ga, wa)
+    close(gb, wb)
+
+
+@pytest.mark.parametrize("shift", [1, 2, 3])
+@pytest.mark.parametrize("mode", [0, 3])
+def test_operands_off_the_16_byte_grid(gpu, shift, mode):
+    n, a_lu, a_ld, b_lu, b_ld = 150, 13, 14, 15, 12
+    torch.manual_seed(shift)
+    a, b = pair(n, a_lu, a_ld, b_lu, b_ld)
+    g = torch.randn(2, n, a.shape[2] + b.shape[2] - 1)
+    ad = offset_copy(a, gpu, shift).requires_grad_(True)
+    bd = offset_copy(b, gpu, shift + 1).requires_grad_(True)
+    X, Y = BandedMatrix(ad, a_lu, a_ld), BandedMatrix(bd, b_lu, b_ld)
+    res = (X.multiply_log if mode == 0 else X.multiply)(Y)
+    want, _, _ = oracle.seq_band_fwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, mode, dtype=np.float64)
+    close(res.data, want)
+    ga, gb = torch.autograd.grad(res.data, (ad, bd), offset_copy(g, gpu, shift + 2))
+    wa, wb = oracle.seq_band_bwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, g.double(), mode, dtype=np.float64)
+    close(ga, wa)
+    close(gb, wb)
+
+
+def test_values_that_are_not_finite(gpu):
+    """inf and NaN in an operand reach exactly the cells the reference lets them reach: a
+    strip that holds one is computed cell by cell."""
+    n, lu, ld = 200, 14, 15
+    torch.manual_seed(5)
+    a, b = pair(n, lu, ld, ld, lu)
+    a[0, 40, 3] = float("inf")
+    a[1, 101, 7] = float("nan")
+    b[0, 77, 20] = -float("inf")
+    b[1, 150, 0] = float("inf")
+    ad, bd = a.to(gpu), b.to(gpu)
+    res = BandedMatrix(ad, lu, ld).multiply(BandedMatrix(bd, ld, lu))
+    want, _, _ = oracle.seq_band_fwd(a.double(), lu, ld, b.double(), ld, lu, 3, dtype=np.float64)
+    got = res.data.cpu().double()
+    assert torch.equal(torch.isnan(got), torch.isnan(want))
+    assert torch.equal(torch.isinf(got), torch.isinf(want))
+    close(got.nan_to_num(posinf=0.0, neginf=0.0), want.nan_to_num(posinf=0.0, neginf=0.0))
+    # gradients with a finite g: rows away from the special values are untouched by them
+    g = torch.randn(2, n, res.data.shape[2])
+    ar, br = ad.clone().requires_grad_(True), bd.clone().requires_grad_(True)
+    out = BandedMatrix(ar, lu, ld).multiply(BandedMatrix(br, ld, lu))
+    ga, gb = torch.autograd.grad(out.data, (ar, br), g.to(gpu))
+    wa, wb = oracle.seq_band_bwd(a.double(), lu, ld, b.double(), ld, lu, g.double(), 3, dtype=np.float64)
+    for got_g, want_g in ((ga, wa), (gb, wb)):
+        got_g = got_g.cpu().double()
+        fin = torch.isfinite(want_g)
+        assert torch.equal(torch.isfinite(got_g), fin)
+        close(got_g[fin], want_g[fin])
+
+
+def test_log_product_with_masked_and_infinite_cells(gpu):
+    n, lu, ld = 160, 16, 16
+    torch.manual_seed(9)
+    a, b = pair(n, lu, ld, ld, lu)
+    a[0, 10:60, 5:9] = -float("inf")
+    b[1, 90, :] = -float("inf")       # a fully masked row
+    a[1, 120, 2] = float("inf")
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    res = BandedMatrix(ad, lu, ld).multiply_log(BandedMatrix(bd, ld, lu))
+    want, _, _ = oracle.seq_band_fwd(a.double(), lu, ld, b.double(), ld, lu, 0, dtype=np.float64)
+    got = res.data.detach().cpu().double()
+    assert torch.equal(torch.isfinite(got), torch.isfinite(want))
+    fin = torch.isfinite(want)
+    close(got[fin], want[fin])
+    assert torch.equal(got[~fin].nan_to_num(nan=7.0), want[~fin].nan_to_num(nan=7.0))
