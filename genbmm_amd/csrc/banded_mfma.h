@@ -315,13 +315,13 @@ __global__ __launch_bounds__(256, 2) void k_band_mm(const BandArgs p, int strips
   const int c4 = FWD ? b_ld : GA ? p.b_lu : p.a_lu;
   const int ny = (Wout + 30) >> 4;
   int total = 0;
-  for (int ty = 0; ty < ny; ++ty) {
+  for (int ty = 0; SPLIT > 1 && ty < ny; ++ty) {
     const int y0t = x0t + cy + 16 * ty;
     const int zlo = max(max(x0t + c1, y0t + c2), 0), zhi = min(min(x0t + 15 + c3, y0t + 15 + c4), n - 1);
     total += zhi >= zlo ? (zhi - zlo + 4) >> 2 : 0;
   }
   const int lo = SPLIT == 1 ? 0 : part ? (total + 1) >> 1 : 0;
-  const int hi = SPLIT == 1 ? total : part ? total : (total + 1) >> 1;
+  const int hi = SPLIT == 1 ? 0x3fffffff : part ? total : (total + 1) >> 1;
 
   // this lane's row of P: the z inside are [plo, plo + pspan]
   constexpr int kNone = 0x3fffffff;
@@ -370,48 +370,53 @@ __global__ __launch_bounds__(256, 2) void k_band_mm(const BandArgs p, int strips
         const int qbase = FWD ? (y - q0) * qp - y + luq : y + luq - q0 * qp;
         const int qz = FWD ? 1 : qp - 1;
         mm_f4 c = acc[ty];
-        // a lane outside feeds zero; what it reads instead (possibly beyond the staged
-        // rows, LDS has no faults) does not matter
-        auto masked = [&](int sa, int sb) {
-          const int z = zlo + 4 * sa + zq;
-          const float* pa = Pt + pbase + psign * z;
-          const float* pb = Qt + qbase + qz * z;
-          unsigned zp = (unsigned)(z - plo), zy = (unsigned)(z - qlo);
-          for (int s = sa; s < sb; ++s) {
-            float a = *pa, b = *pb;
-            a = zp <= (unsigned)pspan ? a : 0.f;
-            b = zy <= (unsigned)qspan ? b : 0.f;
-            c = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
-            pa += 4 * psign;
-            pb += dq;
-            zp += 4;
-            zy += 4;
-          }
-        };
-        masked(s0, sc0);
-        {
-          const int z = zlo + 4 * sc0 + zq;
-          const float* pa = Pt + pbase + psign * z;
-          const float* pb = Qt + qbase + qz * z;
-          int s = sc0;
-          for (; s + 4 <= sc1; s += 4) {
-            const float a0 = pa[0], a1 = pa[4 * psign], a2 = pa[8 * psign], a3 = pa[12 * psign];
-            const float b0 = pb[0], b1 = pb[dq], b2 = pb[2 * dq], b3 = pb[3 * dq];
-            pa += 16 * psign;
-            pb += 4 * dq;
-            c = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b0, c, 0, 0, 0);
-            c = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b1, c, 0, 0, 0);
-            c = __builtin_amdgcn_mfma_f32_16x16x4f32(a2, b2, c, 0, 0, 0);
-            c = __builtin_amdgcn_mfma_f32_16x16x4f32(a3, b3, c, 0, 0, 0);
-          }
-          for (; s < sc1; ++s) {
-            const float a0 = pa[0], b0 = pb[0];
-            pa += 4 * psign;
-            pb += dq;
-            c = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b0, c, 0, 0, 0);
-          }
+        // One walk through the tile's steps: first steps with the test, the steps in
+        // which every lane is inside without it, last steps with it again.  A lane outside
+        // feeds zero; what it reads instead (possibly beyond the staged rows, LDS has no
+        // faults) does not matter.
+        const int z = zlo + 4 * s0 + zq;
+        const float* pa = Pt + pbase + psign * z;
+        const float* pb = Qt + qbase + qz * z;
+        unsigned zp = (unsigned)(z - plo), zy = (unsigned)(z - qlo);
+        int s = s0;
+        for (; s < sc0; ++s) {
+          float a = *pa, b = *pb;
+          a = zp <= (unsigned)pspan ? a : 0.f;
+          b = zy <= (unsigned)qspan ? b : 0.f;
+          c = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+          pa += 4 * psign;
+          pb += dq;
+          zp += 4;
+          zy += 4;
         }
-        masked(sc1, s1);
+        zp += 4 * (sc1 - sc0);
+        zy += 4 * (sc1 - sc0);
+        for (; s + 4 <= sc1; s += 4) {
+          const float a0 = pa[0], a1 = pa[4 * psign], a2 = pa[8 * psign], a3 = pa[12 * psign];
+          const float b0 = pb[0], b1 = pb[dq], b2 = pb[2 * dq], b3 = pb[3 * dq];
+          pa += 16 * psign;
+          pb += 4 * dq;
+          c = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b0, c, 0, 0, 0);
+          c = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b1, c, 0, 0, 0);
+          c = __builtin_amdgcn_mfma_f32_16x16x4f32(a2, b2, c, 0, 0, 0);
+          c = __builtin_amdgcn_mfma_f32_16x16x4f32(a3, b3, c, 0, 0, 0);
+        }
+        for (; s < sc1; ++s) {
+          const float a0 = pa[0], b0 = pb[0];
+          pa += 4 * psign;
+          pb += dq;
+          c = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b0, c, 0, 0, 0);
+        }
+        for (; s < s1; ++s) {
+          float a = *pa, b = *pb;
+          a = zp <= (unsigned)pspan ? a : 0.f;
+          b = zy <= (unsigned)qspan ? b : 0.f;
+          c = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+          pa += 4 * psign;
+          pb += dq;
+          zp += 4;
+          zy += 4;
+        }
         acc[ty] = c;
       }
     }
