@@ -1,4 +1,4 @@
-"""The dense products as `torch.library` custom operators (float32).
+"""The dense and banded products as `torch.library` custom operators (float32).
 
 `genbmm_amd.logbmm` and friends are `torch.autograd.Function`s, which `torch.compile`
 cannot trace through.  This module registers the same library calls as operators of the
@@ -10,6 +10,7 @@ autograd Functions only (genbmm/genmul.py).
 
     from genbmm_amd import ops
     y = ops.logbmm(a, b)          # also ops.maxbmm, ops.prodmaxbmm, ops.samplebmm
+    c = ops.banded_multiply_log(a_band, a_lu, a_ld, b_band, b_lu, b_ld)   # also banded_multiply, _max
 
 The arithmetic is that of genmul.py's Functions: the same C-ABI entry points with the
 same workspaces.
@@ -252,3 +253,144 @@ def samplebmm(a: Tensor, b: Tensor, seed: int, offset: int = 0) -> Tensor:
     """The Philox stream (seed, offset) is an explicit argument: a traced graph must not
     read the global generator."""
     return torch.ops.genbmm_amd.samplebmm_fwd(a, b, seed, offset)[0]
+
+
+# ----------------------------------------------------------------------- banded
+# The three banded products of genbmm_amd.sparse (reference sparse.py:404-637) as
+# operators on the band tensors themselves: a (B, n, a_lu + a_ld + 1), b likewise.
+# mode: 0 log, 1 max, 3 (+,*) - the library's GENBMM_BAND_* values.
+_BAND_LOG, _BAND_MAX, _BAND_MUL = 0, 1, 3
+
+
+def _band_dims(a: Tensor, b: Tensor, a_lu: int, a_ld: int, b_lu: int, b_ld: int):
+    if a.dtype != _F32 or b.dtype != _F32:
+        raise RuntimeError("genbmm_amd.ops: float32 tensors only (use BandedMatrix for others)")
+    if a.dim() != 3 or b.dim() != 3 or a.shape[:2] != b.shape[:2]:
+        raise RuntimeError("band tensors must be (batch, n, width) with equal batch and n")
+    if a.shape[2] != a_lu + a_ld + 1 or b.shape[2] != b_lu + b_ld + 1:
+        raise RuntimeError("band widths do not match lu + ld + 1")
+    return a.shape[0], a.shape[1], a.shape[2] + b.shape[2] - 1
+
+
+def _band_ws_size(a_lu, a_ld, b_lu, b_ld, B, n):
+    return int(_lib.load().genbmm_banded_workspace_size(int(a_lu), int(a_ld), int(b_lu), int(b_ld), int(B), int(n)))
+
+
+@torch.library.custom_op("genbmm_amd::banded_fwd", mutates_args=())
+def banded_fwd(a: Tensor, b: Tensor, a_lu: int, a_ld: int, b_lu: int, b_ld: int, mode: int) -> Tuple[Tensor, Tensor]:
+    """(out, aux): the product's band tensor (lu = a_lu + b_ld, ld = a_ld + b_lu) and what the
+    backward needs beside the operands - the arg-max (int32) for max, the library's
+    workspace for log, nothing (an empty tensor) for (+,*)."""
+    B, n, wo = _band_dims(a, b, a_lu, a_ld, b_lu, b_ld)
+    a, b = a.contiguous(), b.contiguous()
+    out = torch.empty(B, n, wo, dtype=_F32, device=a.device)
+    if mode == _BAND_MAX:
+        aux = torch.empty(B, n, wo, dtype=torch.int32, device=a.device)
+        idx, ws = aux, None
+    elif mode == _BAND_LOG:
+        aux = torch.empty(_band_ws_size(a_lu, a_ld, b_lu, b_ld, B, n), dtype=_F32, device=a.device)
+        idx, ws = None, aux
+    else:
+        aux = torch.empty(0, dtype=_F32, device=a.device)
+        idx, ws = None, None
+    _call("genbmm_banded_fwd", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld, _lib.ptr(out), _lib.ptr(idx),
+          _lib.ptr(ws), B, n, mode)
+    return out, aux
+
+
+@banded_fwd.register_fake
+def _(a, b, a_lu, a_ld, b_lu, b_ld, mode):
+    B, n, wo = a.shape[0], a.shape[1], a.shape[2] + b.shape[2] - 1
+    if mode == _BAND_MAX:
+        aux = a.new_empty((B, n, wo), dtype=torch.int32)
+    elif mode == _BAND_LOG:
+        aux = a.new_empty(_band_ws_size(a_lu, a_ld, b_lu, b_ld, B, n))
+    else:
+        aux = a.new_empty(0)
+    return a.new_empty(B, n, wo), aux
+
+
+@torch.library.custom_op("genbmm_amd::banded_bwd", mutates_args=())
+def banded_bwd(a: Tensor, b: Tensor, out: Tensor, aux: Tensor, g: Tensor, a_lu: int, a_ld: int, b_lu: int,
+               b_ld: int, mode: int) -> Tuple[Tensor, Tensor]:
+    """(grad_a, grad_b).  For the log product the library keeps g / sum in a part of the
+    workspace that nothing else reads: scratch, not a result, so `aux` is not declared
+    as mutated."""
+    B, n, _ = _band_dims(a, b, a_lu, a_ld, b_lu, b_ld)
+    a, b, g = a.contiguous(), b.contiguous(), g.contiguous()
+    grad_a, grad_b = torch.empty_like(a), torch.empty_like(b)
+    idx = aux if mode == _BAND_MAX else None
+    ws = aux if mode == _BAND_LOG else None
+    o = out if mode == _BAND_LOG else None
+    _call("genbmm_banded_bwd", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld, _lib.ptr(o), _lib.ptr(idx),
+          _lib.ptr(ws), _lib.ptr(g), _lib.ptr(grad_a), _lib.ptr(grad_b), B, n, mode)
+    return grad_a, grad_b
+
+
+@banded_bwd.register_fake
+def _(a, b, out, aux, g, a_lu, a_ld, b_lu, b_ld, mode):
+    return torch.empty_like(a), torch.empty_like(b)
+
+
+@torch.library.custom_op("genbmm_amd::banded_bwdbwd", mutates_args=())
+def banded_bwdbwd(a: Tensor, b: Tensor, out: Tensor, g: Tensor, u_a: Tensor, u_b: Tensor, a_lu: int, a_ld: int,
+                  b_lu: int, b_ld: int) -> Tuple[Tensor, Tensor, Tensor]:
+    """Log product: gradients of <u_a, grad_a> + <u_b, grad_b> with respect to (a, b, g)."""
+    B, n, _ = _band_dims(a, b, a_lu, a_ld, b_lu, b_ld)
+    a, b, g, u_a, u_b = a.contiguous(), b.contiguous(), g.contiguous(), u_a.contiguous(), u_b.contiguous()
+    ga, gb, gg = torch.empty_like(a), torch.empty_like(b), torch.empty_like(g)
+    _call("genbmm_banded_bwdbwd", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld, _lib.ptr(out), _lib.ptr(g),
+          _lib.ptr(u_a), _lib.ptr(u_b), _lib.ptr(ga), _lib.ptr(gb), _lib.ptr(gg), B, n)
+    return ga, gb, gg
+
+
+@banded_bwdbwd.register_fake
+def _(a, b, out, g, u_a, u_b, a_lu, a_ld, b_lu, b_ld):
+    return torch.empty_like(a), torch.empty_like(b), torch.empty_like(g)
+
+
+def _banded_setup(ctx, inputs, output):
+    a, b, a_lu, a_ld, b_lu, b_ld, mode = inputs
+    out, aux = output
+    ctx.save_for_backward(a, b, out, aux)
+    ctx.band = (a_lu, a_ld, b_lu, b_ld, mode)
+
+
+def _banded_backward(ctx, g_out, g_aux):
+    a, b, out, aux = ctx.saved_tensors
+    ga, gb = torch.ops.genbmm_amd.banded_bwd(a, b, out, aux, g_out, *ctx.band)
+    return ga, gb, None, None, None, None, None
+
+
+def _banded_bwd_setup(ctx, inputs, output):
+    a, b, out, _, g, a_lu, a_ld, b_lu, b_ld, mode = inputs
+    ctx.save_for_backward(a, b, out, g)
+    ctx.band = (a_lu, a_ld, b_lu, b_ld, mode)
+
+
+def _banded_bwd_backward(ctx, u_a, u_b):
+    a, b, out, g = ctx.saved_tensors
+    a_lu, a_ld, b_lu, b_ld, mode = ctx.band
+    if mode != _BAND_LOG:  # as in the reference: only the log product has second-order terms
+        raise RuntimeError("genbmm_amd.ops: only the banded log product is twice differentiable")
+    u_a = torch.zeros_like(a) if u_a is None else u_a
+    u_b = torch.zeros_like(b) if u_b is None else u_b
+    ga, gb, gg = torch.ops.genbmm_amd.banded_bwdbwd(a, b, out, g, u_a, u_b, a_lu, a_ld, b_lu, b_ld)
+    return ga, gb, None, None, gg, None, None, None, None, None
+
+
+torch.library.register_autograd("genbmm_amd::banded_fwd", _banded_backward, setup_context=_banded_setup)
+torch.library.register_autograd("genbmm_amd::banded_bwd", _banded_bwd_backward, setup_context=_banded_bwd_setup)
+
+
+def banded_multiply(a: Tensor, a_lu: int, a_ld: int, b: Tensor, b_lu: int, b_ld: int) -> Tensor:
+    """Band tensor of the (+,*) product; its band is (a_lu + b_ld, a_ld + b_lu)."""
+    return torch.ops.genbmm_amd.banded_fwd(a, b, a_lu, a_ld, b_lu, b_ld, _BAND_MUL)[0]
+
+
+def banded_multiply_log(a: Tensor, a_lu: int, a_ld: int, b: Tensor, b_lu: int, b_ld: int) -> Tensor:
+    return torch.ops.genbmm_amd.banded_fwd(a, b, a_lu, a_ld, b_lu, b_ld, _BAND_LOG)[0]
+
+
+def banded_multiply_max(a: Tensor, a_lu: int, a_ld: int, b: Tensor, b_lu: int, b_ld: int) -> Tensor:
+    return torch.ops.genbmm_amd.banded_fwd(a, b, a_lu, a_ld, b_lu, b_ld, _BAND_MAX)[0]

@@ -65,3 +65,60 @@ def test_graphs_compile_and_differentiate(gpu):
     got = compiled(a, b)
     ga, gb = torch.autograd.grad(got, (a, b))
     assert torch.equal(got, want) and torch.equal(ga, wa) and torch.equal(gb, wb)
+
+
+def band_pair(gpu, n=90, a_lu=9, a_ld=4, b_lu=6, b_ld=11, grid=False):
+    from genbmm_amd.sparse import banddiag
+    torch.manual_seed(n)
+    mk = (lambda *s: torch.round(torch.randn(*s) * 8) / 8) if grid else torch.randn
+    a = banddiag(mk(2, n, n), a_lu, a_ld)[0].contiguous().to(gpu).requires_grad_(True)
+    b = banddiag(mk(2, n, n), b_lu, b_ld)[0].contiguous().to(gpu).requires_grad_(True)
+    return a, b, (a_lu, a_ld, b_lu, b_ld)
+
+
+def test_banded_operators_match_the_band_matrix_methods(gpu):
+    from genbmm_amd.sparse import BandedMatrix
+    for grid, op, name in ((False, ops.banded_multiply, "multiply"), (False, ops.banded_multiply_log, "multiply_log"),
+                           (True, ops.banded_multiply_max, "multiply_max")):
+        a, b, (a_lu, a_ld, b_lu, b_ld) = band_pair(gpu, grid=grid)
+        y = op(a, a_lu, a_ld, b, b_lu, b_ld)
+        want = getattr(BandedMatrix(a, a_lu, a_ld), name)(BandedMatrix(b, b_lu, b_ld)).data
+        assert torch.equal(y, want)
+        g = torch.randn_like(y)
+        ga, gb = torch.autograd.grad(y, (a, b), g)
+        wa, wb = torch.autograd.grad(want, (a, b), g)
+        assert torch.equal(ga, wa) and torch.equal(gb, wb)
+    # the log product twice
+    a, b, (a_lu, a_ld, b_lu, b_ld) = band_pair(gpu)
+    u = torch.randn_like(a)
+    res = []
+    for f in (lambda: ops.banded_multiply_log(a, a_lu, a_ld, b, b_lu, b_ld),
+              lambda: BandedMatrix(a, a_lu, a_ld).multiply_log(BandedMatrix(b, b_lu, b_ld)).data):
+        y = f()
+        torch.manual_seed(3)
+        g = torch.randn_like(y)
+        (ga,) = torch.autograd.grad(y, a, g, create_graph=True)
+        res.append(torch.autograd.grad((ga * u).sum(), (a, b)))
+    assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
+
+
+def test_banded_registrations_pass_opcheck_and_compile(gpu):
+    a, b, band = band_pair(gpu, n=20, a_lu=2, a_ld=1, b_lu=1, b_ld=3)
+    ad, bd = a.detach(), b.detach()
+    tests = ("test_schema", "test_faketensor", "test_autograd_registration")
+    for mode in (0, 1, 3):
+        torch.library.opcheck(torch.ops.genbmm_amd.banded_fwd.default, (ad, bd) + band + (mode,), test_utils=tests)
+        out, aux = torch.ops.genbmm_amd.banded_fwd(ad, bd, *band, mode)
+        torch.library.opcheck(torch.ops.genbmm_amd.banded_bwd.default,
+                              (ad, bd, out, aux, torch.randn_like(out)) + band + (mode,), test_utils=tests)
+
+    def chain(x, y):
+        z = ops.banded_multiply_log(x, 2, 1, y, 1, 3)      # band (5, 2)
+        w = ops.banded_multiply(z, 5, 2, y, 1, 3)          # band (8, 3)
+        return (w * w).sum() + ops.banded_multiply_max(x, 2, 1, y, 1, 3).sum()
+
+    want = chain(a, b)
+    wa, wb = torch.autograd.grad(want, (a, b))
+    got = torch.compile(chain, backend="aot_eager", fullgraph=True)(a, b)
+    ga, gb = torch.autograd.grad(got, (a, b))
+    assert torch.equal(got, want) and torch.equal(ga, wa) and torch.equal(gb, wb)
