@@ -783,7 +783,7 @@ void k_sample_sweep_mfma(const float* __restrict__ ws_ea, const float* __restric
     for (int x = 0; x < 4; ++x)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int v = (__float_as_int(acc[x >> 1][x & 1][i]) & ~63) | tag;
+        const int v = (__float_as_int(acc[x >> 1][x & 1][i]) & ~63) | (tag & 63);  // one v_bfi_b32
         low[x >> 1][x & 1][i] = min(low[x >> 1][x & 1][i], v);
       }
     __syncthreads();
