@@ -74,13 +74,31 @@ __global__ __launch_bounds__(G * G) void k_log_item_fwd(const float* __restrict_
   const int tid = threadIdx.x, batch = blockIdx.x;
   const float* ab = a + (long)batch * M * K;
   const float* bb = b + (long)batch * K * N;
-  for (RowMajorWalk w(tid, NT, K); w.r < M; w.next()) {
-    const int m = w.r, k = w.c, e = w.r * K + w.c;
-    At[k * LD + m] = ab[e];
+  // All reads of the item are issued before the first one is waited for (a thread owns
+  // elements tid, tid + NT, ... of each operand): one trip to memory, not one per element.
+  constexpr int PER = TB * TB;  // S * S / NT
+  float ra[PER], rb[PER];
+#pragma unroll
+  for (int u = 0; u < PER; ++u) {
+    const int e = tid + u * NT;
+    ra[u] = e < M * K ? ab[e] : 0.f;
+    rb[u] = e < K * N ? bb[e] : 0.f;
   }
-  for (RowMajorWalk w(tid, NT, N); w.r < K; w.next()) {
-    const int k = w.r, n = w.c, e = w.r * N + w.c;
-    Bs[k * LD + n] = bb[e];
+  {
+    RowMajorWalk w(tid, NT, K);
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      if (w.r < M) At[w.c * LD + w.r] = ra[u];
+      w.next();
+    }
+  }
+  {
+    RowMajorWalk w(tid, NT, N);
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      if (w.r < K) Bs[w.r * LD + w.c] = rb[u];
+      w.next();
+    }
   }
   __syncthreads();
   // row / column maxima: one thread per row, one per column (LDS atomics on the
@@ -171,13 +189,32 @@ __global__ __launch_bounds__(G * G) void k_log_item_bwd(const float* __restrict_
   const float* gb = g + (long)batch * M * N;
   float* gab = grad_a ? grad_a + (long)batch * M * K : nullptr;
   float* gbb = grad_b ? grad_b + (long)batch * K * N : nullptr;
-  for (RowMajorWalk w(tid, NT, K); w.r < M; w.next()) {
-    const int m = w.r, k = w.c, e = w.r * K + w.c;
-    Ea[m * LD + k] = ab[e];
+  // all reads of the item in flight together (see the forward)
+  constexpr int PER = TB * TB;
+  float ra[PER], rb[PER], ro[PER], rg[PER];
+#pragma unroll
+  for (int u = 0; u < PER; ++u) {
+    const int e = tid + u * NT;
+    ra[u] = e < M * K ? ab[e] : 0.f;
+    rb[u] = e < K * N ? bb[e] : 0.f;
+    ro[u] = e < M * N ? ob[e] : 0.f;
+    rg[u] = e < M * N ? gb[e] : 0.f;
   }
-  for (RowMajorWalk w(tid, NT, N); w.r < K; w.next()) {
-    const int k = w.r, n = w.c, e = w.r * N + w.c;
-    Eb[k * LD + n] = bb[e];
+  {
+    RowMajorWalk w(tid, NT, K);
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      if (w.r < M) Ea[w.r * LD + w.c] = ra[u];
+      w.next();
+    }
+  }
+  {
+    RowMajorWalk w(tid, NT, N);
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      if (w.r < K) Eb[w.r * LD + w.c] = rb[u];
+      w.next();
+    }
   }
   __syncthreads();
   if (tid < M) {
@@ -200,11 +237,18 @@ __global__ __launch_bounds__(G * G) void k_log_item_bwd(const float* __restrict_
     const int k = w.r, n = w.c, e = w.r * N + w.c;
     Eb[k * LD + n] = item_exp(Eb[k * LD + n], be[n]);
   }
-  for (RowMajorWalk w(tid, NT, N); w.r < M; w.next()) {
-    const int m = w.r, n = w.c, e = w.r * N + w.c;
-    const float ex = al[m] + be[n] - ob[e];
-    if (!(ex <= lim) || !(ex > -INFINITY)) bad = 1;  // S < 2^-40, NaN or infinities: not exact
-    Hs[m * LD + n] = gb[e] * fast_exp2(ex * kLog2e);
+  {
+    RowMajorWalk w(tid, NT, N);
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      if (w.r < M) {
+        const int m = w.r, n = w.c;
+        const float ex = al[m] + be[n] - ro[u];
+        if (!(ex <= lim) || !(ex > -INFINITY)) bad = 1;  // S < 2^-40, NaN or infinities: not exact
+        Hs[m * LD + n] = rg[u] * fast_exp2(ex * kLog2e);
+      }
+      w.next();
+    }
   }
   bad = __syncthreads_or(bad);
   if (bad) {
