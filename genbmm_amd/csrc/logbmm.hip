@@ -871,7 +871,11 @@ int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats, 
   if (missing(a, mk) || missing(b, kn) || missing(out, mn)) return GENBMM_E_NULLPTR;
   hipStream_t s = (hipStream_t)stream;
   if (stats && B > 0 && item_shape(M, K, N) && g_path.load() == 0) {  // whole items per workgroup
-    if (max(max(M, K), N) <= 32)
+    if (M == 32 && K == 32 && N == 32)
+      hipLaunchKernelGGL((k_log_item_fwd<16, 2, true>), dim3(B), dim3(256), 0, s, a, b, out, stats, M, K, N);
+    else if (M == 64 && K == 64 && N == 64)
+      hipLaunchKernelGGL((k_log_item_fwd<16, 4, true>), dim3(B), dim3(256), 0, s, a, b, out, stats, M, K, N);
+    else if (max(max(M, K), N) <= 32)
       hipLaunchKernelGGL((k_log_item_fwd<16, 2>), dim3(B), dim3(256), 0, s, a, b, out, stats, M, K, N);
     else
       hipLaunchKernelGGL((k_log_item_fwd<16, 4>), dim3(B), dim3(256), 0, s, a, b, out, stats, M, K, N);
@@ -921,7 +925,11 @@ int genbmm_logbmm_bwd(const float* a, const float* b, const float* out, const fl
   hipStream_t s = (hipStream_t)stream;
   const float* st = (g_path.load() == 1 || mn == 0) ? nullptr : stats;
   if (st && B > 0 && item_shape(M, K, N) && g_path.load() == 0) {
-    if (max(max(M, K), N) <= 32)
+    if (M == 32 && K == 32 && N == 32)
+      hipLaunchKernelGGL((k_log_item_bwd<16, 2, true>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
+    else if (M == 64 && K == 64 && N == 64)
+      hipLaunchKernelGGL((k_log_item_bwd<16, 4, true>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
+    else if (max(max(M, K), N) <= 32)
       hipLaunchKernelGGL((k_log_item_bwd<16, 2>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
     else
       hipLaunchKernelGGL((k_log_item_bwd<16, 4>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);

@@ -60,13 +60,16 @@ __device__ __forceinline__ float item_exp(float x, float shift) {
 // covers items up to 32 x 32, TB = 4 up to 64 x 64.  (One wave per item, G = 8 and
 // TB = 4, measured slower at 8192 items of 32^3: the chain of dependent phases of
 // an item gets longer than the extra items in flight make up for.)
-template <int G, int TB>
+// FULL: M = K = N = G * TB, known to the compiler - the index arithmetic that is most of
+// the general kernel's instructions (it is issue-bound, not memory-bound) folds away.
+template <int G, int TB, bool FULL = false>
 __global__ __launch_bounds__(G * G) void k_log_item_fwd(const float* __restrict__ a,
                                                       const float* __restrict__ b,
                                                       float* __restrict__ out,
-                                                      float* __restrict__ stats, int M, int K,
-                                                      int N) {
+                                                      float* __restrict__ stats, int M_, int K_,
+                                                      int N_) {
   constexpr int NT = G * G, S = G * TB, LD = S + 1;
+  const int M = FULL ? S : M_, K = FULL ? S : K_, N = FULL ? S : N_;
   static_assert(2 * S <= NT, "row and column scans use 2*S threads");
   __shared__ float At[S * LD];  // [k][m]: a, then EA; finally the output tile [m][n]
   __shared__ float Bs[S * LD];  // [k][n]: b, then EB
@@ -168,15 +171,16 @@ __global__ __launch_bounds__(G * G) void k_log_item_fwd(const float* __restrict_
   }
 }
 
-template <int G, int TB>
-__global__ __launch_bounds__(G * G) void k_log_item_bwd(const float* __restrict__ a,
+template <int G, int TB, bool FULL = false>
+__global__ __launch_bounds__(G * G, TB == 2 ? 6 : 1) void k_log_item_bwd(const float* __restrict__ a,
                                                       const float* __restrict__ b,
                                                       const float* __restrict__ outp,
                                                       const float* __restrict__ g,
                                                       float* __restrict__ grad_a,
-                                                      float* __restrict__ grad_b, int M, int K,
-                                                      int N) {
+                                                      float* __restrict__ grad_b, int M_, int K_,
+                                                      int N_) {
   constexpr int NT = G * G, S = G * TB, LD = S + 1;
+  const int M = FULL ? S : M_, K = FULL ? S : K_, N = FULL ? S : N_;
   static_assert(2 * S <= NT, "row and column scans use 2*S threads");
   __shared__ float Ea[S * LD];  // [m][k]: a, EA, finally grad_a
   __shared__ float Eb[S * LD];  // [k][n]: b, EB, finally grad_b
