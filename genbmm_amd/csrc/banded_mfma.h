@@ -262,6 +262,13 @@ __global__ __launch_bounds__(256, 2) void k_band_mm(const BandArgs p, int strips
     sp.init(pt, pt + (FWD ? cells_a : cells_o), (bn + x0) * Wp, (pr1 - x0) * Wp, Wp, d.pp);
     sp.load(pt, pt + (FWD ? cells_a : cells_o), 0, tid);
   }
+  // forward of the log product: the row maxima too are requested before anything is waited for
+  float alv = 0.f, bev = 0.f;
+  if (FWD && PREP) {
+    if (tid < ROWS && x0 + tid < n) alv = p.ws_al[bn + x0 + tid];
+    const int o = q0 + tid;
+    if (tid < d.q_rows && o >= 0 && o < n) bev = p.ws_be[bn + o];
+  }
   if (tid <= ROWS) badrow[tid] = 0;
   __syncthreads();
   bool bad = sq.store(QL, 0, tid);
@@ -290,8 +297,9 @@ __global__ __launch_bounds__(256, 2) void k_band_mm(const BandArgs p, int strips
   }
   if (bad) *redo = 1;
   if (FWD && PREP) {
-    if (tid < ROWS) al[tid] = x0 + tid < n ? p.ws_al[bn + x0 + tid] : 0.f;
-    for (int t = tid; t < d.q_rows; t += 256) {
+    if (tid < ROWS) al[tid] = alv;
+    if (tid < d.q_rows) be[tid] = bev;
+    for (int t = tid + 256; t < d.q_rows; t += 256) {
       const int o = q0 + t;
       be[t] = (o >= 0 && o < n) ? p.ws_be[bn + o] : 0.f;
     }
@@ -471,6 +479,72 @@ __global__ __launch_bounds__(256, 2) void k_band_mm(const BandArgs p, int strips
   const float thr = fast_exp2(-kBandGuardBits);
   const float* xe = PREP && !FWD ? (GA ? p.ws_ea : p.ws_eb) + (bn + x0) * Wout : nullptr;
   float* rb = PREP && FWD ? p.ws_r + (bn + x0) * Wout : nullptr;
+  // Prepared log product away from trouble: four cells per lane, 16-byte loads and stores
+  // (4-byte stores of a wave reach memory as more than their bytes: 426 MiB were
+  // written for the forward's 258 MiB of out and 1/S).
+  const bool vec_ok = PREP && !whole && (cells & 3) == 0 && Wout >= 4 && (reinterpret_cast<uintptr_t>(ob) & 15) == 0 &&
+                      (FWD ? (reinterpret_cast<uintptr_t>(rb) & 15) == 0 : (reinterpret_cast<uintptr_t>(xe) & 15) == 0);
+  if (PREP && vec_ok) {
+    for (int e = 4 * tid; e < cells; e += 1024) {
+      const mm_f4 sv = *reinterpret_cast<const mm_f4*>(S + e);
+      const int r0 = (int)__umulhi((unsigned)e, magic), k0 = e - r0 * Wout;
+      mm_f4 ov, rv4;
+      bool redo_cell[4];
+      if (FWD) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const bool wrap = k0 + t >= Wout;  // Wout >= 4: one row change at most
+          const int r = r0 + (wrap ? 1 : 0), k = k0 + t - (wrap ? Wout : 0);
+          const int o = x0 + r + k - r_lu;
+          float v = sv[t], rv = 0.f;
+          redo_cell[t] = false;
+          if (o >= 0 && o < n) {
+            const float sh = al[r] + be[o - q0];
+            if ((v >= thr) && (v < INFINITY) && (sh > 0.9f * kFloor) && (sh < INFINITY)) {
+              rv = __builtin_amdgcn_rcpf(v);
+              v = __builtin_fmaf(fast_log2(v), kLn2, sh);
+            } else {
+              redo_cell[t] = true;
+              rv = -1.f;  // tells the backward that 1/S is not usable here
+            }
+          } else {
+            v = 0.f;  // outside the matrix: the reference's zero fill
+          }
+          ov[t] = v;
+          rv4[t] = rv;
+        }
+        // factoring not exact for a cell: recompute it from memory
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          if (redo_cell[t]) {
+            const bool wrap = k0 + t >= Wout;
+            const int r = r0 + (wrap ? 1 : 0), k = k0 + t - (wrap ? Wout : 0);
+            ov[t] = band_fwd_cell_log_exact(p, bn + x0 + r, x0 + r, k);
+          }
+        *reinterpret_cast<mm_f4*>(ob + e) = ov;
+        *reinterpret_cast<mm_f4*>(rb + e) = rv4;
+      } else {
+        const mm_f4 xv = *reinterpret_cast<const mm_f4*>(xe + e);
+        const bool wrapped = k0 + 3 >= Wout;
+        if (!badrow[r0] && !(wrapped && badrow[r0 + 1])) {
+          *reinterpret_cast<mm_f4*>(ob + e) = xv * sv;
+        } else {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const bool wrap = k0 + t >= Wout;
+            const int r = r0 + (wrap ? 1 : 0), k = k0 + t - (wrap ? Wout : 0);
+            if (badrow[r]) {
+              if (GA) band_bwd_a_cell<GENBMM_BAND_LOG>(p, bn + x0 + r, x0 + r, k);
+              else band_bwd_b_cell<GENBMM_BAND_LOG>(p, bn + x0 + r, x0 + r, k);
+            } else {
+              ob[e + t] = xv[t] * sv[t];
+            }
+          }
+        }
+      }
+    }
+    return;
+  }
   for (int e = tid; e < cells; e += 256) {
     float v = S[e];
     const int r = Wout == 1 ? e : (int)__umulhi((unsigned)e, magic), k = e - r * Wout;
