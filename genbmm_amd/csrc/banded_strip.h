@@ -132,7 +132,7 @@ struct RowStage {
 };
 
 // ------------------------------------------------------------ prepared operands
-// One wave per band row: shift = maximum over the cells inside the matrix (-inf if
+// Four lanes per band row: shift = maximum over the cells inside the matrix (-inf if
 // there is none), e = exp(x - shift), 0 for cells outside.  With these the log
 // product is a (+,x) product of e's plus an epilogue, and no kernel downstream
 // takes an exponential per staged element again.
@@ -147,26 +147,42 @@ __global__ __launch_bounds__(256) void k_band_prep(const float* __restrict__ x, 
   const int nr = (int)min((long)kPrepRows, rows - row0);
   const float* xb = x + row0 * W;
   float* eb = e + row0 * W;
-  // the block is contiguous in memory: coalesced in, row per lane inside, coalesced out
-  for (int i = tid, r = tid / W, k = tid - (tid / W) * W; i < nr * W; i += 256) {
-    tile[r * ld + k] = xb[i];
-    r += 256 / W;
-    k += 256 % W;
-    if (k >= W) {
-      k -= W;
-      ++r;
+  // the block is contiguous in memory: coalesced in (batches of reads in flight together),
+  // rows inside, coalesced out
+  constexpr int U = 8;
+  for (int i0 = tid, r = tid / W, k = tid - (tid / W) * W; i0 < nr * W; i0 += 256 * U) {
+    float v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = i0 + 256 * u < nr * W ? xb[i0 + 256 * u] : 0.f;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (i0 + 256 * u < nr * W) tile[r * ld + k] = v[u];
+      r += 256 / W;
+      k += 256 % W;
+      if (k >= W) {
+        k -= W;
+        ++r;
+      }
     }
   }
   __syncthreads();
-  if (tid < nr) {
-    const int c = (int)((row0 + tid) % n);
+  {  // four lanes per row, a quarter of its cells each
+    const int r = tid >> 2, part = tid & 3;
+    const int q = (W + 3) >> 2, k0 = part * q, k1 = min(W, k0 + q);
+    const bool live = r < nr;
+    const int c = live ? (int)((row0 + r) % n) : 0;
     const int klo = max(0, lu - c), khi = min(W - 1, n - 1 + lu - c);  // cells inside the matrix
-    float* tr = tile + tid * ld;
+    float* tr = tile + r * ld;
     float m = -INFINITY;
-    for (int k = klo; k <= khi; ++k) m = fmaxf(m, tr[k]);
-    shift[row0 + tid] = m;
-    const float sh = m == -INFINITY ? 0.f : m;
-    for (int k = 0; k < W; ++k) tr[k] = (k >= klo && k <= khi) ? fast_exp2((tr[k] - sh) * kLog2e) : 0.f;
+    if (live)
+      for (int k = max(k0, klo); k < min(k1, khi + 1); ++k) m = fmaxf(m, tr[k]);
+    m = fmaxf(m, __shfl_xor(m, 1, 64));
+    m = fmaxf(m, __shfl_xor(m, 2, 64));
+    if (live) {
+      if (part == 0) shift[row0 + r] = m;
+      const float sh = m == -INFINITY ? 0.f : m;
+      for (int k = k0; k < k1; ++k) tr[k] = (k >= klo && k <= khi) ? fast_exp2((tr[k] - sh) * kLog2e) : 0.f;
+    }
   }
   __syncthreads();
   for (int i = tid, r = tid / W, k = tid - (tid / W) * W; i < nr * W; i += 256) {
