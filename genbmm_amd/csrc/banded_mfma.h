@@ -214,6 +214,13 @@ struct MmSkew {
 
 __device__ __forceinline__ int mm_clamp(int x, int lo, int hi) { return min(max(x, lo), hi); }
 
+// The exact recompute of one cell, inline: a call would give the kernel a stack frame
+// that every lane writes to memory (168 bytes each, 168 MiB per launch at 64 x 4096).
+__device__ __forceinline__ float mm_fwd_cell_log_exact(const BandArgs& p, long bi, int i, int j) {
+  band_fwd_cell<GENBMM_BAND_LOG>(p, bi, i, j);
+  return p.o0[bi * p.Wo + j];
+}
+
 template <int KIND, bool PREP>
 __global__ __launch_bounds__(256, 2) void k_band_mm(const BandArgs p, int strips, const MmDims d, long cells_a,
                                                     long cells_b, long cells_o) {
@@ -519,7 +526,7 @@ __global__ __launch_bounds__(256, 2) void k_band_mm(const BandArgs p, int strips
           if (redo_cell[t]) {
             const bool wrap = k0 + t >= Wout;
             const int r = r0 + (wrap ? 1 : 0), k = k0 + t - (wrap ? Wout : 0);
-            ov[t] = band_fwd_cell_log_exact(p, bn + x0 + r, x0 + r, k);
+            ov[t] = mm_fwd_cell_log_exact(p, bn + x0 + r, x0 + r, k);
           }
         *reinterpret_cast<mm_f4*>(ob + e) = ov;
         *reinterpret_cast<mm_f4*>(rb + e) = rv4;
@@ -558,7 +565,7 @@ __global__ __launch_bounds__(256, 2) void k_band_mm(const BandArgs p, int strips
           rv = __builtin_amdgcn_rcpf(v);
           v = __builtin_fmaf(fast_log2(v), kLn2, sh);
         } else {  // factoring not exact for this cell: recompute it from memory
-          v = band_fwd_cell_log_exact(p, bn + xx, xx, k);
+          v = mm_fwd_cell_log_exact(p, bn + xx, xx, k);
           rv = -1.f;  // tells the backward that 1/S is not usable here
         }
       } else {
