@@ -39,6 +39,7 @@ SIGNATURES = {
     "genbmm_prodmax_bwd": [_c_float_p] * 2 + [_c_int_p] + [_c_float_p] * 4 + _DENSE_DIMS,
     "genbmm_banded_fwd": _BAND + [_c_float_p, _c_int_p, _c_float_p, _i, _i, _i, _vp],
     "genbmm_banded_bwd": _BAND + [_c_float_p, _c_int_p] + [_c_float_p] * 4 + [_i, _i, _i, _vp],
+    "genbmm_banded_bwd_scratch": _BAND + [_c_float_p, _c_int_p] + [_c_float_p] * 5 + [_i, _i, _i, _vp],
     "genbmm_banded_bwdbwd": _BAND + [_c_float_p] * 7 + [_i, _i, _vp],
     "genbmm_logbmm_fwd_f64": [_c_float_p] * 3 + _DENSE_DIMS,
     "genbmm_logbmm_bwd_f64": [_c_float_p] * 6 + _DENSE_DIMS,

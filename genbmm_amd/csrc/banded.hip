@@ -47,29 +47,34 @@ inline bool bwd_strip_ok(const BandArgs& p) {
   return max(bwd_strip_bytes(da, true), bwd_strip_bytes(db, true)) <= kStripLdsLimit &&
          max(max(da.ld_own, da.ld_sl), max(db.ld_own, db.ld_sl)) <= 128;
 }
-// The workspace is filled and used only when both directions run strip kernels, so
-// that forward and backward always agree on whether it holds anything.
-inline bool workspace_used(const BandArgs& p) {
-  return fwd_strip_ok(p) && bwd_strip_ok(p) &&
-         strip_dims(p.Wa, p.Wb).bytes + sizeof(float) * (kBT + p.Wo + kBJ) <= kStripLdsLimit;
-}
-
-inline bool prep_fwd(const BandArgs& p, int mode, const float* workspace) {
-  return mode == GENBMM_BAND_LOG && workspace != nullptr && workspace_used(p);
-}
-
 // Which bands the matrix-core kernels take: wide enough for 16 x 16 tiles to pay (measured
 // against the strip kernels at 64 x 4096: forward from 9 diagonals on, gradients from 25),
 // and two workgroups' tiles fit in a compute unit's LDS.
 constexpr size_t kMmLdsLimit = 80 * 1024;
-inline bool mm_fwd_ok(const BandArgs& p) {
-  return mm_tiles_ok(p.Wa, p.Wb, p.Wo) && min(p.Wa, p.Wb) >= 8 &&
+// (the log product takes the forward from 4 diagonals on: what it replaces there is the
+// per-cell kernel pair with an exponential per term, 0.26 ms against 0.18 at 5 diagonals)
+inline bool mm_fwd_ok(const BandArgs& p, int min_w = 8) {
+  return mm_tiles_ok(p.Wa, p.Wb, p.Wo) && min(p.Wa, p.Wb) >= min_w &&
          mm_dims(kMmFwd, p.Wa, p.Wb, p.Wo).bytes <= kMmLdsLimit;
 }
 inline bool mm_bwd_ok(const BandArgs& p) {
   return mm_tiles_ok(p.Wa, p.Wb, p.Wo) && min(p.Wa, p.Wb) >= 25 &&
          max(mm_dims(kMmGradA, p.Wa, p.Wb, p.Wo).bytes, mm_dims(kMmGradB, p.Wa, p.Wb, p.Wo).bytes) <= kMmLdsLimit;
 }
+// The workspace of the log product is filled and used only when both directions have a
+// kernel that works on it (matrix-core or strip), so that forward and backward always agree
+// on whether it holds anything.
+inline bool workspace_used(const BandArgs& p) {
+  const bool fwd = mm_fwd_ok(p, 4) ||
+                   (fwd_strip_ok(p) &&
+                    strip_dims(p.Wa, p.Wb).bytes + sizeof(float) * (kBT + p.Wo + kBJ) <= kStripLdsLimit);
+  return fwd && (mm_bwd_ok(p) || bwd_strip_ok(p));
+}
+
+inline bool prep_fwd(const BandArgs& p, int mode, const float* workspace) {
+  return mode == GENBMM_BAND_LOG && workspace != nullptr && workspace_used(p);
+}
+
 template <int KIND, bool PREP>
 inline void launch_mm(const BandArgs& p, int B, hipStream_t s) {
   const MmDims d = mm_dims(KIND, p.Wa, p.Wb, p.Wo);
@@ -120,7 +125,7 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   if (total == 0) return GENBMM_OK;
   hipStream_t s = (hipStream_t)stream;
   const StripDims sd = strip_dims(p.Wa, p.Wb);
-  if (mode != GENBMM_BAND_MAX && mm_fwd_ok(p) && (mode == GENBMM_BAND_MUL || prep_fwd(p, mode, workspace))) {
+  if ((mode == GENBMM_BAND_MUL && mm_fwd_ok(p)) || (prep_fwd(p, mode, workspace) && mm_fwd_ok(p, 4))) {
     if (mode == GENBMM_BAND_LOG) {
       set_workspace(p, workspace, B);
       const long rows = (long)B * n;
@@ -177,10 +182,12 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   return launch_status();
 }
 
-int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
-                      const float* out, const int32_t* idx, float* workspace, const float* g,
-                      float* grad_a, float* grad_b, int B, int n, int mode, void* stream) {
-  using namespace genbmm;
+namespace genbmm {
+namespace {
+// `scratch`: where g / S goes in the prepared log product; NULL: the workspace's own part
+int banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
+               const float* out, const int32_t* idx, float* workspace, float* scratch, const float* g,
+               float* grad_a, float* grad_b, int B, int n, int mode, void* stream) {
   if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
     return GENBMM_E_MODE;
   BandArgs p{};
@@ -200,6 +207,7 @@ int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   }
   if (mode == GENBMM_BAND_LOG && workspace && workspace_used(p) && mm_bwd_ok(p)) {
     set_workspace(p, workspace, B);
+    if (scratch) p.ws_h = scratch;
     const long cells = (long)B * n * p.Wo;
     hipLaunchKernelGGL(k_band_h, dim3((unsigned)min((cells + 1023) / 1024, (long)0x7fffffff)), dim3(256), 0,
                        s, g, p.ws_r, p.ws_h, cells);
@@ -217,6 +225,7 @@ int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_
       const int nq = ceil_div(max(max(da.ld_own, da.ld_sl), max(db.ld_own, db.ld_sl)), 64);
       if (lg && workspace && workspace_used(p)) {  // on the forward's workspace: a (+,x) backward plus epilogue
         set_workspace(p, workspace, B);
+        if (scratch) p.ws_h = scratch;
         // H = g * R once for both gradients (NaN marks a cell whose R is not usable)
         const long cells = (long)B * n * p.Wo;
         hipLaunchKernelGGL(k_band_h, dim3((unsigned)min((cells + 1023) / 1024, (long)0x7fffffff)),
@@ -270,6 +279,25 @@ int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   }
   return launch_status();
 }
+}  // namespace
+}  // namespace genbmm
+
+int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
+                      const float* out, const int32_t* idx, float* workspace, const float* g,
+                      float* grad_a, float* grad_b, int B, int n, int mode, void* stream) {
+  return genbmm::banded_bwd(a, a_lu, a_ld, b, b_lu, b_ld, out, idx, workspace, nullptr, g, grad_a, grad_b, B, n,
+                            mode, stream);
+}
+
+int genbmm_banded_bwd_scratch(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
+                              const float* out, const int32_t* idx, const float* workspace, float* scratch,
+                              const float* g, float* grad_a, float* grad_b, int B, int n, int mode,
+                              void* stream) {
+  if (workspace && !scratch) return GENBMM_E_NULLPTR;
+  return genbmm::banded_bwd(a, a_lu, a_ld, b, b_lu, b_ld, out, idx, const_cast<float*>(workspace), scratch, g,
+                            grad_a, grad_b, B, n, mode, stream);
+}
+
 
 int genbmm_banded_bwdbwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
                          const float* out, const float* g, const float* u_a, const float* u_b,

@@ -206,7 +206,7 @@ __device__ __forceinline__ int xcd_strip_id() {
 
 // The exact recompute of one cell, kept out of line: it is rare, and inlined it costs
 // the strip kernels registers they do not have.
-__device__ __attribute__((noinline)) float band_fwd_cell_log_exact(const BandArgs& p, long bi, int i, int j) {
+__device__ __forceinline__ float band_fwd_cell_log_exact(const BandArgs& p, long bi, int i, int j) {
   band_fwd_cell<GENBMM_BAND_LOG>(p, bi, i, j);
   return p.o0[bi * p.Wo + j];
 }

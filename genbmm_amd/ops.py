@@ -313,17 +313,17 @@ def _(a, b, a_lu, a_ld, b_lu, b_ld, mode):
 @torch.library.custom_op("genbmm_amd::banded_bwd", mutates_args=())
 def banded_bwd(a: Tensor, b: Tensor, out: Tensor, aux: Tensor, g: Tensor, a_lu: int, a_ld: int, b_lu: int,
                b_ld: int, mode: int) -> Tuple[Tensor, Tensor]:
-    """(grad_a, grad_b).  For the log product the library keeps g / sum in a part of the
-    workspace that nothing else reads: scratch, not a result, so `aux` is not declared
-    as mutated."""
-    B, n, _ = _band_dims(a, b, a_lu, a_ld, b_lu, b_ld)
+    """(grad_a, grad_b).  For the log product the library keeps g / sum per output cell
+    beside the workspace: in a buffer of this call's own, so that `aux` is only read."""
+    B, n, wo = _band_dims(a, b, a_lu, a_ld, b_lu, b_ld)
     a, b, g = a.contiguous(), b.contiguous(), g.contiguous()
     grad_a, grad_b = torch.empty_like(a), torch.empty_like(b)
     idx = aux if mode == _BAND_MAX else None
     ws = aux if mode == _BAND_LOG else None
     o = out if mode == _BAND_LOG else None
-    _call("genbmm_banded_bwd", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld, _lib.ptr(o), _lib.ptr(idx),
-          _lib.ptr(ws), _lib.ptr(g), _lib.ptr(grad_a), _lib.ptr(grad_b), B, n, mode)
+    scratch = torch.empty(B * n * wo, dtype=_F32, device=a.device) if mode == _BAND_LOG else None
+    _call("genbmm_banded_bwd_scratch", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld, _lib.ptr(o),
+          _lib.ptr(idx), _lib.ptr(ws), _lib.ptr(scratch), _lib.ptr(g), _lib.ptr(grad_a), _lib.ptr(grad_b), B, n, mode)
     return grad_a, grad_b
 
 

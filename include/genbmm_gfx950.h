@@ -240,6 +240,22 @@ int genbmm_banded_bwd(const float* a, int a_lu, int a_ld,
                       int B, int n, int mode, void* stream);
 
 /*
+ * genbmm_banded_bwd with the workspace left untouched: what the backward keeps
+ * beside it (g/S per output cell, mode LOG with a workspace only) goes to
+ * `scratch`, B * n * Wo floats, which must be given whenever `workspace` is.
+ * For callers that must not write to what the forward returned - operator
+ * frameworks that check their inputs for mutation, or several backward calls
+ * on one workspace at a time, each with a scratch buffer of its own.  Same
+ * reference counterpart as genbmm_banded_bwd.
+ */
+int genbmm_banded_bwd_scratch(const float* a, int a_lu, int a_ld,
+                              const float* b, int b_lu, int b_ld,
+                              const float* out, const int32_t* idx,
+                              const float* workspace, float* scratch,
+                              const float* g, float* grad_a, float* grad_b,
+                              int B, int n, int mode, void* stream);
+
+/*
  * Log-semiring second-order terms: gradients with respect to (a, b, g) of
  * <u_a, grad_a> + <u_b, grad_b> for the outputs of genbmm_banded_bwd in mode
  * LOG.  u_a or u_b may be NULL (zeros), not both.

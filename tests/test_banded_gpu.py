@@ -236,3 +236,36 @@ def test_banded_log_without_workspace(gpu, n, a_lu, a_ld, b_lu, b_ld):
     close(out, want)
     close(ga, wa)
     close(gb, wb)
+
+
+@pytest.mark.parametrize("n,a_lu,a_ld,b_lu,b_ld", [(70, 3, 5, 4, 2), (150, 14, 13, 12, 15), (64, 8, 8, 8, 8)])
+def test_backward_with_separate_scratch_leaves_the_workspace_alone(gpu, n, a_lu, a_ld, b_lu, b_ld):
+    """genbmm_banded_bwd_scratch: same gradients as genbmm_banded_bwd, bit for bit, and the
+    workspace the forward filled is not written."""
+    lib = _lib.load()
+    torch.manual_seed(n)
+    a, b = pair(n, a_lu, a_ld, b_lu, b_ld)
+    B, W = 3, a.shape[2] + b.shape[2] - 1
+    ad, bd, g = a.to(gpu), b.to(gpu), torch.randn(B, n, W).to(gpu)
+    out = torch.empty(B, n, W, device=gpu)
+    ws = torch.zeros(lib.genbmm_banded_workspace_size(a_lu, a_ld, b_lu, b_ld, B, n), device=gpu)
+    s, p = _lib.stream_of(ad), _lib.ptr
+    assert lib.genbmm_banded_fwd(p(ad), a_lu, a_ld, p(bd), b_lu, b_ld, p(out), p(None), p(ws), B, n, 0, s) == 0
+    before = ws.clone()
+    scratch = torch.empty(B * n * W, device=gpu)
+    ga, gb = torch.empty_like(ad), torch.empty_like(bd)
+    assert lib.genbmm_banded_bwd_scratch(p(ad), a_lu, a_ld, p(bd), b_lu, b_ld, p(out), p(None), p(ws), p(scratch),
+                                         p(g), p(ga), p(gb), B, n, 0, s) == 0
+    assert torch.equal(ws, before)
+    wa, wb = torch.empty_like(ad), torch.empty_like(bd)
+    assert lib.genbmm_banded_bwd(p(ad), a_lu, a_ld, p(bd), b_lu, b_ld, p(out), p(None), p(ws), p(g), p(wa), p(wb),
+                                 B, n, 0, s) == 0
+    assert torch.equal(ga, wa) and torch.equal(gb, wb)
+    # a workspace without scratch is refused; the other modes take neither
+    assert lib.genbmm_banded_bwd_scratch(p(ad), a_lu, a_ld, p(bd), b_lu, b_ld, p(out), p(None), p(ws), p(None),
+                                         p(g), p(ga), p(gb), B, n, 0, s) != 0
+    assert lib.genbmm_banded_bwd_scratch(p(ad), a_lu, a_ld, p(bd), b_lu, b_ld, p(None), p(None), p(None), p(None),
+                                         p(g), p(ga), p(gb), B, n, 3, s) == 0
+    assert lib.genbmm_banded_bwd(p(ad), a_lu, a_ld, p(bd), b_lu, b_ld, p(None), p(None), p(None), p(g), p(wa), p(wb),
+                                 B, n, 3, s) == 0
+    assert torch.equal(ga, wa) and torch.equal(gb, wb)
