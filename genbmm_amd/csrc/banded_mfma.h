@@ -487,8 +487,7 @@ __global__ __launch_bounds__(256, 2) void k_band_mm(const BandArgs p, int strips
   const float* xe = PREP && !FWD ? (GA ? p.ws_ea : p.ws_eb) + (bn + x0) * Wout : nullptr;
   float* rb = PREP && FWD ? p.ws_r + (bn + x0) * Wout : nullptr;
   // Prepared log product away from trouble: four cells per lane, 16-byte loads and stores
-  // (4-byte stores of a wave reach memory as more than their bytes: 426 MiB were
-  // written for the forward's 258 MiB of out and 1/S).
+  // (a quarter of the index arithmetic and memory instructions of the cell-by-cell loop).
   const bool vec_ok = PREP && !whole && (cells & 3) == 0 && Wout >= 4 && (reinterpret_cast<uintptr_t>(ob) & 15) == 0 &&
                       (FWD ? (reinterpret_cast<uintptr_t>(rb) & 15) == 0 : (reinterpret_cast<uintptr_t>(xe) & 15) == 0);
   if (PREP && vec_ok) {
