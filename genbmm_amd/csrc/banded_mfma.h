@@ -186,27 +186,33 @@ struct MmSkew {
 
   __device__ __forceinline__ void init(int Wo) { total = (Wo + 31) * 32; }
   __device__ __forceinline__ bool more(int batch) const { return batch * 256 * U < total; }
+  // Cell number tid + 256 u is (row r of g' counted from ilo, column c of the strip) with
+  // c = tid % 32 fixed and r = tid / 32 + 8 u: its address moves by 8 (Wo - 1) floats per
+  // u, its band index j = c + Wo - 1 - r by -8.  j is inside the band for r in
+  // [c, c + Wo); the cell exists for the r that are also rows of the matrix.
   __device__ __forceinline__ void load(const float* __restrict__ src, int Wo, int r_lu, int n, int x0,
                                        int batch, int tid) {
-    const int ilo = x0 + r_lu - (Wo - 1);
+    const int ilo = x0 + r_lu - (Wo - 1), c = tid & 31, r0 = (tid >> 5) + 8 * U * batch;
+    const int rlo = max(c, -ilo), rhi = x0 + c < n ? min(c + Wo, n - ilo) : rlo;
+    const float* q = src + ((long)(ilo + r0) * Wo + (c + Wo - 1 - r0));
+    const long step = 8L * (Wo - 1);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int eu = tid + 256 * (u + batch * U), r = eu >> 5, c = eu & 31;
-      const int i = ilo + r, j = c + Wo - 1 - r;
-      const bool ok = eu < total && j >= 0 && j < Wo && i >= 0 && i < n && x0 + c < n;
-      v[u] = ok ? src[(long)i * Wo + j] : 0.f;
+      const int r = r0 + 8 * u;
+      v[u] = (r >= rlo && r < rhi) ? q[u * step] : 0.f;
     }
   }
   __device__ __forceinline__ void store(float* __restrict__ T, int pitch, int Wo, int batch, int tid,
                                         int* flags) const {
+    const int c = tid & 31, r0 = (tid >> 5) + 8 * U * batch;
+    float* t = T + c * pitch + (c + Wo - 1 - r0);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int eu = tid + 256 * (u + batch * U), r = eu >> 5, c = eu & 31;
-      const int j = c + Wo - 1 - r;
-      if (eu < total && j >= 0 && j < Wo) {
+      const int r = r0 + 8 * u;
+      if (r >= c && r < c + Wo) {
         const float x = v[u];
         if (!(fabsf(x) <= FLT_MAX)) flags[ROWFLAG ? c : 0] = 1;
-        T[c * pitch + j] = x;
+        t[-8 * u] = x;
       }
     }
   }
