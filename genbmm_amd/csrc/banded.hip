@@ -76,7 +76,7 @@ inline bool prep_fwd(const BandArgs& p, int mode, const float* workspace) {
 }
 
 template <int KIND, bool PREP>
-inline void launch_mm(const BandArgs& p, int B, hipStream_t s) {
+inline void launch_mm(const BandArgs& p, int B, hipStream_t s, int fuse_h = 0) {
   const MmDims d = mm_dims(KIND, p.Wa, p.Wb, p.Wo);
   const int strips = ceil_div(p.n, mm_rows(KIND));
   auto kern = k_band_mm<KIND, PREP>;
@@ -85,7 +85,7 @@ inline void launch_mm(const BandArgs& p, int B, hipStream_t s) {
                               (int)d.bytes);
   const long rows = (long)B * p.n;
   hipLaunchKernelGGL(kern, dim3((unsigned)((long)B * strips)), dim3(256), d.bytes, s, p, strips, d,
-                     rows * p.Wa, rows * p.Wb, rows * p.Wo);
+                     rows * p.Wa, rows * p.Wb, rows * p.Wo, fuse_h);
 }
 
 inline void set_workspace(BandArgs& p, float* ws, int B) {
@@ -208,10 +208,16 @@ int banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int
   if (mode == GENBMM_BAND_LOG && workspace && workspace_used(p) && mm_bwd_ok(p)) {
     set_workspace(p, workspace, B);
     if (scratch) p.ws_h = scratch;
-    const long cells = (long)B * n * p.Wo;
-    hipLaunchKernelGGL(k_band_h, dim3((unsigned)min((cells + 1023) / 1024, (long)0x7fffffff)), dim3(256), 0,
-                       s, g, p.ws_r, p.ws_h, cells);
-    launch_mm<kMmGradA, true>(p, B, s);
+    // H = g / S: formed by the grad_a kernel while it stages it and left in the workspace for
+    // grad_b, if the three arrays start on the same 16-byte phase; else by a pass of its own
+    const auto phase = [](const void* q) { return reinterpret_cast<uintptr_t>(q) & 15; };
+    const int fuse_h = phase(g) == phase(p.ws_r) && phase(g) == phase(p.ws_h);
+    if (!fuse_h) {
+      const long cells = (long)B * n * p.Wo;
+      hipLaunchKernelGGL(k_band_h, dim3((unsigned)min((cells + 1023) / 1024, (long)0x7fffffff)), dim3(256), 0,
+                         s, g, p.ws_r, p.ws_h, cells);
+    }
+    launch_mm<kMmGradA, true>(p, B, s, fuse_h);
     launch_mm<kMmGradB, true>(p, B, s);
     return launch_status();
   }

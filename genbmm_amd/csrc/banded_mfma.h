@@ -160,6 +160,34 @@ struct MmFlat {
     }
     return bad;
   }
+  // v = g, rs.v = R = 1/S of the same cells (read with the same lead): v becomes
+  // H = g * R, NaN where R < 0 (the cell was computed exactly, its 1/S is not usable), and
+  // this strip's cells of it go to `h`, laid out like g - the other gradient reads them
+  // there.  h_vec: h + (abeg - tensor) is 16-byte aligned and every piece lies inside.
+  __device__ __forceinline__ void make_h(const MmFlat& rs, float* __restrict__ h, const float* tensor,
+                                         bool h_vec, int count, int batch, int tid) {
+    float* hb = h + (abeg - tensor);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int vi = tid + 256 * (u + batch * U);
+      if (vi < nvec) {
+        mm_f4 x = v[u];
+        const mm_f4 r = rs.v[u];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) x[t] = r[t] < 0.f ? __builtin_nanf("") : x[t] * r[t];
+        v[u] = x;
+        if (h_vec) {
+          *reinterpret_cast<mm_f4*>(hb + 4 * vi) = x;
+        } else {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const int e = 4 * vi + t - lead;
+            if (e >= 0 && e < count) hb[4 * vi + t] = x[t];
+          }
+        }
+      }
+    }
+  }
   // the rows (first one row_first) that hold a value that is not finite
   __device__ __forceinline__ void flag_rows(int batch, int tid, int count, int row_first, int* flags) const {
 #pragma unroll
@@ -229,7 +257,7 @@ __device__ __forceinline__ float mm_fwd_cell_log_exact(const BandArgs& p, long b
 
 template <int KIND, bool PREP>
 __global__ __launch_bounds__(256, 2) void k_band_mm(const BandArgs p, int strips, const MmDims d, long cells_a,
-                                                    long cells_b, long cells_o) {
+                                                    long cells_b, long cells_o, int fuse_h) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   constexpr bool FWD = KIND == kMmFwd, GA = KIND == kMmGradA, GB = KIND == kMmGradB;
   constexpr int ROWS = FWD ? 64 : 32;   // result rows per workgroup
@@ -263,17 +291,24 @@ __global__ __launch_bounds__(256, 2) void k_band_mm(const BandArgs p, int strips
   const int qr0 = max(q0, 0), qr1 = min(q0 + d.q_rows, n);  // existing rows of Q
   const int pr1 = min(x0 + ROWS, n);
   MmFlat<14> sq;
-  MmFlat<6> sp;
+  MmFlat<6> sp, sr;
   MmSkew<PREP, 20> sk;
+  // grad_a of the prepared log product can form H = g / S itself while it stages it, and
+  // leave it in the workspace for grad_b (fuse_h: g, 1/S and H start on the same 16-byte phase)
+  const bool mk_h = GA && PREP && fuse_h != 0;
+  const float* pt = FWD ? at : (mk_h ? p.g : gt);
   sq.init(qt, qt + cells_q, (bn + qr0) * Wq, (qr1 - qr0) * Wq, Wq, d.qp);
   sq.load(qt, qt + cells_q, 0, tid);
   if (GB) {
     sk.init(Wo);
     sk.load(gt + bn * Wo, Wo, r_lu, n, x0, 0, tid);
   } else {
-    const float* pt = FWD ? at : gt;
     sp.init(pt, pt + (FWD ? cells_a : cells_o), (bn + x0) * Wp, (pr1 - x0) * Wp, Wp, d.pp);
     sp.load(pt, pt + (FWD ? cells_a : cells_o), 0, tid);
+    if (mk_h) {
+      sr.init(p.ws_r, p.ws_r + cells_o, (bn + x0) * Wp, (pr1 - x0) * Wp, Wp, d.pp);
+      sr.load(p.ws_r, p.ws_r + cells_o, 0, tid);
+    }
   }
   // forward of the log product: the row maxima too are requested before anything is waited for
   float alv = 0.f, bev = 0.f;
@@ -297,9 +332,12 @@ __global__ __launch_bounds__(256, 2) void k_band_mm(const BandArgs p, int strips
       sk.store(PL, d.pp, Wo, b, tid, pflags);
     }
   } else {
-    const float* pt = FWD ? at : gt;
     for (int b = 0; b == 0 || sp.more(b); ++b) {
-      if (b > 0) sp.load(pt, pt + (FWD ? cells_a : cells_o), b, tid);
+      if (b > 0) {
+        sp.load(pt, pt + (FWD ? cells_a : cells_o), b, tid);
+        if (mk_h) sr.load(p.ws_r, p.ws_r + cells_o, b, tid);
+      }
+      if (mk_h) sp.make_h(sr, p.ws_h, pt, sp.inside, (pr1 - x0) * Wp, b, tid);
       const bool pbad = sp.store(PL, b, tid);
       if (PREP && GA) {
         if (pbad) sp.flag_rows(b, tid, (pr1 - x0) * Wp, 0, badrow);
