@@ -120,3 +120,31 @@ def test_log_product_with_masked_and_infinite_cells(gpu):
     fin = torch.isfinite(want)
     close(got[fin], want[fin])
     assert torch.equal(got[~fin].nan_to_num(nan=7.0), want[~fin].nan_to_num(nan=7.0))
+
+
+def test_random_bands_against_the_oracle(gpu):
+    """Seeded sweep over band shapes around the kernels' switching points (4, 8, 25
+    diagonals; strips of 32 and 64 rows; tiles of 16): forward and both gradients of the
+    (+,x) and the log product."""
+    rng = np.random.default_rng(20240607)
+    for case in range(36):
+        a_lu, a_ld, b_lu, b_ld = (int(v) for v in rng.integers(0, 19, size=4))
+        if case % 3 == 0:  # keep some operands on the narrow side
+            a_lu, a_ld = a_lu % 4, a_ld % 3
+        n = int(rng.choice([1, 2, 7, 15, 16, 17, 31, 32, 33, 63, 64, 65, 97, 128, 131, 200]))
+        mode = 0 if case % 2 else 3
+        torch.manual_seed(case)
+        a, b = pair(n, a_lu, a_ld, b_lu, b_ld)
+        W = a.shape[2] + b.shape[2] - 1
+        g = torch.randn(2, n, W)
+        X = BandedMatrix(a.to(gpu).requires_grad_(True), a_lu, a_ld)
+        Y = BandedMatrix(b.to(gpu).requires_grad_(True), b_lu, b_ld)
+        res = (X.multiply_log if mode == 0 else X.multiply)(Y)
+        want, _, _ = oracle.seq_band_fwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, mode, dtype=np.float64)
+        tag = (case, n, a_lu, a_ld, b_lu, b_ld, mode)
+        assert torch.allclose(res.data.detach().cpu().double(), want, rtol=1e-5, atol=1e-5), tag
+        ga, gb = torch.autograd.grad(res.data, (X.data, Y.data), g.to(gpu))
+        wa, wb = oracle.seq_band_bwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, g.double(), mode,
+                                     dtype=np.float64)
+        assert torch.allclose(ga.cpu().double(), wa, rtol=1e-5, atol=1e-5), tag
+        assert torch.allclose(gb.cpu().double(), wb, rtol=1e-5, atol=1e-5), tag
