@@ -210,6 +210,11 @@ __device__ __forceinline__ float band_fwd_cell_log_exact(const BandArgs& p, long
   band_fwd_cell<GENBMM_BAND_LOG>(p, bi, i, j);
   return p.o0[bi * p.Wo + j];
 }
+// Out of line for the wide-band variants of the strip kernels, which have no registers to
+// spare for it (the narrow ones take it inline: a call costs every lane a stack frame).
+__device__ __attribute__((noinline)) float band_fwd_cell_log_exact_call(const BandArgs& p, long bi, int i, int j) {
+  return band_fwd_cell_log_exact(p, bi, i, j);
+}
 
 template <int SEM, int NQ>
 __global__ __launch_bounds__(256, (SEM == kSemMul || SEM == kSemLogPrep) ? 3 : 2) void k_band_fwd_strip(const BandArgs p, int strips,
@@ -327,7 +332,7 @@ __global__ __launch_bounds__(256, (SEM == kSemMul || SEM == kSemLogPrep) ? 3 : 2
             rv = __builtin_amdgcn_rcpf(v);
             v = __builtin_fmaf(fast_log2(v), kLn2, sh[t]);
           } else {  // factoring not exact for this cell: recompute it from memory
-            v = band_fwd_cell_log_exact(p, bn + i, i, j);
+            v = NQ == 1 ? band_fwd_cell_log_exact(p, bn + i, i, j) : band_fwd_cell_log_exact_call(p, bn + i, i, j);
             rv = -1.f;  // tells the backward that 1/S is not usable here
           }
         } else {
