@@ -63,7 +63,7 @@ __device__ __forceinline__ float item_exp(float x, float shift) {
 // FULL: M = K = N = G * TB, known to the compiler - the index arithmetic that is most of
 // the general kernel's instructions (it is issue-bound, not memory-bound) folds away.
 template <int G, int TB, bool FULL = false>
-__global__ __launch_bounds__(G * G) void k_log_item_fwd(const float* __restrict__ a,
+__global__ __launch_bounds__(G * G, TB == 2 ? 8 : 1) void k_log_item_fwd(const float* __restrict__ a,
                                                       const float* __restrict__ b,
                                                       float* __restrict__ out,
                                                       float* __restrict__ stats, int M_, int K_,
