@@ -148,3 +148,38 @@ def test_random_bands_against_the_oracle(gpu):
                                      dtype=np.float64)
         assert torch.allclose(ga.cpu().double(), wa, rtol=1e-5, atol=1e-5), tag
         assert torch.allclose(gb.cpu().double(), wb, rtol=1e-5, atol=1e-5), tag
+
+
+def test_random_bands_max_product_bit_exact(gpu):
+    """The whole-strip max-plus forward against the oracle, values on a grid of 1/8 so that
+    ties occur: values, arg-max indices (through the C ABI) and gradients must be equal."""
+    from genbmm_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(77)
+    for case in range(24):
+        a_lu, a_ld, b_lu, b_ld = (int(v) for v in rng.integers(0, 21, size=4))
+        if case % 4 == 0:
+            b_lu, b_ld = b_lu % 5, b_ld % 4
+        n = int(rng.choice([3, 16, 33, 63, 64, 65, 100, 128, 150, 257]))
+        torch.manual_seed(100 + case)
+        grid = lambda *s: torch.round(torch.randn(*s) * 8) / 8
+        a = banddiag(grid(2, n, n), a_lu, a_ld)[0].contiguous()
+        b = banddiag(grid(2, n, n), b_lu, b_ld)[0].contiguous()
+        W = a.shape[2] + b.shape[2] - 1
+        ad, bd = a.to(gpu), b.to(gpu)
+        out = torch.empty(2, n, W, device=gpu)
+        idx = torch.empty(2, n, W, dtype=torch.int32, device=gpu)
+        rc = lib.genbmm_banded_fwd(_lib.ptr(ad), a_lu, a_ld, _lib.ptr(bd), b_lu, b_ld, _lib.ptr(out), _lib.ptr(idx),
+                                   _lib.ptr(None), 2, n, 1, _lib.stream_of(ad))
+        assert rc == 0
+        want, widx, _ = oracle.seq_band_fwd(a, a_lu, a_ld, b, b_lu, b_ld, 1)
+        tag = (case, n, a_lu, a_ld, b_lu, b_ld)
+        assert torch.equal(out.cpu(), want), tag
+        assert torch.equal(idx.cpu(), widx), tag
+        g = grid(2, n, W).clamp(-4, 4)
+        X = BandedMatrix(ad.clone().requires_grad_(True), a_lu, a_ld)
+        Y = BandedMatrix(bd.clone().requires_grad_(True), b_lu, b_ld)
+        res = X.multiply_max(Y)
+        ga, gb = torch.autograd.grad(res.data, (X.data, Y.data), g.to(gpu))
+        wa, wb = oracle.seq_band_bwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, g.double(), 1, dtype=np.float64)
+        assert torch.equal(ga.cpu().double(), wa) and torch.equal(gb.cpu().double(), wb), tag
