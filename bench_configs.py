@@ -284,7 +284,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--cpu", action="store_true")
-    ap.add_argument("--only", default="", help="comma-separated subset: log,max,sample,banded,struct,f64")
+    ap.add_argument("--only", default="", help="comma-separated subset: log,max,sample,banded,struct,f64; "
+                    "widths (not in the default set): the banded products at 5 ... 81 diagonals per operand")
     args = ap.parse_args()
     want = set(args.only.split(",")) if args.only else {"log", "max", "sample", "banded", "struct", "f64"}
     lib = _lib.load()
@@ -304,6 +305,10 @@ def main():
     if "banded" in want:
         for mode in (3, 0, 1):
             banded(lib, dev, 64, 4096, 32, 32, mode, r)
+    if "widths" in want:
+        for lu in (2, 4, 8, 16, 24, 32, 40):
+            for mode in (3, 0, 1):
+                banded(lib, dev, 64, 4096, lu, lu, mode, r)
     if "struct" in want:
         band_structure(lib, dev, 64, 4096, 32, 32, r)
     if "f64" in want:
