@@ -65,13 +65,12 @@ def dense_log(lib, dev, B, M, K, N, reps, name, dist="randn", path=0, graph=Fals
     out, ga, gb = torch.empty(B, M, N, device=dev), torch.empty_like(a), torch.empty_like(b)
     stats = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=dev)
     s, p = _lib.stream_of(a), _lib.ptr
-    lib.genbmm_logbmm_force_exact(path)
 
     def f():
-        _lib.check(lib.genbmm_logbmm_fwd(p(a), p(b), p(out), p(stats), B, M, K, N, s), "fwd")
+        _lib.check(lib.genbmm_logbmm_fwd_path(p(a), p(b), p(out), p(stats), B, M, K, N, path, s), "fwd")
 
     def bw():
-        _lib.check(lib.genbmm_logbmm_bwd(p(a), p(b), p(out), p(g), p(stats), p(ga), p(gb), B, M, K, N, s), "bwd")
+        _lib.check(lib.genbmm_logbmm_bwd_path(p(a), p(b), p(out), p(g), p(stats), p(ga), p(gb), B, M, K, N, path, s), "bwd")
 
     def step():
         f()
@@ -87,7 +86,6 @@ def dense_log(lib, dev, B, M, K, N, reps, name, dist="randn", path=0, graph=Fals
             step()
         s = _lib.stream_of(a)
         extra_graph = {"ms_graph_replay": round(timed(gr.replay, reps), 4)}
-    lib.genbmm_logbmm_force_exact(0)
     bmkn = float(B) * M * K * N
     nbytes = 4.0 * B * (3 * M * K + 3 * K * N + 3 * M * N)
     report(name, ms, 6 * bmkn, nbytes, {"path": {0: "factored", 1: "online-exact", 2: "factored-valu"}[path],

@@ -31,6 +31,8 @@ _BAND = [_c_float_p, _i, _i, _c_float_p, _i, _i]  # a, a_lu, a_ld, b, b_lu, b_ld
 SIGNATURES = {
     "genbmm_logbmm_fwd": [_c_float_p] * 4 + _DENSE_DIMS,
     "genbmm_logbmm_bwd": [_c_float_p] * 7 + _DENSE_DIMS,
+    "genbmm_logbmm_fwd_path": [_c_float_p] * 4 + [_i, _i, _i, _i, _i, _vp],  # ..., B, M, K, N, path, stream
+    "genbmm_logbmm_bwd_path": [_c_float_p] * 7 + [_i, _i, _i, _i, _i, _vp],
     "genbmm_logbmm_bwdbwd": [_c_float_p] * 9 + _DENSE_DIMS,
     "genbmm_maxbmm_fwd": [_c_float_p] * 3 + [_c_int_p] + _DENSE_DIMS,
     "genbmm_prodmaxbmm_fwd": [_c_float_p] * 3 + [_c_int_p, _c_float_p] + _DENSE_DIMS,
@@ -59,7 +61,6 @@ SIGNATURES = {
     "genbmm_band_from_dense": [_c_float_p, _c_float_p, _i, _i, _i, _i, _i, _vp],
 }
 STRING_FUNCS = {"genbmm_version": [], "genbmm_error_string": [_i]}
-VOID_FUNCS = {"genbmm_logbmm_force_exact": [_i]}
 SIZE_FUNCS = {"genbmm_logbmm_stats_size": [_i, _i, _i, _i],
               "genbmm_banded_workspace_size": [_i, _i, _i, _i, _i, _i]}
 
@@ -87,10 +88,6 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = argtypes
         fn.restype = ctypes.c_char_p
-    for name, argtypes in VOID_FUNCS.items():
-        fn = getattr(lib, name)
-        fn.argtypes = argtypes
-        fn.restype = None
     for name, argtypes in SIZE_FUNCS.items():
         fn = getattr(lib, name)
         fn.argtypes = argtypes

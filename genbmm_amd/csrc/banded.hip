@@ -355,7 +355,7 @@ const char* genbmm_error_string(int code) {
     case GENBMM_OK: return "ok";
     case GENBMM_E_NULLPTR: return "a required pointer argument is NULL";
     case GENBMM_E_SHAPE: return "a dimension is negative or too large";
-    case GENBMM_E_MODE: return "unknown semiring mode";
+    case GENBMM_E_MODE: return "unknown semiring mode or kernel path";
     case GENBMM_E_BAND: return "negative band width";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
   }

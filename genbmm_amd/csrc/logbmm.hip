@@ -28,7 +28,6 @@
 // (any shape, this file) and the fp32 matrix-core instruction for problems made
 // of full 128x128 tiles (logbmm_mfma.h).
 #include <algorithm>
-#include <atomic>
 
 #include "dense_tiles.h"
 #include "log_bwd_tile.h"
@@ -168,7 +167,8 @@ __global__ __launch_bounds__(C::NT) void k_log_bwd_exact(const LogBwdArgs p) {
 template <class C>
 __global__ __launch_bounds__(C::NT, 2) void k_log_fwd_fast(const DenseArgs p,
                                                            const float* __restrict__ stats,
-                                                           int* __restrict__ flags) {
+                                                           int* __restrict__ flags,
+                                                           int* __restrict__ hdr) {
   __shared__ __attribute__((aligned(16))) float smem[C::KT * (C::LDA + C::LDB) + C::BM + C::BN];
   float* As = smem;
   float* Bs = As + C::KT * C::LDA;
@@ -178,6 +178,11 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_fwd_fast(const DenseArgs p,
   int batch, m0, n0;
   decode_tile<C>(p, batch, m0, n0);
   const int M = p.M, K = p.K, N = p.N;
+  if (blockIdx.x == 0 && tid == 0) {  // whose flags these are, and their tile shape
+    hdr[1] = C::BM;
+    hdr[2] = C::BN;
+    hdr[0] = kWsFast;
+  }
   const float* ab = p.a + (long)batch * M * K;
   const float* bb = p.b + (long)batch * K * N;
   const float* st = stats + (long)batch * (M + N);
@@ -307,18 +312,25 @@ __global__ __launch_bounds__(CX::NT) void k_sample_fixup(const DenseArgs p,
   }
 }
 
+// Backward fix-up: recompute, with the exact routine, the tiles of a factored backward
+// launch that left their work undone.  Whether a tile did is a function of what the
+// forward left in the workspace (bwd_tile_flagged), evaluated here exactly as in the
+// launch itself; the workspace is only read.
 template <class CX, int FBR, int FBC, bool GRAD_A>
 __global__ __launch_bounds__(CX::NT) void k_log_bwd_fixup(const LogBwdArgs p,
-                                                          const int* __restrict__ flags,
-                                                          int total_tiles) {
+                                                          const int* __restrict__ hdr,
+                                                          const int* __restrict__ fwd_flags,
+                                                          int need_factors, int total_tiles) {
   static_assert(FBR % CX::BR == 0 && FBC % CX::BC == 0, "");
   __shared__ __attribute__((aligned(16))) float smem[LogBwdLds<CX, GRAD_A>::FLOATS];
   const int per = p.tiles_r * p.tiles_c;  // of the factored launch
   const int R = GRAD_A ? p.M : p.K, Cc = GRAD_A ? p.K : p.N;
   for (int t = blockIdx.x; t < total_tiles; t += gridDim.x) {
-    if (!flags[t]) continue;
     const int batch = t / per, r = t - batch * per;
     const int r0 = (r / p.tiles_c) * FBR, c0 = (r % p.tiles_c) * FBC;
+    if (!bwd_tile_flagged(hdr, fwd_flags, need_factors, GRAD_A, GRAD_A ? r0 : c0, GRAD_A ? FBR : FBC,
+                          batch, p.M, p.N, threadIdx.x, CX::NT))
+      continue;
     for (int h = 0; h < FBR / CX::BR; ++h)
       for (int w = 0; w < FBC / CX::BC; ++w)
         if (r0 + h * CX::BR < R && c0 + w * CX::BC < Cc) {
@@ -328,26 +340,28 @@ __global__ __launch_bounds__(CX::NT) void k_log_bwd_fixup(const LogBwdArgs p,
   }
 }
 
-// Fix-up of both gradients' flagged tiles in one launch (workgroups stride over
-// the grad_a list, then over the grad_b list).
+// Fix-up of both gradients' tiles in one launch (workgroups stride over the grad_a
+// list, then over the grad_b list).
 template <class CX, int AR, int AC, int BR, int BC>
 __global__ __launch_bounds__(CX::NT) void k_log_bwd_fixup_both(const LogBwdArgs pa,
                                                                const LogBwdArgs pb,
-                                                               const int* __restrict__ flags_a,
-                                                               const int* __restrict__ flags_b,
+                                                               const int* __restrict__ hdr,
+                                                               const int* __restrict__ fwd_flags,
                                                                int tiles_a, int tiles_b) {
   constexpr int kFa = LogBwdLds<CX, true>::FLOATS, kFb = LogBwdLds<CX, false>::FLOATS;
   __shared__ __attribute__((aligned(16))) float smem[kFa > kFb ? kFa : kFb];
   for (int t = blockIdx.x; t < tiles_a + tiles_b; t += gridDim.x) {
     const bool is_a = t < tiles_a;
     const int u = is_a ? t : t - tiles_a;
-    if (!(is_a ? flags_a[u] : flags_b[u])) continue;
     const LogBwdArgs& p = is_a ? pa : pb;
     const int per = p.tiles_r * p.tiles_c;
     const int batch = u / per, r = u - batch * per;
     const int FR = is_a ? AR : BR, FC = is_a ? AC : BC;
     const int R = is_a ? p.M : p.K, Cc = is_a ? p.K : p.N;
     const int r0 = (r / p.tiles_c) * FR, c0 = (r % p.tiles_c) * FC;
+    if (!bwd_tile_flagged(hdr, fwd_flags, true, is_a, is_a ? r0 : c0, is_a ? FR : FC, batch, p.M, p.N,
+                          threadIdx.x, CX::NT))
+      continue;
     for (int h = 0; h < FR / CX::BR; ++h)
       for (int w = 0; w < FC / CX::BC; ++w)
         if (r0 + h * CX::BR < R && c0 + w * CX::BC < Cc) {
@@ -366,7 +380,8 @@ __global__ __launch_bounds__(CX::NT) void k_log_bwd_fixup_both(const LogBwdArgs 
 template <class C, bool GRAD_A>
 __global__ __launch_bounds__(C::NT, 2) void k_log_bwd_fast(const LogBwdArgs p,
                                                            const float* __restrict__ stats,
-                                                           int* __restrict__ flags) {
+                                                           const int* __restrict__ hdr,
+                                                           const int* __restrict__ fwd_flags) {
   constexpr int BY = GRAD_A ? C::BC : C::BR;
   constexpr int BO = GRAD_A ? C::BR : C::BC;
   using TYt = std::conditional_t<GRAD_A, TileOutMajor<BY, C::RT, C::NT>, TileRedMajor<BY, C::RT, C::NT>>;
@@ -383,6 +398,12 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_bwd_fast(const LogBwdArgs p,
   const int batch = blockIdx.x / per;
   const int rem = blockIdx.x - batch * per;
   const int r0 = (rem / p.tiles_c) * C::BR, c0 = (rem % p.tiles_c) * C::BC;
+  // Every cell this tile reduces over must come from a forward tile that passed the
+  // factoring guard (S >= 2^-40, finite shifts): H = g * exp(alpha + beta - out) is then
+  // at most |g| * 2^40.  Otherwise the fix-up launch recomputes this tile.
+  if (bwd_tile_flagged(hdr, fwd_flags, false, GRAD_A, GRAD_A ? r0 : c0, GRAD_A ? C::BR : C::BC, batch, M,
+                       N, tid, C::NT))
+    return;
 
   const float* ab = p.a + (long)batch * M * K;
   const float* bb = p.b + (long)batch * K * N;
@@ -398,7 +419,6 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_bwd_fast(const LogBwdArgs p,
   const bool vec_o = p.vec_n;
   const int y0 = GRAD_A ? c0 : r0;
   const int o0 = GRAD_A ? r0 : c0, olim = GRAD_A ? M : N;
-  const float lim = kGuardBits * kLn2 + 1e-3f;  // alpha+beta-out above this: S < 2^-40
 
   auto col_of = [&](int j) { return (j >> 2) * (C::TX * 4) + tx * 4 + (j & 3); };
   auto safe = [](const float* v, int i, int n) { return i < n ? v[i] : 0.f; };
@@ -432,7 +452,6 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_bwd_fast(const LogBwdArgs p,
     tol.gload(ob, N, o0, q0, olim, Q, vec_o, tid);
     tgl.gload(gb, N, o0, q0, olim, Q, vec_o, tid);
   };
-  int bad = 0;
   if (Q > 0) load(0);
   for (int q0 = 0; q0 < Q; q0 += C::RT) {
     __syncthreads();
@@ -448,15 +467,8 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_bwd_fast(const LogBwdArgs p,
         }
 #pragma unroll
         for (int l = 0; l < TOt::PER; ++l) {
-          const int m = o0 + (tid + l * C::NT) / TOt::C4;
           const float ex = fix_s[l] + bq.x - tol.r[l].x, ey = fix_s[l] + bq.y - tol.r[l].y;
           const float ez = fix_s[l] + bq.z - tol.r[l].z, ew = fix_s[l] + bq.w - tol.r[l].w;
-          if (m < M) {
-            if (n < N && !(ex <= lim)) bad = 1;
-            if (n + 1 < N && !(ey <= lim)) bad = 1;
-            if (n + 2 < N && !(ez <= lim)) bad = 1;
-            if (n + 3 < N && !(ew <= lim)) bad = 1;
-          }
           tol.r[l].x = tgl.r[l].x * exp_stage(ex); tol.r[l].y = tgl.r[l].y * exp_stage(ey);
           tol.r[l].z = tgl.r[l].z * exp_stage(ez); tol.r[l].w = tgl.r[l].w * exp_stage(ew);
         }
@@ -471,17 +483,9 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_bwd_fast(const LogBwdArgs p,
       }
 #pragma unroll
       for (int l = 0; l < TOt::PER; ++l) {
-        const int idx = tid + l * C::NT;
-        const int m = q0 + idx / TOt::C4, n = o0 + (idx % TOt::C4) * 4;
-        const float s = safe(al, m, M);
+        const float s = safe(al, q0 + (tid + l * C::NT) / TOt::C4, M);
         const float ex = s + fix_v[l].x - tol.r[l].x, ey = s + fix_v[l].y - tol.r[l].y;
         const float ez = s + fix_v[l].z - tol.r[l].z, ew = s + fix_v[l].w - tol.r[l].w;
-        if (m < M) {
-          if (n < N && !(ex <= lim)) bad = 1;
-          if (n + 1 < N && !(ey <= lim)) bad = 1;
-          if (n + 2 < N && !(ez <= lim)) bad = 1;
-          if (n + 3 < N && !(ew <= lim)) bad = 1;
-        }
         tol.r[l].x = tgl.r[l].x * exp_stage(ex); tol.r[l].y = tgl.r[l].y * exp_stage(ey);
         tol.r[l].z = tgl.r[l].z * exp_stage(ez); tol.r[l].w = tgl.r[l].w * exp_stage(ew);
       }
@@ -517,10 +521,6 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_bwd_fast(const LogBwdArgs p,
       for (int qq = 0; qq < qn; ++qq) step(qq);
     }
   }
-
-  bad = __syncthreads_or(bad);
-  if (tid == 0) flags[blockIdx.x] = bad;
-  if (bad) return;  // the fix-up launch recomputes this tile
 
   // epilogue: grad = exp(x - shift) * acc, x re-read from global memory
   float* gradb = p.grad + (long)batch * R * Cc;
@@ -562,24 +562,28 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_bwd_fast(const LogBwdArgs p,
 }
 
 // ----------------------------------------------------------------- dispatch
-std::atomic<int> g_path{0};  // 0 default, 1 exact only, 2 factored without matrix cores
+// `path` (GENBMM_PATH_*): which family of kernels a call may use.  AUTO: whole-item
+// kernels for small matrices, the matrix cores where the shape allows, the factored
+// vector-ALU kernels otherwise.  EXACT: the online / exp-per-term kernels only (what a
+// NULL workspace gives).  VALU: the factored kernels on v_fma_f32, never the matrix cores
+// nor the whole-item kernels.
 constexpr int kFixupGrid = 1024;
 
-// Layout of the caller's stats buffer: B*(M+N) shifts; one int flag per 32x32
-// tile of (M,N), of (M,K) and of (K,N) (an upper bound on any launch's tile
-// count); a header of four ints; and, for shapes the matrix-core forward can
-// take, its by-products EA (B*M*K), EB (B*K*N) and R (B*M*N) on a 16-byte
-// boundary.
-inline int64_t tiles32(int B, int X, int Y) { return (int64_t)B * ceil_div(X, 32) * ceil_div(Y, 32); }
-inline int* flags_of(const float* stats, int B, int M, int K, int N, int which) {
-  int* f = reinterpret_cast<int*>(const_cast<float*>(stats) + (int64_t)B * (M + N));
-  if (which >= 1) f += tiles32(B, M, N);
-  if (which >= 2) f += tiles32(B, M, K);
-  if (which >= 3) f += tiles32(B, K, N);
-  return f;
+inline bool valid_path(int path) {
+  return path == GENBMM_PATH_AUTO || path == GENBMM_PATH_EXACT || path == GENBMM_PATH_VALU;
 }
-inline int64_t header_offset(int B, int M, int K, int N) {
-  const int64_t o = (int64_t)B * (M + N) + tiles32(B, M, N) + tiles32(B, M, K) + tiles32(B, K, N);
+
+// Layout of the caller's stats buffer: B*(M+N) shifts; one int flag per 32x32
+// tile of (M,N) (an upper bound on any forward launch's tile count); a header of
+// four ints (which forward filled the buffer, and its tile shape); and, for shapes
+// the matrix-core forward can take, its by-products EA (B*M*K), EB (B*K*N) and
+// R (B*M*N) on a 16-byte boundary.  Only the forward writes to it.
+inline int64_t tiles32(int B, int X, int Y) { return (int64_t)B * ceil_div(X, 32) * ceil_div(Y, 32); }
+inline int* fwd_flags_of(const float* stats, int B, int M, int N) {
+  return reinterpret_cast<int*>(const_cast<float*>(stats) + (int64_t)B * (M + N));
+}
+inline int64_t header_offset(int B, int M, int N) {
+  const int64_t o = (int64_t)B * (M + N) + tiles32(B, M, N);
   return (o + 3) & ~(int64_t)3;
 }
 // Small matrices: a whole batch item per workgroup (logbmm_item.h).
@@ -603,7 +607,7 @@ inline bool fwd_mfma_shape(int B, int M, int K, int N) {
   return t128 <= 0x7fffffff;
 }
 inline LogPrepared prepared_of(const float* stats, int B, int M, int K, int N) {
-  float* base = const_cast<float*>(stats) + header_offset(B, M, K, N);
+  float* base = const_cast<float*>(stats) + header_offset(B, M, N);
   LogPrepared w;
   w.hdr = reinterpret_cast<int*>(base);
   w.ea = base + 4;
@@ -628,11 +632,12 @@ int launch_fwd_fixup(const DenseArgs& p, const int* flags, int tiles, hipStream_
 }
 
 template <class C, class CX>
-int launch_fwd_fast(DenseArgs p, const float* stats, int* flags, int B, int M, int K, int N,
-                    hipStream_t s) {
+int launch_fwd_fast(DenseArgs p, float* stats, int B, int M, int K, int N, hipStream_t s) {
   dim3 grid;
   if (int e = fill_args<C>(p, B, M, K, N, grid)) return e;
-  hipLaunchKernelGGL((k_log_fwd_fast<C>), grid, dim3(C::NT), 0, s, p, stats, flags);
+  int* flags = fwd_flags_of(stats, B, M, N);
+  hipLaunchKernelGGL((k_log_fwd_fast<C>), grid, dim3(C::NT), 0, s, p, stats, flags,
+                     prepared_of(stats, B, M, K, N).hdr);
   if (int e = launch_status()) return e;
   return launch_fwd_fixup<CX, C::BM, C::BN>(p, flags, (int)grid.x, s);
 }
@@ -640,14 +645,14 @@ int launch_fwd_fast(DenseArgs p, const float* stats, int* flags, int B, int M, i
 // Matrix-core launches: T is the MTile; the ragged variant of a kernel is used only
 // when some extent is not a multiple of its tile / slab.
 template <class T>
-int launch_fwd_mfma(DenseArgs p, const float* stats, int* flags, int B, int M, int K, int N,
-                    hipStream_t s) {
+int launch_fwd_mfma(DenseArgs p, float* stats, int B, int M, int K, int N, hipStream_t s) {
   p.M = M; p.K = K; p.N = N;
   p.tiles_m = ceil_div(M, T::TR);
   p.tiles_n = ceil_div(N, T::TC);
   p.vec_a = p.vec_b = p.vec_o = 1;
   const int total = B * p.tiles_m * p.tiles_n;
   const LogPrepared ws = prepared_of(stats, B, M, K, N);
+  int* flags = fwd_flags_of(stats, B, M, N);
   auto go = [&](auto kern) {
     hipLaunchKernelGGL(kern, dim3(total), dim3(T::NT), 0, s, p.a, p.b, p.out, stats, flags, ws.ea,
                        ws.eb, ws.r, ws.hdr, M, K, N, p.tiles_m, p.tiles_n);
@@ -708,38 +713,40 @@ int launch_bwd_exact(LogBwdArgs p, int B, hipStream_t s) {
 }
 
 template <class C, class CX, bool GRAD_A>
-int launch_bwd_fast(LogBwdArgs p, const float* stats, int* flags, int B, hipStream_t s) {
+int launch_bwd_fast(LogBwdArgs p, const float* stats, int B, hipStream_t s) {
   const int R = GRAD_A ? p.M : p.K, Cc = GRAD_A ? p.K : p.N;
   p.tiles_r = ceil_div(R, C::BR);
   p.tiles_c = ceil_div(Cc, C::BC);
   const int64_t total = (int64_t)B * p.tiles_r * p.tiles_c;
   if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
+  const int* hdr = prepared_of(stats, B, p.M, p.K, p.N).hdr;
+  const int* ff = fwd_flags_of(stats, B, p.M, p.N);
   hipLaunchKernelGGL((k_log_bwd_fast<C, GRAD_A>), dim3((unsigned)total), dim3(C::NT), 0, s, p,
-                     stats, flags);
+                     stats, hdr, ff);
   if (int e = launch_status()) return e;
   hipLaunchKernelGGL((k_log_bwd_fixup<CX, C::BR, C::BC, GRAD_A>),
-                     dim3(min((int)total, kFixupGrid)), dim3(CX::NT), 0, s, p, flags, (int)total);
+                     dim3(min((int)total, kFixupGrid)), dim3(CX::NT), 0, s, p, hdr, ff, 0, (int)total);
   return launch_status();
 }
 
 template <class T, bool GRAD_A>
-int launch_bwd_mfma(LogBwdArgs p, const float* stats, int* flags, int B, hipStream_t s) {
+int launch_bwd_mfma(LogBwdArgs p, const float* stats, int B, hipStream_t s) {
   const int R = GRAD_A ? p.M : p.K, Cc = GRAD_A ? p.K : p.N;
   const int Q = GRAD_A ? p.N : p.M;
   p.tiles_r = ceil_div(R, T::TR);
   p.tiles_c = ceil_div(Cc, T::TC);
   const int total = B * p.tiles_r * p.tiles_c;
   const LogPrepared ws = prepared_of(stats, B, p.M, p.K, p.N);
+  const int* ff = fwd_flags_of(stats, B, p.M, p.N);
   auto go = [&](auto kern) {
-    hipLaunchKernelGGL(kern, dim3(total), dim3(T::NT), 0, s, p.g, ws.ea, ws.eb, ws.r, ws.hdr,
-                       flags_of(stats, B, p.M, p.K, p.N, 0), p.grad, flags, p.M, p.K, p.N,
-                       p.tiles_r, p.tiles_c);
+    hipLaunchKernelGGL(kern, dim3(total), dim3(T::NT), 0, s, p.g, ws.ea, ws.eb, ws.r, ws.hdr, ff,
+                       p.grad, p.M, p.K, p.N, p.tiles_r, p.tiles_c);
   };
   if (R % T::TR != 0 || Cc % T::TC != 0 || Q % kMS != 0) go(k_log_bwd_mfma<T, GRAD_A, true>);
   else go(k_log_bwd_mfma<T, GRAD_A, false>);
   if (int e = launch_status()) return e;
   hipLaunchKernelGGL((k_log_bwd_fixup<BCfgWide, T::TR, T::TC, GRAD_A>),
-                     dim3(min(total, kFixupGrid)), dim3(BCfgWide::NT), 0, s, p, flags, total);
+                     dim3(min(total, kFixupGrid)), dim3(BCfgWide::NT), 0, s, p, ws.hdr, ff, 1, total);
   return launch_status();
 }
 
@@ -752,12 +759,11 @@ int launch_bwd_mfma_both(LogBwdArgs pa, LogBwdArgs pb, const float* stats, int B
   const int64_t ta = (int64_t)B * pa.tiles_r * pa.tiles_c, tb = (int64_t)B * pb.tiles_r * pb.tiles_c;
   if (ta + tb > 0x7fffffffLL) return GENBMM_E_SHAPE;
   const LogPrepared ws = prepared_of(stats, B, M, K, N);
-  int* fa = flags_of(stats, B, M, K, N, 1);
-  int* fb = flags_of(stats, B, M, K, N, 2);
+  const int* ff = fwd_flags_of(stats, B, M, N);
   auto go = [&](auto kern) {
     hipLaunchKernelGGL(kern, dim3((unsigned)(ta + tb)), dim3(TA::NT), 0, s, pa.g, ws.ea, ws.eb, ws.r,
-                       ws.hdr, flags_of(stats, B, M, K, N, 0), pa.grad, pb.grad, fa, fb, M, K, N,
-                       (int)ta, pa.tiles_r, pa.tiles_c, pb.tiles_r, pb.tiles_c);
+                       ws.hdr, ff, pa.grad, pb.grad, M, K, N, (int)ta, pa.tiles_r, pa.tiles_c,
+                       pb.tiles_r, pb.tiles_c);
   };
   const bool ragged = M % TA::TR != 0 || K % TA::TC != 0 || N % kMS != 0 || K % TB::TR != 0 ||
                       N % TB::TC != 0 || M % kMS != 0;
@@ -766,17 +772,17 @@ int launch_bwd_mfma_both(LogBwdArgs pa, LogBwdArgs pb, const float* stats, int B
   if (int e = launch_status()) return e;
   hipLaunchKernelGGL((k_log_bwd_fixup_both<BCfgWide, TA::TR, TA::TC, TB::TR, TB::TC>),
                      dim3((unsigned)std::min<int64_t>(ta + tb, kFixupGrid)), dim3(BCfgWide::NT), 0,
-                     s, pa, pb, fa, fb, (int)ta, (int)tb);
+                     s, pa, pb, ws.hdr, ff, (int)ta, (int)tb);
   return launch_status();
 }
 
 // Which matrix-core tiling an output of out_r x out_c (reduction over red) gets:
 // 2 for the 256-wide tile (when the long side splits into 256s without extra
 // padding and there are tiles enough to give every compute unit two workgroups of
-// eight waves), 1 for 128x128, 0 for none (extents too small or not multiples of 4).  `long_cols`: the 256 side is the
-// column side of the output.
-inline int mfma_kind(int B, int out_r, int out_c, int red, bool aligned, bool long_cols) {
-  if (g_path.load() != 0 || !aligned || !mfma_extents(out_r, out_c, red)) return 0;
+// eight waves), 1 for 128x128, 0 for none (path, or extents too small).  `long_cols`:
+// the 256 side is the column side of the output.
+inline int mfma_kind(int path, int B, int out_r, int out_c, int red, bool long_cols) {
+  if (path != GENBMM_PATH_AUTO || !mfma_extents(out_r, out_c, red)) return 0;
   const int64_t t128 = tiles128(B, out_r, out_c);
   if (t128 > 0x7fffffff) return 0;
   const int L = long_cols ? out_c : out_r;
@@ -789,41 +795,131 @@ using MTWide = MTile<128, 256>;  // grad_a (m x k)
 using MTTall = MTile<256, 128>;  // forward (m x n; measured 1-2 % ahead of 128x256) and grad_b (k x n)
 
 template <bool GRAD_A>
-int run_bwd(const LogBwdArgs& p, const float* stats, int B, hipStream_t s) {
+int run_bwd(const LogBwdArgs& p, const float* stats, int path, int B, hipStream_t s) {
   const int R = GRAD_A ? p.M : p.K, Cc = GRAD_A ? p.K : p.N, Q = GRAD_A ? p.N : p.M;
   if ((int64_t)B * R * Cc == 0) return GENBMM_OK;
   auto wgs = [&](int br, int bc) { return (int64_t)B * ceil_div(R, br) * ceil_div(Cc, bc); };
   const bool small = R <= 32 && Cc <= 32;
   if (stats) {
-    int* fl = flags_of(stats, B, p.M, p.K, p.N, GRAD_A ? 1 : 2);
-    const bool al = true;  // the matrix-core kernels assume 4-byte alignment only
     // the matrix-core kernels run on what the matrix-core forward left behind
-    switch (fwd_mfma_shape(B, p.M, p.K, p.N) ? mfma_kind(B, R, Cc, Q, al, GRAD_A) : 0) {
+    switch (fwd_mfma_shape(B, p.M, p.K, p.N) ? mfma_kind(path, B, R, Cc, Q, GRAD_A) : 0) {
       case 2:
-        if constexpr (GRAD_A) return launch_bwd_mfma<MTWide, true>(p, stats, fl, B, s);
-        else return launch_bwd_mfma<MTTall, false>(p, stats, fl, B, s);
-      case 1: return launch_bwd_mfma<MT128, GRAD_A>(p, stats, fl, B, s);
+        if constexpr (GRAD_A) return launch_bwd_mfma<MTWide, true>(p, stats, B, s);
+        else return launch_bwd_mfma<MTTall, false>(p, stats, B, s);
+      case 1: return launch_bwd_mfma<MT128, GRAD_A>(p, stats, B, s);
       default: break;
     }
-    if (small) return launch_bwd_fast<BCfgSmall, BCfgSmall, GRAD_A>(p, stats, fl, B, s);
+    if (small) return launch_bwd_fast<BCfgSmall, BCfgSmall, GRAD_A>(p, stats, B, s);
     if (R >= 128 && Cc >= 128 && wgs(128, 128) >= 512)
-      return launch_bwd_fast<BCfgBig, BCfgWide, GRAD_A>(p, stats, fl, B, s);
-    return launch_bwd_fast<BCfgMid, BCfgMid, GRAD_A>(p, stats, fl, B, s);
+      return launch_bwd_fast<BCfgBig, BCfgWide, GRAD_A>(p, stats, B, s);
+    return launch_bwd_fast<BCfgMid, BCfgMid, GRAD_A>(p, stats, B, s);
   }
   if (small) return launch_bwd_exact<BCfgSmall, GRAD_A>(p, B, s);
   if (R >= 64 && Cc >= 128 && wgs(64, 128) >= 512) return launch_bwd_exact<BCfgWide, GRAD_A>(p, B, s);
   return launch_bwd_exact<BCfgMid, GRAD_A>(p, B, s);
 }
 
+template <int G, int TB, bool FULL>
+void launch_item_fwd(const float* a, const float* b, float* out, float* stats, int* hdr, int B, int M,
+                     int K, int N, hipStream_t s) {
+  hipLaunchKernelGGL((k_log_item_fwd<G, TB, FULL>), dim3(B), dim3(G * G), 0, s, a, b, out, stats, hdr, M, K, N);
+}
+
+int run_fwd(const float* a, const float* b, float* out, float* stats, int B, int M, int K, int N,
+            int path, hipStream_t s) {
+  if (int e = check_dense_dims(B, M, K, N)) return e;
+  if (!valid_path(path)) return GENBMM_E_MODE;
+  const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
+  if (missing(a, mk) || missing(b, kn) || missing(out, mn)) return GENBMM_E_NULLPTR;
+  if (stats && B > 0 && item_shape(M, K, N) && path == GENBMM_PATH_AUTO) {  // whole items per workgroup
+    int* hdr = prepared_of(stats, B, M, K, N).hdr;
+    if (M == 32 && K == 32 && N == 32) launch_item_fwd<16, 2, true>(a, b, out, stats, hdr, B, M, K, N, s);
+    else if (M == 64 && K == 64 && N == 64) launch_item_fwd<16, 4, true>(a, b, out, stats, hdr, B, M, K, N, s);
+    else if (max(max(M, K), N) <= 32) launch_item_fwd<16, 2, false>(a, b, out, stats, hdr, B, M, K, N, s);
+    else launch_item_fwd<16, 4, false>(a, b, out, stats, hdr, B, M, K, N, s);
+    return launch_status();
+  }
+  if (stats) {
+    if (int e = launch_stats(a, b, stats, B, M, K, N, s)) return e;
+  }
+  if (mn == 0) return GENBMM_OK;
+  DenseArgs p{};
+  p.a = a; p.b = b; p.out = out; p.idx = nullptr;
+  if (stats && K > 0 && path != GENBMM_PATH_EXACT) {
+    const int64_t big_tiles = (int64_t)B * ceil_div(M, 128) * ceil_div(N, 128);
+    switch (fwd_mfma_shape(B, M, K, N) ? mfma_kind(path, B, M, N, K, false) : 0) {
+      case 2: return launch_fwd_mfma<MTTall>(p, stats, B, M, K, N, s);
+      case 1: return launch_fwd_mfma<MT128>(p, stats, B, M, K, N, s);
+      default: break;
+    }
+    if (M <= 32 && N <= 32) return launch_fwd_fast<CfgSmall, CfgSmall>(p, stats, B, M, K, N, s);
+    if (M >= 128 && N >= 128 && big_tiles >= 512)
+      return launch_fwd_fast<CfgBig, CfgWide>(p, stats, B, M, K, N, s);
+    return launch_fwd_fast<CfgMid, CfgMid>(p, stats, B, M, K, N, s);
+  }
+  switch (pick_shape(B, M, N, false)) {
+    case kWide: return launch_fwd_exact<CfgWide>(p, B, M, K, N, s);
+    case kMid: return launch_fwd_exact<CfgMid>(p, B, M, K, N, s);
+    default: return launch_fwd_exact<CfgSmall>(p, B, M, K, N, s);
+  }
+}
+
+int run_bwd_both(const float* a, const float* b, const float* out, const float* g,
+                 const float* stats, float* grad_a, float* grad_b, int B, int M, int K, int N,
+                 int path, hipStream_t s) {
+  if (int e = check_dense_dims(B, M, K, N)) return e;
+  if (!valid_path(path)) return GENBMM_E_MODE;
+  const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
+  if (missing(a, mk) || missing(b, kn) || missing(out, mn) || missing(g, mn) ||
+      (missing(grad_a, mk) && missing(grad_b, kn)))
+    return GENBMM_E_NULLPTR;
+  LogBwdArgs p{};
+  p.a = a; p.b = b; p.out = out; p.g = g;
+  p.M = M; p.K = K; p.N = N;
+  p.vec_k = (K % 4 == 0) && aligned16(a) && aligned16(grad_a);
+  p.vec_n = (N % 4 == 0) && aligned16(b) && aligned16(out) && aligned16(g) && aligned16(grad_b);
+  const float* st = (path == GENBMM_PATH_EXACT || mn == 0) ? nullptr : stats;
+  if (st && B > 0 && item_shape(M, K, N) && path == GENBMM_PATH_AUTO) {
+    if (M == 32 && K == 32 && N == 32)
+      hipLaunchKernelGGL((k_log_item_bwd<16, 2, true>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
+    else if (M == 64 && K == 64 && N == 64)
+      hipLaunchKernelGGL((k_log_item_bwd<16, 4, true>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
+    else if (max(max(M, K), N) <= 32)
+      hipLaunchKernelGGL((k_log_item_bwd<16, 2>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
+    else
+      hipLaunchKernelGGL((k_log_item_bwd<16, 4>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
+    return launch_status();
+  }
+  if (st && grad_a && grad_b && mk > 0 && kn > 0 && fwd_mfma_shape(B, M, K, N)) {
+    const int ka = mfma_kind(path, B, M, K, N, true), kb = mfma_kind(path, B, K, N, M, false);
+    if (ka == kb && ka != 0) {
+      LogBwdArgs pa = p, pb = p;
+      pa.grad = grad_a;
+      pb.grad = grad_b;
+      return ka == 2 ? launch_bwd_mfma_both<MTWide, MTTall>(pa, pb, st, B, s)
+                     : launch_bwd_mfma_both<MT128, MT128>(pa, pb, st, B, s);
+    }
+  }
+  if (grad_a) {
+    p.grad = grad_a;
+    if (int e = run_bwd<true>(p, st, path, B, s)) return e;
+  }
+  if (grad_b) {
+    p.grad = grad_b;
+    if (int e = run_bwd<false>(p, st, path, B, s)) return e;
+  }
+  return GENBMM_OK;
+}
+
 }  // namespace
 
-// The forward's own decision (genbmm_logbmm_fwd below): factors are written by the
+// The forward's own decision (run_fwd above, path AUTO): factors are written by the
 // matrix-core kernels only.
 bool log_fwd_writes_factors(const float* stats, int B, int M, int K, int N, LogFactors* f) {
   if (!stats || K <= 0 || (int64_t)B * M * N == 0) return false;
-  if (B > 0 && item_shape(M, K, N) && g_path.load() == 0) return false;   // whole-item kernels
-  if (g_path.load() == 1 || !fwd_mfma_shape(B, M, K, N)) return false;
-  if (mfma_kind(B, M, N, K, true, false) == 0) return false;
+  if (B > 0 && item_shape(M, K, N)) return false;   // whole-item kernels
+  if (!fwd_mfma_shape(B, M, K, N)) return false;
+  if (mfma_kind(GENBMM_PATH_AUTO, B, M, N, K, false) == 0) return false;
   const LogPrepared ws = prepared_of(stats, B, M, K, N);
   f->ea = ws.ea;
   f->eb = ws.eb;
@@ -840,9 +936,9 @@ int log_sample_sweep_mfma(const float* a, const float* b, float* out, int32_t* i
   DenseArgs p{};
   p.a = a; p.b = b; p.out = out; p.idx = idx; p.seed = seed; p.offset = offset;
   if (ceil_div(K, kMS) > kSampleSlabs) return GENBMM_E_SHAPE;  // the caller checks log_sample_mfma_ok
-  int* fl = flags_of(stats, B, M, K, N, 0);
+  int* fl = fwd_flags_of(stats, B, M, N);
   // the forward's tile shape: its flags are indexed by it
-  switch (mfma_kind(B, M, N, K, true, false)) {
+  switch (mfma_kind(GENBMM_PATH_AUTO, B, M, N, K, false)) {
     case 2: return launch_sample_sweep_mfma<MTTall>(p, stats, fl, B, M, K, N, s);
     case 1: return launch_sample_sweep_mfma<MT128>(p, stats, fl, B, M, K, N, s);
     default: return GENBMM_E_SHAPE;
@@ -856,105 +952,33 @@ extern "C" {
 size_t genbmm_logbmm_stats_size(int B, int M, int K, int N) {
   using namespace genbmm;
   if (check_dense_dims(B, M, K, N)) return 0;
-  int64_t n = header_offset(B, M, K, N) + 4;
+  int64_t n = header_offset(B, M, N) + 4;
   if (fwd_mfma_shape(B, M, K, N)) n += (int64_t)B * ((int64_t)M * K + (int64_t)K * N + (int64_t)M * N);
   return (size_t)n;
 }
 
-void genbmm_logbmm_force_exact(int on) { genbmm::g_path.store(on == 1 || on == 2 ? on : 0); }
-
 int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats, int B, int M,
                       int K, int N, void* stream) {
-  using namespace genbmm;
-  if (int e = check_dense_dims(B, M, K, N)) return e;
-  const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
-  if (missing(a, mk) || missing(b, kn) || missing(out, mn)) return GENBMM_E_NULLPTR;
-  hipStream_t s = (hipStream_t)stream;
-  if (stats && B > 0 && item_shape(M, K, N) && g_path.load() == 0) {  // whole items per workgroup
-    if (M == 32 && K == 32 && N == 32)
-      hipLaunchKernelGGL((k_log_item_fwd<16, 2, true>), dim3(B), dim3(256), 0, s, a, b, out, stats, M, K, N);
-    else if (M == 64 && K == 64 && N == 64)
-      hipLaunchKernelGGL((k_log_item_fwd<16, 4, true>), dim3(B), dim3(256), 0, s, a, b, out, stats, M, K, N);
-    else if (max(max(M, K), N) <= 32)
-      hipLaunchKernelGGL((k_log_item_fwd<16, 2>), dim3(B), dim3(256), 0, s, a, b, out, stats, M, K, N);
-    else
-      hipLaunchKernelGGL((k_log_item_fwd<16, 4>), dim3(B), dim3(256), 0, s, a, b, out, stats, M, K, N);
-    return launch_status();
-  }
-  if (stats) {
-    if (int e = launch_stats(a, b, stats, B, M, K, N, s)) return e;
-  }
-  if (mn == 0) return GENBMM_OK;
-  DenseArgs p{};
-  p.a = a; p.b = b; p.out = out; p.idx = nullptr;
-  if (stats && K > 0 && g_path.load() != 1) {
-    int* fl = flags_of(stats, B, M, K, N, 0);
-    const int64_t big_tiles = (int64_t)B * ceil_div(M, 128) * ceil_div(N, 128);
-    const bool al = true;  // the matrix-core kernels assume 4-byte alignment only
-    switch (fwd_mfma_shape(B, M, K, N) ? mfma_kind(B, M, N, K, al, false) : 0) {
-      case 2: return launch_fwd_mfma<MTTall>(p, stats, fl, B, M, K, N, s);
-      case 1: return launch_fwd_mfma<MT128>(p, stats, fl, B, M, K, N, s);
-      default: break;
-    }
-    if (M <= 32 && N <= 32) return launch_fwd_fast<CfgSmall, CfgSmall>(p, stats, fl, B, M, K, N, s);
-    if (M >= 128 && N >= 128 && big_tiles >= 512)
-      return launch_fwd_fast<CfgBig, CfgWide>(p, stats, fl, B, M, K, N, s);
-    return launch_fwd_fast<CfgMid, CfgMid>(p, stats, fl, B, M, K, N, s);
-  }
-  switch (pick_shape(B, M, N, false)) {
-    case kWide: return launch_fwd_exact<CfgWide>(p, B, M, K, N, s);
-    case kMid: return launch_fwd_exact<CfgMid>(p, B, M, K, N, s);
-    default: return launch_fwd_exact<CfgSmall>(p, B, M, K, N, s);
-  }
+  return genbmm::run_fwd(a, b, out, stats, B, M, K, N, GENBMM_PATH_AUTO, (hipStream_t)stream);
+}
+
+int genbmm_logbmm_fwd_path(const float* a, const float* b, float* out, float* stats, int B, int M,
+                           int K, int N, int path, void* stream) {
+  return genbmm::run_fwd(a, b, out, stats, B, M, K, N, path, (hipStream_t)stream);
 }
 
 int genbmm_logbmm_bwd(const float* a, const float* b, const float* out, const float* g,
                       const float* stats, float* grad_a, float* grad_b, int B, int M, int K,
                       int N, void* stream) {
-  using namespace genbmm;
-  if (int e = check_dense_dims(B, M, K, N)) return e;
-  const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
-  if (missing(a, mk) || missing(b, kn) || missing(out, mn) || missing(g, mn) ||
-      (missing(grad_a, mk) && missing(grad_b, kn)))
-    return GENBMM_E_NULLPTR;
-  LogBwdArgs p{};
-  p.a = a; p.b = b; p.out = out; p.g = g;
-  p.M = M; p.K = K; p.N = N;
-  p.vec_k = (K % 4 == 0) && aligned16(a) && aligned16(grad_a);
-  p.vec_n = (N % 4 == 0) && aligned16(b) && aligned16(out) && aligned16(g) && aligned16(grad_b);
-  hipStream_t s = (hipStream_t)stream;
-  const float* st = (g_path.load() == 1 || mn == 0) ? nullptr : stats;
-  if (st && B > 0 && item_shape(M, K, N) && g_path.load() == 0) {
-    if (M == 32 && K == 32 && N == 32)
-      hipLaunchKernelGGL((k_log_item_bwd<16, 2, true>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
-    else if (M == 64 && K == 64 && N == 64)
-      hipLaunchKernelGGL((k_log_item_bwd<16, 4, true>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
-    else if (max(max(M, K), N) <= 32)
-      hipLaunchKernelGGL((k_log_item_bwd<16, 2>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
-    else
-      hipLaunchKernelGGL((k_log_item_bwd<16, 4>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
-    return launch_status();
-  }
-  if (st && grad_a && grad_b && mk > 0 && kn > 0 && fwd_mfma_shape(B, M, K, N)) {
-    const bool al = true;
-    const int ka = mfma_kind(B, M, K, N, al, true), kb = mfma_kind(B, K, N, M, al, false);
-    if (ka == kb && ka != 0) {
-      LogBwdArgs pa = p, pb = p;
-      pa.grad = grad_a;
-      pb.grad = grad_b;
-      return ka == 2 ? launch_bwd_mfma_both<MTWide, MTTall>(pa, pb, st, B, s)
-                     : launch_bwd_mfma_both<MT128, MT128>(pa, pb, st, B, s);
-    }
-  }
-  if (grad_a) {
-    p.grad = grad_a;
-    if (int e = run_bwd<true>(p, st, B, s)) return e;
-  }
-  if (grad_b) {
-    p.grad = grad_b;
-    if (int e = run_bwd<false>(p, st, B, s)) return e;
-  }
-  return GENBMM_OK;
+  return genbmm::run_bwd_both(a, b, out, g, stats, grad_a, grad_b, B, M, K, N, GENBMM_PATH_AUTO,
+                              (hipStream_t)stream);
+}
+
+int genbmm_logbmm_bwd_path(const float* a, const float* b, const float* out, const float* g,
+                           const float* stats, float* grad_a, float* grad_b, int B, int M, int K,
+                           int N, int path, void* stream) {
+  return genbmm::run_bwd_both(a, b, out, g, stats, grad_a, grad_b, B, M, K, N, path,
+                              (hipStream_t)stream);
 }
 
 }  // extern "C"

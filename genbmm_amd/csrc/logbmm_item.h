@@ -14,6 +14,7 @@
 #pragma once
 
 #include "common.h"
+#include "logbmm_ws.h"
 
 namespace genbmm {
 
@@ -66,11 +67,13 @@ template <int G, int TB, bool FULL = false>
 __global__ __launch_bounds__(G * G, TB == 2 ? 8 : 1) void k_log_item_fwd(const float* __restrict__ a,
                                                       const float* __restrict__ b,
                                                       float* __restrict__ out,
-                                                      float* __restrict__ stats, int M_, int K_,
+                                                      float* __restrict__ stats,
+                                                      int* __restrict__ hdr, int M_, int K_,
                                                       int N_) {
   constexpr int NT = G * G, S = G * TB, LD = S + 1;
   const int M = FULL ? S : M_, K = FULL ? S : K_, N = FULL ? S : N_;
   static_assert(2 * S <= NT, "row and column scans use 2*S threads");
+  if (hdr && blockIdx.x == 0 && threadIdx.x == 0) hdr[0] = kWsNone;  // no per-tile flags in this workspace
   __shared__ float At[S * LD];  // [k][m]: a, then EA; finally the output tile [m][n]
   __shared__ float Bs[S * LD];  // [k][n]: b, then EB
   __shared__ float al[S], be[S];

@@ -12,6 +12,7 @@
 #pragma once
 
 #include "common.h"
+#include "logbmm_ws.h"
 
 namespace genbmm {
 
@@ -181,6 +182,32 @@ struct LogPrepared {
   int* hdr;
 };
 
+// Must a backward tile be left to the exact routine?  Yes if the workspace does not
+// hold what the tile's kernel reads (need_factors: EA, EB, 1/S of the matrix-core
+// forward; otherwise the flags of any factored forward), or if the forward flagged a
+// tile among the cells this tile reduces over - rows [lo, lo + extent) of out and
+// every column (by_rows: a grad_a tile), or columns [lo, lo + extent) and every row (a
+// grad_b tile).  A pure function of what the forward left, so the backward kernel and
+// its fix-up launch derive the same answer and nothing is written to the workspace.
+// Every thread of the workgroup must call it (one barrier inside).
+__device__ __forceinline__ int bwd_tile_flagged(const int* __restrict__ hdr,
+                                                const int* __restrict__ fwd_flags,
+                                                bool need_factors, bool by_rows, int lo, int extent,
+                                                int batch, int M, int N, int tid, int nt) {
+  const int tag = hdr[0], ftr = hdr[1], ftc = hdr[2];
+  // flag words exist per 32 x 32 cells at the densest
+  int bad = !(need_factors ? tag == kWsMfma : (tag == kWsMfma || tag == kWsFast)) || ftr < 32 || ftc < 32;
+  if (!bad) {
+    const int fm = (M + ftr - 1) / ftr, fn = (N + ftc - 1) / ftc;
+    const int mlo = by_rows ? lo / ftr : 0, mhi = by_rows ? min((lo + extent - 1) / ftr, fm - 1) : fm - 1;
+    const int nlo = by_rows ? 0 : lo / ftc, nhi = by_rows ? fn - 1 : min((lo + extent - 1) / ftc, fn - 1);
+    const int nn = nhi - nlo + 1, cnt = (mhi - mlo + 1) * nn;
+    for (int t = tid; t < cnt; t += nt)
+      bad |= fwd_flags[((long)batch * fm + mlo + t / nn) * fn + nlo + t % nn];
+  }
+  return __syncthreads_or(bad);
+}
+
 // Compiler-level ordering point for a wave's own LDS traffic (the hardware
 // executes one wave's LDS instructions in order).
 __device__ __forceinline__ void wave_lds_sync() {
@@ -281,7 +308,7 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
   if (tile == 0 && tid == 0) {
     ws_hdr[1] = T::TR;
     ws_hdr[2] = T::TC;
-    ws_hdr[0] = 1;
+    ws_hdr[0] = kWsMfma;
   }
 
   floatx16 acc[2][2];
@@ -421,8 +448,8 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
 // GRAD_B: tile (k,n) of grad_b = EB * sum_m EA[m][k] H[m][n]; rows <- EA,
 //         columns <- H, both sources [red][out].
 // A tile that touches a cell the forward flagged (R unusable there), or runs
-// on a workspace the matrix-core forward did not fill, raises its own flag and
-// leaves the work to the fix-up launch.
+// on a workspace the matrix-core forward did not fill, leaves its work to the
+// fix-up launch, which finds it by the same test (bwd_tile_flagged).
 // RAGGED (any sizes): lines of a tile beyond the matrix re-read the last line (they
 // only feed results that are not stored); pieces straddling the right edge are
 // read element by element; the reduction tail is zero-filled in both operands by
@@ -432,8 +459,8 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
     float* __restrict__ smem, int tile, const float* __restrict__ g,
     const float* __restrict__ ws_ea, const float* __restrict__ ws_eb,
     const float* __restrict__ ws_r, const int* __restrict__ ws_hdr,
-    const int* __restrict__ fwd_flags, float* __restrict__ grad, int* __restrict__ flags, int M,
-    int K, int N, int tiles_r, int tiles_c) {
+    const int* __restrict__ fwd_flags, float* __restrict__ grad, int M, int K, int N, int tiles_r,
+    int tiles_c) {
   constexpr int NT = T::NT, LDR = T::LDR, LDC = T::LDC;
   using SH = std::conditional_t<GRAD_A, StageT<T::TR, NT, LDR>, StageS<T::TC, NT, LDC>>;
   using SY = std::conditional_t<GRAD_A, StageT<T::TC, NT, LDC>, StageS<T::TR, NT, LDR>>;
@@ -449,20 +476,10 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
   const int Q = GRAD_A ? N : M;                      // reduction extent
   const int R = GRAD_A ? M : K, Cc = GRAD_A ? K : N;  // output extents
 
-  {  // forward flags over the cells this tile reduces over
-    int bad = ws_hdr[0] != 1;
-    const int ftr = max(ws_hdr[1], 1), ftc = max(ws_hdr[2], 1);
-    const int fm = (M + ftr - 1) / ftr, fn = (N + ftc - 1) / ftc;
-    const int mlo = GRAD_A ? r0 / ftr : 0, mhi = GRAD_A ? min((r0 + T::TR - 1) / ftr, fm - 1) : fm - 1;
-    const int nlo = GRAD_A ? 0 : c0 / ftc, nhi = GRAD_A ? fn - 1 : min((c0 + T::TC - 1) / ftc, fn - 1);
-    const int nn = nhi - nlo + 1, cnt = (mhi - mlo + 1) * nn;
-    if (!bad)
-      for (int t = tid; t < cnt; t += NT)
-        bad |= fwd_flags[((long)batch * fm + mlo + t / nn) * fn + nlo + t % nn];
-    bad = __syncthreads_or(bad);
-    if (tid == 0) flags[tile] = bad;
-    if (bad) return;
-  }
+  // forward flags over the cells this tile reduces over: the fix-up launch takes the tile
+  if (bwd_tile_flagged(ws_hdr, fwd_flags, true, GRAD_A, GRAD_A ? r0 : c0, GRAD_A ? T::TR : T::TC, batch,
+                       M, N, tid, NT))
+    return;
 
   floatx16 acc[2][2];
 #pragma unroll
@@ -589,11 +606,10 @@ __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WPE, T
 void k_log_bwd_mfma(const float* __restrict__ g, const float* __restrict__ ws_ea,
                     const float* __restrict__ ws_eb, const float* __restrict__ ws_r,
                     const int* __restrict__ ws_hdr, const int* __restrict__ fwd_flags,
-                    float* __restrict__ grad, int* __restrict__ flags, int M, int K, int N,
-                    int tiles_r, int tiles_c) {
+                    float* __restrict__ grad, int M, int K, int N, int tiles_r, int tiles_c) {
   __shared__ __attribute__((aligned(16))) float smem[2 * kMS * (T::LDR + T::LDC)];
   log_bwd_mfma_tile<T, GRAD_A, RAGGED>(smem, xcd_tile_id(), g, ws_ea, ws_eb, ws_r, ws_hdr, fwd_flags,
-                                       grad, flags, M, K, N, tiles_r, tiles_c);
+                                       grad, M, K, N, tiles_r, tiles_c);
 }
 
 // Both gradients in one launch: workgroups [0, tiles_a) take the tiles of grad_a
@@ -605,8 +621,7 @@ __global__ __launch_bounds__(TA::NT) __attribute__((amdgpu_waves_per_eu(TA::WPE,
 void k_log_bwd_mfma_both(const float* __restrict__ g, const float* __restrict__ ws_ea,
                          const float* __restrict__ ws_eb, const float* __restrict__ ws_r,
                          const int* __restrict__ ws_hdr, const int* __restrict__ fwd_flags,
-                         float* __restrict__ grad_a, float* __restrict__ grad_b,
-                         int* __restrict__ flags_a, int* __restrict__ flags_b, int M, int K, int N,
+                         float* __restrict__ grad_a, float* __restrict__ grad_b, int M, int K, int N,
                          int tiles_a, int ar, int ac, int br, int bc) {
   static_assert(TA::NT == TB::NT && TA::WPE == TB::WPE, "");
   constexpr int kA = 2 * kMS * (TA::LDR + TA::LDC), kB = 2 * kMS * (TB::LDR + TB::LDC);
@@ -616,11 +631,11 @@ void k_log_bwd_mfma_both(const float* __restrict__ g, const float* __restrict__ 
   const bool renum = (tiles_a & 7) == 0 && (n & 7) == 0;
   if (w < tiles_a)
     log_bwd_mfma_tile<TA, true, RAGGED>(smem, renum ? xcd_renumber(w, tiles_a) : w, g, ws_ea, ws_eb,
-                                        ws_r, ws_hdr, fwd_flags, grad_a, flags_a, M, K, N, ar, ac);
+                                        ws_r, ws_hdr, fwd_flags, grad_a, M, K, N, ar, ac);
   else
     log_bwd_mfma_tile<TB, false, RAGGED>(smem, renum ? xcd_renumber(w - tiles_a, n - tiles_a) : w - tiles_a,
-                                         g, ws_ea, ws_eb, ws_r, ws_hdr, fwd_flags, grad_b, flags_b, M,
-                                         K, N, br, bc);
+                                         g, ws_ea, ws_eb, ws_r, ws_hdr, fwd_flags, grad_b, M, K, N, br,
+                                         bc);
 }
 
 // ------------------------------------------------------- sampling sweep

@@ -7,6 +7,11 @@
 
 namespace genbmm {
 
+// First word of the workspace's header: which forward filled the workspace last.
+constexpr int kWsNone = 0;  // one that leaves no per-tile flags (exact and whole-item kernels)
+constexpr int kWsMfma = 1;  // the matrix-core forward: flags, EA, EB and 1/S
+constexpr int kWsFast = 2;  // the factored vector-ALU forward: flags only
+
 struct LogFactors {
   const float* ea;   // exp(a - row maximum), (B, M, K)
   const float* eb;   // exp(b - column maximum), (B, K, N)

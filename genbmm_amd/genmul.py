@@ -22,9 +22,16 @@ Differences in mechanism (not in results):
     (matmul_cuda_kernel.cu:517).
 
 Element types: float32 takes the kernels above; float64 takes the library's
-double-precision entry points (`*_f64`, the reference's algorithms as they stand,
-no workspaces); float16 / bfloat16 are widened to float32 and the result is
-narrowed again.
+double-precision entry points (`*_f64`, no workspaces); float16 / bfloat16 are
+widened to float32 and the result is narrowed again.
+
+Beyond the reference's contract the four functions also take operands with any
+number of leading batch dimensions (equal or broadcastable; they are flattened to
+one and restored on the result) and non-contiguous operands (made contiguous;
+the reference raises).  Both conversions, and the widening of half types, happen
+outside the autograd Functions with differentiable torch operations, so first-
+and second-order gradients reach the tensors the caller passed.  CPU tensors
+raise RuntimeError, as in the reference (matmul_cuda.cpp:65-67).
 """
 import torch
 
@@ -38,22 +45,60 @@ def _f64(t):
     return t.dtype == torch.float64
 
 
+PATH_AUTO, PATH_EXACT, PATH_VALU = 0, 1, 2  # GENBMM_PATH_* of the C header
+
+
 def _prep(a, b):
-    """Validate, and widen half types to float32; float32 and float64 stay."""
+    """Checks in front of the library for operands that are already in its form
+    (3-D, contiguous, float32 or float64, on one device)."""
     if not isinstance(a, torch.Tensor) or not isinstance(b, torch.Tensor):
         raise RuntimeError("a and b must be tensors")
     if a.dtype != b.dtype:
         raise RuntimeError("a and b must have the same dtype, got %s and %s" % (a.dtype, b.dtype))
-    if a.dtype in _UPCAST:
-        _lib.require(a, "a", dtype=a.dtype)
-        _lib.require(b, "b", dtype=b.dtype)
-        a, b = a.float(), b.float()
-    elif a.dtype not in (_COMPUTE, torch.float64):
+    if a.dtype not in (_COMPUTE, torch.float64):
         raise RuntimeError(
             "genbmm_amd computes in float32 or float64; %s inputs are not supported" % a.dtype
         )
-    dims = _lib.dense_dims(a, b)
-    return a, b, dims
+    return _lib.dense_dims(a, b)
+
+
+def _canonical(a, b):
+    """(a3, b3, restore): the operands as contiguous 3-D float32 / float64 tensors and
+    the function that gives the (B, M, N) result the caller's batch shape and dtype.
+    Everything done here is an ordinary differentiable torch operation."""
+    if not isinstance(a, torch.Tensor) or not isinstance(b, torch.Tensor):
+        raise RuntimeError("a and b must be tensors")
+    if not a.is_cuda or not b.is_cuda:
+        raise RuntimeError("a and b must be CUDA tensors")
+    if a.dtype != b.dtype:
+        raise RuntimeError("a and b must have the same dtype, got %s and %s" % (a.dtype, b.dtype))
+    if a.dim() < 2 or b.dim() < 2:
+        raise RuntimeError("a and b must have at least 2 dimensions")
+    if a.shape[-1] != b.shape[-2]:
+        raise RuntimeError("shape mismatch: a is %s, b is %s" % (tuple(a.shape), tuple(b.shape)))
+    in_dtype = a.dtype
+    if in_dtype in _UPCAST:
+        a, b = a.float(), b.float()
+    elif in_dtype not in (_COMPUTE, torch.float64):
+        raise RuntimeError(
+            "genbmm_amd computes in float32 or float64; %s inputs are not supported" % in_dtype
+        )
+    batch = None
+    if a.dim() != 3 or b.dim() != 3 or a.shape[0] != b.shape[0]:
+        try:
+            batch = torch.broadcast_shapes(a.shape[:-2], b.shape[:-2])
+        except RuntimeError:
+            raise RuntimeError("shape mismatch: a is %s, b is %s" % (tuple(a.shape), tuple(b.shape)))
+        a = a.expand(batch + a.shape[-2:]).reshape((-1,) + a.shape[-2:])
+        b = b.expand(batch + b.shape[-2:]).reshape((-1,) + b.shape[-2:])
+    a, b = a.contiguous(), b.contiguous()
+
+    def restore(out):
+        if batch is not None:
+            out = out.reshape(batch + out.shape[-2:])
+        return out if out.dtype == in_dtype else out.to(in_dtype)
+
+    return a, b, restore
 
 
 def _call(name, t, *args):
@@ -71,7 +116,7 @@ class _LogBmmGrad(torch.autograd.Function):
     """
 
     @staticmethod
-    def forward(ctx, a, b, g, out, stats):
+    def forward(ctx, a, b, g, out, stats, path):
         B, M, K, N = _lib.dense_dims(a, b)
         grad_a = torch.empty_like(a)
         grad_b = torch.empty_like(b)
@@ -79,8 +124,8 @@ class _LogBmmGrad(torch.autograd.Function):
             _call("genbmm_logbmm_bwd_f64", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g),
                   _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
         else:
-            _call("genbmm_logbmm_bwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g),
-                  _lib.ptr(stats), _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
+            _call("genbmm_logbmm_bwd_path", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g),
+                  _lib.ptr(stats), _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N, path)
         ctx.save_for_backward(a, b, g, out)
         ctx.set_materialize_grads(False)
         return grad_a, grad_b
@@ -88,7 +133,7 @@ class _LogBmmGrad(torch.autograd.Function):
     @staticmethod
     def backward(ctx, u_a, u_b):
         if u_a is None and u_b is None:
-            return None, None, None, None, None
+            return None, None, None, None, None, None
         a, b, g, out = ctx.saved_tensors
         B, M, K, N = _lib.dense_dims(a, b)
         u_a = None if u_a is None else u_a.contiguous()
@@ -99,16 +144,16 @@ class _LogBmmGrad(torch.autograd.Function):
         _call("genbmm_logbmm_bwdbwd_f64" if _f64(a) else "genbmm_logbmm_bwdbwd", a, _lib.ptr(a),
               _lib.ptr(b), _lib.ptr(out), _lib.ptr(g), _lib.ptr(u_a), _lib.ptr(u_b), _lib.ptr(ga),
               _lib.ptr(gb), _lib.ptr(gg), B, M, K, N)
-        return ga, gb, gg, None, None
+        return ga, gb, gg, None, None, None
 
 
 class LogMatMul(torch.autograd.Function):
-    """out[b,m,n] = logsumexp_k(a[b,m,k] + b[b,k,n])   (reference genmul.py:27-41)."""
+    """out[b,m,n] = logsumexp_k(a[b,m,k] + b[b,k,n])   (reference genmul.py:27-41).
+    `path` names the library's kernel family (PATH_AUTO unless a test says otherwise)."""
 
     @staticmethod
-    def forward(ctx, a, b):
-        in_dtype = a.dtype if isinstance(a, torch.Tensor) else None
-        a, b, (B, M, K, N) = _prep(a, b)
+    def forward(ctx, a, b, path=PATH_AUTO):
+        B, M, K, N = _prep(a, b)
         out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)
         if _f64(a):
             stats = a.new_empty(0)
@@ -117,17 +162,17 @@ class LogMatMul(torch.autograd.Function):
             # the library's workspace: what the reference's `maxes` becomes
             stats = torch.empty(_lib.load().genbmm_logbmm_stats_size(B, M, K, N), dtype=_COMPUTE,
                                 device=a.device)
-            _call("genbmm_logbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(stats),
-                  B, M, K, N)
+            _call("genbmm_logbmm_fwd_path", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(stats),
+                  B, M, K, N, path)
         ctx.save_for_backward(a, b, out, stats)
-        ctx.in_dtype = in_dtype
-        return out.to(in_dtype)
+        ctx.path = path
+        return out
 
     @staticmethod
     def backward(ctx, grad_output):
         a, b, out, stats = ctx.saved_tensors
-        grad_a, grad_b = _LogBmmGrad.apply(a, b, grad_output.to(a.dtype).contiguous(), out, stats)
-        return grad_a.to(ctx.in_dtype), grad_b.to(ctx.in_dtype)
+        grad_a, grad_b = _LogBmmGrad.apply(a, b, grad_output.to(a.dtype).contiguous(), out, stats, ctx.path)
+        return grad_a, grad_b, None
 
 
 # ------------------------------------------------- max / sample / prod-max
@@ -155,7 +200,7 @@ def _argmax_backward(ctx, grad_output, prod):
     else:
         _call("genbmm_argmax_bwd", g, _lib.ptr(idx), _lib.ptr(g), _lib.ptr(grad_a),
               _lib.ptr(grad_b), B, M, K, N)
-    return grad_a.to(ctx.in_dtype), grad_b.to(ctx.in_dtype)
+    return grad_a, grad_b
 
 
 class MaxMatMul(torch.autograd.Function):
@@ -163,16 +208,15 @@ class MaxMatMul(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, a, b):
-        in_dtype = a.dtype if isinstance(a, torch.Tensor) else None
-        a, b, dims = _prep(a, b)
+        dims = _prep(a, b)
         B, M, K, N = dims
         out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)
         idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
         _call("genbmm_maxbmm_fwd_f64" if _f64(a) else "genbmm_maxbmm_fwd", a, _lib.ptr(a),
               _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), B, M, K, N)
         ctx.save_for_backward(idx)
-        ctx.dims, ctx.in_dtype, ctx.compute = dims, in_dtype, a.dtype
-        return out.to(in_dtype)
+        ctx.dims, ctx.compute = dims, a.dtype
+        return out
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -184,8 +228,7 @@ class ProdMaxMatMul(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, a, b):
-        in_dtype = a.dtype if isinstance(a, torch.Tensor) else None
-        a, b, dims = _prep(a, b)
+        dims = _prep(a, b)
         B, M, K, N = dims
         out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)
         idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
@@ -199,8 +242,8 @@ class ProdMaxMatMul(torch.autograd.Function):
             _call("genbmm_prodmaxbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
                   _lib.ptr(factors), B, M, K, N)
             ctx.save_for_backward(idx, factors, empty, empty)
-        ctx.dims, ctx.in_dtype, ctx.compute = dims, in_dtype, a.dtype
-        return out.to(in_dtype)
+        ctx.dims, ctx.compute = dims, a.dtype
+        return out
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -227,8 +270,7 @@ class SampleMatMul(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, a, b, stream=None):
-        in_dtype = a.dtype if isinstance(a, torch.Tensor) else None
-        a, b, dims = _prep(a, b)
+        dims = _prep(a, b)
         B, M, K, N = dims
         seed, offset = _next_stream(a.device) if stream is None else stream
         out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)
@@ -243,19 +285,40 @@ class SampleMatMul(torch.autograd.Function):
             _call("genbmm_samplebmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
                   _lib.ptr(stats), seed, offset, B, M, K, N)
         ctx.save_for_backward(idx)
-        ctx.dims, ctx.in_dtype, ctx.compute = dims, in_dtype, a.dtype
-        return out.to(in_dtype)
+        ctx.dims, ctx.compute = dims, a.dtype
+        return out
 
     @staticmethod
     def backward(ctx, grad_output):
         return _argmax_backward(ctx, grad_output, prod=False) + (None,)
 
 
+def logbmm(a, b):
+    """genbmm.logbmm(a, b): out[..., m, n] = logsumexp_k(a[..., m, k] + b[..., k, n])."""
+    a, b, restore = _canonical(a, b)
+    return restore(LogMatMul.apply(a, b, PATH_AUTO))
+
+
+def logbmm_on_path(a, b, path):
+    """logbmm with the library's kernel family named (PATH_AUTO / PATH_EXACT / PATH_VALU);
+    forward and backward both use it.  For tests and measurements."""
+    a, b, restore = _canonical(a, b)
+    return restore(LogMatMul.apply(a, b, path))
+
+
+def maxbmm(a, b):
+    """genbmm.maxbmm(a, b): max_k(a + b); the gradient goes to the lowest arg-max."""
+    a, b, restore = _canonical(a, b)
+    return restore(MaxMatMul.apply(a, b))
+
+
+def prodmaxbmm(a, b):
+    """genbmm.prodmaxbmm(a, b): max_k(a * b)."""
+    a, b, restore = _canonical(a, b)
+    return restore(ProdMaxMatMul.apply(a, b))
+
+
 def samplebmm(a, b, stream=None):
     """genbmm.samplebmm(a, b); `stream=(seed, offset)` makes the draw reproducible."""
-    return SampleMatMul.apply(a, b, stream)
-
-
-logbmm = LogMatMul.apply
-maxbmm = MaxMatMul.apply
-prodmaxbmm = ProdMaxMatMul.apply
+    a, b, restore = _canonical(a, b)
+    return restore(SampleMatMul.apply(a, b, stream))

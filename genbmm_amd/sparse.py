@@ -20,6 +20,7 @@ when its extension is absent, have no counterpart here: a product on CPU
 tensors raises.
 """
 import operator
+import os
 
 import torch
 import torch.nn.functional as F
@@ -27,6 +28,10 @@ import torch.nn.functional as F
 from . import _lib
 
 MODE_LOG, MODE_MAX, MODE_MUL = 0, 1, 3
+
+# The reference sets this when its extension imports (sparse.py:3-9); here: the HIP
+# library has been built.  (It selects nothing: there is no other path to fall back to.)
+has_cuda = os.path.exists(_lib.LIB_PATH)
 
 
 def _band_rows(n_cols, lu, ld, n_rows, device):
@@ -159,6 +164,33 @@ def _band_transpose(data, lu, ld):
     return torch.where(ok, gathered, torch.zeros((), dtype=data.dtype, device=data.device))
 
 
+def repdiag(x, lu, ld):
+    """out[..., i, j] = x[..., i + j - ld, j], 0 where that row does not exist: the
+    diagonals of a band tensor re-read as rows (reference sparse.py:33-47, which pads,
+    unfolds and takes a diagonal).  `repdiag(data.flip(-1), lu, ld)` is the band of the
+    transposed matrix."""
+    return _band_transpose(x.flip(-1), lu, ld)
+
+
+class Transpose(torch.autograd.Function):
+    """Band data of the transposed matrix, `Transpose.apply(val, lu, ld)` as in the
+    reference (sparse.py:64-77); differentiable any number of times (the adjoint of a
+    band transpose is the transpose back)."""
+
+    @staticmethod
+    def forward(ctx, val, lu, ld):
+        ctx.bands = (lu, ld)
+        return _band_transpose(val.detach(), lu, ld)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        lu, ld = ctx.bands
+        return Transpose.apply(grad_output, ld, lu), None, None
+
+
+Transpose2 = Transpose  # the reference's helper for the second derivative (sparse.py:50-61)
+
+
 class BandedMatrix:
     def __init__(self, data, lu, ld, fill=0):
         batch, n, off = data.shape
@@ -278,7 +310,10 @@ class BandedMatrix:
         assert other.data.shape[1] == n
         lu = self.lu + other.ld
         ld = self.ld + other.lu
-        out = fn(self.data, self.lu, self.ld, other.data, other.lu, other.ld, lu, ld)
+        # views are copied here, by a differentiable torch operation, so that the
+        # Functions save (and differentiate with respect to) what they were given
+        out = fn(self.data.contiguous(), self.lu, self.ld, other.data.contiguous(), other.lu, other.ld,
+                 lu, ld)
         return BandedMatrix(out, lu, ld, self.fill)
 
     def multiply(self, other):
@@ -292,6 +327,14 @@ class BandedMatrix:
     def multiply_max(self, other):
         """The same product in the (max, +) semiring (reference sparse.py:255-266)."""
         return self._product(other, bandedmaxbmm)
+
+    def multiply_back(self, other, out, grad_out):
+        """Gradient of `self.multiply(other)` with respect to self, given the gradient of
+        the product's band tensor (reference sparse.py:363-379; `out` is not needed)."""
+        a, b = self.data.detach().contiguous(), other.data.detach().contiguous()
+        g = grad_out.data if isinstance(grad_out, BandedMatrix) else grad_out
+        grad_a, _ = _backward(a, b, (self.lu, self.ld, other.lu, other.ld), None, None, g, MODE_MUL)
+        return BandedMatrix(grad_a, self.lu, self.ld, self.fill)
 
 
 # ------------------------------------------------------------------ autograd
@@ -348,8 +391,12 @@ def _backward(a, b, bands, out, idx, g, mode, ws=None):
         _call("genbmm_banded_bwd_f64", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
               _lib.ptr(out), _lib.ptr(idx), _lib.ptr(g), _lib.ptr(grad_a), _lib.ptr(grad_b), B, n, mode)
         return grad_a, grad_b
-    _call("genbmm_banded_bwd", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
-          _lib.ptr(out), _lib.ptr(idx), _lib.ptr(ws), _lib.ptr(g), _lib.ptr(grad_a),
+    # g / sum per output cell, which both gradients of the log product share, goes to a
+    # buffer of this call's own: the forward's workspace stays as the forward left it, so
+    # backward passes over one forward may overlap (other streams, retained graphs)
+    scratch = torch.empty_like(out) if (mode == MODE_LOG and ws is not None) else None
+    _call("genbmm_banded_bwd_scratch", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
+          _lib.ptr(out), _lib.ptr(idx), _lib.ptr(ws), _lib.ptr(scratch), _lib.ptr(g), _lib.ptr(grad_a),
           _lib.ptr(grad_b), B, n, mode)
     return grad_a, grad_b
 
@@ -362,14 +409,14 @@ class BandedMul(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, a, a_lu, a_ld, b, b_lu, b_ld, o_lu, o_ld):
-        a, b, out, _ = _forward(a, a_lu, a_ld, b, b_lu, b_ld, MODE_MUL)
+        _, _, out, _ = _forward(a, a_lu, a_ld, b, b_lu, b_ld, MODE_MUL)
         ctx.save_for_backward(a, b)
         ctx.bands = (a_lu, a_ld, b_lu, b_ld)
         return out
 
     @staticmethod
     def backward(ctx, grad_output):
-        a, b = ctx.saved_tensors
+        a, b = (t.contiguous() for t in ctx.saved_tensors)
         grad_a, grad_b = _backward(a, b, ctx.bands, None, None, grad_output, MODE_MUL)
         return (grad_a, None, None, grad_b) + (None,) * 4
 
@@ -408,7 +455,10 @@ class BandedLogMul(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, a, a_lu, a_ld, b, b_lu, b_ld, o_lu, o_ld):
-        a, b, out, ws = _forward(a, a_lu, a_ld, b, b_lu, b_ld, MODE_LOG)
+        _, _, out, ws = _forward(a, a_lu, a_ld, b, b_lu, b_ld, MODE_LOG)
+        # the operands as given (the reference does the same, sparse.py:510-520): when they
+        # are views, the copies are taken in backward, where autograd records them, so
+        # that second-order gradients flow to the caller's tensors
         ctx.save_for_backward(a, b, out, ws)
         ctx.bands = (a_lu, a_ld, b_lu, b_ld)
         return out
@@ -416,6 +466,7 @@ class BandedLogMul(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         a, b, out, ws = ctx.saved_tensors
+        a, b = a.contiguous(), b.contiguous()
         g = grad_output.to(a.dtype).contiguous()
         grad_a, grad_b = _BandedLogGrad.apply(a, b, g, out, ws, ctx.bands)
         return (grad_a, None, None, grad_b) + (None,) * 4
@@ -428,7 +479,7 @@ class BandedMaxMul(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, a, a_lu, a_ld, b, b_lu, b_ld, o_lu, o_ld):
-        a, b, out, idx = _forward(a, a_lu, a_ld, b, b_lu, b_ld, MODE_MAX)
+        _, _, out, idx = _forward(a, a_lu, a_ld, b, b_lu, b_ld, MODE_MAX)
         ctx.save_for_backward(a, b, idx)
         ctx.bands = (a_lu, a_ld, b_lu, b_ld)
         return out
@@ -436,6 +487,7 @@ class BandedMaxMul(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         a, b, idx = ctx.saved_tensors
+        a, b = a.contiguous(), b.contiguous()
         grad_a, grad_b = _backward(a, b, ctx.bands, None, idx, grad_output, MODE_MAX)
         return (grad_a, None, None, grad_b) + (None,) * 4
 

@@ -19,8 +19,8 @@
  *     legacy default stream);
  *   - return value: 0 = enqueued; < 0 = argument error (GENBMM_E_*);
  *     > 0 = the hipError_t reported by the launch;
- *   - calls are re-entrant and thread safe; the only global state is the
- *     switch genbmm_logbmm_force_exact().
+ *   - calls are re-entrant and thread safe: the library keeps no mutable global
+ *     state, and a pointer declared const is only read.
  *
  * Dense operands: a is (B, M, K), b is (B, K, N), results are (B, M, N).
  * Banded operands: band data is (B, n, W) with W = lu + ld + 1 and
@@ -40,7 +40,7 @@ extern "C" {
 #define GENBMM_OK 0
 #define GENBMM_E_NULLPTR (-1) /* a required pointer is NULL            */
 #define GENBMM_E_SHAPE (-2)   /* a dimension is < 0 or overflows int32 */
-#define GENBMM_E_MODE (-3)    /* unknown semiring mode                 */
+#define GENBMM_E_MODE (-3)    /* unknown semiring mode or kernel path  */
 #define GENBMM_E_BAND (-4)    /* negative band width                   */
 
 /* Banded semiring modes (reference banded_cuda_kernel.cu:42,64,76). */
@@ -69,11 +69,13 @@ const char* genbmm_error_string(int code);
  * for every m followed by max_k b[k,n] for every n, and the forward uses them
  * to factor exp(a+b) = exp(a-max)*exp(b-max) wherever that is exact to fp32;
  * behind them sit per-tile flags naming the tiles where it is not, which a
- * fix-up launch recomputes with the online kernel's routine, and - for shapes
- * that run on the matrix cores (M and N at least 96, K at least 16) - exp(a-max), exp(b-max) and 1/sum, which the backward then reads
- * instead of taking any exponential itself.  The contents belong to the
- * library; the buffer takes the place of the reference's (B, M, N) `maxes`
- * output; pass the same buffer, unchanged, to genbmm_logbmm_bwd.
+ * fix-up launch recomputes with the online kernel's routine, a header naming
+ * the kernels that filled the buffer, and - for shapes that run on the matrix
+ * cores (M and N at least 96, K at least 16) - exp(a-max), exp(b-max) and
+ * 1/sum, which the backward then reads instead of taking any exponential
+ * itself.  The contents belong to the library; the buffer takes the place of
+ * the reference's (B, M, N) `maxes` output; pass the same buffer, unchanged,
+ * to genbmm_logbmm_bwd.
  */
 int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats,
                       int B, int M, int K, int N, void* stream);
@@ -85,10 +87,13 @@ int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats,
  * LogMatMul.backward (genmul.py:35-41; matmul_cuda.cpp:79-92;
  * matmul_cuda_kernel.cu:625-664, kernel :159-184).
  * grad_a or grad_b may be NULL (that gradient is then not computed), not both.
- * `stats`: NULL, or the buffer genbmm_logbmm_fwd filled for the same (a, b)
- * (the per-tile flags in it are rewritten, hence usable for any number of
- * backward calls).  With both gradients requested a matrix-core problem is one
- * launch.
+ * `stats`: NULL, or the buffer genbmm_logbmm_fwd filled for the same (a, b).
+ * It is only read: any number of backward calls, on any streams, may share it.
+ * Its header tells which forward kernels filled it; a backward kernel that
+ * needs by-products the buffer does not hold (or meets a tile the forward
+ * flagged) leaves that tile to the exact routine, so a mismatch costs time,
+ * never correctness.  With both gradients requested a matrix-core problem is
+ * one launch.
  */
 int genbmm_logbmm_bwd(const float* a, const float* b, const float* out,
                       const float* g, const float* stats,
@@ -99,14 +104,28 @@ int genbmm_logbmm_bwd(const float* a, const float* b, const float* out,
 size_t genbmm_logbmm_stats_size(int B, int M, int K, int N);
 
 /*
- * Process-wide switch for tests and measurements.  1: genbmm_logbmm_fwd / _bwd
- * ignore `stats` and always run the online / exact kernels.  2: the factored
- * kernels contract with v_fma_f32 on the vector ALU instead of the fp32
- * matrix-core instruction.  0 (default): factored kernels, on the matrix cores
- * wherever the shape allows.  The only piece of global state in the library.
- * No counterpart in the reference.
+ * The same two functions with the kernel family named per call (tests and
+ * measurements; the plain functions are GENBMM_PATH_AUTO).
+ *   GENBMM_PATH_AUTO   whole-item kernels for matrices up to 64^3, the fp32
+ *                      matrix cores where the shape allows, else the factored
+ *                      kernels on the vector ALU;
+ *   GENBMM_PATH_EXACT  the online / exp-per-term kernels only (what a NULL
+ *                      `stats` gives; a non-NULL one still receives the maxima);
+ *   GENBMM_PATH_VALU   the factored kernels contracting with v_fma_f32 on the
+ *                      vector ALU, never the matrix cores or whole-item kernels.
+ * Any other value: GENBMM_E_MODE.  Forward and backward of one problem need not
+ * name the same path (see genbmm_logbmm_bwd).  No counterpart in the reference.
  */
-void genbmm_logbmm_force_exact(int on);
+#define GENBMM_PATH_AUTO 0
+#define GENBMM_PATH_EXACT 1
+#define GENBMM_PATH_VALU 2
+int genbmm_logbmm_fwd_path(const float* a, const float* b, float* out,
+                           float* stats, int B, int M, int K, int N, int path,
+                           void* stream);
+int genbmm_logbmm_bwd_path(const float* a, const float* b, const float* out,
+                           const float* g, const float* stats,
+                           float* grad_a, float* grad_b,
+                           int B, int M, int K, int N, int path, void* stream);
 
 /*
  * Second-order terms of logbmm: the gradients with respect to (a, b, g) of

@@ -13,7 +13,7 @@ import torch
 
 import oracle
 import genbmm_amd as genbmm
-from genbmm_amd import _lib
+from genbmm_amd import _lib, genmul
 
 pytestmark = pytest.mark.gpu
 
@@ -37,12 +37,15 @@ def lse64(a, b, chunk=4):
 
 @pytest.fixture(params=["factored", "exact", "factored-valu"])
 def path(request, gpu):
-    """Run a logbmm test on every code path: the factored kernels (default: matrix cores
-    for 128x128 tiles), the online/exact kernels alone, the factored kernels on v_fma."""
-    lib = _lib.load()
-    lib.genbmm_logbmm_force_exact({"factored": 0, "exact": 1, "factored-valu": 2}[request.param])
-    yield request.param
-    lib.genbmm_logbmm_force_exact(0)
+    """Run a logbmm test on every kernel family of the library: the default one (whole-item
+    kernels for small matrices, matrix cores for large ones, factored vector-ALU kernels
+    between), the online / exact kernels alone, and the factored kernels on v_fma only.
+    The value is the `path` argument of genbmm_logbmm_fwd_path / _bwd_path."""
+    return {"factored": genmul.PATH_AUTO, "exact": genmul.PATH_EXACT, "factored-valu": genmul.PATH_VALU}[request.param]
+
+
+def logbmm_on(path):
+    return lambda a, b: genmul.logbmm_on_path(a, b, path)
 
 
 SHAPES = [(16, 64, 64, 64), (3, 7, 9, 5), (2, 1, 1, 1), (4, 5, 1, 6), (5, 33, 70, 129), (2, 130, 17, 66),
@@ -55,7 +58,7 @@ def test_logbmm_forward_and_grads(gpu, path, B, M, K, N):
     a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
     want, wa, wb = oracle.logbmm_grads64(a, b, g)
     ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
-    out = genbmm.logbmm(ad, bd)
+    out = logbmm_on(path)(ad, bd)
     close(out, want)
     ga, gb = torch.autograd.grad(out, (ad, bd), g.to(gpu))
     close(ga, wa)
@@ -72,7 +75,7 @@ def test_logbmm_config_c1_uniform_ones(gpu, path):
     g = torch.ones(16, 64, 64)
     want, wa, wb = oracle.logbmm_grads64(a, b, g)
     ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
-    out = genbmm.logbmm(ad, bd)
+    out = logbmm_on(path)(ad, bd)
     ga, gb = torch.autograd.grad(out.sum(), (ad, bd))
     close(out, want)
     close(ga, wa)
@@ -86,16 +89,16 @@ def test_logbmm_special_values(gpu, path):
     b[0, 2, :] = -math.inf          # masked k
     a[1, 3, :] = -math.inf          # fully masked row -> -inf
     a[0, 1, :] = -2e9               # below the -1e9 floor -> -inf, as in the reference
-    got = genbmm.logbmm(a.to(gpu), b.to(gpu)).cpu()
+    got = logbmm_on(path)(a.to(gpu), b.to(gpu)).cpu()
     want, _ = oracle.seq_logbmm_fwd(a, b)
     assert torch.equal(torch.isinf(got), torch.isinf(want))
     fin = ~torch.isinf(want)
     close(got[fin], want[fin])
     big = torch.randn(2, 9, 33) * 30 + 200  # large magnitudes
     bb = torch.randn(2, 33, 7) * 30 - 500
-    close(genbmm.logbmm(big.to(gpu), bb.to(gpu)), lse64(big, bb))
+    close(logbmm_on(path)(big.to(gpu), bb.to(gpu)), lse64(big, bb))
     a1, b1 = torch.randn(2, 5, 1), torch.randn(2, 1, 4)               # K = 1: out = a + b
-    close(genbmm.logbmm(a1.to(gpu), b1.to(gpu)), a1 + b1, rtol=1e-6, atol=1e-6)
+    close(logbmm_on(path)(a1.to(gpu), b1.to(gpu)), a1 + b1, rtol=1e-6, atol=1e-6)
 
 
 @pytest.mark.parametrize("B,M,K,N,sub", [(512, 128, 128, 128, 8), (8192, 32, 32, 32, 256), (64, 512, 512, 512, 1)])
@@ -105,7 +108,7 @@ def test_logbmm_baseline_shapes(gpu, path, B, M, K, N, sub):
     torch.manual_seed(0)
     a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
     ad, bd, gd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True), g.to(gpu)
-    out = genbmm.logbmm(ad, bd)
+    out = logbmm_on(path)(ad, bd)
     ga, gb = torch.autograd.grad(out, (ad, bd), gd)
     pick = torch.linspace(0, B - 1, sub).long()
     want, wa, wb = oracle.logbmm_grads64(a[pick], b[pick], g[pick])
@@ -142,13 +145,8 @@ def test_logbmm_factoring_guard(gpu, B, M, K, N):
     close(ga[:-1], wa)
     close(gb[:-1], wb)
     # the two paths agree with each other on these inputs as well
-    lib = _lib.load()
-    lib.genbmm_logbmm_force_exact(1)
-    try:
-        out2 = genbmm.logbmm(ad, bd)
-        ga2, gb2 = torch.autograd.grad((out2[:-1] * g[:-1].to(gpu)).sum(), (ad, bd))
-    finally:
-        lib.genbmm_logbmm_force_exact(0)
+    out2 = genmul.logbmm_on_path(ad, bd, genmul.PATH_EXACT)
+    ga2, gb2 = torch.autograd.grad((out2[:-1] * g[:-1].to(gpu)).sum(), (ad, bd))
     close(out2[:-1], want)
     close(ga2[:-1], wa)
     close(gb2[:-1], wb)
@@ -193,12 +191,10 @@ def test_logbmm_backward_on_foreign_workspace(gpu):
     out, ga, gb = torch.empty(B, M, N, device=gpu), torch.empty_like(ad), torch.empty_like(bd)
     stats = torch.full((lib.genbmm_logbmm_stats_size(B, M, K, N),), float("nan"), device=gpu)
     p, s = _lib.ptr, _lib.stream_of(ad)
-    lib.genbmm_logbmm_force_exact(2)
-    try:
-        assert lib.genbmm_logbmm_fwd(p(ad), p(bd), p(out), p(stats), B, M, K, N, s) == 0
-    finally:
-        lib.genbmm_logbmm_force_exact(0)
+    assert lib.genbmm_logbmm_fwd_path(p(ad), p(bd), p(out), p(stats), B, M, K, N, genmul.PATH_VALU, s) == 0
+    before = stats.clone()
     assert lib.genbmm_logbmm_bwd(p(ad), p(bd), p(out), p(gd), p(stats), p(ga), p(gb), B, M, K, N, s) == 0
+    assert torch.equal(before.view(torch.int32), stats.view(torch.int32))  # the backward only reads it
     pick = torch.tensor([0, B - 1])
     want, wa, wb = oracle.logbmm_grads64(a[pick], b[pick], g[pick])
     close(out[pick.to(gpu)], want)
@@ -483,6 +479,82 @@ def test_sample_config_c4_chi_square(gpu):
     assert worst > 0
 
 
+def test_sample_config_c4_at_full_size(gpu):
+    """Benchmark configuration 3 at its own size, through the C ABI: a, b = 2 * randn
+    (64, 512, 512) from seed 0, Philox seed 1234 - the shape whose sweep runs on the
+    matrix cores in 128 x 128 tiles behind a 256 x 128 forward.
+    out against the float64 log-sum-exp and every index against the float64 CDF of its
+    cell on a batch subset; over everything: 0 <= idx < K, the picked term carries mass,
+    and the one-hot gradients add up to g along k (exactly, g on the 1/8 grid).  Then the
+    chi-square of the slice test above, with the 10^4 draws per cell taken from 10^4
+    full-size calls (distinct Philox offsets) instead of from a tiled copy of the slice."""
+    from scipy.stats import chi2 as chi2_dist
+
+    torch.manual_seed(0)
+    B, M, K, N = 64, 512, 512, 512
+    a, b = 2 * torch.randn(B, M, K), 2 * torch.randn(B, K, N)
+    lib = _lib.load()
+    ad, bd = a.to(gpu), b.to(gpu)
+    out = torch.empty(B, M, N, device=gpu)
+    idx = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
+    stats = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=gpu)
+    p, s = _lib.ptr, _lib.stream_of(ad)
+
+    def draw(offset):
+        assert lib.genbmm_samplebmm_fwd(p(ad), p(bd), p(out), p(idx), p(stats), 1234, offset, B, M, K, N, s) == 0
+
+    draw(0)
+    u = oracle.philox_uniform(0, B * M * N, 1234, 0).view(B, M, N)
+    for item in (0, 37, 63):
+        close(out[item:item + 1], lse64(a[item:item + 1], b[item:item + 1]))
+        # the oracle's float64 CDF, evaluated on the device (1 GiB per batch item)
+        cdf = oracle.sample_cdf64(ad[item:item + 1], bd[item:item + 1])
+        got = idx[item:item + 1].long()
+        hi = torch.gather(cdf, 2, got.unsqueeze(2)).squeeze(2)
+        lo = torch.where(got > 0, torch.gather(cdf, 2, (got - 1).clamp(min=0).unsqueeze(2)).squeeze(2),
+                         torch.zeros_like(hi))
+        ui = u[item:item + 1].to(gpu).double()
+        ok = (lo - 2e-5 <= ui) & (ui <= hi + 2e-5)
+        assert bool(ok.all()), (item, float((~ok).float().mean()))
+        want = oracle.sample_index_from_cdf(cdf, ui).long()
+        assert float((got != want).float().mean()) < 2e-3
+        del cdf, want
+    il = idx.long()
+    assert int(il.min()) >= 0 and int(il.max()) < K
+    picked = torch.gather(ad, 2, il) + torch.gather(bd, 1, il)       # a[m, idx] + b[idx, n]
+    assert bool((picked - out > -40.0).all())                         # a term of visible mass
+    g = (torch.round(torch.randn(B, M, N) * 8) / 8).clamp(-4, 4).to(gpu)
+    ga, gb = torch.empty_like(ad), torch.empty_like(bd)
+    assert lib.genbmm_argmax_bwd(p(idx), p(g), p(ga), p(gb), B, M, K, N, s) == 0
+    assert torch.equal(ga.sum(-1), g.sum(-1)) and torch.equal(gb.sum(-2), g.sum(-2))
+    onehot = torch.zeros(M, K, device=gpu).scatter_add_(1, il[5], g[5])
+    assert torch.equal(ga[5], onehot)
+
+    # chi-square on the (4,16,16) slice from full-size draws
+    draws = 10000
+    counts = torch.zeros(4 * 16 * 16, K, device=gpu)
+    cells = torch.arange(4 * 16 * 16, device=gpu)
+    one = torch.ones(4 * 16 * 16, device=gpu)
+    for d in range(draws):
+        draw(4 * d + 4)
+        counts.index_put_((cells, idx[:4, :16, :16].reshape(-1).long()), one, accumulate=True)
+    counts = counts.cpu().double().view(4, 16, 16, K)
+    pr = torch.softmax(a[:4, :16, :].double().unsqueeze(-1) + b[:4, :, :16].double().unsqueeze(-3), -2)
+    expc = pr.permute(0, 1, 3, 2) * draws                             # (4,16,16,K)
+    for cell in range(4 * 16 * 16):
+        e, c = expc.reshape(-1, K)[cell], counts.reshape(-1, K)[cell]
+        keep = e >= 5
+        stat = float((((c - e) ** 2) / e)[keep].sum())
+        dof = int(keep.sum())
+        if (~keep).any():
+            ep, cp = float(e[~keep].sum()), float(c[~keep].sum())
+            if ep >= 1:
+                stat += (cp - ep) ** 2 / ep
+                dof += 1
+        dof = max(dof - 1, 1)
+        assert stat < chi2_dist.ppf(1 - 1e-6, dof), (cell, stat, dof)
+
+
 def test_sample_distribution_on_the_matrix_core_sweep(gpu):
     """A shape whose sweep runs on the matrix cores (slabs of 16 terms + resolve): 1500
     draws per cell with distinct Philox offsets; the empirical CDF of every cell stays
@@ -528,17 +600,19 @@ def test_errors(gpu):
     for op in (genbmm.logbmm, genbmm.maxbmm, genbmm.samplebmm, genbmm.prodmaxbmm):
         with pytest.raises(RuntimeError, match="CUDA tensor"):
             op(a, b)                                                   # matmul_cuda.cpp:65
-        with pytest.raises(RuntimeError, match="contiguous"):
-            op(a.to(gpu).transpose(1, 2).contiguous().transpose(1, 2), b.to(gpu))  # :66
         with pytest.raises(RuntimeError, match="shape mismatch"):
             op(a.to(gpu), torch.randn(2, 3, 5, device=gpu))
         with pytest.raises(RuntimeError, match="same dtype"):
             op(a.to(gpu).double(), b.to(gpu))
         with pytest.raises(RuntimeError, match="not supported"):
             op(a.to(gpu).long(), b.to(gpu).long())
+    # the autograd Functions themselves keep the reference's contract (matmul_cuda.cpp:66)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        genmul.LogMatMul.apply(a.to(gpu).transpose(1, 2).contiguous().transpose(1, 2), b.to(gpu))
     lib = _lib.load()
     null = ctypes.c_void_p(0)
     ad = a.to(gpu)
+    assert lib.genbmm_logbmm_fwd_path(_lib.ptr(ad), _lib.ptr(ad), _lib.ptr(ad), null, 1, 1, 1, 1, 7, null) == -3
     assert lib.genbmm_logbmm_fwd(null, _lib.ptr(ad), _lib.ptr(ad), null, 1, 1, 1, 1, null) == -1
     assert lib.genbmm_logbmm_fwd(_lib.ptr(ad), _lib.ptr(ad), _lib.ptr(ad), null, 1, -1, 1, 1, null) == -2
     assert lib.genbmm_banded_fwd(_lib.ptr(ad), 0, 0, _lib.ptr(ad), 0, 0, _lib.ptr(ad), null, null, 1, 1, 2, null) == -3
@@ -559,6 +633,58 @@ def test_empty_and_half(gpu):
     close(out.float(), lse64(a.float().cpu(), b.float().cpu()), rtol=2e-3, atol=2e-3)
     (ga,) = torch.autograd.grad(out.sum(), a)
     assert ga.dtype == torch.float16
+
+
+def test_views_and_batch_dimensions(gpu):
+    """Operands that are views (transposed, strided) are made contiguous, and any number
+    of leading batch dimensions - equal or broadcastable - is accepted; gradients arrive
+    in the callers' own tensors.  (The reference takes 3-D contiguous tensors only.)"""
+    torch.manual_seed(11)
+    at, b = torch.randn(3, 9, 14), torch.randn(3, 9, 6)       # a is given as the transpose of `at`
+    g = torch.randn(3, 14, 6)
+    want, wa, wb = oracle.logbmm_grads64(at.transpose(1, 2).contiguous(), b, g)
+    atd, bd = at.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    out = genbmm.logbmm(atd.transpose(1, 2), bd)
+    ga, gb = torch.autograd.grad(out, (atd, bd), g.to(gpu))
+    close(out, want)
+    close(ga, wa.transpose(1, 2))
+    close(gb, wb)
+    grid8 = lambda *s: torch.round(torch.randn(*s) * 8) / 8
+    a5, b5 = grid8(2, 3, 4, 7, 5), grid8(3, 1, 5, 8)          # batch (2, 3, 4) against (3, 1): broadcast
+    for op, ref in ((genbmm.maxbmm, lambda x, y: (x.unsqueeze(-1) + y.unsqueeze(-3)).amax(-2)),
+                    (genbmm.prodmaxbmm, lambda x, y: (x.unsqueeze(-1) * y.unsqueeze(-3)).amax(-2))):
+        x, y = a5.to(gpu).requires_grad_(True), b5.to(gpu).requires_grad_(True)
+        got = op(x, y)
+        assert got.shape == (2, 3, 4, 7, 8)
+        assert torch.equal(got.cpu(), ref(a5, b5.expand(2, 3, 4, 5, 8)))
+        gx, gy = torch.autograd.grad(got.sum(), (x, y))
+        assert gx.shape == a5.shape and gy.shape == b5.shape
+    s5 = genbmm.samplebmm(a5.to(gpu), b5.to(gpu), (7, 0))
+    close(s5, lse64(a5.reshape(-1, 7, 5), b5.expand(2, 3, 4, 5, 8).reshape(-1, 5, 8)).reshape(2, 3, 4, 7, 8))
+    a2, b2 = torch.randn(6, 5), torch.randn(5, 4)              # plain matrices
+    close(genbmm.logbmm(a2.to(gpu), b2.to(gpu)), lse64(a2[None], b2[None])[0])
+
+
+def test_half_inputs_are_twice_differentiable(gpu):
+    """float16 / bfloat16 operands are widened by a differentiable cast outside the
+    autograd Function, so second-order terms reach the half tensors as well."""
+    torch.manual_seed(12)
+    for dt in (torch.float16, torch.bfloat16):
+        a = torch.randn(2, 6, 7).to(dt)
+        b = torch.randn(2, 7, 5).to(dt)
+        g, u = torch.randn(2, 6, 5).to(dt).float(), torch.randn(2, 6, 7)
+        want = oracle.logbmm_second_order64(a.float(), b.float(), g, u, None)
+        ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+        out = genbmm.logbmm(ad, bd)
+        assert out.dtype == dt
+        (ga,) = torch.autograd.grad(out, ad, g.to(gpu).to(dt), create_graph=True)
+        assert ga.dtype == dt and ga.requires_grad
+        da, db = torch.autograd.grad((ga.float() * u.to(gpu)).sum(), (ad, bd))
+        assert da.dtype == dt and float(da.float().abs().max()) > 0 and float(db.float().abs().max()) > 0
+        # half rounding of g, of grad_a and of the results: 3 roundings of 2^-8 (bf16) / 2^-11
+        tol = 4e-2 if dt == torch.bfloat16 else 6e-3
+        close(da.float(), want[0], rtol=tol, atol=tol)
+        close(db.float(), want[1], rtol=tol, atol=tol)
 
 
 # ------------------------------------------------------- streams and HIP graphs

@@ -92,11 +92,37 @@ def test_transpose_is_differentiable():
     assert torch.equal(g, inside)
 
 
+def test_module_level_names_of_the_reference():
+    """has_cuda, repdiag, Transpose / Transpose2 (sparse.py:3-9, 33-77): repdiag against its
+    definition by padding and diagonals, Transpose against the dense transpose."""
+    from genbmm_amd import sparse
+
+    assert sparse.has_cuda == os.path.exists(_lib.LIB_PATH)
+    torch.manual_seed(4)
+    x, lu, ld = torch.randn(2, 7, 6), 2, 3
+    want = torch.zeros(2, 7, 6)
+    for i in range(7):
+        for j in range(6):
+            if 0 <= i + j - ld < 7:
+                want[:, i, j] = x[:, i + j - ld, j]
+    assert torch.equal(sparse.repdiag(x, lu, ld), want)
+    dense = torch.randn(2, 7, 7)
+    band = banddiag(dense, lu, ld)[0].clone().requires_grad_(True)
+    t = sparse.Transpose.apply(band, lu, ld)
+    assert torch.equal(t, banddiag(dense.transpose(1, 2), ld, lu)[0])
+    (g,) = torch.autograd.grad((t * t).sum(), band, create_graph=True)
+    inside = oracle.band_from_dense(torch.ones(2, 7, 7), lu, ld)
+    assert torch.allclose(g, 2 * band * inside)
+    (gg,) = torch.autograd.grad(g.sum(), band)
+    assert torch.allclose(gg, 2 * inside)
+    assert sparse.Transpose2 is sparse.Transpose
+
+
 def test_library_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "genbmm_gfx950.h")).read()
     declared = set(re.findall(r"\b(genbmm_[a-z_0-9]+)\s*\(", header))
-    assert len(declared) == 33
-    assert declared == set(_lib.SIGNATURES) | set(_lib.STRING_FUNCS) | set(_lib.VOID_FUNCS) | set(_lib.SIZE_FUNCS)
+    assert len(declared) == 34
+    assert declared == set(_lib.SIGNATURES) | set(_lib.STRING_FUNCS) | set(_lib.SIZE_FUNCS)
     assert os.path.exists(_lib.LIB_PATH), "build with `python -m genbmm_amd.build`"
     lib = ctypes.CDLL(_lib.LIB_PATH)
     for name in declared:

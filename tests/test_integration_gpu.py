@@ -69,9 +69,12 @@ def test_five_dimensional_operands(gpu):
     want = (a.double().unsqueeze(-1) + b.double().unsqueeze(-3)).logsumexp(-2)
     assert got.shape == (2, 3, 4, 17, 21)
     assert torch.allclose(got.cpu().double(), want, rtol=1e-5, atol=1e-5)
-    # a transposed view must be made contiguous by the caller, as with the reference
-    with pytest.raises(RuntimeError):
-        genbmm.logbmm(a.to(gpu).view(-1, 17, 9).transpose(1, 2), b.to(gpu).view(-1, 9, 21))
+    # the same operands handed over as they are: leading dimensions are flattened inside
+    direct = genbmm.logbmm(a.to(gpu), b.to(gpu))
+    assert torch.equal(direct, got)
+    # and a transposed view is made contiguous inside (the reference raises here)
+    at = a.to(gpu).transpose(-1, -2).contiguous()
+    assert torch.equal(genbmm.logbmm(at.transpose(-1, -2), b.to(gpu)), got)
 
 
 @pytest.mark.parametrize("n,lu,ld", [(24, 2, 3), (70, 5, 1)])

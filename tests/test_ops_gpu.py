@@ -48,7 +48,18 @@ def test_registrations_pass_opcheck(gpu):
     torch.library.opcheck(torch.ops.genbmm_amd.prodmaxbmm_fwd.default, (ad, bd), test_utils=tests)
     torch.library.opcheck(torch.ops.genbmm_amd.samplebmm_fwd.default, (ad, bd, 5, 0), test_utils=tests)
     out, idx = torch.ops.genbmm_amd.maxbmm_fwd(ad, bd)
-    torch.library.opcheck(torch.ops.genbmm_amd.argmax_bwd.default, (idx, torch.randn_like(out), 12), test_utils=tests)
+    g = torch.randn_like(out)
+    torch.library.opcheck(torch.ops.genbmm_amd.argmax_bwd.default, (idx, g, 12), test_utils=tests)
+    _, idx, factors = torch.ops.genbmm_amd.prodmaxbmm_fwd(ad, bd)
+    torch.library.opcheck(torch.ops.genbmm_amd.prodmax_bwd.default, (idx, factors, g, 12), test_utils=tests)
+    # the backward operators declare no mutation: the forward's workspace is only read
+    # (checked by test_schema), on a small shape and on one that runs on the matrix cores
+    for a2, b2 in ((ad, bd), (torch.randn(2, 128, 32, device=gpu), torch.randn(2, 32, 128, device=gpu))):
+        out, stats = torch.ops.genbmm_amd.logbmm_fwd(a2, b2)
+        g = torch.randn_like(out)
+        torch.library.opcheck(torch.ops.genbmm_amd.logbmm_bwd.default, (a2, b2, out, g, stats), test_utils=tests)
+        torch.library.opcheck(torch.ops.genbmm_amd.logbmm_bwdbwd.default,
+                              (a2, b2, out, g, torch.randn_like(a2), torch.randn_like(b2)), test_utils=tests)
 
 
 def test_graphs_compile_and_differentiate(gpu):
