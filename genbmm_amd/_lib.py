@@ -31,6 +31,7 @@ _BAND = [_c_float_p, _i, _i, _c_float_p, _i, _i]  # a, a_lu, a_ld, b, b_lu, b_ld
 SIGNATURES = {
     "genbmm_logbmm_fwd": [_c_float_p] * 4 + _DENSE_DIMS,
     "genbmm_logbmm_bwd": [_c_float_p] * 7 + _DENSE_DIMS,
+    "genbmm_logbmm_fwd_static": [_c_float_p] * 3 + _DENSE_DIMS,
     "genbmm_logbmm_fwd_path": [_c_float_p] * 4 + [_i, _i, _i, _i, _i, _vp],  # ..., B, M, K, N, path, stream
     "genbmm_logbmm_bwd_path": [_c_float_p] * 7 + [_i, _i, _i, _i, _i, _vp],
     "genbmm_logbmm_bwdbwd": [_c_float_p] * 9 + _DENSE_DIMS,
@@ -62,6 +63,7 @@ SIGNATURES = {
 }
 STRING_FUNCS = {"genbmm_version": [], "genbmm_error_string": [_i]}
 SIZE_FUNCS = {"genbmm_logbmm_stats_size": [_i, _i, _i, _i],
+              "genbmm_logbmm_static_limit": [],
               "genbmm_banded_workspace_size": [_i, _i, _i, _i, _i, _i]}
 
 _lib = None

@@ -357,6 +357,7 @@ const char* genbmm_error_string(int code) {
     case GENBMM_E_SHAPE: return "a dimension is negative or too large";
     case GENBMM_E_MODE: return "unknown semiring mode or kernel path";
     case GENBMM_E_BAND: return "negative band width";
+    case GENBMM_E_TOOBIG: return "problem exceeds the fixed workspace of this entry point";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
   }
 }

@@ -28,6 +28,7 @@
 // (any shape, this file) and the fp32 matrix-core instruction for problems made
 // of full 128x128 tiles (logbmm_mfma.h).
 #include <algorithm>
+#include <mutex>
 
 #include "dense_tiles.h"
 #include "log_bwd_tile.h"
@@ -645,7 +646,7 @@ int launch_fwd_fast(DenseArgs p, float* stats, int B, int M, int K, int N, hipSt
 // Matrix-core launches: T is the MTile; the ragged variant of a kernel is used only
 // when some extent is not a multiple of its tile / slab.
 template <class T>
-int launch_fwd_mfma(DenseArgs p, float* stats, int B, int M, int K, int N, hipStream_t s) {
+int launch_fwd_mfma(DenseArgs p, float* stats, int B, int M, int K, int N, bool keep, hipStream_t s) {
   p.M = M; p.K = K; p.N = N;
   p.tiles_m = ceil_div(M, T::TR);
   p.tiles_n = ceil_div(N, T::TC);
@@ -657,8 +658,14 @@ int launch_fwd_mfma(DenseArgs p, float* stats, int B, int M, int K, int N, hipSt
     hipLaunchKernelGGL(kern, dim3(total), dim3(T::NT), 0, s, p.a, p.b, p.out, stats, flags, ws.ea,
                        ws.eb, ws.r, ws.hdr, M, K, N, p.tiles_m, p.tiles_n);
   };
-  if (M % T::TR != 0 || N % T::TC != 0 || K % kMS != 0) go(k_log_fwd_mfma<T, true>);
-  else go(k_log_fwd_mfma<T, false>);
+  const bool ragged = M % T::TR != 0 || N % T::TC != 0 || K % kMS != 0;
+  if (keep) {
+    if (ragged) go(k_log_fwd_mfma<T, true, true>);
+    else go(k_log_fwd_mfma<T, false, true>);
+  } else {
+    if (ragged) go(k_log_fwd_mfma<T, true, false>);
+    else go(k_log_fwd_mfma<T, false, false>);
+  }
   if (int e = launch_status()) return e;
   return launch_fwd_fixup<CfgWide, T::TR, T::TC>(p, flags, total, s);
 }
@@ -825,8 +832,10 @@ void launch_item_fwd(const float* a, const float* b, float* out, float* stats, i
   hipLaunchKernelGGL((k_log_item_fwd<G, TB, FULL>), dim3(B), dim3(G * G), 0, s, a, b, out, stats, hdr, M, K, N);
 }
 
+// keep: the workspace is as large as genbmm_logbmm_stats_size says and receives what a
+// backward wants beside the maxima; false: header_offset() + 4 floats of it are used.
 int run_fwd(const float* a, const float* b, float* out, float* stats, int B, int M, int K, int N,
-            int path, hipStream_t s) {
+            int path, bool keep, hipStream_t s) {
   if (int e = check_dense_dims(B, M, K, N)) return e;
   if (!valid_path(path)) return GENBMM_E_MODE;
   const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
@@ -848,8 +857,8 @@ int run_fwd(const float* a, const float* b, float* out, float* stats, int B, int
   if (stats && K > 0 && path != GENBMM_PATH_EXACT) {
     const int64_t big_tiles = (int64_t)B * ceil_div(M, 128) * ceil_div(N, 128);
     switch (fwd_mfma_shape(B, M, K, N) ? mfma_kind(path, B, M, N, K, false) : 0) {
-      case 2: return launch_fwd_mfma<MTTall>(p, stats, B, M, K, N, s);
-      case 1: return launch_fwd_mfma<MT128>(p, stats, B, M, K, N, s);
+      case 2: return launch_fwd_mfma<MTTall>(p, stats, B, M, K, N, keep, s);
+      case 1: return launch_fwd_mfma<MT128>(p, stats, B, M, K, N, keep, s);
       default: break;
     }
     if (M <= 32 && N <= 32) return launch_fwd_fast<CfgSmall, CfgSmall>(p, stats, B, M, K, N, s);
@@ -911,6 +920,35 @@ int run_bwd_both(const float* a, const float* b, const float* out, const float* 
   return GENBMM_OK;
 }
 
+// ------------------------------------------------ forward on a workspace of the library's own
+// For callers that cannot allocate (code under HIP graph capture, serving loops,
+// harnesses that forbid it): the forward's workspace - maxima, per-tile flags, header;
+// no by-products for a backward - lives in this array, one copy per GPU for the life
+// of the process.  Host code never passes the array's name to a kernel (on the host
+// it names a stand-in, not device memory): the device address is looked up once per
+// device with that device current and kept in scratch_ptr[].
+constexpr size_t kStaticFloats = (size_t)1 << 20;  // 4 MiB
+static __device__ __align__(256) float scratch[kStaticFloats];
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mu;
+float* scratch_ptr[kMaxDevices] = {};
+
+int static_workspace(float** ws) {
+  int dev = -1;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return GENBMM_E_SHAPE;
+  std::lock_guard<std::mutex> lock(scratch_mu);
+  if (!scratch_ptr[dev]) {
+    float* p = nullptr;
+    if (hipError_t e = hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch)); e != hipSuccess)
+      return (int)e;
+    if (!p) return (int)hipErrorInvalidSymbol;
+    scratch_ptr[dev] = p;
+  }
+  *ws = scratch_ptr[dev];
+  return GENBMM_OK;
+}
+
 }  // namespace
 
 // The forward's own decision (run_fwd above, path AUTO): factors are written by the
@@ -959,12 +997,24 @@ size_t genbmm_logbmm_stats_size(int B, int M, int K, int N) {
 
 int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats, int B, int M,
                       int K, int N, void* stream) {
-  return genbmm::run_fwd(a, b, out, stats, B, M, K, N, GENBMM_PATH_AUTO, (hipStream_t)stream);
+  return genbmm::run_fwd(a, b, out, stats, B, M, K, N, GENBMM_PATH_AUTO, true, (hipStream_t)stream);
 }
 
 int genbmm_logbmm_fwd_path(const float* a, const float* b, float* out, float* stats, int B, int M,
                            int K, int N, int path, void* stream) {
-  return genbmm::run_fwd(a, b, out, stats, B, M, K, N, path, (hipStream_t)stream);
+  return genbmm::run_fwd(a, b, out, stats, B, M, K, N, path, true, (hipStream_t)stream);
+}
+
+size_t genbmm_logbmm_static_limit(void) { return genbmm::kStaticFloats; }
+
+int genbmm_logbmm_fwd_static(const float* a, const float* b, float* out, int B, int M, int K, int N,
+                             void* stream) {
+  using namespace genbmm;
+  if (int e = check_dense_dims(B, M, K, N)) return e;
+  if ((uint64_t)header_offset(B, M, N) + 4 > kStaticFloats) return GENBMM_E_TOOBIG;
+  float* ws = nullptr;
+  if (int e = static_workspace(&ws)) return e;
+  return run_fwd(a, b, out, ws, B, M, K, N, GENBMM_PATH_AUTO, false, (hipStream_t)stream);
 }
 
 int genbmm_logbmm_bwd(const float* a, const float* b, const float* out, const float* g,

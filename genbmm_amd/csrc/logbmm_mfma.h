@@ -257,7 +257,9 @@ __device__ __forceinline__ void acc_rows(const floatx16 (&acc)[2][2], float* __r
 // tail is filled with -inf (exp -> 0) by a loader used for the last slab only;
 // results and by-products are stored under masks.  Full-tile problems compile
 // without any of it.
-template <class T, bool RAGGED>
+// KEEP: leave EA, EB and 1/S in the workspace for the backward (false: a forward
+// for its own sake - the workspace then holds the maxima, flags and header only).
+template <class T, bool RAGGED, bool KEEP = true>
 __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WPE, T::WPE)))
 void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
                     float* __restrict__ out, const float* __restrict__ stats,
@@ -308,7 +310,7 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
   if (tile == 0 && tid == 0) {
     ws_hdr[1] = T::TR;
     ws_hdr[2] = T::TC;
-    ws_hdr[0] = kWsMfma;
+    ws_hdr[0] = KEEP ? kWsMfma : kWsFast;
   }
 
   floatx16 acc[2][2];
@@ -368,14 +370,14 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
   };
 
   load(slabs == 1 && ktail != 0);
-  stage(0, nblk == 0, mblk == 0);
+  stage(0, KEEP && nblk == 0, KEEP && mblk == 0);
   __syncthreads();
   int sa = 1 % tiles_n, sb = 1 % tiles_m;  // (s + 1) mod tiles_n, mod tiles_m
   for (int s = 0; s < slabs; ++s) {
     const bool more = s + 1 < slabs;
     if (more) load(s + 2 == slabs && ktail != 0);
     mfma_slab<LDR, LDC>(As[s & 1], Bs[s & 1], wm0, wn0, lane, acc);
-    if (more) stage((s + 1) & 1, sa == nblk, sb == mblk);
+    if (more) stage((s + 1) & 1, KEEP && sa == nblk, KEEP && sb == mblk);
     sa = sa + 1 == tiles_n ? 0 : sa + 1;
     sb = sb + 1 == tiles_m ? 0 : sb + 1;
     __syncthreads();
@@ -432,10 +434,10 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
                                            __builtin_fmaf(fast_log2(sv.z), kLn2, alr + be4.z),
                                            __builtin_fmaf(fast_log2(sv.w), kLn2, alr + be4.w));
              if (RAGGED) {
-               st4m(ws_r + u + voff, cc, rv);
+               if (KEEP) st4m(ws_r + u + voff, cc, rv);
                st4m(out + u + voff, cc, ov);
              } else {
-               st4(ws_r + u + voff, rv);
+               if (KEEP) st4(ws_r + u + voff, rv);
                st4(out + u + voff, ov);
              }
            });

@@ -19,8 +19,10 @@
  *     legacy default stream);
  *   - return value: 0 = enqueued; < 0 = argument error (GENBMM_E_*);
  *     > 0 = the hipError_t reported by the launch;
- *   - calls are re-entrant and thread safe: the library keeps no mutable global
- *     state, and a pointer declared const is only read.
+ *   - calls are re-entrant and thread safe: a pointer declared const is only
+ *     read, and the library keeps no mutable global state - except in
+ *     genbmm_logbmm_fwd_static, whose fixed workspace is shared by all calls on
+ *     a GPU (see there).
  *
  * Dense operands: a is (B, M, K), b is (B, K, N), results are (B, M, N).
  * Banded operands: band data is (B, n, W) with W = lu + ld + 1 and
@@ -42,6 +44,7 @@ extern "C" {
 #define GENBMM_E_SHAPE (-2)   /* a dimension is < 0 or overflows int32 */
 #define GENBMM_E_MODE (-3)    /* unknown semiring mode or kernel path  */
 #define GENBMM_E_BAND (-4)    /* negative band width                   */
+#define GENBMM_E_TOOBIG (-5)  /* beyond a fixed-size workspace's limit */
 
 /* Banded semiring modes (reference banded_cuda_kernel.cu:42,64,76). */
 #define GENBMM_BAND_LOG 0
@@ -126,6 +129,27 @@ int genbmm_logbmm_bwd_path(const float* a, const float* b, const float* out,
                            const float* g, const float* stats,
                            float* grad_a, float* grad_b,
                            int B, int M, int K, int N, int path, void* stream);
+
+/*
+ * genbmm_logbmm_fwd for callers that cannot allocate device memory - code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It
+ * has no counterpart in the reference.  The workspace that genbmm_logbmm_fwd takes
+ * as `stats` is a fixed array inside the library instead (4 MiB, one copy on every
+ * GPU the library runs on, held until the process ends), and nothing is kept for a
+ * backward: this is a forward for its own sake, on the same kernels, with results
+ * identical to genbmm_logbmm_fwd's.  No hipMalloc / hipFree inside, ever.
+ * Limit: B*(M+N) + B*ceil(M/32)*ceil(N/32) + 8 <= genbmm_logbmm_static_limit()
+ * (= 1048576 floats; the headline 64 x 512^3 needs 81928); beyond it the call
+ * returns GENBMM_E_TOOBIG and does nothing.
+ * Every call on a GPU uses that GPU's one array: calls that overlap in time on the
+ * same GPU (two streams, two threads) race on it - serialise them.  Nothing in the
+ * array needs clearing between calls (each call writes what it reads).  The first
+ * call on a device looks the array's address up (hipGetSymbolAddress, no stream
+ * work); make that call before starting a graph capture.
+ */
+int genbmm_logbmm_fwd_static(const float* a, const float* b, float* out,
+                             int B, int M, int K, int N, void* stream);
+size_t genbmm_logbmm_static_limit(void);
 
 /*
  * Second-order terms of logbmm: the gradients with respect to (a, b, g) of
