@@ -23,6 +23,7 @@
 #include "banded_argmax.h"
 #include "banded_mfma.h"
 #include "banded_max.h"
+#include "banded_stream.h"
 #include "banded_strip.h"
 
 namespace genbmm {
@@ -93,6 +94,48 @@ inline void launch_max_fwd(const BandArgs& p, int B, hipStream_t s) {
                      rows * p.Wa, rows * p.Wb);
 }
 
+// The streaming kernels (banded_stream.h): operands wide enough for 16 x 16 tiles and within
+// the registers that carry a block's new rows to LDS, tiles within a compute unit's LDS.
+// Rows per block: 64 if two such workgroups fit a compute unit, else 32 if two of those
+// do, else 64 with the compute unit to itself; 0: the band is not for these kernels.
+constexpr size_t kStreamLdsLimit = 160 * 1024;
+inline int stream_rows(int kind, const BandArgs& p) {
+  const int wp = kind == kStFwd ? p.Wa : p.Wo, wout = kind == kStFwd ? p.Wo : p.Wa;
+  if (min(p.Wa, p.Wb) < 8 || p.Wb > 95 || wp > (kind == kStFwd ? 95 : 191) || wout > 162) return 0;
+  auto fits = [&](int rows, int per_cu) {
+    const StreamDims d = stream_dims(kind, rows, p.Wa, p.Wb, p.Wo);
+    return (d.qr - rows) * d.qp <= 4 * 8 * rows * kSShift && d.bytes * per_cu <= kStreamLdsLimit;
+  };
+  if (fits(64, 2)) return 64;
+  if (fits(32, 2)) return 32;
+  return fits(64, 1) ? 64 : 0;
+}
+inline bool stream_ok(int kind, const BandArgs& p) { return stream_rows(kind, p) != 0; }
+
+template <int KIND, bool PREP, int ROWS>
+inline void launch_stream_rows(const BandArgs& p, int B, hipStream_t s, int fuse_h) {
+  const StreamDims d = stream_dims(KIND, ROWS, p.Wa, p.Wb, p.Wo);
+  // Runs: about as many workgroups as the chip holds at once (256 compute units, one or
+  // two workgroups each), runs of whole blocks.
+  const int per_cu = d.bytes * 2 <= kStreamLdsLimit ? 2 : 1;
+  const int blocks = ceil_div(p.n, ROWS);
+  int runs = (int)min((long)blocks, max(1L, (256L * per_cu + B - 1) / B));
+  const int run_rows = ceil_div(blocks, runs) * ROWS;
+  runs = ceil_div(p.n, run_rows);
+  auto kern = k_band_stream<KIND, PREP, ROWS>;
+  if (d.bytes > kStripLdsLimit)
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)d.bytes);
+  const long rows = (long)B * p.n;
+  hipLaunchKernelGGL(kern, dim3((unsigned)((long)B * runs)), dim3(8 * ROWS), d.bytes, s, p, d, runs, run_rows,
+                     rows * p.Wa, rows * p.Wb, rows * p.Wo, fuse_h);
+}
+template <int KIND, bool PREP>
+inline void launch_stream(const BandArgs& p, int B, hipStream_t s, int fuse_h = 0) {
+  if (stream_rows(KIND, p) == 32) launch_stream_rows<KIND, PREP, 32>(p, B, s, fuse_h);
+  else launch_stream_rows<KIND, PREP, 64>(p, B, s, fuse_h);
+}
+
 template <int KIND, bool PREP>
 inline void launch_mm(const BandArgs& p, int B, hipStream_t s, int fuse_h = 0) {
   const MmDims d = mm_dims(KIND, p.Wa, p.Wb, p.Wo);
@@ -153,9 +196,11 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
                          p.ws_al, p.Wa, a_lu, n, rows, lda);
       hipLaunchKernelGGL(k_band_prep, pg, dim3(256), sizeof(float) * kPrepRows * ldb, s, b, p.ws_eb,
                          p.ws_be, p.Wb, b_lu, n, rows, ldb);
-      launch_mm<kMmFwd, true>(p, B, s);
+      if (stream_ok(kStFwd, p)) launch_stream<kStFwd, true>(p, B, s);
+      else launch_mm<kMmFwd, true>(p, B, s);
     } else {
-      launch_mm<kMmFwd, false>(p, B, s);
+      if (stream_ok(kStFwd, p)) launch_stream<kStFwd, false>(p, B, s);
+      else launch_mm<kMmFwd, false>(p, B, s);
     }
     return launch_status();
   }
@@ -223,7 +268,8 @@ int banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int
   if (ta == 0) return GENBMM_OK;
   hipStream_t s = (hipStream_t)stream;
   if (mode == GENBMM_BAND_MUL && mm_bwd_ok(p)) {
-    launch_mm<kMmGradA, false>(p, B, s);
+    if (stream_ok(kStGradA, p)) launch_stream<kStGradA, false>(p, B, s);
+    else launch_mm<kMmGradA, false>(p, B, s);
     launch_mm<kMmGradB, false>(p, B, s);
     return launch_status();
   }
@@ -239,7 +285,8 @@ int banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int
       hipLaunchKernelGGL(k_band_h, dim3((unsigned)min((cells + 1023) / 1024, (long)0x7fffffff)), dim3(256), 0,
                          s, g, p.ws_r, p.ws_h, cells);
     }
-    launch_mm<kMmGradA, true>(p, B, s, fuse_h);
+    if (stream_ok(kStGradA, p)) launch_stream<kStGradA, true>(p, B, s, fuse_h);
+    else launch_mm<kMmGradA, true>(p, B, s, fuse_h);
     launch_mm<kMmGradB, true>(p, B, s);
     return launch_status();
   }

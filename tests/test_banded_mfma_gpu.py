@@ -183,3 +183,64 @@ def test_random_bands_max_product_bit_exact(gpu):
         ga, gb = torch.autograd.grad(res.data, (X.data, Y.data), g.to(gpu))
         wa, wb = oracle.seq_band_bwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, g.double(), 1, dtype=np.float64)
         assert torch.equal(ga.cpu().double(), wa) and torch.equal(gb.cpu().double(), wb), tag
+
+
+def _max_through_abi(gpu, ad, bd, a_lu, a_ld, b_lu, b_ld):
+    from genbmm_amd import _lib
+    lib = _lib.load()
+    B, n = ad.shape[0], ad.shape[1]
+    W = ad.shape[2] + bd.shape[2] - 1
+    out = torch.empty(B, n, W, device=gpu)
+    idx = torch.empty(B, n, W, dtype=torch.int32, device=gpu)
+    rc = lib.genbmm_banded_fwd(_lib.ptr(ad), a_lu, a_ld, _lib.ptr(bd), b_lu, b_ld, _lib.ptr(out), _lib.ptr(idx),
+                               _lib.ptr(None), B, n, 1, _lib.stream_of(ad))
+    assert rc == 0
+    return out, idx
+
+
+@pytest.mark.parametrize("shift", [1, 2, 3])
+def test_max_product_operands_off_the_16_byte_grid(gpu, shift):
+    """The whole-strip max-plus forward on operands that start 4, 8, 12 bytes past a 16-byte
+    boundary (its flat copy into LDS then has a lead), values and indices bit-exact."""
+    n, a_lu, a_ld, b_lu, b_ld = 150, 13, 14, 15, 12
+    torch.manual_seed(40 + shift)
+    grid = lambda *s: torch.round(torch.randn(*s) * 8) / 8
+    a = banddiag(grid(2, n, n), a_lu, a_ld)[0].contiguous()
+    b = banddiag(grid(2, n, n), b_lu, b_ld)[0].contiguous()
+    out, idx = _max_through_abi(gpu, offset_copy(a, gpu, shift), offset_copy(b, gpu, shift + 1), a_lu, a_ld, b_lu, b_ld)
+    want, widx, _ = oracle.seq_band_fwd(a, a_lu, a_ld, b, b_lu, b_ld, 1)
+    assert torch.equal(out.cpu(), want) and torch.equal(idx.cpu(), widx)
+
+
+def test_max_product_values_that_are_not_finite(gpu):
+    """+-inf and NaN operands next to the -inf padding between the staged rows of b: the same
+    cells become non-finite as in the oracle's walk, the same k wins everywhere (NaN never
+    wins a strict '>'; -inf + inf is NaN)."""
+    n, lu, ld = 200, 14, 15
+    torch.manual_seed(6)
+    a, b = pair(n, lu, ld, ld, lu)
+    a[0, 40, 3] = float("inf")
+    a[1, 101, 7] = float("nan")
+    b[0, 77, 20] = -float("inf")
+    b[1, 150, 0] = float("inf")
+    a[1, 30, :] = -float("inf")
+    for shift in (0, 1):
+        ad = offset_copy(a, gpu, shift) if shift else a.to(gpu)
+        out, idx = _max_through_abi(gpu, ad, b.to(gpu), lu, ld, ld, lu)
+        want, widx, _ = oracle.seq_band_fwd(a, lu, ld, b, ld, lu, 1)
+        assert torch.equal(out.cpu().view(torch.int32), want.view(torch.int32))
+        assert torch.equal(idx.cpu(), widx)
+
+
+@pytest.mark.parametrize("n,a_lu,a_ld,b_lu,b_ld", [(700, 75, 74, 4, 3), (513, 60, 60, 12, 12), (330, 0, 139, 10, 0)])
+def test_max_product_on_the_widest_whole_strip_bands(gpu, n, a_lu, a_ld, b_lu, b_ld):
+    """Result bands of 145 to 157 diagonals (twenty blocks of eight per row, the fifth block
+    of the waves in use; a wide first operand against a narrow second keeps the tiles within
+    the kernel's LDS budget) on matrices long enough for interior strips."""
+    torch.manual_seed(n)
+    grid = lambda *s: torch.round(torch.randn(*s) * 8) / 8
+    a = banddiag(grid(2, n, n), a_lu, a_ld)[0].contiguous()
+    b = banddiag(grid(2, n, n), b_lu, b_ld)[0].contiguous()
+    out, idx = _max_through_abi(gpu, a.to(gpu), b.to(gpu), a_lu, a_ld, b_lu, b_ld)
+    want, widx, _ = oracle.seq_band_fwd(a, a_lu, a_ld, b, b_lu, b_ld, 1)
+    assert torch.equal(out.cpu(), want) and torch.equal(idx.cpu(), widx)
