@@ -35,6 +35,13 @@ HIPCC_FLAGS = [
 ]
 
 
+# Per-source additions.  The banded kernels keep their 16 x 16 accumulators in ordinary vector
+# registers: a tile's four values are read by vector instructions right after its last matrix
+# instruction, and copies to and from the accumulation registers around every step cost
+# more than the registers they free.
+EXTRA_FLAGS = {"banded.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
 def lib_path():
     return os.path.join(LIBDIR, LIBNAME)
 
@@ -55,7 +62,7 @@ def build(verbose=True):
     procs = []
     for src in SOURCES:
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        cmd = [cc] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [cc] + HIPCC_FLAGS + EXTRA_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, obj, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))

@@ -21,6 +21,7 @@
 #include <type_traits>
 
 #include "banded_argmax.h"
+#include "banded_direct.h"
 #include "banded_mfma.h"
 #include "banded_max.h"
 #include "banded_stream.h"
@@ -136,6 +137,24 @@ inline void launch_stream(const BandArgs& p, int B, hipStream_t s, int fuse_h = 
   else launch_stream_rows<KIND, PREP, 64>(p, B, s, fuse_h);
 }
 
+// The memory-fed forward (banded_direct.h): at most 16 tiles per tile row and 6 chunks of the
+// first operand, offsets inside a batch item within 32 bits.
+inline bool dir_fwd_ok(const BandArgs& p) {
+  DirPlan plan;
+  return min(p.Wa, p.Wb) >= 8 && (long)p.n * p.Wo < (1L << 30) && dir_plan(plan, p.a_lu, p.Wa, p.b_lu, p.Wb, p.r_lu, p.Wo);
+}
+template <bool PREP>
+inline void launch_dir_fwd(const BandArgs& p, int B, hipStream_t s) {
+  const int blocks = ceil_div(p.n, 16 * kDirWaves);
+  const int nblocks = B * blocks;
+  const long rows = (long)B * p.n;
+  const int wave_lds = dir_wave_lds(p.Wa, p.Wo, PREP);
+  DirPlan plan;
+  dir_plan(plan, p.a_lu, p.Wa, p.b_lu, p.Wb, p.r_lu, p.Wo);
+  hipLaunchKernelGGL(k_band_dir_fwd<PREP>, dim3((unsigned)nblocks), dim3(64 * kDirWaves), kDirWaves * wave_lds, s, p, plan, blocks,
+                     nblocks, rows * p.Wa, rows * p.Wb, wave_lds);
+}
+
 template <int KIND, bool PREP>
 inline void launch_mm(const BandArgs& p, int B, hipStream_t s, int fuse_h = 0) {
   const MmDims d = mm_dims(KIND, p.Wa, p.Wb, p.Wo);
@@ -196,10 +215,12 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
                          p.ws_al, p.Wa, a_lu, n, rows, lda);
       hipLaunchKernelGGL(k_band_prep, pg, dim3(256), sizeof(float) * kPrepRows * ldb, s, b, p.ws_eb,
                          p.ws_be, p.Wb, b_lu, n, rows, ldb);
-      if (stream_ok(kStFwd, p)) launch_stream<kStFwd, true>(p, B, s);
+      if (dir_fwd_ok(p)) launch_dir_fwd<true>(p, B, s);
+      else if (stream_ok(kStFwd, p)) launch_stream<kStFwd, true>(p, B, s);
       else launch_mm<kMmFwd, true>(p, B, s);
     } else {
-      if (stream_ok(kStFwd, p)) launch_stream<kStFwd, false>(p, B, s);
+      if (dir_fwd_ok(p)) launch_dir_fwd<false>(p, B, s);
+      else if (stream_ok(kStFwd, p)) launch_stream<kStFwd, false>(p, B, s);
       else launch_mm<kMmFwd, false>(p, B, s);
     }
     return launch_status();
