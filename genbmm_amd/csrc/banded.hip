@@ -64,11 +64,17 @@ inline bool mm_bwd_ok(const BandArgs& p) {
   return mm_tiles_ok(p.Wa, p.Wb, p.Wo) && min(p.Wa, p.Wb) >= 25 &&
          max(mm_dims(kMmGradA, p.Wa, p.Wb, p.Wo).bytes, mm_dims(kMmGradB, p.Wa, p.Wb, p.Wo).bytes) <= kMmLdsLimit;
 }
+// The memory-fed forward (banded_direct.h): at most 16 tiles per tile row and 6 chunks of the
+// first operand, offsets inside a batch item within 32 bits.
+inline bool dir_fwd_ok(const BandArgs& p) {
+  DirPlan plan;
+  return min(p.Wa, p.Wb) >= 8 && (long)p.n * p.Wo < (1L << 30) && dir_plan(plan, p.a_lu, p.Wa, p.b_lu, p.Wb, p.r_lu, p.Wo);
+}
 // The workspace of the log product is filled and used only when both directions have a
 // kernel that works on it (matrix-core or strip), so that forward and backward always agree
 // on whether it holds anything.
 inline bool workspace_used(const BandArgs& p) {
-  const bool fwd = mm_fwd_ok(p, 4) ||
+  const bool fwd = dir_fwd_ok(p) || mm_fwd_ok(p, 4) ||
                    (fwd_strip_ok(p) &&
                     strip_dims(p.Wa, p.Wb).bytes + sizeof(float) * (kBT + p.Wo + kBJ) <= kStripLdsLimit);
   return fwd && (mm_bwd_ok(p) || bwd_strip_ok(p));
@@ -111,7 +117,12 @@ inline int stream_rows(int kind, const BandArgs& p) {
   if (fits(32, 2)) return 32;
   return fits(64, 1) ? 64 : 0;
 }
-inline bool stream_ok(int kind, const BandArgs& p) { return stream_rows(kind, p) != 0; }
+// grad_a as a stream pays from about 57 diagonals on (measured at 64 x 4096 against the
+// strip-owning matrix-core kernel, whole backward: 33 diagonals 0.171 ms against 0.166, 49:
+// 0.214 against 0.201, 65: 0.326 against 0.387)
+inline bool stream_ok(int kind, const BandArgs& p) {
+  return stream_rows(kind, p) != 0 && (kind == kStFwd || min(p.Wa, p.Wb) >= 57);
+}
 
 template <int KIND, bool PREP, int ROWS>
 inline void launch_stream_rows(const BandArgs& p, int B, hipStream_t s, int fuse_h) {
@@ -137,12 +148,6 @@ inline void launch_stream(const BandArgs& p, int B, hipStream_t s, int fuse_h = 
   else launch_stream_rows<KIND, PREP, 64>(p, B, s, fuse_h);
 }
 
-// The memory-fed forward (banded_direct.h): at most 16 tiles per tile row and 6 chunks of the
-// first operand, offsets inside a batch item within 32 bits.
-inline bool dir_fwd_ok(const BandArgs& p) {
-  DirPlan plan;
-  return min(p.Wa, p.Wb) >= 8 && (long)p.n * p.Wo < (1L << 30) && dir_plan(plan, p.a_lu, p.Wa, p.b_lu, p.Wb, p.r_lu, p.Wo);
-}
 template <bool PREP>
 inline void launch_dir_fwd(const BandArgs& p, int B, hipStream_t s) {
   const int blocks = ceil_div(p.n, 16 * kDirWaves);
@@ -151,6 +156,9 @@ inline void launch_dir_fwd(const BandArgs& p, int B, hipStream_t s) {
   const int wave_lds = dir_wave_lds(p.Wa, p.Wo, PREP);
   DirPlan plan;
   dir_plan(plan, p.a_lu, p.Wa, p.b_lu, p.Wb, p.r_lu, p.Wo);
+  if ((size_t)kDirWaves * wave_lds > kStripLdsLimit)
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_band_dir_fwd<PREP>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kDirWaves * wave_lds);
   hipLaunchKernelGGL(k_band_dir_fwd<PREP>, dim3((unsigned)nblocks), dim3(64 * kDirWaves), kDirWaves * wave_lds, s, p, plan, blocks,
                      nblocks, rows * p.Wa, rows * p.Wb, wave_lds);
 }
@@ -205,7 +213,8 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   if (total == 0) return GENBMM_OK;
   hipStream_t s = (hipStream_t)stream;
   const StripDims sd = strip_dims(p.Wa, p.Wb);
-  if ((mode == GENBMM_BAND_MUL && mm_fwd_ok(p)) || (prep_fwd(p, mode, workspace) && mm_fwd_ok(p, 4))) {
+  const bool dir = dir_fwd_ok(p);
+  if ((mode == GENBMM_BAND_MUL && (dir || mm_fwd_ok(p))) || (prep_fwd(p, mode, workspace) && (dir || mm_fwd_ok(p, 4)))) {
     if (mode == GENBMM_BAND_LOG) {
       set_workspace(p, workspace, B);
       const long rows = (long)B * n;
@@ -215,11 +224,11 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
                          p.ws_al, p.Wa, a_lu, n, rows, lda);
       hipLaunchKernelGGL(k_band_prep, pg, dim3(256), sizeof(float) * kPrepRows * ldb, s, b, p.ws_eb,
                          p.ws_be, p.Wb, b_lu, n, rows, ldb);
-      if (dir_fwd_ok(p)) launch_dir_fwd<true>(p, B, s);
+      if (dir) launch_dir_fwd<true>(p, B, s);
       else if (stream_ok(kStFwd, p)) launch_stream<kStFwd, true>(p, B, s);
       else launch_mm<kMmFwd, true>(p, B, s);
     } else {
-      if (dir_fwd_ok(p)) launch_dir_fwd<false>(p, B, s);
+      if (dir) launch_dir_fwd<false>(p, B, s);
       else if (stream_ok(kStFwd, p)) launch_stream<kStFwd, false>(p, B, s);
       else launch_mm<kMmFwd, false>(p, B, s);
     }
