@@ -64,11 +64,22 @@ inline bool mm_bwd_ok(const BandArgs& p) {
   return mm_tiles_ok(p.Wa, p.Wb, p.Wo) && min(p.Wa, p.Wb) >= 25 &&
          max(mm_dims(kMmGradA, p.Wa, p.Wb, p.Wo).bytes, mm_dims(kMmGradB, p.Wa, p.Wb, p.Wo).bytes) <= kMmLdsLimit;
 }
-// The memory-fed forward (banded_direct.h): at most 16 tiles per tile row and 6 chunks of the
-// first operand, offsets inside a batch item within 32 bits.
-inline bool dir_fwd_ok(const BandArgs& p) {
+// The memory-fed kernels (banded_direct.h): a plan within their limits, offsets inside a
+// batch item within 32 bits.
+inline bool dir_ok(int kind, const BandArgs& p, int min_w) {
   DirPlan plan;
-  return min(p.Wa, p.Wb) >= 8 && (long)p.n * p.Wo < (1L << 30) && dir_plan(plan, p.a_lu, p.Wa, p.b_lu, p.Wb, p.r_lu, p.Wo);
+  return min(p.Wa, p.Wb) >= min_w && (long)p.n * p.Wo < (1L << 30) &&
+         dir_plan(plan, kind, p.a_lu, p.Wa, p.b_lu, p.Wb);
+}
+// From 3 diagonals on, except the forward of the plain product, which one lane per cell does
+// faster below 7 (measured at 64 x 4096, memory-fed against what it replaces: 3 diagonals plain
+// forward 0.020 ms against 0.009, backward 0.044 against 0.074, log forward with its
+// preparation 0.043 against 0.011 without a workspace, log backward 0.060 against 0.219; 7
+// diagonals plain forward 0.020 against 0.023).
+constexpr int kDirMinW = 3, kDirMinWPlainFwd = 7;
+inline bool dir_fwd_ok(const BandArgs& p, int min_w = kDirMinW) { return dir_ok(kDirFwd, p, min_w); }
+inline bool dir_bwd_ok(const BandArgs& p) {
+  return dir_ok(kDirGradA, p, kDirMinW) && dir_ok(kDirGradB, p, kDirMinW);
 }
 // The workspace of the log product is filled and used only when both directions have a
 // kernel that works on it (matrix-core or strip), so that forward and backward always agree
@@ -77,7 +88,7 @@ inline bool workspace_used(const BandArgs& p) {
   const bool fwd = dir_fwd_ok(p) || mm_fwd_ok(p, 4) ||
                    (fwd_strip_ok(p) &&
                     strip_dims(p.Wa, p.Wb).bytes + sizeof(float) * (kBT + p.Wo + kBJ) <= kStripLdsLimit);
-  return fwd && (mm_bwd_ok(p) || bwd_strip_ok(p));
+  return fwd && (dir_bwd_ok(p) || mm_bwd_ok(p) || bwd_strip_ok(p));
 }
 
 inline bool prep_fwd(const BandArgs& p, int mode, const float* workspace) {
@@ -148,19 +159,19 @@ inline void launch_stream(const BandArgs& p, int B, hipStream_t s, int fuse_h = 
   else launch_stream_rows<KIND, PREP, 64>(p, B, s, fuse_h);
 }
 
-template <bool PREP>
-inline void launch_dir_fwd(const BandArgs& p, int B, hipStream_t s) {
+template <int KIND, bool PREP>
+inline void launch_dir(const BandArgs& p, int B, hipStream_t s) {
   const int blocks = ceil_div(p.n, 16 * kDirWaves);
   const int nblocks = B * blocks;
-  const long rows = (long)B * p.n;
-  const int wave_lds = dir_wave_lds(p.Wa, p.Wo, PREP);
   DirPlan plan;
-  dir_plan(plan, p.a_lu, p.Wa, p.b_lu, p.Wb, p.r_lu, p.Wo);
+  dir_plan(plan, KIND, p.a_lu, p.Wa, p.b_lu, p.Wb);
+  const int wave_lds = dir_wave_lds(plan, KIND, PREP);
+  auto kern = k_band_dir<KIND, PREP>;
   if ((size_t)kDirWaves * wave_lds > kStripLdsLimit)
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_band_dir_fwd<PREP>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, kDirWaves * wave_lds);
-  hipLaunchKernelGGL(k_band_dir_fwd<PREP>, dim3((unsigned)nblocks), dim3(64 * kDirWaves), kDirWaves * wave_lds, s, p, plan, blocks,
-                     nblocks, rows * p.Wa, rows * p.Wb, wave_lds);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              kDirWaves * wave_lds);
+  hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64 * kDirWaves), kDirWaves * wave_lds, s, p, plan, blocks,
+                     nblocks, (long)B * p.n, wave_lds);
 }
 
 template <int KIND, bool PREP>
@@ -213,7 +224,7 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   if (total == 0) return GENBMM_OK;
   hipStream_t s = (hipStream_t)stream;
   const StripDims sd = strip_dims(p.Wa, p.Wb);
-  const bool dir = dir_fwd_ok(p);
+  const bool dir = dir_fwd_ok(p, mode == GENBMM_BAND_MUL ? kDirMinWPlainFwd : kDirMinW);
   if ((mode == GENBMM_BAND_MUL && (dir || mm_fwd_ok(p))) || (prep_fwd(p, mode, workspace) && (dir || mm_fwd_ok(p, 4)))) {
     if (mode == GENBMM_BAND_LOG) {
       set_workspace(p, workspace, B);
@@ -224,11 +235,11 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
                          p.ws_al, p.Wa, a_lu, n, rows, lda);
       hipLaunchKernelGGL(k_band_prep, pg, dim3(256), sizeof(float) * kPrepRows * ldb, s, b, p.ws_eb,
                          p.ws_be, p.Wb, b_lu, n, rows, ldb);
-      if (dir) launch_dir_fwd<true>(p, B, s);
+      if (dir) launch_dir<kDirFwd, true>(p, B, s);
       else if (stream_ok(kStFwd, p)) launch_stream<kStFwd, true>(p, B, s);
       else launch_mm<kMmFwd, true>(p, B, s);
     } else {
-      if (dir) launch_dir_fwd<false>(p, B, s);
+      if (dir) launch_dir<kDirFwd, false>(p, B, s);
       else if (stream_ok(kStFwd, p)) launch_stream<kStFwd, false>(p, B, s);
       else launch_mm<kMmFwd, false>(p, B, s);
     }
@@ -297,6 +308,17 @@ int banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int
   const long ta = (long)B * n * p.Wa, tb = (long)B * n * p.Wb;
   if (ta == 0) return GENBMM_OK;
   hipStream_t s = (hipStream_t)stream;
+  if (mode != GENBMM_BAND_MAX && (mode == GENBMM_BAND_MUL || (workspace && workspace_used(p))) && dir_bwd_ok(p)) {
+    if (mode == GENBMM_BAND_MUL) {
+      launch_dir<kDirGradA, false>(p, B, s);
+      launch_dir<kDirGradB, false>(p, B, s);
+    } else {  // H = g / S is formed by both kernels as they read g: the workspace is only read
+      set_workspace(p, workspace, B);
+      launch_dir<kDirGradA, true>(p, B, s);
+      launch_dir<kDirGradB, true>(p, B, s);
+    }
+    return launch_status();
+  }
   if (mode == GENBMM_BAND_MUL && mm_bwd_ok(p)) {
     if (stream_ok(kStGradA, p)) launch_stream<kStGradA, false>(p, B, s);
     else launch_mm<kMmGradA, false>(p, B, s);

@@ -1,21 +1,33 @@
-// Banded (+,*) forward on the matrix cores, operands fed from memory: no operand tiles
-// shared through LDS, no barrier.
+// Banded (+,*) products on the matrix cores, operands fed from memory: forward, grad_a and
+// grad_b of the plain product and of the log product on the forward's workspace.  No
+// operand tiles shared through LDS, no barrier.
 //
-// Dense coordinates as in banded_mfma.h: C[x, y] = sum_z P(x, z) Q(z, y) with
-// P(x, z) = a[x][z - x + lu_a] and Q(z, y) = b[y][z - y + lu_b], 16 x 16 tiles of (x, y).
-// One wave owns a tile row (16 rows x) and walks its tiles along y; waves never meet.
+// Dense coordinates as in banded_mfma.h.  Each of the three is C[i, j] = sum_k P(i, k) Q(k, j)
+// cut into 16 x 16 tiles of (i, j); one wave owns a tile row (16 rows i) and walks its
+// tiles along j; waves never meet.
 //
-// v_mfma_f32_16x16x4_f32 sums over four values of z; which four is free as long as both
+//   forward  i = x, k = z, j = y   P = a[x][z - x + lu_a]    Q = b[y][z - y + lu_b]   -> out[x][y - x + lu_o]
+//   grad_a   i = x, k = y, j = z   P = g[x][y - x + lu_o]    Q = b[y][z - y + lu_b]   -> ga[x][z - x + lu_a]
+//   grad_b   i = y, k = x, j = z   P = g[x][y - x + lu_o]    Q = a[x][z - x + lu_a]   -> gb[y][z - y + lu_b]
+//
+// v_mfma_f32_16x16x4_f32 sums over four values of k; which four is free as long as both
 // operands agree.  Here lane (l15, zq) feeds, in the t-th of four consecutive
-// instructions, z = Z + 4 zq + t: the four values a lane needs for the four
-// instructions are four neighbouring cells of its band row, for P (lane l15 is row x)
-// and for Q (lane l15 is row y of b) alike.  A chunk of 16 z is thus 64 contiguous
-// bytes of each of 16 band rows: it is read by one 16-byte load per lane (4-byte
-// aligned) with four neighbouring lanes on one row - which the memory pipeline takes as
-// one access per row - and the cells then change lanes to where the instruction wants
-// them: P once per tile row through the wave's own piece of LDS, Q by ds_bpermute.
+// instructions, k = K + 4 zq + t, for a chunk of 16 k starting at K.  An operand is read
+// in one of two ways:
 //
-// z runs on a grid of such chunks that starts at x0 - lu_a for the tile row at x0.  A
+//  * its band row is the operand's own row or column (l15) and k runs along the row (a
+//    and b in the forward, g in grad_a): the four values a lane needs are four
+//    neighbouring cells, and a chunk is 64 contiguous bytes of each of 16 band rows.  It
+//    is read by one 16-byte load per lane (4-byte aligned) with four neighbouring
+//    lanes on one row - which the memory pipeline takes as one access per row - and
+//    the cells then change lanes to where the instruction wants them (ds_bpermute for
+//    Q; P goes through the wave's own piece of LDS anyway).
+//  * its band row is k (b in grad_a, g and a in grad_b): 16 lanes l15 read 16
+//    neighbouring cells of row k - four 4-byte loads per lane for the four k, each
+//    already in the lane that feeds it.
+//
+// k runs on a grid of chunks that starts at the first k the tile row's P can meet.  The
+// wave puts its NU chunks of P into LDS once, laid out as the instruction reads them.  A
 // tile uses the chunks that its cells can meet; the (tile, chunk) pairs of a tile row
 // form one list, the same for every tile row of a product, which the host writes once
 // and the wave walks with the loads of Q four pairs ahead of the instructions.  Every
@@ -26,11 +38,16 @@
 // matrix, or whose loads could leave the tensors, read cell by cell from addresses held
 // inside the tensor and test every cell (EDGE).
 //
-// A result that is not finite (an operand that is not, against a zero of the padding),
-// and in the prepared log product a sum outside the guard, is noted per lane or per cell
-// and recomputed from memory by the per-cell routine once the tile row is done.
+// The log product on the forward's workspace: the forward multiplies EA and EB and takes
+// the logarithm per cell (and leaves 1/S); the gradients form H = g / S while they read g
+// and multiply the sums by EA / EB on the way out.
 //
-// Measured at 64 x 4096 with 65 diagonals the kernel issues about 1 700 instructions per
+// A result that is not finite (an operand that is not, against a zero of the padding; an
+// H that is marked unusable), and in the forward of the log product a sum outside the
+// guard, is noted per lane or per cell and recomputed from memory by the per-cell
+// routine once the tile row is done.
+//
+// Measured at 64 x 4096 with 65 diagonals the forward issues about 1 700 instructions per
 // tile row for its 100 matrix instructions and is bound by that count (a SIMD of this
 // chip issues one instruction of any kind about every 4.4 cycles and nothing beside a
 // matrix instruction's 32).
@@ -42,207 +59,273 @@
 
 namespace genbmm {
 
+constexpr int kDirFwd = 0, kDirGradA = 1, kDirGradB = 2;
 constexpr int kDirTiles = 16;   // tiles per tile row, at most (a bit per cell in 64 bits)
-constexpr int kDirChunks = 6;   // chunks of the first operand per tile row, at most
-constexpr int kDirDepth = 4;    // pairs whose loads are in flight
+constexpr int kDirChunks = 12;  // chunks of the first operand per tile row, at most
+constexpr int kDirDepth = 4;    // pairs whose loads of Q are in flight
+constexpr int kDirWaves = 2;    // waves (tile rows) per workgroup
+constexpr int kDirMargin = 48;  // floats a load can stray from the band rows it is meant for
 typedef float dir_f4u __attribute__((ext_vector_type(4), aligned(4)));
 
-constexpr int kDirWaves = 2;    // waves (tile rows) per workgroup
-
-inline int dir_chunks(int Wp) { return (Wp + 30) >> 4; }  // chunks of 16 z that a tile row's P meets
-// LDS of one wave: its chunks of P and one of zeros, 1 KB each; then the row maxima of b for
-// its tiles (prepared log product) or the tile row's results (plain product), which then
-// leave as one contiguous run of memory
-inline int dir_wave_lds(int Wa, int Wo, bool prep) {
-  return (dir_chunks(Wa) + 1) * 1024 + (prep ? 64 * ((Wo + 30) >> 4) : 64 * Wo);
-}
-
-// The walk over a tile row's (tile, chunk) pairs is the same for every tile row of a
-// product: the host lists it once.  One word per step:
-//   bits 0-11  (ty (Wb - 1) + u): where the pair's cells of Q start, in units of 16 floats
-//   bits 12-14 chunk of P (the one past the last holds zeros)
-//   bits 15-18 tile ty          bit 19  the tile is complete after this step
-//   bit 20 / 21  some lane's cells lie past the upper / lower end of the band of b
-//   bits 22-26 (u - ty) + 16    bit 27  a filling step (nothing to multiply)
-//   (bit 21: u - ty is the plan's lowest, bit 28: the one above it)
-//   bit 29  every cell of the tile is inside the result band
-// and beside it the word of the step kDirDepth further on, whose cells of Q are asked for now.
-constexpr int kDirSteps = 64;
+// The walk over a tile row's (tile, chunk) pairs.  One word per step:
+//   bits 0-11  where the pair's cells of Q start, in units of 16 floats
+//   bits 12-15 chunk of P (the one past the last holds zeros)
+//   bits 16-19 tile      bit 20  the tile is complete after this step
+//   bit 21  some lane's cells of Q lie past the upper end of its band (D = 0)
+//   bit 22 / 23  ... below the lower end: D is the plan's lowest / the one above it
+//   bit 24  a filling step (nothing to multiply)
+//   bit 25  every cell of the tile is inside the result band
+// (D: chunk minus tile, or tile minus chunk for an operand whose band row is k; a lane's
+// cell t of Q is Wq - 1 + 16 D + s_t with s_t in [-15, 15]), and beside it the word of
+// the step kDirDepth further on, whose cells of Q are asked for now.
+constexpr int kDirSteps = 72;
 struct DirStep {
   unsigned now, ahead;
 };
 struct DirPlan {
   int steps;  // a multiple of kDirDepth
-  int d_lo;   // the lowest u - ty of the plan
+  int d_lo;   // the lowest D of the plan
+  int Wp, Wq, Wout;
+  int plo, phi;  // P(i, k) is inside its band for k in [i - plo, i + phi]
+  int lu_out;    // out[i][j - i + lu_out]
+  int NU, nt;    // chunks of P, tiles per tile row
   DirStep e[kDirSteps + 1];
 };
 
-inline bool dir_plan(DirPlan& plan, int a_lu, int Wa, int b_lu, int Wb, int r_lu, int Wo) {
-  const int NU = dir_chunks(Wa), ny = (Wo + 30) >> 4;
+inline int dir_chunks(int Wp) { return (Wp + 30) >> 4; }  // chunks of 16 k that a tile row's P meets
+// LDS of one wave: its chunks of P and one of zeros, 1 KB each; then the row maxima of b for
+// its tiles (forward of the log product) or the tile row's results (all others), which then
+// leave as one contiguous run of memory
+inline int dir_wave_lds(const DirPlan& g, int kind, bool prep) {
+  return (g.NU + 1) * 1024 + (kind == kDirFwd && prep ? 64 * g.nt : 64 * g.Wout);
+}
+
+inline bool dir_plan(DirPlan& g, int kind, int a_lu, int Wa, int b_lu, int Wb) {
   const int a_ld = Wa - 1 - a_lu, b_ld = Wb - 1 - b_lu;
-  if (NU > kDirChunks || ny > kDirTiles || 15 * (Wb - 1) + NU >= 4096) return false;
+  const int Wo = Wa + Wb - 1, r_lu = a_lu + b_ld, r_ld = Wo - 1 - r_lu;
+  int qlo, qhi;  // Q(k, j) is inside its band for k in [j - qlo, j + qhi]
+  if (kind == kDirFwd) {
+    g.Wp = Wa; g.Wq = Wb; g.Wout = Wo; g.plo = a_lu; g.phi = a_ld; g.lu_out = r_lu; qlo = b_lu; qhi = b_ld;
+  } else if (kind == kDirGradA) {
+    g.Wp = Wo; g.Wq = Wb; g.Wout = Wa; g.plo = r_lu; g.phi = r_ld; g.lu_out = a_lu; qlo = b_ld; qhi = b_lu;
+  } else {
+    g.Wp = Wo; g.Wq = Wa; g.Wout = Wb; g.plo = r_ld; g.phi = r_lu; g.lu_out = b_lu; qlo = a_ld; qhi = a_lu;
+  }
+  const bool qrow = kind != kDirFwd;
+  const int NU = g.NU = dir_chunks(g.Wp), nt = g.nt = (g.Wout + 30) >> 4;
+  if (NU > kDirChunks || nt > kDirTiles || max(NU, nt) * g.Wq >= 4096) return false;
   unsigned list[kDirTiles * kDirChunks];
   int np = 0, d_lo = 0;
-  for (int ty = 0; ty < ny; ++ty) {
-    const int dlo = max(-a_lu, 16 * ty - r_lu - b_lu);
-    const int ulo = min(NU - 1, (dlo + a_lu) >> 4);
-    d_lo = min(d_lo, ulo - ty);
-  }
-  plan.d_lo = d_lo;
-  for (int ty = 0; ty < ny; ++ty) {
-    // the tile's z relative to x0 in [dlo, dhi]; chunk u covers [16 u - lu_a, 16 u - lu_a + 15].  A
-    // tile whose cells meet no z gets one chunk all the same (every product then has a zero
-    // of the band masks in it).
-    const int dlo = max(-a_lu, 16 * ty - r_lu - b_lu);
-    const int dhi = min(15 + a_ld, 16 * ty - r_lu + 15 + b_ld);
-    const int ulo = min(NU - 1, (dlo + a_lu) >> 4);
-    const int uhi = max(ulo, min(NU - 1, (dhi + a_lu) >> 4));
-    for (int u = ulo; u <= uhi; ++u) {
-      const int d = u - ty;
-      if (d + 16 < 0 || d + 16 > 31) return false;
-      // below the lower end: only the plan's lowest two u - ty can be (30 cells apart at most)
-      const unsigned hi = d >= 0, lo = 16 * d < 16 - Wb;
-      if (d > 0 || (lo && d > d_lo + 1)) return false;
-      const unsigned whole = 16 * ty - 15 >= 0 && 16 * ty + 15 < Wo;
-      list[np++] = (unsigned)(ty * (Wb - 1) + u) | (unsigned)u << 12 | (unsigned)ty << 15 |
-                   (unsigned)(u == uhi) << 19 | hi << 20 | (unsigned)(lo && d == d_lo) << 21 |
-                   (unsigned)(d + 16) << 22 | (unsigned)(lo && d == d_lo + 1) << 28 | whole << 29;
+  for (int pass = 0; pass < 2; ++pass) {
+    np = 0;
+    for (int tj = 0; tj < nt; ++tj) {
+      // the tile's k relative to i0 in [dlo, dhi]; chunk u covers [16 u - plo, 16 u - plo + 15].  A
+      // tile whose cells meet no k gets one chunk all the same (every product then has a zero
+      // of the band masks in it).
+      const int dlo = max(-g.plo, 16 * tj - g.lu_out - qlo);
+      const int dhi = min(15 + g.phi, 16 * tj - g.lu_out + 15 + qhi);
+      const int ulo = min(NU - 1, max(0, (dlo + g.plo) >> 4));
+      const int uhi = max(ulo, min(NU - 1, (dhi + g.plo) >> 4));
+      for (int u = ulo; u <= uhi; ++u) {
+        const int d = qrow ? tj - u : u - tj;
+        if (pass == 0) {
+          d_lo = min(d_lo, d);
+          continue;
+        }
+        // past the upper end only for D = 0, below the lower end only for the lowest two D (a
+        // lane's cells of one chunk are at most 30 apart)
+        const unsigned hi = d >= 0, lo = 16 * d < 16 - g.Wq;
+        if (d > 0 || (lo && d > d_lo + 1)) return false;
+        const unsigned whole = 16 * tj - 15 >= 0 && 16 * tj + 15 < g.Wout;
+        const int q16 = qrow ? u * (g.Wq - 1) + tj : tj * (g.Wq - 1) + u;
+        list[np++] = (unsigned)q16 | (unsigned)u << 12 | (unsigned)tj << 16 | (unsigned)(u == uhi) << 20 | hi << 21 |
+                     (unsigned)(lo && d == d_lo) << 22 | (unsigned)(lo && d == d_lo + 1) << 23 | whole << 25;
+      }
     }
   }
+  g.d_lo = d_lo;
   const int pad = (kDirDepth - (np & (kDirDepth - 1))) & (kDirDepth - 1);
   if (np + pad > kDirSteps) return false;
-  plan.steps = np + pad;
-  for (int i = 0; i < pad; ++i)
-    plan.e[i].now = (list[0] & 0xfffu) | (unsigned)NU << 12 | (list[0] & (31u << 22)) | 1u << 27;
-  for (int i = 0; i < np; ++i) plan.e[pad + i].now = list[i];
-  plan.e[plan.steps].now = plan.e[plan.steps - 1].now;
-  for (int i = 0; i <= plan.steps; ++i) plan.e[i].ahead = plan.e[min(i + kDirDepth, plan.steps - 1)].now;
+  g.steps = np + pad;
+  for (int i = 0; i < pad; ++i) g.e[i].now = (list[0] & 0xfffu) | (unsigned)NU << 12 | 1u << 24;
+  for (int i = 0; i < np; ++i) g.e[pad + i].now = list[i];
+  g.e[g.steps].now = g.e[g.steps - 1].now;
+  for (int i = 0; i <= g.steps; ++i) g.e[i].ahead = g.e[min(i + kDirDepth, g.steps - 1)].now;
   return true;
 }
 
 // One tile row.  All arguments but `lane` are uniform.  lds: this wave's piece.
-template <bool PREP, bool EDGE>
-__device__ __forceinline__ void dir_fwd_row(const BandArgs& p, const DirPlan& plan, long bn, int x0, int lane,
-                                            float* lds, long cells_a, long cells_b) {
-  const int n = p.n, Wa = p.Wa, Wb = p.Wb, Wo = p.Wo, r_lu = p.r_lu, a_lu = p.a_lu;
-  const int NU = (Wa + 30) >> 4, ny = (Wo + 30) >> 4;
+template <int KIND, bool PREP, bool EDGE>
+__device__ __forceinline__ void dir_row(const BandArgs& p, const DirPlan& g, long bn, int i0, int lane, float* lds,
+                                        long rows) {
+  constexpr bool FWD = KIND == kDirFwd, GA = KIND == kDirGradA;
+  constexpr bool PROW = KIND == kDirGradB;  // P's band row is k
+  constexpr bool QROW = KIND != kDirFwd;    // Q's band row is k
+  constexpr bool MKH = PREP && !FWD;        // P = g / S, formed while it is read
+  constexpr bool STAGE = !EDGE && !(FWD && PREP);
+  const int n = p.n, Wp = g.Wp, Wq = g.Wq, Wout = g.Wout, NU = g.NU, nt = g.nt;
   const int l15 = lane & 15, zq = lane >> 4;
-  // loading lane 4 r + c: row r, cells 4 c .. 4 c + 3 of the chunk; the instruction wants
-  // them in lane 16 c + r
+  // a lane that loads 16 bytes: lane 4 r + c takes row r, cells 4 c .. 4 c + 3 of the chunk; the
+  // instruction wants them in lane 16 c + r
   const int lr = lane >> 2, lc = lane & 3;
   const int from = 4 * (4 * l15 + zq);  // byte index of the lane this one takes its cells from
-  const int y0 = x0 - r_lu;             // first column of tile 0
-  const float* at = PREP ? p.ws_ea : p.a;
-  const float* bt = PREP ? p.ws_eb : p.b;
+  const int K0 = i0 - g.plo;            // first k of chunk 0
+  const int J0 = i0 - g.lu_out;         // first column of tile 0
+  const float* pt = FWD ? (PREP ? p.ws_ea : p.a) : p.g;
+  const float* qt = FWD ? (PREP ? p.ws_eb : p.b) : GA ? (PREP ? p.ws_eb : p.b) : (PREP ? p.ws_ea : p.a);
   // offsets from the first cell of the batch item; EDGE keeps them inside the tensor
-  const float* aitem = at + bn * (long)Wa;
-  const float* bitem = bt + bn * (long)Wb;
-  const int a_min = (int)max(-bn * (long)Wa, -(1L << 30)), a_max = (int)min(cells_a - bn * (long)Wa - 1, 1L << 30);
-  const int b_min = (int)max(-bn * (long)Wb, -(1L << 30)), b_max = (int)min(cells_b - bn * (long)Wb - 1, 1L << 30);
+  const float* pitem = pt + bn * (long)Wp;
+  const float* ritem = MKH ? p.ws_r + bn * (long)Wp : nullptr;
+  const float* qitem = qt + bn * (long)Wq;
+  const long cells_p = rows * Wp, cells_q = rows * Wq;
+  const int p_min = (int)max(-bn * (long)Wp, -(1L << 30)), p_max = (int)min(cells_p - bn * (long)Wp - 1, 1L << 30);
+  const int q_min = (int)max(-bn * (long)Wq, -(1L << 30)), q_max = (int)min(cells_q - bn * (long)Wq - 1, 1L << 30);
   auto clamped = [](int v, int lo, int hi) __attribute__((always_inline)) { return min(max(v, lo), hi); };
+  // H = g / S; NaN where 1/S is marked unusable (the cell's gradients are then recomputed)
+  auto mk_h = [](float gv, float rv) __attribute__((always_inline)) {
+    return rv < 0.f ? __builtin_nanf("") : gv * rv;
+  };
 
-  // ---- P: row x0 + lr, cells k = 16 u + 4 lc - lr + t at dense position x0 - lu_a + 16 u + 4 lc + t,
-  // to LDS where lane 16 lc + lr will read them as 16 bytes; after the last chunk one of zeros
-  {
-    const int kb = 4 * lc - lr;
-    const int off = (x0 + lr) * Wa + kb;
-    mm_f4 v[kDirChunks];
+  // ---- Q.  A lane's cell t is Wq - 1 + 16 D + st with
+  //   band row j: loading lane (lr, lc), row J0 + 16 tj + lr, st = 4 lc - lr + t, D = u - tj
+  //   band row k: lane (l15, zq), row K0 + 16 u + 4 zq + t, st = l15 - 4 zq - t, D = tj - u
+  // and its cells of step (tj, u) start 16 * (bits 0-11 of the step's word) floats on.
+  const int s0 = QROW ? l15 - 4 * zq : 4 * lc - lr;  // st = s0 -/+ t
+  int qoff[4];
 #pragma unroll
-    for (int u = 0; u < kDirChunks; ++u) {
-      const int uu = min(u, NU - 1);  // same number of loads whatever NU
-      if (EDGE) {
+  for (int t = 0; t < 4; ++t)
+    qoff[t] = QROW ? (K0 + 4 * zq + t) * (Wq - 1) + J0 + l15 + (Wq - 1 - g.plo + g.lu_out)  // k (Wq - 1) + j + lu_q
+                   : (J0 + lr) * Wq + Wq - 1 + s0 + t;
+  auto issue = [&](unsigned e, mm_f4& q) __attribute__((always_inline)) {
+    const int soff = 16 * (int)(e & 0xfffu);  // uniform
+    if (QROW || EDGE) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) v[u][t] = aitem[clamped(off + 16 * uu + t, a_min, a_max)];
-      } else {
-        const dir_f4u w = *reinterpret_cast<const dir_f4u*>(aitem + (off + 16 * uu));
-        v[u] = mm_f4{w[0], w[1], w[2], w[3]};
+      for (int t = 0; t < 4; ++t) {
+        int o = qoff[t] + soff;
+        if (EDGE) o = clamped(o, q_min, q_max);
+        q[t] = qitem[o];
       }
+    } else {
+      const dir_f4u w = *reinterpret_cast<const dir_f4u*>((qitem + soff) + qoff[0]);
+      q = mm_f4{w[0], w[1], w[2], w[3]};
     }
-    mm_f4* pl = reinterpret_cast<mm_f4*>(lds) + (16 * lc + lr);
+  };
+  // the first steps' cells of Q are asked for before anything else
+  mm_f4 qraw[kDirDepth];
 #pragma unroll
-    for (int u = 0; u < kDirChunks; ++u) {
-      if (u < NU) {
-        mm_f4 x = v[u];
+  for (int s = 0; s < kDirDepth; ++s) issue(g.e[s].now, qraw[s]);
+
+  // ---- P into LDS, as the instruction reads it (lane, t); after the last chunk one of zeros.
+  //   band row i: loading lane (lr, lc), row i0 + lr, cells 16 u + 4 lc - lr + t, k = K0 + 16 u + 4 lc + t
+  //   band row k: lane (l15, zq), row k = K0 + 16 u + 4 zq + t, cell Wp - 1 - 16 u + l15 - 4 zq - t
+  {
+    mm_f4* pl = reinterpret_cast<mm_f4*>(lds);
+    const int off_i = (i0 + lr) * Wp + 4 * lc - lr;                 // + 16 u + t
+    const int lu_row = Wp - 1 - g.plo;  // band row k: cell = i - k + lu_row, at k (Wp - 1) + i + lu_row
+    const int off_k = (K0 + 4 * zq) * (Wp - 1) + i0 + l15 + lu_row;  // + (16 u + t) (Wp - 1)
+    // chunks whose loads are in flight together: all of them for bands up to 65 diagonals
+    // (the registers are free: LDS, not registers, bounds the waves per compute unit)
+    constexpr int kDirGroup = FWD ? 6 : 10;
+    for (int u0 = 0; u0 < NU; u0 += kDirGroup) {
+      mm_f4 v[kDirGroup], w[kDirGroup];
+#pragma unroll
+      for (int s = 0; s < kDirGroup; ++s) {
+        const int u = min(u0 + s, NU - 1);  // same number of loads whatever NU
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          bool ok = (unsigned)(kb + 16 * u + t) < (unsigned)Wa;
-          if (EDGE) ok = ok && x0 + lr < n && (unsigned)(x0 - a_lu + 16 * u + 4 * lc + t) < (unsigned)n;
-          x[t] = ok ? x[t] : 0.f;
+          if (PROW || EDGE) {
+            int o = PROW ? off_k + (16 * u + t) * (Wp - 1) : off_i + 16 * u + t;
+            if (EDGE) o = clamped(o, p_min, p_max);
+            v[s][t] = pitem[o];
+            if (MKH) w[s][t] = ritem[o];
+          }
         }
-        pl[64 * u] = x;
+        if (!PROW && !EDGE) {
+          const dir_f4u x = *reinterpret_cast<const dir_f4u*>(pitem + (off_i + 16 * u));
+          v[s] = mm_f4{x[0], x[1], x[2], x[3]};
+          if (MKH) {
+            const dir_f4u y = *reinterpret_cast<const dir_f4u*>(ritem + (off_i + 16 * u));
+            w[s] = mm_f4{y[0], y[1], y[2], y[3]};
+          }
+        }
+      }
+#pragma unroll
+      for (int s = 0; s < kDirGroup; ++s) {
+        const int u = u0 + s;
+        if (u < NU) {
+          mm_f4 x = v[s];
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const int cell = PROW ? Wp - 1 - 16 * u + l15 - 4 * zq - t : 16 * u + 4 * lc - lr + t;
+            bool ok = (unsigned)cell < (unsigned)Wp;
+            if (EDGE) {
+              const int k = K0 + 16 * u + (PROW ? 4 * zq : 4 * lc) + t;
+              ok = ok && i0 + (PROW ? l15 : lr) < n && (unsigned)k < (unsigned)n;
+            }
+            const float val = MKH ? mk_h(x[t], w[s][t]) : x[t];
+            x[t] = ok ? val : 0.f;
+          }
+          pl[64 * u + (PROW ? lane : 16 * lc + lr)] = x;
+        }
       }
     }
-    reinterpret_cast<mm_f4*>(lds)[64 * NU + lane] = mm_f4{0.f, 0.f, 0.f, 0.f};
+    pl[64 * NU + lane] = mm_f4{0.f, 0.f, 0.f, 0.f};
   }
-  // behind the chunks: beta of every column the wave's tiles cover (prepared log product), or
-  // the tile row's 16 x Wo results (plain product)
+  // behind the chunks: beta of every column the wave's tiles cover (forward of the log
+  // product), or the tile row's 16 x Wout results
   float* aux = lds + 256 * (NU + 1);
-  if (PREP) {
-    for (int t = lane; t < 16 * ny; t += 64) {
-      const int y = y0 + t;
+  if (FWD && PREP) {
+    for (int t = lane; t < 16 * nt; t += 64) {
+      const int y = J0 + t;
       aux[t] = (unsigned)y < (unsigned)n ? p.ws_be[bn + y] : 0.f;
     }
   }
 
-  // ---- Q(z, y) = b[y][k2], k2 = z - y + lu_b = 16 (u - ty) + 4 lc - lr + t + (Wb - 1) in the
-  // loading lane, which takes row y = y0 + 16 ty + lr
-  const int kq = 4 * lc - lr + Wb - 1;
-  const int qoff = (y0 + lr) * Wb + kq;  // pair (0, 0), t = 0
-  constexpr int kBias = 64;              // kq >= -15 + Wb - 1: offsets from (row y0's first cell - kBias) are unsigned
-  const float* qbase = bitem + (long)y0 * Wb - kBias;
-  const unsigned qlane = (unsigned)(lr * Wb + kq + kBias);
-  auto issue = [&](unsigned soff16, mm_f4& q) __attribute__((always_inline)) {
-    const unsigned soff = 16u * (soff16 & 0xfffu);  // uniform
-    if (EDGE) {
-#pragma unroll
-      for (int t = 0; t < 4; ++t) q[t] = bitem[clamped(qoff + (int)soff + t, b_min, b_max)];
-    } else {
-      const dir_f4u w = *reinterpret_cast<const dir_f4u*>((qbase + soff) + qlane);
-      q = mm_f4{w[0], w[1], w[2], w[3]};
-    }
-  };
-  // Factors 1 / 0 for the cells of a chunk at the ends of the band of b: a lane's cell t of a
-  // chunk with u - ty = d is b[y][k2], k2 = kq + 16 d + t.  Past the upper end (k2 >= Wb) only
-  // for d = 0; below the lower end (k2 < 0) for the lowest one or two d of the plan.
+  // Factors 1 / 0 for the cells of a chunk at the ends of Q's band: past the upper end
+  // (cell >= Wq) only for D = 0; below the lower end (cell < 0) for the lowest one or two D.
   float m_hi[4], m_lo0[4], m_lo1[4];
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
-    m_hi[t] = kq + t < Wb ? 1.f : 0.f;
-    m_lo0[t] = kq + 16 * plan.d_lo + t >= 0 ? 1.f : 0.f;
-    m_lo1[t] = kq + 16 * (plan.d_lo + 1) + t >= 0 ? 1.f : 0.f;
+    const int st = QROW ? s0 - t : s0 + t;
+    m_hi[t] = st <= 0 ? 1.f : 0.f;
+    m_lo0[t] = Wq - 1 + 16 * g.d_lo + st >= 0 ? 1.f : 0.f;
+    m_lo1[t] = Wq - 1 + 16 * (g.d_lo + 1) + st >= 0 ? 1.f : 0.f;
   }
   // the loaded cells of step e, zero where the lane is outside the band (EDGE: or the matrix).
   // (A factor 0 on a cell that is not finite leaves a NaN, which the test of the result catches;
   // the cell belongs to a neighbouring band row.)
   auto mask = [&](unsigned e, mm_f4& x) __attribute__((always_inline)) {
     if (EDGE) {
-      const int k2 = kq + 16 * ((int)((e >> 22) & 31u) - 16);
-      const int ty = (e >> 15) & 15u, u = (e >> 12) & 7u;
-      const int y = y0 + 16 * ty + lr, z = x0 - a_lu + 16 * u + 4 * lc;
+      const int tj = (e >> 16) & 15u, u = (e >> 12) & 15u;
+      const int D = QROW ? tj - u : u - tj;
+      const int j = J0 + 16 * tj + (QROW ? l15 : lr);
+      const int k = K0 + 16 * u + (QROW ? 4 * zq : 4 * lc);
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const bool ok = (unsigned)(k2 + t) < (unsigned)Wb && (unsigned)y < (unsigned)n && (unsigned)(z + t) < (unsigned)n;
+        const int cell = Wq - 1 + 16 * D + (QROW ? s0 - t : s0 + t);
+        const bool ok = (unsigned)cell < (unsigned)Wq && (unsigned)j < (unsigned)n && (unsigned)(k + t) < (unsigned)n;
         x[t] = ok ? x[t] : 0.f;
       }
     } else {
-      if (e & (1u << 20)) {  // uniform
+      if (e & (1u << 21)) {  // uniform
         asm volatile("" ::: "memory");  // keeps this a branch: most steps have nothing to mask
 #pragma unroll
         for (int t = 0; t < 4; ++t) x[t] *= m_hi[t];
       }
-      if (e & (1u << 21)) {  // uniform
-        asm volatile("" ::: "memory");  // keeps this a branch: most steps have nothing to mask
+      if (e & (1u << 22)) {  // uniform
+        asm volatile("" ::: "memory");
 #pragma unroll
         for (int t = 0; t < 4; ++t) x[t] *= m_lo0[t];
       }
-      if (e & (1u << 28)) {  // uniform
-        asm volatile("" ::: "memory");  // keeps this a branch: most steps have nothing to mask
+      if (e & (1u << 23)) {  // uniform
+        asm volatile("" ::: "memory");
 #pragma unroll
         for (int t = 0; t < 4; ++t) x[t] *= m_lo1[t];
       }
     }
   };
   auto to_mfma = [&](const mm_f4& v) __attribute__((always_inline)) {
+    if (QROW) return v;
     const float r0 = __int_as_float(__builtin_amdgcn_ds_bpermute(from, __float_as_int(v[0])));
     const float r1 = __int_as_float(__builtin_amdgcn_ds_bpermute(from, __float_as_int(v[1])));
     const float r2 = __int_as_float(__builtin_amdgcn_ds_bpermute(from, __float_as_int(v[2])));
@@ -251,64 +334,74 @@ __device__ __forceinline__ void dir_fwd_row(const BandArgs& p, const DirPlan& pl
   };
   const mm_f4* pl = reinterpret_cast<const mm_f4*>(lds) + lane;
 
-  // ---- results: accumulator element r is row x0 + 4 zq + r, column y0 + 16 ty + l15,
-  // band cell j = 16 ty + l15 - 4 zq - r
+  // ---- results: accumulator element r is row i0 + 4 zq + r, column J0 + 16 tj + l15,
+  // band cell jj = 16 tj + l15 - 4 zq - r
   const float thr = fast_exp2(-kBandGuardBits);
-  float* orow = p.o0 + (bn + x0) * (long)Wo;
-  float* rrow = PREP ? p.ws_r + (bn + x0) * (long)Wo : nullptr;
+  float* dst = KIND == kDirGradB ? p.o1 : p.o0;
+  float* orow = dst + (bn + i0) * (long)Wout;
+  float* rrow = FWD && PREP ? p.ws_r + (bn + i0) * (long)Wout : nullptr;
+  const float* erow = MKH ? (GA ? p.ws_ea : p.ws_eb) + (bn + i0) * (long)Wout : nullptr;  // factor on the way out
   unsigned ooff[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) ooff[r] = (unsigned)((4 * zq + r) * (Wo - 1) + l15);
+  for (int r = 0; r < 4; ++r) ooff[r] = (unsigned)((4 * zq + r) * (Wout - 1) + l15);
   float al[4] = {0.f, 0.f, 0.f, 0.f};
-  if (PREP) {
+  if (FWD && PREP) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r) al[r] = x0 + 4 * zq + r < n ? p.ws_al[bn + x0 + 4 * zq + r] : 0.f;
+    for (int r = 0; r < 4; ++r) al[r] = i0 + 4 * zq + r < n ? p.ws_al[bn + i0 + 4 * zq + r] : 0.f;
   }
-  const bool tail = x0 + 15 > n - 1;                   // rows beyond the matrix in this tile row
-  const bool y_all = y0 >= 0 && y0 + 16 * ny - 1 < n;  // every column of every tile inside the matrix
-  // cells to recompute: the prepared log product keeps a bit per cell (bit 4 ty + r), the plain
-  // product one flag per lane (all the lane's cells are then done again)
+  // the factors that the staged results of the log product's gradients leave with: asked for
+  // now, used when the tile row is done (16 bytes per lane and round of the final copy)
+  constexpr int kDirEf = 6;
+  mm_f4 ef[kDirEf];
+  if (MKH && STAGE) {
+#pragma unroll
+    for (int s = 0; s < kDirEf; ++s) {
+      const dir_f4u f = *reinterpret_cast<const dir_f4u*>(erow + 4 * min(lane + 64 * s, 4 * Wout - 1));
+      ef[s] = mm_f4{f[0], f[1], f[2], f[3]};
+    }
+  }
+  const bool tail = i0 + 15 > n - 1;                   // rows beyond the matrix in this tile row
+  const bool y_all = J0 >= 0 && J0 + 16 * nt - 1 < n;  // every column of every tile inside the matrix
+  // cells to recompute: the forward of the log product keeps a bit per cell (bit 4 tj + r), the
+  // others one flag per lane (all the lane's cells are then done again)
   unsigned long long redo = 0;
-  float worst = 0.f;  // plain product: stays 0 while every result is finite
-  // The plain product's tile rows away from the edges collect their 16 x Wo results in LDS
-  // (aux) and write them as one contiguous run of memory.  (Measured for the prepared log
-  // product too, with 1/S beside: the LDS it takes leaves three waves per compute unit fewer
-  // and the kernel 10 % slower.)
-  constexpr bool STAGE = !PREP && !EDGE;
-  float* st_o = aux;
-  const bool plain_rows = !PREP && !EDGE && y_all;
+  float worst = 0.f;  // stays 0 while every sum is finite
+  // Tile rows away from the edges collect their 16 x Wout results in LDS (aux) and write
+  // them as one contiguous run of memory.  (Measured for the forward of the log product too,
+  // with 1/S beside: the LDS it takes leaves three waves per compute unit fewer and the
+  // kernel 10 % slower.)
+  const bool plain_rows = STAGE && y_all;
   auto finish = [&](unsigned e, const mm_f4& c) __attribute__((always_inline)) {
-    const int ty = (e >> 15) & 15u;
+    const int tj = (e >> 16) & 15u;
     if (plain_rows) {  // uniform: nothing to test but the values
       const float s = (c[0] + c[1]) + (c[2] + c[3]);  // not finite if a cell is not (or the sum overflows: no harm)
       worst = __builtin_fmaf(s, 0.f, worst);          // 0 * s is NaN exactly when s is not finite
-      float* st = st_o + 16 * ty;
-      if (e & (1u << 29)) {
+      float* st = aux + 16 * tj;
+      if (e & (1u << 25)) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) st[ooff[r]] = c[r];
       } else {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int j = 16 * ty + l15 - 4 * zq - r;
-          if (j >= 0 && j < Wo) st[ooff[r]] = c[r];
+          const int jj = 16 * tj + l15 - 4 * zq - r;
+          if (jj >= 0 && jj < Wout) st[ooff[r]] = c[r];
         }
       }
       return;
     }
-    const bool whole = (e & (1u << 29)) && !tail;
-    const int y = y0 + 16 * ty + l15;
+    const bool whole = (e & (1u << 25)) && !tail;
+    const int y = J0 + 16 * tj + l15;
     const bool y_in = y_all || (unsigned)y < (unsigned)n;
-    float* ot = (STAGE ? st_o : orow) + 16 * ty;
-    float* rt = rrow + 16 * ty;
+    float* ot = (STAGE ? aux : orow) + 16 * tj;
     unsigned bits = 0;
     float be = 0.f;
-    if (PREP) be = aux[16 * ty + l15];
+    if (FWD && PREP) be = aux[16 * tj + l15];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int j = 16 * ty + l15 - 4 * zq - r;
-      if (whole || (x0 + 4 * zq + r < n && j >= 0 && j < Wo)) {
+      const int jj = 16 * tj + l15 - 4 * zq - r;
+      if (whole || (i0 + 4 * zq + r < n && jj >= 0 && jj < Wout)) {
         float v = y_in ? c[r] : 0.f;  // outside the matrix: the reference's zero fill
-        if (PREP) {
+        if (FWD && PREP) {
           float rv = 0.f;
           if (y_in) {
             const float sh = al[r] + be;
@@ -317,97 +410,118 @@ __device__ __forceinline__ void dir_fwd_row(const BandArgs& p, const DirPlan& pl
             v = __builtin_fmaf(fast_log2(v), kLn2, sh);
             if (!ok) bits |= 1u << r;
           }
-          rt[ooff[r]] = rv;
-        } else if (!(fabsf(v) <= FLT_MAX)) {
-          redo = 1;
+          (rrow + 16 * tj)[ooff[r]] = rv;
+        } else {
+          if (!(fabsf(v) <= FLT_MAX)) redo = 1;
+          if (MKH && !STAGE) v *= (erow + 16 * tj)[ooff[r]];
         }
         ot[ooff[r]] = v;
       }
     }
-    if (PREP) redo |= (unsigned long long)bits << (4 * ty);
+    if (FWD && PREP) redo |= (unsigned long long)bits << (4 * tj);
   };
 
   // ---- the walk: the loads of Q run kDirDepth steps ahead (past the end they repeat the
   // last step's and are never used); the words of the plan are read a step before their use
-  const int steps = plan.steps;
-  mm_f4 qraw[kDirDepth];
-#pragma unroll
-  for (int s = 0; s < kDirDepth; ++s) issue(plan.e[s].now, qraw[s]);
+  const int steps = g.steps;
   mm_f4 c = mm_f4{0.f, 0.f, 0.f, 0.f};
-  DirStep w = plan.e[0];
+  DirStep w = g.e[0];
   for (int i = 0; i < steps; i += kDirDepth) {
 #pragma unroll
     for (int s = 0; s < kDirDepth; ++s) {
       const DirStep cur = w;
-      w = plan.e[i + s + 1];  // one entry past the last exists
+      w = g.e[i + s + 1];  // one entry past the last exists
       const unsigned e = cur.now;
       mask(e, qraw[s]);
       const mm_f4 qv = to_mfma(qraw[s]);
-      const mm_f4 pv = pl[64 * ((e >> 12) & 7u)];
+      const mm_f4 pv = pl[64 * ((e >> 12) & 15u)];
       issue(cur.ahead, qraw[s]);
-      if (!(e & (1u << 27))) {  // uniform: not one of the filling steps
+      if (!(e & (1u << 24))) {  // uniform: not one of the filling steps
 #pragma unroll
         for (int t = 0; t < 4; ++t) c = __builtin_amdgcn_mfma_f32_16x16x4f32(pv[t], qv[t], c, 0, 0, 0);
       }
-      if (e & (1u << 19)) {  // uniform: the tile is complete
+      if (e & (1u << 20)) {  // uniform: the tile is complete
         finish(e, c);
         c = mm_f4{0.f, 0.f, 0.f, 0.f};
       }
     }
   }
 
-  if (STAGE) {  // the tile row's 16 Wo results: one contiguous run of memory
-    const mm_f4* so4 = reinterpret_cast<const mm_f4*>(st_o);
-    for (int i = lane; i < 4 * Wo; i += 64) {
-      const mm_f4 v = so4[i];
+  if (STAGE) {  // the tile row's 16 Wout results: one contiguous run of memory
+    const mm_f4* so4 = reinterpret_cast<const mm_f4*>(aux);
+#pragma unroll
+    for (int s = 0; s < kDirEf; ++s) {
+      const int i = lane + 64 * s;
+      if (i < 4 * Wout) {
+        mm_f4 v = so4[i];
+        if (MKH) v = mm_f4{v[0] * ef[s][0], v[1] * ef[s][1], v[2] * ef[s][2], v[3] * ef[s][3]};
+        *reinterpret_cast<dir_f4u*>(orow + 4 * i) = dir_f4u{v[0], v[1], v[2], v[3]};
+      }
+    }
+    for (int i = lane + 64 * kDirEf; i < 4 * Wout; i += 64) {
+      mm_f4 v = so4[i];
+      if (MKH) {
+        const dir_f4u f = *reinterpret_cast<const dir_f4u*>(erow + 4 * i);
+        v = mm_f4{v[0] * f[0], v[1] * f[1], v[2] * f[2], v[3] * f[3]};
+      }
       *reinterpret_cast<dir_f4u*>(orow + 4 * i) = dir_f4u{v[0], v[1], v[2], v[3]};
     }
   }
 
   // ---- cells to recompute (rare).  The stores above are to the same addresses from the
   // same lane: they stay in order.
-  if (!PREP && !(worst == 0.f)) redo = ~0ull;
+  if (!(FWD && PREP) && !(worst == 0.f)) redo = 1;
   if (__builtin_amdgcn_ballot_w64(redo != 0) != 0) {
-    if (!PREP && redo) redo = ~0ull;
+    if (STAGE) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // the run above was written by other lanes
+    if (!(FWD && PREP) && redo) redo = ~0ull;
     while (redo) {
       const int bit = __builtin_ctzll(redo);
       redo &= redo - 1;
-      const int ty = bit >> 2, r = bit & 3;
-      const int x = x0 + 4 * zq + r, j = 16 * ty + l15 - 4 * zq - r;
-      if (ty < ny && x < n && j >= 0 && j < Wo) {
-        if (PREP) band_fwd_cell<GENBMM_BAND_LOG>(p, bn + x, x, j);
-        else band_fwd_cell<GENBMM_BAND_MUL>(p, bn + x, x, j);
+      const int tj = bit >> 2, r = bit & 3;
+      const int i = i0 + 4 * zq + r, jj = 16 * tj + l15 - 4 * zq - r;
+      if (tj < nt && i < n && jj >= 0 && jj < Wout) {
+        if (FWD) {
+          if (PREP) band_fwd_cell<GENBMM_BAND_LOG>(p, bn + i, i, jj);
+          else band_fwd_cell<GENBMM_BAND_MUL>(p, bn + i, i, jj);
+        } else if (GA) {
+          if (PREP) band_bwd_a_cell<GENBMM_BAND_LOG>(p, bn + i, i, jj);
+          else band_bwd_a_cell<GENBMM_BAND_MUL>(p, bn + i, i, jj);
+        } else {
+          if (PREP) band_bwd_b_cell<GENBMM_BAND_LOG>(p, bn + i, i, jj);
+          else band_bwd_b_cell<GENBMM_BAND_MUL>(p, bn + i, i, jj);
+        }
       }
     }
   }
 }
 
 // One wave per tile row, kDirWaves tile rows per workgroup.  blocks: workgroups per batch item;
-// wave_lds: bytes of LDS per wave.
-template <bool PREP>
-__global__ __launch_bounds__(64 * kDirWaves) void k_band_dir_fwd(const BandArgs p, const DirPlan plan, int blocks, int nblocks,
-                                                     long cells_a, long cells_b, int wave_lds) {
+// wave_lds: bytes of LDS per wave; rows: band rows of every tensor (batch * n).
+template <int KIND, bool PREP>
+__global__ __launch_bounds__(64 * kDirWaves) void k_band_dir(const BandArgs p, const DirPlan g, int blocks, int nblocks,
+                                                            long rows, int wave_lds) {
   extern __shared__ __attribute__((aligned(16))) float dir_smem[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int blk = xcd_renumber(blockIdx.x, nblocks);
   const int batch = blk / blocks;
-  const int x0 = ((blk - batch * blocks) * kDirWaves + wave) * 16;
-  const int n = p.n, Wa = p.Wa, Wb = p.Wb;
-  if (x0 >= n) return;
+  const int i0 = ((blk - batch * blocks) * kDirWaves + wave) * 16;
+  const int n = p.n;
+  if (i0 >= n) return;
   const long bn = (long)batch * n;
   float* lds = dir_smem + wave * (wave_lds >> 2);
-  // May the wave take 16-byte loads and skip the tests against the matrix?  Every band cell of
-  // its rows of a inside the matrix (a cell of b that is not then only ever meets a zero), and
-  // the cells that the loads can touch beside the band rows inside the tensors.
-  const int ny = (p.Wo + 30) >> 4;
-  const long y0 = bn + x0 - p.r_lu;
-  const bool inside_matrix = x0 - p.a_lu >= 0 && x0 + 15 + (Wa - 1 - p.a_lu) <= n - 1;
-  const bool inside_tensor = (bn + x0) * (long)Wa >= 16 && (bn + x0 + 15) * (long)Wa + 16 * kDirChunks + 4 <= cells_a &&
-                             y0 * (long)Wb >= 16 * kDirChunks + 32 &&
-                             (y0 + 16 * ny) * (long)Wb + 16 * kDirChunks + 32 <= cells_b;
-  if (inside_matrix && inside_tensor) dir_fwd_row<PREP, false>(p, plan, bn, x0, lane, lds, cells_a, cells_b);
-  else dir_fwd_row<PREP, true>(p, plan, bn, x0, lane, lds, cells_a, cells_b);
+  // May the wave take its loads as they come and skip the tests against the matrix?  Every band
+  // cell of its rows of P inside the matrix (a cell of Q that is not then only ever meets a
+  // zero), and the cells that the loads can touch beside the band rows inside the tensors.
+  constexpr bool PROW = KIND == kDirGradB, QROW = KIND != kDirFwd;
+  const long K0 = bn + i0 - g.plo, J0 = bn + i0 - g.lu_out;
+  const long rp0 = PROW ? K0 : bn + i0, rp1 = PROW ? K0 + 16 * g.NU : bn + i0 + 16;  // band rows of P, of Q
+  const long rq0 = QROW ? K0 : J0, rq1 = QROW ? K0 + 16 * g.NU : J0 + 16 * g.nt;
+  const bool inside_matrix = i0 - g.plo >= 0 && i0 + 15 + g.phi <= n - 1;
+  const bool inside_tensor = rp0 * g.Wp >= kDirMargin && rp1 * g.Wp + kDirMargin <= rows * g.Wp &&
+                             rq0 * g.Wq >= kDirMargin && rq1 * g.Wq + kDirMargin <= rows * g.Wq;
+  if (inside_matrix && inside_tensor) dir_row<KIND, PREP, false>(p, g, bn, i0, lane, lds, rows);
+  else dir_row<KIND, PREP, true>(p, g, bn, i0, lane, lds, rows);
 }
 
 }  // namespace genbmm
