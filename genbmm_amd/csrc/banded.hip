@@ -22,9 +22,8 @@
 
 #include "banded_argmax.h"
 #include "banded_direct.h"
-#include "banded_mfma.h"
+#include "banded_flat.h"
 #include "banded_max.h"
-#include "banded_stream.h"
 #include "banded_strip.h"
 
 namespace genbmm {
@@ -50,20 +49,7 @@ inline bool bwd_strip_ok(const BandArgs& p) {
   return max(bwd_strip_bytes(da, true), bwd_strip_bytes(db, true)) <= kStripLdsLimit &&
          max(max(da.ld_own, da.ld_sl), max(db.ld_own, db.ld_sl)) <= 128;
 }
-// Which bands the matrix-core kernels take: wide enough for 16 x 16 tiles to pay (measured
-// against the strip kernels at 64 x 4096: forward from 9 diagonals on, gradients from 25),
-// and two workgroups' tiles fit in a compute unit's LDS.
-constexpr size_t kMmLdsLimit = 80 * 1024;
-// (the log product takes the forward from 4 diagonals on: what it replaces there is the
-// per-cell kernel pair with an exponential per term, 0.26 ms against 0.18 at 5 diagonals)
-inline bool mm_fwd_ok(const BandArgs& p, int min_w = 8) {
-  return mm_tiles_ok(p.Wa, p.Wb, p.Wo) && min(p.Wa, p.Wb) >= min_w &&
-         mm_dims(kMmFwd, p.Wa, p.Wb, p.Wo).bytes <= kMmLdsLimit;
-}
-inline bool mm_bwd_ok(const BandArgs& p) {
-  return mm_tiles_ok(p.Wa, p.Wb, p.Wo) && min(p.Wa, p.Wb) >= 25 &&
-         max(mm_dims(kMmGradA, p.Wa, p.Wb, p.Wo).bytes, mm_dims(kMmGradB, p.Wa, p.Wb, p.Wo).bytes) <= kMmLdsLimit;
-}
+constexpr size_t kMmLdsLimit = 80 * 1024;  // two workgroups' tiles in a compute unit's LDS
 // The memory-fed kernels (banded_direct.h): a plan within their limits, offsets inside a
 // batch item within 32 bits.
 inline bool dir_ok(int kind, const BandArgs& p, int min_w) {
@@ -82,13 +68,13 @@ inline bool dir_bwd_ok(const BandArgs& p) {
   return dir_ok(kDirGradA, p, kDirMinW) && dir_ok(kDirGradB, p, kDirMinW);
 }
 // The workspace of the log product is filled and used only when both directions have a
-// kernel that works on it (matrix-core or strip), so that forward and backward always agree
+// kernel that works on it (memory-fed or strip), so that forward and backward always agree
 // on whether it holds anything.
 inline bool workspace_used(const BandArgs& p) {
-  const bool fwd = dir_fwd_ok(p) || mm_fwd_ok(p, 4) ||
+  const bool fwd = dir_fwd_ok(p) ||
                    (fwd_strip_ok(p) &&
                     strip_dims(p.Wa, p.Wb).bytes + sizeof(float) * (kBT + p.Wo + kBJ) <= kStripLdsLimit);
-  return fwd && (dir_bwd_ok(p) || mm_bwd_ok(p) || bwd_strip_ok(p));
+  return fwd && (dir_bwd_ok(p) || bwd_strip_ok(p));
 }
 
 inline bool prep_fwd(const BandArgs& p, int mode, const float* workspace) {
@@ -112,53 +98,6 @@ inline void launch_max_fwd(const BandArgs& p, int B, hipStream_t s) {
                      rows * p.Wa, rows * p.Wb);
 }
 
-// The streaming kernels (banded_stream.h): operands wide enough for 16 x 16 tiles and within
-// the registers that carry a block's new rows to LDS, tiles within a compute unit's LDS.
-// Rows per block: 64 if two such workgroups fit a compute unit, else 32 if two of those
-// do, else 64 with the compute unit to itself; 0: the band is not for these kernels.
-constexpr size_t kStreamLdsLimit = 160 * 1024;
-inline int stream_rows(int kind, const BandArgs& p) {
-  const int wp = kind == kStFwd ? p.Wa : p.Wo, wout = kind == kStFwd ? p.Wo : p.Wa;
-  if (min(p.Wa, p.Wb) < 8 || p.Wb > 95 || wp > (kind == kStFwd ? 95 : 191) || wout > 162) return 0;
-  auto fits = [&](int rows, int per_cu) {
-    const StreamDims d = stream_dims(kind, rows, p.Wa, p.Wb, p.Wo);
-    return (d.qr - rows) * d.qp <= 4 * 8 * rows * kSShift && d.bytes * per_cu <= kStreamLdsLimit;
-  };
-  if (fits(64, 2)) return 64;
-  if (fits(32, 2)) return 32;
-  return fits(64, 1) ? 64 : 0;
-}
-// grad_a as a stream pays from about 57 diagonals on (measured at 64 x 4096 against the
-// strip-owning matrix-core kernel, whole backward: 33 diagonals 0.171 ms against 0.166, 49:
-// 0.214 against 0.201, 65: 0.326 against 0.387)
-inline bool stream_ok(int kind, const BandArgs& p) {
-  return stream_rows(kind, p) != 0 && (kind == kStFwd || min(p.Wa, p.Wb) >= 57);
-}
-
-template <int KIND, bool PREP, int ROWS>
-inline void launch_stream_rows(const BandArgs& p, int B, hipStream_t s, int fuse_h) {
-  const StreamDims d = stream_dims(KIND, ROWS, p.Wa, p.Wb, p.Wo);
-  // Runs: about as many workgroups as the chip holds at once (256 compute units, one or
-  // two workgroups each), runs of whole blocks.
-  const int per_cu = d.bytes * 2 <= kStreamLdsLimit ? 2 : 1;
-  const int blocks = ceil_div(p.n, ROWS);
-  int runs = (int)min((long)blocks, max(1L, (256L * per_cu + B - 1) / B));
-  const int run_rows = ceil_div(blocks, runs) * ROWS;
-  runs = ceil_div(p.n, run_rows);
-  auto kern = k_band_stream<KIND, PREP, ROWS>;
-  if (d.bytes > kStripLdsLimit)
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)d.bytes);
-  const long rows = (long)B * p.n;
-  hipLaunchKernelGGL(kern, dim3((unsigned)((long)B * runs)), dim3(8 * ROWS), d.bytes, s, p, d, runs, run_rows,
-                     rows * p.Wa, rows * p.Wb, rows * p.Wo, fuse_h);
-}
-template <int KIND, bool PREP>
-inline void launch_stream(const BandArgs& p, int B, hipStream_t s, int fuse_h = 0) {
-  if (stream_rows(KIND, p) == 32) launch_stream_rows<KIND, PREP, 32>(p, B, s, fuse_h);
-  else launch_stream_rows<KIND, PREP, 64>(p, B, s, fuse_h);
-}
-
 template <int KIND, bool PREP>
 inline void launch_dir(const BandArgs& p, int B, hipStream_t s) {
   const int blocks = ceil_div(p.n, 16 * kDirWaves);
@@ -172,19 +111,6 @@ inline void launch_dir(const BandArgs& p, int B, hipStream_t s) {
                               kDirWaves * wave_lds);
   hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64 * kDirWaves), kDirWaves * wave_lds, s, p, plan, blocks,
                      nblocks, (long)B * p.n, wave_lds);
-}
-
-template <int KIND, bool PREP>
-inline void launch_mm(const BandArgs& p, int B, hipStream_t s, int fuse_h = 0) {
-  const MmDims d = mm_dims(KIND, p.Wa, p.Wb, p.Wo);
-  const int strips = ceil_div(p.n, mm_rows(KIND));
-  auto kern = k_band_mm<KIND, PREP>;
-  if (d.bytes > kStripLdsLimit)
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)d.bytes);
-  const long rows = (long)B * p.n;
-  hipLaunchKernelGGL(kern, dim3((unsigned)((long)B * strips)), dim3(256), d.bytes, s, p, strips, d,
-                     rows * p.Wa, rows * p.Wb, rows * p.Wo, fuse_h);
 }
 
 inline void set_workspace(BandArgs& p, float* ws, int B) {
@@ -225,7 +151,7 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   hipStream_t s = (hipStream_t)stream;
   const StripDims sd = strip_dims(p.Wa, p.Wb);
   const bool dir = dir_fwd_ok(p, mode == GENBMM_BAND_MUL ? kDirMinWPlainFwd : kDirMinW);
-  if ((mode == GENBMM_BAND_MUL && (dir || mm_fwd_ok(p))) || (prep_fwd(p, mode, workspace) && (dir || mm_fwd_ok(p, 4)))) {
+  if (dir && (mode == GENBMM_BAND_MUL || prep_fwd(p, mode, workspace))) {
     if (mode == GENBMM_BAND_LOG) {
       set_workspace(p, workspace, B);
       const long rows = (long)B * n;
@@ -235,13 +161,9 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
                          p.ws_al, p.Wa, a_lu, n, rows, lda);
       hipLaunchKernelGGL(k_band_prep, pg, dim3(256), sizeof(float) * kPrepRows * ldb, s, b, p.ws_eb,
                          p.ws_be, p.Wb, b_lu, n, rows, ldb);
-      if (dir) launch_dir<kDirFwd, true>(p, B, s);
-      else if (stream_ok(kStFwd, p)) launch_stream<kStFwd, true>(p, B, s);
-      else launch_mm<kMmFwd, true>(p, B, s);
+      launch_dir<kDirFwd, true>(p, B, s);
     } else {
-      if (dir) launch_dir<kDirFwd, false>(p, B, s);
-      else if (stream_ok(kStFwd, p)) launch_stream<kStFwd, false>(p, B, s);
-      else launch_mm<kMmFwd, false>(p, B, s);
+      launch_dir<kDirFwd, false>(p, B, s);
     }
     return launch_status();
   }
@@ -317,29 +239,6 @@ int banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int
       launch_dir<kDirGradA, true>(p, B, s);
       launch_dir<kDirGradB, true>(p, B, s);
     }
-    return launch_status();
-  }
-  if (mode == GENBMM_BAND_MUL && mm_bwd_ok(p)) {
-    if (stream_ok(kStGradA, p)) launch_stream<kStGradA, false>(p, B, s);
-    else launch_mm<kMmGradA, false>(p, B, s);
-    launch_mm<kMmGradB, false>(p, B, s);
-    return launch_status();
-  }
-  if (mode == GENBMM_BAND_LOG && workspace && workspace_used(p) && mm_bwd_ok(p)) {
-    set_workspace(p, workspace, B);
-    if (scratch) p.ws_h = scratch;
-    // H = g / S: formed by the grad_a kernel while it stages it and left in the workspace for
-    // grad_b, if the three arrays start on the same 16-byte phase; else by a pass of its own
-    const auto phase = [](const void* q) { return reinterpret_cast<uintptr_t>(q) & 15; };
-    const int fuse_h = phase(g) == phase(p.ws_r) && phase(g) == phase(p.ws_h);
-    if (!fuse_h) {
-      const long cells = (long)B * n * p.Wo;
-      hipLaunchKernelGGL(k_band_h, dim3((unsigned)min((cells + 1023) / 1024, (long)0x7fffffff)), dim3(256), 0,
-                         s, g, p.ws_r, p.ws_h, cells);
-    }
-    if (stream_ok(kStGradA, p)) launch_stream<kStGradA, true>(p, B, s, fuse_h);
-    else launch_mm<kMmGradA, true>(p, B, s, fuse_h);
-    launch_mm<kMmGradB, true>(p, B, s);
     return launch_status();
   }
   if (mode != GENBMM_BAND_MAX && bwd_strip_ok(p)) {

@@ -2,7 +2,7 @@
 // grad_b of the plain product and of the log product on the forward's workspace.  No
 // operand tiles shared through LDS, no barrier.
 //
-// Dense coordinates as in banded_mfma.h.  Each of the three is C[i, j] = sum_k P(i, k) Q(k, j)
+// In dense coordinates each of the three is C[i, j] = sum_k P(i, k) Q(k, j)
 // cut into 16 x 16 tiles of (i, j); one wave owns a tile row (16 rows i) and walks its
 // tiles along j; waves never meet.
 //
@@ -55,7 +55,7 @@
 
 #include <cfloat>
 
-#include "banded_mfma.h"
+#include "banded_flat.h"
 
 namespace genbmm {
 

@@ -17,7 +17,7 @@
 // once instead of once per 32 diagonals, and the result leaves in 16-byte stores.
 #pragma once
 
-#include "banded_mfma.h"
+#include "banded_flat.h"
 
 namespace genbmm {
 

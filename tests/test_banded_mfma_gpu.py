@@ -1,7 +1,7 @@
-"""GPU parity of the banded (+,x) and log products on bands wide enough for the
-matrix-core kernels (9 diagonals forward, 25 backward): edges of the matrix inside a
-strip, strips cut by n, one-sided bands, operands that do not start on 16 bytes, values
-that are not finite.  All against the float64 sequential restatement of the reference
+"""GPU parity of the banded (+,x) and log products on the bands that the matrix-core
+kernels take (from 3 diagonals on, up to about 160 in the result): edges of the matrix
+inside a tile row, tile rows cut by n, one-sided bands, the widest first operands,
+operands that do not start on 16 bytes, values that are not finite.  All against the float64 sequential restatement of the reference
 kernel (oracle.seq_band_fwd / seq_band_bwd)."""
 import numpy as np
 import pytest
@@ -15,7 +15,8 @@ pytestmark = pytest.mark.gpu
 # (n, a_lu, a_ld, b_lu, b_ld)
 WIDE = [(300, 12, 12, 12, 12), (95, 20, 9, 14, 16), (513, 32, 32, 32, 32), (64, 30, 0, 0, 30),
         (33, 16, 16, 16, 16), (1000, 3, 30, 28, 2), (129, 4, 4, 20, 20), (40, 28, 28, 30, 30),
-        (257, 0, 31, 31, 0), (70, 10, 5, 3, 8)]
+        (257, 0, 31, 31, 0), (70, 10, 5, 3, 8), (400, 40, 40, 40, 40), (210, 0, 60, 60, 0),
+        (150, 70, 0, 2, 1), (47, 1, 1, 1, 1)]
 
 
 def close(x, ref, rtol=1e-5, atol=1e-5):
