@@ -1,0 +1,246 @@
+// Double-precision logbmm on the matrix cores (v_mfma_f64_16x16x4_f64): forward, grad_a
+// and grad_b in the factored form of the float path, with no workspace.
+//
+//   alpha[m] = max_k a[m,k], beta[n] = max_k b[k,n], EA = exp(a - alpha), EB = exp(b - beta)
+//   S = EA EB,  out = log S + alpha + beta,  H = g / S = g exp(alpha + beta - out)
+//   grad_a = EA .* (H EB^T),  grad_b = EB .* (EA^T H)
+//
+// so that (M K + K N + M N) exponentials replace the M K N of the reference's loops
+// (matmul_cuda_kernel.cu:27-41, 159-217), and the contraction is a plain product.  All
+// three are C[i,j] = sum_l P[i,l] Q[l,j] on 128 x 128 (or 64 x 64) tiles of (i,j), one
+// workgroup of four waves per tile (each wave a quarter: sixteen or four 16 x 16
+// accumulators), the contraction in chunks of 16 staged in LDS with the exponential taken
+// on the way in; the next chunk's operands are in flight while the current one is
+// multiplied.  The exponentials of a staged chunk are vector work of about the same cost as
+// the chunk's matrix instructions at 64 x 64 and half of it at 128 x 128.
+//
+// The entry points have no workspace to keep the maxima in, so a workgroup takes them itself
+// before its tile: the forward for its own rows and columns, grad_a for its rows and
+// every column of the item, grad_b for every row and its columns (a pass over a and b that
+// the L2 serves; a few percent of the tile's work up to a few hundred rows).
+//
+// Exact wherever the factors lose nothing: a sum S below 1e-280 (terms that underflow in the
+// factored form could matter), a shift at the reference's -1e9 floor or anything not finite
+// sends the cell to the reference's own loops (a forward cell: two passes over k; a
+// gradient cell: the sum of exp(a + b - out) g), inside the same kernel.  H is NaN where S
+// is not usable, which carries the flag through the product to every cell it feeds.
+#pragma once
+
+#include "common.h"
+
+namespace genbmm {
+
+constexpr int kDC = 16;        // contraction chunk
+constexpr int kDP = kDC + 2;   // row pitch of a staged chunk, in doubles
+constexpr double kDFloor = -1e9;
+constexpr double kDThr = 1e-280;
+constexpr double kDLogThr = -644.7;  // log(kDThr), rounded up
+constexpr int kDMaxAll = 4096;  // grad_a keeps beta of every column in LDS, grad_b alpha of every row
+typedef double mmd4 __attribute__((ext_vector_type(4)));
+
+constexpr int kD64Fwd = 0, kD64GradA = 1, kD64GradB = 2;
+
+__device__ __forceinline__ double d64_shift(double mx) { return mx == -INFINITY ? 0.0 : mx; }
+__device__ __forceinline__ bool d64_usable(double shift) { return shift > 0.9 * kDFloor && shift < INFINITY; }
+
+// kDT: tile edge, 64 or 128 (a wave's share 32 x 32 or 64 x 64).  tiles: (ceil(I / kDT),
+// ceil(J / kDT)) per item; grid = B * tiles_i * tiles_j
+template <int KIND, int kDT>
+__global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ a, const double* __restrict__ b,
+                                                 const double* __restrict__ out, const double* __restrict__ g,
+                                                 double* __restrict__ dst, int M, int K, int N, int tiles_i,
+                                                 int tiles_j) {
+  extern __shared__ __attribute__((aligned(16))) double smem64[];
+  constexpr bool FWD = KIND == kD64Fwd, GA = KIND == kD64GradA, GB = KIND == kD64GradB;
+  const int I = GB ? K : M, J = FWD ? N : GA ? K : N, L = FWD ? K : GA ? N : M;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tile = blockIdx.x % (tiles_i * tiles_j), batch = blockIdx.x / (tiles_i * tiles_j);
+  const int i0 = (tile / tiles_j) * kDT, j0 = (tile % tiles_j) * kDT;
+  const double* ab = a + (long)batch * M * K;
+  const double* bb = b + (long)batch * K * N;
+  const double* ob = FWD ? nullptr : out + (long)batch * M * N;
+  const double* gb = FWD ? nullptr : g + (long)batch * M * N;
+  double* db = dst + (long)batch * I * J;
+
+  constexpr int kH = kDT / 64, kW = kDT / 32;  // staging rounds per chunk; 16 x 16 accumulators per wave and side
+  double* Ps = smem64;              // [kDT][kDP]: P[i][l]
+  double* Qs = Ps + kDT * kDP;      // [kDT][kDP]: Q[l][j] as [j][l]
+  double* al = Qs + kDT * kDP;      // alpha: the tile's rows m (forward, grad_a) or all M (grad_b)
+  double* be = al + (GB ? M : kDT); // beta: the tile's columns n (forward, grad_b) or all N (grad_a)
+  const int m_lo = GB ? 0 : i0, m_cnt = GB ? M : min(kDT, M - i0);
+  const int n_lo = FWD ? j0 : GA ? 0 : j0, n_cnt = GA ? N : min(kDT, N - n_lo);
+
+  // ---- maxima.  alpha: one wave per row, lanes along k.  beta: 64 columns at a time, four
+  // groups of 64 threads over k, combined through LDS (Ps is free yet).
+  for (int r = wave; r < m_cnt; r += 4) {
+    const double* row = ab + (long)(m_lo + r) * K;
+    double mx = -INFINITY;
+    for (int k = lane; k < K; k += 64) mx = fmax(mx, row[k]);
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) mx = fmax(mx, __shfl_xor(mx, s, 64));
+    if (lane == 0) al[r] = mx;
+  }
+  for (int c0 = 0; c0 < n_cnt; c0 += 64) {
+    const int c = c0 + lane;
+    double mx = -INFINITY;
+    if (c < n_cnt)
+      for (int k = wave; k < K; k += 4) mx = fmax(mx, bb[(long)k * N + n_lo + c]);
+    Ps[wave * 64 + lane] = mx;
+    __syncthreads();
+    if (wave == 0 && c < n_cnt) be[c] = fmax(fmax(Ps[lane], Ps[64 + lane]), fmax(Ps[128 + lane], Ps[192 + lane]));
+    __syncthreads();
+  }
+  __syncthreads();
+
+  // ---- staging.  A thread owns four neighbouring elements along the operand's contiguous
+  // axis: (line = tid / 4, l = 4 (tid % 4) ..) where the contraction index is contiguous,
+  // (l = tid / 16, line = 4 (tid % 16) ..) where the line index is.  raw_*: what memory
+  // holds (the next chunk's, in flight during the products); put(): exponentials, LDS.
+  constexpr bool P_L = !GB;  // P's contiguous axis is l (a[m][k] forward, g[m][n] grad_a); grad_b: i (a[m][k], i = k)
+  constexpr bool Q_L = GA;   // Q's contiguous axis is l only in grad_a (b[k][n], l = n)
+  const int pl_line = P_L ? tid >> 2 : 4 * (tid & 15), pl_l = P_L ? 4 * (tid & 3) : tid >> 4;
+  const int ql_line = Q_L ? tid >> 2 : 4 * (tid & 15), ql_l = Q_L ? 4 * (tid & 3) : tid >> 4;
+  double rp[4 * kH], rp2[4 * kH], rq[4 * kH], rq2[4 * kH];
+  auto load = [&](int l0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int eh = 0; eh < 4 * kH; ++eh) {
+      const int e = eh & 3, h = eh >> 2;
+      {  // P[i][l]
+        const int i = i0 + 64 * h + pl_line + (P_L ? 0 : e), l = l0 + pl_l + (P_L ? e : 0);
+        const bool ok = i < I && l < L;
+        long off = 0;
+        if (FWD) off = (long)i * K + l;  // a[m = i][k = l]
+        if (GA) off = (long)i * N + l;   // g, out [m = i][n = l]
+        if (GB) off = (long)l * K + i;   // a[m = l][k = i]
+        rp[eh] = ok ? (GA ? gb[off] : ab[off]) : 0.0;
+        if (GA) rp2[eh] = ok ? ob[off] : 0.0;
+      }
+      {  // Q[l][j]
+        const int j = j0 + 64 * h + ql_line + (Q_L ? 0 : e), l = l0 + ql_l + (Q_L ? e : 0);
+        const bool ok = j < J && l < L;
+        long off = 0;
+        if (FWD) off = (long)l * N + j;  // b[k = l][n = j]
+        if (GA) off = (long)j * N + l;   // b[k = j][n = l]
+        if (GB) off = (long)l * N + j;   // g, out [m = l][n = j]
+        rq[eh] = ok ? (GB ? gb[off] : bb[off]) : 0.0;
+        if (GB) rq2[eh] = ok ? ob[off] : 0.0;
+      }
+    }
+  };
+  // H = g exp(alpha + beta - out); NaN where S = exp(out - alpha - beta) is not usable
+  auto h_of = [&](double gv, double ov, double am, double bn) __attribute__((always_inline)) {
+    const double sh = d64_shift(am) + d64_shift(bn), ls = ov - sh;  // ls = log S
+    const bool ok = d64_usable(sh) && ls >= kDLogThr && ls < INFINITY;
+    return ok ? gv * exp(-ls) : __builtin_nan("");
+  };
+  auto put = [&](int l0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int eh = 0; eh < 4 * kH; ++eh) {
+      const int e = eh & 3, h = eh >> 2;
+      {
+        const int il = 64 * h + pl_line + (P_L ? 0 : e), ll = pl_l + (P_L ? e : 0);
+        const int i = i0 + il, l = l0 + ll;
+        double v = 0.0;
+        if (i < I && l < L) {
+          if (FWD) v = exp(rp[eh] - d64_shift(al[il]));
+          if (GA) v = h_of(rp[eh], rp2[eh], al[il], be[l]);
+          if (GB) v = exp(rp[eh] - d64_shift(al[l]));
+        }
+        Ps[il * kDP + ll] = v;
+      }
+      {
+        const int jl = 64 * h + ql_line + (Q_L ? 0 : e), ll = ql_l + (Q_L ? e : 0);
+        const int j = j0 + jl, l = l0 + ll;
+        double v = 0.0;
+        if (j < J && l < L) {
+          if (FWD) v = exp(rq[eh] - d64_shift(be[jl]));
+          if (GA) v = exp(rq[eh] - d64_shift(be[l]));
+          if (GB) v = h_of(rq[eh], rq2[eh], al[l], be[jl]);
+        }
+        Qs[jl * kDP + ll] = v;
+      }
+    }
+  };
+
+  // ---- products: wave (wi, wj) owns rows (kDT / 2) wi .., columns (kDT / 2) wj .. of the tile
+  constexpr int kS = kDT / 2;
+  const int wi = wave >> 1, wj = wave & 1, l15 = lane & 15, zq = lane >> 4;
+  mmd4 acc[kW][kW];
+#pragma unroll
+  for (int x = 0; x < kW; ++x)
+#pragma unroll
+    for (int y = 0; y < kW; ++y) acc[x][y] = mmd4{0.0, 0.0, 0.0, 0.0};
+  load(0);
+  for (int l0 = 0; l0 < L; l0 += kDC) {
+    put(l0);
+    __syncthreads();
+    if (l0 + kDC < L) load(l0 + kDC);
+#pragma unroll
+    for (int ks = 0; ks < kDC / 4; ++ks) {
+      double pa[kW], qb[kW];
+#pragma unroll
+      for (int x = 0; x < kW; ++x) pa[x] = Ps[(kS * wi + 16 * x + l15) * kDP + 4 * ks + zq];
+#pragma unroll
+      for (int y = 0; y < kW; ++y) qb[y] = Qs[(kS * wj + 16 * y + l15) * kDP + 4 * ks + zq];
+#pragma unroll
+      for (int x = 0; x < kW; ++x)
+#pragma unroll
+        for (int y = 0; y < kW; ++y) acc[x][y] = __builtin_amdgcn_mfma_f64_16x16x4f64(pa[x], qb[y], acc[x][y], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  // ---- results: accumulator element r of tile (x, y) is row kS wi + 16 x + 4 r + zq, column
+  // kS wj + 16 y + l15
+#pragma unroll
+  for (int x = 0; x < kW; ++x)
+#pragma unroll
+    for (int y = 0; y < kW; ++y)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int il = kS * wi + 16 * x + 4 * r + zq, jl = kS * wj + 16 * y + l15;
+        const int i = i0 + il, j = j0 + jl;
+        if (i >= I || j >= J) continue;
+        const double v = acc[x][y][r];
+        double res;
+        if (FWD) {
+          const double sh = d64_shift(al[il]) + d64_shift(be[jl]);
+          if (d64_usable(sh) && v >= kDThr && v < INFINITY) {
+            res = log(v) + sh;
+          } else {  // the reference's two passes (matmul_cuda_kernel.cu:27-41)
+            const double* arow = ab + (long)i * K;
+            const double* bcol = bb + j;
+            double mx = kDFloor;
+            for (int k = 0; k < K; ++k) mx = fmax(mx, arow[k] + bcol[(long)k * N]);
+            double s = 0.0;
+            for (int k = 0; k < K; ++k) s += exp(arow[k] + bcol[(long)k * N] - mx);
+            res = log(s) + mx;
+          }
+        } else if (GA) {  // i = m, j = k
+          const double av = ab[(long)i * K + j];
+          res = exp(av - d64_shift(al[il])) * v;
+          if (!(fabs(res) <= DBL_MAX)) {  // matmul_cuda_kernel.cu:159-184
+            double s = 0.0;
+            for (int n = 0; n < N; ++n)
+              s = __builtin_fma(exp(av + bb[(long)j * N + n] - ob[(long)i * N + n]), gb[(long)i * N + n], s);
+            res = s;
+          }
+        } else {  // i = k, j = n
+          const double bv = bb[(long)i * N + j];
+          res = exp(bv - d64_shift(be[jl])) * v;
+          if (!(fabs(res) <= DBL_MAX)) {  // matmul_cuda_kernel.cu:190-217
+            double s = 0.0;
+            for (int m = 0; m < M; ++m)
+              s = __builtin_fma(exp(ab[(long)m * K + i] + bv - ob[(long)m * N + j]), gb[(long)m * N + j], s);
+            res = s;
+          }
+        }
+        db[(long)i * J + j] = res;
+      }
+}
+
+inline size_t d64_mm_lds(int kind, int tile, int M, int N) {
+  return sizeof(double) * (2 * tile * kDP + (kind == kD64GradB ? M : tile) + (kind == kD64GradA ? N : tile));
+}
+
+}  // namespace genbmm

@@ -60,6 +60,37 @@ def test_logbmm_f64_special_values(gpu):
     assert abs(got - np.log1p(np.exp(-30.0))) < 3e-16 and got != 0.0
 
 
+def test_logbmm_f64_factoring_guard(gpu):
+    """Shapes that take the factored matrix-core kernels, with rows and columns whose maxima
+    sit on cells that never meet (exp(a - rowmax) * exp(b - colmax) underflows although the
+    true terms do not), entries at the reference's -1e9 floor, -inf entries and a row that is
+    all -inf: every such cell and every gradient fed by it must come from the exact loops."""
+    torch.manual_seed(11)
+    B, M, K, N = 2, 70, 40, 97
+    a, b = torch.randn(B, M, K).double() * 3, torch.randn(B, K, N).double() * 3
+    g = torch.randn(B, M, N).double()
+    a[:, ::3, 0] += 800.0    # the row maximum, on k = 0 ...
+    b[:, 0, :] -= 800.0      # ... which every column makes irrelevant
+    b[:, 5, 1::4] += 700.0   # column maxima on k = 5
+    a[0, 7, 3:9] = float("-inf")
+    a[1, 10, :] = -1e9
+    a[1, 20, :] = float("-inf")
+    out = genbmm.logbmm(a.to(gpu), b.to(gpu)).cpu()
+    want = oracle.seq_logbmm_fwd(a, b, dtype=F64)[0]
+    live = torch.isfinite(want)
+    assert bool(live.sum() > 0.9 * want.numel()) and torch.equal(torch.isfinite(out), live)
+    close(out[live], want[live], 1e-12, 1e-9)
+    close(out[live], oracle.logbmm_broadcast(a, b)[live], 1e-12, 1e-9)
+    # gradients, without the all -inf row (its weights are NaN in the reference's own arithmetic)
+    a[1, 20, :] = torch.randn(K).double()
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    ga, gb = torch.autograd.grad(genbmm.logbmm(ad, bd), (ad, bd), g.to(gpu))
+    wa, wb = oracle.seq_logbmm_bwd(a, b, g, dtype=F64)
+    assert torch.isfinite(wa).all() and torch.isfinite(wb).all()
+    close(ga, wa, 1e-10, 1e-9)
+    close(gb, wb, 1e-10, 1e-9)
+
+
 @pytest.mark.parametrize("B,M,K,N", SHAPES)
 @pytest.mark.parametrize("prod", [False, True])
 def test_max_f64_bit_exact(gpu, B, M, K, N, prod):
