@@ -34,6 +34,7 @@
 #include "log_bwd_tile.h"
 #include "logbmm_item.h"
 #include "logbmm_mfma.h"
+#include "logbmm_item32.h"
 #include "logbmm_ws.h"
 
 namespace genbmm {
@@ -842,7 +843,8 @@ int run_fwd(const float* a, const float* b, float* out, float* stats, int B, int
   if (missing(a, mk) || missing(b, kn) || missing(out, mn)) return GENBMM_E_NULLPTR;
   if (stats && B > 0 && item_shape(M, K, N) && path == GENBMM_PATH_AUTO) {  // whole items per workgroup
     int* hdr = prepared_of(stats, B, M, K, N).hdr;
-    if (M == 32 && K == 32 && N == 32) launch_item_fwd<16, 2, true>(a, b, out, stats, hdr, B, M, K, N, s);
+    if (M == 32 && K == 32 && N == 32)  // one wave per item on the matrix cores
+      hipLaunchKernelGGL(k_log_item32_fwd, dim3((B + 3) / 4), dim3(256), 0, s, a, b, out, stats, hdr, B);
     else if (M == 64 && K == 64 && N == 64) launch_item_fwd<16, 4, true>(a, b, out, stats, hdr, B, M, K, N, s);
     else if (max(max(M, K), N) <= 32) launch_item_fwd<16, 2, false>(a, b, out, stats, hdr, B, M, K, N, s);
     else launch_item_fwd<16, 4, false>(a, b, out, stats, hdr, B, M, K, N, s);
@@ -890,7 +892,7 @@ int run_bwd_both(const float* a, const float* b, const float* out, const float* 
   const float* st = (path == GENBMM_PATH_EXACT || mn == 0) ? nullptr : stats;
   if (st && B > 0 && item_shape(M, K, N) && path == GENBMM_PATH_AUTO) {
     if (M == 32 && K == 32 && N == 32)
-      hipLaunchKernelGGL((k_log_item_bwd<16, 2, true>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
+      hipLaunchKernelGGL(k_log_item32_bwd, dim3((B + 3) / 4), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, B);
     else if (M == 64 && K == 64 && N == 64)
       hipLaunchKernelGGL((k_log_item_bwd<16, 4, true>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
     else if (max(max(M, K), N) <= 32)
