@@ -92,6 +92,28 @@ def dense_log(lib, dev, B, M, K, N, reps, name, dist="randn", path=0, graph=Fals
                                         "ms_fwd": round(mf, 4), "ms_bwd": round(mb, 4), **extra_graph})
 
 
+def dense_log2(lib, dev, B, M, K, N, reps):
+    """The second-order terms of logbmm (both cotangents given): one library call."""
+    torch.manual_seed(0)
+    a, b, g = torch.randn(B, M, K).to(dev), torch.randn(B, K, N).to(dev), torch.randn(B, M, N).to(dev)
+    ua, ub = torch.randn(B, M, K).to(dev), torch.randn(B, K, N).to(dev)
+    out = torch.empty(B, M, N, device=dev)
+    stats = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=dev)
+    ga, gb, gg = torch.empty_like(a), torch.empty_like(b), torch.empty_like(g)
+    s, p = _lib.stream_of(a), _lib.ptr
+    _lib.check(lib.genbmm_logbmm_fwd(p(a), p(b), p(out), p(stats), B, M, K, N, s), "fwd")
+
+    def bb():
+        _lib.check(lib.genbmm_logbmm_bwdbwd(p(a), p(b), p(out), p(g), p(ua), p(ub), p(ga), p(gb), p(gg), B, M, K, N, s),
+                   "bwdbwd")
+
+    ms = timed(bb, reps)
+    bmkn = float(B) * M * K * N
+    # three passes over (m, k, n), a weight and a multiply-add or two each: counted as 6 per term
+    report("logbmm double backward (%d,%d,%d,%d)" % (B, M, K, N), ms, 6 * bmkn,
+           4.0 * B * (3 * M * K + 3 * K * N + 4 * M * N))
+
+
 def dense_max(lib, dev, B, M, K, N, reps, prod):
     torch.manual_seed(0)
     if prod:
@@ -293,6 +315,7 @@ def main():
         dense_log(lib, dev, 16, 64, 64, 64, r, "logbmm fwd+bwd (16,64,64,64) config 0", dist="rand", graph=True)
         dense_log(lib, dev, 512, 128, 128, 128, r, "logbmm fwd+bwd (512,128,128,128) config 1")
         dense_log(lib, dev, 8192, 32, 32, 32, r, "logbmm fwd+bwd (8192,32,32,32) config 1 skinny")
+        dense_log2(lib, dev, 512, 128, 128, 128, max(3, r // 4))
         for path in (0, 2, 1):
             dense_log(lib, dev, 64, 512, 512, 512, r, "logbmm fwd+bwd (64,512,512,512) headline", path=path)
     if "max" in want:

@@ -33,8 +33,10 @@ constexpr size_t kStripLdsLimit = 64 * 1024;  // dynamic LDS available without o
 
 // Workspace of the log product: EA (B*n*Wa), EB (B*n*Wb), alpha (B*n), beta (B*n),
 // R (B*n*Wo) floats from the forward, and H (B*n*Wo) that the backward fills.
+inline bool dir_bwd_ok(const BandArgs& p);
+// (H only where the backward is not the memory-fed one, which forms it on the fly)
 inline size_t band_ws_floats(const BandArgs& p, int B) {
-  return (size_t)B * p.n * ((size_t)p.Wa + p.Wb + 2 * (size_t)p.Wo + 2);
+  return (size_t)B * p.n * ((size_t)p.Wa + p.Wb + (dir_bwd_ok(p) ? 1 : 2) * (size_t)p.Wo + 2);
 }
 // Which bands the strip kernels take (forward / backward): tiles within 64 KB of
 // LDS, the sliding tile large enough to double as the output staging tiles.
@@ -120,7 +122,7 @@ inline void set_workspace(BandArgs& p, float* ws, int B) {
   p.ws_al = p.ws_eb + rows * p.Wb;
   p.ws_be = p.ws_al + rows;
   p.ws_r = p.ws_be + rows;
-  p.ws_h = p.ws_r + rows * p.Wo;
+  p.ws_h = dir_bwd_ok(p) ? nullptr : p.ws_r + rows * p.Wo;
 }
 
 }  // namespace
@@ -133,6 +135,13 @@ size_t genbmm_banded_workspace_size(int a_lu, int a_ld, int b_lu, int b_ld, int 
   BandArgs p{};
   if (fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return 0;
   return band_ws_floats(p, B);
+}
+
+size_t genbmm_banded_scratch_size(int a_lu, int a_ld, int b_lu, int b_ld, int B, int n) {
+  using namespace genbmm;
+  BandArgs p{};
+  if (fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return 0;
+  return dir_bwd_ok(p) || !workspace_used(p) ? 0 : (size_t)B * n * p.Wo;
 }
 
 int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
@@ -319,7 +328,9 @@ int genbmm_banded_bwd_scratch(const float* a, int a_lu, int a_ld, const float* b
                               const float* out, const int32_t* idx, const float* workspace, float* scratch,
                               const float* g, float* grad_a, float* grad_b, int B, int n, int mode,
                               void* stream) {
-  if (workspace && !scratch) return GENBMM_E_NULLPTR;
+  if (workspace && !scratch && mode == GENBMM_BAND_LOG &&
+      genbmm_banded_scratch_size(a_lu, a_ld, b_lu, b_ld, B, n) != 0)
+    return GENBMM_E_NULLPTR;
   return genbmm::banded_bwd(a, a_lu, a_ld, b, b_lu, b_ld, out, idx, const_cast<float*>(workspace), scratch, g,
                             grad_a, grad_b, B, n, mode, stream);
 }

@@ -321,7 +321,10 @@ def banded_bwd(a: Tensor, b: Tensor, out: Tensor, aux: Tensor, g: Tensor, a_lu: 
     idx = aux if mode == _BAND_MAX else None
     ws = aux if mode == _BAND_LOG else None
     o = out if mode == _BAND_LOG else None
-    scratch = torch.empty(B * n * wo, dtype=_F32, device=a.device) if mode == _BAND_LOG else None
+    scratch = None
+    if mode == _BAND_LOG:
+        need = int(_lib.load().genbmm_banded_scratch_size(int(a_lu), int(a_ld), int(b_lu), int(b_ld), int(B), int(n)))
+        scratch = torch.empty(need, dtype=_F32, device=a.device) if need else None
     _call("genbmm_banded_bwd_scratch", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld, _lib.ptr(o),
           _lib.ptr(idx), _lib.ptr(ws), _lib.ptr(scratch), _lib.ptr(g), _lib.ptr(grad_a), _lib.ptr(grad_b), B, n, mode)
     return grad_a, grad_b

@@ -394,7 +394,10 @@ def _backward(a, b, bands, out, idx, g, mode, ws=None):
     # g / sum per output cell, which both gradients of the log product share, goes to a
     # buffer of this call's own: the forward's workspace stays as the forward left it, so
     # backward passes over one forward may overlap (other streams, retained graphs)
-    scratch = torch.empty_like(out) if (mode == MODE_LOG and ws is not None) else None
+    scratch = None
+    if mode == MODE_LOG and ws is not None:
+        need = _lib.load().genbmm_banded_scratch_size(a_lu, a_ld, b_lu, b_ld, B, n)
+        scratch = torch.empty(need, dtype=torch.float32, device=a.device) if need else None
     _call("genbmm_banded_bwd_scratch", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
           _lib.ptr(out), _lib.ptr(idx), _lib.ptr(ws), _lib.ptr(scratch), _lib.ptr(g), _lib.ptr(grad_a),
           _lib.ptr(grad_b), B, n, mode)

@@ -283,9 +283,19 @@ int genbmm_banded_bwd(const float* a, int a_lu, int a_ld,
                       int B, int n, int mode, void* stream);
 
 /*
+ * Floats that genbmm_banded_bwd_scratch needs in `scratch` for a log product of these
+ * bands; 0 where the backward keeps nothing beside the workspace (the kernels that
+ * form g/S while they read g: from 3 diagonals per operand up to about 160 in the
+ * result).  No counterpart in the reference, which allocates its temporaries itself.
+ */
+size_t genbmm_banded_scratch_size(int a_lu, int a_ld, int b_lu, int b_ld,
+                                  int B, int n);
+
+/*
  * genbmm_banded_bwd with the workspace left untouched: what the backward keeps
  * beside it (g/S per output cell, mode LOG with a workspace only) goes to
- * `scratch`, B * n * Wo floats, which must be given whenever `workspace` is.
+ * `scratch`, genbmm_banded_scratch_size floats, which must be given whenever
+ * `workspace` is and that size is not 0.
  * For callers that must not write to what the forward returned - operator
  * frameworks that check their inputs for mutation, or several backward calls
  * on one workspace at a time, each with a scratch buffer of its own.  Same

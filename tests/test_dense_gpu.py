@@ -226,6 +226,25 @@ def test_logbmm_double_backward(gpu, B, M, K, N):
         close(x, y, rtol=1e-9, atol=1e-11)
 
 
+def test_logbmm_double_backward_at_a_matrix_core_shape(gpu):
+    """Second-order terms on a shape whose forward and backward run on the matrix cores
+    ((8, 256, 128, 256): ragged nowhere, two 128-wide tiles a side), against float64
+    autograd with create_graph on two of the batch items."""
+    torch.manual_seed(17)
+    B, M, K, N = 8, 256, 128, 256
+    a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
+    ua, ub = torch.randn(B, M, K), torch.randn(B, K, N)
+    ad, bd, gd = (t.to(gpu).requires_grad_(True) for t in (a, b, g))
+    out = genbmm.logbmm(ad, bd)
+    ga, gb = torch.autograd.grad(out, (ad, bd), gd, create_graph=True)
+    got = torch.autograd.grad((ga, gb), (ad, bd, gd), (ua.to(gpu), ub.to(gpu)))
+    pick = [1, 6]
+    want = oracle.logbmm_second_order64(a[pick], b[pick], g[pick], ua[pick], ub[pick])
+    for x, y in zip(got, want):
+        # sums of up to 256 terms of magnitude |g u| <= ~20: absolute fp32 error well under 1e-4
+        close(x[pick], y, rtol=1e-4, atol=1e-4)
+
+
 # ------------------------------------------------------------ max / prod-max
 def grid(*shape):
     return torch.round(torch.randn(*shape) * 8) / 8
