@@ -63,6 +63,7 @@ SIGNATURES = {
 }
 STRING_FUNCS = {"genbmm_version": [], "genbmm_error_string": [_i]}
 SIZE_FUNCS = {"genbmm_logbmm_stats_size": [_i, _i, _i, _i],
+              "genbmm_samplebmm_stats_size": [_i, _i, _i, _i],
               "genbmm_logbmm_static_limit": [],
               "genbmm_banded_workspace_size": [_i, _i, _i, _i, _i, _i],
               "genbmm_banded_scratch_size": [_i, _i, _i, _i, _i, _i]}

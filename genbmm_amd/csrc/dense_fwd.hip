@@ -705,7 +705,7 @@ int run_sample(const float* a, const float* b, float* out, int32_t* idx, float* 
   p.a = a; p.b = b; p.out = out; p.idx = idx; p.seed = seed; p.offset = offset;
   hipStream_t s = (hipStream_t)stream;
   if (stats && K > 0) {  // log-sum-exp by the logbmm forward, then the multiply-only sweep
-    if (int e = genbmm_logbmm_fwd(a, b, out, stats, B, M, K, N, stream)) return e;
+    if (int e = log_fwd_with_factors(a, b, out, stats, B, M, K, N, s)) return e;
     LogFactors f;
     if (log_fwd_writes_factors(stats, B, M, K, N, &f)) {
       if (log_sample_mfma_ok(K)) {  // sweep on the matrix cores, groups of 16 terms

@@ -35,6 +35,7 @@
 #include "logbmm_item.h"
 #include "logbmm_mfma.h"
 #include "logbmm_item32.h"
+#include "logbmm_self.h"
 #include "logbmm_ws.h"
 
 namespace genbmm {
@@ -593,6 +594,12 @@ inline bool item_shape(int M, int K, int N) {
   return M >= 1 && K >= 1 && N >= 1 && M <= 64 && K <= 64 && N <= 64;
 }
 
+// Items of one 128 x 128 tile, each extent large enough for the tile to pay: forward
+// and backward form everything they need themselves (logbmm_self.h).
+inline bool self_shape(int M, int K, int N) {
+  return max(max(M, K), N) <= kSelfMax && min(min(M, K), N) >= 64 && !item_shape(M, K, N);
+}
+
 // Shapes whose forward runs on the matrix cores (given alignment and path).
 // Extents large enough for 128-wide tiles to pay; ragged edges, odd sizes and
 // unaligned rows are handled by the kernels.  (Measured down to a single batch item of 512^3, 16 tiles: the
@@ -835,8 +842,21 @@ void launch_item_fwd(const float* a, const float* b, float* out, float* stats, i
 
 // keep: the workspace is as large as genbmm_logbmm_stats_size says and receives what a
 // backward wants beside the maxima; false: header_offset() + 4 floats of it are used.
+int launch_self_fwd(DenseArgs p, float* stats, int B, int M, int K, int N, hipStream_t s) {
+  dim3 grid;
+  if (int e = fill_args<CfgWide>(p, B, M, K, N, grid)) return e;  // what the exact routine reads
+  int* hdr = prepared_of(stats, B, M, K, N).hdr;
+  if (M == kSelfMax && K == kSelfMax && N == kSelfMax)
+    hipLaunchKernelGGL(k_log_self_fwd<false>, dim3(B), dim3(256), 0, s, p, stats, hdr);
+  else
+    hipLaunchKernelGGL(k_log_self_fwd<true>, dim3(B), dim3(256), 0, s, p, stats, hdr);
+  return launch_status();
+}
+
+// factors: the caller wants EA, EB and 1/S in the workspace wherever a forward can leave
+// them (the sampling sweep), so the kernels that keep no by-products are not used.
 int run_fwd(const float* a, const float* b, float* out, float* stats, int B, int M, int K, int N,
-            int path, bool keep, hipStream_t s) {
+            int path, bool keep, hipStream_t s, bool factors = false) {
   if (int e = check_dense_dims(B, M, K, N)) return e;
   if (!valid_path(path)) return GENBMM_E_MODE;
   const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
@@ -850,12 +870,14 @@ int run_fwd(const float* a, const float* b, float* out, float* stats, int B, int
     else launch_item_fwd<16, 4, false>(a, b, out, stats, hdr, B, M, K, N, s);
     return launch_status();
   }
+  DenseArgs p{};
+  p.a = a; p.b = b; p.out = out; p.idx = nullptr;
+  if (stats && B > 0 && self_shape(M, K, N) && path == GENBMM_PATH_AUTO && !factors)
+    return launch_self_fwd(p, stats, B, M, K, N, s);
   if (stats) {
     if (int e = launch_stats(a, b, stats, B, M, K, N, s)) return e;
   }
   if (mn == 0) return GENBMM_OK;
-  DenseArgs p{};
-  p.a = a; p.b = b; p.out = out; p.idx = nullptr;
   if (stats && K > 0 && path != GENBMM_PATH_EXACT) {
     const int64_t big_tiles = (int64_t)B * ceil_div(M, 128) * ceil_div(N, 128);
     switch (fwd_mfma_shape(B, M, K, N) ? mfma_kind(path, B, M, N, K, false) : 0) {
@@ -899,6 +921,18 @@ int run_bwd_both(const float* a, const float* b, const float* out, const float* 
       hipLaunchKernelGGL((k_log_item_bwd<16, 2>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
     else
       hipLaunchKernelGGL((k_log_item_bwd<16, 4>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
+    return launch_status();
+  }
+  if (st && B > 0 && self_shape(M, K, N) && path == GENBMM_PATH_AUTO) {
+    LogBwdArgs pa = p, pb = p;
+    pa.grad = grad_a;
+    pb.grad = grad_b;
+    const int* hdr = prepared_of(st, B, M, K, N).hdr;
+    const dim3 grid((unsigned)ceil_div(B, 8) * 16);
+    if (M == kSelfMax && K == kSelfMax && N == kSelfMax)
+      hipLaunchKernelGGL(k_log_self_bwd<false>, grid, dim3(256), 0, s, pa, pb, st, hdr, B);
+    else
+      hipLaunchKernelGGL(k_log_self_bwd<true>, grid, dim3(256), 0, s, pa, pb, st, hdr, B);
     return launch_status();
   }
   if (st && grad_a && grad_b && mk > 0 && kn > 0 && fwd_mfma_shape(B, M, K, N)) {
@@ -968,6 +1002,11 @@ bool log_fwd_writes_factors(const float* stats, int B, int M, int K, int N, LogF
   return true;
 }
 
+int log_fwd_with_factors(const float* a, const float* b, float* out, float* stats, int B, int M, int K,
+                         int N, hipStream_t s) {
+  return run_fwd(a, b, out, stats, B, M, K, N, GENBMM_PATH_AUTO, true, s, true);
+}
+
 bool log_sample_mfma_ok(int K) { return ceil_div(K, kMS) <= kSampleSlabs; }
 
 int log_sample_sweep_mfma(const float* a, const float* b, float* out, int32_t* idx,
@@ -990,6 +1029,16 @@ int log_sample_sweep_mfma(const float* a, const float* b, float* out, int32_t* i
 extern "C" {
 
 size_t genbmm_logbmm_stats_size(int B, int M, int K, int N) {
+  using namespace genbmm;
+  if (check_dense_dims(B, M, K, N)) return 0;
+  int64_t n = header_offset(B, M, N) + 4;
+  // the one-tile kernels keep the maxima only
+  if (fwd_mfma_shape(B, M, K, N) && !self_shape(M, K, N))
+    n += (int64_t)B * ((int64_t)M * K + (int64_t)K * N + (int64_t)M * N);
+  return (size_t)n;
+}
+
+size_t genbmm_samplebmm_stats_size(int B, int M, int K, int N) {
   using namespace genbmm;
   if (check_dense_dims(B, M, K, N)) return 0;
   int64_t n = header_offset(B, M, N) + 4;

@@ -11,6 +11,7 @@ namespace genbmm {
 constexpr int kWsNone = 0;  // one that leaves no per-tile flags (exact and whole-item kernels)
 constexpr int kWsMfma = 1;  // the matrix-core forward: flags, EA, EB and 1/S
 constexpr int kWsFast = 2;  // the factored vector-ALU forward: flags only
+constexpr int kWsSelf = 3;  // the one-tile-per-item forward: the maxima only
 
 struct LogFactors {
   const float* ea;   // exp(a - row maximum), (B, M, K)
@@ -19,7 +20,12 @@ struct LogFactors {
   int* valid;        // the workspace's "factors present" word; clear it when scratch is overwritten
 };
 
-// True (and *f filled) if a genbmm_logbmm_fwd call with this workspace and these sizes
+// genbmm_logbmm_fwd, except that shapes whose forward would keep nothing but the maxima
+// take the kernels that leave the factors (what log_fwd_writes_factors() describes).
+int log_fwd_with_factors(const float* a, const float* b, float* out, float* stats, int B, int M, int K,
+                         int N, hipStream_t s);
+
+// True (and *f filled) if a log_fwd_with_factors call with this workspace and these sizes
 // writes the factors: the same decision the forward takes, made on the host.
 bool log_fwd_writes_factors(const float* stats, int B, int M, int K, int N, LogFactors* f);
 

@@ -280,7 +280,7 @@ class SampleMatMul(torch.autograd.Function):
             _call("genbmm_samplebmm_fwd_f64", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out),
                   _lib.ptr(idx), seed, offset, B, M, K, N)
         else:
-            stats = torch.empty(_lib.load().genbmm_logbmm_stats_size(B, M, K, N), dtype=_COMPUTE,
+            stats = torch.empty(_lib.load().genbmm_samplebmm_stats_size(B, M, K, N), dtype=_COMPUTE,
                                 device=a.device)
             _call("genbmm_samplebmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
                   _lib.ptr(stats), seed, offset, B, M, K, N)

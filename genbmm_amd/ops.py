@@ -148,7 +148,8 @@ def samplebmm_fwd(a: Tensor, b: Tensor, seed: int, offset: int) -> Tuple[Tensor,
     B, M, K, N = _check(a, b)
     out = torch.empty(B, M, N, dtype=_F32, device=a.device)
     idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
-    stats = torch.empty(_stats_size(B, M, K, N), dtype=_F32, device=a.device)
+    stats = torch.empty(int(_lib.load().genbmm_samplebmm_stats_size(int(B), int(M), int(K), int(N))),
+                        dtype=_F32, device=a.device)
     _call("genbmm_samplebmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), _lib.ptr(stats),
           seed & 0xFFFFFFFFFFFFFFFF, offset & 0xFFFFFFFFFFFFFFFF, B, M, K, N)
     return out, idx

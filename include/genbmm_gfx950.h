@@ -74,9 +74,13 @@ const char* genbmm_error_string(int code);
  * behind them sit per-tile flags naming the tiles where it is not, which a
  * fix-up launch recomputes with the online kernel's routine, a header naming
  * the kernels that filled the buffer, and - for shapes that run on the matrix
- * cores (M and N at least 96, K at least 16) - exp(a-max), exp(b-max) and
- * 1/sum, which the backward then reads instead of taking any exponential
- * itself.  The contents belong to the library; the buffer takes the place of
+ * cores (M and N at least 96, K at least 16) and do not fit one 128 x 128 tile
+ * per batch item - exp(a-max), exp(b-max) and 1/sum, which the backward then
+ * reads instead of taking any exponential itself.  Items of one tile (every
+ * extent between 64 and 128) keep the maxima alone: forward and backward each
+ * form what they need in one launch, and a tile that cannot be factored is
+ * redone by the exact routine inside that launch.
+ * The contents belong to the library; the buffer takes the place of
  * the reference's (B, M, N) `maxes` output; pass the same buffer, unchanged,
  * to genbmm_logbmm_bwd.
  */
@@ -105,6 +109,13 @@ int genbmm_logbmm_bwd(const float* a, const float* b, const float* out,
 
 /* Number of fp32 elements genbmm_logbmm_fwd / _bwd need in `stats`. */
 size_t genbmm_logbmm_stats_size(int B, int M, int K, int N);
+
+/*
+ * Number of fp32 elements genbmm_samplebmm_fwd needs in its `stats` (never less
+ * than genbmm_logbmm_stats_size: the sampling sweep always wants the factors
+ * where a forward can leave them).  No counterpart in the reference.
+ */
+size_t genbmm_samplebmm_stats_size(int B, int M, int K, int N);
 
 /*
  * The same two functions with the kernel family named per call (tests and
@@ -196,8 +207,8 @@ int genbmm_prodmaxbmm_fwd(const float* a, const float* b, float* out,
  * A cell whose scan never crosses its uniform keeps index 0, as in the
  * reference.  Replaces _genbmm.forward(a, b, 2): matmul_cuda_kernel.cu:512-526
  * (torch::rand at :517), kernel :77-121.
- * `stats`: NULL, or a buffer of genbmm_logbmm_stats_size(B,M,K,N) floats as for
- * genbmm_logbmm_fwd; with it the log-sum-exp comes from the logbmm forward and
+ * `stats`: NULL, or a buffer of genbmm_samplebmm_stats_size(B,M,K,N) floats, used
+ * like that of genbmm_logbmm_fwd; with it the log-sum-exp comes from the logbmm forward and
  * the CDF walk multiplies staged exp(a-max)*exp(b-max) instead of taking one
  * exponential per term (tiles where that is not exact walk the exact way).
  */

@@ -49,7 +49,8 @@ def logbmm_on(path):
 
 
 SHAPES = [(16, 64, 64, 64), (3, 7, 9, 5), (2, 1, 1, 1), (4, 5, 1, 6), (5, 33, 70, 129), (2, 130, 17, 66),
-          (3, 64, 64, 128), (2, 200, 96, 260), (9, 32, 32, 32), (7, 31, 33, 29), (1, 256, 40, 256)]
+          (3, 64, 64, 128), (2, 200, 96, 260), (9, 32, 32, 32), (7, 31, 33, 29), (1, 256, 40, 256),
+          (6, 128, 128, 128), (11, 100, 70, 128), (3, 65, 64, 64), (9, 127, 99, 101)]
 
 
 @pytest.mark.parametrize("B,M,K,N", SHAPES)
@@ -178,6 +179,65 @@ def test_logbmm_factoring_guard_matrix_core_tiles(gpu, B, M, K, N):
     close(gb[pick.to(gpu)], wb)
     close(ga.sum(-1), g.double().sum(-1), atol=2e-4)
     close(gb.sum(-2), g.double().sum(-2), atol=2e-4)
+
+
+@pytest.mark.parametrize("B,M,K,N", [(20, 128, 128, 128), (17, 100, 70, 128), (12, 64, 128, 65), (9, 127, 99, 101)])
+def test_logbmm_one_tile_items(gpu, B, M, K, N):
+    """Items of at most 128 in every extent: one workgroup per item (and gradient) that
+    takes the maxima, the factors and the guard itself.  Items that need the exact routine
+    (underflowing factors in every row, in one row, masked terms, a fully masked row) sit
+    between items that do not; either gradient alone; a workspace another forward filled."""
+    lib = _lib.load()
+    torch.manual_seed(B + M)
+    a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
+    a[1, ::2, 0] += 200.0
+    b[1, 0, :] -= 200.0
+    a[4, 37, 5] += 200.0
+    b[4, 5, :] -= 200.0
+    a[6, :, ::2] = -2e9   # every term of item 6 below the -1e9 floor -> -inf
+    b[6, 1::2, :] = -2e9
+    b[7, 3, :] = -math.inf  # one masked k
+    fin = torch.tensor([i for i in range(B) if i != 6])
+    want, wa, wb = oracle.logbmm_grads64(a[fin], b[fin], g[fin])
+    ad, bd, gd = a.to(gpu), b.to(gpu), g.to(gpu)
+    out, ga, gb = torch.empty(B, M, N, device=gpu), torch.empty_like(ad), torch.empty_like(bd)
+    size = lib.genbmm_logbmm_stats_size(B, M, K, N)
+    # maxima, one flag word per 32 x 32 cells, header: no copy of any operand
+    assert size <= B * (M + N) + B * 16 + 8 and lib.genbmm_samplebmm_stats_size(B, M, K, N) >= size
+    stats = torch.full((size,), float("nan"), device=gpu)
+    p, s = _lib.ptr, _lib.stream_of(ad)
+    assert lib.genbmm_logbmm_fwd(p(ad), p(bd), p(out), p(stats), B, M, K, N, s) == 0
+    close(out[fin.to(gpu)], want)
+    assert bool(torch.isinf(out[6]).all())
+    # the maxima are in the workspace for the backward
+    close(stats[: B * (M + N)].view(B, M + N)[:, :M], a.amax(-1), rtol=0, atol=0)
+    close(stats[: B * (M + N)].view(B, M + N)[:, M:], b.amax(-2), rtol=0, atol=0)
+    before = stats.clone()
+    assert lib.genbmm_logbmm_bwd(p(ad), p(bd), p(out), p(gd), p(stats), p(ga), p(gb), B, M, K, N, s) == 0
+    assert torch.equal(before.view(torch.int32), stats.view(torch.int32))  # the backward only reads it
+    close(ga[fin.to(gpu)], wa)
+    close(gb[fin.to(gpu)], wb)
+    ok = torch.tensor([i for i in range(B) if i not in (6, 7)])
+    close(ga[ok.to(gpu)].sum(-1), g[ok].double().sum(-1), atol=2e-4)
+    close(gb[ok.to(gpu)].sum(-2), g[ok].double().sum(-2), atol=2e-4)
+    # either gradient alone
+    ga1, gb1 = torch.full_like(ad, 7.0), torch.full_like(bd, 7.0)
+    assert lib.genbmm_logbmm_bwd(p(ad), p(bd), p(out), p(gd), p(stats), p(ga1), p(None), B, M, K, N, s) == 0
+    assert lib.genbmm_logbmm_bwd(p(ad), p(bd), p(out), p(gd), p(stats), p(None), p(gb1), B, M, K, N, s) == 0
+    assert torch.equal(ga1[fin.to(gpu)], ga[fin.to(gpu)]) and torch.equal(gb1[fin.to(gpu)], gb[fin.to(gpu)])
+    # a workspace filled by the vector-ALU forward (same maxima, other tag), and one filled by
+    # nothing at all (every item falls back to the exact routine)
+    out2 = torch.empty_like(out)
+    assert lib.genbmm_logbmm_fwd_path(p(ad), p(bd), p(out2), p(stats), B, M, K, N, genmul.PATH_VALU, s) == 0
+    close(out2[fin.to(gpu)], want)
+    ga2, gb2 = torch.empty_like(ad), torch.empty_like(bd)
+    assert lib.genbmm_logbmm_bwd(p(ad), p(bd), p(out2), p(gd), p(stats), p(ga2), p(gb2), B, M, K, N, s) == 0
+    close(ga2[fin.to(gpu)], wa)
+    close(gb2[fin.to(gpu)], wb)
+    stats.zero_()
+    assert lib.genbmm_logbmm_bwd(p(ad), p(bd), p(out), p(gd), p(stats), p(ga2), p(gb2), B, M, K, N, s) == 0
+    close(ga2[fin.to(gpu)], wa)
+    close(gb2[fin.to(gpu)], wb)
 
 
 def test_logbmm_backward_on_foreign_workspace(gpu):
@@ -423,7 +483,7 @@ def test_sample_index_brackets_cdf(gpu, use_stats, B, M, K, N):
     ad, bd = a.to(gpu), b.to(gpu)
     out = torch.empty(B, M, N, device=gpu)
     idx = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
-    stats = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=gpu) if use_stats else None
+    stats = torch.empty(lib.genbmm_samplebmm_stats_size(B, M, K, N), device=gpu) if use_stats else None
     rc = lib.genbmm_samplebmm_fwd(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx), _lib.ptr(stats),
                                   seed, offset, B, M, K, N, _lib.stream_of(ad))
     assert rc == 0
@@ -467,7 +527,7 @@ def test_sample_config_c4_chi_square(gpu):
     lib = _lib.load()
     idx = torch.empty(A.shape[0], 16, 16, dtype=torch.int32, device=gpu)
     o2 = torch.empty_like(out)
-    st = torch.empty(lib.genbmm_logbmm_stats_size(A.shape[0], 16, 512, 16), device=gpu)
+    st = torch.empty(lib.genbmm_samplebmm_stats_size(A.shape[0], 16, 512, 16), device=gpu)
     lib.genbmm_samplebmm_fwd(_lib.ptr(A), _lib.ptr(Bm), _lib.ptr(o2), _lib.ptr(idx), _lib.ptr(st), 1234, 0,
                              A.shape[0], 16, 512, 16, _lib.stream_of(A))
     assert torch.equal(o2, out.detach())
@@ -516,7 +576,7 @@ def test_sample_config_c4_at_full_size(gpu):
     ad, bd = a.to(gpu), b.to(gpu)
     out = torch.empty(B, M, N, device=gpu)
     idx = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
-    stats = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=gpu)
+    stats = torch.empty(lib.genbmm_samplebmm_stats_size(B, M, K, N), device=gpu)
     p, s = _lib.ptr, _lib.stream_of(ad)
 
     def draw(offset):
@@ -586,7 +646,7 @@ def test_sample_distribution_on_the_matrix_core_sweep(gpu):
     ad, bd = a.to(gpu), b.to(gpu)
     out = torch.empty(B, M, N, device=gpu)
     idx = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
-    stats = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=gpu)
+    stats = torch.empty(lib.genbmm_samplebmm_stats_size(B, M, K, N), device=gpu)
     counts = torch.zeros(B * M * N, K, device=gpu)
     cells = torch.arange(B * M * N, device=gpu)
     for d in range(draws):

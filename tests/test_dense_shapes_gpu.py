@@ -78,7 +78,7 @@ def test_sample_on_many_shapes(gpu):
         ad, bd = a.to(gpu), b.to(gpu)
         out = torch.empty(B, M, N, device=gpu)
         idx = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
-        stats = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=gpu)
+        stats = torch.empty(lib.genbmm_samplebmm_stats_size(B, M, K, N), device=gpu)
         assert lib.genbmm_samplebmm_fwd(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx), _lib.ptr(stats),
                                         77, 3, B, M, K, N, _lib.stream_of(ad)) == 0
         u = oracle.philox_uniform(0, B * M * N, 77, 3).view(B, M, N).double()
@@ -108,7 +108,7 @@ def test_sample_on_flat_and_peaked_distributions(gpu, scale):
     ad, bd = a.to(gpu), b.to(gpu)
     out = torch.empty(B, M, N, device=gpu)
     idx = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
-    stats = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=gpu)
+    stats = torch.empty(lib.genbmm_samplebmm_stats_size(B, M, K, N), device=gpu)
     assert lib.genbmm_samplebmm_fwd(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx), _lib.ptr(stats),
                                     5, 11, B, M, K, N, _lib.stream_of(ad)) == 0
     u = oracle.philox_uniform(0, B * M * N, 5, 11).view(B, M, N).double()
