@@ -155,7 +155,7 @@ def dense_sample(lib, dev, B, M, K, N, reps):
     ga, gb = torch.empty_like(a), torch.empty_like(b)
     s, p = _lib.stream_of(a), _lib.ptr
 
-    stats = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=dev)
+    stats = torch.empty(lib.genbmm_samplebmm_stats_size(B, M, K, N), device=dev)
 
     def f():
         _lib.check(lib.genbmm_samplebmm_fwd(p(a), p(b), p(out), p(idx), p(stats), 1234, 0, B, M, K, N, s), "fwd")
@@ -323,6 +323,7 @@ def main():
         dense_max(lib, dev, 256, 256, 256, 256, r, prod=True)
     if "sample" in want:
         dense_sample(lib, dev, 64, 512, 512, 512, r)
+        dense_sample(lib, dev, 16, 512, 1024, 512, r)  # K beyond the matrix-core sweep's 992
     if "banded" in want:
         for mode in (3, 0, 1):
             banded(lib, dev, 64, 4096, 32, 32, mode, r)

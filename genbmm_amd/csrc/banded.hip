@@ -100,6 +100,21 @@ inline void launch_max_fwd(const BandArgs& p, int B, hipStream_t s) {
                      rows * p.Wa, rows * p.Wb);
 }
 
+// EA, alpha and EB, beta of a log product into the workspace set_workspace() has laid out.
+inline void launch_prep(const BandArgs& p, const float* a, int a_lu, const float* b, int b_lu, int B,
+                        hipStream_t s) {
+  const long rows = (long)B * p.n;
+  const PrepSide pa{a, p.ws_ea, p.ws_al, p.Wa, a_lu, odd(p.Wa)}, pb{b, p.ws_eb, p.ws_be, p.Wb, b_lu, odd(p.Wb)};
+  const int blocks_a = (int)((rows + kPrepRows - 1) / kPrepRows), blocks_b = blocks_a;
+  const size_t lds = sizeof(float) * (size_t)kPrepRows * max(pa.ld, pb.ld);
+  const int vec = aligned16(a) && aligned16(b) && aligned16(p.ws_ea) && aligned16(p.ws_eb);
+  if (lds > kStripLdsLimit)
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_band_prep), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)lds);
+  hipLaunchKernelGGL(k_band_prep, dim3((unsigned)(blocks_a + blocks_b)), dim3(256), lds, s, pa, pb, p.n, rows,
+                     blocks_a, vec);
+}
+
 template <int KIND, bool PREP>
 inline void launch_dir(const BandArgs& p, int B, hipStream_t s) {
   const int blocks = ceil_div(p.n, 16 * kDirWaves);
@@ -163,13 +178,7 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   if (dir && (mode == GENBMM_BAND_MUL || prep_fwd(p, mode, workspace))) {
     if (mode == GENBMM_BAND_LOG) {
       set_workspace(p, workspace, B);
-      const long rows = (long)B * n;
-      const dim3 pg((unsigned)((rows + kPrepRows - 1) / kPrepRows));
-      const int lda = odd(p.Wa), ldb = odd(p.Wb);
-      hipLaunchKernelGGL(k_band_prep, pg, dim3(256), sizeof(float) * kPrepRows * lda, s, a, p.ws_ea,
-                         p.ws_al, p.Wa, a_lu, n, rows, lda);
-      hipLaunchKernelGGL(k_band_prep, pg, dim3(256), sizeof(float) * kPrepRows * ldb, s, b, p.ws_eb,
-                         p.ws_be, p.Wb, b_lu, n, rows, ldb);
+      launch_prep(p, a, a_lu, b, b_lu, B, s);
       launch_dir<kDirFwd, true>(p, B, s);
     } else {
       launch_dir<kDirFwd, false>(p, B, s);
@@ -192,13 +201,7 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
     const bool prep = prep_fwd(p, mode, workspace);
     if (prep) {  // EA, alpha and EB, beta once, instead of per strip and chunk
       set_workspace(p, workspace, B);
-      const long rows = (long)B * n;
-      const dim3 pg((unsigned)((rows + kPrepRows - 1) / kPrepRows));
-      const int lda = odd(p.Wa), ldb = odd(p.Wb);
-      hipLaunchKernelGGL(k_band_prep, pg, dim3(256), sizeof(float) * kPrepRows * lda, s, a, p.ws_ea,
-                         p.ws_al, p.Wa, a_lu, n, rows, lda);
-      hipLaunchKernelGGL(k_band_prep, pg, dim3(256), sizeof(float) * kPrepRows * ldb, s, b, p.ws_eb,
-                         p.ws_be, p.Wb, b_lu, n, rows, ldb);
+      launch_prep(p, a, a_lu, b, b_lu, B, s);
     }
     auto pick = [&](auto nqc) {
       constexpr int Q = decltype(nqc)::value;

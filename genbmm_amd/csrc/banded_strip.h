@@ -136,64 +136,113 @@ struct RowStage {
 // there is none), e = exp(x - shift), 0 for cells outside.  With these the log
 // product is a (+,x) product of e's plus an epilogue, and no kernel downstream
 // takes an exponential per staged element again.
-constexpr int kPrepRows = 64;  // band rows per workgroup: one contiguous block of memory
+// Both operands in one launch.  A workgroup takes R consecutive band rows of one operand -
+// one contiguous block of memory, moved 16 bytes per lane in both directions - and turns them
+// in LDS (row stride ld, odd) so that 256 / R lanes share a row.
+struct PrepSide {
+  const float* x;
+  float* e;
+  float* shift;
+  int W, lu, ld;
+};
+constexpr int kPrepRows = 64;  // measured against 128 and 256: the row pass is the slow part, and
+                               // it is faster with four lanes to a row
 
-__global__ __launch_bounds__(256) void k_band_prep(const float* __restrict__ x, float* __restrict__ e,
-                                                   float* __restrict__ shift, int W, int lu, int n,
-                                                   long rows, int ld) {
-  extern __shared__ __attribute__((aligned(16))) float tile[];  // [64][ld], ld odd
-  const int tid = threadIdx.x;
-  const long row0 = (long)blockIdx.x * kPrepRows;
-  const int nr = (int)min((long)kPrepRows, rows - row0);
-  const float* xb = x + row0 * W;
-  float* eb = e + row0 * W;
-  // the block is contiguous in memory: coalesced in (batches of reads in flight together),
-  // rows inside, coalesced out
+template <int R>
+__device__ __forceinline__ void band_prep_block(const PrepSide& q, float* __restrict__ tile, int n, long rows,
+                                                long row0, int vec) {
+  constexpr int PARTS = 256 / R;
+  const int tid = threadIdx.x, W = q.W, ld = q.ld;
+  const int nr = (int)min((long)R, rows - row0);
+  const int cells = nr * W;
+  const float* xb = q.x + row0 * W;
+  float* eb = q.e + row0 * W;
   constexpr int U = 8;
-  for (int i0 = tid, r = tid / W, k = tid - (tid / W) * W; i0 < nr * W; i0 += 256 * U) {
-    float v[U];
+  // Index arithmetic is what this kernel would otherwise spend its time on: the LDS offset of a
+  // lane's 16-byte piece advances by a fixed step with one carry, and each of its four cells
+  // adds the row gap if it lies past the row end - no division, no branch.
+  const int quads = (vec && W >= 4) ? cells >> 2 : 0;  // W >= 4: a piece straddles at most one row end
+  const int dr = 1024 / W, dk = 1024 - dr * W;        // 256 lanes x 4 cells between a lane's pieces
+  const int gap = ld - W, step = dr * ld + dk;
+  const int r_first = (4 * tid) / W, k_first = 4 * tid - r_first * W;
+  {
+    int k = k_first, base = r_first * ld + k_first;  // base: LDS offset of the piece's first cell
+    for (int i0 = tid; i0 < quads; i0 += 256 * U) {
+      float4 v[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) v[u] = i0 + 256 * u < nr * W ? xb[i0 + 256 * u] : 0.f;
+      for (int u = 0; u < U; ++u)
+        if (i0 + 256 * u < quads) v[u] = *reinterpret_cast<const float4*>(xb + 4 * (i0 + 256 * u));
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      if (i0 + 256 * u < nr * W) tile[r * ld + k] = v[u];
-      r += 256 / W;
-      k += 256 % W;
-      if (k >= W) {
-        k -= W;
-        ++r;
+      for (int u = 0; u < U; ++u) {
+        if (i0 + 256 * u < quads) {
+          tile[base] = v[u].x;
+          tile[base + 1 + (k + 1 >= W ? gap : 0)] = v[u].y;
+          tile[base + 2 + (k + 2 >= W ? gap : 0)] = v[u].z;
+          tile[base + 3 + (k + 3 >= W ? gap : 0)] = v[u].w;
+        }
+        k += dk;
+        base += step;
+        if (k >= W) {
+          k -= W;
+          base += gap;
+        }
       }
     }
+    for (int i = 4 * quads + tid; i < cells; i += 256) tile[(i / W) * ld + i % W] = xb[i];
   }
   __syncthreads();
-  {  // four lanes per row, a quarter of its cells each
-    const int r = tid >> 2, part = tid & 3;
-    const int q = (W + 3) >> 2, k0 = part * q, k1 = min(W, k0 + q);
+  {
+    const int r = tid / PARTS, part = tid % PARTS;
+    const int per = (W + PARTS - 1) / PARTS, k0 = part * per, k1 = min(W, k0 + per);
     const bool live = r < nr;
-    const int c = live ? (int)((row0 + r) % n) : 0;
-    const int klo = max(0, lu - c), khi = min(W - 1, n - 1 + lu - c);  // cells inside the matrix
+    const int c = live ? (int)((unsigned)((row0 + r) % n)) : 0;
+    // cells of this lane's share that lie inside the matrix: k in [lo, hi)
+    const int lo = max(k0, max(0, q.lu - c)), hi = live ? min(k1, min(W - 1, n - 1 + q.lu - c) + 1) : lo;
     float* tr = tile + r * ld;
     float m = -INFINITY;
-    if (live)
-      for (int k = max(k0, klo); k < min(k1, khi + 1); ++k) m = fmaxf(m, tr[k]);
-    m = fmaxf(m, __shfl_xor(m, 1, 64));
-    m = fmaxf(m, __shfl_xor(m, 2, 64));
-    if (live) {
-      if (part == 0) shift[row0 + r] = m;
-      const float sh = m == -INFINITY ? 0.f : m;
-      for (int k = k0; k < k1; ++k) tr[k] = (k >= klo && k <= khi) ? fast_exp2((tr[k] - sh) * kLog2e) : 0.f;
+    // every lane walks its whole share (a uniform trip count); cells outside take no part
+#pragma unroll 4
+    for (int k = k0; k < k0 + per; ++k) {
+      const bool in = k >= lo && k < hi;
+      const float x = tr[in ? k : 0];
+      m = in ? fmaxf(m, x) : m;
+    }
+#pragma unroll
+    for (int o = 1; o < PARTS; o <<= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    if (live && part == 0) q.shift[row0 + r] = m;
+    const float sh = m == -INFINITY ? 0.f : m;
+#pragma unroll 4
+    for (int k = k0; k < k0 + per; ++k) {
+      const bool in = k >= lo && k < hi;
+      const float e = fast_exp2((tr[in ? k : 0] - sh) * kLog2e);
+      if (live && k < k1) tr[k] = in ? e : 0.f;
     }
   }
   __syncthreads();
-  for (int i = tid, r = tid / W, k = tid - (tid / W) * W; i < nr * W; i += 256) {
-    eb[i] = tile[r * ld + k];
-    r += 256 / W;
-    k += 256 % W;
-    if (k >= W) {
-      k -= W;
-      ++r;
+  {
+    int k = k_first, base = r_first * ld + k_first;
+    for (int i = tid; i < quads; i += 256) {
+      const float4 w = make_float4(tile[base], tile[base + 1 + (k + 1 >= W ? gap : 0)],
+                                   tile[base + 2 + (k + 2 >= W ? gap : 0)], tile[base + 3 + (k + 3 >= W ? gap : 0)]);
+      *reinterpret_cast<float4*>(eb + 4 * i) = w;
+      k += dk;
+      base += step;
+      if (k >= W) {
+        k -= W;
+        base += gap;
+      }
     }
+    for (int i = 4 * quads + tid; i < cells; i += 256) eb[i] = tile[(i / W) * ld + i % W];
   }
+}
+
+// Workgroups [0, blocks_a) take the first operand, the rest the second.
+__global__ __launch_bounds__(256) void k_band_prep(const PrepSide pa, const PrepSide pb, int n, long rows,
+                                                   int blocks_a, int vec) {
+  extern __shared__ __attribute__((aligned(16))) float tile[];
+  const bool first = (int)blockIdx.x < blocks_a;
+  const long row0 = (long)(first ? blockIdx.x : blockIdx.x - blocks_a) * kPrepRows;
+  band_prep_block<kPrepRows>(first ? pa : pb, tile, n, rows, row0, vec);
 }
 
 // ------------------------------------------------------------------ forward
