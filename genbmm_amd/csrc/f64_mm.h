@@ -31,10 +31,41 @@
 namespace genbmm {
 
 constexpr int kDC = 16;        // contraction chunk
-constexpr int kDP = kDC + 2;   // row pitch of a staged chunk, in doubles
+constexpr int kDP = kDC + 1;   // row pitch of a staged chunk, in doubles: odd, so that lanes four rows apart
+                               // (the staging stores of an operand whose rows run along the reduction) and
+                               // lanes one row apart (everything else) both spread over all LDS banks
 constexpr double kDFloor = -1e9;
 constexpr double kDThr = 1e-280;
 constexpr double kDLogThr = -644.7;  // log(kDThr), rounded up
+
+// exp for the factors (one per staged element: what these kernels spend their vector time on).
+// The arguments are shifted operands (<= 0) and -log S (guarded to <= 645): finite results
+// only, so no overflow handling; anything below -800 gives 0 and NaN stays NaN.  Reduction by
+// ln 2 in two parts (the high part has 21 trailing zero bits, so n * hi is exact), Taylor
+// polynomial of degree 13 on |r| <= 0.347 (truncation 4e-18), scaling by v_ldexp_f64:
+// about 20 instructions against the 80 of the library routine, within 2 ulp of it.
+// The coefficients live in constant memory and are not `const`: the compiler then reads them
+// with scalar loads into scalar registers, where v_fma_f64 takes them as its addend.  As
+// literals every one of them costs a 64-bit move per use (the instruction has no room for a
+// 64-bit immediate), which doubles the polynomial.
+__constant__ double d64_exp_c[16] = {1.0 / 6227020800.0, 1.0 / 479001600.0, 1.0 / 39916800.0, 1.0 / 3628800.0,
+                                     1.0 / 362880.0,     1.0 / 40320.0,     1.0 / 5040.0,     1.0 / 720.0,
+                                     1.0 / 120.0,        1.0 / 24.0,        1.0 / 6.0,        0.5,
+                                     1.44269504088896340736, -6.93147180369123816490e-01,
+                                     -1.90821492927058770002e-10, -800.0};
+__device__ __forceinline__ double d64_exp(double x) {
+  const double* c = d64_exp_c;
+  x = x < c[15] ? c[15] : x;
+  const double n = __builtin_rint(x * c[12]);
+  double r = __builtin_fma(n, c[13], x);
+  r = __builtin_fma(n, c[14], r);
+  double p = c[0];
+#pragma unroll
+  for (int i = 1; i < 12; ++i) p = __builtin_fma(p, r, c[i]);
+  p = __builtin_fma(p, r, 1.0);
+  p = __builtin_fma(p, r, 1.0);
+  return __builtin_ldexp(p, (int)n);
+}
 constexpr int kDMaxAll = 4096;  // grad_a keeps beta of every column in LDS, grad_b alpha of every row
 typedef double mmd4 __attribute__((ext_vector_type(4)));
 
@@ -131,7 +162,7 @@ __global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ 
   auto h_of = [&](double gv, double ov, double am, double bn) __attribute__((always_inline)) {
     const double sh = d64_shift(am) + d64_shift(bn), ls = ov - sh;  // ls = log S
     const bool ok = d64_usable(sh) && ls >= kDLogThr && ls < INFINITY;
-    return ok ? gv * exp(-ls) : __builtin_nan("");
+    return ok ? gv * d64_exp(-ls) : __builtin_nan("");
   };
   auto put = [&](int l0) __attribute__((always_inline)) {
 #pragma unroll
@@ -140,24 +171,23 @@ __global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ 
       {
         const int il = 64 * h + pl_line + (P_L ? 0 : e), ll = pl_l + (P_L ? e : 0);
         const int i = i0 + il, l = l0 + ll;
-        double v = 0.0;
-        if (i < I && l < L) {
-          if (FWD) v = exp(rp[eh] - d64_shift(al[il]));
-          if (GA) v = h_of(rp[eh], rp2[eh], al[il], be[l]);
-          if (GB) v = exp(rp[eh] - d64_shift(al[l]));
-        }
-        Ps[il * kDP + ll] = v;
+        // (computed for cells beyond the matrix too, then dropped: a select, not a branch)
+        const int lc = min(l, L - 1);
+        double v;
+        if (FWD) v = d64_exp(rp[eh] - d64_shift(al[il]));
+        if (GA) v = h_of(rp[eh], rp2[eh], al[il], be[lc]);
+        if (GB) v = d64_exp(rp[eh] - d64_shift(al[lc]));
+        Ps[il * kDP + ll] = (i < I && l < L) ? v : 0.0;
       }
       {
         const int jl = 64 * h + ql_line + (Q_L ? 0 : e), ll = ql_l + (Q_L ? e : 0);
         const int j = j0 + jl, l = l0 + ll;
-        double v = 0.0;
-        if (j < J && l < L) {
-          if (FWD) v = exp(rq[eh] - d64_shift(be[jl]));
-          if (GA) v = exp(rq[eh] - d64_shift(be[l]));
-          if (GB) v = h_of(rq[eh], rq2[eh], al[l], be[jl]);
-        }
-        Qs[jl * kDP + ll] = v;
+        const int lc = min(l, L - 1);
+        double v;
+        if (FWD) v = d64_exp(rq[eh] - d64_shift(be[jl]));
+        if (GA) v = d64_exp(rq[eh] - d64_shift(be[lc]));
+        if (GB) v = h_of(rq[eh], rq2[eh], al[lc], be[jl]);
+        Qs[jl * kDP + ll] = (j < J && l < L) ? v : 0.0;
       }
     }
   };
@@ -218,7 +248,7 @@ __global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ 
           }
         } else if (GA) {  // i = m, j = k
           const double av = ab[(long)i * K + j];
-          res = exp(av - d64_shift(al[il])) * v;
+          res = d64_exp(av - d64_shift(al[il])) * v;
           if (!(fabs(res) <= DBL_MAX)) {  // matmul_cuda_kernel.cu:159-184
             double s = 0.0;
             for (int n = 0; n < N; ++n)
@@ -227,7 +257,7 @@ __global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ 
           }
         } else {  // i = k, j = n
           const double bv = bb[(long)i * N + j];
-          res = exp(bv - d64_shift(be[jl])) * v;
+          res = d64_exp(bv - d64_shift(be[jl])) * v;
           if (!(fabs(res) <= DBL_MAX)) {  // matmul_cuda_kernel.cu:190-217
             double s = 0.0;
             for (int m = 0; m < M; ++m)
