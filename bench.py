@@ -32,9 +32,12 @@ def cpu_baseline(torch, sample_batches=64):
     chunk (a 512 MB fp32 intermediate each)."""
     import oracle
 
-    cores = os.cpu_count() or 1
-    cores = min(cores, 16)  # the GPU box grants 16 host cores to a one-GPU job
-    torch.set_num_threads(cores)
+    # the threads torch's CPU kernels run on: OMP_NUM_THREADS where the host sets it, else the
+    # cores this process may be scheduled on
+    cores = torch.get_num_threads()
+    if "OMP_NUM_THREADS" not in os.environ and hasattr(os, "sched_getaffinity"):
+        cores = len(os.sched_getaffinity(0))
+        torch.set_num_threads(cores)
     torch.manual_seed(0)
     a = torch.randn(sample_batches, M, K)
     b = torch.randn(sample_batches, K, N)

@@ -478,11 +478,6 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
   const int Q = GRAD_A ? N : M;                      // reduction extent
   const int R = GRAD_A ? M : K, Cc = GRAD_A ? K : N;  // output extents
 
-  // forward flags over the cells this tile reduces over: the fix-up launch takes the tile
-  if (bwd_tile_flagged(ws_hdr, fwd_flags, true, GRAD_A, GRAD_A ? r0 : c0, GRAD_A ? T::TR : T::TC, batch,
-                       M, N, tid, NT))
-    return;
-
   floatx16 acc[2][2];
 #pragma unroll
   for (int x = 0; x < 4; ++x)
@@ -563,6 +558,12 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
   };
 
   load(slabs == 1 && qtail != 0);
+  // Forward flags over the cells this tile reduces over: the fix-up launch takes a flagged tile.
+  // Asked while the first slab's loads are in flight (the workspace is allocated whatever it
+  // holds, so the loads are harmless for a tile that then leaves).
+  if (bwd_tile_flagged(ws_hdr, fwd_flags, true, GRAD_A, GRAD_A ? r0 : c0, GRAD_A ? T::TR : T::TC, batch,
+                       M, N, tid, NT))
+    return;
   stage(0);
   __syncthreads();
   for (int s = 0; s < slabs; ++s) {
