@@ -397,9 +397,14 @@ int genbmm_band_from_dense(const float* dense, float* out, int B, int n_rows,
  * banded_cuda_kernel.cu:389 and on).  The functions below are the same
  * operations as their float namesakes above on double buffers, with the same
  * argument meaning and return codes, minus the float path's workspaces
- * (stats / factors / workspace): one lane per result cell, the reduction walked
- * in ascending order as the reference does.  samplebmm draws the same uniform
- * (24 random bits) per cell as the float function for a given seed and offset.
+ * (stats / factors / workspace).  logbmm forward and backward run factored on
+ * the double-precision matrix instruction (64 x 64 tiles; row and column
+ * maxima, exponentials and the guard S >= 1e-280 inside the one kernel, cells
+ * that fail it redone by the reference's own two passes) for problems of at
+ * least 4096 terms with M, N <= 4096; everything else is one lane per result
+ * cell, the reduction walked in ascending order as the reference does.
+ * samplebmm draws the same uniform (24 random bits) per cell as the float
+ * function for a given seed and offset.
  */
 int genbmm_logbmm_fwd_f64(const double* a, const double* b, double* out,
                           int B, int M, int K, int N, void* stream);
