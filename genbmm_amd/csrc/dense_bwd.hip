@@ -12,7 +12,7 @@ namespace {
 //   grad_b[k,n] = sum_m g[m,n]*p*(w - t[m,n])
 // With u_b = 0 these are the reference's three quartic kernels
 // (matmul_cuda_kernel.cu:220-331: inner = sum_k2 (delta*s - s*s2)*u[k2]
-// = s*(u[k] - t)), computed in O(M*K*N).  One lane per output element.
+// = s*(u[k] - t)), computed in O(M*K*N).  One lane per output element for t and grad_b.
 struct BB {
   const float* a; const float* b; const float* out; const float* g;
   const float* ua; const float* ub;
@@ -40,26 +40,65 @@ __global__ __launch_bounds__(256) void k_log_bwdbwd_t(const BB p, long total) {
   p.gg[e] = t;
 }
 
-__global__ __launch_bounds__(256) void k_log_bwdbwd_a(const BB p, long total) {
-  const long e = (long)blockIdx.x * 256 + threadIdx.x;
-  if (e >= total) return;
-  const int k = (int)(e % p.K);
-  const long bm = e / p.K;
+// grad_a: a wave per row (batch, m), its lanes along n - the one axis on which b, u_b, out, g and
+// t are all contiguous (with a lane per cell (m, k) the reads of b run down a column, one cache
+// line per lane).  The row's out, g and t stay in registers for N <= 256; per k the lanes'
+// partial sums are added across the wave and 64 finished cells are written at once.
+constexpr int kBBChunks = 4;  // n chunks of 64 a lane keeps in registers
+__global__ __launch_bounds__(256) void k_log_bwdbwd_a(const BB p, long rows) {
+  const int lane = threadIdx.x & 63;
+  const long bm = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (bm >= rows) return;
   const long batch = bm / p.M;
-  const float av = p.a[e];
-  const float uav = p.ua ? p.ua[e] : 0.f;
-  const float* brow = p.b + (batch * p.K + k) * p.N;
-  const float* ubrow = p.ub ? p.ub + (batch * p.K + k) * p.N : nullptr;
-  const float* orow = p.out + bm * p.N;
-  const float* grow = p.g + bm * p.N;
-  const float* trow = p.gg + bm * p.N;
-  float acc = 0.f;
-  for (int n = 0; n < p.N; ++n) {
-    const float pr = fast_exp(av + brow[n] - orow[n]);
-    const float w = uav + (ubrow ? ubrow[n] : 0.f) - trow[n];
-    acc = __builtin_fmaf(grow[n] * pr, w, acc);
+  const int K = p.K, N = p.N;
+  const float* arow = p.a + bm * K;
+  const float* uarow = p.ua ? p.ua + bm * K : nullptr;
+  const float* bmat = p.b + batch * K * N;
+  const float* ubmat = p.ub ? p.ub + batch * K * N : nullptr;
+  const float* orow = p.out + bm * N;
+  const float* grow = p.g + bm * N;
+  const float* trow = p.gg + bm * N;
+  const bool cached = N <= 64 * kBBChunks;
+  float oc[kBBChunks], gc[kBBChunks], tc[kBBChunks];
+#pragma unroll
+  for (int j = 0; j < kBBChunks; ++j) {
+    const int n = lane + 64 * j;
+    const bool in = cached && n < N;
+    oc[j] = in ? orow[n] : 0.f;
+    gc[j] = in ? grow[n] : 0.f;
+    tc[j] = in ? trow[n] : 0.f;
   }
-  p.ga[e] = acc;
+  float mine = 0.f;  // the finished cell k with k % 64 == lane
+  for (int k = 0; k < K; ++k) {
+    const float av = arow[k], uav = uarow ? uarow[k] : 0.f;
+    const float* brow = bmat + (long)k * N;
+    const float* ubrow = ubmat ? ubmat + (long)k * N : nullptr;
+    float acc = 0.f;
+    if (cached) {
+#pragma unroll
+      for (int j = 0; j < kBBChunks; ++j) {
+        const int n = lane + 64 * j;
+        if (n < N) {
+          const float pr = fast_exp(av + brow[n] - oc[j]);
+          const float w = uav + (ubrow ? ubrow[n] : 0.f) - tc[j];
+          acc = __builtin_fmaf(gc[j] * pr, w, acc);
+        }
+      }
+    } else {
+      for (int n = lane; n < N; n += 64) {
+        const float pr = fast_exp(av + brow[n] - orow[n]);
+        const float w = uav + (ubrow ? ubrow[n] : 0.f) - trow[n];
+        acc = __builtin_fmaf(grow[n] * pr, w, acc);
+      }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    if ((k & 63) == lane) mine = acc;
+    if ((k & 63) == 63 || k == K - 1) {
+      const int k0 = k & ~63;
+      if (k0 + lane <= k) p.ga[bm * K + k0 + lane] = mine;
+    }
+  }
 }
 
 __global__ __launch_bounds__(256) void k_log_bwdbwd_b(const BB p, long total) {
@@ -352,7 +391,8 @@ int genbmm_logbmm_bwdbwd(const float* a, const float* b, const float* out, const
     if (int e = launch_status()) return e;
   }
   if (tmk > 0) {
-    hipLaunchKernelGGL(k_log_bwdbwd_a, blocks(tmk), dim3(256), 0, s, p, tmk);
+    const long rows = (long)B * M;  // four rows per workgroup
+    hipLaunchKernelGGL(k_log_bwdbwd_a, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, p, rows);
     if (int e = launch_status()) return e;
   }
   if (tkn > 0) {
