@@ -101,21 +101,33 @@ __global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ 
   const int m_lo = GB ? 0 : i0, m_cnt = GB ? M : min(kDT, M - i0);
   const int n_lo = FWD ? j0 : GA ? 0 : j0, n_cnt = GA ? N : min(kDT, N - n_lo);
 
-  // ---- maxima.  alpha: one wave per row, lanes along k.  beta: 64 columns at a time, four
+  // ---- maxima.  alpha: a wave per eight rows, lanes along k.  beta: 64 columns at a time, four
   // groups of 64 threads over k, combined through LDS (Ps is free yet).
-  for (int r = wave; r < m_cnt; r += 4) {
-    const double* row = ab + (long)(m_lo + r) * K;
-    double mx = -INFINITY;
-    for (int k = lane; k < K; k += 64) mx = fmax(mx, row[k]);
+  // (eight rows, resp. eight steps of k, are requested before the first is used: taken one at a
+  // time, each waits out a full memory latency and the pre-pass costs a quarter of the kernel)
+  for (int r0 = 8 * wave; r0 < m_cnt; r0 += 32) {
+    double mx[8];
 #pragma unroll
-    for (int s = 32; s >= 1; s >>= 1) mx = fmax(mx, __shfl_xor(mx, s, 64));
-    if (lane == 0) al[r] = mx;
+    for (int j = 0; j < 8; ++j) mx[j] = -INFINITY;
+    for (int k = lane; k < K; k += 64) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (r0 + j < m_cnt) mx[j] = fmax(mx[j], ab[(long)(m_lo + r0 + j) * K + k]);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+#pragma unroll
+      for (int s = 32; s >= 1; s >>= 1) mx[j] = fmax(mx[j], __shfl_xor(mx[j], s, 64));
+      if (lane == 0 && r0 + j < m_cnt) al[r0 + j] = mx[j];
+    }
   }
   for (int c0 = 0; c0 < n_cnt; c0 += 64) {
     const int c = c0 + lane;
     double mx = -INFINITY;
-    if (c < n_cnt)
+    if (c < n_cnt) {
+#pragma unroll 8
       for (int k = wave; k < K; k += 4) mx = fmax(mx, bb[(long)k * N + n_lo + c]);
+    }
     Ps[wave * 64 + lane] = mx;
     __syncthreads();
     if (wave == 0 && c < n_cnt) be[c] = fmax(fmax(Ps[lane], Ps[64 + lane]), fmax(Ps[128 + lane], Ps[192 + lane]));

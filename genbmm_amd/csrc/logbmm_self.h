@@ -394,7 +394,7 @@ __device__ __forceinline__ void log_self_bwd_tile(float* __restrict__ smem, floa
     for (int i = 0; i < 16; ++i) acc[x >> 1][x & 1][i] = 0.f;
 
   // Slab s is formed and staged while slab s-1 is multiplied, so the products start as soon as
-  // the first pieces have arrived; the guard's verdict is only needed before the results are
+  // the first pieces have arrived; the guard's answer is only needed before the results are
   // stored (an item that fails it has been multiplied in vain).
   static_for<0, kSelfSlabs>([&](auto sc_) __attribute__((always_inline)) {
     constexpr int s = decltype(sc_)::value;
