@@ -294,15 +294,20 @@ inline void launch_d64_mm_t(const double* a, const double* b, const double* out,
                             int M, int K, int N, hipStream_t s) {
   const int I = KIND == kD64GradB ? K : M, J = KIND == kD64GradA ? K : N;
   const int ti = (I + T - 1) / T, tj = (J + T - 1) / T;
-  hipLaunchKernelGGL((k64_log_mm<KIND, T>), dim3((unsigned)((long)B * ti * tj)), dim3(256),
+  hipLaunchKernelGGL((k64_log_mm<KIND, T>), dim3((unsigned)((long)B * ti * tj)), dim3(4 * T),
                      d64_mm_lds(KIND, T, M, N), s, a, b, out, g, dst, M, K, N, ti, tj);
 }
-// (128 x 128 tiles, which halve the exponentials per product, measured slower at 512 items of
-// 128^3 - 0.32 ms against 0.20 for the forward: one workgroup per compute unit hides nothing.)
+// 128 x 128 tiles (eight waves) where the result is wider than one 64 x 64 tile in both directions
+// and the tile's LDS stays within the default 64 KB: half the exponentials per product, and an
+// item of 128 x 128 takes its maxima and reads its operands once instead of four times.
 template <int KIND>
 inline void launch_d64_mm(const double* a, const double* b, const double* out, const double* g, double* dst, int B,
                           int M, int K, int N, hipStream_t s) {
-  launch_d64_mm_t<KIND, 64>(a, b, out, g, dst, B, M, K, N, s);
+  const int I = KIND == kD64GradB ? K : M, J = KIND == kD64GradA ? K : N;
+  if (I > 64 && J > 64 && d64_mm_lds(KIND, 128, M, N) <= 64 * 1024)
+    launch_d64_mm_t<KIND, 128>(a, b, out, g, dst, B, M, K, N, s);
+  else
+    launch_d64_mm_t<KIND, 64>(a, b, out, g, dst, B, M, K, N, s);
 }
 }  // namespace
 }  // namespace genbmm
@@ -348,6 +353,12 @@ int genbmm_logbmm_bwd_f64(const double* a, const double* b, const double* out, c
     return GENBMM_E_NULLPTR;
   hipStream_t s = (hipStream_t)stream;
   if (d64_mm_ok(B, M, K, N)) {
+    const size_t lds = max(d64_mm_lds(kD64GradA, 128, M, N), d64_mm_lds(kD64GradB, 128, M, N));
+    if (max(max(M, K), N) <= 128 && min(min(M, K), N) > 64 && lds <= 64 * 1024) {  // one tile per item and gradient
+      hipLaunchKernelGGL(k64_log_mm_both<128>, dim3((unsigned)((B + 7) / 8 * 16)), dim3(512), lds, s, a, b, out, g,
+                         grad_a, grad_b, B, M, K, N);
+      return launch_status();
+    }
     launch_d64_mm<kD64GradA>(a, b, out, g, grad_a, B, M, K, N, s);
     launch_d64_mm<kD64GradB>(a, b, out, g, grad_b, B, M, K, N, s);
     return launch_status();

@@ -8,8 +8,8 @@
 // so that (M K + K N + M N) exponentials replace the M K N of the reference's loops
 // (matmul_cuda_kernel.cu:27-41, 159-217), and the contraction is a plain product.  All
 // three are C[i,j] = sum_l P[i,l] Q[l,j] on 128 x 128 (or 64 x 64) tiles of (i,j), one
-// workgroup of four waves per tile (each wave a quarter: sixteen or four 16 x 16
-// accumulators), the contraction in chunks of 16 staged in LDS with the exponential taken
+// workgroup of eight (four) waves per tile (each wave 32 x 64 or 32 x 32 of it: eight or four
+// 16 x 16 accumulators), the contraction in chunks of 16 staged in LDS with the exponential taken
 // on the way in; the next chunk's operands are in flight while the current one is
 // multiplied.  The exponentials of a staged chunk are vector work of about the same cost as
 // the chunk's matrix instructions at 64 x 64 and half of it at 128 x 128.
@@ -74,18 +74,19 @@ constexpr int kD64Fwd = 0, kD64GradA = 1, kD64GradB = 2;
 __device__ __forceinline__ double d64_shift(double mx) { return mx == -INFINITY ? 0.0 : mx; }
 __device__ __forceinline__ bool d64_usable(double shift) { return shift > 0.9 * kDFloor && shift < INFINITY; }
 
-// kDT: tile edge, 64 or 128 (a wave's share 32 x 32 or 64 x 64).  tiles: (ceil(I / kDT),
-// ceil(J / kDT)) per item; grid = B * tiles_i * tiles_j
+// kDT: tile edge, 64 (four waves, a wave's share 32 x 32) or 128 (eight waves, 32 x 64: every staged
+// element - one exponential each - then feeds twice the products, and an item of 128 x 128 is one
+// tile, so its maxima are taken once and its operands read once).  4 kDT threads.  tiles:
+// (ceil(I / kDT), ceil(J / kDT)) per item; grid = B * tiles_i * tiles_j
 template <int KIND, int kDT>
-__global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ a, const double* __restrict__ b,
-                                                 const double* __restrict__ out, const double* __restrict__ g,
-                                                 double* __restrict__ dst, int M, int K, int N, int tiles_i,
-                                                 int tiles_j) {
-  extern __shared__ __attribute__((aligned(16))) double smem64[];
+__device__ __forceinline__ void d64_log_mm_tile(double* __restrict__ smem64, int block, const double* __restrict__ a,
+                                                const double* __restrict__ b, const double* __restrict__ out,
+                                                const double* __restrict__ g, double* __restrict__ dst, int M,
+                                                int K, int N, int tiles_i, int tiles_j) {
   constexpr bool FWD = KIND == kD64Fwd, GA = KIND == kD64GradA, GB = KIND == kD64GradB;
   const int I = GB ? K : M, J = FWD ? N : GA ? K : N, L = FWD ? K : GA ? N : M;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int tile = blockIdx.x % (tiles_i * tiles_j), batch = blockIdx.x / (tiles_i * tiles_j);
+  const int tile = block % (tiles_i * tiles_j), batch = block / (tiles_i * tiles_j);
   const int i0 = (tile / tiles_j) * kDT, j0 = (tile % tiles_j) * kDT;
   const double* ab = a + (long)batch * M * K;
   const double* bb = b + (long)batch * K * N;
@@ -93,7 +94,8 @@ __global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ 
   const double* gb = FWD ? nullptr : g + (long)batch * M * N;
   double* db = dst + (long)batch * I * J;
 
-  constexpr int kH = kDT / 64, kW = kDT / 32;  // staging rounds per chunk; 16 x 16 accumulators per wave and side
+  constexpr int NT = 4 * kDT, kWaves = NT / 64;
+  constexpr int kWI = 2, kWJ = kDT / 32;  // 16 x 16 accumulators per wave: rows, columns
   double* Ps = smem64;              // [kDT][kDP]: P[i][l]
   double* Qs = Ps + kDT * kDP;      // [kDT][kDP]: Q[l][j] as [j][l]
   double* al = Qs + kDT * kDP;      // alpha: the tile's rows m (forward, grad_a) or all M (grad_b)
@@ -102,10 +104,10 @@ __global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ 
   const int n_lo = FWD ? j0 : GA ? 0 : j0, n_cnt = GA ? N : min(kDT, N - n_lo);
 
   // ---- maxima.  alpha: a wave per eight rows, lanes along k.  beta: 64 columns at a time, four
-  // groups of 64 threads over k, combined through LDS (Ps is free yet).
+  // groups of 64 threads (one per wave) over k, combined through LDS (Ps is free yet).
   // (eight rows, resp. eight steps of k, are requested before the first is used: taken one at a
   // time, each waits out a full memory latency and the pre-pass costs a quarter of the kernel)
-  for (int r0 = 8 * wave; r0 < m_cnt; r0 += 32) {
+  for (int r0 = 8 * wave; r0 < m_cnt; r0 += 8 * kWaves) {
     double mx[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) mx[j] = -INFINITY;
@@ -126,11 +128,16 @@ __global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ 
     double mx = -INFINITY;
     if (c < n_cnt) {
 #pragma unroll 8
-      for (int k = wave; k < K; k += 4) mx = fmax(mx, bb[(long)k * N + n_lo + c]);
+      for (int k = wave; k < K; k += kWaves) mx = fmax(mx, bb[(long)k * N + n_lo + c]);
     }
     Ps[wave * 64 + lane] = mx;
     __syncthreads();
-    if (wave == 0 && c < n_cnt) be[c] = fmax(fmax(Ps[lane], Ps[64 + lane]), fmax(Ps[128 + lane], Ps[192 + lane]));
+    if (wave == 0 && c < n_cnt) {
+      double m = Ps[lane];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) m = fmax(m, Ps[64 * w + lane]);
+      be[c] = m;
+    }
     __syncthreads();
   }
   __syncthreads();
@@ -141,15 +148,16 @@ __global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ 
   // holds (the next chunk's, in flight during the products); put(): exponentials, LDS.
   constexpr bool P_L = !GB;  // P's contiguous axis is l (a[m][k] forward, g[m][n] grad_a); grad_b: i (a[m][k], i = k)
   constexpr bool Q_L = GA;   // Q's contiguous axis is l only in grad_a (b[k][n], l = n)
-  const int pl_line = P_L ? tid >> 2 : 4 * (tid & 15), pl_l = P_L ? 4 * (tid & 3) : tid >> 4;
-  const int ql_line = Q_L ? tid >> 2 : 4 * (tid & 15), ql_l = Q_L ? 4 * (tid & 3) : tid >> 4;
-  double rp[4 * kH], rp2[4 * kH], rq[4 * kH], rq2[4 * kH];
+  constexpr int kLQ = kDT / 4;  // groups of four lines
+  const int pl_line = P_L ? tid >> 2 : 4 * (tid % kLQ), pl_l = P_L ? 4 * (tid & 3) : tid / kLQ;
+  const int ql_line = Q_L ? tid >> 2 : 4 * (tid % kLQ), ql_l = Q_L ? 4 * (tid & 3) : tid / kLQ;
+  double rp[4], rp2[4], rq[4], rq2[4];
   auto load = [&](int l0) __attribute__((always_inline)) {
 #pragma unroll
-    for (int eh = 0; eh < 4 * kH; ++eh) {
-      const int e = eh & 3, h = eh >> 2;
+    for (int eh = 0; eh < 4; ++eh) {
+      const int e = eh;
       {  // P[i][l]
-        const int i = i0 + 64 * h + pl_line + (P_L ? 0 : e), l = l0 + pl_l + (P_L ? e : 0);
+        const int i = i0 + pl_line + (P_L ? 0 : e), l = l0 + pl_l + (P_L ? e : 0);
         const bool ok = i < I && l < L;
         long off = 0;
         if (FWD) off = (long)i * K + l;  // a[m = i][k = l]
@@ -159,7 +167,7 @@ __global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ 
         if (GA) rp2[eh] = ok ? ob[off] : 0.0;
       }
       {  // Q[l][j]
-        const int j = j0 + 64 * h + ql_line + (Q_L ? 0 : e), l = l0 + ql_l + (Q_L ? e : 0);
+        const int j = j0 + ql_line + (Q_L ? 0 : e), l = l0 + ql_l + (Q_L ? e : 0);
         const bool ok = j < J && l < L;
         long off = 0;
         if (FWD) off = (long)l * N + j;  // b[k = l][n = j]
@@ -178,10 +186,10 @@ __global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ 
   };
   auto put = [&](int l0) __attribute__((always_inline)) {
 #pragma unroll
-    for (int eh = 0; eh < 4 * kH; ++eh) {
-      const int e = eh & 3, h = eh >> 2;
+    for (int eh = 0; eh < 4; ++eh) {
+      const int e = eh;
       {
-        const int il = 64 * h + pl_line + (P_L ? 0 : e), ll = pl_l + (P_L ? e : 0);
+        const int il = pl_line + (P_L ? 0 : e), ll = pl_l + (P_L ? e : 0);
         const int i = i0 + il, l = l0 + ll;
         // (computed for cells beyond the matrix too, then dropped: a select, not a branch)
         const int lc = min(l, L - 1);
@@ -192,7 +200,7 @@ __global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ 
         Ps[il * kDP + ll] = (i < I && l < L) ? v : 0.0;
       }
       {
-        const int jl = 64 * h + ql_line + (Q_L ? 0 : e), ll = ql_l + (Q_L ? e : 0);
+        const int jl = ql_line + (Q_L ? 0 : e), ll = ql_l + (Q_L ? e : 0);
         const int j = j0 + jl, l = l0 + ll;
         const int lc = min(l, L - 1);
         double v;
@@ -205,13 +213,13 @@ __global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ 
   };
 
   // ---- products: wave (wi, wj) owns rows (kDT / 2) wi .., columns (kDT / 2) wj .. of the tile
-  constexpr int kS = kDT / 2;
+  constexpr int kSI = 16 * kWI, kSJ = 16 * kWJ;  // a wave's rows and columns
   const int wi = wave >> 1, wj = wave & 1, l15 = lane & 15, zq = lane >> 4;
-  mmd4 acc[kW][kW];
+  mmd4 acc[kWI][kWJ];
 #pragma unroll
-  for (int x = 0; x < kW; ++x)
+  for (int x = 0; x < kWI; ++x)
 #pragma unroll
-    for (int y = 0; y < kW; ++y) acc[x][y] = mmd4{0.0, 0.0, 0.0, 0.0};
+    for (int y = 0; y < kWJ; ++y) acc[x][y] = mmd4{0.0, 0.0, 0.0, 0.0};
   load(0);
   for (int l0 = 0; l0 < L; l0 += kDC) {
     put(l0);
@@ -219,28 +227,28 @@ __global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ 
     if (l0 + kDC < L) load(l0 + kDC);
 #pragma unroll
     for (int ks = 0; ks < kDC / 4; ++ks) {
-      double pa[kW], qb[kW];
+      double pa[kWI], qb[kWJ];
 #pragma unroll
-      for (int x = 0; x < kW; ++x) pa[x] = Ps[(kS * wi + 16 * x + l15) * kDP + 4 * ks + zq];
+      for (int x = 0; x < kWI; ++x) pa[x] = Ps[(kSI * wi + 16 * x + l15) * kDP + 4 * ks + zq];
 #pragma unroll
-      for (int y = 0; y < kW; ++y) qb[y] = Qs[(kS * wj + 16 * y + l15) * kDP + 4 * ks + zq];
+      for (int y = 0; y < kWJ; ++y) qb[y] = Qs[(kSJ * wj + 16 * y + l15) * kDP + 4 * ks + zq];
 #pragma unroll
-      for (int x = 0; x < kW; ++x)
+      for (int x = 0; x < kWI; ++x)
 #pragma unroll
-        for (int y = 0; y < kW; ++y) acc[x][y] = __builtin_amdgcn_mfma_f64_16x16x4f64(pa[x], qb[y], acc[x][y], 0, 0, 0);
+        for (int y = 0; y < kWJ; ++y) acc[x][y] = __builtin_amdgcn_mfma_f64_16x16x4f64(pa[x], qb[y], acc[x][y], 0, 0, 0);
     }
     __syncthreads();
   }
 
-  // ---- results: accumulator element r of tile (x, y) is row kS wi + 16 x + 4 r + zq, column
-  // kS wj + 16 y + l15
+  // ---- results: accumulator element r of tile (x, y) is row kSI wi + 16 x + 4 r + zq, column
+  // kSJ wj + 16 y + l15
 #pragma unroll
-  for (int x = 0; x < kW; ++x)
+  for (int x = 0; x < kWI; ++x)
 #pragma unroll
-    for (int y = 0; y < kW; ++y)
+    for (int y = 0; y < kWJ; ++y)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int il = kS * wi + 16 * x + 4 * r + zq, jl = kS * wj + 16 * y + l15;
+        const int il = kSI * wi + 16 * x + 4 * r + zq, jl = kSJ * wj + 16 * y + l15;
         const int i = i0 + il, j = j0 + jl;
         if (i >= I || j >= J) continue;
         const double v = acc[x][y][r];
@@ -279,6 +287,34 @@ __global__ __launch_bounds__(256, 4) void k64_log_mm(const double* __restrict__ 
         }
         db[(long)i * J + j] = res;
       }
+}
+
+template <int KIND, int kDT>
+__global__ __launch_bounds__(4 * kDT, 4) void k64_log_mm(const double* __restrict__ a, const double* __restrict__ b,
+                                                         const double* __restrict__ out,
+                                                         const double* __restrict__ g, double* __restrict__ dst,
+                                                         int M, int K, int N, int tiles_i, int tiles_j) {
+  extern __shared__ __attribute__((aligned(16))) double smem64[];
+  d64_log_mm_tile<KIND, kDT>(smem64, blockIdx.x, a, b, out, g, dst, M, K, N, tiles_i, tiles_j);
+}
+
+// Both gradients of items that are one tile each, in one launch.  Workgroups come in groups of
+// 16: the first eight take grad_a of eight consecutive items, the next eight grad_b of the same
+// items (workgroup w runs on XCD w mod 8, so an item's second reader finds a, b, out and g in that
+// XCD's L2).
+template <int kDT>
+__global__ __launch_bounds__(4 * kDT, 4) void k64_log_mm_both(const double* __restrict__ a,
+                                                              const double* __restrict__ b,
+                                                              const double* __restrict__ out,
+                                                              const double* __restrict__ g,
+                                                              double* __restrict__ grad_a,
+                                                              double* __restrict__ grad_b, int B, int M, int K,
+                                                              int N) {
+  extern __shared__ __attribute__((aligned(16))) double smem64[];
+  const int w = blockIdx.x, item = (w >> 4) * 8 + (w & 7);
+  if (item >= B) return;
+  if (((w >> 3) & 1) == 0) d64_log_mm_tile<kD64GradA, kDT>(smem64, item, a, b, out, g, grad_a, M, K, N, 1, 1);
+  else d64_log_mm_tile<kD64GradB, kDT>(smem64, item, a, b, out, g, grad_b, M, K, N, 1, 1);
 }
 
 inline size_t d64_mm_lds(int kind, int tile, int M, int N) {

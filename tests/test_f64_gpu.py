@@ -48,6 +48,24 @@ def test_logbmm_f64(gpu, B, M, K, N):
     close(got[1], want[1], 1e-9, 1e-11)
 
 
+@pytest.mark.parametrize("B,M,K,N", [(9, 128, 128, 128), (11, 100, 97, 120), (3, 200, 130, 96), (2, 65, 300, 129)])
+def test_logbmm_f64_wide_tiles(gpu, B, M, K, N):
+    """Shapes on the eight-wave 128 x 128 tiles: items that are one tile per gradient (both gradients
+    in one launch), ragged edges, several tiles per item; one item needs the exact loops."""
+    torch.manual_seed(B + N)
+    a, b, g = torch.randn(B, M, K).double() * 3, torch.randn(B, K, N).double() * 3, torch.randn(B, M, N).double()
+    a[1, ::3, 0] += 800.0
+    b[1, 0, :] -= 800.0
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    out = genbmm.logbmm(ad, bd)
+    close(out, oracle.logbmm_broadcast(a, b), 1e-12, 1e-9)
+    ga, gb = torch.autograd.grad(out, (ad, bd), g.to(gpu))
+    _, wa, wb = oracle.logbmm_grads64(a, b, g)
+    close(ga, wa, 1e-10, 1e-9)
+    close(gb, wb, 1e-10, 1e-9)
+    close(ga.sum(-1), g.sum(-1), 1e-10, 1e-9)
+
+
 def test_logbmm_f64_special_values(gpu):
     a = torch.tensor([[[0.0, -1e9, float("-inf")], [5.0, 5.0, 5.0]]], dtype=torch.float64)
     b = torch.zeros(1, 3, 2, dtype=torch.float64)
