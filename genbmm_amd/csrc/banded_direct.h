@@ -97,7 +97,7 @@ inline int dir_chunks(int Wp) { return (Wp + 30) >> 4; }  // chunks of 16 k that
 // its tiles (forward of the log product) or the tile row's results (all others), which then
 // leave as one contiguous run of memory
 inline int dir_wave_lds(const DirPlan& g, int kind, bool prep) {
-  return (g.NU + 1) * 1024 + (kind == kDirFwd && prep ? 64 * g.nt : 64 * g.Wout);
+  return (g.NU + 1) * 1024 + 64 * g.Wout + (kind == kDirFwd && prep ? 64 * g.nt + 64 : 0);
 }
 
 inline bool dir_plan(DirPlan& g, int kind, int a_lu, int Wa, int b_lu, int Wb) {
@@ -162,7 +162,7 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const DirPlan& g, lon
   constexpr bool PROW = KIND == kDirGradB;  // P's band row is k
   constexpr bool QROW = KIND != kDirFwd;    // Q's band row is k
   constexpr bool MKH = PREP && !FWD;        // P = g / S, formed while it is read
-  constexpr bool STAGE = !EDGE && !(FWD && PREP);
+  constexpr bool STAGE = !EDGE;
   const int n = p.n, Wp = g.Wp, Wq = g.Wq, Wout = g.Wout, NU = g.NU, nt = g.nt;
   const int l15 = lane & 15, zq = lane >> 4;
   // a lane that loads 16 bytes: lane 4 r + c takes row r, cells 4 c .. 4 c + 3 of the chunk; the
@@ -271,14 +271,17 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const DirPlan& g, lon
     }
     pl[64 * NU + lane] = mm_f4{0.f, 0.f, 0.f, 0.f};
   }
-  // behind the chunks: beta of every column the wave's tiles cover (forward of the log
-  // product), or the tile row's 16 x Wout results
+  // behind the chunks: the tile row's 16 x Wout results, then (forward of the log product) beta
+  // of every column the wave's tiles cover and alpha of its 16 rows
   float* aux = lds + 256 * (NU + 1);
+  float* bet = aux + 16 * Wout;
+  float* alp = bet + 16 * nt;
   if (FWD && PREP) {
     for (int t = lane; t < 16 * nt; t += 64) {
       const int y = J0 + t;
-      aux[t] = (unsigned)y < (unsigned)n ? p.ws_be[bn + y] : 0.f;
+      bet[t] = (unsigned)y < (unsigned)n ? p.ws_be[bn + y] : 0.f;
     }
+    if (lane < 16) alp[lane] = i0 + lane < n ? p.ws_al[bn + i0 + lane] : 0.f;
   }
 
   // Factors 1 / 0 for the cells of a chunk at the ends of Q's band: past the upper end
@@ -395,7 +398,7 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const DirPlan& g, lon
     float* ot = (STAGE ? aux : orow) + 16 * tj;
     unsigned bits = 0;
     float be = 0.f;
-    if (FWD && PREP) be = aux[16 * tj + l15];
+    if (FWD && PREP) be = bet[16 * tj + l15];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int jj = 16 * tj + l15 - 4 * zq - r;
@@ -447,7 +450,43 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const DirPlan& g, lon
     }
   }
 
-  if (STAGE) {  // the tile row's 16 Wout results: one contiguous run of memory
+  if (FWD && PREP && plain_rows) {
+    // The sums S of the tile row are in LDS: out = log S + alpha + beta and 1/S leave as two
+    // contiguous runs, four cells per lane.  A cell outside the guard gets 1/S = -1 (not usable,
+    // the backward then takes the exact way) and its value from the per-cell routine right
+    // behind the store (same lane, same address: in order).
+    const mm_f4* so4 = reinterpret_cast<const mm_f4*>(aux);
+    const float rw = 1.f / (float)Wout;
+    for (int i = lane; i < 4 * Wout; i += 64) {
+      const mm_f4 sv = so4[i];
+      int row = (int)((float)(4 * i) * rw);  // 4 i / Wout, exact after one correction either way
+      int jj = 4 * i - row * Wout;
+      if (jj < 0) { --row; jj += Wout; }
+      if (jj >= Wout) { ++row; jj -= Wout; }
+      mm_f4 ov, rv;
+      unsigned bad = 0;
+#pragma unroll
+      for (int c4 = 0; c4 < 4; ++c4) {
+        const float sh = alp[row] + bet[row + jj], v = sv[c4];
+        const bool ok = (v >= thr) && (v < INFINITY) && (sh > 0.9f * kFloor) && (sh < INFINITY);
+        rv[c4] = ok ? __builtin_amdgcn_rcpf(v) : -1.f;
+        ov[c4] = __builtin_fmaf(fast_log2(v), kLn2, sh);
+        if (!ok) bad |= 0x80000000u >> c4;
+        if (++jj == Wout) { jj = 0; ++row; }
+      }
+      *reinterpret_cast<dir_f4u*>(orow + 4 * i) = dir_f4u{ov[0], ov[1], ov[2], ov[3]};
+      *reinterpret_cast<dir_f4u*>(rrow + 4 * i) = dir_f4u{rv[0], rv[1], rv[2], rv[3]};
+      if (bad) {  // rare
+        int r2 = (int)((float)(4 * i) * rw), j2 = 4 * i - r2 * Wout;
+        if (j2 < 0) { --r2; j2 += Wout; }
+        if (j2 >= Wout) { ++r2; j2 -= Wout; }
+        for (int c4 = 0; c4 < 4; ++c4) {
+          if (bad & (0x80000000u >> c4)) band_fwd_cell<GENBMM_BAND_LOG>(p, bn + i0 + r2, i0 + r2, j2);
+          if (++j2 == Wout) { j2 = 0; ++r2; }
+        }
+      }
+    }
+  } else if (STAGE) {  // the tile row's 16 Wout results: one contiguous run of memory
     const mm_f4* so4 = reinterpret_cast<const mm_f4*>(aux);
 #pragma unroll
     for (int s = 0; s < kDirEf; ++s) {
