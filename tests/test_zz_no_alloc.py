@@ -36,8 +36,9 @@ def test_static_workspace_forward_matches_the_allocating_one(gpu):
     lib = _lib.load()
     torch.manual_seed(5)
     # matrix-core tiles (one batch item with rows that defeat the factoring -> flagged
-    # tiles), then smaller: ragged matrix-core, vector-ALU tiles, whole-item kernels
-    shapes = [(6, 256, 128, 256), (3, 130, 97, 200), (4, 70, 33, 50), (9, 32, 32, 32), (2, 5, 3, 4)]
+    # tiles), then smaller: ragged matrix-core, one tile per item, vector-ALU tiles, whole-item kernels
+    shapes = [(6, 256, 128, 256), (3, 130, 97, 200), (5, 128, 100, 96), (4, 70, 33, 50), (9, 32, 32, 32),
+              (2, 5, 3, 4)]
     for rep in range(2):          # the second round starts from the smallest shape's leftovers
         for B, M, K, N in shapes:
             a, b = torch.randn(B, M, K), torch.randn(B, K, N)
