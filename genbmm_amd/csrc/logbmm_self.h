@@ -51,11 +51,8 @@ __device__ __forceinline__ void static_for(F&& f) {
 __device__ __forceinline__ bool shift_ok(float sh) { return (sh > 0.45f * kFloor) && (sh < INFINITY); }
 
 // ----------------------------------------------------------------- forward
-// An item that fails the guard: the online routine, two 64 x 128 tiles.  
-__device__ __forceinline__ void self_fwd_exact(DenseArgs p, int batch, float* smem) {
-  // (reads some of the addresses the caller has loaded from: hidden from the compiler, which
-  // would otherwise keep the caller's registers of a and b alive for this routine)
-  asm volatile("" : "+s"(p.a), "+s"(p.b));
+// An item that fails the guard: the online routine, two 64 x 128 tiles.
+__device__ __forceinline__ void self_fwd_exact(const DenseArgs& p, int batch, float* smem) {
   for (int h = 0; h < kSelfMax / CfgWide::BM; ++h)
     if (h * CfgWide::BM < p.M) {
       log_fwd_tile<CfgWide, false>(p, batch, h * CfgWide::BM, 0, smem, smem + CfgWide::KT * CfgWide::LDA);
@@ -236,12 +233,9 @@ void k_log_self_fwd(const DenseArgs p, float* __restrict__ stats, int* __restric
 }
 
 // ---------------------------------------------------------------- backward
-// An item that fails the guard: the exact routine, two 64 x 128 tiles.  
+// An item that fails the guard: the exact routine, two 64 x 128 tiles.
 template <bool GRAD_A>
-__device__ __forceinline__ void self_bwd_exact(LogBwdArgs p, int batch, float* smem) {
-  // The routine reads some of the very addresses the caller has loaded from: hide that from the
-  // compiler, which would otherwise keep the caller's 128 registers of g and out alive for it.
-  asm volatile("" : "+s"(p.a), "+s"(p.b), "+s"(p.out), "+s"(p.g));
+__device__ __forceinline__ void self_bwd_exact(const LogBwdArgs& p, int batch, float* smem) {
   const int R = GRAD_A ? p.M : p.K;
   for (int h = 0; h < kSelfMax / BCfgWide::BR; ++h)
     if (h * BCfgWide::BR < R) {
