@@ -421,7 +421,11 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
         if (m < M && n < N) {
           const float e = al[r] + be[c] - ob[(long)m * N + n];   // -log S
           if (!(e <= lim) || !(e > -INFINITY)) bad = 1;
-          rem[i][j] = u[q] * fast_exp2(-e * kLog2e);
+          // S = exp(-e) carries the rounding of `out` (2^-24 |out|) and the sweep adds the terms up in
+          // another order than the forward did: a target that close to the total could lie beyond
+          // the last prefix sum and never be passed, so every target is shrunk by 2^-17 of itself
+          // (the boundaries between the terms move by 7.6e-6 of the total mass).
+          rem[i][j] = (u[q] * (1.f - 0x1p-17f)) * fast_exp2(-e * kLog2e);
         }
         if (TWO) {
           low[i][j] = __float_as_uint(rem[i][j]);

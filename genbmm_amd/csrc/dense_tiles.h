@@ -196,8 +196,12 @@ __device__ __forceinline__ void log_fwd_tile(const DenseArgs& p, int batch, int 
   // ---- second sweep: inverse CDF.  rem = uniform - (mass scanned so far);
   // cell takes index k at the first k with rem > 0 and p_k > rem, which is
   // the reference's `total < r && total + p > r` with total = r - rem.
+  // The masses exp(a + b - out) add up to 1 only within the rounding of `out` (2^-24 |out| in the
+  // exponent), so a uniform that close to 1 can lie beyond the last prefix sum: such a cell takes
+  // the last term that has any mass (`last`), not the reference's default of 0, which may name
+  // a masked term.
   float rem[C::TM][C::TN];
-  int ind[C::TM][C::TN];
+  int ind[C::TM][C::TN], last[C::TM][C::TN];
   const bool blocks = (N & 3) == 0;  // a lane's four adjacent cells then share one Philox block
 #pragma unroll
   for (int i = 0; i < C::TM; ++i)
@@ -211,6 +215,7 @@ __device__ __forceinline__ void log_fwd_tile(const DenseArgs& p, int batch, int 
       for (int q = 0; q < 4; ++q) {
         rem[i][jq + q] = u[q];
         ind[i][jq + q] = 0;
+        last[i][jq + q] = 0;
         mx[i][jq + q] = -mx[i][jq + q] * kLog2e;  // -out*log2e
       }
     }
@@ -240,6 +245,7 @@ __device__ __forceinline__ void log_fwd_tile(const DenseArgs& p, int batch, int 
           const float pk = fast_exp2(__builtin_fmaf(av[i] + bv[j], kLog2e, mx[i][j]));
           const float r = rem[i][j];
           if (r > 0.f && pk > r) ind[i][j] = k;
+          if (pk > 0.f) last[i][j] = k;
           rem[i][j] = r - pk;
         }
     };
@@ -250,6 +256,11 @@ __device__ __forceinline__ void log_fwd_tile(const DenseArgs& p, int batch, int 
       for (int kk = 0; kk < kn; ++kk) scan(kk);
     }
   }
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+      if (rem[i][j] > 0.f) ind[i][j] = last[i][j];  // the walk never passed its target
   store_tile_i<C>(p.idx + (long)batch * M * N, ind, m0, n0, M, N, p.vec_o, tx, ty);
 }
 

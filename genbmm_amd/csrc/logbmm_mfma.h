@@ -644,7 +644,7 @@ void k_log_bwd_mfma_both(const float* __restrict__ g, const float* __restrict__ 
 // ------------------------------------------------------- sampling sweep
 // samplebmm on the forward's factors: index = first k whose prefix sum
 // sum_{k' <= k} EA[m,k'] EB[k',n] passes the target t = u * S (one Philox uniform
-// u per cell, S = exp(out - alpha - beta)).  The accumulators start at -t, so after
+// u per cell, S = the reciprocal of the forward's 1 / S).  The accumulators start at -t, so after
 // every slab they hold prefix - t: negative while the prefix is below the target, and
 // closer to zero slab by slab.  One register per cell keeps what is needed of that
 // history: the low six bits of the value's bit pattern are replaced by 62 - slab and
@@ -662,6 +662,10 @@ void k_log_bwd_mfma_both(const float* __restrict__ g, const float* __restrict__ 
 // waves lets two workgroups share a compute unit within the 256 registers per lane,
 // so that one's vector work overlaps the other's matrix-core work.
 constexpr int kSampleSlabs = 62;
+// The reciprocal of the forward's 1 / S is S within two roundings; a target within 2^-22 of the sum
+// the sweep adds up could lie beyond it and never be passed.  Every target is shrunk by that
+// much instead (the boundaries between the terms move by 2.4e-7 of the total mass).
+constexpr float kSampleShrink = 1.f - 0x1p-22f;
 
 // (Always the any-size form of the loaders: with this kernel's register budget the
 // full-tile form compiled to spills and measured no faster.)
@@ -709,13 +713,18 @@ void k_sample_sweep_mfma(const float* __restrict__ ws_ea, const float* __restric
       philox_uniform4((uint64_t)cell, blocks, seed, offset, u);
       const float alr = st[m];
       const float4 be4 = ld4m(st + M + n, cn, 0.f), o4 = ld4m(out + cell, cn, 0.f);
+      // S from the forward's 1 / S, which still sits where the targets go (valid in every tile the
+      // forward did not flag): exp(out - alpha - beta) carries the rounding of `out`, up to 6e-5
+      // of S at |out| ~ 1000, and a target u S beyond the sum the sweep adds up is never passed
+      const float4 r4 = ld4m(remw + cell, cn, 1.f);
       const float bev[4] = {be4.x, be4.y, be4.z, be4.w}, ov[4] = {o4.x, o4.y, o4.z, o4.w};
+      const float rv[4] = {r4.x, r4.y, r4.z, r4.w};
       float tv[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const float e = alr + bev[j] - ov[j];  // -log S
         if (j < cn && (!(e <= lim) || !(e > -INFINITY))) bad = 1;
-        tv[j] = -u[j] * fast_exp2(-e * kLog2e);
+        tv[j] = -(u[j] * kSampleShrink) * __builtin_amdgcn_rcpf(rv[j]);
       }
       st4m(remw + cell, cn, make_float4(tv[0], tv[1], tv[2], tv[3]));
     }

@@ -204,8 +204,12 @@ int genbmm_prodmaxbmm_fwd(const float* a, const float* b, float* out,
  * (x >> 8) * 2^-24 with x = word (i & 3) of Philox4x32-10(counter = {lo32(i >> 2),
  * hi32(i >> 2), lo32(offset), hi32(offset)}, key = {lo32(seed), hi32(seed)}):
  * four consecutive cells share one Philox block.
- * A cell whose scan never crosses its uniform keeps index 0, as in the
- * reference.  Replaces _genbmm.forward(a, b, 2): matmul_cuda_kernel.cu:512-526
+ * A cell without any mass (every term masked) keeps index 0, as in the
+ * reference.  A uniform within rounding of 1 never falls past the last term:
+ * the exact walk then names the last term that has mass, and the walks on the
+ * factors shrink every target by 2^-22 (matrix cores) or 2^-17 (vector ALU) of
+ * itself - where the reference's own scan can run out and leave index 0.
+ * Replaces _genbmm.forward(a, b, 2): matmul_cuda_kernel.cu:512-526
  * (torch::rand at :517), kernel :77-121.
  * `stats`: NULL, or a buffer of genbmm_samplebmm_stats_size(B,M,K,N) floats, used
  * like that of genbmm_logbmm_fwd; with it the log-sum-exp comes from the logbmm forward and

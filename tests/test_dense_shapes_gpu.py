@@ -94,13 +94,16 @@ def test_sample_on_many_shapes(gpu):
         assert float((got != want).float().mean()) < 5e-3, (B, M, K, N)
 
 
-@pytest.mark.parametrize("scale", [0.05, 2.0, 12.0, 40.0])
-def test_sample_on_flat_and_peaked_distributions(gpu, scale):
-    """From nearly uniform to one-term-takes-all, with masked terms (-inf, -1e9), on a shape
-    that takes the matrix-core sweep (and its exact fix-up where S underflows)."""
+@pytest.mark.parametrize("shape", [(2, 128, 200, 160), (2, 256, 512, 128)])
+@pytest.mark.parametrize("scale", [0.05, 2.0, 12.0, 40.0, 100.0, 400.0])
+def test_sample_on_flat_and_peaked_distributions(gpu, scale, shape):
+    """From nearly uniform to one-term-takes-all (at the largest scales the winning term leads by
+    hundreds: the remainder the matrix-core sweep hands to the resolve step, six mantissa bits
+    short, must still name the right term), with masked terms (-inf, -1e9), on shapes that take
+    the matrix-core sweep (and its exact fix-up where S underflows): 13 and 32 slabs."""
     lib = _lib.load()
     torch.manual_seed(int(scale * 10))
-    B, M, K, N = 2, 128, 200, 160
+    B, M, K, N = shape
     a, b = scale * torch.randn(B, M, K), scale * torch.randn(B, K, N)
     a[:, ::3, ::5] = float("-inf")
     b[:, 1::7, ::2] = -1e9
@@ -121,8 +124,12 @@ def test_sample_on_flat_and_peaked_distributions(gpu, scale):
     cdf = oracle.sample_cdf64(a, b)
     hi = torch.gather(cdf, 2, got.unsqueeze(2)).squeeze(2)
     lo = torch.where(got > 0, torch.gather(cdf, 2, (got - 1).clamp(min=0).unsqueeze(2)).squeeze(2), torch.zeros_like(hi))
-    ok = ((lo - 2e-5 <= u) & (u <= hi + 2e-5)) | ~live
-    assert bool(ok.all()), float((~ok).float().mean())
+    # fp32 prefix sums over K terms (the reference's too): K roundings of 2^-24 of the running mass;
+    # and the masses are exp(a + b - out) with `out` rounded to fp32: 2^-24 |out| in the exponent
+    tol = max(2e-5, 2.0 * K * 2.0 ** -24, 2.0 * float(want_out[live].abs().max()) * 2.0 ** -23)
+    viol = torch.maximum(lo - u, u - hi).clamp(min=0)
+    ok = (viol <= tol) | ~live
+    assert bool(ok.all()), (float((~ok).float().mean()), float(viol[live].max()), tol)
     # a sampled term always has mass (never a masked one)
     picked = torch.gather(a.unsqueeze(-1) + b.unsqueeze(-3), 2, got.unsqueeze(2)).squeeze(2)
     assert bool((picked[live] > -1e8).all())
