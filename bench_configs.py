@@ -57,20 +57,24 @@ def report(name, ms, ops, nbytes, extra=None):
     print(json.dumps(line), flush=True)
 
 
-def dense_log(lib, dev, B, M, K, N, reps, name, dist="randn", path=0, graph=False):
+def dense_log(lib, dev, B, M, K, N, reps, name, dist="randn", path=0, graph=False, dtype=torch.float32):
+    """dtype float16 / bfloat16: the `_f16` / `_bf16` entry points on tensors of that type (and, for
+    comparison, the float entry points with the widening and narrowing copies around them)."""
     torch.manual_seed(0)
     mk = torch.randn if dist == "randn" else torch.rand
-    a, b = mk(B, M, K).to(dev), mk(B, K, N).to(dev)
-    g = (torch.ones(B, M, N) if dist == "rand" else torch.randn(B, M, N)).to(dev)
-    out, ga, gb = torch.empty(B, M, N, device=dev), torch.empty_like(a), torch.empty_like(b)
+    a, b = mk(B, M, K).to(dev).to(dtype), mk(B, K, N).to(dev).to(dtype)
+    g = (torch.ones(B, M, N) if dist == "rand" else torch.randn(B, M, N)).to(dev).to(dtype)
+    out, ga, gb = torch.empty(B, M, N, device=dev, dtype=dtype), torch.empty_like(a), torch.empty_like(b)
     stats = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=dev)
     s, p = _lib.stream_of(a), _lib.ptr
+    sfx = _lib.HALF_SUFFIX.get(dtype, "")
+    fwd, bwd = getattr(lib, "genbmm_logbmm_fwd_path" + sfx), getattr(lib, "genbmm_logbmm_bwd_path" + sfx)
 
     def f():
-        _lib.check(lib.genbmm_logbmm_fwd_path(p(a), p(b), p(out), p(stats), B, M, K, N, path, s), "fwd")
+        _lib.check(fwd(p(a), p(b), p(out), p(stats), B, M, K, N, path, s), "fwd")
 
     def bw():
-        _lib.check(lib.genbmm_logbmm_bwd_path(p(a), p(b), p(out), p(g), p(stats), p(ga), p(gb), B, M, K, N, path, s), "bwd")
+        _lib.check(bwd(p(a), p(b), p(out), p(g), p(stats), p(ga), p(gb), B, M, K, N, path, s), "bwd")
 
     def step():
         f()
@@ -86,8 +90,20 @@ def dense_log(lib, dev, B, M, K, N, reps, name, dist="randn", path=0, graph=Fals
             step()
         s = _lib.stream_of(a)
         extra_graph = {"ms_graph_replay": round(timed(gr.replay, reps), 4)}
+    if sfx:  # the same step through the float kernels: widen a, b, g; narrow out and the gradients
+        o32, ga32, gb32 = torch.empty(B, M, N, device=dev), torch.empty(B, M, K, device=dev), torch.empty(B, K, N, device=dev)
+
+        def widened():
+            x, y = a.float(), b.float()
+            _lib.check(lib.genbmm_logbmm_fwd_path(p(x), p(y), p(o32), p(stats), B, M, K, N, path, s), "fwd")
+            o = o32.to(dtype)
+            gg = g.float()
+            _lib.check(lib.genbmm_logbmm_bwd_path(p(x), p(y), p(o32), p(gg), p(stats), p(ga32), p(gb32), B, M, K, N, path, s), "bwd")
+            return o, ga32.to(dtype), gb32.to(dtype)
+
+        extra_graph["ms_float_kernels_with_casts"] = round(timed(widened, reps), 4)
     bmkn = float(B) * M * K * N
-    nbytes = 4.0 * B * (3 * M * K + 3 * K * N + 3 * M * N)
+    nbytes = float(a.element_size()) * B * (3 * M * K + 3 * K * N + 3 * M * N)
     report(name, ms, 6 * bmkn, nbytes, {"path": {0: "factored", 1: "online-exact", 2: "factored-valu"}[path],
                                         "ms_fwd": round(mf, 4), "ms_bwd": round(mb, 4), **extra_graph})
 
@@ -304,10 +320,10 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--cpu", action="store_true")
-    ap.add_argument("--only", default="", help="comma-separated subset: log,max,sample,banded,struct,f64; "
+    ap.add_argument("--only", default="", help="comma-separated subset: log,half,max,sample,banded,struct,f64; "
                     "widths (not in the default set): the banded products at 5 ... 81 diagonals per operand")
     args = ap.parse_args()
-    want = set(args.only.split(",")) if args.only else {"log", "max", "sample", "banded", "struct", "f64"}
+    want = set(args.only.split(",")) if args.only else {"log", "half", "max", "sample", "banded", "struct", "f64"}
     lib = _lib.load()
     dev = torch.device("cuda:0")
     r = args.reps
@@ -318,6 +334,11 @@ def main():
         dense_log2(lib, dev, 512, 128, 128, 128, max(3, r // 4))
         for path in (0, 2, 1):
             dense_log(lib, dev, 64, 512, 512, 512, r, "logbmm fwd+bwd (64,512,512,512) headline", path=path)
+    if "half" in want:
+        for dt, nm in ((torch.float16, "float16"), (torch.bfloat16, "bfloat16")):
+            dense_log(lib, dev, 64, 512, 512, 512, r, "logbmm fwd+bwd (64,512,512,512) headline, %s tensors" % nm, dtype=dt)
+            dense_log(lib, dev, 512, 128, 128, 128, r, "logbmm fwd+bwd (512,128,128,128) config 1, %s tensors" % nm, dtype=dt)
+            dense_log(lib, dev, 8192, 32, 32, 32, r, "logbmm fwd+bwd (8192,32,32,32) config 1 skinny, %s tensors" % nm, dtype=dt)
     if "max" in want:
         dense_max(lib, dev, 256, 256, 256, 256, r, prod=False)
         dense_max(lib, dev, 256, 256, 256, 256, r, prod=True)

@@ -61,6 +61,15 @@ SIGNATURES = {
     "genbmm_band_to_dense": [_c_float_p, _c_float_p, _i, _i, _i, _i, ctypes.c_float, _vp],
     "genbmm_band_from_dense": [_c_float_p, _c_float_p, _i, _i, _i, _i, _i, _vp],
 }
+# Entry points that also exist for float16 (`*_f16`) and bfloat16 (`*_bf16`) tensors: the same
+# arguments, the caller's tensors in that type, every workspace still float32.
+HALF_VARIANTS = ("genbmm_logbmm_fwd", "genbmm_logbmm_bwd", "genbmm_logbmm_fwd_path", "genbmm_logbmm_bwd_path",
+                 "genbmm_maxbmm_fwd", "genbmm_prodmaxbmm_fwd", "genbmm_samplebmm_fwd", "genbmm_argmax_bwd",
+                 "genbmm_prodmax_bwd")
+for _name in HALF_VARIANTS:
+    for _suffix in ("_f16", "_bf16"):
+        SIGNATURES[_name + _suffix] = SIGNATURES[_name]
+HALF_SUFFIX = {torch.float16: "_f16", torch.bfloat16: "_bf16"}
 STRING_FUNCS = {"genbmm_version": [], "genbmm_error_string": [_i]}
 SIZE_FUNCS = {"genbmm_logbmm_stats_size": [_i, _i, _i, _i],
               "genbmm_samplebmm_stats_size": [_i, _i, _i, _i],
@@ -137,8 +146,10 @@ def require(t, name, dtype=torch.float32, ndim=3, device=None):
 
 def dense_dims(a, b):
     """(B, M, K, N) of a (B,M,K) x (B,K,N) product, with agreement checks; a's element
-    type (float32 or float64) is the one both must have."""
-    dtype = torch.float64 if isinstance(a, torch.Tensor) and a.dtype == torch.float64 else torch.float32
+    type (float32, float64, float16 or bfloat16) is the one both must have."""
+    dtype = torch.float32
+    if isinstance(a, torch.Tensor) and (a.dtype == torch.float64 or a.dtype in HALF_SUFFIX):
+        dtype = a.dtype
     require(a, "a", dtype=dtype)
     require(b, "b", dtype=dtype, device=a.device)
     B, M, K = a.shape

@@ -18,6 +18,10 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIBNAME = "libgenbmm_gfx950.so"
 SOURCES = ["logbmm.hip", "dense_fwd.hip", "dense_bwd.hip", "banded.hip", "band_struct.hip", "f64.hip"]
+# Sources that are compiled once per element type of the caller's tensors: float (entry points
+# genbmm_*), IEEE binary16 (genbmm_*_f16) and bfloat16 (genbmm_*_bf16); see csrc/common.h.
+_ELEMENTS = (("", 0), ("_f16", 1), ("_bf16", 2))
+PER_ELEMENT = {"logbmm.hip": _ELEMENTS, "dense_fwd.hip": _ELEMENTS, "dense_bwd.hip": _ELEMENTS}
 
 # -packed-fp32-ops is switched OFF: v_pk_{add,mul,fma}_f32 are not used by any
 # kernel here, and the compiler must not form them on its own either.
@@ -61,11 +65,14 @@ def build(verbose=True):
     cc = hipcc()
     procs = []
     for src in SOURCES:
-        obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        cmd = [cc] + HIPCC_FLAGS + EXTRA_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
-        if verbose:
-            print(" ".join(cmd), flush=True)
-        procs.append((src, obj, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
+        for suffix, elem in PER_ELEMENT.get(src, (("", 0),)):
+            obj = os.path.join(objdir, src.replace(".hip", suffix + ".o"))
+            cmd = ([cc] + HIPCC_FLAGS + EXTRA_FLAGS.get(src, []) + ["-DGENBMM_ELEM=%d" % elem, "-c",
+                   os.path.join(CSRC, src), "-o", obj])
+            if verbose:
+                print(" ".join(cmd), flush=True)
+            procs.append((src + suffix, obj,
+                          subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
     objs = []
     for src, obj, proc in procs:
         out = proc.communicate()[0].decode()

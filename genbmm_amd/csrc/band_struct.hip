@@ -7,7 +7,7 @@
 // an LDS tile).
 #include "common.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 namespace {
 
 constexpr int kST = 256;                 // lanes per workgroup
@@ -280,13 +280,13 @@ int shift_of(int v) {
 }
 
 }  // namespace
-}  // namespace genbmm
+}  // namespace GENBMM_NS
 
 extern "C" {
 
 int genbmm_band_shift(const float* data, float* out, int B, int n, int w_in, int w_out, int dcol,
                       int dband, float fill, void* stream) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   if (int e = check_band(B, n, w_in)) return e;
   if (int e = check_band(B, n, w_out)) return e;
   const int64_t cells = (int64_t)B * n * w_out;
@@ -302,7 +302,7 @@ int genbmm_band_shift(const float* data, float* out, int B, int n, int w_in, int
 
 int genbmm_band_op(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
                    float* out, int B, int n, int op, float zero, void* stream) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   if (a_lu < 0 || a_ld < 0 || b_lu < 0 || b_ld < 0) return GENBMM_E_BAND;
   if (op < kOpAdd || op > kOpMin) return GENBMM_E_MODE;
   const int64_t wa = (int64_t)a_lu + a_ld + 1, wb = (int64_t)b_lu + b_ld + 1;
@@ -324,7 +324,7 @@ int genbmm_band_op(const float* a, int a_lu, int a_ld, const float* b, int b_lu,
 
 int genbmm_band_transpose(const float* data, float* out, int B, int n, int lu, int ld,
                           void* stream) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   if (lu < 0 || ld < 0) return GENBMM_E_BAND;
   const int64_t w = (int64_t)lu + ld + 1;
   if (int e = check_band(B, n, w)) return e;
@@ -353,7 +353,7 @@ int genbmm_band_transpose(const float* data, float* out, int B, int n, int lu, i
 
 int genbmm_band_to_dense(const float* data, float* out, int B, int n, int lu, int ld, float fill,
                          void* stream) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   if (lu < 0 || ld < 0) return GENBMM_E_BAND;
   const int64_t w = (int64_t)lu + ld + 1;
   if (int e = check_band(B, n, w)) return e;
@@ -376,7 +376,7 @@ int genbmm_band_to_dense(const float* data, float* out, int B, int n, int lu, in
 
 int genbmm_band_from_dense(const float* dense, float* out, int B, int n_rows, int n, int lu,
                            int ld, void* stream) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   if (lu < 0 || ld < 0) return GENBMM_E_BAND;
   if (n_rows < 0 || n_rows > kMaxLine) return GENBMM_E_SHAPE;
   const int64_t w = (int64_t)lu + ld + 1;

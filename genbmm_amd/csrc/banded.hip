@@ -26,7 +26,7 @@
 #include "banded_max.h"
 #include "banded_strip.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 namespace {
 
 constexpr size_t kStripLdsLimit = 64 * 1024;  // dynamic LDS available without opting in
@@ -141,19 +141,19 @@ inline void set_workspace(BandArgs& p, float* ws, int B) {
 }
 
 }  // namespace
-}  // namespace genbmm
+}  // namespace GENBMM_NS
 
 extern "C" {
 
 size_t genbmm_banded_workspace_size(int a_lu, int a_ld, int b_lu, int b_ld, int B, int n) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   BandArgs p{};
   if (fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return 0;
   return band_ws_floats(p, B);
 }
 
 size_t genbmm_banded_scratch_size(int a_lu, int a_ld, int b_lu, int b_ld, int B, int n) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   BandArgs p{};
   if (fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return 0;
   return dir_bwd_ok(p) || !workspace_used(p) ? 0 : (size_t)B * n * p.Wo;
@@ -162,7 +162,7 @@ size_t genbmm_banded_scratch_size(int a_lu, int a_ld, int b_lu, int b_ld, int B,
 int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
                       float* out, int32_t* idx, float* workspace, int B, int n, int mode,
                       void* stream) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
     return GENBMM_E_MODE;
   BandArgs p{};
@@ -224,7 +224,7 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   return launch_status();
 }
 
-namespace genbmm {
+namespace GENBMM_NS {
 namespace {
 // `scratch`: where g / S goes in the prepared log product; NULL: the workspace's own part
 int banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
@@ -318,12 +318,12 @@ int banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int
   return launch_status();
 }
 }  // namespace
-}  // namespace genbmm
+}  // namespace GENBMM_NS
 
 int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
                       const float* out, const int32_t* idx, float* workspace, const float* g,
                       float* grad_a, float* grad_b, int B, int n, int mode, void* stream) {
-  return genbmm::banded_bwd(a, a_lu, a_ld, b, b_lu, b_ld, out, idx, workspace, nullptr, g, grad_a, grad_b, B, n,
+  return GENBMM_NS::banded_bwd(a, a_lu, a_ld, b, b_lu, b_ld, out, idx, workspace, nullptr, g, grad_a, grad_b, B, n,
                             mode, stream);
 }
 
@@ -334,7 +334,7 @@ int genbmm_banded_bwd_scratch(const float* a, int a_lu, int a_ld, const float* b
   if (workspace && !scratch && mode == GENBMM_BAND_LOG &&
       genbmm_banded_scratch_size(a_lu, a_ld, b_lu, b_ld, B, n) != 0)
     return GENBMM_E_NULLPTR;
-  return genbmm::banded_bwd(a, a_lu, a_ld, b, b_lu, b_ld, out, idx, const_cast<float*>(workspace), scratch, g,
+  return GENBMM_NS::banded_bwd(a, a_lu, a_ld, b, b_lu, b_ld, out, idx, const_cast<float*>(workspace), scratch, g,
                             grad_a, grad_b, B, n, mode, stream);
 }
 
@@ -343,7 +343,7 @@ int genbmm_banded_bwdbwd(const float* a, int a_lu, int a_ld, const float* b, int
                          const float* out, const float* g, const float* u_a, const float* u_b,
                          float* grad_a, float* grad_b, float* grad_g, int B, int n,
                          void* stream) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   BandArgs p{};
   if (int e = fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return e;
   if ((int64_t)B * n == 0) return GENBMM_OK;

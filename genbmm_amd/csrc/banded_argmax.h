@@ -18,7 +18,7 @@
 
 #include "banded_cells.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 
 constexpr int kAT = 64;        // rows per strip
 constexpr int kAJ = 32;        // diagonals per tile
@@ -163,4 +163,4 @@ __global__ __launch_bounds__(256) void k_band_argmax_bwd_b(const BandArgs p, int
   }
 }
 
-}  // namespace genbmm
+}  // namespace GENBMM_NS

@@ -6,7 +6,7 @@
 
 #include "common.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 
 // T: element type of the operands and results (float; double for the fp64 entry
 // points, which run these per-cell kernels only).
@@ -293,4 +293,4 @@ inline int fill_band(BandArgsT<T>& p, int a_lu, int a_ld, int b_lu, int b_ld, in
 
 inline dim3 blocks_for(long total) { return dim3((unsigned)((total + 255) / 256)); }
 
-}  // namespace genbmm
+}  // namespace GENBMM_NS

@@ -57,7 +57,7 @@
 
 #include "banded_flat.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 
 constexpr int kDirFwd = 0, kDirGradA = 1, kDirGradB = 2;
 constexpr int kDirTiles = 16;   // tiles per tile row, at most (a bit per cell in 64 bits)
@@ -563,4 +563,4 @@ __global__ __launch_bounds__(64 * kDirWaves) void k_band_dir(const BandArgs p, c
   else dir_row<KIND, PREP, true>(p, g, bn, i0, lane, lds, rows);
 }
 
-}  // namespace genbmm
+}  // namespace GENBMM_NS

@@ -7,7 +7,7 @@
 
 #include "banded_strip.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 
 constexpr int kMmSlack = 8;    // spare floats around a staged block
 typedef float mm_f4 __attribute__((ext_vector_type(4)));
@@ -128,4 +128,4 @@ struct MmFlat {
   }
 };
 
-}  // namespace genbmm
+}  // namespace GENBMM_NS

@@ -19,7 +19,7 @@
 
 #include "banded_flat.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 
 constexpr int kMaxRows = 64;
 
@@ -189,4 +189,4 @@ __global__ __launch_bounds__(256, 2) void k_band_max_fwd(const BandArgs p, int s
   }
 }
 
-}  // namespace genbmm
+}  // namespace GENBMM_NS

@@ -29,7 +29,7 @@
 
 #include "banded_cells.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 
 constexpr int kBT = 64;              // rows per strip = lanes of a wave
 constexpr int kBJ = 32;              // band-axis chunk: 4 waves x 8
@@ -694,4 +694,4 @@ inline StripDims strip_dims(int w_own, int w_sl) {
   return d;
 }
 
-}  // namespace genbmm
+}  // namespace GENBMM_NS

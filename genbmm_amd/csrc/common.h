@@ -6,7 +6,42 @@
 
 #include "../../include/genbmm_gfx950.h"
 
-namespace genbmm {
+// Element type of the caller's tensors.  The dense sources are compiled once per element
+// type (GENBMM_ELEM: 0 float, 1 IEEE binary16, 2 bfloat16), each into a namespace and a
+// set of entry-point names of its own; arithmetic, LDS and every workspace are fp32 in all
+// three: a half value is widened by the load that fetches it and a result is rounded
+// (to nearest even) by the store that writes it.
+#ifndef GENBMM_ELEM
+#define GENBMM_ELEM 0
+#endif
+#if GENBMM_ELEM == 0
+#define GENBMM_NS genbmm_f32
+#define GENBMM_API(name) genbmm_##name
+#elif GENBMM_ELEM == 1
+#define GENBMM_NS genbmm_f16
+#define GENBMM_API(name) genbmm_##name##_f16
+#elif GENBMM_ELEM == 2
+#define GENBMM_NS genbmm_bf16
+#define GENBMM_API(name) genbmm_##name##_bf16
+#else
+#error "GENBMM_ELEM: 0 (float), 1 (binary16) or 2 (bfloat16)"
+#endif
+
+namespace GENBMM_NS {
+
+#if GENBMM_ELEM == 0
+typedef float elem_t;
+typedef float abi_t;       // what the C header declares for an element
+#elif GENBMM_ELEM == 1
+typedef _Float16 elem_t;
+typedef uint16_t abi_t;
+#else
+typedef __bf16 elem_t;
+typedef uint16_t abi_t;
+#endif
+constexpr bool kElemF32 = GENBMM_ELEM == 0;
+inline const elem_t* el(const abi_t* p) { return reinterpret_cast<const elem_t*>(p); }
+inline elem_t* el(abi_t* p) { return reinterpret_cast<elem_t*>(p); }
 
 // Floor of every running maximum, as in the reference kernels
 // (matmul_cuda_kernel.cu:31,62,93,139; banded_cuda_kernel.cu:44,79).
@@ -22,6 +57,92 @@ __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_lo
 __device__ __forceinline__ float fast_exp(float x) { return fast_exp2(x * kLog2e); }
 
 constexpr int kPad = 4;  // LDS row padding (floats); keeps float4 alignment
+
+// ------------------------------------------------------- four elements at a time
+// ld4 / st4: element alignment only (the hardware takes misaligned dwordx4 / dwordx2;
+// rows of odd-sized matrices start anywhere).  ld4a / st4a: the address is a multiple of
+// four elements.  The masked forms touch the first cnt (<= 0: none, >= 4: all) elements.
+typedef float f4v __attribute__((ext_vector_type(4)));
+typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
+typedef _Float16 h4v __attribute__((ext_vector_type(4)));
+typedef _Float16 h4u __attribute__((ext_vector_type(4), aligned(2)));
+typedef __bf16 b4v __attribute__((ext_vector_type(4)));
+typedef __bf16 b4u __attribute__((ext_vector_type(4), aligned(2)));
+__device__ __forceinline__ float4 from_f4v(f4v f) { return make_float4(f.x, f.y, f.z, f.w); }
+// A result is rounded to fp32 first and to the half type second, exactly as if the float
+// kernel's output were converted afterwards.  Left alone, the compiler folds a multiply that
+// feeds the conversion into one instruction with a single rounding (v_fma_mixlo_f16), which
+// differs on ties; `settled` hides the value's origin from it (no instruction is emitted).
+__device__ __forceinline__ float settled(float x) {
+  asm volatile("" : "+v"(x));
+  return x;
+}
+__device__ __forceinline__ f4v to_f4v(float4 v) {
+  f4v f;
+  f.x = settled(v.x); f.y = settled(v.y); f.z = settled(v.z); f.w = settled(v.w);
+  return f;
+}
+// float -> element, for scalar stores
+template <class E>
+__device__ __forceinline__ E to_elem(float x) {
+  if constexpr (sizeof(E) == 4) return x;
+  else return (E)settled(x);
+}
+__device__ __forceinline__ float4 ld4(const float* p) {
+  const float4u v = *reinterpret_cast<const float4u*>(p);
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ float4 ld4(const _Float16* p) {
+  return from_f4v(__builtin_convertvector(*reinterpret_cast<const h4u*>(p), f4v));
+}
+__device__ __forceinline__ float4 ld4(const __bf16* p) {
+  return from_f4v(__builtin_convertvector(*reinterpret_cast<const b4u*>(p), f4v));
+}
+__device__ __forceinline__ float4 ld4a(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 ld4a(const _Float16* p) {
+  return from_f4v(__builtin_convertvector(*reinterpret_cast<const h4v*>(p), f4v));
+}
+__device__ __forceinline__ float4 ld4a(const __bf16* p) {
+  return from_f4v(__builtin_convertvector(*reinterpret_cast<const b4v*>(p), f4v));
+}
+__device__ __forceinline__ void st4(float* p, float4 v) {
+  float4u u;
+  u.x = v.x; u.y = v.y; u.z = v.z; u.w = v.w;
+  *reinterpret_cast<float4u*>(p) = u;
+}
+__device__ __forceinline__ void st4(_Float16* p, float4 v) {
+  *reinterpret_cast<h4u*>(p) = __builtin_convertvector(to_f4v(v), h4u);
+}
+__device__ __forceinline__ void st4(__bf16* p, float4 v) {
+  *reinterpret_cast<b4u*>(p) = __builtin_convertvector(to_f4v(v), b4u);
+}
+__device__ __forceinline__ void st4a(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void st4a(_Float16* p, float4 v) {
+  *reinterpret_cast<h4v*>(p) = __builtin_convertvector(to_f4v(v), h4v);
+}
+__device__ __forceinline__ void st4a(__bf16* p, float4 v) {
+  *reinterpret_cast<b4v*>(p) = __builtin_convertvector(to_f4v(v), b4v);
+}
+template <class E>
+__device__ __forceinline__ float4 ld4m(const E* p, int cnt, float fill) {
+  if (cnt >= 4) return ld4(p);
+  float4 r = make_float4(fill, fill, fill, fill);
+  if (cnt > 0) r.x = p[0];
+  if (cnt > 1) r.y = p[1];
+  if (cnt > 2) r.z = p[2];
+  return r;
+}
+template <class E>
+__device__ __forceinline__ void st4m(E* p, int cnt, float4 v) {
+  if (cnt >= 4) {
+    st4(p, v);
+    return;
+  }
+  if (cnt > 0) p[0] = to_elem<E>(v.x);
+  if (cnt > 1) p[1] = to_elem<E>(v.y);
+  if (cnt > 2) p[2] = to_elem<E>(v.z);
+}
+__device__ __forceinline__ int clamp4(int x) { return min(max(x, 0), 4); }
 
 // ---------------------------------------------------------------- tile loaders
 //
@@ -41,7 +162,8 @@ struct TileOutMajor {
   static constexpr int LD = OUT + kPad;
   float4 r[PER];
 
-  __device__ __forceinline__ void gload(const float* __restrict__ base, long ld,
+  template <class E>
+  __device__ __forceinline__ void gload(const E* __restrict__ base, long ld,
                                         int out0, int red0, int out_lim,
                                         int red_lim, bool vec, int tid) {
 #pragma unroll
@@ -52,9 +174,9 @@ struct TileOutMajor {
         const int row = idx / C4, c4 = idx % C4;
         const int go = out0 + row, gr = red0 + c4 * 4;
         if (go < out_lim && gr < red_lim) {
-          const float* p = base + (long)go * ld + gr;
+          const E* p = base + (long)go * ld + gr;
           if (vec && gr + 3 < red_lim) {
-            v = *reinterpret_cast<const float4*>(p);
+            v = ld4a(p);
           } else {
             v.x = p[0];
             if (gr + 1 < red_lim) v.y = p[1];
@@ -93,7 +215,8 @@ struct TileRedMajor {
   static constexpr int LD = OUT + kPad;
   float4 r[PER];
 
-  __device__ __forceinline__ void gload(const float* __restrict__ base, long ld,
+  template <class E>
+  __device__ __forceinline__ void gload(const E* __restrict__ base, long ld,
                                         int out0, int red0, int out_lim,
                                         int red_lim, bool vec, int tid) {
 #pragma unroll
@@ -104,9 +227,9 @@ struct TileRedMajor {
         const int row = idx / C4, c4 = idx % C4;
         const int gr = red0 + row, go = out0 + c4 * 4;
         if (gr < red_lim && go < out_lim) {
-          const float* p = base + (long)gr * ld + go;
+          const E* p = base + (long)gr * ld + go;
           if (vec && go + 3 < out_lim) {
-            v = *reinterpret_cast<const float4*>(p);
+            v = ld4a(p);
           } else {
             v.x = p[0];
             if (go + 1 < out_lim) v.y = p[1];
@@ -145,7 +268,8 @@ __device__ __forceinline__ void lds_frag(const float* __restrict__ row, int off,
   }
 }
 
-// 16-byte alignment test used to enable float4 global accesses.
+// 16-byte alignment test used to enable four-element global accesses (stricter than
+// needed for the half types).
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // ------------------------------------------------------------------- Philox
@@ -257,4 +381,4 @@ inline int launch_status() {
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-}  // namespace genbmm
+}  // namespace GENBMM_NS

@@ -1,9 +1,10 @@
 // Dense semiring batched matmul, backward and second-order kernels (gfx950).
 #include "common.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 namespace {
 
+#if GENBMM_ELEM == 0  // second order: float tensors only (grad_g is re-read as an operand)
 // ===================================================== logbmm second order
 //
 // With p = exp(a+b-out), w = u_a[m,k] + u_b[k,n]  (a missing u counts as 0):
@@ -125,6 +126,8 @@ __global__ __launch_bounds__(256) void k_log_bwdbwd_b(const BB p, long total) {
   p.gb[e] = acc;
 }
 
+#endif
+
 // ===================================================== argmax backward
 //
 // maxbmm / samplebmm:  grad_a[m,k] = sum_n [k == idx[m,n]] g[m,n]
@@ -149,11 +152,11 @@ constexpr int kKC = 128;  // cells of the reduction axis per lane
 // grad_a: line = row m.  The row is read 16 cells at a time (int4 / float4 when the
 // rows are 16-byte aligned), then the 16 additions are made in order.
 template <int PROD>
-__global__ __launch_bounds__(64) void k_argmax_bwd_a(const float* __restrict__ bmat,
+__global__ __launch_bounds__(64) void k_argmax_bwd_a(const elem_t* __restrict__ bmat,
                                                     const float* __restrict__ fac,
                                                     const int32_t* __restrict__ idx,
-                                                    const float* __restrict__ g,
-                                                    float* __restrict__ grad_a, int M, int K,
+                                                    const elem_t* __restrict__ g,
+                                                    elem_t* __restrict__ grad_a, int M, int K,
                                                     int N, int row_tiles, int k_chunks, int ps,
                                                     int vec) {
   __shared__ float accs[64 * kKC + 64 + 64];
@@ -169,8 +172,8 @@ __global__ __launch_bounds__(64) void k_argmax_bwd_a(const float* __restrict__ b
   const int m = m0 + line;
   const bool live = m < M;
   const int32_t* irow = idx + ((long)batch * M + (live ? m : 0)) * N;
-  const float* grow = g + ((long)batch * M + (live ? m : 0)) * N;
-  const float* bb = PROD == 1 ? bmat + (long)batch * K * N : nullptr;
+  const elem_t* grow = g + ((long)batch * M + (live ? m : 0)) * N;
+  const elem_t* bb = PROD == 1 ? bmat + (long)batch * K * N : nullptr;
   const float* frow = PROD == 2 ? fac + ((long)batch * M + (live ? m : 0)) * N : nullptr;
   const int base = line * (kw + 1) + part * kKC;
   float* mine = accs + base;
@@ -200,7 +203,7 @@ __global__ __launch_bounds__(64) void k_argmax_bwd_a(const float* __restrict__ b
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           iv[q] = *reinterpret_cast<const int4*>(irow + n + 4 * q);
-          gv[q] = *reinterpret_cast<const float4*>(grow + n + 4 * q);
+          gv[q] = ld4a(grow + n + 4 * q);
         }
         if (PROD == 2) {
 #pragma unroll
@@ -234,19 +237,19 @@ __global__ __launch_bounds__(64) void k_argmax_bwd_a(const float* __restrict__ b
   __syncthreads();
   const int rows = min(lines, M - m0), kn = min(kw, K - w0);
   for (int r = 0; r < rows; ++r) {
-    float* dst = grad_a + ((long)batch * M + m0 + r) * K + w0;
-    for (int kk = lane; kk < kn; kk += 64) dst[kk] = accs[r * (kw + 1) + kk];
+    elem_t* dst = grad_a + ((long)batch * M + m0 + r) * K + w0;
+    for (int kk = lane; kk < kn; kk += 64) dst[kk] = to_elem<elem_t>(accs[r * (kw + 1) + kk]);
   }
 }
 
 // grad_b: line = column n; the column is read 16 rows at a time, then added in order.
 // Accumulators are [k][line].
 template <int PROD>
-__global__ __launch_bounds__(64) void k_argmax_bwd_b(const float* __restrict__ amat,
+__global__ __launch_bounds__(64) void k_argmax_bwd_b(const elem_t* __restrict__ amat,
                                                     const float* __restrict__ fac,
                                                     const int32_t* __restrict__ idx,
-                                                    const float* __restrict__ g,
-                                                    float* __restrict__ grad_b, int M, int K,
+                                                    const elem_t* __restrict__ g,
+                                                    elem_t* __restrict__ grad_b, int M, int K,
                                                     int N, int col_tiles, int k_chunks, int ps) {
   __shared__ float accs[kKC * 64 + 64];
   const int lane = threadIdx.x, parts = 1 << ps, lines = 64 >> ps;
@@ -261,8 +264,8 @@ __global__ __launch_bounds__(64) void k_argmax_bwd_b(const float* __restrict__ a
   const bool live = n < N;
   const int nn = live ? n : N - 1;
   const int32_t* icol = idx + (long)batch * M * N + nn;
-  const float* gcol = g + (long)batch * M * N + nn;
-  const float* ab = PROD == 1 ? amat + (long)batch * M * K : nullptr;
+  const elem_t* gcol = g + (long)batch * M * N + nn;
+  const elem_t* ab = PROD == 1 ? amat + (long)batch * M * K : nullptr;
   const float* fcol = PROD == 2 ? fac + (long)batch * M * N + nn : nullptr;
   const int base = (part * kKC) * lines + line;  // cell k of this lane: accs[base + k * lines]
   float* mine = accs + base;
@@ -309,7 +312,7 @@ __global__ __launch_bounds__(64) void k_argmax_bwd_b(const float* __restrict__ a
   const int lc = lane & (lines - 1), lk = lane / lines;
   if (lc < cols)
     for (int kk = lk; kk < kn; kk += parts)
-      grad_b[((long)batch * K + w0 + kk) * N + n0 + lc] = accs[kk * lines + lc];
+      grad_b[((long)batch * K + w0 + kk) * N + n0 + lc] = to_elem<elem_t>(accs[kk * lines + lc]);
 }
 
 // Parts per workgroup for a reduction axis of K cells: the smallest power of two that
@@ -321,8 +324,8 @@ inline int argmax_parts_shift(int K) {
 }
 
 template <bool PROD>
-int run_argmax_bwd(const float* a, const float* b, const int32_t* idx, const float* factors,
-                   const float* g, float* grad_a, float* grad_b, int B, int M, int K, int N,
+int run_argmax_bwd(const elem_t* a, const elem_t* b, const int32_t* idx, const float* factors,
+                   const elem_t* g, elem_t* grad_a, elem_t* grad_b, int B, int M, int K, int N,
                    void* stream) {
   if (int e = check_dense_dims(B, M, K, N)) return e;
   const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
@@ -366,14 +369,15 @@ int run_argmax_bwd(const float* a, const float* b, const int32_t* idx, const flo
 }
 
 }  // namespace
-}  // namespace genbmm
+}  // namespace GENBMM_NS
 
 extern "C" {
 
+#if GENBMM_ELEM == 0
 int genbmm_logbmm_bwdbwd(const float* a, const float* b, const float* out, const float* g,
                          const float* u_a, const float* u_b, float* grad_a, float* grad_b,
                          float* grad_g, int B, int M, int K, int N, void* stream) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   if (int e = check_dense_dims(B, M, K, N)) return e;
   {
     const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
@@ -402,16 +406,22 @@ int genbmm_logbmm_bwdbwd(const float* a, const float* b, const float* out, const
   return GENBMM_OK;
 }
 
-int genbmm_argmax_bwd(const int32_t* idx, const float* g, float* grad_a, float* grad_b, int B,
-                      int M, int K, int N, void* stream) {
-  return genbmm::run_argmax_bwd<false>(nullptr, nullptr, idx, nullptr, g, grad_a, grad_b, B, M,
-                                       K, N, stream);
+#endif
+
+// One set per element type: genbmm_argmax_bwd, genbmm_argmax_bwd_f16, ..._bf16, ...
+int GENBMM_API(argmax_bwd)(const int32_t* idx, const GENBMM_NS::abi_t* g, GENBMM_NS::abi_t* grad_a,
+                           GENBMM_NS::abi_t* grad_b, int B, int M, int K, int N, void* stream) {
+  using namespace GENBMM_NS;
+  return run_argmax_bwd<false>(nullptr, nullptr, idx, nullptr, el(g), el(grad_a), el(grad_b), B, M, K, N,
+                               stream);
 }
 
-int genbmm_prodmax_bwd(const float* a, const float* b, const int32_t* idx, const float* factors,
-                       const float* g, float* grad_a, float* grad_b, int B, int M, int K, int N,
-                       void* stream) {
-  return genbmm::run_argmax_bwd<true>(a, b, idx, factors, g, grad_a, grad_b, B, M, K, N, stream);
+int GENBMM_API(prodmax_bwd)(const GENBMM_NS::abi_t* a, const GENBMM_NS::abi_t* b, const int32_t* idx,
+                            const float* factors, const GENBMM_NS::abi_t* g, GENBMM_NS::abi_t* grad_a,
+                            GENBMM_NS::abi_t* grad_b, int B, int M, int K, int N, void* stream) {
+  using namespace GENBMM_NS;
+  return run_argmax_bwd<true>(el(a), el(b), idx, factors, el(g), el(grad_a), el(grad_b), B, M, K, N,
+                              stream);
 }
 
 }  // extern "C"

@@ -13,7 +13,7 @@
 #include "dense_tiles.h"
 #include "logbmm_ws.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 namespace {
 
 // ------------------------------------------------------- max / prod-max forward
@@ -43,8 +43,8 @@ __global__ __launch_bounds__(C::NT) void k_max_fwd(const DenseArgs p) {
   int batch, m0, n0;
   decode_tile<C>(p, batch, m0, n0);
   const int M = p.M, K = p.K, N = p.N;
-  const float* ab = p.a + (long)batch * M * K;
-  const float* bb = p.b + (long)batch * K * N;
+  const elem_t* ab = p.a + (long)batch * M * K;
+  const elem_t* bb = p.b + (long)batch * K * N;
 
   float mx[C::TM][C::TN];
   int ind[C::TM][C::TN];
@@ -143,10 +143,10 @@ constexpr int kResGroup = 8, kResWaves = 8, kResRows = 4, kResStage = 8;
 constexpr int kResFloats = 16384;  // 64 KB of LDS
 static_assert(kMaxGroup == kResGroup, "");
 
-typedef float float4_u __attribute__((ext_vector_type(4), aligned(4)));
-
-template <int COLS, bool TAIL, int G, int R, class Op>
-__device__ __forceinline__ void resolve_walk(const float* __restrict__ first, const float* __restrict__ second,
+// E: element type of the two operands (the caller's for max / prod-max, fp32 for the
+// factors the sampling sweep runs on).
+template <int COLS, bool TAIL, int G, int R, class E, class Op>
+__device__ __forceinline__ void resolve_walk(const E* __restrict__ first, const E* __restrict__ second,
                                              int32_t* __restrict__ idx, Op& op, int M, int K, int N,
                                              int panels, int row_chunks, int rows_per, float* Bs) {
   constexpr int RPW = 64 / COLS;           // rows a wave takes per step
@@ -165,8 +165,8 @@ __device__ __forceinline__ void resolve_walk(const float* __restrict__ first, co
   const bool live = n < N;
   const int nc = min(n, N - 1);
   const int m_beg = chunk * rows_per, m_end = min(M, m_beg + rows_per);
-  const float* ab = first + (long)batch * M * K;
-  const float* bb = second + (long)batch * K * N;
+  const E* ab = first + (long)batch * M * K;
+  const E* bb = second + (long)batch * K * N;
   const long cell0 = (long)batch * M * N;
   const int32_t* ib = idx + cell0;
   using Extra = typename Op::Extra;
@@ -193,11 +193,11 @@ __device__ __forceinline__ void resolve_walk(const float* __restrict__ first, co
       const bool act = code[r] <= -2 && k >= kc && k < kc + KSTAGE;
       kb[r] = act ? k : -1;
       const int ks = act ? k : kc;
-      const float* ar = ab + (long)min(row_of(mb, r), M - 1) * K + ks;
+      const E* ar = ab + (long)min(row_of(mb, r), M - 1) * K + ks;
       if (!TAIL) {
 #pragma unroll
         for (int q = 0; q < G / 4; ++q) {
-          const float4_u x = *reinterpret_cast<const float4_u*>(ar + 4 * q);
+          const float4 x = ld4(ar + 4 * q);
           av[r][4 * q] = x.x; av[r][4 * q + 1] = x.y; av[r][4 * q + 2] = x.z; av[r][4 * q + 3] = x.w;
         }
       } else {
@@ -281,13 +281,13 @@ inline int resolve_grid(int B, int M, int N, int cols, int rows_step, int& panel
 template <bool PROD>
 struct MaxResolve {
   struct Extra {};
-  float* out;
+  elem_t* out;
   int32_t* idx;
   float* fa;  // optional: the two factors of the winning term per cell (product semiring)
   float* fb;
   __device__ __forceinline__ Extra load(long) const { return Extra{}; }
   __device__ __forceinline__ void none(long e) const {
-    out[e] = kFloor;
+    out[e] = to_elem<elem_t>(kFloor);
     if (fa) {
       fa[e] = 0.f;
       fb[e] = 0.f;
@@ -317,7 +317,7 @@ struct MaxResolve {
         if (j == first) v = t[j];
     }
     idx[e] = kb + first;
-    out[e] = v;
+    out[e] = to_elem<elem_t>(v);
     if (fa) {
       float sa = av[0], sb = bv[0];
 #pragma unroll
@@ -334,7 +334,7 @@ struct MaxResolve {
 // TAIL: K is not a multiple of the group, the last group is cut at K.
 template <bool PROD, int COLS, bool TAIL>
 __global__ __launch_bounds__(kResWaves * 64, 4) void k_max_resolve(
-    const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ out,
+    const elem_t* __restrict__ a, const elem_t* __restrict__ b, elem_t* __restrict__ out,
     int32_t* __restrict__ idx, float* __restrict__ fac_a, float* __restrict__ fac_b, int M, int K,
     int N, int panels, int row_chunks, int rows_per) {
   __shared__ float Bs[kResFloats];
@@ -384,9 +384,16 @@ __global__ __launch_bounds__(C::NT, 2) void k_sample_sweep(const DenseArgs p,
   int batch, m0, n0;
   decode_tile<C>(p, batch, m0, n0);
   const int M = p.M, K = p.K, N = p.N;
-  const float* ab = (TWO ? ws_ea : p.a) + (long)batch * M * K;
-  const float* bb = (TWO ? ws_eb : p.b) + (long)batch * K * N;
-  const float* ob = p.out + (long)batch * M * N;
+  using SrcT = std::conditional_t<TWO, float, elem_t>;  // the factors are fp32, the operands the caller's
+  const SrcT *ab, *bb;
+  if constexpr (TWO) {
+    ab = ws_ea + (long)batch * M * K;
+    bb = ws_eb + (long)batch * K * N;
+  } else {
+    ab = p.a + (long)batch * M * K;
+    bb = p.b + (long)batch * K * N;
+  }
+  const elem_t* ob = p.out + (long)batch * M * N;
   const float* st = stats + (long)batch * (M + N);
   for (int t = tid; t < C::BM; t += C::NT) al[t] = (m0 + t < M) ? st[m0 + t] : 0.f;
   for (int t = tid; t < C::BN; t += C::NT) be[t] = (n0 + t < N) ? st[M + n0 + t] : 0.f;
@@ -634,7 +641,7 @@ int launch_sample(DenseArgs p, int B, int M, int K, int N, hipStream_t s) {
 }
 
 template <bool PROD>
-int run_max(const float* a, const float* b, float* out, int32_t* idx, float* factors, int B,
+int run_max(const elem_t* a, const elem_t* b, elem_t* out, int32_t* idx, float* factors, int B,
             int M, int K, int N, void* stream) {
   if (int e = check_dense_dims(B, M, K, N)) return e;
   const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
@@ -698,7 +705,7 @@ int launch_sweep_two(DenseArgs p, const float* stats, const LogFactors& f, int B
   return launch_sample_resolve<kSampleGroup>(p, f, B, M, K, N, s);
 }
 
-int run_sample(const float* a, const float* b, float* out, int32_t* idx, float* stats,
+int run_sample(const elem_t* a, const elem_t* b, elem_t* out, int32_t* idx, float* stats,
                uint64_t seed, uint64_t offset, int B, int M, int K, int N, void* stream) {
   if (int e = check_dense_dims(B, M, K, N)) return e;
   const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
@@ -708,9 +715,14 @@ int run_sample(const float* a, const float* b, float* out, int32_t* idx, float* 
   DenseArgs p{};
   p.a = a; p.b = b; p.out = out; p.idx = idx; p.seed = seed; p.offset = offset;
   hipStream_t s = (hipStream_t)stream;
-  if (stats && K > 0) {  // log-sum-exp by the logbmm forward, then the multiply-only sweep
+  LogFactors f;
+  // The vector-ALU sweeps take S = exp(out - alpha - beta) from `out` as stored; rounded to a
+  // half type that is S within 2^-9 |out| at best, and targets u S past the true sum would be
+  // common.  Half tensors therefore sweep only where 1/S itself is at hand in fp32 (the
+  // matrix-core sweep) and walk exactly otherwise.
+  const bool sweep = kElemF32 || (stats && log_fwd_writes_factors(stats, B, M, K, N, &f) && log_sample_mfma_ok(K));
+  if (stats && K > 0 && sweep) {  // log-sum-exp by the logbmm forward, then the multiply-only sweep
     if (int e = log_fwd_with_factors(a, b, out, stats, B, M, K, N, s)) return e;
-    LogFactors f;
     if (log_fwd_writes_factors(stats, B, M, K, N, &f)) {
       if (log_sample_mfma_ok(K)) {  // sweep on the matrix cores, groups of 16 terms
         if (int e = log_sample_sweep_mfma(a, b, out, idx, stats, seed, offset, B, M, K, N, s)) return e;
@@ -735,24 +747,29 @@ int run_sample(const float* a, const float* b, float* out, int32_t* idx, float* 
 }
 
 }  // namespace
-}  // namespace genbmm
+}  // namespace GENBMM_NS
 
 extern "C" {
 
-int genbmm_samplebmm_fwd(const float* a, const float* b, float* out, int32_t* idx, float* stats,
-                         uint64_t seed, uint64_t offset, int B, int M, int K, int N,
-                         void* stream) {
-  return genbmm::run_sample(a, b, out, idx, stats, seed, offset, B, M, K, N, stream);
+// One set per element type: genbmm_samplebmm_fwd, genbmm_samplebmm_fwd_f16, ..._bf16, ...
+int GENBMM_API(samplebmm_fwd)(const GENBMM_NS::abi_t* a, const GENBMM_NS::abi_t* b, GENBMM_NS::abi_t* out,
+                              int32_t* idx, float* stats, uint64_t seed, uint64_t offset, int B, int M,
+                              int K, int N, void* stream) {
+  using namespace GENBMM_NS;
+  return run_sample(el(a), el(b), el(out), idx, stats, seed, offset, B, M, K, N, stream);
 }
 
-int genbmm_maxbmm_fwd(const float* a, const float* b, float* out, int32_t* idx, int B, int M,
-                      int K, int N, void* stream) {
-  return genbmm::run_max<false>(a, b, out, idx, nullptr, B, M, K, N, stream);
+int GENBMM_API(maxbmm_fwd)(const GENBMM_NS::abi_t* a, const GENBMM_NS::abi_t* b, GENBMM_NS::abi_t* out,
+                           int32_t* idx, int B, int M, int K, int N, void* stream) {
+  using namespace GENBMM_NS;
+  return run_max<false>(el(a), el(b), el(out), idx, nullptr, B, M, K, N, stream);
 }
 
-int genbmm_prodmaxbmm_fwd(const float* a, const float* b, float* out, int32_t* idx,
-                          float* factors, int B, int M, int K, int N, void* stream) {
-  return genbmm::run_max<true>(a, b, out, idx, factors, B, M, K, N, stream);
+int GENBMM_API(prodmaxbmm_fwd)(const GENBMM_NS::abi_t* a, const GENBMM_NS::abi_t* b,
+                               GENBMM_NS::abi_t* out, int32_t* idx, float* factors, int B, int M, int K,
+                               int N, void* stream) {
+  using namespace GENBMM_NS;
+  return run_max<true>(el(a), el(b), el(out), idx, factors, B, M, K, N, stream);
 }
 
 }  // extern "C"

@@ -5,7 +5,7 @@
 
 #include "common.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 
 template <int BM_, int BN_, int TM_, int TN_, int KT_>
 struct Cfg {
@@ -16,9 +16,9 @@ struct Cfg {
 };
 
 struct DenseArgs {
-  const float* a;
-  const float* b;
-  float* out;
+  const elem_t* a;
+  const elem_t* b;
+  elem_t* out;
   int32_t* idx;
   int M, K, N;
   int tiles_m, tiles_n;
@@ -46,8 +46,8 @@ __device__ __forceinline__ int col_of(int tx, int j) {
   return (j >> 2) * (C::TX * 4) + tx * 4 + (j & 3);
 }
 
-template <class C>
-__device__ __forceinline__ void store_tile_f(float* __restrict__ outb, const float (&v)[C::TM][C::TN],
+template <class C, class E>
+__device__ __forceinline__ void store_tile_f(E* __restrict__ outb, const float (&v)[C::TM][C::TN],
                                              int m0, int n0, int M, int N, bool vec, int tx,
                                              int ty) {
 #pragma unroll
@@ -57,14 +57,13 @@ __device__ __forceinline__ void store_tile_f(float* __restrict__ outb, const flo
 #pragma unroll
     for (int q = 0; q < C::TN / 4; ++q) {
       const int n = n0 + col_of<C>(tx, 4 * q);
-      float* dst = outb + (long)m * N + n;
+      E* dst = outb + (long)m * N + n;
       if (vec && n + 3 < N) {
-        *reinterpret_cast<float4*>(dst) =
-            make_float4(v[i][4 * q], v[i][4 * q + 1], v[i][4 * q + 2], v[i][4 * q + 3]);
+        st4a(dst, make_float4(v[i][4 * q], v[i][4 * q + 1], v[i][4 * q + 2], v[i][4 * q + 3]));
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          if (n + e < N) dst[e] = v[i][4 * q + e];
+          if (n + e < N) dst[e] = to_elem<E>(v[i][4 * q + e]);
       }
     }
   }
@@ -106,8 +105,8 @@ __device__ __forceinline__ void log_fwd_tile(const DenseArgs& p, int batch, int 
                                              float* __restrict__ As, float* __restrict__ Bs) {
   const int tid = threadIdx.x, tx = tid % C::TX, ty = tid / C::TX;
   const int M = p.M, K = p.K, N = p.N;
-  const float* ab = p.a + (long)batch * M * K;
-  const float* bb = p.b + (long)batch * K * N;
+  const elem_t* ab = p.a + (long)batch * M * K;
+  const elem_t* bb = p.b + (long)batch * K * N;
 
   float mx[C::TM][C::TN], acc[C::TM][C::TN];
 #pragma unroll
@@ -297,4 +296,4 @@ inline int fill_args(DenseArgs& p, int B, int M, int K, int N, dim3& grid) {
   return GENBMM_OK;
 }
 
-}  // namespace genbmm
+}  // namespace GENBMM_NS

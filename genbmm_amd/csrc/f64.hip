@@ -10,7 +10,7 @@
 #include "banded_cells.h"
 #include "f64_mm.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 namespace {
 
 constexpr double kFloorD = -1e9;
@@ -310,13 +310,13 @@ inline void launch_d64_mm(const double* a, const double* b, const double* out, c
     launch_d64_mm_t<KIND, 64>(a, b, out, g, dst, B, M, K, N, s);
 }
 }  // namespace
-}  // namespace genbmm
+}  // namespace GENBMM_NS
 
 extern "C" {
 
 int genbmm_logbmm_fwd_f64(const double* a, const double* b, double* out, int B, int M, int K, int N,
                           void* stream) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   if (d64_mm_ok(B, M, K, N)) {
     if (int e = check_dense_dims(B, M, K, N)) return e;
     if (!a || !b || !out) return GENBMM_E_NULLPTR;
@@ -328,24 +328,24 @@ int genbmm_logbmm_fwd_f64(const double* a, const double* b, double* out, int B, 
 
 int genbmm_maxbmm_fwd_f64(const double* a, const double* b, double* out, int32_t* idx, int B, int M,
                           int K, int N, void* stream) {
-  return genbmm::run_fwd64<genbmm::kMax>(a, b, out, idx, 0, 0, B, M, K, N, stream);
+  return GENBMM_NS::run_fwd64<GENBMM_NS::kMax>(a, b, out, idx, 0, 0, B, M, K, N, stream);
 }
 
 int genbmm_prodmaxbmm_fwd_f64(const double* a, const double* b, double* out, int32_t* idx, int B,
                               int M, int K, int N, void* stream) {
-  return genbmm::run_fwd64<genbmm::kProdMax>(a, b, out, idx, 0, 0, B, M, K, N, stream);
+  return GENBMM_NS::run_fwd64<GENBMM_NS::kProdMax>(a, b, out, idx, 0, 0, B, M, K, N, stream);
 }
 
 int genbmm_samplebmm_fwd_f64(const double* a, const double* b, double* out, int32_t* idx,
                              uint64_t seed, uint64_t offset, int B, int M, int K, int N,
                              void* stream) {
-  return genbmm::run_fwd64<genbmm::kSample>(a, b, out, idx, seed, offset, B, M, K, N, stream);
+  return GENBMM_NS::run_fwd64<GENBMM_NS::kSample>(a, b, out, idx, seed, offset, B, M, K, N, stream);
 }
 
 int genbmm_logbmm_bwd_f64(const double* a, const double* b, const double* out, const double* g,
                           double* grad_a, double* grad_b, int B, int M, int K, int N,
                           void* stream) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   if (int e = check_dense_dims(B, M, K, N)) return e;
   const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
   if (missing(a, mk) || missing(b, kn) || missing(out, mn) || missing(g, mn) ||
@@ -378,7 +378,7 @@ int genbmm_logbmm_bwd_f64(const double* a, const double* b, const double* out, c
 int genbmm_logbmm_bwdbwd_f64(const double* a, const double* b, const double* out, const double* g,
                              const double* u_a, const double* u_b, double* grad_a, double* grad_b,
                              double* grad_g, int B, int M, int K, int N, void* stream) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   if (int e = check_dense_dims(B, M, K, N)) return e;
   const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
   if (missing(a, mk) || missing(b, kn) || missing(out, mn) || missing(g, mn) ||
@@ -395,19 +395,19 @@ int genbmm_logbmm_bwdbwd_f64(const double* a, const double* b, const double* out
 
 int genbmm_argmax_bwd_f64(const int32_t* idx, const double* g, double* grad_a, double* grad_b, int B,
                           int M, int K, int N, void* stream) {
-  return genbmm::run_argmax_bwd64<false>(nullptr, nullptr, idx, g, grad_a, grad_b, B, M, K, N,
+  return GENBMM_NS::run_argmax_bwd64<false>(nullptr, nullptr, idx, g, grad_a, grad_b, B, M, K, N,
                                          stream);
 }
 
 int genbmm_prodmax_bwd_f64(const double* a, const double* b, const int32_t* idx, const double* g,
                            double* grad_a, double* grad_b, int B, int M, int K, int N,
                            void* stream) {
-  return genbmm::run_argmax_bwd64<true>(a, b, idx, g, grad_a, grad_b, B, M, K, N, stream);
+  return GENBMM_NS::run_argmax_bwd64<true>(a, b, idx, g, grad_a, grad_b, B, M, K, N, stream);
 }
 
 int genbmm_banded_fwd_f64(const double* a, int a_lu, int a_ld, const double* b, int b_lu, int b_ld,
                           double* out, int32_t* idx, int B, int n, int mode, void* stream) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
     return GENBMM_E_MODE;
   BandArgsT<double> p{};
@@ -429,7 +429,7 @@ int genbmm_banded_fwd_f64(const double* a, int a_lu, int a_ld, const double* b, 
 int genbmm_banded_bwd_f64(const double* a, int a_lu, int a_ld, const double* b, int b_lu, int b_ld,
                           const double* out, const int32_t* idx, const double* g, double* grad_a,
                           double* grad_b, int B, int n, int mode, void* stream) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
     return GENBMM_E_MODE;
   BandArgsT<double> p{};
@@ -458,7 +458,7 @@ int genbmm_banded_bwdbwd_f64(const double* a, int a_lu, int a_ld, const double* 
                              int b_ld, const double* out, const double* g, const double* u_a,
                              const double* u_b, double* grad_a, double* grad_b, double* grad_g,
                              int B, int n, void* stream) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   BandArgsT<double> p{};
   if (int e = fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return e;
   if ((int64_t)B * n == 0) return GENBMM_OK;

@@ -28,7 +28,7 @@
 
 #include "common.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 
 constexpr int kDC = 16;        // contraction chunk
 constexpr int kDP = kDC + 1;   // row pitch of a staged chunk, in doubles: odd, so that lanes four rows apart
@@ -321,4 +321,4 @@ inline size_t d64_mm_lds(int kind, int tile, int M, int N) {
   return sizeof(double) * (2 * tile * kDP + (kind == kD64GradB ? M : tile) + (kind == kD64GradA ? N : tile));
 }
 
-}  // namespace genbmm
+}  // namespace GENBMM_NS

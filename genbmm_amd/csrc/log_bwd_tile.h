@@ -5,7 +5,7 @@
 
 #include "common.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 
 // ===================================================== logbmm backward
 //
@@ -31,11 +31,11 @@ struct BCfg {
 };
 
 struct LogBwdArgs {
-  const float* a;
-  const float* b;
-  const float* out;
-  const float* g;
-  float* grad;
+  const elem_t* a;
+  const elem_t* b;
+  const elem_t* out;
+  const elem_t* g;
+  elem_t* grad;
   int M, K, N;
   int tiles_r, tiles_c;
   int vec_k, vec_n;  // float4 access allowed along K-contiguous / N-contiguous rows
@@ -67,12 +67,12 @@ __device__ __forceinline__ void log_bwd_tile(const LogBwdArgs& p, int batch, int
   const int M = p.M, K = p.K, N = p.N;
   const int R = GRAD_A ? M : K, Cc = GRAD_A ? K : N, Q = GRAD_A ? N : M;
 
-  const float* ab = p.a + (long)batch * M * K;
-  const float* bb = p.b + (long)batch * K * N;
-  const float* ob = p.out + (long)batch * M * N;
-  const float* gb = p.g + (long)batch * M * N;
-  const float* xb = GRAD_A ? ab : bb;
-  const float* yb = GRAD_A ? bb : ab;
+  const elem_t* ab = p.a + (long)batch * M * K;
+  const elem_t* bb = p.b + (long)batch * K * N;
+  const elem_t* ob = p.out + (long)batch * M * N;
+  const elem_t* gb = p.g + (long)batch * M * N;
+  const elem_t* xb = GRAD_A ? ab : bb;
+  const elem_t* yb = GRAD_A ? bb : ab;
   const long ldy = GRAD_A ? N : K;
   const bool vec_x = GRAD_A ? p.vec_k : p.vec_n;  // X and grad rows are Cc long
   const bool vec_y = GRAD_A ? p.vec_n : p.vec_k;
@@ -93,9 +93,9 @@ __device__ __forceinline__ void log_bwd_tile(const LogBwdArgs& p, int batch, int
       const int c = c0 + col_of(4 * q4);
       float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
       if (r < R && c < Cc) {
-        const float* src = xb + (long)r * Cc + c;
+        const elem_t* src = xb + (long)r * Cc + c;
         if (vec_x && c + 3 < Cc) {
-          v = *reinterpret_cast<const float4*>(src);
+          v = ld4a(src);
         } else {
           v.x = src[0];
           if (c + 1 < Cc) v.y = src[1];
@@ -164,7 +164,7 @@ __device__ __forceinline__ void log_bwd_tile(const LogBwdArgs& p, int batch, int
     }
   }
 
-  float* gradb = p.grad + (long)batch * R * Cc;
+  elem_t* gradb = p.grad + (long)batch * R * Cc;
 #pragma unroll
   for (int i = 0; i < C::TR; ++i) {
     const int r = r0 + ty * C::TR + i;
@@ -172,14 +172,13 @@ __device__ __forceinline__ void log_bwd_tile(const LogBwdArgs& p, int batch, int
 #pragma unroll
     for (int q4 = 0; q4 < C::TC / 4; ++q4) {
       const int c = c0 + col_of(4 * q4);
-      float* dst = gradb + (long)r * Cc + c;
+      elem_t* dst = gradb + (long)r * Cc + c;
       if (vec_x && c + 3 < Cc) {
-        *reinterpret_cast<float4*>(dst) =
-            make_float4(acc[i][4 * q4], acc[i][4 * q4 + 1], acc[i][4 * q4 + 2], acc[i][4 * q4 + 3]);
+        st4a(dst, make_float4(acc[i][4 * q4], acc[i][4 * q4 + 1], acc[i][4 * q4 + 2], acc[i][4 * q4 + 3]));
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          if (c + e < Cc) dst[e] = acc[i][4 * q4 + e];
+          if (c + e < Cc) dst[e] = to_elem<elem_t>(acc[i][4 * q4 + e]);
       }
     }
   }
@@ -190,4 +189,4 @@ using BCfgWide = BCfg<64, 128, 4, 8, 16>;
 using BCfgMid = BCfg<64, 64, 4, 4, 16>;
 using BCfgSmall = BCfg<32, 32, 4, 4, 32>;
 
-}  // namespace genbmm
+}  // namespace GENBMM_NS

@@ -38,7 +38,7 @@
 #include "logbmm_self.h"
 #include "logbmm_ws.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 namespace {
 
 constexpr float kLog2eLo = 1.92596299e-8f;  // log2(e) - (float)log2(e)
@@ -65,8 +65,8 @@ __device__ __forceinline__ float exp_comp(float d) {
 // groups down, reduced through LDS).
 constexpr int kStatRows = 16, kStatCols = 32;
 
-__global__ __launch_bounds__(256) void k_log_stats(const float* __restrict__ a,
-                                                   const float* __restrict__ b,
+__global__ __launch_bounds__(256) void k_log_stats(const elem_t* __restrict__ a,
+                                                   const elem_t* __restrict__ b,
                                                    float* __restrict__ stats, int* __restrict__ hdr,
                                                    int M, int K, int N, int row_wgs, int col_wgs,
                                                    int vec_a, int vec_b) {
@@ -79,13 +79,13 @@ __global__ __launch_bounds__(256) void k_log_stats(const float* __restrict__ a,
   float* st = stats + (long)batch * (M + N);
   if (wg < row_wgs) {
     const int lane = tid & 63, m0 = wg * kStatRows + (tid >> 6) * 4;
-    const float* base = a + ((long)batch * M + m0) * K;
+    const elem_t* base = a + ((long)batch * M + m0) * K;
     float v[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
     if (vec_a && m0 + 3 < M) {
       for (int k = lane * 4; k < K; k += 256) {
         float4 x[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) x[r] = *reinterpret_cast<const float4*>(base + (long)r * K + k);
+        for (int r = 0; r < 4; ++r) x[r] = ld4a(base + (long)r * K + k);
 #pragma unroll
         for (int r = 0; r < 4; ++r) v[r] = fmaxf(v[r], fmaxf(fmaxf(x[r].x, x[r].y), fmaxf(x[r].z, x[r].w)));
       }
@@ -104,7 +104,7 @@ __global__ __launch_bounds__(256) void k_log_stats(const float* __restrict__ a,
   } else {
     const int c4 = tid & 7, rg = tid >> 3;
     const int n = (wg - row_wgs) * kStatCols + c4 * 4;
-    const float* col = b + (long)batch * K * N + n;
+    const elem_t* col = b + (long)batch * K * N + n;
     float4 v = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
     if (n < N) {
       if (vec_b) {
@@ -112,7 +112,7 @@ __global__ __launch_bounds__(256) void k_log_stats(const float* __restrict__ a,
         for (; k + 96 < K; k += 128) {  // four rows in flight
           float4 x[4];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) x[r] = *reinterpret_cast<const float4*>(col + (long)(k + 32 * r) * N);
+          for (int r = 0; r < 4; ++r) x[r] = ld4a(col + (long)(k + 32 * r) * N);
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             v.x = fmaxf(v.x, x[r].x); v.y = fmaxf(v.y, x[r].y);
@@ -120,12 +120,12 @@ __global__ __launch_bounds__(256) void k_log_stats(const float* __restrict__ a,
           }
         }
         for (; k < K; k += 32) {
-          const float4 x = *reinterpret_cast<const float4*>(col + (long)k * N);
+          const float4 x = ld4a(col + (long)k * N);
           v.x = fmaxf(v.x, x.x); v.y = fmaxf(v.y, x.y); v.z = fmaxf(v.z, x.z); v.w = fmaxf(v.w, x.w);
         }
       } else {
         for (int k = rg; k < K; k += 32) {
-          const float* p = col + (long)k * N;
+          const elem_t* p = col + (long)k * N;
           v.x = fmaxf(v.x, p[0]);
           if (n + 1 < N) v.y = fmaxf(v.y, p[1]);
           if (n + 2 < N) v.z = fmaxf(v.z, p[2]);
@@ -186,8 +186,8 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_fwd_fast(const DenseArgs p,
     hdr[2] = C::BN;
     hdr[0] = kWsFast;
   }
-  const float* ab = p.a + (long)batch * M * K;
-  const float* bb = p.b + (long)batch * K * N;
+  const elem_t* ab = p.a + (long)batch * M * K;
+  const elem_t* bb = p.b + (long)batch * K * N;
   const float* st = stats + (long)batch * (M + N);
   for (int t = tid; t < C::BM; t += C::NT) al[t] = (m0 + t < M) ? st[m0 + t] : 0.f;
   for (int t = tid; t < C::BN; t += C::NT) be[t] = (n0 + t < N) ? st[M + n0 + t] : 0.f;
@@ -408,12 +408,12 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_bwd_fast(const LogBwdArgs p,
                        N, tid, C::NT))
     return;
 
-  const float* ab = p.a + (long)batch * M * K;
-  const float* bb = p.b + (long)batch * K * N;
-  const float* ob = p.out + (long)batch * M * N;
-  const float* gb = p.g + (long)batch * M * N;
-  const float* xb = GRAD_A ? ab : bb;
-  const float* yb = GRAD_A ? bb : ab;
+  const elem_t* ab = p.a + (long)batch * M * K;
+  const elem_t* bb = p.b + (long)batch * K * N;
+  const elem_t* ob = p.out + (long)batch * M * N;
+  const elem_t* gb = p.g + (long)batch * M * N;
+  const elem_t* xb = GRAD_A ? ab : bb;
+  const elem_t* yb = GRAD_A ? bb : ab;
   const float* al = stats + (long)batch * (M + N);  // alpha[m]
   const float* be = al + M;                         // beta[n]
   const long ldy = GRAD_A ? N : K;
@@ -526,7 +526,7 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_bwd_fast(const LogBwdArgs p,
   }
 
   // epilogue: grad = exp(x - shift) * acc, x re-read from global memory
-  float* gradb = p.grad + (long)batch * R * Cc;
+  elem_t* gradb = p.grad + (long)batch * R * Cc;
   const float* xshift = GRAD_A ? al : be;  // alpha by row (m) / beta by column (n)
 #pragma unroll
   for (int i = 0; i < C::TR; ++i) {
@@ -537,12 +537,12 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_bwd_fast(const LogBwdArgs p,
     for (int q4 = 0; q4 < C::TC / 4; ++q4) {
       const int c = c0 + col_of(4 * q4);
       if (c >= Cc) continue;
-      const float* src = xb + (long)r * Cc + c;
-      float* dst = gradb + (long)r * Cc + c;
+      const elem_t* src = xb + (long)r * Cc + c;
+      elem_t* dst = gradb + (long)r * Cc + c;
       float xv[4], sv[4];
       const bool full = vec_x && c + 3 < Cc;
       if (full) {
-        const float4 v = *reinterpret_cast<const float4*>(src);
+        const float4 v = ld4a(src);
         xv[0] = v.x; xv[1] = v.y; xv[2] = v.z; xv[3] = v.w;
       } else {
 #pragma unroll
@@ -554,11 +554,11 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_bwd_fast(const LogBwdArgs p,
         xv[e] = exp_comp(xv[e] - sv[e]) * acc[i][4 * q4 + e];
       }
       if (full) {
-        *reinterpret_cast<float4*>(dst) = make_float4(xv[0], xv[1], xv[2], xv[3]);
+        st4a(dst, make_float4(xv[0], xv[1], xv[2], xv[3]));
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          if (c + e < Cc) dst[e] = xv[e];
+          if (c + e < Cc) dst[e] = to_elem<elem_t>(xv[e]);
       }
     }
   }
@@ -704,7 +704,7 @@ int launch_sample_sweep_mfma(DenseArgs p, const float* stats, int* flags, int B,
   return launch_status();
 }
 
-int launch_stats(const float* a, const float* b, float* stats, int B, int M, int K, int N,
+int launch_stats(const elem_t* a, const elem_t* b, float* stats, int B, int M, int K, int N,
                  hipStream_t s) {
   const int row_wgs = ceil_div(M, kStatRows), col_wgs = ceil_div(N, kStatCols);
   const int64_t total = (int64_t)B * (row_wgs + col_wgs);
@@ -835,7 +835,7 @@ int run_bwd(const LogBwdArgs& p, const float* stats, int path, int B, hipStream_
 }
 
 template <int G, int TB, bool FULL>
-void launch_item_fwd(const float* a, const float* b, float* out, float* stats, int* hdr, int B, int M,
+void launch_item_fwd(const elem_t* a, const elem_t* b, elem_t* out, float* stats, int* hdr, int B, int M,
                      int K, int N, hipStream_t s) {
   hipLaunchKernelGGL((k_log_item_fwd<G, TB, FULL>), dim3(B), dim3(G * G), 0, s, a, b, out, stats, hdr, M, K, N);
 }
@@ -855,7 +855,7 @@ int launch_self_fwd(DenseArgs p, float* stats, int B, int M, int K, int N, hipSt
 
 // factors: the caller wants EA, EB and 1/S in the workspace wherever a forward can leave
 // them (the sampling sweep), so the kernels that keep no by-products are not used.
-int run_fwd(const float* a, const float* b, float* out, float* stats, int B, int M, int K, int N,
+int run_fwd(const elem_t* a, const elem_t* b, elem_t* out, float* stats, int B, int M, int K, int N,
             int path, bool keep, hipStream_t s, bool factors = false) {
   if (int e = check_dense_dims(B, M, K, N)) return e;
   if (!valid_path(path)) return GENBMM_E_MODE;
@@ -897,8 +897,8 @@ int run_fwd(const float* a, const float* b, float* out, float* stats, int B, int
   }
 }
 
-int run_bwd_both(const float* a, const float* b, const float* out, const float* g,
-                 const float* stats, float* grad_a, float* grad_b, int B, int M, int K, int N,
+int run_bwd_both(const elem_t* a, const elem_t* b, const elem_t* out, const elem_t* g,
+                 const float* stats, elem_t* grad_a, elem_t* grad_b, int B, int M, int K, int N,
                  int path, hipStream_t s) {
   if (int e = check_dense_dims(B, M, K, N)) return e;
   if (!valid_path(path)) return GENBMM_E_MODE;
@@ -956,6 +956,7 @@ int run_bwd_both(const float* a, const float* b, const float* out, const float* 
   return GENBMM_OK;
 }
 
+#if GENBMM_ELEM == 0
 // ------------------------------------------------ forward on a workspace of the library's own
 // For callers that cannot allocate (code under HIP graph capture, serving loops,
 // harnesses that forbid it): the forward's workspace - maxima, per-tile flags, header;
@@ -984,6 +985,7 @@ int static_workspace(float** ws) {
   *ws = scratch_ptr[dev];
   return GENBMM_OK;
 }
+#endif
 
 }  // namespace
 
@@ -1002,14 +1004,14 @@ bool log_fwd_writes_factors(const float* stats, int B, int M, int K, int N, LogF
   return true;
 }
 
-int log_fwd_with_factors(const float* a, const float* b, float* out, float* stats, int B, int M, int K,
+int log_fwd_with_factors(const elem_t* a, const elem_t* b, elem_t* out, float* stats, int B, int M, int K,
                          int N, hipStream_t s) {
   return run_fwd(a, b, out, stats, B, M, K, N, GENBMM_PATH_AUTO, true, s, true);
 }
 
 bool log_sample_mfma_ok(int K) { return ceil_div(K, kMS) <= kSampleSlabs; }
 
-int log_sample_sweep_mfma(const float* a, const float* b, float* out, int32_t* idx,
+int log_sample_sweep_mfma(const elem_t* a, const elem_t* b, elem_t* out, int32_t* idx,
                           const float* stats, uint64_t seed, uint64_t offset, int B, int M, int K,
                           int N, hipStream_t s) {
   DenseArgs p{};
@@ -1024,12 +1026,13 @@ int log_sample_sweep_mfma(const float* a, const float* b, float* out, int32_t* i
   }
 }
 
-}  // namespace genbmm
+}  // namespace GENBMM_NS
 
 extern "C" {
 
+#if GENBMM_ELEM == 0
 size_t genbmm_logbmm_stats_size(int B, int M, int K, int N) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   if (check_dense_dims(B, M, K, N)) return 0;
   int64_t n = header_offset(B, M, N) + 4;
   // the one-tile kernels keep the maxima only
@@ -1039,47 +1042,57 @@ size_t genbmm_logbmm_stats_size(int B, int M, int K, int N) {
 }
 
 size_t genbmm_samplebmm_stats_size(int B, int M, int K, int N) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   if (check_dense_dims(B, M, K, N)) return 0;
   int64_t n = header_offset(B, M, N) + 4;
   if (fwd_mfma_shape(B, M, K, N)) n += (int64_t)B * ((int64_t)M * K + (int64_t)K * N + (int64_t)M * N);
   return (size_t)n;
 }
 
-int genbmm_logbmm_fwd(const float* a, const float* b, float* out, float* stats, int B, int M,
-                      int K, int N, void* stream) {
-  return genbmm::run_fwd(a, b, out, stats, B, M, K, N, GENBMM_PATH_AUTO, true, (hipStream_t)stream);
-}
-
-int genbmm_logbmm_fwd_path(const float* a, const float* b, float* out, float* stats, int B, int M,
-                           int K, int N, int path, void* stream) {
-  return genbmm::run_fwd(a, b, out, stats, B, M, K, N, path, true, (hipStream_t)stream);
-}
-
-size_t genbmm_logbmm_static_limit(void) { return genbmm::kStaticFloats; }
+size_t genbmm_logbmm_static_limit(void) { return GENBMM_NS::kStaticFloats; }
 
 int genbmm_logbmm_fwd_static(const float* a, const float* b, float* out, int B, int M, int K, int N,
                              void* stream) {
-  using namespace genbmm;
+  using namespace GENBMM_NS;
   if (int e = check_dense_dims(B, M, K, N)) return e;
   if ((uint64_t)header_offset(B, M, N) + 4 > kStaticFloats) return GENBMM_E_TOOBIG;
   float* ws = nullptr;
   if (int e = static_workspace(&ws)) return e;
   return run_fwd(a, b, out, ws, B, M, K, N, GENBMM_PATH_AUTO, false, (hipStream_t)stream);
 }
+#endif
 
-int genbmm_logbmm_bwd(const float* a, const float* b, const float* out, const float* g,
-                      const float* stats, float* grad_a, float* grad_b, int B, int M, int K,
-                      int N, void* stream) {
-  return genbmm::run_bwd_both(a, b, out, g, stats, grad_a, grad_b, B, M, K, N, GENBMM_PATH_AUTO,
-                              (hipStream_t)stream);
+// The four entry points below exist once per element type: genbmm_logbmm_fwd,
+// genbmm_logbmm_fwd_f16, genbmm_logbmm_fwd_bf16, ...
+int GENBMM_API(logbmm_fwd)(const GENBMM_NS::abi_t* a, const GENBMM_NS::abi_t* b, GENBMM_NS::abi_t* out,
+                           float* stats, int B, int M, int K, int N, void* stream) {
+  using namespace GENBMM_NS;
+  return run_fwd(el(a), el(b), el(out), stats, B, M, K, N, GENBMM_PATH_AUTO, true, (hipStream_t)stream);
 }
 
-int genbmm_logbmm_bwd_path(const float* a, const float* b, const float* out, const float* g,
-                           const float* stats, float* grad_a, float* grad_b, int B, int M, int K,
-                           int N, int path, void* stream) {
-  return genbmm::run_bwd_both(a, b, out, g, stats, grad_a, grad_b, B, M, K, N, path,
-                              (hipStream_t)stream);
+int GENBMM_API(logbmm_fwd_path)(const GENBMM_NS::abi_t* a, const GENBMM_NS::abi_t* b,
+                                GENBMM_NS::abi_t* out, float* stats, int B, int M, int K, int N,
+                                int path, void* stream) {
+  using namespace GENBMM_NS;
+  return run_fwd(el(a), el(b), el(out), stats, B, M, K, N, path, true, (hipStream_t)stream);
+}
+
+int GENBMM_API(logbmm_bwd)(const GENBMM_NS::abi_t* a, const GENBMM_NS::abi_t* b,
+                           const GENBMM_NS::abi_t* out, const GENBMM_NS::abi_t* g, const float* stats,
+                           GENBMM_NS::abi_t* grad_a, GENBMM_NS::abi_t* grad_b, int B, int M, int K,
+                           int N, void* stream) {
+  using namespace GENBMM_NS;
+  return run_bwd_both(el(a), el(b), el(out), el(g), stats, el(grad_a), el(grad_b), B, M, K, N,
+                      GENBMM_PATH_AUTO, (hipStream_t)stream);
+}
+
+int GENBMM_API(logbmm_bwd_path)(const GENBMM_NS::abi_t* a, const GENBMM_NS::abi_t* b,
+                                const GENBMM_NS::abi_t* out, const GENBMM_NS::abi_t* g,
+                                const float* stats, GENBMM_NS::abi_t* grad_a, GENBMM_NS::abi_t* grad_b,
+                                int B, int M, int K, int N, int path, void* stream) {
+  using namespace GENBMM_NS;
+  return run_bwd_both(el(a), el(b), el(out), el(g), stats, el(grad_a), el(grad_b), B, M, K, N, path,
+                      (hipStream_t)stream);
 }
 
 }  // extern "C"

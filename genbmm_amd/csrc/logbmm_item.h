@@ -16,19 +16,20 @@
 #include "common.h"
 #include "logbmm_ws.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 
 constexpr float kItemGuardBits = 40.f;
 
 // log-sum-exp of a[m,:] + b[:,n] the way the reference's kernel does it
 // (matmul_cuda_kernel.cu:27-41): running maximum from -1e9, then the sum.
-__device__ __forceinline__ float item_exact_out(const float* __restrict__ arow,
-                                                const float* __restrict__ bcol, int K, int N) {
+__device__ __forceinline__ float item_exact_out(const elem_t* __restrict__ arow,
+                                                const elem_t* __restrict__ bcol, int K, int N) {
   float mx = kFloor;
-  for (int k = 0; k < K; ++k) mx = fmaxf(mx, arow[k] + bcol[(long)k * N]);
+  for (int k = 0; k < K; ++k) mx = fmaxf(mx, (float)arow[k] + (float)bcol[(long)k * N]);
   const float nm = -mx * kLog2e;
   float s = 0.f;
-  for (int k = 0; k < K; ++k) s += fast_exp2(__builtin_fmaf(arow[k] + bcol[(long)k * N], kLog2e, nm));
+  for (int k = 0; k < K; ++k)
+    s += fast_exp2(__builtin_fmaf((float)arow[k] + (float)bcol[(long)k * N], kLog2e, nm));
   return logf(s) + mx;
 }
 
@@ -64,9 +65,9 @@ __device__ __forceinline__ float item_exp(float x, float shift) {
 // FULL: M = K = N = G * TB, known to the compiler - the index arithmetic that is most of
 // the general kernel's instructions (it is issue-bound, not memory-bound) folds away.
 template <int G, int TB, bool FULL = false>
-__global__ __launch_bounds__(G * G, TB == 2 ? 8 : 1) void k_log_item_fwd(const float* __restrict__ a,
-                                                      const float* __restrict__ b,
-                                                      float* __restrict__ out,
+__global__ __launch_bounds__(G * G, TB == 2 ? 8 : 1) void k_log_item_fwd(const elem_t* __restrict__ a,
+                                                      const elem_t* __restrict__ b,
+                                                      elem_t* __restrict__ out,
                                                       float* __restrict__ stats,
                                                       int* __restrict__ hdr, int M_, int K_,
                                                       int N_) {
@@ -78,8 +79,8 @@ __global__ __launch_bounds__(G * G, TB == 2 ? 8 : 1) void k_log_item_fwd(const f
   __shared__ float Bs[S * LD];  // [k][n]: b, then EB
   __shared__ float al[S], be[S];
   const int tid = threadIdx.x, batch = blockIdx.x;
-  const float* ab = a + (long)batch * M * K;
-  const float* bb = b + (long)batch * K * N;
+  const elem_t* ab = a + (long)batch * M * K;
+  const elem_t* bb = b + (long)batch * K * N;
   // All reads of the item are issued before the first one is waited for (a thread owns
   // elements tid, tid + NT, ... of each operand): one trip to memory, not one per element.
   constexpr int PER = TB * TB;  // S * S / NT
@@ -167,20 +168,20 @@ __global__ __launch_bounds__(G * G, TB == 2 ? 8 : 1) void k_log_item_fwd(const f
       }
     }
   __syncthreads();
-  float* ob = out + (long)batch * M * N;
+  elem_t* ob = out + (long)batch * M * N;
   for (RowMajorWalk w(tid, NT, N); w.r < M; w.next()) {
     const int m = w.r, n = w.c, e = w.r * N + w.c;
-    ob[e] = At[m * LD + n];
+    ob[e] = to_elem<elem_t>(At[m * LD + n]);
   }
 }
 
 template <int G, int TB, bool FULL = false>
-__global__ __launch_bounds__(G * G, TB == 2 ? 6 : 1) void k_log_item_bwd(const float* __restrict__ a,
-                                                      const float* __restrict__ b,
-                                                      const float* __restrict__ outp,
-                                                      const float* __restrict__ g,
-                                                      float* __restrict__ grad_a,
-                                                      float* __restrict__ grad_b, int M_, int K_,
+__global__ __launch_bounds__(G * G, TB == 2 ? 6 : 1) void k_log_item_bwd(const elem_t* __restrict__ a,
+                                                      const elem_t* __restrict__ b,
+                                                      const elem_t* __restrict__ outp,
+                                                      const elem_t* __restrict__ g,
+                                                      elem_t* __restrict__ grad_a,
+                                                      elem_t* __restrict__ grad_b, int M_, int K_,
                                                       int N_) {
   constexpr int NT = G * G, S = G * TB, LD = S + 1;
   const int M = FULL ? S : M_, K = FULL ? S : K_, N = FULL ? S : N_;
@@ -190,12 +191,12 @@ __global__ __launch_bounds__(G * G, TB == 2 ? 6 : 1) void k_log_item_bwd(const f
   __shared__ float Hs[S * LD];  // [m][n]: H
   __shared__ float al[S], be[S];
   const int tid = threadIdx.x, batch = blockIdx.x;
-  const float* ab = a + (long)batch * M * K;
-  const float* bb = b + (long)batch * K * N;
-  const float* ob = outp + (long)batch * M * N;
-  const float* gb = g + (long)batch * M * N;
-  float* gab = grad_a ? grad_a + (long)batch * M * K : nullptr;
-  float* gbb = grad_b ? grad_b + (long)batch * K * N : nullptr;
+  const elem_t* ab = a + (long)batch * M * K;
+  const elem_t* bb = b + (long)batch * K * N;
+  const elem_t* ob = outp + (long)batch * M * N;
+  const elem_t* gb = g + (long)batch * M * N;
+  elem_t* gab = grad_a ? grad_a + (long)batch * M * K : nullptr;
+  elem_t* gbb = grad_b ? grad_b + (long)batch * K * N : nullptr;
   // all reads of the item in flight together (see the forward)
   constexpr int PER = TB * TB;
   float ra[PER], rb[PER], ro[PER], rg[PER];
@@ -267,8 +268,8 @@ __global__ __launch_bounds__(G * G, TB == 2 ? 6 : 1) void k_log_item_bwd(const f
         const float av = ab[e];
         float s = 0.f;
         for (int n = 0; n < N; ++n)
-          s = __builtin_fmaf(fast_exp(av + bb[(long)k * N + n] - ob[(long)m * N + n]), gb[(long)m * N + n], s);
-        gab[e] = s;
+          s = __builtin_fmaf(fast_exp(av + (float)bb[(long)k * N + n] - (float)ob[(long)m * N + n]), (float)gb[(long)m * N + n], s);
+        gab[e] = to_elem<elem_t>(s);
       }
     if (gbb)
       for (int e = tid; e < K * N; e += NT) {
@@ -276,8 +277,8 @@ __global__ __launch_bounds__(G * G, TB == 2 ? 6 : 1) void k_log_item_bwd(const f
         const float bv = bb[e];
         float s = 0.f;
         for (int m = 0; m < M; ++m)
-          s = __builtin_fmaf(fast_exp(ab[(long)m * K + k] + bv - ob[(long)m * N + n]), gb[(long)m * N + n], s);
-        gbb[e] = s;
+          s = __builtin_fmaf(fast_exp((float)ab[(long)m * K + k] + bv - (float)ob[(long)m * N + n]), (float)gb[(long)m * N + n], s);
+        gbb[e] = to_elem<elem_t>(s);
       }
     return;
   }
@@ -327,9 +328,9 @@ __global__ __launch_bounds__(G * G, TB == 2 ? 6 : 1) void k_log_item_bwd(const f
     }
   __syncthreads();
   if (gab)
-    for (RowMajorWalk w(tid, NT, K); w.r < M; w.next()) gab[w.r * K + w.c] = Ea[w.r * LD + w.c];
+    for (RowMajorWalk w(tid, NT, K); w.r < M; w.next()) gab[w.r * K + w.c] = to_elem<elem_t>(Ea[w.r * LD + w.c]);
   if (gbb)
-    for (RowMajorWalk w(tid, NT, N); w.r < K; w.next()) gbb[w.r * N + w.c] = Eb[w.r * LD + w.c];
+    for (RowMajorWalk w(tid, NT, N); w.r < K; w.next()) gbb[w.r * N + w.c] = to_elem<elem_t>(Eb[w.r * LD + w.c]);
 }
 
-}  // namespace genbmm
+}  // namespace GENBMM_NS

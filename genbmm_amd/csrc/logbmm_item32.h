@@ -31,7 +31,7 @@
 #include "logbmm_item.h"
 #include "logbmm_mfma.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 
 constexpr int kI32 = 32;  // M = K = N
 
@@ -40,7 +40,7 @@ struct Item32Lane {
 };
 
 // 16 values x[row][16 h + s] of a row-major 32 x 32 item
-__device__ __forceinline__ void item32_rows(const float* __restrict__ x, int row, int h, float (&v)[16]) {
+__device__ __forceinline__ void item32_rows(const elem_t* __restrict__ x, int row, int h, float (&v)[16]) {
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     const float4 t = ld4(x + row * kI32 + 16 * h + 4 * q);
@@ -48,12 +48,12 @@ __device__ __forceinline__ void item32_rows(const float* __restrict__ x, int row
   }
 }
 // 16 values x[k][c] for k = 16 h + s
-__device__ __forceinline__ void item32_cols_k(const float* __restrict__ x, int c, int h, float (&v)[16]) {
+__device__ __forceinline__ void item32_cols_k(const elem_t* __restrict__ x, int c, int h, float (&v)[16]) {
 #pragma unroll
   for (int s = 0; s < 16; ++s) v[s] = x[(16 * h + s) * kI32 + c];
 }
 // 16 values x[rho(r, h)][c]
-__device__ __forceinline__ void item32_cols(const float* __restrict__ x, int c, int h, float (&v)[16]) {
+__device__ __forceinline__ void item32_cols(const elem_t* __restrict__ x, int c, int h, float (&v)[16]) {
 #pragma unroll
   for (int r = 0; r < 16; ++r) v[r] = x[(mfma_row_u(r) + 4 * h) * kI32 + c];
 }
@@ -65,8 +65,8 @@ __device__ __forceinline__ float max16(const float (&v)[16]) {
 }
 
 // One wave per item, four items per workgroup.
-__global__ __launch_bounds__(256) void k_log_item32_fwd(const float* __restrict__ a, const float* __restrict__ b,
-                                                       float* __restrict__ out, float* __restrict__ stats,
+__global__ __launch_bounds__(256) void k_log_item32_fwd(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
+                                                       elem_t* __restrict__ out, float* __restrict__ stats,
                                                        int* __restrict__ hdr, int B) {
   __shared__ float sh[4][64];
   if (hdr && blockIdx.x == 0 && threadIdx.x == 0) hdr[0] = kWsNone;  // no per-tile flags in this workspace
@@ -74,8 +74,8 @@ __global__ __launch_bounds__(256) void k_log_item32_fwd(const float* __restrict_
   const int item = blockIdx.x * 4 + wave;
   if (item >= B) return;
   const int c = lane & 31, h = lane >> 5;
-  const float* ab = a + (long)item * kI32 * kI32;
-  const float* bb = b + (long)item * kI32 * kI32;
+  const elem_t* ab = a + (long)item * kI32 * kI32;
+  const elem_t* bb = b + (long)item * kI32 * kI32;
   float av[16], bv[16];
   item32_rows(ab, c, h, av);      // a[i = c][16 h + s]
   item32_cols_k(bb, c, h, bv);    // b[16 h + s][j = c]
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void k_log_item32_fwd(const float* __restrict_
     st[lane] = h == 0 ? al : be;  // alpha[0..32), beta[0..32)
   }
   const float thr = fast_exp2(-kItemGuardBits);
-  float* ob = out + (long)item * kI32 * kI32;
+  elem_t* ob = out + (long)item * kI32 * kI32;
   unsigned redo = 0;  // bit r: the cell is recomputed by the reference's form (rare)
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
@@ -108,19 +108,19 @@ __global__ __launch_bounds__(256) void k_log_item32_fwd(const float* __restrict_
     const float shift = ar[r] + be, s = acc[r];
     const bool ok = (s >= thr) && (s < INFINITY) && (shift > 0.9f * kFloor) && (shift < INFINITY);
     if (!ok) redo |= 1u << r;
-    ob[i * kI32 + c] = __builtin_fmaf(fast_log2(s), kLn2, shift);
+    ob[i * kI32 + c] = to_elem<elem_t>(__builtin_fmaf(fast_log2(s), kLn2, shift));
   }
   while (redo) {  // same lane, same address as the store above: they stay in order
     const int r = __builtin_ctz(redo);
     redo &= redo - 1;
     const int i = 8 * (r >> 2) + (r & 3) + 4 * h;
-    ob[i * kI32 + c] = item_exact_out(ab + i * kI32, bb + c, kI32, kI32);
+    ob[i * kI32 + c] = to_elem<elem_t>(item_exact_out(ab + i * kI32, bb + c, kI32, kI32));
   }
 }
 
-__global__ __launch_bounds__(256, 3) void k_log_item32_bwd(const float* __restrict__ a, const float* __restrict__ b,
-                                                       const float* __restrict__ outp, const float* __restrict__ g,
-                                                       float* __restrict__ grad_a, float* __restrict__ grad_b,
+__global__ __launch_bounds__(256, 3) void k_log_item32_bwd(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
+                                                       const elem_t* __restrict__ outp, const elem_t* __restrict__ g,
+                                                       elem_t* __restrict__ grad_a, elem_t* __restrict__ grad_b,
                                                        int B) {
   __shared__ float sh[4][64];
   __shared__ float tr[4][kI32 * 33];  // a wave's 32 x 32 values on their way from columns to rows
@@ -139,12 +139,12 @@ __global__ __launch_bounds__(256, 3) void k_log_item32_bwd(const float* __restri
     for (int s2 = 0; s2 < 16; ++s2) row[s2] = tw[c * 33 + 16 * h + s2];
     wave_lds_sync();
   };
-  const float* ab = a + (long)item * E;
-  const float* bb = b + (long)item * E;
-  const float* ob = outp + (long)item * E;
-  const float* gb = g + (long)item * E;
-  float* gab = grad_a ? grad_a + (long)item * E : nullptr;
-  float* gbb = grad_b ? grad_b + (long)item * E : nullptr;
+  const elem_t* ab = a + (long)item * E;
+  const elem_t* bb = b + (long)item * E;
+  const elem_t* ob = outp + (long)item * E;
+  const elem_t* gb = g + (long)item * E;
+  elem_t* gab = grad_a ? grad_a + (long)item * E : nullptr;
+  elem_t* gbb = grad_b ? grad_b + (long)item * E : nullptr;
 
   // ---- maxima: alpha from a in rows, beta from b in columns; both to LDS
   float a_col[16], b_col[16], al, be;
@@ -189,8 +189,8 @@ __global__ __launch_bounds__(256, 3) void k_log_item32_bwd(const float* __restri
         const float av = ab[e];
         float s = 0.f;
         for (int n = 0; n < kI32; ++n)
-          s = __builtin_fmaf(fast_exp(av + bb[k * kI32 + n] - ob[m * kI32 + n]), gb[m * kI32 + n], s);
-        gab[e] = s;
+          s = __builtin_fmaf(fast_exp(av + (float)bb[k * kI32 + n] - (float)ob[m * kI32 + n]), (float)gb[m * kI32 + n], s);
+        gab[e] = to_elem<elem_t>(s);
       }
     if (gbb)
       for (int e = lane; e < E; e += 64) {
@@ -198,8 +198,8 @@ __global__ __launch_bounds__(256, 3) void k_log_item32_bwd(const float* __restri
         const float bv = bb[e];
         float s = 0.f;
         for (int m = 0; m < kI32; ++m)
-          s = __builtin_fmaf(fast_exp(ab[m * kI32 + k] + bv - ob[m * kI32 + n]), gb[m * kI32 + n], s);
-        gbb[e] = s;
+          s = __builtin_fmaf(fast_exp((float)ab[m * kI32 + k] + bv - (float)ob[m * kI32 + n]), (float)gb[m * kI32 + n], s);
+        gbb[e] = to_elem<elem_t>(s);
       }
     return;
   }
@@ -219,7 +219,7 @@ __global__ __launch_bounds__(256, 3) void k_log_item32_bwd(const float* __restri
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc = mfma_32x32x2(a_col[r], h_col[r], acc);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) gbb[(mfma_row_u(r) + 4 * h) * kI32 + c] = b_col[r] * acc[r];
+    for (int r = 0; r < 16; ++r) gbb[(mfma_row_u(r) + 4 * h) * kI32 + c] = to_elem<elem_t>((b_col[r] * acc[r]));
   }
   if (gab) {  // T[i][k] = sum_j H[i][j] EB[k][j], j = 16 h + s: both operands in rows
     float h_row[16], eb_row[16];
@@ -231,8 +231,8 @@ __global__ __launch_bounds__(256, 3) void k_log_item32_bwd(const float* __restri
 #pragma unroll
     for (int s2 = 0; s2 < 16; ++s2) acc = mfma_32x32x2(h_row[s2], eb_row[s2], acc);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) gab[(mfma_row_u(r) + 4 * h) * kI32 + c] = a_col[r] * acc[r];
+    for (int r = 0; r < 16; ++r) gab[(mfma_row_u(r) + 4 * h) * kI32 + c] = to_elem<elem_t>((a_col[r] * acc[r]));
   }
 }
 
-}  // namespace genbmm
+}  // namespace GENBMM_NS

@@ -14,7 +14,7 @@
 #include "common.h"
 #include "logbmm_ws.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
@@ -119,46 +119,28 @@ struct StageS {
   }
 };
 
-// Global memory is touched four floats at a time with only 4-byte alignment
-// assumed (the hardware takes misaligned dwordx4; rows of odd-sized matrices start
-// anywhere).  The masked forms touch the first cnt (<= 0: none, >= 4: all) elements.
-typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
-__device__ __forceinline__ float4 ld4(const float* p) {
-  const float4u v = *reinterpret_cast<const float4u*>(p);
-  return make_float4(v.x, v.y, v.z, v.w);
+// Two arrays of the same shape - one of the caller's elements, one of fp32 workspace -
+// are walked with one pointer: the element at the same index of the other array is
+// found by integer arithmetic on addresses (not pointer arithmetic across objects).
+// ws_twin: from an element pointer to the fp32 array; elem_twin: the other way round.
+// The distance may carry a fixed offset in bytes of the target array.
+template <class E>
+constexpr uintptr_t kWiden = 4 / sizeof(E);  // bytes of workspace per byte of element
+template <class E>
+__device__ __forceinline__ long ws_distance(const float* ws, const E* from) {
+  return (long)(reinterpret_cast<uintptr_t>(ws) - reinterpret_cast<uintptr_t>(from) * kWiden<E>);
 }
-__device__ __forceinline__ void st4(float* p, float4 v) {
-  float4u u;
-  u.x = v.x; u.y = v.y; u.z = v.z; u.w = v.w;
-  *reinterpret_cast<float4u*>(p) = u;
+template <class E>
+__device__ __forceinline__ float* ws_twin(const E* p, long d) {
+  return reinterpret_cast<float*>(reinterpret_cast<uintptr_t>(p) * kWiden<E> + (uintptr_t)d);
 }
-__device__ __forceinline__ float4 ld4m(const float* p, int cnt, float fill) {
-  if (cnt >= 4) return ld4(p);
-  float4 r = make_float4(fill, fill, fill, fill);
-  if (cnt > 0) r.x = p[0];
-  if (cnt > 1) r.y = p[1];
-  if (cnt > 2) r.z = p[2];
-  return r;
+template <class E>
+__device__ __forceinline__ long elem_distance(const E* to, const float* ws) {
+  return (long)(reinterpret_cast<uintptr_t>(to) - reinterpret_cast<uintptr_t>(ws) / kWiden<E>);
 }
-__device__ __forceinline__ void st4m(float* p, int cnt, float4 v) {
-  if (cnt >= 4) {
-    st4(p, v);
-    return;
-  }
-  if (cnt > 0) p[0] = v.x;
-  if (cnt > 1) p[1] = v.y;
-  if (cnt > 2) p[2] = v.z;
-}
-__device__ __forceinline__ int clamp4(int x) { return min(max(x, 0), 4); }
-
-// Two arrays of the same shape are walked with one pointer plus the byte distance
-// between them (integer arithmetic on addresses, not pointer arithmetic across
-// objects).
-__device__ __forceinline__ long byte_distance(const void* to, const void* from) {
-  return (long)(reinterpret_cast<uintptr_t>(to) - reinterpret_cast<uintptr_t>(from));
-}
-__device__ __forceinline__ float* shifted(const float* p, long bytes) {
-  return reinterpret_cast<float*>(reinterpret_cast<uintptr_t>(p) + (uintptr_t)bytes);
+template <class E>
+__device__ __forceinline__ const E* elem_twin(const float* p, long d) {
+  return reinterpret_cast<const E*>(reinterpret_cast<uintptr_t>(p) / kWiden<E> + (uintptr_t)d);
 }
 __device__ __forceinline__ float4 exp4(float4 x, float4 s) {
   return make_float4(exp_st(x.x - s.x), exp_st(x.y - s.y), exp_st(x.z - s.z), exp_st(x.w - s.w));
@@ -261,8 +243,8 @@ __device__ __forceinline__ void acc_rows(const floatx16 (&acc)[2][2], float* __r
 // for its own sake - the workspace then holds the maxima, flags and header only).
 template <class T, bool RAGGED, bool KEEP = true>
 __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WPE, T::WPE)))
-void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
-                    float* __restrict__ out, const float* __restrict__ stats,
+void k_log_fwd_mfma(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
+                    elem_t* __restrict__ out, const float* __restrict__ stats,
                     int* __restrict__ flags, float* __restrict__ ws_ea,
                     float* __restrict__ ws_eb, float* __restrict__ ws_r, int* __restrict__ ws_hdr,
                     int M, int K, int N, int tiles_m, int tiles_n) {
@@ -290,8 +272,8 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
   const int cb = RAGGED ? clamp4(N - bcol) : 4;  // columns of this lane's b pieces inside the matrix
   const bool vb = cb > 0;
   bool va[SA::PER];
-  const float* pa[SA::PER];
-  const float* pb[SB::PER];
+  const elem_t* pa[SA::PER];
+  const elem_t* pb[SB::PER];
   float al[SA::PER];
 #pragma unroll
   for (int l = 0; l < SA::PER; ++l) {
@@ -306,7 +288,7 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
   const float4 be = RAGGED ? ld4m(st + M + (vb ? bcol : 0), cb, INFINITY) : ld4(st + M + bcol);
   // by-products live at the same offsets in their own arrays
   // (the source pointers run one slab ahead of what is being staged)
-  const long da = byte_distance(ws_ea, a) - 4l * kMS, db = byte_distance(ws_eb, b) - 4l * kMS * N;
+  const long da = ws_distance(ws_ea, a) - 4l * kMS, db = ws_distance(ws_eb, b) - 4l * kMS * N;
   if (tile == 0 && tid == 0) {
     ws_hdr[1] = T::TR;
     ws_hdr[2] = T::TC;
@@ -354,8 +336,8 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
       const float4 e = exp4(ra[l], al[l]);
       SA::put(As[buf], tid, l, e);
       if (keep_a) {
-        if (!RAGGED) st4(shifted(pa[l], da), e);
-        else if (va[l]) st4m(shifted(pa[l], da), ca, e);
+        if (!RAGGED) st4(ws_twin(pa[l], da), e);
+        else if (va[l]) st4m(ws_twin(pa[l], da), ca, e);
       }
     }
 #pragma unroll
@@ -363,8 +345,8 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
       const float4 e = exp4(rb[l], be);
       SB::put(Bs[buf], tid, l, e);
       if (keep_b) {
-        if (!RAGGED) st4(shifted(pb[l], db), e);
-        else if (tb[l]) st4m(shifted(pb[l], db), cb, e);
+        if (!RAGGED) st4(ws_twin(pb[l], db), e);
+        else if (tb[l]) st4m(ws_twin(pb[l], db), cb, e);
       }
     }
   };
@@ -458,10 +440,10 @@ void k_log_fwd_mfma(const float* __restrict__ a, const float* __restrict__ b,
 // the loader of the last slab; the epilogue is masked.
 template <class T, bool GRAD_A, bool RAGGED>
 __device__ __forceinline__ void log_bwd_mfma_tile(
-    float* __restrict__ smem, int tile, const float* __restrict__ g,
+    float* __restrict__ smem, int tile, const elem_t* __restrict__ g,
     const float* __restrict__ ws_ea, const float* __restrict__ ws_eb,
     const float* __restrict__ ws_r, const int* __restrict__ ws_hdr,
-    const int* __restrict__ fwd_flags, float* __restrict__ grad, int M, int K, int N, int tiles_r,
+    const int* __restrict__ fwd_flags, elem_t* __restrict__ grad, int M, int K, int N, int tiles_r,
     int tiles_c) {
   constexpr int NT = T::NT, LDR = T::LDR, LDC = T::LDC;
   using SH = std::conditional_t<GRAD_A, StageT<T::TR, NT, LDR>, StageS<T::TC, NT, LDC>>;
@@ -487,7 +469,7 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
   float4 ry[SY::PER], rr[SH::PER], rg[SH::PER];
   const float* py[SY::PER];
   const float* pr[SH::PER];
-  long dg;  // g sits at the same offsets as R: byte distance between the arrays
+  long dg;  // g sits at the same element offsets as R
   // elements of this lane's pieces inside the matrix: grad_b pieces run along the
   // output axis (fixed per lane), grad_a pieces along the reduction (last slab only)
   int cy = 4, ch = 4;
@@ -513,7 +495,7 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
     for (int l = 0; l < SH::PER; ++l)
       pr[l] = ws_r + ((long)batch * M + SH::red(tid, l)) * N + (ch > 0 ? nc : 0);
   }
-  dg = byte_distance(g, ws_r);
+  dg = elem_distance(g, ws_r);
   const int qtail = RAGGED ? Q % kMS : 0;
   const int slabs = RAGGED ? (Q + kMS - 1) / kMS : Q / kMS;
   const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -524,7 +506,7 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
 #pragma unroll
       for (int l = 0; l < SH::PER; ++l) {
         rr[l] = ld4(pr[l]);
-        rg[l] = ld4(shifted(pr[l], dg));
+        rg[l] = ld4(elem_twin<elem_t>(pr[l], dg));
       }
     } else {
       // grad_a: a piece covers reduction steps redpos .. redpos+3; grad_b: one step
@@ -538,7 +520,7 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
         const int left = tail ? qtail - SH::redpos(tid, l) : 4;
         const int cnt = GRAD_A ? left : (left > 0 ? ch : 0);
         rr[l] = ld4m(pr[l], cnt, 0.f);
-        rg[l] = ld4m(shifted(pr[l], dg), cnt, 0.f);
+        rg[l] = ld4m(elem_twin<elem_t>(pr[l], dg), cnt, 0.f);
       }
     }
 #pragma unroll
@@ -580,7 +562,7 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
   const int voff = lr * Cc + lc;
   const long ubase = ((long)batch * R + r0 + wr0) * Cc + c0 + wc0;
   const float* xb = (GRAD_A ? ws_ea : ws_eb) + ubase + voff;
-  float* gp = grad + ubase + voff;
+  elem_t* gp = grad + ubase + voff;
   const int cc = RAGGED ? clamp4(Cc - (c0 + wc0 + lc)) : 4;  // columns of this lane's pieces that exist
   const bool cok = cc > 0;
   const int rows_left = R - (r0 + wr0) - lr;
@@ -606,10 +588,10 @@ __device__ __forceinline__ void log_bwd_mfma_tile(
 
 template <class T, bool GRAD_A, bool RAGGED>
 __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WPE, T::WPE)))
-void k_log_bwd_mfma(const float* __restrict__ g, const float* __restrict__ ws_ea,
+void k_log_bwd_mfma(const elem_t* __restrict__ g, const float* __restrict__ ws_ea,
                     const float* __restrict__ ws_eb, const float* __restrict__ ws_r,
                     const int* __restrict__ ws_hdr, const int* __restrict__ fwd_flags,
-                    float* __restrict__ grad, int M, int K, int N, int tiles_r, int tiles_c) {
+                    elem_t* __restrict__ grad, int M, int K, int N, int tiles_r, int tiles_c) {
   __shared__ __attribute__((aligned(16))) float smem[2 * kMS * (T::LDR + T::LDC)];
   log_bwd_mfma_tile<T, GRAD_A, RAGGED>(smem, xcd_tile_id(), g, ws_ea, ws_eb, ws_r, ws_hdr, fwd_flags,
                                        grad, M, K, N, tiles_r, tiles_c);
@@ -621,10 +603,10 @@ void k_log_bwd_mfma(const float* __restrict__ g, const float* __restrict__ ws_ea
 // still writing their results back.
 template <class TA, class TB, bool RAGGED>
 __global__ __launch_bounds__(TA::NT) __attribute__((amdgpu_waves_per_eu(TA::WPE, TA::WPE)))
-void k_log_bwd_mfma_both(const float* __restrict__ g, const float* __restrict__ ws_ea,
+void k_log_bwd_mfma_both(const elem_t* __restrict__ g, const float* __restrict__ ws_ea,
                          const float* __restrict__ ws_eb, const float* __restrict__ ws_r,
                          const int* __restrict__ ws_hdr, const int* __restrict__ fwd_flags,
-                         float* __restrict__ grad_a, float* __restrict__ grad_b, int M, int K, int N,
+                         elem_t* __restrict__ grad_a, elem_t* __restrict__ grad_b, int M, int K, int N,
                          int tiles_a, int ar, int ac, int br, int bc) {
   static_assert(TA::NT == TB::NT && TA::WPE == TB::WPE, "");
   constexpr int kA = 2 * kMS * (TA::LDR + TA::LDC), kB = 2 * kMS * (TB::LDR + TB::LDC);
@@ -672,7 +654,7 @@ constexpr float kSampleShrink = 1.f - 0x1p-22f;
 template <class T>
 __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void k_sample_sweep_mfma(const float* __restrict__ ws_ea, const float* __restrict__ ws_eb,
-                         const float* __restrict__ out, const float* __restrict__ stats,
+                         const elem_t* __restrict__ out, const float* __restrict__ stats,
                          int* __restrict__ flags, float* __restrict__ remw,
                          int32_t* __restrict__ idx, uint64_t seed, uint64_t offset, int M, int K,
                          int N, int tiles_m, int tiles_n, int ftr, int ftc, int ftiles_m,
@@ -835,4 +817,4 @@ void k_sample_sweep_mfma(const float* __restrict__ ws_ea, const float* __restric
     }
 }
 
-}  // namespace genbmm
+}  // namespace GENBMM_NS

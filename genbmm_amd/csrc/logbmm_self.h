@@ -25,7 +25,7 @@
 #include "logbmm_mfma.h"
 #include "logbmm_ws.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 
 constexpr int kSelfMax = 128;               // largest extent these kernels take
 constexpr int kSelfSlabs = kSelfMax / kMS;  // reduction slabs at that extent
@@ -78,8 +78,8 @@ void k_log_self_fwd(const DenseArgs p, float* __restrict__ stats, int* __restric
   const int wm0 = (wave >> 1) * 64, wn0 = (wave & 1) * 64;
   const int batch = blockIdx.x;
   const int M = p.M, K = p.K, N = p.N;
-  const float* ab = p.a + (long)batch * M * K;
-  const float* bb = p.b + (long)batch * K * N;
+  const elem_t* ab = p.a + (long)batch * M * K;
+  const elem_t* bb = p.b + (long)batch * K * N;
   float* st = stats + (long)batch * (M + N);
   const int slabs = RAGGED ? (K + kMS - 1) / kMS : kSelfSlabs;
   const float4 ninf = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
@@ -104,7 +104,7 @@ void k_log_self_fwd(const DenseArgs p, float* __restrict__ stats, int* __restric
 #pragma unroll
   for (int s = 0; s < kSelfSlabs; ++s)
     if (!RAGGED || s < slabs) {
-      const float* bs = bb + (size_t)(kMS * s) * N;  // uniform
+      const elem_t* bs = bb + (size_t)(kMS * s) * N;  // uniform
 #pragma unroll
       for (int l = 0; l < 2; ++l) {
         const int m = SA::line(tid, l), k = kMS * s + SB::red(tid, l);
@@ -216,7 +216,7 @@ void k_log_self_fwd(const DenseArgs p, float* __restrict__ stats, int* __restric
   const bool cok = cc > 0;
   const float4 be4 = *reinterpret_cast<const float4*>(&s_be[wn0 + lc]);
   const float* alw = s_al + wm0 + lr;
-  float* ob = p.out + ((long)batch * M + wm0 + lr) * N + wn0 + lc;
+  elem_t* ob = p.out + ((long)batch * M + wm0 + lr) * N + wn0 + lc;
   const int rows_left = M - wm0 - lr;
   acc_rows(acc, smem + wave * kStripFloats, lane, [](int) {},
            [&](int q, int t, float4 sv) __attribute__((always_inline)) {
@@ -282,10 +282,10 @@ __device__ __forceinline__ void log_self_bwd_tile(float* __restrict__ smem, floa
   const int wr0 = (wave >> 1) * 64, wc0 = (wave & 1) * 64;
   const int M = p.M, K = p.K, N = p.N;
   const int Q = GRAD_A ? N : M, R = GRAD_A ? M : K, Cc = GRAD_A ? K : N;
-  const float* ab = p.a + (long)batch * M * K;
-  const float* bb = p.b + (long)batch * K * N;
-  const float* ob = p.out + (long)batch * M * N;
-  const float* gb = p.g + (long)batch * M * N;
+  const elem_t* ab = p.a + (long)batch * M * K;
+  const elem_t* bb = p.b + (long)batch * K * N;
+  const elem_t* ob = p.out + (long)batch * M * N;
+  const elem_t* gb = p.g + (long)batch * M * N;
   const float* st = stats + (long)batch * (M + N);
   const int slabs = RAGGED ? (Q + kMS - 1) / kMS : kSelfSlabs;
   const float4 ninf = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
@@ -322,8 +322,8 @@ __device__ __forceinline__ void log_self_bwd_tile(float* __restrict__ smem, floa
     constexpr int s = decltype(sc_)::value;
     if (RAGGED && s >= slabs) return;
     const size_t dn = GRAD_A ? (size_t)(kMS * s) : (size_t)(kMS * s) * N;
-    const float* gs = gb + dn;
-    const float* os = ob + dn;
+    const elem_t* gs = gb + dn;
+    const elem_t* os = ob + dn;
 #pragma unroll
     for (int l = 0; l < 2; ++l) {
       if (!RAGGED) {
@@ -340,7 +340,7 @@ __device__ __forceinline__ void log_self_bwd_tile(float* __restrict__ smem, floa
   auto load_y = [&](auto sc_) __attribute__((always_inline)) {
     constexpr int s = decltype(sc_)::value;
     if (RAGGED && s >= slabs) return;
-    const float* ys = (GRAD_A ? bb : ab) + (GRAD_A ? (size_t)(kMS * s) : (size_t)(kMS * s) * K);
+    const elem_t* ys = (GRAD_A ? bb : ab) + (GRAD_A ? (size_t)(kMS * s) : (size_t)(kMS * s) * K);
 #pragma unroll
     for (int l = 0; l < 2; ++l) {
       if (!RAGGED) ry[s][l] = ld4(ys + oy[l]);
@@ -425,8 +425,8 @@ __device__ __forceinline__ void log_self_bwd_tile(float* __restrict__ smem, floa
   // grad = exp(x - shift) * acc, x = a (shift alpha per row) or b (beta per column)
   const int lr = lane >> 4, lc = (lane & 15) * 4;
   const long ubase = ((long)batch * R + wr0 + lr) * Cc + wc0 + lc;
-  const float* xb = (GRAD_A ? p.a : p.b) + ubase;
-  float* gp = p.grad + ubase;
+  const elem_t* xb = (GRAD_A ? p.a : p.b) + ubase;
+  elem_t* gp = p.grad + ubase;
   const int cc = RAGGED ? clamp4(Cc - (wc0 + lc)) : 4;
   const bool cok = cc > 0;
   const int rows_left = R - wr0 - lr;
@@ -475,4 +475,4 @@ void k_log_self_bwd(const LogBwdArgs pa, const LogBwdArgs pb, const float* __res
   }
 }
 
-}  // namespace genbmm
+}  // namespace GENBMM_NS

@@ -2,10 +2,9 @@
 // library (the sampling sweep reads the factors instead of taking exponentials again).
 #pragma once
 
-#include <hip/hip_runtime.h>
-#include <stdint.h>
+#include "common.h"
 
-namespace genbmm {
+namespace GENBMM_NS {
 
 // First word of the workspace's header: which forward filled the workspace last.
 constexpr int kWsNone = 0;  // one that leaves no per-tile flags (exact and whole-item kernels)
@@ -22,7 +21,7 @@ struct LogFactors {
 
 // genbmm_logbmm_fwd, except that shapes whose forward would keep nothing but the maxima
 // take the kernels that leave the factors (what log_fwd_writes_factors() describes).
-int log_fwd_with_factors(const float* a, const float* b, float* out, float* stats, int B, int M, int K,
+int log_fwd_with_factors(const elem_t* a, const elem_t* b, elem_t* out, float* stats, int B, int M, int K,
                          int N, hipStream_t s);
 
 // True (and *f filled) if a log_fwd_with_factors call with this workspace and these sizes
@@ -35,8 +34,8 @@ bool log_fwd_writes_factors(const float* stats, int B, int M, int K, int N, LogF
 // group; tiles that the forward or the sweep flagged are redone exactly (out and the
 // final index).  The caller resolves the codes.
 bool log_sample_mfma_ok(int K);  // the sweep below takes reductions up to 62 slabs of 16 terms
-int log_sample_sweep_mfma(const float* a, const float* b, float* out, int32_t* idx,
+int log_sample_sweep_mfma(const elem_t* a, const elem_t* b, elem_t* out, int32_t* idx,
                           const float* stats, uint64_t seed, uint64_t offset, int B, int M, int K,
                           int N, hipStream_t s);
 
-}  // namespace genbmm
+}  // namespace GENBMM_NS

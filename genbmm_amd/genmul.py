@@ -22,13 +22,16 @@ Differences in mechanism (not in results):
     (matmul_cuda_kernel.cu:517).
 
 Element types: float32 takes the kernels above; float64 takes the library's
-double-precision entry points (`*_f64`, no workspaces); float16 / bfloat16 are
-widened to float32 and the result is narrowed again.
+double-precision entry points (`*_f64`, no workspaces); float16 / bfloat16 take the
+same kernels compiled for that element type (`*_f16` / `*_bf16`: the loads widen,
+arithmetic and workspaces are float32, the stores round to nearest), the reference's
+AT_DISPATCH_FLOATING_TYPES_AND_HALF (matmul_cuda_kernel.cu:489).  Only logbmm's
+double backward widens half tensors on the host.
 
 Beyond the reference's contract the four functions also take operands with any
 number of leading batch dimensions (equal or broadcastable; they are flattened to
 one and restored on the result) and non-contiguous operands (made contiguous;
-the reference raises).  Both conversions, and the widening of half types, happen
+the reference raises).  Both conversions happen
 outside the autograd Functions with differentiable torch operations, so first-
 and second-order gradients reach the tensors the caller passed.  CPU tensors
 raise RuntimeError, as in the reference (matmul_cuda.cpp:65-67).
@@ -37,12 +40,17 @@ import torch
 
 from . import _lib
 
-_COMPUTE = torch.float32
-_UPCAST = (torch.float16, torch.bfloat16)
+_COMPUTE = torch.float32   # every workspace, whatever the tensors' element type
+_DTYPES = (torch.float32, torch.float64, torch.float16, torch.bfloat16)
 
 
 def _f64(t):
     return t.dtype == torch.float64
+
+
+def _sfx(t):
+    """Suffix of the entry points for t's element type ('' for float32)."""
+    return _lib.HALF_SUFFIX.get(t.dtype, "")
 
 
 PATH_AUTO, PATH_EXACT, PATH_VALU = 0, 1, 2  # GENBMM_PATH_* of the C header
@@ -55,16 +63,16 @@ def _prep(a, b):
         raise RuntimeError("a and b must be tensors")
     if a.dtype != b.dtype:
         raise RuntimeError("a and b must have the same dtype, got %s and %s" % (a.dtype, b.dtype))
-    if a.dtype not in (_COMPUTE, torch.float64):
+    if a.dtype not in _DTYPES:
         raise RuntimeError(
-            "genbmm_amd computes in float32 or float64; %s inputs are not supported" % a.dtype
+            "genbmm_amd takes float32, float64, float16 or bfloat16 tensors; %s is not supported" % a.dtype
         )
     return _lib.dense_dims(a, b)
 
 
 def _canonical(a, b):
-    """(a3, b3, restore): the operands as contiguous 3-D float32 / float64 tensors and
-    the function that gives the (B, M, N) result the caller's batch shape and dtype.
+    """(a3, b3, restore): the operands as contiguous 3-D tensors and the function that
+    gives the (B, M, N) result the caller's batch shape.
     Everything done here is an ordinary differentiable torch operation."""
     if not isinstance(a, torch.Tensor) or not isinstance(b, torch.Tensor):
         raise RuntimeError("a and b must be tensors")
@@ -76,12 +84,9 @@ def _canonical(a, b):
         raise RuntimeError("a and b must have at least 2 dimensions")
     if a.shape[-1] != b.shape[-2]:
         raise RuntimeError("shape mismatch: a is %s, b is %s" % (tuple(a.shape), tuple(b.shape)))
-    in_dtype = a.dtype
-    if in_dtype in _UPCAST:
-        a, b = a.float(), b.float()
-    elif in_dtype not in (_COMPUTE, torch.float64):
+    if a.dtype not in _DTYPES:
         raise RuntimeError(
-            "genbmm_amd computes in float32 or float64; %s inputs are not supported" % in_dtype
+            "genbmm_amd takes float32, float64, float16 or bfloat16 tensors; %s is not supported" % a.dtype
         )
     batch = None
     if a.dim() != 3 or b.dim() != 3 or a.shape[0] != b.shape[0]:
@@ -96,7 +101,7 @@ def _canonical(a, b):
     def restore(out):
         if batch is not None:
             out = out.reshape(batch + out.shape[-2:])
-        return out if out.dtype == in_dtype else out.to(in_dtype)
+        return out
 
     return a, b, restore
 
@@ -124,7 +129,7 @@ class _LogBmmGrad(torch.autograd.Function):
             _call("genbmm_logbmm_bwd_f64", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g),
                   _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
         else:
-            _call("genbmm_logbmm_bwd_path", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g),
+            _call("genbmm_logbmm_bwd_path" + _sfx(a), a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g),
                   _lib.ptr(stats), _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N, path)
         ctx.save_for_backward(a, b, g, out)
         ctx.set_materialize_grads(False)
@@ -136,15 +141,18 @@ class _LogBmmGrad(torch.autograd.Function):
             return None, None, None, None, None, None
         a, b, g, out = ctx.saved_tensors
         B, M, K, N = _lib.dense_dims(a, b)
-        u_a = None if u_a is None else u_a.contiguous()
-        u_b = None if u_b is None else u_b.contiguous()
+        dtype = a.dtype
+        if _sfx(a):  # the second-order kernels re-read their own grad_g: float32 tensors only
+            a, b, g, out = a.float(), b.float(), g.float(), out.float()
+        u_a = None if u_a is None else u_a.to(a.dtype).contiguous()
+        u_b = None if u_b is None else u_b.to(a.dtype).contiguous()
         ga = torch.empty_like(a)
         gb = torch.empty_like(b)
         gg = torch.empty_like(g)
         _call("genbmm_logbmm_bwdbwd_f64" if _f64(a) else "genbmm_logbmm_bwdbwd", a, _lib.ptr(a),
               _lib.ptr(b), _lib.ptr(out), _lib.ptr(g), _lib.ptr(u_a), _lib.ptr(u_b), _lib.ptr(ga),
               _lib.ptr(gb), _lib.ptr(gg), B, M, K, N)
-        return ga, gb, gg, None, None, None
+        return ga.to(dtype), gb.to(dtype), gg.to(dtype), None, None, None
 
 
 class LogMatMul(torch.autograd.Function):
@@ -162,8 +170,8 @@ class LogMatMul(torch.autograd.Function):
             # the library's workspace: what the reference's `maxes` becomes
             stats = torch.empty(_lib.load().genbmm_logbmm_stats_size(B, M, K, N), dtype=_COMPUTE,
                                 device=a.device)
-            _call("genbmm_logbmm_fwd_path", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(stats),
-                  B, M, K, N, path)
+            _call("genbmm_logbmm_fwd_path" + _sfx(a), a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out),
+                  _lib.ptr(stats), B, M, K, N, path)
         ctx.save_for_backward(a, b, out, stats)
         ctx.path = path
         return out
@@ -195,10 +203,10 @@ def _argmax_backward(ctx, grad_output, prod):
                   _lib.ptr(grad_b), B, M, K, N)
     elif prod:
         # the factors a[m, idx], b[idx, n] were stored by the forward: a and b are not read
-        _call("genbmm_prodmax_bwd", g, _lib.ptr(None), _lib.ptr(None), _lib.ptr(idx), _lib.ptr(factors), _lib.ptr(g),
-              _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
+        _call("genbmm_prodmax_bwd" + _sfx(g), g, _lib.ptr(None), _lib.ptr(None), _lib.ptr(idx),
+              _lib.ptr(factors), _lib.ptr(g), _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
     else:
-        _call("genbmm_argmax_bwd", g, _lib.ptr(idx), _lib.ptr(g), _lib.ptr(grad_a),
+        _call("genbmm_argmax_bwd" + _sfx(g), g, _lib.ptr(idx), _lib.ptr(g), _lib.ptr(grad_a),
               _lib.ptr(grad_b), B, M, K, N)
     return grad_a, grad_b
 
@@ -212,7 +220,7 @@ class MaxMatMul(torch.autograd.Function):
         B, M, K, N = dims
         out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)
         idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
-        _call("genbmm_maxbmm_fwd_f64" if _f64(a) else "genbmm_maxbmm_fwd", a, _lib.ptr(a),
+        _call("genbmm_maxbmm_fwd_f64" if _f64(a) else "genbmm_maxbmm_fwd" + _sfx(a), a, _lib.ptr(a),
               _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), B, M, K, N)
         ctx.save_for_backward(idx)
         ctx.dims, ctx.compute = dims, a.dtype
@@ -239,7 +247,7 @@ class ProdMaxMatMul(torch.autograd.Function):
             ctx.save_for_backward(idx, empty, a, b)
         else:
             factors = torch.empty(2, B, M, N, dtype=_COMPUTE, device=a.device)
-            _call("genbmm_prodmaxbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
+            _call("genbmm_prodmaxbmm_fwd" + _sfx(a), a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
                   _lib.ptr(factors), B, M, K, N)
             ctx.save_for_backward(idx, factors, empty, empty)
         ctx.dims, ctx.compute = dims, a.dtype
@@ -282,7 +290,7 @@ class SampleMatMul(torch.autograd.Function):
         else:
             stats = torch.empty(_lib.load().genbmm_samplebmm_stats_size(B, M, K, N), dtype=_COMPUTE,
                                 device=a.device)
-            _call("genbmm_samplebmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
+            _call("genbmm_samplebmm_fwd" + _sfx(a), a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
                   _lib.ptr(stats), seed, offset, B, M, K, N)
         ctx.save_for_backward(idx)
         ctx.dims, ctx.compute = dims, a.dtype

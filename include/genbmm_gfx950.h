@@ -449,6 +449,86 @@ int genbmm_banded_bwdbwd_f64(const double* a, int a_lu, int a_ld,
                              double* grad_a, double* grad_b, double* grad_g,
                              int B, int n, void* stream);
 
+/* --------------------------------------------------------- half precision */
+
+/*
+ * The reference instantiates its dense kernels for Half too
+ * (AT_DISPATCH_FLOATING_TYPES_AND_HALF, matmul_cuda_kernel.cu:489, :503, :518,
+ * :533 for the four forwards, :654-:709 for the backwards), computing in
+ * scalar_t = Half.
+ * The functions below are the float functions of the same name compiled for
+ * tensors of IEEE binary16 (`_f16`) and bfloat16 (`_bf16`) elements, passed as
+ * their 16-bit patterns: a, b, out, g, grad_a and grad_b are of that type;
+ * stats, factors and idx keep their float / int32 types and the sizes the float
+ * functions use (genbmm_logbmm_stats_size, genbmm_samplebmm_stats_size,
+ * 2*B*M*N factors).  A value is widened by the load that fetches it, all
+ * arithmetic and every workspace is fp32, a result is rounded to nearest-even
+ * by the store that writes it: each function returns exactly what its float
+ * namesake returns on the widened tensors, rounded once (indices: identical).
+ * The backward functions that read `out` read the rounded one, as the
+ * reference's do.  samplebmm sweeps only where the forward left 1/S in the
+ * workspace (matrix-core shapes, K <= 992) and walks the terms exactly
+ * otherwise: `out` rounded to 11 or 8 bits does not give S well enough for the
+ * other sweeps.  genbmm_logbmm_bwdbwd and the banded functions have no half
+ * form: callers widen those tensors.
+ */
+int genbmm_logbmm_fwd_f16(const uint16_t* a, const uint16_t* b, uint16_t* out,
+                          float* stats, int B, int M, int K, int N, void* stream);
+int genbmm_logbmm_fwd_bf16(const uint16_t* a, const uint16_t* b, uint16_t* out,
+                           float* stats, int B, int M, int K, int N, void* stream);
+int genbmm_logbmm_bwd_f16(const uint16_t* a, const uint16_t* b, const uint16_t* out,
+                          const uint16_t* g, const float* stats,
+                          uint16_t* grad_a, uint16_t* grad_b,
+                          int B, int M, int K, int N, void* stream);
+int genbmm_logbmm_bwd_bf16(const uint16_t* a, const uint16_t* b, const uint16_t* out,
+                           const uint16_t* g, const float* stats,
+                           uint16_t* grad_a, uint16_t* grad_b,
+                           int B, int M, int K, int N, void* stream);
+int genbmm_logbmm_fwd_path_f16(const uint16_t* a, const uint16_t* b, uint16_t* out,
+                               float* stats, int B, int M, int K, int N, int path,
+                               void* stream);
+int genbmm_logbmm_fwd_path_bf16(const uint16_t* a, const uint16_t* b, uint16_t* out,
+                                float* stats, int B, int M, int K, int N, int path,
+                                void* stream);
+int genbmm_logbmm_bwd_path_f16(const uint16_t* a, const uint16_t* b, const uint16_t* out,
+                               const uint16_t* g, const float* stats,
+                               uint16_t* grad_a, uint16_t* grad_b,
+                               int B, int M, int K, int N, int path, void* stream);
+int genbmm_logbmm_bwd_path_bf16(const uint16_t* a, const uint16_t* b, const uint16_t* out,
+                                const uint16_t* g, const float* stats,
+                                uint16_t* grad_a, uint16_t* grad_b,
+                                int B, int M, int K, int N, int path, void* stream);
+int genbmm_maxbmm_fwd_f16(const uint16_t* a, const uint16_t* b, uint16_t* out,
+                          int32_t* idx, int B, int M, int K, int N, void* stream);
+int genbmm_maxbmm_fwd_bf16(const uint16_t* a, const uint16_t* b, uint16_t* out,
+                           int32_t* idx, int B, int M, int K, int N, void* stream);
+int genbmm_prodmaxbmm_fwd_f16(const uint16_t* a, const uint16_t* b, uint16_t* out,
+                              int32_t* idx, float* factors,
+                              int B, int M, int K, int N, void* stream);
+int genbmm_prodmaxbmm_fwd_bf16(const uint16_t* a, const uint16_t* b, uint16_t* out,
+                               int32_t* idx, float* factors,
+                               int B, int M, int K, int N, void* stream);
+int genbmm_samplebmm_fwd_f16(const uint16_t* a, const uint16_t* b, uint16_t* out,
+                             int32_t* idx, float* stats, uint64_t seed, uint64_t offset,
+                             int B, int M, int K, int N, void* stream);
+int genbmm_samplebmm_fwd_bf16(const uint16_t* a, const uint16_t* b, uint16_t* out,
+                              int32_t* idx, float* stats, uint64_t seed, uint64_t offset,
+                              int B, int M, int K, int N, void* stream);
+int genbmm_argmax_bwd_f16(const int32_t* idx, const uint16_t* g,
+                          uint16_t* grad_a, uint16_t* grad_b,
+                          int B, int M, int K, int N, void* stream);
+int genbmm_argmax_bwd_bf16(const int32_t* idx, const uint16_t* g,
+                           uint16_t* grad_a, uint16_t* grad_b,
+                           int B, int M, int K, int N, void* stream);
+int genbmm_prodmax_bwd_f16(const uint16_t* a, const uint16_t* b, const int32_t* idx,
+                           const float* factors, const uint16_t* g,
+                           uint16_t* grad_a, uint16_t* grad_b,
+                           int B, int M, int K, int N, void* stream);
+int genbmm_prodmax_bwd_bf16(const uint16_t* a, const uint16_t* b, const int32_t* idx,
+                            const float* factors, const uint16_t* g,
+                            uint16_t* grad_a, uint16_t* grad_b,
+                            int B, int M, int K, int N, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -745,8 +745,9 @@ def test_views_and_batch_dimensions(gpu):
 
 
 def test_half_inputs_are_twice_differentiable(gpu):
-    """float16 / bfloat16 operands are widened by a differentiable cast outside the
-    autograd Function, so second-order terms reach the half tensors as well."""
+    """float16 / bfloat16 operands stay in their type through forward and backward; the
+    double backward widens what the first backward saved, so second-order terms reach the
+    half tensors as well."""
     torch.manual_seed(12)
     for dt in (torch.float16, torch.bfloat16):
         a = torch.randn(2, 6, 7).to(dt)

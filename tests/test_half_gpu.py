@@ -1,0 +1,177 @@
+"""float16 / bfloat16 tensors through the dense entry points (`*_f16`, `*_bf16`): the kernels
+are the float kernels compiled for that element type - loads widen, arithmetic and workspaces
+are fp32, stores round to nearest - so the contract tested here is exact: every result equals
+what the float entry point returns on the widened tensors, rounded once (indices identical),
+for every kernel family a shape can take.  On top of that the results are compared with the
+float64 closed forms / the sequential oracle at the tolerance of one rounding of the output
+type.  (The reference computes in scalar_t = Half, matmul_cuda_kernel.cu:489; it has no test
+for it.)"""
+import pytest
+import torch
+
+import oracle
+import genbmm_amd as genbmm
+from genbmm_amd import _lib
+
+pytestmark = pytest.mark.gpu
+
+TYPES = [(torch.float16, "_f16", 2.0 ** -11), (torch.bfloat16, "_bf16", 2.0 ** -8)]
+# whole items (32^3 on the matrix cores, up to 64^3 in LDS), one 128 x 128 tile per item, tiled
+# matrix-core shapes (full tiles, ragged, 256-wide tiles), vector-ALU shapes, odd alignments
+SHAPES = [(3, 32, 32, 32), (2, 64, 64, 64), (3, 20, 33, 50), (5, 128, 128, 128), (3, 100, 96, 120),
+          (2, 256, 128, 256), (2, 200, 77, 131), (2, 70, 50, 90), (1, 33, 17, 200), (2, 129, 513, 257),
+          (8, 512, 256, 512)]
+P = _lib.ptr
+
+
+def lse64(a, b, chunk=2):
+    """float64 logsumexp of the broadcast form (README.md:23-30 of the reference), in batch chunks."""
+    outs = [oracle.logbmm_broadcast(a[i:i + chunk].double(), b[i:i + chunk].double())
+            for i in range(0, a.shape[0], chunk)]
+    return torch.cat(outs) if outs else a.new_zeros((0, a.shape[1], b.shape[2])).double()
+
+
+def _operands(gpu, dt, B, M, K, N, scale=2.0):
+    a = (scale * torch.randn(B, M, K, device=gpu)).to(dt)
+    b = (scale * torch.randn(B, K, N, device=gpu)).to(dt)
+    g = torch.randn(B, M, N, device=gpu).to(dt)
+    return a, b, g
+
+
+@pytest.mark.parametrize("dt,suffix,eps", TYPES)
+@pytest.mark.parametrize("path", [genbmm.genmul.PATH_AUTO, genbmm.genmul.PATH_EXACT, genbmm.genmul.PATH_VALU])
+def test_logbmm_half_equals_float_kernels_rounded(gpu, dt, suffix, eps, path):
+    lib = _lib.load()
+    torch.manual_seed(3)
+    for B, M, K, N in SHAPES:
+        a, b, g = _operands(gpu, dt, B, M, K, N)
+        a32, b32, g32 = a.float(), b.float(), g.float()
+        n = lib.genbmm_logbmm_stats_size(B, M, K, N)
+        st, st32 = torch.empty(n, device=gpu), torch.empty(n, device=gpu)
+        out, out32 = torch.empty(B, M, N, device=gpu, dtype=dt), torch.empty(B, M, N, device=gpu)
+        s = _lib.stream_of(a)
+        assert getattr(lib, "genbmm_logbmm_fwd_path" + suffix)(P(a), P(b), P(out), P(st), B, M, K, N, path, s) == 0
+        assert lib.genbmm_logbmm_fwd_path(P(a32), P(b32), P(out32), P(st32), B, M, K, N, path, s) == 0
+        assert torch.equal(out, out32.to(dt)), (B, M, K, N)
+        if B * M * K * N <= 40_000_000:
+            want = lse64(a32.cpu(), b32.cpu())
+            # one rounding of the result (half an ulp: eps relative) on top of the fp32 kernel's own error
+            err = (out.double().cpu() - want).abs()
+            assert bool((err <= eps * want.abs() + 1e-5 * want.abs() + 1e-6).all()), (B, M, K, N, float(err.max()))
+        # the backward reads `out` as stored (rounded): the float kernels get the same values
+        ga, gb = torch.empty_like(a), torch.empty_like(b)
+        ga32, gb32 = torch.empty_like(a32), torch.empty_like(b32)
+        oh = out.float()
+        assert getattr(lib, "genbmm_logbmm_bwd_path" + suffix)(P(a), P(b), P(out), P(g), P(st), P(ga), P(gb),
+                                                              B, M, K, N, path, s) == 0
+        assert lib.genbmm_logbmm_bwd_path(P(a32), P(b32), P(oh), P(g32), P(st32), P(ga32), P(gb32),
+                                          B, M, K, N, path, s) == 0
+        assert torch.equal(ga, ga32.to(dt)) and torch.equal(gb, gb32.to(dt)), (B, M, K, N)
+
+
+@pytest.mark.parametrize("dt,suffix,eps", TYPES)
+def test_logbmm_half_gradients_against_float64(gpu, dt, suffix, eps):
+    """Through the autograd layer, against float64 autograd of the closed form on the same
+    (half-valued) operands.  The weights exp(a + b - out) are formed with `out` as stored:
+    its rounding (eps |out|) enters every gradient term as a relative error."""
+    torch.manual_seed(4)
+    for B, M, K, N in [(3, 32, 32, 32), (2, 50, 40, 70), (4, 128, 128, 128), (2, 256, 128, 256), (2, 130, 97, 150)]:
+        a, b, g = _operands(gpu, dt, B, M, K, N, scale=1.0)
+        want, wa, wb = oracle.logbmm_grads64(a.float().cpu(), b.float().cpu(), g.float().cpu())
+        ad, bd = a.clone().requires_grad_(True), b.clone().requires_grad_(True)
+        out = genbmm.logbmm(ad, bd)
+        assert out.dtype == dt
+        ga, gb = torch.autograd.grad(out, (ad, bd), g)
+        assert ga.dtype == dt and gb.dtype == dt
+        omax = float(want.abs().max())
+        for got, ref in ((ga, wa), (gb, wb)):
+            scale = float(ref.abs().max())
+            tol = (2.0 * eps * omax + 2.0 * eps) * scale + 1e-6
+            assert float((got.double().cpu() - ref).abs().max()) <= tol, (B, M, K, N)
+
+
+@pytest.mark.parametrize("dt,suffix,eps", TYPES)
+@pytest.mark.parametrize("prod", [False, True])
+def test_max_products_half_bit_exact(gpu, dt, suffix, eps, prod):
+    """Values and indices equal the sequential oracle's on the widened operands (values
+    rounded once: a + b and a * b of two half values are exact in fp32), and so do the
+    gradients, whose ordered fp32 sums are rounded once."""
+    torch.manual_seed(5)
+    for B, M, K, N in [(3, 20, 33, 50), (2, 64, 64, 64), (2, 200, 77, 131), (1, 33, 300, 200), (2, 129, 513, 70)]:
+        a, b, g = _operands(gpu, dt, B, M, K, N)
+        g = (torch.round(g.float() * 8) / 8).to(dt)
+        sv, si = oracle.seq_maxbmm_fwd(a.float().cpu(), b.float().cpu(), prod)
+        ad, bd = a.clone().requires_grad_(True), b.clone().requires_grad_(True)
+        out = (genbmm.prodmaxbmm if prod else genbmm.maxbmm)(ad, bd)
+        assert out.dtype == dt
+        assert torch.equal(out.detach().cpu(), sv.to(dt)), (B, M, K, N)
+        ga, gb = torch.autograd.grad(out, (ad, bd), g)
+        wa, wb = oracle.seq_argmax_bwd(a.float().cpu() if prod else K, b.float().cpu(), si, g.float().cpu(), prod)
+        assert torch.equal(ga.cpu(), wa.to(dt)) and torch.equal(gb.cpu(), wb.to(dt)), (B, M, K, N)
+        # the gathering form of the product backward (no stored factors) agrees
+        if prod:
+            lib = _lib.load()
+            idx = si.to(gpu).to(torch.int32)
+            ga2, gb2 = torch.empty_like(a), torch.empty_like(b)
+            assert getattr(lib, "genbmm_prodmax_bwd" + suffix)(P(a), P(b), P(idx), P(None), P(g), P(ga2), P(gb2),
+                                                              B, M, K, N, _lib.stream_of(a)) == 0
+            assert torch.equal(ga2, ga) and torch.equal(gb2, gb)
+
+
+@pytest.mark.parametrize("dt,suffix,eps", TYPES)
+def test_samplebmm_half(gpu, dt, suffix, eps):
+    """Every index brackets its uniform in the float64 CDF of the (half-valued) operands;
+    shapes that take the matrix-core sweep (1/S from the fp32 workspace) and shapes that walk
+    exactly; out is the float result rounded once."""
+    lib = _lib.load()
+    torch.manual_seed(6)
+    for B, M, K, N in [(3, 20, 33, 50), (5, 128, 128, 128), (2, 200, 77, 131), (2, 256, 512, 128), (1, 128, 1040, 160),
+                       (2, 64, 300, 96)]:
+        a, b, _ = _operands(gpu, dt, B, M, K, N)
+        out = torch.empty(B, M, N, device=gpu, dtype=dt)
+        idx = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
+        stats = torch.empty(lib.genbmm_samplebmm_stats_size(B, M, K, N), device=gpu)
+        assert getattr(lib, "genbmm_samplebmm_fwd" + suffix)(P(a), P(b), P(out), P(idx), P(stats), 21, 4, B, M, K, N,
+                                                            _lib.stream_of(a)) == 0
+        a32, b32 = a.float().cpu(), b.float().cpu()
+        want = lse64(a32, b32)
+        err = (out.double().cpu() - want).abs()
+        assert bool((err <= eps * want.abs() + 1e-5 * want.abs() + 1e-6).all()), (B, M, K, N)
+        u = oracle.philox_uniform(0, B * M * N, 21, 4).view(B, M, N).double()
+        cdf = oracle.sample_cdf64(a32, b32)
+        got = idx.cpu().long()
+        assert int(got.min()) >= 0 and int(got.max()) < K
+        hi = torch.gather(cdf, 2, got.unsqueeze(2)).squeeze(2)
+        lo = torch.where(got > 0, torch.gather(cdf, 2, (got - 1).clamp(min=0).unsqueeze(2)).squeeze(2),
+                         torch.zeros_like(hi))
+        tol = max(2e-5, 2.0 * K * 2.0 ** -24)
+        assert bool(((lo - tol <= u) & (u <= hi + tol)).all()), (B, M, K, N)
+        # through the autograd layer: one-hot gradient of the sampled term
+        ad = a.clone().requires_grad_(True)
+        s = genbmm.samplebmm(ad, b, (21, 4))
+        (ga,) = torch.autograd.grad(s.sum(), ad)
+        assert ga.dtype == dt and float(ga.float().sum()) == pytest.approx(B * M * N, rel=1e-2)
+
+
+def test_half_masks_and_empty(gpu):
+    """-inf masks, rows without mass, the reference's -1e9 floor (which is -inf in
+    binary16, as `scalar_t m = -1e9` is in the reference) and empty extents."""
+    for dt in (torch.float16, torch.bfloat16):
+        torch.manual_seed(8)
+        a = torch.randn(2, 70, 40, device=gpu).to(dt)
+        b = torch.randn(2, 40, 90, device=gpu).to(dt)
+        a[:, ::3, ::5] = float("-inf")
+        a[1, 5, :] = float("-inf")
+        out = genbmm.logbmm(a, b)
+        want = lse64(a.float().cpu(), b.float().cpu())
+        assert bool(torch.isneginf(out[1, 5]).all())
+        live = torch.isfinite(want)
+        eps = 2.0 ** -11 if dt == torch.float16 else 2.0 ** -8
+        assert bool(((out.double().cpu() - want).abs()[live] <= eps * want.abs()[live] + 1e-4).all())
+        for shape in [(0, 3, 4, 5), (2, 0, 4, 5), (2, 3, 4, 0)]:
+            B, M, K, N = shape
+            z = genbmm.logbmm(torch.randn(B, M, K, device=gpu).to(dt), torch.randn(B, K, N, device=gpu).to(dt))
+            assert z.shape == (B, M, N) and z.dtype == dt
+        e = genbmm.maxbmm(torch.randn(2, 3, 0, device=gpu).to(dt), torch.randn(2, 0, 5, device=gpu).to(dt))
+        floor = torch.full(e.shape, -1e9, device=gpu).to(dt)   # rounded to the type (-inf in binary16)
+        assert torch.equal(e, floor)
