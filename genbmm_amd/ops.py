@@ -1,4 +1,5 @@
-"""The dense and banded products as `torch.library` custom operators (float32).
+"""The dense and banded products as `torch.library` custom operators (float32; the dense
+ones also float16 / bfloat16).
 
 `genbmm_amd.logbmm` and friends are `torch.autograd.Function`s, which `torch.compile`
 cannot trace through.  This module registers the same library calls as operators of the
@@ -31,9 +32,15 @@ def _dims(a: Tensor, b: Tensor):
 
 
 def _check(a: Tensor, b: Tensor):
-    if a.dtype != _F32 or b.dtype != _F32:
-        raise RuntimeError("genbmm_amd.ops: float32 tensors only (use genbmm_amd.logbmm etc. for others)")
+    if a.dtype != b.dtype or (a.dtype != _F32 and a.dtype not in _lib.HALF_SUFFIX):
+        raise RuntimeError("genbmm_amd.ops: float32, float16 or bfloat16 tensors of one type "
+                           "(use genbmm_amd.logbmm etc. for others)")
     return _lib.dense_dims(a, b)
+
+
+def _sfx(t: Tensor):
+    """Suffix of the library's entry points for t's element type."""
+    return _lib.HALF_SUFFIX.get(t.dtype, "")
 
 
 def _call(name, t, *args):
@@ -51,24 +58,24 @@ def _stats_size(B, M, K, N):
 def logbmm_fwd(a: Tensor, b: Tensor) -> Tuple[Tensor, Tensor]:
     """(out, stats): out = logsumexp_k(a + b); stats is the library's workspace."""
     B, M, K, N = _check(a, b)
-    out = torch.empty(B, M, N, dtype=_F32, device=a.device)
+    out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)
     stats = torch.empty(_stats_size(B, M, K, N), dtype=_F32, device=a.device)
-    _call("genbmm_logbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(stats), B, M, K, N)
+    _call("genbmm_logbmm_fwd" + _sfx(a), a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(stats), B, M, K, N)
     return out, stats
 
 
 @logbmm_fwd.register_fake
 def _(a, b):
     B, M, K, N = _dims(a, b)
-    return a.new_empty(B, M, N), a.new_empty(_stats_size(B, M, K, N))
+    return a.new_empty(B, M, N), a.new_empty(_stats_size(B, M, K, N), dtype=_F32)
 
 
 @torch.library.custom_op("genbmm_amd::logbmm_bwd", mutates_args=())
 def logbmm_bwd(a: Tensor, b: Tensor, out: Tensor, g: Tensor, stats: Tensor) -> Tuple[Tensor, Tensor]:
     B, M, K, N = _check(a, b)
-    g = g.contiguous()
+    g = g.to(a.dtype).contiguous()
     grad_a, grad_b = torch.empty_like(a), torch.empty_like(b)
-    _call("genbmm_logbmm_bwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g), _lib.ptr(stats),
+    _call("genbmm_logbmm_bwd" + _sfx(a), a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g), _lib.ptr(stats),
           _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
     return grad_a, grad_b
 
@@ -83,11 +90,14 @@ def logbmm_bwdbwd(a: Tensor, b: Tensor, out: Tensor, g: Tensor, u_a: Tensor,
                   u_b: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
     """Gradients of <u_a, grad_a> + <u_b, grad_b> with respect to (a, b, g)."""
     B, M, K, N = _check(a, b)
-    g, u_a, u_b = g.contiguous(), u_a.contiguous(), u_b.contiguous()
+    dtype = a.dtype
+    if _sfx(a):  # the second-order kernels take float tensors: half ones are widened here
+        a, b, out = a.float(), b.float(), out.float()
+    g, u_a, u_b = g.to(a.dtype).contiguous(), u_a.to(a.dtype).contiguous(), u_b.to(a.dtype).contiguous()
     ga, gb, gg = torch.empty_like(a), torch.empty_like(b), torch.empty_like(g)
     _call("genbmm_logbmm_bwdbwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g), _lib.ptr(u_a),
           _lib.ptr(u_b), _lib.ptr(ga), _lib.ptr(gb), _lib.ptr(gg), B, M, K, N)
-    return ga, gb, gg
+    return ga.to(dtype), gb.to(dtype), gg.to(dtype)
 
 
 @logbmm_bwdbwd.register_fake
@@ -131,9 +141,9 @@ def logbmm(a: Tensor, b: Tensor) -> Tensor:
 @torch.library.custom_op("genbmm_amd::maxbmm_fwd", mutates_args=())
 def maxbmm_fwd(a: Tensor, b: Tensor) -> Tuple[Tensor, Tensor]:
     B, M, K, N = _check(a, b)
-    out = torch.empty(B, M, N, dtype=_F32, device=a.device)
+    out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)
     idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
-    _call("genbmm_maxbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), B, M, K, N)
+    _call("genbmm_maxbmm_fwd" + _sfx(a), a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), B, M, K, N)
     return out, idx
 
 
@@ -146,11 +156,11 @@ def _(a, b):
 @torch.library.custom_op("genbmm_amd::samplebmm_fwd", mutates_args=())
 def samplebmm_fwd(a: Tensor, b: Tensor, seed: int, offset: int) -> Tuple[Tensor, Tensor]:
     B, M, K, N = _check(a, b)
-    out = torch.empty(B, M, N, dtype=_F32, device=a.device)
+    out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)
     idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
     stats = torch.empty(int(_lib.load().genbmm_samplebmm_stats_size(int(B), int(M), int(K), int(N))),
                         dtype=_F32, device=a.device)
-    _call("genbmm_samplebmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), _lib.ptr(stats),
+    _call("genbmm_samplebmm_fwd" + _sfx(a), a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), _lib.ptr(stats),
           seed & 0xFFFFFFFFFFFFFFFF, offset & 0xFFFFFFFFFFFFFFFF, B, M, K, N)
     return out, idx
 
@@ -166,9 +176,9 @@ def argmax_bwd(idx: Tensor, g: Tensor, K: int) -> Tuple[Tensor, Tensor]:
     """One-hot(idx) * g summed over n (grad_a) and over m (grad_b)."""
     B, M, N = idx.shape
     g = g.contiguous()
-    grad_a = torch.empty(B, M, K, dtype=_F32, device=g.device)
-    grad_b = torch.empty(B, K, N, dtype=_F32, device=g.device)
-    _call("genbmm_argmax_bwd", g, _lib.ptr(idx), _lib.ptr(g), _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
+    grad_a = torch.empty(B, M, K, dtype=g.dtype, device=g.device)
+    grad_b = torch.empty(B, K, N, dtype=g.dtype, device=g.device)
+    _call("genbmm_argmax_bwd" + _sfx(g), g, _lib.ptr(idx), _lib.ptr(g), _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
     return grad_a, grad_b
 
 
@@ -198,10 +208,10 @@ torch.library.register_autograd("genbmm_amd::samplebmm_fwd", _argmax_backward, s
 def prodmaxbmm_fwd(a: Tensor, b: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
     """(out, idx, factors): factors holds a[m, idx] and b[idx, n] per cell for the backward."""
     B, M, K, N = _check(a, b)
-    out = torch.empty(B, M, N, dtype=_F32, device=a.device)
+    out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)
     idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
     factors = torch.empty(2, B, M, N, dtype=_F32, device=a.device)
-    _call("genbmm_prodmaxbmm_fwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), _lib.ptr(factors),
+    _call("genbmm_prodmaxbmm_fwd" + _sfx(a), a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), _lib.ptr(factors),
           B, M, K, N)
     return out, idx, factors
 
@@ -209,16 +219,16 @@ def prodmaxbmm_fwd(a: Tensor, b: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
 @prodmaxbmm_fwd.register_fake
 def _(a, b):
     B, M, K, N = _dims(a, b)
-    return a.new_empty(B, M, N), a.new_empty(B, M, N, dtype=torch.int32), a.new_empty(2, B, M, N)
+    return a.new_empty(B, M, N), a.new_empty(B, M, N, dtype=torch.int32), a.new_empty(2, B, M, N, dtype=_F32)
 
 
 @torch.library.custom_op("genbmm_amd::prodmax_bwd", mutates_args=())
 def prodmax_bwd(idx: Tensor, factors: Tensor, g: Tensor, K: int) -> Tuple[Tensor, Tensor]:
     B, M, N = idx.shape
     g = g.contiguous()
-    grad_a = torch.empty(B, M, K, dtype=_F32, device=g.device)
-    grad_b = torch.empty(B, K, N, dtype=_F32, device=g.device)
-    _call("genbmm_prodmax_bwd", g, _lib.ptr(None), _lib.ptr(None), _lib.ptr(idx), _lib.ptr(factors), _lib.ptr(g),
+    grad_a = torch.empty(B, M, K, dtype=g.dtype, device=g.device)
+    grad_b = torch.empty(B, K, N, dtype=g.dtype, device=g.device)
+    _call("genbmm_prodmax_bwd" + _sfx(g), g, _lib.ptr(None), _lib.ptr(None), _lib.ptr(idx), _lib.ptr(factors), _lib.ptr(g),
           _lib.ptr(grad_a), _lib.ptr(grad_b), B, M, K, N)
     return grad_a, grad_b
 

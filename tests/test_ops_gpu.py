@@ -39,6 +39,37 @@ def test_operators_match_the_functions(gpu):
     assert torch.equal(first[0], r[0]) and torch.equal(first[1], r[1])
 
 
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_operators_on_half_tensors(gpu, dt):
+    """float16 / bfloat16 tensors: the operators and the autograd Functions call the same
+    entry points (same bits), the registrations pass torch's checks, a graph compiles."""
+    a, b = pair(gpu)
+    a, b = a.detach().to(dt).requires_grad_(True), b.detach().to(dt).requires_grad_(True)
+    g = torch.randn(3, 70, 66, device=gpu).to(dt)
+    for op, fn in ((ops.logbmm, genbmm.logbmm), (ops.maxbmm, genbmm.maxbmm), (ops.prodmaxbmm, genbmm.prodmaxbmm)):
+        y, want = op(a, b), fn(a, b)
+        assert y.dtype == dt and torch.equal(y, want)
+        ga, gb = torch.autograd.grad(y, (a, b), g)
+        wa, wb = torch.autograd.grad(want, (a, b), g)
+        assert ga.dtype == dt and torch.equal(ga, wa) and torch.equal(gb, wb)
+    assert torch.equal(ops.samplebmm(a, b, 99, 4), genbmm.samplebmm(a, b, (99, 4)))
+    u = torch.randn_like(a)
+    res = []
+    for op in (ops.logbmm, genbmm.logbmm):
+        (ga,) = torch.autograd.grad(op(a, b), a, g, create_graph=True)
+        res.append(torch.autograd.grad((ga * u).sum(), (a, b)))
+    assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
+    ad, bd = a.detach()[:, :9, :12].contiguous(), b.detach()[:, :12, :7].contiguous()
+    tests = ("test_schema", "test_faketensor", "test_autograd_registration")
+    torch.library.opcheck(torch.ops.genbmm_amd.logbmm_fwd.default, (ad, bd), test_utils=tests)
+    torch.library.opcheck(torch.ops.genbmm_amd.prodmaxbmm_fwd.default, (ad, bd), test_utils=tests)
+    out, stats = torch.ops.genbmm_amd.logbmm_fwd(ad, bd)
+    torch.library.opcheck(torch.ops.genbmm_amd.logbmm_bwd.default, (ad, bd, out, torch.randn_like(out), stats),
+                          test_utils=tests)
+    compiled = torch.compile(lambda x, y: ops.logbmm(x, y).float().sum(), backend="aot_eager", fullgraph=True)
+    assert torch.equal(compiled(a, b), genbmm.logbmm(a, b).float().sum())
+
+
 def test_registrations_pass_opcheck(gpu):
     a, b = pair(gpu, 2, 9, 12, 7)
     ad, bd = a.detach(), b.detach()
