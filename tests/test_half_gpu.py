@@ -69,6 +69,62 @@ def test_logbmm_half_equals_float_kernels_rounded(gpu, dt, suffix, eps, path):
         assert torch.equal(ga, ga32.to(dt)) and torch.equal(gb, gb32.to(dt)), (B, M, K, N)
 
 
+def _odd_shapes(seed, count, kmax):
+    """Extents on both sides of every tile, slab and vector boundary, odd row lengths (rows of a
+    half tensor then start at any 2-byte address)."""
+    import random
+    rng = random.Random(seed)
+    edge = [1, 2, 3, 7, 8, 9, 31, 32, 33, 63, 64, 65, 95, 96, 97, 127, 128, 129, 130, 255, 257]
+    out = []
+    for _ in range(count):
+        M = rng.choice(edge + [rng.randint(1, 300)])
+        N = rng.choice(edge + [rng.randint(1, 300)])
+        K = rng.choice([1, 2, 7, 8, 9, 15, 16, 17, 31, 33, 127, 128, 129, 255, 257, rng.randint(1, kmax)])
+        B = rng.randint(1, 3)
+        if B * M * K * N > 8_000_000:
+            K = max(1, 8_000_000 // (B * M * N))
+        out.append((B, M, K, N))
+    return out
+
+
+@pytest.mark.parametrize("dt,suffix,eps", TYPES)
+def test_half_equals_float_kernels_on_many_shapes(gpu, dt, suffix, eps):
+    """The bit-for-bit contract on sixty seeded shapes: logbmm forward and backward (default
+    path), maxbmm and prodmaxbmm values, indices and gradients."""
+    lib = _lib.load()
+    torch.manual_seed(9)
+    for B, M, K, N in _odd_shapes(17, 60, 600):
+        a, b, g = _operands(gpu, dt, B, M, K, N)
+        a32, b32, g32 = a.float(), b.float(), g.float()
+        s = _lib.stream_of(a)
+        n = lib.genbmm_logbmm_stats_size(B, M, K, N)
+        st, st32 = torch.empty(n, device=gpu), torch.empty(n, device=gpu)
+        out, out32 = torch.empty(B, M, N, device=gpu, dtype=dt), torch.empty(B, M, N, device=gpu)
+        assert getattr(lib, "genbmm_logbmm_fwd" + suffix)(P(a), P(b), P(out), P(st), B, M, K, N, s) == 0
+        assert lib.genbmm_logbmm_fwd(P(a32), P(b32), P(out32), P(st32), B, M, K, N, s) == 0
+        assert torch.equal(out, out32.to(dt)), ("logbmm", B, M, K, N)
+        ga, gb = torch.empty_like(a), torch.empty_like(b)
+        ga32, gb32 = torch.empty_like(a32), torch.empty_like(b32)
+        oh = out.float()
+        assert getattr(lib, "genbmm_logbmm_bwd" + suffix)(P(a), P(b), P(out), P(g), P(st), P(ga), P(gb), B, M, K, N, s) == 0
+        assert lib.genbmm_logbmm_bwd(P(a32), P(b32), P(oh), P(g32), P(st32), P(ga32), P(gb32), B, M, K, N, s) == 0
+        assert torch.equal(ga, ga32.to(dt)) and torch.equal(gb, gb32.to(dt)), ("logbmm bwd", B, M, K, N)
+        idx, idx32 = (torch.empty(B, M, N, device=gpu, dtype=torch.int32) for _ in range(2))
+        fac, fac32 = (torch.empty(2, B, M, N, device=gpu) for _ in range(2))
+        assert getattr(lib, "genbmm_maxbmm_fwd" + suffix)(P(a), P(b), P(out), P(idx), B, M, K, N, s) == 0
+        assert lib.genbmm_maxbmm_fwd(P(a32), P(b32), P(out32), P(idx32), B, M, K, N, s) == 0
+        assert torch.equal(out, out32.to(dt)) and torch.equal(idx, idx32), ("maxbmm", B, M, K, N)
+        assert getattr(lib, "genbmm_argmax_bwd" + suffix)(P(idx), P(g), P(ga), P(gb), B, M, K, N, s) == 0
+        assert lib.genbmm_argmax_bwd(P(idx32), P(g32), P(ga32), P(gb32), B, M, K, N, s) == 0
+        assert torch.equal(ga, ga32.to(dt)) and torch.equal(gb, gb32.to(dt)), ("argmax bwd", B, M, K, N)
+        assert getattr(lib, "genbmm_prodmaxbmm_fwd" + suffix)(P(a), P(b), P(out), P(idx), P(fac), B, M, K, N, s) == 0
+        assert lib.genbmm_prodmaxbmm_fwd(P(a32), P(b32), P(out32), P(idx32), P(fac32), B, M, K, N, s) == 0
+        assert torch.equal(out, out32.to(dt)) and torch.equal(idx, idx32) and torch.equal(fac, fac32), ("prodmax", B, M, K, N)
+        assert getattr(lib, "genbmm_prodmax_bwd" + suffix)(P(None), P(None), P(idx), P(fac), P(g), P(ga), P(gb), B, M, K, N, s) == 0
+        assert lib.genbmm_prodmax_bwd(P(None), P(None), P(idx32), P(fac32), P(g32), P(ga32), P(gb32), B, M, K, N, s) == 0
+        assert torch.equal(ga, ga32.to(dt)) and torch.equal(gb, gb32.to(dt)), ("prodmax bwd", B, M, K, N)
+
+
 @pytest.mark.parametrize("dt,suffix,eps", TYPES)
 def test_logbmm_half_gradients_against_float64(gpu, dt, suffix, eps):
     """Through the autograd layer, against float64 autograd of the closed form on the same
