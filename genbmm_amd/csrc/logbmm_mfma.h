@@ -130,9 +130,15 @@ template <class E>
 __device__ __forceinline__ long ws_distance(const float* ws, const E* from) {
   return (long)(reinterpret_cast<uintptr_t>(ws) - reinterpret_cast<uintptr_t>(from) * kWiden<E>);
 }
+// (The address is handed back through a pointer typed as global memory: a pointer made from a
+// bare integer is of unknown address space, its accesses become flat_load / flat_store, and the
+// compiler drains every outstanding global load before it issues one - the slab in flight
+// under the matrix instructions would be waited for at the top of each step.)
+template <class T>
+using global_ptr = __attribute__((address_space(1))) T*;
 template <class E>
 __device__ __forceinline__ float* ws_twin(const E* p, long d) {
-  return reinterpret_cast<float*>(reinterpret_cast<uintptr_t>(p) * kWiden<E> + (uintptr_t)d);
+  return (float*)reinterpret_cast<global_ptr<float>>(reinterpret_cast<uintptr_t>(p) * kWiden<E> + (uintptr_t)d);
 }
 template <class E>
 __device__ __forceinline__ long elem_distance(const E* to, const float* ws) {
@@ -140,7 +146,7 @@ __device__ __forceinline__ long elem_distance(const E* to, const float* ws) {
 }
 template <class E>
 __device__ __forceinline__ const E* elem_twin(const float* p, long d) {
-  return reinterpret_cast<const E*>(reinterpret_cast<uintptr_t>(p) / kWiden<E> + (uintptr_t)d);
+  return (const E*)reinterpret_cast<global_ptr<const E>>(reinterpret_cast<uintptr_t>(p) / kWiden<E> + (uintptr_t)d);
 }
 __device__ __forceinline__ float4 exp4(float4 x, float4 s) {
   return make_float4(exp_st(x.x - s.x), exp_st(x.y - s.y), exp_st(x.z - s.z), exp_st(x.w - s.w));
