@@ -146,14 +146,19 @@ __global__ __launch_bounds__(256, 3) void k_log_item32_bwd(const elem_t* __restr
   elem_t* gab = grad_a ? grad_a + (long)item * E : nullptr;
   elem_t* gbb = grad_b ? grad_b + (long)item * E : nullptr;
 
-  // ---- maxima: alpha from a in rows, beta from b in columns; both to LDS
-  float a_col[16], b_col[16], al, be;
+  // ---- everything the item needs is requested at once (one trip to memory, not one per phase)
+  float a_col[16], b_col[16], g_col[16], o_col[16], al, be;
   {
     float a_row[16];
     item32_rows(ab, c, h, a_row);
+    item32_cols(bb, c, h, b_col);   // b[rho][j = c]
+    item32_cols(gb, c, h, g_col);
+    item32_cols(ob, c, h, o_col);
+    item32_cols(ab, c, h, a_col);   // a[rho][k = c]: the second read of a comes from the cache
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- maxima: alpha from a in rows, beta from b in columns; both to LDS
     al = max16(a_row);  // alpha[c]
   }
-  item32_cols(bb, c, h, b_col);   // b[rho][j = c]
   be = max16(b_col);              // beta[c]
   float* shw = sh[wave];
   if (h == 0) shw[c] = al;
@@ -169,16 +174,11 @@ __global__ __launch_bounds__(256, 3) void k_log_item32_bwd(const elem_t* __restr
   float h_col[16];
   const float lim = kItemGuardBits * kLn2 + 1e-3f;
   int bad = 0;
-  {
-    float g_col[16], o_col[16];
-    item32_cols(gb, c, h, g_col);
-    item32_cols(ob, c, h, o_col);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const float ex = al_rho[r] + be - o_col[r];
-      if (!(ex <= lim) || !(ex > -INFINITY)) bad = 1;  // S < 2^-40, NaN or infinities: not exact
-      h_col[r] = g_col[r] * fast_exp2(ex * kLog2e);
-    }
+  for (int r = 0; r < 16; ++r) {
+    const float ex = al_rho[r] + be - o_col[r];
+    if (!(ex <= lim) || !(ex > -INFINITY)) bad = 1;  // S < 2^-40, NaN or infinities: not exact
+    h_col[r] = g_col[r] * fast_exp2(ex * kLog2e);
   }
   if (__builtin_amdgcn_ballot_w64(bad != 0) != 0) {
     // the reference's form for the whole item (matmul_cuda_kernel.cu:159-184):
@@ -205,7 +205,6 @@ __global__ __launch_bounds__(256, 3) void k_log_item32_bwd(const elem_t* __restr
   }
 
   // ---- EA in columns: the factor of grad_a and the first operand of grad_b
-  item32_cols(ab, c, h, a_col);
 #pragma unroll
   for (int r = 0; r < 16; ++r) a_col[r] = item_exp(a_col[r], al_rho[r]);
 
