@@ -209,6 +209,41 @@ def test_samplebmm_half(gpu, dt, suffix, eps):
         assert ga.dtype == dt and float(ga.float().sum()) == pytest.approx(B * M * N, rel=1e-2)
 
 
+@pytest.mark.parametrize("dt,suffix,eps", TYPES)
+def test_half_tensors_at_any_two_byte_address(gpu, dt, suffix, eps):
+    """Operands, results and gradients that start one element past a 16-byte boundary (views
+    into larger buffers): the same bits as from aligned tensors, on shapes of every family."""
+    lib = _lib.load()
+    torch.manual_seed(10)
+
+    def shifted(t):   # the same values at an address that is 2 mod 16
+        buf = torch.empty(t.numel() + 9, device=gpu, dtype=dt)
+        v = buf[1:1 + t.numel()].view(t.shape)
+        v.copy_(t)
+        assert v.data_ptr() % 16 == 2
+        return v
+
+    for B, M, K, N in [(3, 32, 32, 32), (2, 40, 24, 36), (2, 128, 128, 128), (2, 100, 96, 120), (2, 256, 128, 256),
+                       (1, 129, 77, 131)]:
+        a, b, g = _operands(gpu, dt, B, M, K, N)
+        s = _lib.stream_of(a)
+        n = lib.genbmm_logbmm_stats_size(B, M, K, N)
+        res = []
+        for move in (lambda t: t, shifted):
+            x, y, gg = move(a), move(b), move(g)
+            st = torch.empty(n, device=gpu)
+            out, ga, gb = move(torch.zeros(B, M, N, device=gpu, dtype=dt)), move(torch.zeros_like(a)), move(torch.zeros_like(b))
+            assert getattr(lib, "genbmm_logbmm_fwd" + suffix)(P(x), P(y), P(out), P(st), B, M, K, N, s) == 0
+            assert getattr(lib, "genbmm_logbmm_bwd" + suffix)(P(x), P(y), P(out), P(gg), P(st), P(ga), P(gb), B, M, K, N, s) == 0
+            mo, idx = move(torch.zeros(B, M, N, device=gpu, dtype=dt)), torch.empty(B, M, N, device=gpu, dtype=torch.int32)
+            assert getattr(lib, "genbmm_maxbmm_fwd" + suffix)(P(x), P(y), P(mo), P(idx), B, M, K, N, s) == 0
+            ma, mb = move(torch.zeros_like(a)), move(torch.zeros_like(b))
+            assert getattr(lib, "genbmm_argmax_bwd" + suffix)(P(idx), P(gg), P(ma), P(mb), B, M, K, N, s) == 0
+            res.append([t.clone() for t in (out, ga, gb, mo, idx, ma, mb)])
+        for u, v in zip(*res):
+            assert torch.equal(u, v), (B, M, K, N)
+
+
 def test_half_masks_and_empty(gpu):
     """-inf masks, rows without mass, the reference's -1e9 floor (which is -inf in
     binary16, as `scalar_t m = -1e9` is in the reference) and empty extents."""
