@@ -312,8 +312,15 @@ class BandedMatrix:
         ld = self.ld + other.lu
         # views are copied here, by a differentiable torch operation, so that the
         # Functions save (and differentiate with respect to) what they were given
-        out = fn(self.data.contiguous(), self.lu, self.ld, other.data.contiguous(), other.lu, other.ld,
-                 lu, ld)
+        a, b = self.data, other.data
+        # float16 / bfloat16 bands are widened for the kernels and the result narrowed again (the
+        # banded entry points exist for float and double); the casts are differentiable
+        half = a.dtype if a.dtype in (torch.float16, torch.bfloat16) and b.dtype == a.dtype else None
+        if half is not None:
+            a, b = a.float(), b.float()
+        out = fn(a.contiguous(), self.lu, self.ld, b.contiguous(), other.lu, other.ld, lu, ld)
+        if half is not None:
+            out = out.to(half)
         return BandedMatrix(out, lu, ld, self.fill)
 
     def multiply(self, other):

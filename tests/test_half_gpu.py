@@ -266,3 +266,22 @@ def test_half_masks_and_empty(gpu):
         e = genbmm.maxbmm(torch.randn(2, 3, 0, device=gpu).to(dt), torch.randn(2, 0, 5, device=gpu).to(dt))
         floor = torch.full(e.shape, -1e9, device=gpu).to(dt)   # rounded to the type (-inf in binary16)
         assert torch.equal(e, floor)
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_banded_products_on_half_bands(gpu, dt):
+    """BandedMatrix widens half bands for the banded kernels and narrows the result: the float
+    product of the widened bands, rounded once; gradients arrive in the half tensors."""
+    from genbmm_amd.sparse import BandedMatrix, banddiag
+    torch.manual_seed(11)
+    n, (alu, ald, blu, bld) = 70, (5, 3, 2, 6)
+    x = banddiag(torch.randn(2, n, n), alu, ald)[0].contiguous().to(gpu).to(dt)
+    y = banddiag(torch.randn(2, n, n), blu, bld)[0].contiguous().to(gpu).to(dt)
+    for name in ("multiply", "multiply_log", "multiply_max"):
+        xh, yh = x.clone().requires_grad_(True), y.clone().requires_grad_(True)
+        got = getattr(BandedMatrix(xh, alu, ald), name)(BandedMatrix(yh, blu, bld))
+        want = getattr(BandedMatrix(x.float(), alu, ald), name)(BandedMatrix(y.float(), blu, bld))
+        assert got.data.dtype == dt and (got.lu, got.ld) == (want.lu, want.ld)
+        assert torch.equal(got.data, want.data.to(dt)), name
+        ga, gb = torch.autograd.grad(got.data.float().sum(), (xh, yh))
+        assert ga.dtype == dt and gb.dtype == dt and float(ga.float().abs().sum()) > 0
