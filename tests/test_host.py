@@ -133,6 +133,36 @@ def test_library_exports_every_declared_symbol():
     assert lib.genbmm_error_string(-2) == b"a dimension is negative or too large"
 
 
+def test_half_builds_compute_in_float():
+    """The float16 / bfloat16 builds of the dense sources widen on load and narrow on store
+    and do nothing else in the narrow type: their device code (LLVM IR) holds no arithmetic,
+    comparison or min / max on half or bfloat values, scalar or vector."""
+    import shutil
+    import subprocess
+    from concurrent.futures import ThreadPoolExecutor
+    from genbmm_amd import build as hip_build
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not present")
+    jobs = [(src, elem) for src, variants in hip_build.PER_ELEMENT.items() for _, elem in variants if elem]
+    assert len(jobs) == 6
+
+    def ir(job):
+        src, elem = job
+        cmd = [hipcc, "-O1", "-std=c++17", "--offload-arch=gfx950", "-ffp-contract=on", "-fno-gpu-rdc",
+               "-DGENBMM_ELEM=%d" % elem, "-S", "-emit-llvm", "--cuda-device-only", "-o", "-",
+               os.path.join(hip_build.CSRC, src)]
+        return subprocess.run(cmd, check=True, capture_output=True, text=True).stdout
+
+    narrow = re.compile(r"= (fadd|fsub|fmul|fdiv|frem|fneg|fcmp \w+) [^\n]*?(<\d+ x )?(half|bfloat)\b"
+                        r"|call [^\n]*llvm\.(maxnum|minnum|fma|fmuladd|maximum|minimum)\.(v\d+)?(f16|bf16)")
+    with ThreadPoolExecutor(max_workers=6) as pool:
+        for job, text in zip(jobs, pool.map(ir, jobs)):
+            assert "define" in text and ("half" in text or "bfloat" in text), job
+            hits = [m.group(0) for m in narrow.finditer(text)]
+            assert not hits, (job, hits[:3])
+
+
 def test_no_cpu_fallback():
     a, b = torch.randn(2, 3, 4), torch.randn(2, 4, 5)
     for op in (genbmm_amd.logbmm, genbmm_amd.maxbmm, genbmm_amd.samplebmm, genbmm_amd.prodmaxbmm):
