@@ -61,7 +61,7 @@ namespace GENBMM_NS {
 
 constexpr int kDirFwd = 0, kDirGradA = 1, kDirGradB = 2;
 constexpr int kDirTiles = 16;   // tiles per tile row, at most (a bit per cell in 64 bits)
-constexpr int kDirChunks = 12;  // chunks of the first operand per tile row, at most
+constexpr int kDirChunks = 15;  // chunks of the first operand per tile row, at most (4 bits of a step word, one value for the chunk of zeros)
 constexpr int kDirDepth = 4;    // pairs whose loads of Q are in flight
 constexpr int kDirWaves = 2;    // waves (tile rows) per workgroup
 constexpr int kDirMargin = 48;  // floats a load can stray from the band rows it is meant for
@@ -78,7 +78,7 @@ typedef float dir_f4u __attribute__((ext_vector_type(4), aligned(4)));
 // (D: chunk minus tile, or tile minus chunk for an operand whose band row is k; a lane's
 // cell t of Q is Wq - 1 + 16 D + s_t with s_t in [-15, 15]), and beside it the word of
 // the step kDirDepth further on, whose cells of Q are asked for now.
-constexpr int kDirSteps = 72;
+constexpr int kDirSteps = 176;
 struct DirStep {
   unsigned now, ahead;
 };

@@ -13,7 +13,9 @@ pytestmark = pytest.mark.gpu
 # (n, a_lu, a_ld, b_lu, b_ld): bands narrower and wider than the matrix, empty sides
 BANDS = [(5, 1, 1, 2, 0), (6, 2, 1, 1, 3), (4, 3, 3, 3, 3), (7, 0, 2, 2, 0), (3, 4, 5, 5, 4),
          (40, 3, 5, 4, 2), (33, 0, 0, 0, 0), (64, 8, 8, 8, 8), (1, 0, 0, 0, 0), (130, 17, 2, 5, 20),
-         (257, 32, 32, 32, 32), (100, 60, 50, 40, 70)]
+         (257, 32, 32, 32, 32), (100, 60, 50, 40, 70),
+         # 97 and 102 / 101 diagonals: the widest bands the memory-fed matrix-core kernels take
+         (300, 48, 48, 48, 48), (260, 52, 49, 50, 50), (230, 64, 64, 64, 64)]
 
 
 def close(x, ref, rtol=1e-5, atol=1e-5):
