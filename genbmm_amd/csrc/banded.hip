@@ -122,12 +122,15 @@ inline void launch_dir(const BandArgs& p, int B, hipStream_t s) {
   DirPlan plan;
   dir_plan(plan, KIND, p.a_lu, p.Wa, p.b_lu, p.Wb);
   const int wave_lds = dir_wave_lds(plan, KIND, PREP);
-  auto kern = k_band_dir<KIND, PREP>;
-  if ((size_t)kDirWaves * wave_lds > kStripLdsLimit)
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              kDirWaves * wave_lds);
-  hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64 * kDirWaves), kDirWaves * wave_lds, s, p, plan, blocks,
-                     nblocks, (long)B * p.n, wave_lds);
+  auto go = [&](auto kern, const auto& table) {
+    if ((size_t)kDirWaves * wave_lds > kStripLdsLimit)
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kDirWaves * wave_lds);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64 * kDirWaves), kDirWaves * wave_lds, s, p, table,
+                       blocks, nblocks, (long)B * p.n, wave_lds);
+  };
+  if (plan.steps <= kDirStepsSmall) go(k_band_dir<KIND, PREP, DirPlanSmall>, dir_plan_small(plan));
+  else go(k_band_dir<KIND, PREP, DirPlan>, plan);
 }
 
 inline void set_workspace(BandArgs& p, float* ws, int B) {

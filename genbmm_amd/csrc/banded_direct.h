@@ -60,37 +60,55 @@
 namespace GENBMM_NS {
 
 constexpr int kDirFwd = 0, kDirGradA = 1, kDirGradB = 2;
-constexpr int kDirTiles = 16;   // tiles per tile row, at most (a bit per cell in 64 bits)
-constexpr int kDirChunks = 15;  // chunks of the first operand per tile row, at most (4 bits of a step word, one value for the chunk of zeros)
+constexpr int kDirTiles = 32;   // tiles per tile row, at most (5 bits of a step word; a bit per cell in 128 bits)
+constexpr int kDirChunks = 30;  // chunks of the first operand per tile row, at most (5 bits, one value for the chunk of zeros)
 constexpr int kDirDepth = 4;    // pairs whose loads of Q are in flight
 constexpr int kDirWaves = 2;    // waves (tile rows) per workgroup
 constexpr int kDirMargin = 48;  // floats a load can stray from the band rows it is meant for
 typedef float dir_f4u __attribute__((ext_vector_type(4), aligned(4)));
 
 // The walk over a tile row's (tile, chunk) pairs.  One word per step:
-//   bits 0-11  where the pair's cells of Q start, in units of 16 floats
-//   bits 12-15 chunk of P (the one past the last holds zeros)
-//   bits 16-19 tile      bit 20  the tile is complete after this step
-//   bit 21  some lane's cells of Q lie past the upper end of its band (D = 0)
-//   bit 22 / 23  ... below the lower end: D is the plan's lowest / the one above it
-//   bit 24  a filling step (nothing to multiply)
-//   bit 25  every cell of the tile is inside the result band
+//   bits 0-12  where the pair's cells of Q start, in units of 16 floats
+//   bits 13-17 chunk of P (the one past the last holds zeros)
+//   bits 18-22 tile      bit 23  the tile is complete after this step
+//   bit 24  some lane's cells of Q lie past the upper end of its band (D = 0)
+//   bit 25 / 26  ... below the lower end: D is the plan's lowest / the one above it
+//   bit 27  a filling step (nothing to multiply)
+//   bit 28  every cell of the tile is inside the result band
 // (D: chunk minus tile, or tile minus chunk for an operand whose band row is k; a lane's
 // cell t of Q is Wq - 1 + 16 D + s_t with s_t in [-15, 15]), and beside it the word of
 // the step kDirDepth further on, whose cells of Q are asked for now.
-constexpr int kDirSteps = 176;
+constexpr int kDirSteps = 400;  // of a tile row (the table travels as a kernel argument: 3.2 KB)
+constexpr unsigned kDirQMask = 0x1fffu;
+constexpr int kDirChunkShift = 13, kDirTileShift = 18;
+constexpr unsigned kDirDone = 1u << 23, kDirPastHi = 1u << 24, kDirBelowLo0 = 1u << 25, kDirBelowLo1 = 1u << 26,
+                   kDirFill = 1u << 27, kDirWhole = 1u << 28;
+constexpr size_t kDirLdsLimit = 160 * 1024;  // of a workgroup (one compute unit's LDS)
 struct DirStep {
   unsigned now, ahead;
 };
-struct DirPlan {
+// (CAP: steps the table has room for.  Narrow bands travel in the small form - a kernel
+// argument of 3 KB costs every launch a few microseconds.)
+constexpr int kDirStepsSmall = 88;
+template <int CAP>
+struct DirPlanT {
   int steps;  // a multiple of kDirDepth
   int d_lo;   // the lowest D of the plan
   int Wp, Wq, Wout;
   int plo, phi;  // P(i, k) is inside its band for k in [i - plo, i + phi]
   int lu_out;    // out[i][j - i + lu_out]
   int NU, nt;    // chunks of P, tiles per tile row
-  DirStep e[kDirSteps + 1];
+  DirStep e[CAP + 1];
 };
+using DirPlan = DirPlanT<kDirSteps>;
+using DirPlanSmall = DirPlanT<kDirStepsSmall>;
+inline DirPlanSmall dir_plan_small(const DirPlan& g) {  // g.steps <= kDirStepsSmall
+  DirPlanSmall r;
+  r.steps = g.steps; r.d_lo = g.d_lo; r.Wp = g.Wp; r.Wq = g.Wq; r.Wout = g.Wout;
+  r.plo = g.plo; r.phi = g.phi; r.lu_out = g.lu_out; r.NU = g.NU; r.nt = g.nt;
+  for (int i = 0; i <= g.steps; ++i) r.e[i] = g.e[i];
+  return r;
+}
 
 inline int dir_chunks(int Wp) { return (Wp + 30) >> 4; }  // chunks of 16 k that a tile row's P meets
 // LDS of one wave: its chunks of P and one of zeros, 1 KB each; then the row maxima of b for
@@ -113,7 +131,8 @@ inline bool dir_plan(DirPlan& g, int kind, int a_lu, int Wa, int b_lu, int Wb) {
   }
   const bool qrow = kind != kDirFwd;
   const int NU = g.NU = dir_chunks(g.Wp), nt = g.nt = (g.Wout + 30) >> 4;
-  if (NU > kDirChunks || nt > kDirTiles || max(NU, nt) * g.Wq >= 4096) return false;
+  if (NU > kDirChunks || nt > kDirTiles || max(NU, nt) * g.Wq > (int)kDirQMask) return false;
+  if ((size_t)kDirWaves * dir_wave_lds(g, kDirFwd, true) > kDirLdsLimit) return false;
   unsigned list[kDirTiles * kDirChunks];
   int np = 0, d_lo = 0;
   for (int pass = 0; pass < 2; ++pass) {
@@ -138,8 +157,9 @@ inline bool dir_plan(DirPlan& g, int kind, int a_lu, int Wa, int b_lu, int Wb) {
         if (d > 0 || (lo && d > d_lo + 1)) return false;
         const unsigned whole = 16 * tj - 15 >= 0 && 16 * tj + 15 < g.Wout;
         const int q16 = qrow ? u * (g.Wq - 1) + tj : tj * (g.Wq - 1) + u;
-        list[np++] = (unsigned)q16 | (unsigned)u << 12 | (unsigned)tj << 16 | (unsigned)(u == uhi) << 20 | hi << 21 |
-                     (unsigned)(lo && d == d_lo) << 22 | (unsigned)(lo && d == d_lo + 1) << 23 | whole << 25;
+        list[np++] = (unsigned)q16 | (unsigned)u << kDirChunkShift | (unsigned)tj << kDirTileShift |
+                     (u == uhi ? kDirDone : 0u) | (hi ? kDirPastHi : 0u) | (lo && d == d_lo ? kDirBelowLo0 : 0u) |
+                     (lo && d == d_lo + 1 ? kDirBelowLo1 : 0u) | (whole ? kDirWhole : 0u);
       }
     }
   }
@@ -147,7 +167,7 @@ inline bool dir_plan(DirPlan& g, int kind, int a_lu, int Wa, int b_lu, int Wb) {
   const int pad = (kDirDepth - (np & (kDirDepth - 1))) & (kDirDepth - 1);
   if (np + pad > kDirSteps) return false;
   g.steps = np + pad;
-  for (int i = 0; i < pad; ++i) g.e[i].now = (list[0] & 0xfffu) | (unsigned)NU << 12 | 1u << 24;
+  for (int i = 0; i < pad; ++i) g.e[i].now = (list[0] & kDirQMask) | (unsigned)NU << kDirChunkShift | kDirFill;
   for (int i = 0; i < np; ++i) g.e[pad + i].now = list[i];
   g.e[g.steps].now = g.e[g.steps - 1].now;
   for (int i = 0; i <= g.steps; ++i) g.e[i].ahead = g.e[min(i + kDirDepth, g.steps - 1)].now;
@@ -155,8 +175,8 @@ inline bool dir_plan(DirPlan& g, int kind, int a_lu, int Wa, int b_lu, int Wb) {
 }
 
 // One tile row.  All arguments but `lane` are uniform.  lds: this wave's piece.
-template <int KIND, bool PREP, bool EDGE>
-__device__ __forceinline__ void dir_row(const BandArgs& p, const DirPlan& g, long bn, int i0, int lane, float* lds,
+template <int KIND, bool PREP, bool EDGE, class Plan>
+__device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long bn, int i0, int lane, float* lds,
                                         long rows) {
   constexpr bool FWD = KIND == kDirFwd, GA = KIND == kDirGradA;
   constexpr bool PROW = KIND == kDirGradB;  // P's band row is k
@@ -197,7 +217,7 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const DirPlan& g, lon
     qoff[t] = QROW ? (K0 + 4 * zq + t) * (Wq - 1) + J0 + l15 + (Wq - 1 - g.plo + g.lu_out)  // k (Wq - 1) + j + lu_q
                    : (J0 + lr) * Wq + Wq - 1 + s0 + t;
   auto issue = [&](unsigned e, mm_f4& q) __attribute__((always_inline)) {
-    const int soff = 16 * (int)(e & 0xfffu);  // uniform
+    const int soff = 16 * (int)(e & kDirQMask);  // uniform
     if (QROW || EDGE) {
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
@@ -299,7 +319,7 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const DirPlan& g, lon
   // the cell belongs to a neighbouring band row.)
   auto mask = [&](unsigned e, mm_f4& x) __attribute__((always_inline)) {
     if (EDGE) {
-      const int tj = (e >> 16) & 15u, u = (e >> 12) & 15u;
+      const int tj = (e >> kDirTileShift) & 31u, u = (e >> kDirChunkShift) & 31u;
       const int D = QROW ? tj - u : u - tj;
       const int j = J0 + 16 * tj + (QROW ? l15 : lr);
       const int k = K0 + 16 * u + (QROW ? 4 * zq : 4 * lc);
@@ -310,17 +330,17 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const DirPlan& g, lon
         x[t] = ok ? x[t] : 0.f;
       }
     } else {
-      if (e & (1u << 21)) {  // uniform
+      if (e & kDirPastHi) {  // uniform
         asm volatile("" ::: "memory");  // keeps this a branch: most steps have nothing to mask
 #pragma unroll
         for (int t = 0; t < 4; ++t) x[t] *= m_hi[t];
       }
-      if (e & (1u << 22)) {  // uniform
+      if (e & kDirBelowLo0) {  // uniform
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int t = 0; t < 4; ++t) x[t] *= m_lo0[t];
       }
-      if (e & (1u << 23)) {  // uniform
+      if (e & kDirBelowLo1) {  // uniform
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int t = 0; t < 4; ++t) x[t] *= m_lo1[t];
@@ -367,7 +387,7 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const DirPlan& g, lon
   const bool y_all = J0 >= 0 && J0 + 16 * nt - 1 < n;  // every column of every tile inside the matrix
   // cells to recompute: the forward of the log product keeps a bit per cell (bit 4 tj + r), the
   // others one flag per lane (all the lane's cells are then done again)
-  unsigned long long redo = 0;
+  unsigned __int128 redo = 0;
   float worst = 0.f;  // stays 0 while every sum is finite
   // Tile rows away from the edges collect their 16 x Wout results in LDS (aux) and write
   // them as one contiguous run of memory; the forward of the log product collects its sums S
@@ -375,12 +395,12 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const DirPlan& g, lon
   // LDS, measured 10 % slower than no staging at all).
   const bool plain_rows = STAGE && y_all;
   auto finish = [&](unsigned e, const mm_f4& c) __attribute__((always_inline)) {
-    const int tj = (e >> 16) & 15u;
+    const int tj = (e >> kDirTileShift) & 31u;
     if (plain_rows) {  // uniform: nothing to test but the values
       const float s = (c[0] + c[1]) + (c[2] + c[3]);  // not finite if a cell is not (or the sum overflows: no harm)
       worst = __builtin_fmaf(s, 0.f, worst);          // 0 * s is NaN exactly when s is not finite
       float* st = aux + 16 * tj;
-      if (e & (1u << 25)) {
+      if (e & kDirWhole) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) st[ooff[r]] = c[r];
       } else {
@@ -392,7 +412,7 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const DirPlan& g, lon
       }
       return;
     }
-    const bool whole = (e & (1u << 25)) && !tail;
+    const bool whole = (e & kDirWhole) && !tail;
     const int y = J0 + 16 * tj + l15;
     const bool y_in = y_all || (unsigned)y < (unsigned)n;
     float* ot = (STAGE ? aux : orow) + 16 * tj;
@@ -421,7 +441,7 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const DirPlan& g, lon
         ot[ooff[r]] = v;
       }
     }
-    if (FWD && PREP) redo |= (unsigned long long)bits << (4 * tj);
+    if (FWD && PREP) redo |= (unsigned __int128)bits << (4 * tj);
   };
 
   // ---- the walk: the loads of Q run kDirDepth steps ahead (past the end they repeat the
@@ -437,13 +457,13 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const DirPlan& g, lon
       const unsigned e = cur.now;
       mask(e, qraw[s]);
       const mm_f4 qv = to_mfma(qraw[s]);
-      const mm_f4 pv = pl[64 * ((e >> 12) & 15u)];
+      const mm_f4 pv = pl[64 * ((e >> kDirChunkShift) & 31u)];
       issue(cur.ahead, qraw[s]);
-      if (!(e & (1u << 24))) {  // uniform: not one of the filling steps
+      if (!(e & kDirFill)) {  // uniform: not one of the filling steps
 #pragma unroll
         for (int t = 0; t < 4; ++t) c = __builtin_amdgcn_mfma_f32_16x16x4f32(pv[t], qv[t], c, 0, 0, 0);
       }
-      if (e & (1u << 20)) {  // uniform: the tile is complete
+      if (e & kDirDone) {  // uniform: the tile is complete
         finish(e, c);
         c = mm_f4{0.f, 0.f, 0.f, 0.f};
       }
@@ -512,9 +532,10 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const DirPlan& g, lon
   if (!(FWD && PREP) && !(worst == 0.f)) redo = 1;
   if (__builtin_amdgcn_ballot_w64(redo != 0) != 0) {
     if (STAGE) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // the run above was written by other lanes
-    if (!(FWD && PREP) && redo) redo = ~0ull;
+    if (!(FWD && PREP) && redo) redo = ~(unsigned __int128)0;
     while (redo) {
-      const int bit = __builtin_ctzll(redo);
+      const unsigned long long half = (unsigned long long)redo;
+      const int bit = half ? __builtin_ctzll(half) : 64 + __builtin_ctzll((unsigned long long)(redo >> 64));
       redo &= redo - 1;
       const int tj = bit >> 2, r = bit & 3;
       const int i = i0 + 4 * zq + r, jj = 16 * tj + l15 - 4 * zq - r;
@@ -536,8 +557,8 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const DirPlan& g, lon
 
 // One wave per tile row, kDirWaves tile rows per workgroup.  blocks: workgroups per batch item;
 // wave_lds: bytes of LDS per wave; rows: band rows of every tensor (batch * n).
-template <int KIND, bool PREP>
-__global__ __launch_bounds__(64 * kDirWaves) void k_band_dir(const BandArgs p, const DirPlan g, int blocks, int nblocks,
+template <int KIND, bool PREP, class Plan>
+__global__ __launch_bounds__(64 * kDirWaves) void k_band_dir(const BandArgs p, const Plan g, int blocks, int nblocks,
                                                             long rows, int wave_lds) {
   extern __shared__ __attribute__((aligned(16))) float dir_smem[];
   const int lane = threadIdx.x & 63;
