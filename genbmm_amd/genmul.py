@@ -301,9 +301,33 @@ class SampleMatMul(torch.autograd.Function):
         return _argmax_backward(ctx, grad_output, prod=False) + (None,)
 
 
+def _reduction_splits(B, M, K, N):
+    """How many pieces to cut the reduction axis into.  The kernels give every output tile to one
+    workgroup that walks all of K: a problem with few tiles and a long K would run on a few
+    of the 256 compute units.  Such a problem is cut into S pieces of K (S divides K), each a
+    batch item of its own; the pieces are joined by a logsumexp over S."""
+    tiles = B * ((M + 127) // 128) * ((N + 127) // 128)
+    # (from K = 4096 on: below, the extra launches of the split cost what it saves)
+    if tiles >= 128 or K < 4096 or M * N == 0:
+        return 1
+    want = min(K // 256, (255 + tiles) // tiles)
+    for s in range(want, 1, -1):
+        if K % s == 0:
+            return s
+    return 1
+
+
 def logbmm(a, b):
     """genbmm.logbmm(a, b): out[..., m, n] = logsumexp_k(a[..., m, k] + b[..., k, n])."""
     a, b, restore = _canonical(a, b)
+    B, M, K = a.shape
+    N = b.shape[2]
+    S = 1 if _f64(a) else _reduction_splits(B, M, K, N)
+    if S > 1:  # differentiable torch operations around the same kernels (any order of derivative)
+        a_s = a.view(B, M, S, K // S).transpose(1, 2).reshape(B * S, M, K // S).contiguous()
+        b_s = b.view(B * S, K // S, N)
+        parts = LogMatMul.apply(a_s, b_s, PATH_AUTO).view(B, S, M, N)
+        return restore(torch.logsumexp(parts.float(), dim=1).to(a.dtype))
     return restore(LogMatMul.apply(a, b, PATH_AUTO))
 
 

@@ -744,6 +744,30 @@ def test_views_and_batch_dimensions(gpu):
     close(genbmm.logbmm(a2.to(gpu), b2.to(gpu)), lse64(a2[None], b2[None])[0])
 
 
+@pytest.mark.parametrize("B,M,K,N", [(2, 40, 4096, 30), (1, 7, 8192, 5), (1, 100, 4608, 96), (1, 16, 6000, 16)])
+def test_long_reductions_with_few_tiles_are_split(gpu, B, M, K, N):
+    """logbmm cuts a long reduction axis of a problem with few output tiles into batch items of
+    its own and joins them by a logsumexp (host layer): same values, first and second
+    derivatives as the float64 closed form.  (6000 = 2^4 * 3 * 5^3: the cut takes a divisor.)"""
+    assert genmul._reduction_splits(B, M, K, N) > 1
+    assert genmul._reduction_splits(64, 512, 512, 512) == 1 and genmul._reduction_splits(512, 128, 128, 128) == 1
+    torch.manual_seed(K + M)
+    a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
+    want, wa, wb = oracle.logbmm_grads64(a, b, g)
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    out = genbmm.logbmm(ad, bd)
+    close(out, want)
+    ga, gb = torch.autograd.grad(out, (ad, bd), g.to(gpu), create_graph=True)
+    close(ga, wa)
+    close(gb, wb)
+    if B * M * K * N <= 3_000_000:
+        u = torch.randn(B, M, K)
+        w2 = oracle.logbmm_second_order64(a, b, g, u, None)
+        da, db = torch.autograd.grad((ga * u.to(gpu)).sum(), (ad, bd))
+        close(da, w2[0], rtol=1e-4, atol=1e-5)
+        close(db, w2[1], rtol=1e-4, atol=1e-5)
+
+
 def test_half_inputs_are_twice_differentiable(gpu):
     """float16 / bfloat16 operands stay in their type through forward and backward; the
     double backward widens what the first backward saved, so second-order terms reach the
