@@ -86,21 +86,33 @@ inline bool prep_fwd(const BandArgs& p, int mode, const float* workspace) {
 // The whole-strip max-plus forward: from 8 diagonals on (measured at 64 x 4096: 9 diagonals
 // 0.035 ms against 0.042, 17: 0.046 against 0.126, 65: 0.29 against 0.36; 5: 0.031 against
 // 0.015 for one lane per cell), bands whose tiles fit two workgroups per compute unit.
-inline bool max_fwd_ok(const BandArgs& p) {
-  return min(p.Wa, p.Wb) >= 8 && p.Wo <= 160 && max_dims(p.Wa, p.Wb, p.Wo).bytes <= kMmLdsLimit;
+// Diagonals per workgroup: the whole result while it has at most 160 diagonals and its tiles
+// fit two workgroups per compute unit; otherwise the widest segment (a multiple of 8) whose
+// tiles fit - two workgroups per compute unit if possible, else one.  0: none fits.
+inline int max_fwd_segment(const BandArgs& p) {
+  if (min(p.Wa, p.Wb) < 8) return 0;
+  if (p.Wo <= 160 && max_dims(p.Wa, p.Wb, p.Wo).bytes <= kMmLdsLimit) return p.Wo;
+  // just past that the chunked strip kernel is the faster one (81 diagonals per operand at
+  // 16 x 4096: 0.14 ms against 0.23 in two segments); segments take over where it ends
+  if (fwd_strip_ok(p)) return 0;
+  for (size_t limit : {kMmLdsLimit, (size_t)160 * 1024})
+    for (int w = min(160, p.Wo & ~7); w >= 16; w -= 8)
+      if (max_dims(p.Wa, p.Wb, w).bytes <= limit) return w;
+  return 0;
 }
+inline bool max_fwd_ok(const BandArgs& p) { return max_fwd_segment(p) > 0; }
 inline void launch_max_fwd(const BandArgs& p, int B, hipStream_t s) {
-  const MaxDims d = max_dims(p.Wa, p.Wb, p.Wo);
+  const int Wseg = max_fwd_segment(p), nseg = ceil_div(p.Wo, Wseg);
+  const MaxDims d = max_dims(p.Wa, p.Wb, Wseg);
   const int strips = ceil_div(p.n, kMaxRows);
   if (d.bytes > kStripLdsLimit)
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_band_max_fwd),
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)d.bytes);
   const long rows = (long)B * p.n;
-  hipLaunchKernelGGL(k_band_max_fwd, dim3((unsigned)((long)B * strips)), dim3(256), d.bytes, s, p, strips, d,
-                     rows * p.Wa, rows * p.Wb);
+  hipLaunchKernelGGL(k_band_max_fwd, dim3((unsigned)((long)B * strips * nseg)), dim3(256), d.bytes, s, p, strips, d,
+                     rows * p.Wa, rows * p.Wb, nseg, Wseg);
 }
 
-// EA, alpha and EB, beta of a log product into the workspace set_workspace() has laid out.
 inline void launch_prep(const BandArgs& p, const float* a, int a_lu, const float* b, int b_lu, int B,
                         hipStream_t s) {
   const long rows = (long)B * p.n;
@@ -301,11 +313,18 @@ int banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int
     }
   }
   if (mode == GENBMM_BAND_MAX &&
-      max(argmax_bwd_a_bytes(p.Wa), argmax_bwd_b_bytes(p.Wb)) <= kStripLdsLimit) {
+      max(argmax_bwd_a_bytes(p.Wa), argmax_bwd_b_bytes(p.Wb)) <= kDirLdsLimit) {  // a compute unit's LDS
     const int strips = ceil_div(n, kAT);
     const dim3 grid((unsigned)((long)B * strips));
-    hipLaunchKernelGGL(k_band_argmax_bwd_a, grid, dim3(256), argmax_bwd_a_bytes(p.Wa), s, p, strips);
-    hipLaunchKernelGGL(k_band_argmax_bwd_b, grid, dim3(256), argmax_bwd_b_bytes(p.Wb), s, p, strips);
+    const size_t na = argmax_bwd_a_bytes(p.Wa), nb = argmax_bwd_b_bytes(p.Wb);
+    if (na > kStripLdsLimit)
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_band_argmax_bwd_a),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)na);
+    if (nb > kStripLdsLimit)
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_band_argmax_bwd_b),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)nb);
+    hipLaunchKernelGGL(k_band_argmax_bwd_a, grid, dim3(256), na, s, p, strips);
+    hipLaunchKernelGGL(k_band_argmax_bwd_b, grid, dim3(256), nb, s, p, strips);
     return launch_status();
   }
   if (mode == GENBMM_BAND_LOG) {

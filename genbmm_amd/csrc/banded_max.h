@@ -15,6 +15,10 @@
 //
 // Compared with the chunked strip kernel (banded_strip.h) the sliding operand is staged
 // once instead of once per 32 diagonals, and the result leaves in 16-byte stores.
+//
+// Wide results are cut into segments of Wseg <= 160 adjacent diagonals, one workgroup per strip
+// and segment: a segment needs only the 64 + Wseg - 1 rows of b that its diagonals meet, so the
+// tiles fit in LDS whatever the band width; its cells leave as one run of Wseg per row.
 #pragma once
 
 #include "banded_flat.h"
@@ -28,6 +32,7 @@ struct MaxDims {
   size_t bytes;
 };
 
+// Wo: the diagonals one workgroup takes (the whole result or a segment of it)
 inline MaxDims max_dims(int Wa, int Wb, int Wo) {
   MaxDims d;
   d.pp = Wa | 1;
@@ -43,19 +48,22 @@ inline MaxDims max_dims(int Wa, int Wb, int Wo) {
 }
 
 __global__ __launch_bounds__(256, 2) void k_band_max_fwd(const BandArgs p, int strips, const MaxDims d,
-                                                         long cells_a, long cells_b) {
+                                                         long cells_a, long cells_b, int nseg, int Wseg) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wg = xcd_strip_id();
+  int wg = xcd_strip_id();
+  const int seg = wg % nseg;  // the segments of a strip run side by side: they share its rows of a
+  wg /= nseg;
   const int batch = wg / strips, x0 = (wg - batch * strips) * kMaxRows;
   const int n = p.n, Wa = p.Wa, Wb = p.Wb, Wo = p.Wo, r_lu = p.r_lu;
+  const int j_lo = seg * Wseg, Ws = min(Wseg, Wo - j_lo);  // this workgroup's diagonals [j_lo, j_lo + Ws)
   const long bn = (long)batch * n;
   float* PL = smem + kMmSlack;
   float* QL = smem + d.q_off;
 
   // ---- staging
-  const int q0 = x0 - r_lu;
+  const int q0 = x0 - r_lu + j_lo;  // first row of b that the segment's cells meet
   const int qr0 = max(q0, 0), qr1 = min(q0 + d.q_rows, n);
   const int pr1 = min(x0 + kMaxRows, n);
   MmFlat<14> sq;
@@ -92,8 +100,8 @@ __global__ __launch_bounds__(256, 2) void k_band_max_fwd(const BandArgs p, int s
   // every row of the strip is inside the matrix with its whole band, and so is every b row
   const bool interior = x0 >= max(p.a_lu, r_lu) && x0 + kMaxRows - 1 <= n - 1 - max(Wa - 1 - p.a_lu, Wo - 1 - r_lu);
   const float* ap = Pt + lane * pp;
-  const int nblocks = (Wo + 7) >> 3;
-  float val[5][8];  // blocks wave, wave + 4, ...: at most 5 of them (Wo <= 160)
+  const int nblocks = (Ws + 7) >> 3;
+  float val[5][8];  // blocks wave, wave + 4, ...: at most 5 of them (Ws <= 160)
   int ind[5][8];
 #pragma unroll
   for (int s = 0; s < 5; ++s) {
@@ -104,9 +112,9 @@ __global__ __launch_bounds__(256, 2) void k_band_max_fwd(const BandArgs p, int s
     }
     const int jb = wave + 4 * s;
     if (jb < nblocks) {
-      const int j0 = 8 * jb;
-      // b[o][k2] of cell t at step k: Qt[(lane + j0 + t) * qp + k - j0 - t + Wb - 1]
-      const float* bp = Qt + (lane + j0) * qp + (Wb - 1 - j0);
+      const int j0 = j_lo + 8 * jb;
+      // b[o][k2] of cell t at step k: Qt[(lane + j0 - j_lo + t) * qp + k - j0 - t + Wb - 1]
+      const float* bp = Qt + (lane + j0 - j_lo) * qp + (Wb - 1 - j0);
       const int dt = qp - 1;
       auto fold = [&](int t, float av, float bv, int k) __attribute__((always_inline)) {
         const float v = av + bv;
@@ -143,7 +151,7 @@ __global__ __launch_bounds__(256, 2) void k_band_max_fwd(const BandArgs p, int s
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
           const int j = j0 + t, o = x + j - r_lu;
-          if (j < Wo && o >= 0 && o < n) {
+          if (j < j_lo + Ws && o >= 0 && o < n) {
             const int klo = max(max(0, j - (Wb - 1)), p.a_lu - x), khi = min(min(Wa - 1, j), n - 1 + p.a_lu - x);
             for (int k = klo; k <= khi; ++k) fold(t, ap[k], bp[t * dt + k], k);
           }
@@ -154,37 +162,39 @@ __global__ __launch_bounds__(256, 2) void k_band_max_fwd(const BandArgs p, int s
   __syncthreads();  // the operands are consumed: their place becomes the result tiles
 
   float* Sv = smem;
-  int* Si = reinterpret_cast<int*>(smem + ((kMaxRows * Wo + 3) & ~3));
+  int* Si = reinterpret_cast<int*>(smem + ((kMaxRows * Ws + 3) & ~3));
 #pragma unroll
   for (int s = 0; s < 5; ++s) {
     const int jb = wave + 4 * s;
     if (jb < nblocks) {
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
-        const int j = 8 * jb + t, o = x + j - r_lu;
-        if (j < Wo) {
+        const int js = 8 * jb + t, o = x + j_lo + js - r_lu;
+        if (js < Ws) {
           const bool inside = x < n && o >= 0 && o < n;  // outside: the reference's zero fill
-          Sv[lane * Wo + j] = inside ? val[s][t] : 0.f;
-          Si[lane * Wo + j] = inside ? ind[s][t] : 0;
+          Sv[lane * Ws + js] = inside ? val[s][t] : 0.f;
+          Si[lane * Ws + js] = inside ? ind[s][t] : 0;
         }
       }
     }
   }
   __syncthreads();
 
-  const int rows = min(kMaxRows, n - x0), cells = rows * Wo;
-  float* ob = p.o0 + (bn + x0) * Wo;
-  int32_t* ib = p.oidx + (bn + x0) * Wo;
-  if ((cells & 3) == 0 && ((reinterpret_cast<uintptr_t>(ob) | reinterpret_cast<uintptr_t>(ib)) & 15) == 0) {
-    typedef int mm_i4 __attribute__((ext_vector_type(4)));
-    for (int e = 4 * tid; e < cells; e += 1024) {
+  const int rows = min(kMaxRows, n - x0), cells = rows * Ws;
+  float* ob = p.o0 + (bn + x0) * Wo + j_lo;
+  int32_t* ib = p.oidx + (bn + x0) * Wo + j_lo;
+  typedef int mm_i4 __attribute__((ext_vector_type(4)));
+  if (Ws == Wo && (cells & 3) == 0 &&
+      ((reinterpret_cast<uintptr_t>(ob) | reinterpret_cast<uintptr_t>(ib)) & 15) == 0) {
+    for (int e = 4 * tid; e < cells; e += 1024) {  // the strip's rows are one contiguous run
       *reinterpret_cast<mm_f4*>(ob + e) = *reinterpret_cast<const mm_f4*>(Sv + e);
       *reinterpret_cast<mm_i4*>(ib + e) = *reinterpret_cast<const mm_i4*>(Si + e);
     }
   } else {
-    for (int e = tid; e < cells; e += 256) {
-      ob[e] = Sv[e];
-      ib[e] = Si[e];
+    for (int e = tid; e < cells; e += 256) {  // runs of Ws cells, one per row
+      const int r = e / Ws, c = e - r * Ws;
+      ob[(long)r * Wo + c] = Sv[e];
+      ib[(long)r * Wo + c] = Si[e];
     }
   }
 }
