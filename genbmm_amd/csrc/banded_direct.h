@@ -61,7 +61,7 @@ namespace GENBMM_NS {
 
 constexpr int kDirFwd = 0, kDirGradA = 1, kDirGradB = 2;
 constexpr int kDirTiles = 32;   // tiles per tile row, at most (5 bits of a step word; a bit per cell in 128 bits)
-constexpr int kDirChunks = 30;  // chunks of the first operand per tile row, at most (5 bits, one value for the chunk of zeros)
+constexpr int kDirChunks = 30;  // chunks of the first operand per tile row, at most (5 bits)
 constexpr int kDirDepth = 4;    // pairs whose loads of Q are in flight
 constexpr int kDirWaves = 2;    // waves (tile rows) per workgroup
 constexpr int kDirMargin = 48;  // floats a load can stray from the band rows it is meant for
@@ -69,7 +69,7 @@ typedef float dir_f4u __attribute__((ext_vector_type(4), aligned(4)));
 
 // The walk over a tile row's (tile, chunk) pairs.  One word per step:
 //   bits 0-12  where the pair's cells of Q start, in units of 16 floats
-//   bits 13-17 chunk of P (the one past the last holds zeros)
+//   bits 13-17 chunk of P
 //   bits 18-22 tile      bit 23  the tile is complete after this step
 //   bit 24  some lane's cells of Q lie past the upper end of its band (D = 0)
 //   bit 25 / 26  ... below the lower end: D is the plan's lowest / the one above it
@@ -111,11 +111,13 @@ inline DirPlanSmall dir_plan_small(const DirPlan& g) {  // g.steps <= kDirStepsS
 }
 
 inline int dir_chunks(int Wp) { return (Wp + 30) >> 4; }  // chunks of 16 k that a tile row's P meets
-// LDS of one wave: its chunks of P and one of zeros, 1 KB each; then the row maxima of b for
-// its tiles (forward of the log product) or the tile row's results (all others), which then
-// leave as one contiguous run of memory
+// LDS of one wave: its chunks of P, 1 KB each; then the tile row's results, which leave as one
+// contiguous run of memory.  The forward of the log product puts the row maxima of b for its
+// tiles and of a for its rows where the chunks were, once the walk is done with them.  (LDS
+// bounds the waves per compute unit, and the kernels' time follows their number: at 65
+// diagonals per operand 13.4 KB per wave are twelve waves, a KB more ten.)
 inline int dir_wave_lds(const DirPlan& g, int kind, bool prep) {
-  return (g.NU + 1) * 1024 + 64 * g.Wout + (kind == kDirFwd && prep ? 64 * g.nt + 64 : 0);
+  return max(g.NU * 1024, kind == kDirFwd && prep ? 64 * g.nt + 64 : 0) + 64 * g.Wout;
 }
 
 inline bool dir_plan(DirPlan& g, int kind, int a_lu, int Wa, int b_lu, int Wb) {
@@ -167,7 +169,7 @@ inline bool dir_plan(DirPlan& g, int kind, int a_lu, int Wa, int b_lu, int Wb) {
   const int pad = (kDirDepth - (np & (kDirDepth - 1))) & (kDirDepth - 1);
   if (np + pad > kDirSteps) return false;
   g.steps = np + pad;
-  for (int i = 0; i < pad; ++i) g.e[i].now = (list[0] & kDirQMask) | (unsigned)NU << kDirChunkShift | kDirFill;
+  for (int i = 0; i < pad; ++i) g.e[i].now = (list[0] & kDirQMask) | kDirFill;  // chunk 0, read and not used
   for (int i = 0; i < np; ++i) g.e[pad + i].now = list[i];
   g.e[g.steps].now = g.e[g.steps - 1].now;
   for (int i = 0; i <= g.steps; ++i) g.e[i].ahead = g.e[min(i + kDirDepth, g.steps - 1)].now;
@@ -235,7 +237,7 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long b
 #pragma unroll
   for (int s = 0; s < kDirDepth; ++s) issue(g.e[s].now, qraw[s]);
 
-  // ---- P into LDS, as the instruction reads it (lane, t); after the last chunk one of zeros.
+  // ---- P into LDS, as the instruction reads it (lane, t).
   //   band row i: loading lane (lr, lc), row i0 + lr, cells 16 u + 4 lc - lr + t, k = K0 + 16 u + 4 lc + t
   //   band row k: lane (l15, zq), row k = K0 + 16 u + 4 zq + t, cell Wp - 1 - 16 u + l15 - 4 zq - t
   {
@@ -289,19 +291,21 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long b
         }
       }
     }
-    pl[64 * NU + lane] = mm_f4{0.f, 0.f, 0.f, 0.f};
   }
-  // behind the chunks: the tile row's 16 x Wout results, then (forward of the log product) beta
-  // of every column the wave's tiles cover and alpha of its 16 rows
-  float* aux = lds + 256 * (NU + 1);
-  float* bet = aux + 16 * Wout;
-  float* alp = bet + 16 * nt;
+  // the tile row's 16 x Wout results, in the last 64 Wout bytes of the wave's piece
+  float* aux = lds + ((FWD && PREP) ? max(256 * NU, 16 * nt + 16) : 256 * NU);
+  // forward of the log product: beta of every column the wave's tiles cover and alpha of its 16
+  // rows, asked for now, put into LDS over the chunks when the walk is over
+  float* bet = lds;
+  float* alp = lds + 16 * nt;
+  float betr[kDirTiles / 4], alpr = 0.f;
   if (FWD && PREP) {
-    for (int t = lane; t < 16 * nt; t += 64) {
-      const int y = J0 + t;
-      bet[t] = (unsigned)y < (unsigned)n ? p.ws_be[bn + y] : 0.f;
+#pragma unroll
+    for (int s = 0; s < kDirTiles / 4; ++s) {
+      const int t = lane + 64 * s, y = J0 + t;
+      betr[s] = t < 16 * nt && (unsigned)y < (unsigned)n ? p.ws_be[bn + y] : 0.f;
     }
-    if (lane < 16) alp[lane] = i0 + lane < n ? p.ws_al[bn + i0 + lane] : 0.f;
+    if (lane < 16) alpr = i0 + lane < n ? p.ws_al[bn + i0 + lane] : 0.f;
   }
 
   // Factors 1 / 0 for the cells of a chunk at the ends of Q's band: past the upper end
@@ -418,7 +422,7 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long b
     float* ot = (STAGE ? aux : orow) + 16 * tj;
     unsigned bits = 0;
     float be = 0.f;
-    if (FWD && PREP) be = bet[16 * tj + l15];
+    if (FWD && PREP) be = y_in ? p.ws_be[bn + y] : 0.f;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int jj = 16 * tj + l15 - 4 * zq - r;
@@ -471,6 +475,10 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long b
   }
 
   if (FWD && PREP && plain_rows) {
+#pragma unroll
+    for (int s = 0; s < kDirTiles / 4; ++s)
+      if (lane + 64 * s < 16 * nt) bet[lane + 64 * s] = betr[s];
+    if (lane < 16) alp[lane] = alpr;
     // The sums S of the tile row are in LDS: out = log S + alpha + beta and 1/S leave as two
     // contiguous runs, four cells per lane.  A cell outside the guard gets 1/S = -1 (not usable,
     // the backward then takes the exact way) and its value from the per-cell routine right
