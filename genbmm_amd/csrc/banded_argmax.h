@@ -40,15 +40,18 @@ struct ArgTile {
   float gv[PER];
   int iv[PER];
   // row0: g row of tile row 0; the cell (row0 + r, jc + c) counts if its row is in
-  // [0, n), j < Wo and, for need_o, its o = i + j - r_lu is in [0, n)
+  // [0, n), j < Wo and, for need_o, its o = i + j - r_lu is in [0, n); for skew (a tile
+  // whose rows of b run along its diagonals) only if it lies on the diagonal of one of the
+  // strip's 64 rows - the corners of the tile are not read
   __device__ __forceinline__ void load(const float* __restrict__ gb, const int32_t* __restrict__ ib,
                                        int row0, int jc, int n, int Wo, int r_lu, bool need_o,
-                                       int tid) {
+                                       bool skew, int tid) {
 #pragma unroll
     for (int u = 0; u < PER; ++u) {
       const int e = tid + 256 * u, r = e >> 5, c = e & 31;
       const int i = row0 + r, j = jc + c, o = i + j - r_lu;
-      const bool ok = r < ROWS && i >= 0 && i < n && j < Wo && (!need_o || (o >= 0 && o < n));
+      const bool ok = r < ROWS && i >= 0 && i < n && j < Wo && (!need_o || (o >= 0 && o < n)) &&
+                      (!skew || (unsigned)(r - (kAJ - 1) + c) < (unsigned)kAT);
       gv[u] = ok ? gb[(long)i * Wo + j] : 0.f;
       iv[u] = ok ? ib[(long)i * Wo + j] : -1;
     }
@@ -83,12 +86,12 @@ __global__ __launch_bounds__(256) void k_band_argmax_bwd_a(const BandArgs p, int
   for (int e = tid; e < Wa * kAS + 256; e += 256) acc[e] = 0.f;
   const int spare = Wa * kAS + tid;
   ArgTile<kAT> tile;
-  tile.load(gb, ib, i0, 0, n, Wo, p.r_lu, true, tid);
+  tile.load(gb, ib, i0, 0, n, Wo, p.r_lu, true, false, tid);
   for (int jc = 0; jc < Wo; jc += kAJ) {
     __syncthreads();
     tile.store(gt, it, tid);
     __syncthreads();
-    if (jc + kAJ < Wo) tile.load(gb, ib, i0, jc + kAJ, n, Wo, p.r_lu, true, tid);
+    if (jc + kAJ < Wo) tile.load(gb, ib, i0, jc + kAJ, n, Wo, p.r_lu, true, false, tid);
 #pragma unroll 2
     for (int c = 0; c < kAJ; c += 4) {
       int sl[4];
@@ -130,12 +133,12 @@ __global__ __launch_bounds__(256) void k_band_argmax_bwd_b(const BandArgs p, int
   const int jlast = ((Wo - 1) / kAJ) * kAJ;
   auto row0_of = [&](int jc) { return o0 + p.r_lu - jc - (kAJ - 1); };
   ArgTile<kRows> tile;
-  tile.load(gb, ib, row0_of(jlast), jlast, n, Wo, p.r_lu, false, tid);
+  tile.load(gb, ib, row0_of(jlast), jlast, n, Wo, p.r_lu, false, true, tid);
   for (int jc = jlast; jc >= 0; jc -= kAJ) {
     __syncthreads();
     tile.store(gt, it, tid);
     __syncthreads();
-    if (jc > 0) tile.load(gb, ib, row0_of(jc - kAJ), jc - kAJ, n, Wo, p.r_lu, false, tid);
+    if (jc > 0) tile.load(gb, ib, row0_of(jc - kAJ), jc - kAJ, n, Wo, p.r_lu, false, true, tid);
     if (o0 + lane < n) {
 #pragma unroll 2
       for (int c4 = kAJ - 1; c4 >= 0; c4 -= 4) {
