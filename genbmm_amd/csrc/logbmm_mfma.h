@@ -371,9 +371,7 @@ void k_log_fwd_mfma(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
     __syncthreads();
   }
 
-  // guard: S >= 2^-40 and finite; every shift of the tile finite and far above
-  // the reference's -1e9 floor (checked per row and column, which is stricter
-  // than per cell and only sends more tiles to the exact routine).
+  // guard: S >= 2^-40 and finite; ...
   const float thr = fast_exp2(-kMfmaGuardBits);
   int bad = 0;
   {
@@ -388,13 +386,29 @@ void k_log_fwd_mfma(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
         if (here && !((s >= thr) && (s < INFINITY))) bad = 1;
       }
   }
-  for (int t = tid; t < T::TR + T::TC; t += NT) {
+  // ... every shift finite and not below the floor; and, since the reference keeps its running
+  // maximum at the floor or above, alpha + beta of every cell within reach of the floor must not
+  // be so far below it that the reference's terms would vanish (they do from 104 below): a row
+  // at the floor (an operand row masked with -1e9) is factored as long as every column's shift
+  // is above -30, and the other way round.  (1 / S is kept as computed, not derived from `out`,
+  // so the backward loses nothing to the rounding of results near -1e9.)
+  static_assert(T::TR + T::TC <= NT, "one shift per thread");
+  int low = 0, neg = 0;  // bit 0: of a row, bit 1: of a column
+  {
+    const int t = tid;
     const bool row = t < T::TR;
-    const bool here = !RAGGED || (row ? m0 + t < M : n0 + t - T::TR < N);
+    const bool here = t < T::TR + T::TC && (!RAGGED || (row ? m0 + t < M : n0 + t - T::TR < N));
     if (here) {
       const float sh = row ? st[m0 + t] : st[M + n0 + t - T::TR];
-      if (!((sh > 0.45f * kFloor) && (sh < INFINITY))) bad = 1;
+      if (!((sh >= kFloor) && (sh < INFINITY))) bad = 1;
+      if (sh <= 0.45f * kFloor) low = row ? 1 : 2;
+      if (sh < -30.f) neg = row ? 1 : 2;
     }
+  }
+  const int row_low = __syncthreads_or(low & 1), col_low = __syncthreads_or(low & 2);
+  if (row_low | col_low) {  // uniform, and rare
+    const int row_neg = __syncthreads_or(neg & 1), col_neg = __syncthreads_or(neg & 2);
+    if ((row_low && col_neg) || (col_low && row_neg)) bad = 1;
   }
   bad = __syncthreads_or(bad);  // also: every wave is done with the staging buffers
   if (tid == 0) flags[tile] = bad;

@@ -181,6 +181,55 @@ def test_logbmm_factoring_guard_matrix_core_tiles(gpu, B, M, K, N):
     close(gb.sum(-2), g.double().sum(-2), atol=2e-4)
 
 
+@pytest.mark.parametrize("B,M,K,N", [(8, 256, 128, 256), (6, 300, 100, 260), (4, 512, 64, 384)])
+def test_logbmm_rows_masked_at_the_floor(gpu, B, M, K, N):
+    """Padding written as -1e9, the reference's own floor (matmul_cuda_kernel.cu:31): whole
+    rows of a, whole columns of b, or - one batch item - both.  A cell of a masked row has
+    max_k(a + b) = -1e9 + max_k b, not below the floor, so the reference's result is the
+    plain log-sum-exp there (float64: -1e9 + logsumexp_k b[k, n]; a float holds it to within
+    64); where a masked row meets a masked column every term is at -2e9 and the reference
+    gives -inf.  The gradient flowing into the padding is zero, as after any masked loss;
+    the gradients of everything else must not notice the padding.  Matrix-core shapes: the
+    tiles with masked rows or columns are factored like any other (their 1 / S comes from the
+    sums, not from `out`), only the tiles of the item with both take the exact routine."""
+    torch.manual_seed(B + N)
+    a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
+    rows, cols = M - M // 5, N - N // 7
+    a[: B // 2, rows:, :] = -1e9          # padded rows
+    b[B // 2:, :, cols:] = -1e9           # padded columns
+    a[B - 1, rows:, :] = -1e9             # the last item: both
+    g[: B // 2, rows:, :] = 0.0
+    g[B // 2:, :, cols:] = 0.0
+    g[B - 1, rows:, :] = 0.0
+    want, wa, wb = oracle.logbmm_grads64(a, b, g)
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    out = genbmm.logbmm(ad, bd)
+    ga, gb = torch.autograd.grad(out, (ad, bd), g.to(gpu))
+    both = torch.zeros(B, M, N, dtype=torch.bool)
+    both[B - 1, rows:, cols:] = True
+    pad = torch.zeros(B, M, N, dtype=torch.bool)
+    pad[: B // 2, rows:, :] = True
+    pad[B // 2:, :, cols:] = True
+    pad[B - 1, rows:, :] = True
+    pad &= ~both
+    oc = out.cpu()
+    assert bool(torch.isinf(oc[both]).all()) and bool((oc[both] < 0).all())
+    close(oc[~pad & ~both], want[~pad & ~both])
+    close(oc[pad], want[pad], rtol=0, atol=128.0)   # a float near -1e9 is a multiple of 64
+    # the exact routine and the factored vector-ALU kernels (the reference's own steps at the padding) agree
+    for other in (genmul.PATH_EXACT, genmul.PATH_VALU):
+        alt = genmul.logbmm_on_path(ad.detach(), bd.detach(), other).cpu()
+        assert torch.equal(torch.isinf(alt), torch.isinf(oc))
+        close(oc[~pad & ~both], alt[~pad & ~both])
+        close(oc[pad], alt[pad], rtol=0, atol=128.0)
+    # gradients: the item with both has infinite weights where the reference has them (0 * inf);
+    # the others are finite everywhere and equal to float64's
+    ok = torch.arange(B) != B - 1
+    close(ga[ok.to(gpu)], wa[ok])
+    close(gb[ok.to(gpu)], wb[ok])
+    assert bool(torch.isfinite(ga[ok.to(gpu)]).all()) and bool(torch.isfinite(gb[ok.to(gpu)]).all())
+
+
 @pytest.mark.parametrize("B,M,K,N", [(20, 128, 128, 128), (17, 100, 70, 128), (12, 64, 128, 65), (9, 127, 99, 101)])
 def test_logbmm_one_tile_items(gpu, B, M, K, N):
     """Items of at most 128 in every extent: one workgroup per item (and gradient) that
