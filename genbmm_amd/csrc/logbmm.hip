@@ -258,7 +258,7 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_fwd_fast(const DenseArgs p,
       const int c = col_of<C>(tx, j);
       const float shift = ai + be[c];
       const float s = acc[i][j];
-      const bool ok = (s >= thr) && (s < INFINITY) && (shift > 0.9f * kFloor) && (shift < INFINITY);
+      const bool ok = (s >= thr) && (s < INFINITY) && (shift >= kFloor) && (shift < INFINITY);
       if (!ok && m0 + r < M && n0 + c < N) bad = 1;
       acc[i][j] = __builtin_fmaf(fast_log2(s), kLn2, shift);  // v_log_f32
     }

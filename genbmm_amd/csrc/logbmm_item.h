@@ -162,7 +162,7 @@ __global__ __launch_bounds__(G * G, TB == 2 ? 8 : 1) void k_log_item_fwd(const e
       const int m = ty * TB + i, n = tx * TB + j;
       if (m < M && n < N) {
         const float shift = al[m] + be[n], s = acc[i][j];
-        const bool ok = (s >= thr) && (s < INFINITY) && (shift > 0.9f * kFloor) && (shift < INFINITY);
+        const bool ok = (s >= thr) && (s < INFINITY) && (shift >= kFloor) && (shift < INFINITY);
         At[m * LD + n] = ok ? __builtin_fmaf(fast_log2(s), kLn2, shift)
                             : item_exact_out(ab + (long)m * K, bb + n, K, N);
       }

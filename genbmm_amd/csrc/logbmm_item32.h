@@ -106,7 +106,7 @@ __global__ __launch_bounds__(256) void k_log_item32_fwd(const elem_t* __restrict
   for (int r = 0; r < 16; ++r) {
     const int i = mfma_row_u(r) + 4 * h;
     const float shift = ar[r] + be, s = acc[r];
-    const bool ok = (s >= thr) && (s < INFINITY) && (shift > 0.9f * kFloor) && (shift < INFINITY);
+    const bool ok = (s >= thr) && (s < INFINITY) && (shift >= kFloor) && (shift < INFINITY);
     if (!ok) redo |= 1u << r;
     ob[i * kI32 + c] = to_elem<elem_t>(__builtin_fmaf(fast_log2(s), kLn2, shift));
   }

@@ -181,7 +181,8 @@ def test_logbmm_factoring_guard_matrix_core_tiles(gpu, B, M, K, N):
     close(gb.sum(-2), g.double().sum(-2), atol=2e-4)
 
 
-@pytest.mark.parametrize("B,M,K,N", [(8, 256, 128, 256), (6, 300, 100, 260), (4, 512, 64, 384)])
+@pytest.mark.parametrize("B,M,K,N", [(8, 256, 128, 256), (6, 300, 100, 260), (4, 512, 64, 384), (9, 32, 32, 32),
+                                     (6, 64, 64, 64), (5, 40, 48, 36), (7, 128, 128, 128), (4, 100, 70, 128)])
 def test_logbmm_rows_masked_at_the_floor(gpu, B, M, K, N):
     """Padding written as -1e9, the reference's own floor (matmul_cuda_kernel.cu:31): whole
     rows of a, whole columns of b, or - one batch item - both.  A cell of a masked row has
@@ -189,9 +190,11 @@ def test_logbmm_rows_masked_at_the_floor(gpu, B, M, K, N):
     plain log-sum-exp there (float64: -1e9 + logsumexp_k b[k, n]; a float holds it to within
     64); where a masked row meets a masked column every term is at -2e9 and the reference
     gives -inf.  The gradient flowing into the padding is zero, as after any masked loss;
-    the gradients of everything else must not notice the padding.  Matrix-core shapes: the
-    tiles with masked rows or columns are factored like any other (their 1 / S comes from the
-    sums, not from `out`), only the tiles of the item with both take the exact routine."""
+    the gradients of everything else must not notice the padding.  On the matrix-core shapes
+    the tiles with masked rows or columns are factored like any other (their 1 / S comes from
+    the sums, not from `out`), only the tiles of the item with both take the exact routine;
+    the smaller shapes run the whole-item kernels, the factored vector-ALU kernels and the
+    one-tile-per-item kernels (whose padded items take the exact routine)."""
     torch.manual_seed(B + N)
     a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
     rows, cols = M - M // 5, N - N // 7
