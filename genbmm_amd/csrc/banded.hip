@@ -138,8 +138,7 @@ inline void launch_dir(const BandArgs& p, int B, hipStream_t s) {
     if ((size_t)kDirWaves * wave_lds > kStripLdsLimit)
       (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 kDirWaves * wave_lds);
-    const int extra = getenv("GENBMM_LDSX") ? atoi(getenv("GENBMM_LDSX")) : 0;
-    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64 * kDirWaves), kDirWaves * wave_lds + extra, s, p, table,
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64 * kDirWaves), kDirWaves * wave_lds, s, p, table,
                        blocks, nblocks, (long)B * p.n, wave_lds);
   };
   if (plan.steps <= kDirStepsSmall) go(k_band_dir<KIND, PREP, DirPlanSmall>, dir_plan_small(plan));

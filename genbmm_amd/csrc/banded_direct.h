@@ -63,7 +63,7 @@ constexpr int kDirFwd = 0, kDirGradA = 1, kDirGradB = 2;
 constexpr int kDirTiles = 32;   // tiles per tile row, at most (5 bits of a step word; a bit per cell in 128 bits)
 constexpr int kDirChunks = 30;  // chunks of the first operand per tile row, at most (5 bits)
 constexpr int kDirDepth = 4;    // pairs whose loads of Q are in flight
-constexpr int kDirWaves = 2;    // waves (tile rows) per workgroup
+constexpr int kDirWaves = 1;    // waves (tile rows) per workgroup
 constexpr int kDirMargin = 48;  // floats a load can stray from the band rows it is meant for
 typedef float dir_f4u __attribute__((ext_vector_type(4), aligned(4)));
 
