@@ -48,7 +48,26 @@ __device__ __forceinline__ void static_for(F&& f) {
     static_for<I + 1, E>(f);
   }
 }
-__device__ __forceinline__ bool shift_ok(float sh) { return (sh > 0.45f * kFloor) && (sh < INFINITY); }
+// The shifts of an item, one per thread (`row`: a row's maximum, else a column's; `here`: the
+// thread has one): may the item be factored?  Every shift finite and not below the reference's
+// floor, and - the reference keeps its running maximum at the floor or above, and its terms
+// vanish from about 100 below it - no row at the floor (an operand row padded with -1e9) together
+// with a column whose shift is below -30, nor the other way round.  Every thread of the
+// workgroup calls this (it synchronizes); the answer is uniform.
+__device__ __forceinline__ int self_shifts_bad(bool here, bool row, float sh) {
+  int bad = 0, low = 0, neg = 0;  // bit 0: of a row, bit 1: of a column
+  if (here) {
+    bad = !((sh >= kFloor) && (sh < INFINITY));
+    if (sh <= 0.45f * kFloor) low = row ? 1 : 2;
+    if (sh < -30.f) neg = row ? 1 : 2;
+  }
+  const int row_low = __syncthreads_or(low & 1), col_low = __syncthreads_or(low & 2);
+  if (row_low | col_low) {  // uniform, and rare
+    const int row_neg = __syncthreads_or(neg & 1), col_neg = __syncthreads_or(neg & 2);
+    if ((row_low && col_neg) || (col_low && row_neg)) bad = 1;
+  }
+  return __syncthreads_or(bad);
+}
 
 // ----------------------------------------------------------------- forward
 // An item that fails the guard: the online routine, two 64 x 128 tiles.
@@ -202,7 +221,7 @@ void k_log_self_fwd(const DenseArgs p, float* __restrict__ stats, int* __restric
     const bool row = tid < kSelfMax;
     const int t = row ? tid : tid - kSelfMax;
     const bool here = !RAGGED || t < (row ? M : N);
-    if (here && !shift_ok(row ? s_al[t] : s_be[t])) bad = 1;
+    bad |= self_shifts_bad(here, row, here ? (row ? s_al[t] : s_be[t]) : 0.f);
   }
   bad = __builtin_amdgcn_readfirstlane(__syncthreads_or(bad));
   if (bad) {
@@ -294,13 +313,13 @@ __device__ __forceinline__ void log_self_bwd_tile(float* __restrict__ smem, floa
   // the shifts the forward left (any forward that writes them will do)
   const int tag = hdr[0];
   int bad = !(tag == kWsSelf || tag == kWsMfma || tag == kWsFast);
+  float my_shift;
   {
     const bool row = tid < kSelfMax;
     const int t = row ? tid : tid - kSelfMax;
     const bool here = !RAGGED || t < (row ? M : N);
-    const float sh = here ? st[row ? t : M + t] : 0.f;
-    if (!shift_ok(sh)) bad = 1;
-    (row ? s_al : s_be)[t] = sh;
+    my_shift = here ? st[row ? t : M + t] : 0.f;
+    (row ? s_al : s_be)[t] = my_shift;
   }
 
   // What this tile stages: rg/ro = g and out, ry = the other operand.  g and out are requested at
@@ -380,6 +399,11 @@ __device__ __forceinline__ void log_self_bwd_tile(float* __restrict__ smem, floa
   static_for<0, kSelfSlabs>(load_h);
   __builtin_amdgcn_sched_barrier(0);
   __syncthreads();  // s_al, s_be
+  {  // (asked here, behind the loads: it waits for the shifts)
+    const bool row = tid < kSelfMax;
+    const int t = row ? tid : tid - kSelfMax;
+    bad |= self_shifts_bad(!RAGGED || t < (row ? M : N), row, my_shift);
+  }
 
   floatx16 acc[2][2];
 #pragma unroll
