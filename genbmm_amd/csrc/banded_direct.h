@@ -432,7 +432,7 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long b
           float rv = 0.f;
           if (y_in) {
             const float sh = al[r] + be;
-            const bool ok = (v >= thr) && (v < INFINITY) && (sh > 0.9f * kFloor) && (sh < INFINITY);
+            const bool ok = (v >= thr) && (v < INFINITY) && (sh >= kFloor) && (sh < INFINITY);
             rv = ok ? __builtin_amdgcn_rcpf(v) : -1.f;  // -1 tells the backward that 1/S is not usable here
             v = __builtin_fmaf(fast_log2(v), kLn2, sh);
             if (!ok) bits |= 1u << r;
@@ -496,7 +496,7 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long b
 #pragma unroll
       for (int c4 = 0; c4 < 4; ++c4) {
         const float sh = alp[row] + bet[row + jj], v = sv[c4];
-        const bool ok = (v >= thr) && (v < INFINITY) && (sh > 0.9f * kFloor) && (sh < INFINITY);
+        const bool ok = (v >= thr) && (v < INFINITY) && (sh >= kFloor) && (sh < INFINITY);
         rv[c4] = ok ? __builtin_amdgcn_rcpf(v) : -1.f;
         ov[c4] = __builtin_fmaf(fast_log2(v), kLn2, sh);
         if (!ok) bad |= 0x80000000u >> c4;

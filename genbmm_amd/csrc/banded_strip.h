@@ -377,7 +377,7 @@ __global__ __launch_bounds__(256, (SEM == kSemMul || SEM == kSemLogPrep) ? 3 : 2
         const int j = j0 + t, o = i + j - p.r_lu;
         float rv = 0.f;
         if (i < n && j < Wo && o >= 0 && o < n) {
-          if ((v >= thr) && (v < INFINITY) && (sh[t] > 0.9f * kFloor) && (sh[t] < INFINITY)) {
+          if ((v >= thr) && (v < INFINITY) && (sh[t] >= kFloor) && (sh[t] < INFINITY)) {
             rv = __builtin_amdgcn_rcpf(v);
             v = __builtin_fmaf(fast_log2(v), kLn2, sh[t]);
           } else {  // factoring not exact for this cell: recompute it from memory

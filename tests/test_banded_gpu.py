@@ -96,6 +96,42 @@ def test_banded_log_factoring_guard(gpu, n, a_lu, a_ld, b_lu, b_ld):
     close(gb, wb, rtol=tol, atol=tol)
 
 
+@pytest.mark.parametrize("n,a_lu,a_ld,b_lu,b_ld", [(200, 6, 5, 4, 7), (600, 32, 32, 32, 32), (300, 12, 20, 30, 3)])
+def test_banded_log_rows_padded_at_the_floor(gpu, n, a_lu, a_ld, b_lu, b_ld):
+    """Band rows written as -1e9 throughout (padding at the reference's floor,
+    banded_cuda_kernel.cu:31-33): max_k(a + b) of their cells is -1e9 + max b, not below the
+    floor, so the result is the plain log-sum-exp (float64: -1e9 + logsumexp of the cells of b
+    it meets; a float near -1e9 is a multiple of 64).  No gradient flows into the padding;
+    everything else must not notice it.  These rows are factored like any other (their 1 / S
+    comes from the sums); where a padded row of a meets a padded row of b every term is at
+    -2e9 and the per-cell routine gives the reference's -inf."""
+    torch.manual_seed(n + a_lu)
+    a, b = pair(n, a_lu, a_ld, b_lu, b_ld)
+    W = a.shape[2] + b.shape[2] - 1
+    g = torch.randn(3, n, W)
+    pad = slice(n - n // 6, n)
+    a[:2, pad, :] = -1e9                      # the last rows of a (items 0, 1)
+    b[1:, pad, :] = -1e9                      # the last rows of b (items 1, 2): item 1 has both
+    want, _, _ = oracle.seq_band_fwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, 0, dtype=np.float64)
+    want32, _, _ = oracle.seq_band_fwd(a, a_lu, a_ld, b, b_lu, b_ld, 0)
+    at_floor = want < -5e8                    # cells fed by padding: near -1e9, or -inf in float where both meet
+    g[at_floor] = 0.0
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    res = BandedMatrix(ad, a_lu, a_ld).multiply_log(BandedMatrix(bd, b_lu, b_ld))
+    got = res.data.detach().cpu()
+    gone = torch.isinf(want32)                # the reference's own float arithmetic: terms at -2e9 vanish
+    assert torch.equal(torch.isinf(got), gone)
+    close(got[~at_floor], want[~at_floor])
+    close(got[at_floor & ~gone], want[at_floor & ~gone], rtol=0, atol=128.0)
+    ga, gb = torch.autograd.grad(res.data, (ad, bd), g.to(gpu))
+    wa, wb = oracle.seq_band_bwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, g.double(), 0, dtype=np.float64)
+    # item 1, where results are -inf, has 0 * inf among its weights in the reference's own arithmetic
+    ok = torch.tensor([0, 2])
+    assert bool(torch.isfinite(ga[ok.to(gpu)]).all()) and bool(torch.isfinite(gb[ok.to(gpu)]).all())
+    close(ga[ok.to(gpu)], wa[ok], atol=2e-5)
+    close(gb[ok.to(gpu)], wb[ok], atol=2e-5)
+
+
 def test_banded_max_index_through_c_abi(gpu):
     torch.manual_seed(2)
     n, a_lu, a_ld, b_lu, b_ld = 50, 4, 6, 5, 3
