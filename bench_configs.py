@@ -57,13 +57,17 @@ def report(name, ms, ops, nbytes, extra=None):
     print(json.dumps(line), flush=True)
 
 
-def dense_log(lib, dev, B, M, K, N, reps, name, dist="randn", path=0, graph=False, dtype=torch.float32):
+def dense_log(lib, dev, B, M, K, N, reps, name, dist="randn", path=0, graph=False, dtype=torch.float32, pad=None):
     """dtype float16 / bfloat16: the `_f16` / `_bf16` entry points on tensors of that type (and, for
-    comparison, the float entry points with the widening and narrowing copies around them)."""
+    comparison, the float entry points with the widening and narrowing copies around them).
+    pad = (value, rows): the last `rows` rows of every a hold `value` (padding), no gradient flows into them."""
     torch.manual_seed(0)
     mk = torch.randn if dist == "randn" else torch.rand
     a, b = mk(B, M, K).to(dev).to(dtype), mk(B, K, N).to(dev).to(dtype)
     g = (torch.ones(B, M, N) if dist == "rand" else torch.randn(B, M, N)).to(dev).to(dtype)
+    if pad is not None:
+        a[:, M - pad[1]:, :] = pad[0]
+        g[:, M - pad[1]:, :] = 0
     out, ga, gb = torch.empty(B, M, N, device=dev, dtype=dtype), torch.empty_like(a), torch.empty_like(b)
     stats = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=dev)
     s, p = _lib.stream_of(a), _lib.ptr
@@ -186,12 +190,16 @@ def dense_sample(lib, dev, B, M, K, N, reps):
            {"ms_fwd": round(mf, 4), "ms_bwd": round(mb, 4)})
 
 
-def banded(lib, dev, B, n, lu, ld, mode, reps):
+def banded(lib, dev, B, n, lu, ld, mode, reps, pad=None):
+    """pad = (value, rows): the last `rows` band rows of a hold `value`, no gradient flows into them."""
     torch.manual_seed(7)
     W = lu + ld + 1
     Wo = 2 * W - 1
     a, b = (torch.rand(B, n, W) * 2 - 1).to(dev), (torch.rand(B, n, W) * 2 - 1).to(dev)
     g = torch.randn(B, n, Wo).to(dev)
+    if pad is not None:
+        a[:, n - pad[1]:, :] = pad[0]
+        g[:, n - pad[1]:, :] = 0
     out = torch.empty(B, n, Wo, device=dev)
     idx = torch.empty(B, n, Wo, dtype=torch.int32, device=dev) if mode == 1 else None
     ga, gb = torch.empty_like(a), torch.empty_like(b)
@@ -210,7 +218,8 @@ def banded(lib, dev, B, n, lu, ld, mode, reps):
     fb = 4.0 * B * n * (2 * W + Wo) + (4.0 * B * n * Wo if mode == 1 else 0)
     bb = 4.0 * B * n * (4 * W + Wo + (Wo if mode in (0, 1) else 0))
     name = {0: "multiply_log", 1: "multiply_max", 3: "multiply"}[mode]
-    report("banded %s fwd+bwd (B=%d,n=%d,lu=ld=%d)" % (name, B, n, lu), mf + mb, 6 * pairs, fb + bb,
+    report("banded %s fwd+bwd (B=%d,n=%d,lu=ld=%d)%s" % (name, B, n, lu, "" if pad is None else ", last %d rows of a = %g" % (pad[1], pad[0])),
+           mf + mb, 6 * pairs, fb + bb,
            {"ms_fwd": round(mf, 4), "ms_bwd": round(mb, 4),
             "fwd_GBs": round(fb / mf / 1e6, 1), "bwd_GBs": round(bb / mb / 1e6, 1)})
 
@@ -321,7 +330,8 @@ def main():
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--cpu", action="store_true")
     ap.add_argument("--only", default="", help="comma-separated subset: log,half,max,sample,banded,struct,f64; "
-                    "widths (not in the default set): the banded products at 5 ... 81 diagonals per operand")
+                    "widths (not in the default set): the banded products at 5 ... 81 diagonals per operand; "
+                    "pad (not in the default set): the log products with whole rows of padding (-1e9, -1e5, -inf)")
     args = ap.parse_args()
     want = set(args.only.split(",")) if args.only else {"log", "half", "max", "sample", "banded", "struct", "f64"}
     lib = _lib.load()
@@ -352,6 +362,13 @@ def main():
         for lu in (2, 4, 8, 16, 24, 32, 40):
             for mode in (3, 0, 1):
                 banded(lib, dev, 64, 4096, lu, lu, mode, r)
+    if "pad" in want:
+        for value in (-1e9, -1e5, float("-inf")):
+            for (B, M, K, N, rows) in ((64, 512, 512, 512, 8), (512, 128, 128, 128, 4), (2048, 64, 64, 64, 4), (8192, 32, 32, 32, 4)):
+                dense_log(lib, dev, B, M, K, N, r, "logbmm fwd+bwd (%d,%d,%d,%d), last %d rows of a = %g" % (B, M, K, N, rows, value),
+                          pad=(value, rows))
+            if value != float("-inf"):
+                banded(lib, dev, 64, 4096, 32, 32, 0, r, pad=(value, 400))
     if "struct" in want:
         band_structure(lib, dev, 64, 4096, 32, 32, r)
     if "f64" in want:
