@@ -617,10 +617,8 @@ void k_log_bwd_mfma(const elem_t* __restrict__ g, const float* __restrict__ ws_e
                                        grad, M, K, N, tiles_r, tiles_c);
 }
 
-// Both gradients in one launch: workgroups [0, tiles_a) take the tiles of grad_a
-// (shape TA), the rest those of grad_b (shape TB).  Workgroups are dispatched in
-// index order, so the first grad_b tiles start while the last grad_a tiles are
-// still writing their results back.
+// Both gradients in one launch: the tiles of grad_a (shape TA) and of grad_b (shape TB),
+// tiles_a of the former in all.
 template <class TA, class TB, bool RAGGED>
 __global__ __launch_bounds__(TA::NT) __attribute__((amdgpu_waves_per_eu(TA::WPE, TA::WPE)))
 void k_log_bwd_mfma_both(const elem_t* __restrict__ g, const float* __restrict__ ws_ea,
@@ -631,16 +629,21 @@ void k_log_bwd_mfma_both(const elem_t* __restrict__ g, const float* __restrict__
   static_assert(TA::NT == TB::NT && TA::WPE == TB::WPE, "");
   constexpr int kA = 2 * kMS * (TA::LDR + TA::LDC), kB = 2 * kMS * (TB::LDR + TB::LDC);
   __shared__ __attribute__((aligned(16))) float smem[kA > kB ? kA : kB];
+  // Item by item, the tiles of grad_a then those of grad_b: both gradients of an item read the
+  // same four arrays (g, 1/S, EA, EB: one's operand is the other's epilogue factor), so with
+  // an item's tiles in flight together the second use of each comes from the XCD's L2
+  // (all grad_a tiles first, then all grad_b tiles: 0.3125 against 0.3015 ms at the headline
+  // shape, build against build on one box).  XCD-aware numbering over the whole launch.
   const int w = blockIdx.x, n = gridDim.x;
-  // XCD-aware numbering inside each half (needs both halves to be multiples of 8)
-  const bool renum = (tiles_a & 7) == 0 && (n & 7) == 0;
-  if (w < tiles_a)
-    log_bwd_mfma_tile<TA, true, RAGGED>(smem, renum ? xcd_renumber(w, tiles_a) : w, g, ws_ea, ws_eb,
-                                        ws_r, ws_hdr, fwd_flags, grad_a, M, K, N, ar, ac);
+  const int per_a = ar * ac, per_b = br * bc;
+  const int v = xcd_renumber(w, n);
+  const int item = v / (per_a + per_b), r = v - item * (per_a + per_b);
+  if (r < per_a)
+    log_bwd_mfma_tile<TA, true, RAGGED>(smem, item * per_a + r, g, ws_ea, ws_eb, ws_r, ws_hdr, fwd_flags,
+                                        grad_a, M, K, N, ar, ac);
   else
-    log_bwd_mfma_tile<TB, false, RAGGED>(smem, renum ? xcd_renumber(w - tiles_a, n - tiles_a) : w - tiles_a,
-                                         g, ws_ea, ws_eb, ws_r, ws_hdr, fwd_flags, grad_b, M, K, N, br,
-                                         bc);
+    log_bwd_mfma_tile<TB, false, RAGGED>(smem, item * per_b + r - per_a, g, ws_ea, ws_eb, ws_r, ws_hdr,
+                                         fwd_flags, grad_b, M, K, N, br, bc);
 }
 
 // ------------------------------------------------------- sampling sweep
