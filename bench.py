@@ -23,7 +23,7 @@ FP32_VALU_PEAK_TFLOPS = 157.3  # MI355X FP32 peak (vector with packed FMA = fp32
 # HBM bytes per launch of the dominant kernel (k_log_bwd_mfma_both): rocprofv3 --pmc
 # FETCH_SIZE 274150 KiB + WRITE_SIZE 131070 KiB per dispatch, scale factor 1.00 against a
 # known-size copy in the same run (profiles/logbmm_headline_B64_512.md).
-DOMINANT_TRAFFIC_BYTES = (276060 + 131070) * 1024
+DOMINANT_TRAFFIC_BYTES = (243860 + 131070) * 1024
 
 
 def cpu_baseline(torch, sample_batches=64):
