@@ -145,6 +145,28 @@ inline void launch_dir(const BandArgs& p, int B, hipStream_t s) {
   else go(k_band_dir<KIND, PREP, DirPlan>, plan);
 }
 
+// grad_a and grad_b in one launch where both plans travel in the small form, else one launch each.
+template <bool PREP>
+inline void launch_dir_grads(const BandArgs& p, int B, hipStream_t s) {
+  DirPlan pa, pb;
+  dir_plan(pa, kDirGradA, p.a_lu, p.Wa, p.b_lu, p.Wb);
+  dir_plan(pb, kDirGradB, p.a_lu, p.Wa, p.b_lu, p.Wb);
+  if (pa.steps > kDirStepsSmall || pb.steps > kDirStepsSmall) {
+    launch_dir<kDirGradA, PREP>(p, B, s);
+    launch_dir<kDirGradB, PREP>(p, B, s);
+    return;
+  }
+  const int blocks = ceil_div(p.n, 16 * kDirWaves);
+  const int nblocks = B * blocks;
+  const int wave_lds = max(dir_wave_lds(pa, kDirGradA, PREP), dir_wave_lds(pb, kDirGradB, PREP));
+  auto kern = k_band_dir_grads<PREP, DirPlanSmall>;
+  if ((size_t)kDirWaves * wave_lds > kStripLdsLimit)
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              kDirWaves * wave_lds);
+  hipLaunchKernelGGL(kern, dim3(2u * (unsigned)nblocks), dim3(64 * kDirWaves), kDirWaves * wave_lds, s, p,
+                     dir_plan_small(pa), dir_plan_small(pb), blocks, nblocks, (long)B * p.n, wave_lds);
+}
+
 inline void set_workspace(BandArgs& p, float* ws, int B) {
   const size_t rows = (size_t)B * p.n;
   p.ws_ea = ws;
@@ -259,12 +281,10 @@ int banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int
   hipStream_t s = (hipStream_t)stream;
   if (mode != GENBMM_BAND_MAX && (mode == GENBMM_BAND_MUL || (workspace && workspace_used(p))) && dir_bwd_ok(p)) {
     if (mode == GENBMM_BAND_MUL) {
-      launch_dir<kDirGradA, false>(p, B, s);
-      launch_dir<kDirGradB, false>(p, B, s);
+      launch_dir_grads<false>(p, B, s);
     } else {  // H = g / S is formed by both kernels as they read g: the workspace is only read
       set_workspace(p, workspace, B);
-      launch_dir<kDirGradA, true>(p, B, s);
-      launch_dir<kDirGradB, true>(p, B, s);
+      launch_dir_grads<true>(p, B, s);
     }
     return launch_status();
   }

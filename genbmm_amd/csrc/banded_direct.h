@@ -563,15 +563,14 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long b
   }
 }
 
-// One wave per tile row, kDirWaves tile rows per workgroup.  blocks: workgroups per batch item;
-// wave_lds: bytes of LDS per wave; rows: band rows of every tensor (batch * n).
+// One wave per tile row, kDirWaves tile rows per workgroup: the tile rows of workgroup `blk` of a
+// product.  blocks: workgroups per batch item; wave_lds: bytes of LDS per wave; rows: band rows of
+// every tensor (batch * n).
 template <int KIND, bool PREP, class Plan>
-__global__ __launch_bounds__(64 * kDirWaves) void k_band_dir(const BandArgs p, const Plan g, int blocks, int nblocks,
-                                                            long rows, int wave_lds) {
-  extern __shared__ __attribute__((aligned(16))) float dir_smem[];
+__device__ __forceinline__ void dir_block(const BandArgs& p, const Plan& g, int blk, int blocks, long rows,
+                                          int wave_lds, float* dir_smem) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int blk = xcd_renumber(blockIdx.x, nblocks);
   const int batch = blk / blocks;
   const int i0 = ((blk - batch * blocks) * kDirWaves + wave) * 16;
   const int n = p.n;
@@ -590,6 +589,25 @@ __global__ __launch_bounds__(64 * kDirWaves) void k_band_dir(const BandArgs p, c
                              rq0 * g.Wq >= kDirMargin && rq1 * g.Wq + kDirMargin <= rows * g.Wq;
   if (inside_matrix && inside_tensor) dir_row<KIND, PREP, false>(p, g, bn, i0, lane, lds, rows);
   else dir_row<KIND, PREP, true>(p, g, bn, i0, lane, lds, rows);
+}
+
+template <int KIND, bool PREP, class Plan>
+__global__ __launch_bounds__(64 * kDirWaves) void k_band_dir(const BandArgs p, const Plan g, int blocks, int nblocks,
+                                                            long rows, int wave_lds) {
+  extern __shared__ __attribute__((aligned(16))) float dir_smem[];
+  dir_block<KIND, PREP>(p, g, xcd_renumber(blockIdx.x, nblocks), blocks, rows, wave_lds, dir_smem);
+}
+
+// Both gradients in one launch, workgroup by workgroup in turn: grad_a and grad_b of
+// neighbouring rows read the same rows of g (and of 1 / S), which then come from memory once.
+// nblocks: workgroups of one gradient.
+template <bool PREP, class Plan>
+__global__ __launch_bounds__(64 * kDirWaves) void k_band_dir_grads(const BandArgs p, const Plan ga, const Plan gb,
+                                                                  int blocks, int nblocks, long rows, int wave_lds) {
+  extern __shared__ __attribute__((aligned(16))) float dir_smem[];
+  const int v = xcd_renumber(blockIdx.x, 2 * nblocks);
+  if ((v & 1) == 0) dir_block<kDirGradA, PREP>(p, ga, v >> 1, blocks, rows, wave_lds, dir_smem);
+  else dir_block<kDirGradB, PREP>(p, gb, v >> 1, blocks, rows, wave_lds, dir_smem);
 }
 
 }  // namespace GENBMM_NS
