@@ -151,19 +151,21 @@ constexpr int kKC = 128;  // cells of the reduction axis per lane
 
 // grad_a: line = row m.  The row is read 16 cells at a time (int4 / float4 when the
 // rows are 16-byte aligned), then the 16 additions are made in order.
+constexpr int kArgAccA = 64 * kKC + 64 + 64, kArgAccB = kKC * 64 + 64;  // floats of LDS
+// (blk: the workgroup's number among those of grad_a; accs: kArgAccA floats of LDS)
 template <int PROD>
-__global__ __launch_bounds__(64) void k_argmax_bwd_a(const elem_t* __restrict__ bmat,
-                                                    const float* __restrict__ fac,
-                                                    const int32_t* __restrict__ idx,
-                                                    const elem_t* __restrict__ g,
-                                                    elem_t* __restrict__ grad_a, int M, int K,
-                                                    int N, int row_tiles, int k_chunks, int ps,
-                                                    int vec) {
-  __shared__ float accs[64 * kKC + 64 + 64];
+__device__ __forceinline__ void argmax_bwd_a_block(float* __restrict__ accs, int blk,
+                                                   const elem_t* __restrict__ bmat,
+                                                   const float* __restrict__ fac,
+                                                   const int32_t* __restrict__ idx,
+                                                   const elem_t* __restrict__ g,
+                                                   elem_t* __restrict__ grad_a, int M, int K,
+                                                   int N, int row_tiles, int k_chunks, int ps,
+                                                   int vec) {
   const int lane = threadIdx.x, parts = 1 << ps, lines = 64 >> ps;
   const int part = lane & (parts - 1), line = lane >> ps;
   const int spare = 64 * kKC + 64 + lane;
-  const int kc_id = blockIdx.x % k_chunks, rt = blockIdx.x / k_chunks;
+  const int kc_id = blk % k_chunks, rt = blk / k_chunks;
   const int batch = rt / row_tiles;
   const int m0 = (rt - batch * row_tiles) * lines;
   const int kw = parts * kKC;                       // k covered by the workgroup
@@ -244,18 +246,19 @@ __global__ __launch_bounds__(64) void k_argmax_bwd_a(const elem_t* __restrict__ 
 
 // grad_b: line = column n; the column is read 16 rows at a time, then added in order.
 // Accumulators are [k][line].
+// (blk: the workgroup's number among those of grad_b; accs: kArgAccB floats of LDS)
 template <int PROD>
-__global__ __launch_bounds__(64) void k_argmax_bwd_b(const elem_t* __restrict__ amat,
-                                                    const float* __restrict__ fac,
-                                                    const int32_t* __restrict__ idx,
-                                                    const elem_t* __restrict__ g,
-                                                    elem_t* __restrict__ grad_b, int M, int K,
-                                                    int N, int col_tiles, int k_chunks, int ps) {
-  __shared__ float accs[kKC * 64 + 64];
+__device__ __forceinline__ void argmax_bwd_b_block(float* __restrict__ accs, int blk,
+                                                   const elem_t* __restrict__ amat,
+                                                   const float* __restrict__ fac,
+                                                   const int32_t* __restrict__ idx,
+                                                   const elem_t* __restrict__ g,
+                                                   elem_t* __restrict__ grad_b, int M, int K,
+                                                   int N, int col_tiles, int k_chunks, int ps) {
   const int lane = threadIdx.x, parts = 1 << ps, lines = 64 >> ps;
   const int part = lane & (parts - 1), line = lane >> ps;
   const int spare = kKC * 64 + lane;
-  const int kc_id = blockIdx.x % k_chunks, ct = blockIdx.x / k_chunks;
+  const int kc_id = blk % k_chunks, ct = blk / k_chunks;
   const int batch = ct / col_tiles;
   const int n0 = (ct - batch * col_tiles) * lines, n = n0 + line;
   const int kw = parts * kKC;
@@ -315,6 +318,30 @@ __global__ __launch_bounds__(64) void k_argmax_bwd_b(const elem_t* __restrict__ 
       grad_b[((long)batch * K + w0 + kk) * N + n0 + lc] = to_elem<elem_t>(accs[kk * lines + lc]);
 }
 
+// Both gradients in one launch, batch item by batch item (ta workgroups of grad_a, then tb of
+// grad_b, per item; XCD-aware numbering): both read the item's idx and g, which then come from
+// memory once.
+template <int PROD>
+__global__ __launch_bounds__(64) void k_argmax_bwd_both(const elem_t* __restrict__ amat,
+                                                       const elem_t* __restrict__ bmat,
+                                                       const float* __restrict__ fac_a,
+                                                       const float* __restrict__ fac_b,
+                                                       const int32_t* __restrict__ idx,
+                                                       const elem_t* __restrict__ g,
+                                                       elem_t* __restrict__ grad_a,
+                                                       elem_t* __restrict__ grad_b, int M, int K, int N,
+                                                       int row_tiles, int kc_a, int ps_a, int vec,
+                                                       int col_tiles, int kc_b, int ps_b) {
+  __shared__ float accs[kArgAccA > kArgAccB ? kArgAccA : kArgAccB];
+  const int ta = row_tiles * kc_a, tb = col_tiles * kc_b;
+  const int v = xcd_renumber(blockIdx.x, gridDim.x);
+  const int item = v / (ta + tb), r = v - item * (ta + tb);
+  if (r < ta)
+    argmax_bwd_a_block<PROD>(accs, item * ta + r, bmat, fac_a, idx, g, grad_a, M, K, N, row_tiles, kc_a, ps_a, vec);
+  else
+    argmax_bwd_b_block<PROD>(accs, item * tb + r - ta, amat, fac_b, idx, g, grad_b, M, K, N, col_tiles, kc_b, ps_b);
+}
+
 // Parts per workgroup for a reduction axis of K cells: the smallest power of two that
 // covers it (at most 64).
 inline int argmax_parts_shift(int K) {
@@ -335,36 +362,26 @@ int run_argmax_bwd(const elem_t* a, const elem_t* b, const int32_t* idx, const f
   // factors = [a[m, idx] | b[idx, n]], each B*M*N: grad_a needs the second, grad_b the first
   constexpr int kGather = PROD ? 1 : 0;
   hipStream_t s = (hipStream_t)stream;
-  if ((int64_t)B * M * K > 0) {
-    const int ps = argmax_parts_shift(K);
-    const int row_tiles = ceil_div(M, 64 >> ps), k_chunks = ceil_div(K, kKC << ps);
-    const int64_t total = (int64_t)B * row_tiles * k_chunks;
-    if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
-    const int vec = (N % 4 == 0) && aligned16(idx) && aligned16(g);
-    if (PROD && factors && mn > 0)
-      hipLaunchKernelGGL((k_argmax_bwd_a<2>), dim3((unsigned)total), dim3(64), 0, s, b,
-                         factors + mn, idx, g, grad_a, M, K, N, row_tiles,
-                         k_chunks, ps, vec && aligned16(factors + mn));
-    else
-      hipLaunchKernelGGL((k_argmax_bwd_a<kGather>), dim3((unsigned)total), dim3(64), 0, s, b,
-                         (const float*)nullptr, idx, g, grad_a, M, K, N, row_tiles, k_chunks, ps, vec);
-    if (int e = launch_status()) return e;
-  }
-  if ((int64_t)B * K * N > 0) {
-    // columns: two parts at most - narrower groups of columns cost more in the strided
-    // reads of idx and g than reading them again saves
-    const int ps = min(argmax_parts_shift(K), 1);
-    const int col_tiles = ceil_div(N, 64 >> ps), k_chunks = ceil_div(K, kKC << ps);
-    const int64_t total = (int64_t)B * col_tiles * k_chunks;
-    if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
-    if (PROD && factors && mn > 0)
-      hipLaunchKernelGGL((k_argmax_bwd_b<2>), dim3((unsigned)total), dim3(64), 0, s, a, factors,
-                         idx, g, grad_b, M, K, N, col_tiles, k_chunks, ps);
-    else
-      hipLaunchKernelGGL((k_argmax_bwd_b<kGather>), dim3((unsigned)total), dim3(64), 0, s, a,
-                         (const float*)nullptr, idx, g, grad_b, M, K, N, col_tiles, k_chunks, ps);
-    if (int e = launch_status()) return e;
-  }
+  if (mk == 0 && kn == 0) return GENBMM_OK;
+  // (an empty M or N leaves one gradient without workgroups; the other is then all zeros)
+  const int ps_a = argmax_parts_shift(K);
+  const int row_tiles = ceil_div(M, 64 >> ps_a), kc_a = ceil_div(K, kKC << ps_a);
+  // columns: two parts at most - narrower groups of columns cost more in the strided
+  // reads of idx and g than reading them again saves
+  const int ps_b = min(argmax_parts_shift(K), 1);
+  const int col_tiles = ceil_div(N, 64 >> ps_b), kc_b = ceil_div(K, kKC << ps_b);
+  const int64_t total = (int64_t)B * ((int64_t)row_tiles * kc_a + (int64_t)col_tiles * kc_b);
+  if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
+  const int vec = (N % 4 == 0) && aligned16(idx) && aligned16(g);
+  if (PROD && factors)
+    hipLaunchKernelGGL((k_argmax_bwd_both<2>), dim3((unsigned)total), dim3(64), 0, s, a, b, factors + mn, factors,
+                       idx, g, grad_a, grad_b, M, K, N, row_tiles, kc_a, ps_a, vec && aligned16(factors + mn),
+                       col_tiles, kc_b, ps_b);
+  else
+    hipLaunchKernelGGL((k_argmax_bwd_both<kGather>), dim3((unsigned)total), dim3(64), 0, s, a, b,
+                       (const float*)nullptr, (const float*)nullptr, idx, g, grad_a, grad_b, M, K, N, row_tiles,
+                       kc_a, ps_a, vec, col_tiles, kc_b, ps_b);
+  if (int e = launch_status()) return e;
   return GENBMM_OK;
 }
 
