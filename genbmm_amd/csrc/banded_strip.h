@@ -248,10 +248,7 @@ __global__ __launch_bounds__(256) void k_band_prep(const PrepSide pa, const Prep
 // ------------------------------------------------------------------ forward
 // Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each): renumber so
 // that an XCD works on consecutive strips, whose halos overlap.
-__device__ __forceinline__ int xcd_strip_id() {
-  const int w = blockIdx.x, n = gridDim.x;
-  return (n & 7) == 0 ? (w & 7) * (n >> 3) + (w >> 3) : w;
-}
+__device__ __forceinline__ int xcd_strip_id() { return xcd_renumber(blockIdx.x, gridDim.x); }
 
 // The exact recompute of one cell, kept out of line: it is rare, and inlined it costs
 // the strip kernels registers they do not have.

@@ -341,9 +341,11 @@ __host__ __device__ inline void philox_uniform4(uint64_t i, bool aligned, uint64
 
 // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
 // Renumber them so that every XCD works on one contiguous run of tiles (the
-// tiles of a batch item share their operands).
+// tiles of a batch item share their operands): XCD x takes n / 8 of them, one
+// more if x < n % 8, and workgroup w is the (w / 8)-th of XCD w % 8.
 __device__ __forceinline__ int xcd_renumber(int w, int n) {
-  return (n & 7) == 0 ? (w & 7) * (n >> 3) + (w >> 3) : w;
+  const int q = n >> 3, r = n & 7, x = w & 7;
+  return x * q + min(x, r) + (w >> 3);
 }
 // Four ordered additions with one LDS round trip: the four cells are read together,
 // the sums are chained in registers (a cell that was already hit earlier in the group
