@@ -30,7 +30,7 @@ struct DenseArgs {
 template <class C>
 __device__ __forceinline__ void decode_tile(const DenseArgs& p, int& batch, int& m0, int& n0) {
   const int per = p.tiles_m * p.tiles_n;
-  const int wg = blockIdx.x;
+  const int wg = xcd_renumber(blockIdx.x, gridDim.x);  // an XCD works on a contiguous run of tiles
   batch = wg / per;
   const int r = wg - batch * per;
   const int mt = r / p.tiles_n;

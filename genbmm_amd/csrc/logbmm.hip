@@ -161,8 +161,9 @@ template <class C, bool GRAD_A>
 __global__ __launch_bounds__(C::NT) void k_log_bwd_exact(const LogBwdArgs p) {
   __shared__ __attribute__((aligned(16))) float smem[LogBwdLds<C, GRAD_A>::FLOATS];
   const int per = p.tiles_r * p.tiles_c;
-  const int batch = blockIdx.x / per;
-  const int rem = blockIdx.x - batch * per;
+  const int tile = xcd_renumber(blockIdx.x, gridDim.x);
+  const int batch = tile / per;
+  const int rem = tile - batch * per;
   log_bwd_tile<C, GRAD_A>(p, batch, (rem / p.tiles_c) * C::BR, (rem % p.tiles_c) * C::BC, smem);
 }
 
@@ -264,7 +265,7 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_fwd_fast(const DenseArgs p,
     }
   }
   bad = __syncthreads_or(bad);
-  if (tid == 0) flags[blockIdx.x] = bad;
+  if (tid == 0) flags[xcd_renumber(blockIdx.x, gridDim.x)] = bad;  // the tile's number, as decode_tile has it
   if (bad) return;  // the fix-up launch recomputes this tile
   store_tile_f<C>(p.out + (long)batch * M * N, acc, m0, n0, M, N, p.vec_o, tx, ty);
 }
@@ -398,8 +399,9 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_bwd_fast(const LogBwdArgs p,
   const int M = p.M, K = p.K, N = p.N;
   const int R = GRAD_A ? M : K, Cc = GRAD_A ? K : N, Q = GRAD_A ? N : M;
   const int per = p.tiles_r * p.tiles_c;
-  const int batch = blockIdx.x / per;
-  const int rem = blockIdx.x - batch * per;
+  const int tile = xcd_renumber(blockIdx.x, gridDim.x);
+  const int batch = tile / per;
+  const int rem = tile - batch * per;
   const int r0 = (rem / p.tiles_c) * C::BR, c0 = (rem % p.tiles_c) * C::BC;
   // Every cell this tile reduces over must come from a forward tile that passed the
   // factoring guard (S >= 2^-40, finite shifts): H = g * exp(alpha + beta - out) is then
