@@ -22,7 +22,7 @@ struct BB {
 };
 
 __global__ __launch_bounds__(256) void k_log_bwdbwd_t(const BB p, long total) {
-  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  const long e = (long)xcd_renumber(blockIdx.x, gridDim.x) * 256 + threadIdx.x;  // an item's workgroups on one XCD
   if (e >= total) return;
   const int n = (int)(e % p.N);
   const long bm = e / p.N;  // batch*M + m
@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void k_log_bwdbwd_t(const BB p, long total) {
 constexpr int kBBChunks = 4;  // n chunks of 64 a lane keeps in registers
 __global__ __launch_bounds__(256) void k_log_bwdbwd_a(const BB p, long rows) {
   const int lane = threadIdx.x & 63;
-  const long bm = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const long bm = (long)xcd_renumber(blockIdx.x, gridDim.x) * 4 + (threadIdx.x >> 6);
   if (bm >= rows) return;
   const long batch = bm / p.M;
   const int K = p.K, N = p.N;
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(256) void k_log_bwdbwd_a(const BB p, long rows) {
 }
 
 __global__ __launch_bounds__(256) void k_log_bwdbwd_b(const BB p, long total) {
-  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  const long e = (long)xcd_renumber(blockIdx.x, gridDim.x) * 256 + threadIdx.x;  // an item's workgroups on one XCD
   if (e >= total) return;
   const int n = (int)(e % p.N);
   const long bk = e / p.N;  // batch*K + k
