@@ -41,6 +41,7 @@ SIGNATURES = {
     "genbmm_argmax_bwd": [_c_int_p] + [_c_float_p] * 3 + _DENSE_DIMS,
     "genbmm_prodmax_bwd": [_c_float_p] * 2 + [_c_int_p] + [_c_float_p] * 4 + _DENSE_DIMS,
     "genbmm_banded_fwd": _BAND + [_c_float_p, _c_int_p, _c_float_p, _i, _i, _i, _vp],
+    "genbmm_banded_sample_fwd": _BAND + [_c_float_p, _c_int_p, _c_float_p, _u64, _u64, _i, _i, _vp],
     "genbmm_banded_bwd": _BAND + [_c_float_p, _c_int_p] + [_c_float_p] * 4 + [_i, _i, _i, _vp],
     "genbmm_banded_bwd_scratch": _BAND + [_c_float_p, _c_int_p] + [_c_float_p] * 5 + [_i, _i, _i, _vp],
     "genbmm_banded_bwdbwd": _BAND + [_c_float_p] * 7 + [_i, _i, _vp],
@@ -53,6 +54,7 @@ SIGNATURES = {
     "genbmm_argmax_bwd_f64": [_c_int_p] + [_c_float_p] * 3 + _DENSE_DIMS,
     "genbmm_prodmax_bwd_f64": [_c_float_p] * 2 + [_c_int_p] + [_c_float_p] * 3 + _DENSE_DIMS,
     "genbmm_banded_fwd_f64": _BAND + [_c_float_p, _c_int_p, _i, _i, _i, _vp],
+    "genbmm_banded_sample_fwd_f64": _BAND + [_c_float_p, _c_int_p, _u64, _u64, _i, _i, _vp],
     "genbmm_banded_bwd_f64": _BAND + [_c_float_p, _c_int_p] + [_c_float_p] * 3 + [_i, _i, _i, _vp],
     "genbmm_banded_bwdbwd_f64": _BAND + [_c_float_p] * 7 + [_i, _i, _vp],
     "genbmm_band_shift": [_c_float_p, _c_float_p] + [_i] * 6 + [ctypes.c_float, _vp],

@@ -24,6 +24,7 @@
 #include "banded_direct.h"
 #include "banded_flat.h"
 #include "banded_max.h"
+#include "banded_sample.h"
 #include "banded_strip.h"
 
 namespace GENBMM_NS {
@@ -261,12 +262,49 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
   return launch_status();
 }
 
+int genbmm_banded_sample_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
+                             float* out, int32_t* idx, float* workspace, uint64_t seed, uint64_t offset,
+                             int B, int n, void* stream) {
+  using namespace GENBMM_NS;
+  BandArgs p{};
+  if (int e = fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return e;
+  if ((int64_t)B * n == 0) return GENBMM_OK;
+  if (!a || !b || !out || !idx) return GENBMM_E_NULLPTR;
+  // out: the log product, on the workspace where there is one
+  if (int e = genbmm_banded_fwd(a, a_lu, a_ld, b, b_lu, b_ld, out, nullptr, workspace, B, n, GENBMM_BAND_LOG, stream))
+    return e;
+  p.a = a; p.b = b; p.out = out; p.oidx = idx;
+  const long total = (long)B * n * p.Wo;
+  hipStream_t s = (hipStream_t)stream;
+  const bool dir = dir_fwd_ok(p, kDirMinW);
+  const bool prepared = prep_fwd(p, GENBMM_BAND_LOG, workspace) && (dir || fwd_strip_ok(p));
+  const int Wseg = max_fwd_segment(p);
+  if (prepared && Wseg > 0) {
+    set_workspace(p, workspace, B);
+    const int nseg = ceil_div(p.Wo, Wseg), strips = ceil_div(p.n, kMaxRows);
+    const MaxDims d = max_dims(p.Wa, p.Wb, Wseg);
+    if ((long)B * strips * nseg > 0x7fffffffL) return GENBMM_E_SHAPE;
+    hipLaunchKernelGGL(k_band_sample_targets, blocks_for((total + 3) / 4), dim3(256), 0, s, p.ws_r, idx, total, seed,
+                       offset);
+    if (d.bytes > kStripLdsLimit)
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_band_sample_fwd<float>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)d.bytes);
+    const long rows = (long)B * p.n;
+    hipLaunchKernelGGL(k_band_sample_fwd<float>, dim3((unsigned)((long)B * strips * nseg)), dim3(256), d.bytes, s, p,
+                       strips, d, rows * p.Wa, rows * p.Wb, nseg, Wseg, seed, offset);
+    return launch_status();
+  }
+  hipLaunchKernelGGL(k_band_sample_cells<float>, blocks_for(total), dim3(256), 0, s, p, total, seed, offset);
+  return launch_status();
+}
+
 namespace GENBMM_NS {
 namespace {
 // `scratch`: where g / S goes in the prepared log product; NULL: the workspace's own part
 int banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
                const float* out, const int32_t* idx, float* workspace, float* scratch, const float* g,
                float* grad_a, float* grad_b, int B, int n, int mode, void* stream) {
+  if (mode == GENBMM_BAND_SAMPLE) mode = GENBMM_BAND_MAX;  // a drawn index scatters like an arg-max
   if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
     return GENBMM_E_MODE;
   BandArgs p{};

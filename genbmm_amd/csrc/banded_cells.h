@@ -191,6 +191,64 @@ __global__ __launch_bounds__(256) void k_band_bwd_b(const BandArgsT<T> p, long t
   band_bwd_b_cell<MODE>(p, bo, (int)(bo % p.n), (int)(e - bo * p.Wb));
 }
 
+// ------------------------------------------------------------------ sample
+// The banded sample product (no counterpart among the reference's band modes): the dense
+// sampling rule (sample_cuda_forward_kernel, matmul_cuda_kernel.cu:107-118) on the terms of
+// a band cell in ascending k.
+// The exact walk of one cell inside the matrix, u its uniform; returns the index.
+template <class T>
+__device__ __forceinline__ int band_sample_cell(const BandArgsT<T>& p, long bi, int i, int j, float u) {
+  const int o = i + j - p.r_lu;
+  int klo, khi;
+  k_range(p, i, j, klo, khi);
+  const T* ar = p.a + bi * p.Wa;
+  const T* br = p.b + (bi + (o - i)) * p.Wb + (p.Wb - 1 - j);
+  if constexpr (sizeof(T) == sizeof(double)) {
+    double m = kFloor;
+    for (int k = klo; k <= khi; ++k) m = fmax(m, (double)ar[k] + (double)br[k]);
+    double s = 0;
+    for (int k = klo; k <= khi; ++k) s += exp((double)ar[k] + (double)br[k] - m);
+    const double t = (double)u * s;
+    double tot = 0;
+    int last = klo;
+    for (int k = klo; k <= khi; ++k) {
+      const double pr = exp((double)ar[k] + (double)br[k] - m);
+      if (tot + pr > t) return k;  // (total < t holds until then, except on an exact tie, which the next term takes)
+      tot += pr;
+      if (pr > 0) last = k;
+    }
+    return u > 0.f ? last : klo;
+  } else {
+    float m = kFloor;
+    for (int k = klo; k <= khi; ++k) m = fmaxf(m, (float)ar[k] + (float)br[k]);
+    const float nm = -m * kLog2e;
+    float s = 0.f;
+    for (int k = klo; k <= khi; ++k) s += fast_exp2(__builtin_fmaf((float)ar[k] + (float)br[k], kLog2e, nm));
+    const float t = u * s;
+    float tot = 0.f;
+    int last = klo;
+    for (int k = klo; k <= khi; ++k) {
+      const float pr = fast_exp2(__builtin_fmaf((float)ar[k] + (float)br[k], kLog2e, nm));
+      if (tot + pr > t) return k;  // (total < t holds until then, except on an exact tie, which the next term takes)
+      tot += pr;
+      if (pr > 0.f) last = k;
+    }
+    // ran out by rounding: the last term that had mass (r = 0 brackets nothing: first term)
+    return u > 0.f ? last : klo;
+  }
+}
+
+// One lane per cell: the exact walk everywhere.
+template <class T>
+__global__ __launch_bounds__(256) void k_band_sample_cells(const BandArgsT<T> p, long total, uint64_t seed,
+                                                           uint64_t offset) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const long bi = e / p.Wo;
+  const int i = (int)(bi % p.n), j = (int)(e - bi * p.Wo), o = i + j - p.r_lu;
+  p.oidx[e] = (o < 0 || o >= p.n) ? 0 : band_sample_cell(p, bi, i, j, philox_uniform((uint64_t)e, seed, offset));
+}
+
 // ------------------------------------------------------ log second order
 // p = exp(a[i,k] + b[o,k2] - out[i,j]),  w = u_a[i,k] + u_b[o,k2]:
 //   t[i,j]       = sum_k p*w                        (gradient w.r.t. g)

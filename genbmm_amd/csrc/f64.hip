@@ -426,10 +426,27 @@ int genbmm_banded_fwd_f64(const double* a, int a_lu, int a_ld, const double* b, 
   return launch_status();
 }
 
+int genbmm_banded_sample_fwd_f64(const double* a, int a_lu, int a_ld, const double* b, int b_lu, int b_ld,
+                                 double* out, int32_t* idx, uint64_t seed, uint64_t offset, int B, int n,
+                                 void* stream) {
+  using namespace GENBMM_NS;
+  BandArgsT<double> p{};
+  if (int e = fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return e;
+  const long total = (long)B * n * p.Wo;
+  if (total == 0) return GENBMM_OK;
+  if (!a || !b || !out || !idx) return GENBMM_E_NULLPTR;
+  p.a = a; p.b = b; p.o0 = out; p.oidx = idx;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL((k_band_fwd<GENBMM_BAND_LOG, double>), blocks_for(total), dim3(256), 0, s, p, total);
+  hipLaunchKernelGGL(k_band_sample_cells<double>, blocks_for(total), dim3(256), 0, s, p, total, seed, offset);
+  return launch_status();
+}
+
 int genbmm_banded_bwd_f64(const double* a, int a_lu, int a_ld, const double* b, int b_lu, int b_ld,
                           const double* out, const int32_t* idx, const double* g, double* grad_a,
                           double* grad_b, int B, int n, int mode, void* stream) {
   using namespace GENBMM_NS;
+  if (mode == GENBMM_BAND_SAMPLE) mode = GENBMM_BAND_MAX;  // a drawn index scatters like an arg-max
   if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
     return GENBMM_E_MODE;
   BandArgsT<double> p{};

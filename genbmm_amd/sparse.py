@@ -27,7 +27,7 @@ import torch.nn.functional as F
 
 from . import _lib
 
-MODE_LOG, MODE_MAX, MODE_MUL = 0, 1, 3
+MODE_LOG, MODE_MAX, MODE_SAMPLE, MODE_MUL = 0, 1, 2, 3
 
 # The reference sets this when its extension imports (sparse.py:3-9); here: the HIP
 # library has been built.  (It selects nothing: there is no other path to fall back to.)
@@ -335,6 +335,15 @@ class BandedMatrix:
         """The same product in the (max, +) semiring (reference sparse.py:255-266)."""
         return self._product(other, bandedmaxbmm)
 
+    def multiply_sample(self, other, stream=None):
+        """The log product whose gradient is a one-hot sample: every result cell draws one of
+        its terms k with probability exp(a + b - out) and hands its incoming gradient to that
+        term's two cells, as `samplebmm` does for dense operands.  The reference's band kernel
+        stops at the log, max and (+, *) products (banded_cuda_kernel.cu:42, 65, 76); this is
+        its dense sampling rule (matmul_cuda_kernel.cu:107-118) on a band cell's terms.
+        `stream` = (seed, offset) pins the Philox stream; None follows torch's CUDA generator."""
+        return self._product(other, lambda *args: BandedSampleMul.apply(*args, stream))
+
     def multiply_back(self, other, out, grad_out):
         """Gradient of `self.multiply(other)` with respect to self, given the gradient of
         the product's band tensor (reference sparse.py:363-379; `out` is not needed)."""
@@ -500,6 +509,43 @@ class BandedMaxMul(torch.autograd.Function):
         a, b = a.contiguous(), b.contiguous()
         grad_a, grad_b = _backward(a, b, ctx.bands, None, idx, grad_output, MODE_MAX)
         return (grad_a, None, None, grad_b) + (None,) * 4
+
+
+class BandedSampleMul(torch.autograd.Function):
+    """Banded sample product (`BandedMatrix.multiply_sample`): the log product forward, the
+    arg-max scatter of the drawn indices backward - the banded form of the reference's
+    SampleMatMul (genmul.py:68-81)."""
+
+    @staticmethod
+    def forward(ctx, a, a_lu, a_ld, b, b_lu, b_ld, o_lu, o_ld, stream=None):
+        from .genmul import _next_stream
+
+        a, b = a.contiguous(), b.contiguous()
+        B, n = _check_pair(a, b)
+        if a.shape[2] != a_lu + a_ld + 1 or b.shape[2] != b_lu + b_ld + 1:
+            raise RuntimeError("band widths do not match lu + ld + 1")
+        seed, offset = _next_stream(a.device) if stream is None else stream
+        seed, offset = int(seed) & 0xFFFFFFFFFFFFFFFF, int(offset) & 0xFFFFFFFFFFFFFFFF
+        wo = a.shape[2] + b.shape[2] - 1
+        out = torch.empty(B, n, wo, dtype=a.dtype, device=a.device)
+        idx = torch.empty(B, n, wo, dtype=torch.int32, device=a.device)
+        if _f64(a):
+            _call("genbmm_banded_sample_fwd_f64", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
+                  _lib.ptr(out), _lib.ptr(idx), seed, offset, B, n)
+        else:
+            size = _lib.load().genbmm_banded_workspace_size(a_lu, a_ld, b_lu, b_ld, B, n)
+            ws = torch.empty(size, dtype=torch.float32, device=a.device)
+            _call("genbmm_banded_sample_fwd", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
+                  _lib.ptr(out), _lib.ptr(idx), _lib.ptr(ws), seed, offset, B, n)
+        ctx.save_for_backward(a, b, idx)
+        ctx.bands = (a_lu, a_ld, b_lu, b_ld)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        a, b, idx = ctx.saved_tensors
+        grad_a, grad_b = _backward(a, b, ctx.bands, None, idx, grad_output, MODE_SAMPLE)
+        return (grad_a, None, None, grad_b) + (None,) * 5
 
 
 bandedbmm = BandedMul.apply

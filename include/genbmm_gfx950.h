@@ -49,6 +49,7 @@ extern "C" {
 /* Banded semiring modes (reference banded_cuda_kernel.cu:42,64,76). */
 #define GENBMM_BAND_LOG 0
 #define GENBMM_BAND_MAX 1
+#define GENBMM_BAND_SAMPLE 2  /* backward only: a drawn index scatters like an arg-max */
 #define GENBMM_BAND_MUL 3
 
 /* Library version string, e.g. "genbmm-gfx950 0.1". */
@@ -272,6 +273,28 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld,
                       float* out, int32_t* idx, float* workspace,
                       int B, int n, int mode, void* stream);
 
+/*
+ * Banded sample product: out = the log product (mode GENBMM_BAND_LOG above),
+ * idx[i,j] = one term k of the cell (index into a's band, as mode MAX stores
+ * its arg-max) drawn with probability exp(a[i,k] + b[o,k2] - out[i,j]).  The
+ * reference's band kernel has modes 0, 1 and 3 only
+ * (banded_cuda_kernel.cu:42, 65, 76); this is its dense sampling rule
+ * (sample_cuda_forward_kernel, matmul_cuda_kernel.cu:107-118: ascending
+ * terms, the first with total < r && total + p > r) applied to a band cell's
+ * terms, with r the Philox4x32-10 uniform of the cell's linear index for
+ * (seed, offset), exactly as genbmm_samplebmm_fwd draws it.  A cell whose walk
+ * never brackets r keeps its first term; cells outside the matrix get 0.
+ * `workspace`: NULL or genbmm_banded_workspace_size floats (then the walk runs
+ * on the log product's factors and takes no exponential).  The gradients are
+ * genbmm_banded_bwd's with mode GENBMM_BAND_SAMPLE (one-hot scatter of g, as
+ * the dense sample op uses the arg-max backward, matmul_cuda_kernel.cu:676).
+ */
+int genbmm_banded_sample_fwd(const float* a, int a_lu, int a_ld,
+                             const float* b, int b_lu, int b_ld,
+                             float* out, int32_t* idx, float* workspace,
+                             uint64_t seed, uint64_t offset,
+                             int B, int n, void* stream);
+
 /* Number of fp32 elements of the log product's workspace (0 on bad arguments). */
 size_t genbmm_banded_workspace_size(int a_lu, int a_ld, int b_lu, int b_ld,
                                     int B, int n);
@@ -437,6 +460,11 @@ int genbmm_banded_fwd_f64(const double* a, int a_lu, int a_ld,
                           const double* b, int b_lu, int b_ld,
                           double* out, int32_t* idx,
                           int B, int n, int mode, void* stream);
+int genbmm_banded_sample_fwd_f64(const double* a, int a_lu, int a_ld,
+                                 const double* b, int b_lu, int b_ld,
+                                 double* out, int32_t* idx,
+                                 uint64_t seed, uint64_t offset,
+                                 int B, int n, void* stream);
 int genbmm_banded_bwd_f64(const double* a, int a_lu, int a_ld,
                           const double* b, int b_lu, int b_ld,
                           const double* out, const int32_t* idx, const double* g,

@@ -337,6 +337,56 @@ def seq_band_fwd(a, a_lu, a_ld, b, b_lu, b_ld, mode, dtype=np.float32):
     return torch.from_numpy(out), torch.from_numpy(idx), torch.from_numpy(mx)
 
 
+def seq_band_sample_fwd(a, a_lu, a_ld, b, b_lu, b_ld, rnd, dtype=np.float32):
+    """Banded sample product: (out, idx) for the uniforms `rnd` (B, n, Wo)."""
+    pre, dt = _prefix(dtype)
+    a, b, rnd = _np(a, dt), _np(b, dt), _np(rnd, dt)
+    B, n, _ = a.shape
+    W = a.shape[2] + b.shape[2] - 1
+    out, idx = np.empty((B, n, W), dt), np.empty((B, n, W), np.int32)
+    getattr(lib(), pre + "band_sample_fwd")(_p(a), a_lu, a_ld, _p(b), b_lu, b_ld, _p(rnd), _p(out), _p(idx), B, n)
+    return torch.from_numpy(out), torch.from_numpy(idx)
+
+
+def band_terms64(a, a_lu, a_ld, b, b_lu, b_ld):
+    """Every term of every band cell in float64, by index arithmetic (works on any device):
+    v[b, i, j, k] = a[b, i, k] + b[b, o, k2] with o = i + j - lu_out, k2 = k - j + Wb - 1, and
+    valid[i, j, k] = 0 <= o < n and 0 <= k2 < Wb and 0 <= i + k - a_lu < n
+    (banded_cuda_kernel.cu:32-51).  Returns (v, valid); v holds -inf where not valid."""
+    B, n, Wa = a.shape
+    Wb = b.shape[2]
+    Wo, r_lu = Wa + Wb - 1, a_lu + b_ld
+    dev = a.device
+    i = torch.arange(n, device=dev).view(n, 1, 1)
+    j = torch.arange(Wo, device=dev).view(1, Wo, 1)
+    k = torch.arange(Wa, device=dev).view(1, 1, Wa)
+    o, k2, pos = i + j - r_lu, k - j + (Wb - 1), i + k - a_lu
+    valid = (o >= 0) & (o < n) & (k2 >= 0) & (k2 < Wb) & (pos >= 0) & (pos < n)
+    bv = b.double()[:, o.clamp(0, n - 1).expand(n, Wo, Wa), k2.clamp(0, Wb - 1).expand(n, Wo, Wa)]
+    v = a.double().unsqueeze(2) + bv
+    return torch.where(valid, v, torch.full_like(v, -float("inf"))), valid
+
+
+def band_sample_cdf64(a, a_lu, a_ld, b, b_lu, b_ld):
+    """Inclusive CDF over k of softmax_k of a band cell's terms, float64, (B, n, Wo, Wa);
+    cells outside the matrix (no term) hold zeros."""
+    v, valid = band_terms64(a, a_lu, a_ld, b, b_lu, b_ld)
+    has = valid.any(-1, keepdim=True)
+    p = torch.softmax(torch.where(has, v, torch.zeros_like(v)), -1)
+    return torch.where(has & valid, p, torch.zeros_like(p)).cumsum(-1), valid
+
+
+def band_sample_index_from_cdf(cdf, valid, u):
+    """The dense rule (matmul_cuda_kernel.cu:109-118) on a band cell's CDF: first k with
+    C[k-1] < r and C[k] > r; the cell's first term if there is none; 0 outside the matrix."""
+    r = u.double().unsqueeze(-1)
+    prev = torch.cat([torch.zeros_like(cdf[..., :1]), cdf[..., :-1]], dim=-1)
+    hit = valid & (prev < r) & (cdf > r)
+    first_hit = hit.to(torch.int8).argmax(-1)
+    first_term = valid.to(torch.int8).argmax(-1).expand_as(first_hit)
+    return torch.where(hit.any(-1), first_hit, first_term).to(torch.int32)
+
+
 def _seq_band_bwd_first(pre, dt, a, a_lu, a_ld, b, b_lu, b_ld, part, g, mode):
     a, b, part, g = _np(a, dt), _np(b, dt), _np(part, dt), _np(g, dt)
     B, n, _ = a.shape

@@ -233,6 +233,41 @@ void FN(band_fwd)(const REAL* a, int a_lu, int a_lb, const REAL* b, int b_lu, in
       }
 }
 
+/* Banded sample product.  The reference's band kernel has modes 0, 1 and 3 only
+ * (banded_cuda_kernel.cu:42, 65, 76), so there is no reference function to follow line
+ * by line: this is its dense sampling rule (sample_cuda_forward_kernel,
+ * matmul_cuda_kernel.cu:107-118: walk the terms in ascending order, take the first one
+ * with total < r && total + exp(v - out) > r) applied to the term list of a band cell
+ * (banded_cuda_kernel.cu:32-51, ascending k with the two range tests).  out = banded
+ * log-sum-exp (mode 0 above); indices[i][j] = the chosen k (index into a's band, as
+ * mode 1 stores it); a cell whose walk never brackets r keeps the first term of its
+ * list, cells outside the matrix keep the zero fill.  `rnd` is (B, n, W). */
+void FN(band_sample_fwd)(const REAL* a, int a_lu, int a_lb, const REAL* b, int b_lu, int b_lb,
+                         const REAL* rnd, REAL* out, int32_t* indices, int B, int n) {
+  const int result_lu = a_lu + b_lb, result_lb = a_lb + b_lu;
+  const int self_width = a_lu + a_lb + 1, b_width = b_lu + b_lb + 1;
+  const int W = result_lu + result_lb + 1;
+  FN(band_fwd)(a, a_lu, a_lb, b, b_lu, b_lb, out, indices, NULL, B, n, 0);
+  for (int batch = 0; batch < B; ++batch)
+    for (int i = 0; i < n; ++i)
+      for (int j = 0; j < W; ++j) {
+        const int o = i + (j - result_lu);
+        if (o < 0 || o >= n) continue;
+        REAL total = 0, r = A3(rnd, n, W, batch, i, j);
+        int first = -1, hit = -1;
+        for (int k = 0; k < self_width; ++k) {
+          int pos = i + (k - a_lu), k2 = (pos - o) + b_lu;
+          if (k2 < 0 || k2 >= b_width) continue;
+          if (pos < 0 || pos >= n) continue;
+          if (first < 0) first = k;
+          REAL v = A3(a, n, self_width, batch, i, k) + A3(b, n, b_width, batch, o, k2) - A3(out, n, W, batch, i, j);
+          if (total < r && total + EXP(v) > r) { hit = k; break; }
+          total += EXP(v);
+        }
+        A3(indices, n, W, batch, i, j) = hit >= 0 ? hit : first;
+      }
+}
+
 /* banded_cuda_backward_kernel_mul :104-152: gradient with respect to the FIRST
  * operand; `part` is out (mode 0) or the arg-max as REAL (mode 1); grad_a is
  * zero-filled first (:436). */

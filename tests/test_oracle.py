@@ -234,6 +234,63 @@ def test_seq_band_fwd_matches_dense_identity(n, a_lu, a_ld, b_lu, b_ld, mode):
     assert (out[:, ~mask] == 0).all()  # cells outside the matrix keep the zero fill
 
 
+@pytest.mark.parametrize("n,a_lu,a_ld,b_lu,b_ld", BANDS)
+def test_seq_band_sample_matches_dense_sample_rule(n, a_lu, a_ld, b_lu, b_ld):
+    """The banded sample product has no reference function (the band kernel stops at modes 0, 1,
+    3); its oracle is pinned through the dense identity of test_sparse.py:181-195 and the dense
+    sampling oracle (itself pinned above): sampling Dense(b)^T (x) Dense(a) with -1e9 outside the
+    bands picks, for result cell (r, c), a dense row p of a's column c, i.e. k = p - c + a_lu."""
+    a, b = _band_pair(n, a_lu, a_ld, b_lu, b_ld)
+    a, b = 2 * a.double(), 2 * b.double()
+    lu, ld = a_lu + b_ld, a_ld + b_lu
+    W = lu + ld + 1
+    u = oracle.philox_uniform(0, 2 * n * W, 7, 3).view(2, n, W).double().clamp(min=1e-3)
+    out, idx = oracle.seq_band_sample_fwd(a, a_lu, a_ld, b, b_lu, b_ld, u, dtype=np.float64)
+    want, mask = oracle.band_product_dense(a, a_lu, a_ld, b, b_lu, b_ld, 0)
+    assert torch.allclose(out[:, mask], want[:, mask], rtol=1e-12, atol=1e-12)
+    assert (out[:, ~mask] == 0).all() and (idx[:, ~mask] == 0).all()
+    X = oracle.band_to_dense(a, a_lu, a_ld, -1e9)
+    Y = oracle.band_to_dense(b, b_lu, b_ld, -1e9)
+    ud = oracle.band_to_dense(u, lu, ld, 0.5)                 # uniforms at their dense cells (r, c)
+    _, p = oracle.seq_samplebmm_fwd(Y.transpose(-2, -1).contiguous(), X, ud, dtype=np.float64)
+    k_dense = p - torch.arange(n).view(1, 1, n) + a_lu            # (B, r, c)
+    k_band = oracle.band_from_dense(k_dense.double(), lu, ld).long()
+    assert torch.equal(idx.long()[:, mask], k_band[:, mask])
+    # and the float64 CDF rule evaluated by index arithmetic agrees
+    cdf, valid = oracle.band_sample_cdf64(a, a_lu, a_ld, b, b_lu, b_ld)
+    assert torch.equal(idx, oracle.band_sample_index_from_cdf(cdf, valid, u))
+    # the terms tensor itself: its log-sum-exp is the product
+    v, _ = oracle.band_terms64(a, a_lu, a_ld, b, b_lu, b_ld)
+    assert torch.allclose(v.logsumexp(-1)[:, mask], want[:, mask], rtol=1e-12, atol=1e-12)
+
+
+def test_seq_band_sample_distribution_and_defaults():
+    n, a_lu, a_ld, b_lu, b_ld = 4, 1, 2, 2, 1
+    a, b = _band_pair(n, a_lu, a_ld, b_lu, b_ld, batch=1)
+    a, b = 2 * a.double(), 2 * b.double()
+    W = a.shape[2] + b.shape[2] - 1
+    draws = 20000
+    A, Bm = a.expand(draws, -1, -1).contiguous(), b.expand(draws, -1, -1).contiguous()
+    u = oracle.philox_uniform(0, draws * n * W, 5, 1).view(draws, n, W).double()
+    _, idx = oracle.seq_band_sample_fwd(A, a_lu, a_ld, Bm, b_lu, b_ld, u, dtype=np.float64)
+    cdf, valid = oracle.band_sample_cdf64(a, a_lu, a_ld, b, b_lu, b_ld)
+    pr = torch.diff(cdf[0], dim=-1, prepend=torch.zeros(n, W, 1, dtype=torch.float64))
+    for i in range(n):
+        for j in range(W):
+            if not valid[i, j].any():
+                assert (idx[:, i, j] == 0).all()
+                continue
+            cnt = torch.bincount(idx[:, i, j].long(), minlength=a.shape[2]).double()
+            assert (cnt[~valid[i, j]] == 0).all()              # only terms of the cell are drawn
+            exp = pr[i, j] * draws
+            keep = exp >= 5
+            assert float((((cnt - exp) ** 2) / exp)[keep].sum()) < 45, (i, j)
+    # r = 0 never brackets: every cell keeps its first term
+    _, idx0 = oracle.seq_band_sample_fwd(a, a_lu, a_ld, b, b_lu, b_ld, torch.zeros(1, n, W), dtype=np.float64)
+    first = valid.to(torch.int8).argmax(-1)
+    assert torch.equal(idx0[0].long(), torch.where(valid.any(-1), first, torch.zeros_like(first)))
+
+
 def _dense_band_fn(a_lu, a_ld, b_lu, b_ld, mode):
     fill = 0.0 if mode == 3 else -1e9
 
