@@ -348,11 +348,12 @@ def seq_band_sample_fwd(a, a_lu, a_ld, b, b_lu, b_ld, rnd, dtype=np.float32):
     return torch.from_numpy(out), torch.from_numpy(idx)
 
 
-def band_terms64(a, a_lu, a_ld, b, b_lu, b_ld):
-    """Every term of every band cell in float64, by index arithmetic (works on any device):
-    v[b, i, j, k] = a[b, i, k] + b[b, o, k2] with o = i + j - lu_out, k2 = k - j + Wb - 1, and
-    valid[i, j, k] = 0 <= o < n and 0 <= k2 < Wb and 0 <= i + k - a_lu < n
-    (banded_cuda_kernel.cu:32-51).  Returns (v, valid); v holds -inf where not valid."""
+def band_pairs(a, a_lu, a_ld, b, b_lu, b_ld):
+    """The factor pairs of every band cell, by index arithmetic (works on any device, keeps
+    the dtype, differentiable): av[b, i, j, k] = a[b, i, k], bv[b, i, j, k] = b[b, o, k2] with
+    o = i + j - lu_out, k2 = k - j + Wb - 1, and valid[i, j, k] = 0 <= o < n and 0 <= k2 < Wb
+    and 0 <= i + k - a_lu < n (banded_cuda_kernel.cu:32-51).  bv holds an arbitrary cell of b
+    where not valid."""
     B, n, Wa = a.shape
     Wb = b.shape[2]
     Wo, r_lu = Wa + Wb - 1, a_lu + b_ld
@@ -362,9 +363,44 @@ def band_terms64(a, a_lu, a_ld, b, b_lu, b_ld):
     k = torch.arange(Wa, device=dev).view(1, 1, Wa)
     o, k2, pos = i + j - r_lu, k - j + (Wb - 1), i + k - a_lu
     valid = (o >= 0) & (o < n) & (k2 >= 0) & (k2 < Wb) & (pos >= 0) & (pos < n)
-    bv = b.double()[:, o.clamp(0, n - 1).expand(n, Wo, Wa), k2.clamp(0, Wb - 1).expand(n, Wo, Wa)]
-    v = a.double().unsqueeze(2) + bv
+    bv = b[:, o.clamp(0, n - 1).expand(n, Wo, Wa), k2.clamp(0, Wb - 1).expand(n, Wo, Wa)]
+    return a.unsqueeze(2).expand(B, n, Wo, Wa), bv, valid
+
+
+def band_terms64(a, a_lu, a_ld, b, b_lu, b_ld):
+    """Every term a[i, k] + b[o, k2] of every band cell in float64, (B, n, Wo, Wa), -inf where
+    the pair is not valid.  Returns (v, valid)."""
+    av, bv, valid = band_pairs(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld)
+    v = av + bv
     return torch.where(valid, v, torch.full_like(v, -float("inf"))), valid
+
+
+def band_product64(a, a_lu, a_ld, b, b_lu, b_ld, mode):
+    """The banded product as a closed form over band_pairs in float64 (any device,
+    differentiable in a and b): mode 3 sum of products, mode 0 log-sum-exp of sums; cells
+    outside the matrix are 0.  The same arithmetic as band_product_dense without the dense
+    detour, for sizes where that is too large; pinned against it in tests/test_oracle.py."""
+    av, bv, valid = band_pairs(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld)
+    inside = valid.any(-1)
+    if mode == 3:
+        return torch.where(valid, av * bv, torch.zeros_like(av)).sum(-1)
+    v = torch.where(valid, av + bv, torch.full_like(av, -float("inf")))
+    v = torch.where(inside.unsqueeze(-1), v, torch.zeros_like(v))
+    return torch.where(inside, v.logsumexp(-1), torch.zeros_like(v[..., 0]))
+
+
+def band_max_first(a, a_lu, a_ld, b, b_lu, b_ld):
+    """Max-plus band product in the operands' own dtype (one rounding per sum, as the
+    reference) with the lowest k that attains the maximum, any device: (values, idx);
+    cells outside the matrix are 0 / 0.  Assumes every cell has a term above the -1e9
+    floor (banded_cuda_kernel.cu:79)."""
+    av, bv, valid = band_pairs(a, a_lu, a_ld, b, b_lu, b_ld)
+    inside = valid.any(-1)
+    v = torch.where(valid, av + bv, torch.full_like(av, -float("inf")))
+    m = v.max(-1).values
+    k = torch.arange(a.shape[2], device=a.device).expand_as(v)
+    first = torch.where(v == m.unsqueeze(-1), k, torch.full_like(k, a.shape[2])).min(-1).values
+    return torch.where(inside, m, torch.zeros_like(m)), torch.where(inside, first, torch.zeros_like(first)).to(torch.int32)
 
 
 def band_sample_cdf64(a, a_lu, a_ld, b, b_lu, b_ld):

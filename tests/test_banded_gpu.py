@@ -240,33 +240,62 @@ def test_double_backward_reaches_operands_given_as_views(gpu):
 
 def test_banded_config_c5(gpu):
     """Benchmark configuration 4: batch 64, n = 4096, lu = ld = 32 for both operands, Uniform[-1,1)
-    band data from seed 7; standard and log semiring, forward + backward.  Full-size run;
-    float64 oracle on two batch items; dense closed form at reduced n."""
+    band data from seed 7; standard, log and max semiring, forward + backward, at full size.
+    EVERY batch item: out, grad_a and grad_b against the float64 closed form over the cells'
+    factor pairs (oracle.band_product64 and its autograd gradients, evaluated on the device
+    item by item); the max product bit-exact (values, lowest-k indices, one-hot gradients with
+    g on the 1/8 grid); two items against the sequential float64 restatement of the
+    reference kernel; the dense closed form at reduced n."""
     torch.manual_seed(7)
     B, n, lu, ld = 64, 4096, 32, 32
     a, b = torch.rand(B, n, 65) * 2 - 1, torch.rand(B, n, 65) * 2 - 1
     g = torch.randn(B, n, 129)
     ad, bd, gd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True), g.to(gpu)
     pick = [0, 63]
+    # absolute bound of a K-term fp32 sum against float64: 4 u K max|x| max|y| (u = 2^-24; the
+    # textbook K u sum|x y| with room for the order of summation); the log product's
+    # weights are at most 1, so its gradients obey the same bound with |y| = 1
+    u, K = 2.0 ** -24, 65
+    fwd_tol = 4 * u * K * float(a.abs().max()) * float(b.abs().max())
+    bwd_tol = 4 * u * K * float(g.abs().max()) * max(float(a.abs().max()), float(b.abs().max()))
+    assert fwd_tol < 2e-5 and bwd_tol < 1e-4
     for mode in (3, 0):
         X, Y = BandedMatrix(ad, lu, ld), BandedMatrix(bd, lu, ld)
         res = (X.multiply if mode == 3 else X.multiply_log)(Y)
         ga, gb = torch.autograd.grad(res.data, (ad, bd), gd)
         want, _, _ = oracle.seq_band_fwd(a[pick].double(), lu, ld, b[pick].double(), lu, ld, mode, dtype=np.float64)
-        # absolute bound of a K-term fp32 sum against float64: 4 u K max|x| max|y| (u = 2^-24; the
-        # textbook K u sum|x y| with room for the order of summation); the log product's
-        # weights are at most 1, so its gradients obey the same bound with |y| = 1
-        u, K = 2.0 ** -24, 65
-        fwd_tol = 4 * u * K * float(a.abs().max()) * float(b.abs().max())
-        bwd_tol = 4 * u * K * float(g.abs().max()) * max(float(a.abs().max()), float(b.abs().max()))
-        assert fwd_tol < 2e-5 and bwd_tol < 1e-4
         close(res.data[pick], want, rtol=1e-5, atol=fwd_tol)
         wa, wb = oracle.seq_band_bwd(a[pick].double(), lu, ld, b[pick].double(), lu, ld, g[pick].double(), mode,
                                      dtype=np.float64)
         close(ga[pick], wa, rtol=1e-5, atol=bwd_tol)
         close(gb[pick], wb, rtol=1e-5, atol=bwd_tol)
-        if mode == 0:  # softmax weights of every in-matrix output cell sum to one
-            pass
+        for item in range(B):
+            sl = slice(item, item + 1)
+            a64 = ad[sl].detach().double().requires_grad_(True)
+            b64 = bd[sl].detach().double().requires_grad_(True)
+            w = oracle.band_product64(a64, lu, ld, b64, lu, ld, mode)
+            wa, wb = torch.autograd.grad(w, (a64, b64), gd[sl].double())
+            for got, ref, tol in ((res.data[sl].detach(), w.detach(), fwd_tol), (ga[sl], wa, bwd_tol), (gb[sl], wb, bwd_tol)):
+                assert torch.allclose(got.double(), ref, rtol=1e-5, atol=tol), (mode, item, float((got.double() - ref).abs().max()))
+            del w, wa, wb, a64, b64
+    # max product, every item, bit for bit
+    torch.manual_seed(8)
+    aq, bq = grid(B, n, 65).to(gpu).requires_grad_(True), grid(B, n, 65).to(gpu).requires_grad_(True)
+    gq = grid(B, n, 129).clamp(-4, 4).to(gpu)
+    res = BandedMatrix(aq, lu, ld).multiply_max(BandedMatrix(bq, lu, ld))
+    ga, gb = torch.autograd.grad(res.data, (aq, bq), gq)
+    i = torch.arange(n, device=gpu).view(n, 1)
+    jj = torch.arange(129, device=gpu).view(1, 129)
+    o = i + jj - (lu + ld)
+    inside = (o >= 0) & (o < n)
+    for item in range(B):
+        sl = slice(item, item + 1)
+        mv, mi = oracle.band_max_first(aq[sl].detach(), lu, ld, bq[sl].detach(), lu, ld)
+        assert torch.equal(res.data[sl].detach(), mv), item
+        li = mi[0].long()
+        wa = torch.zeros(n, 65, device=gpu).index_put_((i.expand(n, 129)[inside], li[inside]), gq[item][inside], accumulate=True)
+        wb = torch.zeros(n, 65, device=gpu).index_put_((o[inside], (li - jj + 64)[inside]), gq[item][inside], accumulate=True)
+        assert torch.equal(ga[item], wa) and torch.equal(gb[item], wb), item
     # dense closed form at n = 256, same bandwidths (test_sparse.py:141-142, 181-195)
     n2 = 256
     a2, b2 = a[:4, :n2].contiguous(), b[:4, :n2].contiguous()

@@ -291,6 +291,21 @@ def test_seq_band_sample_distribution_and_defaults():
     assert torch.equal(idx0[0].long(), torch.where(valid.any(-1), first, torch.zeros_like(first)))
 
 
+@pytest.mark.parametrize("n,a_lu,a_ld,b_lu,b_ld", BANDS)
+def test_band_closed_forms_by_index_arithmetic_match_the_dense_identity(n, a_lu, a_ld, b_lu, b_ld):
+    """band_product64 / band_max_first (used on the device for full-size checks) against the
+    dense identities of test_sparse.py:141-142, 181-195 and the sequential kernel restatement."""
+    a, b = _band_pair(n, a_lu, a_ld, b_lu, b_ld, grid=True)
+    for mode in (3, 0):
+        want, mask = oracle.band_product_dense(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, mode)
+        got = oracle.band_product64(a, a_lu, a_ld, b, b_lu, b_ld, mode)
+        assert torch.allclose(got[:, mask], want[:, mask], rtol=1e-12, atol=1e-12)
+        assert (got[:, ~mask] == 0).all()
+    sv, si, _ = oracle.seq_band_fwd(a, a_lu, a_ld, b, b_lu, b_ld, 1)
+    mv, mi = oracle.band_max_first(a, a_lu, a_ld, b, b_lu, b_ld)
+    assert torch.equal(mv, sv) and torch.equal(mi, si)          # ties present on the 1/8 grid
+
+
 def _dense_band_fn(a_lu, a_ld, b_lu, b_ld, mode):
     fill = 0.0 if mode == 3 else -1e9
 
