@@ -120,6 +120,28 @@ def main():
 
     ms_fwd = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
     ms_bwd = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+    # The same events, first and last five timed steps apart: after any idle period (the host-side
+    # set-up above is one) this GPU runs its first ~25 ms of work slower and then settles, whatever
+    # the kernel - a short run (few warm-up steps) is timed inside that window, a long one past it.
+    head, tail = ev[:5], ev[-5:]
+
+    def mean(pairs):
+        return round(sum(x.elapsed_time(y) for x, y in pairs) / len(pairs), 4)
+
+    trend = {
+        "ms_step_first5": mean([(e[0], e[2]) for e in head]), "ms_step_last5": mean([(e[0], e[2]) for e in tail]),
+        "ms_fwd_first5": mean([(e[0], e[1]) for e in head]), "ms_fwd_last5": mean([(e[0], e[1]) for e in tail]),
+        "ms_bwd_first5": mean([(e[1], e[2]) for e in head]), "ms_bwd_last5": mean([(e[1], e[2]) for e in tail]),
+    }
+    # and, outside the timed region and of no influence on `value`: the step time once settled
+    # (60 more steps straight behind the timed ones, the last 20 of them averaged)
+    more = [torch.cuda.Event(enable_timing=True) for _ in range(61)]
+    more[0].record()
+    for i in range(60):
+        fwd(); bwd()
+        more[i + 1].record()
+    torch.cuda.synchronize()
+    trend["ms_step_settled"] = round(more[40].elapsed_time(more[60]) / 20, 4)
     ms_step = dt * 1e3 / args.steps
     bmkn = float(B) * M * K * N
     value = 6.0 * bmkn / (ms_step * 1e-3) / 1e9
@@ -172,6 +194,7 @@ def main():
         "pct_fp32_valu_peak": round(100.0 * value / 1e3 / FP32_VALU_PEAK_TFLOPS, 3),
         "ms_fwd": round(ms_fwd, 4),
         "ms_bwd": round(ms_bwd, 4),
+        "step_time_trend": trend,
         "ms_per_step_autograd_api": round(ms_autograd, 4),
         "roofline": roofline,
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(torch),

@@ -67,10 +67,13 @@ SIGNATURES = {
 # arguments, the caller's tensors in that type, every workspace still float32.
 HALF_VARIANTS = ("genbmm_logbmm_fwd", "genbmm_logbmm_bwd", "genbmm_logbmm_fwd_path", "genbmm_logbmm_bwd_path",
                  "genbmm_maxbmm_fwd", "genbmm_prodmaxbmm_fwd", "genbmm_samplebmm_fwd", "genbmm_argmax_bwd",
-                 "genbmm_prodmax_bwd")
+                 "genbmm_prodmax_bwd", "genbmm_banded_fwd", "genbmm_banded_sample_fwd", "genbmm_banded_bwd",
+                 "genbmm_banded_bwd_scratch")
 for _name in HALF_VARIANTS:
     for _suffix in ("_f16", "_bf16"):
         SIGNATURES[_name + _suffix] = SIGNATURES[_name]
+for _suffix in ("_f16", "_bf16"):  # one more buffer than the float function: t_scratch (B * n * Wo floats)
+    SIGNATURES["genbmm_banded_bwdbwd" + _suffix] = _BAND + [_c_float_p] * 8 + [_i, _i, _vp]
 HALF_SUFFIX = {torch.float16: "_f16", torch.bfloat16: "_bf16"}
 STRING_FUNCS = {"genbmm_version": [], "genbmm_error_string": [_i]}
 SIZE_FUNCS = {"genbmm_logbmm_stats_size": [_i, _i, _i, _i],

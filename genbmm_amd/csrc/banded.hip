@@ -114,7 +114,7 @@ inline void launch_max_fwd(const BandArgs& p, int B, hipStream_t s) {
                      rows * p.Wa, rows * p.Wb, nseg, Wseg);
 }
 
-inline void launch_prep(const BandArgs& p, const float* a, int a_lu, const float* b, int b_lu, int B,
+inline void launch_prep(const BandArgs& p, const elem_t* a, int a_lu, const elem_t* b, int b_lu, int B,
                         hipStream_t s) {
   const long rows = (long)B * p.n;
   const PrepSide pa{a, p.ws_ea, p.ws_al, p.Wa, a_lu, odd(p.Wa)}, pb{b, p.ws_eb, p.ws_be, p.Wb, b_lu, odd(p.Wb)};
@@ -183,6 +183,7 @@ inline void set_workspace(BandArgs& p, float* ws, int B) {
 
 extern "C" {
 
+#if GENBMM_ELEM == 0  // sizes do not depend on the element type: every workspace is float
 size_t genbmm_banded_workspace_size(int a_lu, int a_ld, int b_lu, int b_ld, int B, int n) {
   using namespace GENBMM_NS;
   BandArgs p{};
@@ -196,11 +197,15 @@ size_t genbmm_banded_scratch_size(int a_lu, int a_ld, int b_lu, int b_ld, int B,
   if (fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return 0;
   return dir_bwd_ok(p) || !workspace_used(p) ? 0 : (size_t)B * n * p.Wo;
 }
+#endif
 
-int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
-                      float* out, int32_t* idx, float* workspace, int B, int n, int mode,
-                      void* stream) {
+int GENBMM_API(banded_fwd)(const GENBMM_NS::abi_t* a_, int a_lu, int a_ld, const GENBMM_NS::abi_t* b_, int b_lu,
+                           int b_ld, GENBMM_NS::abi_t* out_, int32_t* idx, float* workspace, int B, int n, int mode,
+                           void* stream) {
   using namespace GENBMM_NS;
+  const elem_t* a = el(a_);
+  const elem_t* b = el(b_);
+  elem_t* out = el(out_);
   if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
     return GENBMM_E_MODE;
   BandArgs p{};
@@ -254,24 +259,28 @@ int genbmm_banded_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_
     return launch_status();
   }
   if (mode == GENBMM_BAND_LOG)
-    hipLaunchKernelGGL((k_band_fwd<GENBMM_BAND_LOG, float>), blocks_for(total), dim3(256), 0, s, p, total);
+    hipLaunchKernelGGL((k_band_fwd<GENBMM_BAND_LOG, elem_t>), blocks_for(total), dim3(256), 0, s, p, total);
   else if (mode == GENBMM_BAND_MAX)
-    hipLaunchKernelGGL((k_band_fwd<GENBMM_BAND_MAX, float>), blocks_for(total), dim3(256), 0, s, p, total);
+    hipLaunchKernelGGL((k_band_fwd<GENBMM_BAND_MAX, elem_t>), blocks_for(total), dim3(256), 0, s, p, total);
   else
-    hipLaunchKernelGGL((k_band_fwd<GENBMM_BAND_MUL, float>), blocks_for(total), dim3(256), 0, s, p, total);
+    hipLaunchKernelGGL((k_band_fwd<GENBMM_BAND_MUL, elem_t>), blocks_for(total), dim3(256), 0, s, p, total);
   return launch_status();
 }
 
-int genbmm_banded_sample_fwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
-                             float* out, int32_t* idx, float* workspace, uint64_t seed, uint64_t offset,
-                             int B, int n, void* stream) {
+int GENBMM_API(banded_sample_fwd)(const GENBMM_NS::abi_t* a_, int a_lu, int a_ld, const GENBMM_NS::abi_t* b_,
+                                  int b_lu, int b_ld, GENBMM_NS::abi_t* out_, int32_t* idx, float* workspace,
+                                  uint64_t seed, uint64_t offset, int B, int n, void* stream) {
   using namespace GENBMM_NS;
+  const elem_t* a = el(a_);
+  const elem_t* b = el(b_);
+  elem_t* out = el(out_);
   BandArgs p{};
   if (int e = fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return e;
   if ((int64_t)B * n == 0) return GENBMM_OK;
   if (!a || !b || !out || !idx) return GENBMM_E_NULLPTR;
   // out: the log product, on the workspace where there is one
-  if (int e = genbmm_banded_fwd(a, a_lu, a_ld, b, b_lu, b_ld, out, nullptr, workspace, B, n, GENBMM_BAND_LOG, stream))
+  if (int e = GENBMM_API(banded_fwd)(a_, a_lu, a_ld, b_, b_lu, b_ld, out_, nullptr, workspace, B, n, GENBMM_BAND_LOG,
+                                     stream))
     return e;
   p.a = a; p.b = b; p.out = out; p.oidx = idx;
   const long total = (long)B * n * p.Wo;
@@ -287,23 +296,23 @@ int genbmm_banded_sample_fwd(const float* a, int a_lu, int a_ld, const float* b,
     hipLaunchKernelGGL(k_band_sample_targets, blocks_for((total + 3) / 4), dim3(256), 0, s, p.ws_r, idx, total, seed,
                        offset);
     if (d.bytes > kStripLdsLimit)
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_band_sample_fwd<float>),
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k_band_sample_fwd<elem_t>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)d.bytes);
     const long rows = (long)B * p.n;
-    hipLaunchKernelGGL(k_band_sample_fwd<float>, dim3((unsigned)((long)B * strips * nseg)), dim3(256), d.bytes, s, p,
+    hipLaunchKernelGGL(k_band_sample_fwd<elem_t>, dim3((unsigned)((long)B * strips * nseg)), dim3(256), d.bytes, s, p,
                        strips, d, rows * p.Wa, rows * p.Wb, nseg, Wseg, seed, offset);
     return launch_status();
   }
-  hipLaunchKernelGGL(k_band_sample_cells<float>, blocks_for(total), dim3(256), 0, s, p, total, seed, offset);
+  hipLaunchKernelGGL(k_band_sample_cells<elem_t>, blocks_for(total), dim3(256), 0, s, p, total, seed, offset);
   return launch_status();
 }
 
 namespace GENBMM_NS {
 namespace {
 // `scratch`: where g / S goes in the prepared log product; NULL: the workspace's own part
-int banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
-               const float* out, const int32_t* idx, float* workspace, float* scratch, const float* g,
-               float* grad_a, float* grad_b, int B, int n, int mode, void* stream) {
+static int banded_bwd(const elem_t* a, int a_lu, int a_ld, const elem_t* b, int b_lu, int b_ld,
+               const elem_t* out, const int32_t* idx, float* workspace, float* scratch, const elem_t* g,
+               elem_t* grad_a, elem_t* grad_b, int B, int n, int mode, void* stream) {
   if (mode == GENBMM_BAND_SAMPLE) mode = GENBMM_BAND_MAX;  // a drawn index scatters like an arg-max
   if (mode != GENBMM_BAND_LOG && mode != GENBMM_BAND_MAX && mode != GENBMM_BAND_MUL)
     return GENBMM_E_MODE;
@@ -334,7 +343,11 @@ int banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int
       const int strips = ceil_div(n, kBT);
       const dim3 grid((unsigned)((long)B * strips));
       const int nq = ceil_div(max(max(da.ld_own, da.ld_sl), max(db.ld_own, db.ld_sl)), 64);
-      if (lg && workspace && workspace_used(p)) {  // on the forward's workspace: a (+,x) backward plus epilogue
+      // on the forward's workspace: a (+,x) backward plus epilogue.  H = g / S needs a place: the
+      // caller's scratch, or the workspace's own part - which exists exactly for the bands whose
+      // backward is not the memory-fed one (band_ws_floats); without one, the kernels below
+      // rebuild the weights from `out`
+      if (lg && workspace && workspace_used(p) && (scratch || !dir_bwd_ok(p))) {
         set_workspace(p, workspace, B);
         if (scratch) p.ws_h = scratch;
         // H = g * R once for both gradients (NaN marks a cell whose R is not usable)
@@ -386,60 +399,80 @@ int banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int
     return launch_status();
   }
   if (mode == GENBMM_BAND_LOG) {
-    hipLaunchKernelGGL((k_band_bwd_a<GENBMM_BAND_LOG, float>), blocks_for(ta), dim3(256), 0, s, p, ta);
-    hipLaunchKernelGGL((k_band_bwd_b<GENBMM_BAND_LOG, float>), blocks_for(tb), dim3(256), 0, s, p, tb);
+    hipLaunchKernelGGL((k_band_bwd_a<GENBMM_BAND_LOG, elem_t>), blocks_for(ta), dim3(256), 0, s, p, ta);
+    hipLaunchKernelGGL((k_band_bwd_b<GENBMM_BAND_LOG, elem_t>), blocks_for(tb), dim3(256), 0, s, p, tb);
   } else if (mode == GENBMM_BAND_MAX) {
-    hipLaunchKernelGGL((k_band_bwd_a<GENBMM_BAND_MAX, float>), blocks_for(ta), dim3(256), 0, s, p, ta);
-    hipLaunchKernelGGL((k_band_bwd_b<GENBMM_BAND_MAX, float>), blocks_for(tb), dim3(256), 0, s, p, tb);
+    hipLaunchKernelGGL((k_band_bwd_a<GENBMM_BAND_MAX, elem_t>), blocks_for(ta), dim3(256), 0, s, p, ta);
+    hipLaunchKernelGGL((k_band_bwd_b<GENBMM_BAND_MAX, elem_t>), blocks_for(tb), dim3(256), 0, s, p, tb);
   } else {
-    hipLaunchKernelGGL((k_band_bwd_a<GENBMM_BAND_MUL, float>), blocks_for(ta), dim3(256), 0, s, p, ta);
-    hipLaunchKernelGGL((k_band_bwd_b<GENBMM_BAND_MUL, float>), blocks_for(tb), dim3(256), 0, s, p, tb);
+    hipLaunchKernelGGL((k_band_bwd_a<GENBMM_BAND_MUL, elem_t>), blocks_for(ta), dim3(256), 0, s, p, ta);
+    hipLaunchKernelGGL((k_band_bwd_b<GENBMM_BAND_MUL, elem_t>), blocks_for(tb), dim3(256), 0, s, p, tb);
   }
   return launch_status();
 }
 }  // namespace
 }  // namespace GENBMM_NS
 
-int genbmm_banded_bwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
-                      const float* out, const int32_t* idx, float* workspace, const float* g,
-                      float* grad_a, float* grad_b, int B, int n, int mode, void* stream) {
-  return GENBMM_NS::banded_bwd(a, a_lu, a_ld, b, b_lu, b_ld, out, idx, workspace, nullptr, g, grad_a, grad_b, B, n,
-                            mode, stream);
+int GENBMM_API(banded_bwd)(const GENBMM_NS::abi_t* a, int a_lu, int a_ld, const GENBMM_NS::abi_t* b, int b_lu,
+                           int b_ld, const GENBMM_NS::abi_t* out, const int32_t* idx, float* workspace,
+                           const GENBMM_NS::abi_t* g, GENBMM_NS::abi_t* grad_a, GENBMM_NS::abi_t* grad_b, int B, int n,
+                           int mode, void* stream) {
+  using namespace GENBMM_NS;
+  return banded_bwd(el(a), a_lu, a_ld, el(b), b_lu, b_ld, el(out), idx, workspace, nullptr, el(g), el(grad_a),
+                    el(grad_b), B, n, mode, stream);
 }
 
-int genbmm_banded_bwd_scratch(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
-                              const float* out, const int32_t* idx, const float* workspace, float* scratch,
-                              const float* g, float* grad_a, float* grad_b, int B, int n, int mode,
-                              void* stream) {
+int GENBMM_API(banded_bwd_scratch)(const GENBMM_NS::abi_t* a, int a_lu, int a_ld, const GENBMM_NS::abi_t* b,
+                                   int b_lu, int b_ld, const GENBMM_NS::abi_t* out, const int32_t* idx,
+                                   const float* workspace, float* scratch, const GENBMM_NS::abi_t* g,
+                                   GENBMM_NS::abi_t* grad_a, GENBMM_NS::abi_t* grad_b, int B, int n, int mode,
+                                   void* stream) {
+  using namespace GENBMM_NS;
   if (workspace && !scratch && mode == GENBMM_BAND_LOG &&
       genbmm_banded_scratch_size(a_lu, a_ld, b_lu, b_ld, B, n) != 0)
     return GENBMM_E_NULLPTR;
-  return GENBMM_NS::banded_bwd(a, a_lu, a_ld, b, b_lu, b_ld, out, idx, const_cast<float*>(workspace), scratch, g,
-                            grad_a, grad_b, B, n, mode, stream);
+  return banded_bwd(el(a), a_lu, a_ld, el(b), b_lu, b_ld, el(out), idx, const_cast<float*>(workspace), scratch,
+                    el(g), el(grad_a), el(grad_b), B, n, mode, stream);
 }
 
 
+// `t_scratch`: B * n * Wo floats for the half element types, where t (the gradient with respect
+// to g, which the other two gradients read back) must stay unrounded; the float build keeps it in
+// grad_g itself and takes no such argument.
+#if GENBMM_ELEM == 0
 int genbmm_banded_bwdbwd(const float* a, int a_lu, int a_ld, const float* b, int b_lu, int b_ld,
                          const float* out, const float* g, const float* u_a, const float* u_b,
                          float* grad_a, float* grad_b, float* grad_g, int B, int n,
                          void* stream) {
+  float* t_scratch = grad_g;
+#else
+int GENBMM_API(banded_bwdbwd)(const GENBMM_NS::abi_t* a_, int a_lu, int a_ld, const GENBMM_NS::abi_t* b_, int b_lu,
+                              int b_ld, const GENBMM_NS::abi_t* out_, const GENBMM_NS::abi_t* g_,
+                              const GENBMM_NS::abi_t* ua_, const GENBMM_NS::abi_t* ub_, GENBMM_NS::abi_t* ga_,
+                              GENBMM_NS::abi_t* gb_, GENBMM_NS::abi_t* gg_, float* t_scratch, int B, int n,
+                              void* stream) {
+  using GENBMM_NS::el;
+  const GENBMM_NS::elem_t *a = el(a_), *b = el(b_), *out = el(out_), *g = el(g_), *u_a = el(ua_), *u_b = el(ub_);
+  GENBMM_NS::elem_t *grad_a = el(ga_), *grad_b = el(gb_), *grad_g = el(gg_);
+#endif
   using namespace GENBMM_NS;
   BandArgs p{};
   if (int e = fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return e;
   if ((int64_t)B * n == 0) return GENBMM_OK;
-  if (!a || !b || !out || !g || !grad_a || !grad_b || !grad_g || (!u_a && !u_b))
+  if (!a || !b || !out || !g || !grad_a || !grad_b || !grad_g || !t_scratch || (!u_a && !u_b))
     return GENBMM_E_NULLPTR;
   p.a = a; p.b = b; p.out = out; p.g = g; p.ua = u_a; p.ub = u_b;
   p.o0 = grad_a; p.o1 = grad_b; p.o2 = grad_g;
   const long ta = (long)B * n * p.Wa, tb = (long)B * n * p.Wb, to = (long)B * n * p.Wo;
   if (to == 0) return GENBMM_OK;
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(k_band_bb_t<float>, blocks_for(to), dim3(256), 0, s, p, to);
-  hipLaunchKernelGGL(k_band_bb_a<float>, blocks_for(ta), dim3(256), 0, s, p, ta);
-  hipLaunchKernelGGL(k_band_bb_b<float>, blocks_for(tb), dim3(256), 0, s, p, tb);
+  hipLaunchKernelGGL(k_band_bb_t<elem_t>, blocks_for(to), dim3(256), 0, s, p, t_scratch, to);
+  hipLaunchKernelGGL(k_band_bb_a<elem_t>, blocks_for(ta), dim3(256), 0, s, p, t_scratch, ta);
+  hipLaunchKernelGGL(k_band_bb_b<elem_t>, blocks_for(tb), dim3(256), 0, s, p, t_scratch, tb);
   return launch_status();
 }
 
+#if GENBMM_ELEM == 0
 const char* genbmm_version(void) { return "genbmm-gfx950 0.1"; }
 
 const char* genbmm_error_string(int code) {
@@ -453,5 +486,6 @@ const char* genbmm_error_string(int code) {
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
   }
 }
+#endif
 
 }  // extern "C"

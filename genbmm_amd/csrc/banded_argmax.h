@@ -43,7 +43,7 @@ struct ArgTile {
   // [0, n), j < Wo and, for need_o, its o = i + j - r_lu is in [0, n); for skew (a tile
   // whose rows of b run along its diagonals) only if it lies on the diagonal of one of the
   // strip's 64 rows - the corners of the tile are not read
-  __device__ __forceinline__ void load(const float* __restrict__ gb, const int32_t* __restrict__ ib,
+  __device__ __forceinline__ void load(const elem_t* __restrict__ gb, const int32_t* __restrict__ ib,
                                        int row0, int jc, int n, int Wo, int r_lu, bool need_o,
                                        bool skew, int tid) {
 #pragma unroll
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(256) void k_band_argmax_bwd_a(const BandArgs p, int
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int batch = blockIdx.x / strips, i0 = (blockIdx.x - batch * strips) * kAT;
   const long bn = (long)batch * n;
-  const float* gb = p.g + bn * Wo;
+  const elem_t* gb = p.g + bn * Wo;
   const int32_t* ib = p.idx + bn * Wo;
   for (int e = tid; e < Wa * kAS + 256; e += 256) acc[e] = 0.f;
   const int spare = Wa * kAS + tid;
@@ -106,11 +106,11 @@ __global__ __launch_bounds__(256) void k_band_argmax_bwd_a(const BandArgs p, int
     }
   }
   __syncthreads();
-  float* out = p.o0 + (bn + i0) * Wa;
+  elem_t* out = p.o0 + (bn + i0) * Wa;
   const int rows = min(kAT, n - i0);
   for (int e = tid; e < rows * Wa; e += 256) {
     const int r = e / Wa, k = e - r * Wa;
-    out[e] = acc[k * kAS + r];
+    out[e] = to_elem<elem_t>(acc[k * kAS + r]);
   }
 }
 
@@ -124,7 +124,7 @@ __global__ __launch_bounds__(256) void k_band_argmax_bwd_b(const BandArgs p, int
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int batch = blockIdx.x / strips, o0 = (blockIdx.x - batch * strips) * kAT;
   const long bn = (long)batch * n;
-  const float* gb = p.g + bn * Wo;
+  const elem_t* gb = p.g + bn * Wo;
   const int32_t* ib = p.idx + bn * Wo;
   for (int e = tid; e < Wb * kAS + 256; e += 256) acc[e] = 0.f;
   const int spare = Wb * kAS + tid;
@@ -158,11 +158,11 @@ __global__ __launch_bounds__(256) void k_band_argmax_bwd_b(const BandArgs p, int
     }
   }
   __syncthreads();
-  float* out = p.o1 + (bn + o0) * Wb;
+  elem_t* out = p.o1 + (bn + o0) * Wb;
   const int rows = min(kAT, n - o0);
   for (int e = tid; e < rows * Wb; e += 256) {
     const int r = e / Wb, k = e - r * Wb;
-    out[e] = acc[k * kAS + r];
+    out[e] = to_elem<elem_t>(acc[k * kAS + r]);
   }
 }
 

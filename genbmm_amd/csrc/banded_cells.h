@@ -34,7 +34,19 @@ struct BandArgsT {
   float* ws_h;    // backward scratch: g * R per output cell (NaN where R is not usable)
   int n, a_lu, Wa, b_lu, Wb, r_lu, Wo;
 };
-using BandArgs = BandArgsT<float>;
+using BandArgs = BandArgsT<elem_t>;  // the caller's tensors; workspaces are float whatever the element type
+
+// The type a cell is computed in: double for double tensors, float for float, binary16 and
+// bfloat16 ones (widened by the load, rounded once by the store).
+template <class T> struct band_acc { typedef float type; };
+template <> struct band_acc<double> { typedef double type; };
+template <class T> using band_acc_t = typename band_acc<T>::type;
+// result -> element: one rounding to nearest even for the half types
+template <class T, class A>
+__device__ __forceinline__ T band_store(A x) {
+  if constexpr (sizeof(T) == 2) return (T)settled((float)x);
+  else return (T)x;
+}
 
 // exp of a difference and fused multiply-add per element type: float takes the
 // hardware base-2 exponential, double the library routine.
@@ -58,10 +70,11 @@ __device__ __forceinline__ void k_range(const BandArgsT<T>& p, int i, int j, int
 // One output cell e = (bi*Wo + j), bi = batch*n + i.
 template <int MODE, class T>
 __device__ __forceinline__ void band_fwd_cell(const BandArgsT<T>& p, long bi, int i, int j) {
+  typedef band_acc_t<T> A;
   const long e = bi * p.Wo + j;
   const int o = i + j - p.r_lu;
   if (o < 0 || o >= p.n) {  // outside the matrix: the reference leaves its zero fill
-    p.o0[e] = 0;
+    p.o0[e] = (T)0;
     if (MODE == GENBMM_BAND_MAX) p.oidx[e] = 0;
     return;
   }
@@ -70,32 +83,32 @@ __device__ __forceinline__ void band_fwd_cell(const BandArgsT<T>& p, long bi, in
   const T* ar = p.a + bi * p.Wa;
   const T* br = p.b + (bi + (o - i)) * p.Wb + (p.Wb - 1 - j);  // br[k] = b[o][k2(k)]
   if (MODE == GENBMM_BAND_MUL) {
-    T v = 0;
-    for (int k = klo; k <= khi; ++k) v = sr_fma(ar[k], br[k], v);
-    p.o0[e] = v;
+    A v = 0;
+    for (int k = klo; k <= khi; ++k) v = sr_fma((A)ar[k], (A)br[k], v);
+    p.o0[e] = band_store<T>(v);
   } else if (MODE == GENBMM_BAND_MAX) {
-    T m = kFloor;
+    A m = kFloor;
     int ind = -1;
     for (int k = klo; k <= khi; ++k) {
-      const T v = ar[k] + br[k];
+      const A v = (A)ar[k] + (A)br[k];
       if (v > m) {
         m = v;
         ind = k;
       }
     }
-    p.o0[e] = m;
+    p.o0[e] = band_store<T>(m);
     p.oidx[e] = ind;
-  } else if constexpr (sizeof(T) == sizeof(float)) {
+  } else if constexpr (sizeof(A) == sizeof(float)) {
     float m = kFloor;
-    for (int k = klo; k <= khi; ++k) m = fmaxf(m, ar[k] + br[k]);
+    for (int k = klo; k <= khi; ++k) m = fmaxf(m, (float)ar[k] + (float)br[k]);
     const float nm = -m * kLog2e;
     float s = 0.f;
-    for (int k = klo; k <= khi; ++k) s += fast_exp2(__builtin_fmaf(ar[k] + br[k], kLog2e, nm));
-    p.o0[e] = logf(s) + m;
+    for (int k = klo; k <= khi; ++k) s += fast_exp2(__builtin_fmaf((float)ar[k] + (float)br[k], kLog2e, nm));
+    p.o0[e] = band_store<T>(logf(s) + m);
   } else {
-    T m = kFloor;
+    A m = kFloor;
     for (int k = klo; k <= khi; ++k) m = fmax(m, ar[k] + br[k]);
-    T s = 0;
+    A s = 0;
     for (int k = klo; k <= khi; ++k) s += exp(ar[k] + br[k] - m);
     p.o0[e] = log(s) + m;
   }
@@ -107,9 +120,10 @@ __device__ __forceinline__ void band_fwd_cell(const BandArgsT<T>& p, long bi, in
 // banded_cuda_backward_kernel_mul, banded_cuda_kernel.cu:104-152).
 template <int MODE, class T>
 __device__ __forceinline__ void band_bwd_a_cell(const BandArgsT<T>& p, long bi, int i, int k) {
+  typedef band_acc_t<T> A;
   const long e = bi * p.Wa + k;
   const int pos = i + k - p.a_lu;
-  T acc = 0;
+  A acc = 0;
   if (pos >= 0 && pos < p.n) {
     const int jlo = imax3(k, p.r_lu - i, 0);
     const int jhi = imin3(k + p.Wb - 1, p.n - 1 + p.r_lu - i, p.Wo - 1);
@@ -117,20 +131,20 @@ __device__ __forceinline__ void band_bwd_a_cell(const BandArgsT<T>& p, long bi, 
     // b[o][k2] = bw[j * (Wb - 1)] with o = i + j - r_lu, k2 = k - j + Wb - 1
     const T* bw = p.b + (bi - p.r_lu) * p.Wb + k + p.Wb - 1;
     if (MODE == GENBMM_BAND_MUL) {
-      for (int j = jlo; j <= jhi; ++j) acc = sr_fma(bw[(long)j * (p.Wb - 1)], gr[j], acc);
+      for (int j = jlo; j <= jhi; ++j) acc = sr_fma((A)bw[(long)j * (p.Wb - 1)], (A)gr[j], acc);
     } else if (MODE == GENBMM_BAND_MAX) {
       const int32_t* ir = p.idx + bi * p.Wo;
-      for (int j = jlo; j <= jhi; ++j) acc += (ir[j] == k) ? gr[j] : T(0);
+      for (int j = jlo; j <= jhi; ++j) acc += (ir[j] == k) ? (A)gr[j] : A(0);
     } else {
-      const T av = p.a[e];
+      const A av = p.a[e];
       const T* orow = p.out + bi * p.Wo;
       for (int j = jlo; j <= jhi; ++j) {
-        const T w = sr_exp(av + bw[(long)j * (p.Wb - 1)] - orow[j]);
-        acc = sr_fma(w, gr[j], acc);
+        const A w = sr_exp(av + (A)bw[(long)j * (p.Wb - 1)] - (A)orow[j]);
+        acc = sr_fma(w, (A)gr[j], acc);
       }
     }
   }
-  p.o0[e] = acc;
+  p.o0[e] = band_store<T>(acc);
 }
 
 // grad_b[o,k2] sums, in ascending i, over the cells (i, j = o - i + r_lu) that
@@ -139,31 +153,32 @@ __device__ __forceinline__ void band_bwd_a_cell(const BandArgsT<T>& p, long bi, 
 // kernel above with the operands swapped (sparse.py:436-446, 523-545, 625-635).
 template <int MODE, class T>
 __device__ __forceinline__ void band_bwd_b_cell(const BandArgsT<T>& p, long bo, int o, int k2) {
+  typedef band_acc_t<T> A;
   const long e = bo * p.Wb + k2;
   const int prow = o + k2 - p.b_lu;
-  T acc = 0;
+  A acc = 0;
   if (prow >= 0 && prow < p.n) {
     const int jhi_k = p.Wb - 1 - k2 + p.Wa - 1;  // j with k = Wa-1
     const int jlo_k = p.Wb - 1 - k2;             // j with k = 0
     const int ilo = imax3(0, o + p.r_lu - min(jhi_k, p.Wo - 1), o + p.r_lu - (p.Wo - 1));
     const int ihi = imin3(p.n - 1, o + p.r_lu - max(jlo_k, 0), o + p.r_lu);
     const long base = bo - o;  // batch*n
-    const T bv = p.b[e];
+    const A bv = p.b[e];
     for (int i = ilo; i <= ihi; ++i) {
       const int j = o - i + p.r_lu;
       const int k = k2 + j - (p.Wb - 1);
       const long gi = (base + i) * p.Wo + j;
       if (MODE == GENBMM_BAND_MUL) {
-        acc = sr_fma(p.a[(base + i) * p.Wa + k], p.g[gi], acc);
+        acc = sr_fma((A)p.a[(base + i) * p.Wa + k], (A)p.g[gi], acc);
       } else if (MODE == GENBMM_BAND_MAX) {
-        acc += (p.idx[gi] == k) ? p.g[gi] : T(0);
+        acc += (p.idx[gi] == k) ? (A)p.g[gi] : A(0);
       } else {
-        const T w = sr_exp(p.a[(base + i) * p.Wa + k] + bv - p.out[gi]);
-        acc = sr_fma(w, p.g[gi], acc);
+        const A w = sr_exp((A)p.a[(base + i) * p.Wa + k] + bv - (A)p.out[gi]);
+        acc = sr_fma(w, (A)p.g[gi], acc);
       }
     }
   }
-  p.o1[e] = acc;
+  p.o1[e] = band_store<T>(acc);
 }
 
 // ------------------------------------------------ one lane per cell kernels
@@ -257,83 +272,91 @@ __global__ __launch_bounds__(256) void k_band_sample_cells(const BandArgsT<T> p,
 // With u_b = 0 these equal the reference's banded_cuda_backbackward_kernel_A/
 // _B/_C (banded_cuda_kernel.cu:154-350), whose inner loop sum_m (delta*s -
 // s*s2)*u[m] is s*(u[k] - t).
+// `tt`: t per output cell in the accumulation type (a float buffer of the caller's for
+// the half element types, whose grad_g output holds t rounded; else grad_g itself).
 template <class T>
-__global__ __launch_bounds__(256) void k_band_bb_t(const BandArgsT<T> p, long total) {
+__global__ __launch_bounds__(256) void k_band_bb_t(const BandArgsT<T> p, band_acc_t<T>* __restrict__ tt, long total) {
+  typedef band_acc_t<T> A;
   const long e = (long)blockIdx.x * 256 + threadIdx.x;
   if (e >= total) return;
   const int j = (int)(e % p.Wo);
   const long bi = e / p.Wo;
   const int i = (int)(bi % p.n);
   const int o = i + j - p.r_lu;
-  T t = 0;
+  A t = 0;
   if (o >= 0 && o < p.n) {
     int klo, khi;
     k_range(p, i, j, klo, khi);
     const long boff = (bi + (o - i)) * p.Wb + (p.Wb - 1 - j);
-    const T ov = p.out[e];
+    const A ov = p.out[e];
     for (int k = klo; k <= khi; ++k) {
-      const T pr = sr_exp(p.a[bi * p.Wa + k] + p.b[boff + k] - ov);
-      const T w = (p.ua ? p.ua[bi * p.Wa + k] : T(0)) + (p.ub ? p.ub[boff + k] : T(0));
+      const A pr = sr_exp((A)p.a[bi * p.Wa + k] + (A)p.b[boff + k] - ov);
+      const A w = (p.ua ? (A)p.ua[bi * p.Wa + k] : A(0)) + (p.ub ? (A)p.ub[boff + k] : A(0));
       t = sr_fma(pr, w, t);
     }
   }
-  p.o2[e] = t;
+  tt[e] = t;
+  if constexpr (sizeof(T) != sizeof(A)) p.o2[e] = band_store<T>(t);
 }
 
 template <class T>
-__global__ __launch_bounds__(256) void k_band_bb_a(const BandArgsT<T> p, long total) {
+__global__ __launch_bounds__(256) void k_band_bb_a(const BandArgsT<T> p, const band_acc_t<T>* __restrict__ tt,
+                                                   long total) {
+  typedef band_acc_t<T> A;
   const long e = (long)blockIdx.x * 256 + threadIdx.x;
   if (e >= total) return;
   const int k = (int)(e % p.Wa);
   const long bi = e / p.Wa;
   const int i = (int)(bi % p.n);
   const int pos = i + k - p.a_lu;
-  T acc = 0;
+  A acc = 0;
   if (pos >= 0 && pos < p.n) {
     const int jlo = imax3(k, p.r_lu - i, 0);
     const int jhi = imin3(k + p.Wb - 1, p.n - 1 + p.r_lu - i, p.Wo - 1);
     const long bw = (bi - p.r_lu) * p.Wb + k + p.Wb - 1;
-    const T av = p.a[e];
-    const T uav = p.ua ? p.ua[e] : T(0);
+    const A av = p.a[e];
+    const A uav = p.ua ? (A)p.ua[e] : A(0);
     for (int j = jlo; j <= jhi; ++j) {
       const long bj = bw + (long)j * (p.Wb - 1);
       const long gi = bi * p.Wo + j;
-      const T pr = sr_exp(av + p.b[bj] - p.out[gi]);
-      const T w = uav + (p.ub ? p.ub[bj] : T(0)) - p.o2[gi];
-      acc = sr_fma(p.g[gi] * pr, w, acc);
+      const A pr = sr_exp(av + (A)p.b[bj] - (A)p.out[gi]);
+      const A w = uav + (p.ub ? (A)p.ub[bj] : A(0)) - tt[gi];
+      acc = sr_fma((A)p.g[gi] * pr, w, acc);
     }
   }
-  p.o0[e] = acc;
+  p.o0[e] = band_store<T>(acc);
 }
 
 template <class T>
-__global__ __launch_bounds__(256) void k_band_bb_b(const BandArgsT<T> p, long total) {
+__global__ __launch_bounds__(256) void k_band_bb_b(const BandArgsT<T> p, const band_acc_t<T>* __restrict__ tt,
+                                                   long total) {
+  typedef band_acc_t<T> A;
   const long e = (long)blockIdx.x * 256 + threadIdx.x;
   if (e >= total) return;
   const int k2 = (int)(e % p.Wb);
   const long bo = e / p.Wb;
   const int o = (int)(bo % p.n);
   const int prow = o + k2 - p.b_lu;
-  T acc = 0;
+  A acc = 0;
   if (prow >= 0 && prow < p.n) {
     const int jhi_k = p.Wb - 1 - k2 + p.Wa - 1;
     const int jlo_k = p.Wb - 1 - k2;
     const int ilo = imax3(0, o + p.r_lu - min(jhi_k, p.Wo - 1), o + p.r_lu - (p.Wo - 1));
     const int ihi = imin3(p.n - 1, o + p.r_lu - max(jlo_k, 0), o + p.r_lu);
     const long base = bo - o;
-    const T bv = p.b[e];
-    const T ubv = p.ub ? p.ub[e] : T(0);
+    const A bv = p.b[e];
+    const A ubv = p.ub ? (A)p.ub[e] : A(0);
     for (int i = ilo; i <= ihi; ++i) {
       const int j = o - i + p.r_lu;
       const int k = k2 + j - (p.Wb - 1);
       const long gi = (base + i) * p.Wo + j;
       const long ai = (base + i) * p.Wa + k;
-      const T pr = sr_exp(p.a[ai] + bv - p.out[gi]);
-      const T w = (p.ua ? p.ua[ai] : T(0)) + ubv - p.o2[gi];
-      acc = sr_fma(p.g[gi] * pr, w, acc);
+      const A pr = sr_exp((A)p.a[ai] + bv - (A)p.out[gi]);
+      const A w = (p.ua ? (A)p.ua[ai] : A(0)) + ubv - tt[gi];
+      acc = sr_fma((A)p.g[gi] * pr, w, acc);
     }
   }
-  p.o1[e] = acc;
+  p.o1[e] = band_store<T>(acc);
 }
 
 // ------------------------------------------------------------------- host
@@ -343,7 +366,11 @@ inline int fill_band(BandArgsT<T>& p, int a_lu, int a_ld, int b_lu, int b_ld, in
   if (B < 0 || n < 0) return GENBMM_E_SHAPE;
   const int64_t Wa = (int64_t)a_lu + a_ld + 1, Wb = (int64_t)b_lu + b_ld + 1;
   const int64_t Wo = Wa + Wb - 1;
-  if (Wo > 0x3fffffff || (int64_t)B * n * Wo > ((int64_t)1 << 40)) return GENBMM_E_SHAPE;
+  // 2^37 cells: beyond any device buffer, and one-lane-per-cell grids (cells / 256) stay within
+  // 32 bits; the strip and tile-row kernels launch at most two workgroups per 16 rows and
+  // segment of 8 result diagonals - a grid beyond 2^31 - 1 workgroups would wrap silently
+  if (Wo > 0x3fffffff || (int64_t)B * n * Wo > ((int64_t)1 << 37)) return GENBMM_E_SHAPE;
+  if ((int64_t)B * ((n + 15) / 16) * ((Wo + 7) / 8) > ((int64_t)1 << 30)) return GENBMM_E_SHAPE;
   p.n = n; p.a_lu = a_lu; p.Wa = (int)Wa; p.b_lu = b_lu; p.Wb = (int)Wb;
   p.r_lu = a_lu + b_ld; p.Wo = (int)Wo;
   return GENBMM_OK;

@@ -193,12 +193,19 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long b
   const int from = 4 * (4 * l15 + zq);  // byte index of the lane this one takes its cells from
   const int K0 = i0 - g.plo;            // first k of chunk 0
   const int J0 = i0 - g.lu_out;         // first column of tile 0
-  const float* pt = FWD ? (PREP ? p.ws_ea : p.a) : p.g;
-  const float* qt = FWD ? (PREP ? p.ws_eb : p.b) : GA ? (PREP ? p.ws_eb : p.b) : (PREP ? p.ws_ea : p.a);
+  // P and Q: the workspace's factors (float) in the prepared product, else the caller's tensors
+  // (element type, widened by the loads); g always is the caller's.
   // offsets from the first cell of the batch item; EDGE keeps them inside the tensor
-  const float* pitem = pt + bn * (long)Wp;
+  auto pitem = [&] {
+    if constexpr (FWD && PREP) return static_cast<const float*>(p.ws_ea) + bn * (long)Wp;
+    else if constexpr (FWD) return p.a + bn * (long)Wp;
+    else return p.g + bn * (long)Wp;
+  }();
   const float* ritem = MKH ? p.ws_r + bn * (long)Wp : nullptr;
-  const float* qitem = qt + bn * (long)Wq;
+  auto qitem = [&] {
+    if constexpr (PREP) return static_cast<const float*>(KIND == kDirGradB ? p.ws_ea : p.ws_eb) + bn * (long)Wq;
+    else return (KIND == kDirGradB ? p.a : p.b) + bn * (long)Wq;
+  }();
   const long cells_p = rows * Wp, cells_q = rows * Wq;
   const int p_min = (int)max(-bn * (long)Wp, -(1L << 30)), p_max = (int)min(cells_p - bn * (long)Wp - 1, 1L << 30);
   const int q_min = (int)max(-bn * (long)Wq, -(1L << 30)), q_max = (int)min(cells_q - bn * (long)Wq - 1, 1L << 30);
@@ -228,8 +235,8 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long b
         q[t] = qitem[o];
       }
     } else {
-      const dir_f4u w = *reinterpret_cast<const dir_f4u*>((qitem + soff) + qoff[0]);
-      q = mm_f4{w[0], w[1], w[2], w[3]};
+      const float4 w = ld4((qitem + soff) + qoff[0]);
+      q = mm_f4{w.x, w.y, w.z, w.w};
     }
   };
   // the first steps' cells of Q are asked for before anything else
@@ -263,8 +270,8 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long b
           }
         }
         if (!PROW && !EDGE) {
-          const dir_f4u x = *reinterpret_cast<const dir_f4u*>(pitem + (off_i + 16 * u));
-          v[s] = mm_f4{x[0], x[1], x[2], x[3]};
+          const float4 x = ld4(pitem + (off_i + 16 * u));
+          v[s] = mm_f4{x.x, x.y, x.z, x.w};
           if (MKH) {
             const dir_f4u y = *reinterpret_cast<const dir_f4u*>(ritem + (off_i + 16 * u));
             w[s] = mm_f4{y[0], y[1], y[2], y[3]};
@@ -364,8 +371,8 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long b
   // ---- results: accumulator element r is row i0 + 4 zq + r, column J0 + 16 tj + l15,
   // band cell jj = 16 tj + l15 - 4 zq - r
   const float thr = fast_exp2(-kBandGuardBits);
-  float* dst = KIND == kDirGradB ? p.o1 : p.o0;
-  float* orow = dst + (bn + i0) * (long)Wout;
+  elem_t* dst = KIND == kDirGradB ? p.o1 : p.o0;
+  elem_t* orow = dst + (bn + i0) * (long)Wout;
   float* rrow = FWD && PREP ? p.ws_r + (bn + i0) * (long)Wout : nullptr;
   const float* erow = MKH ? (GA ? p.ws_ea : p.ws_eb) + (bn + i0) * (long)Wout : nullptr;  // factor on the way out
   unsigned ooff[4];
@@ -419,7 +426,6 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long b
     const bool whole = (e & kDirWhole) && !tail;
     const int y = J0 + 16 * tj + l15;
     const bool y_in = y_all || (unsigned)y < (unsigned)n;
-    float* ot = (STAGE ? aux : orow) + 16 * tj;
     unsigned bits = 0;
     float be = 0.f;
     if (FWD && PREP) be = y_in ? p.ws_be[bn + y] : 0.f;
@@ -442,7 +448,8 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long b
           if (!(fabsf(v) <= FLT_MAX)) redo = 1;
           if (MKH && !STAGE) v *= (erow + 16 * tj)[ooff[r]];
         }
-        ot[ooff[r]] = v;
+        if (STAGE) (aux + 16 * tj)[ooff[r]] = v;
+        else (orow + 16 * tj)[ooff[r]] = to_elem<elem_t>(v);
       }
     }
     if (FWD && PREP) redo |= (unsigned __int128)bits << (4 * tj);
@@ -502,7 +509,7 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long b
         if (!ok) bad |= 0x80000000u >> c4;
         if (++jj == Wout) { jj = 0; ++row; }
       }
-      *reinterpret_cast<dir_f4u*>(orow + 4 * i) = dir_f4u{ov[0], ov[1], ov[2], ov[3]};
+      st4(orow + 4 * i, make_float4(ov[0], ov[1], ov[2], ov[3]));
       *reinterpret_cast<dir_f4u*>(rrow + 4 * i) = dir_f4u{rv[0], rv[1], rv[2], rv[3]};
       if (bad) {  // rare
         int r2 = (int)((float)(4 * i) * rw), j2 = 4 * i - r2 * Wout;
@@ -522,7 +529,7 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long b
       if (i < 4 * Wout) {
         mm_f4 v = so4[i];
         if (MKH) v = mm_f4{v[0] * ef[s][0], v[1] * ef[s][1], v[2] * ef[s][2], v[3] * ef[s][3]};
-        *reinterpret_cast<dir_f4u*>(orow + 4 * i) = dir_f4u{v[0], v[1], v[2], v[3]};
+        st4(orow + 4 * i, make_float4(v[0], v[1], v[2], v[3]));
       }
     }
     for (int i = lane + 64 * kDirEf; i < 4 * Wout; i += 64) {
@@ -531,7 +538,7 @@ __device__ __forceinline__ void dir_row(const BandArgs& p, const Plan& g, long b
         const dir_f4u f = *reinterpret_cast<const dir_f4u*>(erow + 4 * i);
         v = mm_f4{v[0] * f[0], v[1] * f[1], v[2] * f[2], v[3] * f[3]};
       }
-      *reinterpret_cast<dir_f4u*>(orow + 4 * i) = dir_f4u{v[0], v[1], v[2], v[3]};
+      st4(orow + 4 * i, make_float4(v[0], v[1], v[2], v[3]));
     }
   }
 

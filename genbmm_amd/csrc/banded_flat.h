@@ -12,23 +12,25 @@ namespace GENBMM_NS {
 constexpr int kMmSlack = 8;    // spare floats around a staged block
 typedef float mm_f4 __attribute__((ext_vector_type(4)));
 
-// `count` floats starting at tensor[first] - rows of W floats - read in 16-byte pieces
-// from the aligned address below and laid down with row stride `pitch`:
-// tensor[first + r * W + k] lands at L[origin() + r * pitch + k].
+// `count` elements starting at tensor[first] - rows of W elements - read in pieces of four
+// elements (16 bytes of floats, 8 of a half type) from the aligned address below and laid
+// down as floats with row stride `pitch`: tensor[first + r * W + k] lands at
+// L[origin() + r * pitch + k].
 // load() only issues the reads of one batch of 256 * U pieces, store() consumes them.
-template <int U>
+// E: float (a workspace) or the element type of the caller's tensors (widened by the load).
+template <int U, class E = float>
 struct MmFlat {
   mm_f4 v[U];
   int nvec, lead, W, gap;
   unsigned magic;  // ceil(2^32 / W)
-  const float* abeg;
+  const E* abeg;
   bool inside;     // every piece lies inside the tensor
 
-  // [tensor, tensor_end): the whole tensor; a piece that crosses its ends is read float by float
-  __device__ __forceinline__ void init(const float* tensor, const float* tensor_end, long first, int count,
+  // [tensor, tensor_end): the whole tensor; a piece that crosses its ends is read element by element
+  __device__ __forceinline__ void init(const E* tensor, const E* tensor_end, long first, int count,
                                        int W_, int pitch) {
-    const float* beg = tensor + first;
-    lead = (int)((reinterpret_cast<uintptr_t>(beg) & 15) >> 2);
+    const E* beg = tensor + first;
+    lead = (int)((reinterpret_cast<uintptr_t>(beg) & (4 * sizeof(E) - 1)) / sizeof(E));
     abeg = beg - lead;
     nvec = count > 0 ? (lead + count + 3) >> 2 : 0;
     W = W_;
@@ -38,13 +40,16 @@ struct MmFlat {
   }
   __device__ __forceinline__ int origin() const { return lead + gap; }
   __device__ __forceinline__ bool more(int batch) const { return batch * 256 * U < nvec; }
-  __device__ __forceinline__ void load(const float* lo, const float* hi, int batch, int tid) {
+  __device__ __forceinline__ void load(const E* lo, const E* hi, int batch, int tid) {
     if (inside) {  // uniform
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int vi = tid + 256 * (u + batch * U);
         v[u] = mm_f4{0.f, 0.f, 0.f, 0.f};
-        if (vi < nvec) v[u] = *reinterpret_cast<const mm_f4*>(abeg + 4 * vi);
+        if (vi < nvec) {
+          const float4 x = ld4a(abeg + 4 * vi);
+          v[u] = mm_f4{x.x, x.y, x.z, x.w};
+        }
       }
       return;
     }
@@ -53,7 +58,7 @@ struct MmFlat {
       const int vi = tid + 256 * (u + batch * U);
       mm_f4 x = mm_f4{0.f, 0.f, 0.f, 0.f};
       if (vi < nvec) {
-        const float* q = abeg + 4 * vi;
+        const E* q = abeg + 4 * vi;
         for (int t = 0; t < 4; ++t)
           if (q + t >= lo && q + t < hi) x[t] = q[t];
       }
@@ -83,48 +88,6 @@ struct MmFlat {
       }
     }
     return bad;
-  }
-  // v = g, rs.v = R = 1/S of the same cells (read with the same lead): v becomes
-  // H = g * R, NaN where R < 0 (the cell was computed exactly, its 1/S is not usable), and
-  // this strip's cells of it go to `h`, laid out like g - the other gradient reads them
-  // there.  h_vec: h + (abeg - tensor) is 16-byte aligned and every piece lies inside.
-  __device__ __forceinline__ void make_h(const MmFlat& rs, float* __restrict__ h, const float* tensor,
-                                         bool h_vec, int count, int batch, int tid) {
-    float* hb = h + (abeg - tensor);
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int vi = tid + 256 * (u + batch * U);
-      if (vi < nvec) {
-        mm_f4 x = v[u];
-        const mm_f4 r = rs.v[u];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) x[t] = r[t] < 0.f ? __builtin_nanf("") : x[t] * r[t];
-        v[u] = x;
-        if (h_vec) {
-          *reinterpret_cast<mm_f4*>(hb + 4 * vi) = x;
-        } else {
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const int e = 4 * vi + t - lead;
-            if (e >= 0 && e < count) hb[4 * vi + t] = x[t];
-          }
-        }
-      }
-    }
-  }
-  // the rows (first one row_first) that hold a value that is not finite
-  __device__ __forceinline__ void flag_rows(int batch, int tid, int count, int row_first, int* flags) const {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int vi = tid + 256 * (u + batch * U);
-      if (vi < nvec) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int e = 4 * vi + t - lead;
-          if (e >= 0 && e < count && !(fabsf(v[u][t]) <= FLT_MAX)) flags[row_first + e / W] = 1;
-        }
-      }
-    }
   }
 };
 

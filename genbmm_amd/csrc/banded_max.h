@@ -66,8 +66,8 @@ __global__ __launch_bounds__(256, 2) void k_band_max_fwd(const BandArgs p, int s
   const int q0 = x0 - r_lu + j_lo;  // first row of b that the segment's cells meet
   const int qr0 = max(q0, 0), qr1 = min(q0 + d.q_rows, n);
   const int pr1 = min(x0 + kMaxRows, n);
-  MmFlat<14> sq;
-  MmFlat<6> sp;
+  MmFlat<14, elem_t> sq;
+  MmFlat<6, elem_t> sp;
   sq.init(p.b, p.b + cells_b, (bn + qr0) * Wb, (qr1 - qr0) * Wb, Wb, d.qp);
   sq.load(p.b, p.b + cells_b, 0, tid);
   sp.init(p.a, p.a + cells_a, (bn + x0) * Wa, (pr1 - x0) * Wa, Wa, d.pp);
@@ -181,19 +181,19 @@ __global__ __launch_bounds__(256, 2) void k_band_max_fwd(const BandArgs p, int s
   __syncthreads();
 
   const int rows = min(kMaxRows, n - x0), cells = rows * Ws;
-  float* ob = p.o0 + (bn + x0) * Wo + j_lo;
+  elem_t* ob = p.o0 + (bn + x0) * Wo + j_lo;
   int32_t* ib = p.oidx + (bn + x0) * Wo + j_lo;
   typedef int mm_i4 __attribute__((ext_vector_type(4)));
   if (Ws == Wo && (cells & 3) == 0 &&
       ((reinterpret_cast<uintptr_t>(ob) | reinterpret_cast<uintptr_t>(ib)) & 15) == 0) {
     for (int e = 4 * tid; e < cells; e += 1024) {  // the strip's rows are one contiguous run
-      *reinterpret_cast<mm_f4*>(ob + e) = *reinterpret_cast<const mm_f4*>(Sv + e);
+      st4a(ob + e, *reinterpret_cast<const float4*>(Sv + e));
       *reinterpret_cast<mm_i4*>(ib + e) = *reinterpret_cast<const mm_i4*>(Si + e);
     }
   } else {
     for (int e = tid; e < cells; e += 256) {  // runs of Ws cells, one per row
       const int r = e / Ws, c = e - r * Ws;
-      ob[(long)r * Wo + c] = Sv[e];
+      ob[(long)r * Wo + c] = to_elem<elem_t>(Sv[e]);
       ib[(long)r * Wo + c] = Si[e];
     }
   }

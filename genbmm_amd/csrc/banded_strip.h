@@ -69,7 +69,9 @@ struct RowStage {
   static constexpr int U = (ROWS + 3) / 4;
   float v[U][NQ];
 
-  __device__ __forceinline__ void load(const float* __restrict__ src, int W, int lu, int n, int row0,
+  // E: float (a workspace) or the element type of the caller's tensors (widened here)
+  template <class E>
+  __device__ __forceinline__ void load(const E* __restrict__ src, int W, int lu, int n, int row0,
                                        int ld, int pad, int wave, int lane) {
     const float fill = SEM == kSemMul ? 0.f : -INFINITY;
     // Strips away from the matrix edges (all but a few per batch item): every staged
@@ -78,7 +80,7 @@ struct RowStage {
     // five comparisons per element.
     const bool interior = row0 - lu >= 0 && row0 + ROWS + W - 2 - lu <= n - 1;  // uniform
     if (interior) {
-      const float* base = src + (long)(row0 + wave) * W - pad + lane;
+      const E* base = src + (long)(row0 + wave) * W - pad + lane;
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
         const int col = lane + 64 * q, k = col - pad;
@@ -140,7 +142,7 @@ struct RowStage {
 // one contiguous block of memory, moved 16 bytes per lane in both directions - and turns them
 // in LDS (row stride ld, odd) so that 256 / R lanes share a row.
 struct PrepSide {
-  const float* x;
+  const elem_t* x;
   float* e;
   float* shift;
   int W, lu, ld;
@@ -155,7 +157,7 @@ __device__ __forceinline__ void band_prep_block(const PrepSide& q, float* __rest
   const int tid = threadIdx.x, W = q.W, ld = q.ld;
   const int nr = (int)min((long)R, rows - row0);
   const int cells = nr * W;
-  const float* xb = q.x + row0 * W;
+  const elem_t* xb = q.x + row0 * W;
   float* eb = q.e + row0 * W;
   constexpr int U = 8;
   // Index arithmetic is what this kernel would otherwise spend its time on: the LDS offset of a
@@ -171,7 +173,7 @@ __device__ __forceinline__ void band_prep_block(const PrepSide& q, float* __rest
       float4 v[U];
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        if (i0 + 256 * u < quads) v[u] = *reinterpret_cast<const float4*>(xb + 4 * (i0 + 256 * u));
+        if (i0 + 256 * u < quads) v[u] = ld4a(xb + 4 * (i0 + 256 * u));
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         if (i0 + 256 * u < quads) {
@@ -279,9 +281,16 @@ __global__ __launch_bounds__(256, (SEM == kSemMul || SEM == kSemLogPrep) ? 3 : 2
   const int wg = xcd_strip_id();
   const int batch = wg / strips, i0 = (wg - batch * strips) * kBT;
   const int n = p.n, Wa = p.Wa, Wb = p.Wb, Wo = p.Wo;
-  const float* ab = (PREP ? p.ws_ea : p.a) + (long)batch * n * Wa;
-  const float* bb = (PREP ? p.ws_eb : p.b) + (long)batch * n * Wb;
-  float* ob = p.o0 + (long)batch * n * Wo;
+  // the prepared product reads the workspace's factors (float), the others the caller's tensors
+  auto ab = [&] {
+    if constexpr (PREP) return static_cast<const float*>(p.ws_ea) + (long)batch * n * Wa;
+    else return p.a + (long)batch * n * Wa;
+  }();
+  auto bb = [&] {
+    if constexpr (PREP) return static_cast<const float*>(p.ws_eb) + (long)batch * n * Wb;
+    else return p.b + (long)batch * n * Wb;
+  }();
+  elem_t* ob = p.o0 + (long)batch * n * Wo;
   int32_t* ib = MAXP ? p.oidx + (long)batch * n * Wo : nullptr;
   float* rb = PREP ? p.ws_r + (long)batch * n * Wo : nullptr;
   const long bn = (long)batch * n;
@@ -399,7 +408,7 @@ __global__ __launch_bounds__(256, (SEM == kSemMul || SEM == kSemLogPrep) ? 3 : 2
     for (int e = tid; e < kBT * kBJ; e += 256) {
       const int r = e >> 5, c = e & 31;
       if (i0 + r < n && jc + c < Wo) {
-        ob[(long)(i0 + r) * Wo + jc + c] = Cs[r * kBC + c];
+        ob[(long)(i0 + r) * Wo + jc + c] = to_elem<elem_t>(Cs[r * kBC + c]);
         if (MAXP) ib[(long)(i0 + r) * Wo + jc + c] = Is[r * kBC + c];
         if (PREP) rb[(long)(i0 + r) * Wo + jc + c] = Rt[r * kBC + c];
       }
@@ -429,8 +438,8 @@ struct GStage {
 
   // [U0, U1): the pieces handled by this call (all of them, or a few at a time where
   // registers are short)
-  template <int U0 = 0, int U1 = PER>
-  __device__ __forceinline__ void load(const float* __restrict__ gb, const float* __restrict__ ob,
+  template <int U0 = 0, int U1 = PER, class G, class O>
+  __device__ __forceinline__ void load(const G* __restrict__ gb, const O* __restrict__ ob,
                                        int x0, int yb, int jc, int n, int Wo, int r_lu, int tid) {
     if (U0 == 0) used = 0;
 #pragma unroll
@@ -479,7 +488,7 @@ constexpr int kMaxKB = 3;  // band-axis blocks of 8 per wave: widths up to 96
 // H = g * R for the prepared log backward, once for both gradients; R < 0 marks a
 // cell that the forward computed exactly (its 1/S is not usable): NaN there, which
 // the gradient kernels turn into "redo this row exactly".
-__global__ __launch_bounds__(256) void k_band_h(const float* __restrict__ g,
+__global__ __launch_bounds__(256) void k_band_h(const elem_t* __restrict__ g,
                                                const float* __restrict__ r,
                                                float* __restrict__ h, long cells) {
   const long stride = (long)gridDim.x * 1024;
@@ -489,7 +498,7 @@ __global__ __launch_bounds__(256) void k_band_h(const float* __restrict__ g,
       const long i = e + 256 * u;
       if (i < cells) {
         const float rv = r[i];
-        h[i] = rv < 0.f ? __builtin_nanf("") : g[i] * rv;
+        h[i] = rv < 0.f ? __builtin_nanf("") : (float)g[i] * rv;
       }
     }
   }
@@ -519,16 +528,26 @@ __global__ __launch_bounds__(256, 3) void k_band_bwd_strip(const BandArgs p, int
   const int batch = wg / strips, x0 = (wg - batch * strips) * kBT;
   const int n = p.n, Wa = p.Wa, Wb = p.Wb, Wo = p.Wo;
   const long bn = (long)batch * n;
-  const float* ab = (PREP ? p.ws_ea : p.a) + bn * Wa;
-  const float* bb = (PREP ? p.ws_eb : p.b) + bn * Wb;
-  const float* gb = (PREP ? p.ws_h : p.g) + bn * Wo;  // PREP: H = g / S, staged once for both gradients
-  const float* ob = LOG ? p.out + bn * Wo : nullptr;
+  // the prepared product reads the workspace (float), the others the caller's tensors
+  auto ab = [&] {
+    if constexpr (PREP) return static_cast<const float*>(p.ws_ea) + bn * Wa;
+    else return p.a + bn * Wa;
+  }();
+  auto bb = [&] {
+    if constexpr (PREP) return static_cast<const float*>(p.ws_eb) + bn * Wb;
+    else return p.b + bn * Wb;
+  }();
+  auto gb = [&] {  // PREP: H = g / S, staged once for both gradients
+    if constexpr (PREP) return static_cast<const float*>(p.ws_h) + bn * Wo;
+    else return p.g + bn * Wo;
+  }();
+  const elem_t* ob = LOG ? p.out + bn * Wo : nullptr;
   // output operand / other operand
-  const float* xo = GRAD_A ? ab : bb;
-  const float* yo = GRAD_A ? bb : ab;
+  auto xo = GRAD_A ? ab : bb;
+  auto yo = GRAD_A ? bb : ab;
   const int Wx = GRAD_A ? Wa : Wb, Wy = GRAD_A ? Wb : Wa;
   const int lux = GRAD_A ? p.a_lu : p.b_lu, luy = GRAD_A ? p.b_lu : p.a_lu;
-  float* gradb = (GRAD_A ? p.o0 : p.o1) + bn * Wx;
+  elem_t* gradb = (GRAD_A ? p.o0 : p.o1) + bn * Wx;
   const float lim = kBandGuardBits * kLn2 + 1e-3f;
 
   if (tid < kBT) badrow[tid] = 0;
@@ -567,9 +586,9 @@ __global__ __launch_bounds__(256, 3) void k_band_bwd_strip(const BandArgs p, int
         if (inside && (GRAD_A || (o >= x0 && o < x0 + kBT))) {
           const float sa = GRAD_A ? sh_own[r] : sh_sl[r];
           const float sb = GRAD_A ? sh_sl[r + c] : sh_own[o - x0];
-          const float ex = sa + sb - ob[(long)i * Wo + j];  // alpha[i] + beta[o] - out[i,j]
+          const float ex = sa + sb - (float)ob[(long)i * Wo + j];  // alpha[i] + beta[o] - out[i,j]
           if (!(ex <= lim)) badrow[GRAD_A ? r : o - x0] = 1;  // factoring not exact: row redone
-          v = gb[(long)i * Wo + j] * fast_exp2(ex * kLog2e);
+          v = (float)gb[(long)i * Wo + j] * fast_exp2(ex * kLog2e);
         }
         gt[r * kBC + c] = v;
       }
@@ -663,16 +682,16 @@ __global__ __launch_bounds__(256, 3) void k_band_bwd_strip(const BandArgs p, int
         // exp(x - shift); cells outside the matrix are excluded from the row maximum
         // and their sum is 0
         const float acv = ct[r * ld_own + k];
-        gradb[(long)x * Wx + k] = acv == 0.f ? 0.f : fast_exp2((xv[rr][q] - sh) * kLog2e) * acv;
+        gradb[(long)x * Wx + k] = to_elem<elem_t>(acv == 0.f ? 0.f : fast_exp2((xv[rr][q] - sh) * kLog2e) * acv);
       }
     } else if (PREP) {
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
         const int k = lane + 64 * q;
-        if (k < Wx) gradb[(long)x * Wx + k] = xv[rr][q] * ct[r * ld_own + k];
+        if (k < Wx) gradb[(long)x * Wx + k] = to_elem<elem_t>(xv[rr][q] * ct[r * ld_own + k]);
       }
     } else {
-      for (int k = lane; k < Wx; k += 64) gradb[(long)x * Wx + k] = ct[r * ld_own + k];
+      for (int k = lane; k < Wx; k += 64) gradb[(long)x * Wx + k] = to_elem<elem_t>(ct[r * ld_own + k]);
     }
   }
 }

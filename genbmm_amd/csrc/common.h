@@ -367,8 +367,16 @@ __device__ __forceinline__ void add4_ordered(float* __restrict__ accs, const int
 // ------------------------------------------------------------- host helpers
 inline int check_dense_dims(int B, int M, int K, int N) {
   if (B < 0 || M < 0 || K < 0 || N < 0) return GENBMM_E_SHAPE;
-  const int64_t lim = (int64_t)1 << 40;  // element counts are 64-bit inside
+  // element counts are 64-bit inside; 2^37 elements (half a terabyte of floats) is beyond
+  // any device buffer and keeps one-lane-per-cell grids (cells / 256) within 32 bits
+  const int64_t lim = (int64_t)1 << 37;
   if ((int64_t)B * M * K > lim || (int64_t)B * K * N > lim || (int64_t)B * M * N > lim)
+    return GENBMM_E_SHAPE;
+  // launch grids: one workgroup per tile of 32 x 32 at the smallest, two tile lists in one
+  // launch at the most - a grid beyond 2^31 - 1 workgroups would wrap silently
+  const int64_t grid_lim = (int64_t)1 << 30;
+  auto tiles = [](int64_t batch, int x, int y) { return batch * ((x + 31) / 32) * ((y + 31) / 32); };
+  if (tiles(B, M, N) > grid_lim || tiles(B, M, K) > grid_lim || tiles(B, K, N) > grid_lim)
     return GENBMM_E_SHAPE;
   return GENBMM_OK;
 }

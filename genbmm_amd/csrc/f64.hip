@@ -485,9 +485,9 @@ int genbmm_banded_bwdbwd_f64(const double* a, int a_lu, int a_ld, const double* 
   p.o0 = grad_a; p.o1 = grad_b; p.o2 = grad_g;
   const long ta = (long)B * n * p.Wa, tb = (long)B * n * p.Wb, to = (long)B * n * p.Wo;
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(k_band_bb_t<double>, blocks_for(to), dim3(256), 0, s, p, to);
-  hipLaunchKernelGGL(k_band_bb_a<double>, blocks_for(ta), dim3(256), 0, s, p, ta);
-  hipLaunchKernelGGL(k_band_bb_b<double>, blocks_for(tb), dim3(256), 0, s, p, tb);
+  hipLaunchKernelGGL(k_band_bb_t<double>, blocks_for(to), dim3(256), 0, s, p, grad_g, to);
+  hipLaunchKernelGGL(k_band_bb_a<double>, blocks_for(ta), dim3(256), 0, s, p, grad_g, ta);
+  hipLaunchKernelGGL(k_band_bb_b<double>, blocks_for(tb), dim3(256), 0, s, p, grad_g, tb);
   return launch_status();
 }
 

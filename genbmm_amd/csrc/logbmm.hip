@@ -660,7 +660,11 @@ int launch_fwd_mfma(DenseArgs p, float* stats, int B, int M, int K, int N, bool 
   p.M = M; p.K = K; p.N = N;
   p.tiles_m = ceil_div(M, T::TR);
   p.tiles_n = ceil_div(N, T::TC);
-  p.vec_a = p.vec_b = p.vec_o = 1;
+  // what the exact fix-up may read and write four aligned elements at a time (the matrix-core
+  // kernel itself takes any alignment and ignores these)
+  p.vec_a = (K % 4 == 0) && aligned16(p.a);
+  p.vec_b = (N % 4 == 0) && aligned16(p.b);
+  p.vec_o = (N % 4 == 0) && aligned16(p.out);
   const int total = B * p.tiles_m * p.tiles_n;
   const LogPrepared ws = prepared_of(stats, B, M, K, N);
   int* flags = fwd_flags_of(stats, B, M, N);

@@ -324,10 +324,13 @@ def logbmm(a, b):
     N = b.shape[2]
     S = 1 if _f64(a) else _reduction_splits(B, M, K, N)
     if S > 1:  # differentiable torch operations around the same kernels (any order of derivative)
-        a_s = a.view(B, M, S, K // S).transpose(1, 2).reshape(B * S, M, K // S).contiguous()
-        b_s = b.view(B * S, K // S, N)
+        # float16 / bfloat16 operands: the pieces are formed and joined in float32 and the result is
+        # rounded once, as the unsplit kernels do (a piece stored in the half type would round twice)
+        wide = a.float() if a.dtype in _lib.HALF_SUFFIX else a
+        a_s = wide.view(B, M, S, K // S).transpose(1, 2).reshape(B * S, M, K // S).contiguous()
+        b_s = (b.float() if b.dtype in _lib.HALF_SUFFIX else b).view(B * S, K // S, N)
         parts = LogMatMul.apply(a_s, b_s, PATH_AUTO).view(B, S, M, N)
-        return restore(torch.logsumexp(parts.float(), dim=1).to(a.dtype))
+        return restore(torch.logsumexp(parts, dim=1).to(a.dtype))
     return restore(LogMatMul.apply(a, b, PATH_AUTO))
 
 

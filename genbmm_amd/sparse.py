@@ -312,15 +312,9 @@ class BandedMatrix:
         ld = self.ld + other.lu
         # views are copied here, by a differentiable torch operation, so that the
         # Functions save (and differentiate with respect to) what they were given
+        # (float16 / bfloat16 bands go to the `_f16` / `_bf16` entry points as they are)
         a, b = self.data, other.data
-        # float16 / bfloat16 bands are widened for the kernels and the result narrowed again (the
-        # banded entry points exist for float and double); the casts are differentiable
-        half = a.dtype if a.dtype in (torch.float16, torch.bfloat16) and b.dtype == a.dtype else None
-        if half is not None:
-            a, b = a.float(), b.float()
         out = fn(a.contiguous(), self.lu, self.ld, b.contiguous(), other.lu, other.ld, lu, ld)
-        if half is not None:
-            out = out.to(half)
         return BandedMatrix(out, lu, ld, self.fill)
 
     def multiply(self, other):
@@ -358,8 +352,15 @@ def _f64(t):
     return t.dtype == torch.float64
 
 
+def _sfx(t):
+    """Entry-point suffix for the tensor's element type ("", "_f16", "_bf16")."""
+    return _lib.HALF_SUFFIX.get(t.dtype, "")
+
+
 def _check_pair(a, b):
-    dtype = torch.float64 if isinstance(a, torch.Tensor) and _f64(a) else torch.float32
+    dtype = torch.float32
+    if isinstance(a, torch.Tensor) and (_f64(a) or a.dtype in _lib.HALF_SUFFIX):
+        dtype = a.dtype
     _lib.require(a, "a", dtype=dtype)
     _lib.require(b, "b", dtype=dtype, device=a.device)
     if a.shape[:2] != b.shape[:2]:
@@ -392,7 +393,7 @@ def _forward(a, a_lu, a_ld, b, b_lu, b_ld, mode):
     if mode == MODE_LOG:
         size = _lib.load().genbmm_banded_workspace_size(a_lu, a_ld, b_lu, b_ld, B, n)
         ws = torch.empty(size, dtype=torch.float32, device=a.device)
-    _call("genbmm_banded_fwd", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
+    _call("genbmm_banded_fwd" + _sfx(a), a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
           _lib.ptr(out), _lib.ptr(idx), _lib.ptr(ws), B, n, mode)
     return a, b, out, (ws if mode == MODE_LOG else idx)
 
@@ -414,7 +415,7 @@ def _backward(a, b, bands, out, idx, g, mode, ws=None):
     if mode == MODE_LOG and ws is not None:
         need = _lib.load().genbmm_banded_scratch_size(a_lu, a_ld, b_lu, b_ld, B, n)
         scratch = torch.empty(need, dtype=torch.float32, device=a.device) if need else None
-    _call("genbmm_banded_bwd_scratch", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
+    _call("genbmm_banded_bwd_scratch" + _sfx(a), a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
           _lib.ptr(out), _lib.ptr(idx), _lib.ptr(ws), _lib.ptr(scratch), _lib.ptr(g), _lib.ptr(grad_a),
           _lib.ptr(grad_b), B, n, mode)
     return grad_a, grad_b
@@ -463,6 +464,13 @@ class _BandedLogGrad(torch.autograd.Function):
         u_a = None if u_a is None else u_a.contiguous()
         u_b = None if u_b is None else u_b.contiguous()
         ga, gb, gg = torch.empty_like(a), torch.empty_like(b), torch.empty_like(g)
+        if a.dtype in _lib.HALF_SUFFIX:
+            # the gradient with respect to g is read back by the other two: a float copy of it
+            t = torch.empty(g.shape, dtype=torch.float32, device=g.device)
+            _call("genbmm_banded_bwdbwd" + _sfx(a), a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
+                  _lib.ptr(out), _lib.ptr(g), _lib.ptr(u_a), _lib.ptr(u_b), _lib.ptr(ga), _lib.ptr(gb),
+                  _lib.ptr(gg), _lib.ptr(t), a.shape[0], a.shape[1])
+            return ga, gb, gg, None, None, None
         _call("genbmm_banded_bwdbwd_f64" if _f64(a) else "genbmm_banded_bwdbwd", a, _lib.ptr(a),
               a_lu, a_ld, _lib.ptr(b), b_lu, b_ld, _lib.ptr(out), _lib.ptr(g), _lib.ptr(u_a), _lib.ptr(u_b),
               _lib.ptr(ga), _lib.ptr(gb), _lib.ptr(gg), a.shape[0], a.shape[1])
@@ -535,7 +543,7 @@ class BandedSampleMul(torch.autograd.Function):
         else:
             size = _lib.load().genbmm_banded_workspace_size(a_lu, a_ld, b_lu, b_ld, B, n)
             ws = torch.empty(size, dtype=torch.float32, device=a.device)
-            _call("genbmm_banded_sample_fwd", a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
+            _call("genbmm_banded_sample_fwd" + _sfx(a), a, _lib.ptr(a), a_lu, a_ld, _lib.ptr(b), b_lu, b_ld,
                   _lib.ptr(out), _lib.ptr(idx), _lib.ptr(ws), seed, offset, B, n)
         ctx.save_for_backward(a, b, idx)
         ctx.bands = (a_lu, a_ld, b_lu, b_ld)

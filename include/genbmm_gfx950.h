@@ -498,8 +498,14 @@ int genbmm_banded_bwdbwd_f64(const double* a, int a_lu, int a_ld,
  * workspace (matrix-core shapes, K <= 992) and walks the terms exactly
  * otherwise (`out` rounded to 11 or 8 bits does not give S well enough for the
  * other sweeps): its index is the float function's on those shapes and the
- * index of the float function called with stats = NULL on all others.  genbmm_logbmm_bwdbwd and the banded functions have no half
- * form: callers widen those tensors.
+ * index of the float function called with stats = NULL on all others.
+ * The banded functions likewise (the reference instantiates every banded kernel
+ * for Half too, banded_cuda_kernel.cu:389, :435, :484, :508, :530): band data,
+ * results, g and gradients in the 16-bit type, `workspace` and `scratch` float
+ * with the sizes of the float functions.  The second-order function takes one
+ * more buffer, `t_scratch` (B * n * Wo floats): the gradient with respect to g
+ * is read back by the other two gradients and must stay unrounded there
+ * (grad_g receives it rounded).
  */
 int genbmm_logbmm_fwd_f16(const uint16_t* a, const uint16_t* b, uint16_t* out,
                           float* stats, int B, int M, int K, int N, void* stream);
@@ -557,6 +563,61 @@ int genbmm_prodmax_bwd_bf16(const uint16_t* a, const uint16_t* b, const int32_t*
                             const float* factors, const uint16_t* g,
                             uint16_t* grad_a, uint16_t* grad_b,
                             int B, int M, int K, int N, void* stream);
+
+int genbmm_banded_fwd_f16(const uint16_t* a, int a_lu, int a_ld,
+                          const uint16_t* b, int b_lu, int b_ld,
+                          uint16_t* out, int32_t* idx, float* workspace,
+                          int B, int n, int mode, void* stream);
+int genbmm_banded_sample_fwd_f16(const uint16_t* a, int a_lu, int a_ld,
+                                 const uint16_t* b, int b_lu, int b_ld,
+                                 uint16_t* out, int32_t* idx, float* workspace,
+                                 uint64_t seed, uint64_t offset,
+                                 int B, int n, void* stream);
+int genbmm_banded_bwd_f16(const uint16_t* a, int a_lu, int a_ld,
+                          const uint16_t* b, int b_lu, int b_ld,
+                          const uint16_t* out, const int32_t* idx,
+                          float* workspace, const uint16_t* g,
+                          uint16_t* grad_a, uint16_t* grad_b,
+                          int B, int n, int mode, void* stream);
+int genbmm_banded_bwd_scratch_f16(const uint16_t* a, int a_lu, int a_ld,
+                                  const uint16_t* b, int b_lu, int b_ld,
+                                  const uint16_t* out, const int32_t* idx,
+                                  const float* workspace, float* scratch,
+                                  const uint16_t* g, uint16_t* grad_a, uint16_t* grad_b,
+                                  int B, int n, int mode, void* stream);
+int genbmm_banded_bwdbwd_f16(const uint16_t* a, int a_lu, int a_ld,
+                             const uint16_t* b, int b_lu, int b_ld,
+                             const uint16_t* out, const uint16_t* g,
+                             const uint16_t* u_a, const uint16_t* u_b,
+                             uint16_t* grad_a, uint16_t* grad_b, uint16_t* grad_g,
+                             float* t_scratch, int B, int n, void* stream);
+int genbmm_banded_fwd_bf16(const uint16_t* a, int a_lu, int a_ld,
+                          const uint16_t* b, int b_lu, int b_ld,
+                          uint16_t* out, int32_t* idx, float* workspace,
+                          int B, int n, int mode, void* stream);
+int genbmm_banded_sample_fwd_bf16(const uint16_t* a, int a_lu, int a_ld,
+                                 const uint16_t* b, int b_lu, int b_ld,
+                                 uint16_t* out, int32_t* idx, float* workspace,
+                                 uint64_t seed, uint64_t offset,
+                                 int B, int n, void* stream);
+int genbmm_banded_bwd_bf16(const uint16_t* a, int a_lu, int a_ld,
+                          const uint16_t* b, int b_lu, int b_ld,
+                          const uint16_t* out, const int32_t* idx,
+                          float* workspace, const uint16_t* g,
+                          uint16_t* grad_a, uint16_t* grad_b,
+                          int B, int n, int mode, void* stream);
+int genbmm_banded_bwd_scratch_bf16(const uint16_t* a, int a_lu, int a_ld,
+                                  const uint16_t* b, int b_lu, int b_ld,
+                                  const uint16_t* out, const int32_t* idx,
+                                  const float* workspace, float* scratch,
+                                  const uint16_t* g, uint16_t* grad_a, uint16_t* grad_b,
+                                  int B, int n, int mode, void* stream);
+int genbmm_banded_bwdbwd_bf16(const uint16_t* a, int a_lu, int a_ld,
+                             const uint16_t* b, int b_lu, int b_ld,
+                             const uint16_t* out, const uint16_t* g,
+                             const uint16_t* u_a, const uint16_t* u_b,
+                             uint16_t* grad_a, uint16_t* grad_b, uint16_t* grad_g,
+                             float* t_scratch, int B, int n, void* stream);
 
 #ifdef __cplusplus
 }

@@ -859,6 +859,27 @@ def test_long_reductions_with_few_tiles_are_split(gpu, B, M, K, N):
         close(db, w2[1], rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_long_reductions_split_with_half_tensors(gpu, dtype):
+    """The split of a long reduction on float16 / bfloat16 operands keeps the half contract: what
+    the float function returns on the widened tensors, rounded once (pieces are formed and joined
+    in float32) - forward and gradients, bit for bit."""
+    B, M, K, N = 2, 40, 4096, 30
+    assert genmul._reduction_splits(B, M, K, N) > 1
+    torch.manual_seed(3)
+    a, b, g = torch.randn(B, M, K).to(dtype), torch.randn(B, K, N).to(dtype), torch.randn(B, M, N).to(dtype)
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    out = genbmm.logbmm(ad, bd)
+    assert out.dtype == dtype
+    ga, gb = torch.autograd.grad(out, (ad, bd), g.to(gpu))
+    af, bf = a.float().to(gpu).requires_grad_(True), b.float().to(gpu).requires_grad_(True)
+    ref = genbmm.logbmm(af, bf)
+    ra, rb = torch.autograd.grad(ref, (af, bf), g.float().to(gpu))
+    assert torch.equal(out, ref.to(dtype))
+    assert torch.equal(ga, ra.to(dtype)) and torch.equal(gb, rb.to(dtype))
+    close(out.float(), oracle.logbmm_grads64(a.float(), b.float(), g.float())[0], rtol=2.0 ** -8, atol=1e-3)
+
+
 def test_half_inputs_are_twice_differentiable(gpu):
     """float16 / bfloat16 operands stay in their type through forward and backward; the
     double backward widens what the first backward saved, so second-order terms reach the

@@ -121,7 +121,7 @@ def test_module_level_names_of_the_reference():
 def test_library_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "genbmm_gfx950.h")).read()
     declared = set(re.findall(r"\b(genbmm_[a-z_0-9]+)\s*\(", header))
-    assert len(declared) == 58
+    assert len(declared) == 68
     assert declared == set(_lib.SIGNATURES) | set(_lib.STRING_FUNCS) | set(_lib.SIZE_FUNCS)
     assert os.path.exists(_lib.LIB_PATH), "build with `python -m genbmm_amd.build`"
     lib = ctypes.CDLL(_lib.LIB_PATH)
@@ -131,6 +131,60 @@ def test_library_exports_every_declared_symbol():
     assert lib.genbmm_version().startswith(b"genbmm-gfx950")
     lib.genbmm_error_string.restype = ctypes.c_char_p
     assert lib.genbmm_error_string(-2) == b"a dimension is negative or too large"
+
+
+def test_banded_workspace_and_scratch_sizes_agree_on_the_backward_path():
+    """The log product's workspace holds a place for H = g / S exactly when the backward is not
+    the memory-fed one (which forms H on the fly and needs no scratch either): for every band
+    shape, either workspace = rows * (Wa + Wb + Wo + 2) and scratch = 0, or the workspace has
+    Wo more floats per row and scratch is 0 (workspace unused) or rows * Wo.  Host code only."""
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in ("genbmm_banded_workspace_size", "genbmm_banded_scratch_size"):
+        getattr(lib, name).restype = ctypes.c_size_t
+        getattr(lib, name).argtypes = [ctypes.c_int] * 6
+    B, n = 3, 500
+    rows = B * n
+    lean = full = 0
+    widths = list(range(0, 9)) + [15, 16, 32, 48, 60, 100, 110, 111, 112, 113, 120, 127, 128, 140]
+    for lu in widths:
+        for ld in (lu, max(lu - 1, 0), 0):
+            for blu, bld in ((lu, ld), (1, 2), (ld, lu)):
+                Wa, Wb = lu + ld + 1, blu + bld + 1
+                Wo = Wa + Wb - 1
+                ws = lib.genbmm_banded_workspace_size(lu, ld, blu, bld, B, n)
+                sc = lib.genbmm_banded_scratch_size(lu, ld, blu, bld, B, n)
+                if ws == rows * (Wa + Wb + Wo + 2):
+                    assert sc == 0, (lu, ld, blu, bld)
+                    lean += 1
+                else:
+                    assert ws == rows * (Wa + Wb + 2 * Wo + 2), (lu, ld, blu, bld)
+                    assert sc in (0, rows * Wo), (lu, ld, blu, bld)
+                    full += 1
+    assert lean > 20 and full > 5
+    assert lib.genbmm_banded_workspace_size(-1, 0, 0, 0, B, n) == 0
+
+
+def test_launch_grids_beyond_32_bits_are_refused():
+    """Shapes whose launch grid would exceed 2^31 - 1 workgroups (and wrap silently) return
+    GENBMM_E_SHAPE before anything is launched or any pointer is read.  Host code only."""
+    lib = _lib.load()
+    fake = ctypes.c_void_p(256)      # never dereferenced: the shape check comes first
+    E_SHAPE = -2
+    # banded: 2^30 batch items of 64 rows -> 2^32 tile rows
+    for mode in (0, 1, 3):
+        assert lib.genbmm_banded_fwd(fake, 1, 1, fake, 1, 1, fake, fake, None, 1 << 30, 64, mode, None) == E_SHAPE
+    assert lib.genbmm_banded_bwd(fake, 1, 1, fake, 1, 1, fake, fake, None, fake, fake, fake, 1 << 30, 64, 3, None) == E_SHAPE
+    assert lib.genbmm_banded_sample_fwd(fake, 1, 1, fake, 1, 1, fake, fake, None, 1, 0, 1 << 30, 64, None) == E_SHAPE
+    # dense: 2^37 result cells pass the element count, their 2^32 tiles of 32 x 32 do not
+    B, M, K, N = 1 << 20, 1, 1, 1 << 17
+    assert lib.genbmm_maxbmm_fwd(fake, fake, fake, fake, B, M, K, N, None) == E_SHAPE
+    assert lib.genbmm_logbmm_fwd(fake, fake, fake, None, B, M, K, N, None) == E_SHAPE
+    assert lib.genbmm_logbmm_bwd(fake, fake, fake, fake, None, fake, fake, B, M, K, N, None) == E_SHAPE
+    assert lib.genbmm_samplebmm_fwd(fake, fake, fake, fake, None, 1, 0, B, M, K, N, None) == E_SHAPE
+    assert lib.genbmm_argmax_bwd(fake, fake, fake, fake, B, M, K, N, None) == E_SHAPE
+    assert lib.genbmm_logbmm_fwd_f64(fake, fake, fake, B, M, K, N, None) == E_SHAPE
+    # an ordinary large problem is still accepted by the size functions
+    assert lib.genbmm_logbmm_stats_size(64, 512, 512, 512) > 0
 
 
 def test_half_builds_compute_in_float():
@@ -145,7 +199,7 @@ def test_half_builds_compute_in_float():
     if not os.path.exists(hipcc):
         pytest.skip("hipcc not present")
     jobs = [(src, elem) for src, variants in hip_build.PER_ELEMENT.items() for _, elem in variants if elem]
-    assert len(jobs) == 6
+    assert len(jobs) == 8
 
     def ir(job):
         src, elem = job
@@ -156,7 +210,7 @@ def test_half_builds_compute_in_float():
 
     narrow = re.compile(r"= (fadd|fsub|fmul|fdiv|frem|fneg|fcmp \w+) [^\n]*?(<\d+ x )?(half|bfloat)\b"
                         r"|call [^\n]*llvm\.(maxnum|minnum|fma|fmuladd|maximum|minimum)\.(v\d+)?(f16|bf16)")
-    with ThreadPoolExecutor(max_workers=6) as pool:
+    with ThreadPoolExecutor(max_workers=8) as pool:
         for job, text in zip(jobs, pool.map(ir, jobs)):
             assert "define" in text and ("half" in text or "bfloat" in text), job
             hits = [m.group(0) for m in narrow.finditer(text)]
