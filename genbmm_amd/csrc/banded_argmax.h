@@ -10,9 +10,12 @@
 // which are the reference's summation orders (banded_cuda_kernel.cu:104-152 and
 // the transposed call of sparse.py:625-635), so the sums come out bit for bit.
 // One workgroup per strip of 64 rows; a lane owns a row of the gradient and walks
-// its cells in that order, accumulating in LDS (stride 65: conflict-free both for
-// lanes on one k and for the row-wise write-out).  g and idx pass through LDS
-// tiles of 32 diagonals so that global memory is read in runs along the band.
+// its cells in that order, accumulating in LDS at [k][lane]: whatever k each of the 64
+// lanes adds to, the lanes stay in 64 different banks (with the rows 65 apart a wave's
+// additions met at random: 11.6 M conflict cycles per launch at 64 x 4096, 65 diagonals).
+// For the row-wise write-out the sums change places once, through registers, to [row][k]
+// with an odd row length.  g and idx pass through LDS tiles of 32 diagonals so that global
+// memory is read in runs along the band.
 // Cells outside the matrix carry index 0 from the forward and are masked here.
 #pragma once
 
@@ -23,12 +26,34 @@ namespace GENBMM_NS {
 constexpr int kAT = 64;        // rows per strip
 constexpr int kAJ = 32;        // diagonals per tile
 constexpr int kAC = kAJ + 1;   // tile row stride
-constexpr int kAS = kAT + 1;   // accumulator stride
+constexpr int kAS = kAT;       // accumulators: [k][lane]
 
-// accumulators [W][65], one spare cell per lane (terms that are not the lane's), tiles
-inline size_t argmax_bwd_a_bytes(int Wa) { return sizeof(float) * ((size_t)Wa * kAS + 256 + 2 * kAT * kAC); }
+// accumulators [W][64], one spare cell per lane (terms that are not the lane's), tiles
+__host__ __device__ inline int argmax_acc_floats(int W) { return kAT * W + 256; }
+inline size_t argmax_bwd_a_bytes(int Wa) { return sizeof(float) * ((size_t)argmax_acc_floats(Wa) + 2 * kAT * kAC); }
 inline size_t argmax_bwd_b_bytes(int Wb) {
-  return sizeof(float) * ((size_t)Wb * kAS + 256 + 2 * (kAT + kAJ - 1) * kAC);
+  return sizeof(float) * ((size_t)argmax_acc_floats(Wb) + 2 * (kAT + kAJ - 1) * kAC);
+}
+
+// The sums leave as rows, 32 cells of the band at a time: [k][lane] -> `tile` as [row][33]
+// (a wave moving one k for 64 rows meets 64 banks on both sides) -> memory in runs along the
+// band.  tile: kAT * kAC floats (the g tile, no longer needed).
+__device__ __forceinline__ void argmax_write_out(const float* __restrict__ acc, float* __restrict__ tile, int W,
+                                                 elem_t* __restrict__ out, int rows, int tid) {
+  const int lane = tid & 63, wave = tid >> 6;
+  for (int kc = 0; kc < W; kc += kAJ) {
+    __syncthreads();  // the sums are complete / the previous chunk has left the tile
+#pragma unroll
+    for (int q = 0; q < kAJ / 4; ++q) {
+      const int kk = wave + 4 * q;
+      if (kc + kk < W) tile[lane * kAC + kk] = acc[(kc + kk) * kAS + lane];
+    }
+    __syncthreads();
+    for (int e = tid; e < kAT * kAJ; e += 256) {
+      const int r = e >> 5, c = e & 31;
+      if (r < rows && kc + c < W) out[(long)r * W + kc + c] = to_elem<elem_t>(tile[r * kAC + c]);
+    }
+  }
 }
 
 // Tile of ROWS x 32 cells of g and idx: load() starts the global reads (masked
@@ -76,15 +101,15 @@ __global__ __launch_bounds__(256) void k_band_argmax_bwd_a(const BandArgs p, int
   extern __shared__ __attribute__((aligned(16))) float smem[];
   const int n = p.n, Wa = p.Wa, Wo = p.Wo;
   float* acc = smem;                                      // [Wa][65] + 256 spare cells
-  float* gt = acc + Wa * kAS + 256;                       // [64][33]
+  float* gt = acc + argmax_acc_floats(Wa);                // [64][33]
   int* it = reinterpret_cast<int*>(gt + kAT * kAC);       // [64][33]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int batch = blockIdx.x / strips, i0 = (blockIdx.x - batch * strips) * kAT;
   const long bn = (long)batch * n;
   const elem_t* gb = p.g + bn * Wo;
   const int32_t* ib = p.idx + bn * Wo;
-  for (int e = tid; e < Wa * kAS + 256; e += 256) acc[e] = 0.f;
-  const int spare = Wa * kAS + tid;
+  for (int e = tid; e < argmax_acc_floats(Wa); e += 256) acc[e] = 0.f;
+  const int spare = argmax_acc_floats(Wa) - 256 + tid;
   ArgTile<kAT> tile;
   tile.load(gb, ib, i0, 0, n, Wo, p.r_lu, true, false, tid);
   for (int jc = 0; jc < Wo; jc += kAJ) {
@@ -105,13 +130,7 @@ __global__ __launch_bounds__(256) void k_band_argmax_bwd_a(const BandArgs p, int
       add4_ordered(acc, sl, tv);
     }
   }
-  __syncthreads();
-  elem_t* out = p.o0 + (bn + i0) * Wa;
-  const int rows = min(kAT, n - i0);
-  for (int e = tid; e < rows * Wa; e += 256) {
-    const int r = e / Wa, k = e - r * Wa;
-    out[e] = to_elem<elem_t>(acc[k * kAS + r]);
-  }
+  argmax_write_out(acc, gt, Wa, p.o0 + (bn + i0) * Wa, min(kAT, n - i0), tid);
 }
 
 __global__ __launch_bounds__(256) void k_band_argmax_bwd_b(const BandArgs p, int strips) {
@@ -119,15 +138,15 @@ __global__ __launch_bounds__(256) void k_band_argmax_bwd_b(const BandArgs p, int
   constexpr int kRows = kAT + kAJ - 1;  // 95 rows of g / idx feed 64 rows of b per tile
   const int n = p.n, Wb = p.Wb, Wo = p.Wo;
   float* acc = smem;                                      // [Wb][65] + 256 spare cells
-  float* gt = acc + Wb * kAS + 256;                       // [95][33]
+  float* gt = acc + argmax_acc_floats(Wb);                // [95][33]
   int* it = reinterpret_cast<int*>(gt + kRows * kAC);     // [95][33]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int batch = blockIdx.x / strips, o0 = (blockIdx.x - batch * strips) * kAT;
   const long bn = (long)batch * n;
   const elem_t* gb = p.g + bn * Wo;
   const int32_t* ib = p.idx + bn * Wo;
-  for (int e = tid; e < Wb * kAS + 256; e += 256) acc[e] = 0.f;
-  const int spare = Wb * kAS + tid;
+  for (int e = tid; e < argmax_acc_floats(Wb); e += 256) acc[e] = 0.f;
+  const int spare = argmax_acc_floats(Wb) - 256 + tid;
   // i = o + r_lu - j ascends as j descends: last tile first, columns right to left;
   // tile row 0 holds g row o0 + r_lu - jc - 31
   const int jlast = ((Wo - 1) / kAJ) * kAJ;
@@ -157,13 +176,7 @@ __global__ __launch_bounds__(256) void k_band_argmax_bwd_b(const BandArgs p, int
       }
     }
   }
-  __syncthreads();
-  elem_t* out = p.o1 + (bn + o0) * Wb;
-  const int rows = min(kAT, n - o0);
-  for (int e = tid; e < rows * Wb; e += 256) {
-    const int r = e / Wb, k = e - r * Wb;
-    out[e] = to_elem<elem_t>(acc[k * kAS + r]);
-  }
+  argmax_write_out(acc, gt, Wb, p.o1 + (bn + o0) * Wb, min(kAT, n - o0), tid);
 }
 
 }  // namespace GENBMM_NS
