@@ -123,7 +123,17 @@ def dense_log2(lib, dev, B, M, K, N, reps):
     s, p = _lib.stream_of(a), _lib.ptr
     _lib.check(lib.genbmm_logbmm_fwd(p(a), p(b), p(out), p(stats), B, M, K, N, s), "fwd")
 
-    def bb():
+    ws = torch.empty(lib.genbmm_logbmm_bwdbwd_ws_size(B, M, K, N), device=dev)
+
+    def bb():  # factored, on the matrix cores
+        _lib.check(lib.genbmm_logbmm_bwdbwd_ws(p(a), p(b), p(out), p(g), p(ua), p(ub), p(ga), p(gb), p(gg), p(ws),
+                                               B, M, K, N, s), "bwdbwd_ws")
+
+    def bb_ua():  # the reference's case: the cotangent of grad_a only
+        _lib.check(lib.genbmm_logbmm_bwdbwd_ws(p(a), p(b), p(out), p(g), p(ua), p(None), p(ga), p(gb), p(gg), p(ws),
+                                               B, M, K, N, s), "bwdbwd_ws")
+
+    def bb_exact():  # three vector-ALU passes, one exponential per term in each
         _lib.check(lib.genbmm_logbmm_bwdbwd(p(a), p(b), p(out), p(g), p(ua), p(ub), p(ga), p(gb), p(gg), B, M, K, N, s),
                    "bwdbwd")
 
@@ -131,7 +141,8 @@ def dense_log2(lib, dev, B, M, K, N, reps):
     bmkn = float(B) * M * K * N
     # three passes over (m, k, n), a weight and a multiply-add or two each: counted as 6 per term
     report("logbmm double backward (%d,%d,%d,%d)" % (B, M, K, N), ms, 6 * bmkn,
-           4.0 * B * (3 * M * K + 3 * K * N + 4 * M * N))
+           4.0 * B * (3 * M * K + 3 * K * N + 4 * M * N),
+           {"ms_u_a_only": round(timed(bb_ua, reps), 4), "ms_exact_passes": round(timed(bb_exact, max(reps // 4, 2)), 4)})
 
 
 def dense_max(lib, dev, B, M, K, N, reps, prod):

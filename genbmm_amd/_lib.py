@@ -35,6 +35,7 @@ SIGNATURES = {
     "genbmm_logbmm_fwd_path": [_c_float_p] * 4 + [_i, _i, _i, _i, _i, _vp],  # ..., B, M, K, N, path, stream
     "genbmm_logbmm_bwd_path": [_c_float_p] * 7 + [_i, _i, _i, _i, _i, _vp],
     "genbmm_logbmm_bwdbwd": [_c_float_p] * 9 + _DENSE_DIMS,
+    "genbmm_logbmm_bwdbwd_ws": [_c_float_p] * 10 + _DENSE_DIMS,
     "genbmm_maxbmm_fwd": [_c_float_p] * 3 + [_c_int_p] + _DENSE_DIMS,
     "genbmm_prodmaxbmm_fwd": [_c_float_p] * 3 + [_c_int_p, _c_float_p] + _DENSE_DIMS,
     "genbmm_samplebmm_fwd": [_c_float_p] * 3 + [_c_int_p, _c_float_p, _u64, _u64] + _DENSE_DIMS,
@@ -67,7 +68,7 @@ SIGNATURES = {
 # arguments, the caller's tensors in that type, every workspace still float32.
 HALF_VARIANTS = ("genbmm_logbmm_fwd", "genbmm_logbmm_bwd", "genbmm_logbmm_fwd_path", "genbmm_logbmm_bwd_path",
                  "genbmm_maxbmm_fwd", "genbmm_prodmaxbmm_fwd", "genbmm_samplebmm_fwd", "genbmm_argmax_bwd",
-                 "genbmm_prodmax_bwd", "genbmm_banded_fwd", "genbmm_banded_sample_fwd", "genbmm_banded_bwd",
+                 "genbmm_prodmax_bwd", "genbmm_logbmm_bwdbwd_ws", "genbmm_banded_fwd", "genbmm_banded_sample_fwd", "genbmm_banded_bwd",
                  "genbmm_banded_bwd_scratch")
 for _name in HALF_VARIANTS:
     for _suffix in ("_f16", "_bf16"):
@@ -77,6 +78,7 @@ for _suffix in ("_f16", "_bf16"):  # one more buffer than the float function: t_
 HALF_SUFFIX = {torch.float16: "_f16", torch.bfloat16: "_bf16"}
 STRING_FUNCS = {"genbmm_version": [], "genbmm_error_string": [_i]}
 SIZE_FUNCS = {"genbmm_logbmm_stats_size": [_i, _i, _i, _i],
+              "genbmm_logbmm_bwdbwd_ws_size": [_i, _i, _i, _i],
               "genbmm_samplebmm_stats_size": [_i, _i, _i, _i],
               "genbmm_logbmm_static_limit": [],
               "genbmm_banded_workspace_size": [_i, _i, _i, _i, _i, _i],

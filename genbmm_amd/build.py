@@ -17,11 +17,11 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIBNAME = "libgenbmm_gfx950.so"
-SOURCES = ["logbmm.hip", "dense_fwd.hip", "dense_bwd.hip", "banded.hip", "band_struct.hip", "f64.hip"]
+SOURCES = ["logbmm.hip", "logbmm_bb.hip", "dense_fwd.hip", "dense_bwd.hip", "banded.hip", "band_struct.hip", "f64.hip"]
 # Sources that are compiled once per element type of the caller's tensors: float (entry points
 # genbmm_*), IEEE binary16 (genbmm_*_f16) and bfloat16 (genbmm_*_bf16); see csrc/common.h.
 _ELEMENTS = (("", 0), ("_f16", 1), ("_bf16", 2))
-PER_ELEMENT = {"logbmm.hip": _ELEMENTS, "dense_fwd.hip": _ELEMENTS, "dense_bwd.hip": _ELEMENTS,
+PER_ELEMENT = {"logbmm.hip": _ELEMENTS, "logbmm_bb.hip": _ELEMENTS, "dense_fwd.hip": _ELEMENTS, "dense_bwd.hip": _ELEMENTS,
                "banded.hip": _ELEMENTS}
 
 # -packed-fp32-ops is switched OFF: v_pk_{add,mul,fma}_f32 are not used by any

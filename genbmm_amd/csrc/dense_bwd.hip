@@ -1,132 +1,8 @@
-// Dense semiring batched matmul, backward and second-order kernels (gfx950).
+// Dense semiring batched matmul: the arg-max backward kernels (gfx950).
 #include "common.h"
 
 namespace GENBMM_NS {
 namespace {
-
-#if GENBMM_ELEM == 0  // second order: float tensors only (grad_g is re-read as an operand)
-// ===================================================== logbmm second order
-//
-// With p = exp(a+b-out), w = u_a[m,k] + u_b[k,n]  (a missing u counts as 0):
-//   t[m,n]      = sum_k p*w                        (gradient w.r.t. g)
-//   grad_a[m,k] = sum_n g[m,n]*p*(w - t[m,n])
-//   grad_b[k,n] = sum_m g[m,n]*p*(w - t[m,n])
-// With u_b = 0 these are the reference's three quartic kernels
-// (matmul_cuda_kernel.cu:220-331: inner = sum_k2 (delta*s - s*s2)*u[k2]
-// = s*(u[k] - t)), computed in O(M*K*N).  One lane per output element for t and grad_b.
-struct BB {
-  const float* a; const float* b; const float* out; const float* g;
-  const float* ua; const float* ub;
-  float* ga; float* gb; float* gg;
-  int M, K, N;
-};
-
-__global__ __launch_bounds__(256) void k_log_bwdbwd_t(const BB p, long total) {
-  const long e = (long)xcd_renumber(blockIdx.x, gridDim.x) * 256 + threadIdx.x;  // an item's workgroups on one XCD
-  if (e >= total) return;
-  const int n = (int)(e % p.N);
-  const long bm = e / p.N;  // batch*M + m
-  const long batch = bm / p.M;
-  const float* arow = p.a + bm * p.K;
-  const float* uarow = p.ua ? p.ua + bm * p.K : nullptr;
-  const float* bcol = p.b + batch * p.K * p.N + n;
-  const float* ubcol = p.ub ? p.ub + batch * p.K * p.N + n : nullptr;
-  const float o = p.out[e];
-  float t = 0.f;
-  for (int k = 0; k < p.K; ++k) {
-    const float pr = fast_exp(arow[k] + bcol[(long)k * p.N] - o);
-    const float w = (uarow ? uarow[k] : 0.f) + (ubcol ? ubcol[(long)k * p.N] : 0.f);
-    t = __builtin_fmaf(pr, w, t);
-  }
-  p.gg[e] = t;
-}
-
-// grad_a: a wave per row (batch, m), its lanes along n - the one axis on which b, u_b, out, g and
-// t are all contiguous (with a lane per cell (m, k) the reads of b run down a column, one cache
-// line per lane).  The row's out, g and t stay in registers for N <= 256; per k the lanes'
-// partial sums are added across the wave and 64 finished cells are written at once.
-constexpr int kBBChunks = 4;  // n chunks of 64 a lane keeps in registers
-__global__ __launch_bounds__(256) void k_log_bwdbwd_a(const BB p, long rows) {
-  const int lane = threadIdx.x & 63;
-  const long bm = (long)xcd_renumber(blockIdx.x, gridDim.x) * 4 + (threadIdx.x >> 6);
-  if (bm >= rows) return;
-  const long batch = bm / p.M;
-  const int K = p.K, N = p.N;
-  const float* arow = p.a + bm * K;
-  const float* uarow = p.ua ? p.ua + bm * K : nullptr;
-  const float* bmat = p.b + batch * K * N;
-  const float* ubmat = p.ub ? p.ub + batch * K * N : nullptr;
-  const float* orow = p.out + bm * N;
-  const float* grow = p.g + bm * N;
-  const float* trow = p.gg + bm * N;
-  const bool cached = N <= 64 * kBBChunks;
-  float oc[kBBChunks], gc[kBBChunks], tc[kBBChunks];
-#pragma unroll
-  for (int j = 0; j < kBBChunks; ++j) {
-    const int n = lane + 64 * j;
-    const bool in = cached && n < N;
-    oc[j] = in ? orow[n] : 0.f;
-    gc[j] = in ? grow[n] : 0.f;
-    tc[j] = in ? trow[n] : 0.f;
-  }
-  float mine = 0.f;  // the finished cell k with k % 64 == lane
-  for (int k = 0; k < K; ++k) {
-    const float av = arow[k], uav = uarow ? uarow[k] : 0.f;
-    const float* brow = bmat + (long)k * N;
-    const float* ubrow = ubmat ? ubmat + (long)k * N : nullptr;
-    float acc = 0.f;
-    if (cached) {
-#pragma unroll
-      for (int j = 0; j < kBBChunks; ++j) {
-        const int n = lane + 64 * j;
-        if (n < N) {
-          const float pr = fast_exp(av + brow[n] - oc[j]);
-          const float w = uav + (ubrow ? ubrow[n] : 0.f) - tc[j];
-          acc = __builtin_fmaf(gc[j] * pr, w, acc);
-        }
-      }
-    } else {
-      for (int n = lane; n < N; n += 64) {
-        const float pr = fast_exp(av + brow[n] - orow[n]);
-        const float w = uav + (ubrow ? ubrow[n] : 0.f) - trow[n];
-        acc = __builtin_fmaf(grow[n] * pr, w, acc);
-      }
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-    if ((k & 63) == lane) mine = acc;
-    if ((k & 63) == 63 || k == K - 1) {
-      const int k0 = k & ~63;
-      if (k0 + lane <= k) p.ga[bm * K + k0 + lane] = mine;
-    }
-  }
-}
-
-__global__ __launch_bounds__(256) void k_log_bwdbwd_b(const BB p, long total) {
-  const long e = (long)xcd_renumber(blockIdx.x, gridDim.x) * 256 + threadIdx.x;  // an item's workgroups on one XCD
-  if (e >= total) return;
-  const int n = (int)(e % p.N);
-  const long bk = e / p.N;  // batch*K + k
-  const long batch = bk / p.K;
-  const int k = (int)(bk - batch * p.K);
-  const float bv = p.b[e];
-  const float ubv = p.ub ? p.ub[e] : 0.f;
-  const float* acol = p.a + batch * p.M * p.K + k;
-  const float* uacol = p.ua ? p.ua + batch * p.M * p.K + k : nullptr;
-  const float* ocol = p.out + batch * p.M * p.N + n;
-  const float* gcol = p.g + batch * p.M * p.N + n;
-  const float* tcol = p.gg + batch * p.M * p.N + n;
-  float acc = 0.f;
-  for (int m = 0; m < p.M; ++m) {
-    const long mn = (long)m * p.N;
-    const float pr = fast_exp(acol[(long)m * p.K] + bv - ocol[mn]);
-    const float w = (uacol ? uacol[(long)m * p.K] : 0.f) + ubv - tcol[mn];
-    acc = __builtin_fmaf(gcol[mn] * pr, w, acc);
-  }
-  p.gb[e] = acc;
-}
-
-#endif
 
 // ===================================================== argmax backward
 //
@@ -389,41 +265,6 @@ int run_argmax_bwd(const elem_t* a, const elem_t* b, const int32_t* idx, const f
 }  // namespace GENBMM_NS
 
 extern "C" {
-
-#if GENBMM_ELEM == 0
-int genbmm_logbmm_bwdbwd(const float* a, const float* b, const float* out, const float* g,
-                         const float* u_a, const float* u_b, float* grad_a, float* grad_b,
-                         float* grad_g, int B, int M, int K, int N, void* stream) {
-  using namespace GENBMM_NS;
-  if (int e = check_dense_dims(B, M, K, N)) return e;
-  {
-    const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
-    if (missing(a, mk) || missing(b, kn) || missing(out, mn) || missing(g, mn) ||
-        missing(grad_a, mk) || missing(grad_b, kn) || missing(grad_g, mn) ||
-        (missing(u_a, mk) && missing(u_b, kn)))
-      return GENBMM_E_NULLPTR;
-  }
-  BB p{a, b, out, g, u_a, u_b, grad_a, grad_b, grad_g, M, K, N};
-  hipStream_t s = (hipStream_t)stream;
-  auto blocks = [](long total) { return dim3((unsigned)((total + 255) / 256)); };
-  const long tmn = (long)B * M * N, tmk = (long)B * M * K, tkn = (long)B * K * N;
-  if (tmn > 0) {
-    hipLaunchKernelGGL(k_log_bwdbwd_t, blocks(tmn), dim3(256), 0, s, p, tmn);
-    if (int e = launch_status()) return e;
-  }
-  if (tmk > 0) {
-    const long rows = (long)B * M;  // four rows per workgroup
-    hipLaunchKernelGGL(k_log_bwdbwd_a, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, p, rows);
-    if (int e = launch_status()) return e;
-  }
-  if (tkn > 0) {
-    hipLaunchKernelGGL(k_log_bwdbwd_b, blocks(tkn), dim3(256), 0, s, p, tkn);
-    if (int e = launch_status()) return e;
-  }
-  return GENBMM_OK;
-}
-
-#endif
 
 // One set per element type: genbmm_argmax_bwd, genbmm_argmax_bwd_f16, ..._bf16, ...
 int GENBMM_API(argmax_bwd)(const int32_t* idx, const GENBMM_NS::abi_t* g, GENBMM_NS::abi_t* grad_a,

@@ -141,18 +141,21 @@ class _LogBmmGrad(torch.autograd.Function):
             return None, None, None, None, None, None
         a, b, g, out = ctx.saved_tensors
         B, M, K, N = _lib.dense_dims(a, b)
-        dtype = a.dtype
-        if _sfx(a):  # the second-order kernels re-read their own grad_g: float32 tensors only
-            a, b, g, out = a.float(), b.float(), g.float(), out.float()
         u_a = None if u_a is None else u_a.to(a.dtype).contiguous()
         u_b = None if u_b is None else u_b.to(a.dtype).contiguous()
         ga = torch.empty_like(a)
         gb = torch.empty_like(b)
         gg = torch.empty_like(g)
-        _call("genbmm_logbmm_bwdbwd_f64" if _f64(a) else "genbmm_logbmm_bwdbwd", a, _lib.ptr(a),
-              _lib.ptr(b), _lib.ptr(out), _lib.ptr(g), _lib.ptr(u_a), _lib.ptr(u_b), _lib.ptr(ga),
-              _lib.ptr(gb), _lib.ptr(gg), B, M, K, N)
-        return ga.to(dtype), gb.to(dtype), gg.to(dtype), None, None, None
+        if _f64(a):
+            _call("genbmm_logbmm_bwdbwd_f64", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g),
+                  _lib.ptr(u_a), _lib.ptr(u_b), _lib.ptr(ga), _lib.ptr(gb), _lib.ptr(gg), B, M, K, N)
+        else:
+            # scratch for the factored form on the matrix cores (and, for float16 / bfloat16 tensors, where
+            # the gradient with respect to g stays unrounded for the other two gradients)
+            ws = torch.empty(_lib.load().genbmm_logbmm_bwdbwd_ws_size(B, M, K, N), dtype=_COMPUTE, device=a.device)
+            _call("genbmm_logbmm_bwdbwd_ws" + _sfx(a), a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g),
+                  _lib.ptr(u_a), _lib.ptr(u_b), _lib.ptr(ga), _lib.ptr(gb), _lib.ptr(gg), _lib.ptr(ws), B, M, K, N)
+        return ga, gb, gg, None, None, None
 
 
 class LogMatMul(torch.autograd.Function):

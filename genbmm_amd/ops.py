@@ -90,14 +90,12 @@ def logbmm_bwdbwd(a: Tensor, b: Tensor, out: Tensor, g: Tensor, u_a: Tensor,
                   u_b: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
     """Gradients of <u_a, grad_a> + <u_b, grad_b> with respect to (a, b, g)."""
     B, M, K, N = _check(a, b)
-    dtype = a.dtype
-    if _sfx(a):  # the second-order kernels take float tensors: half ones are widened here
-        a, b, out = a.float(), b.float(), out.float()
     g, u_a, u_b = g.to(a.dtype).contiguous(), u_a.to(a.dtype).contiguous(), u_b.to(a.dtype).contiguous()
     ga, gb, gg = torch.empty_like(a), torch.empty_like(b), torch.empty_like(g)
-    _call("genbmm_logbmm_bwdbwd", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g), _lib.ptr(u_a),
-          _lib.ptr(u_b), _lib.ptr(ga), _lib.ptr(gb), _lib.ptr(gg), B, M, K, N)
-    return ga.to(dtype), gb.to(dtype), gg.to(dtype)
+    ws = torch.empty(_lib.load().genbmm_logbmm_bwdbwd_ws_size(B, M, K, N), dtype=torch.float32, device=a.device)
+    _call("genbmm_logbmm_bwdbwd_ws" + _sfx(a), a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(g), _lib.ptr(u_a),
+          _lib.ptr(u_b), _lib.ptr(ga), _lib.ptr(gb), _lib.ptr(gg), _lib.ptr(ws), B, M, K, N)
+    return ga, gb, gg
 
 
 @logbmm_bwdbwd.register_fake

@@ -176,6 +176,28 @@ int genbmm_logbmm_bwdbwd(const float* a, const float* b, const float* out,
                          int B, int M, int K, int N, void* stream);
 
 /*
+ * The same function on a caller-allocated workspace of
+ * genbmm_logbmm_bwdbwd_ws_size(B, M, K, N) floats (NULL: as the function above).
+ * With it, problems whose extents are all at least 64 take the factored form on
+ * the matrix cores: with EA = exp(a - rowmax), EB = exp(b - colmax),
+ * R = exp(rowmax + colmax - out), H = g R, X = EA u_a, Y = EB u_b:
+ *   grad_g = t = R (X EB + EA Y),
+ *   grad_a = X (H EB^T) + EA (H Y^T - (H t) EB^T),
+ *   grad_b = Y (EA^T H) + EB (X^T H - EA^T (H t))
+ * - eight batched matrix products (five without u_b) instead of one
+ * exponential per (m, k, n) in each of three passes.  Batch items with a cell
+ * whose rowmax + colmax - out exceeds 40 ln 2 or is not finite are redone by
+ * the exact passes.  Same reference counterpart as genbmm_logbmm_bwdbwd; the
+ * workspace is scratch (nothing in it outlives the call).
+ */
+size_t genbmm_logbmm_bwdbwd_ws_size(int B, int M, int K, int N);
+int genbmm_logbmm_bwdbwd_ws(const float* a, const float* b, const float* out,
+                            const float* g, const float* u_a, const float* u_b,
+                            float* grad_a, float* grad_b, float* grad_g,
+                            float* workspace, int B, int M, int K, int N,
+                            void* stream);
+
+/*
  * out[b,m,n] = max_k (a[m,k] + b[k,n]); idx = the k attaining it.
  * Ascending k, strict '>' against a running maximum that starts at -1e9
  * with index -1: ties resolve to the lowest k.
@@ -499,6 +521,9 @@ int genbmm_banded_bwdbwd_f64(const double* a, int a_lu, int a_ld,
  * otherwise (`out` rounded to 11 or 8 bits does not give S well enough for the
  * other sweeps): its index is the float function's on those shapes and the
  * index of the float function called with stats = NULL on all others.
+ * The second-order function exists in its workspace form only
+ * (genbmm_logbmm_bwdbwd_ws_f16 / _bf16; the workspace is required: the gradient
+ * with respect to g is read back by the other two and stays unrounded there).
  * The banded functions likewise (the reference instantiates every banded kernel
  * for Half too, banded_cuda_kernel.cu:389, :435, :484, :508, :530): band data,
  * results, g and gradients in the 16-bit type, `workspace` and `scratch` float
@@ -564,6 +589,16 @@ int genbmm_prodmax_bwd_bf16(const uint16_t* a, const uint16_t* b, const int32_t*
                             uint16_t* grad_a, uint16_t* grad_b,
                             int B, int M, int K, int N, void* stream);
 
+int genbmm_logbmm_bwdbwd_ws_f16(const uint16_t* a, const uint16_t* b, const uint16_t* out,
+                                const uint16_t* g, const uint16_t* u_a, const uint16_t* u_b,
+                                uint16_t* grad_a, uint16_t* grad_b, uint16_t* grad_g,
+                                float* workspace, int B, int M, int K, int N,
+                                void* stream);
+int genbmm_logbmm_bwdbwd_ws_bf16(const uint16_t* a, const uint16_t* b, const uint16_t* out,
+                                 const uint16_t* g, const uint16_t* u_a, const uint16_t* u_b,
+                                 uint16_t* grad_a, uint16_t* grad_b, uint16_t* grad_g,
+                                 float* workspace, int B, int M, int K, int N,
+                                 void* stream);
 int genbmm_banded_fwd_f16(const uint16_t* a, int a_lu, int a_ld,
                           const uint16_t* b, int b_lu, int b_ld,
                           uint16_t* out, int32_t* idx, float* workspace,

@@ -370,6 +370,100 @@ def test_logbmm_double_backward_at_a_matrix_core_shape(gpu):
         close(x[pick], y, rtol=1e-4, atol=1e-4)
 
 
+def _bwdbwd_abi(gpu, a, b, out, g, u_a, u_b, use_ws):
+    lib = _lib.load()
+    B, M, K = a.shape
+    N = b.shape[2]
+    ga, gb, gg = torch.empty_like(a), torch.empty_like(b), torch.empty_like(g)
+    p, s = _lib.ptr, _lib.stream_of(a)
+    if use_ws:
+        ws = torch.empty(lib.genbmm_logbmm_bwdbwd_ws_size(B, M, K, N), device=gpu)
+        rc = lib.genbmm_logbmm_bwdbwd_ws(p(a), p(b), p(out), p(g), p(u_a), p(u_b), p(ga), p(gb), p(gg), p(ws), B, M, K, N, s)
+    else:
+        rc = lib.genbmm_logbmm_bwdbwd(p(a), p(b), p(out), p(g), p(u_a), p(u_b), p(ga), p(gb), p(gg), B, M, K, N, s)
+    assert rc == 0
+    return ga, gb, gg
+
+
+@pytest.mark.parametrize("B,M,K,N", [(16, 128, 128, 128), (9, 100, 70, 130), (3, 200, 96, 260), (5, 64, 300, 65),
+                                     (2, 512, 128, 384), (40, 64, 64, 64)])
+def test_logbmm_double_backward_factored_on_the_matrix_cores(gpu, B, M, K, N):
+    """genbmm_logbmm_bwdbwd_ws (eight matrix products on exp(a - max), exp(b - max), exp(max - out))
+    against float64 second-order autograd, and against the exact vector-ALU passes of
+    genbmm_logbmm_bwdbwd; full tiles, ragged extents in every position, each cotangent alone.
+    Sums of up to 300 terms of magnitude |g u| <= ~20: absolute fp32 error well under 1e-4."""
+    lib = _lib.load()
+    assert lib.genbmm_logbmm_bwdbwd_ws_size(B, M, K, N) > B * M * N      # the factored form applies
+    torch.manual_seed(M + N)
+    a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
+    ua, ub = torch.randn(B, M, K), torch.randn(B, K, N)
+    ad, bd, gd, uad, ubd = (t.to(gpu) for t in (a, b, g, ua, ub))
+    out = genbmm.logbmm(ad, bd)
+    pick = sorted({0, B // 2, B - 1})
+    for u_a, u_b, ha, hb in ((uad, ubd, ua, ub), (uad, None, ua, None), (None, ubd, None, ub)):
+        got = _bwdbwd_abi(gpu, ad, bd, out, gd, u_a, u_b, True)
+        exact = _bwdbwd_abi(gpu, ad, bd, out, gd, u_a, u_b, False)
+        for x, y in zip(got, exact):
+            close(x, y, rtol=1e-4, atol=1e-4)
+        want = oracle.logbmm_second_order64(a[pick], b[pick], g[pick], None if ha is None else ha[pick],
+                                            None if hb is None else hb[pick])
+        for x, y in zip(got, want):
+            close(x[pick], y, rtol=1e-4, atol=1e-4)
+
+
+def test_logbmm_double_backward_factored_guard(gpu):
+    """Batch items with rows whose maxima sit on terms that never meet (the factors underflow
+    against terms that matter), a -inf mask and a row at the floor: those items are redone by
+    the exact passes, the others stay on the matrix cores; all agree with the exact passes."""
+    torch.manual_seed(23)
+    B, M, K, N = 6, 128, 96, 160
+    a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
+    a[1, ::2, 0] += 200.0          # item 1: exp(a - rowmax) underflows for every k > 0 of those rows ...
+    b[1, 0, :] -= 200.0            # ... while the true terms do not
+    b[3, 5, :] = -float("inf")     # item 3: a masked k (stays factorable: exp -> 0)
+    a[4, 7, :] = -1e9              # item 4: a row at the floor
+    ua, ub = torch.randn(B, M, K), torch.randn(B, K, N)
+    ad, bd, gd, uad, ubd = (t.to(gpu) for t in (a, b, g, ua, ub))
+    gd[4, 7, :] = 0                # no gradient flows into the padding row
+    out = genbmm.logbmm(ad, bd)
+    got = _bwdbwd_abi(gpu, ad, bd, out, gd, uad, ubd, True)
+    exact = _bwdbwd_abi(gpu, ad, bd, out, gd, uad, ubd, False)
+    # (the weights of the row at the floor are a matter of rounding - a + b = out = -1e9 in float,
+    # every weight 1, in the exact passes; the softmax of b's column in exact arithmetic and in the
+    # factored form - so its own cells of grad_a and grad_g are left out; nothing flows out of it)
+    for x, y, rowwise in zip(got, exact, (True, False, True)):
+        x, y = x.clone(), y.clone()
+        if rowwise:
+            assert bool(torch.isfinite(x[4, 7]).all())
+            x[4, 7], y[4, 7] = 0, 0
+        fin = torch.isfinite(y)
+        assert torch.equal(torch.isfinite(x), fin)
+        close(x[fin], y[fin], rtol=1e-4, atol=1e-4)
+    keep = [0, 1, 2, 3, 5]
+    want = oracle.logbmm_second_order64(a[keep], b[keep], g[keep], ua[keep], ub[keep])
+    for x, y in zip(got, want):
+        close(x[keep], y, rtol=1e-4, atol=2e-4)
+
+
+def test_logbmm_double_backward_at_the_headline_shape(gpu):
+    """(64, 512, 512, 512) through autograd with create_graph; three batch items against float64
+    second-order autograd evaluated on the device."""
+    torch.manual_seed(29)
+    B, M, K, N = 64, 512, 512, 512
+    ad, bd, gd = (torch.randn(B, M, K, device=gpu).requires_grad_(True), torch.randn(B, K, N, device=gpu).requires_grad_(True),
+                  torch.randn(B, M, N, device=gpu).requires_grad_(True))
+    ua = torch.randn(B, M, K, device=gpu)
+    out = genbmm.logbmm(ad, bd)
+    ga, gb = torch.autograd.grad(out, (ad, bd), gd, create_graph=True)
+    got = torch.autograd.grad(ga, (ad, bd, gd), ua)                   # the reference's case: u_b absent
+    for item in (0, 31, 63):
+        sl = slice(item, item + 1)
+        want = oracle.logbmm_second_order64(ad[sl], bd[sl], gd[sl], ua[sl], None)
+        for x, y, what in zip(got, want, ("grad_a", "grad_b", "grad_g")):
+            close_on_device(x[sl], y, "%s item %d" % (what, item), rtol=1e-4, atol=2e-4)
+        del want
+
+
 # ------------------------------------------------------------ max / prod-max
 def grid(*shape):
     return torch.round(torch.randn(*shape) * 8) / 8

@@ -285,3 +285,33 @@ def test_banded_products_on_half_bands(gpu, dt):
         assert torch.equal(got.data, want.data.to(dt)), name
         ga, gb = torch.autograd.grad(got.data.float().sum(), (xh, yh))
         assert ga.dtype == dt and gb.dtype == dt and float(ga.float().abs().sum()) > 0
+
+
+@pytest.mark.parametrize("dt,suffix,eps", TYPES)
+@pytest.mark.parametrize("B,M,K,N", [(3, 20, 33, 50), (6, 128, 128, 128), (4, 100, 70, 130)])
+def test_logbmm_second_order_half_equals_float_kernels_rounded(gpu, dt, suffix, eps, B, M, K, N):
+    """genbmm_logbmm_bwdbwd_ws_f16 / _bf16 (exact passes for the small shape, matrix cores for the
+    others): the float function on the widened tensors, rounded once - the gradient with respect
+    to g stays unrounded in the workspace for the other two gradients."""
+    lib = _lib.load()
+    torch.manual_seed(B + M)
+    a, b, g = _operands(gpu, dt, B, M, K, N, scale=1.0)
+    ua, ub = torch.randn(B, M, K, device=gpu).to(dt), torch.randn(B, K, N, device=gpu).to(dt)
+    s = _lib.stream_of(a)
+    out = torch.empty(B, M, N, device=gpu, dtype=dt)
+    st = torch.empty(lib.genbmm_logbmm_stats_size(B, M, K, N), device=gpu)
+    assert getattr(lib, "genbmm_logbmm_fwd" + suffix)(P(a), P(b), P(out), P(st), B, M, K, N, s) == 0
+    wide = [t.float() for t in (a, b, out, g, ua, ub)]
+    nws = lib.genbmm_logbmm_bwdbwd_ws_size(B, M, K, N)
+    for u_a, u_b, w_a, w_b in ((ua, ub, wide[4], wide[5]), (ua, None, wide[4], None), (None, ub, None, wide[5])):
+        ws, ws32 = torch.empty(nws, device=gpu), torch.empty(nws, device=gpu)
+        ga, gb, gg = torch.empty_like(a), torch.empty_like(b), torch.empty_like(g)
+        ga32, gb32, gg32 = (torch.empty_like(t) for t in (wide[0], wide[1], wide[3]))
+        assert getattr(lib, "genbmm_logbmm_bwdbwd_ws" + suffix)(P(a), P(b), P(out), P(g), P(u_a), P(u_b), P(ga), P(gb),
+                                                               P(gg), P(ws), B, M, K, N, s) == 0
+        assert lib.genbmm_logbmm_bwdbwd_ws(P(wide[0]), P(wide[1]), P(wide[2]), P(wide[3]), P(w_a), P(w_b), P(ga32),
+                                           P(gb32), P(gg32), P(ws32), B, M, K, N, s) == 0
+        assert torch.equal(ga, ga32.to(dt)) and torch.equal(gb, gb32.to(dt)) and torch.equal(gg, gg32.to(dt))
+    # the workspace is required for the half types
+    assert getattr(lib, "genbmm_logbmm_bwdbwd_ws" + suffix)(P(a), P(b), P(out), P(g), P(ua), P(ub), P(ga), P(gb), P(gg),
+                                                           P(None), B, M, K, N, s) == -1
