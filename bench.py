@@ -20,10 +20,11 @@ if ROOT not in sys.path:
 
 B, M, K, N = 64, 512, 512, 512
 FP32_VALU_PEAK_TFLOPS = 157.3  # MI355X FP32 peak (vector with packed FMA = fp32 matrix cores)
-# HBM bytes per launch of the dominant kernel (k_log_bwd_mfma_both): rocprofv3 --pmc
-# FETCH_SIZE 274150 KiB + WRITE_SIZE 131070 KiB per dispatch, scale factor 1.00 against a
-# known-size copy in the same run (profiles/logbmm_headline_B64_512.md).
-DOMINANT_TRAFFIC_BYTES = (243860 + 131070) * 1024
+# HBM bytes per launch of the dominant kernel (k_log_bwd_mfma_both_lean): rocprofv3 --pmc
+# FETCH_SIZE + WRITE_SIZE in KiB per dispatch, scale factor 1.00 against a known-size copy in
+# the same run; the two figures are those of profiles/logbmm_headline_B64_512.md.
+DOMINANT_FETCH_KIB, DOMINANT_WRITE_KIB = 243860, 131070
+DOMINANT_TRAFFIC_BYTES = (DOMINANT_FETCH_KIB + DOMINANT_WRITE_KIB) * 1024
 
 
 def cpu_baseline(torch, sample_batches=64):
@@ -153,7 +154,8 @@ def main():
     achieved = 4.0 * bmkn / (ms_dom * 1e-3) / 1e12
     roofline = {
         "bound": "mfma",
-        "kernel": "k_log_bwd_mfma_both (grad_a and grad_b tiles in one launch)",
+        "kernel": "k_log_bwd_mfma_both_lean (grad_a and grad_b tiles in one launch, operands formed "
+                  "again from a, b, out and the maxima)",
         "achieved": round(achieved, 3),
         "peak": FP32_VALU_PEAK_TFLOPS,
         "unit": "TFLOP/s",

@@ -79,6 +79,7 @@ HALF_SUFFIX = {torch.float16: "_f16", torch.bfloat16: "_bf16"}
 STRING_FUNCS = {"genbmm_version": [], "genbmm_error_string": [_i]}
 SIZE_FUNCS = {"genbmm_logbmm_stats_size": [_i, _i, _i, _i],
               "genbmm_logbmm_bwdbwd_ws_size": [_i, _i, _i, _i],
+              "genbmm_logbmm_stats_size_path": [_i, _i, _i, _i, _i],
               "genbmm_samplebmm_stats_size": [_i, _i, _i, _i],
               "genbmm_logbmm_static_limit": [],
               "genbmm_banded_workspace_size": [_i, _i, _i, _i, _i, _i],

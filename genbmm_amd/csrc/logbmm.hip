@@ -351,7 +351,7 @@ __global__ __launch_bounds__(CX::NT) void k_log_bwd_fixup_both(const LogBwdArgs 
                                                                const LogBwdArgs pb,
                                                                const int* __restrict__ hdr,
                                                                const int* __restrict__ fwd_flags,
-                                                               int tiles_a, int tiles_b) {
+                                                               int tiles_a, int tiles_b, int need_factors) {
   constexpr int kFa = LogBwdLds<CX, true>::FLOATS, kFb = LogBwdLds<CX, false>::FLOATS;
   __shared__ __attribute__((aligned(16))) float smem[kFa > kFb ? kFa : kFb];
   for (int t = blockIdx.x; t < tiles_a + tiles_b; t += gridDim.x) {
@@ -363,7 +363,7 @@ __global__ __launch_bounds__(CX::NT) void k_log_bwd_fixup_both(const LogBwdArgs 
     const int FR = is_a ? AR : BR, FC = is_a ? AC : BC;
     const int R = is_a ? p.M : p.K, Cc = is_a ? p.K : p.N;
     const int r0 = (r / p.tiles_c) * FR, c0 = (r % p.tiles_c) * FC;
-    if (!bwd_tile_flagged(hdr, fwd_flags, true, is_a, is_a ? r0 : c0, is_a ? FR : FC, batch, p.M, p.N,
+    if (!bwd_tile_flagged(hdr, fwd_flags, need_factors, is_a, is_a ? r0 : c0, is_a ? FR : FC, batch, p.M, p.N,
                           threadIdx.x, CX::NT))
       continue;
     for (int h = 0; h < FR / CX::BR; ++h)
@@ -571,12 +571,16 @@ __global__ __launch_bounds__(C::NT, 2) void k_log_bwd_fast(const LogBwdArgs p,
 // kernels for small matrices, the matrix cores where the shape allows, the factored
 // vector-ALU kernels otherwise.  EXACT: the online / exp-per-term kernels only (what a
 // NULL workspace gives).  VALU: the factored kernels on v_fma_f32, never the matrix cores
-// nor the whole-item kernels.
+// nor the whole-item kernels.  FACTORS: as AUTO, but the matrix-core forward leaves EA, EB and 1/S in
+// the workspace and the matrix-core backward reads them instead of forming its operands again from
+// a, b, out and the maxima (what AUTO does: the workspace then holds the maxima and flags only).
 constexpr int kFixupGrid = 1024;
 
 inline bool valid_path(int path) {
-  return path == GENBMM_PATH_AUTO || path == GENBMM_PATH_EXACT || path == GENBMM_PATH_VALU;
+  return path == GENBMM_PATH_AUTO || path == GENBMM_PATH_EXACT || path == GENBMM_PATH_VALU ||
+         path == GENBMM_PATH_FACTORS;
 }
+inline bool auto_path(int path) { return path == GENBMM_PATH_AUTO || path == GENBMM_PATH_FACTORS; }
 
 // Layout of the caller's stats buffer: B*(M+N) shifts; one int flag per 32x32
 // tile of (M,N) (an upper bound on any forward launch's tile count); a header of
@@ -751,7 +755,7 @@ int launch_bwd_fast(LogBwdArgs p, const float* stats, int B, hipStream_t s) {
 }
 
 template <class T, bool GRAD_A>
-int launch_bwd_mfma(LogBwdArgs p, const float* stats, int B, hipStream_t s) {
+int launch_bwd_mfma(LogBwdArgs p, const float* stats, int B, hipStream_t s, bool lean = false) {
   const int R = GRAD_A ? p.M : p.K, Cc = GRAD_A ? p.K : p.N;
   const int Q = GRAD_A ? p.N : p.M;
   p.tiles_r = ceil_div(R, T::TR);
@@ -763,17 +767,27 @@ int launch_bwd_mfma(LogBwdArgs p, const float* stats, int B, hipStream_t s) {
     hipLaunchKernelGGL(kern, dim3(total), dim3(T::NT), 0, s, p.g, ws.ea, ws.eb, ws.r, ws.hdr, ff,
                        p.grad, p.M, p.K, p.N, p.tiles_r, p.tiles_c);
   };
-  if (R % T::TR != 0 || Cc % T::TC != 0 || Q % kMS != 0) go(k_log_bwd_mfma<T, GRAD_A, true>);
-  else go(k_log_bwd_mfma<T, GRAD_A, false>);
+  auto go_lean = [&](auto kern) {
+    hipLaunchKernelGGL(kern, dim3(total), dim3(T::NT), 0, s, p.g, LeanSrc{p.a, p.b, p.out, stats}, ws.hdr, ff, p.grad,
+                       p.M, p.K, p.N, p.tiles_r, p.tiles_c);
+  };
+  const bool ragged = R % T::TR != 0 || Cc % T::TC != 0 || Q % kMS != 0;
+  if (lean) {
+    if (ragged) go_lean(k_log_bwd_mfma_lean<T, GRAD_A, true>);
+    else go_lean(k_log_bwd_mfma_lean<T, GRAD_A, false>);
+  } else {
+    if (ragged) go(k_log_bwd_mfma<T, GRAD_A, true>);
+    else go(k_log_bwd_mfma<T, GRAD_A, false>);
+  }
   if (int e = launch_status()) return e;
   hipLaunchKernelGGL((k_log_bwd_fixup<BCfgWide, T::TR, T::TC, GRAD_A>),
-                     dim3(min(total, kFixupGrid)), dim3(BCfgWide::NT), 0, s, p, ws.hdr, ff, 1, total);
+                     dim3(min(total, kFixupGrid)), dim3(BCfgWide::NT), 0, s, p, ws.hdr, ff, lean ? 0 : 1, total);
   return launch_status();
 }
 
 // grad_a and grad_b of a matrix-core problem in one launch (+ one fix-up launch).
 template <class TA, class TB>
-int launch_bwd_mfma_both(LogBwdArgs pa, LogBwdArgs pb, const float* stats, int B, hipStream_t s) {
+int launch_bwd_mfma_both(LogBwdArgs pa, LogBwdArgs pb, const float* stats, int B, hipStream_t s, bool lean = false) {
   const int M = pa.M, K = pa.K, N = pa.N;
   pa.tiles_r = ceil_div(M, TA::TR); pa.tiles_c = ceil_div(K, TA::TC);
   pb.tiles_r = ceil_div(K, TB::TR); pb.tiles_c = ceil_div(N, TB::TC);
@@ -788,12 +802,22 @@ int launch_bwd_mfma_both(LogBwdArgs pa, LogBwdArgs pb, const float* stats, int B
   };
   const bool ragged = M % TA::TR != 0 || K % TA::TC != 0 || N % kMS != 0 || K % TB::TR != 0 ||
                       N % TB::TC != 0 || M % kMS != 0;
-  if (ragged) go(k_log_bwd_mfma_both<TA, TB, true>);
-  else go(k_log_bwd_mfma_both<TA, TB, false>);
+  auto go_lean = [&](auto kern) {
+    hipLaunchKernelGGL(kern, dim3((unsigned)(ta + tb)), dim3(TA::NT), 0, s, pa.g, LeanSrc{pa.a, pa.b, pa.out, stats},
+                       ws.hdr, ff, pa.grad, pb.grad, M, K, N, (int)ta, pa.tiles_r, pa.tiles_c, pb.tiles_r,
+                       pb.tiles_c);
+  };
+  if (lean) {
+    if (ragged) go_lean(k_log_bwd_mfma_both_lean<TA, TB, true>);
+    else go_lean(k_log_bwd_mfma_both_lean<TA, TB, false>);
+  } else {
+    if (ragged) go(k_log_bwd_mfma_both<TA, TB, true>);
+    else go(k_log_bwd_mfma_both<TA, TB, false>);
+  }
   if (int e = launch_status()) return e;
   hipLaunchKernelGGL((k_log_bwd_fixup_both<BCfgWide, TA::TR, TA::TC, TB::TR, TB::TC>),
                      dim3((unsigned)std::min<int64_t>(ta + tb, kFixupGrid)), dim3(BCfgWide::NT), 0,
-                     s, pa, pb, ws.hdr, ff, (int)ta, (int)tb);
+                     s, pa, pb, ws.hdr, ff, (int)ta, (int)tb, lean ? 0 : 1);
   return launch_status();
 }
 
@@ -803,7 +827,7 @@ int launch_bwd_mfma_both(LogBwdArgs pa, LogBwdArgs pb, const float* stats, int B
 // eight waves), 1 for 128x128, 0 for none (path, or extents too small).  `long_cols`:
 // the 256 side is the column side of the output.
 inline int mfma_kind(int path, int B, int out_r, int out_c, int red, bool long_cols) {
-  if (path != GENBMM_PATH_AUTO || !mfma_extents(out_r, out_c, red)) return 0;
+  if (!auto_path(path) || !mfma_extents(out_r, out_c, red)) return 0;
   const int64_t t128 = tiles128(B, out_r, out_c);
   if (t128 > 0x7fffffff) return 0;
   const int L = long_cols ? out_c : out_r;
@@ -825,9 +849,9 @@ int run_bwd(const LogBwdArgs& p, const float* stats, int path, int B, hipStream_
     // the matrix-core kernels run on what the matrix-core forward left behind
     switch (fwd_mfma_shape(B, p.M, p.K, p.N) ? mfma_kind(path, B, R, Cc, Q, GRAD_A) : 0) {
       case 2:
-        if constexpr (GRAD_A) return launch_bwd_mfma<MTWide, true>(p, stats, B, s);
-        else return launch_bwd_mfma<MTTall, false>(p, stats, B, s);
-      case 1: return launch_bwd_mfma<MT128, GRAD_A>(p, stats, B, s);
+        if constexpr (GRAD_A) return launch_bwd_mfma<MTWide, true>(p, stats, B, s, path != GENBMM_PATH_FACTORS);
+        else return launch_bwd_mfma<MTTall, false>(p, stats, B, s, path != GENBMM_PATH_FACTORS);
+      case 1: return launch_bwd_mfma<MT128, GRAD_A>(p, stats, B, s, path != GENBMM_PATH_FACTORS);
       default: break;
     }
     if (small) return launch_bwd_fast<BCfgSmall, BCfgSmall, GRAD_A>(p, stats, B, s);
@@ -867,7 +891,8 @@ int run_fwd(const elem_t* a, const elem_t* b, elem_t* out, float* stats, int B, 
   if (!valid_path(path)) return GENBMM_E_MODE;
   const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
   if (missing(a, mk) || missing(b, kn) || missing(out, mn)) return GENBMM_E_NULLPTR;
-  if (stats && B > 0 && item_shape(M, K, N) && path == GENBMM_PATH_AUTO) {  // whole items per workgroup
+  if (path != GENBMM_PATH_FACTORS && !factors) keep = false;
+  if (stats && B > 0 && item_shape(M, K, N) && auto_path(path)) {  // whole items per workgroup
     int* hdr = prepared_of(stats, B, M, K, N).hdr;
     if (M == 32 && K == 32 && N == 32)  // one wave per item on the matrix cores
       hipLaunchKernelGGL(k_log_item32_fwd, dim3((B + 3) / 4), dim3(256), 0, s, a, b, out, stats, hdr, B);
@@ -878,7 +903,7 @@ int run_fwd(const elem_t* a, const elem_t* b, elem_t* out, float* stats, int B, 
   }
   DenseArgs p{};
   p.a = a; p.b = b; p.out = out; p.idx = nullptr;
-  if (stats && B > 0 && self_shape(M, K, N) && path == GENBMM_PATH_AUTO && !factors)
+  if (stats && B > 0 && self_shape(M, K, N) && auto_path(path) && !factors)
     return launch_self_fwd(p, stats, B, M, K, N, s);
   if (stats) {
     if (int e = launch_stats(a, b, stats, B, M, K, N, s)) return e;
@@ -918,7 +943,7 @@ int run_bwd_both(const elem_t* a, const elem_t* b, const elem_t* out, const elem
   p.vec_k = (K % 4 == 0) && aligned16(a) && aligned16(grad_a);
   p.vec_n = (N % 4 == 0) && aligned16(b) && aligned16(out) && aligned16(g) && aligned16(grad_b);
   const float* st = (path == GENBMM_PATH_EXACT || mn == 0) ? nullptr : stats;
-  if (st && B > 0 && item_shape(M, K, N) && path == GENBMM_PATH_AUTO) {
+  if (st && B > 0 && item_shape(M, K, N) && auto_path(path)) {
     if (M == 32 && K == 32 && N == 32)
       hipLaunchKernelGGL(k_log_item32_bwd, dim3((B + 3) / 4), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, B);
     else if (M == 64 && K == 64 && N == 64)
@@ -929,7 +954,7 @@ int run_bwd_both(const elem_t* a, const elem_t* b, const elem_t* out, const elem
       hipLaunchKernelGGL((k_log_item_bwd<16, 4>), dim3(B), dim3(256), 0, s, a, b, out, g, grad_a, grad_b, M, K, N);
     return launch_status();
   }
-  if (st && B > 0 && self_shape(M, K, N) && path == GENBMM_PATH_AUTO) {
+  if (st && B > 0 && self_shape(M, K, N) && auto_path(path)) {
     LogBwdArgs pa = p, pb = p;
     pa.grad = grad_a;
     pb.grad = grad_b;
@@ -947,8 +972,9 @@ int run_bwd_both(const elem_t* a, const elem_t* b, const elem_t* out, const elem
       LogBwdArgs pa = p, pb = p;
       pa.grad = grad_a;
       pb.grad = grad_b;
-      return ka == 2 ? launch_bwd_mfma_both<MTWide, MTTall>(pa, pb, st, B, s)
-                     : launch_bwd_mfma_both<MT128, MT128>(pa, pb, st, B, s);
+      const bool lean = path != GENBMM_PATH_FACTORS;
+      return ka == 2 ? launch_bwd_mfma_both<MTWide, MTTall>(pa, pb, st, B, s, lean)
+                     : launch_bwd_mfma_both<MT128, MT128>(pa, pb, st, B, s, lean);
     }
   }
   if (grad_a) {
@@ -1037,14 +1063,18 @@ int log_sample_sweep_mfma(const elem_t* a, const elem_t* b, elem_t* out, int32_t
 extern "C" {
 
 #if GENBMM_ELEM == 0
-size_t genbmm_logbmm_stats_size(int B, int M, int K, int N) {
+size_t genbmm_logbmm_stats_size_path(int B, int M, int K, int N, int path) {
   using namespace GENBMM_NS;
   if (check_dense_dims(B, M, K, N)) return 0;
-  int64_t n = header_offset(B, M, N) + 4;
-  // the one-tile kernels keep the maxima only
-  if (fwd_mfma_shape(B, M, K, N) && !self_shape(M, K, N))
+  int64_t n = header_offset(B, M, N) + 4;  // maxima, flags and the header
+  // the by-products of the matrix-core forward (the one-tile kernels keep the maxima only)
+  if (path == GENBMM_PATH_FACTORS && fwd_mfma_shape(B, M, K, N) && !self_shape(M, K, N))
     n += (int64_t)B * ((int64_t)M * K + (int64_t)K * N + (int64_t)M * N);
   return (size_t)n;
+}
+
+size_t genbmm_logbmm_stats_size(int B, int M, int K, int N) {
+  return genbmm_logbmm_stats_size_path(B, M, K, N, GENBMM_PATH_AUTO);
 }
 
 size_t genbmm_samplebmm_stats_size(int B, int M, int K, int N) {

@@ -650,6 +650,244 @@ void k_log_bwd_mfma_both(const elem_t* __restrict__ g, const float* __restrict__
                                          fwd_flags, grad_b, M, K, N, br, bc);
 }
 
+// ------------------------------------------------- backward without by-products
+// The same two contractions for a forward that kept nothing but the maxima and its flags (a
+// workspace of B (M + N) floats and a flag per tile instead of EA, EB and 1/S: at 64 x 512^3,
+// 0.3 MB instead of 201 MB): the operands are formed again while they are staged -
+// EA = exp(a - alpha), EB = exp(b - beta), H = g exp(alpha + beta - out) - and so is the
+// epilogue's factor: exponentials per staged element where the kernels above multiply once.
+// Shifts: alpha[m] of a piece's line (grad_a) or reduction step (grad_b), beta[n] of its four
+// columns.  RAGGED as above, with fills that make the exponential vanish: -inf for a and b,
+// +inf for out, 0 for g.
+struct LeanSrc {
+  const elem_t* a;
+  const elem_t* b;
+  const elem_t* out;
+  const float* stats;  // alpha (M) then beta (N) per batch item
+};
+__device__ __forceinline__ float4 mul_exp4(float4 g, float4 sh, float4 o) {  // g * exp(sh - o)
+  return make_float4(g.x * exp_st(sh.x - o.x), g.y * exp_st(sh.y - o.y), g.z * exp_st(sh.z - o.z),
+                     g.w * exp_st(sh.w - o.w));
+}
+template <class T, bool GRAD_A, bool RAGGED>
+__device__ __forceinline__ void log_bwd_mfma_tile_lean(
+    float* __restrict__ smem, int tile, const elem_t* __restrict__ g, const LeanSrc src,
+    const int* __restrict__ ws_hdr, const int* __restrict__ fwd_flags, elem_t* __restrict__ grad,
+    int M, int K, int N, int tiles_r, int tiles_c) {
+  constexpr int NT = T::NT, LDR = T::LDR, LDC = T::LDC;
+  using SH = std::conditional_t<GRAD_A, StageT<T::TR, NT, LDR>, StageS<T::TC, NT, LDC>>;
+  using SY = std::conditional_t<GRAD_A, StageT<T::TC, NT, LDC>, StageS<T::TR, NT, LDR>>;
+  float(*Rs)[kMS * LDR] = reinterpret_cast<float(*)[kMS * LDR]>(smem);
+  float(*Cs)[kMS * LDC] = reinterpret_cast<float(*)[kMS * LDC]>(smem + 2 * kMS * LDR);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wr0 = (wave / T::WC) * 64, wc0 = (wave % T::WC) * 64;
+  const int per = tiles_r * tiles_c;
+  const int batch = tile / per, rem = tile - batch * per;
+  const int r0 = (rem / tiles_c) * T::TR, c0 = (rem % tiles_c) * T::TC;
+  const int Q = GRAD_A ? N : M;
+  const int R = GRAD_A ? M : K, Cc = GRAD_A ? K : N;
+  const float* al = src.stats + (long)batch * (M + N);
+  const float* be = al + M;
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int x = 0; x < 4; ++x)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[x >> 1][x & 1][i] = 0.f;
+
+  float4 ry[SY::PER], ro[SH::PER], rg[SH::PER];
+  const elem_t* py[SY::PER];
+  const elem_t* po[SH::PER];
+  // g sits at the same element offsets as out (address arithmetic on integers, the result typed
+  // as global memory: see ws_twin)
+  const long dg = (long)(reinterpret_cast<uintptr_t>(g) - reinterpret_cast<uintptr_t>(src.out));
+  auto g_of = [&](const elem_t* o) __attribute__((always_inline)) {
+    return (const elem_t*)reinterpret_cast<global_ptr<const elem_t>>(reinterpret_cast<uintptr_t>(o) + (uintptr_t)dg);
+  };
+  // shifts.  grad_a: alpha of the H pieces' lines (fixed), beta of the slab's four columns (one
+  // float4 per slab, the same for every piece: all pieces of a thread share their quad).
+  // grad_b: beta of the lane's four columns (fixed), alpha of every piece's reduction step.
+  float alh[SH::PER];
+  const float* pbe = be + SH::quad(tid) * 4;  // grad_a: + kMS per slab
+  float4 be4 = make_float4(0.f, 0.f, 0.f, 0.f), bslab = be4;
+  float ay[SY::PER], ah[SH::PER];
+  int cy = 4, ch = 4;
+  if constexpr (GRAD_A) {
+#pragma unroll
+    for (int l = 0; l < SY::PER; ++l) {  // b[k][n]: line k, four n from quad*4
+      const int k = c0 + SY::line(tid, l);
+      py[l] = src.b + ((long)batch * K + (RAGGED ? min(k, K - 1) : k)) * N + SY::quad(tid) * 4;
+    }
+#pragma unroll
+    for (int l = 0; l < SH::PER; ++l) {
+      const int m = r0 + SH::line(tid, l);
+      const int mc = RAGGED ? min(m, M - 1) : m;
+      po[l] = src.out + ((long)batch * M + mc) * N + SH::quad(tid) * 4;
+      alh[l] = al[mc];
+    }
+  } else {
+    const int kc = r0 + SY::quad(tid) * 4, nc = c0 + SH::quad(tid) * 4;
+    cy = RAGGED ? clamp4(K - kc) : 4;
+    ch = RAGGED ? clamp4(N - nc) : 4;
+#pragma unroll
+    for (int l = 0; l < SY::PER; ++l)    // a[m][k]: row m = red, four k
+      py[l] = src.a + ((long)batch * M + SY::red(tid, l)) * K + (cy > 0 ? kc : 0);
+#pragma unroll
+    for (int l = 0; l < SH::PER; ++l)
+      po[l] = src.out + ((long)batch * M + SH::red(tid, l)) * N + (ch > 0 ? nc : 0);
+    be4 = RAGGED ? ld4m(be + (ch > 0 ? nc : 0), ch, 0.f) : ld4(be + nc);
+  }
+  const int qtail = RAGGED ? Q % kMS : 0;
+  const int slabs = RAGGED ? (Q + kMS - 1) / kMS : Q / kMS;
+  int s_load = 0;  // slab the next load() fetches
+  auto load = [&](bool tail) __attribute__((always_inline)) {
+    const int q0 = s_load * kMS;
+    if constexpr (GRAD_A) {
+      const int left = tail ? qtail - SH::redpos(tid, 0) : 4;  // all pieces share their quad
+      if (!RAGGED) {
+#pragma unroll
+        for (int l = 0; l < SY::PER; ++l) ry[l] = ld4(py[l]);
+#pragma unroll
+        for (int l = 0; l < SH::PER; ++l) {
+          ro[l] = ld4(po[l]);
+          rg[l] = ld4(g_of(po[l]));
+        }
+        bslab = ld4(pbe);
+      } else {
+#pragma unroll
+        for (int l = 0; l < SY::PER; ++l) ry[l] = ld4m(py[l], left, -INFINITY);
+#pragma unroll
+        for (int l = 0; l < SH::PER; ++l) {
+          ro[l] = ld4m(po[l], left, INFINITY);
+          rg[l] = ld4m(g_of(po[l]), left, 0.f);
+        }
+        bslab = ld4m(pbe, left, 0.f);
+      }
+      pbe += kMS;
+    } else {
+#pragma unroll
+      for (int l = 0; l < SY::PER; ++l) {
+        const bool in = !RAGGED || !tail || SY::redpos(tid, l) < qtail;
+        ry[l] = RAGGED ? ld4m(py[l], in ? cy : 0, -INFINITY) : ld4(py[l]);
+        ay[l] = in ? al[q0 + SY::red(tid, l)] : 0.f;
+      }
+#pragma unroll
+      for (int l = 0; l < SH::PER; ++l) {
+        const bool in = !RAGGED || !tail || SH::redpos(tid, l) < qtail;
+        ro[l] = RAGGED ? ld4m(po[l], in ? ch : 0, INFINITY) : ld4(po[l]);
+        rg[l] = RAGGED ? ld4m(g_of(po[l]), in ? ch : 0, 0.f) : ld4(g_of(po[l]));
+        ah[l] = in ? al[q0 + SH::red(tid, l)] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int l = 0; l < SY::PER; ++l) py[l] += GRAD_A ? (long)kMS : (long)kMS * K;
+#pragma unroll
+    for (int l = 0; l < SH::PER; ++l) po[l] += GRAD_A ? (long)kMS : (long)kMS * N;
+    ++s_load;
+  };
+  auto stage = [&](int buf) __attribute__((always_inline)) {
+    float* ybuf = GRAD_A ? Cs[buf] : Rs[buf];
+    float* hbuf = GRAD_A ? Rs[buf] : Cs[buf];
+#pragma unroll
+    for (int l = 0; l < SY::PER; ++l) {
+      if constexpr (GRAD_A) SY::put(ybuf, tid, l, exp4(ry[l], bslab));
+      else SY::put(ybuf, tid, l, exp4(ry[l], ay[l]));
+    }
+#pragma unroll
+    for (int l = 0; l < SH::PER; ++l) {
+      float4 sh;
+      if constexpr (GRAD_A) sh = make_float4(alh[l] + bslab.x, alh[l] + bslab.y, alh[l] + bslab.z, alh[l] + bslab.w);
+      else sh = make_float4(ah[l] + be4.x, ah[l] + be4.y, ah[l] + be4.z, ah[l] + be4.w);
+      SH::put(hbuf, tid, l, mul_exp4(rg[l], sh, ro[l]));
+    }
+  };
+
+  load(slabs == 1 && qtail != 0);
+  if (bwd_tile_flagged(ws_hdr, fwd_flags, false, GRAD_A, GRAD_A ? r0 : c0, GRAD_A ? T::TR : T::TC, batch,
+                       M, N, tid, NT))
+    return;
+  stage(0);
+  __syncthreads();
+  for (int s = 0; s < slabs; ++s) {
+    const bool more = s + 1 < slabs;
+    if (more) load(s + 2 == slabs && qtail != 0);
+    mfma_slab<LDR, LDC>(Rs[s & 1], Cs[s & 1], wr0, wc0, lane, acc);
+    if (more) stage((s + 1) & 1);
+    __syncthreads();
+  }
+
+  // grad = EX * acc with EX = exp(a - alpha) (grad_a) or exp(b - beta) (grad_b), row-wise
+  const int lr = lane >> 4, lc = (lane & 15) * 4;
+  const int voff = lr * Cc + lc;
+  const long ubase = ((long)batch * R + r0 + wr0) * Cc + c0 + wc0;
+  const elem_t* xb = (GRAD_A ? src.a : src.b) + ubase + voff;
+  elem_t* gp = grad + ubase + voff;
+  const int cc = RAGGED ? clamp4(Cc - (c0 + wc0 + lc)) : 4;
+  const bool cok = cc > 0;
+  const int rows_left = R - (r0 + wr0) - lr;
+  float4 becol = make_float4(0.f, 0.f, 0.f, 0.f);
+  if constexpr (!GRAD_A) becol = RAGGED ? ld4m(be + (cok ? c0 + wc0 + lc : 0), cc, 0.f) : ld4(be + c0 + wc0 + lc);
+  const float* alrow = al + r0 + wr0 + lr;
+  float4 xq[2][4];
+  float xa[2][4];
+  auto fetch = [&](int q) __attribute__((always_inline)) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const bool live = !RAGGED || (cok && 16 * q + 4 * t < rows_left);
+      if (live) {
+        xq[q & 1][t] = RAGGED ? ld4m(xb + (long)(16 * q + 4 * t) * Cc, cc, -INFINITY) : ld4(xb + (long)(16 * q + 4 * t) * Cc);
+        if constexpr (GRAD_A) xa[q & 1][t] = alrow[16 * q + 4 * t];
+      }
+    }
+  };
+  fetch(0);
+  acc_rows(acc, smem + wave * kStripFloats, lane,
+           [&](int q) __attribute__((always_inline)) { if (q + 1 < 4) fetch(q + 1); },
+           [&](int q, int t, float4 v) __attribute__((always_inline)) {
+             if (RAGGED && !(cok && 16 * q + 4 * t < rows_left)) return;
+             float4 x;
+             if constexpr (GRAD_A) x = exp4(xq[q & 1][t], xa[q & 1][t]);
+             else x = exp4(xq[q & 1][t], becol);
+             const float4 r = make_float4(x.x * v.x, x.y * v.y, x.z * v.z, x.w * v.w);
+             if (RAGGED) st4m(gp + (long)(16 * q + 4 * t) * Cc, cc, r);
+             else st4(gp + (long)(16 * q + 4 * t) * Cc, r);
+           });
+}
+
+template <class T, bool GRAD_A, bool RAGGED>
+__global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WPE, T::WPE)))
+void k_log_bwd_mfma_lean(const elem_t* __restrict__ g, const LeanSrc src, const int* __restrict__ ws_hdr,
+                         const int* __restrict__ fwd_flags, elem_t* __restrict__ grad, int M, int K, int N,
+                         int tiles_r, int tiles_c) {
+  __shared__ __attribute__((aligned(16))) float smem[2 * kMS * (T::LDR + T::LDC)];
+  log_bwd_mfma_tile_lean<T, GRAD_A, RAGGED>(smem, xcd_tile_id(), g, src, ws_hdr, fwd_flags, grad, M, K, N, tiles_r,
+                                            tiles_c);
+}
+
+// Both gradients in one launch, item by item (see k_log_bwd_mfma_both): here the two share
+// a, b, out and g.
+template <class TA, class TB, bool RAGGED>
+__global__ __launch_bounds__(TA::NT) __attribute__((amdgpu_waves_per_eu(TA::WPE, TA::WPE)))
+void k_log_bwd_mfma_both_lean(const elem_t* __restrict__ g, const LeanSrc src, const int* __restrict__ ws_hdr,
+                              const int* __restrict__ fwd_flags, elem_t* __restrict__ grad_a,
+                              elem_t* __restrict__ grad_b, int M, int K, int N, int tiles_a, int ar, int ac,
+                              int br, int bc) {
+  static_assert(TA::NT == TB::NT && TA::WPE == TB::WPE, "");
+  constexpr int kA = 2 * kMS * (TA::LDR + TA::LDC), kB = 2 * kMS * (TB::LDR + TB::LDC);
+  __shared__ __attribute__((aligned(16))) float smem[kA > kB ? kA : kB];
+  const int per_a = ar * ac, per_b = br * bc;
+  const int v = xcd_renumber(blockIdx.x, gridDim.x);
+  const int item = v / (per_a + per_b), r = v - item * (per_a + per_b);
+  const bool alt = per_a == per_b;
+  const bool is_a = alt ? (r & 1) == 0 : r < per_a;
+  const int idx = alt ? r >> 1 : (r < per_a ? r : r - per_a);
+  if (is_a)
+    log_bwd_mfma_tile_lean<TA, true, RAGGED>(smem, item * per_a + idx, g, src, ws_hdr, fwd_flags, grad_a, M, K, N, ar, ac);
+  else
+    log_bwd_mfma_tile_lean<TB, false, RAGGED>(smem, item * per_b + idx, g, src, ws_hdr, fwd_flags, grad_b, M, K, N, br, bc);
+}
+
 // ------------------------------------------------------- sampling sweep
 // samplebmm on the forward's factors: index = first k whose prefix sum
 // sum_{k' <= k} EA[m,k'] EB[k',n] passes the target t = u * S (one Philox uniform

@@ -53,7 +53,7 @@ def _sfx(t):
     return _lib.HALF_SUFFIX.get(t.dtype, "")
 
 
-PATH_AUTO, PATH_EXACT, PATH_VALU = 0, 1, 2  # GENBMM_PATH_* of the C header
+PATH_AUTO, PATH_EXACT, PATH_VALU, PATH_FACTORS = 0, 1, 2, 3  # GENBMM_PATH_* of the C header
 
 
 def _prep(a, b):
@@ -171,7 +171,7 @@ class LogMatMul(torch.autograd.Function):
             _call("genbmm_logbmm_fwd_f64", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), B, M, K, N)
         else:
             # the library's workspace: what the reference's `maxes` becomes
-            stats = torch.empty(_lib.load().genbmm_logbmm_stats_size(B, M, K, N), dtype=_COMPUTE,
+            stats = torch.empty(_lib.load().genbmm_logbmm_stats_size_path(B, M, K, N, path), dtype=_COMPUTE,
                                 device=a.device)
             _call("genbmm_logbmm_fwd_path" + _sfx(a), a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out),
                   _lib.ptr(stats), B, M, K, N, path)
@@ -334,11 +334,15 @@ def logbmm(a, b):
         b_s = (b.float() if b.dtype in _lib.HALF_SUFFIX else b).view(B * S, K // S, N)
         parts = LogMatMul.apply(a_s, b_s, PATH_AUTO).view(B, S, M, N)
         return restore(torch.logsumexp(parts, dim=1).to(a.dtype))
-    return restore(LogMatMul.apply(a, b, PATH_AUTO))
+    # float16 / bfloat16 tensors keep 1 / sum in float32 for the backward (PATH_FACTORS): with the
+    # maxima alone it would be rebuilt from `out` as stored, i.e. rounded to 11 or 8 bits
+    return restore(LogMatMul.apply(a, b, PATH_FACTORS if a.dtype in _lib.HALF_SUFFIX else PATH_AUTO))
 
 
 def logbmm_on_path(a, b, path):
-    """logbmm with the library's kernel family named (PATH_AUTO / PATH_EXACT / PATH_VALU);
+    """logbmm with the library's kernel family named (PATH_AUTO / PATH_EXACT / PATH_VALU / PATH_FACTORS:
+    as PATH_AUTO, but autograd saves exp(a - max), exp(b - max) and 1 / sum beside the maxima - three
+    more tensors than the reference saves - and the matrix-core backward takes no exponential);
     forward and backward both use it.  For tests and measurements."""
     a, b, restore = _canonical(a, b)
     return restore(LogMatMul.apply(a, b, path))

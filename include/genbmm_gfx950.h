@@ -128,12 +128,29 @@ size_t genbmm_samplebmm_stats_size(int B, int M, int K, int N);
  *                      `stats` gives; a non-NULL one still receives the maxima);
  *   GENBMM_PATH_VALU   the factored kernels contracting with v_fma_f32 on the
  *                      vector ALU, never the matrix cores or whole-item kernels.
+ *   GENBMM_PATH_FACTORS as AUTO, but the matrix-core forward leaves
+ *                      exp(a - max), exp(b - max) and 1 / sum in `stats`
+ *                      (201 MB at 64 x 512^3) and the matrix-core backward
+ *                      reads them instead of forming them again: a backward
+ *                      without an exponential, at 600 times the workspace.
+ * Under AUTO the matrix-core kernels keep the reference's memory footprint (it
+ * saves one `maxes` tensor, genmul.py:29-32): `stats` holds the row / column
+ * maxima and a flag per tile (0.3 MB at 64 x 512^3), and the backward forms
+ * exp(a - max), exp(b - max) and g exp(max - out) again while it stages them -
+ * measured 3 % faster per forward + backward than keeping the factors (the
+ * forward writes 200 MB less, the backward takes three exponentials per staged
+ * element).  With float16 / bfloat16 tensors that backward reads `out` as stored
+ * (rounded); FACTORS keeps 1 / sum in fp32.
  * Any other value: GENBMM_E_MODE.  Forward and backward of one problem need not
  * name the same path (see genbmm_logbmm_bwd).  No counterpart in the reference.
  */
 #define GENBMM_PATH_AUTO 0
 #define GENBMM_PATH_EXACT 1
 #define GENBMM_PATH_VALU 2
+#define GENBMM_PATH_FACTORS 3
+/* Number of fp32 elements of `stats` for a forward / backward pair on `path`
+ * (genbmm_logbmm_stats_size is this for GENBMM_PATH_AUTO). */
+size_t genbmm_logbmm_stats_size_path(int B, int M, int K, int N, int path);
 int genbmm_logbmm_fwd_path(const float* a, const float* b, float* out,
                            float* stats, int B, int M, int K, int N, int path,
                            void* stream);

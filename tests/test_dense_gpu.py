@@ -35,13 +35,16 @@ def lse64(a, b, chunk=4):
     return torch.cat(outs) if outs else a.new_zeros((0, a.shape[1], b.shape[2])).double()
 
 
-@pytest.fixture(params=["factored", "exact", "factored-valu"])
+@pytest.fixture(params=["factored", "exact", "factored-valu", "factors-kept"])
 def path(request, gpu):
     """Run a logbmm test on every kernel family of the library: the default one (whole-item
     kernels for small matrices, matrix cores for large ones, factored vector-ALU kernels
-    between), the online / exact kernels alone, and the factored kernels on v_fma only.
+    between; the matrix-core kernels keep the maxima only and form their operands again in the
+    backward), the online / exact kernels alone, the factored kernels on v_fma only, and the
+    default kernels with the forward's factors kept for an exponent-free backward.
     The value is the `path` argument of genbmm_logbmm_fwd_path / _bwd_path."""
-    return {"factored": genmul.PATH_AUTO, "exact": genmul.PATH_EXACT, "factored-valu": genmul.PATH_VALU}[request.param]
+    return {"factored": genmul.PATH_AUTO, "exact": genmul.PATH_EXACT, "factored-valu": genmul.PATH_VALU,
+            "factors-kept": genmul.PATH_FACTORS}[request.param]
 
 
 def logbmm_on(path):
@@ -169,13 +172,16 @@ def test_logbmm_factoring_guard(gpu, B, M, K, N):
 @pytest.mark.parametrize("B,M,K,N", [(32, 256, 128, 256), (64, 512, 128, 512), (64, 200, 100, 260),
                                      (64, 500, 132, 500), (128, 260, 388, 132), (24, 201, 103, 259),
                                      (3, 130, 97, 391), (64, 257, 255, 129)])
-def test_logbmm_factoring_guard_matrix_core_tiles(gpu, B, M, K, N):
+@pytest.mark.parametrize("keep", [False, True])
+def test_logbmm_factoring_guard_matrix_core_tiles(gpu, keep, B, M, K, N):
     """Shapes that run on the matrix-core kernels (128x128 and 128x256 / 256x128 tiles),
     all but the first two with ragged edges in every dimension (partial tiles, partial slabs),
     the last three with odd sizes (rows not 16-byte aligned, pieces straddling the edge).
     Some batch items need the exact fall-back in every tile, one in a single row, the
     rest in none: flagged and unflagged tiles side by side, and the backward kernels
-    must honour the forward's flags (they read 1/S from the forward's workspace)."""
+    must honour the forward's flags.  keep: the forward's factors are kept and the backward
+    reads 1/S from the workspace (GENBMM_PATH_FACTORS); else only the maxima are kept and the
+    backward forms its operands again."""
     torch.manual_seed(B + M)
     a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
     a[: B // 4, ::2, 0] += 200.0
@@ -185,7 +191,7 @@ def test_logbmm_factoring_guard_matrix_core_tiles(gpu, B, M, K, N):
     pick = torch.tensor([0, 1, B // 4, B // 4 + 1, B - 1])
     want, wa, wb = oracle.logbmm_grads64(a[pick], b[pick], g[pick])
     ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
-    out = genbmm.logbmm(ad, bd)
+    out = genmul.logbmm_on_path(ad, bd, genmul.PATH_FACTORS) if keep else genbmm.logbmm(ad, bd)
     ga, gb = torch.autograd.grad(out, (ad, bd), g.to(gpu))
     close(out[pick.to(gpu)], want)
     close(ga[pick.to(gpu)], wa)
@@ -196,7 +202,8 @@ def test_logbmm_factoring_guard_matrix_core_tiles(gpu, B, M, K, N):
 
 @pytest.mark.parametrize("B,M,K,N", [(8, 256, 128, 256), (6, 300, 100, 260), (4, 512, 64, 384), (9, 32, 32, 32),
                                      (6, 64, 64, 64), (5, 40, 48, 36), (7, 128, 128, 128), (4, 100, 70, 128)])
-def test_logbmm_rows_masked_at_the_floor(gpu, B, M, K, N):
+@pytest.mark.parametrize("keep", [False, True])
+def test_logbmm_rows_masked_at_the_floor(gpu, keep, B, M, K, N):
     """Padding written as -1e9, the reference's own floor (matmul_cuda_kernel.cu:31): whole
     rows of a, whole columns of b, or - one batch item - both.  A cell of a masked row has
     max_k(a + b) = -1e9 + max_k b, not below the floor, so the reference's result is the
@@ -219,7 +226,7 @@ def test_logbmm_rows_masked_at_the_floor(gpu, B, M, K, N):
     g[B - 1, rows:, :] = 0.0
     want, wa, wb = oracle.logbmm_grads64(a, b, g)
     ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
-    out = genbmm.logbmm(ad, bd)
+    out = genmul.logbmm_on_path(ad, bd, genmul.PATH_FACTORS) if keep else genbmm.logbmm(ad, bd)
     ga, gb = torch.autograd.grad(out, (ad, bd), g.to(gpu))
     both = torch.zeros(B, M, N, dtype=torch.bool)
     both[B - 1, rows:, cols:] = True
@@ -306,26 +313,33 @@ def test_logbmm_one_tile_items(gpu, B, M, K, N):
 
 
 def test_logbmm_backward_on_foreign_workspace(gpu):
-    """The matrix-core backward runs on by-products of the matrix-core forward; handed
-    a workspace that another forward path filled, it must notice and still be right."""
+    """The exponent-free matrix-core backward (GENBMM_PATH_FACTORS) runs on by-products of the
+    matrix-core forward; handed a workspace that another forward path filled - the vector-ALU
+    forward, or the default matrix-core forward, which keeps the maxima only - it must notice
+    and still be right (every tile then goes to the exact routine).  The default backward takes
+    any of them as they are."""
     lib = _lib.load()
     torch.manual_seed(3)
     B, M, K, N = 32, 256, 128, 256
     a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
     ad, bd, gd = a.to(gpu), b.to(gpu), g.to(gpu)
-    out, ga, gb = torch.empty(B, M, N, device=gpu), torch.empty_like(ad), torch.empty_like(bd)
-    stats = torch.full((lib.genbmm_logbmm_stats_size(B, M, K, N),), float("nan"), device=gpu)
     p, s = _lib.ptr, _lib.stream_of(ad)
-    assert lib.genbmm_logbmm_fwd_path(p(ad), p(bd), p(out), p(stats), B, M, K, N, genmul.PATH_VALU, s) == 0
-    before = stats.clone()
-    assert lib.genbmm_logbmm_bwd(p(ad), p(bd), p(out), p(gd), p(stats), p(ga), p(gb), B, M, K, N, s) == 0
-    assert torch.equal(before.view(torch.int32), stats.view(torch.int32))  # the backward only reads it
+    big = lib.genbmm_logbmm_stats_size_path(B, M, K, N, genmul.PATH_FACTORS)
+    assert big > B * (M * K + K * N + M * N) > lib.genbmm_logbmm_stats_size(B, M, K, N)
     pick = torch.tensor([0, B - 1])
     want, wa, wb = oracle.logbmm_grads64(a[pick], b[pick], g[pick])
-    close(out[pick.to(gpu)], want)
-    close(ga[pick.to(gpu)], wa)
-    close(gb[pick.to(gpu)], wb)
-    close(ga.sum(-1), g.double().sum(-1), atol=2e-4)
+    for fwd_path in (genmul.PATH_VALU, genmul.PATH_AUTO, genmul.PATH_FACTORS):
+        for bwd_path in (genmul.PATH_FACTORS, genmul.PATH_AUTO):
+            out, ga, gb = torch.empty(B, M, N, device=gpu), torch.empty_like(ad), torch.empty_like(bd)
+            stats = torch.full((big,), float("nan"), device=gpu)
+            assert lib.genbmm_logbmm_fwd_path(p(ad), p(bd), p(out), p(stats), B, M, K, N, fwd_path, s) == 0
+            before = stats.clone()
+            assert lib.genbmm_logbmm_bwd_path(p(ad), p(bd), p(out), p(gd), p(stats), p(ga), p(gb), B, M, K, N, bwd_path, s) == 0
+            assert torch.equal(before.view(torch.int32), stats.view(torch.int32))  # the backward only reads it
+            close(out[pick.to(gpu)], want)
+            close(ga[pick.to(gpu)], wa)
+            close(gb[pick.to(gpu)], wb)
+            close(ga.sum(-1), g.double().sum(-1), atol=2e-4)
 
 
 @pytest.mark.parametrize("B,M,K,N", [(2, 4, 5, 3), (3, 9, 12, 7), (2, 33, 20, 40)])

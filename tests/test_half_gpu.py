@@ -39,14 +39,15 @@ def _operands(gpu, dt, B, M, K, N, scale=2.0):
 
 
 @pytest.mark.parametrize("dt,suffix,eps", TYPES)
-@pytest.mark.parametrize("path", [genbmm.genmul.PATH_AUTO, genbmm.genmul.PATH_EXACT, genbmm.genmul.PATH_VALU])
+@pytest.mark.parametrize("path", [genbmm.genmul.PATH_AUTO, genbmm.genmul.PATH_EXACT, genbmm.genmul.PATH_VALU,
+                                  genbmm.genmul.PATH_FACTORS])
 def test_logbmm_half_equals_float_kernels_rounded(gpu, dt, suffix, eps, path):
     lib = _lib.load()
     torch.manual_seed(3)
     for B, M, K, N in SHAPES:
         a, b, g = _operands(gpu, dt, B, M, K, N)
         a32, b32, g32 = a.float(), b.float(), g.float()
-        n = lib.genbmm_logbmm_stats_size(B, M, K, N)
+        n = lib.genbmm_logbmm_stats_size_path(B, M, K, N, path)
         st, st32 = torch.empty(n, device=gpu), torch.empty(n, device=gpu)
         out, out32 = torch.empty(B, M, N, device=gpu, dtype=dt), torch.empty(B, M, N, device=gpu)
         s = _lib.stream_of(a)
