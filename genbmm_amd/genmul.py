@@ -214,17 +214,63 @@ def _argmax_backward(ctx, grad_output, prod):
     return grad_a, grad_b
 
 
+def _max_forward(a, b, prod, factors=None):
+    """(out, idx) of the max / prod-max product through the library; `factors` (2, B, M, N) receives
+    a[m, idx], b[idx, n] of prod-max.  A long reduction over few output tiles is cut into S pieces
+    of K, each a batch item of its own (see _reduction_splits): the pieces' maxima are joined
+    here - the first piece that attains the maximum wins, as the lowest k does inside a piece -
+    and the indices become indices into the whole of K."""
+    B, M, K = a.shape
+    N = b.shape[2]
+    S = 1 if _f64(a) else _reduction_splits(B, M, K, N)
+    name = "genbmm_prodmaxbmm_fwd" if prod else "genbmm_maxbmm_fwd"
+    if S == 1:
+        out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)
+        idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
+        if _f64(a):
+            _call(name + "_f64", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), B, M, K, N)
+        elif prod:
+            _call(name + _sfx(a), a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), _lib.ptr(factors), B, M, K, N)
+        else:
+            _call(name + _sfx(a), a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), B, M, K, N)
+        return out, idx
+    Ks = K // S
+    # (float16 / bfloat16 operands: the pieces are compared unrounded, in float32 - two pieces whose
+    # maxima round to the same half value must still be told apart - and the result is rounded once)
+    wide_a = a.float() if a.dtype in _lib.HALF_SUFFIX else a
+    wide_b = b.float() if b.dtype in _lib.HALF_SUFFIX else b
+    a_s = wide_a.view(B, M, S, Ks).transpose(1, 2).reshape(B * S, M, Ks).contiguous()
+    b_s = wide_b.view(B * S, Ks, N)
+    vals = torch.empty(B * S, M, N, dtype=a_s.dtype, device=a.device)
+    idxs = torch.empty(B * S, M, N, dtype=torch.int32, device=a.device)
+    if prod:
+        fac_s = torch.empty(2, B * S, M, N, dtype=_COMPUTE, device=a.device)
+        _call(name, a, _lib.ptr(a_s), _lib.ptr(b_s), _lib.ptr(vals), _lib.ptr(idxs), _lib.ptr(fac_s), B * S, M, Ks, N)
+    else:
+        _call(name, a, _lib.ptr(a_s), _lib.ptr(b_s), _lib.ptr(vals), _lib.ptr(idxs), B * S, M, Ks, N)
+    vals, idxs = vals.view(B, S, M, N), idxs.view(B, S, M, N)
+    # a piece without a term above the -1e9 floor reports the floor and index -1: it never wins
+    # against a piece with one, and if no piece has one the result is the floor and -1 as well
+    top = vals.amax(1, keepdim=True)
+    pieces = torch.arange(S, device=a.device).view(1, S, 1, 1)
+    first = torch.where(vals == top, pieces, torch.full_like(pieces, S)).amin(1, keepdim=True)   # lowest piece on ties
+    first = first.clamp(max=S - 1)      # (all NaN: cannot happen, NaN terms never win inside a piece)
+    out = torch.gather(vals, 1, first).squeeze(1)
+    local = torch.gather(idxs, 1, first).squeeze(1)
+    idx = torch.where(local >= 0, local + (first.squeeze(1) * Ks).to(torch.int32), local).contiguous()
+    if prod:
+        fac = fac_s.view(2, B, S, M, N)
+        factors.copy_(torch.gather(fac, 2, first.unsqueeze(0).expand(2, -1, -1, -1, -1)).squeeze(2))
+    return out.to(a.dtype).contiguous(), idx
+
+
 class MaxMatMul(torch.autograd.Function):
     """out = max_k(a + b), ties to the lowest k   (reference genmul.py:52-65)."""
 
     @staticmethod
     def forward(ctx, a, b):
         dims = _prep(a, b)
-        B, M, K, N = dims
-        out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)
-        idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
-        _call("genbmm_maxbmm_fwd_f64" if _f64(a) else "genbmm_maxbmm_fwd" + _sfx(a), a, _lib.ptr(a),
-              _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx), B, M, K, N)
+        out, idx = _max_forward(a, b, False)
         ctx.save_for_backward(idx)
         ctx.dims, ctx.compute = dims, a.dtype
         return out
@@ -241,17 +287,13 @@ class ProdMaxMatMul(torch.autograd.Function):
     def forward(ctx, a, b):
         dims = _prep(a, b)
         B, M, K, N = dims
-        out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)
-        idx = torch.empty(B, M, N, dtype=torch.int32, device=a.device)
         empty = a.new_empty(0)
         if _f64(a):
-            _call("genbmm_prodmaxbmm_fwd_f64", a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out),
-                  _lib.ptr(idx), B, M, K, N)
+            out, idx = _max_forward(a, b, True)
             ctx.save_for_backward(idx, empty, a, b)
         else:
             factors = torch.empty(2, B, M, N, dtype=_COMPUTE, device=a.device)
-            _call("genbmm_prodmaxbmm_fwd" + _sfx(a), a, _lib.ptr(a), _lib.ptr(b), _lib.ptr(out), _lib.ptr(idx),
-                  _lib.ptr(factors), B, M, K, N)
+            out, idx = _max_forward(a, b, True, factors)
             ctx.save_for_backward(idx, factors, empty, empty)
         ctx.dims, ctx.compute = dims, a.dtype
         return out

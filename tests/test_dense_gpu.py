@@ -967,6 +967,33 @@ def test_long_reductions_with_few_tiles_are_split(gpu, B, M, K, N):
         close(db, w2[1], rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("B,M,K,N", [(2, 40, 4096, 30), (1, 7, 8192, 5), (1, 100, 4608, 96), (1, 16, 6000, 16)])
+@pytest.mark.parametrize("prod", [False, True])
+def test_long_reductions_of_the_max_products_are_split(gpu, prod, B, M, K, N):
+    """maxbmm / prodmaxbmm cut a long reduction over few output tiles into batch items of its own
+    and join the pieces' maxima (host layer): values, indices into the whole of K (ties to the
+    lowest k, also across pieces) and gradients equal the sequential oracle's bit for bit."""
+    assert genmul._reduction_splits(B, M, K, N) > 1
+    torch.manual_seed(K + N)
+    if prod:
+        a, b = 1 - torch.rand(B, M, K), 1 - torch.rand(B, K, N)
+    else:
+        a, b = grid(B, M, K), grid(B, K, N)      # multiples of 1/8: many ties, within and across pieces
+    g = grid(B, M, N).clamp(-4, 4)
+    sv, si = oracle.seq_maxbmm_fwd(a, b, prod)
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    out = (genbmm.prodmaxbmm if prod else genbmm.maxbmm)(ad, bd)
+    assert torch.equal(out.detach().cpu(), sv)
+    ga, gb = torch.autograd.grad(out, (ad, bd), g.to(gpu))
+    wa, wb = oracle.seq_argmax_bwd(a if prod else K, b, si, g, prod)
+    assert torch.equal(ga.cpu(), wa) and torch.equal(gb.cpu(), wb)
+    # half tensors: the float function on the widened tensors, rounded once
+    ah, bh = a.half().to(gpu), b.half().to(gpu)
+    oh = (genbmm.prodmaxbmm if prod else genbmm.maxbmm)(ah, bh)
+    of = (genbmm.prodmaxbmm if prod else genbmm.maxbmm)(ah.float(), bh.float())
+    assert oh.dtype == torch.float16 and torch.equal(oh, of.half())
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_long_reductions_split_with_half_tensors(gpu, dtype):
     """The split of a long reduction on float16 / bfloat16 operands keeps the half contract: what
