@@ -202,34 +202,44 @@ def dense_sample(lib, dev, B, M, K, N, reps):
            {"ms_fwd": round(mf, 4), "ms_bwd": round(mb, 4)})
 
 
-def banded(lib, dev, B, n, lu, ld, mode, reps, pad=None):
-    """pad = (value, rows): the last `rows` band rows of a hold `value`, no gradient flows into them."""
+def banded(lib, dev, B, n, lu, ld, mode, reps, pad=None, dtype=torch.float32):
+    """pad = (value, rows): the last `rows` band rows of a hold `value`, no gradient flows into them.
+    mode 2: the sample product (forward = log product + index walk, backward = one-hot scatter).
+    dtype float16 / bfloat16: the `_f16` / `_bf16` entry points on band tensors of that type."""
     torch.manual_seed(7)
     W = lu + ld + 1
     Wo = 2 * W - 1
-    a, b = (torch.rand(B, n, W) * 2 - 1).to(dev), (torch.rand(B, n, W) * 2 - 1).to(dev)
-    g = torch.randn(B, n, Wo).to(dev)
+    a, b = (torch.rand(B, n, W) * 2 - 1).to(dev).to(dtype), (torch.rand(B, n, W) * 2 - 1).to(dev).to(dtype)
+    g = torch.randn(B, n, Wo).to(dev).to(dtype)
     if pad is not None:
         a[:, n - pad[1]:, :] = pad[0]
         g[:, n - pad[1]:, :] = 0
-    out = torch.empty(B, n, Wo, device=dev)
-    idx = torch.empty(B, n, Wo, dtype=torch.int32, device=dev) if mode == 1 else None
+    out = torch.empty(B, n, Wo, device=dev, dtype=dtype)
+    idx = torch.empty(B, n, Wo, dtype=torch.int32, device=dev) if mode in (1, 2) else None
     ga, gb = torch.empty_like(a), torch.empty_like(b)
-    ws = torch.empty(lib.genbmm_banded_workspace_size(lu, ld, lu, ld, B, n), device=dev) if mode == 0 else None
+    ws = torch.empty(lib.genbmm_banded_workspace_size(lu, ld, lu, ld, B, n), device=dev) if mode in (0, 2) else None
     s, p = _lib.stream_of(a), _lib.ptr
+    sfx = _lib.HALF_SUFFIX.get(dtype, "")
+    fwd, bwd, smp = (getattr(lib, nm + sfx) for nm in ("genbmm_banded_fwd", "genbmm_banded_bwd", "genbmm_banded_sample_fwd"))
 
     def f():
-        _lib.check(lib.genbmm_banded_fwd(p(a), lu, ld, p(b), lu, ld, p(out), p(idx), p(ws), B, n, mode, s), "fwd")
+        if mode == 2:
+            _lib.check(smp(p(a), lu, ld, p(b), lu, ld, p(out), p(idx), p(ws), 1234, 0, B, n, s), "sample fwd")
+        else:
+            _lib.check(fwd(p(a), lu, ld, p(b), lu, ld, p(out), p(idx), p(ws), B, n, mode, s), "fwd")
 
     def bw():
-        _lib.check(lib.genbmm_banded_bwd(p(a), lu, ld, p(b), lu, ld, p(out), p(idx), p(ws), p(g), p(ga), p(gb), B, n, mode, s),
+        _lib.check(bwd(p(a), lu, ld, p(b), lu, ld, p(out), p(idx), p(None) if mode == 2 else p(ws), p(g), p(ga), p(gb), B, n, mode, s),
                    "bwd")
 
     mf, mb = timed(f, reps), timed(bw, reps)
     pairs = float(B) * n * W * W
-    fb = 4.0 * B * n * (2 * W + Wo) + (4.0 * B * n * Wo if mode == 1 else 0)
-    bb = 4.0 * B * n * (4 * W + Wo + (Wo if mode in (0, 1) else 0))
-    name = {0: "multiply_log", 1: "multiply_max", 3: "multiply"}[mode]
+    es = float(a.element_size())
+    fb = es * B * n * (2 * W + Wo) + (4.0 * B * n * Wo if mode in (1, 2) else 0)
+    bb = es * B * n * (4 * W + Wo) + (es * B * n * Wo if mode == 0 else 0) + (4.0 * B * n * Wo if mode in (1, 2) else 0)
+    name = {0: "multiply_log", 1: "multiply_max", 2: "multiply_sample", 3: "multiply"}[mode]
+    if sfx:
+        name += ", %s bands" % str(dtype).replace("torch.", "")
     report("banded %s fwd+bwd (B=%d,n=%d,lu=ld=%d)%s" % (name, B, n, lu, "" if pad is None else ", last %d rows of a = %g" % (pad[1], pad[0])),
            mf + mb, 6 * pairs, fb + bb,
            {"ms_fwd": round(mf, 4), "ms_bwd": round(mb, 4),
@@ -368,8 +378,11 @@ def main():
         dense_sample(lib, dev, 64, 512, 512, 512, r)
         dense_sample(lib, dev, 16, 512, 1024, 512, r)  # K beyond the matrix-core sweep's 992
     if "banded" in want:
-        for mode in (3, 0, 1):
+        for mode in (3, 0, 1, 2):
             banded(lib, dev, 64, 4096, 32, 32, mode, r)
+        for dt in (torch.float16, torch.bfloat16):
+            for mode in (3, 0, 1):
+                banded(lib, dev, 64, 4096, 32, 32, mode, r, dtype=dt)
     if "widths" in want:
         for lu in (2, 4, 8, 16, 24, 32, 40):
             for mode in (3, 0, 1):
