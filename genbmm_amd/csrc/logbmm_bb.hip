@@ -28,6 +28,7 @@
 //    alpha + beta - out is beyond 40 ln 2 or not finite (a factor could underflow against a
 //    term that matters) is flagged by the pass that forms H and redone by the exact kernels,
 //    which run behind the factored ones on the flagged items only.
+#include <algorithm>
 #include <type_traits>
 
 #include "logbmm_mfma.h"
@@ -48,8 +49,25 @@ struct BB {
   int M, K, N;
 };
 
+// Workgroup blocks of a pass: launched one per workgroup (numbered so that an item's workgroups share
+// an XCD), or - the pass over flagged items only, which usually finds none - walked by a small
+// grid in strides: tens of thousands of workgroups that exit at once still cost 60 us a launch.
+constexpr int kBBOnlyGrid = 2048;
+template <class F>
+__device__ __forceinline__ void bb_blocks(const BB& p, long nblocks, F&& f) {
+  if (p.only == nullptr) {
+    f((long)xcd_renumber(blockIdx.x, gridDim.x));
+    return;
+  }
+  for (long blk = blockIdx.x; blk < nblocks; blk += gridDim.x) f(blk);
+}
+inline dim3 bb_grid(const BB& p, long nblocks) {
+  return dim3((unsigned)(p.only ? std::min<long>(nblocks, kBBOnlyGrid) : nblocks));
+}
+
 __global__ __launch_bounds__(256) void k_log_bwdbwd_t(const BB p, long total) {
-  const long e = (long)xcd_renumber(blockIdx.x, gridDim.x) * 256 + threadIdx.x;  // an item's workgroups on one XCD
+  bb_blocks(p, (total + 255) / 256, [&](long blk) __attribute__((always_inline)) {
+  const long e = blk * 256 + threadIdx.x;
   if (e >= total) return;
   const int n = (int)(e % p.N);
   const long bm = e / p.N;  // batch*M + m
@@ -68,6 +86,7 @@ __global__ __launch_bounds__(256) void k_log_bwdbwd_t(const BB p, long total) {
   }
   p.tt[e] = t;
   if constexpr (!kElemF32) p.gg[e] = to_elem<elem_t>(t);
+  });
 }
 
 // grad_a: a wave per row (batch, m), its lanes along n - the one axis on which b, u_b, out, g and
@@ -76,8 +95,9 @@ __global__ __launch_bounds__(256) void k_log_bwdbwd_t(const BB p, long total) {
 // partial sums are added across the wave and 64 finished cells are written at once.
 constexpr int kBBChunks = 4;  // n chunks of 64 a lane keeps in registers
 __global__ __launch_bounds__(256) void k_log_bwdbwd_a(const BB p, long rows) {
+  bb_blocks(p, (rows + 3) / 4, [&](long blk) __attribute__((always_inline)) {
   const int lane = threadIdx.x & 63;
-  const long bm = (long)xcd_renumber(blockIdx.x, gridDim.x) * 4 + (threadIdx.x >> 6);
+  const long bm = blk * 4 + (threadIdx.x >> 6);
   if (bm >= rows) return;
   const long batch = bm / p.M;
   if (p.only && !p.only[batch]) return;
@@ -130,10 +150,12 @@ __global__ __launch_bounds__(256) void k_log_bwdbwd_a(const BB p, long rows) {
       if (k0 + lane <= k) p.ga[bm * K + k0 + lane] = to_elem<elem_t>(mine);
     }
   }
+  });
 }
 
 __global__ __launch_bounds__(256) void k_log_bwdbwd_b(const BB p, long total) {
-  const long e = (long)xcd_renumber(blockIdx.x, gridDim.x) * 256 + threadIdx.x;  // an item's workgroups on one XCD
+  bb_blocks(p, (total + 255) / 256, [&](long blk) __attribute__((always_inline)) {
+  const long e = blk * 256 + threadIdx.x;
   if (e >= total) return;
   const int n = (int)(e % p.N);
   const long bk = e / p.N;  // batch*K + k
@@ -155,10 +177,11 @@ __global__ __launch_bounds__(256) void k_log_bwdbwd_b(const BB p, long total) {
     acc = __builtin_fmaf((float)gcol[mn] * pr, w, acc);
   }
   p.gb[e] = to_elem<elem_t>(acc);
+  });
 }
 
 int launch_exact(const BB& p, int B, hipStream_t s) {
-  auto blocks = [](long total) { return dim3((unsigned)((total + 255) / 256)); };
+  auto blocks = [&](long total) { return bb_grid(p, (total + 255) / 256); };
   const long tmn = (long)B * p.M * p.N, tmk = (long)B * p.M * p.K, tkn = (long)B * p.K * p.N;
   if (tmn > 0) {
     hipLaunchKernelGGL(k_log_bwdbwd_t, blocks(tmn), dim3(256), 0, s, p, tmn);
@@ -166,7 +189,7 @@ int launch_exact(const BB& p, int B, hipStream_t s) {
   }
   if (tmk > 0) {
     const long rows = (long)B * p.M;  // four rows per workgroup
-    hipLaunchKernelGGL(k_log_bwdbwd_a, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, p, rows);
+    hipLaunchKernelGGL(k_log_bwdbwd_a, bb_grid(p, (rows + 3) / 4), dim3(256), 0, s, p, rows);
     if (int e = launch_status()) return e;
   }
   if (tkn > 0) {
@@ -219,6 +242,14 @@ inline size_t bb_ws_floats(int B, int M, int K, int N, BBWs* w, float* base) {
   return off;
 }
 
+// The three passes move four cells per lane and instruction (the padded extents are multiples of
+// 128; rows of the caller's tensors start at any element, which the loads take).
+__device__ __forceinline__ float4 exp4_st(float4 v, float m) {
+  return make_float4(exp_st(v.x - m), exp_st(v.y - m), exp_st(v.z - m), exp_st(v.w - m));
+}
+__device__ __forceinline__ float4 mul4(float4 a, float4 b) { return make_float4(a.x * b.x, a.y * b.y, a.z * b.z, a.w * b.w); }
+__device__ __forceinline__ float max4(float m, float4 v) { return fmaxf(fmaxf(m, fmaxf(v.x, v.y)), fmaxf(v.z, v.w)); }
+
 // alpha, EA, X: a wave per padded row (b, mp); rows and columns of the padding hold zeros.
 __global__ __launch_bounds__(256) void k_bb_prep_a(const elem_t* __restrict__ a, const elem_t* __restrict__ ua,
                                                    float* __restrict__ alpha, float* __restrict__ ea,
@@ -232,80 +263,108 @@ __global__ __launch_bounds__(256) void k_bb_prep_a(const elem_t* __restrict__ a,
   if (row < (rows / Mp) && lane == 0) flags[row] = 0;  // (rows / Mp = B words, cleared by the first B waves)
   float* er = ea + row * Kp;
   float* xr = x + row * Kp;
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
   if (m >= M) {
-    for (int k = lane; k < Kp; k += 64) { er[k] = 0.f; xr[k] = 0.f; }
+    for (int k = lane * 4; k < Kp; k += 256) { st4(er + k, zero); st4(xr + k, zero); }
     if (lane == 0) alpha[row] = 0.f;
     return;
   }
   const elem_t* ar = a + (batch * M + m) * K;
   const elem_t* ur = ua ? ua + (batch * M + m) * K : nullptr;
   float mx = -INFINITY;
-  for (int k = lane; k < K; k += 64) mx = fmaxf(mx, (float)ar[k]);
+  for (int k = lane * 4; k < K; k += 256) mx = max4(mx, ld4m(ar + k, K - k, -INFINITY));
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
   if (lane == 0) alpha[row] = mx;
-  for (int k = lane; k < Kp; k += 64) {
-    const float e = k < K ? exp_st((float)ar[k] - mx) : 0.f;
-    er[k] = e;
-    xr[k] = (ur && k < K) ? e * (float)ur[k] : 0.f;
+  for (int k = lane * 4; k < Kp; k += 256) {
+    // (the fill -inf gives exp = 0 in the padding; a row of -inf has mx = -inf and NaN here, and is
+    //  flagged by the pass that forms H)
+    const float4 e = k < K ? exp4_st(ld4m(ar + k, K - k, -INFINITY), mx) : zero;
+    st4(er + k, e);
+    st4(xr + k, (ur && k < K) ? mul4(e, ld4m(ur + k, K - k, 0.f)) : zero);
   }
 }
 
-// beta, EB, Y: a workgroup per (batch item, 64 columns); four waves split the rows of b.
+// beta, EB, Y: a workgroup per (batch item, 64 columns): 16 lanes x 4 columns across, the 16 lane
+// groups of the four waves split the rows of b.
 __global__ __launch_bounds__(256) void k_bb_prep_b(const elem_t* __restrict__ b, const elem_t* __restrict__ ub,
                                                    float* __restrict__ beta, float* __restrict__ eb,
                                                    float* __restrict__ y, int K, int N, int Kp, int Np) {
-  __shared__ float part[4][64];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __shared__ float part[16][64];
+  const int cq = threadIdx.x & 15, rg = threadIdx.x >> 4;
   const int cblocks = Np / 64;
   const long batch = blockIdx.x / cblocks;
-  const int n = (blockIdx.x - batch * cblocks) * 64 + lane;
-  const bool live = n < N;
-  const elem_t* bc = b + batch * K * N + (live ? n : 0);
-  const elem_t* uc = ub ? ub + batch * K * N + (live ? n : 0) : nullptr;
-  float mx = -INFINITY;
-  if (live)
-    for (int k = wave; k < K; k += 4) mx = fmaxf(mx, (float)bc[(long)k * N]);
-  part[wave][lane] = mx;
+  const int n = (blockIdx.x - batch * cblocks) * 64 + cq * 4;
+  const int cnt = N - n;  // live columns of this lane's four (<= 0: none)
+  const elem_t* bc = b + batch * K * N + (cnt > 0 ? n : 0);
+  const elem_t* uc = ub ? ub + batch * K * N + (cnt > 0 ? n : 0) : nullptr;
+  float4 mx = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+  for (int k = rg; k < K; k += 16) {
+    const float4 v = ld4m(bc + (long)k * N, cnt, -INFINITY);
+    mx = make_float4(fmaxf(mx.x, v.x), fmaxf(mx.y, v.y), fmaxf(mx.z, v.z), fmaxf(mx.w, v.w));
+  }
+  st4a(&part[rg][cq * 4], mx);
   __syncthreads();
-  mx = fmaxf(fmaxf(part[0][lane], part[1][lane]), fmaxf(part[2][lane], part[3][lane]));
-  if (wave == 0) beta[batch * Np + n] = live ? mx : 0.f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const float4 v = ld4a(&part[r][cq * 4]);
+    mx = make_float4(fmaxf(mx.x, v.x), fmaxf(mx.y, v.y), fmaxf(mx.z, v.z), fmaxf(mx.w, v.w));
+  }
+  if (rg == 0)
+    st4(beta + batch * Np + n, make_float4(cnt > 0 ? mx.x : 0.f, cnt > 1 ? mx.y : 0.f, cnt > 2 ? mx.z : 0.f,
+                                           cnt > 3 ? mx.w : 0.f));
   float* ec = eb + batch * Kp * Np + n;
   float* yc = y + batch * Kp * Np + n;
-  for (int k = wave; k < Kp; k += 4) {
-    const bool in = live && k < K;
-    const float e = in ? exp_st((float)bc[(long)k * N] - mx) : 0.f;
-    ec[(long)k * Np] = e;
-    yc[(long)k * Np] = (uc && in) ? e * (float)uc[(long)k * N] : 0.f;
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int k = rg; k < Kp; k += 16) {
+    const bool in = cnt > 0 && k < K;
+    float4 e = zero;
+    if (in) {
+      const float4 v = ld4m(bc + (long)k * N, cnt, -INFINITY);
+      e = make_float4(exp_st(v.x - mx.x), cnt > 1 ? exp_st(v.y - mx.y) : 0.f, cnt > 2 ? exp_st(v.z - mx.z) : 0.f,
+                      cnt > 3 ? exp_st(v.w - mx.w) : 0.f);
+    }
+    st4(ec + (long)k * Np, e);
+    st4(yc + (long)k * Np, (uc && in) ? mul4(e, ld4m(uc + (long)k * N, cnt, 0.f)) : zero);
   }
 }
 
-// R = exp(alpha + beta - out), H = g R over the padded (Mp, Np) grid (zeros in the padding); an
-// item with a cell beyond the guard is flagged.
+// R = exp(alpha + beta - out), H = g R over the padded (Mp, Np) grid (zeros in the padding), four
+// cells of a row per lane; an item with a cell beyond the guard is flagged.
 __global__ __launch_bounds__(256) void k_bb_prep_h(const elem_t* __restrict__ out, const elem_t* __restrict__ g,
                                                    const float* __restrict__ alpha, const float* __restrict__ beta,
                                                    float* __restrict__ r, float* __restrict__ h,
                                                    int* __restrict__ flags, int M, int N, int Mp, int Np,
-                                                   long total) {
-  const long e = (long)blockIdx.x * 256 + threadIdx.x;
-  if (e >= total) return;
-  const int n = (int)(e % Np);
-  const long bm = e / Np;
+                                                   long quads) {
+  const long q = (long)blockIdx.x * 256 + threadIdx.x;
+  if (q >= quads) return;
+  const int nq = Np / 4;
+  const int n = (int)(q % nq) * 4;
+  const long bm = q / nq;
   const long batch = bm / Mp;
   const int m = (int)(bm - batch * Mp);
-  float rv = 0.f, hv = 0.f;
-  if (m < M && n < N) {
+  float rv[4] = {0.f, 0.f, 0.f, 0.f}, hv[4] = {0.f, 0.f, 0.f, 0.f};
+  const int cnt = N - n;
+  if (m < M && cnt > 0) {
     const long src = (batch * M + m) * N + n;
-    const float al = alpha[bm], be = beta[batch * Np + n];
-    const float ex = al + be - (float)out[src];
+    const float al = alpha[bm];
+    const float4 be4 = ld4(beta + batch * Np + n), o4 = ld4m(out + src, cnt, 0.f), g4 = ld4m(g + src, cnt, 0.f);
+    const float be[4] = {be4.x, be4.y, be4.z, be4.w}, o[4] = {o4.x, o4.y, o4.z, o4.w}, gv[4] = {g4.x, g4.y, g4.z, g4.w};
     const float lim = kMfmaGuardBits * kLn2 + 1e-3f;
-    // (a negated comparison: NaN and +inf fail it; alpha, beta not finite make ex not finite or NaN)
-    if (!(ex <= lim) || !(al > -INFINITY) || !(be > -INFINITY)) flags[batch] = 1;
-    rv = exp_st(ex);
-    hv = (float)g[src] * rv;
+    bool bad = !(al > -INFINITY);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i < cnt) {
+        const float ex = al + be[i] - o[i];
+        // (a negated comparison: NaN and +inf fail it; alpha, beta not finite make ex not finite or NaN)
+        bad = bad || !(ex <= lim) || !(be[i] > -INFINITY);
+        rv[i] = exp_st(ex);
+        hv[i] = gv[i] * rv[i];
+      }
+    if (bad) flags[batch] = 1;
   }
-  r[e] = rv;
-  h[e] = hv;
+  st4(r + bm * Np + n, make_float4(rv[0], rv[1], rv[2], rv[3]));
+  st4(h + bm * Np + n, make_float4(hv[0], hv[1], hv[2], hv[3]));
 }
 
 // One tile of C = P1 Q1 (+ P2 Q2) and its epilogue.  Operands are padded workspace arrays:
@@ -450,9 +509,9 @@ int bwdbwd_factored(const BB& p, const BBWs& w, int B, hipStream_t s) {
                        w.x, w.flags, M, K, Mp, Kp, rows);
     hipLaunchKernelGGL(k_bb_prep_b, dim3((unsigned)(B * (Np / 64))), dim3(256), 0, s, p.b, p.ub, w.beta, w.eb, w.y,
                        K, N, Kp, Np);
-    const long cells = (long)B * Mp * Np;
-    hipLaunchKernelGGL(k_bb_prep_h, dim3((unsigned)((cells + 255) / 256)), dim3(256), 0, s, p.out, p.g, w.alpha,
-                       w.beta, w.r, w.h, w.flags, M, N, Mp, Np, cells);
+    const long quads = (long)B * Mp * (Np / 4);
+    hipLaunchKernelGGL(k_bb_prep_h, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, p.out, p.g, w.alpha,
+                       w.beta, w.r, w.h, w.flags, M, N, Mp, Np, quads);
     if (int e = launch_status()) return e;
   }
   const bool has_a = p.ua != nullptr, has_b = p.ub != nullptr;
