@@ -23,7 +23,7 @@ FP32_VALU_PEAK_TFLOPS = 157.3  # MI355X FP32 peak (vector with packed FMA = fp32
 # HBM bytes per launch of the dominant kernel (k_log_bwd_mfma_both_lean): rocprofv3 --pmc
 # FETCH_SIZE + WRITE_SIZE in KiB per dispatch, scale factor 1.00 against a known-size copy in
 # the same run; the two figures are those of profiles/logbmm_headline_B64_512.md.
-DOMINANT_FETCH_KIB, DOMINANT_WRITE_KIB = 243860, 131070
+DOMINANT_FETCH_KIB, DOMINANT_WRITE_KIB = 240100, 131072
 DOMINANT_TRAFFIC_BYTES = (DOMINANT_FETCH_KIB + DOMINANT_WRITE_KIB) * 1024
 
 
@@ -73,6 +73,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-verify", action="store_true", help="skip the float64 check of all items before timing")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU only; every batch item is independent, so more GPUs "
@@ -100,6 +101,29 @@ def main():
 
     def bwd():  # both gradients in one call, like the reference's _genbmm.backward
         _lib.check(lib.genbmm_logbmm_bwd(p(a), p(b), p(out), p(g), p(stats), p(ga), p(gb), B, M, K, N, stream), "bwd")
+
+    # Before anything is timed: the buffers the timed steps write are checked, every batch item,
+    # against float64 torch on the device (the broadcast form of README.md:31-35 and its autograd
+    # gradients, an item at a time - 1 GB of float64 terms each).  A wrong kernel ends the run here.
+    checked = None
+    if not args.no_verify:
+        fwd(); bwd()
+        worst = [0.0, 0.0, 0.0]
+        for i in range(B):
+            a64, b64 = a[i].double().requires_grad_(True), b[i].double().requires_grad_(True)
+            ref = torch.logsumexp(a64[:, :, None] + b64[None, :, :], dim=1)
+            ra, rb = torch.autograd.grad(ref, (a64, b64), g[i].double())
+            for j, (got, want) in enumerate(((out[i], ref.detach()), (ga[i], ra), (gb[i], rb))):
+                err = float(((got.double() - want).abs() / (1e-5 + 1e-5 * want.abs())).max())
+                worst[j] = max(worst[j], err)
+            del a64, b64, ref, ra, rb
+        if not max(worst) <= 1.0:
+            sys.exit("bench.py: results differ from float64 beyond rtol 1e-5 + atol 1e-5 (out, grad_a, grad_b: "
+                     "%s x the tolerance)" % worst)
+        checked = {"items": B, "reference": "float64 torch broadcast logsumexp + autograd on the device",
+                   "rtol": 1e-5, "atol": 1e-5,
+                   "worst_error_over_tolerance": {"out": round(worst[0], 4), "grad_a": round(worst[1], 4),
+                                                  "grad_b": round(worst[2], 4)}}
 
     for _ in range(args.warmup):
         fwd(); bwd()
@@ -136,13 +160,14 @@ def main():
     }
     # and, outside the timed region and of no influence on `value`: the step time once settled
     # (60 more steps straight behind the timed ones, the last 20 of them averaged)
-    more = [torch.cuda.Event(enable_timing=True) for _ in range(61)]
-    more[0].record()
-    for i in range(60):
-        fwd(); bwd()
-        more[i + 1].record()
+    more = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(60)]
+    for e in more:
+        e[0].record(); fwd()
+        e[1].record(); bwd()
+        e[2].record()
     torch.cuda.synchronize()
-    trend["ms_step_settled"] = round(more[40].elapsed_time(more[60]) / 20, 4)
+    trend["ms_step_settled"] = round(more[40][0].elapsed_time(more[59][2]) / 20, 4)
+    trend["ms_bwd_settled"] = mean([(e[1], e[2]) for e in more[40:]])
     ms_step = dt * 1e3 / args.steps
     bmkn = float(B) * M * K * N
     value = 6.0 * bmkn / (ms_step * 1e-3) / 1e9
@@ -197,6 +222,7 @@ def main():
         "ms_fwd": round(ms_fwd, 4),
         "ms_bwd": round(ms_bwd, 4),
         "step_time_trend": trend,
+        "verified_before_timing": checked,
         "ms_per_step_autograd_api": round(ms_autograd, 4),
         "roofline": roofline,
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(torch),

@@ -47,28 +47,52 @@ struct BB {
   float* tt;
   const int* only;
   int M, K, N;
+  int B;
 };
 
-// Workgroup blocks of a pass: launched one per workgroup (numbered so that an item's workgroups share
-// an XCD), or - the pass over flagged items only, which usually finds none - walked by a small
-// grid in strides: tens of thousands of workgroups that exit at once still cost 60 us a launch.
+// The blocks of a pass.  A block is `per_block` consecutive units (cells or rows) starting at `base`
+// and ending before `limit`; f(base, limit) works on one.  Without `only`: one block per workgroup
+// over all units (numbered so that an item's workgroups share an XCD).  With it - the pass over
+// flagged items, which usually finds none - a small grid reads the flags 64 at a time; its workgroups
+// form groups of one item's blocks (or one group that strides, for items of more blocks than the
+// grid), and the flagged items go to the groups in turn: tens of thousands of workgroups that look
+// up a flag and exit cost 60 us a launch, this costs 2.
 constexpr int kBBOnlyGrid = 2048;
-template <class F>
-__device__ __forceinline__ void bb_blocks(const BB& p, long nblocks, F&& f) {
-  if (p.only == nullptr) {
-    f((long)xcd_renumber(blockIdx.x, gridDim.x));
+template <bool ONLY, class F>
+__device__ __forceinline__ void bb_blocks(const BB& p, long total, long per_item, int per_block, F&& f) {
+  if constexpr (!ONLY) {
+    f((long)xcd_renumber(blockIdx.x, gridDim.x) * per_block, total);
     return;
   }
-  for (long blk = blockIdx.x; blk < nblocks; blk += gridDim.x) f(blk);
+  const int lane = threadIdx.x & 63;
+  const long bpi = (per_item + per_block - 1) / per_block;  // blocks per item
+  const bool fits = bpi <= (long)gridDim.x;
+  const long groups = fits ? (long)gridDim.x / bpi : 1;
+  const long grp = fits ? (long)blockIdx.x / bpi : 0;
+  if (grp >= groups) return;
+  const long first = fits ? (long)blockIdx.x - grp * bpi : (long)blockIdx.x;
+  const long stride = fits ? bpi : (long)gridDim.x;
+  long seen = 0;
+  for (int b0 = 0; b0 < p.B; b0 += 64) {
+    unsigned long long live = __ballot(b0 + lane < p.B && p.only[b0 + lane] != 0);
+    while (live) {
+      const long batch = b0 + __builtin_ctzll(live);
+      live &= live - 1;
+      if (seen++ % groups != grp) continue;
+      for (long u = first * per_block; u < per_item; u += stride * per_block)
+        f(batch * per_item + u, (batch + 1) * per_item);
+    }
+  }
 }
 inline dim3 bb_grid(const BB& p, long nblocks) {
   return dim3((unsigned)(p.only ? std::min<long>(nblocks, kBBOnlyGrid) : nblocks));
 }
 
+template <bool ONLY>
 __global__ __launch_bounds__(256) void k_log_bwdbwd_t(const BB p, long total) {
-  bb_blocks(p, (total + 255) / 256, [&](long blk) __attribute__((always_inline)) {
-  const long e = blk * 256 + threadIdx.x;
-  if (e >= total) return;
+  bb_blocks<ONLY>(p, total, (long)p.M * p.N, 256, [&](long base, long limit) __attribute__((always_inline)) {
+  const long e = base + threadIdx.x;
+  if (e >= limit) return;
   const int n = (int)(e % p.N);
   const long bm = e / p.N;  // batch*M + m
   const long batch = bm / p.M;
@@ -94,11 +118,12 @@ __global__ __launch_bounds__(256) void k_log_bwdbwd_t(const BB p, long total) {
 // line per lane).  The row's out, g and t stay in registers for N <= 256; per k the lanes'
 // partial sums are added across the wave and 64 finished cells are written at once.
 constexpr int kBBChunks = 4;  // n chunks of 64 a lane keeps in registers
+template <bool ONLY>
 __global__ __launch_bounds__(256) void k_log_bwdbwd_a(const BB p, long rows) {
-  bb_blocks(p, (rows + 3) / 4, [&](long blk) __attribute__((always_inline)) {
+  bb_blocks<ONLY>(p, rows, (long)p.M, 4, [&](long base, long limit) __attribute__((always_inline)) {
   const int lane = threadIdx.x & 63;
-  const long bm = blk * 4 + (threadIdx.x >> 6);
-  if (bm >= rows) return;
+  const long bm = base + (threadIdx.x >> 6);
+  if (bm >= limit) return;
   const long batch = bm / p.M;
   if (p.only && !p.only[batch]) return;
   const int K = p.K, N = p.N;
@@ -153,10 +178,11 @@ __global__ __launch_bounds__(256) void k_log_bwdbwd_a(const BB p, long rows) {
   });
 }
 
+template <bool ONLY>
 __global__ __launch_bounds__(256) void k_log_bwdbwd_b(const BB p, long total) {
-  bb_blocks(p, (total + 255) / 256, [&](long blk) __attribute__((always_inline)) {
-  const long e = blk * 256 + threadIdx.x;
-  if (e >= total) return;
+  bb_blocks<ONLY>(p, total, (long)p.K * p.N, 256, [&](long base, long limit) __attribute__((always_inline)) {
+  const long e = base + threadIdx.x;
+  if (e >= limit) return;
   const int n = (int)(e % p.N);
   const long bk = e / p.N;  // batch*K + k
   const long batch = bk / p.K;
@@ -184,16 +210,17 @@ int launch_exact(const BB& p, int B, hipStream_t s) {
   auto blocks = [&](long total) { return bb_grid(p, (total + 255) / 256); };
   const long tmn = (long)B * p.M * p.N, tmk = (long)B * p.M * p.K, tkn = (long)B * p.K * p.N;
   if (tmn > 0) {
-    hipLaunchKernelGGL(k_log_bwdbwd_t, blocks(tmn), dim3(256), 0, s, p, tmn);
+    hipLaunchKernelGGL(p.only ? k_log_bwdbwd_t<true> : k_log_bwdbwd_t<false>, blocks(tmn), dim3(256), 0, s, p, tmn);
     if (int e = launch_status()) return e;
   }
   if (tmk > 0) {
     const long rows = (long)B * p.M;  // four rows per workgroup
-    hipLaunchKernelGGL(k_log_bwdbwd_a, bb_grid(p, (rows + 3) / 4), dim3(256), 0, s, p, rows);
+    hipLaunchKernelGGL(p.only ? k_log_bwdbwd_a<true> : k_log_bwdbwd_a<false>, bb_grid(p, (rows + 3) / 4), dim3(256), 0, s,
+                       p, rows);
     if (int e = launch_status()) return e;
   }
   if (tkn > 0) {
-    hipLaunchKernelGGL(k_log_bwdbwd_b, blocks(tkn), dim3(256), 0, s, p, tkn);
+    hipLaunchKernelGGL(p.only ? k_log_bwdbwd_b<true> : k_log_bwdbwd_b<false>, blocks(tkn), dim3(256), 0, s, p, tkn);
     if (int e = launch_status()) return e;
   }
   return GENBMM_OK;
@@ -250,33 +277,38 @@ __device__ __forceinline__ float4 exp4_st(float4 v, float m) {
 __device__ __forceinline__ float4 mul4(float4 a, float4 b) { return make_float4(a.x * b.x, a.y * b.y, a.z * b.z, a.w * b.w); }
 __device__ __forceinline__ float max4(float m, float4 v) { return fmaxf(fmaxf(m, fmaxf(v.x, v.y)), fmaxf(v.z, v.w)); }
 
-// alpha, EA, X: a wave per padded row (b, mp); rows and columns of the padding hold zeros.
+// alpha, EA, X: a wave per padded row (b, mp) - half a wave where a row is 128 cells, 32 lanes' worth;
+// rows and columns of the padding hold zeros.
 __global__ __launch_bounds__(256) void k_bb_prep_a(const elem_t* __restrict__ a, const elem_t* __restrict__ ua,
                                                    float* __restrict__ alpha, float* __restrict__ ea,
                                                    float* __restrict__ x, int* __restrict__ flags, int M, int K,
                                                    int Mp, int Kp, long rows) {
-  const int lane = threadIdx.x & 63;
-  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lpr = Kp == 128 ? 32 : 64;  // lanes per row
+  const int lane = threadIdx.x & (lpr - 1);
+  const long row = ((long)blockIdx.x * 256 + threadIdx.x) / lpr;
   if (row >= rows) return;
   const long batch = row / Mp;
   const int m = (int)(row - batch * Mp);
-  if (row < (rows / Mp) && lane == 0) flags[row] = 0;  // (rows / Mp = B words, cleared by the first B waves)
+  if (row < (rows / Mp) && lane == 0) flags[row] = 0;  // (rows / Mp = B words, cleared by the first B rows)
   float* er = ea + row * Kp;
   float* xr = x + row * Kp;
   const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  const int step = lpr * 4;
   if (m >= M) {
-    for (int k = lane * 4; k < Kp; k += 256) { st4(er + k, zero); st4(xr + k, zero); }
+    for (int k = lane * 4; k < Kp; k += step) { st4(er + k, zero); st4(xr + k, zero); }
     if (lane == 0) alpha[row] = 0.f;
     return;
   }
   const elem_t* ar = a + (batch * M + m) * K;
   const elem_t* ur = ua ? ua + (batch * M + m) * K : nullptr;
   float mx = -INFINITY;
-  for (int k = lane * 4; k < K; k += 256) mx = max4(mx, ld4m(ar + k, K - k, -INFINITY));
+  for (int k = lane * 4; k < K; k += step) mx = max4(mx, ld4m(ar + k, K - k, -INFINITY));
+  // (the exchange stays within the row's own lanes, all of which are here)
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+  for (int off = 32; off > 0; off >>= 1)
+    if (off < lpr) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
   if (lane == 0) alpha[row] = mx;
-  for (int k = lane * 4; k < Kp; k += 256) {
+  for (int k = lane * 4; k < Kp; k += step) {
     // (the fill -inf gives exp = 0 in the padding; a row of -inf has mx = -inf and NaN here, and is
     //  flagged by the pass that forms H)
     const float4 e = k < K ? exp4_st(ld4m(ar + k, K - k, -INFINITY), mx) : zero;
@@ -505,7 +537,8 @@ int bwdbwd_factored(const BB& p, const BBWs& w, int B, hipStream_t s) {
   const int M = p.M, K = p.K, N = p.N, Mp = bb_pad(M), Kp = bb_pad(K), Np = bb_pad(N);
   {
     const long rows = (long)B * Mp;
-    hipLaunchKernelGGL(k_bb_prep_a, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, p.a, p.ua, w.alpha, w.ea,
+    const long per_wg = Kp == 128 ? 8 : 4;  // rows per workgroup: 32 or 64 lanes each
+    hipLaunchKernelGGL(k_bb_prep_a, dim3((unsigned)((rows + per_wg - 1) / per_wg)), dim3(256), 0, s, p.a, p.ua, w.alpha, w.ea,
                        w.x, w.flags, M, K, Mp, Kp, rows);
     hipLaunchKernelGGL(k_bb_prep_b, dim3((unsigned)(B * (Np / 64))), dim3(256), 0, s, p.b, p.ub, w.beta, w.eb, w.y,
                        K, N, Kp, Np);
@@ -573,7 +606,7 @@ int bwdbwd(const elem_t* a, const elem_t* b, const elem_t* out, const elem_t* g,
     if (!kElemF32 && missing(workspace, mn)) return GENBMM_E_NULLPTR;  // t must stay unrounded somewhere
   }
   hipStream_t s = (hipStream_t)stream;
-  BB p{a, b, out, g, u_a, u_b, grad_a, grad_b, grad_g, nullptr, nullptr, M, K, N};
+  BB p{a, b, out, g, u_a, u_b, grad_a, grad_b, grad_g, nullptr, nullptr, M, K, N, B};
   BBWs w{};
   if (workspace) bb_ws_floats(B, M, K, N, &w, workspace);
   if constexpr (kElemF32) p.tt = reinterpret_cast<float*>(grad_g);

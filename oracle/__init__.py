@@ -17,7 +17,11 @@ has no stored vectors for this path and cannot be built here (CUDA only), so
 there is no oracle/_ref; the band products are additionally pinned by vectors
 that the reference's own CPU loops produced (tests/golden/band_struct.npz).
 Parity unpinned: only the random stream of samplebmm (the reference draws from
-torch's CUDA generator); its decision rule and distribution are pinned.
+torch's CUDA generator); its decision rule and distribution are pinned.  The
+banded sample product has no reference function at all (the reference's band
+kernel has no sample mode): its restatement is the reference's dense sampling
+rule on a band cell's terms and is pinned through the dense sampling oracle on
+the equivalent dense operands, not against the reference.
 """
 import ctypes
 import os

@@ -459,6 +459,30 @@ def test_logbmm_double_backward_factored_guard(gpu):
         close(x[keep], y, rtol=1e-4, atol=2e-4)
 
 
+@pytest.mark.parametrize("B,M,K,N,flagged", [
+    (40, 64, 64, 64, list(range(0, 40, 3)) + [39]),   # many flagged items, several to a group of workgroups
+    (70, 128, 64, 64, [0, 63, 64, 69]),               # more than 64 items: two words of flags
+    (2, 768, 64, 768, [1]),                           # an item of more blocks than the walking grid has workgroups
+])
+def test_logbmm_double_backward_flagged_items_walk(gpu, B, M, K, N, flagged):
+    """The exact passes behind the factored form visit the flagged items only, a group of workgroups
+    per item: every flagged item comes out as the exact passes alone give it (bit for bit), every
+    other item within the factored form's tolerance."""
+    torch.manual_seed(B + M)
+    a, b = torch.randn(B, M, K, device=gpu), torch.randn(B, K, N, device=gpu)
+    g, ua, ub = torch.randn(B, M, N, device=gpu), torch.randn(B, M, K, device=gpu), torch.randn(B, K, N, device=gpu)
+    for i in flagged:              # rows whose maximum sits on a term that never meets a live one
+        a[i, ::2, 0] += 200.0
+        b[i, 0, :] -= 200.0
+    out = genbmm.logbmm(a, b)
+    got = _bwdbwd_abi(gpu, a, b, out, g, ua, ub, True)
+    exact = _bwdbwd_abi(gpu, a, b, out, g, ua, ub, False)
+    rest = [i for i in range(B) if i not in flagged]
+    for x, y in zip(got, exact):
+        assert torch.equal(x[flagged], y[flagged])
+        close(x[rest], y[rest], rtol=1e-4, atol=2e-4)
+
+
 def test_logbmm_double_backward_at_the_headline_shape(gpu):
     """(64, 512, 512, 512) through autograd with create_graph; three batch items against float64
     second-order autograd evaluated on the device."""
