@@ -34,6 +34,7 @@
 #include "log_bwd_tile.h"
 #include "logbmm_item.h"
 #include "logbmm_mfma.h"
+#include "logbmm_split.h"
 #include "logbmm_item32.h"
 #include "logbmm_self.h"
 #include "logbmm_ws.h"
@@ -54,7 +55,8 @@ __device__ __forceinline__ float exp_comp(float d) {
   const float hi = d * kLog2e;
   const float lo = __builtin_fmaf(d, kLog2e, -hi) + d * kLog2eLo;
   const float e = fast_exp2(hi);
-  return __builtin_fmaf(e, lo * kLn2, e);
+  // (d = -inf, a masked entry: hi - hi is NaN in `lo`; the result is the plain 0)
+  return hi == -INFINITY ? 0.f : __builtin_fmaf(e, lo * kLn2, e);
 }
 
 // ------------------------------------------------------------------ stats
@@ -578,9 +580,19 @@ constexpr int kFixupGrid = 1024;
 
 inline bool valid_path(int path) {
   return path == GENBMM_PATH_AUTO || path == GENBMM_PATH_EXACT || path == GENBMM_PATH_VALU ||
-         path == GENBMM_PATH_FACTORS;
+         path == GENBMM_PATH_FACTORS || path == GENBMM_PATH_MFMA32;
 }
-inline bool auto_path(int path) { return path == GENBMM_PATH_AUTO || path == GENBMM_PATH_FACTORS; }
+inline bool auto_path(int path) {
+  return path == GENBMM_PATH_AUTO || path == GENBMM_PATH_FACTORS || path == GENBMM_PATH_MFMA32;
+}
+// MFMA32: as AUTO, but the tiled matrix-core kernels always use the fp32 matrix instruction; under
+// AUTO, full-tile shapes run on the bf16 instruction with every factor in three parts (logbmm_split.h).
+inline bool split_path(int path) { return path == GENBMM_PATH_AUTO; }
+// dynamic LDS beyond 64 KB must be asked for
+template <class Kern>
+inline void allow_lds(Kern kern, int bytes) {
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
 
 // Layout of the caller's stats buffer: B*(M+N) shifts; one int flag per 32x32
 // tile of (M,N) (an upper bound on any forward launch's tile count); a header of
@@ -821,6 +833,51 @@ int launch_bwd_mfma_both(LogBwdArgs pa, LogBwdArgs pb, const float* stats, int B
   return launch_status();
 }
 
+// The bf16 three-part kernels (logbmm_split.h): full tiles only; the 256 x 256 tile (one
+// workgroup of sixteen waves per compute unit) when it fills the chip.
+template <class T>
+inline bool split_fits(int B, int out_r, int out_c, int red, bool fill_chip) {
+  if (out_r % T::TR != 0 || out_c % T::TC != 0 || red % kMS != 0) return false;
+  return !fill_chip || (int64_t)B * (out_r / T::TR) * (out_c / T::TC) >= 192;
+}
+template <class T>
+int launch_fwd_split(DenseArgs p, float* stats, int B, int M, int K, int N, hipStream_t s) {
+  p.M = M; p.K = K; p.N = N;
+  p.tiles_m = M / T::TR;
+  p.tiles_n = N / T::TC;
+  p.vec_a = (K % 4 == 0) && aligned16(p.a);
+  p.vec_b = (N % 4 == 0) && aligned16(p.b);
+  p.vec_o = (N % 4 == 0) && aligned16(p.out);
+  const int total = B * p.tiles_m * p.tiles_n;
+  int* flags = fwd_flags_of(stats, B, M, N);
+  constexpr int lds = 4 * split_lds_words<SplitT<T::TR, T::NT>, SplitS<T::TC, T::NT>>();
+  allow_lds(k_log_fwd_split<T>, lds);
+  hipLaunchKernelGGL(k_log_fwd_split<T>, dim3(total), dim3(T::NT), lds, s, p.a, p.b, p.out, stats, flags,
+                     prepared_of(stats, B, M, K, N).hdr, M, K, N, p.tiles_m, p.tiles_n);
+  if (int e = launch_status()) return e;
+  return launch_fwd_fixup<CfgWide, T::TR, T::TC>(p, flags, total, s);
+}
+template <class TA, class TB>
+int launch_bwd_split_both(LogBwdArgs pa, LogBwdArgs pb, const float* stats, int B, hipStream_t s) {
+  const int M = pa.M, K = pa.K, N = pa.N;
+  pa.tiles_r = M / TA::TR; pa.tiles_c = K / TA::TC;
+  pb.tiles_r = K / TB::TR; pb.tiles_c = N / TB::TC;
+  const int64_t ta = (int64_t)B * pa.tiles_r * pa.tiles_c, tb = (int64_t)B * pb.tiles_r * pb.tiles_c;
+  if (ta + tb > 0x7fffffffLL) return GENBMM_E_SHAPE;
+  const int* hdr = prepared_of(stats, B, M, K, N).hdr;
+  const int* ff = fwd_flags_of(stats, B, M, N);
+  constexpr int lds = split_bwd_lds_bytes<TA, TB>();
+  allow_lds(k_log_bwd_split_both<TA, TB>, lds);
+  hipLaunchKernelGGL((k_log_bwd_split_both<TA, TB>), dim3((unsigned)(ta + tb)), dim3(TA::NT), lds, s, pa.g,
+                     LeanSrc{pa.a, pa.b, pa.out, stats}, hdr, ff, pa.grad, pb.grad, M, K, N, pa.tiles_r, pa.tiles_c,
+                     pb.tiles_r, pb.tiles_c);
+  if (int e = launch_status()) return e;
+  hipLaunchKernelGGL((k_log_bwd_fixup_both<BCfgWide, TA::TR, TA::TC, TB::TR, TB::TC>),
+                     dim3((unsigned)std::min<int64_t>(ta + tb, kFixupGrid)), dim3(BCfgWide::NT), 0, s, pa, pb, hdr, ff,
+                     (int)ta, (int)tb, 0);
+  return launch_status();
+}
+
 // Which matrix-core tiling an output of out_r x out_c (reduction over red) gets:
 // 2 for the 256-wide tile (when the long side splits into 256s without extra
 // padding and there are tiles enough to give every compute unit two workgroups of
@@ -838,6 +895,7 @@ inline int mfma_kind(int path, int B, int out_r, int out_c, int red, bool long_c
 using MT128 = MTile<128, 128>;
 using MTWide = MTile<128, 256>;  // grad_a (m x k)
 using MTTall = MTile<256, 128>;  // forward (m x n; measured 1-2 % ahead of 128x256) and grad_b (k x n)
+using MTBig = MTile<256, 256>;   // sixteen waves, one workgroup per compute unit (the bf16 three-part kernels)
 
 template <bool GRAD_A>
 int run_bwd(const LogBwdArgs& p, const float* stats, int path, int B, hipStream_t s) {
@@ -912,7 +970,12 @@ int run_fwd(const elem_t* a, const elem_t* b, elem_t* out, float* stats, int B, 
   if (stats && K > 0 && path != GENBMM_PATH_EXACT) {
     const int64_t big_tiles = (int64_t)B * ceil_div(M, 128) * ceil_div(N, 128);
     switch (fwd_mfma_shape(B, M, K, N) ? mfma_kind(path, B, M, N, K, false) : 0) {
-      case 2: return launch_fwd_mfma<MTTall>(p, stats, B, M, K, N, keep, s);
+      case 2:
+        if (!keep && split_path(path)) {
+          if (split_fits<MTBig>(B, M, N, K, true)) return launch_fwd_split<MTBig>(p, stats, B, M, K, N, s);
+          if (split_fits<MTTall>(B, M, N, K, false)) return launch_fwd_split<MTTall>(p, stats, B, M, K, N, s);
+        }
+        return launch_fwd_mfma<MTTall>(p, stats, B, M, K, N, keep, s);
       case 1: return launch_fwd_mfma<MT128>(p, stats, B, M, K, N, keep, s);
       default: break;
     }
@@ -973,6 +1036,12 @@ int run_bwd_both(const elem_t* a, const elem_t* b, const elem_t* out, const elem
       pa.grad = grad_a;
       pb.grad = grad_b;
       const bool lean = path != GENBMM_PATH_FACTORS;
+      if (ka == 2 && lean && split_path(path)) {
+        if (split_fits<MTBig>(B, M, K, N, true) && split_fits<MTBig>(B, K, N, M, true))
+          return launch_bwd_split_both<MTBig, MTBig>(pa, pb, st, B, s);
+        if (split_fits<MTWide>(B, M, K, N, false) && split_fits<MTTall>(B, K, N, M, false))
+          return launch_bwd_split_both<MTWide, MTTall>(pa, pb, st, B, s);
+      }
       return ka == 2 ? launch_bwd_mfma_both<MTWide, MTTall>(pa, pb, st, B, s, lean)
                      : launch_bwd_mfma_both<MT128, MT128>(pa, pb, st, B, s, lean);
     }

@@ -1,0 +1,523 @@
+// Factored logbmm on the bf16 matrix instruction with fp32 accuracy: every staged factor
+// x (fp32) is cut into three bfloat16 parts h + m + l = x exactly (h = x rounded to bf16,
+// m = x - h rounded, l = the rest: 8 + 8 + 8 significant bits), and a product x y is taken
+// as the six partial products h h, h m, m h, m m, h l, l h on v_mfma_f32_32x32x16_bf16
+// (fp32 accumulate; bf16 x bf16 is exact in fp32).  What is left out - m l, l m, l l - is
+// below 2^-23 of x y, the size of one fp32 rounding of the product itself.  The
+// instruction does 16 reduction steps in the time the fp32 one (v_mfma_f32_32x32x2_f32)
+// needs for one, so six of them per 16 steps are 2.7 times less matrix-pipe time, and -
+// unlike the fp32 matrix instruction on this part - they run beside the vector ALU's work.
+//
+// Same tiles, guards, flags, epilogues and fix-up launches as the fp32 kernels of
+// logbmm_mfma.h (a 64 x 64 block per wave as 2 x 2 accumulators, whose layout is that of
+// the fp32 instruction; reduction in slabs of 16 through two LDS buffers); what differs is
+// the staged form and the inner loop.  Full tiles only (every extent a multiple of its
+// tile, the reduction of 16): other shapes stay on the fp32 instruction.
+//
+// LDS layouts, three planes (h, m, l) per operand, words of two bf16:
+//  * an operand whose source is [line][reduction] (reduction contiguous): plane[line][8
+//    words]; a lane stages four consecutive reduction steps of a line (one 8-byte store
+//    per plane) and reads the eight steps of its line that the instruction wants from it
+//    as one 16-byte load.
+//  * an operand whose source is [reduction][line]: plane[8 step pairs][lines + 8]; a lane
+//    stages a pair of reduction steps for LW consecutive lines (the pair shares a word;
+//    one store of LW words per plane) and reads its eight steps as four words a row apart.
+#pragma once
+
+#include "logbmm_mfma.h"
+
+namespace GENBMM_NS {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+
+// (x0, x1) rounded to bf16, x0 in the low half: one v_cvt_pk_bf16_f32
+__device__ __forceinline__ unsigned pk_bf16(float x0, float x1) {
+  floatx2 v;
+  v.x = x0; v.y = x1;
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2));
+}
+__device__ __forceinline__ float bf_lo(unsigned pk) { return __builtin_bit_cast(float, pk << 16); }
+__device__ __forceinline__ float bf_hi(unsigned pk) { return __builtin_bit_cast(float, pk & 0xffff0000u); }
+// h + m + l = x exactly, for both values of a pair
+__device__ __forceinline__ void split2(float x0, float x1, unsigned& h, unsigned& m, unsigned& l) {
+  h = pk_bf16(x0, x1);
+  const float r0 = x0 - bf_lo(h), r1 = x1 - bf_hi(h);
+  m = pk_bf16(r0, r1);
+  l = pk_bf16(r0 - bf_lo(m), r1 - bf_hi(m));
+}
+
+// source [line][reduction]
+template <int OUT, int NT>
+struct SplitT {
+  static constexpr int PLANE = OUT * 8;      // words
+  static constexpr int BUF = 3 * PLANE;
+  static constexpr int PER = OUT * 4 / NT;   // pieces (a line, four reduction steps) per thread
+  static_assert(PER >= 1 && OUT * 4 % NT == 0, "");
+  static __device__ __forceinline__ int line(int tid, int l) { return (tid >> 2) + l * (NT / 4); }
+  static __device__ __forceinline__ int quad(int tid) { return tid & 3; }
+  static __device__ __forceinline__ void put(unsigned* __restrict__ buf, int tid, int l, float4 v) {
+    unsigned h0, m0, l0, h1, m1, l1;
+    split2(v.x, v.y, h0, m0, l0);
+    split2(v.z, v.w, h1, m1, l1);
+    unsigned* p = buf + line(tid, l) * 8 + quad(tid) * 2;
+    uintx2 w;
+    w.x = h0; w.y = h1; *reinterpret_cast<uintx2*>(p) = w;
+    w.x = m0; w.y = m1; *reinterpret_cast<uintx2*>(p + PLANE) = w;
+    w.x = l0; w.y = l1; *reinterpret_cast<uintx2*>(p + 2 * PLANE) = w;
+  }
+  // the lane's operand of one 32-line block: line0 + lane % 32, reduction steps 8 (lane / 32) .. + 7
+  static __device__ __forceinline__ bf16x8 frag(const unsigned* __restrict__ buf, int plane, int line0, int lane) {
+    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4*>(buf + plane * PLANE + (line0 + (lane & 31)) * 8 +
+                                                                       (lane >> 5) * 4));
+  }
+};
+
+// source [reduction][line]
+template <int OUT, int NT>
+struct SplitS {
+  static constexpr int LD = OUT + 8;         // words per step pair (lanes 32.. read four rows on: other banks)
+  static constexpr int PLANE = 8 * LD;
+  static constexpr int BUF = 3 * PLANE;
+  static constexpr int LW = OUT * 8 / NT;    // lines per piece (a pair of reduction steps, LW lines); one piece per thread
+  static_assert(LW == 2 || LW == 4, "");
+  static constexpr int Q = OUT / LW;         // pieces per step pair
+  static __device__ __forceinline__ int pair(int tid) { return tid / Q; }          // reduction steps 2 pair, 2 pair + 1
+  static __device__ __forceinline__ int line0(int tid) { return (tid % Q) * LW; }
+  static __device__ __forceinline__ void put(unsigned* __restrict__ buf, int tid, const float (&even)[LW],
+                                             const float (&odd)[LW]) {
+    unsigned h[LW], m[LW], l[LW];
+#pragma unroll
+    for (int j = 0; j < LW; ++j) split2(even[j], odd[j], h[j], m[j], l[j]);
+    unsigned* p = buf + pair(tid) * LD + line0(tid);
+    if constexpr (LW == 4) {
+      uintx4 w;
+      w.x = h[0]; w.y = h[1]; w.z = h[2]; w.w = h[3]; *reinterpret_cast<uintx4*>(p) = w;
+      w.x = m[0]; w.y = m[1]; w.z = m[2]; w.w = m[3]; *reinterpret_cast<uintx4*>(p + PLANE) = w;
+      w.x = l[0]; w.y = l[1]; w.z = l[2]; w.w = l[3]; *reinterpret_cast<uintx4*>(p + 2 * PLANE) = w;
+    } else {
+      uintx2 w;
+      w.x = h[0]; w.y = h[1]; *reinterpret_cast<uintx2*>(p) = w;
+      w.x = m[0]; w.y = m[1]; *reinterpret_cast<uintx2*>(p + PLANE) = w;
+      w.x = l[0]; w.y = l[1]; *reinterpret_cast<uintx2*>(p + 2 * PLANE) = w;
+    }
+  }
+  static __device__ __forceinline__ bf16x8 frag(const unsigned* __restrict__ buf, int plane, int line0, int lane) {
+    const unsigned* p = buf + plane * PLANE + (lane >> 5) * 4 * LD + line0 + (lane & 31);
+    uintx4 w;
+    w.x = p[0]; w.y = p[LD]; w.z = p[2 * LD]; w.w = p[3 * LD];
+    return __builtin_bit_cast(bf16x8, w);
+  }
+};
+
+// LW consecutive elements as floats
+template <int LW>
+__device__ __forceinline__ void ldw(const elem_t* p, float (&v)[LW]) {
+  if constexpr (LW == 4) {
+    const float4 t = ld4(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  } else {
+    typedef elem_t e2u __attribute__((ext_vector_type(2), aligned(sizeof(elem_t))));
+    const e2u t = *reinterpret_cast<const e2u*>(p);
+    v[0] = (float)t.x; v[1] = (float)t.y;
+  }
+}
+
+__device__ __forceinline__ floatx16 mfma_bf16(bf16x8 a, bf16x8 b, floatx16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+// The six partial products of one staged slab, for the wave's 2 x 2 blocks.  Products of one
+// kind go to the four accumulators in turn (no instruction waits for the one before it);
+// the small ones first.
+template <class SR, class SC>
+__device__ __forceinline__ void split_slab(const unsigned* __restrict__ R, const unsigned* __restrict__ Cs, int wr0,
+                                           int wc0, int lane, floatx16 (&acc)[2][2]) {
+  // Operand registers are asked for a phase ahead of their products and given up after them
+  // (at most 40 of them live beside the 64 accumulators; the fences keep the compiler from
+  // asking for all twelve operands up front).
+  bf16x8 rh[2], ch[2], cl[2], rl[2], rm[2], cm[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    rh[i] = SR::frag(R, 0, wr0 + 32 * i, lane);
+    cl[i] = SC::frag(Cs, 2, wc0 + 32 * i, lane);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    ch[i] = SC::frag(Cs, 0, wc0 + 32 * i, lane);
+    rl[i] = SR::frag(R, 2, wr0 + 32 * i, lane);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+  for (int x = 0; x < 4; ++x) acc[x >> 1][x & 1] = mfma_bf16(rh[x >> 1], cl[x & 1], acc[x >> 1][x & 1]);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) cm[i] = SC::frag(Cs, 1, wc0 + 32 * i, lane);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int x = 0; x < 4; ++x) acc[x >> 1][x & 1] = mfma_bf16(rl[x >> 1], ch[x & 1], acc[x >> 1][x & 1]);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) rm[i] = SR::frag(R, 1, wr0 + 32 * i, lane);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int x = 0; x < 4; ++x) acc[x >> 1][x & 1] = mfma_bf16(rh[x >> 1], cm[x & 1], acc[x >> 1][x & 1]);
+#pragma unroll
+  for (int x = 0; x < 4; ++x) acc[x >> 1][x & 1] = mfma_bf16(rm[x >> 1], cm[x & 1], acc[x >> 1][x & 1]);
+#pragma unroll
+  for (int x = 0; x < 4; ++x) acc[x >> 1][x & 1] = mfma_bf16(rm[x >> 1], ch[x & 1], acc[x >> 1][x & 1]);
+#pragma unroll
+  for (int x = 0; x < 4; ++x) acc[x >> 1][x & 1] = mfma_bf16(rh[x >> 1], ch[x & 1], acc[x >> 1][x & 1]);
+  __builtin_amdgcn_s_setprio(0);
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+// LDS words of a kernel on tile T whose row operand is staged by SR and column operand by SC
+template <class SR, class SC>
+constexpr int split_lds_words() { return 2 * (SR::BUF + SC::BUF); }
+
+// ----------------------------------------------------------------- forward
+// rows <- EA from a[m][k] ([line][reduction]), columns <- EB from b[k][n] ([reduction][line]).
+// Leaves the maxima, the tile flags and the header (no factors), like k_log_fwd_mfma<T, false, false>.
+template <class T>
+__global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WPE, T::WPE)))
+void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b, elem_t* __restrict__ out,
+                     const float* __restrict__ stats, int* __restrict__ flags, int* __restrict__ ws_hdr, int M,
+                     int K, int N, int tiles_m, int tiles_n) {
+  constexpr int NT = T::NT;
+  using SA = SplitT<T::TR, NT>;
+  using SB = SplitS<T::TC, NT>;
+  constexpr int LW = SB::LW;
+  extern __shared__ __attribute__((aligned(16))) unsigned split_smem[];
+  static_assert(split_lds_words<SA, SB>() >= (NT / 64) * kStripFloats, "");
+  auto As = [&](int buf) __attribute__((always_inline)) { return split_smem + buf * SA::BUF; };
+  auto Bs = [&](int buf) __attribute__((always_inline)) { return split_smem + 2 * SA::BUF + buf * SB::BUF; };
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = (wave / T::WC) * 64, wn0 = (wave % T::WC) * 64;
+  const int per = tiles_m * tiles_n, tile = xcd_tile_id();
+  const int batch = tile / per, rem = tile - batch * per;
+  const int m0 = (rem / tiles_n) * T::TR, n0 = (rem % tiles_n) * T::TC;
+  const float* st = stats + (long)batch * (M + N);
+
+  const elem_t* pa[SA::PER];
+  float al[SA::PER];
+#pragma unroll
+  for (int l = 0; l < SA::PER; ++l) {
+    const int line = m0 + SA::line(tid, l);
+    pa[l] = a + ((long)batch * M + line) * K + SA::quad(tid) * 4;
+    al[l] = st[line];
+  }
+  const int bcol = n0 + SB::line0(tid);
+  const elem_t* pb = b + ((long)batch * K + 2 * SB::pair(tid)) * N + bcol;
+  float be[LW];
+#pragma unroll
+  for (int j = 0; j < LW; ++j) be[j] = st[M + bcol + j];
+  if (tile == 0 && tid == 0) {
+    ws_hdr[1] = T::TR;
+    ws_hdr[2] = T::TC;
+    ws_hdr[0] = kWsFast;
+  }
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int x = 0; x < 4; ++x)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[x >> 1][x & 1][i] = 0.f;
+
+  const int slabs = K / kMS;
+  float4 ra[SA::PER];
+  float rbe[LW], rbo[LW];
+  auto load = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int l = 0; l < SA::PER; ++l) {
+      ra[l] = ld4(pa[l]);
+      pa[l] += kMS;
+    }
+    ldw<LW>(pb, rbe);
+    ldw<LW>(pb + N, rbo);
+    pb += (long)kMS * N;
+  };
+  auto stage = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int l = 0; l < SA::PER; ++l) SA::put(As(buf), tid, l, exp4(ra[l], al[l]));
+    float ee[LW], eo[LW];
+#pragma unroll
+    for (int j = 0; j < LW; ++j) {
+      ee[j] = exp_st(rbe[j] - be[j]);
+      eo[j] = exp_st(rbo[j] - be[j]);
+    }
+    SB::put(Bs(buf), tid, ee, eo);
+  };
+
+  load();
+  stage(0);
+  __syncthreads();
+  for (int s = 0; s < slabs; ++s) {
+    const bool more = s + 1 < slabs;
+    if (more) load();
+    split_slab<SA, SB>(As(s & 1), Bs(s & 1), wm0, wn0, lane, acc);
+    if (more) stage((s + 1) & 1);
+    __syncthreads();
+  }
+
+  // guard (as k_log_fwd_mfma): S >= 2^-40 and finite; every shift finite and not below the floor;
+  // no shift below -30 opposite a row or column at the floor
+  const float thr = fast_exp2(-kMfmaGuardBits);
+  int bad = 0;
+#pragma unroll
+  for (int x = 0; x < 4; ++x)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float s = acc[x >> 1][x & 1][i];
+      if (!((s >= thr) && (s < INFINITY))) bad = 1;
+    }
+  static_assert(T::TR + T::TC <= NT, "one shift per thread");
+  int low = 0, neg = 0;  // bit 0: of a row, bit 1: of a column
+  if (tid < T::TR + T::TC) {
+    const bool row = tid < T::TR;
+    const float sh = row ? st[m0 + tid] : st[M + n0 + tid - T::TR];
+    if (!((sh >= kFloor) && (sh < INFINITY))) bad = 1;
+    if (sh <= 0.45f * kFloor) low = row ? 1 : 2;
+    if (sh < -30.f) neg = row ? 1 : 2;
+  }
+  const int row_low = __syncthreads_or(low & 1), col_low = __syncthreads_or(low & 2);
+  if (row_low | col_low) {  // uniform, and rare
+    const int row_neg = __syncthreads_or(neg & 1), col_neg = __syncthreads_or(neg & 2);
+    if ((row_low && col_neg) || (col_low && row_neg)) bad = 1;
+  }
+  bad = __syncthreads_or(bad);  // also: every wave is done with the staging buffers
+  if (tid == 0) flags[tile] = bad;
+  if (bad) return;  // the fix-up launch recomputes this tile
+
+  // out = log S + alpha + beta, written row-wise
+  const int lr = lane >> 4, lc = (lane & 15) * 4;
+  const float4 be4 = ld4(st + M + n0 + wn0 + lc);
+  const float* alw = st + m0 + wm0 + lr;
+  const long ubase = ((long)batch * M + m0 + wm0) * N + n0 + wn0;
+  const int voff = lr * N + lc;
+  acc_rows(acc, reinterpret_cast<float*>(split_smem) + wave * kStripFloats, lane, [](int) {},
+           [&](int q, int t, float4 sv) __attribute__((always_inline)) {
+             const int ru = 16 * q + 4 * t;
+             const float alr = alw[ru];
+             const float4 ov = make_float4(__builtin_fmaf(fast_log2(sv.x), kLn2, alr + be4.x),
+                                           __builtin_fmaf(fast_log2(sv.y), kLn2, alr + be4.y),
+                                           __builtin_fmaf(fast_log2(sv.z), kLn2, alr + be4.z),
+                                           __builtin_fmaf(fast_log2(sv.w), kLn2, alr + be4.w));
+             st4(out + ubase + (long)ru * N + voff, ov);
+           });
+}
+
+// ---------------------------------------------------------------- backward
+// Operands formed from a, b, out, g and the maxima while they are staged (as
+// log_bwd_mfma_tile_lean): EA = exp(a - alpha), EB = exp(b - beta), H = g exp(alpha + beta - out).
+// GRAD_A: tile (m,k) of grad_a = EA * sum_n H[m][n] EB[k][n]; rows <- H, columns <- EB, both
+//         sources [line][reduction].
+// GRAD_B: tile (k,n) of grad_b = EB * sum_m EA[m][k] H[m][n]; rows <- EA, columns <- H, both
+//         sources [reduction][line].
+template <class T, bool GRAD_A>
+struct SplitBwd {
+  static constexpr int NT = T::NT;
+  using SR = std::conditional_t<GRAD_A, SplitT<T::TR, NT>, SplitS<T::TR, NT>>;
+  using SC = std::conditional_t<GRAD_A, SplitT<T::TC, NT>, SplitS<T::TC, NT>>;
+  static constexpr int WORDS = split_lds_words<SR, SC>();
+};
+
+template <class T, bool GRAD_A>
+__device__ __forceinline__ void log_bwd_split_tile(unsigned* __restrict__ smem, int tile, const elem_t* __restrict__ g,
+                                                   const LeanSrc src, const int* __restrict__ ws_hdr,
+                                                   const int* __restrict__ fwd_flags, elem_t* __restrict__ grad, int M,
+                                                   int K, int N, int tiles_r, int tiles_c) {
+  using W = SplitBwd<T, GRAD_A>;
+  using SR = typename W::SR;
+  using SC = typename W::SC;
+  constexpr int NT = T::NT;
+  static_assert(W::WORDS >= (NT / 64) * kStripFloats, "");
+  auto Rs = [&](int buf) __attribute__((always_inline)) { return smem + buf * SR::BUF; };
+  auto Cs = [&](int buf) __attribute__((always_inline)) { return smem + 2 * SR::BUF + buf * SC::BUF; };
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wr0 = (wave / T::WC) * 64, wc0 = (wave % T::WC) * 64;
+  const int per = tiles_r * tiles_c;
+  const int batch = tile / per, rem = tile - batch * per;
+  const int r0 = (rem / tiles_c) * T::TR, c0 = (rem % tiles_c) * T::TC;
+  const int Q = GRAD_A ? N : M;
+  const int R = GRAD_A ? M : K, Cc = GRAD_A ? K : N;
+  const float* al = src.stats + (long)batch * (M + N);
+  const float* be = al + M;
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int x = 0; x < 4; ++x)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[x >> 1][x & 1][i] = 0.f;
+  const int slabs = Q / kMS;
+
+  // Addresses are a base per workgroup (scalar registers, stepped slab by slab) plus a fixed
+  // 32-bit offset per thread: the vector registers go to operands and accumulators.
+  if constexpr (GRAD_A) {
+    // rows: H pieces (line m, four n); columns: EB pieces (line k, four n); beta of the slab's four
+    // columns is the same for every piece of a thread (all share their quad)
+    const elem_t* ob = src.out + (long)batch * M * N;
+    const elem_t* gb = g + (long)batch * M * N;
+    const elem_t* bb = src.b + (long)batch * K * N;
+    const float* beb = be;
+    int oo[SR::PER], yo[SC::PER];
+    float alh[SR::PER];
+#pragma unroll
+    for (int l = 0; l < SR::PER; ++l) {
+      const int m = r0 + SR::line(tid, l);
+      oo[l] = m * N + SR::quad(tid) * 4;
+      alh[l] = al[m];
+    }
+#pragma unroll
+    for (int l = 0; l < SC::PER; ++l) yo[l] = (c0 + SC::line(tid, l)) * N + SC::quad(tid) * 4;
+    const int beo = SR::quad(tid) * 4;
+    float4 ro[SR::PER], rg[SR::PER], ry[SC::PER], bslab;
+    auto load = [&]() __attribute__((always_inline)) {
+#pragma unroll
+      for (int l = 0; l < SC::PER; ++l) ry[l] = ld4(bb + yo[l]);
+#pragma unroll
+      for (int l = 0; l < SR::PER; ++l) {
+        ro[l] = ld4(ob + oo[l]);
+        rg[l] = ld4(gb + oo[l]);
+      }
+      bslab = ld4(beb + beo);
+      ob += kMS; gb += kMS; bb += kMS; beb += kMS;
+    };
+    auto stage = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+      for (int l = 0; l < SC::PER; ++l) SC::put(Cs(buf), tid, l, exp4(ry[l], bslab));
+#pragma unroll
+      for (int l = 0; l < SR::PER; ++l) {
+        const float4 sh = make_float4(alh[l] + bslab.x, alh[l] + bslab.y, alh[l] + bslab.z, alh[l] + bslab.w);
+        SR::put(Rs(buf), tid, l, mul_exp4(rg[l], sh, ro[l]));
+      }
+    };
+    load();
+    if (bwd_tile_flagged(ws_hdr, fwd_flags, false, true, r0, T::TR, batch, M, N, tid, NT)) return;
+    stage(0);
+    __syncthreads();
+    for (int s = 0; s < slabs; ++s) {
+      const bool more = s + 1 < slabs;
+      if (more) load();
+      split_slab<SR, SC>(Rs(s & 1), Cs(s & 1), wr0, wc0, lane, acc);
+      if (more) stage((s + 1) & 1);
+      __syncthreads();
+    }
+  } else {
+    // rows: EA pieces (steps m, m + 1; LW lines k); columns: H pieces (steps m, m + 1; LW lines n);
+    // both operands' pieces of a thread are on the same pair of steps
+    constexpr int LR = SR::LW, LC = SC::LW;
+    static_assert(SR::Q == SC::Q, "");
+    const int m2 = 2 * SR::pair(tid);
+    const elem_t* ab = src.a + (long)batch * M * K;
+    const elem_t* ob = src.out + (long)batch * M * N;
+    const elem_t* gb = g + (long)batch * M * N;
+    const float* alb = al;
+    const int yo = m2 * K + r0 + SR::line0(tid), oo = m2 * N + c0 + SC::line0(tid);
+    float bec[LC];
+#pragma unroll
+    for (int j = 0; j < LC; ++j) bec[j] = be[c0 + SC::line0(tid) + j];
+    float ye[LR], yd[LR], oe[LC], od[LC], ge[LC], gd[LC];
+    float a0, a1;
+    auto load = [&]() __attribute__((always_inline)) {
+      ldw<LR>(ab + yo, ye);
+      ldw<LR>(ab + yo + K, yd);
+      ldw<LC>(ob + oo, oe);
+      ldw<LC>(ob + oo + N, od);
+      ldw<LC>(gb + oo, ge);
+      ldw<LC>(gb + oo + N, gd);
+      a0 = alb[m2]; a1 = alb[m2 + 1];
+      ab += (long)kMS * K;
+      ob += (long)kMS * N;
+      gb += (long)kMS * N;
+      alb += kMS;
+    };
+    auto stage = [&](int buf) __attribute__((always_inline)) {
+      float e0[LR], e1[LR], h0[LC], h1[LC];
+#pragma unroll
+      for (int j = 0; j < LR; ++j) {
+        e0[j] = exp_st(ye[j] - a0);
+        e1[j] = exp_st(yd[j] - a1);
+      }
+#pragma unroll
+      for (int j = 0; j < LC; ++j) {
+        h0[j] = ge[j] * exp_st(a0 + bec[j] - oe[j]);
+        h1[j] = gd[j] * exp_st(a1 + bec[j] - od[j]);
+      }
+      SR::put(Rs(buf), tid, e0, e1);
+      SC::put(Cs(buf), tid, h0, h1);
+    };
+    load();
+    if (bwd_tile_flagged(ws_hdr, fwd_flags, false, false, c0, T::TC, batch, M, N, tid, NT)) return;
+    stage(0);
+    __syncthreads();
+    for (int s = 0; s < slabs; ++s) {
+      const bool more = s + 1 < slabs;
+      if (more) load();
+      split_slab<SR, SC>(Rs(s & 1), Cs(s & 1), wr0, wc0, lane, acc);
+      if (more) stage((s + 1) & 1);
+      __syncthreads();
+    }
+  }
+
+  // grad = EX * acc with EX = exp(a - alpha) (grad_a) or exp(b - beta) (grad_b), row-wise
+  const int lr = lane >> 4, lc = (lane & 15) * 4;
+  const int voff = lr * Cc + lc;
+  const long ubase = ((long)batch * R + r0 + wr0) * Cc + c0 + wc0;
+  const elem_t* xb = (GRAD_A ? src.a : src.b) + ubase + voff;
+  elem_t* gp = grad + ubase + voff;
+  float4 becol = make_float4(0.f, 0.f, 0.f, 0.f);
+  if constexpr (!GRAD_A) becol = ld4(be + c0 + wc0 + lc);
+  const float* alrow = al + r0 + wr0 + lr;
+  float4 xq[2][4];
+  float xa[2][4];
+  auto fetch = [&](int q) __attribute__((always_inline)) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      xq[q & 1][t] = ld4(xb + (long)(16 * q + 4 * t) * Cc);
+      if constexpr (GRAD_A) xa[q & 1][t] = alrow[16 * q + 4 * t];
+    }
+  };
+  fetch(0);
+  acc_rows(acc, reinterpret_cast<float*>(smem) + wave * kStripFloats, lane,
+           [&](int q) __attribute__((always_inline)) { if (q + 1 < 4) fetch(q + 1); },
+           [&](int q, int t, float4 v) __attribute__((always_inline)) {
+             float4 x;
+             if constexpr (GRAD_A) x = exp4(xq[q & 1][t], xa[q & 1][t]);
+             else x = exp4(xq[q & 1][t], becol);
+             st4(gp + (long)(16 * q + 4 * t) * Cc, make_float4(x.x * v.x, x.y * v.y, x.z * v.z, x.w * v.w));
+           });
+}
+
+// Both gradients in one launch, item by item, a tile of each in turn (see k_log_bwd_mfma_both).
+template <class TA, class TB>
+__global__ __launch_bounds__(TA::NT) __attribute__((amdgpu_waves_per_eu(TA::WPE, TA::WPE)))
+void k_log_bwd_split_both(const elem_t* __restrict__ g, const LeanSrc src, const int* __restrict__ ws_hdr,
+                          const int* __restrict__ fwd_flags, elem_t* __restrict__ grad_a,
+                          elem_t* __restrict__ grad_b, int M, int K, int N, int ar, int ac, int br, int bc) {
+  static_assert(TA::NT == TB::NT && TA::WPE == TB::WPE, "");
+  extern __shared__ __attribute__((aligned(16))) unsigned split_smem[];
+  const int per_a = ar * ac, per_b = br * bc;
+  const int v = xcd_renumber(blockIdx.x, gridDim.x);
+  const int item = v / (per_a + per_b), r = v - item * (per_a + per_b);
+  const bool alt = per_a == per_b;
+  const bool is_a = alt ? (r & 1) == 0 : r < per_a;
+  const int idx = alt ? r >> 1 : (r < per_a ? r : r - per_a);
+  if (is_a)
+    log_bwd_split_tile<TA, true>(split_smem, item * per_a + idx, g, src, ws_hdr, fwd_flags, grad_a, M, K, N, ar, ac);
+  else
+    log_bwd_split_tile<TB, false>(split_smem, item * per_b + idx, g, src, ws_hdr, fwd_flags, grad_b, M, K, N, br, bc);
+}
+
+template <class TA, class TB>
+constexpr int split_bwd_lds_bytes() {
+  constexpr int a = SplitBwd<TA, true>::WORDS, b = SplitBwd<TB, false>::WORDS;
+  return 4 * (a > b ? a : b);
+}
+
+}  // namespace GENBMM_NS

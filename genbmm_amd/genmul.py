@@ -53,7 +53,7 @@ def _sfx(t):
     return _lib.HALF_SUFFIX.get(t.dtype, "")
 
 
-PATH_AUTO, PATH_EXACT, PATH_VALU, PATH_FACTORS = 0, 1, 2, 3  # GENBMM_PATH_* of the C header
+PATH_AUTO, PATH_EXACT, PATH_VALU, PATH_FACTORS, PATH_MFMA32 = 0, 1, 2, 3, 4  # GENBMM_PATH_* of the C header
 
 
 def _prep(a, b):
@@ -384,7 +384,8 @@ def logbmm(a, b):
 def logbmm_on_path(a, b, path):
     """logbmm with the library's kernel family named (PATH_AUTO / PATH_EXACT / PATH_VALU / PATH_FACTORS:
     as PATH_AUTO, but autograd saves exp(a - max), exp(b - max) and 1 / sum beside the maxima - three
-    more tensors than the reference saves - and the matrix-core backward takes no exponential);
+    more tensors than the reference saves - and the matrix-core backward takes no exponential /
+    PATH_MFMA32: as PATH_AUTO with the fp32 matrix instruction for every tiled shape);
     forward and backward both use it.  For tests and measurements."""
     a, b, restore = _canonical(a, b)
     return restore(LogMatMul.apply(a, b, path))

@@ -141,6 +141,14 @@ size_t genbmm_samplebmm_stats_size(int B, int M, int K, int N);
  * forward writes 200 MB less, the backward takes three exponentials per staged
  * element).  With float16 / bfloat16 tensors that backward reads `out` as stored
  * (rounded); FACTORS keeps 1 / sum in fp32.
+ *   GENBMM_PATH_MFMA32 as AUTO, but the tiled matrix-core kernels use the fp32
+ *                      matrix instruction for every shape.  Under AUTO,
+ *                      problems made of full tiles (M and K multiples of 256,
+ *                      N of 128) run on the bf16 matrix instruction with every
+ *                      factor cut into three bf16 parts that add up to it
+ *                      exactly and six partial products per product - what is
+ *                      dropped is below 2^-23 of a product, one fp32 rounding -
+ *                      at 2.7 times less matrix-pipe time.
  * Any other value: GENBMM_E_MODE.  Forward and backward of one problem need not
  * name the same path (see genbmm_logbmm_bwd).  No counterpart in the reference.
  */
@@ -148,6 +156,7 @@ size_t genbmm_samplebmm_stats_size(int B, int M, int K, int N);
 #define GENBMM_PATH_EXACT 1
 #define GENBMM_PATH_VALU 2
 #define GENBMM_PATH_FACTORS 3
+#define GENBMM_PATH_MFMA32 4
 /* Number of fp32 elements of `stats` for a forward / backward pair on `path`
  * (genbmm_logbmm_stats_size is this for GENBMM_PATH_AUTO). */
 size_t genbmm_logbmm_stats_size_path(int B, int M, int K, int N, int path);

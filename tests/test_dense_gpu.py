@@ -35,16 +35,17 @@ def lse64(a, b, chunk=4):
     return torch.cat(outs) if outs else a.new_zeros((0, a.shape[1], b.shape[2])).double()
 
 
-@pytest.fixture(params=["factored", "exact", "factored-valu", "factors-kept"])
+@pytest.fixture(params=["factored", "exact", "factored-valu", "factors-kept", "fp32-matrix"])
 def path(request, gpu):
     """Run a logbmm test on every kernel family of the library: the default one (whole-item
     kernels for small matrices, matrix cores for large ones, factored vector-ALU kernels
     between; the matrix-core kernels keep the maxima only and form their operands again in the
     backward), the online / exact kernels alone, the factored kernels on v_fma only, and the
-    default kernels with the forward's factors kept for an exponent-free backward.
-    The value is the `path` argument of genbmm_logbmm_fwd_path / _bwd_path."""
+    default kernels with the forward's factors kept for an exponent-free backward, and the default
+    kernels with the fp32 matrix instruction wherever the default uses the bf16 one on three-part
+    factors.  The value is the `path` argument of genbmm_logbmm_fwd_path / _bwd_path."""
     return {"factored": genmul.PATH_AUTO, "exact": genmul.PATH_EXACT, "factored-valu": genmul.PATH_VALU,
-            "factors-kept": genmul.PATH_FACTORS}[request.param]
+            "factors-kept": genmul.PATH_FACTORS, "fp32-matrix": genmul.PATH_MFMA32}[request.param]
 
 
 def logbmm_on(path):
@@ -251,6 +252,53 @@ def test_logbmm_rows_masked_at_the_floor(gpu, keep, B, M, K, N):
     close(ga[ok.to(gpu)], wa[ok])
     close(gb[ok.to(gpu)], wb[ok])
     assert bool(torch.isfinite(ga[ok.to(gpu)]).all()) and bool(torch.isfinite(gb[ok.to(gpu)]).all())
+
+
+@pytest.mark.parametrize("B,M,K,N", [(64, 512, 256, 512), (64, 512, 512, 384), (64, 512, 512, 512), (48, 768, 64, 512)])
+def test_logbmm_three_part_kernels(gpu, B, M, K, N):
+    """Shapes made of full tiles, which the default path runs on the bf16 matrix instruction with
+    every factor cut into three bf16 parts (256 x 256 tiles where they fill the chip, 256 x 128 /
+    128 x 256 otherwise; forward and backward switch independently): every batch item against
+    float64 on the device, among them items whose tiles must take the exact routine (factors that
+    underflow against live terms: everywhere, and in a single row), an item with rows padded at
+    the floor, one with a masked reduction step, one with magnitudes near 1000 - and the whole
+    result against the fp32 matrix instruction (GENBMM_PATH_MFMA32) at twice the tolerance."""
+    torch.manual_seed(M + N)
+    a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
+    a[1, ::2, 0] += 200.0
+    b[1, 0, :] -= 200.0
+    a[2, 37, 5] += 200.0
+    b[2, 5, :] -= 200.0
+    a[3, M - 50:, :] = -1e9
+    g[3, M - 50:, :] = 0.0
+    a[4] *= 300.0
+    b[5, 7, :] = -float("inf")
+    ad, bd, gd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True), g.to(gpu)
+    out = genbmm.logbmm(ad, bd)
+    ga, gb = torch.autograd.grad(out, (ad, bd), gd)
+    for i in range(B):
+        want, wa, wb = oracle.logbmm_grads64(ad[i:i + 1], bd[i:i + 1], gd[i:i + 1])
+        rows = slice(0, M - 50) if i == 3 else slice(0, M)   # the padded rows' own cells: rounding artefacts
+        # (item 4: `out` near 1000 is rounded to 6e-5, and every backward that forms its weights from
+        #  `out` - the reference's included - inherits that as a relative error of the weights)
+        tol = dict(rtol=1e-3, atol=5e-3) if i == 4 else {}
+        close_on_device(out[i:i + 1, rows].detach(), want[:, rows], "out, item %d" % i)
+        close_on_device(ga[i:i + 1, rows], wa[:, rows], "grad_a, item %d" % i, **tol)
+        close_on_device(gb[i:i + 1], wb, "grad_b, item %d" % i, **tol)
+        del want, wa, wb
+    assert bool(torch.isfinite(ga).all()) and bool(torch.isfinite(gb).all())
+    ar, br = ad.detach().clone().requires_grad_(True), bd.detach().clone().requires_grad_(True)
+    ref = genmul.logbmm_on_path(ar, br, genmul.PATH_MFMA32)
+    ra, rb = torch.autograd.grad(ref, (ar, br), gd)
+    keep = torch.ones(M, dtype=torch.bool, device=gpu)
+    for x, y, rowwise, grad in ((out.detach(), ref.detach(), True, False), (ga, ra, True, True), (gb, rb, False, True)):
+        x, y = x.clone(), y.clone()
+        if rowwise:   # item 3's padded rows again
+            x[3, M - 50:], y[3, M - 50:] = 0, 0
+        if grad:
+            close_on_device(x[4], y[4].double(), "item 4 against the fp32 matrix instruction", rtol=1e-3, atol=5e-3)
+            x[4], y[4] = 0, 0
+        close_on_device(x, y.double(), "against the fp32 matrix instruction", rtol=2e-5, atol=2e-5)
 
 
 @pytest.mark.parametrize("B,M,K,N", [(20, 128, 128, 128), (17, 100, 70, 128), (12, 64, 128, 65), (9, 127, 99, 101)])
