@@ -130,12 +130,26 @@ __device__ __forceinline__ floatx16 mfma_bf16(bf16x8 a, bf16x8 b, floatx16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
+// The waves of a SIMD (waves i, i + 4, ... of the workgroup) run their matrix instructions at
+// different priorities, all above the priority of staging: behind a barrier they would otherwise
+// take turns instruction by instruction, finish their products together and then all stage at
+// once with the matrix pipe idle; this way the first is through early and stages - vector work,
+// which issues beside the others' matrix instructions - while the next one multiplies.
+__device__ __forceinline__ void mfma_prio(int wave) {
+  switch ((wave >> 2) & 3) {
+    case 0: __builtin_amdgcn_s_setprio(3); break;
+    case 1: __builtin_amdgcn_s_setprio(2); break;
+    case 2: __builtin_amdgcn_s_setprio(1); break;
+    default: __builtin_amdgcn_s_setprio(1); break;
+  }
+}
+
 // The six partial products of one staged slab, for the wave's 2 x 2 blocks.  Products of one
 // kind go to the four accumulators in turn (no instruction waits for the one before it);
 // the small ones first.
 template <class SR, class SC>
 __device__ __forceinline__ void split_slab(const unsigned* __restrict__ R, const unsigned* __restrict__ Cs, int wr0,
-                                           int wc0, int lane, floatx16 (&acc)[2][2]) {
+                                           int wc0, int wave, int lane, floatx16 (&acc)[2][2]) {
   // Operand registers are asked for a phase ahead of their products and given up after them
   // (at most 40 of them live beside the 64 accumulators; the fences keep the compiler from
   // asking for all twelve operands up front).
@@ -151,7 +165,7 @@ __device__ __forceinline__ void split_slab(const unsigned* __restrict__ R, const
     rl[i] = SR::frag(R, 2, wr0 + 32 * i, lane);
   }
   __builtin_amdgcn_sched_barrier(0);
-  __builtin_amdgcn_s_setprio(1);
+  mfma_prio(wave);
 #pragma unroll
   for (int x = 0; x < 4; ++x) acc[x >> 1][x & 1] = mfma_bf16(rh[x >> 1], cl[x & 1], acc[x >> 1][x & 1]);
   __builtin_amdgcn_sched_barrier(0);
@@ -180,6 +194,34 @@ __device__ __forceinline__ void split_slab(const unsigned* __restrict__ R, const
 template <class SR, class SC>
 constexpr int split_lds_words() { return 2 * (SR::BUF + SC::BUF); }
 
+// The slab loop.  On entry slab 0 is loaded and staged (no barrier yet).
+// The four waves of a SIMD (waves i, i + 4, i + 8, i + 12 of a workgroup of sixteen) issue their
+// matrix instructions at descending priority (mfma_prio), so behind the barrier the first is
+// through its products early and the last late.  The first half ("late" waves) stages the next
+// slab behind its products, while the others still multiply; the second half ("early" waves),
+// which must wait for the matrix pipe anyway, stages the next slab AHEAD of its products - from
+// registers loaded a whole slab before - while the first half multiplies.  Nobody's staging is
+// left for the end of the slab with the matrix pipe idle.  One load in flight per wave either way.
+template <class Load, class Stage, class Mma>
+__device__ __forceinline__ void split_loop(int slabs, bool early, Load&& load, Stage&& stage, Mma&& mma) {
+  if (early && slabs > 1) load();
+  __syncthreads();
+  for (int s = 0; s < slabs; ++s) {
+    const bool more = s + 1 < slabs;
+    if (early) {
+      if (more) stage((s + 1) & 1);
+      if (s + 2 < slabs) load();
+    } else {
+      if (more) load();
+    }
+    mma(s & 1);
+    if (!early && more) stage((s + 1) & 1);
+    __syncthreads();
+  }
+}
+// the second half of a workgroup's waves
+template <int NT>
+__device__ __forceinline__ bool split_early(int wave) { return wave >= NT / 128; }
 // ----------------------------------------------------------------- forward
 // rows <- EA from a[m][k] ([line][reduction]), columns <- EB from b[k][n] ([reduction][line]).
 // Leaves the maxima, the tile flags and the header (no factors), like k_log_fwd_mfma<T, false, false>.
@@ -256,14 +298,9 @@ void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
 
   load();
   stage(0);
-  __syncthreads();
-  for (int s = 0; s < slabs; ++s) {
-    const bool more = s + 1 < slabs;
-    if (more) load();
-    split_slab<SA, SB>(As(s & 1), Bs(s & 1), wm0, wn0, lane, acc);
-    if (more) stage((s + 1) & 1);
-    __syncthreads();
-  }
+  split_loop(slabs, split_early<NT>(wave), load, stage, [&](int buf) __attribute__((always_inline)) {
+    split_slab<SA, SB>(As(buf), Bs(buf), wm0, wn0, wave, lane, acc);
+  });
 
   // guard (as k_log_fwd_mfma): S >= 2^-40 and finite; every shift finite and not below the floor;
   // no shift below -30 opposite a row or column at the floor
@@ -400,14 +437,9 @@ __device__ __forceinline__ void log_bwd_split_tile(unsigned* __restrict__ smem, 
     load();
     if (bwd_tile_flagged(ws_hdr, fwd_flags, false, true, r0, T::TR, batch, M, N, tid, NT)) return;
     stage(0);
-    __syncthreads();
-    for (int s = 0; s < slabs; ++s) {
-      const bool more = s + 1 < slabs;
-      if (more) load();
-      split_slab<SR, SC>(Rs(s & 1), Cs(s & 1), wr0, wc0, lane, acc);
-      if (more) stage((s + 1) & 1);
-      __syncthreads();
-    }
+    split_loop(slabs, split_early<NT>(wave), load, stage, [&](int buf) __attribute__((always_inline)) {
+      split_slab<SR, SC>(Rs(buf), Cs(buf), wr0, wc0, wave, lane, acc);
+    });
   } else {
     // rows: EA pieces (steps m, m + 1; LW lines k); columns: H pieces (steps m, m + 1; LW lines n);
     // both operands' pieces of a thread are on the same pair of steps
@@ -455,14 +487,9 @@ __device__ __forceinline__ void log_bwd_split_tile(unsigned* __restrict__ smem, 
     load();
     if (bwd_tile_flagged(ws_hdr, fwd_flags, false, false, c0, T::TC, batch, M, N, tid, NT)) return;
     stage(0);
-    __syncthreads();
-    for (int s = 0; s < slabs; ++s) {
-      const bool more = s + 1 < slabs;
-      if (more) load();
-      split_slab<SR, SC>(Rs(s & 1), Cs(s & 1), wr0, wc0, lane, acc);
-      if (more) stage((s + 1) & 1);
-      __syncthreads();
-    }
+    split_loop(slabs, split_early<NT>(wave), load, stage, [&](int buf) __attribute__((always_inline)) {
+      split_slab<SR, SC>(Rs(buf), Cs(buf), wr0, wc0, wave, lane, acc);
+    });
   }
 
   // grad = EX * acc with EX = exp(a - alpha) (grad_a) or exp(b - beta) (grad_b), row-wise
