@@ -108,7 +108,7 @@ def dense_log(lib, dev, B, M, K, N, reps, name, dist="randn", path=0, graph=Fals
         extra_graph["ms_float_kernels_with_casts"] = round(timed(widened, reps), 4)
     bmkn = float(B) * M * K * N
     nbytes = float(a.element_size()) * B * (3 * M * K + 3 * K * N + 3 * M * N)
-    report(name, ms, 6 * bmkn, nbytes, {"path": {0: "factored", 1: "online-exact", 2: "factored-valu", 3: "factored, factors kept"}[path],
+    report(name, ms, 6 * bmkn, nbytes, {"path": {0: "factored (bf16 matrix instruction on three-part factors where the shape is made of full tiles)", 1: "online-exact", 2: "factored-valu", 3: "factored, factors kept (fp32 matrix instruction)", 4: "factored, fp32 matrix instruction"}[path],
                                         "workspace_MB": round(stats.numel() * 4 / 1e6, 2),
                                         "ms_fwd": round(mf, 4), "ms_bwd": round(mb, 4), **extra_graph})
 
@@ -364,7 +364,7 @@ def main():
         dense_log(lib, dev, 512, 128, 128, 128, r, "logbmm fwd+bwd (512,128,128,128) config 1")
         dense_log(lib, dev, 8192, 32, 32, 32, r, "logbmm fwd+bwd (8192,32,32,32) config 1 skinny")
         dense_log2(lib, dev, 512, 128, 128, 128, max(3, r // 4))
-        for path in (0, 3, 2, 1):
+        for path in (0, 4, 3, 2, 1):
             dense_log(lib, dev, 64, 512, 512, 512, r, "logbmm fwd+bwd (64,512,512,512) headline", path=path)
     if "half" in want:
         for dt, nm in ((torch.float16, "float16"), (torch.bfloat16, "bfloat16")):

@@ -930,14 +930,19 @@ void launch_item_fwd(const elem_t* a, const elem_t* b, elem_t* out, float* stats
 
 // keep: the workspace is as large as genbmm_logbmm_stats_size says and receives what a
 // backward wants beside the maxima; false: header_offset() + 4 floats of it are used.
-int launch_self_fwd(DenseArgs p, float* stats, int B, int M, int K, int N, hipStream_t s) {
+int launch_self_fwd(DenseArgs p, float* stats, int B, int M, int K, int N, bool split, hipStream_t s) {
   dim3 grid;
   if (int e = fill_args<CfgWide>(p, B, M, K, N, grid)) return e;  // what the exact routine reads
   int* hdr = prepared_of(stats, B, M, K, N).hdr;
-  if (M == kSelfMax && K == kSelfMax && N == kSelfMax)
-    hipLaunchKernelGGL(k_log_self_fwd<false>, dim3(B), dim3(256), 0, s, p, stats, hdr);
-  else
-    hipLaunchKernelGGL(k_log_self_fwd<true>, dim3(B), dim3(256), 0, s, p, stats, hdr);
+  const bool full = M == kSelfMax && K == kSelfMax && N == kSelfMax;
+  auto go = [&](auto kern) { hipLaunchKernelGGL(kern, dim3(B), dim3(256), 0, s, p, stats, hdr); };
+  if (split) {
+    if (full) go(k_log_self_fwd<false, true>);
+    else go(k_log_self_fwd<true, true>);
+  } else {
+    if (full) go(k_log_self_fwd<false, false>);
+    else go(k_log_self_fwd<true, false>);
+  }
   return launch_status();
 }
 
@@ -962,7 +967,7 @@ int run_fwd(const elem_t* a, const elem_t* b, elem_t* out, float* stats, int B, 
   DenseArgs p{};
   p.a = a; p.b = b; p.out = out; p.idx = nullptr;
   if (stats && B > 0 && self_shape(M, K, N) && auto_path(path) && !factors)
-    return launch_self_fwd(p, stats, B, M, K, N, s);
+    return launch_self_fwd(p, stats, B, M, K, N, split_path(path), s);
   if (stats) {
     if (int e = launch_stats(a, b, stats, B, M, K, N, s)) return e;
   }
@@ -1023,10 +1028,15 @@ int run_bwd_both(const elem_t* a, const elem_t* b, const elem_t* out, const elem
     pb.grad = grad_b;
     const int* hdr = prepared_of(st, B, M, K, N).hdr;
     const dim3 grid((unsigned)ceil_div(B, 8) * 16);
-    if (M == kSelfMax && K == kSelfMax && N == kSelfMax)
-      hipLaunchKernelGGL(k_log_self_bwd<false>, grid, dim3(256), 0, s, pa, pb, st, hdr, B);
-    else
-      hipLaunchKernelGGL(k_log_self_bwd<true>, grid, dim3(256), 0, s, pa, pb, st, hdr, B);
+    const bool full = M == kSelfMax && K == kSelfMax && N == kSelfMax;
+    auto go = [&](auto kern) { hipLaunchKernelGGL(kern, grid, dim3(256), 0, s, pa, pb, st, hdr, B); };
+    if (split_path(path)) {
+      if (full) go(k_log_self_bwd<false, true>);
+      else go(k_log_self_bwd<true, true>);
+    } else {
+      if (full) go(k_log_self_bwd<false, false>);
+      else go(k_log_self_bwd<true, false>);
+    }
     return launch_status();
   }
   if (st && grad_a && grad_b && mk > 0 && kn > 0 && fwd_mfma_shape(B, M, K, N)) {

@@ -23,6 +23,7 @@
 #include "dense_tiles.h"
 #include "log_bwd_tile.h"
 #include "logbmm_mfma.h"
+#include "logbmm_split.h"
 #include "logbmm_ws.h"
 
 namespace GENBMM_NS {
@@ -30,7 +31,27 @@ namespace GENBMM_NS {
 constexpr int kSelfMax = 128;               // largest extent these kernels take
 constexpr int kSelfSlabs = kSelfMax / kMS;  // reduction slabs at that extent
 using SelfTile = MTile<kSelfMax, kSelfMax, 2>;
-constexpr int kSelfLds = 2 * kMS * (SelfTile::LDR + SelfTile::LDC);
+// SPLIT kernels: the products on the bf16 matrix instruction, every staged factor in three bf16
+// parts (logbmm_split.h); the staged form takes more LDS than the fp32 one, which sets the size.
+using SelfSplitT = SplitT<kSelfMax, SelfTile::NT>;
+using SelfSplitS = SplitS<kSelfMax, SelfTile::NT>;
+constexpr int kSelfLds = 4 * SelfSplitS::BUF;  // two buffers of two operands, each the size of the larger form
+static_assert(kSelfLds >= 2 * kMS * (SelfTile::LDR + SelfTile::LDC) && SelfSplitT::BUF <= SelfSplitS::BUF, "");
+// Pieces of an operand stored [reduction][line]: rows red(tid, l), l = 0, 1, of a slab, four
+// lines from quad * 4.  The bf16 form wants a thread's two rows to be neighbours (a pair shares
+// a word); the fp32 form has them eight apart (StageS).
+template <bool SPLIT>
+struct SelfS {
+  static __device__ __forceinline__ int red(int tid, int l) { return SPLIT ? 2 * (tid >> 5) + l : (tid >> 5) + 8 * l; }
+  static __device__ __forceinline__ int quad(int tid) { return tid & 31; }
+};
+// the two LDS buffers of a split operand pair, rows operand first (sizes of the larger form)
+__device__ __forceinline__ unsigned* self_split_rows(float* smem, int buf) {
+  return reinterpret_cast<unsigned*>(smem) + buf * SelfSplitS::BUF;
+}
+__device__ __forceinline__ unsigned* self_split_cols(float* smem, int buf) {
+  return reinterpret_cast<unsigned*>(smem) + (2 + buf) * SelfSplitS::BUF;
+}
 static_assert(kSelfLds >= CfgWide::KT * (CfgWide::LDA + CfgWide::LDB), "exact forward routine fits");
 static_assert(kSelfLds >= LogBwdLds<BCfgWide, true>::FLOATS && kSelfLds >= LogBwdLds<BCfgWide, false>::FLOATS,
               "exact backward routine fits");
@@ -79,7 +100,7 @@ __device__ __forceinline__ void self_fwd_exact(const DenseArgs& p, int batch, fl
     }
 }
 
-template <bool RAGGED>
+template <bool RAGGED, bool SPLIT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void k_log_self_fwd(const DenseArgs p, float* __restrict__ stats, int* __restrict__ hdr) {
   using T = SelfTile;
@@ -87,7 +108,8 @@ void k_log_self_fwd(const DenseArgs p, float* __restrict__ stats, int* __restric
   static_assert(NT == 256 && T::LDR == T::LDC && CfgWide::NT == 256, "");
   using SA = StageT<kSelfMax, NT, LD>;
   using SB = StageS<kSelfMax, NT, LD>;
-  static_assert(SA::PER == 2 && SB::PER == 2, "");
+  using SBr = SelfS<SPLIT>;
+  static_assert(SA::PER == 2 && SB::PER == 2 && SelfSplitT::PER == 2, "");
   __shared__ __attribute__((aligned(16))) float smem[kSelfLds];
   __shared__ __attribute__((aligned(16))) float s_al[kSelfMax], s_be[kSelfMax], s_part[4][kSelfMax];
   float(*As)[kMS * LD] = reinterpret_cast<float(*)[kMS * LD]>(smem);
@@ -118,7 +140,7 @@ void k_log_self_fwd(const DenseArgs p, float* __restrict__ stats, int* __restric
 #pragma unroll
   for (int l = 0; l < 2; ++l) {
     oa[l] = (unsigned)(SA::line(tid, l) * K + aq);
-    obb[l] = (unsigned)(SB::red(tid, l) * N + bcol);
+    obb[l] = (unsigned)(SBr::red(tid, l) * N + bcol);
   }
 #pragma unroll
   for (int s = 0; s < kSelfSlabs; ++s)
@@ -126,7 +148,7 @@ void k_log_self_fwd(const DenseArgs p, float* __restrict__ stats, int* __restric
       const elem_t* bs = bb + (size_t)(kMS * s) * N;  // uniform
 #pragma unroll
       for (int l = 0; l < 2; ++l) {
-        const int m = SA::line(tid, l), k = kMS * s + SB::red(tid, l);
+        const int m = SA::line(tid, l), k = kMS * s + SBr::red(tid, l);
         if (!RAGGED) {
           ra[s][l] = ld4(ab + oa[l] + kMS * s);
           rb[s][l] = ld4(bs + obb[l]);
@@ -192,13 +214,25 @@ void k_log_self_fwd(const DenseArgs p, float* __restrict__ stats, int* __restric
   for (int s = 0; s <= kSelfSlabs; ++s) {
     // slab s is staged while slab s-1 is multiplied
     if (s < kSelfSlabs && (!RAGGED || s < slabs)) {
+      if constexpr (SPLIT) {
 #pragma unroll
-      for (int l = 0; l < 2; ++l) {
-        SA::put(As[s & 1], tid, l, exp4(ra[s][l], al[l]));
-        SB::put(Bs[s & 1], tid, l, exp4(rb[s][l], be));
+        for (int l = 0; l < 2; ++l) SelfSplitT::put(self_split_rows(smem, s & 1), tid, l, exp4(ra[s][l], al[l]));
+        SelfSplitS::put(self_split_cols(smem, s & 1), tid, exp4(rb[s][0], be), exp4(rb[s][1], be));
+      } else {
+#pragma unroll
+        for (int l = 0; l < 2; ++l) {
+          SA::put(As[s & 1], tid, l, exp4(ra[s][l], al[l]));
+          SB::put(Bs[s & 1], tid, l, exp4(rb[s][l], be));
+        }
       }
     }
-    if (s > 0 && (!RAGGED || s <= slabs)) mfma_slab<LD, LD>(As[(s - 1) & 1], Bs[(s - 1) & 1], wm0, wn0, lane, acc);
+    if (s > 0 && (!RAGGED || s <= slabs)) {
+      if constexpr (SPLIT)
+        split_slab<SelfSplitT, SelfSplitS>(self_split_rows(smem, (s - 1) & 1), self_split_cols(smem, (s - 1) & 1), wm0, wn0,
+                                           wave, lane, acc);
+      else
+        mfma_slab<LD, LD>(As[(s - 1) & 1], Bs[(s - 1) & 1], wm0, wn0, lane, acc);
+    }
     __syncthreads();
   }
 
@@ -285,7 +319,7 @@ __device__ __forceinline__ float4 self_h(float4 g, float4 o, float4 sh, int cnt,
   return h;
 }
 
-template <bool GRAD_A, bool RAGGED>
+template <bool GRAD_A, bool RAGGED, bool SPLIT>
 __device__ __forceinline__ void log_self_bwd_tile(float* __restrict__ smem, float* __restrict__ s_al,
                                                   float* __restrict__ s_be, const LogBwdArgs& p,
                                                   const float* __restrict__ stats,
@@ -293,7 +327,8 @@ __device__ __forceinline__ void log_self_bwd_tile(float* __restrict__ smem, floa
   using T = SelfTile;
   constexpr int NT = T::NT, LD = T::LDR;
   using ST = StageT<kSelfMax, NT, LD>;  // sources [out][red]: both operands of grad_a
-  using SS = StageS<kSelfMax, NT, LD>;  // sources [red][out]: both operands of grad_b
+  using SP = StageS<kSelfMax, NT, LD>;  // sources [red][out]: both operands of grad_b ...
+  using SS = SelfS<SPLIT>;              // ... and which pieces a thread holds of them
   float(*Rs)[kMS * LD] = reinterpret_cast<float(*)[kMS * LD]>(smem);
   float(*Cs)[kMS * LD] = reinterpret_cast<float(*)[kMS * LD]>(smem + 2 * kMS * LD);
   const int tid = threadIdx.x, lane = tid & 63;
@@ -411,6 +446,13 @@ __device__ __forceinline__ void log_self_bwd_tile(float* __restrict__ smem, floa
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[x >> 1][x & 1][i] = 0.f;
 
+  auto multiply = [&](int buf) __attribute__((always_inline)) {
+    if constexpr (!SPLIT) mfma_slab<LD, LD>(Rs[buf], Cs[buf], wr0, wc0, lane, acc);
+    else if constexpr (GRAD_A)
+      split_slab<SelfSplitT, SelfSplitT>(self_split_rows(smem, buf), self_split_cols(smem, buf), wr0, wc0, wave, lane, acc);
+    else
+      split_slab<SelfSplitS, SelfSplitS>(self_split_rows(smem, buf), self_split_cols(smem, buf), wr0, wc0, wave, lane, acc);
+  };
   // Slab s is formed and staged while slab s-1 is multiplied, so the products start as soon as
   // the first pieces have arrived; the guard's answer is only needed before the results are
   // stored (an item that fails it has been multiplied in vain).
@@ -423,23 +465,31 @@ __device__ __forceinline__ void log_self_bwd_tile(float* __restrict__ smem, floa
         make_y(sc_);
 #pragma unroll
         for (int l = 0; l < 2; ++l) {
-          if constexpr (GRAD_A) {  // rows <- H[m][n], columns <- EB[k][n]
+          if constexpr (SPLIT) {
+            if constexpr (GRAD_A) {
+              SelfSplitT::put(self_split_rows(smem, s & 1), tid, l, rg[s][l]);
+              SelfSplitT::put(self_split_cols(smem, s & 1), tid, l, ry[s][l]);
+            }
+          } else if constexpr (GRAD_A) {  // rows <- H[m][n], columns <- EB[k][n]
             ST::put(Rs[s & 1], tid, l, rg[s][l]);
             ST::put(Cs[s & 1], tid, l, ry[s][l]);
           } else {                 // rows <- EA[m][k], columns <- H[m][n]
-            SS::put(Rs[s & 1], tid, l, ry[s][l]);
-            SS::put(Cs[s & 1], tid, l, rg[s][l]);
+            SP::put(Rs[s & 1], tid, l, ry[s][l]);
+            SP::put(Cs[s & 1], tid, l, rg[s][l]);
           }
+        }
+        if constexpr (SPLIT && !GRAD_A) {
+          SelfSplitS::put(self_split_rows(smem, s & 1), tid, ry[s][0], ry[s][1]);
+          SelfSplitS::put(self_split_cols(smem, s & 1), tid, rg[s][0], rg[s][1]);
         }
       }
     }
     if constexpr (s > 0) {
-      if (!RAGGED || s <= slabs) mfma_slab<LD, LD>(Rs[(s - 1) & 1], Cs[(s - 1) & 1], wr0, wc0, lane, acc);
+      if (!RAGGED || s <= slabs) multiply((s - 1) & 1);
     }
     __syncthreads();
   });
-  if (!RAGGED || slabs == kSelfSlabs)
-    mfma_slab<LD, LD>(Rs[(kSelfSlabs - 1) & 1], Cs[(kSelfSlabs - 1) & 1], wr0, wc0, lane, acc);
+  if (!RAGGED || slabs == kSelfSlabs) multiply((kSelfSlabs - 1) & 1);
   bad = __builtin_amdgcn_readfirstlane(__syncthreads_or(bad));
   if (bad) {
     self_bwd_exact<GRAD_A>(p, batch, smem);
@@ -483,7 +533,7 @@ __device__ __forceinline__ void log_self_bwd_tile(float* __restrict__ smem, floa
 // Workgroups come in groups of 16: the first eight take grad_a of eight consecutive
 // items, the next eight grad_b of the same items (workgroup w runs on XCD w mod 8).
 // A gradient whose pointer is null is skipped.
-template <bool RAGGED>
+template <bool RAGGED, bool SPLIT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void k_log_self_bwd(const LogBwdArgs pa, const LogBwdArgs pb, const float* __restrict__ stats,
                     const int* __restrict__ hdr, int B) {
@@ -493,9 +543,9 @@ void k_log_self_bwd(const LogBwdArgs pa, const LogBwdArgs pb, const float* __res
   const int item = (w >> 4) * 8 + (w & 7);
   if (item >= B) return;
   if (((w >> 3) & 1) == 0) {
-    if (pa.grad) log_self_bwd_tile<true, RAGGED>(smem, s_al, s_be, pa, stats, hdr, item);
+    if (pa.grad) log_self_bwd_tile<true, RAGGED, SPLIT>(smem, s_al, s_be, pa, stats, hdr, item);
   } else {
-    if (pb.grad) log_self_bwd_tile<false, RAGGED>(smem, s_al, s_be, pb, stats, hdr, item);
+    if (pb.grad) log_self_bwd_tile<false, RAGGED, SPLIT>(smem, s_al, s_be, pb, stats, hdr, item);
   }
 }
 

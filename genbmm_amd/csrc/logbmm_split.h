@@ -105,6 +105,11 @@ struct SplitS {
       w.x = l[0]; w.y = l[1]; *reinterpret_cast<uintx2*>(p + 2 * PLANE) = w;
     }
   }
+  static __device__ __forceinline__ void put(unsigned* __restrict__ buf, int tid, float4 even, float4 odd) {
+    static_assert(LW == 4, "");
+    const float e[4] = {even.x, even.y, even.z, even.w}, o[4] = {odd.x, odd.y, odd.z, odd.w};
+    put(buf, tid, e, o);
+  }
   static __device__ __forceinline__ bf16x8 frag(const unsigned* __restrict__ buf, int plane, int line0, int lane) {
     const unsigned* p = buf + plane * PLANE + (lane >> 5) * 4 * LD + line0 + (lane & 31);
     uintx4 w;
