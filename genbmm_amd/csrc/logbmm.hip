@@ -833,44 +833,55 @@ int launch_bwd_mfma_both(LogBwdArgs pa, LogBwdArgs pb, const float* stats, int B
   return launch_status();
 }
 
-// The bf16 three-part kernels (logbmm_split.h): full tiles only; the 256 x 256 tile (one
-// workgroup of sixteen waves per compute unit) when it fills the chip.
-template <class T>
-inline bool split_fits(int B, int out_r, int out_c, int red, bool fill_chip) {
-  if (out_r % T::TR != 0 || out_c % T::TC != 0 || red % kMS != 0) return false;
-  return !fill_chip || (int64_t)B * (out_r / T::TR) * (out_c / T::TC) >= 192;
+// The bf16 three-part kernels (logbmm_split.h).  The 256 x 256 tile (one workgroup of sixteen waves
+// per compute unit) where both extents split into 256s without more padding than 128-wide tiles
+// would add and there are tiles enough to fill the chip; the caller falls back to 256 x 128 /
+// 128 x 256.
+inline bool pads_to_256(int x) { return ceil_div(x, 256) * 2 == ceil_div(x, 128); }
+inline bool split_big_fits(int B, int out_r, int out_c) {
+  return pads_to_256(out_r) && pads_to_256(out_c) && (int64_t)B * ceil_div(out_r, 256) * ceil_div(out_c, 256) >= 192;
 }
 template <class T>
 int launch_fwd_split(DenseArgs p, float* stats, int B, int M, int K, int N, hipStream_t s) {
   p.M = M; p.K = K; p.N = N;
-  p.tiles_m = M / T::TR;
-  p.tiles_n = N / T::TC;
+  p.tiles_m = ceil_div(M, T::TR);
+  p.tiles_n = ceil_div(N, T::TC);
   p.vec_a = (K % 4 == 0) && aligned16(p.a);
   p.vec_b = (N % 4 == 0) && aligned16(p.b);
   p.vec_o = (N % 4 == 0) && aligned16(p.out);
-  const int total = B * p.tiles_m * p.tiles_n;
+  const int64_t total64 = (int64_t)B * p.tiles_m * p.tiles_n;
+  if (total64 > 0x7fffffffLL) return GENBMM_E_SHAPE;
+  const int total = (int)total64;
   int* flags = fwd_flags_of(stats, B, M, N);
   constexpr int lds = 4 * split_lds_words<SplitT<T::TR, T::NT>, SplitS<T::TC, T::NT>>();
-  allow_lds(k_log_fwd_split<T>, lds);
-  hipLaunchKernelGGL(k_log_fwd_split<T>, dim3(total), dim3(T::NT), lds, s, p.a, p.b, p.out, stats, flags,
-                     prepared_of(stats, B, M, K, N).hdr, M, K, N, p.tiles_m, p.tiles_n);
+  auto go = [&](auto kern) {
+    allow_lds(kern, lds);
+    hipLaunchKernelGGL(kern, dim3(total), dim3(T::NT), lds, s, p.a, p.b, p.out, stats, flags,
+                       prepared_of(stats, B, M, K, N).hdr, M, K, N, p.tiles_m, p.tiles_n);
+  };
+  if (M % T::TR != 0 || N % T::TC != 0 || K % kMS != 0) go(k_log_fwd_split<T, true>);
+  else go(k_log_fwd_split<T, false>);
   if (int e = launch_status()) return e;
   return launch_fwd_fixup<CfgWide, T::TR, T::TC>(p, flags, total, s);
 }
 template <class TA, class TB>
 int launch_bwd_split_both(LogBwdArgs pa, LogBwdArgs pb, const float* stats, int B, hipStream_t s) {
   const int M = pa.M, K = pa.K, N = pa.N;
-  pa.tiles_r = M / TA::TR; pa.tiles_c = K / TA::TC;
-  pb.tiles_r = K / TB::TR; pb.tiles_c = N / TB::TC;
+  pa.tiles_r = ceil_div(M, TA::TR); pa.tiles_c = ceil_div(K, TA::TC);
+  pb.tiles_r = ceil_div(K, TB::TR); pb.tiles_c = ceil_div(N, TB::TC);
   const int64_t ta = (int64_t)B * pa.tiles_r * pa.tiles_c, tb = (int64_t)B * pb.tiles_r * pb.tiles_c;
   if (ta + tb > 0x7fffffffLL) return GENBMM_E_SHAPE;
   const int* hdr = prepared_of(stats, B, M, K, N).hdr;
   const int* ff = fwd_flags_of(stats, B, M, N);
   constexpr int lds = split_bwd_lds_bytes<TA, TB>();
-  allow_lds(k_log_bwd_split_both<TA, TB>, lds);
-  hipLaunchKernelGGL((k_log_bwd_split_both<TA, TB>), dim3((unsigned)(ta + tb)), dim3(TA::NT), lds, s, pa.g,
-                     LeanSrc{pa.a, pa.b, pa.out, stats}, hdr, ff, pa.grad, pb.grad, M, K, N, pa.tiles_r, pa.tiles_c,
-                     pb.tiles_r, pb.tiles_c);
+  auto go = [&](auto kern) {
+    allow_lds(kern, lds);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(ta + tb)), dim3(TA::NT), lds, s, pa.g, LeanSrc{pa.a, pa.b, pa.out, stats},
+                       hdr, ff, pa.grad, pb.grad, M, K, N, pa.tiles_r, pa.tiles_c, pb.tiles_r, pb.tiles_c);
+  };
+  const bool ragged = M % TA::TR != 0 || K % TA::TC != 0 || K % TB::TR != 0 || N % TB::TC != 0;
+  if (ragged) go(k_log_bwd_split_both<TA, TB, true>);
+  else go(k_log_bwd_split_both<TA, TB, false>);
   if (int e = launch_status()) return e;
   hipLaunchKernelGGL((k_log_bwd_fixup_both<BCfgWide, TA::TR, TA::TC, TB::TR, TB::TC>),
                      dim3((unsigned)std::min<int64_t>(ta + tb, kFixupGrid)), dim3(BCfgWide::NT), 0, s, pa, pb, hdr, ff,
@@ -977,8 +988,8 @@ int run_fwd(const elem_t* a, const elem_t* b, elem_t* out, float* stats, int B, 
     switch (fwd_mfma_shape(B, M, K, N) ? mfma_kind(path, B, M, N, K, false) : 0) {
       case 2:
         if (!keep && split_path(path)) {
-          if (split_fits<MTBig>(B, M, N, K, true)) return launch_fwd_split<MTBig>(p, stats, B, M, K, N, s);
-          if (split_fits<MTTall>(B, M, N, K, false)) return launch_fwd_split<MTTall>(p, stats, B, M, K, N, s);
+          if (split_big_fits(B, M, N)) return launch_fwd_split<MTBig>(p, stats, B, M, K, N, s);
+          return launch_fwd_split<MTTall>(p, stats, B, M, K, N, s);
         }
         return launch_fwd_mfma<MTTall>(p, stats, B, M, K, N, keep, s);
       case 1: return launch_fwd_mfma<MT128>(p, stats, B, M, K, N, keep, s);
@@ -1046,11 +1057,12 @@ int run_bwd_both(const elem_t* a, const elem_t* b, const elem_t* out, const elem
       pa.grad = grad_a;
       pb.grad = grad_b;
       const bool lean = path != GENBMM_PATH_FACTORS;
-      if (ka == 2 && lean && split_path(path)) {
-        if (split_fits<MTBig>(B, M, K, N, true) && split_fits<MTBig>(B, K, N, M, true))
+      // (the three-part backward takes output extents of any size but reductions - N, M - of whole
+      //  slabs and rows of K in whole pieces of four; the forward takes any sizes)
+      if (ka == 2 && lean && split_path(path) && M % kMS == 0 && N % kMS == 0 && K % 4 == 0) {
+        if (split_big_fits(B, M, K) && split_big_fits(B, K, N))
           return launch_bwd_split_both<MTBig, MTBig>(pa, pb, st, B, s);
-        if (split_fits<MTWide>(B, M, K, N, false) && split_fits<MTTall>(B, K, N, M, false))
-          return launch_bwd_split_both<MTWide, MTTall>(pa, pb, st, B, s);
+        return launch_bwd_split_both<MTWide, MTTall>(pa, pb, st, B, s);
       }
       return ka == 2 ? launch_bwd_mfma_both<MTWide, MTTall>(pa, pb, st, B, s, lean)
                      : launch_bwd_mfma_both<MT128, MT128>(pa, pb, st, B, s, lean);

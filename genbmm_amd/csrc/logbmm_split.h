@@ -11,8 +11,11 @@
 // Same tiles, guards, flags, epilogues and fix-up launches as the fp32 kernels of
 // logbmm_mfma.h (a 64 x 64 block per wave as 2 x 2 accumulators, whose layout is that of
 // the fp32 instruction; reduction in slabs of 16 through two LDS buffers); what differs is
-// the staged form and the inner loop.  Full tiles only (every extent a multiple of its
-// tile, the reduction of 16): other shapes stay on the fp32 instruction.
+// the staged form and the inner loop.  Any sizes: ragged edges are a second instantiation
+// of each kernel (RAGGED), handled as in logbmm_mfma.h - lines of a tile beyond the matrix
+// re-read the last line with a shift that makes the factor vanish, pieces that straddle the
+// right edge are read element by element, the reduction tail is filled by the loader of the
+// last slab, stores are masked.
 //
 // LDS layouts, three planes (h, m, l) per operand, words of two bf16:
 //  * an operand whose source is [line][reduction] (reduction contiguous): plane[line][8
@@ -131,6 +134,18 @@ __device__ __forceinline__ void ldw(const elem_t* p, float (&v)[LW]) {
   }
 }
 
+// the first cnt of them (<= 0: none), `fill` for the rest
+template <int LW>
+__device__ __forceinline__ void ldwm(const elem_t* p, int cnt, float fill, float (&v)[LW]) {
+  if (cnt >= LW) {
+    ldw<LW>(p, v);
+    return;
+  }
+#pragma unroll
+  for (int j = 0; j < LW; ++j) v[j] = j < cnt ? (float)p[j] : fill;
+}
+__device__ __forceinline__ int clampw(int x, int w) { return min(max(x, 0), w); }
+
 __device__ __forceinline__ floatx16 mfma_bf16(bf16x8 a, bf16x8 b, floatx16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
@@ -230,7 +245,7 @@ __device__ __forceinline__ bool split_early(int wave) { return wave >= NT / 128;
 // ----------------------------------------------------------------- forward
 // rows <- EA from a[m][k] ([line][reduction]), columns <- EB from b[k][n] ([reduction][line]).
 // Leaves the maxima, the tile flags and the header (no factors), like k_log_fwd_mfma<T, false, false>.
-template <class T>
+template <class T, bool RAGGED>
 __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WPE, T::WPE)))
 void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b, elem_t* __restrict__ out,
                      const float* __restrict__ stats, int* __restrict__ flags, int* __restrict__ ws_hdr, int M,
@@ -251,19 +266,24 @@ void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
   const int m0 = (rem / tiles_n) * T::TR, n0 = (rem % tiles_n) * T::TC;
   const float* st = stats + (long)batch * (M + N);
 
+  // a pieces: line m0 + line(l), four k from quad * 4;  the b piece: rows 2 pair, 2 pair + 1 of the
+  // slab, LW columns from bcol
   const elem_t* pa[SA::PER];
   float al[SA::PER];
 #pragma unroll
   for (int l = 0; l < SA::PER; ++l) {
     const int line = m0 + SA::line(tid, l);
-    pa[l] = a + ((long)batch * M + line) * K + SA::quad(tid) * 4;
-    al[l] = st[line];
+    const bool in = !RAGGED || line < M;
+    pa[l] = a + ((long)batch * M + (in ? line : M - 1)) * K + SA::quad(tid) * 4;
+    al[l] = in ? st[line] : INFINITY;  // lines beyond the matrix: exp -> 0
   }
   const int bcol = n0 + SB::line0(tid);
-  const elem_t* pb = b + ((long)batch * K + 2 * SB::pair(tid)) * N + bcol;
+  const int cb = RAGGED ? clampw(N - bcol, LW) : LW;  // columns of the b piece inside the matrix
+  const int brow = 2 * SB::pair(tid);
+  const elem_t* pb = b + ((long)batch * K + brow) * N + (cb > 0 ? bcol : 0);
   float be[LW];
 #pragma unroll
-  for (int j = 0; j < LW; ++j) be[j] = st[M + bcol + j];
+  for (int j = 0; j < LW; ++j) be[j] = j < cb ? st[M + bcol + j] : INFINITY;
   if (tile == 0 && tid == 0) {
     ws_hdr[1] = T::TR;
     ws_hdr[2] = T::TC;
@@ -276,18 +296,33 @@ void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[x >> 1][x & 1][i] = 0.f;
 
-  const int slabs = K / kMS;
+  const int ktail = RAGGED ? K % kMS : 0;          // reduction steps of a partial last slab
+  const int slabs = RAGGED ? (K + kMS - 1) / kMS : K / kMS;
+  int s_load = 0;                                  // the slab the next load() fetches
   float4 ra[SA::PER];
   float rbe[LW], rbo[LW];
   auto load = [&]() __attribute__((always_inline)) {
+    if (RAGGED && ktail != 0 && s_load == slabs - 1) {
+      const int ca = clamp4(ktail - SA::quad(tid) * 4);
 #pragma unroll
-    for (int l = 0; l < SA::PER; ++l) {
-      ra[l] = ld4(pa[l]);
-      pa[l] += kMS;
+      for (int l = 0; l < SA::PER; ++l) ra[l] = ld4m(pa[l], ca, -INFINITY);
+      ldwm<LW>(pb, brow < ktail ? cb : 0, -INFINITY, rbe);
+      ldwm<LW>(pb + N, brow + 1 < ktail ? cb : 0, -INFINITY, rbo);
+    } else {
+#pragma unroll
+      for (int l = 0; l < SA::PER; ++l) ra[l] = ld4(pa[l]);
+      if (RAGGED) {
+        ldwm<LW>(pb, cb, -INFINITY, rbe);
+        ldwm<LW>(pb + N, cb, -INFINITY, rbo);
+      } else {
+        ldw<LW>(pb, rbe);
+        ldw<LW>(pb + N, rbo);
+      }
     }
-    ldw<LW>(pb, rbe);
-    ldw<LW>(pb + N, rbo);
+#pragma unroll
+    for (int l = 0; l < SA::PER; ++l) pa[l] += kMS;
     pb += (long)kMS * N;
+    ++s_load;
   };
   auto stage = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
@@ -311,21 +346,29 @@ void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
   // no shift below -30 opposite a row or column at the floor
   const float thr = fast_exp2(-kMfmaGuardBits);
   int bad = 0;
+  {
+    const int rlim = M - (m0 + wm0) - mfma_row_l(lane);   // rows of this lane below rlim exist
+    const int clim = N - (n0 + wn0) - (lane & 31);        // column blocks at offset < clim exist
 #pragma unroll
-  for (int x = 0; x < 4; ++x)
+    for (int x = 0; x < 4; ++x)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const float s = acc[x >> 1][x & 1][i];
-      if (!((s >= thr) && (s < INFINITY))) bad = 1;
-    }
+      for (int i = 0; i < 16; ++i) {
+        const float s = acc[x >> 1][x & 1][i];
+        const bool here = !RAGGED || ((x >> 1) * 32 + mfma_row_u(i) < rlim && (x & 1) * 32 < clim);
+        if (here && !((s >= thr) && (s < INFINITY))) bad = 1;
+      }
+  }
   static_assert(T::TR + T::TC <= NT, "one shift per thread");
   int low = 0, neg = 0;  // bit 0: of a row, bit 1: of a column
-  if (tid < T::TR + T::TC) {
+  {
     const bool row = tid < T::TR;
-    const float sh = row ? st[m0 + tid] : st[M + n0 + tid - T::TR];
-    if (!((sh >= kFloor) && (sh < INFINITY))) bad = 1;
-    if (sh <= 0.45f * kFloor) low = row ? 1 : 2;
-    if (sh < -30.f) neg = row ? 1 : 2;
+    const bool here = tid < T::TR + T::TC && (!RAGGED || (row ? m0 + tid < M : n0 + tid - T::TR < N));
+    if (here) {
+      const float sh = row ? st[m0 + tid] : st[M + n0 + tid - T::TR];
+      if (!((sh >= kFloor) && (sh < INFINITY))) bad = 1;
+      if (sh <= 0.45f * kFloor) low = row ? 1 : 2;
+      if (sh < -30.f) neg = row ? 1 : 2;
+    }
   }
   const int row_low = __syncthreads_or(low & 1), col_low = __syncthreads_or(low & 2);
   if (row_low | col_low) {  // uniform, and rare
@@ -338,19 +381,24 @@ void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
 
   // out = log S + alpha + beta, written row-wise
   const int lr = lane >> 4, lc = (lane & 15) * 4;
-  const float4 be4 = ld4(st + M + n0 + wn0 + lc);
+  const int cc = RAGGED ? clamp4(N - (n0 + wn0 + lc)) : 4;  // columns of this lane's pieces that exist
+  const bool cok = cc > 0;
+  const float4 be4 = RAGGED ? ld4m(st + M + (cok ? n0 + wn0 + lc : 0), cc, 0.f) : ld4(st + M + n0 + wn0 + lc);
   const float* alw = st + m0 + wm0 + lr;
   const long ubase = ((long)batch * M + m0 + wm0) * N + n0 + wn0;
   const int voff = lr * N + lc;
+  const int rows_left = M - (m0 + wm0) - lr;
   acc_rows(acc, reinterpret_cast<float*>(split_smem) + wave * kStripFloats, lane, [](int) {},
            [&](int q, int t, float4 sv) __attribute__((always_inline)) {
              const int ru = 16 * q + 4 * t;
+             if (RAGGED && !(cok && ru < rows_left)) return;
              const float alr = alw[ru];
              const float4 ov = make_float4(__builtin_fmaf(fast_log2(sv.x), kLn2, alr + be4.x),
                                            __builtin_fmaf(fast_log2(sv.y), kLn2, alr + be4.y),
                                            __builtin_fmaf(fast_log2(sv.z), kLn2, alr + be4.z),
                                            __builtin_fmaf(fast_log2(sv.w), kLn2, alr + be4.w));
-             st4(out + ubase + (long)ru * N + voff, ov);
+             if (RAGGED) st4m(out + ubase + (long)ru * N + voff, cc, ov);
+             else st4(out + ubase + (long)ru * N + voff, ov);
            });
 }
 
@@ -369,7 +417,7 @@ struct SplitBwd {
   static constexpr int WORDS = split_lds_words<SR, SC>();
 };
 
-template <class T, bool GRAD_A>
+template <class T, bool GRAD_A, bool RAGGED>
 __device__ __forceinline__ void log_bwd_split_tile(unsigned* __restrict__ smem, int tile, const elem_t* __restrict__ g,
                                                    const LeanSrc src, const int* __restrict__ ws_hdr,
                                                    const int* __restrict__ fwd_flags, elem_t* __restrict__ grad, int M,
@@ -396,13 +444,16 @@ __device__ __forceinline__ void log_bwd_split_tile(unsigned* __restrict__ smem, 
   for (int x = 0; x < 4; ++x)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[x >> 1][x & 1][i] = 0.f;
-  const int slabs = Q / kMS;
+  const int slabs = Q / kMS;  // (the backward takes reductions of whole slabs only)
 
   // Addresses are a base per workgroup (scalar registers, stepped slab by slab) plus a fixed
   // 32-bit offset per thread: the vector registers go to operands and accumulators.
+  // RAGGED: output extents of any size (K a multiple of four); the reductions - N for grad_a, M for
+  // grad_b - are multiples of the slab (other shapes run their backward on the fp32 instruction).
   if constexpr (GRAD_A) {
     // rows: H pieces (line m, four n); columns: EB pieces (line k, four n); beta of the slab's four
-    // columns is the same for every piece of a thread (all share their quad)
+    // columns is the same for every piece of a thread (all share their quad).  Lines beyond the
+    // matrix re-read the last line: they only feed results that are not stored.
     const elem_t* ob = src.out + (long)batch * M * N;
     const elem_t* gb = g + (long)batch * M * N;
     const elem_t* bb = src.b + (long)batch * K * N;
@@ -411,12 +462,15 @@ __device__ __forceinline__ void log_bwd_split_tile(unsigned* __restrict__ smem, 
     float alh[SR::PER];
 #pragma unroll
     for (int l = 0; l < SR::PER; ++l) {
-      const int m = r0 + SR::line(tid, l);
+      const int m = RAGGED ? min(r0 + SR::line(tid, l), M - 1) : r0 + SR::line(tid, l);
       oo[l] = m * N + SR::quad(tid) * 4;
       alh[l] = al[m];
     }
 #pragma unroll
-    for (int l = 0; l < SC::PER; ++l) yo[l] = (c0 + SC::line(tid, l)) * N + SC::quad(tid) * 4;
+    for (int l = 0; l < SC::PER; ++l) {
+      const int k = RAGGED ? min(c0 + SC::line(tid, l), K - 1) : c0 + SC::line(tid, l);
+      yo[l] = k * N + SC::quad(tid) * 4;
+    }
     const int beo = SR::quad(tid) * 4;
     float4 ro[SR::PER], rg[SR::PER], ry[SC::PER], bslab;
     auto load = [&]() __attribute__((always_inline)) {
@@ -447,7 +501,8 @@ __device__ __forceinline__ void log_bwd_split_tile(unsigned* __restrict__ smem, 
     });
   } else {
     // rows: EA pieces (steps m, m + 1; LW lines k); columns: H pieces (steps m, m + 1; LW lines n);
-    // both operands' pieces of a thread are on the same pair of steps
+    // both operands' pieces of a thread are on the same pair of steps.  RAGGED: lines beyond the
+    // matrix re-read the last LW lines - they only feed results that are not stored.
     constexpr int LR = SR::LW, LC = SC::LW;
     static_assert(SR::Q == SC::Q, "");
     const int m2 = 2 * SR::pair(tid);
@@ -455,10 +510,12 @@ __device__ __forceinline__ void log_bwd_split_tile(unsigned* __restrict__ smem, 
     const elem_t* ob = src.out + (long)batch * M * N;
     const elem_t* gb = g + (long)batch * M * N;
     const float* alb = al;
-    const int yo = m2 * K + r0 + SR::line0(tid), oo = m2 * N + c0 + SC::line0(tid);
+    const int kc = RAGGED ? min(r0 + SR::line0(tid), K - LR) : r0 + SR::line0(tid);
+    const int nc = RAGGED ? min(c0 + SC::line0(tid), N - LC) : c0 + SC::line0(tid);
+    const int yo = m2 * K + kc, oo = m2 * N + nc;
     float bec[LC];
 #pragma unroll
-    for (int j = 0; j < LC; ++j) bec[j] = be[c0 + SC::line0(tid) + j];
+    for (int j = 0; j < LC; ++j) bec[j] = be[nc + j];
     float ye[LR], yd[LR], oe[LC], od[LC], ge[LC], gd[LC];
     float a0, a1;
     auto load = [&]() __attribute__((always_inline)) {
@@ -468,7 +525,8 @@ __device__ __forceinline__ void log_bwd_split_tile(unsigned* __restrict__ smem, 
       ldw<LC>(ob + oo + N, od);
       ldw<LC>(gb + oo, ge);
       ldw<LC>(gb + oo + N, gd);
-      a0 = alb[m2]; a1 = alb[m2 + 1];
+      a0 = alb[m2];
+      a1 = alb[m2 + 1];
       ab += (long)kMS * K;
       ob += (long)kMS * N;
       gb += (long)kMS * N;
@@ -503,31 +561,40 @@ __device__ __forceinline__ void log_bwd_split_tile(unsigned* __restrict__ smem, 
   const long ubase = ((long)batch * R + r0 + wr0) * Cc + c0 + wc0;
   const elem_t* xb = (GRAD_A ? src.a : src.b) + ubase + voff;
   elem_t* gp = grad + ubase + voff;
+  const int cc = RAGGED ? clamp4(Cc - (c0 + wc0 + lc)) : 4;
+  const bool cok = cc > 0;
+  const int rows_left = R - (r0 + wr0) - lr;
   float4 becol = make_float4(0.f, 0.f, 0.f, 0.f);
-  if constexpr (!GRAD_A) becol = ld4(be + c0 + wc0 + lc);
+  if constexpr (!GRAD_A) becol = RAGGED ? ld4m(be + (cok ? c0 + wc0 + lc : 0), cc, 0.f) : ld4(be + c0 + wc0 + lc);
   const float* alrow = al + r0 + wr0 + lr;
   float4 xq[2][4];
   float xa[2][4];
   auto fetch = [&](int q) __attribute__((always_inline)) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      xq[q & 1][t] = ld4(xb + (long)(16 * q + 4 * t) * Cc);
-      if constexpr (GRAD_A) xa[q & 1][t] = alrow[16 * q + 4 * t];
+      const bool live = !RAGGED || (cok && 16 * q + 4 * t < rows_left);
+      if (live) {
+        xq[q & 1][t] = RAGGED ? ld4m(xb + (long)(16 * q + 4 * t) * Cc, cc, -INFINITY) : ld4(xb + (long)(16 * q + 4 * t) * Cc);
+        if constexpr (GRAD_A) xa[q & 1][t] = alrow[16 * q + 4 * t];
+      }
     }
   };
   fetch(0);
   acc_rows(acc, reinterpret_cast<float*>(smem) + wave * kStripFloats, lane,
            [&](int q) __attribute__((always_inline)) { if (q + 1 < 4) fetch(q + 1); },
            [&](int q, int t, float4 v) __attribute__((always_inline)) {
+             if (RAGGED && !(cok && 16 * q + 4 * t < rows_left)) return;
              float4 x;
              if constexpr (GRAD_A) x = exp4(xq[q & 1][t], xa[q & 1][t]);
              else x = exp4(xq[q & 1][t], becol);
-             st4(gp + (long)(16 * q + 4 * t) * Cc, make_float4(x.x * v.x, x.y * v.y, x.z * v.z, x.w * v.w));
+             const float4 r = make_float4(x.x * v.x, x.y * v.y, x.z * v.z, x.w * v.w);
+             if (RAGGED) st4m(gp + (long)(16 * q + 4 * t) * Cc, cc, r);
+             else st4(gp + (long)(16 * q + 4 * t) * Cc, r);
            });
 }
 
 // Both gradients in one launch, item by item, a tile of each in turn (see k_log_bwd_mfma_both).
-template <class TA, class TB>
+template <class TA, class TB, bool RAGGED>
 __global__ __launch_bounds__(TA::NT) __attribute__((amdgpu_waves_per_eu(TA::WPE, TA::WPE)))
 void k_log_bwd_split_both(const elem_t* __restrict__ g, const LeanSrc src, const int* __restrict__ ws_hdr,
                           const int* __restrict__ fwd_flags, elem_t* __restrict__ grad_a,
@@ -541,9 +608,9 @@ void k_log_bwd_split_both(const elem_t* __restrict__ g, const LeanSrc src, const
   const bool is_a = alt ? (r & 1) == 0 : r < per_a;
   const int idx = alt ? r >> 1 : (r < per_a ? r : r - per_a);
   if (is_a)
-    log_bwd_split_tile<TA, true>(split_smem, item * per_a + idx, g, src, ws_hdr, fwd_flags, grad_a, M, K, N, ar, ac);
+    log_bwd_split_tile<TA, true, RAGGED>(split_smem, item * per_a + idx, g, src, ws_hdr, fwd_flags, grad_a, M, K, N, ar, ac);
   else
-    log_bwd_split_tile<TB, false>(split_smem, item * per_b + idx, g, src, ws_hdr, fwd_flags, grad_b, M, K, N, br, bc);
+    log_bwd_split_tile<TB, false, RAGGED>(split_smem, item * per_b + idx, g, src, ws_hdr, fwd_flags, grad_b, M, K, N, br, bc);
 }
 
 template <class TA, class TB>

@@ -254,11 +254,15 @@ def test_logbmm_rows_masked_at_the_floor(gpu, keep, B, M, K, N):
     assert bool(torch.isfinite(ga[ok.to(gpu)]).all()) and bool(torch.isfinite(gb[ok.to(gpu)]).all())
 
 
-@pytest.mark.parametrize("B,M,K,N", [(64, 512, 256, 512), (64, 512, 512, 384), (64, 512, 512, 512), (48, 768, 64, 512)])
+@pytest.mark.parametrize("B,M,K,N", [(64, 512, 256, 512), (64, 512, 512, 384), (64, 512, 512, 512), (48, 768, 64, 512),
+                                     (64, 500, 300, 500), (64, 500, 500, 300), (64, 509, 253, 499), (64, 1000, 250, 300),
+                                     (64, 496, 500, 496), (64, 496, 508, 304), (40, 1008, 252, 400)])
 def test_logbmm_three_part_kernels(gpu, B, M, K, N):
-    """Shapes made of full tiles, which the default path runs on the bf16 matrix instruction with
+    """Shapes which the default path runs on the bf16 matrix instruction with
     every factor cut into three bf16 parts (256 x 256 tiles where they fill the chip, 256 x 128 /
-    128 x 256 otherwise; forward and backward switch independently): every batch item against
+    128 x 256 otherwise; forward and backward switch independently; the last seven with ragged
+    edges - partial tiles, partial slabs, odd row lengths; the backward takes ragged output extents
+    where its reductions, M and N, are multiples of 16 - the last three): every batch item against
     float64 on the device, among them items whose tiles must take the exact routine (factors that
     underflow against live terms: everywhere, and in a single row), an item with rows padded at
     the floor, one with a masked reduction step, one with magnitudes near 1000 - and the whole
