@@ -907,6 +907,7 @@ using MT128 = MTile<128, 128>;
 using MTWide = MTile<128, 256>;  // grad_a (m x k)
 using MTTall = MTile<256, 128>;  // forward (m x n; measured 1-2 % ahead of 128x256) and grad_b (k x n)
 using MTBig = MTile<256, 256>;   // sixteen waves, one workgroup per compute unit (the bf16 three-part kernels)
+using MT128S = MTile<128, 128, 2>;  // the three-part kernels' 128 x 128 tile: a thread stages twice as much, 256 registers
 
 template <bool GRAD_A>
 int run_bwd(const LogBwdArgs& p, const float* stats, int path, int B, hipStream_t s) {
@@ -992,7 +993,9 @@ int run_fwd(const elem_t* a, const elem_t* b, elem_t* out, float* stats, int B, 
           return launch_fwd_split<MTTall>(p, stats, B, M, K, N, s);
         }
         return launch_fwd_mfma<MTTall>(p, stats, B, M, K, N, keep, s);
-      case 1: return launch_fwd_mfma<MT128>(p, stats, B, M, K, N, keep, s);
+      case 1:
+        if (!keep && split_path(path)) return launch_fwd_split<MT128S>(p, stats, B, M, K, N, s);
+        return launch_fwd_mfma<MT128>(p, stats, B, M, K, N, keep, s);
       default: break;
     }
     if (M <= 32 && N <= 32) return launch_fwd_fast<CfgSmall, CfgSmall>(p, stats, B, M, K, N, s);
@@ -1059,7 +1062,8 @@ int run_bwd_both(const elem_t* a, const elem_t* b, const elem_t* out, const elem
       const bool lean = path != GENBMM_PATH_FACTORS;
       // (the three-part backward takes output extents of any size but reductions - N, M - of whole
       //  slabs and rows of K in whole pieces of four; the forward takes any sizes)
-      if (ka == 2 && lean && split_path(path) && M % kMS == 0 && N % kMS == 0 && K % 4 == 0) {
+      if (lean && split_path(path) && M % kMS == 0 && N % kMS == 0 && K % 4 == 0) {
+        if (ka == 1) return launch_bwd_split_both<MT128S, MT128S>(pa, pb, st, B, s);
         if (split_big_fits(B, M, K) && split_big_fits(B, K, N))
           return launch_bwd_split_both<MTBig, MTBig>(pa, pb, st, B, s);
         return launch_bwd_split_both<MTWide, MTTall>(pa, pb, st, B, s);
