@@ -121,8 +121,9 @@ size_t genbmm_samplebmm_stats_size(int B, int M, int K, int N);
 /*
  * The same two functions with the kernel family named per call (tests and
  * measurements; the plain functions are GENBMM_PATH_AUTO).
- *   GENBMM_PATH_AUTO   whole-item kernels for matrices up to 64^3, the fp32
- *                      matrix cores where the shape allows, else the factored
+ *   GENBMM_PATH_AUTO   whole-item kernels for matrices up to 64^3, the matrix
+ *                      cores where the shape allows (every extent at least
+ *                      96, or items of one 128 x 128 tile), else the factored
  *                      kernels on the vector ALU;
  *   GENBMM_PATH_EXACT  the online / exp-per-term kernels only (what a NULL
  *                      `stats` gives; a non-NULL one still receives the maxima);
@@ -141,14 +142,15 @@ size_t genbmm_samplebmm_stats_size(int B, int M, int K, int N);
  * forward writes 200 MB less, the backward takes three exponentials per staged
  * element).  With float16 / bfloat16 tensors that backward reads `out` as stored
  * (rounded); FACTORS keeps 1 / sum in fp32.
- *   GENBMM_PATH_MFMA32 as AUTO, but the tiled matrix-core kernels use the fp32
- *                      matrix instruction for every shape.  Under AUTO,
- *                      problems made of full tiles (M and K multiples of 256,
- *                      N of 128) run on the bf16 matrix instruction with every
- *                      factor cut into three bf16 parts that add up to it
- *                      exactly and six partial products per product - what is
+ *   GENBMM_PATH_MFMA32 as AUTO, but the matrix-core kernels use the fp32 matrix
+ *                      instruction.  Under AUTO they run on the bf16 matrix
+ *                      instruction with every factor cut into three bf16
+ *                      parts that add up to it exactly and six partial
+ *                      products per product, accumulated in fp32 - what is
  *                      dropped is below 2^-23 of a product, one fp32 rounding -
- *                      at 2.7 times less matrix-pipe time.
+ *                      at 2.7 times less matrix-pipe time (the forward for any
+ *                      sizes; the backward where M and N are multiples of 16
+ *                      and K of 4, else it stays on the fp32 instruction).
  * Any other value: GENBMM_E_MODE.  Forward and backward of one problem need not
  * name the same path (see genbmm_logbmm_bwd).  No counterpart in the reference.
  */
