@@ -879,7 +879,8 @@ int launch_bwd_split_both(LogBwdArgs pa, LogBwdArgs pb, const float* stats, int 
     hipLaunchKernelGGL(kern, dim3((unsigned)(ta + tb)), dim3(TA::NT), lds, s, pa.g, LeanSrc{pa.a, pa.b, pa.out, stats},
                        hdr, ff, pa.grad, pb.grad, M, K, N, pa.tiles_r, pa.tiles_c, pb.tiles_r, pb.tiles_c);
   };
-  const bool ragged = M % TA::TR != 0 || K % TA::TC != 0 || K % TB::TR != 0 || N % TB::TC != 0;
+  const bool ragged = M % TA::TR != 0 || K % TA::TC != 0 || K % TB::TR != 0 || N % TB::TC != 0 || N % kMS != 0 ||
+                      M % kMS != 0;
   if (ragged) go(k_log_bwd_split_both<TA, TB, true>);
   else go(k_log_bwd_split_both<TA, TB, false>);
   if (int e = launch_status()) return e;
@@ -1060,9 +1061,8 @@ int run_bwd_both(const elem_t* a, const elem_t* b, const elem_t* out, const elem
       pa.grad = grad_a;
       pb.grad = grad_b;
       const bool lean = path != GENBMM_PATH_FACTORS;
-      // (the three-part backward takes output extents of any size but reductions - N, M - of whole
-      //  slabs and rows of K in whole pieces of four; the forward takes any sizes)
-      if (lean && split_path(path) && M % kMS == 0 && N % kMS == 0 && K % 4 == 0) {
+      // (the three-part backward takes any M, and K and N in whole pieces of four; the forward any sizes)
+      if (lean && split_path(path) && N % 4 == 0 && K % 4 == 0) {
         if (ka == 1) return launch_bwd_split_both<MT128S, MT128S>(pa, pb, st, B, s);
         if (split_big_fits(B, M, K) && split_big_fits(B, K, N))
           return launch_bwd_split_both<MTBig, MTBig>(pa, pb, st, B, s);

@@ -444,12 +444,16 @@ __device__ __forceinline__ void log_bwd_split_tile(unsigned* __restrict__ smem, 
   for (int x = 0; x < 4; ++x)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[x >> 1][x & 1][i] = 0.f;
-  const int slabs = Q / kMS;  // (the backward takes reductions of whole slabs only)
+  const int slabs = Q / kMS;                // whole slabs: the loop
+  const int qtail = RAGGED ? Q % kMS : 0;   // reduction steps of a partial last slab: one more step behind the
+                                            // loop, with a loader of its own (inside the loop's loader it cost
+                                            // 19 spilled registers and the kernel ran 1.7 times slower)
 
   // Addresses are a base per workgroup (scalar registers, stepped slab by slab) plus a fixed
   // 32-bit offset per thread: the vector registers go to operands and accumulators.
-  // RAGGED: output extents of any size (K a multiple of four); the reductions - N for grad_a, M for
-  // grad_b - are multiples of the slab (other shapes run their backward on the fp32 instruction).
+  // RAGGED: any M; K and N multiples of four, so that no piece straddles the right edge of its
+  // matrix (other shapes run their backward on the fp32 instruction).  Fills of the partial last
+  // slab make a factor vanish: -inf for a and b, +inf for out, 0 for g.
   if constexpr (GRAD_A) {
     // rows: H pieces (line m, four n); columns: EB pieces (line k, four n); beta of the slab's four
     // columns is the same for every piece of a thread (all share their quad).  Lines beyond the
@@ -499,6 +503,21 @@ __device__ __forceinline__ void log_bwd_split_tile(unsigned* __restrict__ smem, 
     split_loop(slabs, split_early<NT>(wave), load, stage, [&](int buf) __attribute__((always_inline)) {
       split_slab<SR, SC>(Rs(buf), Cs(buf), wr0, wc0, wave, lane, acc);
     });
+    if (RAGGED && qtail != 0) {  // uniform
+      const int left = qtail - beo;  // all pieces of a thread share their quad
+#pragma unroll
+      for (int l = 0; l < SC::PER; ++l) ry[l] = ld4m(bb + yo[l], left, -INFINITY);
+#pragma unroll
+      for (int l = 0; l < SR::PER; ++l) {
+        ro[l] = ld4m(ob + oo[l], left, INFINITY);
+        rg[l] = ld4m(gb + oo[l], left, 0.f);
+      }
+      bslab = ld4m(beb + beo, left, 0.f);
+      stage(0);
+      __syncthreads();
+      split_slab<SR, SC>(Rs(0), Cs(0), wr0, wc0, wave, lane, acc);
+      __syncthreads();
+    }
   } else {
     // rows: EA pieces (steps m, m + 1; LW lines k); columns: H pieces (steps m, m + 1; LW lines n);
     // both operands' pieces of a thread are on the same pair of steps.  RAGGED: lines beyond the
@@ -553,6 +572,32 @@ __device__ __forceinline__ void log_bwd_split_tile(unsigned* __restrict__ smem, 
     split_loop(slabs, split_early<NT>(wave), load, stage, [&](int buf) __attribute__((always_inline)) {
       split_slab<SR, SC>(Rs(buf), Cs(buf), wr0, wc0, wave, lane, acc);
     });
+    if (RAGGED && qtail != 0) {  // uniform; steps beyond M re-read row M - 1 and are replaced by the fills
+      const int c0r = min(m2, qtail - 1), c1r = min(m2 + 1, qtail - 1);
+      ldw<LR>(ab + c0r * K + kc, ye);
+      ldw<LR>(ab + c1r * K + kc, yd);
+      ldw<LC>(ob + c0r * N + nc, oe);
+      ldw<LC>(ob + c1r * N + nc, od);
+      ldw<LC>(gb + c0r * N + nc, ge);
+      ldw<LC>(gb + c1r * N + nc, gd);
+      a0 = alb[c0r];
+      a1 = alb[c1r];
+      const bool in0 = m2 < qtail, in1 = m2 + 1 < qtail;
+#pragma unroll
+      for (int j = 0; j < LR; ++j) {
+        ye[j] = in0 ? ye[j] : -INFINITY;
+        yd[j] = in1 ? yd[j] : -INFINITY;
+      }
+#pragma unroll
+      for (int j = 0; j < LC; ++j) {
+        ge[j] = in0 ? ge[j] : 0.f;
+        gd[j] = in1 ? gd[j] : 0.f;
+      }
+      stage(0);
+      __syncthreads();
+      split_slab<SR, SC>(Rs(0), Cs(0), wr0, wc0, wave, lane, acc);
+      __syncthreads();
+    }
   }
 
   // grad = EX * acc with EX = exp(a - alpha) (grad_a) or exp(b - beta) (grad_b), row-wise

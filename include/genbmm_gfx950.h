@@ -149,8 +149,8 @@ size_t genbmm_samplebmm_stats_size(int B, int M, int K, int N);
  *                      products per product, accumulated in fp32 - what is
  *                      dropped is below 2^-23 of a product, one fp32 rounding -
  *                      at 2.7 times less matrix-pipe time (the forward for any
- *                      sizes; the backward where M and N are multiples of 16
- *                      and K of 4, else it stays on the fp32 instruction).
+ *                      sizes; the backward where K and N are multiples of 4,
+ *                      else it stays on the fp32 instruction).
  * Any other value: GENBMM_E_MODE.  Forward and backward of one problem need not
  * name the same path (see genbmm_logbmm_bwd).  No counterpart in the reference.
  */

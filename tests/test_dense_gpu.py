@@ -261,8 +261,8 @@ def test_logbmm_three_part_kernels(gpu, B, M, K, N):
     """Shapes which the default path runs on the bf16 matrix instruction with
     every factor cut into three bf16 parts (256 x 256 tiles where they fill the chip, 256 x 128 /
     128 x 256 otherwise; forward and backward switch independently; the last seven with ragged
-    edges - partial tiles, partial slabs, odd row lengths; the backward takes ragged output extents
-    where its reductions, M and N, are multiples of 16 - the last three): every batch item against
+    edges - partial tiles, partial slabs, odd row lengths; the backward takes any M, and K and N in
+    multiples of four): every batch item against
     float64 on the device, among them items whose tiles must take the exact routine (factors that
     underflow against live terms: everywhere, and in a single row), an item with rows padded at
     the floor, one with a masked reduction step, one with magnitudes near 1000 - and the whole
