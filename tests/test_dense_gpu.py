@@ -305,6 +305,37 @@ def test_logbmm_three_part_kernels(gpu, B, M, K, N):
         close_on_device(x, y.double(), "against the fp32 matrix instruction", rtol=2e-5, atol=2e-5)
 
 
+def test_logbmm_matrix_core_shape_sweep(gpu):
+    """A seeded sweep of 48 shapes around the switching points of the matrix-core kernels (tile forms
+    256 x 256 / 256 x 128 / 128 x 128, full and ragged, extents in multiples of 16, of 4 and odd -
+    the backward takes the bf16 instruction for K and N in multiples of four, else the fp32 one):
+    the default path against float64 on the device, and against GENBMM_PATH_MFMA32."""
+    rng = np.random.RandomState(7)
+    shapes = []
+    for i in range(48):
+        step = (16, 4, 1)[i % 3]
+        M, K, N = (int(rng.randint(96 // step, 700 // step + 1)) * step for _ in range(3))
+        B = int(rng.choice([1, 3, 8, 24, 64]))
+        if B * M * N > 64 * 512 * 512:
+            B = max(1, (64 * 512 * 512) // (M * N))
+        shapes.append((B, M, K, N))
+    shapes += [(64, 256, 96, 512), (24, 512, 16, 768), (5, 1024, 272, 256)]
+    for B, M, K, N in shapes:
+        torch.manual_seed(M * 7 + N)
+        a, b, g = (torch.randn(B, M, K, device=gpu), torch.randn(B, K, N, device=gpu), torch.randn(B, M, N, device=gpu))
+        res = []
+        for path in (genmul.PATH_AUTO, genmul.PATH_MFMA32):
+            ad, bd = a.clone().requires_grad_(True), b.clone().requires_grad_(True)
+            out = genmul.logbmm_on_path(ad, bd, path)
+            res.append((out.detach(),) + torch.autograd.grad(out, (ad, bd), g))
+        pick = slice(0, min(B, 4))
+        want = oracle.logbmm_grads64(a[pick], b[pick], g[pick])
+        for x, y, w, what in zip(res[0], res[1], want, ("out", "grad_a", "grad_b")):
+            close_on_device(x[pick], w, "%s of %s" % (what, (B, M, K, N)))
+            close_on_device(x, y.double(), "%s of %s against the fp32 matrix instruction" % (what, (B, M, K, N)),
+                            rtol=2e-5, atol=2e-5)
+
+
 @pytest.mark.parametrize("B,M,K,N", [(20, 128, 128, 128), (17, 100, 70, 128), (12, 64, 128, 65), (9, 127, 99, 101)])
 def test_logbmm_one_tile_items(gpu, B, M, K, N):
     """Items of at most 128 in every extent: one workgroup per item (and gradient) that
