@@ -705,7 +705,7 @@ int launch_fwd_mfma(DenseArgs p, float* stats, int B, int M, int K, int N, bool 
 template <class TF>
 int launch_sample_sweep_mfma(DenseArgs p, const float* stats, int* flags, int B, int M, int K, int N,
                              hipStream_t s) {
-  using T = MTile<128, 128>;
+  using T = MTile<128, 128, 2>;
   p.M = M; p.K = K; p.N = N;
   const int tiles_m = ceil_div(M, T::TR), tiles_n = ceil_div(N, T::TC);
   p.tiles_m = ceil_div(M, TF::TR);
@@ -716,7 +716,7 @@ int launch_sample_sweep_mfma(DenseArgs p, const float* stats, int* flags, int B,
   const int64_t total = (int64_t)B * tiles_m * tiles_n;
   if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
   const LogPrepared ws = prepared_of(stats, B, M, K, N);
-  hipLaunchKernelGGL(k_sample_sweep_mfma<T>, dim3((unsigned)total), dim3(T::NT), 0, s, ws.ea, ws.eb,
+  hipLaunchKernelGGL(k_sample_sweep_split<T>, dim3((unsigned)total), dim3(T::NT), 0, s, ws.ea, ws.eb,
                      p.out, stats, flags, ws.r, p.idx, p.seed, p.offset, M, K, N, tiles_m, tiles_n,
                      TF::TR, TF::TC, p.tiles_m, p.tiles_n);
   if (int e = launch_status()) return e;
@@ -842,7 +842,7 @@ inline bool split_big_fits(int B, int out_r, int out_c) {
   return pads_to_256(out_r) && pads_to_256(out_c) && (int64_t)B * ceil_div(out_r, 256) * ceil_div(out_c, 256) >= 192;
 }
 template <class T>
-int launch_fwd_split(DenseArgs p, float* stats, int B, int M, int K, int N, hipStream_t s) {
+int launch_fwd_split(DenseArgs p, float* stats, int B, int M, int K, int N, bool keep, hipStream_t s) {
   p.M = M; p.K = K; p.N = N;
   p.tiles_m = ceil_div(M, T::TR);
   p.tiles_n = ceil_div(N, T::TC);
@@ -854,13 +854,20 @@ int launch_fwd_split(DenseArgs p, float* stats, int B, int M, int K, int N, hipS
   const int total = (int)total64;
   int* flags = fwd_flags_of(stats, B, M, N);
   constexpr int lds = 4 * split_lds_words<SplitT<T::TR, T::NT>, SplitS<T::TC, T::NT>>();
+  const LogPrepared ws = prepared_of(stats, B, M, K, N);
   auto go = [&](auto kern) {
     allow_lds(kern, lds);
-    hipLaunchKernelGGL(kern, dim3(total), dim3(T::NT), lds, s, p.a, p.b, p.out, stats, flags,
-                       prepared_of(stats, B, M, K, N).hdr, M, K, N, p.tiles_m, p.tiles_n);
+    hipLaunchKernelGGL(kern, dim3(total), dim3(T::NT), lds, s, p.a, p.b, p.out, stats, flags, ws.ea, ws.eb, ws.r,
+                       ws.hdr, M, K, N, p.tiles_m, p.tiles_n);
   };
-  if (M % T::TR != 0 || N % T::TC != 0 || K % kMS != 0) go(k_log_fwd_split<T, true>);
-  else go(k_log_fwd_split<T, false>);
+  const bool ragged = M % T::TR != 0 || N % T::TC != 0 || K % kMS != 0;
+  if (keep) {
+    if (ragged) go(k_log_fwd_split<T, true, true>);
+    else go(k_log_fwd_split<T, false, true>);
+  } else {
+    if (ragged) go(k_log_fwd_split<T, true, false>);
+    else go(k_log_fwd_split<T, false, false>);
+  }
   if (int e = launch_status()) return e;
   return launch_fwd_fixup<CfgWide, T::TR, T::TC>(p, flags, total, s);
 }
@@ -989,13 +996,13 @@ int run_fwd(const elem_t* a, const elem_t* b, elem_t* out, float* stats, int B, 
     const int64_t big_tiles = (int64_t)B * ceil_div(M, 128) * ceil_div(N, 128);
     switch (fwd_mfma_shape(B, M, K, N) ? mfma_kind(path, B, M, N, K, false) : 0) {
       case 2:
-        if (!keep && split_path(path)) {
-          if (split_big_fits(B, M, N)) return launch_fwd_split<MTBig>(p, stats, B, M, K, N, s);
-          return launch_fwd_split<MTTall>(p, stats, B, M, K, N, s);
+        if (split_path(path)) {
+          if (split_big_fits(B, M, N)) return launch_fwd_split<MTBig>(p, stats, B, M, K, N, keep, s);
+          return launch_fwd_split<MTTall>(p, stats, B, M, K, N, keep, s);
         }
         return launch_fwd_mfma<MTTall>(p, stats, B, M, K, N, keep, s);
       case 1:
-        if (!keep && split_path(path)) return launch_fwd_split<MT128S>(p, stats, B, M, K, N, s);
+        if (split_path(path)) return launch_fwd_split<MT128S>(p, stats, B, M, K, N, keep, s);
         return launch_fwd_mfma<MT128>(p, stats, B, M, K, N, keep, s);
       default: break;
     }
@@ -1147,7 +1154,9 @@ int log_sample_sweep_mfma(const elem_t* a, const elem_t* b, elem_t* out, int32_t
   int* fl = fwd_flags_of(stats, B, M, N);
   // the forward's tile shape: its flags are indexed by it
   switch (mfma_kind(GENBMM_PATH_AUTO, B, M, N, K, false)) {
-    case 2: return launch_sample_sweep_mfma<MTTall>(p, stats, fl, B, M, K, N, s);
+    case 2:
+      if (split_big_fits(B, M, N)) return launch_sample_sweep_mfma<MTBig>(p, stats, fl, B, M, K, N, s);
+      return launch_sample_sweep_mfma<MTTall>(p, stats, fl, B, M, K, N, s);
     case 1: return launch_sample_sweep_mfma<MT128>(p, stats, fl, B, M, K, N, s);
     default: return GENBMM_E_SHAPE;
   }

@@ -914,172 +914,4 @@ constexpr int kSampleSlabs = 62;
 // much instead (the boundaries between the terms move by 2.4e-7 of the total mass).
 constexpr float kSampleShrink = 1.f - 0x1p-22f;
 
-// (Always the any-size form of the loaders: with this kernel's register budget the
-// full-tile form compiled to spills and measured no faster.)
-template <class T>
-__global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void k_sample_sweep_mfma(const float* __restrict__ ws_ea, const float* __restrict__ ws_eb,
-                         const elem_t* __restrict__ out, const float* __restrict__ stats,
-                         int* __restrict__ flags, float* __restrict__ remw,
-                         int32_t* __restrict__ idx, uint64_t seed, uint64_t offset, int M, int K,
-                         int N, int tiles_m, int tiles_n, int ftr, int ftc, int ftiles_m,
-                         int ftiles_n) {
-  constexpr bool RAGGED = true;
-  constexpr int NT = T::NT, LDR = T::LDR, LDC = T::LDC;
-  using SA = StageT<T::TR, NT, LDR>;
-  using SB = StageS<T::TC, NT, LDC>;
-  __shared__ __attribute__((aligned(16))) float smem[2 * kMS * (LDR + LDC)];
-  float(*As)[kMS * LDR] = reinterpret_cast<float(*)[kMS * LDR]>(smem);
-  float(*Bs)[kMS * LDC] = reinterpret_cast<float(*)[kMS * LDC]>(smem + 2 * kMS * LDR);
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm0 = (wave / T::WC) * 64, wn0 = (wave % T::WC) * 64;
-  const int per = tiles_m * tiles_n, tile = xcd_tile_id();
-  const int batch = tile / per, rem = tile - batch * per;
-  const int m0 = (rem / tiles_n) * T::TR, n0 = (rem % tiles_n) * T::TC;
-  const float* st = stats + (long)batch * (M + N);
-
-  // ---- targets.  First -t = -u * S per cell into `remw`, row by row, four adjacent
-  // cells per lane and step (they share one Philox block when rows are a multiple of
-  // four cells); a rolled loop, its body is long.  Then the accumulators pick their
-  // cells up in the matrix-core layout.
-  // the flags are the forward's, one per tile of ITS shape (ftr x ftc)
-  int* flag = flags + (batch * ftiles_m + m0 / ftr) * ftiles_n + n0 / ftc;
-  const float lim = kMfmaGuardBits * kLn2 + 1e-3f;
-  int bad = *flag;
-  {
-    constexpr int QR = T::TC / 4;  // quads per tile row
-    const bool blocks = (N & 3) == 0;
-#pragma unroll 4
-    for (int q = tid; q < T::TR * QR; q += NT) {
-      const int r = q / QR, m = m0 + r, n = n0 + (q - r * QR) * 4;
-      if (RAGGED && (m >= M || n >= N)) continue;
-      const long cell = ((long)batch * M + m) * N + n;
-      const int cn = RAGGED ? clamp4(N - n) : 4;
-      float u[4];
-      philox_uniform4((uint64_t)cell, blocks, seed, offset, u);
-      const float alr = st[m];
-      const float4 be4 = ld4m(st + M + n, cn, 0.f), o4 = ld4m(out + cell, cn, 0.f);
-      // S from the forward's 1 / S, which still sits where the targets go (valid in every tile the
-      // forward did not flag): exp(out - alpha - beta) carries the rounding of `out`, up to 6e-5
-      // of S at |out| ~ 1000, and a target u S beyond the sum the sweep adds up is never passed
-      const float4 r4 = ld4m(remw + cell, cn, 1.f);
-      const float bev[4] = {be4.x, be4.y, be4.z, be4.w}, ov[4] = {o4.x, o4.y, o4.z, o4.w};
-      const float rv[4] = {r4.x, r4.y, r4.z, r4.w};
-      float tv[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float e = alr + bev[j] - ov[j];  // -log S
-        if (j < cn && (!(e <= lim) || !(e > -INFINITY))) bad = 1;
-        tv[j] = -(u[j] * kSampleShrink) * __builtin_amdgcn_rcpf(rv[j]);
-      }
-      st4m(remw + cell, cn, make_float4(tv[0], tv[1], tv[2], tv[3]));
-    }
-  }
-  bad = __syncthreads_or(bad);  // also: the tile's -t are visible to the whole workgroup
-  if (bad) {
-    if (tid == 0) *flag = 1;
-    return;
-  }
-  floatx16 acc[2][2];
-  int low[2][2][16];
-  const int col = lane & 31;
-#pragma unroll
-  for (int br = 0; br < 2; ++br)
-#pragma unroll
-    for (int bc = 0; bc < 2; ++bc) {
-      const int n = n0 + wn0 + bc * 32 + col;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int m = m0 + wm0 + br * 32 + mfma_row(i, lane);
-        const bool ok = !RAGGED || (m < M && n < N);
-        const float nt = ok ? remw[((long)batch * M + m) * N + n] : 0.f;
-        acc[br][bc][i] = nt;
-        low[br][bc][i] = __float_as_int(nt) | 63;  // tag 63: no slab has ended below t
-      }
-    }
-
-  // ---- staging of EA (transposed) and EB, one slab ahead
-  const int bcol = n0 + SB::quad(tid) * 4;
-  const int cb = RAGGED ? clamp4(N - bcol) : 4;
-  const bool vb = cb > 0;
-  bool va[SA::PER];
-  const float* pa[SA::PER];
-  const float* pb[SB::PER];
-#pragma unroll
-  for (int l = 0; l < SA::PER; ++l) {
-    const int line = m0 + SA::line(tid, l);
-    va[l] = !RAGGED || line < M;
-    pa[l] = ws_ea + ((long)batch * M + (va[l] ? line : M - 1)) * K + SA::quad(tid) * 4;
-  }
-#pragma unroll
-  for (int l = 0; l < SB::PER; ++l)
-    pb[l] = ws_eb + ((long)batch * K + SB::red(tid, l)) * N + (vb ? bcol : 0);
-  const int ktail = RAGGED ? K % kMS : 0;
-  const int slabs = RAGGED ? (K + kMS - 1) / kMS : K / kMS;
-  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
-  float4 ra[SA::PER], rb[SB::PER];
-  auto load = [&](bool tail) __attribute__((always_inline)) {
-    if (RAGGED && tail) {
-      const int ca = clamp4(ktail - SA::quad(tid) * 4);
-#pragma unroll
-      for (int l = 0; l < SA::PER; ++l) ra[l] = va[l] ? ld4m(pa[l], ca, 0.f) : zero;
-#pragma unroll
-      for (int l = 0; l < SB::PER; ++l) rb[l] = SB::red(tid, l) < ktail ? ld4m(pb[l], cb, 0.f) : zero;
-    } else {
-#pragma unroll
-      for (int l = 0; l < SA::PER; ++l) ra[l] = (!RAGGED || va[l]) ? ld4(pa[l]) : zero;
-#pragma unroll
-      for (int l = 0; l < SB::PER; ++l) rb[l] = RAGGED ? ld4m(pb[l], cb, 0.f) : ld4(pb[l]);
-    }
-#pragma unroll
-    for (int l = 0; l < SA::PER; ++l) pa[l] += kMS;
-#pragma unroll
-    for (int l = 0; l < SB::PER; ++l) pb[l] += (long)kMS * N;
-  };
-  auto stage = [&](int buf) __attribute__((always_inline)) {
-#pragma unroll
-    for (int l = 0; l < SA::PER; ++l) SA::put(As[buf], tid, l, ra[l]);
-#pragma unroll
-    for (int l = 0; l < SB::PER; ++l) SB::put(Bs[buf], tid, l, rb[l]);
-  };
-
-  load(slabs == 1 && ktail != 0);
-  stage(0);
-  __syncthreads();
-  for (int s = 0; s < slabs; ++s) {
-    const bool more = s + 1 < slabs;
-    if (more) load(s + 2 == slabs && ktail != 0);
-    mfma_slab<LDR, LDC>(As[s & 1], Bs[s & 1], wm0, wn0, lane, acc);
-    if (more) stage((s + 1) & 1);
-    const int tag = 62 - s;
-#pragma unroll
-    for (int x = 0; x < 4; ++x)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int v = (__float_as_int(acc[x >> 1][x & 1][i]) & ~63) | (tag & 63);  // one v_bfi_b32
-        low[x >> 1][x & 1][i] = min(low[x >> 1][x & 1][i], v);
-      }
-    __syncthreads();
-  }
-
-  // ---- slab in which the prefix passes t, and rem at its start
-#pragma unroll
-  for (int br = 0; br < 2; ++br)
-#pragma unroll
-    for (int bc = 0; bc < 2; ++bc) {
-      const int n = n0 + wn0 + bc * 32 + col;
-      if (RAGGED && n >= N) continue;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int m = m0 + wm0 + br * 32 + mfma_row(i, lane);
-        if (RAGGED && m >= M) continue;
-        const long cell = ((long)batch * M + m) * N + n;
-        const int below = 63 - (low[br][bc][i] & 63);
-        idx[cell] = below >= slabs ? 0 : -2 - below;
-        remw[cell] = -__int_as_float(low[br][bc][i] & ~63);
-      }
-    }
-}
-
 }  // namespace GENBMM_NS

@@ -244,12 +244,16 @@ template <int NT>
 __device__ __forceinline__ bool split_early(int wave) { return wave >= NT / 128; }
 // ----------------------------------------------------------------- forward
 // rows <- EA from a[m][k] ([line][reduction]), columns <- EB from b[k][n] ([reduction][line]).
-// Leaves the maxima, the tile flags and the header (no factors), like k_log_fwd_mfma<T, false, false>.
-template <class T, bool RAGGED>
+// Leaves the maxima, the tile flags and the header; KEEP: also the factors EA, EB (fp32, written
+// by the tiles that stage them anyway: slab s of a row block's EA by its column block s mod
+// tiles_n, likewise EB) and 1 / S, as k_log_fwd_mfma<T, RAGGED, true> does - what the sampling
+// sweep reads.
+template <class T, bool RAGGED, bool KEEP>
 __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WPE, T::WPE)))
 void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b, elem_t* __restrict__ out,
-                     const float* __restrict__ stats, int* __restrict__ flags, int* __restrict__ ws_hdr, int M,
-                     int K, int N, int tiles_m, int tiles_n) {
+                     const float* __restrict__ stats, int* __restrict__ flags, float* __restrict__ ws_ea,
+                     float* __restrict__ ws_eb, float* __restrict__ ws_r, int* __restrict__ ws_hdr, int M, int K,
+                     int N, int tiles_m, int tiles_n) {
   constexpr int NT = T::NT;
   using SA = SplitT<T::TR, NT>;
   using SB = SplitS<T::TC, NT>;
@@ -270,13 +274,19 @@ void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
   // slab, LW columns from bcol
   const elem_t* pa[SA::PER];
   float al[SA::PER];
+  bool va[SA::PER];
 #pragma unroll
   for (int l = 0; l < SA::PER; ++l) {
     const int line = m0 + SA::line(tid, l);
-    const bool in = !RAGGED || line < M;
-    pa[l] = a + ((long)batch * M + (in ? line : M - 1)) * K + SA::quad(tid) * 4;
-    al[l] = in ? st[line] : INFINITY;  // lines beyond the matrix: exp -> 0
+    va[l] = !RAGGED || line < M;
+    pa[l] = a + ((long)batch * M + (va[l] ? line : M - 1)) * K + SA::quad(tid) * 4;
+    al[l] = va[l] ? st[line] : INFINITY;  // lines beyond the matrix: exp -> 0
   }
+  // the factors live at the same offsets in their own arrays (the source pointers run one slab
+  // ahead of what is being staged, whichever side of its products a wave stages on)
+  const int nblk = rem % tiles_n, mblk = rem / tiles_n;
+  const long da = KEEP ? ws_distance(ws_ea, a) - 4l * kMS : 0, db = KEEP ? ws_distance(ws_eb, b) - 4l * kMS * N : 0;
+  int s_stage = 0, sa = 0, sb = 0;  // the slab the next stage() forms; s_stage mod tiles_n, mod tiles_m
   const int bcol = n0 + SB::line0(tid);
   const int cb = RAGGED ? clampw(N - bcol, LW) : LW;  // columns of the b piece inside the matrix
   const int brow = 2 * SB::pair(tid);
@@ -287,7 +297,7 @@ void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
   if (tile == 0 && tid == 0) {
     ws_hdr[1] = T::TR;
     ws_hdr[2] = T::TC;
-    ws_hdr[0] = kWsFast;
+    ws_hdr[0] = KEEP ? kWsMfma : kWsFast;
   }
 
   floatx16 acc[2][2];
@@ -325,8 +335,16 @@ void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
     ++s_load;
   };
   auto stage = [&](int buf) __attribute__((always_inline)) {
+    const bool tail = RAGGED && ktail != 0 && s_stage == slabs - 1;
 #pragma unroll
-    for (int l = 0; l < SA::PER; ++l) SA::put(As(buf), tid, l, exp4(ra[l], al[l]));
+    for (int l = 0; l < SA::PER; ++l) {
+      const float4 e = exp4(ra[l], al[l]);
+      SA::put(As(buf), tid, l, e);
+      if (KEEP && sa == nblk) {
+        if (!RAGGED) st4(ws_twin(pa[l], da), e);
+        else if (va[l]) st4m(ws_twin(pa[l], da), tail ? clamp4(ktail - SA::quad(tid) * 4) : 4, e);
+      }
+    }
     float ee[LW], eo[LW];
 #pragma unroll
     for (int j = 0; j < LW; ++j) {
@@ -334,6 +352,19 @@ void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
       eo[j] = exp_st(rbo[j] - be[j]);
     }
     SB::put(Bs(buf), tid, ee, eo);
+    if (KEEP && sb == mblk) {
+      float* we = ws_twin(pb, db);
+#pragma unroll
+      for (int j = 0; j < LW; ++j) {
+        if (j < cb && (!tail || brow < ktail)) we[j] = ee[j];
+        if (j < cb && (!tail || brow + 1 < ktail)) we[N + j] = eo[j];
+      }
+    }
+    if (KEEP) {
+      ++s_stage;
+      sa = sa + 1 == tiles_n ? 0 : sa + 1;
+      sb = sb + 1 == tiles_m ? 0 : sb + 1;
+    }
   };
 
   load();
@@ -399,7 +430,180 @@ void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
                                            __builtin_fmaf(fast_log2(sv.w), kLn2, alr + be4.w));
              if (RAGGED) st4m(out + ubase + (long)ru * N + voff, cc, ov);
              else st4(out + ubase + (long)ru * N + voff, ov);
+             if constexpr (KEEP) {
+               const float4 rv = make_float4(__builtin_amdgcn_rcpf(sv.x), __builtin_amdgcn_rcpf(sv.y),
+                                             __builtin_amdgcn_rcpf(sv.z), __builtin_amdgcn_rcpf(sv.w));
+               if (RAGGED) st4m(ws_r + ubase + (long)ru * N + voff, cc, rv);
+               else st4(ws_r + ubase + (long)ru * N + voff, rv);
+             }
            });
+}
+
+// ------------------------------------------------------- sampling sweep
+// The sampling sweep described in logbmm_mfma.h: the forward's contraction again on its fp32
+// factors EA, EB - cut into their three parts while they are staged, no exponential - with the
+// accumulators started at -t, t = u S the cell's target; after every slab of 16 terms a
+// register per cell keeps, by a signed-integer minimum over (value with its low six bits
+// replaced by 62 - slab), the slab in which the prefix sum passes t and -rem at the start of
+// that slab.  S is the reciprocal of the forward's 1 / S, the targets are shrunk by 2^-22;
+// results: the code -2 - slab in idx, rem in `remw`.  The partial products are added in the
+// forward's order, so the sums the sweep compares with its targets are the forward's.  A tile
+// with a cell whose S is below 2^-40 or not finite, or that lies in a tile the forward
+// flagged, sets that flag and leaves: the forward's tile is redone exactly.  128 x 128 tiles of
+// four waves with 256 registers (64 accumulators and 64 history registers per lane); always
+// the any-size form of the loaders.
+template <class T>
+__global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void k_sample_sweep_split(const float* __restrict__ ws_ea, const float* __restrict__ ws_eb,
+                          const elem_t* __restrict__ out, const float* __restrict__ stats,
+                          int* __restrict__ flags, float* __restrict__ remw, int32_t* __restrict__ idx,
+                          uint64_t seed, uint64_t offset, int M, int K, int N, int tiles_m, int tiles_n, int ftr,
+                          int ftc, int ftiles_m, int ftiles_n) {
+  constexpr bool RAGGED = true;
+  constexpr int NT = T::NT;
+  using SA = SplitT<T::TR, NT>;
+  using SB = SplitS<T::TC, NT>;
+  static_assert(SB::LW == 4, "");
+  __shared__ __attribute__((aligned(16))) unsigned smem[split_lds_words<SA, SB>()];
+  auto As = [&](int buf) __attribute__((always_inline)) { return smem + buf * SA::BUF; };
+  auto Bs = [&](int buf) __attribute__((always_inline)) { return smem + 2 * SA::BUF + buf * SB::BUF; };
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = (wave / T::WC) * 64, wn0 = (wave % T::WC) * 64;
+  const int per = tiles_m * tiles_n, tile = xcd_tile_id();
+  const int batch = tile / per, rem = tile - batch * per;
+  const int m0 = (rem / tiles_n) * T::TR, n0 = (rem % tiles_n) * T::TC;
+  const float* st = stats + (long)batch * (M + N);
+
+  // ---- targets: -t = -u S per cell into `remw`, row by row, four adjacent cells per lane and
+  // step (they share one Philox block when rows are a multiple of four cells); then the
+  // accumulators pick their cells up in the matrix-core layout.  The flags are the forward's,
+  // one per tile of ITS shape (ftr x ftc).
+  int* flag = flags + (batch * ftiles_m + m0 / ftr) * ftiles_n + n0 / ftc;
+  const float lim = kMfmaGuardBits * kLn2 + 1e-3f;
+  int bad = *flag;
+  {
+    constexpr int QR = T::TC / 4;  // quads per tile row
+    const bool blocks = (N & 3) == 0;
+#pragma unroll 4
+    for (int q = tid; q < T::TR * QR; q += NT) {
+      const int r = q / QR, m = m0 + r, n = n0 + (q - r * QR) * 4;
+      if (RAGGED && (m >= M || n >= N)) continue;
+      const long cell = ((long)batch * M + m) * N + n;
+      const int cn = RAGGED ? clamp4(N - n) : 4;
+      float u[4];
+      philox_uniform4((uint64_t)cell, blocks, seed, offset, u);
+      const float alr = st[m];
+      const float4 be4 = ld4m(st + M + n, cn, 0.f), o4 = ld4m(out + cell, cn, 0.f);
+      const float4 r4 = ld4m(remw + cell, cn, 1.f);  // the forward's 1 / S
+      const float bev[4] = {be4.x, be4.y, be4.z, be4.w}, ov[4] = {o4.x, o4.y, o4.z, o4.w};
+      const float rv[4] = {r4.x, r4.y, r4.z, r4.w};
+      float tv[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float e = alr + bev[j] - ov[j];  // -log S
+        if (j < cn && (!(e <= lim) || !(e > -INFINITY))) bad = 1;
+        tv[j] = -(u[j] * kSampleShrink) * __builtin_amdgcn_rcpf(rv[j]);
+      }
+      st4m(remw + cell, cn, make_float4(tv[0], tv[1], tv[2], tv[3]));
+    }
+  }
+  bad = __syncthreads_or(bad);  // also: the tile's -t are visible to the whole workgroup
+  if (bad) {
+    if (tid == 0) *flag = 1;
+    return;
+  }
+  floatx16 acc[2][2];
+  int low[2][2][16];
+  const int col = lane & 31;
+#pragma unroll
+  for (int br = 0; br < 2; ++br)
+#pragma unroll
+    for (int bc = 0; bc < 2; ++bc) {
+      const int n = n0 + wn0 + bc * 32 + col;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int m = m0 + wm0 + br * 32 + mfma_row(i, lane);
+        const bool ok = !RAGGED || (m < M && n < N);
+        const float nt = ok ? remw[((long)batch * M + m) * N + n] : 0.f;
+        acc[br][bc][i] = nt;
+        low[br][bc][i] = __float_as_int(nt) | 63;  // tag 63: no slab has ended below t
+      }
+    }
+
+  // ---- staging of EA ([line][reduction]) and EB (pairs of reduction steps), zeros beyond the matrix
+  const int bcol = n0 + SB::line0(tid);
+  const int cb = clamp4(N - bcol);
+  const int brow = 2 * SB::pair(tid);
+  bool va[SA::PER];
+  const float* pa[SA::PER];
+#pragma unroll
+  for (int l = 0; l < SA::PER; ++l) {
+    const int line = m0 + SA::line(tid, l);
+    va[l] = line < M;
+    pa[l] = ws_ea + ((long)batch * M + (va[l] ? line : M - 1)) * K + SA::quad(tid) * 4;
+  }
+  const float* pb = ws_eb + ((long)batch * K + brow) * N + (cb > 0 ? bcol : 0);
+  const int ktail = K % kMS;
+  const int slabs = (K + kMS - 1) / kMS;
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 ra[SA::PER], rbe, rbo;
+  int s_load = 0, s_mma = 0;
+  auto load = [&]() __attribute__((always_inline)) {
+    if (ktail != 0 && s_load == slabs - 1) {
+      const int ca = clamp4(ktail - SA::quad(tid) * 4);
+#pragma unroll
+      for (int l = 0; l < SA::PER; ++l) ra[l] = va[l] ? ld4m(pa[l], ca, 0.f) : zero;
+      rbe = brow < ktail ? ld4m(pb, cb, 0.f) : zero;
+      rbo = brow + 1 < ktail ? ld4m(pb + N, cb, 0.f) : zero;
+    } else {
+#pragma unroll
+      for (int l = 0; l < SA::PER; ++l) ra[l] = va[l] ? ld4(pa[l]) : zero;
+      rbe = ld4m(pb, cb, 0.f);
+      rbo = ld4m(pb + N, cb, 0.f);
+    }
+#pragma unroll
+    for (int l = 0; l < SA::PER; ++l) pa[l] += kMS;
+    pb += (long)kMS * N;
+    ++s_load;
+  };
+  auto stage = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int l = 0; l < SA::PER; ++l) SA::put(As(buf), tid, l, ra[l]);
+    SB::put(Bs(buf), tid, rbe, rbo);
+  };
+  load();
+  stage(0);
+  split_loop(slabs, split_early<NT>(wave), load, stage, [&](int buf) __attribute__((always_inline)) {
+    split_slab<SA, SB>(As(buf), Bs(buf), wm0, wn0, wave, lane, acc);
+    const int tag = 62 - s_mma;
+    ++s_mma;
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int v = (__float_as_int(acc[x >> 1][x & 1][i]) & ~63) | (tag & 63);  // one v_bfi_b32
+        low[x >> 1][x & 1][i] = min(low[x >> 1][x & 1][i], v);
+      }
+  });
+
+  // ---- slab in which the prefix passes t, and rem at its start
+#pragma unroll
+  for (int br = 0; br < 2; ++br)
+#pragma unroll
+    for (int bc = 0; bc < 2; ++bc) {
+      const int n = n0 + wn0 + bc * 32 + col;
+      if (RAGGED && n >= N) continue;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int m = m0 + wm0 + br * 32 + mfma_row(i, lane);
+        if (RAGGED && m >= M) continue;
+        const long cell = ((long)batch * M + m) * N + n;
+        const int below = 63 - (low[br][bc][i] & 63);
+        idx[cell] = below >= slabs ? 0 : -2 - below;
+        remw[cell] = -__int_as_float(low[br][bc][i] & ~63);
+      }
+    }
 }
 
 // ---------------------------------------------------------------- backward
