@@ -1068,8 +1068,10 @@ int run_bwd_both(const elem_t* a, const elem_t* b, const elem_t* out, const elem
       pa.grad = grad_a;
       pb.grad = grad_b;
       const bool lean = path != GENBMM_PATH_FACTORS;
-      // (the three-part backward takes any M, and K and N in whole pieces of four; the forward any sizes)
-      if (lean && split_path(path) && N % 4 == 0 && K % 4 == 0) {
+      // (the three-part backward takes any M, and K and N in whole pieces of four - the forward any
+      //  sizes -; it addresses a batch item's matrices by 32-bit offsets)
+      const bool small_items = (int64_t)M * N < (1ll << 31) && (int64_t)K * N < (1ll << 31) && (int64_t)M * K < (1ll << 31);
+      if (lean && split_path(path) && N % 4 == 0 && K % 4 == 0 && small_items) {
         if (ka == 1) return launch_bwd_split_both<MT128S, MT128S>(pa, pb, st, B, s);
         if (split_big_fits(B, M, K) && split_big_fits(B, K, N))
           return launch_bwd_split_both<MTBig, MTBig>(pa, pb, st, B, s);

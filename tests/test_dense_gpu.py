@@ -305,6 +305,30 @@ def test_logbmm_three_part_kernels(gpu, B, M, K, N):
         close_on_device(x, y.double(), "against the fp32 matrix instruction", rtol=2e-5, atol=2e-5)
 
 
+@pytest.mark.parametrize("B,M,K,N,scale", [(64, 512, 512, 512, 1.0), (8, 1024, 2048, 512, 1.0), (32, 500, 1000, 400, 3.0),
+                                            (512, 128, 128, 128, 1.0)])
+def test_three_part_products_are_as_accurate_as_fp32_products(gpu, B, M, K, N, scale):
+    """The default kernels take every product as six bf16 partial products of three-part factors;
+    GENBMM_PATH_MFMA32 takes it on the fp32 matrix instruction.  Against float64 (four batch items,
+    on the device) the two must be equally good: maximum and mean absolute error of out, grad_a
+    and grad_b on the default path at most 1.5 times the fp32 instruction's (+ 1e-7)."""
+    torch.manual_seed(K)
+    a, b, g = (torch.randn(B, M, K, device=gpu) * scale, torch.randn(B, K, N, device=gpu) * scale,
+               torch.randn(B, M, N, device=gpu))
+    pick = slice(0, 4)
+    want = oracle.logbmm_grads64(a[pick], b[pick], g[pick])
+    errs = []
+    for path in (genmul.PATH_AUTO, genmul.PATH_MFMA32):
+        ad, bd = a.clone().requires_grad_(True), b.clone().requires_grad_(True)
+        out = genmul.logbmm_on_path(ad, bd, path)
+        res = (out.detach(),) + torch.autograd.grad(out, (ad, bd), g)
+        errs.append([((x[pick].double() - w).abs().max().item(), (x[pick].double() - w).abs().mean().item())
+                     for x, w in zip(res, want)])
+    for (mx3, mean3), (mx32, mean32), what in zip(errs[0], errs[1], ("out", "grad_a", "grad_b")):
+        assert mx3 <= 1.5 * mx32 + 1e-7, (what, mx3, mx32)
+        assert mean3 <= 1.5 * mean32 + 1e-7, (what, mean3, mean32)
+
+
 def test_logbmm_matrix_core_shape_sweep(gpu):
     """A seeded sweep of 48 shapes around the switching points of the matrix-core kernels (tile forms
     256 x 256 / 256 x 128 / 128 x 128, full and ragged, extents in multiples of 16, of 4 and odd -

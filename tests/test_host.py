@@ -288,3 +288,35 @@ def test_band_structural_ops_match_reference_vectors(case):
     same("op_max", bm.op(om, torch.max, zero=-1e9))
     same("transpose", bm.transpose())
     assert torch.equal(bm.to_dense(), torch.from_numpy(z[p + "to_dense"]))
+
+
+def test_three_bf16_parts_of_a_float_add_up_to_it_exactly():
+    """The arithmetic behind the default logbmm kernels' products (genbmm_amd/csrc/logbmm_split.h):
+    a float x is cut into three bfloat16 parts by rounding and subtracting twice; the parts add up
+    to x exactly (8 + 8 + 8 significant bits; below 2^-100 the last part can fall into the
+    denormals, far beneath any factor the kernels' guard lets matter), and the six partial
+    products the kernels take - all but m l, l m, l l - give x y within 2^-22 of it: the size of
+    the rounding of one fp32 product."""
+    import torch
+    torch.manual_seed(0)
+    mag = torch.exp2(torch.empty(400000).uniform_(-60.0, 60.0))
+    x = torch.cat([torch.rand(200000), torch.randn(200000) * 1e3, mag * torch.sign(torch.randn(400000)),
+                   torch.tensor([0.0, 1.0, 2.0 ** -40, 1 - 2.0 ** -24, 3.0e38, -7.25])])
+
+    def parts(v):
+        h = v.bfloat16().float()
+        r = v - h
+        m = r.bfloat16().float()
+        l = (r - m).bfloat16().float()
+        return h, m, l
+
+    h, m, l = parts(x)
+    assert torch.equal((h.double() + m.double()) + l.double(), x.double())
+    y = x[torch.randperm(x.numel())]
+    hy, my, ly = parts(y)
+    d = lambda t: t.double()
+    six = d(h) * d(hy) + d(h) * d(my) + d(m) * d(hy) + d(m) * d(my) + d(h) * d(ly) + d(l) * d(hy)
+    exact = d(x) * d(y)
+    fin = torch.isfinite(exact) & (exact != 0)
+    rel = ((six - exact).abs() / exact.abs())[fin]
+    assert float(rel.max()) <= 2.0 ** -22, float(rel.max())
