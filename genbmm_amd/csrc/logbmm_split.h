@@ -6,16 +6,19 @@
 // below 2^-23 of x y, the size of one fp32 rounding of the product itself.  The
 // instruction does 16 reduction steps in the time the fp32 one (v_mfma_f32_32x32x2_f32)
 // needs for one, so six of them per 16 steps are 2.7 times less matrix-pipe time, and -
-// unlike the fp32 matrix instruction on this part - they run beside the vector ALU's work.
+// unlike the fp32 matrix instruction on this part - vector instructions of other waves can
+// execute beside them (the counters show it for about a third of the pipe's busy cycles).
 //
 // Same tiles, guards, flags, epilogues and fix-up launches as the fp32 kernels of
 // logbmm_mfma.h (a 64 x 64 block per wave as 2 x 2 accumulators, whose layout is that of
 // the fp32 instruction; reduction in slabs of 16 through two LDS buffers); what differs is
-// the staged form and the inner loop.  Any sizes: ragged edges are a second instantiation
-// of each kernel (RAGGED), handled as in logbmm_mfma.h - lines of a tile beyond the matrix
-// re-read the last line with a shift that makes the factor vanish, pieces that straddle the
-// right edge are read element by element, the reduction tail is filled by the loader of the
-// last slab, stores are masked.
+// the staged form and the inner loop.  Ragged edges are a second instantiation of each
+// kernel (RAGGED), handled as in logbmm_mfma.h: lines of a tile beyond the matrix re-read
+// the last line (under a shift that makes the factor vanish where the line feeds stored
+// results), stores are masked.  The forward takes any sizes: pieces that straddle the right
+// edge are read element by element, the reduction tail is filled by the loader of the last
+// slab.  The backward takes any M but K and N in multiples of four (no piece straddles an
+// edge), and its partial last slab is a step of its own behind the loop.
 //
 // LDS layouts, three planes (h, m, l) per operand, words of two bf16:
 //  * an operand whose source is [line][reduction] (reduction contiguous): plane[line][8
