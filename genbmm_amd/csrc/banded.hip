@@ -21,6 +21,7 @@
 #include <type_traits>
 
 #include "banded_argmax.h"
+#include "banded_block.h"
 #include "banded_direct.h"
 #include "banded_flat.h"
 #include "banded_max.h"
@@ -128,6 +129,30 @@ inline void launch_prep(const BandArgs& p, const elem_t* a, int a_lu, const elem
                      blocks_a, vec);
 }
 
+// The block kernel (banded_block.h) takes the forward where it is the faster one: from about 53
+// diagonals per operand (measured at 64 x 4096, block against memory-fed: 49 diagonals 0.067 ms
+// against 0.063, 57: 0.078 against 0.084, 65: 0.083 against 0.098; log product with its
+// preparation 0.145 / 0.138, 0.165 / 0.177, 0.193 / 0.214) up to where its staged blocks still fit
+// a compute unit's LDS (65 diagonals per operand; 73 do not).
+constexpr int kBlkMinW = 53;
+inline bool blk_fwd_ok(const BandArgs& p, int B) {
+  BlkPlan g;
+  return min(p.Wa, p.Wb) >= kBlkMinW && (long)p.n * p.Wo < (1L << 30) && blk_plan_fwd(g, p.Wa, p.Wb, p.n, B, 8);
+}
+template <bool PREP>
+inline void launch_blk_fwd(const BandArgs& p, int B, hipStream_t s) {
+  BlkPlan g;
+  blk_plan_fwd(g, p.Wa, p.Wb, p.n, B, 8);
+  const int nblocks = B * g.chunks;
+  const size_t lds = blk_lds_bytes(g);
+  auto go = [&](auto kern, int sw) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64 * (g.ncw + sw)), lds, s, p, g, nblocks, (long)B * p.n);
+  };
+  if (max(g.NSa, g.NSb) <= 6) go(k_band_blk_fwd<PREP, 4, 3, 3>, 4);
+  else go(k_band_blk_fwd<PREP, 4, 4, 4>, 4);
+}
+
 template <int KIND, bool PREP>
 inline void launch_dir(const BandArgs& p, int B, hipStream_t s) {
   const int blocks = ceil_div(p.n, 16 * kDirWaves);
@@ -219,12 +244,15 @@ int GENBMM_API(banded_fwd)(const GENBMM_NS::abi_t* a_, int a_lu, int a_ld, const
   const StripDims sd = strip_dims(p.Wa, p.Wb);
   const bool dir = dir_fwd_ok(p, mode == GENBMM_BAND_MUL ? kDirMinWPlainFwd : kDirMinW);
   if (dir && (mode == GENBMM_BAND_MUL || prep_fwd(p, mode, workspace))) {
+    const bool blk = blk_fwd_ok(p, B);
     if (mode == GENBMM_BAND_LOG) {
       set_workspace(p, workspace, B);
       launch_prep(p, a, a_lu, b, b_lu, B, s);
-      launch_dir<kDirFwd, true>(p, B, s);
+      if (blk) launch_blk_fwd<true>(p, B, s);
+      else launch_dir<kDirFwd, true>(p, B, s);
     } else {
-      launch_dir<kDirFwd, false>(p, B, s);
+      if (blk) launch_blk_fwd<false>(p, B, s);
+      else launch_dir<kDirFwd, false>(p, B, s);
     }
     return launch_status();
   }
