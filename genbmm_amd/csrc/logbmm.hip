@@ -858,7 +858,7 @@ int launch_fwd_split(DenseArgs p, float* stats, int B, int M, int K, int N, bool
   auto go = [&](auto kern) {
     allow_lds(kern, lds);
     hipLaunchKernelGGL(kern, dim3(total), dim3(T::NT), lds, s, p.a, p.b, p.out, stats, flags, ws.ea, ws.eb, ws.r,
-                       ws.hdr, M, K, N, p.tiles_m, p.tiles_n);
+                       ws.hdr, M, K, N, p.tiles_m, p.tiles_n, 1);
   };
   const bool ragged = M % T::TR != 0 || N % T::TC != 0 || K % kMS != 0;
   if (keep) {
@@ -968,8 +968,44 @@ int launch_self_fwd(DenseArgs p, float* stats, int B, int M, int K, int N, bool 
 
 // factors: the caller wants EA, EB and 1/S in the workspace wherever a forward can leave
 // them (the sampling sweep), so the kernels that keep no by-products are not used.
+// Few output tiles and a long reduction: how many pieces to cut the reduction axis into (1: none).
+// At most one round of workgroups over the chip, pieces of at least 32 slabs (512 steps), none empty.
+inline int fwd_pieces(int B, int M, int K, int N) {
+  const int64_t tiles = tiles128(B, M, N);
+  const int slabs = ceil_div(K, kMS);
+  if (tiles <= 0 || tiles >= 128 || slabs < 128) return 1;
+  const int want = (int)std::min<int64_t>((255 + tiles) / tiles, slabs / 32);
+  if (want < 2) return 1;
+  return ceil_div(slabs, ceil_div(slabs, want));
+}
+// The forward in pieces of the reduction axis: 128 x 128 tiles, the pieces' sums in the workspace
+// behind the header ([piece][B][M][N]), joined by k_log_fwd_join.
+int launch_fwd_pieces(DenseArgs p, float* stats, int B, int M, int K, int N, int pieces, hipStream_t s) {
+  using T = MT128S;
+  p.M = M; p.K = K; p.N = N;
+  p.tiles_m = ceil_div(M, T::TR);
+  p.tiles_n = ceil_div(N, T::TC);
+  p.vec_a = (K % 4 == 0) && aligned16(p.a);
+  p.vec_b = (N % 4 == 0) && aligned16(p.b);
+  p.vec_o = (N % 4 == 0) && aligned16(p.out);
+  const int total = B * p.tiles_m * p.tiles_n;  // below 128
+  int* flags = fwd_flags_of(stats, B, M, N);
+  constexpr int lds = 4 * split_lds_words<SplitT<T::TR, T::NT>, SplitS<T::TC, T::NT>>();
+  const LogPrepared ws = prepared_of(stats, B, M, K, N);
+  float* parts = ws.ea;
+  auto kern = k_log_fwd_split<T, true, false, true>;
+  allow_lds(kern, lds);
+  hipLaunchKernelGGL(kern, dim3(total * pieces), dim3(T::NT), lds, s, p.a, p.b, p.out, stats, flags, nullptr, nullptr,
+                     parts, ws.hdr, M, K, N, p.tiles_m, p.tiles_n, pieces);
+  if (int e = launch_status()) return e;
+  hipLaunchKernelGGL((k_log_fwd_join<T::TR, T::TC>), dim3(total), dim3(256), 0, s, parts, p.out, stats, flags, ws.hdr,
+                     B, M, N, p.tiles_m, p.tiles_n, pieces);
+  if (int e = launch_status()) return e;
+  return launch_fwd_fixup<CfgWide, T::TR, T::TC>(p, flags, total, s);
+}
+// pieces_ok: the workspace has room for the sums of a forward in pieces (fwd_pieces)
 int run_fwd(const elem_t* a, const elem_t* b, elem_t* out, float* stats, int B, int M, int K, int N,
-            int path, bool keep, hipStream_t s, bool factors = false) {
+            int path, bool keep, hipStream_t s, bool factors = false, bool pieces_ok = true) {
   if (int e = check_dense_dims(B, M, K, N)) return e;
   if (!valid_path(path)) return GENBMM_E_MODE;
   const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
@@ -992,6 +1028,10 @@ int run_fwd(const elem_t* a, const elem_t* b, elem_t* out, float* stats, int B, 
     if (int e = launch_stats(a, b, stats, B, M, K, N, s)) return e;
   }
   if (mn == 0) return GENBMM_OK;
+  if (stats && split_path(path) && !keep && pieces_ok) {
+    const int pieces = fwd_pieces(B, M, K, N);
+    if (pieces > 1) return launch_fwd_pieces(p, stats, B, M, K, N, pieces, s);
+  }
   if (stats && K > 0 && path != GENBMM_PATH_EXACT) {
     const int64_t big_tiles = (int64_t)B * ceil_div(M, 128) * ceil_div(N, 128);
     switch (fwd_mfma_shape(B, M, K, N) ? mfma_kind(path, B, M, N, K, false) : 0) {
@@ -1176,11 +1216,22 @@ size_t genbmm_logbmm_stats_size_path(int B, int M, int K, int N, int path) {
   // the by-products of the matrix-core forward (the one-tile kernels keep the maxima only)
   if (path == GENBMM_PATH_FACTORS && fwd_mfma_shape(B, M, K, N) && !self_shape(M, K, N))
     n += (int64_t)B * ((int64_t)M * K + (int64_t)K * N + (int64_t)M * N);
+  // the sums of a forward that cuts a long reduction into pieces
+  if (path == GENBMM_PATH_AUTO) {
+    const int pieces = fwd_pieces(B, M, K, N);
+    if (pieces > 1) n += (int64_t)pieces * B * M * N;
+  }
   return (size_t)n;
 }
 
 size_t genbmm_logbmm_stats_size(int B, int M, int K, int N) {
   return genbmm_logbmm_stats_size_path(B, M, K, N, GENBMM_PATH_AUTO);
+}
+
+int genbmm_logbmm_fwd_pieces(int B, int M, int K, int N) {
+  using namespace GENBMM_NS;
+  if (check_dense_dims(B, M, K, N) || (int64_t)B * M * N == 0 || item_shape(M, K, N) || self_shape(M, K, N)) return 1;
+  return fwd_pieces(B, M, K, N);
 }
 
 size_t genbmm_samplebmm_stats_size(int B, int M, int K, int N) {
@@ -1200,7 +1251,7 @@ int genbmm_logbmm_fwd_static(const float* a, const float* b, float* out, int B, 
   if ((uint64_t)header_offset(B, M, N) + 4 > kStaticFloats) return GENBMM_E_TOOBIG;
   float* ws = nullptr;
   if (int e = static_workspace(&ws)) return e;
-  return run_fwd(a, b, out, ws, B, M, K, N, GENBMM_PATH_AUTO, false, (hipStream_t)stream);
+  return run_fwd(a, b, out, ws, B, M, K, N, GENBMM_PATH_AUTO, false, (hipStream_t)stream, false, false);
 }
 #endif
 

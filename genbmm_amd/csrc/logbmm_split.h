@@ -226,12 +226,18 @@ __device__ __forceinline__ bool split_early(int wave) { return wave >= NT / 128;
 // by the tiles that stage them anyway: slab s of a row block's EA by its column block s mod
 // tiles_n, likewise EB) and 1 / S, as k_log_fwd_mfma<T, RAGGED, true> does - what the sampling
 // sweep reads.
-template <class T, bool RAGGED, bool KEEP>
+// PIECES: the reduction axis is cut into `pieces` runs of slabs, each a workgroup of its own
+// (workgroup = tile * pieces + piece); a piece leaves its sums S for its tile in ws_r
+// ([piece][batch][M][N]) and k_log_fwd_join adds them, tests the guard and takes the logarithm.
+// For problems with few output tiles and a long reduction, which would otherwise run on a few
+// compute units.
+template <class T, bool RAGGED, bool KEEP, bool PIECES = false>
 __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WPE, T::WPE)))
 void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b, elem_t* __restrict__ out,
                      const float* __restrict__ stats, int* __restrict__ flags, float* __restrict__ ws_ea,
                      float* __restrict__ ws_eb, float* __restrict__ ws_r, int* __restrict__ ws_hdr, int M, int K,
-                     int N, int tiles_m, int tiles_n) {
+                     int N, int tiles_m, int tiles_n, int pieces = 1) {
+  static_assert(!PIECES || (RAGGED && !KEEP), "");
   constexpr int NT = T::NT;
   using SA = SplitT<T::TR, NT>;
   using SB = SplitS<T::TC, NT>;
@@ -243,10 +249,15 @@ void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = (wave / T::WC) * 64, wn0 = (wave % T::WC) * 64;
-  const int per = tiles_m * tiles_n, tile = xcd_tile_id();
+  const int per = tiles_m * tiles_n, wg = xcd_tile_id();
+  const int tile = PIECES ? wg / pieces : wg, piece = PIECES ? wg - tile * pieces : 0;
   const int batch = tile / per, rem = tile - batch * per;
   const int m0 = (rem / tiles_n) * T::TR, n0 = (rem % tiles_n) * T::TC;
   const float* st = stats + (long)batch * (M + N);
+  // the slabs of this workgroup: all of them, or the piece's run (no piece is empty)
+  const int slabs_all = RAGGED ? (K + kMS - 1) / kMS : K / kMS;
+  const int slabs_piece = PIECES ? (slabs_all + pieces - 1) / pieces : slabs_all;
+  const int slab0 = piece * slabs_piece;
 
   // a pieces: line m0 + line(l), four k from quad * 4;  the b piece: rows 2 pair, 2 pair + 1 of the
   // slab, LW columns from bcol
@@ -257,7 +268,7 @@ void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
   for (int l = 0; l < SA::PER; ++l) {
     const int line = m0 + SA::line(tid, l);
     va[l] = !RAGGED || line < M;
-    pa[l] = a + ((long)batch * M + (va[l] ? line : M - 1)) * K + SA::quad(tid) * 4;
+    pa[l] = a + ((long)batch * M + (va[l] ? line : M - 1)) * K + SA::quad(tid) * 4 + (long)slab0 * kMS;
     al[l] = va[l] ? st[line] : INFINITY;  // lines beyond the matrix: exp -> 0
   }
   // the factors live at the same offsets in their own arrays (the source pointers run one slab
@@ -268,11 +279,11 @@ void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
   const int bcol = n0 + SB::line0(tid);
   const int cb = RAGGED ? clampw(N - bcol, LW) : LW;  // columns of the b piece inside the matrix
   const int brow = 2 * SB::pair(tid);
-  const elem_t* pb = b + ((long)batch * K + brow) * N + (cb > 0 ? bcol : 0);
+  const elem_t* pb = b + ((long)batch * K + brow + (long)slab0 * kMS) * N + (cb > 0 ? bcol : 0);
   float be[LW];
 #pragma unroll
   for (int j = 0; j < LW; ++j) be[j] = j < cb ? st[M + bcol + j] : INFINITY;
-  if (tile == 0 && tid == 0) {
+  if (!PIECES && tile == 0 && tid == 0) {
     ws_hdr[1] = T::TR;
     ws_hdr[2] = T::TC;
     ws_hdr[0] = KEEP ? kWsMfma : kWsFast;
@@ -284,8 +295,9 @@ void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[x >> 1][x & 1][i] = 0.f;
 
-  const int ktail = RAGGED ? K % kMS : 0;          // reduction steps of a partial last slab
-  const int slabs = RAGGED ? (K + kMS - 1) / kMS : K / kMS;
+  const int slabs = PIECES ? min(slabs_piece, slabs_all - slab0) : slabs_all;
+  // reduction steps of a partial last slab (of the last piece)
+  const int ktail = RAGGED && (!PIECES || slab0 + slabs == slabs_all) ? K % kMS : 0;
   int s_load = 0;                                  // the slab the next load() fetches
   float4 ra[SA::PER];
   float rbe[LW], rbo[LW];
@@ -351,6 +363,19 @@ void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
     split_slab<SA, SB>(As(buf), Bs(buf), wm0, wn0, wave, lane, acc);
   });
 
+  if constexpr (PIECES) {  // the piece's sums, row-wise; the guard is k_log_fwd_join's
+    __syncthreads();       // every wave is done with the staging buffers
+    const int lr = lane >> 4, lc = (lane & 15) * 4;
+    const int cc = clamp4(N - (n0 + wn0 + lc));
+    const long ubase = (((long)piece * (gridDim.x / (pieces * per)) + batch) * M + m0 + wm0) * N + n0 + wn0;
+    const int voff = lr * N + lc, rows_left = M - (m0 + wm0) - lr;
+    acc_rows(acc, reinterpret_cast<float*>(split_smem) + wave * kStripFloats, lane, [](int) {},
+             [&](int q, int t, float4 sv) __attribute__((always_inline)) {
+               const int ru = 16 * q + 4 * t;
+               if (cc > 0 && ru < rows_left) st4m(ws_r + ubase + (long)ru * N + voff, cc, sv);
+             });
+    return;
+  }
   // guard (as k_log_fwd_mfma): S >= 2^-40 and finite; every shift finite and not below the floor;
   // no shift below -30 opposite a row or column at the floor
   const float thr = fast_exp2(-kMfmaGuardBits);
@@ -415,6 +440,62 @@ void k_log_fwd_split(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
                else st4(ws_r + ubase + (long)ru * N + voff, rv);
              }
            });
+}
+
+// The pieces of k_log_fwd_split<.., PIECES> joined: S = the sum of the pieces' sums for a cell, then
+// the forward's guard - per tile of TR x TC cells, the tile shape that the flags, the header and the
+// exact fix-up launch behind this kernel go by - and out = log S + alpha + beta.  One workgroup per tile.
+template <int TR, int TC>
+__global__ __launch_bounds__(256) void k_log_fwd_join(const float* __restrict__ parts, elem_t* __restrict__ out,
+                                                      const float* __restrict__ stats, int* __restrict__ flags,
+                                                      int* __restrict__ ws_hdr, int B, int M, int N, int tiles_m,
+                                                      int tiles_n, int pieces) {
+  const int tid = threadIdx.x, tile = blockIdx.x, per = tiles_m * tiles_n;
+  const int batch = tile / per, rem = tile - batch * per;
+  const int m0 = (rem / tiles_n) * TR, n0 = (rem % tiles_n) * TC;
+  const float* st = stats + (long)batch * (M + N);
+  const long piece_stride = (long)B * M * N;
+  const float thr = fast_exp2(-kMfmaGuardBits);
+  int bad = 0, low = 0, neg = 0;  // bit 0: of a row, bit 1: of a column
+  for (int c = tid; c < TR * (TC / 4); c += 256) {
+    const int m = m0 + c / (TC / 4), n = n0 + (c % (TC / 4)) * 4;
+    const int cc = clamp4(N - n);
+    if (m >= M || cc <= 0) continue;
+    const long at = ((long)batch * M + m) * N + n;
+    float4 sv = ld4m(parts + at, cc, 0.f);
+    for (int p = 1; p < pieces; ++p) {
+      const float4 x = ld4m(parts + p * piece_stride + at, cc, 0.f);
+      sv.x += x.x; sv.y += x.y; sv.z += x.z; sv.w += x.w;
+    }
+    const float alr = st[m];
+    const float4 be4 = ld4m(st + M + n, cc, 0.f);
+    const float s4[4] = {sv.x, sv.y, sv.z, sv.w}, b4[4] = {be4.x, be4.y, be4.z, be4.w};
+    if (!((alr >= kFloor) && (alr < INFINITY))) bad = 1;
+    if (alr <= 0.45f * kFloor) low |= 1;
+    if (alr < -30.f) neg |= 1;
+    float o4[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      o4[j] = 0.f;
+      if (j < cc) {
+        if (!((s4[j] >= thr) && (s4[j] < INFINITY)) || !((b4[j] >= kFloor) && (b4[j] < INFINITY))) bad = 1;
+        if (b4[j] <= 0.45f * kFloor) low |= 2;
+        if (b4[j] < -30.f) neg |= 2;
+        o4[j] = __builtin_fmaf(fast_log2(s4[j]), kLn2, alr + b4[j]);
+      }
+    }
+    st4m(out + at, cc, make_float4(o4[0], o4[1], o4[2], o4[3]));
+  }
+  const int row_low = __syncthreads_or(low & 1), col_low = __syncthreads_or(low & 2);
+  const int row_neg = __syncthreads_or(neg & 1), col_neg = __syncthreads_or(neg & 2);
+  if ((row_low && col_neg) || (col_low && row_neg)) bad = 1;
+  bad = __syncthreads_or(bad);
+  if (tid == 0) flags[tile] = bad;  // the fix-up launch recomputes a flagged tile
+  if (tile == 0 && tid == 0) {
+    ws_hdr[1] = TR;
+    ws_hdr[2] = TC;
+    ws_hdr[0] = kWsFast;
+  }
 }
 
 // ------------------------------------------------------- sampling sweep

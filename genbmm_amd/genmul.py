@@ -368,6 +368,12 @@ def logbmm(a, b):
     B, M, K = a.shape
     N = b.shape[2]
     S = 1 if _f64(a) else _reduction_splits(B, M, K, N)
+    if S > 1 and _lib.load().genbmm_logbmm_fwd_pieces(B, M, K, N) > 1:
+        # the library's forward cuts the reduction axis of this problem itself (float16 / bfloat16
+        # operands: the float function on the widened tensors, rounded once)
+        if a.dtype in _lib.HALF_SUFFIX:
+            return restore(LogMatMul.apply(a.float(), b.float(), PATH_AUTO).to(a.dtype))
+        S = 1
     if S > 1:  # differentiable torch operations around the same kernels (any order of derivative)
         # float16 / bfloat16 operands: the pieces are formed and joined in float32 and the result is
         # rounded once, as the unsplit kernels do (a piece stored in the half type would round twice)

@@ -171,13 +171,29 @@ int genbmm_logbmm_bwd_path(const float* a, const float* b, const float* out,
                            int B, int M, int K, int N, int path, void* stream);
 
 /*
+ * Into how many pieces genbmm_logbmm_fwd (path GENBMM_PATH_AUTO, and its _f16 /
+ * _bf16 forms) cuts the reduction axis of this problem: 1 (it does not) unless
+ * the result has fewer than 128 tiles of 128 x 128 and K is at least 2048 -
+ * every output tile belongs to one workgroup that walks all of K, and such a
+ * problem would run on a few of the chip's 256 compute units.  The pieces'
+ * sums are added in the workspace (genbmm_logbmm_stats_size counts the room)
+ * before the guard is tested and the logarithm taken, so the result is the
+ * unsplit one up to the order of the additions.  No counterpart in the
+ * reference, whose kernel gives every output cell one thread that walks all
+ * of K (matmul_cuda_kernel.cu:13-45).  genbmm_logbmm_fwd_static never cuts.
+ */
+int genbmm_logbmm_fwd_pieces(int B, int M, int K, int N);
+
+/*
  * genbmm_logbmm_fwd for callers that cannot allocate device memory - code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It
  * has no counterpart in the reference.  The workspace that genbmm_logbmm_fwd takes
  * as `stats` is a fixed array inside the library instead (4 MiB, one copy on every
  * GPU the library runs on, held until the process ends), and nothing is kept for a
  * backward: this is a forward for its own sake, on the same kernels, with results
- * identical to genbmm_logbmm_fwd's.  No hipMalloc / hipFree inside, ever.
+ * identical to genbmm_logbmm_fwd's (a problem that genbmm_logbmm_fwd cuts into
+ * pieces, genbmm_logbmm_fwd_pieces > 1, runs uncut here: equal up to the order
+ * of the additions, and slower).  No hipMalloc / hipFree inside, ever.
  * Limit: B*(M+N) + B*ceil(M/32)*ceil(N/32) + 8 <= genbmm_logbmm_static_limit()
  * (= 1048576 floats; the headline 64 x 512^3 needs 81928); beyond it the call
  * returns GENBMM_E_TOOBIG and does nothing.

@@ -1098,6 +1098,68 @@ def test_long_reductions_with_few_tiles_are_split(gpu, B, M, K, N):
         close(db, w2[1], rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("B,M,K,N", [(16, 96, 4096, 96), (1, 16, 65536, 16), (64, 7, 4100, 7), (3, 130, 2101, 97),
+                                     (2, 300, 5000, 200), (1, 128, 2048, 128), (100, 120, 2300, 127)])
+def test_library_cuts_long_reductions_into_pieces(gpu, B, M, K, N):
+    """genbmm_logbmm_fwd cuts the reduction axis of a problem with few output tiles into pieces,
+    one workgroup each, and joins their sums before the guard and the logarithm: values and both
+    gradients (the ordinary backward on the forward's workspace) against float64; items whose
+    tiles must take the exact routine (a factor that underflows against live terms), a row at the
+    floor, a masked reduction step and a masked row; the workspace is larger by the pieces' sums;
+    float16 / bfloat16 tensors on the same kernels; the entry point without allocation never cuts."""
+    lib = _lib.load()
+    pieces = lib.genbmm_logbmm_fwd_pieces(B, M, K, N)
+    assert pieces > 1
+    assert lib.genbmm_logbmm_fwd_pieces(64, 512, 512, 512) == 1 and lib.genbmm_logbmm_fwd_pieces(512, 128, 128, 128) == 1
+    assert lib.genbmm_logbmm_fwd_pieces(1, 512, 8192, 4096) == 1 and lib.genbmm_logbmm_fwd_pieces(16, 64, 64, 64) == 1
+    size = lib.genbmm_logbmm_stats_size(B, M, K, N)
+    assert size >= pieces * B * M * N + B * (M + N)
+    torch.manual_seed(K + M)
+    a, b, g = torch.randn(B, M, K), torch.randn(B, K, N), torch.randn(B, M, N)
+    a[0, ::2, 0] += 200.0           # the other terms' factors underflow: exact routine
+    b[0, 0, :] -= 200.0
+    a[B - 1, M - 1, :] = -1e9      # a row at the floor
+    g[B - 1, M - 1, :] = 0.0
+    b[B // 2, K - 3, :] = -float("inf")
+    b[B // 2, :, N - 1] = -float("inf")   # a masked column: out = -inf
+    ad, bd, gd = a.to(gpu), b.to(gpu), g.to(gpu)
+    P, s = _lib.ptr, _lib.stream_of(ad)
+    out, st = torch.empty(B, M, N, device=gpu), torch.empty(size, device=gpu)
+    ga, gb = torch.empty_like(ad), torch.empty_like(bd)
+    assert lib.genbmm_logbmm_fwd(P(ad), P(bd), P(out), P(st), B, M, K, N, s) == 0
+    assert lib.genbmm_logbmm_bwd(P(ad), P(bd), P(out), P(gd), P(st), P(ga), P(gb), B, M, K, N, s) == 0
+    torch.cuda.synchronize()
+    want, wa, wb = oracle.logbmm_grads64(a, b, g)
+    col = torch.ones(B, 1, N, dtype=torch.bool)
+    col[B // 2, 0, N - 1] = False   # the masked column: -inf in out, nothing to compare in the gradients
+    rows = torch.ones(B, M, 1, dtype=torch.bool)
+    rows[B - 1, M - 1, 0] = False   # the floor row's own cells: rounding artefacts of 1e9
+    assert bool(torch.isneginf(out[B // 2, :, N - 1]).all())
+    keep = (col & rows).expand(B, M, N)
+    close(out.cpu()[keep], want[keep])
+    close(torch.where(rows.expand(B, M, K), ga.cpu(), torch.zeros(())), torch.where(rows.expand(B, M, K), wa, torch.zeros(())))
+    close(torch.where(col.expand(B, K, N), gb.cpu(), torch.zeros(())), torch.where(col.expand(B, K, N), wb, torch.zeros(())))
+    # the public function takes the same route (and its second derivative the library's)
+    ar, br = ad.clone().requires_grad_(True), bd.clone().requires_grad_(True)
+    o2 = genbmm.logbmm(ar, br)
+    assert torch.equal(o2.detach(), out)
+    # the entry point without allocation: no room for the pieces' sums, the unsplit kernels
+    if lib.genbmm_logbmm_stats_size_path(B, M, K, N, genmul.PATH_MFMA32) <= lib.genbmm_logbmm_static_limit():
+        o3 = torch.empty_like(out)
+        assert lib.genbmm_logbmm_fwd_static(P(ad), P(bd), P(o3), B, M, K, N, s) == 0
+        torch.cuda.synchronize()
+        close(o3.cpu()[keep], want[keep])
+    for dt, sfx, eps in ((torch.float16, "_f16", 2.0 ** -11), (torch.bfloat16, "_bf16", 2.0 ** -8)):
+        ah, bh = ad.to(dt), bd.to(dt)
+        oh = torch.empty(B, M, N, device=gpu, dtype=dt)
+        assert getattr(lib, "genbmm_logbmm_fwd" + sfx)(P(ah), P(bh), P(oh), P(st), B, M, K, N, s) == 0
+        o32 = torch.empty(B, M, N, device=gpu)
+        a32, b32 = ah.float(), bh.float()
+        assert lib.genbmm_logbmm_fwd(P(a32), P(b32), P(o32), P(st), B, M, K, N, s) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(oh, o32.to(dt))
+
+
 @pytest.mark.parametrize("B,M,K,N", [(2, 40, 4096, 30), (1, 7, 8192, 5), (1, 100, 4608, 96), (1, 16, 6000, 16)])
 @pytest.mark.parametrize("prod", [False, True])
 def test_long_reductions_of_the_max_products_are_split(gpu, prod, B, M, K, N):
