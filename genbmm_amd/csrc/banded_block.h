@@ -17,7 +17,8 @@
 // from memory and cut into its parts once.  One wave per block of a step multiplies and writes
 // its 32 x 32 results from the accumulators; four more waves only stage, their loads two steps
 // ahead of their use (two steps' worth of rows in flight per compute unit); all meet at one
-// barrier per step.  The staging waves issue the same loads every step whatever the step meets
+// barrier per step.  (Ahead of the first step, which needs NT + 1 blocks staged, four of the
+// multiplying waves stage half of them.)  The staging waves issue the same loads every step whatever the step meets
 // - addresses are held inside the tensors, rows outside the matrix zeroed when they are staged -
 // so that the counted waits for loads stay exact; a branch around a load costs every wait
 // behind it its count.
@@ -193,172 +194,179 @@ __global__ __launch_bounds__(64 * (kBlkNT + SW)) void k_band_blk_fwd(const BandA
   if (!PREP && tid == 0) *inexact = 0u;
 
   const int role = wave < g.ncw ? wave : wave - g.ncw;  // among the waves of its kind
-  if (wave >= g.ncw) {
-    // ------------------------------------------------------------------ staging
-    constexpr int SP = SW / 2;
-    const int lt = role * 64 + lane, quad = lt & 3, line = (lt >> 2) & 31, half = lt >> 7;  // half: the wave pair
-    auto asrc = [&] {
-      if constexpr (PREP) return static_cast<const float*>(p.ws_ea);
-      else return p.a;
-    }();
-    auto bsrc = [&] {
-      if constexpr (PREP) return static_cast<const float*>(p.ws_eb);
-      else return p.b;
-    }();
-    constexpr int ES = sizeof(*asrc);
-    const long cells_a = rows * Wa, cells_b = rows * Wb;
-    int low = 0;
-    // What does not change from step to step: where a piece lies from its block's first cell
-    // (a piece with no cell inside the band reads its row's first cells instead) and which of
-    // its cells are inside the band.
-    int offa[UA], offb[UB];
-    unsigned ma[UA][4], mb[UB][4];
+  // ------------------------------------------------------------------ staging
+  // The staging waves; the first four multiplying waves stage too, once: before the first step half
+  // of the blocks that it needs are theirs (they would only wait for them).
+  const bool helps = wave < g.ncw && wave < 4;
+  constexpr int SP = SW / 2;
+  const int lt = (wave < g.ncw ? wave & 3 : role) * 64 + lane, quad = lt & 3, line = (lt >> 2) & 31, half = lt >> 7;  // half: the wave pair
+  auto asrc = [&] {
+    if constexpr (PREP) return static_cast<const float*>(p.ws_ea);
+    else return p.a;
+  }();
+  auto bsrc = [&] {
+    if constexpr (PREP) return static_cast<const float*>(p.ws_eb);
+    else return p.b;
+  }();
+  constexpr int ES = sizeof(*asrc);
+  const long cells_a = rows * Wa, cells_b = rows * Wb;
+  int low = 0;
+  // What does not change from step to step: where a piece lies from its block's first cell
+  // (a piece with no cell inside the band reads its row's first cells instead) and which of
+  // its cells are inside the band.
+  int offa[UA], offb[UB];
+  unsigned ma[UA][4], mb[UB][4];
+#pragma unroll
+  for (int u = 0; u < UA; ++u) {
+    const int slab = SP * u + half, c = 16 * slab + 4 * quad - line;
+    offa[u] = line * Wa + (slab < NSa && c > -4 && c < Wa ? c : 0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ma[u][e] = slab < NSa && (unsigned)(c + e) < (unsigned)Wa ? ~0u : 0u;
+  }
+#pragma unroll
+  for (int u = 0; u < UB; ++u) {
+    const int slab = SP * u + half, c = 16 * slab + 4 * quad - g.delta - line;
+    offb[u] = line * Wb + (slab < NSb && c > -4 && c < Wb ? c : 0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) mb[u][e] = slab < NSb && (unsigned)(c + e) < (unsigned)Wb ? ~0u : 0u;
+  }
+  // a piece's place in a plane: [half of the slab's z][line][4 words], the lines of the second
+  // half swapped in fours (the sixteen lanes that store together then meet sixteen banks)
+  const int place = (quad >> 1) * 128 + ((line ^ ((quad >> 1) << 2)) << 2) + (quad & 1) * 2;
+  unsigned* const dst_a = As + half * kBlkSlabWords + place;
+  unsigned* const dst_b = Bs + half * kBlkSlabWords + place;
+
+  // Every step issues the same loads whatever it meets (the waits then count exactly what is
+  // in flight, two steps' worth): all of a block's pieces are read, from addresses held inside
+  // the tensor.  A block's rows outside the matrix read their neighbours in memory and are
+  // zeroed when they are staged; a piece that would cross an end of the tensor is read from
+  // the four cells at that end and moved into place then.
+  struct Where {
+    long first;  // the cell of the tensor that offset 0 stands for
+    int add;     // what a piece's offset from its block's first cell becomes an offset from `first` by
+    int hi;      // the largest offset to read at
+  };
+  // (a piece may begin up to three cells ahead of its block's first cell)
+  const long cell_a0 = (bn + i_start) * Wa, cell_b0 = (bn + i_start - p.r_lu) * Wb;  // first cells of block 0
+  // uniform: no block of this workgroup comes near an end of its tensor
+  const bool inner = cell_a0 >= 4 && cell_a0 + (32L * steps + 31) * Wa + 16 * NSa + 8 <= cells_a && cell_b0 >= 4 &&
+                     cell_b0 + (32L * (steps + NT) + 31) * Wb + 16 * NSb + 8 <= cells_b;
+  auto where = [&](long r0, long cells) __attribute__((always_inline)) {
+    Where w;
+    if (inner) {
+      w.first = r0 - 4;
+      w.add = 4;
+      w.hi = 1 << 30;
+    } else {
+      w.first = min(max(r0 - 4, 0L), cells - 4);
+      w.add = (int)min(max(r0 - w.first, -(1L << 30)), 1L << 30);
+      w.hi = (int)min(cells - 4 - w.first, 1L << 30);
+    }
+    return w;
+  };
+  // a piece as it was meant, from what was read `shift` cells before it (cells that were not read: 0,
+  // they lie outside the tensor)
+  auto moved = [](float4 v, int shift) __attribute__((always_inline)) {
+    const float x[4] = {v.x, v.y, v.z, v.w};
+    float y[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      y[e] = 0.f;
+#pragma unroll
+      for (int f = 0; f < 4; ++f) y[e] = f - e == shift ? x[f] : y[e];
+    }
+    return make_float4(y[0], y[1], y[2], y[3]);
+  };
+  // block k of the first operand: rows i_start + 32 k ..., z from i_start + 32 k - lu_a.
+  // ab: alpha of the block's rows (lanes 0-31 of the first staging wave)
+  auto load_a = [&](int k, float4 (&r)[UA], float& ab) __attribute__((always_inline)) {
+    const int ib = i_start + 32 * k;
+    const Where w = where(cell_a0 + 32 * k * Wa, cells_a);
+    const auto* base = asrc + w.first;
+#pragma unroll
+    for (int u = 0; u < UA; ++u) r[u] = ld4(blk_at(base, (unsigned)(ES * min(max(offa[u] + w.add, 0), w.hi))));
+    if (PREP) ab = p.ws_al[min(bn + ib + (lt & 31), rows - 1)];
+  };
+  // block q of the second: rows i_start - lu_out + 32 q ..., z from that - lu_b - delta.
+  // ab: beta of the block's rows (lanes 32-63 of the first staging wave)
+  auto load_b = [&](int q, float4 (&r)[UB], float& ab) __attribute__((always_inline)) {
+    const int ob = i_start - p.r_lu + 32 * q;
+    const Where w = where(cell_b0 + 32 * q * Wb, cells_b);
+    const auto* base = bsrc + w.first;
+#pragma unroll
+    for (int u = 0; u < UB; ++u) r[u] = ld4(blk_at(base, (unsigned)(ES * min(max(offb[u] + w.add, 0), w.hi))));
+    if (PREP) {
+      const float be = p.ws_be[min(max(bn + ob + (lt & 31), 0L), rows - 1)];
+      ab = lt & 32 ? be : ab;
+    }
+  };
+  auto stage_a = [&](int k, const float4 (&r)[UA], float ab) __attribute__((always_inline)) {
+    unsigned* dst = dst_a + (k & 1) * NSa * kBlkSlabWords;
+    const int ib = i_start + 32 * k, z0 = ib - p.a_lu;
+    const Where w = where(cell_a0 + 32 * k * Wa, cells_a);
+    // uniform: every row of the block is a row of the matrix and every z of its slabs a column; no
+    // piece had to be read elsewhere
+    const bool plain = ib + 31 < n && z0 >= 0 && z0 + 16 * NSa <= n && w.add == 4 && w.hi >= 31 * Wa + 16 * NSa + 4;
 #pragma unroll
     for (int u = 0; u < UA; ++u) {
-      const int slab = SP * u + half, c = 16 * slab + 4 * quad - line;
-      offa[u] = line * Wa + (slab < NSa && c > -4 && c < Wa ? c : 0);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) ma[u][e] = slab < NSa && (unsigned)(c + e) < (unsigned)Wa ? ~0u : 0u;
+      if (SP * u + half < NSa) {
+        float4 v = r[u];
+        if (!plain) {
+          const int at = offa[u] + w.add;
+          v = moved(v, at - min(max(at, 0), w.hi));
+          const int z = z0 + 16 * (SP * u + half) + 4 * quad;
+          const bool row = ib + line < n;
+          v.x = row && (unsigned)(z + 0) < (unsigned)n ? v.x : 0.f;
+          v.y = row && (unsigned)(z + 1) < (unsigned)n ? v.y : 0.f;
+          v.z = row && (unsigned)(z + 2) < (unsigned)n ? v.z : 0.f;
+          v.w = row && (unsigned)(z + 3) < (unsigned)n ? v.w : 0.f;
+        }
+        blk_put<!PREP>(dst + SP * u * kBlkSlabWords, blk_and(v, ma[u]), low);
+      }
     }
+    if (PREP && lt < 32) alpha[(k & 1) * 32 + lt] = ib + lt < n ? ab : 0.f;
+  };
+  auto stage_b = [&](int q, const float4 (&r)[UB], float ab) __attribute__((always_inline)) {
+    const int slot = q % RING;
+    unsigned* dst = dst_b + slot * NSb * kBlkSlabWords;
+    const int ob = i_start - p.r_lu + 32 * q;
+    const Where w = where(cell_b0 + 32 * q * Wb, cells_b);
+    const bool plain = ob >= 0 && ob + 31 < n && w.add == 4 && w.hi >= 31 * Wb + 16 * NSb + 4;  // uniform
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
-      const int slab = SP * u + half, c = 16 * slab + 4 * quad - g.delta - line;
-      offb[u] = line * Wb + (slab < NSb && c > -4 && c < Wb ? c : 0);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) mb[u][e] = slab < NSb && (unsigned)(c + e) < (unsigned)Wb ? ~0u : 0u;
+      if (SP * u + half < NSb) {
+        float4 v = r[u];
+        if (!plain) {
+          const int at = offb[u] + w.add;
+          v = moved(v, at - min(max(at, 0), w.hi));
+          const bool row = (unsigned)(ob + line) < (unsigned)n;
+          v.x = row ? v.x : 0.f;
+          v.y = row ? v.y : 0.f;
+          v.z = row ? v.z : 0.f;
+          v.w = row ? v.w : 0.f;
+        }
+        blk_put<!PREP>(dst + SP * u * kBlkSlabWords, blk_and(v, mb[u]), low);
+      }
     }
-    // a piece's place in a plane: [half of the slab's z][line][4 words], the lines of the second
-    // half swapped in fours (the sixteen lanes that store together then meet sixteen banks)
-    const int place = (quad >> 1) * 128 + ((line ^ ((quad >> 1) << 2)) << 2) + (quad & 1) * 2;
-    unsigned* const dst_a = As + half * kBlkSlabWords + place;
-    unsigned* const dst_b = Bs + half * kBlkSlabWords + place;
+    if (PREP && lt >= 32 && lt < 64) beta[slot * 32 + lt - 32] = (unsigned)(ob + lt - 32) < (unsigned)n ? ab : 0.f;
+  };
 
-    // Every step issues the same loads whatever it meets (the waits then count exactly what is
-    // in flight, two steps' worth): all of a block's pieces are read, from addresses held inside
-    // the tensor.  A block's rows outside the matrix read their neighbours in memory and are
-    // zeroed when they are staged; a piece that would cross an end of the tensor is read from
-    // the four cells at that end and moved into place then.
-    struct Where {
-      long first;  // the cell of the tensor that offset 0 stands for
-      int add;     // what a piece's offset from its block's first cell becomes an offset from `first` by
-      int hi;      // the largest offset to read at
-    };
-    // (a piece may begin up to three cells ahead of its block's first cell)
-    const long cell_a0 = (bn + i_start) * Wa, cell_b0 = (bn + i_start - p.r_lu) * Wb;  // first cells of block 0
-    // uniform: no block of this workgroup comes near an end of its tensor
-    const bool inner = cell_a0 >= 4 && cell_a0 + (32L * steps + 31) * Wa + 16 * NSa + 8 <= cells_a && cell_b0 >= 4 &&
-                       cell_b0 + (32L * (steps + NT) + 31) * Wb + 16 * NSb + 8 <= cells_b;
-    auto where = [&](long r0, long cells) __attribute__((always_inline)) {
-      Where w;
-      if (inner) {
-        w.first = r0 - 4;
-        w.add = 4;
-        w.hi = 1 << 30;
-      } else {
-        w.first = min(max(r0 - 4, 0L), cells - 4);
-        w.add = (int)min(max(r0 - w.first, -(1L << 30)), 1L << 30);
-        w.hi = (int)min(cells - 4 - w.first, 1L << 30);
-      }
-      return w;
-    };
-    // a piece as it was meant, from what was read `shift` cells before it (cells that were not read: 0,
-    // they lie outside the tensor)
-    auto moved = [](float4 v, int shift) __attribute__((always_inline)) {
-      const float x[4] = {v.x, v.y, v.z, v.w};
-      float y[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        y[e] = 0.f;
-#pragma unroll
-        for (int f = 0; f < 4; ++f) y[e] = f - e == shift ? x[f] : y[e];
-      }
-      return make_float4(y[0], y[1], y[2], y[3]);
-    };
-    // block k of the first operand: rows i_start + 32 k ..., z from i_start + 32 k - lu_a.
-    // ab: alpha of the block's rows (lanes 0-31 of the first staging wave)
-    auto load_a = [&](int k, float4 (&r)[UA], float& ab) __attribute__((always_inline)) {
-      const int ib = i_start + 32 * k;
-      const Where w = where(cell_a0 + 32 * k * Wa, cells_a);
-      const auto* base = asrc + w.first;
-#pragma unroll
-      for (int u = 0; u < UA; ++u) r[u] = ld4(blk_at(base, (unsigned)(ES * min(max(offa[u] + w.add, 0), w.hi))));
-      if (PREP) ab = p.ws_al[min(bn + ib + (lt & 31), rows - 1)];
-    };
-    // block q of the second: rows i_start - lu_out + 32 q ..., z from that - lu_b - delta.
-    // ab: beta of the block's rows (lanes 32-63 of the first staging wave)
-    auto load_b = [&](int q, float4 (&r)[UB], float& ab) __attribute__((always_inline)) {
-      const int ob = i_start - p.r_lu + 32 * q;
-      const Where w = where(cell_b0 + 32 * q * Wb, cells_b);
-      const auto* base = bsrc + w.first;
-#pragma unroll
-      for (int u = 0; u < UB; ++u) r[u] = ld4(blk_at(base, (unsigned)(ES * min(max(offb[u] + w.add, 0), w.hi))));
-      if (PREP) {
-        const float be = p.ws_be[min(max(bn + ob + (lt & 31), 0L), rows - 1)];
-        ab = lt & 32 ? be : ab;
-      }
-    };
-    auto stage_a = [&](int k, const float4 (&r)[UA], float ab) __attribute__((always_inline)) {
-      unsigned* dst = dst_a + (k & 1) * NSa * kBlkSlabWords;
-      const int ib = i_start + 32 * k, z0 = ib - p.a_lu;
-      const Where w = where(cell_a0 + 32 * k * Wa, cells_a);
-      // uniform: every row of the block is a row of the matrix and every z of its slabs a column; no
-      // piece had to be read elsewhere
-      const bool plain = ib + 31 < n && z0 >= 0 && z0 + 16 * NSa <= n && w.add == 4 && w.hi >= 31 * Wa + 16 * NSa + 4;
-#pragma unroll
-      for (int u = 0; u < UA; ++u) {
-        if (SP * u + half < NSa) {
-          float4 v = r[u];
-          if (!plain) {
-            const int at = offa[u] + w.add;
-            v = moved(v, at - min(max(at, 0), w.hi));
-            const int z = z0 + 16 * (SP * u + half) + 4 * quad;
-            const bool row = ib + line < n;
-            v.x = row && (unsigned)(z + 0) < (unsigned)n ? v.x : 0.f;
-            v.y = row && (unsigned)(z + 1) < (unsigned)n ? v.y : 0.f;
-            v.z = row && (unsigned)(z + 2) < (unsigned)n ? v.z : 0.f;
-            v.w = row && (unsigned)(z + 3) < (unsigned)n ? v.w : 0.f;
-          }
-          blk_put<!PREP>(dst + SP * u * kBlkSlabWords, blk_and(v, ma[u]), low);
-        }
-      }
-      if (PREP && lt < 32) alpha[(k & 1) * 32 + lt] = ib + lt < n ? ab : 0.f;
-    };
-    auto stage_b = [&](int q, const float4 (&r)[UB], float ab) __attribute__((always_inline)) {
-      const int slot = q % RING;
-      unsigned* dst = dst_b + slot * NSb * kBlkSlabWords;
-      const int ob = i_start - p.r_lu + 32 * q;
-      const Where w = where(cell_b0 + 32 * q * Wb, cells_b);
-      const bool plain = ob >= 0 && ob + 31 < n && w.add == 4 && w.hi >= 31 * Wb + 16 * NSb + 4;  // uniform
-#pragma unroll
-      for (int u = 0; u < UB; ++u) {
-        if (SP * u + half < NSb) {
-          float4 v = r[u];
-          if (!plain) {
-            const int at = offb[u] + w.add;
-            v = moved(v, at - min(max(at, 0), w.hi));
-            const bool row = (unsigned)(ob + line) < (unsigned)n;
-            v.x = row ? v.x : 0.f;
-            v.y = row ? v.y : 0.f;
-            v.z = row ? v.z : 0.f;
-            v.w = row ? v.w : 0.f;
-          }
-          blk_put<!PREP>(dst + SP * u * kBlkSlabWords, blk_and(v, mb[u]), low);
-        }
-      }
-      if (PREP && lt >= 32 && lt < 64) beta[slot * 32 + lt - 32] = (unsigned)(ob + lt - 32) < (unsigned)n ? ab : 0.f;
-    };
-
+  // of the NT - 1 older blocks of the second operand that step 0 meets, the first `helped` are staged by
+  // the multiplying waves: half of the NT + 1 blocks to stage before the first step
+  const int helped = g.ncw >= 4 ? min(NT - 1, (NT + 2) / 2) : 0;
+  if (wave >= g.ncw) {
     float4 ra0[UA], rb0[UB], ra1[UA], rb1[UB];
     float aa0 = 0.f, aa1 = 0.f;  // alpha (lanes 0-31 of the first staging wave) or beta (its lanes 32-63)
     const int last = steps - 1;
     {
       // the blocks of the second operand that step 0 meets beside its own newest one
+      // (blocks helped ... NT - 2 here, 0 ... helped - 1 by the multiplying waves that help)
       float4 pro[kBlkNT - 1][UB];
       float pab[kBlkNT - 1];
 #pragma unroll
       for (int q = 0; q < kBlkNT - 1; ++q) {
         pab[q] = 0.f;
-        load_b(min(q, NT - 1), pro[q], pab[q]);
+        load_b(min(helped + q, NT - 1), pro[q], pab[q]);
       }
       load_a(0, ra0, aa0);
       load_b(NT - 1, rb0, aa0);
@@ -366,7 +374,7 @@ __global__ __launch_bounds__(64 * (kBlkNT + SW)) void k_band_blk_fwd(const BandA
       load_b(min(1, last) + NT - 1, rb1, aa1);
 #pragma unroll
       for (int q = 0; q < kBlkNT - 1; ++q)
-        if (q < NT - 1) stage_b(q, pro[q], pab[q]);
+        if (helped + q < NT - 1) stage_b(helped + q, pro[q], pab[q]);
     }
     stage_a(0, ra0, aa0);
     stage_b(NT - 1, rb0, aa0);
@@ -414,7 +422,20 @@ __global__ __launch_bounds__(64 * (kBlkNT + SW)) void k_band_blk_fwd(const BandA
       asm volatile("" : "+v"(x));
       return x;
     };
+    if (helps) {
+      float4 pro[(kBlkNT + 1) / 2][UB];
+      float pab[(kBlkNT + 1) / 2];
+#pragma unroll
+      for (int q = 0; q < (kBlkNT + 1) / 2; ++q) {
+        pab[q] = 0.f;
+        load_b(min(q, NT - 1), pro[q], pab[q]);
+      }
+#pragma unroll
+      for (int q = 0; q < (kBlkNT + 1) / 2; ++q)
+        if (q < helped) stage_b(q, pro[q], pab[q]);
+    }
     __syncthreads();
+    if (!PREP && low < kBlkLowExp) *inexact = 1u;  // (behind the barrier: thread 0 has cleared the flag)
     for (int s = 0; s < steps; ++s) {
       const int ib = i_start + 32 * s;
 
