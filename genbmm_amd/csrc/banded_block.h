@@ -248,12 +248,18 @@ __global__ __launch_bounds__(64 * (kBlkNT + SW)) void k_band_blk_fwd(const BandA
   };
   // (a piece may begin up to three cells ahead of its block's first cell)
   const long cell_a0 = (bn + i_start) * Wa, cell_b0 = (bn + i_start - p.r_lu) * Wb;  // first cells of block 0
-  // uniform: no block of this workgroup comes near an end of its tensor
-  const bool inner = cell_a0 >= 4 && cell_a0 + (32L * steps + 31) * Wa + 16 * NSa + 8 <= cells_a && cell_b0 >= 4 &&
-                     cell_b0 + (32L * (steps + NT) + 31) * Wb + 16 * NSb + 8 <= cells_b;
-  auto where = [&](long r0, long cells) __attribute__((always_inline)) {
+  // the blocks of this workgroup (first operand: k, second: q) that lie clear of their tensor's ends
+  auto clear_of_ends = [](long cell0, long per_block, long span, long cells, int& lo, int& hi) {
+    lo = cell0 >= 4 ? 0 : (int)min((4 - cell0 + per_block - 1) / per_block, 1L << 30);
+    const long room = cells - span - cell0;
+    hi = room < 0 ? -1 : (int)min(room / per_block, 1L << 30);
+  };
+  int ka_lo, ka_hi, qb_lo, qb_hi;
+  clear_of_ends(cell_a0, 32L * Wa, 31L * Wa + 16 * NSa + 8, cells_a, ka_lo, ka_hi);
+  clear_of_ends(cell_b0, 32L * Wb, 31L * Wb + 16 * NSb + 8, cells_b, qb_lo, qb_hi);
+  auto where = [&](long r0, long cells, bool clear) __attribute__((always_inline)) {
     Where w;
-    if (inner) {
+    if (clear) {  // uniform
       w.first = r0 - 4;
       w.add = 4;
       w.hi = 1 << 30;
@@ -281,7 +287,7 @@ __global__ __launch_bounds__(64 * (kBlkNT + SW)) void k_band_blk_fwd(const BandA
   // ab: alpha of the block's rows (lanes 0-31 of the first staging wave)
   auto load_a = [&](int k, float4 (&r)[UA], float& ab) __attribute__((always_inline)) {
     const int ib = i_start + 32 * k;
-    const Where w = where(cell_a0 + 32 * k * Wa, cells_a);
+    const Where w = where(cell_a0 + 32 * k * Wa, cells_a, k >= ka_lo && k <= ka_hi);
     const auto* base = asrc + w.first;
 #pragma unroll
     for (int u = 0; u < UA; ++u) r[u] = ld4(blk_at(base, (unsigned)(ES * min(max(offa[u] + w.add, 0), w.hi))));
@@ -291,7 +297,7 @@ __global__ __launch_bounds__(64 * (kBlkNT + SW)) void k_band_blk_fwd(const BandA
   // ab: beta of the block's rows (lanes 32-63 of the first staging wave)
   auto load_b = [&](int q, float4 (&r)[UB], float& ab) __attribute__((always_inline)) {
     const int ob = i_start - p.r_lu + 32 * q;
-    const Where w = where(cell_b0 + 32 * q * Wb, cells_b);
+    const Where w = where(cell_b0 + 32 * q * Wb, cells_b, q >= qb_lo && q <= qb_hi);
     const auto* base = bsrc + w.first;
 #pragma unroll
     for (int u = 0; u < UB; ++u) r[u] = ld4(blk_at(base, (unsigned)(ES * min(max(offb[u] + w.add, 0), w.hi))));
@@ -303,7 +309,7 @@ __global__ __launch_bounds__(64 * (kBlkNT + SW)) void k_band_blk_fwd(const BandA
   auto stage_a = [&](int k, const float4 (&r)[UA], float ab) __attribute__((always_inline)) {
     unsigned* dst = dst_a + (k & 1) * NSa * kBlkSlabWords;
     const int ib = i_start + 32 * k, z0 = ib - p.a_lu;
-    const Where w = where(cell_a0 + 32 * k * Wa, cells_a);
+    const Where w = where(cell_a0 + 32 * k * Wa, cells_a, k >= ka_lo && k <= ka_hi);
     // uniform: every row of the block is a row of the matrix and every z of its slabs a column; no
     // piece had to be read elsewhere
     const bool plain = ib + 31 < n && z0 >= 0 && z0 + 16 * NSa <= n && w.add == 4 && w.hi >= 31 * Wa + 16 * NSa + 4;
@@ -330,7 +336,7 @@ __global__ __launch_bounds__(64 * (kBlkNT + SW)) void k_band_blk_fwd(const BandA
     const int slot = q % RING;
     unsigned* dst = dst_b + slot * NSb * kBlkSlabWords;
     const int ob = i_start - p.r_lu + 32 * q;
-    const Where w = where(cell_b0 + 32 * q * Wb, cells_b);
+    const Where w = where(cell_b0 + 32 * q * Wb, cells_b, q >= qb_lo && q <= qb_hi);
     const bool plain = ob >= 0 && ob + 31 < n && w.add == 4 && w.hi >= 31 * Wb + 16 * NSb + 4;  // uniform
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
