@@ -1,13 +1,15 @@
 // Double-precision entry points (gfx950).  The reference instantiates every kernel
 // for double as well (AT_DISPATCH_FLOATING_TYPES_AND_HALF, matmul_cuda_kernel.cu:489
 // and on, banded_cuda_kernel.cu:389 and on).  logbmm forward and backward run factored on
-// the double-precision matrix instruction (f64_mm.h).  Everything else here is the
+// the double-precision matrix instruction (f64_mm.h); the max / prod-max products run tiled
+// through LDS and their backward is a scatter (f64_max.h).  Everything else here is the
 // reference's algorithm in the plain form - one lane per result cell, the reduction axis
 // walked in ascending order, lanes along the contiguous axis so that loads and stores
 // coalesce.
 #include <cfloat>
 
 #include "banded_cells.h"
+#include "f64_max.h"
 #include "f64_mm.h"
 
 namespace GENBMM_NS {
@@ -18,9 +20,8 @@ constexpr double kFloorD = -1e9;
 enum { kLog = 0, kMax = 1, kSample = 2, kProdMax = 3 };  // the reference's dense modes
 
 // --------------------------------------------------------------- dense forward
-// Reference kernels matmul_cuda_kernel.cu:13-45 (log), :47-75 (max), :77-121
-// (sample), :124-152 (prod-max): two passes (maximum, then sum of exponentials)
-// for the log-sum-exp, strict '>' from -1e9 / index -1 for the arg-max modes.
+// Reference kernels matmul_cuda_kernel.cu:13-45 (log) and :77-121 (sample): two passes
+// (maximum, then sum of exponentials) for the log-sum-exp.
 template <int MODE>
 __global__ __launch_bounds__(256) void k64_fwd(const double* __restrict__ a,
                                               const double* __restrict__ b,
@@ -35,19 +36,6 @@ __global__ __launch_bounds__(256) void k64_fwd(const double* __restrict__ a,
   const double* arow = a + bm * K;
   const double* bcol = b + batch * K * N + n;
   double m = kFloorD;
-  if (MODE == kMax || MODE == kProdMax) {
-    int ind = -1;
-    for (int k = 0; k < K; ++k) {
-      const double v = MODE == kProdMax ? arow[k] * bcol[(long)k * N] : arow[k] + bcol[(long)k * N];
-      if (v > m) {
-        m = v;
-        ind = k;
-      }
-    }
-    out[e] = m;
-    idx[e] = ind;
-    return;
-  }
   for (int k = 0; k < K; ++k) {
     const double v = arow[k] + bcol[(long)k * N];
     if (v > m) m = v;
@@ -204,53 +192,6 @@ __global__ __launch_bounds__(256) void k64_bb_b(const BB64 p, long total) {
   p.gb[e] = acc;
 }
 
-// ---------------------------------------------------------- arg-max backward
-// grad_a[m,k] = sum_n [k == idx[m,n]] g[m,n] (* b[k,n]); grad_b[k,n] = sum_m [...]
-// g[m,n] (* a[m,k]): one lane per gradient cell scanning the reduced axis in
-// ascending order, products rounded before the add - the reference's kernels
-// :336-456 as they stand, so the sums are bit-identical to a sequential loop.
-template <bool PROD>
-__global__ __launch_bounds__(256) void k64_argmax_bwd_a(const double* __restrict__ b,
-                                                       const int32_t* __restrict__ idx,
-                                                       const double* __restrict__ g,
-                                                       double* __restrict__ grad_a, int M, int K,
-                                                       int N, long total) {
-  const long e = (long)blockIdx.x * 256 + threadIdx.x;
-  if (e >= total) return;
-  const int k = (int)(e % K);
-  const long bm = e / K;
-  const long batch = bm / M;
-  const int32_t* irow = idx + bm * N;
-  const double* grow = g + bm * N;
-  const double* brow = PROD ? b + (batch * K + k) * N : nullptr;
-  double acc = 0.0;
-  for (int n = 0; n < N; ++n)
-    if (irow[n] == k) acc = __dadd_rn(acc, PROD ? __dmul_rn(brow[n], grow[n]) : grow[n]);
-  grad_a[e] = acc;
-}
-
-template <bool PROD>
-__global__ __launch_bounds__(256) void k64_argmax_bwd_b(const double* __restrict__ a,
-                                                       const int32_t* __restrict__ idx,
-                                                       const double* __restrict__ g,
-                                                       double* __restrict__ grad_b, int M, int K,
-                                                       int N, long total) {
-  const long e = (long)blockIdx.x * 256 + threadIdx.x;
-  if (e >= total) return;
-  const int n = (int)(e % N);
-  const long bk = e / N;
-  const long batch = bk / K;
-  const int k = (int)(bk - batch * K);
-  const int32_t* icol = idx + batch * M * N + n;
-  const double* gcol = g + batch * M * N + n;
-  const double* acol = PROD ? a + batch * M * K + k : nullptr;
-  double acc = 0.0;
-  for (int m = 0; m < M; ++m)
-    if (icol[(long)m * N] == k)
-      acc = __dadd_rn(acc, PROD ? __dmul_rn(acol[(long)m * K], gcol[(long)m * N]) : gcol[(long)m * N]);
-  grad_b[e] = acc;
-}
-
 // ---------------------------------------------------------------- dispatch
 template <int MODE>
 int run_fwd64(const double* a, const double* b, double* out, int32_t* idx, uint64_t seed,
@@ -265,6 +206,31 @@ int run_fwd64(const double* a, const double* b, double* out, int32_t* idx, uint6
   return launch_status();
 }
 
+// max / prod-max forward: one workgroup per 64 x 64 tile of the result
+template <bool PROD>
+int run_max_fwd64(const double* a, const double* b, double* out, int32_t* idx, int B, int M, int K, int N,
+                  void* stream) {
+  if (int e = check_dense_dims(B, M, K, N)) return e;
+  const int64_t mk = (int64_t)B * M * K, kn = (int64_t)B * K * N, mn = (int64_t)B * M * N;
+  if (missing(a, mk) || missing(b, kn) || missing(out, mn) || missing(idx, mn)) return GENBMM_E_NULLPTR;
+  if (mn == 0) return GENBMM_OK;
+  const int tiles_m = ceil_div(M, kD64Tile), tiles_n = ceil_div(N, kD64Tile);
+  const int64_t total = (int64_t)B * tiles_m * tiles_n;
+  if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
+  const int vec_o = (N % 4 == 0) && aligned16(out) && aligned16(idx);
+  hipLaunchKernelGGL((k64_max_fwd<PROD>), dim3((unsigned)total), dim3(256), 0, (hipStream_t)stream, a, b, out, idx,
+                     M, K, N, tiles_m, tiles_n, vec_o);
+  return launch_status();
+}
+
+// Parts per workgroup for a reduction axis of K cells: the smallest power of two that covers it,
+// at most `most` (2^most parts; 64 lanes in all).
+inline int argmax64_parts_shift(int K, int most) {
+  int ps = 0;
+  while (ps < most && (kArg64 << ps) < K) ++ps;
+  return ps;
+}
+
 template <bool PROD>
 int run_argmax_bwd64(const double* a, const double* b, const int32_t* idx, const double* g,
                      double* grad_a, double* grad_b, int B, int M, int K, int N, void* stream) {
@@ -273,14 +239,19 @@ int run_argmax_bwd64(const double* a, const double* b, const int32_t* idx, const
   if (missing(idx, mn) || missing(g, mn) || missing(grad_a, mk) || missing(grad_b, kn) ||
       (PROD && (missing(a, mk) || missing(b, kn))))
     return GENBMM_E_NULLPTR;
-  hipStream_t s = (hipStream_t)stream;
-  if (mk > 0) hipLaunchKernelGGL((k64_argmax_bwd_a<PROD>), blocks_for(mk), dim3(256), 0, s, b, idx, g,
-                                 grad_a, M, K, N, (long)mk);
-  if (kn > 0) hipLaunchKernelGGL((k64_argmax_bwd_b<PROD>), blocks_for(kn), dim3(256), 0, s, a, idx, g,
-                                 grad_b, M, K, N, (long)kn);
+  if (mk == 0 && kn == 0) return GENBMM_OK;
+  // (an empty M or N leaves one gradient without workgroups; the other is then all zeros)
+  const int ps_a = argmax64_parts_shift(K, 6);
+  const int row_tiles = ceil_div(M, 64 >> ps_a), kc_a = ceil_div(K, kArg64 << ps_a);
+  // columns: runs of at least 16 adjacent columns (128 bytes of every row of idx-and-g read)
+  const int ps_b = argmax64_parts_shift(K, 2);
+  const int col_tiles = ceil_div(N, 64 >> ps_b), kc_b = ceil_div(K, kArg64 << ps_b);
+  const int64_t total = (int64_t)B * ((int64_t)row_tiles * kc_a + (int64_t)col_tiles * kc_b);
+  if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
+  hipLaunchKernelGGL((k64_argmax_bwd_both<PROD>), dim3((unsigned)total), dim3(64), 0, (hipStream_t)stream, a, b, idx,
+                     g, grad_a, grad_b, M, K, N, row_tiles, kc_a, ps_a, col_tiles, kc_b, ps_b);
   return launch_status();
 }
-
 
 // The factored matrix-core kernels take problems big enough for their tiles to pay and small
 // enough for a whole row or column of maxima in LDS.
@@ -328,12 +299,12 @@ int genbmm_logbmm_fwd_f64(const double* a, const double* b, double* out, int B, 
 
 int genbmm_maxbmm_fwd_f64(const double* a, const double* b, double* out, int32_t* idx, int B, int M,
                           int K, int N, void* stream) {
-  return GENBMM_NS::run_fwd64<GENBMM_NS::kMax>(a, b, out, idx, 0, 0, B, M, K, N, stream);
+  return GENBMM_NS::run_max_fwd64<false>(a, b, out, idx, B, M, K, N, stream);
 }
 
 int genbmm_prodmaxbmm_fwd_f64(const double* a, const double* b, double* out, int32_t* idx, int B,
                               int M, int K, int N, void* stream) {
-  return GENBMM_NS::run_fwd64<GENBMM_NS::kProdMax>(a, b, out, idx, 0, 0, B, M, K, N, stream);
+  return GENBMM_NS::run_max_fwd64<true>(a, b, out, idx, B, M, K, N, stream);
 }
 
 int genbmm_samplebmm_fwd_f64(const double* a, const double* b, double* out, int32_t* idx,

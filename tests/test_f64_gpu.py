@@ -109,7 +109,12 @@ def test_logbmm_f64_factoring_guard(gpu):
     close(gb, wb, 1e-10, 1e-9)
 
 
-@pytest.mark.parametrize("B,M,K,N", SHAPES)
+# beside SHAPES: several slabs of 16 with a cut last one, reduction axes longer than one workgroup of
+# the backward covers (128 cells of a column, 2048 of a row), tiles cut in both directions
+MAX_SHAPES = SHAPES + [(2, 20, 300, 24), (1, 5, 2100, 3), (3, 70, 40, 130), (1, 64, 16, 64), (2, 67, 17, 4)]
+
+
+@pytest.mark.parametrize("B,M,K,N", MAX_SHAPES)
 @pytest.mark.parametrize("prod", [False, True])
 def test_max_f64_bit_exact(gpu, B, M, K, N, prod):
     torch.manual_seed(M + N)
