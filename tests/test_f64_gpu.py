@@ -144,6 +144,68 @@ def test_max_f64_bit_exact(gpu, B, M, K, N, prod):
     assert torch.equal(i2.cpu(), si) and torch.equal(o2.cpu(), sv)
 
 
+def test_max_f64_at_the_benchmark_size(gpu):
+    """(512,128,128,128) on the 1/8 grid (max) and Uniform(0,1] (prod-max), EVERY batch item: values
+    and indices bit-exact against the broadcast closed form evaluated on the device in float64
+    (index = the lowest k that attains the maximum); max gradients bit-exact against the one-hot
+    scatter (g on the 1/8 grid: the sums are exact in any order), prod-max gradients against the
+    scatter to rtol 1e-12; three items bit-exact against the sequential oracle, which also pins
+    the order of the prod-max sums."""
+    torch.manual_seed(1)
+    B, M, K, N = 512, 128, 128, 128
+    g = grid(B, M, N).clamp(-4, 4)
+    gd = g.to(gpu)
+    for prod in (False, True):
+        if prod:
+            a, b = (1 - torch.rand(B, M, K)).double(), (1 - torch.rand(B, K, N)).double()
+            op = genbmm.prodmaxbmm
+        else:
+            a, b = grid(B, M, K), grid(B, K, N)
+            op = genbmm.maxbmm
+        ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+        out = op(ad, bd)
+        ga, gb = torch.autograd.grad(out, (ad, bd), gd)
+        lib = _lib.load()
+        o2 = torch.empty(B, M, N, dtype=torch.float64, device=gpu)
+        idx = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
+        fn = lib.genbmm_prodmaxbmm_fwd_f64 if prod else lib.genbmm_maxbmm_fwd_f64
+        assert fn(_lib.ptr(ad.detach()), _lib.ptr(bd.detach()), _lib.ptr(o2), _lib.ptr(idx), B, M, K, N,
+                  _lib.stream_of(o2)) == 0
+        pick = [0, 300, 511]
+        sv, si = oracle.seq_maxbmm_fwd(a[pick], b[pick], prod, dtype=F64)
+        assert torch.equal(out[pick].detach().cpu(), sv) and torch.equal(idx[pick].cpu(), si)
+        wa, wb = oracle.seq_argmax_bwd(a[pick] if prod else K, b[pick], si, g[pick], prod, dtype=F64)
+        assert torch.equal(ga[pick].cpu(), wa) and torch.equal(gb[pick].cpu(), wb)
+        ks = torch.arange(K, device=gpu).view(1, 1, K, 1)
+        ties = 0
+        for i in range(0, B, 64):
+            sl = slice(i, i + 64)
+            x, y = ad[sl].detach().unsqueeze(-1), bd[sl].detach().unsqueeze(-3)
+            s = x * y if prod else x + y                                          # (64, M, K, N)
+            mv = s.max(-2).values
+            hit = s == mv.unsqueeze(-2)
+            first = torch.where(hit, ks, torch.full_like(ks, K)).min(-2).values
+            assert torch.equal(out[sl].detach(), mv) and torch.equal(o2[sl], mv), i
+            assert torch.equal(idx[sl].long(), first), i
+            ties += int((hit.sum(-2) > 1).sum())
+            wa64 = torch.zeros(64, M, K, device=gpu, dtype=torch.float64)
+            wb64 = torch.zeros(64, K, N, device=gpu, dtype=torch.float64)
+            if prod:
+                bsel = torch.gather(bd[sl].detach(), 1, first)
+                asel = torch.gather(ad[sl].detach().unsqueeze(2).expand(64, M, N, K), 3, first.unsqueeze(-1)).squeeze(-1)
+                wa64.scatter_add_(2, first, bsel * gd[sl])
+                wb64.scatter_add_(1, first, asel * gd[sl])
+                assert torch.allclose(ga[sl], wa64, rtol=1e-12, atol=1e-12), i
+                assert torch.allclose(gb[sl], wb64, rtol=1e-12, atol=1e-12), i
+            else:
+                wa64.scatter_add_(2, first, gd[sl])
+                wb64.scatter_add_(1, first, gd[sl])
+                assert torch.equal(ga[sl], wa64) and torch.equal(gb[sl], wb64), i
+            del s, hit, first, mv
+        if not prod:
+            assert ties > 100 * B   # ties are present and resolve to the lowest k
+
+
 def test_sample_f64_follows_the_cdf_rule(gpu):
     """Index = the reference's walk (matmul_cuda_kernel.cu:109-118) on the uniform of the
     cell, which is the float path's Philox draw for the same seed and offset."""
