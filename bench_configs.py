@@ -376,7 +376,7 @@ def main():
         dense_max(lib, dev, 256, 256, 256, 256, r, prod=True)
     if "sample" in want:
         dense_sample(lib, dev, 64, 512, 512, 512, r)
-        dense_sample(lib, dev, 16, 512, 1024, 512, r)  # K beyond the matrix-core sweep's 992
+        dense_sample(lib, dev, 16, 512, 1024, 512, r)  # K beyond the 62 slabs of the sweep's six-bit tag
     if "banded" in want:
         for mode in (3, 0, 1, 2):
             banded(lib, dev, 64, 4096, 32, 32, mode, r)

@@ -718,7 +718,7 @@ int launch_sample_sweep_mfma(DenseArgs p, const float* stats, int* flags, int B,
   const LogPrepared ws = prepared_of(stats, B, M, K, N);
   hipLaunchKernelGGL(k_sample_sweep_split<T>, dim3((unsigned)total), dim3(T::NT), 0, s, ws.ea, ws.eb,
                      p.out, stats, flags, ws.r, p.idx, p.seed, p.offset, M, K, N, tiles_m, tiles_n,
-                     TF::TR, TF::TC, p.tiles_m, p.tiles_n);
+                     TF::TR, TF::TC, p.tiles_m, p.tiles_n, ceil_div(K, kMS) <= 62 ? 63 : 127);
   if (int e = launch_status()) return e;
   const int ftotal = B * p.tiles_m * p.tiles_n;
   hipLaunchKernelGGL((k_sample_fixup<CfgWide, TF::TR, TF::TC>), dim3(min(ftotal, kFixupGrid)),

@@ -901,14 +901,18 @@ void k_log_bwd_mfma_both_lean(const elem_t* __restrict__ g, const LeanSrc src, c
 // slabs that ended below the target = the slab in which the prefix passes it, and the
 // value (six mantissa bits short) is -(t - prefix at the start of that slab) = -rem.
 // Two vector instructions per cell and slab beside the matrix-core work.  Results:
-// the code -2 - slab in idx (0 if the prefix never reaches t) and rem in `remw`; the
+// the code -2 - slab in idx (K - 1, the final index, if the prefix never reaches t: the
+// accumulators start at -t, so their roundings are not the forward's, and a draw within some
+// 1e-6 of 1 can end a hair above the sum) and rem in `remw`; the
 // terms of that one slab are walked by the resolve kernel.  At most kSampleSlabs
-// slabs (the tag's range).  A tile with a cell whose S is below 2^-40 or not finite,
+// slabs: up to 62 with a tag of six bits, beyond that with seven (rem is then seven mantissa
+// bits short: 1.5e-5 of itself, which moves a boundary between two terms by at most that
+// share of the cell's total mass).  A tile with a cell whose S is below 2^-40 or not finite,
 // or that lies in a tile the forward flagged, sets that flag and leaves: the forward's
 // tile is redone exactly.  The sweep's own tile shape is free: 128 x 128 with four
 // waves lets two workgroups share a compute unit within the 256 registers per lane,
 // so that one's vector work overlaps the other's matrix-core work.
-constexpr int kSampleSlabs = 62;
+constexpr int kSampleSlabs = 126;
 // The reciprocal of the forward's 1 / S is S within two roundings; a target within 2^-22 of the sum
 // the sweep adds up could lie beyond it and never be passed.  Every target is shrunk by that
 // much instead (the boundaries between the terms move by 2.4e-7 of the total mass).

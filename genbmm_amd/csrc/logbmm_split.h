@@ -503,8 +503,8 @@ __global__ __launch_bounds__(256) void k_log_fwd_join(const float* __restrict__ 
 // factors EA, EB - cut into their three parts while they are staged, no exponential - with the
 // accumulators started at -t, t = u S the cell's target; after every slab of 16 terms a
 // register per cell keeps, by a signed-integer minimum over (value with its low six bits
-// replaced by 62 - slab), the slab in which the prefix sum passes t and -rem at the start of
-// that slab.  S is the reciprocal of the forward's 1 / S, the targets are shrunk by 2^-22;
+// replaced by 62 - slab; seven bits and 126 - slab for more than 62 slabs: `tmask` = 63 or 127),
+// the slab in which the prefix sum passes t and -rem at the start of that slab.  S is the reciprocal of the forward's 1 / S, the targets are shrunk by 2^-22;
 // results: the code -2 - slab in idx, rem in `remw`.  The partial products are added in the
 // forward's order, so the sums the sweep compares with its targets are the forward's.  A tile
 // with a cell whose S is below 2^-40 or not finite, or that lies in a tile the forward
@@ -517,7 +517,7 @@ void k_sample_sweep_split(const float* __restrict__ ws_ea, const float* __restri
                           const elem_t* __restrict__ out, const float* __restrict__ stats,
                           int* __restrict__ flags, float* __restrict__ remw, int32_t* __restrict__ idx,
                           uint64_t seed, uint64_t offset, int M, int K, int N, int tiles_m, int tiles_n, int ftr,
-                          int ftc, int ftiles_m, int ftiles_n) {
+                          int ftc, int ftiles_m, int ftiles_n, int tmask) {
   constexpr bool RAGGED = true;
   constexpr int NT = T::NT;
   using SA = SplitT<T::TR, NT>;
@@ -586,7 +586,7 @@ void k_sample_sweep_split(const float* __restrict__ ws_ea, const float* __restri
         const bool ok = !RAGGED || (m < M && n < N);
         const float nt = ok ? remw[((long)batch * M + m) * N + n] : 0.f;
         acc[br][bc][i] = nt;
-        low[br][bc][i] = __float_as_int(nt) | 63;  // tag 63: no slab has ended below t
+        low[br][bc][i] = __float_as_int(nt) | tmask;  // all tag bits set: no slab has ended below t
       }
     }
 
@@ -635,13 +635,13 @@ void k_sample_sweep_split(const float* __restrict__ ws_ea, const float* __restri
   stage(0);
   split_loop(slabs, split_early<NT>(wave), load, stage, [&](int buf) __attribute__((always_inline)) {
     split_slab<SA, SB>(As(buf), Bs(buf), wm0, wn0, wave, lane, acc);
-    const int tag = 62 - s_mma;
+    const int tag = tmask - 1 - s_mma;
     ++s_mma;
 #pragma unroll
     for (int x = 0; x < 4; ++x)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int v = (__float_as_int(acc[x >> 1][x & 1][i]) & ~63) | (tag & 63);  // one v_bfi_b32
+        const int v = (__float_as_int(acc[x >> 1][x & 1][i]) & ~tmask) | (tag & tmask);  // one v_bfi_b32
         low[x >> 1][x & 1][i] = min(low[x >> 1][x & 1][i], v);
       }
   });
@@ -658,9 +658,10 @@ void k_sample_sweep_split(const float* __restrict__ ws_ea, const float* __restri
         const int m = m0 + wm0 + br * 32 + mfma_row(i, lane);
         if (RAGGED && m >= M) continue;
         const long cell = ((long)batch * M + m) * N + n;
-        const int below = 63 - (low[br][bc][i] & 63);
-        idx[cell] = below >= slabs ? 0 : -2 - below;
-        remw[cell] = -__int_as_float(low[br][bc][i] & ~63);
+        const int below = tmask - (low[br][bc][i] & tmask);
+        // a target that the sums never reach lies within their rounding of the total: the last term
+        idx[cell] = below >= slabs ? K - 1 : -2 - below;
+        remw[cell] = -__int_as_float(low[br][bc][i] & ~tmask);
       }
     }
 }

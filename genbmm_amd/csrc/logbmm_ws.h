@@ -29,11 +29,11 @@ int log_fwd_with_factors(const elem_t* a, const elem_t* b, elem_t* out, float* s
 bool log_fwd_writes_factors(const float* stats, int B, int M, int K, int N, LogFactors* f);
 
 // For a workspace that log_fwd_writes_factors() accepts: the sampling sweep on the
-// matrix cores.  Leaves in idx the code -2 - group (groups of 16 terms; 0: the prefix
-// sums never reach the target) and in the scratch array rem at the start of that
+// matrix cores.  Leaves in idx the code -2 - group (groups of 16 terms; K - 1, final: the
+// prefix sums never reach the target) and in the scratch array rem at the start of that
 // group; tiles that the forward or the sweep flagged are redone exactly (out and the
 // final index).  The caller resolves the codes.
-bool log_sample_mfma_ok(int K);  // the sweep below takes reductions up to 62 slabs of 16 terms
+bool log_sample_mfma_ok(int K);  // the sweep below takes reductions up to 126 slabs of 16 terms
 int log_sample_sweep_mfma(const elem_t* a, const elem_t* b, elem_t* out, int32_t* idx,
                           const float* stats, uint64_t seed, uint64_t offset, int B, int M, int K,
                           int N, hipStream_t s);

@@ -561,7 +561,7 @@ int genbmm_banded_bwdbwd_f64(const double* a, int a_lu, int a_ld,
  * namesake returns on the widened tensors, rounded once (indices: identical).
  * The backward functions that read `out` read the rounded one, as the
  * reference's do.  samplebmm sweeps only where the forward left 1/S in the
- * workspace (matrix-core shapes, K <= 992) and walks the terms exactly
+ * workspace (matrix-core shapes, K <= 2016) and walks the terms exactly
  * otherwise (`out` rounded to 11 or 8 bits does not give S well enough for the
  * other sweeps): its index is the float function's on those shapes and the
  * index of the float function called with stats = NULL on all others.

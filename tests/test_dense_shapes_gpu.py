@@ -66,13 +66,14 @@ def test_argmax_backward_with_many_k_ranges(gpu):
 
 def test_sample_on_many_shapes(gpu):
     """Every index brackets its uniform in the float64 CDF; shapes on both sides of the
-    matrix-core limits (M, N >= 96, K >= 16) and of its 62-slab limit (K <= 992; the last
-    two shapes have a matrix-core forward and, with K = 1040 and 1008, the two-level sweep
-    on the vector ALU behind it)."""
+    matrix-core limits (M, N >= 96, K >= 16), of the 62 slabs that its six-bit tag counts
+    (K <= 992; K = 993, 1008, 1040: seven bits) and of its 126-slab limit (K <= 2016; the last
+    shape has a matrix-core forward and, with K = 2020, the two-level sweep on the vector ALU
+    behind it)."""
     lib = _lib.load()
     torch.manual_seed(7)
     shapes = _shapes(13, 14, 400) + [(1, 96, 16, 96), (1, 97, 993, 100), (1, 130, 992, 96), (2, 100, 500, 131),
-                                     (1, 128, 1040, 160), (2, 256, 1008, 128)]
+                                     (1, 128, 1040, 160), (2, 256, 1008, 128), (1, 128, 2016, 96), (1, 96, 2020, 128)]
     for B, M, K, N in shapes:
         a, b = 2 * torch.randn(B, M, K), 2 * torch.randn(B, K, N)
         ad, bd = a.to(gpu), b.to(gpu)
