@@ -24,7 +24,7 @@ BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
 # HBM bytes per launch of the dominant kernel (k_log_bwd_split_both): rocprofv3 --pmc
 # FETCH_SIZE + WRITE_SIZE in KiB per dispatch, scale factor 1.00 against a known-size copy in
 # the same run; the two figures are those of profiles/logbmm_headline_B64_512.md.
-DOMINANT_FETCH_KIB, DOMINANT_WRITE_KIB = 242745, 131072
+DOMINANT_FETCH_KIB, DOMINANT_WRITE_KIB = 242399, 131072
 DOMINANT_TRAFFIC_BYTES = (DOMINANT_FETCH_KIB + DOMINANT_WRITE_KIB) * 1024
 
 
