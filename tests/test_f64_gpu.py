@@ -144,6 +144,41 @@ def test_max_f64_bit_exact(gpu, B, M, K, N, prod):
     assert torch.equal(i2.cpu(), si) and torch.equal(o2.cpu(), sv)
 
 
+@pytest.mark.parametrize("B,M,K,N", [(2, 70, 261, 65), (1, 40, 600, 130), (3, 33, 7, 20), (2, 64, 512, 128)])
+@pytest.mark.parametrize("prod", [False, True])
+def test_max_f64_index_groups_and_special_values(gpu, prod, B, M, K, N):
+    """The double-precision forward keeps the group of four consecutive k that last raised a
+    cell's maximum and forms that group's terms again at the end: K across many slabs and not a
+    multiple of the group, many ties, NaN / infinite / signed-zero terms, everything below the
+    -1e9 floor.  Values are compared as bit patterns."""
+    torch.manual_seed(K + N)
+    a, b = grid(B, M, K) / 2, grid(B, K, N) / 2
+    if prod:
+        a, b = a.abs(), b.abs()       # zeros stay: products tie at 0 and signs of zero matter
+        b[:, 1::5, :] *= -1
+    a[:, ::7, 3::11] = float("nan")
+    a[:, 1::9, 2::13] = float("inf")
+    b[:, 4::17, ::6] = float("-inf")
+    b[:, 5::19, 1::4] = -0.0
+    a[:, 2::5, 5::19] = -0.0
+    a[0, 0, :] = -0.0                 # a whole row of zero terms of both signs
+    b[0, :, 0] = torch.where(torch.arange(K) % 3 == 0, 0.0, -0.0).double()
+    if not prod:
+        a[-1, 3, :] = -3e9            # every term of the row below the floor: value -1e9, index -1
+    lib = _lib.load()
+    ad, bd = a.to(gpu), b.to(gpu)
+    out = torch.empty(B, M, N, dtype=torch.float64, device=gpu)
+    idx = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
+    fn = lib.genbmm_prodmaxbmm_fwd_f64 if prod else lib.genbmm_maxbmm_fwd_f64
+    assert fn(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx), B, M, K, N, _lib.stream_of(out)) == 0
+    sv, si = oracle.seq_maxbmm_fwd(a, b, prod, dtype=F64)
+    assert torch.equal(idx.cpu(), si)
+    assert torch.equal(out.cpu().view(torch.int64), sv.view(torch.int64))
+    assert int((si >= 0).sum()) > 0
+    if not prod:
+        assert bool((si[-1, 3] == -1).all()) and bool((sv[-1, 3] == -1e9).all())
+
+
 def test_max_f64_at_the_benchmark_size(gpu):
     """(512,128,128,128) on the 1/8 grid (max) and Uniform(0,1] (prod-max), EVERY batch item: values
     and indices bit-exact against the broadcast closed form evaluated on the device in float64
