@@ -23,7 +23,7 @@
 // so that the counted waits for loads stay exact; a branch around a load costs every wait
 // behind it its count.
 //
-// What bounds it (64 x 4096, 65 diagonals per operand: 81 us, of which the matrix instructions
+// What bounds it (64 x 4096, 65 diagonals per operand: 73-78 us, of which the matrix instructions
 // fill a tenth): instruction issue.  A step is about 900 staging instructions (cutting 6 144
 // floats into parts), 220 matrix and LDS instructions and 500 for writing results, on four
 // SIMDs that issue one vector instruction in about 4.4 cycles each; the staged blocks take 144
