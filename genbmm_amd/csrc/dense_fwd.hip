@@ -632,6 +632,178 @@ int launch_max(DenseArgs p, float* factors, int B, int M, int K, int N, hipStrea
   return launch_status();
 }
 
+#if GENBMM_ELEM == 0
+// ------------------------------------------- max / prod-max: a long reduction in pieces
+// Few result tiles and a long K would run on a few compute units, every tile being one
+// workgroup's that walks all of K.  Such a problem is cut into pieces of K, a workgroup per
+// 64 x 64 tile and piece, in two passes over a and b that need nothing beside out and idx:
+//   pass 0  the maximum of a piece's terms joins out by an integer atomic on the value's bit pattern
+//           (max of the pattern for values >= 0, min for negative ones: the order of floats);
+//   pass 1  the lowest k of a piece whose term equals that maximum joins idx by an atomic minimum;
+// then every cell forms the term of its index again (the value of the first term that attains
+// the maximum, as the reference's walk keeps it - +0 and -0 compare equal, so the atomics
+// cannot tell them apart) and, for the product semiring, stores its two factors.  Maximum and
+// minimum commute: the result does not depend on the order in which the pieces arrive, and it is the
+// sequential walk's (matmul_cuda_kernel.cu:47-75, :124-152) bit for bit.  A NaN term never wins
+// (it is no maximum and equals nothing); k beyond a piece are staged as NaN.
+constexpr int kCutTile = 64, kCutSlab = 16, kCutLda = 68;
+
+// pieces of K for (B, M, K, N): 1 = no cut.  About two rounds of workgroups over the chip, pieces of
+// at least 256 terms and a multiple of the slab.
+inline int max_cut_pieces(int B, int M, int K, int N, int& per) {
+  const int64_t tiles = (int64_t)B * ceil_div(M, kCutTile) * ceil_div(N, kCutTile);
+  per = K;
+  if (tiles <= 0 || tiles >= 128 || K < 2048) return 1;
+  const int want = (int)std::min<int64_t>((511 + tiles) / tiles, K / 256);
+  if (want < 2) return 1;
+  per = ceil_div(ceil_div(K, want), kCutSlab) * kCutSlab;
+  return ceil_div(K, per);
+}
+
+__global__ __launch_bounds__(256) void k_max_cut_init(float* __restrict__ out, int32_t* __restrict__ idx, long cells) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e < cells) {
+    out[e] = kFloor;
+    idx[e] = -1;
+  }
+}
+
+// PASS 0 / 1 as above; one workgroup per tile and piece, a lane keeps 4 x 4 cells.
+template <bool PROD, int PASS>
+__global__ __launch_bounds__(256) void k_max_cut(const float* __restrict__ a, const float* __restrict__ b,
+                                                float* __restrict__ out, int32_t* __restrict__ idx, int M, int K,
+                                                int N, int tiles_m, int tiles_n, int pieces, int per) {
+  __shared__ __attribute__((aligned(16))) float As[kCutSlab * kCutLda];   // [k][m]
+  __shared__ __attribute__((aligned(16))) float Bs[kCutSlab * kCutTile];  // [k][n]
+  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  const int wg = xcd_renumber(blockIdx.x, gridDim.x);
+  const int piece = wg % pieces, tile = wg / pieces;  // the pieces of a tile side by side: they share its cells
+  const int per_item = tiles_m * tiles_n, batch = tile / per_item, rem = tile - batch * per_item;
+  const int m0 = (rem / tiles_n) * kCutTile, n0 = (rem % tiles_n) * kCutTile;
+  const int k_lo = piece * per, k_hi = min(K, k_lo + per);
+  const float* ab = a + (long)batch * M * K;
+  const float* bb = b + (long)batch * K * N;
+  float* ob = out + (long)batch * M * N;
+  int32_t* ib = idx + (long)batch * M * N;
+  const int nslabs = (k_hi - k_lo + kCutSlab - 1) / kCutSlab;
+  if (nslabs <= 0) return;
+
+  const int ak = tid & 15, ar = tid >> 4, bn = tid & 63, bk = tid >> 6;
+  float ra[4], rb[4];
+  auto gload = [&](int k0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + ar + 16 * i, k = k0 + ak;
+      ra[i] = k < k_hi ? (m < M ? ab[(long)m * K + k] : 0.f) : __builtin_nanf("");
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = k0 + bk + 4 * i, n = n0 + bn;
+      rb[i] = (k < k_hi && n < N) ? bb[(long)k * N + n] : 0.f;
+    }
+  };
+  auto sstore = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) As[ak * kCutLda + ar + 16 * i] = ra[i];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) Bs[(bk + 4 * i) * kCutTile + bn] = rb[i];
+  };
+  // the cells' state: the running maximum (pass 0) or the maximum to look for and the lowest k found
+  float val[4][4];
+  int cand[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int m = m0 + ty * 4 + i, n = n0 + tx * 4 + j;
+      val[i][j] = PASS == 0 ? kFloor : ((m < M && n < N) ? ob[(long)m * N + n] : kFloor);
+      cand[i][j] = 0x7fffffff;
+    }
+  // pass 1 walks its piece from the end, so that of the terms that match the lowest k is the one that stays
+  auto slab_k0 = [&](int s) { return k_lo + (PASS == 0 ? s : nslabs - 1 - s) * kCutSlab; };
+  gload(slab_k0(0));
+  for (int s = 0; s < nslabs; ++s) {
+    __syncthreads();
+    sstore();
+    __syncthreads();
+    if (s + 1 < nslabs) gload(slab_k0(s + 1));
+    const int k0 = slab_k0(s);
+#pragma unroll
+    for (int q = 0; q < kCutSlab; ++q) {
+      const int kk = PASS == 0 ? q : kCutSlab - 1 - q;
+      const float4 av = *reinterpret_cast<const float4*>(As + kk * kCutLda + ty * 4);
+      const float4 bv = *reinterpret_cast<const float4*>(Bs + kk * kCutTile + tx * 4);
+      const float a4[4] = {av.x, av.y, av.z, av.w}, b4[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float t = PROD ? __fmul_rn(a4[i], b4[j]) : __fadd_rn(a4[i], b4[j]);
+          if (PASS == 0) val[i][j] = __builtin_fmaxf(val[i][j], t);
+          else cand[i][j] = t == val[i][j] ? k0 + kk : cand[i][j];
+        }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int m = m0 + ty * 4 + i, n = n0 + tx * 4 + j;
+      if (m >= M || n >= N) continue;
+      const long e = (long)m * N + n;
+      if (PASS == 0) {
+        const float v = val[i][j] + 0.f;  // -0 joins as +0 (the value itself is formed again at the end)
+        if (v > kFloor) {
+          if (v >= 0.f) atomicMax(reinterpret_cast<int*>(ob + e), __float_as_int(v));
+          else atomicMin(reinterpret_cast<unsigned*>(ob + e), __float_as_uint(v));
+        }
+      } else if (val[i][j] > kFloor && cand[i][j] != 0x7fffffff) {
+        atomicMin(reinterpret_cast<unsigned*>(ib + e), (unsigned)cand[i][j]);  // -1, "none", is the largest
+      }
+    }
+}
+
+// the term of every cell's index again: the value, and the factors of the product semiring
+template <bool PROD>
+__global__ __launch_bounds__(256) void k_max_cut_finish(const float* __restrict__ a, const float* __restrict__ b,
+                                                       float* __restrict__ out, const int32_t* __restrict__ idx,
+                                                       float* __restrict__ fa, float* __restrict__ fb, int M, int K,
+                                                       int N, long cells) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= cells) return;
+  const int n = (int)(e % N);
+  const long bm = e / N, batch = bm / M;
+  const int k = idx[e];
+  float av = 0.f, bv = 0.f;
+  if (k >= 0) {
+    av = a[bm * K + k];
+    bv = b[(batch * K + k) * N + n];
+    out[e] = PROD ? __fmul_rn(av, bv) : __fadd_rn(av, bv);
+  }
+  if (fa) {
+    fa[e] = av;
+    fb[e] = bv;
+  }
+}
+
+template <bool PROD>
+int launch_max_cut(const float* a, const float* b, float* out, int32_t* idx, float* factors, int B, int M, int K,
+                   int N, int pieces, int per, hipStream_t s) {
+  const long cells = (long)B * M * N;
+  const int tiles_m = ceil_div(M, kCutTile), tiles_n = ceil_div(N, kCutTile);
+  const unsigned grid = (unsigned)(B * tiles_m * tiles_n * pieces);  // below 128 tiles, at most 512 pieces
+  const unsigned cgrid = (unsigned)((cells + 255) / 256);
+  hipLaunchKernelGGL(k_max_cut_init, dim3(cgrid), dim3(256), 0, s, out, idx, cells);
+  hipLaunchKernelGGL((k_max_cut<PROD, 0>), dim3(grid), dim3(256), 0, s, a, b, out, idx, M, K, N, tiles_m, tiles_n,
+                     pieces, per);
+  hipLaunchKernelGGL((k_max_cut<PROD, 1>), dim3(grid), dim3(256), 0, s, a, b, out, idx, M, K, N, tiles_m, tiles_n,
+                     pieces, per);
+  hipLaunchKernelGGL((k_max_cut_finish<PROD>), dim3(cgrid), dim3(256), 0, s, a, b, out, idx, factors,
+                     factors ? factors + cells : nullptr, M, K, N, cells);
+  return launch_status();
+}
+#endif
+
 template <class C>
 int launch_sample(DenseArgs p, int B, int M, int K, int N, hipStream_t s) {
   dim3 grid;
@@ -651,6 +823,13 @@ int run_max(const elem_t* a, const elem_t* b, elem_t* out, int32_t* idx, float* 
   DenseArgs p{};
   p.a = a; p.b = b; p.out = out; p.idx = idx;
   hipStream_t s = (hipStream_t)stream;
+#if GENBMM_ELEM == 0
+  {
+    int per;
+    const int pieces = max_cut_pieces(B, M, K, N, per);
+    if (pieces > 1) return launch_max_cut<PROD>(a, b, out, idx, factors, B, M, K, N, pieces, per, s);
+  }
+#endif
   switch (pick_shape(B, M, N, false)) {
     case kBig: return launch_max<CfgBig, PROD>(p, factors, B, M, K, N, s);
     case kWide: return launch_max<CfgWide, PROD>(p, factors, B, M, K, N, s);
@@ -750,6 +929,15 @@ int run_sample(const elem_t* a, const elem_t* b, elem_t* out, int32_t* idx, floa
 }  // namespace GENBMM_NS
 
 extern "C" {
+
+#if GENBMM_ELEM == 0
+int genbmm_maxbmm_fwd_pieces(int B, int M, int K, int N) {
+  using namespace GENBMM_NS;
+  if (check_dense_dims(B, M, K, N) || (int64_t)B * M * N == 0) return 1;
+  int per;
+  return max_cut_pieces(B, M, K, N, per);
+}
+#endif
 
 // One set per element type: genbmm_samplebmm_fwd, genbmm_samplebmm_fwd_f16, ..._bf16, ...
 int GENBMM_API(samplebmm_fwd)(const GENBMM_NS::abi_t* a, const GENBMM_NS::abi_t* b, GENBMM_NS::abi_t* out,

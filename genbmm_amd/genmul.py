@@ -223,6 +223,8 @@ def _max_forward(a, b, prod, factors=None):
     B, M, K = a.shape
     N = b.shape[2]
     S = 1 if _f64(a) else _reduction_splits(B, M, K, N)
+    if S > 1 and a.dtype == torch.float32 and _lib.load().genbmm_maxbmm_fwd_pieces(B, M, K, N) > 1:
+        S = 1       # the library cuts the reduction axis of this problem itself
     name = "genbmm_prodmaxbmm_fwd" if prod else "genbmm_maxbmm_fwd"
     if S == 1:
         out = torch.empty(B, M, N, dtype=a.dtype, device=a.device)

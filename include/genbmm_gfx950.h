@@ -252,6 +252,18 @@ int genbmm_maxbmm_fwd(const float* a, const float* b, float* out, int32_t* idx,
                       int B, int M, int K, int N, void* stream);
 
 /*
+ * Into how many pieces genbmm_maxbmm_fwd and genbmm_prodmaxbmm_fwd (float
+ * operands) cut the reduction axis of this problem: 1 (they do not) unless the
+ * result has fewer than 128 tiles of 64 x 64 and K is at least 2048.  The
+ * pieces' maxima meet in `out` and the lowest k that attains them in `idx` by
+ * integer atomics, which commute: values and indices are those of the uncut
+ * walk, bit for bit, whatever order the pieces arrive in.  No counterpart in
+ * the reference, whose kernel gives every output cell one thread that walks
+ * all of K (matmul_cuda_kernel.cu:47-75, :124-152).
+ */
+int genbmm_maxbmm_fwd_pieces(int B, int M, int K, int N);
+
+/*
  * out[b,m,n] = max_k (a[m,k] * b[k,n]); idx as above.
  * factors (optional, may be NULL): 2*B*M*N floats of workspace for
  * genbmm_prodmax_bwd; receives a[m, idx[m,n]] for every cell, then

@@ -1098,6 +1098,62 @@ def test_long_reductions_with_few_tiles_are_split(gpu, B, M, K, N):
         close(db, w2[1], rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("B,M,K,N", [(16, 96, 4096, 96), (1, 16, 65536, 16), (60, 7, 4100, 7), (3, 130, 2101, 97),
+                                     (2, 300, 5000, 200), (1, 64, 2048, 64)])
+@pytest.mark.parametrize("prod", [False, True])
+def test_library_cuts_long_max_reductions_into_pieces(gpu, prod, B, M, K, N):
+    """genbmm_maxbmm_fwd / genbmm_prodmaxbmm_fwd cut the reduction axis of a problem with few
+    output tiles into pieces whose maxima and lowest indices meet by integer atomics: values (as
+    bit patterns), indices and the product semiring's factors equal to the sequential oracle's,
+    with ties inside and across pieces, NaN / infinite / signed-zero terms, a row below the -1e9
+    floor and a row of NaN; twice in a row into the same buffers; through autograd as well."""
+    lib = _lib.load()
+    assert lib.genbmm_maxbmm_fwd_pieces(B, M, K, N) > 1
+    assert lib.genbmm_maxbmm_fwd_pieces(256, 256, 256, 256) == 1 and lib.genbmm_maxbmm_fwd_pieces(1, 16, 2000, 16) == 1
+    assert lib.genbmm_maxbmm_fwd_pieces(4, 512, 8192, 512) == 1
+    torch.manual_seed(K + N)
+    a, b = grid(B, M, K) / 2, grid(B, K, N) / 2
+    if prod:
+        a, b = a.abs(), b.abs()       # zeros stay: products tie at 0 and signs of zero matter
+        b[:, 1::5, :] *= -1
+    a[:, ::7, 3::11] = float("nan")
+    a[:, 1::9, 2::13] = float("inf")
+    b[:, 4::17, ::6] = float("-inf")
+    b[:, 5::19, 1::4] = -0.0
+    a[:, 2::5, 5::19] = -0.0
+    a[0, 0, :] = -0.0                 # a whole row of zero terms of both signs
+    b[0, :, 0] = torch.where(torch.arange(K) % 3 == 0, 0.0, -0.0)
+    a[-1, M - 1, :] = float("nan")    # no term at all: value -1e9, index -1
+    if not prod:
+        a[-1, 1 % M, :] = -3e9        # every term below the floor
+    ad, bd = a.to(gpu), b.to(gpu)
+    sv, si = oracle.seq_maxbmm_fwd(a, b, prod)
+    fac = torch.full((2, B, M, N), float("nan"), device=gpu) if prod else None
+    for _ in range(2):
+        out, idx = _abi_max(gpu, ad, bd, prod, fac)
+        assert torch.equal(idx.cpu(), si)
+        assert torch.equal(out.cpu().view(torch.int32), sv.view(torch.int32))
+    assert bool((si[-1, M - 1] == -1).all()) and int((si >= 0).sum()) > 0
+    if prod:
+        k = si.long().clamp(min=0)
+        fa = torch.gather(a, 2, k)                                      # a[m, idx]
+        fb = torch.gather(b, 1, k)                                      # b[idx, n]
+        live = si >= 0
+        assert torch.equal(fac[0].cpu()[live], fa[live]) and torch.equal(fac[1].cpu()[live], fb[live])
+        assert bool((fac[0].cpu()[~live] == 0).all()) and bool((fac[1].cpu()[~live] == 0).all())
+    # the public function leaves the cut to the library and its gradient is the one-hot scatter
+    op = genbmm.prodmaxbmm if prod else genbmm.maxbmm
+    a2, b2 = a.nan_to_num(nan=-1.0, posinf=3.0, neginf=-3.0), b.nan_to_num(nan=-1.0, posinf=3.0, neginf=-3.0)
+    ar, br = a2.to(gpu).requires_grad_(True), b2.to(gpu).requires_grad_(True)
+    o = op(ar, br)
+    sv2, si2 = oracle.seq_maxbmm_fwd(a2, b2, prod)
+    assert torch.equal(o.detach().cpu().view(torch.int32), sv2.view(torch.int32))
+    g = grid(B, M, N).clamp(-4, 4)
+    ga, gb = torch.autograd.grad(o, (ar, br), g.to(gpu))
+    wa, wb = oracle.seq_argmax_bwd(a2 if prod else K, b2, si2, g, prod)
+    assert torch.equal(ga.cpu(), wa) and torch.equal(gb.cpu(), wb)
+
+
 @pytest.mark.parametrize("B,M,K,N", [(16, 96, 4096, 96), (1, 16, 65536, 16), (64, 7, 4100, 7), (3, 130, 2101, 97),
                                      (2, 300, 5000, 200), (1, 128, 2048, 128), (100, 120, 2300, 127)])
 def test_library_cuts_long_reductions_into_pieces(gpu, B, M, K, N):
