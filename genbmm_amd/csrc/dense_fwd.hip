@@ -899,6 +899,9 @@ int run_sample(const elem_t* a, const elem_t* b, elem_t* out, int32_t* idx, floa
   // half type that is S within 2^-9 |out| at best, and targets u S past the true sum would be
   // common.  Half tensors therefore sweep only where 1/S itself is at hand in fp32 (the
   // matrix-core sweep) and walk exactly otherwise.
+  // few result tiles and a long reduction: the forward cuts K into pieces, and so does the draw
+  if (K > 0 && log_sample_cut_ok(stats, B, M, K, N))
+    return log_sample_cut(a, b, out, idx, stats, seed, offset, B, M, K, N, s);
   const bool sweep = kElemF32 || (stats && log_fwd_writes_factors(stats, B, M, K, N, &f) && log_sample_mfma_ok(K));
   if (stats && K > 0 && sweep) {  // log-sum-exp by the logbmm forward, then the multiply-only sweep
     if (int e = log_fwd_with_factors(a, b, out, stats, B, M, K, N, s)) return e;

@@ -1204,6 +1204,119 @@ int log_sample_sweep_mfma(const elem_t* a, const elem_t* b, elem_t* out, int32_t
   }
 }
 
+// ------------------------------------------------- sampling on a forward in pieces
+// One lane per cell, lanes along n.  The cell's target t = u S (u its Philox uniform, S the sum of
+// the pieces' sums in the order the join adds them, shrunk by 2^-22 so that it lies inside the
+// total) falls into the piece in which the prefix of the pieces' sums passes it; the cell then
+// walks that piece's terms exp(a - alpha) exp(b - beta) - the factors whose products the piece's
+// sum is - until their prefix passes what was left of t.  The walk's own sum may differ from the
+// piece's in the last bits: a target it never reaches names the piece's last term with mass.
+// A cell of a tile that the forward flagged (its factored sums are not usable) walks the
+// reference's own way: maximum, sum of exponentials, then the decision of
+// matmul_cuda_kernel.cu:109-118 on p = exp(a + b - logsumexp), naming the last term that had mass
+// when the walk runs out.
+__global__ __launch_bounds__(256) void k_sample_cut(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
+                                                   const float* __restrict__ stats, const int* __restrict__ flags,
+                                                   const float* __restrict__ parts, int32_t* __restrict__ idx,
+                                                   uint64_t seed, uint64_t offset, int B, int M, int K, int N,
+                                                   int pieces, int slabs_piece, int tiles_m, int tiles_n, long cells) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= cells) return;
+  const int n = (int)(e % N);
+  const long bm = e / N;
+  const int batch = (int)(bm / M), m = (int)(bm - (long)batch * M);
+  const elem_t* arow = a + bm * K;
+  const elem_t* bcol = b + (long)batch * K * N + n;
+  const float u = philox_uniform((uint64_t)e, seed, offset);
+  int ind = 0;
+  if (flags[((long)batch * tiles_m + m / 128) * tiles_n + n / 128]) {
+    float mx = kFloor;
+    for (int k = 0; k < K; ++k) mx = __builtin_fmaxf(mx, (float)arow[k] + (float)bcol[(long)k * N]);
+    float tot = 0.f;
+    for (int k = 0; k < K; ++k) tot += __expf((float)arow[k] + (float)bcol[(long)k * N] - mx);
+    const float o = __logf(tot) + mx;
+    float acc = 0.f;
+    int last = 0;
+    bool found = false;
+    for (int k = 0; k < K && !found; ++k) {
+      const float p = __expf((float)arow[k] + (float)bcol[(long)k * N] - o);
+      if (acc <= u && acc + p > u) {  // (<=: a prefix that lands on u exactly must not lose the draw)
+        ind = k;
+        found = true;
+      }
+      if (p > 0.f) last = k;
+      acc += p;
+    }
+    if (!found) ind = (acc > 0.f && u >= acc) ? last : 0;  // ran out just below u: the last term with mass
+    idx[e] = ind;
+    return;
+  }
+  const float* sp = parts + bm * N + n;  // piece p: sp[p * cells]
+  float total = sp[0];
+  for (int p = 1; p < pieces; ++p) total += sp[(long)p * cells];
+  const float t = u * kSampleShrink * total;
+  float before = 0.f;
+  int piece = 0;
+  for (; piece < pieces - 1; ++piece) {
+    const float next = before + sp[(long)piece * cells];
+    if (next > t) break;
+    before = next;
+  }
+  const int k0 = piece * slabs_piece * kMS, k1 = min(K, k0 + slabs_piece * kMS);
+  const float al = stats[(long)batch * (M + N) + m], be = stats[(long)batch * (M + N) + M + n];
+  float rem = t - before;
+  int last = k0;
+  ind = -1;
+  // sixteen terms at a time (their loads in flight together): a group whose sum leaves rem
+  // non-negative is passed whole, the group in which rem turns negative is walked term by term
+  for (int kc = k0; kc < k1 && ind < 0; kc += 16) {
+    float tv[16];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const int k = min(kc + q, k1 - 1);
+      tv[q] = fast_exp((float)arow[k] - al) * fast_exp((float)bcol[(long)k * N] - be);
+      if (kc + q >= k1) tv[q] = 0.f;
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) sum += tv[q];
+    const bool whole = rem - sum >= 0.f;
+    float r = rem;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      if (tv[q] > 0.f) last = kc + q;
+      r -= tv[q];
+      if (!whole && ind < 0 && r < 0.f) ind = kc + q;
+    }
+    rem = whole ? rem - sum : r;
+    if (!whole && ind < 0) ind = last;  // the group's sum passed rem, its terms one by one did not: rounding
+  }
+  idx[e] = ind >= 0 ? ind : last;
+}
+
+bool log_sample_cut_ok(const float* stats, int B, int M, int K, int N) {
+  return stats != nullptr && (int64_t)B * M * N > 0 && !item_shape(M, K, N) && !self_shape(M, K, N) &&
+         fwd_pieces(B, M, K, N) > 1;
+}
+int64_t log_sample_cut_floats(int B, int M, int K, int N) {
+  if ((int64_t)B * M * N == 0 || item_shape(M, K, N) || self_shape(M, K, N)) return 0;
+  const int pieces = fwd_pieces(B, M, K, N);
+  return pieces > 1 ? (int64_t)pieces * B * M * N : 0;
+}
+int log_sample_cut(const elem_t* a, const elem_t* b, elem_t* out, int32_t* idx, float* stats, uint64_t seed,
+                   uint64_t offset, int B, int M, int K, int N, hipStream_t s) {
+  // the forward in pieces: out, the maxima, the flags and every piece's sums
+  if (int e = run_fwd(a, b, out, stats, B, M, K, N, GENBMM_PATH_AUTO, false, s, false, true)) return e;
+  const int pieces = fwd_pieces(B, M, K, N);
+  const int slabs_piece = ceil_div(ceil_div(K, kMS), pieces);
+  const long cells = (long)B * M * N;
+  if ((cells + 255) / 256 > 0x7fffffffL) return GENBMM_E_SHAPE;
+  hipLaunchKernelGGL(k_sample_cut, dim3((unsigned)((cells + 255) / 256)), dim3(256), 0, s, a, b, stats,
+                     fwd_flags_of(stats, B, M, N), prepared_of(stats, B, M, K, N).ea, idx, seed, offset, B, M, K, N,
+                     pieces, slabs_piece, ceil_div(M, 128), ceil_div(N, 128), cells);
+  return launch_status();
+}
+
 }  // namespace GENBMM_NS
 
 extern "C" {
@@ -1238,8 +1351,11 @@ size_t genbmm_samplebmm_stats_size(int B, int M, int K, int N) {
   using namespace GENBMM_NS;
   if (check_dense_dims(B, M, K, N)) return 0;
   int64_t n = header_offset(B, M, N) + 4;
-  if (fwd_mfma_shape(B, M, K, N)) n += (int64_t)B * ((int64_t)M * K + (int64_t)K * N + (int64_t)M * N);
-  return (size_t)n;
+  // the factors of the matrix-core forward, or the sums of a forward in pieces
+  int64_t room = 0;
+  if (fwd_mfma_shape(B, M, K, N)) room = (int64_t)B * ((int64_t)M * K + (int64_t)K * N + (int64_t)M * N);
+  room = std::max(room, log_sample_cut_floats(B, M, K, N));
+  return (size_t)(n + room);
 }
 
 size_t genbmm_logbmm_static_limit(void) { return GENBMM_NS::kStaticFloats; }

@@ -38,4 +38,13 @@ int log_sample_sweep_mfma(const elem_t* a, const elem_t* b, elem_t* out, int32_t
                           const float* stats, uint64_t seed, uint64_t offset, int B, int M, int K,
                           int N, hipStream_t s);
 
+// samplebmm on a problem whose forward cuts its reduction into pieces (few result tiles, a long
+// K): log_sample_cut_ok() tells whether this is one; log_sample_cut() runs that forward - out, the
+// maxima and every piece's sum stay in the workspace - and draws every cell's index from the sums:
+// the piece in which the prefix passes the cell's target, then the terms of that one piece.
+bool log_sample_cut_ok(const float* stats, int B, int M, int K, int N);
+int64_t log_sample_cut_floats(int B, int M, int K, int N);  // workspace floats behind the header (0: no cut)
+int log_sample_cut(const elem_t* a, const elem_t* b, elem_t* out, int32_t* idx, float* stats, uint64_t seed,
+                   uint64_t offset, int B, int M, int K, int N, hipStream_t s);
+
 }  // namespace GENBMM_NS

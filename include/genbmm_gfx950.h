@@ -114,7 +114,10 @@ size_t genbmm_logbmm_stats_size(int B, int M, int K, int N);
 /*
  * Number of fp32 elements genbmm_samplebmm_fwd needs in its `stats` (never less
  * than genbmm_logbmm_stats_size: the sampling sweep always wants the factors
- * where a forward can leave them).  No counterpart in the reference.
+ * where a forward can leave them, and on a problem whose forward cuts its
+ * reduction into pieces - genbmm_logbmm_fwd_pieces > 1 - the draw reads the
+ * pieces' sums: it picks the piece in which their prefix passes the cell's
+ * target, then walks that piece's terms).  No counterpart in the reference.
  */
 size_t genbmm_samplebmm_stats_size(int B, int M, int K, int N);
 

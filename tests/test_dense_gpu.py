@@ -840,6 +840,56 @@ def test_sample_index_brackets_cdf(gpu, use_stats, B, M, K, N):
     assert not torch.equal(idx, idx2)
 
 
+@pytest.mark.parametrize("B,M,K,N", [(2, 40, 4096, 30), (1, 16, 6000, 16), (2, 100, 2101, 97), (1, 7, 8192, 5)])
+def test_sample_on_long_reductions_with_few_tiles(gpu, B, M, K, N):
+    """samplebmm on a problem whose forward cuts the reduction axis into pieces: the draw picks the
+    piece in which the prefix of the pieces' sums passes the cell's target and walks that piece.
+    out against float64; every index brackets its Philox uniform in the float64 CDF (tolerance:
+    the rounding of an fp32 sum of K terms); batch item 0 holds rows that defeat the factoring
+    (flagged tiles walk the reference's own way); same stream, same draw; float16 operands too."""
+    lib = _lib.load()
+    assert lib.genbmm_logbmm_fwd_pieces(B, M, K, N) > 1
+    torch.manual_seed(K + N)
+    a, b = 2 * torch.randn(B, M, K), 2 * torch.randn(B, K, N)
+    a[0, ::2, 0] += 150.0
+    b[0, 0, :] -= 150.0
+    seed, offset = 4321, 2
+    u = oracle.philox_uniform(0, B * M * N, seed, offset).view(B, M, N).double()
+    tol = max(2e-5, K * 2.0 ** -24)
+    for dt, suffix in ((torch.float32, ""), (torch.float16, "_f16")):
+        ad, bd = a.to(gpu).to(dt), b.to(gpu).to(dt)
+        a32, b32 = ad.float().cpu(), bd.float().cpu()
+        out = torch.empty(B, M, N, device=gpu, dtype=dt)
+        idx = torch.empty(B, M, N, dtype=torch.int32, device=gpu)
+        stats = torch.empty(lib.genbmm_samplebmm_stats_size(B, M, K, N), device=gpu)
+        fn = getattr(lib, "genbmm_samplebmm_fwd" + suffix)
+        assert fn(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx), _lib.ptr(stats), seed, offset, B, M, K, N,
+                  _lib.stream_of(ad)) == 0
+        want = lse64(a32, b32)
+        if dt == torch.float32:
+            close(out, want)
+        else:
+            assert bool(((out.double().cpu() - want).abs() <= 2.0 ** -11 * want.abs() + 1e-5 * want.abs() + 1e-6).all())
+        cdf = oracle.sample_cdf64(a32, b32)                               # (B,M,K,N)
+        got = idx.cpu().long()
+        assert int(got.min()) >= 0 and int(got.max()) < K
+        hi = torch.gather(cdf, 2, got.unsqueeze(2)).squeeze(2)
+        lo = torch.where(got > 0, torch.gather(cdf, 2, (got - 1).clamp(min=0).unsqueeze(2)).squeeze(2),
+                         torch.zeros_like(hi))
+        ok = (lo - tol <= u) & (u <= hi + tol)
+        assert bool(ok.all()), (str(dt), float((~ok).float().mean()))
+        assert float((got != oracle.sample_index_from_cdf(cdf, u).long()).float().mean()) < 5e-3
+        idx2 = torch.empty_like(idx)
+        fn(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(out), _lib.ptr(idx2), _lib.ptr(stats), seed, offset, B, M, K, N,
+           _lib.stream_of(ad))
+        assert torch.equal(idx, idx2)
+    # through the public function: the one-hot gradient of the drawn term
+    ar = a.to(gpu).requires_grad_(True)
+    o = genbmm.samplebmm(ar, b.to(gpu), (seed, offset))
+    (ga,) = torch.autograd.grad(o.sum(), ar)
+    assert float(ga.sum()) == pytest.approx(B * M * N, rel=1e-3)
+
+
 def test_sample_config_c4_chi_square(gpu):
     """Benchmark configuration 3: Normal(0,2) (64,512,512) potentials, Philox seed 1234; 10^4
     draws per cell of the (4,16,16) slice; per-cell chi-square against the float64
