@@ -77,7 +77,8 @@ for _suffix in ("_f16", "_bf16"):  # one more buffer than the float function: t_
     SIGNATURES["genbmm_banded_bwdbwd" + _suffix] = _BAND + [_c_float_p] * 8 + [_i, _i, _vp]
 HALF_SUFFIX = {torch.float16: "_f16", torch.bfloat16: "_bf16"}
 STRING_FUNCS = {"genbmm_version": [], "genbmm_error_string": [_i]}
-INT_FUNCS = {"genbmm_logbmm_fwd_pieces": [_i, _i, _i, _i], "genbmm_maxbmm_fwd_pieces": [_i, _i, _i, _i]}
+INT_FUNCS = {"genbmm_logbmm_fwd_pieces": [_i, _i, _i, _i], "genbmm_maxbmm_fwd_pieces": [_i, _i, _i, _i],
+             "genbmm_banded_on_matrix_cores": [_i, _i, _i, _i, _i, _i]}
 SIZE_FUNCS = {"genbmm_logbmm_stats_size": [_i, _i, _i, _i],
               "genbmm_logbmm_bwdbwd_ws_size": [_i, _i, _i, _i],
               "genbmm_logbmm_stats_size_path": [_i, _i, _i, _i, _i],

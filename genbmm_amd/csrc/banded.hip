@@ -216,6 +216,13 @@ size_t genbmm_banded_workspace_size(int a_lu, int a_ld, int b_lu, int b_ld, int 
   return band_ws_floats(p, B);
 }
 
+int genbmm_banded_on_matrix_cores(int a_lu, int a_ld, int b_lu, int b_ld, int B, int n) {
+  using namespace GENBMM_NS;
+  BandArgs p{};
+  if (fill_band(p, a_lu, a_ld, b_lu, b_ld, B, n)) return 0;
+  return workspace_used(p) ? 1 : 0;
+}
+
 size_t genbmm_banded_scratch_size(int a_lu, int a_ld, int b_lu, int b_ld, int B, int n) {
   using namespace GENBMM_NS;
   BandArgs p{};

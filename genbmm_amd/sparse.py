@@ -305,11 +305,51 @@ class BandedMatrix:
         return BandedMatrix(_band_transpose(self.data, self.lu, self.ld), self.ld, self.lu, self.fill)
 
     # ------------------------------------------------------------- products
+    def _dense_pays(self, other, log):
+        """Bands so wide that no banded kernel of the library takes them on the matrix cores (beyond
+        about 225 diagonals per operand they fall to one lane per result cell, 20 to 40 times slower)
+        while the matrices are small enough to multiply as dense ones: the product then goes through
+        `to_dense`, the dense product on the matrix cores and `banddiag`.  Measured, forward +
+        backward, 241 diagonals per operand: (+,x) 64 x 330: 0.49 ms against 7.2, 16 x 1024: 1.2 against
+        9.4, 4 x 2048: 1.7 against 5.1, 4 x 4096: 11.7 against 10.5 (no longer); the log product pays
+        while the result band covers a good part of the matrix - a 128 x 128 tile of the dense result
+        with a cell outside the band has a cell without terms, fails the factored kernels' guard and is
+        redone the exact way (64 x 330: 1.9 ms against 16.7; 16 x 512: 1.4 against 9.2; 16 x 1024: 10
+        against 20; 4 x 2048: 20 against 10, no longer)."""
+        a, b = self.data, other.data
+        if not (_native(a) and _native(b)) or a.shape[:2] != b.shape[:2]:
+            return False
+        batch, n, _ = a.shape
+        if min(self.width, other.width) <= 128 or batch * n * n > (1 << 28):
+            return False
+        if log:  # share of the dense result's cells that lie outside the result band
+            lu, ld = self.lu + other.ld, self.ld + other.lu
+            empty = (max(n - 1 - lu, 0) ** 2 + max(n - 1 - ld, 0) ** 2) / (2.0 * n * n)
+            if empty > 0.6:
+                return False
+        elif n > 2048:
+            return False
+        return _lib.load().genbmm_banded_on_matrix_cores(self.lu, self.ld, other.lu, other.ld, batch, n) == 0
+
+    def _product_dense(self, other, log):
+        """Dense(other)^T (x) Dense(self), re-banded (reference sparse.py:229-253 in dense algebra;
+        cells outside the bands are the semiring's zero, result cells outside the matrix 0)."""
+        from .genmul import logbmm
+
+        zero = -1e9 if log else 0.0       # the reference's own floor for a cell that is no term
+        x = BandedMatrix(self.data, self.lu, self.ld, zero).to_dense()
+        yt = BandedMatrix(other.data, other.lu, other.ld, zero).to_dense().transpose(1, 2).contiguous()
+        d = logbmm(yt, x) if log else torch.bmm(yt, x)
+        lu, ld = self.lu + other.ld, self.ld + other.lu
+        return BandedMatrix(banddiag(d, lu, ld)[0], lu, ld, self.fill)
+
     def _product(self, other, fn):
         batch, n, _ = self.data.shape
         assert other.data.shape[1] == n
         lu = self.lu + other.ld
         ld = self.ld + other.lu
+        if (fn is bandedbmm or fn is bandedlogbmm) and self._dense_pays(other, fn is bandedlogbmm):
+            return self._product_dense(other, fn is bandedlogbmm)
         # views are copied here, by a differentiable torch operation, so that the
         # Functions save (and differentiate with respect to) what they were given
         # (float16 / bfloat16 bands go to the `_f16` / `_bf16` entry points as they are)

@@ -381,6 +381,17 @@ size_t genbmm_banded_workspace_size(int a_lu, int a_ld, int b_lu, int b_ld,
                                     int B, int n);
 
 /*
+ * 1 if the (+,x) and log products of these bands, forward and backward, run on
+ * the kernels that feed the matrix cores (from 3 diagonals per operand up to
+ * about 225); 0 if they fall to one lane per result cell, which is 20 to 40
+ * times slower per cell - a caller whose matrices are small may then prefer
+ * dense algebra (the host layer does: to_dense, the dense product, banddiag).
+ * No counterpart in the reference, which has the one kernel for every width.
+ */
+int genbmm_banded_on_matrix_cores(int a_lu, int a_ld, int b_lu, int b_ld,
+                                  int B, int n);
+
+/*
  * Gradients of genbmm_banded_fwd with respect to BOTH operands, reading g,
  * out and idx in the frame the forward wrote them (no banded transposes).
  * `out` is read in mode LOG only, `idx` in mode MAX only (others may be NULL);

@@ -35,6 +35,44 @@ def pair(n, a_lu, a_ld, b_lu, b_ld, batch=3, mk=torch.randn):
     return a, b
 
 
+@pytest.mark.parametrize("batch,n,a_lu,a_ld,b_lu,b_ld", [(2, 330, 120, 120, 120, 120), (2, 300, 150, 100, 90, 140),
+                                                         (1, 260, 129, 129, 129, 129), (3, 700, 120, 120, 120, 120),
+                                                         (2, 1400, 120, 120, 120, 120)])
+@pytest.mark.parametrize("mode", [0, 3])
+def test_very_wide_bands_multiply_as_dense_matrices(gpu, batch, n, a_lu, a_ld, b_lu, b_ld, mode):
+    """Bands beyond what the matrix-core band kernels take (about 225 diagonals per operand): where
+    the matrices are small enough, BandedMatrix.multiply / multiply_log go through to_dense, the
+    dense product and banddiag instead of one lane per result cell.  Same values and gradients as the
+    sequential oracle, cells of the bands outside the matrix holding anything; the last shape's log
+    product (a band that leaves most of the dense result empty) stays on the band kernels, as do
+    calls through the C ABI (the two routes agree)."""
+    lib = _lib.load()
+    assert lib.genbmm_banded_on_matrix_cores(a_lu, a_ld, b_lu, b_ld, batch, n) == 0
+    assert lib.genbmm_banded_on_matrix_cores(32, 32, 32, 32, 64, 4096) == 1
+    torch.manual_seed(n + mode)
+    a, b = pair(n, a_lu, a_ld, b_lu, b_ld, batch=batch)
+    a[:, :3, :] += 100.0 * (a[:, :3, :] == 0)
+    b[:, -3:, :] += 100.0 * (b[:, -3:, :] == 0)
+    X = BandedMatrix(a.to(gpu).requires_grad_(True), a_lu, a_ld)
+    Y = BandedMatrix(b.to(gpu).requires_grad_(True), b_lu, b_ld)
+    assert X._dense_pays(Y, mode == 0) == (not (mode == 0 and n == 1400))
+    res = (X.multiply_log if mode == 0 else X.multiply)(Y)
+    assert (res.lu, res.ld) == (a_lu + b_ld, a_ld + b_lu)
+    want, _, _ = oracle.seq_band_fwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, mode, dtype=np.float64)
+    W = a.shape[2] + b.shape[2] - 1
+    atol = 1e-5 * max(1.0, W / 64.0)
+    close(res.data, want, atol=atol)
+    g = torch.randn(batch, n, W)
+    ga, gb = torch.autograd.grad(res.data, (X.data, Y.data), g.to(gpu))
+    wa, wb = oracle.seq_band_bwd(a.double(), a_lu, a_ld, b.double(), b_lu, b_ld, g.double(), mode, dtype=np.float64)
+    close(ga, wa, atol=atol)
+    close(gb, wb, atol=atol)
+    # the band kernels on the same operands (the autograd Functions called directly)
+    fn = genbmm.sparse.bandedlogbmm if mode == 0 else genbmm.sparse.bandedbmm
+    direct = fn(X.data.detach(), a_lu, a_ld, Y.data.detach(), b_lu, b_ld, a_lu + b_ld, a_ld + b_lu)
+    close(direct, res.data, atol=atol)
+
+
 @pytest.mark.parametrize("n,a_lu,a_ld,b_lu,b_ld", BANDS)
 @pytest.mark.parametrize("mode", [0, 1, 3])
 def test_banded_forward_backward(gpu, n, a_lu, a_ld, b_lu, b_ld, mode):
