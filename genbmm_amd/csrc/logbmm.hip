@@ -150,6 +150,55 @@ __global__ __launch_bounds__(256) void k_log_stats(const elem_t* __restrict__ a,
   }
 }
 
+// The same maxima for a problem with few rows and columns and a long K, where the kernel above
+// would walk all of K in a handful of workgroups: the reduction axis in parts, a workgroup per
+// batch item, part and operand, joined by an integer atomic on the bit pattern (max of the
+// pattern for values >= 0, min for negative ones - the order of floats), which commutes: the
+// result is the kernel above's whatever order the parts arrive in.  k_log_stats_init fills the
+// maxima with -inf first.
+__global__ __launch_bounds__(256) void k_log_stats_init(float* __restrict__ stats, int* __restrict__ hdr, long count) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e < count) stats[e] = -INFINITY;
+  if (e == 0) hdr[0] = 0;  // by-products of an earlier forward are stale
+}
+__device__ __forceinline__ void stat_join(float* __restrict__ at, float v) {
+  v += 0.f;  // -0 joins as +0
+  if (v >= 0.f) atomicMax(reinterpret_cast<int*>(at), __float_as_int(v));
+  else if (v > -INFINITY) atomicMin(reinterpret_cast<unsigned*>(at), __float_as_uint(v));
+}
+__global__ __launch_bounds__(256) void k_log_stats_parts(const elem_t* __restrict__ a, const elem_t* __restrict__ b,
+                                                        float* __restrict__ stats, int M, int K, int N, int kparts,
+                                                        int klen) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rows = blockIdx.x & 1, part = (blockIdx.x >> 1) % kparts, batch = (blockIdx.x >> 1) / kparts;
+  const int k0 = part * klen, k1 = min(K, k0 + klen);
+  float* st = stats + (long)batch * (M + N);
+  if (rows) {  // a wave per row, its lanes along k
+    for (int m = wave; m < M; m += 4) {
+      const elem_t* row = a + ((long)batch * M + m) * K;
+      float v = -INFINITY;
+      for (int k = k0 + lane; k < k1; k += 64) v = fmaxf(v, (float)row[k]);
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+      if (lane == 0) stat_join(st + m, v);
+    }
+  } else {  // lanes along n, the waves take every fourth k
+    for (int n0 = 0; n0 < N; n0 += 64) {
+      const int n = n0 + lane;
+      if (n >= N) continue;
+      const elem_t* col = b + (long)batch * K * N + n;
+      float v = -INFINITY;
+      int k = k0 + wave;
+      for (; k + 12 < k1; k += 16) {  // four rows in flight
+        const float x0 = col[(long)k * N], x1 = col[(long)(k + 4) * N], x2 = col[(long)(k + 8) * N], x3 = col[(long)(k + 12) * N];
+        v = fmaxf(fmaxf(fmaxf(fmaxf(v, x0), x1), x2), x3);  // (each maximum against the float: none narrows to the element type)
+      }
+      for (; k < k1; k += 4) v = fmaxf(v, (float)col[(long)k * N]);
+      stat_join(st + M + n, v);
+    }
+  }
+}
+
 // ------------------------------------------------------------ exact kernels
 template <class C>
 __global__ __launch_bounds__(C::NT) void k_log_fwd_exact(const DenseArgs p) {
@@ -732,6 +781,16 @@ int launch_stats(const elem_t* a, const elem_t* b, float* stats, int B, int M, i
   const int64_t total = (int64_t)B * (row_wgs + col_wgs);
   if (total > 0x7fffffffLL) return GENBMM_E_SHAPE;
   if (total == 0) return GENBMM_OK;
+  if (total < 64 && K >= 8192) {  // a handful of workgroups would walk all of K: cut it
+    const int kparts = (int)std::min<int64_t>(std::max<int64_t>(256 / (2 * B), 2), K / 2048);
+    const int klen = ceil_div(ceil_div(K, kparts), 4) * 4;
+    const long count = (long)B * (M + N);
+    hipLaunchKernelGGL(k_log_stats_init, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s, stats,
+                       prepared_of(stats, B, M, K, N).hdr, count);
+    hipLaunchKernelGGL(k_log_stats_parts, dim3((unsigned)(2 * B * ceil_div(K, klen))), dim3(256), 0, s, a, b, stats, M, K,
+                       N, ceil_div(K, klen), klen);
+    return launch_status();
+  }
   hipLaunchKernelGGL(k_log_stats, dim3((unsigned)total), dim3(256), 0, s, a, b, stats,
                      prepared_of(stats, B, M, K, N).hdr, M, K, N, row_wgs, col_wgs, (int)((K % 4 == 0) && aligned16(a)),
                      (int)((N % 4 == 0) && aligned16(b)));

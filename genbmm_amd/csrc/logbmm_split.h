@@ -463,7 +463,17 @@ __global__ __launch_bounds__(256) void k_log_fwd_join(const float* __restrict__ 
     if (m >= M || cc <= 0) continue;
     const long at = ((long)batch * M + m) * N + n;
     float4 sv = ld4m(parts + at, cc, 0.f);
-    for (int p = 1; p < pieces; ++p) {
+    int p = 1;
+    for (; p + 8 <= pieces; p += 8) {  // eight pieces' loads in flight; added in the pieces' order
+      float4 x[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) x[q] = ld4m(parts + (p + q) * piece_stride + at, cc, 0.f);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        sv.x += x[q].x; sv.y += x[q].y; sv.z += x[q].z; sv.w += x[q].w;
+      }
+    }
+    for (; p < pieces; ++p) {
       const float4 x = ld4m(parts + p * piece_stride + at, cc, 0.f);
       sv.x += x.x; sv.y += x.y; sv.z += x.z; sv.w += x.w;
     }
