@@ -69,8 +69,13 @@ def test_very_wide_bands_multiply_as_dense_matrices(gpu, batch, n, a_lu, a_ld, b
     close(gb, wb, atol=atol)
     # the band kernels on the same operands (the autograd Functions called directly)
     fn = genbmm.sparse.bandedlogbmm if mode == 0 else genbmm.sparse.bandedbmm
-    direct = fn(X.data.detach(), a_lu, a_ld, Y.data.detach(), b_lu, b_ld, a_lu + b_ld, a_ld + b_lu)
+    ad, bd = a.to(gpu).requires_grad_(True), b.to(gpu).requires_grad_(True)
+    direct = fn(ad, a_lu, a_ld, bd, b_lu, b_ld, a_lu + b_ld, a_ld + b_lu)
     close(direct, res.data, atol=atol)
+    close(direct, want, atol=atol)
+    da, db = torch.autograd.grad(direct, (ad, bd), g.to(gpu))
+    close(da, wa, atol=atol)
+    close(db, wb, atol=atol)
 
 
 @pytest.mark.parametrize("n,a_lu,a_ld,b_lu,b_ld", BANDS)
